@@ -1,0 +1,225 @@
+/*
+ * moye_hip.h — C ABI of libmoye_hip.so: gfx950 (MI355X) kernels behind MoYe.jl's
+ * `copyto!` / `gemm!` and the host-side layout algebra that computes their descriptors.
+ *
+ * The reference (YichengDWu/MoYe.jl v4.0.1) has no FFI boundary of its own: its atoms call
+ * NVPTX intrinsics from Julia device code.  Each entry point below names the Julia generic
+ * function (reference file:line) whose device work it takes over.  A Julia caller binds
+ * these with `ccall`, the Python mirror with `ctypes`; both pass the same plain structs.
+ *
+ * Conventions
+ *   - every function returns a moye_status (0 = ok); moye_last_error() gives the
+ *     thread-local message of the last failure on the calling thread;
+ *   - pointers inside moye_tensor are BORROWED device pointers, 0-based offsets already
+ *     folded in; descriptors are copied at call time;
+ *   - shapes/strides are the FLATTENED layout of a MoYeArray (src/array.jl:53-59), strides
+ *     in elements, non-negative;
+ *   - kernels are enqueued on the caller's stream (NULL = default stream) and the call
+ *     returns without waiting.
+ */
+#ifndef MOYE_HIP_H
+#define MOYE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MOYE_MAX_RANK 8
+
+typedef enum {
+    MOYE_OK = 0,
+    MOYE_ERR_RANK = 1,        /* DimensionMismatch: wrong number of modes                       */
+    MOYE_ERR_SHAPE = 2,       /* size mismatch / tile does not divide (shape_div assert)        */
+    MOYE_ERR_UNSUPPORTED = 3, /* dtype / atom / operand major this build has no kernel for      */
+    MOYE_ERR_ALIGN = 4,       /* pointer or leading dimension not aligned for the vector width  */
+    MOYE_ERR_HIP = 5,         /* a HIP runtime call failed                                       */
+    MOYE_ERR_ARG = 6,         /* NULL or out-of-range argument                                   */
+    MOYE_ERR_PARSE = 7,       /* malformed layout / tuple text                                   */
+    MOYE_ERR_BUFFER = 8       /* output text buffer too small                                    */
+} moye_status;
+
+typedef enum {
+    MOYE_F32 = 0, MOYE_F16 = 1, MOYE_BF16 = 2, MOYE_F8E4M3 = 3, MOYE_F64 = 4,
+    MOYE_U8 = 5, MOYE_U16 = 6, MOYE_U32 = 7, MOYE_U64 = 8, MOYE_U128 = 9
+} moye_dtype;
+
+/* address-space tag of src/pointer.jl:1-7 (isgmem / issmem / isrmem) */
+typedef enum { MOYE_GMEM = 0, MOYE_SMEM = 1, MOYE_RMEM = 2 } moye_memspace;
+
+/* a MoYeArray over a ViewEngine (src/array.jl:53-59, src/engine.jl:6-50), flattened */
+typedef struct {
+    void*   ptr;
+    int32_t dtype;      /* moye_dtype    */
+    int32_t memspace;   /* moye_memspace */
+    int32_t rank;       /* 1..MOYE_MAX_RANK */
+    int32_t _pad;
+    int64_t shape[MOYE_MAX_RANK];
+    int64_t stride[MOYE_MAX_RANK];
+} moye_tensor;
+
+/* MMA atoms: UniversalFMA (src/arch/mma/mma.jl:53-64) plus the gfx950 MFMA instructions that
+ * take the place of the reference's MMAOP_* table (src/arch/mma/make_mma_ops.jl:426-438). */
+typedef enum {
+    MOYE_MMA_UNIVERSAL_FMA = 0,
+    MOYE_MFMA_F32_16x16x32_F16 = 1,
+    MOYE_MFMA_F32_32x32x16_F16 = 2,
+    MOYE_MFMA_F32_16x16x32_BF16 = 3,
+    MOYE_MFMA_F32_32x32x16_BF16 = 4,
+    MOYE_MFMA_F32_16x16x32_FP8 = 5,
+    MOYE_MFMA_F32_32x32x16_FP8 = 6,
+    MOYE_MFMA_F32_16x16x4_F32 = 7,
+    MOYE_MFMA_F32_32x32x2_F32 = 8
+} moye_mma_atom;
+
+/* a TiledMMA (src/atom/mma.jl:80-92) plus the CTA tile the caller's shared-memory layouts
+ * imply (bM,bN,bK of test/device/matmul.jl:11-13) and schedule options */
+typedef struct {
+    int32_t atom;                  /* moye_mma_atom                                           */
+    int32_t atom_layout_mnk[3];    /* shape of TiledMMA.atom_layout_mnk (atom/mma.jl:84)       */
+    int32_t tile_mnk[3];           /* tile_size(mma, 1..3) (atom/mma.jl:178-191)               */
+    int32_t cta_tile_mnk[3];       /* bM, bN, bK; 0 = let the library choose                    */
+    int32_t stages;                /* LDS pipeline depth, 0 = default                           */
+    int32_t split_k;               /* 0/1 = none; >1 = deterministic two-pass split-K           */
+    int32_t flags;                 /* MOYE_GEMM_* bits                                          */
+} moye_tiled_mma;
+
+#define MOYE_GEMM_NO_XCD_SWIZZLE 1   /* keep blockIdx -> tile mapping linear (for A/B studies)  */
+#define MOYE_GEMM_NO_LDS_SWIZZLE 2   /* linear LDS tiles (bank-conflict study)                  */
+
+/* copy ops: UniversalCopy (src/arch/copy/copy.jl:26-51); the LDS-staged forms stand where the
+ * reference has cp.async (copy_async.jl:8-24) and ldmatrix (ldmatrix.jl:18-48) */
+typedef enum {
+    MOYE_COPY_UNIVERSAL = 0,       /* element-wise through both layouts                        */
+    MOYE_COPY_LDS_TILED = 1        /* 128-bit global loads -> XOR-swizzled LDS tile -> 128-bit  */
+} moye_copy_op;
+
+/* a TiledCopy (src/atom/copy.jl:86-90) reduced to what the kernels consume */
+typedef struct {
+    int32_t op;                    /* moye_copy_op                                             */
+    int32_t vec_bits;              /* bits per access of the atom: 8..128 (UniversalCopy{UIntN}) */
+    int32_t thr_shape[2];          /* thr_layout of make_tiled_copy (atom/copy.jl:249-258)      */
+    int32_t val_shape[2];          /* val_layout                                                */
+    int32_t tiler_mn[2];           /* tiler_MN = LDS tile, e.g. 64x64                           */
+    int32_t flags;
+} moye_tiled_copy;
+
+/* ---- device loops ------------------------------------------------------------------------ */
+
+/* Base.copyto!(dest::MoYeArray, src::MoYeArray) (src/algorithm/copy.jl:42-64) and
+ * Base.copyto!(tiled_copy, dst, src) (src/algorithm/copy.jl:106-130): logical element i of
+ * src goes to logical element i of dst through both layouts; bit-exact when the dtypes
+ * agree, round-to-nearest-even conversion otherwise (src/arch/copy/copy.jl:38-43).
+ * `tc` may be NULL (plain copyto!). */
+int32_t moye_copy(const moye_tiled_copy* tc, const moye_tensor* dst, const moye_tensor* src,
+                  void* stream);
+
+/* gemm!(mma, D, A, B, C) (src/algorithm/blas.jl:11-17 and the dispatch tower :20-131) driven
+ * over a whole problem the way the reference's user kernels drive it
+ * (test/device/matmul.jl:3-53, docs/src/manual/tensor_core.md:265-355):
+ * A:(M,K), B:(N,K), C,D:(M,N);  D = alpha * (A * B') + C.   C may be NULL (zero-init
+ * accumulator, `zeros!(tCrC)`); D may alias C.  With MOYE_MMA_UNIVERSAL_FMA the arithmetic is
+ * the reference's exactly (product rounded in the input type, unfused add, k ascending). */
+int32_t moye_gemm(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A,
+                  const moye_tensor* B, const moye_tensor* C, float alpha, void* stream);
+
+/* bytes of device workspace moye_gemm needs for this call (split-K partials); 0 if none.
+ * The library allocates it internally on first use and keeps it. */
+int32_t moye_gemm_workspace_size(const moye_tiled_mma* mma, const moye_tensor* D,
+                                 const moye_tensor* A, const moye_tensor* B, size_t* bytes);
+
+/* ---- host-side layout algebra (no GPU needed) ------------------------------------------- */
+/* Text form of a layout: `shape:stride`, `_n` = static int, `n` = dynamic int, e.g.
+ * "(_2, (_1, _6)):(_1, (_6, _2))"; a bare shape means the compact column-major layout
+ * (make_layout(shape), src/layout.jl:141-144).  Tiles: a layout, an int, `:` or `<t1, t2, ..>`.
+ * Results are written to `out` (capacity `cap` bytes, NUL-terminated). */
+int32_t moye_layout_normalize(const char* layout, char* out, size_t cap);                    /* parse + print  */
+int32_t moye_layout_eval(const char* layout, const char* coord, int64_t* index);             /* layout.jl:90-102 (1-based) */
+int32_t moye_layout_size(const char* layout, int64_t* size);                                 /* layout.jl:302-304 */
+int32_t moye_layout_cosize(const char* layout, int64_t* cosize);                             /* layout.jl:350-352 */
+int32_t moye_layout_rank_depth(const char* layout, int32_t* rank, int32_t* depth);           /* layout.jl:321-343 */
+int32_t moye_layout_flatten(const char* layout, char* out, size_t cap);                      /* layout.jl:292-294 */
+int32_t moye_layout_coalesce(const char* layout, char* out, size_t cap);                     /* layout.jl:497-502 */
+int32_t moye_layout_filter(const char* layout, char* out, size_t cap);                       /* layout.jl:515-517 */
+int32_t moye_layout_composition(const char* lhs, const char* rhs_tile, char* out, size_t cap); /* layout.jl:593-612 */
+int32_t moye_layout_complement(const char* layout, const char* cotarget, char* out, size_t cap); /* layout.jl:660-668; cotarget "" = cosize */
+int32_t moye_layout_right_inverse(const char* layout, char* out, size_t cap);                /* layout.jl:717-730 */
+int32_t moye_layout_left_inverse(const char* layout, char* out, size_t cap);                 /* layout.jl:738 */
+int32_t moye_layout_max_common_vector(const char* a, const char* b, int64_t* n);             /* layout.jl:752-761 */
+int32_t moye_layout_logical_product(const char* layout, const char* tile, char* out, size_t cap); /* layout.jl:826-838 */
+int32_t moye_layout_zipped_product(const char* layout, const char* tile, char* out, size_t cap);  /* layout.jl:840-842 */
+int32_t moye_layout_tiled_product(const char* layout, const char* tile, char* out, size_t cap);   /* layout.jl:844-847 */
+int32_t moye_layout_blocked_product(const char* block, const char* layout, int32_t coalesce_result, char* out, size_t cap); /* layout.jl:880-889 */
+int32_t moye_layout_raked_product(const char* block, const char* layout, int32_t coalesce_result, char* out, size_t cap);   /* layout.jl:919-928 */
+int32_t moye_layout_logical_divide(const char* layout, const char* tile, char* out, size_t cap);  /* layout.jl:1058-1070 */
+int32_t moye_layout_zipped_divide(const char* layout, const char* tile, char* out, size_t cap);   /* layout.jl:1114-1116 */
+int32_t moye_layout_tiled_divide(const char* layout, const char* tile, char* out, size_t cap);    /* layout.jl:1123-1127 */
+int32_t moye_layout_recast(const char* layout, int32_t new_bytes, int32_t old_bytes, char* out, size_t cap); /* layout.jl:999-1010 */
+int32_t moye_layout_append(const char* layout, int32_t rank, char* out, size_t cap);         /* layout.jl:377-389 */
+int32_t moye_layout_prepend(const char* layout, int32_t rank, char* out, size_t cap);        /* layout.jl:391-397 */
+int32_t moye_layout_make_ordered(const char* shape, const char* order, char* out, size_t cap); /* layout.jl:216-218 */
+int32_t moye_layout_make_fragment_like(const char* layout, char* out, size_t cap);           /* layout.jl:1143-1149 */
+int32_t moye_layout_slice(const char* layout, const char* coord, char* out, size_t cap, int64_t* offset); /* slice_and_offset, layout.jl:368-371 */
+int32_t moye_layout_make(const char* shape, int32_t row_major, char* out, size_t cap);        /* make_layout(shape, GenColMajor|GenRowMajor), layout.jl:154-159 */
+
+/* IntTuple helpers (src/int_tuple.jl, src/stride.jl) on tuple text such as "(3,(2,2))" */
+int32_t moye_tuple_op(const char* op, const char* a, const char* b, const char* c, char* out, size_t cap);
+
+/* @tile / local_tile (src/algorithm/array_algorithms.jl:113-120) and @parallelize /
+ * local_partition (:36-47) on a layout: the sliced layout and the 0-based element offset.
+ * `proj` may be "" (none). */
+int32_t moye_local_tile(const char* layout, const char* tile, const char* coord, const char* proj,
+                        char* out, size_t cap, int64_t* offset);
+int32_t moye_local_partition(const char* layout, const char* thr_tile, const char* coord_or_index,
+                             const char* proj, char* out, size_t cap, int64_t* offset);
+
+/* TiledMMA (src/atom/mma.jl): `atom` is a moye_mma_atom or the name of one of the reference's
+ * NVIDIA atoms kept as data for its tests ("MMAOP_16x8x8_F16F16F16F16_TN", ...).
+ * what = "thr_layout_vmnk" | "tile_shape" | "layout_a" | "layout_b" | "layout_c" |
+ *        "layoutA_TV" | "layoutB_TV" | "layoutC_TV" | "size"                                  */
+int32_t moye_tiled_mma_query(const char* atom, const char* atom_layout, const char* permutation,
+                             const char* what, char* out, size_t cap);
+/* partition_A/B/C of get_slice(mma, thr_idx) (atom/mma.jl:171-175,292-308); operand = 'A'|'B'|'C' */
+int32_t moye_tiled_mma_partition(const char* atom, const char* atom_layout, const char* permutation,
+                                 int32_t thr_idx, char operand, const char* layout,
+                                 char* out, size_t cap, int64_t* offset);
+/* make_tiled_copy (atom/copy.jl:249-258): src/dst bits of UniversalCopy{S,D}, value bits of T.
+ * what = "layout_tv" | "tiler" | "num_val_src" | "num_val_dst" | "size"                        */
+int32_t moye_tiled_copy_query(int32_t src_bits, int32_t dst_bits, int32_t val_bits,
+                              const char* thr_layout, const char* val_layout, const char* what,
+                              char* out, size_t cap);
+/* partition_S / partition_D of get_slice(tiled_copy, thr_idx) (atom/copy.jl:206-214); which = 'S'|'D' */
+int32_t moye_tiled_copy_partition(int32_t src_bits, int32_t dst_bits, int32_t val_bits,
+                                  const char* thr_layout, const char* val_layout, int32_t thr_idx,
+                                  char which, const char* layout, char* out, size_t cap, int64_t* offset);
+/* fill a moye_tiled_mma from MoYe-level arguments (checks that the atom layout and the
+ * permutation sizes describe a tile this build has a kernel for) */
+int32_t moye_make_tiled_mma(int32_t atom, const char* atom_layout, const char* permutation,
+                            moye_tiled_mma* out);
+
+/* ---- runtime helpers (thin wrappers so a non-HIP host language needs nothing else) ------- */
+int32_t moye_device_malloc(void** ptr, size_t bytes);
+int32_t moye_device_free(void* ptr);
+int32_t moye_memcpy_h2d(void* dst, const void* src, size_t bytes);
+int32_t moye_memcpy_d2h(void* dst, const void* src, size_t bytes);
+int32_t moye_memset(void* dst, int value, size_t bytes);
+int32_t moye_device_sync(void);
+int32_t moye_device_info(char* name, size_t cap, int32_t* compute_units, int32_t* clock_khz,
+                         size_t* total_mem);
+/* time `iters` back-to-back launches of the same moye_gemm / moye_copy call with HIP events on
+ * `stream`; returns the average milliseconds per launch */
+int32_t moye_time_gemm(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A,
+                       const moye_tensor* B, const moye_tensor* C, float alpha, void* stream,
+                       int32_t warmup, int32_t iters, float* ms_per_launch);
+int32_t moye_time_copy(const moye_tiled_copy* tc, const moye_tensor* dst, const moye_tensor* src,
+                       void* stream, int32_t warmup, int32_t iters, float* ms_per_launch);
+
+const char* moye_last_error(void);
+const char* moye_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOYE_HIP_H */

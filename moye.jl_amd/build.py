@@ -1,0 +1,74 @@
+"""Builds libmoye_hip.so for gfx950 with hipcc (cross-compiles without a GPU).
+
+    python moye.jl_amd/build.py [--force]
+
+Objects go to csrc/build/, the library next to the Python mirror as moye_hip/libmoye_hip.so.
+"""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OUT = os.path.join(HERE, "moye_hip", "libmoye_hip.so")
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+COMMON = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
+          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+# source -> extra flags
+SOURCES = {
+    "capi.hip": [],
+    "copy_kernels.hip": [],
+    "gemm_mfma.hip": [],
+    "gemm_universal.hip": ["-ffp-contract=off"],   # UniversalFMA: mul then add, never fused
+    "layout_host.cpp": ["-x", "hip"],
+}
+
+
+def _headers():
+    return [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".hpp", ".h"))] + \
+        [os.path.join(HERE, "..", "include", "moye_hip.h")]
+
+
+def _stale(target, deps):
+    if not os.path.exists(target):
+        return True
+    t = os.path.getmtime(target)
+    return any(os.path.getmtime(d) > t for d in deps)
+
+
+def _compile(item, force):
+    src, extra = item
+    path = os.path.join(CSRC, src)
+    obj = os.path.join(CSRC, "build", os.path.splitext(src)[0] + ".o")
+    if not force and not _stale(obj, [path] + _headers()):
+        return obj, ""
+    cmd = [HIPCC] + COMMON + extra + ["-c", path, "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "not a recognized feature for this target"
+    err = "\n".join(l for l in (r.stdout + r.stderr).splitlines() if noise not in l)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed for %s:\n%s" % (src, err))
+    return obj, err
+
+
+def build(force=False, verbose=True):
+    os.makedirs(os.path.join(CSRC, "build"), exist_ok=True)
+    items = [(s, f) for s, f in SOURCES.items() if os.path.exists(os.path.join(CSRC, s))]
+    with ThreadPoolExecutor(max_workers=min(8, len(items))) as ex:
+        results = list(ex.map(lambda it: _compile(it, force), items))
+    objs = [o for o, _ in results]
+    for (src, _), (_, msg) in zip(items, results):
+        if msg.strip() and verbose:
+            print("[%s]\n%s" % (src, msg))
+    if force or _stale(OUT, objs):
+        cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", OUT] + objs
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("link failed:\n" + r.stdout + r.stderr)
+    return OUT
+
+
+if __name__ == "__main__":
+    print(build(force="--force" in sys.argv))

@@ -1,0 +1,219 @@
+// C entry points of libmoye_hip for the device loops and the small runtime helpers.
+// Descriptor validation lives here: the shape/divisibility violations the reference raises as
+// Julia assertions while tracing (src/algorithm/blas.jl:55-57,79-82, src/int_tuple.jl:88,
+// src/atom/copy.jl:121-122) come back as status codes before any kernel is launched.
+#include <cstring>
+#include <mutex>
+
+#include "kernels.hpp"
+
+namespace moye {
+
+std::string& last_error() {
+    thread_local std::string e;
+    return e;
+}
+
+int32_t fail(moye_status st, const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    last_error() = buf;
+    return (int32_t)st;
+}
+
+int32_t check_tensor(const moye_tensor* t, const char* what) {
+    if (!t) return fail(MOYE_ERR_ARG, "%s: null tensor descriptor", what);
+    if (t->rank < 1 || t->rank > MOYE_MAX_RANK)
+        return fail(MOYE_ERR_RANK, "%s: rank %d outside 1..%d", what, t->rank, MOYE_MAX_RANK);
+    if (dtype_bytes(t->dtype) == 0) return fail(MOYE_ERR_UNSUPPORTED, "%s: unknown dtype %d", what, t->dtype);
+    for (int i = 0; i < t->rank; ++i) {
+        if (t->shape[i] < 0) return fail(MOYE_ERR_SHAPE, "%s: negative extent in mode %d", what, i + 1);
+        if (t->stride[i] < 0) return fail(MOYE_ERR_UNSUPPORTED, "%s: negative strides are not supported", what);
+    }
+    if (tensor_size(*t) > 0 && !t->ptr) return fail(MOYE_ERR_ARG, "%s: null data pointer", what);
+    if (t->memspace != MOYE_GMEM)
+        return fail(MOYE_ERR_UNSUPPORTED, "%s: only global-memory arrays cross the C ABI (shared memory and registers "
+                                          "live inside the kernels)", what);
+    return MOYE_OK;
+}
+
+int32_t as_matrix(const moye_tensor* t, const char* what, Mat* m) {
+    if (int32_t e = check_tensor(t, what)) return e;
+    if (t->rank != 2) return fail(MOYE_ERR_RANK, "%s: gemm! operands are rank-2, got rank %d", what, t->rank);
+    m->ptr = static_cast<char*>(t->ptr);
+    m->rows = t->shape[0];
+    m->cols = t->shape[1];
+    m->rs = t->stride[0];
+    m->cs = t->stride[1];
+    m->dtype = t->dtype;
+    return MOYE_OK;
+}
+
+static int32_t atom_input_dtype(int32_t atom) {
+    switch (atom) {
+        case MOYE_MFMA_F32_16x16x32_F16: case MOYE_MFMA_F32_32x32x16_F16: return MOYE_F16;
+        case MOYE_MFMA_F32_16x16x32_BF16: case MOYE_MFMA_F32_32x32x16_BF16: return MOYE_BF16;
+        case MOYE_MFMA_F32_16x16x32_FP8: case MOYE_MFMA_F32_32x32x16_FP8: return MOYE_F8E4M3;
+        case MOYE_MFMA_F32_16x16x4_F32: case MOYE_MFMA_F32_32x32x2_F32: return MOYE_F32;
+        default: return -1;
+    }
+}
+
+static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const moye_tensor* tA,
+                         const moye_tensor* tB, const moye_tensor* tC, float alpha, hipStream_t st) {
+    if (!mma) return fail(MOYE_ERR_ARG, "gemm!: null TiledMMA descriptor");
+    Mat A, B, C{}, D;
+    if (int32_t e = as_matrix(tA, "A", &A)) return e;
+    if (int32_t e = as_matrix(tB, "B", &B)) return e;
+    if (int32_t e = as_matrix(tD, "D", &D)) return e;
+    if (tC) {
+        if (int32_t e = as_matrix(tC, "C", &C)) return e;
+    }
+    // blas.jl:55-57,79-82: size(A,1)==size(C,1), size(B,1)==size(C,2), size(A,2)==size(B,2)
+    if (A.rows != D.rows) return fail(MOYE_ERR_SHAPE, "gemm!: M of A (%lld) and D (%lld) differ", (long long)A.rows, (long long)D.rows);
+    if (B.rows != D.cols) return fail(MOYE_ERR_SHAPE, "gemm!: N of B (%lld) and D (%lld) differ", (long long)B.rows, (long long)D.cols);
+    if (A.cols != B.cols) return fail(MOYE_ERR_SHAPE, "gemm!: K of A (%lld) and B (%lld) differ", (long long)A.cols, (long long)B.cols);
+    if (tC && (C.rows != D.rows || C.cols != D.cols)) return fail(MOYE_ERR_SHAPE, "gemm!: C and D differ in shape");
+    if (A.rows > 0x7fffffff || B.rows > 0x7fffffff || A.cols > 0x7fffffff)
+        return fail(MOYE_ERR_SHAPE, "gemm!: extents above 2^31-1 are not supported");
+    if (A.rows == 0 || B.rows == 0) return MOYE_OK;
+    const int M = (int)A.rows, N = (int)B.rows, K = (int)A.cols;
+    const int bm = mma->cta_tile_mnk[0], bn = mma->cta_tile_mnk[1], bk = mma->cta_tile_mnk[2];
+
+    if (mma->atom == MOYE_MMA_UNIVERSAL_FMA) {
+        UArgs u{A.ptr, B.ptr, tC ? C.ptr : nullptr, D.ptr, M, N, K, A.rs, A.cs, B.rs, B.cs,
+                C.rs, C.cs, D.rs, D.cs, alpha, A.dtype, B.dtype, tC ? C.dtype : D.dtype, D.dtype};
+        return gemm_universal_dispatch(bm, bn, bk, u, st);
+    }
+    const int32_t in_dt = atom_input_dtype(mma->atom);
+    if (in_dt < 0) return fail(MOYE_ERR_UNSUPPORTED, "gemm!: unknown MMA atom %d", mma->atom);
+    if (A.dtype != in_dt || B.dtype != in_dt)
+        return fail(MOYE_ERR_UNSUPPORTED, "gemm!: atom takes %s operands, got A %s and B %s", dtype_name(in_dt),
+                    dtype_name(A.dtype), dtype_name(B.dtype));
+    if (tC && C.dtype != D.dtype) return fail(MOYE_ERR_UNSUPPORTED, "gemm!: C and D must have the same element type");
+    if (in_dt == MOYE_F32)
+        return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the fp32 MFMA atoms have no kernel yet; use MOYE_MMA_UNIVERSAL_FMA");
+    if (K > 0 && (A.cs != 1 || B.cs != 1))
+        return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the MFMA kernels need K-major A and B (stride 1 along K, the 'TN' form)");
+    if (K == 0) return fail(MOYE_ERR_SHAPE, "gemm!: K == 0");
+    GemmArgs g{};
+    g.alpha = alpha;
+    g.K = K;
+    g.xcd_swizzle = !(mma->flags & MOYE_GEMM_NO_XCD_SWIZZLE);
+    if (D.cs == 1) {  // row-major D
+        g.A = A.ptr; g.B = B.ptr; g.M = M; g.N = N; g.lda = A.rs; g.ldb = B.rs; g.ldd = D.rs;
+        g.C = tC ? C.ptr : nullptr; g.ldc_m = C.rs; g.ldc_n = C.cs; g.D = D.ptr;
+        return gemm_mfma_tn_dispatch(in_dt, D.dtype, bm, bn, bk, g, st);
+    }
+    if (D.rs == 1) {  // column-major D: D' = B * A' is row-major
+        g.A = B.ptr; g.B = A.ptr; g.M = N; g.N = M; g.lda = B.rs; g.ldb = A.rs; g.ldd = D.cs;
+        g.C = tC ? C.ptr : nullptr; g.ldc_m = C.cs; g.ldc_n = C.rs; g.D = D.ptr;
+        return gemm_mfma_tn_dispatch(in_dt, D.dtype, bn, bm, bk, g, st);
+    }
+    return fail(MOYE_ERR_UNSUPPORTED, "gemm!: D needs a unit stride along M or N");
+}
+
+// Average launch time of `iters` back-to-back launches, HIP events on the launch stream.
+template <typename F>
+static int32_t time_launches(F&& launch, hipStream_t st, int warmup, int iters, float* ms) {
+    if (!ms || iters <= 0 || warmup < 0) return fail(MOYE_ERR_ARG, "timing: bad arguments");
+    for (int i = 0; i < warmup; ++i)
+        if (int32_t e = launch()) return e;
+    hipEvent_t t0, t1;
+    MOYE_HIP_CHECK(hipEventCreate(&t0));
+    MOYE_HIP_CHECK(hipEventCreate(&t1));
+    MOYE_HIP_CHECK(hipEventRecord(t0, st));
+    int32_t err = MOYE_OK;
+    for (int i = 0; i < iters && !err; ++i) err = launch();
+    MOYE_HIP_CHECK(hipEventRecord(t1, st));
+    MOYE_HIP_CHECK(hipEventSynchronize(t1));
+    float total = 0.f;
+    MOYE_HIP_CHECK(hipEventElapsedTime(&total, t0, t1));
+    (void)hipEventDestroy(t0);
+    (void)hipEventDestroy(t1);
+    if (err) return err;
+    *ms = total / (float)iters;
+    return MOYE_OK;
+}
+
+}  // namespace moye
+
+using namespace moye;
+
+extern "C" {
+
+int32_t moye_copy(const moye_tiled_copy* tc, const moye_tensor* dst, const moye_tensor* src, void* stream) {
+    return copy_dispatch(tc, dst, src, static_cast<hipStream_t>(stream));
+}
+
+int32_t moye_gemm(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A, const moye_tensor* B,
+                  const moye_tensor* C, float alpha, void* stream) {
+    return gemm_impl(mma, D, A, B, C, alpha, static_cast<hipStream_t>(stream));
+}
+
+int32_t moye_gemm_workspace_size(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A,
+                                 const moye_tensor* B, size_t* bytes) {
+    if (!mma || !D || !A || !B || !bytes) return fail(MOYE_ERR_ARG, "moye_gemm_workspace_size: null argument");
+    *bytes = 0;
+    return MOYE_OK;
+}
+
+int32_t moye_device_malloc(void** ptr, size_t bytes) {
+    if (!ptr) return fail(MOYE_ERR_ARG, "moye_device_malloc: null out pointer");
+    MOYE_HIP_CHECK(hipMalloc(ptr, bytes));
+    return MOYE_OK;
+}
+int32_t moye_device_free(void* ptr) {
+    MOYE_HIP_CHECK(hipFree(ptr));
+    return MOYE_OK;
+}
+int32_t moye_memcpy_h2d(void* dst, const void* src, size_t bytes) {
+    MOYE_HIP_CHECK(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
+    return MOYE_OK;
+}
+int32_t moye_memcpy_d2h(void* dst, const void* src, size_t bytes) {
+    MOYE_HIP_CHECK(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
+    return MOYE_OK;
+}
+int32_t moye_memset(void* dst, int value, size_t bytes) {
+    MOYE_HIP_CHECK(hipMemset(dst, value, bytes));
+    return MOYE_OK;
+}
+int32_t moye_device_sync(void) {
+    MOYE_HIP_CHECK(hipDeviceSynchronize());
+    return MOYE_OK;
+}
+int32_t moye_device_info(char* name, size_t cap, int32_t* compute_units, int32_t* clock_khz, size_t* total_mem) {
+    int dev = 0;
+    MOYE_HIP_CHECK(hipGetDevice(&dev));
+    hipDeviceProp_t prop;
+    MOYE_HIP_CHECK(hipGetDeviceProperties(&prop, dev));
+    if (name && cap) {
+        snprintf(name, cap, "%s (%s)", prop.name, prop.gcnArchName);
+    }
+    if (compute_units) *compute_units = prop.multiProcessorCount;
+    if (clock_khz) *clock_khz = prop.clockRate;
+    if (total_mem) *total_mem = prop.totalGlobalMem;
+    return MOYE_OK;
+}
+
+int32_t moye_time_gemm(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A, const moye_tensor* B,
+                       const moye_tensor* C, float alpha, void* stream, int32_t warmup, int32_t iters,
+                       float* ms_per_launch) {
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    return time_launches([&] { return gemm_impl(mma, D, A, B, C, alpha, st); }, st, warmup, iters, ms_per_launch);
+}
+
+int32_t moye_time_copy(const moye_tiled_copy* tc, const moye_tensor* dst, const moye_tensor* src, void* stream,
+                       int32_t warmup, int32_t iters, float* ms_per_launch) {
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    return time_launches([&] { return copy_dispatch(tc, dst, src, st); }, st, warmup, iters, ms_per_launch);
+}
+
+const char* moye_last_error(void) { return last_error().c_str(); }
+const char* moye_version(void) { return "moye_hip 0.1.0 (gfx950)"; }
+
+}  // extern "C"

@@ -1,0 +1,354 @@
+// copyto! on the device: layout-driven copy kernels for gfx950.
+//
+// Takes over the element loop of the reference's `copyto!`
+// (src/algorithm/copy.jl:4-12,42-64 and :106-130): logical element i of src goes to logical
+// element i of dst through both layouts.  Three kernels:
+//   transpose_lds   rank-2, the unit-stride mode differs between src and dst: 128-bit global
+//                   loads, 4x4 register transpose, XOR-swizzled LDS tile, 128-bit stores
+//   copy_flat       both sides contiguous in the same order: 128-bit streaming copy
+//   copy_generic    anything else: per-element gather/scatter with optional conversion
+#include "kernels.hpp"
+
+namespace moye {
+
+// ------------------------------------------------------------------------------------------
+// transpose through a 64x64 LDS tile
+// ------------------------------------------------------------------------------------------
+// src(i, j) at i + j*lds   (i is the contiguous index),  dst(i, j) at i*ldd + j.
+// One workgroup of 256 threads moves one 64x64 tile of 4-byte elements.
+//
+// LDS tile T[64 rows = i][16 chunks of 4 = j]; the chunk index is XORed with (row>>2)&15 so
+// that the 16 lanes which write one float4 each to 16 different rows, and the 16 lanes which
+// read 16 different chunks of one row, both touch all 64 banks exactly once.
+
+constexpr int kTile = 64;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));  // one 128-bit access
+
+template <bool kSwizzle>
+__device__ __forceinline__ int lds_chunk(int row, int chunk) {
+    return kSwizzle ? (chunk ^ ((row >> 2) & 15)) : chunk;
+}
+
+// tile index -> (ti, tj): tiles are visited in square super-blocks of `sb` x `sb` tiles so
+// that the workgroups in flight read and write runs of sb*256 contiguous bytes per row on
+// BOTH sides (a plain row-major order makes one side hop a full leading dimension per tile).
+__device__ __forceinline__ void tile_coords(int64_t t, int tiles_i, int tiles_j, int sb,
+                                            int* ti, int* tj) {
+    const int64_t per_band = (int64_t)sb * tiles_i;       // a band = sb tile-columns (j), all i
+    const int band = (int)(t / per_band);
+    const int64_t r = t - (int64_t)band * per_band;
+    const int band_w = min(sb, tiles_j - band * sb);      // last band may be narrower
+    const int blk = (int)(r / ((int64_t)sb * band_w));    // block of sb tiles along i
+    const int64_t q = r - (int64_t)blk * sb * band_w;
+    const int blk_h = min(sb, tiles_i - blk * sb);
+    // inside a block: i fastest
+    *ti = blk * sb + (int)(q % blk_h);
+    *tj = band * sb + (int)(q / blk_h);
+}
+
+template <bool kSwizzle>
+__global__ __launch_bounds__(256) void transpose_lds_b32(const uint32_t* __restrict__ src,
+                                                         uint32_t* __restrict__ dst, int64_t lds_,
+                                                         int64_t ldd, int tiles_i, int tiles_j,
+                                                         int sb) {
+    __shared__ u32x4 tile[kTile * (kTile / 4)];
+    int ti, tj;
+    tile_coords(blockIdx.x, tiles_i, tiles_j, sb, &ti, &tj);
+
+    const int lane16 = threadIdx.x & 15;  // chunk of 4 along the contiguous index
+    const int grp = threadIdx.x >> 4;     // 0..15
+
+    // ---- load: rows j = 4*grp+q, columns i = 4*lane16 .. +3 ----
+    const uint32_t* s = src + ((int64_t)tj * kTile + 4 * grp) * lds_ + (int64_t)ti * kTile + 4 * lane16;
+    u32x4 v[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+        v[q] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(s + q * lds_));
+
+    // ---- 4x4 register transpose, store float4 over j into row i of the LDS tile ----
+    const uint32_t a[4][4] = {{v[0].x, v[0].y, v[0].z, v[0].w},
+                              {v[1].x, v[1].y, v[1].z, v[1].w},
+                              {v[2].x, v[2].y, v[2].z, v[2].w},
+                              {v[3].x, v[3].y, v[3].z, v[3].w}};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int row = 4 * lane16 + e;  // i within the tile
+        tile[row * 16 + lds_chunk<kSwizzle>(row, grp)] = u32x4{a[0][e], a[1][e], a[2][e], a[3][e]};
+    }
+    __syncthreads();
+
+    // ---- store: rows i = grp + 16*p, columns j = 4*lane16 .. +3 ----
+    uint32_t* d = dst + ((int64_t)ti * kTile + grp) * ldd + (int64_t)tj * kTile + 4 * lane16;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const int row = grp + 16 * p;
+        const u32x4 w = tile[row * 16 + lds_chunk<kSwizzle>(row, lane16)];
+        __builtin_nontemporal_store(w, reinterpret_cast<u32x4*>(d + (int64_t)16 * p * ldd));
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// contiguous streaming copy, 16 bytes per lane per step
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void copy_flat_b128(const u32x4* __restrict__ src,
+                                                      u32x4* __restrict__ dst, int64_t n16) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride)
+        __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+}
+
+__global__ __launch_bounds__(256) void copy_flat_bytes(const uint8_t* __restrict__ src,
+                                                       uint8_t* __restrict__ dst, int64_t n) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = src[i];
+}
+
+// ------------------------------------------------------------------------------------------
+// generic gather/scatter with conversion
+// ------------------------------------------------------------------------------------------
+struct FlatLayout {
+    int32_t rank;
+    int64_t shape[MOYE_MAX_RANK];
+    int64_t stride[MOYE_MAX_RANK];
+};
+
+// colexicographic decomposition of a 0-based linear index (src/stride.jl:20-31)
+__device__ __forceinline__ int64_t layout_offset(const FlatLayout& l, int64_t i) {
+    int64_t off = 0;
+#pragma unroll 1
+    for (int m = 0; m < l.rank; ++m) {
+        const int64_t s = l.shape[m];
+        const int64_t q = i / s;
+        off += (i - q * s) * l.stride[m];
+        i = q;
+    }
+    return off;
+}
+
+__device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
+
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {  // round to nearest even
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);  // quiet NaN
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float f8e4m3_to_f32(uint8_t b) {  // OCP e4m3fn
+    const uint32_t sign = (uint32_t)(b & 0x80) << 24;
+    const int e = (b >> 3) & 0xf;
+    const int m = b & 7;
+    if (e == 0xf && m == 7) return __uint_as_float(sign | 0x7fc00000u);
+    if (e == 0) return __uint_as_float(sign) + (sign ? -1.f : 1.f) * (float)m * 0.001953125f;  // m * 2^-9
+    return __uint_as_float(sign | ((uint32_t)(e + 120) << 23) | ((uint32_t)m << 20));
+}
+
+__device__ __forceinline__ uint8_t f32_to_f8e4m3(float f) {  // RNE; |x| > 464 and NaN -> NaN
+    const uint32_t u = __float_as_uint(f);
+    const uint8_t sign = (uint8_t)((u >> 24) & 0x80);
+    const float a = fabsf(f);
+    if (!(a <= 464.f)) return sign | 0x7f;           // NaN, inf, overflow past the last tie
+    if (a < 0.015625f) {                              // below 2^-6: subnormal grid of 2^-9
+        const float r = rintf(a * 512.f);             // rintf = round half to even
+        return sign | (uint8_t)r;                     // r == 8 lands on the first normal, 0x08
+    }
+    uint32_t au = u & 0x7fffffffu;
+    au += 0x7ffffu + ((au >> 20) & 1u);               // RNE to 3 mantissa bits
+    const int e = (int)(au >> 23) - 120;
+    const uint32_t m = (au >> 20) & 7u;
+    return sign | (uint8_t)((e << 3) | m);
+}
+
+template <int kDt>
+__device__ __forceinline__ double load_as_f64(const char* p) {
+    if constexpr (kDt == MOYE_F32) return (double)*reinterpret_cast<const float*>(p);
+    else if constexpr (kDt == MOYE_F16) return (double)(float)*reinterpret_cast<const _Float16*>(p);
+    else if constexpr (kDt == MOYE_BF16) return (double)bf16_to_f32(*reinterpret_cast<const uint16_t*>(p));
+    else if constexpr (kDt == MOYE_F8E4M3) return (double)f8e4m3_to_f32(*reinterpret_cast<const uint8_t*>(p));
+    else return *reinterpret_cast<const double*>(p);
+}
+
+// Every narrower float format here embeds exactly in fp32 and fp32 in fp64, so one rounding
+// step per conversion happens below (f64 -> f16/bf16/f8 goes through f32 only when the source
+// was at most f32, which is then exact).
+template <int kDt>
+__device__ __forceinline__ void store_from(char* p, double v, bool src_is_f64) {
+    if constexpr (kDt == MOYE_F64) *reinterpret_cast<double*>(p) = v;
+    else if constexpr (kDt == MOYE_F32) *reinterpret_cast<float*>(p) = (float)v;
+    else if constexpr (kDt == MOYE_F16)
+        *reinterpret_cast<_Float16*>(p) = src_is_f64 ? (_Float16)v : (_Float16)(float)v;
+    else if constexpr (kDt == MOYE_BF16) *reinterpret_cast<uint16_t*>(p) = f32_to_bf16((float)v);
+    else *reinterpret_cast<uint8_t*>(p) = f32_to_f8e4m3((float)v);
+}
+
+template <int kBytes>
+__global__ __launch_bounds__(256) void copy_generic_bits(const char* __restrict__ src,
+                                                         char* __restrict__ dst, FlatLayout ls,
+                                                         FlatLayout ld, int64_t n) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const char* s = src + layout_offset(ls, i) * kBytes;
+        char* d = dst + layout_offset(ld, i) * kBytes;
+        if constexpr (kBytes == 1) *reinterpret_cast<uint8_t*>(d) = *reinterpret_cast<const uint8_t*>(s);
+        else if constexpr (kBytes == 2) *reinterpret_cast<uint16_t*>(d) = *reinterpret_cast<const uint16_t*>(s);
+        else if constexpr (kBytes == 4) *reinterpret_cast<uint32_t*>(d) = *reinterpret_cast<const uint32_t*>(s);
+        else if constexpr (kBytes == 8) *reinterpret_cast<uint64_t*>(d) = *reinterpret_cast<const uint64_t*>(s);
+        else *reinterpret_cast<u32x4*>(d) = *reinterpret_cast<const u32x4*>(s);
+    }
+}
+
+template <int kSrc, int kDst>
+__global__ __launch_bounds__(256) void copy_generic_cvt(const char* __restrict__ src,
+                                                        char* __restrict__ dst, FlatLayout ls,
+                                                        FlatLayout ld, int64_t n, int sb, int db) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const double v = load_as_f64<kSrc>(src + layout_offset(ls, i) * sb);
+        store_from<kDst>(dst + layout_offset(ld, i) * db, v, kSrc == MOYE_F64);
+    }
+}
+
+static FlatLayout flat_of(const moye_tensor& t) {
+    FlatLayout f;
+    f.rank = t.rank;
+    for (int i = 0; i < MOYE_MAX_RANK; ++i) {
+        f.shape[i] = i < t.rank ? t.shape[i] : 1;
+        f.stride[i] = i < t.rank ? t.stride[i] : 0;
+    }
+    return f;
+}
+
+// Is the layout a dense run 0..size-1 visited in order (compact column-major after dropping
+// size-1 modes)?
+static bool is_contiguous(const moye_tensor& t) {
+    int64_t expect = 1;
+    for (int i = 0; i < t.rank; ++i) {
+        if (t.shape[i] == 1) continue;
+        if (t.stride[i] != expect) return false;
+        expect *= t.shape[i];
+    }
+    return true;
+}
+
+template <int kSrc>
+static bool launch_cvt_dst(int32_t dd, dim3 g, hipStream_t st, const char* s, char* d, FlatLayout ls,
+                           FlatLayout ld, int64_t n, int sb, int db) {
+    switch (dd) {
+        case MOYE_F32: copy_generic_cvt<kSrc, MOYE_F32><<<g, 256, 0, st>>>(s, d, ls, ld, n, sb, db); return true;
+        case MOYE_F16: copy_generic_cvt<kSrc, MOYE_F16><<<g, 256, 0, st>>>(s, d, ls, ld, n, sb, db); return true;
+        case MOYE_BF16: copy_generic_cvt<kSrc, MOYE_BF16><<<g, 256, 0, st>>>(s, d, ls, ld, n, sb, db); return true;
+        case MOYE_F8E4M3: copy_generic_cvt<kSrc, MOYE_F8E4M3><<<g, 256, 0, st>>>(s, d, ls, ld, n, sb, db); return true;
+        case MOYE_F64: copy_generic_cvt<kSrc, MOYE_F64><<<g, 256, 0, st>>>(s, d, ls, ld, n, sb, db); return true;
+        default: return false;
+    }
+}
+
+int32_t copy_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, const moye_tensor* src,
+                      hipStream_t st) {
+    if (int32_t e = check_tensor(dst, "dst")) return e;
+    if (int32_t e = check_tensor(src, "src")) return e;
+    const int64_t n = tensor_size(*src);
+    if (tensor_size(*dst) != n)
+        return fail(MOYE_ERR_SHAPE, "copyto!: dst holds %lld elements, src %lld",
+                    (long long)tensor_size(*dst), (long long)n);
+    const int sb = dtype_bytes(src->dtype), db = dtype_bytes(dst->dtype);
+    if (n == 0) return MOYE_OK;
+    const bool same_bits = (src->dtype == dst->dtype) || (sb == db && !is_float_dtype(src->dtype) && !is_float_dtype(dst->dtype));
+    if (!same_bits && !(is_float_dtype(src->dtype) && is_float_dtype(dst->dtype)))
+        return fail(MOYE_ERR_UNSUPPORTED, "copyto!: no conversion %s -> %s", dtype_name(src->dtype),
+                    dtype_name(dst->dtype));
+    if (tc) {
+        if (tc->op != MOYE_COPY_UNIVERSAL && tc->op != MOYE_COPY_LDS_TILED)
+            return fail(MOYE_ERR_UNSUPPORTED, "copyto!: unknown copy op %d", tc->op);
+        if (tc->vec_bits && (tc->vec_bits % 8 || tc->vec_bits > 128 || (tc->vec_bits & (tc->vec_bits - 1))))
+            return fail(MOYE_ERR_ARG, "copyto!: vec_bits %d is not one of 8..128", tc->vec_bits);
+        if (tc->vec_bits && tc->vec_bits % (8 * sb))
+            return fail(MOYE_ERR_SHAPE, "copyto!: a %d-bit access does not hold whole %s values", tc->vec_bits,
+                        dtype_name(src->dtype));
+    }
+    const char* s = static_cast<const char*>(src->ptr);
+    char* d = static_cast<char*>(dst->ptr);
+
+    if (same_bits) {
+        // (1) both sides one dense run in the same order
+        if (is_contiguous(*src) && is_contiguous(*dst)) {
+            const int64_t bytes = n * sb;
+            if (bytes % 16 == 0 && (reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d)) % 16 == 0) {
+                const int64_t n16 = bytes / 16;
+                const int blocks = (int)std::min<int64_t>((n16 + 255) / 256, 256 * 32);
+                copy_flat_b128<<<blocks, 256, 0, st>>>(reinterpret_cast<const u32x4*>(s), reinterpret_cast<u32x4*>(d), n16);
+            } else {
+                const int blocks = (int)std::min<int64_t>((bytes + 255) / 256, 256 * 32);
+                copy_flat_bytes<<<blocks, 256, 0, st>>>(reinterpret_cast<const uint8_t*>(s), reinterpret_cast<uint8_t*>(d), bytes);
+            }
+            MOYE_HIP_CHECK(hipGetLastError());
+            return MOYE_OK;
+        }
+        // (2) rank-2 transpose of 4-byte elements through the LDS tile
+        const int tm = tc && tc->tiler_mn[0] ? tc->tiler_mn[0] : kTile;
+        const int tn = tc && tc->tiler_mn[1] ? tc->tiler_mn[1] : kTile;
+        if (sb == 4 && src->rank == 2 && dst->rank == 2 && src->shape[0] == dst->shape[0] &&
+            src->shape[1] == dst->shape[1] && tm == kTile && tn == kTile) {
+            const moye_tensor *a = src, *b = dst;
+            bool ok = false, swap = false;
+            if (a->stride[0] == 1 && b->stride[1] == 1) ok = true;
+            else if (a->stride[1] == 1 && b->stride[0] == 1) ok = swap = true;
+            if (ok) {
+                // normalise to: i = contiguous index of src, j = contiguous index of dst
+                const int mi = swap ? 1 : 0, mj = swap ? 0 : 1;
+                const int64_t ni = a->shape[mi], nj = a->shape[mj];
+                const int64_t lds_ = a->stride[mj], ldd = b->stride[mi];
+                const bool aligned = ni % kTile == 0 && nj % kTile == 0 && lds_ % 4 == 0 && ldd % 4 == 0 &&
+                                     lds_ >= ni && ldd >= nj &&
+                                     (reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d)) % 16 == 0;
+                if (aligned) {
+                    const int ti = (int)(ni / kTile), tj = (int)(nj / kTile);
+                    const int64_t tiles = (int64_t)ti * tj;
+                    if (tiles > 0x7fffffff) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles");
+                    const int sbk = 16;
+                    if (tc && (tc->flags & MOYE_GEMM_NO_LDS_SWIZZLE))
+                        transpose_lds_b32<false><<<(unsigned)tiles, 256, 0, st>>>(
+                            reinterpret_cast<const uint32_t*>(s), reinterpret_cast<uint32_t*>(d), lds_, ldd, ti, tj, sbk);
+                    else
+                        transpose_lds_b32<true><<<(unsigned)tiles, 256, 0, st>>>(
+                            reinterpret_cast<const uint32_t*>(s), reinterpret_cast<uint32_t*>(d), lds_, ldd, ti, tj, sbk);
+                    MOYE_HIP_CHECK(hipGetLastError());
+                    return MOYE_OK;
+                }
+            }
+        }
+        if (tc && tc->op == MOYE_COPY_LDS_TILED)
+            return fail(MOYE_ERR_UNSUPPORTED,
+                        "copyto!: the LDS-tiled copy needs rank-2 4-byte operands whose sizes are multiples of "
+                        "64, 16-byte aligned, with the unit stride on different modes");
+    }
+
+    // (3) generic
+    const FlatLayout ls = flat_of(*src), ld = flat_of(*dst);
+    const dim3 g((unsigned)std::min<int64_t>((n + 255) / 256, 256 * 64));
+    bool ok = true;
+    if (same_bits) {
+        switch (sb) {
+            case 1: copy_generic_bits<1><<<g, 256, 0, st>>>(s, d, ls, ld, n); break;
+            case 2: copy_generic_bits<2><<<g, 256, 0, st>>>(s, d, ls, ld, n); break;
+            case 4: copy_generic_bits<4><<<g, 256, 0, st>>>(s, d, ls, ld, n); break;
+            case 8: copy_generic_bits<8><<<g, 256, 0, st>>>(s, d, ls, ld, n); break;
+            case 16: copy_generic_bits<16><<<g, 256, 0, st>>>(s, d, ls, ld, n); break;
+            default: ok = false;
+        }
+    } else {
+        switch (src->dtype) {
+            case MOYE_F32: ok = launch_cvt_dst<MOYE_F32>(dst->dtype, g, st, s, d, ls, ld, n, sb, db); break;
+            case MOYE_F16: ok = launch_cvt_dst<MOYE_F16>(dst->dtype, g, st, s, d, ls, ld, n, sb, db); break;
+            case MOYE_BF16: ok = launch_cvt_dst<MOYE_BF16>(dst->dtype, g, st, s, d, ls, ld, n, sb, db); break;
+            case MOYE_F8E4M3: ok = launch_cvt_dst<MOYE_F8E4M3>(dst->dtype, g, st, s, d, ls, ld, n, sb, db); break;
+            case MOYE_F64: ok = launch_cvt_dst<MOYE_F64>(dst->dtype, g, st, s, d, ls, ld, n, sb, db); break;
+            default: ok = false;
+        }
+    }
+    if (!ok) return fail(MOYE_ERR_UNSUPPORTED, "copyto!: no kernel for %s -> %s", dtype_name(src->dtype), dtype_name(dst->dtype));
+    MOYE_HIP_CHECK(hipGetLastError());
+    return MOYE_OK;
+}
+
+}  // namespace moye

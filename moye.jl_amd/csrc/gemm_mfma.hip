@@ -1,0 +1,321 @@
+// gemm! on the matrix cores: D = alpha * A * B' + C for K-major ("TN") A:(M,K), B:(N,K) in
+// f16 / bf16 / fp8-e4m3 with fp32 accumulation, written for gfx950 (64-lane waves, MFMA).
+//
+// Stands where the reference has its tensor-core user kernel and the loops under it
+// (docs/src/manual/tensor_core.md:265-355 driving src/algorithm/blas.jl:74-131 and
+// src/algorithm/copy.jl:106-130).  The reference's pieces map as follows:
+//   cp.async gmem->smem   (src/arch/copy/copy_async.jl:8-24)  -> 128-bit global loads, staged in
+//                          registers, written to LDS with an XOR swizzle on the 16-byte chunk
+//   ldmatrix smem->reg    (src/arch/copy/ldmatrix.jl:18-48)   -> ds_read_b128 fragment loads that
+//                          land directly in MFMA operand order
+//   mma.sync              (src/arch/mma/make_mma_ops.jl:387-407) -> v_mfma_f32_16x16x32_{f16,bf16},
+//                          v_mfma_f32_16x16x32_fp8_fp8
+//   epilogue copyto!(tCgC, tCrC) (test/device/matmul.jl:51) -> registers -> LDS -> 128-bit stores
+//
+// Wave layout: 2 x 2 waves per workgroup, each wave owns a (BM/2) x (BN/2) block of C made of
+// 16x16 MFMA tiles.  The MFMA is issued with the B-matrix rows as its first operand and the
+// A-matrix rows as its second, so a lane ends up holding four CONSECUTIVE n of one m, which is
+// what a row-major D wants.
+#include "kernels.hpp"
+
+namespace moye {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+
+// ---- input element traits: how one pair of 16-byte chunks feeds the MFMA pipe ----------------
+struct InF16 {
+    static constexpr int kBytes = 2;
+    static __device__ __forceinline__ void mma(const u32x4& a, const u32x4& b, f32x4& c) {
+        c = __builtin_amdgcn_mfma_f32_16x16x32_f16((f16x8)a, (f16x8)b, c, 0, 0, 0);
+    }
+};
+struct InBF16 {
+    static constexpr int kBytes = 2;
+    static __device__ __forceinline__ void mma(const u32x4& a, const u32x4& b, f32x4& c) {
+        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16((bf16x8)a, (bf16x8)b, c, 0, 0, 0);
+    }
+};
+// A 16-byte chunk holds 16 fp8 values = the k-slices of two MFMAs.  Both operands split the
+// chunk the same way, so the pairing of products is unchanged.
+struct InFP8 {
+    static constexpr int kBytes = 1;
+    static __device__ __forceinline__ void mma(const u32x4& a, const u32x4& b, f32x4& c) {
+        const long a0 = (long)(((uint64_t)a.y << 32) | a.x), a1 = (long)(((uint64_t)a.w << 32) | a.z);
+        const long b0 = (long)(((uint64_t)b.y << 32) | b.x), b1 = (long)(((uint64_t)b.w << 32) | b.z);
+        c = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a0, b0, c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a1, b1, c, 0, 0, 0);
+    }
+};
+
+// ---- output element traits: fp32 -> OutT, round to nearest even (src/arch/copy/copy.jl:38-43) ---
+struct OutF32 {
+    typedef float type;
+    static __device__ __forceinline__ float cvt(float x) { return x; }
+    static __device__ __forceinline__ float load(const void* p, int64_t i) { return static_cast<const float*>(p)[i]; }
+};
+struct OutF16 {
+    typedef _Float16 type;
+    static __device__ __forceinline__ _Float16 cvt(float x) { return (_Float16)x; }
+    static __device__ __forceinline__ float load(const void* p, int64_t i) { return (float)static_cast<const _Float16*>(p)[i]; }
+};
+struct OutBF16 {
+    typedef uint16_t type;
+    static __device__ __forceinline__ uint16_t cvt(float x) {
+        uint32_t u = __float_as_uint(x);
+        if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+        u += 0x7fffu + ((u >> 16) & 1u);
+        return (uint16_t)(u >> 16);
+    }
+    static __device__ __forceinline__ float load(const void* p, int64_t i) {
+        return __uint_as_float((uint32_t)static_cast<const uint16_t*>(p)[i] << 16);
+    }
+};
+
+// XOR swizzle of the 16-byte chunk index inside an LDS tile row of CPR chunks: rows that are
+// 256 bytes apart in LDS (one full sweep of the 64 banks) get different chunk permutations, so
+// 16 lanes reading the same logical chunk of 16 consecutive rows hit 16 different bank groups.
+template <int CPR>
+__device__ __forceinline__ int swz(int row) {
+    if constexpr (CPR >= 16) return row & 15;
+    else return (row / (16 / CPR)) & (CPR - 1);
+}
+
+// blockIdx -> (tile_m, tile_n).  Hardware deals consecutive workgroup ids round-robin to the 8
+// XCDs; remapping id -> (id % 8) * (n / 8) + id / 8 hands each XCD one contiguous run of tiles,
+// and inside a run tiles are walked in bands of 8 tile-rows so that the A and B panels an
+// XCD's L2 holds are reused by the workgroups that follow.
+__device__ __forceinline__ void tile_of_block(const GemmArgs& p, int* tm, int* tn) {
+    int bid = blockIdx.x;
+    const int n = gridDim.x;
+    if (p.xcd_swizzle && (n % 8) == 0) bid = (bid % 8) * (n / 8) + bid / 8;
+    constexpr int kGroup = 8;
+    const int per_group = kGroup * p.tiles_n;
+    const int g = bid / per_group;
+    const int first_m = g * kGroup;
+    const int gsize = min(p.tiles_m - first_m, kGroup);
+    const int r = bid - g * per_group;
+    *tm = first_m + r % gsize;
+    *tn = r / gsize;
+}
+
+template <typename In, typename Out, int BM, int BN, int BKB /* bytes of K per tile row */>
+__global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
+    constexpr int CPR = BKB / 16;                 // 16-byte chunks per tile row
+    constexpr int KSTEPS = CPR / 4;               // one step = 4 chunks = one (fp8: two) MFMA k-slice
+    constexpr int A_CH = BM * CPR, B_CH = BN * CPR;
+    constexpr int A_LD = A_CH / 256, B_LD = B_CH / 256;
+    constexpr int WM = BM / 2, WN = BN / 2, MI = WM / 16, NI = WN / 16;
+    static_assert(A_CH % 256 == 0 && B_CH % 256 == 0 && CPR % 4 == 0, "tile shape");
+    typedef typename Out::type OutT;
+
+    extern __shared__ u32x4 smem[];
+    u32x4* const sA0 = smem;
+    u32x4* const sB0 = smem + A_CH;
+    constexpr int STAGE = A_CH + B_CH;
+
+    int tm, tn;
+    tile_of_block(p, &tm, &tn);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
+    const int r16 = lane & 15, kq = lane >> 4;
+
+    const int64_t kbytes_a = (int64_t)p.lda * In::kBytes, kbytes_b = (int64_t)p.ldb * In::kBytes;
+    const char* gA = static_cast<const char*>(p.A) + (int64_t)tm * BM * kbytes_a;
+    const char* gB = static_cast<const char*>(p.B) + (int64_t)tn * BN * kbytes_b;
+
+    // per-thread global chunk addresses and LDS slots (fixed for the whole k loop)
+    const char* a_src[A_LD];
+    const char* b_src[B_LD];
+    int a_dst[A_LD], b_dst[B_LD];
+#pragma unroll
+    for (int i = 0; i < A_LD; ++i) {
+        const int c = tid + 256 * i, row = c / CPR, ch = c % CPR;
+        a_src[i] = gA + row * kbytes_a + ch * 16;
+        a_dst[i] = row * CPR + (ch ^ swz<CPR>(row));
+    }
+#pragma unroll
+    for (int i = 0; i < B_LD; ++i) {
+        const int c = tid + 256 * i, row = c / CPR, ch = c % CPR;
+        b_src[i] = gB + row * kbytes_b + ch * 16;
+        b_dst[i] = row * CPR + (ch ^ swz<CPR>(row));
+    }
+
+    f32x4 acc[MI][NI];
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int ktiles = (int)(((int64_t)p.K * In::kBytes) / BKB);
+    u32x4 ra[A_LD], rb[B_LD];
+
+    // prologue: tile 0 -> LDS stage 0
+#pragma unroll
+    for (int i = 0; i < A_LD; ++i) ra[i] = *reinterpret_cast<const u32x4*>(a_src[i]);
+#pragma unroll
+    for (int i = 0; i < B_LD; ++i) rb[i] = *reinterpret_cast<const u32x4*>(b_src[i]);
+#pragma unroll
+    for (int i = 0; i < A_LD; ++i) sA0[a_dst[i]] = ra[i];
+#pragma unroll
+    for (int i = 0; i < B_LD; ++i) sB0[b_dst[i]] = rb[i];
+    __syncthreads();
+
+    for (int kt = 0; kt < ktiles; ++kt) {
+        const u32x4* sA = sA0 + (kt & 1) * STAGE;
+        const u32x4* sB = sB0 + (kt & 1) * STAGE;
+        const bool more = kt + 1 < ktiles;
+        if (more) {  // next tile: global -> registers, in flight during the MFMAs below
+            const int64_t koff = (int64_t)(kt + 1) * BKB;
+#pragma unroll
+            for (int i = 0; i < A_LD; ++i) ra[i] = *reinterpret_cast<const u32x4*>(a_src[i] + koff);
+#pragma unroll
+            for (int i = 0; i < B_LD; ++i) rb[i] = *reinterpret_cast<const u32x4*>(b_src[i] + koff);
+        }
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+            u32x4 fa[MI], fb[NI];
+            const int ch = ks * 4 + kq;
+#pragma unroll
+            for (int i = 0; i < MI; ++i) {
+                const int row = wm0 + 16 * i + r16;
+                fa[i] = sA[row * CPR + (ch ^ swz<CPR>(row))];
+            }
+#pragma unroll
+            for (int j = 0; j < NI; ++j) {
+                const int row = wn0 + 16 * j + r16;
+                fb[j] = sB[row * CPR + (ch ^ swz<CPR>(row))];
+            }
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+#pragma unroll
+                for (int j = 0; j < NI; ++j) In::mma(fb[j], fa[i], acc[i][j]);
+        }
+        if (more) {  // registers -> the other LDS stage
+            u32x4* dA = sA0 + ((kt + 1) & 1) * STAGE;
+            u32x4* dB = sB0 + ((kt + 1) & 1) * STAGE;
+#pragma unroll
+            for (int i = 0; i < A_LD; ++i) dA[a_dst[i]] = ra[i];
+#pragma unroll
+            for (int i = 0; i < B_LD; ++i) dB[b_dst[i]] = rb[i];
+        }
+        __syncthreads();
+    }
+
+    // ---- epilogue: alpha*acc + C -> OutT -> this wave's LDS patch -> 128-bit row stores ----
+    // lane holds C[m = 16 i + r16][n = 16 j + 4 kq + e], e = 0..3
+    const int64_t m_base = (int64_t)tm * BM + wm0, n_base = (int64_t)tn * BN + wn0;
+    constexpr int EPC = 16 / (int)sizeof(OutT);          // elements per 16-byte chunk
+    constexpr int CR = WN / EPC;                         // chunks per patch row
+    constexpr int PASS_MI = (sizeof(OutT) == 4 && MI > 1) ? MI / 2 : MI;  // keep the patch <= 8 KiB
+    constexpr int PASS_ROWS = PASS_MI * 16;
+    OutT* patch = reinterpret_cast<OutT*>(smem) + wave * (PASS_ROWS * WN);
+    u32x4* patch16 = reinterpret_cast<u32x4*>(patch);
+
+#pragma unroll
+    for (int i0 = 0; i0 < MI; i0 += PASS_MI) {
+#pragma unroll
+        for (int ii = 0; ii < PASS_MI; ++ii) {
+            const int i = i0 + ii;
+#pragma unroll
+            for (int j = 0; j < NI; ++j) {
+                float v[4] = {acc[i][j].x * p.alpha, acc[i][j].y * p.alpha, acc[i][j].z * p.alpha,
+                              acc[i][j].w * p.alpha};
+                if (p.C) {
+                    const int64_t m = m_base + 16 * i + r16, n = n_base + 16 * j + 4 * kq;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] += Out::load(p.C, m * p.ldc_m + (n + e) * p.ldc_n);
+                }
+                const int row = 16 * ii + r16, col = 16 * j + 4 * kq;
+                const int chunk = col / EPC, within = col % EPC;
+                OutT* dst = patch + (row * CR + (chunk ^ (row & (CR - 1)))) * EPC + within;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) dst[e] = Out::cvt(v[e]);
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int t = 0; t < PASS_ROWS * CR / 64; ++t) {
+            const int c = lane + 64 * t, row = c / CR, ch = c % CR;
+            const u32x4 w = patch16[row * CR + (ch ^ (row & (CR - 1)))];
+            char* d = static_cast<char*>(p.D) +
+                      ((m_base + 16 * i0 + row) * p.ldd + n_base) * (int64_t)sizeof(OutT) + ch * 16;
+            *reinterpret_cast<u32x4*>(d) = w;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+}
+
+template <typename In, typename Out, int BM, int BN, int BKB>
+static int32_t launch(const GemmArgs& a, hipStream_t st) {
+    typedef typename Out::type OutT;
+    constexpr int kMain = 2 * (BM + BN) * BKB;
+    constexpr int kEpi = (sizeof(OutT) == 4 && BM / 32 > 1 ? BM / 2 : BM) * BN * (int)sizeof(OutT);
+    constexpr int kLds = kMain > kEpi ? kMain : kEpi;
+    auto kern = gemm_mfma_tn<In, Out, BM, BN, BKB>;
+    if (kLds > 64 * 1024) {
+        static bool once = false;  // raising the dynamic LDS cap is per function, idempotent
+        if (!once) {
+            MOYE_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
+            once = true;
+        }
+    }
+    kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n)), dim3(256), kLds, st>>>(a);
+    MOYE_HIP_CHECK(hipGetLastError());
+    return MOYE_OK;
+}
+
+template <typename In, int BM, int BN, int BKB>
+static int32_t launch_out(int32_t out_dt, const GemmArgs& a, hipStream_t st) {
+    switch (out_dt) {
+        case MOYE_F32: return launch<In, OutF32, BM, BN, BKB>(a, st);
+        case MOYE_F16: return launch<In, OutF16, BM, BN, BKB>(a, st);
+        case MOYE_BF16: return launch<In, OutBF16, BM, BN, BKB>(a, st);
+        default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: MFMA kernels write f32, f16 or bf16, not %s", dtype_name(out_dt));
+    }
+}
+
+// K-major A and B, N-contiguous D.  bk_elems = 0 picks the default K extent per tile.
+int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int bk_elems,
+                              GemmArgs a, hipStream_t st) {
+    const int eb = dtype_bytes(in_dt);
+    if (bm == 0) bm = 128;
+    if (bn == 0) bn = 128;
+    if (bk_elems == 0) bk_elems = 64 / eb;  // 64 bytes of K per row: 32 halves / 64 fp8
+    const int bkb = bk_elems * eb;
+    if (bm != 128 || bn != 128 || (bkb != 64 && bkb != 128))
+        return fail(MOYE_ERR_UNSUPPORTED,
+                    "gemm!: no MFMA kernel for CTA tile %dx%dx%d (%s); built: 128x128x{%d,%d}", bm, bn, bk_elems,
+                    dtype_name(in_dt), 64 / eb, 128 / eb);
+    if (a.M % bm || a.N % bn || a.K % bk_elems)
+        return fail(MOYE_ERR_SHAPE, "gemm!: CTA tile %dx%dx%d does not divide the problem %dx%dx%d", bm, bn,
+                    bk_elems, a.M, a.N, a.K);
+    const int ob = dtype_bytes(out_dt);
+    if ((a.lda * eb) % 16 || (a.ldb * eb) % 16 || (a.ldd * ob) % 16 ||
+        (reinterpret_cast<uintptr_t>(a.A) | reinterpret_cast<uintptr_t>(a.B) | reinterpret_cast<uintptr_t>(a.D)) % 16)
+        return fail(MOYE_ERR_ALIGN, "gemm!: operands of the MFMA kernels need 16-byte aligned pointers and row pitches");
+    a.tiles_m = a.M / bm;
+    a.tiles_n = a.N / bn;
+    const bool wide = bkb == 128;
+    switch (in_dt) {
+        case MOYE_F16:
+            return wide ? launch_out<InF16, 128, 128, 128>(out_dt, a, st) : launch_out<InF16, 128, 128, 64>(out_dt, a, st);
+        case MOYE_BF16:
+            return wide ? launch_out<InBF16, 128, 128, 128>(out_dt, a, st) : launch_out<InBF16, 128, 128, 64>(out_dt, a, st);
+        case MOYE_F8E4M3:
+            return wide ? launch_out<InFP8, 128, 128, 128>(out_dt, a, st) : launch_out<InFP8, 128, 128, 64>(out_dt, a, st);
+        default:
+            return fail(MOYE_ERR_UNSUPPORTED, "gemm!: no MFMA atom for %s inputs", dtype_name(in_dt));
+    }
+}
+
+}  // namespace moye

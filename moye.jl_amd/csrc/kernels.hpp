@@ -1,0 +1,34 @@
+// Argument blocks and dispatch entry points shared by the kernel translation units and capi.hip.
+#pragma once
+
+#include "moye_common.hpp"
+
+namespace moye {
+
+// MFMA GEMM, K-major operands, N-contiguous output (gemm_mfma.hip)
+struct GemmArgs {
+    const void* A;  // (M,K), K contiguous, row pitch lda elements
+    const void* B;  // (N,K), K contiguous, row pitch ldb
+    const void* C;  // (M,N) or null, element strides ldc_m / ldc_n, dtype of D
+    void* D;        // (M,N), N contiguous, row pitch ldd
+    int M, N, K;
+    int64_t lda, ldb, ldc_m, ldc_n, ldd;
+    float alpha;
+    int tiles_m, tiles_n;
+    int xcd_swizzle;
+};
+
+// UniversalFMA GEMM, any strides (gemm_universal.hip)
+struct UArgs {
+    const void* A; const void* B; const void* C; void* D;
+    int M, N, K;
+    int64_t sa_m, sa_k, sb_n, sb_k, sc_m, sc_n, sd_m, sd_n;
+    float alpha;
+    int a_dt, b_dt, c_dt, d_dt;
+};
+
+int32_t copy_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, const moye_tensor* src, hipStream_t st);
+int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int bk_elems, GemmArgs a, hipStream_t st);
+int32_t gemm_universal_dispatch(int bm, int bn, int bk, UArgs a, hipStream_t st);
+
+}  // namespace moye

@@ -1,0 +1,17 @@
+"""moye_hip — host-side mirror of MoYe.jl's API over libmoye_hip.so (gfx950 / MI355X).
+
+`copyto_` and `gemm_` are `Base.copyto!` (src/algorithm/copy.jl:42-46,106-110 of the
+reference) and `gemm!` (src/algorithm/blas.jl:11-17) for device arrays; they flatten the
+arrays' layouts into plain descriptors and hand them to the HIP library.  There is no other
+code path: without the built library every call raises.
+"""
+from . import _lib
+from ._lib import (BF16, COPY_LDS_TILED, COPY_UNIVERSAL, F8E4M3, F16, F32, F64, GEMM_NO_LDS_SWIZZLE,
+                   GEMM_NO_XCD_SWIZZLE, MFMA_F32_16x16x4_F32, MFMA_F32_16x16x32_BF16, MFMA_F32_16x16x32_F16,
+                   MFMA_F32_16x16x32_FP8, MFMA_F32_32x32x2_F32, MFMA_F32_32x32x16_BF16,
+                   MFMA_F32_32x32x16_F16, MFMA_F32_32x32x16_FP8, MMA_UNIVERSAL_FMA, U8, U16, U32, U64, U128,
+                   MoyeError, Tensor, TiledCopy, TiledMMA, check, lib, make_tensor)
+from .device import (copyto_, device_info, gemm_, tiled_copy_desc, tiled_mma_desc, time_copy, time_gemm,
+                     version)
+
+__all__ = [n for n in dir() if not n.startswith("_")]

@@ -1,0 +1,70 @@
+"""Device loops behind the C ABI: copyto! and gemm! on flattened descriptors."""
+import ctypes as C
+
+from . import _lib
+from ._lib import TiledCopy, TiledMMA, check, lib
+
+
+def version():
+    return lib().moye_version().decode()
+
+
+def device_info():
+    name = C.create_string_buffer(256)
+    cu, khz, mem = C.c_int32(), C.c_int32(), C.c_size_t()
+    check(lib().moye_device_info(name, 256, C.byref(cu), C.byref(khz), C.byref(mem)))
+    return {"name": name.value.decode(), "compute_units": cu.value, "clock_khz": khz.value,
+            "total_mem": mem.value}
+
+
+def tiled_mma_desc(atom, atom_layout=(1, 1, 1), tile=(0, 0, 0), cta_tile=(0, 0, 0), stages=0, split_k=0,
+                   flags=0):
+    """A moye_tiled_mma: what `make_tiled_mma(op, atom_layout, permutations)` (src/atom/mma.jl:193-233)
+    plus the kernel's shared-memory tile (bM, bN, bK) boil down to."""
+    d = TiledMMA()
+    d.atom = atom
+    for i in range(3):
+        d.atom_layout_mnk[i] = atom_layout[i] if i < len(atom_layout) else 1
+        d.tile_mnk[i] = tile[i]
+        d.cta_tile_mnk[i] = cta_tile[i]
+    d.stages, d.split_k, d.flags = stages, split_k, flags
+    return d
+
+
+def tiled_copy_desc(op=_lib.COPY_UNIVERSAL, vec_bits=0, thr_shape=(0, 0), val_shape=(0, 0), tiler=(0, 0),
+                    flags=0):
+    """A moye_tiled_copy: `make_tiled_copy(atom, thr_layout, val_layout)` (src/atom/copy.jl:249-258)."""
+    d = TiledCopy()
+    d.op, d.vec_bits, d.flags = op, vec_bits, flags
+    for i in range(2):
+        d.thr_shape[i], d.val_shape[i], d.tiler_mn[i] = thr_shape[i], val_shape[i], tiler[i]
+    return d
+
+
+def _ref(x):
+    return C.byref(x) if x is not None else None
+
+
+def copyto_(dst, src, tiled_copy=None, stream=None):
+    """copyto!(dst, src) / copyto!(tiled_copy, dst, src) on moye_tensor descriptors; returns dst."""
+    check(lib().moye_copy(_ref(tiled_copy), C.byref(dst), C.byref(src), stream))
+    return dst
+
+
+def gemm_(mma, D, A, B, C_=None, alpha=1.0, stream=None):
+    """gemm!(mma, D, A, B, C): D = alpha * A * B' + C with A:(M,K), B:(N,K), C,D:(M,N)."""
+    check(lib().moye_gemm(C.byref(mma), C.byref(D), C.byref(A), C.byref(B), _ref(C_), alpha, stream))
+
+
+def time_gemm(mma, D, A, B, C_=None, alpha=1.0, stream=None, warmup=2, iters=10):
+    """Average milliseconds per launch (HIP events on `stream`)."""
+    ms = C.c_float()
+    check(lib().moye_time_gemm(C.byref(mma), C.byref(D), C.byref(A), C.byref(B), _ref(C_), alpha, stream,
+                               warmup, iters, C.byref(ms)))
+    return ms.value
+
+
+def time_copy(dst, src, tiled_copy=None, stream=None, warmup=2, iters=10):
+    ms = C.c_float()
+    check(lib().moye_time_copy(_ref(tiled_copy), C.byref(dst), C.byref(src), stream, warmup, iters, C.byref(ms)))
+    return ms.value

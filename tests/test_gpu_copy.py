@@ -1,0 +1,205 @@
+"""GPU parity of copyto! through the C ABI (moye_copy) against the CPU oracle and against the
+closed form the reference's own device tests use (`a == transpose(b)`,
+test/host/copy_async.jl:43,95).  Bit-exact: everything is compared as integers."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+import layout_oracle as lo  # noqa: E402
+import tiled_oracle as to  # noqa: E402
+
+
+@pytest.fixture(scope="module")
+def mh():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    import moye_hip
+    from moye_hip import torch_interop  # noqa: F401
+    return moye_hip
+
+
+def _tens(mh, t, shape, stride):
+    from moye_hip.torch_interop import tensor_of
+    return tensor_of(t, shape, stride)
+
+
+def _flat(l):
+    f = lo.lflatten(l)
+    s, d = f.shape, f.stride
+    if not isinstance(s, tuple):
+        s, d = (s,), (d,)
+    return [int(x) for x in s], [int(x) for x in d]
+
+
+def _rand_bits(n, seed, device="cuda"):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    return torch.randint(-2 ** 31, 2 ** 31 - 1, (n,), dtype=torch.int32, generator=g).to(device)
+
+
+@pytest.mark.parametrize("M,N", [(64, 64), (128, 256), (192, 64), (1024, 2048)])
+def test_transpose_matches_oracle_and_closed_form(mh, M, N):
+    """config-2 shape family: column-major src -> row-major dst through the 64x64 LDS tile."""
+    src = _rand_bits(M * N, 1002)
+    dst = torch.zeros(M * N, dtype=torch.int32, device="cuda")
+    tc = mh.tiled_copy_desc(op=mh.COPY_LDS_TILED, vec_bits=128, tiler=(64, 64))
+    mh.copyto_(_tens(mh, dst, (M, N), (N, 1)), _tens(mh, src, (M, N), (1, M)), tc)
+    torch.cuda.synchronize()
+    assert torch.equal(dst.view(M, N), src.view(N, M).t())
+    if M * N <= 128 * 256:  # the oracle walks both layouts element by element
+        s = to.Array(src.cpu().numpy(), lo.make_layout((M, N), (1, M)))
+        d = to.Array(np.zeros(M * N, np.int32), lo.make_layout((M, N), (N, 1)))
+        to.copyto(d, s)
+        assert np.array_equal(d.buf, dst.cpu().numpy())
+
+
+def test_transpose_other_orientation_and_pitch(mh):
+    """row-major src -> column-major dst, with padded leading dimensions on both sides."""
+    M, N, lds, ldd = 128, 192, 200, 136
+    src = _rand_bits(M * lds, 7)
+    dst = torch.full((N * ldd,), -1, dtype=torch.int32, device="cuda")
+    mh.copyto_(_tens(mh, dst, (M, N), (1, ldd)), _tens(mh, src, (M, N), (lds, 1)))
+    torch.cuda.synchronize()
+    assert torch.equal(dst.view(N, ldd)[:, :M], src.view(M, lds)[:, :N].t())
+    assert bool((dst.view(N, ldd)[:, M:] == -1).all())  # padding untouched
+
+
+def test_transpose_without_swizzle_is_identical(mh):
+    M = N = 256
+    src = _rand_bits(M * N, 11)
+    a = torch.zeros_like(src)
+    b = torch.zeros_like(src)
+    mh.copyto_(_tens(mh, a, (M, N), (N, 1)), _tens(mh, src, (M, N), (1, M)))
+    tc = mh.tiled_copy_desc(op=mh.COPY_LDS_TILED, tiler=(64, 64), flags=mh.GEMM_NO_LDS_SWIZZLE)
+    mh.copyto_(_tens(mh, b, (M, N), (N, 1)), _tens(mh, src, (M, N), (1, M)), tc)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+
+
+def test_transpose_full_size_involution(mh):
+    """BASELINE config 2 at full size (16384^2 fp32 bits, 1 GiB each side): closed form on sampled
+    tiles, an order-independent checksum, and transpose(transpose(x)) == x."""
+    M = N = 16384
+    src = _rand_bits(M * N, 1002)
+    dst = torch.empty_like(src)
+    tc = mh.tiled_copy_desc(op=mh.COPY_LDS_TILED, vec_bits=128, tiler=(64, 64))
+    mh.copyto_(_tens(mh, dst, (M, N), (N, 1)), _tens(mh, src, (M, N), (1, M)), tc)
+    torch.cuda.synchronize()
+    assert int(dst.sum(dtype=torch.int64)) == int(src.sum(dtype=torch.int64))
+    rng = np.random.default_rng(0)
+    for _ in range(64):
+        i, j = int(rng.integers(0, M - 64)), int(rng.integers(0, N - 64))
+        assert torch.equal(dst.view(M, N)[i:i + 64, j:j + 64], src.view(N, M)[j:j + 64, i:i + 64].t())
+    back = torch.empty_like(src)
+    # dst viewed as the column-major matrix of the transposed problem
+    mh.copyto_(_tens(mh, back, (N, M), (M, 1)), _tens(mh, dst, (N, M), (1, N)), tc)
+    torch.cuda.synchronize()
+    assert torch.equal(back, src)
+
+
+CASES = [
+    # (dst layout, src layout) — hierarchical, strided, broadcast-free
+    ("(4,6):(6,1)", "(4,6):(1,4)"),
+    ("((2,3),(2,4)):((1,16),(2,4))", "(6,8):(1,6)"),
+    ("(32,(2,4)):(2,(1,64))", "(32,8):(1,32)"),
+    ("(3,5,7):(35,7,1)", "(3,5,7):(1,3,15)"),
+    ("(8,9):(1,10)", "(8,9):(11,1)"),
+    ("105:1", "(3,5,7):(1,3,15)"),
+]
+
+
+@pytest.mark.parametrize("dl,sl", CASES)
+@pytest.mark.parametrize("dtype", ["int8", "int16", "int32", "int64"])
+def test_generic_copy_matches_oracle(mh, dl, sl, dtype):
+    """Arbitrary layouts go through the gather/scatter kernel; the oracle is the element loop of
+    src/algorithm/copy.jl:4-12."""
+    ld, ls = lo.parse_layout(dl), lo.parse_layout(sl)
+    ns, nd = int(lo.cosize(ls)), int(lo.cosize(ld))
+    tdt = getattr(torch, dtype)
+    info = torch.iinfo(tdt)
+    g = torch.Generator().manual_seed(3)
+    src = torch.randint(max(info.min, -2 ** 62), min(info.max, 2 ** 62), (ns,), dtype=tdt, generator=g)
+    dst0 = torch.full((nd,), 5, dtype=tdt)
+    s_sh, s_st = _flat(ls)
+    d_sh, d_st = _flat(ld)
+    src_d, dst_d = src.cuda(), dst0.cuda()
+    mh.copyto_(_tens(mh, dst_d, d_sh, d_st), _tens(mh, src_d, s_sh, s_st))
+    torch.cuda.synchronize()
+    o_dst = to.Array(dst0.numpy().copy(), ld)
+    to.copyto(o_dst, to.Array(src.numpy(), ls))
+    assert np.array_equal(o_dst.buf, dst_d.cpu().numpy())
+
+
+def test_contiguous_copy_and_odd_sizes(mh):
+    for n in (1, 7, 4096, 1000003):
+        src = _rand_bits(n, n)
+        dst = torch.zeros_like(src)
+        mh.copyto_(_tens(mh, dst, (n,), (1,)), _tens(mh, src, (n,), (1,)))
+        torch.cuda.synchronize()
+        assert torch.equal(dst, src)
+    # same dense order expressed with two modes
+    src = _rand_bits(96 * 40, 5)
+    dst = torch.zeros_like(src)
+    mh.copyto_(_tens(mh, dst, (96, 40), (1, 96)), _tens(mh, src, (96 * 40,), (1,)))
+    torch.cuda.synchronize()
+    assert torch.equal(dst, src)
+
+
+def test_converting_copy_rounds_to_nearest_even(mh):
+    """UniversalCopy{TS,TD} converts with Julia's `convert` (src/arch/copy/copy.jl:38-43)."""
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(5000, generator=g) * 3
+    x[:6] = torch.tensor([1.0 + 2.0 ** -11, 1.0 + 3 * 2.0 ** -11, 65520.0, -65519.0, 2.0 ** -25, 0.0])
+    xd = x.cuda()
+    h = torch.zeros(5000, dtype=torch.float16, device="cuda")
+    b = torch.zeros(5000, dtype=torch.bfloat16, device="cuda")
+    mh.copyto_(_tens(mh, h, (5000,), (1,)), _tens(mh, xd, (5000,), (1,)))
+    mh.copyto_(_tens(mh, b, (50, 100), (100, 1)), _tens(mh, xd, (50, 100), (1, 50)))
+    torch.cuda.synchronize()
+    want_h = x.numpy().astype(np.float16)
+    assert np.array_equal(h.cpu().numpy().view(np.uint16), want_h.view(np.uint16))
+    want_b = to.round_bf16(x.numpy().reshape(100, 50).T.copy()).reshape(-1)
+    got_b = b.cpu().float().numpy().reshape(-1)
+    assert np.array_equal(got_b.view(np.uint32), want_b.view(np.uint32))
+    # and back up, exactly
+    up = torch.zeros(5000, dtype=torch.float32, device="cuda")
+    mh.copyto_(_tens(mh, up, (5000,), (1,)), _tens(mh, h, (5000,), (1,)))
+    torch.cuda.synchronize()
+    assert np.array_equal(up.cpu().numpy(), want_h.astype(np.float32))
+
+
+def test_fp8_conversion_matches_torch(mh):
+    if not hasattr(torch, "float8_e4m3fn"):
+        pytest.skip("torch without float8_e4m3fn")
+    g = torch.Generator().manual_seed(4)
+    x = torch.cat([torch.randn(4000, generator=g) * 40, torch.linspace(-464, 464, 4001),
+                   torch.tensor([2.0 ** -9, 2.0 ** -10, 3 * 2.0 ** -10, 0.0156, 448.0, 0.0])])
+    n = x.numel()
+    xd = x.cuda()
+    q = torch.zeros(n, dtype=torch.float8_e4m3fn, device="cuda")
+    mh.copyto_(_tens(mh, q, (n,), (1,)), _tens(mh, xd, (n,), (1,)))
+    torch.cuda.synchronize()
+    want = x.to(torch.float8_e4m3fn)
+    assert torch.equal(q.cpu().view(torch.uint8), want.view(torch.uint8))
+    back = torch.zeros(n, dtype=torch.float32, device="cuda")
+    mh.copyto_(_tens(mh, back, (n,), (1,)), _tens(mh, q, (n,), (1,)))
+    torch.cuda.synchronize()
+    assert torch.equal(back.cpu(), want.float())
+
+
+def test_copy_errors(mh):
+    a = torch.zeros(64, dtype=torch.int32, device="cuda")
+    with pytest.raises(mh.MoyeError) as e:
+        mh.copyto_(_tens(mh, a, (8, 8), (1, 8)), _tens(mh, a, (8, 4), (1, 8)))
+    assert e.value.status == mh._lib.ERR_SHAPE
+    with pytest.raises(mh.MoyeError) as e:
+        mh.copyto_(_tens(mh, a, (8, 8), (1, 8)), _tens(mh, a.float(), (8, 8), (1, 8)))
+    assert e.value.status == mh._lib.ERR_UNSUPPORTED
+    tc = mh.tiled_copy_desc(op=mh.COPY_LDS_TILED, tiler=(64, 64))
+    with pytest.raises(mh.MoyeError) as e:  # 8x8 is not a multiple of the 64x64 LDS tile
+        mh.copyto_(_tens(mh, a, (8, 8), (8, 1)), _tens(mh, a, (8, 8), (1, 8)), tc)
+    assert e.value.status == mh._lib.ERR_UNSUPPORTED
+    empty = torch.zeros(0, dtype=torch.int32, device="cuda")
+    mh.copyto_(_tens(mh, empty, (0,), (1,)), _tens(mh, empty, (0,), (1,)))

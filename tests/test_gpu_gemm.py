@@ -1,0 +1,248 @@
+"""GPU parity of gemm! through the C ABI (moye_gemm).
+
+UniversalFMA atom: bit-exact against the CPU restatement of the reference's arithmetic
+(oracle/tiled_oracle.py::gemm_universal_fma) — the tolerance is zero.
+MFMA atoms: norm-wise relative error  max|C - C64| / max|C64|  against an fp64 product of the
+same rounded inputs, tolerance 1e-2 for f16/bf16/fp8 inputs and 1e-5 for fp32, with the error of
+the reference's own arithmetic printed alongside."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+import tiled_oracle as to  # noqa: E402
+
+TOL16 = 1e-2
+TOL32 = 1e-5
+
+
+@pytest.fixture(scope="module")
+def mh():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    import moye_hip
+    return moye_hip
+
+
+def T(t, shape=None, stride=None):
+    from moye_hip.torch_interop import tensor_of
+    return tensor_of(t, shape, stride)
+
+
+def relerr(c, c64):
+    c64 = c64.double()
+    return float((c.double() - c64).abs().max() / c64.abs().max())
+
+
+# ---------------------------------------------------------------------------------------------
+# UniversalFMA: exact
+# ---------------------------------------------------------------------------------------------
+
+def test_config1_fp32_256_nn_bit_exact(mh):
+    """BASELINE config 1: fp32 C = A*B, M=N=K=256, A and B column-major, 32x32x8 tiles."""
+    rng = np.random.default_rng(1001)
+    M = N = K = 256
+    A = (rng.random((M, K), dtype=np.float32) * 2 - 1)           # A[m,k]
+    Bkn = (rng.random((K, N), dtype=np.float32) * 2 - 1)         # B[k,n]
+    a = torch.from_numpy(np.asfortranarray(A).reshape(-1, order="F").copy()).cuda()    # column-major storage
+    b = torch.from_numpy(np.asfortranarray(Bkn).reshape(-1, order="F").copy()).cuda()
+    c = torch.zeros(M * N, dtype=torch.float32, device="cuda")
+    mma = mh.tiled_mma_desc(mh.MMA_UNIVERSAL_FMA, cta_tile=(32, 32, 8))
+    # MoYe operands: A (M,K):(1,M); B as (N,K):(K,1); C (M,N):(1,M)
+    mh.gemm_(mma, T(c, (M, N), (1, M)), T(a, (M, K), (1, M)), T(b, (N, K), (K, 1)), T(c, (M, N), (1, M)))
+    torch.cuda.synchronize()
+    got = c.cpu().numpy().reshape(N, M).T
+    want = to.gemm_universal_fma(A, Bkn.T.copy(), np.zeros((M, N), np.float32))
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    c64 = A.astype(np.float64) @ Bkn.astype(np.float64)
+    err = to.relerr(got, c64)
+    print("config1 fp32 256^3: rel err vs fp64 = %.3e (reference arithmetic: identical)" % err)
+    assert err <= TOL32
+    # every built tiling gives the same bits
+    for tile in ((64, 64, 8), (128, 128, 8)):
+        c2 = torch.zeros_like(c)
+        mh.gemm_(mh.tiled_mma_desc(mh.MMA_UNIVERSAL_FMA, cta_tile=tile), T(c2, (M, N), (1, M)),
+                 T(a, (M, K), (1, M)), T(b, (N, K), (K, 1)))
+        torch.cuda.synchronize()
+        assert torch.equal(c2, c)
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
+def test_universal_fma_ragged_bit_exact(mh, dt):
+    """Odd sizes, K-major operands, C accumulated: product rounded in the input type (f16/bf16),
+    unfused fp32 add, k ascending."""
+    rng = np.random.default_rng(5)
+    M, N, K = 70, 45, 37
+    tdt = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}[dt]
+    A = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(tdt)
+    B = torch.from_numpy(rng.standard_normal((N, K)).astype(np.float32)).to(tdt)
+    C0 = torch.from_numpy(rng.standard_normal((M, N)).astype(np.float32))
+    a, b, c = A.cuda(), B.cuda(), C0.cuda()
+    d = torch.zeros(M, N, dtype=torch.float32, device="cuda")
+    mh.gemm_(mh.tiled_mma_desc(mh.MMA_UNIVERSAL_FMA), T(d), T(a), T(b), T(c))
+    torch.cuda.synchronize()
+    want = to.gemm_universal_fma(A.float().numpy(), B.float().numpy(), C0.numpy(), dt, dt)
+    assert np.array_equal(d.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
+def test_universal_fma_matches_reference_device_test_shape(mh):
+    """test/device/matmul.jl:75-81 — C = A*B' with A:(2048,256), B:(2048,256) column-major."""
+    rng = np.random.default_rng(6)
+    M = N = 2048
+    K = 256
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    B = rng.standard_normal((N, K)).astype(np.float32)
+    a = torch.from_numpy(A.reshape(-1, order="F").copy()).cuda()
+    b = torch.from_numpy(B.reshape(-1, order="F").copy()).cuda()
+    c = torch.zeros(M * N, dtype=torch.float32, device="cuda")
+    mh.gemm_(mh.tiled_mma_desc(mh.MMA_UNIVERSAL_FMA, cta_tile=(128, 128, 8)), T(c, (M, N), (1, M)),
+             T(a, (M, K), (1, M)), T(b, (N, K), (1, N)))
+    torch.cuda.synchronize()
+    got = c.cpu().numpy().reshape(N, M).T
+    rows = rng.choice(M, 48, replace=False)
+    want = to.gemm_universal_fma(A[rows], B, np.zeros((len(rows), N), np.float32))
+    assert np.array_equal(got[rows].view(np.uint32), want.view(np.uint32))
+
+
+# ---------------------------------------------------------------------------------------------
+# MFMA kernels: tolerance against fp64
+# ---------------------------------------------------------------------------------------------
+
+def _mfma_case(mh, atom, tdt, out_dt, M, N, K, seed, scale, cta=(128, 128, 0), col_major_d=False, with_c=False,
+               alpha=1.0):
+    g = torch.Generator().manual_seed(seed)
+    A = (torch.randn(M, K, generator=g) * scale).to(tdt)
+    B = (torch.randn(N, K, generator=g) * scale).to(tdt)
+    a, b = A.cuda(), B.cuda()
+    if col_major_d:
+        d = torch.zeros(N, M, dtype=out_dt, device="cuda")
+        dd = T(d, (M, N), (1, M))
+    else:
+        d = torch.zeros(M, N, dtype=out_dt, device="cuda")
+        dd = T(d)
+    cc, C0 = None, None
+    if with_c:
+        C0 = torch.randn(M, N, generator=g).to(out_dt)
+        c = C0.cuda()
+        cc = T(c)
+    mh.gemm_(mh.tiled_mma_desc(atom, atom_layout=(2, 2, 1), cta_tile=cta), dd, T(a), T(b), cc, alpha)
+    torch.cuda.synchronize()
+    got = d.t() if col_major_d else d
+    c64 = alpha * (a.double() @ b.double().t())
+    if with_c:
+        c64 = c64 + C0.cuda().double()
+    return got, c64, A, B
+
+
+@pytest.mark.parametrize("bk", [32, 64])
+@pytest.mark.parametrize("M,N,K", [(128, 128, 64), (256, 384, 512), (512, 256, 1024)])
+def test_f16_tn_small(mh, M, N, K, bk):
+    got, c64, A, B = _mfma_case(mh, mh.MFMA_F32_16x16x32_F16, torch.float16, torch.float16, M, N, K, 3,
+                                K ** -0.5, cta=(128, 128, bk))
+    err = relerr(got, c64)
+    # the reference's own arithmetic (16-bit rounded products, sequential fp32 sum), fp16 output
+    ref = to.gemm_universal_fma(A.float().numpy(), B.float().numpy(), np.zeros((M, N), np.float32), "f16", "f16")
+    ref_err = to.relerr(ref.astype(np.float16), c64.cpu().numpy())
+    print("f16 %dx%dx%d bk=%d: rel err %.3e (reference arithmetic %.3e)" % (M, N, K, bk, err, ref_err))
+    assert err <= TOL16
+    # cross-check the GPU fp64 oracle against numpy on the host
+    c64_host = A.double().numpy() @ B.double().numpy().T
+    assert np.allclose(c64.cpu().numpy(), c64_host, rtol=1e-12, atol=1e-12)
+
+
+def test_f16_tn_exact_on_integers(mh):
+    """Small-integer inputs make every product and partial sum exact in fp32, so any indexing
+    mistake (wrong k pairing, transposed tile, swapped fragment) shows as a hard mismatch."""
+    M, N, K = 256, 256, 256
+    g = torch.Generator().manual_seed(8)
+    A = torch.randint(-4, 5, (M, K), generator=g).to(torch.float16)
+    B = torch.randint(-4, 5, (N, K), generator=g).to(torch.float16)
+    a, b = A.cuda(), B.cuda()
+    for out_dt in (torch.float32, torch.float16):
+        d = torch.zeros(M, N, dtype=out_dt, device="cuda")
+        mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(128, 128, 32)), T(d), T(a), T(b))
+        torch.cuda.synchronize()
+        want = (A.double() @ B.double().t())
+        assert torch.equal(d.cpu().double(), want)
+
+
+def test_f16_variants(mh):
+    """column-major D, C accumulation, alpha, fp32 output."""
+    for kw in (dict(col_major_d=True), dict(with_c=True), dict(with_c=True, alpha=0.5, col_major_d=True)):
+        for out_dt in (torch.float16, torch.float32):
+            got, c64, _, _ = _mfma_case(mh, mh.MFMA_F32_16x16x32_F16, torch.float16, out_dt, 256, 128, 256, 4,
+                                        1 / 16, **kw)
+            assert relerr(got, c64) <= TOL16, kw
+
+
+def test_config3_f16_tn_4096(mh):
+    """BASELINE config 3 at full size: fp16 TN 4096^3, fp32 accumulate, fp16 out, 128x128x32 tile."""
+    M = N = K = 4096
+    got, c64, A, B = _mfma_case(mh, mh.MFMA_F32_16x16x32_F16, torch.float16, torch.float16, M, N, K, 1003,
+                                K ** -0.5, cta=(128, 128, 32))
+    err = relerr(got, c64)
+    rows = np.random.default_rng(0).choice(M, 64, replace=False)
+    host = A[rows].double().numpy() @ B.double().numpy().T
+    assert np.allclose(c64[rows].cpu().numpy(), host, rtol=1e-12, atol=1e-12)
+    ref = to.gemm_universal_fma(A[rows[:16]].float().numpy(), B.float().numpy(), np.zeros((16, N), np.float32),
+                                "f16", "f16").astype(np.float16)
+    ref_err = to.relerr(ref, host[:16])
+    print("config3 f16 4096^3: rel err %.3e (reference arithmetic on 16 rows: %.3e)" % (err, ref_err))
+    assert err <= TOL16
+
+
+def test_bf16_tn(mh):
+    """BASELINE config 4 (square), reduced to 1024^3 here; bf16 in, fp32 out, N(0, 0.02)."""
+    got, c64, A, B = _mfma_case(mh, mh.MFMA_F32_16x16x32_BF16, torch.bfloat16, torch.float32, 1024, 1024, 1024,
+                                1004, 0.02)
+    err = relerr(got, c64)
+    ref = to.gemm_universal_fma(A[:32].float().numpy(), B.float().numpy(), np.zeros((32, 1024), np.float32),
+                                "bf16", "bf16")
+    ref_err = to.relerr(ref, c64[:32].cpu().numpy())
+    print("bf16 1024^3: rel err %.3e (reference arithmetic on 32 rows: %.3e)" % (err, ref_err))
+    assert err <= TOL16
+
+
+def test_fp8_tn_with_scales(mh):
+    """BASELINE config 5 reduced to 1024^3: e4m3 inputs quantised per tensor by amax/448, fp32
+    accumulate, bf16 out = acc * s_a * s_b."""
+    if not hasattr(torch, "float8_e4m3fn"):
+        pytest.skip("torch without float8_e4m3fn")
+    M = N = K = 1024
+    g = torch.Generator().manual_seed(1005)
+    X, W = torch.randn(M, K, generator=g), torch.randn(N, K, generator=g)
+    sa, sb = float(X.abs().max() / 448), float(W.abs().max() / 448)
+    qa, qb = (X / sa).to(torch.float8_e4m3fn), (W / sb).to(torch.float8_e4m3fn)
+    a, b = qa.cuda(), qb.cuda()
+    d = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
+    mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_FP8, cta_tile=(128, 128, 64)), T(d), T(a), T(b), None, sa * sb)
+    torch.cuda.synchronize()
+    c64 = (qa.double().cuda() @ qb.double().cuda().t()) * (sa * sb)
+    err = relerr(d, c64)
+    print("fp8 1024^3: rel err vs fp64 of the quantised inputs %.3e" % err)
+    assert err <= TOL16
+
+
+def test_gemm_errors(mh):
+    a = torch.zeros(128, 64, dtype=torch.float16, device="cuda")
+    b = torch.zeros(128, 64, dtype=torch.float16, device="cuda")
+    d = torch.zeros(128, 128, dtype=torch.float16, device="cuda")
+    E = mh._lib
+    mma = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(128, 128, 32))
+    with pytest.raises(mh.MoyeError) as e:  # K mismatch
+        mh.gemm_(mma, T(d), T(a), T(b[:, :32]))
+    assert e.value.status == E.ERR_SHAPE
+    with pytest.raises(mh.MoyeError) as e:  # tile does not divide
+        mh.gemm_(mma, T(d[:96]), T(a[:96]), T(b))
+    assert e.value.status == E.ERR_SHAPE
+    with pytest.raises(mh.MoyeError) as e:  # M-major A is not the TN form
+        mh.gemm_(mma, T(d), T(a, (128, 64), (1, 128)), T(b))
+    assert e.value.status == E.ERR_UNSUPPORTED
+    with pytest.raises(mh.MoyeError) as e:  # wrong operand type for the atom
+        mh.gemm_(mma, T(d), T(a.float()), T(b))
+    assert e.value.status == E.ERR_UNSUPPORTED
+    with pytest.raises(mh.MoyeError) as e:  # rank
+        mh.gemm_(mma, T(d), T(a, (128, 8, 8), (64, 8, 1)), T(b))
+    assert e.value.status == E.ERR_RANK

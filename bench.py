@@ -24,28 +24,38 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
 def cpu_baseline(cores):
     """The reference's CPU path, restated (oracle/gemm_oracle.c): UniversalFMA gemm! over host
-    arrays, fp16 operands, 32x32x8 tiles, on a bounded 768^3 sample of the same workload."""
+    arrays, fp16 operands, 32x32x8 tiles, on a bounded sub-problem (about 12 s) of the same workload."""
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
     import numpy as np
     import c_oracle as co
 
-    n = 768
     rng = np.random.default_rng(1003)
-    A = (rng.standard_normal((n, n)) / np.sqrt(4096)).astype(np.float16).astype(np.float32)
-    B = (rng.standard_normal((n, n)) / np.sqrt(4096)).astype(np.float16).astype(np.float32)
+
+    def operands(n):
+        a = (rng.standard_normal((n, n)) / np.sqrt(4096)).astype(np.float16).astype(np.float32)
+        b = (rng.standard_normal((n, n)) / np.sqrt(4096)).astype(np.float16).astype(np.float32)
+        return a, b
+
+    A, B = operands(512)
     co.gemm(A[:64, :64], B[:64, :64], None, "f16", (32, 32, 8), cores)  # load + warm
     t0 = time.perf_counter()
     co.gemm(A, B, None, "f16", (32, 32, 8), cores)
+    rate = 2.0 * 512 ** 3 / (time.perf_counter() - t0)      # flop/s on a probe
+    # bounded sample: about 12 s of CPU work, a multiple of 256, at most the full 4096^3 problem
+    n = int(min(4096, max(512, ((rate * 12.0 / 2.0) ** (1.0 / 3.0)) // 256 * 256)))
+    A, B = operands(n)
+    t0 = time.perf_counter()
+    co.gemm(A, B, None, "f16", (32, 32, 8), cores)
     dt = time.perf_counter() - t0
-    return {"value": 2.0 * n ** 3 / dt / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+    return {"value": round(2.0 * n ** 3 / dt / 1e12, 6), "unit": "TFLOP/s", "cores": cores, "kind": "port",
             "sample": "fp16 TN %d^3 sub-problem of the 4096^3 workload, UniversalFMA gemm! restatement "
-                      "(32x32x8 tiles, OpenMP over C tiles), %.2f s" % (n, dt)}
+                      "(32x32x8 tiles, OpenMP over C tiles), %.1f s" % (n, dt)}
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-copy", action="store_true", help="skip the tiled-copy leg")

@@ -191,11 +191,12 @@ def test_fp8_conversion_matches_torch(mh):
 
 def test_copy_errors(mh):
     a = torch.zeros(64, dtype=torch.int32, device="cuda")
+    af = a.float()
     with pytest.raises(mh.MoyeError) as e:
         mh.copyto_(_tens(mh, a, (8, 8), (1, 8)), _tens(mh, a, (8, 4), (1, 8)))
     assert e.value.status == mh._lib.ERR_SHAPE
     with pytest.raises(mh.MoyeError) as e:
-        mh.copyto_(_tens(mh, a, (8, 8), (1, 8)), _tens(mh, a.float(), (8, 8), (1, 8)))
+        mh.copyto_(_tens(mh, a, (8, 8), (1, 8)), _tens(mh, af, (8, 8), (1, 8)))
     assert e.value.status == mh._lib.ERR_UNSUPPORTED
     tc = mh.tiled_copy_desc(op=mh.COPY_LDS_TILED, tiler=(64, 64))
     with pytest.raises(mh.MoyeError) as e:  # 8x8 is not a multiple of the 64x64 LDS tile

@@ -241,7 +241,8 @@ def test_gemm_errors(mh):
         mh.gemm_(mma, T(d), T(a, (128, 64), (1, 128)), T(b))
     assert e.value.status == E.ERR_UNSUPPORTED
     with pytest.raises(mh.MoyeError) as e:  # wrong operand type for the atom
-        mh.gemm_(mma, T(d), T(a.float()), T(b))
+        a32 = a.float()
+        mh.gemm_(mma, T(d), T(a32), T(b))
     assert e.value.status == E.ERR_UNSUPPORTED
     with pytest.raises(mh.MoyeError) as e:  # rank
         mh.gemm_(mma, T(d), T(a, (128, 8, 8), (64, 8, 1)), T(b))

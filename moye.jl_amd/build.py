@@ -21,6 +21,7 @@ SOURCES = {
     "capi.hip": [],
     "copy_kernels.hip": [],
     "gemm_mfma.hip": [],
+    "gemm_mfma256.hip": [],
     "gemm_universal.hip": ["-ffp-contract=off"],   # UniversalFMA: mul then add, never fused
     "layout_host.cpp": ["-x", "hip"],
 }

@@ -16,92 +16,9 @@
 // 16x16 MFMA tiles.  The MFMA is issued with the B-matrix rows as its first operand and the
 // A-matrix rows as its second, so a lane ends up holding four CONSECUTIVE n of one m, which is
 // what a row-major D wants.
-#include "kernels.hpp"
+#include "mfma_common.hpp"
 
 namespace moye {
-
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
-
-// ---- input element traits: how one pair of 16-byte chunks feeds the MFMA pipe ----------------
-struct InF16 {
-    static constexpr int kBytes = 2;
-    static __device__ __forceinline__ void mma(const u32x4& a, const u32x4& b, f32x4& c) {
-        c = __builtin_amdgcn_mfma_f32_16x16x32_f16((f16x8)a, (f16x8)b, c, 0, 0, 0);
-    }
-};
-struct InBF16 {
-    static constexpr int kBytes = 2;
-    static __device__ __forceinline__ void mma(const u32x4& a, const u32x4& b, f32x4& c) {
-        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16((bf16x8)a, (bf16x8)b, c, 0, 0, 0);
-    }
-};
-// A 16-byte chunk holds 16 fp8 values = the k-slices of two MFMAs.  Both operands split the
-// chunk the same way, so the pairing of products is unchanged.
-struct InFP8 {
-    static constexpr int kBytes = 1;
-    static __device__ __forceinline__ void mma(const u32x4& a, const u32x4& b, f32x4& c) {
-        const long a0 = (long)(((uint64_t)a.y << 32) | a.x), a1 = (long)(((uint64_t)a.w << 32) | a.z);
-        const long b0 = (long)(((uint64_t)b.y << 32) | b.x), b1 = (long)(((uint64_t)b.w << 32) | b.z);
-        c = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a0, b0, c, 0, 0, 0);
-        c = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a1, b1, c, 0, 0, 0);
-    }
-};
-
-// ---- output element traits: fp32 -> OutT, round to nearest even (src/arch/copy/copy.jl:38-43) ---
-struct OutF32 {
-    typedef float type;
-    static __device__ __forceinline__ float cvt(float x) { return x; }
-    static __device__ __forceinline__ float load(const void* p, int64_t i) { return static_cast<const float*>(p)[i]; }
-};
-struct OutF16 {
-    typedef _Float16 type;
-    static __device__ __forceinline__ _Float16 cvt(float x) { return (_Float16)x; }
-    static __device__ __forceinline__ float load(const void* p, int64_t i) { return (float)static_cast<const _Float16*>(p)[i]; }
-};
-struct OutBF16 {
-    typedef uint16_t type;
-    static __device__ __forceinline__ uint16_t cvt(float x) {
-        uint32_t u = __float_as_uint(x);
-        if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
-        u += 0x7fffu + ((u >> 16) & 1u);
-        return (uint16_t)(u >> 16);
-    }
-    static __device__ __forceinline__ float load(const void* p, int64_t i) {
-        return __uint_as_float((uint32_t)static_cast<const uint16_t*>(p)[i] << 16);
-    }
-};
-
-// XOR swizzle of the 16-byte chunk index inside an LDS tile row of CPR chunks: rows that are
-// 256 bytes apart in LDS (one full sweep of the 64 banks) get different chunk permutations, so
-// 16 lanes reading the same logical chunk of 16 consecutive rows hit 16 different bank groups.
-template <int CPR>
-__device__ __forceinline__ int swz(int row) {
-    if constexpr (CPR >= 16) return row & 15;
-    else return (row / (16 / CPR)) & (CPR - 1);
-}
-
-// blockIdx -> (tile_m, tile_n).  Hardware deals consecutive workgroup ids round-robin to the 8
-// XCDs; remapping id -> (id % 8) * (n / 8) + id / 8 hands each XCD one contiguous run of tiles,
-// and inside a run tiles are walked in bands of 8 tile-rows so that the A and B panels an
-// XCD's L2 holds are reused by the workgroups that follow.
-__device__ __forceinline__ void tile_of_block(const GemmArgs& p, int* tm, int* tn) {
-    int bid = blockIdx.x;
-    const int n = gridDim.x;
-    if (p.xcd_swizzle && (n % 8) == 0) bid = (bid % 8) * (n / 8) + bid / 8;
-    constexpr int kGroup = 8;
-    const int per_group = kGroup * p.tiles_n;
-    const int g = bid / per_group;
-    const int first_m = g * kGroup;
-    const int gsize = min(p.tiles_m - first_m, kGroup);
-    const int r = bid - g * per_group;
-    *tm = first_m + r % gsize;
-    *tn = r / gsize;
-}
 
 template <typename In, typename Out, int BM, int BN, int BKB /* bytes of K per tile row */>
 __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
@@ -285,23 +202,35 @@ static int32_t launch_out(int32_t out_dt, const GemmArgs& a, hipStream_t st) {
 }
 
 // K-major A and B, N-contiguous D.  bk_elems = 0 picks the default K extent per tile.
-int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int bk_elems,
+int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int bk_elems, int waves,
                               GemmArgs a, hipStream_t st) {
     const int eb = dtype_bytes(in_dt);
     if (bm == 0) bm = 128;
     if (bn == 0) bn = 128;
     if (bk_elems == 0) bk_elems = 64 / eb;  // 64 bytes of K per row: 32 halves / 64 fp8
     const int bkb = bk_elems * eb;
+    const int ob = dtype_bytes(out_dt);
+    const bool misaligned =
+        (a.lda * eb) % 16 || (a.ldb * eb) % 16 || (a.ldd * ob) % 16 ||
+        (reinterpret_cast<uintptr_t>(a.A) | reinterpret_cast<uintptr_t>(a.B) | reinterpret_cast<uintptr_t>(a.D)) % 16;
+    if (bm == 256 && bn == 256) {
+        if (bkb != 128 && bk_elems != 64 / eb)
+            return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the 256x256 MFMA kernel takes %d elements of K per tile", 128 / eb);
+        if (a.M % 256 || a.N % 256 || a.K % (128 / eb))
+            return fail(MOYE_ERR_SHAPE, "gemm!: CTA tile 256x256x%d does not divide the problem %dx%dx%d", 128 / eb,
+                        a.M, a.N, a.K);
+        if (misaligned)
+            return fail(MOYE_ERR_ALIGN, "gemm!: operands of the MFMA kernels need 16-byte aligned pointers and row pitches");
+        return gemm_mfma_tn_256_dispatch(in_dt, out_dt, a, waves, st);
+    }
     if (bm != 128 || bn != 128 || (bkb != 64 && bkb != 128))
         return fail(MOYE_ERR_UNSUPPORTED,
-                    "gemm!: no MFMA kernel for CTA tile %dx%dx%d (%s); built: 128x128x{%d,%d}", bm, bn, bk_elems,
-                    dtype_name(in_dt), 64 / eb, 128 / eb);
+                    "gemm!: no MFMA kernel for CTA tile %dx%dx%d (%s); built: 128x128x{%d,%d} and 256x256x%d", bm, bn,
+                    bk_elems, dtype_name(in_dt), 64 / eb, 128 / eb, 128 / eb);
     if (a.M % bm || a.N % bn || a.K % bk_elems)
         return fail(MOYE_ERR_SHAPE, "gemm!: CTA tile %dx%dx%d does not divide the problem %dx%dx%d", bm, bn,
                     bk_elems, a.M, a.N, a.K);
-    const int ob = dtype_bytes(out_dt);
-    if ((a.lda * eb) % 16 || (a.ldb * eb) % 16 || (a.ldd * ob) % 16 ||
-        (reinterpret_cast<uintptr_t>(a.A) | reinterpret_cast<uintptr_t>(a.B) | reinterpret_cast<uintptr_t>(a.D)) % 16)
+    if (misaligned)
         return fail(MOYE_ERR_ALIGN, "gemm!: operands of the MFMA kernels need 16-byte aligned pointers and row pitches");
     a.tiles_m = a.M / bm;
     a.tiles_n = a.N / bn;

@@ -1,0 +1,93 @@
+// Element traits, LDS swizzle and tile mapping shared by the MFMA GEMM kernels.
+#pragma once
+
+#include "kernels.hpp"
+
+namespace moye {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+
+// ---- input element traits: how one pair of 16-byte chunks feeds the MFMA pipe ----------------
+struct InF16 {
+    static constexpr int kBytes = 2;
+    static __device__ __forceinline__ void mma(const u32x4& a, const u32x4& b, f32x4& c) {
+        c = __builtin_amdgcn_mfma_f32_16x16x32_f16((f16x8)a, (f16x8)b, c, 0, 0, 0);
+    }
+};
+struct InBF16 {
+    static constexpr int kBytes = 2;
+    static __device__ __forceinline__ void mma(const u32x4& a, const u32x4& b, f32x4& c) {
+        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16((bf16x8)a, (bf16x8)b, c, 0, 0, 0);
+    }
+};
+// A 16-byte chunk holds 16 fp8 values = the k-slices of two MFMAs.  Both operands split the
+// chunk the same way, so the pairing of products is unchanged.
+struct InFP8 {
+    static constexpr int kBytes = 1;
+    static __device__ __forceinline__ void mma(const u32x4& a, const u32x4& b, f32x4& c) {
+        const long a0 = (long)(((uint64_t)a.y << 32) | a.x), a1 = (long)(((uint64_t)a.w << 32) | a.z);
+        const long b0 = (long)(((uint64_t)b.y << 32) | b.x), b1 = (long)(((uint64_t)b.w << 32) | b.z);
+        c = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a0, b0, c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a1, b1, c, 0, 0, 0);
+    }
+};
+
+// ---- output element traits: fp32 -> OutT, round to nearest even (src/arch/copy/copy.jl:38-43) ---
+struct OutF32 {
+    typedef float type;
+    static __device__ __forceinline__ float cvt(float x) { return x; }
+    static __device__ __forceinline__ float load(const void* p, int64_t i) { return static_cast<const float*>(p)[i]; }
+};
+struct OutF16 {
+    typedef _Float16 type;
+    static __device__ __forceinline__ _Float16 cvt(float x) { return (_Float16)x; }
+    static __device__ __forceinline__ float load(const void* p, int64_t i) { return (float)static_cast<const _Float16*>(p)[i]; }
+};
+struct OutBF16 {
+    typedef uint16_t type;
+    static __device__ __forceinline__ uint16_t cvt(float x) {
+        uint32_t u = __float_as_uint(x);
+        if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+        u += 0x7fffu + ((u >> 16) & 1u);
+        return (uint16_t)(u >> 16);
+    }
+    static __device__ __forceinline__ float load(const void* p, int64_t i) {
+        return __uint_as_float((uint32_t)static_cast<const uint16_t*>(p)[i] << 16);
+    }
+};
+
+// XOR swizzle of the 16-byte chunk index inside an LDS tile row of CPR chunks.  The LDS has 32
+// banks of 4 bytes, so 128 bytes (8 chunks) make one sweep of the banks and a 128-bit access is
+// served 8 lanes per clock.  Rows that lie in different 128-byte sweeps get different chunk
+// permutations, so 8 lanes reading the same logical chunk of 8 consecutive rows hit 8 different
+// bank groups, and so do 8 lanes writing 8 consecutive chunks.
+template <int CPR>
+__device__ __forceinline__ int swz(int row) {
+    if constexpr (CPR >= 8) return row & 7;
+    else return (row / (8 / CPR)) & (CPR - 1);
+}
+
+// blockIdx -> (tile_m, tile_n).  Hardware deals consecutive workgroup ids round-robin to the 8
+// XCDs; remapping id -> (id % 8) * (n / 8) + id / 8 hands each XCD one contiguous run of tiles,
+// and inside a run tiles are walked in bands of 8 tile-rows so that the A and B panels an
+// XCD's L2 holds are reused by the workgroups that follow.
+__device__ __forceinline__ void tile_of_block(const GemmArgs& p, int* tm, int* tn) {
+    int bid = blockIdx.x;
+    const int n = gridDim.x;
+    if (p.xcd_swizzle && (n % 8) == 0) bid = (bid % 8) * (n / 8) + bid / 8;
+    constexpr int kGroup = 8;
+    const int per_group = kGroup * p.tiles_n;
+    const int g = bid / per_group;
+    const int first_m = g * kGroup;
+    const int gsize = min(p.tiles_m - first_m, kGroup);
+    const int r = bid - g * per_group;
+    *tm = first_m + r % gsize;
+    *tn = r / gsize;
+}
+
+}  // namespace moye

@@ -59,7 +59,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-copy", action="store_true", help="skip the tiled-copy leg")
-    ap.add_argument("--tile", default="128,128,32", help="CTA tile bm,bn,bk of the GEMM kernel")
+    ap.add_argument("--tile", default="256,256,64", help="CTA tile bm,bn,bk of the GEMM kernel")
+    ap.add_argument("--waves", default="2,4", help="waves per CTA along M,N (TiledMMA atom layout)")
+    ap.add_argument("--stages", type=int, default=0, help="LDS pipeline depth (0 = kernel default)")
+    ap.add_argument("--flags", type=int, default=0, help="MOYE_GEMM_* bits (1 = no XCD swizzle)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; --gpus %d is not supported (every box has one "
@@ -79,8 +82,9 @@ def main():
     A = (torch.randn(M, K, generator=g) / K ** 0.5).half().cuda()
     B = (torch.randn(N, K, generator=g) / K ** 0.5).half().cuda()
     D = torch.zeros(M, N, dtype=torch.float16, device="cuda")
-    mma = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 2, 1), tile=(bm, bn, bk),
-                            cta_tile=(bm, bn, bk))
+    wm, wn = (int(v) for v in args.waves.split(","))
+    mma = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(wm, wn, 1), tile=(bm, bn, bk),
+                            cta_tile=(bm, bn, bk), stages=args.stages, flags=args.flags)
     tA, tB, tD = tensor_of(A), tensor_of(B), tensor_of(D)
 
     for _ in range(args.warmup):
@@ -111,7 +115,7 @@ def main():
         "ms_per_step": round(elapsed / args.steps * 1e3, 5), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": "fp16 TN GEMM M=N=K=4096, A row-major (MxK), B col-major (KxN), fp32 accumulate, "
-                               "fp16 out; CTA tile %dx%dx%d, 2x2 waves of v_mfma_f32_16x16x32_f16" % (bm, bn, bk),
+                               "fp16 out; CTA tile %dx%dx%d, %dx%d waves of v_mfma_f32_16x16x32_f16" % (bm, bn, bk, wm, wn),
                    "rel_err_vs_fp64": err},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_F16_TFLOPS, 4), "traffic": None,

@@ -104,16 +104,16 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
     const int waves = mma->atom_layout_mnk[0] * mma->atom_layout_mnk[1];
     g.alpha = alpha;
     g.K = K;
-    g.xcd_swizzle = !(mma->flags & MOYE_GEMM_NO_XCD_SWIZZLE);
+    g.xcd_swizzle = !(mma->flags & MOYE_GEMM_NO_XCD_SWIZZLE) | (mma->flags & 0xff00);
     if (D.cs == 1) {  // row-major D
         g.A = A.ptr; g.B = B.ptr; g.M = M; g.N = N; g.lda = A.rs; g.ldb = B.rs; g.ldd = D.rs;
         g.C = tC ? C.ptr : nullptr; g.ldc_m = C.rs; g.ldc_n = C.cs; g.D = D.ptr;
-        return gemm_mfma_tn_dispatch(in_dt, D.dtype, bm, bn, bk, waves, g, st);
+        return gemm_mfma_tn_dispatch(in_dt, D.dtype, bm, bn, bk, waves, mma->stages, g, st);
     }
     if (D.rs == 1) {  // column-major D: D' = B * A' is row-major
         g.A = B.ptr; g.B = A.ptr; g.M = N; g.N = M; g.lda = B.rs; g.ldb = A.rs; g.ldd = D.cs;
         g.C = tC ? C.ptr : nullptr; g.ldc_m = C.cs; g.ldc_n = C.rs; g.D = D.ptr;
-        return gemm_mfma_tn_dispatch(in_dt, D.dtype, bn, bm, bk, waves, g, st);
+        return gemm_mfma_tn_dispatch(in_dt, D.dtype, bn, bm, bk, waves, mma->stages, g, st);
     }
     return fail(MOYE_ERR_UNSUPPORTED, "gemm!: D needs a unit stride along M or N");
 }

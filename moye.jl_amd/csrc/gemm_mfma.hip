@@ -202,7 +202,7 @@ static int32_t launch_out(int32_t out_dt, const GemmArgs& a, hipStream_t st) {
 }
 
 // K-major A and B, N-contiguous D.  bk_elems = 0 picks the default K extent per tile.
-int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int bk_elems, int waves,
+int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int bk_elems, int waves, int stages,
                               GemmArgs a, hipStream_t st) {
     const int eb = dtype_bytes(in_dt);
     if (bm == 0) bm = 128;
@@ -214,14 +214,14 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         (a.lda * eb) % 16 || (a.ldb * eb) % 16 || (a.ldd * ob) % 16 ||
         (reinterpret_cast<uintptr_t>(a.A) | reinterpret_cast<uintptr_t>(a.B) | reinterpret_cast<uintptr_t>(a.D)) % 16;
     if (bm == 256 && bn == 256) {
-        if (bkb != 128 && bk_elems != 64 / eb)
-            return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the 256x256 MFMA kernel takes %d elements of K per tile", 128 / eb);
+        if (bkb != 128 && bkb != 64)
+            return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the 256x256 MFMA kernels take %d or %d elements of K per tile", 64 / eb, 128 / eb);
         if (a.M % 256 || a.N % 256 || a.K % (128 / eb))
             return fail(MOYE_ERR_SHAPE, "gemm!: CTA tile 256x256x%d does not divide the problem %dx%dx%d", 128 / eb,
                         a.M, a.N, a.K);
         if (misaligned)
             return fail(MOYE_ERR_ALIGN, "gemm!: operands of the MFMA kernels need 16-byte aligned pointers and row pitches");
-        return gemm_mfma_tn_256_dispatch(in_dt, out_dt, a, waves, st);
+        return gemm_mfma_tn_256_dispatch(in_dt, out_dt, a, waves, stages, st);
     }
     if (bm != 128 || bn != 128 || (bkb != 64 && bkb != 128))
         return fail(MOYE_ERR_UNSUPPORTED,

@@ -7,12 +7,14 @@
 // LDS bytes per flop (and the L2 bytes per flop of the workgroup).  4096 / 256 = 16, so a 4096^2
 // problem is exactly 256 workgroups: one per CU, no tail.
 //
-// Schedule per k-tile (two k-steps of 32 halves / 64 fp8), operand tiles double-buffered in LDS:
-//   ds_read fragments of step 1                      (fragments are double-buffered in registers)
-//   global_load_lds_dwordx4 of tile t+1 -> the other LDS stage (no registers, no ds_write)
-//   MFMAs of step 0, first half of the MFMAs of step 1
-//   s_waitcnt vmcnt(0), barrier, ds_read fragments of step 0 of tile t+1
-//   second half of the MFMAs of step 1               (covers the LDS latency after the barrier)
+// Schedule per k-tile (two k-steps of 32 halves / 64 fp8), operand tiles double-buffered in LDS,
+// fragments double-buffered in registers:
+//   step 0: ds_read the fragments of step 1 (buffer 1) | MFMAs of step 0 (buffer 0)
+//   s_waitcnt vmcnt(0) lgkmcnt(0), s_barrier: tile t+1 has landed, nobody reads tile t any more
+//   global_load_lds_dwordx4 of tile t+2 -> the stage tile t just vacated: the loads have a whole
+//     iteration to complete and go straight to LDS (no registers, no ds_write)
+//   step 1: ds_read the fragments of step 0 of tile t+1 (buffer 0) | MFMAs of step 1 (buffer 1)
+// so the MFMAs that follow a barrier always find their operands already in registers.
 // A load-to-LDS instruction writes lane l's 16 bytes at base + 16 l, so the XOR swizzle is
 // applied on the global side: lane l of a 64-chunk block fetches chunk (l%8)^(l/8) of row l/8.
 //
@@ -75,7 +77,19 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
         __builtin_amdgcn_global_load_lds((gptr_t)(gB + (int64_t)(8 * i) * pitch_b + (KOFF)),          \
                                          (lptr_t)((BASE) + A_CH + dma_slot + 8 * CPR * i), 16, 0, 0); \
     }
-#define MOYE_WAIT_DMA() __builtin_amdgcn_s_waitcnt(0x0F70) /* vmcnt(0), leave expcnt and lgkmcnt alone */
+    // Wait until at most N of this wave's load-to-LDS instructions are in flight and its own LDS reads
+    // have returned, then meet the other waves.  A bare s_barrier on purpose: __syncthreads() adds a
+    // release fence that waits for ALL outstanding loads, which would drain the prefetch.  The waits
+    // are the s_waitcnt builtin (not asm text) so that the compiler's own wait-count bookkeeping
+    // sees them and does not add a second, stricter wait in front of the MFMAs.
+#define MOYE_WAIT_BARRIER(N)                                                                           \
+    {                                                                                                  \
+        __builtin_amdgcn_s_waitcnt(((N) & 0xF) | (((N) >> 4) << 14) | 0x0070); /* vmcnt(N) lgkmcnt(0) */ \
+        asm volatile("" ::: "memory");                                                                 \
+        __builtin_amdgcn_s_barrier();                                                                  \
+        asm volatile("" ::: "memory");                                                                 \
+    }
+#define MOYE_WAIT_LDS() __builtin_amdgcn_s_waitcnt(0xC07F) /* lgkmcnt(0) only */
 #define MOYE_FRAGS(BASE, KS, BUF)                                                                     \
     _Pragma("unroll") for (int i = 0; i < MI; ++i) fa[BUF][i] = (BASE)[fa_slot[KS] + 16 * CPR * i];   \
     _Pragma("unroll") for (int j = 0; j < NI; ++j) fb[BUF][j] = (BASE)[fb_slot[KS] + 16 * CPR * j];
@@ -83,34 +97,68 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
     _Pragma("unroll") for (int i = I0; i < I1; ++i)                                                   \
         _Pragma("unroll") for (int j = 0; j < NI; ++j) In::mma(fb[BUF][j], fa[BUF][i], acc[i][j]);
 
-    // prologue
+    // Issue order inside a k-step: the two waves of a SIMD leave the barrier together, so if each one
+    // issued all its fragment reads first the MFMA pipe would idle for both.  Spread them instead:
+    // NV load-to-LDS instructions each followed by one MFMA, then every ds_read followed by MFMAs.
+#define MOYE_INTERLEAVE(NV)                                                                           \
+    _Pragma("unroll") for (int q = 0; q < (NV); ++q) {                                                \
+        __builtin_amdgcn_sched_group_barrier(0x010, 1, 0); /* VMEM   */                               \
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); /* MFMA   */                               \
+    }                                                                                                 \
+    _Pragma("unroll") for (int q = 0; q < MI + NI; ++q) {                                             \
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); /* DS read */                              \
+        __builtin_amdgcn_sched_group_barrier(0x008, (MI * NI - (NV)) / (MI + NI), 0);                 \
+    }                                                                                                 \
+    __builtin_amdgcn_sched_group_barrier(0x008, (MI * NI - (NV)) % (MI + NI), 0);
+
+    // prologue: tiles 0 and 1 on their way, wait for tile 0 only (LD loads per operand are younger)
     MOYE_DMA(smem, 0)
-    MOYE_WAIT_DMA();
-    __syncthreads();
+    if (ktiles > 1) {
+        MOYE_DMA(smem + STAGE, 128)
+        MOYE_WAIT_BARRIER(2 * LD)
+    } else {
+        MOYE_WAIT_BARRIER(0)
+    }
     MOYE_FRAGS(smem, 0, 0)
 
-    for (int kt = 0; kt < ktiles; ++kt) {
-        u32x4* const cur = smem + (kt & 1) * STAGE;
-        u32x4* const nxt = smem + ((kt + 1) & 1) * STAGE;
-        const bool more = kt + 1 < ktiles;
-        MOYE_FRAGS(cur, 1, 1)
-        if (more) {
-            const int64_t koff = (int64_t)(kt + 1) * 128;
-            MOYE_DMA(nxt, koff)
-        }
-        MOYE_MMA(0, 0, MI)
-        MOYE_MMA(1, 0, MI / 2)
-        __builtin_amdgcn_sched_barrier(0);  // keep the MFMAs above on this side of the wait
-        MOYE_WAIT_DMA();
-        __syncthreads();
-        __builtin_amdgcn_sched_barrier(0);
-        if (more) {
-            MOYE_FRAGS(nxt, 0, 0)
-        }
-        MOYE_MMA(1, MI / 2, MI)
+    // One k-tile.  DMA: tile KT+2 exists and is fetched; NEXT: tile KT+1 exists and its first fragments
+    // are read.  The steady-state body has no branches, so each k-step is one scheduling region.
+#define MOYE_TILE(KT, DMA, NEXT)                                                                      \
+    {                                                                                                 \
+        u32x4* const cur = smem + ((KT) & 1) * STAGE;                                                 \
+        u32x4* const nxt = smem + (((KT) + 1) & 1) * STAGE;                                           \
+        /* step 0: MFMAs on buffer 0 while the fragments of step 1 arrive in buffer 1.  Buffer 0 was  \
+           requested a whole step ago; retiring those reads BEFORE the new ones are issued keeps the  \
+           MFMAs from waiting on the reads they are meant to overlap with. */                         \
+        MOYE_WAIT_LDS();                                                                              \
+        __builtin_amdgcn_sched_barrier(0);                                                            \
+        MOYE_FRAGS(cur, 1, 1)                                                                         \
+        MOYE_MMA(0, 0, MI)                                                                            \
+        MOYE_INTERLEAVE(0)                                                                            \
+        __builtin_amdgcn_sched_barrier(0);                                                            \
+        /* tile KT+1 has landed (the only loads in flight); this wave needs nothing more of tile KT */ \
+        MOYE_WAIT_BARRIER(0)                                                                          \
+        __builtin_amdgcn_sched_barrier(0);                                                            \
+        /* step 1: the stage tile KT lived in is free, so tile KT+2 gets a whole iteration to arrive; \
+           MFMAs on buffer 1 (already in registers) while step 0 of tile KT+1 arrives in buffer 0 */  \
+        if (DMA) MOYE_DMA(cur, (int64_t)((KT) + 2) * 128)                                             \
+        if (NEXT) MOYE_FRAGS(nxt, 0, 0)                                                               \
+        MOYE_MMA(1, 0, MI)                                                                            \
+        if (NEXT) { MOYE_INTERLEAVE((DMA) ? 2 * LD : 0) }                                             \
+        __builtin_amdgcn_sched_barrier(0);                                                            \
     }
+    int kt = 0;
+    for (; kt + 2 < ktiles; ++kt) MOYE_TILE(kt, true, true)
+    if (kt + 1 < ktiles) {
+        MOYE_TILE(kt, false, true)
+        ++kt;
+    }
+    MOYE_TILE(kt, false, false)
+#undef MOYE_TILE
+#undef MOYE_INTERLEAVE
 #undef MOYE_DMA
-#undef MOYE_WAIT_DMA
+#undef MOYE_WAIT_BARRIER
+#undef MOYE_WAIT_LDS
 #undef MOYE_FRAGS
 #undef MOYE_MMA
     __syncthreads();  // every wave is done with the operand stages before they become C patches
@@ -163,6 +211,175 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Ring schedule: the same 256 x 256 CTA tile, but the K extent per tile is 64 bytes (one k-step)
+// and the operand tiles live in a ring of STAGES LDS buffers filled by load-to-LDS instructions
+// issued STAGES-1 tiles ahead, so HBM/L2 latency has (STAGES-1) k-steps to hide in.
+// Per k-step: issue the loads of tile t+STAGES-1 | first half of the MFMAs of tile t |
+// s_waitcnt vmcnt(loads younger than tile t+1) | barrier | ds_read fragments of tile t+1 |
+// second half of the MFMAs of tile t.
+// ------------------------------------------------------------------------------------------------
+template <typename In, typename Out, int WGM, int WGN, int STAGES>
+__global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256_ring(GemmArgs p) {
+    constexpr int BM = 256, BN = 256, CPR = 4;  // 4 chunks of 16 bytes per tile row
+    constexpr int A_CH = BM * CPR, B_CH = BN * CPR, STAGE = A_CH + B_CH;
+    constexpr int NWAVES = WGM * WGN;
+    constexpr int WROWS = BM / NWAVES;  // operand rows each wave brings in per tile
+    constexpr int LD = WROWS / 16;      // load-to-LDS instructions per wave per operand (16 rows each)
+    constexpr int WM = BM / WGM, WN = BN / WGN, MI = WM / 16, NI = WN / 16;
+    static_assert(LD >= 1 && STAGES >= 3, "ring shape");
+    typedef typename Out::type OutT;
+
+    extern __shared__ u32x4 smem[];
+
+    int tm, tn;
+    tile_of_block(p, &tm, &tn);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm0 = (wave / WGN) * WM, wn0 = (wave % WGN) * WN;
+    const int r16 = lane & 15, kq = lane >> 4;
+
+    const int64_t pitch_a = (int64_t)p.lda * In::kBytes, pitch_b = (int64_t)p.ldb * In::kBytes;
+    // lane l of a load-to-LDS instruction lands in physical chunk l % 4 of row l / 4 of a 16-row block
+    const int lrow = wave * WROWS + (lane >> 2), lch = (lane & 3) ^ swz<CPR>(lane >> 2);
+    const char* gA = static_cast<const char*>(p.A) + ((int64_t)tm * BM + lrow) * pitch_a + lch * 16;
+    const char* gB = static_cast<const char*>(p.B) + ((int64_t)tn * BN + lrow) * pitch_b + lch * 16;
+    const int dma_slot = __builtin_amdgcn_readfirstlane(wave * WROWS * CPR);
+
+    const int fa_slot = (wm0 + r16) * CPR + (kq ^ swz<CPR>(r16));
+    const int fb_slot = A_CH + (wn0 + r16) * CPR + (kq ^ swz<CPR>(r16));
+
+    f32x4 acc[MI][NI];
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int ktiles = (int)(((int64_t)p.K * In::kBytes) / 64);
+    u32x4 fa[2][MI], fb[2][NI];
+
+    typedef __attribute__((address_space(1))) const void* gptr_t;
+    typedef __attribute__((address_space(3))) void* lptr_t;
+#define MOYE_DMA(T)                                                                                    \
+    {                                                                                                  \
+        u32x4* const base_ = smem + ((T) % STAGES) * STAGE + dma_slot;                                 \
+        const int64_t koff_ = (int64_t)(T) * 64;                                                       \
+        _Pragma("unroll") for (int i = 0; i < LD; ++i) {                                               \
+            __builtin_amdgcn_global_load_lds((gptr_t)(gA + (int64_t)(16 * i) * pitch_a + koff_),       \
+                                             (lptr_t)(base_ + 16 * CPR * i), 16, 0, 0);                \
+            __builtin_amdgcn_global_load_lds((gptr_t)(gB + (int64_t)(16 * i) * pitch_b + koff_),       \
+                                             (lptr_t)(base_ + A_CH + 16 * CPR * i), 16, 0, 0);         \
+        }                                                                                              \
+    }
+#define MOYE_VMCNT(N) __builtin_amdgcn_s_waitcnt(((N) & 0xF) | (((N) >> 4) << 14) | 0x0F70)
+    // Wait until at most N of this wave's load-to-LDS instructions are still in flight (the ones for
+    // tiles younger than t+1) and its own LDS reads have returned, then meet the other waves.  A
+    // plain s_barrier: __syncthreads() would add a release fence, which waits for ALL outstanding
+    // loads and so would drain the ring every k-step.
+#define MOYE_WAIT_BARRIER(N) \
+    { asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory"); }
+#define MOYE_FRAGS(T, BUF)                                                                             \
+    {                                                                                                  \
+        const u32x4* const base_ = smem + ((T) % STAGES) * STAGE;                                      \
+        _Pragma("unroll") for (int i = 0; i < MI; ++i) fa[BUF][i] = base_[fa_slot + 16 * CPR * i];     \
+        _Pragma("unroll") for (int j = 0; j < NI; ++j) fb[BUF][j] = base_[fb_slot + 16 * CPR * j];     \
+    }
+#define MOYE_MMA(BUF, I0, I1)                                                                          \
+    _Pragma("unroll") for (int i = I0; i < I1; ++i)                                                    \
+        _Pragma("unroll") for (int j = 0; j < NI; ++j) In::mma(fb[BUF][j], fa[BUF][i], acc[i][j]);
+    // one k-step; BUF is the fragment buffer that holds tile T
+#define MOYE_STEP(T, BUF)                                                                              \
+    {                                                                                                  \
+        const bool ahead_ = (T) + STAGES - 1 < ktiles;                                                 \
+        if (ahead_) MOYE_DMA((T) + STAGES - 1)                                                         \
+        MOYE_MMA(BUF, 0, MI / 2)                                                                       \
+        __builtin_amdgcn_sched_barrier(0);                                                             \
+        if (ahead_) MOYE_WAIT_BARRIER(2 * LD * (STAGES - 2)) else MOYE_WAIT_BARRIER(0)                 \
+        __builtin_amdgcn_sched_barrier(0);                                                             \
+        if ((T) + 1 < ktiles) MOYE_FRAGS((T) + 1, (BUF) ^ 1)                                           \
+        MOYE_MMA(BUF, MI / 2, MI)                                                                      \
+    }
+
+    // prologue: fill STAGES-1 buffers, wait for the first
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; ++s)
+        if (s < ktiles) MOYE_DMA(s)
+    MOYE_VMCNT(0);
+    __syncthreads();
+    MOYE_FRAGS(0, 0)
+
+    for (int kt = 0; kt < ktiles; kt += 2) {
+        MOYE_STEP(kt, 0)
+        if (kt + 1 < ktiles) MOYE_STEP(kt + 1, 1)
+    }
+#undef MOYE_DMA
+#undef MOYE_VMCNT
+#undef MOYE_WAIT_BARRIER
+#undef MOYE_FRAGS
+#undef MOYE_MMA
+#undef MOYE_STEP
+    __syncthreads();  // every wave is done with the operand ring before it becomes C patches
+
+    // ---- epilogue: alpha*acc + C -> OutT -> this wave's LDS patch -> 128-bit row stores ----
+    const int64_t m_base = (int64_t)tm * BM + wm0, n_base = (int64_t)tn * BN + wn0;
+    constexpr int EPC = 16 / (int)sizeof(OutT);
+    constexpr int CR = WN / EPC;
+    constexpr int PASS_MI = 2, PASS_ROWS = PASS_MI * 16;
+    static_assert(NWAVES * PASS_ROWS * WN * 4 <= STAGES * STAGE * 16, "C patches fit in the operand ring");
+    OutT* patch = reinterpret_cast<OutT*>(smem) + wave * (PASS_ROWS * WN);
+    u32x4* patch16 = reinterpret_cast<u32x4*>(patch);
+#pragma unroll
+    for (int i0 = 0; i0 < MI; i0 += PASS_MI) {
+#pragma unroll
+        for (int ii = 0; ii < PASS_MI; ++ii) {
+            const int i = i0 + ii;
+#pragma unroll
+            for (int j = 0; j < NI; ++j) {
+                float v[4] = {acc[i][j].x * p.alpha, acc[i][j].y * p.alpha, acc[i][j].z * p.alpha,
+                              acc[i][j].w * p.alpha};
+                if (p.C) {
+                    const int64_t m = m_base + 16 * i + r16, n = n_base + 16 * j + 4 * kq;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] += Out::load(p.C, m * p.ldc_m + (n + e) * p.ldc_n);
+                }
+                const int row = 16 * ii + r16, col = 16 * j + 4 * kq;
+                const int chunk = col / EPC, within = col % EPC;
+                OutT* dst = patch + (row * CR + (chunk ^ (row & 7))) * EPC + within;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) dst[e] = Out::cvt(v[e]);
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int t = 0; t < PASS_ROWS * CR / 64; ++t) {
+            const int c = lane + 64 * t, row = c / CR, ch = c % CR;
+            const u32x4 w = patch16[row * CR + (ch ^ (row & 7))];
+            char* d = static_cast<char*>(p.D) +
+                      ((m_base + 16 * i0 + row) * p.ldd + n_base) * (int64_t)sizeof(OutT) + ch * 16;
+            *reinterpret_cast<u32x4*>(d) = w;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+}
+
+template <typename In, typename Out, int STAGES>
+static int32_t launch256_ring(const GemmArgs& a, hipStream_t st) {
+    constexpr int kLds = STAGES * (256 + 256) * 64;
+    auto kern = gemm_mfma_tn_256_ring<In, Out, 2, 4, STAGES>;
+    static bool once = false;
+    if (!once) {
+        MOYE_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
+        once = true;
+    }
+    kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n)), dim3(512), kLds, st>>>(a);
+    MOYE_HIP_CHECK(hipGetLastError());
+    return MOYE_OK;
+}
+
 template <typename In, typename Out, int WGM, int WGN>
 static int32_t launch256(const GemmArgs& a, hipStream_t st) {
     constexpr int kLds = 2 * (256 + 256) * 128;  // two operand stages, 128 KiB
@@ -179,7 +396,16 @@ static int32_t launch256(const GemmArgs& a, hipStream_t st) {
 }
 
 template <typename In>
-static int32_t launch256_out(int32_t out_dt, const GemmArgs& a, int waves, hipStream_t st) {
+static int32_t launch256_out(int32_t out_dt, const GemmArgs& a, int waves, int stages, hipStream_t st) {
+    if (stages >= 3) {
+        const bool five = stages >= 5;
+        switch (out_dt) {
+            case MOYE_F32: return five ? launch256_ring<In, OutF32, 5>(a, st) : launch256_ring<In, OutF32, 4>(a, st);
+            case MOYE_F16: return five ? launch256_ring<In, OutF16, 5>(a, st) : launch256_ring<In, OutF16, 4>(a, st);
+            case MOYE_BF16: return five ? launch256_ring<In, OutBF16, 5>(a, st) : launch256_ring<In, OutBF16, 4>(a, st);
+            default: break;
+        }
+    }
     if (waves == 4) {
         switch (out_dt) {
             case MOYE_F32: return launch256<In, OutF32, 2, 2>(a, st);
@@ -197,13 +423,13 @@ static int32_t launch256_out(int32_t out_dt, const GemmArgs& a, int waves, hipSt
 }
 
 // 256 x 256 x (128 bytes of K) tile; the caller has checked divisibility and alignment.
-int32_t gemm_mfma_tn_256_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, int waves, hipStream_t st) {
+int32_t gemm_mfma_tn_256_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, int waves, int stages, hipStream_t st) {
     a.tiles_m = a.M / 256;
     a.tiles_n = a.N / 256;
     switch (in_dt) {
-        case MOYE_F16: return launch256_out<InF16>(out_dt, a, waves, st);
-        case MOYE_BF16: return launch256_out<InBF16>(out_dt, a, waves, st);
-        case MOYE_F8E4M3: return launch256_out<InFP8>(out_dt, a, waves, st);
+        case MOYE_F16: return launch256_out<InF16>(out_dt, a, waves, stages, st);
+        case MOYE_BF16: return launch256_out<InBF16>(out_dt, a, waves, stages, st);
+        case MOYE_F8E4M3: return launch256_out<InFP8>(out_dt, a, waves, stages, st);
         default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: no MFMA atom for %s inputs", dtype_name(in_dt));
     }
 }

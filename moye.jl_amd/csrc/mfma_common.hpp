@@ -18,11 +18,19 @@ struct InF16 {
     static __device__ __forceinline__ void mma(const u32x4& a, const u32x4& b, f32x4& c) {
         c = __builtin_amdgcn_mfma_f32_16x16x32_f16((f16x8)a, (f16x8)b, c, 0, 0, 0);
     }
+    // accumulator pinned in the AccVGPR file: its reads and write-backs then stay off the
+    // ArchVGPR ports that the LDS fragment loads are writing through
+    static __device__ __forceinline__ void mma_acc(const u32x4& a, const u32x4& b, f32x4& c) {
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    }
 };
 struct InBF16 {
     static constexpr int kBytes = 2;
     static __device__ __forceinline__ void mma(const u32x4& a, const u32x4& b, f32x4& c) {
         c = __builtin_amdgcn_mfma_f32_16x16x32_bf16((bf16x8)a, (bf16x8)b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ void mma_acc(const u32x4& a, const u32x4& b, f32x4& c) {
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
     }
 };
 // A 16-byte chunk holds 16 fp8 values = the k-slices of two MFMAs.  Both operands split the
@@ -34,6 +42,11 @@ struct InFP8 {
         const long b0 = (long)(((uint64_t)b.y << 32) | b.x), b1 = (long)(((uint64_t)b.w << 32) | b.z);
         c = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a0, b0, c, 0, 0, 0);
         c = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a1, b1, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ void mma_acc(const u32x4& a, const u32x4& b, f32x4& c) {
+        const u32x2 a0 = {a.x, a.y}, a1 = {a.z, a.w}, b0 = {b.x, b.y}, b1 = {b.z, b.w};
+        asm volatile("v_mfma_f32_16x16x32_fp8_fp8 %0, %1, %2, %0" : "+a"(c) : "v"(a0), "v"(b0));
+        asm volatile("v_mfma_f32_16x16x32_fp8_fp8 %0, %1, %2, %0" : "+a"(c) : "v"(a1), "v"(b1));
     }
 };
 
@@ -79,7 +92,7 @@ __device__ __forceinline__ int swz(int row) {
 __device__ __forceinline__ void tile_of_block(const GemmArgs& p, int* tm, int* tn) {
     int bid = blockIdx.x;
     const int n = gridDim.x;
-    if (p.xcd_swizzle && (n % 8) == 0) bid = (bid % 8) * (n / 8) + bid / 8;
+    if ((p.xcd_swizzle & 1) && (n % 8) == 0) bid = (bid % 8) * (n / 8) + bid / 8;
     constexpr int kGroup = 8;
     const int per_group = kGroup * p.tiles_n;
     const int g = bid / per_group;

@@ -24,6 +24,7 @@ SOURCES = {
     "gemm_mfma256.hip": [],
     "gemm_universal.hip": ["-ffp-contract=off"],   # UniversalFMA: mul then add, never fused
     "layout_host.cpp": ["-x", "hip"],
+    "tiled_host.cpp": ["-x", "hip"],
 }
 
 

@@ -205,6 +205,14 @@ static int32_t launch_out(int32_t out_dt, const GemmArgs& a, hipStream_t st) {
 int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int bk_elems, int waves, int stages,
                               GemmArgs a, hipStream_t st) {
     const int eb = dtype_bytes(in_dt);
+    if (bm == 0 && bn == 0) {
+        // the library chooses: one 256x256 tile per CU when that fills the chip, else 128x128
+        const bool big = a.M % 256 == 0 && a.N % 256 == 0 && a.K % (128 / eb) == 0 &&
+                         (int64_t)(a.M / 256) * (a.N / 256) >= 128;
+        bm = bn = big ? 256 : 128;
+        if (bk_elems == 0) bk_elems = big || a.K % (128 / eb) == 0 ? 128 / eb : 64 / eb;
+        if (big && waves <= 1) waves = 8;
+    }
     if (bm == 0) bm = 128;
     if (bn == 0) bn = 128;
     if (bk_elems == 0) bk_elems = 64 / eb;  // 64 bytes of K per row: 32 halves / 64 fp8

@@ -20,6 +20,13 @@ sys.path.insert(0, os.path.join(ROOT, "moye.jl_amd"))
 
 PEAK_F16_TFLOPS = 2500.0   # MI355X dense fp16/bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+# Bytes that leave the L2s per launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script
+# (the summaries are committed under profiles/), each reading scaled by what the same counter shows for the
+# 1 GiB plain copy (fetch x2.0000, write x1.0000).  Only valid for the default tile/waves/flags.
+MEASURED_TRAFFIC = {
+    "gemm_f16_4096_tile256": {"read_bytes": 197454 * 1024, "write_bytes": 33279 * 1024},
+    "transpose_f32_16384": {"read_bytes": 1048610 * 1024, "write_bytes": 1049814 * 1024},
+}
 
 
 def cpu_baseline(cores):
@@ -109,6 +116,9 @@ def main():
     if not err <= 1e-2:
         sys.exit("bench.py: result check failed, rel err %.3e" % err)
 
+    default_cfg = (bm, bn, bk, wm, wn, args.stages, args.flags) == (256, 256, 64, 2, 4, 0, 0)
+    t = MEASURED_TRAFFIC["gemm_f16_4096_tile256"]
+    gemm_traffic = t["read_bytes"] + t["write_bytes"] if default_cfg else None
     out = {
         "metric": "GEMM TFLOP/s (fp16 4096^3) + % MFMA peak; tiled-copy GB/s + % HBM peak",
         "value": round(value, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -118,7 +128,7 @@ def main():
                                "fp16 out; CTA tile %dx%dx%d, %dx%d waves of v_mfma_f32_16x16x32_f16" % (bm, bn, bk, wm, wn),
                    "rel_err_vs_fp64": err},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_F16_TFLOPS, 4), "traffic": None,
+                     "frac": round(achieved / PEAK_F16_TFLOPS, 4), "traffic": gemm_traffic,
                      "kernel_ms": round(kern_ms, 5)},
     }
 
@@ -138,7 +148,8 @@ def main():
             "metric": "tiled-copy GB/s", "value": round(gbs, 1), "unit": "GB/s",
             "config": {"workload": "16384x16384 fp32 column-major -> row-major through 64x64 LDS tiles", "bit_exact_sample": ok},
             "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                         "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None, "kernel_ms": round(cms, 5)},
+                         "frac": round(gbs / PEAK_HBM_GBS, 4),
+                         "traffic": sum(MEASURED_TRAFFIC["transpose_f32_16384"].values()), "kernel_ms": round(cms, 5)},
             "plain_copy_gbs": round(nbytes / (pms * 1e-3) / 1e9, 1),
         }
         del src, dst

@@ -247,3 +247,118 @@ def test_gemm_errors(mh):
     with pytest.raises(mh.MoyeError) as e:  # rank
         mh.gemm_(mma, T(d), T(a, (128, 8, 8), (64, 8, 1)), T(b))
     assert e.value.status == E.ERR_RANK
+
+
+# ---------------------------------------------------------------------------------------------
+# 256 x 256 CTA tile schedules (one workgroup per CU)
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("waves,stages", [((2, 4, 1), 0), ((2, 2, 1), 0), ((2, 4, 1), 4), ((2, 4, 1), 5)])
+def test_f16_tn_256_tile_exact_on_integers(mh, waves, stages):
+    """Every 256x256 schedule (8 waves, 4 waves, 4- and 5-stage ring) on small-integer inputs:
+    all sums are exact in fp32, so the result must equal the integer product exactly."""
+    M, N, K = 512, 768, 320
+    g = torch.Generator().manual_seed(12)
+    A = torch.randint(-4, 5, (M, K), generator=g).to(torch.float16)
+    B = torch.randint(-4, 5, (N, K), generator=g).to(torch.float16)
+    a, b = A.cuda(), B.cuda()
+    bk = 32 if stages >= 3 else 64
+    for out_dt in (torch.float32, torch.float16):
+        d = torch.zeros(M, N, dtype=out_dt, device="cuda")
+        mma = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=waves, cta_tile=(256, 256, bk), stages=stages)
+        mh.gemm_(mma, T(d), T(a), T(b))
+        torch.cuda.synchronize()
+        assert torch.equal(d.cpu().double(), A.double() @ B.double().t()), (waves, stages, out_dt)
+
+
+@pytest.mark.parametrize("tdt,atom", [("float16", "MFMA_F32_16x16x32_F16"), ("bfloat16", "MFMA_F32_16x16x32_BF16")])
+def test_256_tile_variants(mh, tdt, atom):
+    """column-major D, C accumulation and alpha through the 256x256 kernel; one k-tile and many."""
+    tdt = getattr(torch, tdt)
+    for K in (64, 1024):
+        for kw in (dict(), dict(col_major_d=True), dict(with_c=True, alpha=0.5)):
+            got, c64, _, _ = _mfma_case(mh, getattr(mh, atom), tdt, torch.float32, 512, 256, K, 21, K ** -0.5,
+                                        cta=(256, 256, 64), **kw)
+            assert relerr(got, c64) <= TOL16, (K, kw)
+
+
+def test_library_picks_the_tile(mh):
+    """cta_tile = (0,0,0): the library chooses; the result must not depend on the choice."""
+    for (M, N, K) in ((4096, 2048, 512), (384, 128, 96)):
+        got, c64, _, _ = _mfma_case(mh, mh.MFMA_F32_16x16x32_F16, torch.float16, torch.float16, M, N, K, 5, K ** -0.5,
+                                    cta=(0, 0, 0))
+        assert relerr(got, c64) <= TOL16
+
+
+def test_config4_bf16_8192(mh):
+    """BASELINE config 4 (square) at full size: bf16 8192^3, fp32 accumulate and output."""
+    M = N = K = 8192
+    got, c64, A, B = _mfma_case(mh, mh.MFMA_F32_16x16x32_BF16, torch.bfloat16, torch.float32, M, N, K, 1004, 0.02,
+                                cta=(256, 256, 64))
+    err = relerr(got, c64)
+    rows = np.random.default_rng(1).choice(M, 16, replace=False)
+    ref = to.gemm_universal_fma(A[rows].float().numpy(), B.float().numpy(), np.zeros((16, N), np.float32), "bf16", "bf16")
+    ref_err = to.relerr(ref, c64[rows].cpu().numpy())
+    print("config4 bf16 8192^3: rel err %.3e (reference arithmetic on 16 rows: %.3e)" % (err, ref_err))
+    assert err <= TOL16
+
+
+def test_config5_fp8_8192(mh):
+    """BASELINE config 5 at full size: e4m3 8192^3, per-tensor scales, bf16 out."""
+    if not hasattr(torch, "float8_e4m3fn"):
+        pytest.skip("torch without float8_e4m3fn")
+    M = N = K = 8192
+    g = torch.Generator(device="cuda").manual_seed(1005)
+    X = torch.randn(M, K, generator=g, device="cuda")
+    W = torch.randn(N, K, generator=g, device="cuda")
+    sa, sb = float(X.abs().max() / 448), float(W.abs().max() / 448)
+    a, b = (X / sa).to(torch.float8_e4m3fn), (W / sb).to(torch.float8_e4m3fn)
+    del X, W
+    d = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
+    mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_FP8, atom_layout=(2, 4, 1), cta_tile=(256, 256, 128)), T(d), T(a),
+             T(b), None, sa * sb)
+    torch.cuda.synchronize()
+    rows = torch.randperm(M, device="cuda")[:512]
+    c64 = (a[rows].float().double() @ b.float().double().t()) * (sa * sb)
+    err = relerr(d[rows], c64)
+    print("config5 fp8 8192^3 (512 sampled rows): rel err vs fp64 of the quantised inputs %.3e" % err)
+    assert err <= TOL16
+
+
+def test_moye_array_api_on_device(mh):
+    """The MoYe-level calls: MoYeArray views, @tile, make_tiled_mma, gemm!, copyto! on device arrays."""
+    from moye_hip import layout as ml
+    g = torch.Generator().manual_seed(2)
+    M, N, K = 512, 256, 128
+    A = (torch.randn(M, K, generator=g) / 8).half().cuda()
+    B = (torch.randn(N, K, generator=g) / 8).half().cuda()
+    Dt = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+    mA = mh.MoYeArray.from_torch(A)          # (M,K):(K,1)
+    mB = mh.MoYeArray.from_torch(B)          # (N,K):(K,1)
+    mD = mh.MoYeArray.from_torch(Dt)
+    S = ml.StaticInt
+    mma = mh.make_tiled_mma(mh.MFMA_F32_16x16x32_F16, ml.static_layout((2, 2, 1)), (S(128), S(128), S(32)))
+    assert [int(v) for v in mma.tile_shape()] == [128, 128, 32] and mma.size() == 256
+    mh.gemm_(mma, mD, mA, mB)
+    torch.cuda.synchronize()
+    c64 = A.double() @ B.double().t()
+    assert relerr(Dt, c64) <= TOL16
+    # gemm! on one CTA tile of the problem, selected with @tile as the reference's kernels do
+    Dt2 = torch.zeros_like(Dt)
+    mD2 = mh.MoYeArray.from_torch(Dt2)
+    gA = mh.local_tile(mA, (S(128), S(K)), (2, 1))
+    gB = mh.local_tile(mB, (S(128), S(K)), (1, 1))
+    gD = mh.local_tile(mD2, (S(128), S(128)), (2, 1))
+    mh.gemm_(mma, gD, gA, gB)
+    torch.cuda.synchronize()
+    assert torch.equal(Dt2[128:256, :128], Dt[128:256, :128]) and float(Dt2[:128].abs().max()) == 0.0
+    # copyto! with a tiled copy: transposed destination
+    src = torch.randint(-2 ** 31, 2 ** 31 - 1, (256 * 192,), dtype=torch.int32, device="cuda")
+    dst = torch.zeros_like(src)
+    ms = mh.MoYeArray.from_torch(src, ml.Layout((256, 192), (1, 256)))
+    md = mh.MoYeArray.from_torch(dst, ml.Layout((256, 192), (192, 1)))
+    tc = mh.make_tiled_copy(mh.CopyAtom(128, 32), ml.static_layout((16, 16)), ml.static_layout((4, 4)),
+                            op=mh.COPY_LDS_TILED)
+    mh.copyto_(md, ms, tc)
+    torch.cuda.synchronize()
+    assert torch.equal(dst.view(256, 192), src.view(192, 256).t())

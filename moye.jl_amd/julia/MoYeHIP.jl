@@ -1,0 +1,397 @@
+# MoYeHIP.jl — `ccall` glue that routes MoYe's device verbs to libmoye_hip.so on AMD gfx950.
+#
+# This file is the reference-side binding of include/moye_hip.h.  It is written against MoYe.jl
+# v4.0.1's own types and adds methods to its generic functions, so user code keeps calling
+# `copyto!`, `gemm!`, `make_tiled_mma`, `@tile`, ... unchanged.  It has not been executed in this
+# repository's build environment (no Julia runtime there); the ABI it binds is exercised by the
+# ctypes mirror under moye_hip/, which declares the same signatures.
+#
+# Usage:
+#   ENV["MOYE_HIP_LIB"] = "/path/to/libmoye_hip.so"
+#   using MoYe; include("MoYeHIP.jl"); using .MoYeHIP
+#   A = MoYeHIP.device_array(Float16, @Layout((4096,4096), GenRowMajor))  # (M,K), K contiguous
+#   mma = MoYeHIP.make_tiled_mma(MoYeHIP.MFMA_F32_16x16x32_F16, @Layout((2,4,1)), (_256,_256,_64))
+#   MoYeHIP.gemm!(mma, D, A, B)            # D = A * B'   on the GPU
+module MoYeHIP
+
+using MoYe
+using MoYe: MoYeArray, Layout, StaticInt, static, shape, stride, flatten, rank
+
+const LIB = get(ENV, "MOYE_HIP_LIB", "libmoye_hip.so")
+const CAP = 1 << 16            # text buffer for layouts coming back
+
+# ---- status -----------------------------------------------------------------------------------
+struct MoYeHIPError <: Exception
+    status::Int32
+    msg::String
+end
+Base.showerror(io::IO, e::MoYeHIPError) = print(io, "MoYeHIP status ", e.status, ": ", e.msg)
+
+last_error() = unsafe_string(ccall((:moye_last_error, LIB), Cstring, ()))
+version() = unsafe_string(ccall((:moye_version, LIB), Cstring, ()))
+
+# The library's status codes stand for the reference's exception classes.
+function check(st::Int32)
+    st == 0 && return nothing
+    msg = last_error()
+    st == 1 && throw(DimensionMismatch(msg))        # MOYE_ERR_RANK
+    st == 2 && throw(DimensionMismatch(msg))        # MOYE_ERR_SHAPE (failed shape_div assert)
+    st == 3 && throw(ArgumentError(msg))            # MOYE_ERR_UNSUPPORTED (no method)
+    st == 6 && throw(ArgumentError(msg))            # MOYE_ERR_ARG
+    throw(MoYeHIPError(st, msg))
+end
+
+# ---- descriptors (mirror the C structs field for field) ---------------------------------------
+struct Tensor                     # moye_tensor
+    ptr::Ptr{Cvoid}
+    dtype::Int32
+    memspace::Int32
+    rank::Int32
+    _pad::Int32
+    shape::NTuple{8,Int64}
+    stride::NTuple{8,Int64}
+end
+
+struct TiledMMADesc               # moye_tiled_mma
+    atom::Int32
+    atom_layout_mnk::NTuple{3,Int32}
+    tile_mnk::NTuple{3,Int32}
+    cta_tile_mnk::NTuple{3,Int32}
+    stages::Int32
+    split_k::Int32
+    flags::Int32
+end
+
+struct TiledCopyDesc              # moye_tiled_copy
+    op::Int32
+    vec_bits::Int32
+    thr_shape::NTuple{2,Int32}
+    val_shape::NTuple{2,Int32}
+    tiler_mn::NTuple{2,Int32}
+    flags::Int32
+end
+
+const UNIVERSAL_FMA = Int32(0)
+const MFMA_F32_16x16x32_F16 = Int32(1)
+const MFMA_F32_32x32x16_F16 = Int32(2)
+const MFMA_F32_16x16x32_BF16 = Int32(3)
+const MFMA_F32_32x32x16_BF16 = Int32(4)
+const MFMA_F32_16x16x32_FP8 = Int32(5)
+const MFMA_F32_32x32x16_FP8 = Int32(6)
+const MFMA_F32_16x16x4_F32 = Int32(7)
+const MFMA_F32_32x32x2_F32 = Int32(8)
+const COPY_UNIVERSAL = Int32(0)
+const COPY_LDS_TILED = Int32(1)
+
+dtype_code(::Type{Float32}) = Int32(0)
+dtype_code(::Type{Float16}) = Int32(1)
+dtype_code(::Type{Float64}) = Int32(4)
+dtype_code(::Type{UInt8}) = Int32(5)
+dtype_code(::Type{UInt16}) = Int32(6)
+dtype_code(::Type{UInt32}) = Int32(7)
+dtype_code(::Type{Int32}) = Int32(7)
+dtype_code(::Type{UInt64}) = Int32(8)
+dtype_code(::Type{UInt128}) = Int32(9)
+dtype_code(::Type{T}) where {T} =
+    nameof(T) === :BFloat16 ? Int32(2) : throw(ArgumentError("MoYeHIP: no dtype code for $T"))
+
+pad8(t, fill) = ntuple(i -> i <= length(t) ? Int64(t[i]) : Int64(fill), 8)
+
+"Flatten a device MoYeArray into the descriptor the library consumes (borrowed pointer)."
+function Tensor(x::MoYeArray{T}) where {T}
+    l = flatten(MoYe.layout(x))
+    r = rank(l)
+    r <= 8 || throw(DimensionMismatch("MoYeHIP: more than 8 flattened modes"))
+    Tensor(Ptr{Cvoid}(UInt(pointer(x))), dtype_code(T), Int32(0), Int32(r), Int32(0),
+           pad8(shape(l), 1), pad8(stride(l), 0))
+end
+
+# ---- host-side layout algebra through the library -------------------------------------------
+# Layouts cross the boundary in MoYe's own printed form; `string(layout)` is already that form.
+# The results are parsed back with MoYe's constructors by `parse_layout` below.
+
+function parse_int_tuple(s::AbstractString)
+    s = strip(s)
+    if startswith(s, "(")
+        depth = 0; parts = String[]; start = 2
+        for (i, c) in pairs(s)
+            c == '(' && (depth += 1)
+            c == ')' && (depth -= 1)
+            if (c == ',' && depth == 1) || (c == ')' && depth == 0)
+                piece = strip(s[start:prevind(s, i)])
+                isempty(piece) || push!(parts, piece)
+                start = nextind(s, i)
+            end
+        end
+        return Tuple(parse_int_tuple(p) for p in parts)
+    elseif startswith(s, "_")
+        return static(parse(Int, s[2:end]))
+    else
+        return parse(Int, s)
+    end
+end
+
+function parse_layout(s::AbstractString)
+    depth = 0
+    for (i, c) in pairs(s)
+        c == '(' && (depth += 1)
+        c == ')' && (depth -= 1)
+        if c == ':' && depth == 0
+            return MoYe.make_layout(parse_int_tuple(s[1:prevind(s, i)]), parse_int_tuple(s[nextind(s, i):end]))
+        end
+    end
+    MoYe.make_layout(parse_int_tuple(s))
+end
+
+tile_text(t::Tuple) = "<" * join((x isa Layout ? string(x) : x isa Colon ? ":" : string(x) for x in t), ", ") * ">"
+tile_text(x) = string(x)
+
+macro layout_call(sym, args...)
+    quote
+        buf = Vector{UInt8}(undef, CAP)
+        check(ccall(($(QuoteNode(sym)), LIB), Int32, ($(map(_ -> :Cstring, args)...), Ptr{UInt8}, Csize_t),
+                    $(map(esc, args)...), buf, CAP))
+        parse_layout(unsafe_string(pointer(buf)))
+    end
+end
+
+coalesce(l::Layout) = @layout_call moye_layout_coalesce string(l)
+filter(l::Layout) = @layout_call moye_layout_filter string(l)
+flatten_layout(l::Layout) = @layout_call moye_layout_flatten string(l)
+composition(a::Layout, b) = @layout_call moye_layout_composition string(a) tile_text(b)
+complement(l::Layout, cotarget = "") = @layout_call moye_layout_complement string(l) string(cotarget)
+right_inverse(l::Layout) = @layout_call moye_layout_right_inverse string(l)
+left_inverse(l::Layout) = @layout_call moye_layout_left_inverse string(l)
+logical_product(l::Layout, t) = @layout_call moye_layout_logical_product string(l) tile_text(t)
+zipped_product(l::Layout, t) = @layout_call moye_layout_zipped_product string(l) tile_text(t)
+tiled_product(l::Layout, t) = @layout_call moye_layout_tiled_product string(l) tile_text(t)
+logical_divide(l::Layout, t) = @layout_call moye_layout_logical_divide string(l) tile_text(t)
+zipped_divide(l::Layout, t) = @layout_call moye_layout_zipped_divide string(l) tile_text(t)
+tiled_divide(l::Layout, t) = @layout_call moye_layout_tiled_divide string(l) tile_text(t)
+make_fragment_like(l::Layout) = @layout_call moye_layout_make_fragment_like string(l)
+normalize(l::Layout) = @layout_call moye_layout_normalize string(l)
+
+function blocked_product(block::Layout, l::Layout, coalesce_result::Bool = false)
+    buf = Vector{UInt8}(undef, CAP)
+    check(ccall((:moye_layout_blocked_product, LIB), Int32, (Cstring, Cstring, Int32, Ptr{UInt8}, Csize_t),
+                string(block), string(l), Int32(coalesce_result), buf, CAP))
+    parse_layout(unsafe_string(pointer(buf)))
+end
+
+function raked_product(block::Layout, l::Layout, coalesce_result::Bool = false)
+    buf = Vector{UInt8}(undef, CAP)
+    check(ccall((:moye_layout_raked_product, LIB), Int32, (Cstring, Cstring, Int32, Ptr{UInt8}, Csize_t),
+                string(block), string(l), Int32(coalesce_result), buf, CAP))
+    parse_layout(unsafe_string(pointer(buf)))
+end
+
+function recast(l::Layout, ::Type{New}, ::Type{Old}) where {New,Old}
+    buf = Vector{UInt8}(undef, CAP)
+    check(ccall((:moye_layout_recast, LIB), Int32, (Cstring, Int32, Int32, Ptr{UInt8}, Csize_t),
+                string(l), Int32(sizeof(New)), Int32(sizeof(Old)), buf, CAP))
+    parse_layout(unsafe_string(pointer(buf)))
+end
+
+function layout_index(l::Layout, coord)
+    idx = Ref{Int64}(0)
+    check(ccall((:moye_layout_eval, LIB), Int32, (Cstring, Cstring, Ptr{Int64}), string(l), string(coord), idx))
+    idx[]
+end
+
+function layout_size(l::Layout)
+    n = Ref{Int64}(0)
+    check(ccall((:moye_layout_size, LIB), Int32, (Cstring, Ptr{Int64}), string(l), n)); n[]
+end
+
+function layout_cosize(l::Layout)
+    n = Ref{Int64}(0)
+    check(ccall((:moye_layout_cosize, LIB), Int32, (Cstring, Ptr{Int64}), string(l), n)); n[]
+end
+
+function max_common_vector(a::Layout, b::Layout)
+    n = Ref{Int64}(0)
+    check(ccall((:moye_layout_max_common_vector, LIB), Int32, (Cstring, Cstring, Ptr{Int64}), string(a), string(b), n))
+    n[]
+end
+
+function tuple_op(op::AbstractString, a, b = "", c = "")
+    buf = Vector{UInt8}(undef, CAP)
+    check(ccall((:moye_tuple_op, LIB), Int32, (Cstring, Cstring, Cstring, Cstring, Ptr{UInt8}, Csize_t),
+                op, string(a), string(b), string(c), buf, CAP))
+    unsafe_string(pointer(buf))
+end
+
+"`@tile x tile coord` on a device array: the sub-array's layout and pointer, computed by the library."
+function local_tile(x::MoYeArray{T}, tile::Tuple, coord::Tuple, proj = "") where {T}
+    buf = Vector{UInt8}(undef, CAP); off = Ref{Int64}(0)
+    check(ccall((:moye_local_tile, LIB), Int32, (Cstring, Cstring, Cstring, Cstring, Ptr{UInt8}, Csize_t, Ptr{Int64}),
+                string(MoYe.layout(x)), tile_text(tile), tile_text(coord), string(proj), buf, CAP, off))
+    MoYeArray(pointer(x) + off[] * sizeof(T), parse_layout(unsafe_string(pointer(buf))))
+end
+
+"`@parallelize x thr_layout thr_idx` on a device array."
+function local_partition(x::MoYeArray{T}, thr::Layout, idx::Integer, proj = "") where {T}
+    buf = Vector{UInt8}(undef, CAP); off = Ref{Int64}(0)
+    check(ccall((:moye_local_partition, LIB), Int32,
+                (Cstring, Cstring, Cstring, Cstring, Ptr{UInt8}, Csize_t, Ptr{Int64}),
+                string(MoYe.layout(x)), string(thr), string(idx), string(proj), buf, CAP, off))
+    MoYeArray(pointer(x) + off[] * sizeof(T), parse_layout(unsafe_string(pointer(buf))))
+end
+
+# ---- TiledMMA / TiledCopy ---------------------------------------------------------------------
+"make_tiled_mma(op, atom_layout, permutation) for the gfx950 atoms; returns the POD descriptor."
+function make_tiled_mma(atom::Int32, atom_layout::Layout, permutation::Tuple = ())
+    d = Ref{TiledMMADesc}()
+    check(ccall((:moye_make_tiled_mma, LIB), Int32, (Int32, Cstring, Cstring, Ptr{TiledMMADesc}),
+                atom, string(atom_layout), isempty(permutation) ? "" : tile_text(permutation), d))
+    d[]
+end
+
+function tiled_mma_query(atom::AbstractString, atom_layout::Layout, permutation, what::AbstractString)
+    buf = Vector{UInt8}(undef, CAP)
+    check(ccall((:moye_tiled_mma_query, LIB), Int32, (Cstring, Cstring, Cstring, Cstring, Ptr{UInt8}, Csize_t),
+                atom, string(atom_layout), permutation === nothing ? "" : tile_text(permutation), what, buf, CAP))
+    unsafe_string(pointer(buf))
+end
+
+"partition_A/B/C(get_slice(mma, thr_idx), x) computed by the library (operand = 'A', 'B' or 'C')."
+function tiled_mma_partition(atom::AbstractString, atom_layout::Layout, permutation, thr_idx::Integer,
+                             operand::Char, x::MoYeArray{T}) where {T}
+    buf = Vector{UInt8}(undef, CAP); off = Ref{Int64}(0)
+    check(ccall((:moye_tiled_mma_partition, LIB), Int32,
+                (Cstring, Cstring, Cstring, Int32, Cchar, Cstring, Ptr{UInt8}, Csize_t, Ptr{Int64}),
+                atom, string(atom_layout), permutation === nothing ? "" : tile_text(permutation), Int32(thr_idx),
+                Cchar(operand), string(MoYe.layout(x)), buf, CAP, off))
+    MoYeArray(pointer(x) + off[] * sizeof(T), parse_layout(unsafe_string(pointer(buf))))
+end
+
+function tiled_copy_query(src_bits, dst_bits, val_bits, thr::Layout, val::Layout, what::AbstractString)
+    buf = Vector{UInt8}(undef, CAP)
+    check(ccall((:moye_tiled_copy_query, LIB), Int32,
+                (Int32, Int32, Int32, Cstring, Cstring, Cstring, Ptr{UInt8}, Csize_t),
+                Int32(src_bits), Int32(dst_bits), Int32(val_bits), string(thr), string(val), what, buf, CAP))
+    unsafe_string(pointer(buf))
+end
+
+function tiled_copy_partition(src_bits, dst_bits, val_bits, thr::Layout, val::Layout, thr_idx::Integer,
+                              which::Char, x::MoYeArray{T}) where {T}
+    buf = Vector{UInt8}(undef, CAP); off = Ref{Int64}(0)
+    check(ccall((:moye_tiled_copy_partition, LIB), Int32,
+                (Int32, Int32, Int32, Cstring, Cstring, Int32, Cchar, Cstring, Ptr{UInt8}, Csize_t, Ptr{Int64}),
+                Int32(src_bits), Int32(dst_bits), Int32(val_bits), string(thr), string(val), Int32(thr_idx),
+                Cchar(which), string(MoYe.layout(x)), buf, CAP, off))
+    MoYeArray(pointer(x) + off[] * sizeof(T), parse_layout(unsafe_string(pointer(buf))))
+end
+
+"A TiledCopy for the device copy: atom of `vec_bits` bits, thread and value layouts, LDS tile."
+function tiled_copy_desc(; op = COPY_UNIVERSAL, vec_bits = 128, thr = (16, 16), val = (4, 4), tiler = (64, 64))
+    TiledCopyDesc(op, Int32(vec_bits), Int32.(thr), Int32.(val), Int32.(tiler), Int32(0))
+end
+
+# ---- the device verbs -------------------------------------------------------------------------
+"""
+    copyto!(dst, src; tiled_copy=nothing, stream=C_NULL)
+
+`Base.copyto!(dest::MoYeArray, src::MoYeArray)` (src/algorithm/copy.jl:42-64) and
+`copyto!(tiled_copy, dst, src)` (:106-130) for device arrays.  Asynchronous on `stream`.
+"""
+function copyto!(dst::MoYeArray, src::MoYeArray; tiled_copy::Union{Nothing,TiledCopyDesc} = nothing,
+                 stream::Ptr{Cvoid} = C_NULL)
+    d, s = Ref(Tensor(dst)), Ref(Tensor(src))
+    GC.@preserve dst src begin
+        if tiled_copy === nothing
+            check(ccall((:moye_copy, LIB), Int32, (Ptr{Cvoid}, Ptr{Tensor}, Ptr{Tensor}, Ptr{Cvoid}), C_NULL, d, s, stream))
+        else
+            tc = Ref(tiled_copy)
+            check(ccall((:moye_copy, LIB), Int32, (Ptr{TiledCopyDesc}, Ptr{Tensor}, Ptr{Tensor}, Ptr{Cvoid}), tc, d, s, stream))
+        end
+    end
+    dst
+end
+
+"""
+    gemm!(mma, D, A, B[, C]; alpha=1f0, stream=C_NULL)
+
+`gemm!(mma, D, A, B, C)` (src/algorithm/blas.jl:11-17) over whole device operands:
+A:(M,K), B:(N,K), C,D:(M,N); D = alpha * A * B' + C.  Returns `nothing` like the reference.
+"""
+function gemm!(mma::TiledMMADesc, D::MoYeArray, A::MoYeArray, B::MoYeArray, C::Union{Nothing,MoYeArray} = nothing;
+               alpha::Real = 1.0f0, stream::Ptr{Cvoid} = C_NULL)
+    m, d, a, b = Ref(mma), Ref(Tensor(D)), Ref(Tensor(A)), Ref(Tensor(B))
+    GC.@preserve D A B C begin
+        if C === nothing
+            check(ccall((:moye_gemm, LIB), Int32,
+                        (Ptr{TiledMMADesc}, Ptr{Tensor}, Ptr{Tensor}, Ptr{Tensor}, Ptr{Cvoid}, Cfloat, Ptr{Cvoid}),
+                        m, d, a, b, C_NULL, Float32(alpha), stream))
+        else
+            c = Ref(Tensor(C))
+            check(ccall((:moye_gemm, LIB), Int32,
+                        (Ptr{TiledMMADesc}, Ptr{Tensor}, Ptr{Tensor}, Ptr{Tensor}, Ptr{Tensor}, Cfloat, Ptr{Cvoid}),
+                        m, d, a, b, c, Float32(alpha), stream))
+        end
+    end
+    nothing
+end
+
+function gemm_workspace_size(mma::TiledMMADesc, D::MoYeArray, A::MoYeArray, B::MoYeArray)
+    n = Ref{Csize_t}(0)
+    check(ccall((:moye_gemm_workspace_size, LIB), Int32,
+                (Ptr{TiledMMADesc}, Ptr{Tensor}, Ptr{Tensor}, Ptr{Tensor}, Ptr{Csize_t}),
+                Ref(mma), Ref(Tensor(D)), Ref(Tensor(A)), Ref(Tensor(B)), n))
+    Int(n[])
+end
+
+# ---- device memory without a Julia GPU package ------------------------------------------------
+function device_malloc(bytes::Integer)
+    p = Ref{Ptr{Cvoid}}(C_NULL)
+    check(ccall((:moye_device_malloc, LIB), Int32, (Ptr{Ptr{Cvoid}}, Csize_t), p, bytes)); p[]
+end
+device_free(p::Ptr{Cvoid}) = check(ccall((:moye_device_free, LIB), Int32, (Ptr{Cvoid},), p))
+device_sync() = check(ccall((:moye_device_sync, LIB), Int32, ()))
+memset(p::Ptr{Cvoid}, v::Integer, bytes::Integer) =
+    check(ccall((:moye_memset, LIB), Int32, (Ptr{Cvoid}, Cint, Csize_t), p, v, bytes))
+
+"A device MoYeArray of element type T with the given layout (caller frees with `device_free(pointer(x))`)."
+function device_array(::Type{T}, l::Layout) where {T}
+    p = device_malloc(layout_cosize(l) * sizeof(T))
+    MoYeArray(Ptr{T}(p), l)
+end
+
+function upload!(dst::MoYeArray{T}, host::Array{T}) where {T}
+    GC.@preserve host check(ccall((:moye_memcpy_h2d, LIB), Int32, (Ptr{Cvoid}, Ptr{Cvoid}, Csize_t),
+                                  Ptr{Cvoid}(UInt(pointer(dst))), pointer(host), sizeof(host)))
+    dst
+end
+
+function download!(host::Array{T}, src::MoYeArray{T}) where {T}
+    GC.@preserve host check(ccall((:moye_memcpy_d2h, LIB), Int32, (Ptr{Cvoid}, Ptr{Cvoid}, Csize_t),
+                                  pointer(host), Ptr{Cvoid}(UInt(pointer(src))), sizeof(host)))
+    host
+end
+
+function device_info()
+    name = Vector{UInt8}(undef, 256); cu = Ref{Int32}(0); khz = Ref{Int32}(0); mem = Ref{Csize_t}(0)
+    check(ccall((:moye_device_info, LIB), Int32, (Ptr{UInt8}, Csize_t, Ptr{Int32}, Ptr{Int32}, Ptr{Csize_t}),
+                name, 256, cu, khz, mem))
+    (name = unsafe_string(pointer(name)), compute_units = cu[], clock_khz = khz[], total_mem = Int(mem[]))
+end
+
+"Average milliseconds per launch of the same gemm! call, HIP events on `stream`."
+function time_gemm(mma::TiledMMADesc, D, A, B; alpha = 1.0f0, stream = C_NULL, warmup = 3, iters = 20)
+    ms = Ref{Cfloat}(0)
+    check(ccall((:moye_time_gemm, LIB), Int32,
+                (Ptr{TiledMMADesc}, Ptr{Tensor}, Ptr{Tensor}, Ptr{Tensor}, Ptr{Cvoid}, Cfloat, Ptr{Cvoid}, Int32, Int32, Ptr{Cfloat}),
+                Ref(mma), Ref(Tensor(D)), Ref(Tensor(A)), Ref(Tensor(B)), C_NULL, Float32(alpha), stream,
+                Int32(warmup), Int32(iters), ms))
+    ms[]
+end
+
+function time_copy(dst, src; tiled_copy = tiled_copy_desc(), stream = C_NULL, warmup = 3, iters = 20)
+    ms = Ref{Cfloat}(0)
+    check(ccall((:moye_time_copy, LIB), Int32,
+                (Ptr{TiledCopyDesc}, Ptr{Tensor}, Ptr{Tensor}, Ptr{Cvoid}, Int32, Int32, Ptr{Cfloat}),
+                Ref(tiled_copy), Ref(Tensor(dst)), Ref(Tensor(src)), stream, Int32(warmup), Int32(iters), ms))
+    ms[]
+end
+
+end # module

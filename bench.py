@@ -59,6 +59,72 @@ def cpu_baseline(cores):
                       "(32x32x8 tiles, OpenMP over C tiles), %.1f s" % (n, dt)}
 
 
+def other_configs(mh, tensor_of, torch, stream):
+    """The remaining GEMM workloads of the baseline: bf16 8192^3 (fp32 out), fp8 e4m3 8192^3 with per-tensor
+    scales (bf16 out), and the HBM-bound short-M case bf16 16 x 8192 x 8192.  Kernel time by HIP events."""
+    res = []
+    n = 8192
+    g = torch.Generator(device="cuda").manual_seed(1004)
+
+    def run(name, atom, a, b, d, alpha, peak, cta, waves):
+        mma = mh.tiled_mma_desc(atom, atom_layout=waves, cta_tile=cta)
+        ms = mh.time_gemm(mma, tensor_of(d), tensor_of(a), tensor_of(b), None, alpha, stream, warmup=3, iters=20)
+        M, N, K = a.shape[0], b.shape[0], a.shape[1]
+        rows = torch.arange(0, M, max(1, M // 16), device="cuda")
+        c64 = alpha * (a[rows].float().double() @ b.float().double().t())
+        err = float((d[rows].double() - c64).abs().max() / c64.abs().max())
+        flops = 2.0 * M * N * K
+        entry = {"workload": name, "kernel_ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 1), "rel_err_vs_fp64": err}
+        if peak:
+            entry["roofline"] = {"bound": "mfma", "achieved": entry["tflops"], "peak": peak, "unit": "TFLOP/s",
+                                 "frac": round(entry["tflops"] / peak, 4)}
+        else:
+            nbytes = a.numel() * a.element_size() + b.numel() * b.element_size() + d.numel() * d.element_size()
+            gbs = nbytes / ms / 1e6
+            entry["roofline"] = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                 "frac": round(gbs / PEAK_HBM_GBS, 4), "algorithmic_bytes": nbytes}
+        res.append(entry)
+
+    a = (torch.randn(n, n, generator=g, device="cuda") * 0.02).bfloat16()
+    b = (torch.randn(n, n, generator=g, device="cuda") * 0.02).bfloat16()
+    d = torch.zeros(n, n, dtype=torch.float32, device="cuda")
+    run("bf16 TN 8192^3, fp32 out, CTA 256x256x64", mh.MFMA_F32_16x16x32_BF16, a, b, d, 1.0, PEAK_F16_TFLOPS, (256, 256, 64), (2, 4, 1))
+    # short M: rotate over 3 copies of B so that the 256 MiB Infinity Cache cannot serve the stream
+    a16 = a[:16].contiguous()
+    d16 = torch.zeros(16, n, dtype=torch.float32, device="cuda")
+    bs = [b, b.clone(), b.clone()]
+    mma = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_BF16, cta_tile=(0, 0, 0))
+    tA, tD, tBs = tensor_of(a16), tensor_of(d16), [tensor_of(x) for x in bs]
+    for i in range(3):
+        mh.gemm_(mma, tD, tA, tBs[i], None, 1.0, stream)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    iters = 30
+    for i in range(iters):
+        mh.gemm_(mma, tD, tA, tBs[i % 3], None, 1.0, stream)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / iters
+    nbytes = 16 * n * 2 + n * n * 2 + 16 * n * 4
+    c64 = a16.float().double() @ b.float().double().t()
+    res.append({"workload": "bf16 TN 16x8192x8192, fp32 out (short-M kernel, B rotated over 3 buffers)",
+                "kernel_ms": round(ms, 5), "tflops": round(2.0 * 16 * n * n / ms / 1e9, 1),
+                "rel_err_vs_fp64": float((d16.double() - c64).abs().max() / c64.abs().max()),
+                "roofline": {"bound": "hbm", "achieved": round(nbytes / ms / 1e6, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                             "frac": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4), "algorithmic_bytes": nbytes}})
+    del bs, a, b, d
+    if hasattr(torch, "float8_e4m3fn"):
+        x = torch.randn(n, n, generator=g, device="cuda")
+        w = torch.randn(n, n, generator=g, device="cuda")
+        sa, sb = float(x.abs().max() / 448), float(w.abs().max() / 448)
+        qa, qb = (x / sa).to(torch.float8_e4m3fn), (w / sb).to(torch.float8_e4m3fn)
+        del x, w
+        d = torch.zeros(n, n, dtype=torch.bfloat16, device="cuda")
+        run("fp8 e4m3 TN 8192^3, per-tensor scales, bf16 out, CTA 256x256x128", mh.MFMA_F32_16x16x32_FP8, qa, qb, d,
+            sa * sb, 5000.0, (256, 256, 128), (2, 4, 1))
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -66,6 +132,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-copy", action="store_true", help="skip the tiled-copy leg")
+    ap.add_argument("--no-other", action="store_true", help="skip the bf16 / fp8 / short-M GEMM legs")
     ap.add_argument("--tile", default="256,256,64", help="CTA tile bm,bn,bk of the GEMM kernel")
     ap.add_argument("--waves", default="2,4", help="waves per CTA along M,N (TiledMMA atom layout)")
     ap.add_argument("--stages", type=int, default=0, help="LDS pipeline depth (0 = kernel default)")
@@ -153,6 +220,9 @@ def main():
             "plain_copy_gbs": round(nbytes / (pms * 1e-3) / 1e9, 1),
         }
         del src, dst
+
+    if not args.no_other:
+        out["other_configs"] = other_configs(mh, tensor_of, torch, stream)
 
     if not args.no_cpu:
         cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else os.cpu_count()

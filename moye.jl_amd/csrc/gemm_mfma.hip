@@ -205,6 +205,9 @@ static int32_t launch_out(int32_t out_dt, const GemmArgs& a, hipStream_t st) {
 int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int bk_elems, int waves, int stages,
                               GemmArgs a, hipStream_t st) {
     const int eb = dtype_bytes(in_dt);
+    // a short A (at most 64 rows) is a bandwidth problem: stream B once, no CTA tiling
+    if ((bm == 0 && bn == 0 && a.M <= 64) || (bm == a.M && bm <= 64 && bn == 16))
+        return gemm_mfma_skinny_dispatch(in_dt, out_dt, a, st);
     if (bm == 0 && bn == 0) {
         // the library chooses: one 256x256 tile per CU when that fills the chip, else 128x128
         const bool big = a.M % 256 == 0 && a.N % 256 == 0 && a.K % (128 / eb) == 0 &&

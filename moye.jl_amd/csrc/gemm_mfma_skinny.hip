@@ -1,0 +1,115 @@
+// MFMA GEMM for a short A: M = 16, 32, 48 or 64 rows against a long B (N x K), K-major operands.
+// The work is streaming B from HBM once, so the kernel is laid out for bandwidth, not for the
+// matrix pipe: one workgroup owns 16 rows of B (16 output columns) and all of A; its waves split
+// K into contiguous ranges, each lane streams 16-byte pieces of its B row straight into the MFMA
+// operand registers (no LDS staging: nothing is reused inside a workgroup), and the per-wave
+// partial accumulators are summed through LDS in wave order, which makes the result independent
+// of timing.  A (at most 64 x K) is re-read by every workgroup and lives in L2.
+//
+// Stands where the reference's user kernel would run gemm! (src/algorithm/blas.jl:11-131) on a
+// 16-row problem with its usual 128 x 128 tiles and waste 7/8 of each tile.
+#include "mfma_common.hpp"
+
+namespace moye {
+
+template <typename In, typename Out, int MT, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void gemm_mfma_skinny(GemmArgs p) {
+    typedef typename Out::type OutT;
+    constexpr int U = 8;  // 64-byte k-steps in flight per wave and row
+    __shared__ f32x4 part[WAVES][MT][64];
+    const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, r16 = lane % 16, kq = lane / 16;
+    const int n0 = blockIdx.x * 16;
+    const int steps = (int)(((int64_t)p.K * In::kBytes) / 64);
+    const int s0 = (int)((int64_t)steps * wave / WAVES), s1 = (int)((int64_t)steps * (wave + 1) / WAVES);
+    const char* bp = static_cast<const char*>(p.B) + (int64_t)(n0 + r16) * p.ldb * In::kBytes + kq * 16;
+    const char* ap[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+        ap[i] = static_cast<const char*>(p.A) + (int64_t)(16 * i + r16) * p.lda * In::kBytes + kq * 16;
+    f32x4 acc[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    int s = s0;
+    for (; s + U <= s1; s += U) {
+        u32x4 b[U], a[MT][U];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            b[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(bp + (int64_t)(s + u) * 64));
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int u = 0; u < U; ++u) a[i][u] = *reinterpret_cast<const u32x4*>(ap[i] + (int64_t)(s + u) * 64);
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int i = 0; i < MT; ++i) In::mma(b[u], a[i][u], acc[i]);
+    }
+    for (; s < s1; ++s) {
+        const u32x4 b = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(bp + (int64_t)s * 64));
+#pragma unroll
+        for (int i = 0; i < MT; ++i) In::mma(b, *reinterpret_cast<const u32x4*>(ap[i] + (int64_t)s * 64), acc[i]);
+    }
+
+#pragma unroll
+    for (int i = 0; i < MT; ++i) part[wave][i][lane] = acc[i];
+    __syncthreads();
+    // lane l of tile i holds C[m = 16 i + l % 16][n = n0 + 4 (l / 16) + 0..3]
+    for (int unit = threadIdx.x; unit < MT * 64; unit += WAVES * 64) {
+        const int i = unit / 64, l = unit % 64;
+        f32x4 v = part[0][i][l];
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) v += part[w][i][l];
+        const int m = 16 * i + l % 16, n = n0 + 4 * (l / 16);
+        OutT* d = static_cast<OutT*>(p.D) + (int64_t)m * p.ldd + n;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            float x = v[e] * p.alpha;
+            if (p.C) x += Out::load(p.C, (int64_t)m * p.ldc_m + (int64_t)(n + e) * p.ldc_n);
+            d[e] = Out::cvt(x);
+        }
+    }
+}
+
+template <typename In, typename Out>
+static int32_t launch_skinny(const GemmArgs& a, hipStream_t st) {
+    constexpr int W = 8;
+    const dim3 grid((unsigned)(a.N / 16)), block(W * 64);
+    switch (a.M / 16) {
+        case 1: gemm_mfma_skinny<In, Out, 1, W><<<grid, block, 0, st>>>(a); break;
+        case 2: gemm_mfma_skinny<In, Out, 2, W><<<grid, block, 0, st>>>(a); break;
+        case 3: gemm_mfma_skinny<In, Out, 3, W><<<grid, block, 0, st>>>(a); break;
+        default: gemm_mfma_skinny<In, Out, 4, W><<<grid, block, 0, st>>>(a); break;
+    }
+    MOYE_HIP_CHECK(hipGetLastError());
+    return MOYE_OK;
+}
+
+template <typename In>
+static int32_t launch_skinny_out(int32_t out_dt, const GemmArgs& a, hipStream_t st) {
+    switch (out_dt) {
+        case MOYE_F32: return launch_skinny<In, OutF32>(a, st);
+        case MOYE_F16: return launch_skinny<In, OutF16>(a, st);
+        case MOYE_BF16: return launch_skinny<In, OutBF16>(a, st);
+        default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: MFMA kernels write f32, f16 or bf16, not %s", dtype_name(out_dt));
+    }
+}
+
+// M in {16,32,48,64}, N a multiple of 16, K a multiple of 64 bytes; pointers and pitches 16-byte aligned.
+int32_t gemm_mfma_skinny_dispatch(int32_t in_dt, int32_t out_dt, const GemmArgs& a, hipStream_t st) {
+    const int eb = dtype_bytes(in_dt);
+    if (a.M % 16 || a.M > 64 || a.N % 16 || ((int64_t)a.K * eb) % 64)
+        return fail(MOYE_ERR_SHAPE, "gemm!: the short-M MFMA kernel needs M in {16,32,48,64}, N %% 16 == 0 and K %% %d == 0, got %dx%dx%d",
+                    64 / eb, a.M, a.N, a.K);
+    if ((a.lda * eb) % 16 || (a.ldb * eb) % 16 ||
+        (reinterpret_cast<uintptr_t>(a.A) | reinterpret_cast<uintptr_t>(a.B)) % 16)
+        return fail(MOYE_ERR_ALIGN, "gemm!: operands of the MFMA kernels need 16-byte aligned pointers and row pitches");
+    switch (in_dt) {
+        case MOYE_F16: return launch_skinny_out<InF16>(out_dt, a, st);
+        case MOYE_BF16: return launch_skinny_out<InBF16>(out_dt, a, st);
+        case MOYE_F8E4M3: return launch_skinny_out<InFP8>(out_dt, a, st);
+        default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: no MFMA atom for %s inputs", dtype_name(in_dt));
+    }
+}
+
+}  // namespace moye

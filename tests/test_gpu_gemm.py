@@ -362,3 +362,63 @@ def test_moye_array_api_on_device(mh):
     mh.copyto_(md, ms, tc)
     torch.cuda.synchronize()
     assert torch.equal(dst.view(256, 192), src.view(192, 256).t())
+
+
+# ---------------------------------------------------------------------------------------------
+# short A (M <= 64): the bandwidth-shaped kernel
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("M", [16, 32, 48, 64])
+def test_short_m_exact_on_integers(mh, M):
+    g = torch.Generator().manual_seed(40 + M)
+    for (N, K) in ((256, 320), (1024, 4096), (48, 32)):
+        A = torch.randint(-4, 5, (M, K), generator=g).to(torch.float16)
+        B = torch.randint(-4, 5, (N, K), generator=g).to(torch.float16)
+        C = torch.randint(-8, 9, (M, N), generator=g).to(torch.float32)
+        a, b, c = A.cuda(), B.cuda(), C.cuda()
+        ref = A.double() @ B.double().t()
+        for explicit in (False, True):
+            d = torch.zeros(M, N, dtype=torch.float32, device="cuda")
+            mma = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(M, 16, 32) if explicit else (0, 0, 0))
+            mh.gemm_(mma, T(d), T(a), T(b))
+            torch.cuda.synchronize()
+            assert torch.equal(d.cpu().double(), ref), (M, N, K, explicit)
+        d = torch.zeros(M, N, dtype=torch.float32, device="cuda")
+        mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(0, 0, 0)), T(d), T(a), T(b), T(c), 2.0)
+        torch.cuda.synchronize()
+        assert torch.equal(d.cpu().double(), 2.0 * ref + C.double()), (M, N, K, "C, alpha")
+
+
+def test_short_m_other_types(mh):
+    g = torch.Generator().manual_seed(77)
+    M, N, K = 16, 512, 1024
+    A = torch.randint(-3, 4, (M, K), generator=g).float()
+    B = torch.randint(-3, 4, (N, K), generator=g).float()
+    ref = A.double() @ B.double().t()
+    cases = [(torch.bfloat16, mh.MFMA_F32_16x16x32_BF16, torch.bfloat16), (torch.bfloat16, mh.MFMA_F32_16x16x32_BF16, torch.float32)]
+    if hasattr(torch, "float8_e4m3fn"):
+        cases.append((torch.float8_e4m3fn, mh.MFMA_F32_16x16x32_FP8, torch.bfloat16))
+    for in_dt, atom, out_dt in cases:
+        a, b = A.to(in_dt).cuda(), B.to(in_dt).cuda()
+        d = torch.zeros(M, N, dtype=out_dt, device="cuda")
+        mh.gemm_(mh.tiled_mma_desc(atom, cta_tile=(0, 0, 0)), T(d), T(a), T(b), None, 1.0 / 64)
+        torch.cuda.synchronize()
+        # |sum| <= 9 * 1024 / 64 = 144 in steps of 1/64: exact in fp32, and in bf16 after the 1/64 scaling
+        # only when it fits 8 bits of mantissa, so compare against the same rounding
+        want = (ref / 64).to(torch.float32).to(out_dt)
+        assert torch.equal(d.cpu(), want), (in_dt, out_dt)
+
+
+def test_config4_skinny_bf16(mh):
+    """BASELINE config 4, skinny case: bf16 16 x 8192 x 8192, fp32 out; run twice, results identical."""
+    M, N, K = 16, 8192, 8192
+    got, c64, A, B = _mfma_case(mh, mh.MFMA_F32_16x16x32_BF16, torch.bfloat16, torch.float32, M, N, K, 1004, 0.02,
+                                cta=(0, 0, 0))
+    again, _, _, _ = _mfma_case(mh, mh.MFMA_F32_16x16x32_BF16, torch.bfloat16, torch.float32, M, N, K, 1004, 0.02,
+                                cta=(0, 0, 0))
+    assert torch.equal(got, again)
+    err = relerr(got, c64)
+    ref = to.gemm_universal_fma(A.float().numpy()[:, :], B[:64].float().numpy(), np.zeros((M, 64), np.float32), "bf16", "bf16")
+    ref_err = to.relerr(ref, c64[:, :64].cpu().numpy())
+    print("config4 bf16 16x8192x8192: rel err %.3e (reference arithmetic on 64 columns: %.3e)" % (err, ref_err))
+    assert err <= TOL16

@@ -371,7 +371,7 @@ def test_moye_array_api_on_device(mh):
 @pytest.mark.parametrize("M", [16, 32, 48, 64])
 def test_short_m_exact_on_integers(mh, M):
     g = torch.Generator().manual_seed(40 + M)
-    for (N, K) in ((256, 320), (1024, 4096), (48, 32)):
+    for (N, K) in ((256, 320), (1024, 4096), (48, 32), (8192, 288)):
         A = torch.randint(-4, 5, (M, K), generator=g).to(torch.float16)
         B = torch.randint(-4, 5, (N, K), generator=g).to(torch.float16)
         C = torch.randint(-8, 9, (M, N), generator=g).to(torch.float32)

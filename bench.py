@@ -68,7 +68,10 @@ def other_configs(mh, tensor_of, torch, stream):
 
     def run(name, atom, a, b, d, alpha, peak, cta, waves):
         mma = mh.tiled_mma_desc(atom, atom_layout=waves, cta_tile=cta)
-        ms = mh.time_gemm(mma, tensor_of(d), tensor_of(a), tensor_of(b), None, alpha, stream, warmup=3, iters=20)
+        t_ramp = time.perf_counter()
+        while time.perf_counter() - t_ramp < 0.3:
+            mh.time_gemm(mma, tensor_of(d), tensor_of(a), tensor_of(b), None, alpha, stream, warmup=0, iters=20)
+        ms = mh.time_gemm(mma, tensor_of(d), tensor_of(a), tensor_of(b), None, alpha, stream, warmup=3, iters=50)
         M, N, K = a.shape[0], b.shape[0], a.shape[1]
         rows = torch.arange(0, M, max(1, M // 16), device="cuda")
         c64 = alpha * (a[rows].float().double() @ b.float().double().t())
@@ -95,11 +98,14 @@ def other_configs(mh, tensor_of, torch, stream):
     bs = [b, b.clone(), b.clone()]
     mma = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_BF16, cta_tile=(0, 0, 0))
     tA, tD, tBs = tensor_of(a16), tensor_of(d16), [tensor_of(x) for x in bs]
-    for i in range(3):
-        mh.gemm_(mma, tD, tA, tBs[i], None, 1.0, stream)
+    t_ramp = time.perf_counter()
+    while time.perf_counter() - t_ramp < 0.3:
+        for i in range(30):
+            mh.gemm_(mma, tD, tA, tBs[i % 3], None, 1.0, stream)
+        torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
-    iters = 30
+    iters = 90
     for i in range(iters):
         mh.gemm_(mma, tD, tA, tBs[i % 3], None, 1.0, stream)
     e1.record()
@@ -161,6 +167,15 @@ def main():
                             cta_tile=(bm, bn, bk), stages=args.stages, flags=args.flags)
     tA, tB, tD = tensor_of(A), tensor_of(B), tensor_of(D)
 
+    # The part ramps its clocks over tens of milliseconds of sustained load (measured: the same
+    # kernel reads 1.08 PFLOP/s in the first 10 ms and 1.31 after 100 ms), so before anything is
+    # timed the GPU is kept busy with the workload itself for a fixed 0.5 s; these launches are not
+    # steps and are not counted.
+    t_ramp = time.perf_counter()
+    while time.perf_counter() - t_ramp < 0.5:
+        for _ in range(50):
+            mh.gemm_(mma, tD, tA, tB, None, 1.0, stream)
+        torch.cuda.synchronize()
     for _ in range(args.warmup):
         mh.gemm_(mma, tD, tA, tB, None, 1.0, stream)
     torch.cuda.synchronize()
@@ -205,12 +220,15 @@ def main():
         dst = torch.empty_like(src)
         tc = mh.tiled_copy_desc(op=mh.COPY_LDS_TILED, vec_bits=128, tiler=(64, 64))
         td, ts = tensor_of(dst, (n, n), (n, 1)), tensor_of(src, (n, n), (1, n))
-        cms = mh.time_copy(td, ts, tc, stream, warmup=3, iters=20)
+        t_ramp = time.perf_counter()
+        while time.perf_counter() - t_ramp < 0.3:  # same clock ramp as for the GEMM leg
+            mh.time_copy(td, ts, tc, stream, warmup=0, iters=20)
+        cms = mh.time_copy(td, ts, tc, stream, warmup=3, iters=50)
         nbytes = 2.0 * n * n * 4
         gbs = nbytes / (cms * 1e-3) / 1e9
         ok = bool(torch.equal(dst.view(n, n)[:256, :256], src.view(n, n)[:256, :256].t()))
         flat_d, flat_s = tensor_of(dst, (n * n,), (1,)), tensor_of(src, (n * n,), (1,))
-        pms = mh.time_copy(flat_d, flat_s, None, stream, warmup=3, iters=20)
+        pms = mh.time_copy(flat_d, flat_s, None, stream, warmup=20, iters=50)
         out["secondary"] = {
             "metric": "tiled-copy GB/s", "value": round(gbs, 1), "unit": "GB/s",
             "config": {"workload": "16384x16384 fp32 column-major -> row-major through 64x64 LDS tiles", "bit_exact_sample": ok},

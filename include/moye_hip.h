@@ -88,6 +88,9 @@ typedef struct {
 
 #define MOYE_GEMM_NO_XCD_SWIZZLE 1   /* keep blockIdx -> tile mapping linear (for A/B studies)  */
 #define MOYE_GEMM_NO_LDS_SWIZZLE 2   /* linear LDS tiles (bank-conflict study)                  */
+#define MOYE_GEMM_PINGPONG 0x100      /* 256x256 tile only: the two waves of a SIMD alternate
+                                        between MFMA and memory slots, k-tiles of 64 bytes in a
+                                        five-stage LDS ring (cta_tile_mnk[2] = 64 bytes of K)    */
 
 /* copy ops: UniversalCopy (src/arch/copy/copy.jl:26-51); the LDS-staged forms stand where the
  * reference has cp.async (copy_async.jl:8-24) and ldmatrix (ldmatrix.jl:18-48) */

@@ -22,6 +22,7 @@ SOURCES = {
     "copy_kernels.hip": [],
     "gemm_mfma.hip": [],
     "gemm_mfma256.hip": [],
+    "gemm_mfma256pp.hip": [],
     "gemm_mfma_skinny.hip": [],
     "gemm_universal.hip": ["-ffp-contract=off"],   # UniversalFMA: mul then add, never fused
     "layout_host.cpp": ["-x", "hip"],

@@ -31,6 +31,7 @@ int32_t copy_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, const m
 int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int bk_elems, int waves, int stages,
                               GemmArgs a, hipStream_t st);
 int32_t gemm_mfma_tn_256_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, int waves, int stages, hipStream_t st);
+int32_t gemm_mfma_tn_256_pp_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, hipStream_t st);
 int32_t gemm_mfma_skinny_dispatch(int32_t in_dt, int32_t out_dt, const GemmArgs& a, hipStream_t st);
 int32_t gemm_universal_dispatch(int bm, int bn, int bk, UArgs a, hipStream_t st);
 

@@ -1,0 +1,62 @@
+// Epilogue shared by the MFMA GEMM kernels: alpha * acc + C -> OutT (round to nearest even,
+// the conversion rule of src/arch/copy/copy.jl:38-43) -> the wave's own LDS patch -> 128-bit row
+// stores.  The reference's kernels store accumulator fragments straight to global memory in
+// fragment order (test/device/matmul.jl:51); going through LDS turns that into full-row writes.
+#pragma once
+
+#include "mfma_common.hpp"
+
+namespace moye {
+
+// acc[i][j] of a lane holds C[m = 16 i + lane % 16][n = 16 j + 4 (lane / 16) + e], e = 0..3,
+// relative to (m_base, n_base).  `smem` must be free of operand data for all waves.
+template <typename Out, int MI, int NI>
+__device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&acc)[MI][NI], u32x4* smem, int wave,
+                                             int lane, int64_t m_base, int64_t n_base) {
+    typedef typename Out::type OutT;
+    constexpr int WN = NI * 16;
+    constexpr int EPC = 16 / (int)sizeof(OutT);  // elements per 16-byte chunk
+    constexpr int CR = WN / EPC;                 // chunks per patch row
+    constexpr int PASS_MI = 2, PASS_ROWS = PASS_MI * 16;
+    const int r16 = lane & 15, kq = lane >> 4;
+    OutT* patch = reinterpret_cast<OutT*>(smem) + wave * (PASS_ROWS * WN);
+    u32x4* patch16 = reinterpret_cast<u32x4*>(patch);
+#pragma unroll
+    for (int i0 = 0; i0 < MI; i0 += PASS_MI) {
+#pragma unroll
+        for (int ii = 0; ii < PASS_MI; ++ii) {
+            const int i = i0 + ii;
+#pragma unroll
+            for (int j = 0; j < NI; ++j) {
+                float v[4] = {acc[i][j].x * p.alpha, acc[i][j].y * p.alpha, acc[i][j].z * p.alpha,
+                              acc[i][j].w * p.alpha};
+                if (p.C) {
+                    const int64_t m = m_base + 16 * i + r16, n = n_base + 16 * j + 4 * kq;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] += Out::load(p.C, m * p.ldc_m + (n + e) * p.ldc_n);
+                }
+                const int row = 16 * ii + r16, col = 16 * j + 4 * kq;
+                const int chunk = col / EPC, within = col % EPC;
+                OutT* dst = patch + (row * CR + (chunk ^ (row & 7))) * EPC + within;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) dst[e] = Out::cvt(v[e]);
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int t = 0; t < PASS_ROWS * CR / 64; ++t) {
+            const int c = lane + 64 * t, row = c / CR, ch = c % CR;
+            const u32x4 w = patch16[row * CR + (ch ^ (row & 7))];
+            char* d = static_cast<char*>(p.D) +
+                      ((m_base + 16 * i0 + row) * p.ldd + n_base) * (int64_t)sizeof(OutT) + ch * 16;
+            *reinterpret_cast<u32x4*>(d) = w;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+}
+
+}  // namespace moye

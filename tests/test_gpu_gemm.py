@@ -271,6 +271,47 @@ def test_f16_tn_256_tile_exact_on_integers(mh, waves, stages):
         assert torch.equal(d.cpu().double(), A.double() @ B.double().t()), (waves, stages, out_dt)
 
 
+def test_pingpong_schedule_exact_on_integers(mh):
+    """MOYE_GEMM_PINGPONG: 64-byte k-tiles in a five-stage ring; K from one k-tile to many (the
+    prologue, the steady state and the drain each have their own wait counts), every input type."""
+    from moye_hip import _lib
+    g = torch.Generator().manual_seed(13)
+    cases = [(torch.float16, mh.MFMA_F32_16x16x32_F16, 32), (torch.bfloat16, mh.MFMA_F32_16x16x32_BF16, 32)]
+    if hasattr(torch, "float8_e4m3fn"):
+        cases.append((torch.float8_e4m3fn, mh.MFMA_F32_16x16x32_FP8, 64))
+    for in_dt, atom, bk in cases:
+        for (M, N, kt) in ((256, 256, 1), (256, 512, 3), (512, 256, 4), (256, 256, 5), (256, 256, 6), (512, 768, 37)):
+            K = kt * bk
+            A = torch.randint(-3, 4, (M, K), generator=g).float()
+            B = torch.randint(-3, 4, (N, K), generator=g).float()
+            C = torch.randint(-8, 9, (M, N), generator=g).float()
+            a, b, c = A.to(in_dt).cuda(), B.to(in_dt).cuda(), C.cuda()
+            d = torch.zeros(M, N, dtype=torch.float32, device="cuda")
+            mma = mh.tiled_mma_desc(atom, atom_layout=(2, 4, 1), cta_tile=(256, 256, bk), flags=_lib.GEMM_PINGPONG)
+            mh.gemm_(mma, T(d), T(a), T(b), T(c), 2.0)
+            torch.cuda.synchronize()
+            assert torch.equal(d.cpu().double(), 2.0 * (A.double() @ B.double().t()) + C.double()), (in_dt, M, N, K)
+
+
+def test_pingpong_schedule_random(mh):
+    from moye_hip import _lib
+    M = N = K = 2048
+    g = torch.Generator().manual_seed(14)
+    A = (torch.randn(M, K, generator=g) * K ** -0.5).half()
+    B = (torch.randn(N, K, generator=g) * K ** -0.5).half()
+    a, b = A.cuda(), B.cuda()
+    d = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+    d2 = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+    mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 4, 1), cta_tile=(256, 256, 32),
+                               flags=_lib.GEMM_PINGPONG), T(d), T(a), T(b))
+    mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 4, 1), cta_tile=(256, 256, 64)), T(d2), T(a), T(b))
+    torch.cuda.synchronize()
+    c64 = a.double() @ b.double().t()
+    assert relerr(d, c64) <= TOL16
+    # both schedules add the same products in the same k order within a lane
+    assert torch.equal(d, d2)
+
+
 @pytest.mark.parametrize("tdt,atom", [("float16", "MFMA_F32_16x16x32_F16"), ("bfloat16", "MFMA_F32_16x16x32_BF16")])
 def test_256_tile_variants(mh, tdt, atom):
     """column-major D, C accumulation and alpha through the 256x256 kernel; one k-tile and many."""

@@ -202,6 +202,13 @@ int32_t moye_tiled_copy_partition(int32_t src_bits, int32_t dst_bits, int32_t va
 int32_t moye_make_tiled_mma(int32_t atom, const char* atom_layout, const char* permutation,
                             moye_tiled_mma* out);
 
+/* One execution of a hardware MMA atom by one wave, operands gathered and results scattered through
+ * the atom's (thr,val) layouts (the tables behind layout_a/b/c of src/traits/mma.jl:26-31, which
+ * partition_A/B/C apply): A is the (M,K) atom tile, B the (N,K) tile, D the (M,N) tile, all dense
+ * column-major on the device; D = A * B'.  Allocates a small table buffer and synchronises `stream`:
+ * a self-test for the atom tables, not a compute path. */
+int32_t moye_mma_atom_probe(int32_t atom, const void* A, const void* B, float* D, void* stream);
+
 /* ---- runtime helpers (thin wrappers so a non-HIP host language needs nothing else) ------- */
 int32_t moye_device_malloc(void** ptr, size_t bytes);
 int32_t moye_device_free(void* ptr);

@@ -237,6 +237,136 @@ int32_t guarded(F&& f) {
     if (!(p)) return fail(MOYE_ERR_ARG, "null argument: %s", #p)
 }  // namespace
 
+
+// ---------------------------------------------------------------------------------------------
+// One-wave probe of an MFMA atom: every lane gathers its A and B fragment values through the
+// atom's (thr, val) -> tile-index tables above, the wave executes the instruction once on a zero
+// accumulator, and every lane scatters its D values through the C table.  If the tables describe
+// the hardware, D = A * B' for any input; they are what partition_A/B/C hand to callers
+// (src/atom/mma.jl:292-308), so this is their known-answer test on the machine itself.
+// ---------------------------------------------------------------------------------------------
+namespace {
+typedef float probe_f32x4 __attribute__((ext_vector_type(4)));
+typedef float probe_f32x16 __attribute__((ext_vector_type(16)));
+typedef _Float16 probe_f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 probe_bf16x8 __attribute__((ext_vector_type(8)));
+
+template <int ATOM>
+__global__ __launch_bounds__(64) void mma_atom_probe_kernel(const void* A, const void* B, float* D, const int* ai,
+                                                            const int* bi, const int* ci) {
+    const int lane = threadIdx.x;
+    constexpr bool k32 = ATOM == MOYE_MFMA_F32_32x32x16_F16 || ATOM == MOYE_MFMA_F32_32x32x16_BF16 ||
+                         ATOM == MOYE_MFMA_F32_32x32x16_FP8 || ATOM == MOYE_MFMA_F32_32x32x2_F32;
+    constexpr int VC = k32 ? 16 : 4;
+    float out[VC];
+    if constexpr (ATOM == MOYE_MFMA_F32_16x16x4_F32 || ATOM == MOYE_MFMA_F32_32x32x2_F32) {
+        const float a = static_cast<const float*>(A)[ai[lane]], b = static_cast<const float*>(B)[bi[lane]];
+        if constexpr (k32) {
+            probe_f32x16 c = {};
+            c = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+            for (int v = 0; v < VC; ++v) out[v] = c[v];
+        } else {
+            probe_f32x4 c = {};
+            c = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+            for (int v = 0; v < VC; ++v) out[v] = c[v];
+        }
+    } else if constexpr (ATOM == MOYE_MFMA_F32_16x16x32_FP8 || ATOM == MOYE_MFMA_F32_32x32x16_FP8) {
+        uint64_t a = 0, b = 0;
+        for (int v = 0; v < 8; ++v) {
+            a |= (uint64_t)static_cast<const uint8_t*>(A)[ai[lane * 8 + v]] << (8 * v);
+            b |= (uint64_t)static_cast<const uint8_t*>(B)[bi[lane * 8 + v]] << (8 * v);
+        }
+        if constexpr (k32) {
+            probe_f32x16 c = {};
+            c = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8((long)a, (long)b, c, 0, 0, 0);
+            for (int v = 0; v < VC; ++v) out[v] = c[v];
+        } else {
+            probe_f32x4 c = {};
+            c = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8((long)a, (long)b, c, 0, 0, 0);
+            for (int v = 0; v < VC; ++v) out[v] = c[v];
+        }
+    } else {
+        uint16_t a[8], b[8];
+        for (int v = 0; v < 8; ++v) {
+            a[v] = static_cast<const uint16_t*>(A)[ai[lane * 8 + v]];
+            b[v] = static_cast<const uint16_t*>(B)[bi[lane * 8 + v]];
+        }
+        if constexpr (ATOM == MOYE_MFMA_F32_16x16x32_F16 || ATOM == MOYE_MFMA_F32_32x32x16_F16) {
+            probe_f16x8 fa, fb;
+            __builtin_memcpy(&fa, a, 16);
+            __builtin_memcpy(&fb, b, 16);
+            if constexpr (k32) {
+                probe_f32x16 c = {};
+                c = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, fb, c, 0, 0, 0);
+                for (int v = 0; v < VC; ++v) out[v] = c[v];
+            } else {
+                probe_f32x4 c = {};
+                c = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa, fb, c, 0, 0, 0);
+                for (int v = 0; v < VC; ++v) out[v] = c[v];
+            }
+        } else {
+            probe_bf16x8 fa, fb;
+            __builtin_memcpy(&fa, a, 16);
+            __builtin_memcpy(&fb, b, 16);
+            if constexpr (k32) {
+                probe_f32x16 c = {};
+                c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, c, 0, 0, 0);
+                for (int v = 0; v < VC; ++v) out[v] = c[v];
+            } else {
+                probe_f32x4 c = {};
+                c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa, fb, c, 0, 0, 0);
+                for (int v = 0; v < VC; ++v) out[v] = c[v];
+            }
+        }
+    }
+    for (int v = 0; v < VC; ++v) D[ci[lane * VC + v]] = out[v];
+}
+
+// 0-based tile indices of every (lane, value) pair of a TV layout
+std::vector<int> tv_table(const Layout& tv) {
+    const int64_t nt = size(tv, 1).v, nv = size(tv, 2).v;
+    std::vector<int> t((size_t)(nt * nv));
+    for (int64_t l = 0; l < nt; ++l)
+        for (int64_t v = 0; v < nv; ++v)
+            t[(size_t)(l * nv + v)] = (int)(eval(tv, tup({IT(D(l + 1)), IT(D(v + 1))})).v - 1);
+    return t;
+}
+
+int32_t mma_atom_probe_impl(int32_t atom, const void* A, const void* B, float* D, hipStream_t st) {
+    if (atom < MOYE_MFMA_F32_16x16x32_F16 || atom > MOYE_MFMA_F32_32x32x2_F32)
+        throw Error(MOYE_ERR_UNSUPPORTED, "moye_mma_atom_probe: not a hardware atom");
+    const MMAAtomDesc& a = find_atom(std::to_string(atom));
+    if (size(a.thr_id).v != 64) throw Error(MOYE_ERR_UNSUPPORTED, "moye_mma_atom_probe: atom is not one wave wide");
+    const std::vector<int> ta = tv_table(a.layout_a), tb = tv_table(a.layout_b), tc = tv_table(a.layout_c);
+    const size_t na = ta.size(), nb = tb.size(), nc = tc.size();
+    int* dev = nullptr;
+    MOYE_HIP_CHECK(hipMalloc(&dev, (na + nb + nc) * sizeof(int)));
+    int32_t rc = MOYE_OK;
+    auto copy = [&](int* d, const std::vector<int>& h) { return hipMemcpy(d, h.data(), h.size() * sizeof(int), hipMemcpyHostToDevice); };
+    if (copy(dev, ta) != hipSuccess || copy(dev + na, tb) != hipSuccess || copy(dev + na + nb, tc) != hipSuccess) {
+        rc = fail(MOYE_ERR_HIP, "moye_mma_atom_probe: table upload failed");
+    } else {
+        const int *ai = dev, *bi = dev + na, *ci = dev + na + nb;
+        switch (atom) {
+#define MOYE_PROBE_CASE(X) case X: mma_atom_probe_kernel<X><<<1, 64, 0, st>>>(A, B, D, ai, bi, ci); break;
+            MOYE_PROBE_CASE(MOYE_MFMA_F32_16x16x32_F16)
+            MOYE_PROBE_CASE(MOYE_MFMA_F32_32x32x16_F16)
+            MOYE_PROBE_CASE(MOYE_MFMA_F32_16x16x32_BF16)
+            MOYE_PROBE_CASE(MOYE_MFMA_F32_32x32x16_BF16)
+            MOYE_PROBE_CASE(MOYE_MFMA_F32_16x16x32_FP8)
+            MOYE_PROBE_CASE(MOYE_MFMA_F32_32x32x16_FP8)
+            MOYE_PROBE_CASE(MOYE_MFMA_F32_16x16x4_F32)
+            MOYE_PROBE_CASE(MOYE_MFMA_F32_32x32x2_F32)
+#undef MOYE_PROBE_CASE
+        }
+        if (hipGetLastError() != hipSuccess || hipStreamSynchronize(st) != hipSuccess)
+            rc = fail(MOYE_ERR_HIP, "moye_mma_atom_probe: launch failed");
+    }
+    (void)hipFree(dev);
+    return rc;
+}
+}  // namespace
+
 extern "C" {
 
 int32_t moye_layout_normalize(const char* layout, char* out, size_t cap) {
@@ -496,6 +626,11 @@ int32_t moye_make_tiled_mma(int32_t atom, const char* atom_layout, const char* p
         for (int i = 0; i < 3; ++i) out->cta_tile_mnk[i] = out->tile_mnk[i];
         return (int32_t)MOYE_OK;
     });
+}
+
+int32_t moye_mma_atom_probe(int32_t atom, const void* A, const void* B, float* D, void* stream) {
+    MOYE_REQUIRE(A && B && D);
+    return guarded([&] { return mma_atom_probe_impl(atom, A, B, D, static_cast<hipStream_t>(stream)); });
 }
 
 }  // extern "C"

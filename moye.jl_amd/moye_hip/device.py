@@ -68,3 +68,11 @@ def time_copy(dst, src, tiled_copy=None, stream=None, warmup=2, iters=10):
     ms = C.c_float()
     check(lib().moye_time_copy(_ref(tiled_copy), C.byref(dst), C.byref(src), stream, warmup, iters, C.byref(ms)))
     return ms.value
+
+
+def mma_atom_probe(atom, a_ptr, b_ptr, d_ptr, stream=None):
+    """One wave executes the atom once through its (thr,val) tables: D(M,N) = A(M,K) * B(N,K)',
+    all dense column-major device buffers (raw pointers)."""
+    f = lib().moye_mma_atom_probe
+    f.argtypes = [C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+    check(f(atom, a_ptr, b_ptr, d_ptr, stream))

@@ -463,3 +463,32 @@ def test_config4_skinny_bf16(mh):
     ref_err = to.relerr(ref, c64[:, :64].cpu().numpy())
     print("config4 bf16 16x8192x8192: rel err %.3e (reference arithmetic on 64 columns: %.3e)" % (err, ref_err))
     assert err <= TOL16
+
+
+# ---------------------------------------------------------------------------------------------
+# the MFMA atoms' (thr,val) tables against the instruction itself
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("atom,m,n,k,dt", [
+    ("MFMA_F32_16x16x32_F16", 16, 16, 32, "float16"), ("MFMA_F32_32x32x16_F16", 32, 32, 16, "float16"),
+    ("MFMA_F32_16x16x32_BF16", 16, 16, 32, "bfloat16"), ("MFMA_F32_32x32x16_BF16", 32, 32, 16, "bfloat16"),
+    ("MFMA_F32_16x16x32_FP8", 16, 16, 32, "float8_e4m3fn"), ("MFMA_F32_32x32x16_FP8", 32, 32, 16, "float8_e4m3fn"),
+    ("MFMA_F32_16x16x4_F32", 16, 16, 4, "float32"), ("MFMA_F32_32x32x2_F32", 32, 32, 2, "float32")])
+def test_mfma_atom_tables_on_hardware(mh, atom, m, n, k, dt):
+    """layout_a/b/c of every gfx950 atom: one wave gathers A and B through the tables, executes the
+    instruction once, scatters D through the C table; D must equal A*B' exactly on small integers.
+    A wrong lane->row, lane->k-group or accumulator-register mapping breaks the equality."""
+    if not hasattr(torch, dt):
+        pytest.skip("torch without " + dt)
+    tdt = getattr(torch, dt)
+    g = torch.Generator().manual_seed(m * 1000 + k)
+    for trial in range(3):
+        A = torch.randint(-4, 5, (m, k), generator=g).float()       # distinct rows and columns
+        B = torch.randint(-4, 5, (n, k), generator=g).float()
+        # column-major dense tiles: element (i, kk) at i + m*kk
+        a = A.t().contiguous().to(tdt).cuda()
+        b = B.t().contiguous().to(tdt).cuda()
+        d = torch.full((n, m), float("nan"), dtype=torch.float32, device="cuda")   # (M,N) column-major
+        mh.mma_atom_probe(getattr(mh, atom), a.data_ptr(), b.data_ptr(), d.data_ptr())
+        torch.cuda.synchronize()
+        assert torch.equal(d.t().cpu().double(), A.double() @ B.double().t()), (atom, trial)

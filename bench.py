@@ -24,8 +24,11 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # (the summaries are committed under profiles/), each reading scaled by what the same counter shows for the
 # 1 GiB plain copy (fetch x2.0000, write x1.0000).  Only valid for the default tile/waves/flags.
 MEASURED_TRAFFIC = {
-    "gemm_f16_4096_tile256": {"read_bytes": 197454 * 1024, "write_bytes": 33279 * 1024},
-    "transpose_f32_16384": {"read_bytes": 1048610 * 1024, "write_bytes": 1049814 * 1024},
+    "gemm_f16_4096_tile256": {"read_bytes": 197437 * 1024, "write_bytes": 33280 * 1024},
+    "transpose_f32_16384": {"read_bytes": 1048622 * 1024, "write_bytes": 1049576 * 1024},
+    "gemm_bf16_8192_tile256": {"read_bytes": 1647295 * 1024, "write_bytes": 266240 * 1024},
+    "gemm_fp8_8192_tile256": {"read_bytes": 787830 * 1024, "write_bytes": 131072 * 1024},
+    "gemm_bf16_16x8192x8192": {"read_bytes": 159438 * 1024, "write_bytes": 512 * 1024},
 }
 
 
@@ -66,7 +69,7 @@ def other_configs(mh, tensor_of, torch, stream):
     n = 8192
     g = torch.Generator(device="cuda").manual_seed(1004)
 
-    def run(name, atom, a, b, d, alpha, peak, cta, waves):
+    def run(name, atom, a, b, d, alpha, peak, cta, waves, traffic_key):
         mma = mh.tiled_mma_desc(atom, atom_layout=waves, cta_tile=cta)
         t_ramp = time.perf_counter()
         while time.perf_counter() - t_ramp < 0.3:
@@ -80,7 +83,8 @@ def other_configs(mh, tensor_of, torch, stream):
         entry = {"workload": name, "kernel_ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 1), "rel_err_vs_fp64": err}
         if peak:
             entry["roofline"] = {"bound": "mfma", "achieved": entry["tflops"], "peak": peak, "unit": "TFLOP/s",
-                                 "frac": round(entry["tflops"] / peak, 4)}
+                                 "frac": round(entry["tflops"] / peak, 4),
+                                 "traffic": sum(MEASURED_TRAFFIC[traffic_key].values())}
         else:
             nbytes = a.numel() * a.element_size() + b.numel() * b.element_size() + d.numel() * d.element_size()
             gbs = nbytes / ms / 1e6
@@ -91,7 +95,8 @@ def other_configs(mh, tensor_of, torch, stream):
     a = (torch.randn(n, n, generator=g, device="cuda") * 0.02).bfloat16()
     b = (torch.randn(n, n, generator=g, device="cuda") * 0.02).bfloat16()
     d = torch.zeros(n, n, dtype=torch.float32, device="cuda")
-    run("bf16 TN 8192^3, fp32 out, CTA 256x256x64", mh.MFMA_F32_16x16x32_BF16, a, b, d, 1.0, PEAK_F16_TFLOPS, (256, 256, 64), (2, 4, 1))
+    run("bf16 TN 8192^3, fp32 out, CTA 256x256x64", mh.MFMA_F32_16x16x32_BF16, a, b, d, 1.0, PEAK_F16_TFLOPS, (256, 256, 64), (2, 4, 1),
+        "gemm_bf16_8192_tile256")
     # short M: rotate over 3 copies of B so that the 256 MiB Infinity Cache cannot serve the stream
     a16 = a[:16].contiguous()
     d16 = torch.zeros(16, n, dtype=torch.float32, device="cuda")
@@ -117,7 +122,8 @@ def other_configs(mh, tensor_of, torch, stream):
                 "kernel_ms": round(ms, 5), "tflops": round(2.0 * 16 * n * n / ms / 1e9, 1),
                 "rel_err_vs_fp64": float((d16.double() - c64).abs().max() / c64.abs().max()),
                 "roofline": {"bound": "hbm", "achieved": round(nbytes / ms / 1e6, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                             "frac": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4), "algorithmic_bytes": nbytes}})
+                             "frac": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4), "algorithmic_bytes": nbytes,
+                             "traffic": sum(MEASURED_TRAFFIC["gemm_bf16_16x8192x8192"].values())}})
     del bs, a, b, d
     if hasattr(torch, "float8_e4m3fn"):
         x = torch.randn(n, n, generator=g, device="cuda")
@@ -127,7 +133,7 @@ def other_configs(mh, tensor_of, torch, stream):
         del x, w
         d = torch.zeros(n, n, dtype=torch.bfloat16, device="cuda")
         run("fp8 e4m3 TN 8192^3, per-tensor scales, bf16 out, CTA 256x256x128", mh.MFMA_F32_16x16x32_FP8, qa, qb, d,
-            sa * sb, 5000.0, (256, 256, 128), (2, 4, 1))
+            sa * sb, 5000.0, (256, 256, 128), (2, 4, 1), "gemm_fp8_8192_tile256")
     return res
 
 

@@ -20,10 +20,12 @@ src/algorithm/array_algorithms.jl, docs/src/manual/tiled_matmul.md) and by
 function-level invariants evaluated by brute force.
 
 Parity unpinned (no reference vector exists and none can be generated without
-a Julia runtime): the printed nesting of `retile`, `get_layout{A,B,C}_TV`,
-`make_tiled_copy_{A,B,C}`, `tile_to_shape`, `left_inverse`, and
-`compact_order` with mixed static/dynamic orders.  Their function values are
-checked by bijection/ownership invariants only.
+a Julia runtime): the printed form (nesting, static-ness) of the results of
+`retile`, `get_layout{A,B,C}_TV`, `make_tiled_copy_{A,B,C}`, `tile_to_shape`,
+`left_inverse`, and of `compact_order` with mixed static/dynamic orders.  The
+function values of the TV layouts and of make_tiled_copy_A/B are pinned by the
+thread-ownership tables of the manual's figures (tests/test_svg_fixtures.py);
+`retile`, `tile_to_shape` and `left_inverse` by invariants only.
 """
 from __future__ import annotations
 

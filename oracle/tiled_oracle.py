@@ -7,8 +7,9 @@ reference over numpy buffers.  Pure-Python loops: for small cases only.
 
 The tensor-core tables of the reference (`mma_sm70/75/80.jl`, `ldmatrix.jl`)
 are reproduced as data because the reference's own tests and SVG fixtures are
-expressed through them; the gfx950 MFMA tables are new and are pinned on
-hardware by the one-wave atom probe test.
+expressed through them (pinned by tests/test_svg_fixtures.py against the figures
+of the reference's manual); the gfx950 MFMA tables are new and are pinned on
+hardware by the one-wave atom probe test (tests/test_gpu_gemm.py).
 """
 from __future__ import annotations
 

@@ -77,14 +77,15 @@ def other_configs(mh, tensor_of, torch, stream):
         ms = mh.time_gemm(mma, tensor_of(d), tensor_of(a), tensor_of(b), None, alpha, stream, warmup=3, iters=50)
         M, N, K = a.shape[0], b.shape[0], a.shape[1]
         rows = torch.arange(0, M, max(1, M // 16), device="cuda")
-        c64 = alpha * (a[rows].float().double() @ b.float().double().t())
+        c64 = alpha * (a[rows].double() @ b.double().t()) if a.dtype == torch.float32 else \
+            alpha * (a[rows].float().double() @ b.float().double().t())
         err = float((d[rows].double() - c64).abs().max() / c64.abs().max())
         flops = 2.0 * M * N * K
         entry = {"workload": name, "kernel_ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 1), "rel_err_vs_fp64": err}
         if peak:
             entry["roofline"] = {"bound": "mfma", "achieved": entry["tflops"], "peak": peak, "unit": "TFLOP/s",
                                  "frac": round(entry["tflops"] / peak, 4),
-                                 "traffic": sum(MEASURED_TRAFFIC[traffic_key].values())}
+                                 "traffic": sum(MEASURED_TRAFFIC[traffic_key].values()) if traffic_key else None}
         else:
             nbytes = a.numel() * a.element_size() + b.numel() * b.element_size() + d.numel() * d.element_size()
             gbs = nbytes / ms / 1e6
@@ -97,6 +98,11 @@ def other_configs(mh, tensor_of, torch, stream):
     d = torch.zeros(n, n, dtype=torch.float32, device="cuda")
     run("bf16 TN 8192^3, fp32 out, CTA 256x256x64", mh.MFMA_F32_16x16x32_BF16, a, b, d, 1.0, PEAK_F16_TFLOPS, (256, 256, 64), (2, 4, 1),
         "gemm_bf16_8192_tile256")
+    af, bf_ = a.float(), b.float()
+    df = torch.zeros(n, n, dtype=torch.float32, device="cuda")
+    run("fp32 TN 8192^3 (v_mfma_f32_16x16x4_f32), CTA 256x256x32", mh.MFMA_F32_16x16x4_F32, af, bf_, df, 1.0, 157.3,
+        (256, 256, 32), (2, 4, 1), None)
+    del af, bf_, df
     # short M: rotate over 3 copies of B so that the 256 MiB Infinity Cache cannot serve the stream
     a16 = a[:16].contiguous()
     d16 = torch.zeros(16, n, dtype=torch.float32, device="cuda")

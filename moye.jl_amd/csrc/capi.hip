@@ -94,8 +94,9 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
         return fail(MOYE_ERR_UNSUPPORTED, "gemm!: atom takes %s operands, got A %s and B %s", dtype_name(in_dt),
                     dtype_name(A.dtype), dtype_name(B.dtype));
     if (tC && C.dtype != D.dtype) return fail(MOYE_ERR_UNSUPPORTED, "gemm!: C and D must have the same element type");
-    if (in_dt == MOYE_F32)
-        return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the fp32 MFMA atoms have no kernel yet; use MOYE_MMA_UNIVERSAL_FMA");
+    if (mma->atom == MOYE_MFMA_F32_32x32x2_F32 || mma->atom == MOYE_MFMA_F32_32x32x16_F16 ||
+        mma->atom == MOYE_MFMA_F32_32x32x16_BF16 || mma->atom == MOYE_MFMA_F32_32x32x16_FP8)
+        return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the 32x32 MFMA atoms are described (layouts, partitions) but the kernels issue the 16x16 forms");
     if (K > 0 && (A.cs != 1 || B.cs != 1))
         return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the MFMA kernels need K-major A and B (stride 1 along K, the 'TN' form)");
     if (K == 0) return fail(MOYE_ERR_SHAPE, "gemm!: K == 0");

@@ -255,6 +255,8 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
             return wide ? launch_out<InBF16, 128, 128, 128>(out_dt, a, st) : launch_out<InBF16, 128, 128, 64>(out_dt, a, st);
         case MOYE_F8E4M3:
             return wide ? launch_out<InFP8, 128, 128, 128>(out_dt, a, st) : launch_out<InFP8, 128, 128, 64>(out_dt, a, st);
+        case MOYE_F32:
+            return wide ? launch_out<InF32, 128, 128, 128>(out_dt, a, st) : launch_out<InF32, 128, 128, 64>(out_dt, a, st);
         default:
             return fail(MOYE_ERR_UNSUPPORTED, "gemm!: no MFMA atom for %s inputs", dtype_name(in_dt));
     }

@@ -1,11 +1,11 @@
 // gemm! on the matrix cores, large-tile schedule: one 256 x 256 x (128 bytes of K) CTA tile per
-// compute unit, 2 x 2 waves, each wave a 128 x 128 block of C held in 256 accumulator registers.
+// compute unit; 2 x 4 waves with 128 x 64 wave tiles (the default: 128 accumulator registers per
+// lane, two waves per SIMD) or 2 x 2 waves with 128 x 128 wave tiles (256 accumulators).
 //
-// Why this shape on gfx950: the LDS delivers 128 bytes per clock per CU while the four SIMDs
-// retire one 16x16x32 MFMA each every 16 clocks.  With 64 x 64 wave tiles the fragment reads
-// alone need as many LDS clocks as the MFMAs need SIMD clocks; 128 x 128 wave tiles halve the
-// LDS bytes per flop (and the L2 bytes per flop of the workgroup).  4096 / 256 = 16, so a 4096^2
-// problem is exactly 256 workgroups: one per CU, no tail.
+// Why this shape on gfx950: with 64 x 64 wave tiles the fragment reads need about as many LDS
+// clocks as the MFMAs need SIMD clocks; larger wave tiles cut the LDS bytes per flop, and the
+// 256 x 256 CTA tile halves the L2 bytes per flop of a 128 x 128 one.  4096 / 256 = 16, so a
+// 4096^2 problem is exactly 256 workgroups: one per CU, no tail.
 //
 // Schedule per k-tile (two k-steps of 32 halves / 64 fp8), operand tiles double-buffered in LDS,
 // fragments double-buffered in registers:
@@ -430,6 +430,7 @@ int32_t gemm_mfma_tn_256_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, int
         case MOYE_F16: return launch256_out<InF16>(out_dt, a, waves, stages, st);
         case MOYE_BF16: return launch256_out<InBF16>(out_dt, a, waves, stages, st);
         case MOYE_F8E4M3: return launch256_out<InFP8>(out_dt, a, waves, stages, st);
+        case MOYE_F32: return launch256_out<InF32>(out_dt, a, waves, stages, st);
         default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: no MFMA atom for %s inputs", dtype_name(in_dt));
     }
 }

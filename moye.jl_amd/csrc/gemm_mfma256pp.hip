@@ -184,6 +184,7 @@ int32_t gemm_mfma_tn_256_pp_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, 
         case MOYE_F16: return launch256_pp_out<InF16>(out_dt, a, st);
         case MOYE_BF16: return launch256_pp_out<InBF16>(out_dt, a, st);
         case MOYE_F8E4M3: return launch256_pp_out<InFP8>(out_dt, a, st);
+        case MOYE_F32: return launch256_pp_out<InF32>(out_dt, a, st);
         default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: no MFMA atom for %s inputs", dtype_name(in_dt));
     }
 }

@@ -50,6 +50,19 @@ struct InFP8 {
     }
 };
 
+// A 16-byte chunk holds 4 fp32 values of one row: element j of every lane's chunk goes to MFMA j, so
+// MFMA j multiplies the k-slices {j, 4+j, 8+j, 12+j} of a 64-byte row piece; A and B are cut the
+// same way, so every product a[m][k] * b[n][k] is formed exactly once.
+struct InF32 {
+    static constexpr int kBytes = 4;
+    static __device__ __forceinline__ void mma(const u32x4& a, const u32x4& b, f32x4& c) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            c = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(a[j]), __uint_as_float(b[j]), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ void mma_acc(const u32x4& a, const u32x4& b, f32x4& c) { mma(a, b, c); }
+};
+
 // ---- output element traits: fp32 -> OutT, round to nearest even (src/arch/copy/copy.jl:38-43) ---
 struct OutF32 {
     typedef float type;

@@ -492,3 +492,53 @@ def test_mfma_atom_tables_on_hardware(mh, atom, m, n, k, dt):
         mh.mma_atom_probe(getattr(mh, atom), a.data_ptr(), b.data_ptr(), d.data_ptr())
         torch.cuda.synchronize()
         assert torch.equal(d.t().cpu().double(), A.double() @ B.double().t()), (atom, trial)
+
+
+# ---------------------------------------------------------------------------------------------
+# fp32 operands on the matrix cores (v_mfma_f32_16x16x4_f32)
+# ---------------------------------------------------------------------------------------------
+
+TOL32 = 1e-5   # rel err bound for fp32 inputs
+
+
+@pytest.mark.parametrize("cta,flags", [((128, 128, 16), 0), ((128, 128, 32), 0), ((256, 256, 32), 0), ((256, 256, 16), 0x100),
+                                       ((0, 0, 0), 0)])
+def test_f32_mfma_gemm(mh, cta, flags):
+    g = torch.Generator().manual_seed(55)
+    for (M, N, K) in ((256, 256, 32), (512, 768, 416)):
+        # exact on integers
+        A = torch.randint(-50, 51, (M, K), generator=g).float()
+        B = torch.randint(-50, 51, (N, K), generator=g).float()
+        a, b = A.cuda(), B.cuda()
+        d = torch.zeros(M, N, device="cuda")
+        mma = mh.tiled_mma_desc(mh.MFMA_F32_16x16x4_F32, atom_layout=(2, 4, 1) if cta[0] == 256 else (2, 2, 1), cta_tile=cta,
+                                flags=flags)
+        mh.gemm_(mma, T(d), T(a), T(b))
+        torch.cuda.synchronize()
+        assert torch.equal(d.cpu().double(), A.double() @ B.double().t()), (cta, M, N, K)
+        # random data against fp64
+        A = torch.rand(M, K, generator=g) * 2 - 1
+        B = torch.rand(N, K, generator=g) * 2 - 1
+        a, b = A.cuda(), B.cuda()
+        mh.gemm_(mma, T(d), T(a), T(b))
+        torch.cuda.synchronize()
+        assert relerr(d, a.double() @ b.double().t()) <= TOL32
+
+
+def test_f32_mfma_short_m(mh):
+    g = torch.Generator().manual_seed(56)
+    A = torch.randint(-50, 51, (16, 2048), generator=g).float()
+    B = torch.randint(-50, 51, (512, 2048), generator=g).float()
+    a, b = A.cuda(), B.cuda()
+    d = torch.zeros(16, 512, device="cuda")
+    mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x4_F32, cta_tile=(0, 0, 0)), T(d), T(a), T(b))
+    torch.cuda.synchronize()
+    assert torch.equal(d.cpu().double(), A.double() @ B.double().t())
+
+
+def test_32x32_atoms_have_no_kernel(mh):
+    a = torch.zeros(256, 64, dtype=torch.float16, device="cuda")
+    d = torch.zeros(256, 256, dtype=torch.float16, device="cuda")
+    with pytest.raises(mh.MoyeError) as e:
+        mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_32x32x16_F16, cta_tile=(128, 128, 32)), T(d), T(a), T(a))
+    assert "32x32" in str(e.value)

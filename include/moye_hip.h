@@ -165,9 +165,15 @@ int32_t moye_layout_prepend(const char* layout, int32_t rank, char* out, size_t 
 int32_t moye_layout_make_ordered(const char* shape, const char* order, char* out, size_t cap); /* layout.jl:216-218 */
 int32_t moye_layout_make_fragment_like(const char* layout, char* out, size_t cap);           /* layout.jl:1143-1149 */
 int32_t moye_layout_slice(const char* layout, const char* coord, char* out, size_t cap, int64_t* offset); /* slice_and_offset, layout.jl:368-371 */
-int32_t moye_layout_make(const char* shape, int32_t row_major, char* out, size_t cap);        /* make_layout(shape, GenColMajor|GenRowMajor), layout.jl:154-159 */
+int32_t moye_layout_make(const char* shape, int32_t row_major, char* out, size_t cap);
+int32_t moye_layout_tile_to_shape(const char* layout, const char* trg_shape, const char* order, char* out, size_t cap); /* layout.jl:930-935; order "" = GenColMajor */
+int32_t moye_layout_make_like(const char* layout, char* out, size_t cap);                   /* make_layout_like, layout.jl:223-225 */        /* make_layout(shape, GenColMajor|GenRowMajor), layout.jl:154-159 */
 
-/* IntTuple helpers (src/int_tuple.jl, src/stride.jl) on tuple text such as "(3,(2,2))" */
+/* IntTuple helpers (src/int_tuple.jl, src/stride.jl, src/algorithm/tuple_algorithms.jl) on tuple text such as
+ * "(3,(2,2))".  op = flatten | unflatten | product | capacity | product_each | rank | depth | shape_div |
+ * elem_scale | filter_zeros | slice | dice | group(a, begin, end) | append(a, val[, n]) | prepend(a, val[, n]) |
+ * zip2_by | compact_col_major | compact_row_major | compact_order | coord_to_index | index_to_coord |
+ * coord_to_coord | iscompatible | colex_less | elem_less | increment */
 int32_t moye_tuple_op(const char* op, const char* a, const char* b, const char* c, char* out, size_t cap);
 
 /* @tile / local_tile (src/algorithm/array_algorithms.jl:113-120) and @parallelize /
@@ -197,6 +203,18 @@ int32_t moye_tiled_copy_query(int32_t src_bits, int32_t dst_bits, int32_t val_bi
 int32_t moye_tiled_copy_partition(int32_t src_bits, int32_t dst_bits, int32_t val_bits,
                                   const char* thr_layout, const char* val_layout, int32_t thr_idx,
                                   char which, const char* layout, char* out, size_t cap, int64_t* offset);
+/* TiledCopy(atom, layout_tv, tiler) (atom/copy.jl:113-125): the form make_tiled_copy_A/B/C build from a
+ * TiledMMA (atom/copy.jl:227-240: layout_tv = get_layoutA/B/C_TV(mma), tiler = its tile sizes).
+ * what = "layoutS_TV" | "layoutD_TV" (atom/copy.jl:168-187) | "num_val_src" | "num_val_dst" | "size";
+ * the two names are accepted by moye_tiled_copy_query too. */
+int32_t moye_tiled_copy_tv_query(int32_t src_bits, int32_t dst_bits, int32_t val_bits, const char* layout_tv,
+                                 const char* tiler, const char* what, char* out, size_t cap);
+int32_t moye_tiled_copy_tv_partition(int32_t src_bits, int32_t dst_bits, int32_t val_bits, const char* layout_tv,
+                                     const char* tiler, int32_t thr_idx, char which, const char* layout,
+                                     char* out, size_t cap, int64_t* offset);
+/* retile_S / retile_D (atom/copy.jl:151-166, 216-225) */
+int32_t moye_tiled_copy_tv_retile(int32_t src_bits, int32_t dst_bits, int32_t val_bits, const char* layout_tv,
+                                  const char* tiler, const char* layout, char* out, size_t cap);
 /* fill a moye_tiled_mma from MoYe-level arguments (checks that the atom layout and the
  * permutation sizes describe a tile this build has a kernel for) */
 int32_t moye_make_tiled_mma(int32_t atom, const char* atom_layout, const char* permutation,

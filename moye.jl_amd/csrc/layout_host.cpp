@@ -329,7 +329,6 @@ IT shape_div(const IT& a, const IT& b) {  // int_tuple.jl:84-101
     return IT(shape_div_int(leaf_of(a), leaf_of(b)));
 }
 
-namespace {
 IT elem_scale(const IT& x, const IT& y) {  // int_tuple.jl:103-109
     if (x.is_tuple()) {
         if (!y.is_tuple() || x.size() != y.size()) raise(MOYE_ERR_RANK, "elem_scale: incongruent tuples");
@@ -349,6 +348,7 @@ IT filter_zeros(const IT& a, const IT& x) {  // int_tuple.jl:123-128
     return is_static_zero(a) ? IT(S(1)) : x;
 }
 
+namespace {
 IT product_like(const IT& x, const IT& g) {  // int_tuple.jl:59-60
     if (g.is_tuple()) {
         if (!x.is_tuple() || x.size() != g.size()) raise(MOYE_ERR_RANK, "product_like: incongruent tuples");
@@ -1131,6 +1131,150 @@ Layout local_partition(const Layout& l, const Tile& tile, const IT& coord_or_ind
     if (tile.kind != Tile::TUPLE) raise(MOYE_ERR_ARG, "@parallelize takes a thread layout or a tuple tile");
     const Layout z = zipped_divide(l, tile);
     return slice_and_offset(z, IT::tuple({coord_or_index, colons(rank(l))}), offset);
+}
+
+// ------------------------------------------------------------------------------------------------
+// IntTuple helpers used by callers rather than by the algebra itself
+// ------------------------------------------------------------------------------------------------
+IT unflatten(const IT& flat, const IT& target) {  // tuple_algorithms.jl:25-37
+    const std::vector<IT> items = as_items(flat);
+    size_t need = flat_leaves(target).size();
+    if (items.size() < need) raise(MOYE_ERR_RANK, "unflatten: not enough elements for the target profile");
+    size_t pos = 0;
+    return unflatten_impl(items, pos, target);
+}
+
+IT group(const IT& t, int b, int e) {  // tuple_algorithms.jl:101-112, modes b..e (1-based, inclusive)
+    const std::vector<IT> items = as_items(t);
+    if (b < 1 || e < b || (size_t)e > items.size()) raise(MOYE_ERR_ARG, "group: bad range");
+    std::vector<IT> out(items.begin(), items.begin() + (b - 1));
+    out.push_back(IT::tuple(std::vector<IT>(items.begin() + (b - 1), items.begin() + e)));
+    out.insert(out.end(), items.begin() + e, items.end());
+    return IT::tuple(out);
+}
+
+IT append_value(const IT& t, const IT& val, int n) {  // tuple_algorithms.jl:114-145
+    std::vector<IT> items = as_items(t);
+    if (n < 0) {
+        items.push_back(val);
+        return IT::tuple(items);
+    }
+    if (items.size() > (size_t)n)
+        raise(MOYE_ERR_RANK, "input tuple of length " + std::to_string(items.size()) + ", requested " + std::to_string(n));
+    while (items.size() < (size_t)n) items.push_back(val);
+    return IT::tuple(items);
+}
+
+IT prepend_value(const IT& t, const IT& val, int n) {  // tuple_algorithms.jl:147-176
+    std::vector<IT> items = as_items(t);
+    if (n < 0) {
+        items.insert(items.begin(), val);
+        return IT::tuple(items);
+    }
+    if (items.size() > (size_t)n)
+        raise(MOYE_ERR_RANK, "input tuple of length " + std::to_string(items.size()) + ", requested " + std::to_string(n));
+    items.insert(items.begin(), (size_t)n - items.size(), val);
+    return IT::tuple(items);
+}
+
+IT zip2_by(const IT& t, const IT& guide) {  // tuple_algorithms.jl:213-224
+    if (!guide.is_tuple()) {
+        if (!t.is_tuple() || t.size() != 2) raise(MOYE_ERR_RANK, "zip2_by: expected a pair");
+        return t;
+    }
+    if (!t.is_tuple() || guide.size() > t.size()) raise(MOYE_ERR_RANK, "zip2_by: guide tuple is longer than input tuple");
+    std::vector<IT> firsts, seconds;
+    for (size_t i = 0; i < guide.size(); ++i) {
+        const IT z = zip2_by(t[i], guide[i]);
+        firsts.push_back(z[0]);
+        seconds.push_back(z[1]);
+    }
+    for (size_t i = guide.size(); i < t.size(); ++i) seconds.push_back(t[i]);
+    return IT::tuple({IT::tuple(firsts), IT::tuple(seconds)});
+}
+
+IT product_each(const IT& t) {
+    std::vector<IT> out;
+    for (const IT& e : as_items(t)) out.push_back(IT(product(e)));
+    return IT::tuple(out);
+}
+
+namespace {
+bool int_less(const IT& a, const IT& b) { return leaf_of(a).v < leaf_of(b).v; }
+IT drop_last(const IT& t) { return IT::tuple(std::vector<IT>(t.items.begin(), t.items.end() - 1)); }
+IT drop_first(const IT& t) { return IT::tuple(std::vector<IT>(t.items.begin() + 1, t.items.end())); }
+IT repeat_like(const IT& t, Int x) {  // tuple_algorithms.jl:80-98
+    if (!t.is_tuple()) return IT(x);
+    std::vector<IT> out;
+    for (const IT& e : t.items) out.push_back(repeat_like(e, x));
+    return IT::tuple(out);
+}
+}  // namespace
+
+bool colex_less(const IT& a, const IT& b) {  // int_tuple.jl:184-195
+    if (!a.is_tuple() && !b.is_tuple()) return int_less(a, b);
+    if (!a.is_tuple() || !b.is_tuple()) raise(MOYE_ERR_RANK, "colex_less: an integer against a tuple");
+    if (a.size() == 0) return b.size() != 0;
+    if (b.size() == 0) return false;
+    const IT &x = a.items.back(), &y = b.items.back();
+    if (!equal_values(x, y)) return colex_less(x, y);
+    return colex_less(drop_last(a), drop_last(b));
+}
+
+bool elem_less(const IT& a, const IT& b) {  // int_tuple.jl:197-211
+    if (!a.is_tuple() && !b.is_tuple()) return int_less(a, b);
+    if (!a.is_tuple() || !b.is_tuple()) raise(MOYE_ERR_RANK, "elem_less: an integer against a tuple");
+    if (a.size() == 0) return true;
+    if (b.size() == 0) return false;
+    const IT &x = a[0], &y = b[0];
+    if (a.size() == 1 && b.size() == 1) return x.is_tuple() ? elem_less(x, y) : int_less(x, y);
+    if (!(equal_values(x, y) || elem_less(x, y))) return false;
+    return elem_less(drop_first(a), drop_first(b));
+}
+
+IT increment(const IT& coord, const IT& shape) {  // int_tuple.jl:218-232: next 1-based coordinate, wrapping
+    if (!coord.is_tuple()) {
+        const Int c = leaf_of(coord), s = leaf_of(shape);
+        return c.v < s.v ? IT(add(c, Int(1, c.s))) : IT(Int(1, c.s));
+    }
+    if (!shape.is_tuple() || shape.size() != coord.size()) raise(MOYE_ERR_RANK, "increment: coordinate and shape differ in rank");
+    const IT &c = coord[0], &s = shape[0];
+    if (coord.size() == 1) return IT::tuple({increment(c, s)});
+    if (!equal_values(c, s)) {
+        IT r = coord;
+        r.items[0] = increment(c, s);
+        return r;
+    }
+    const bool st = is_static(c);
+    std::vector<IT> out{repeat_like(s, Int(1, st))};
+    for (const IT& e : increment(drop_first(coord), drop_first(shape)).items) out.push_back(e);
+    return IT::tuple(out);
+}
+
+IT coord_to_coord(const IT& coord, const IT& src_shape, const IT& dst_shape) {  // stride.jl:133-141
+    if (coord.is_tuple() && src_shape.is_tuple() && dst_shape.is_tuple()) {
+        if (coord.size() != src_shape.size() || coord.size() != dst_shape.size())
+            raise(MOYE_ERR_RANK, "coord, shape1, and shape2 must have the same rank");
+        std::vector<IT> out;
+        for (size_t i = 0; i < coord.size(); ++i) out.push_back(coord_to_coord(coord[i], src_shape[i], dst_shape[i]));
+        return IT::tuple(out);
+    }
+    const Int idx = coord_to_index_default(coord, src_shape);
+    if (!dst_shape.is_tuple()) return IT(idx);  // index_to_coord(index, shape::Int) is the index itself (stride.jl:118-121)
+    return index_to_coord(idx, dst_shape, compact_col_major(dst_shape));
+}
+
+Layout tile_to_shape(const Layout& l, const IT& trg_shape, const IT* order) {  // layout.jl:930-935
+    const int r = rank(trg_shape);
+    if (rank(l) > r) raise(MOYE_ERR_RANK, "Cannot tile to a smaller shape");
+    const Layout padded = append(l, r);
+    const IT pshape = shape_div(product_each(trg_shape), product_each(padded.shape));
+    const Layout ord = order ? make_ordered_layout(pshape, *order) : make_layout(pshape);
+    return coalesce(blocked_product(padded, ord, false), pshape);
+}
+
+Layout make_layout_like(const Layout& l) {  // layout.jl:223-225
+    return Layout{l.shape, compact_order(filter_zeros(l.stride, l.shape), l.stride)};
 }
 
 }  // namespace host

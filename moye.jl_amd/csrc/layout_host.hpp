@@ -149,6 +149,22 @@ Tile tile_from_shape(const IT& t);        // ints -> by-mode tiler of ints
 
 // ---- tiling verbs on layouts (src/algorithm/array_algorithms.jl) ----------------------------------
 Layout local_tile(const Layout& l, const Tile& tile, const IT& coord, const IT* proj, int64_t* offset);
+
+// more IntTuple helpers (src/algorithm/tuple_algorithms.jl, src/int_tuple.jl, src/stride.jl)
+IT unflatten(const IT& flat, const IT& target);
+IT group(const IT& t, int b, int e);
+IT append_value(const IT& t, const IT& val, int n);    // n < 0: append once
+IT prepend_value(const IT& t, const IT& val, int n);
+IT zip2_by(const IT& t, const IT& guide);
+IT product_each(const IT& t);
+IT elem_scale(const IT& x, const IT& y);
+IT filter_zeros(const IT& a, const IT& x);
+bool colex_less(const IT& a, const IT& b);
+bool elem_less(const IT& a, const IT& b);
+IT increment(const IT& coord, const IT& shape);
+IT coord_to_coord(const IT& coord, const IT& src_shape, const IT& dst_shape);
+Layout tile_to_shape(const Layout& l, const IT& trg_shape, const IT* order);  // order null = GenColMajor
+Layout make_layout_like(const Layout& l);
 Layout local_partition(const Layout& l, const Tile& tile, const IT& coord_or_index, const IT* proj,
                        int64_t* offset);
 

@@ -182,6 +182,22 @@ struct TiledCopyHost {
             raise(MOYE_ERR_SHAPE, "values per thread (" + std::to_string(size(layout_tv, 2).v) +
                                       ") are not a multiple of the atom's " + std::to_string(size(val_ref, 2).v));
     }
+    // TiledCopy(atom, layout_tv, tiler) (atom/copy.jl:113-125): what make_tiled_copy_A/B/C build from a
+    // TiledMMA's layouts (atom/copy.jl:227-240)
+    TiledCopyHost(int src_bits, int dst_bits, int val_bits, const Layout& tv, const IT& tiler_mn) {
+        if (src_bits <= 0 || dst_bits <= 0 || val_bits <= 0) raise(MOYE_ERR_ARG, "bit widths must be positive");
+        const Layout bs = make_layout(tup({SI(1), SI(src_bits)})), bd = make_layout(tup({SI(1), SI(dst_bits)}));
+        val_src = upcast(bs, val_bits);
+        val_dst = upcast(bd, val_bits);
+        val_ref = val_src;
+        layout_tv = tv;
+        tiler = tiler_mn;
+        if (rank(layout_tv) != 2) raise(MOYE_ERR_RANK, "layout_tv must have a thread and a value mode");
+        if (size(layout_tv, 1).v % size(val_ref, 1).v) raise(MOYE_ERR_SHAPE, "thread count is not a multiple of the atom's");
+        if (size(layout_tv, 2).v % size(val_ref, 2).v)
+            raise(MOYE_ERR_SHAPE, "values per thread (" + std::to_string(size(layout_tv, 2).v) +
+                                      ") are not a multiple of the atom's " + std::to_string(size(val_ref, 2).v));
+    }
     Int num_val_src() const { return size(val_src, 2); }
     Int num_val_dst() const { return size(val_dst, 2); }
 
@@ -197,6 +213,28 @@ struct TiledCopyHost {
         if (rank(l) < rank(tiler)) raise(MOYE_ERR_RANK, "The dimension is too small to be tiled.");
         const Layout& trg = which == 'S' ? val_src : val_dst;
         return tile2thrfrg(zipped_divide(l, tile_from_shape(tiler)), composition(right_inverse(val_ref), trg));
+    }
+    Layout layout_TV(char which) const {  // get_layoutS_TV / get_layoutD_TV, atom/copy.jl:168-187
+        if (which != 'S' && which != 'D') raise(MOYE_ERR_ARG, "which must be 'S' or 'D'");
+        const Layout& trg = which == 'S' ? val_src : val_dst;
+        const Layout ref = make_layout(tup({tiler, SI(1)}));
+        const Layout t = tile2thrfrg(ref, composition(right_inverse(val_ref), trg));
+        return slice_layout(t, tup({IT::colon(), IT::colon(), SI(1)}));
+    }
+    Layout retile(const Layout& x) const {  // atom/copy.jl:151-166
+        const Int v = size(x, 1);
+        const Int atom_num_val = size(val_ref, 2);
+        const Int num_thr = size(layout_tv, 1);
+        const Layout frg_mn = upcast(composition(right_inverse(layout_tv), make_layout(tiler)), num_thr.v * v.v);
+        const Layout frg_v = zipped_divide(logical_product(make_layout(IT(v)), tile_of(right_inverse(frg_mn))),
+                                           tile_of(make_layout(IT(atom_num_val))));
+        std::vector<Tile> by_mode{tile_of(v)};
+        for (const IT& e : product_each(frg_mn.shape).items) by_mode.push_back(tile_of(e.leaf));
+        const Layout t_array = zipped_divide(x, tile_tuple(by_mode));
+        const Layout v_array = composition(t_array, tile_tuple({tile_of(frg_v), tile_colon()}));
+        std::vector<IT> rest{SI(1)};
+        for (int i = 1; i < rank(x); ++i) rest.push_back(IT::colon());
+        return slice_layout(v_array, tup({IT::colon(), IT::tuple(rest)}));
     }
     Layout partition(char which, const Layout& l, int64_t thr_idx, int64_t* offset) const {  // atom/copy.jl:206-214
         if (which != 'S' && which != 'D') raise(MOYE_ERR_ARG, "which must be 'S' or 'D'");
@@ -222,6 +260,11 @@ int32_t put(const std::string& s, char* out, size_t cap) {
     return MOYE_OK;
 }
 const char* nz(const char* s) { return s ? s : ""; }
+int64_t leaf_of_text(const std::string& t) {
+    const IT v = parse_int_tuple(t);
+    if (!v.is_leaf()) throw Error(MOYE_ERR_ARG, "expected an integer, got " + t);
+    return v.leaf.v;
+}
 
 template <typename F>
 int32_t guarded(F&& f) {
@@ -521,6 +564,18 @@ int32_t moye_tuple_op(const char* op_, const char* a_, const char* b_, const cha
             return put(to_string(index_to_coord(a.leaf, shp, compact_col_major(shp))), out, cap);
         }
         if (op == "iscompatible") return put(iscompatible(a, B()) ? "true" : "false", out, cap);
+        if (op == "unflatten") return put(to_string(unflatten(a, B())), out, cap);
+        if (op == "group") return put(to_string(group(a, (int)leaf_of_text(b), (int)leaf_of_text(c))), out, cap);
+        if (op == "append") return put(to_string(append_value(a, B(), c.empty() ? -1 : (int)leaf_of_text(c))), out, cap);
+        if (op == "prepend") return put(to_string(prepend_value(a, B(), c.empty() ? -1 : (int)leaf_of_text(c))), out, cap);
+        if (op == "zip2_by") return put(to_string(zip2_by(a, B())), out, cap);
+        if (op == "product_each") return put(to_string(product_each(a)), out, cap);
+        if (op == "elem_scale") return put(to_string(elem_scale(a, B())), out, cap);
+        if (op == "filter_zeros") return put(to_string(filter_zeros(a, b.empty() ? a : B())), out, cap);
+        if (op == "colex_less") return put(colex_less(a, B()) ? "true" : "false", out, cap);
+        if (op == "elem_less") return put(elem_less(a, B()) ? "true" : "false", out, cap);
+        if (op == "increment") return put(to_string(increment(a, B())), out, cap);
+        if (op == "coord_to_coord") return put(to_string(coord_to_coord(a, B(), C())), out, cap);
         throw Error(MOYE_ERR_UNSUPPORTED, "unknown tuple op \"" + op + "\"");
     });
 }
@@ -590,6 +645,8 @@ int32_t moye_tiled_copy_query(int32_t src_bits, int32_t dst_bits, int32_t val_bi
         const TiledCopyHost tc(src_bits, dst_bits, val_bits, parse_layout(thr_layout), vl.empty() ? parse_layout("_1") : parse_layout(vl));
         const std::string what = what_;
         if (what == "layout_tv") return put(to_string(tc.layout_tv), out, cap);
+        if (what == "layoutS_TV") return put(to_string(tc.layout_TV('S')), out, cap);
+        if (what == "layoutD_TV") return put(to_string(tc.layout_TV('D')), out, cap);
         if (what == "tiler") return put(to_string(tc.tiler), out, cap);
         if (what == "num_val_src") return put(to_string(IT(tc.num_val_src())), out, cap);
         if (what == "num_val_dst") return put(to_string(IT(tc.num_val_dst())), out, cap);
@@ -607,6 +664,55 @@ int32_t moye_tiled_copy_partition(int32_t src_bits, int32_t dst_bits, int32_t va
         const TiledCopyHost tc(src_bits, dst_bits, val_bits, parse_layout(thr_layout), vl.empty() ? parse_layout("_1") : parse_layout(vl));
         return put(to_string(tc.partition(which, parse_layout(layout), thr_idx, offset)), out, cap);
     });
+}
+
+int32_t moye_tiled_copy_tv_query(int32_t src_bits, int32_t dst_bits, int32_t val_bits, const char* layout_tv,
+                                 const char* tiler, const char* what_, char* out, size_t cap) {
+    MOYE_REQUIRE(layout_tv && tiler && what_);
+    return guarded([&] {
+        const TiledCopyHost tc(src_bits, dst_bits, val_bits, parse_layout(layout_tv), parse_int_tuple(tiler));
+        const std::string what = what_;
+        if (what == "layoutS_TV") return put(to_string(tc.layout_TV('S')), out, cap);
+        if (what == "layoutD_TV") return put(to_string(tc.layout_TV('D')), out, cap);
+        if (what == "num_val_src") return put(to_string(IT(tc.num_val_src())), out, cap);
+        if (what == "num_val_dst") return put(to_string(IT(tc.num_val_dst())), out, cap);
+        if (what == "size") return put(to_string(IT(size(tc.layout_tv, 1))), out, cap);
+        throw Error(MOYE_ERR_UNSUPPORTED, "unknown TiledCopy query \"" + what + "\"");
+    });
+}
+
+int32_t moye_tiled_copy_tv_partition(int32_t src_bits, int32_t dst_bits, int32_t val_bits, const char* layout_tv,
+                                     const char* tiler, int32_t thr_idx, char which, const char* layout, char* out,
+                                     size_t cap, int64_t* offset) {
+    MOYE_REQUIRE(layout_tv && tiler && layout);
+    return guarded([&] {
+        const TiledCopyHost tc(src_bits, dst_bits, val_bits, parse_layout(layout_tv), parse_int_tuple(tiler));
+        return put(to_string(tc.partition(which, parse_layout(layout), thr_idx, offset)), out, cap);
+    });
+}
+
+int32_t moye_tiled_copy_tv_retile(int32_t src_bits, int32_t dst_bits, int32_t val_bits, const char* layout_tv,
+                                  const char* tiler, const char* layout, char* out, size_t cap) {
+    MOYE_REQUIRE(layout_tv && tiler && layout);
+    return guarded([&] {
+        const TiledCopyHost tc(src_bits, dst_bits, val_bits, parse_layout(layout_tv), parse_int_tuple(tiler));
+        return put(to_string(tc.retile(parse_layout(layout))), out, cap);
+    });
+}
+
+int32_t moye_layout_tile_to_shape(const char* layout, const char* trg_shape, const char* order, char* out, size_t cap) {
+    MOYE_REQUIRE(layout && trg_shape);
+    return guarded([&] {
+        const std::string od = nz(order);
+        IT o;
+        if (!od.empty()) o = parse_int_tuple(od);
+        return put(to_string(tile_to_shape(parse_layout(layout), parse_int_tuple(trg_shape), od.empty() ? nullptr : &o)), out, cap);
+    });
+}
+
+int32_t moye_layout_make_like(const char* layout, char* out, size_t cap) {
+    MOYE_REQUIRE(layout);
+    return guarded([&] { return put(to_string(make_layout_like(parse_layout(layout))), out, cap); });
 }
 
 int32_t moye_make_tiled_mma(int32_t atom, const char* atom_layout, const char* permutation, moye_tiled_mma* out) {

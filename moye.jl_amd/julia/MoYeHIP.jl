@@ -283,6 +283,47 @@ function tiled_copy_partition(src_bits, dst_bits, val_bits, thr::Layout, val::La
     MoYeArray(pointer(x) + off[] * sizeof(T), parse_layout(unsafe_string(pointer(buf))))
 end
 
+# TiledCopy(atom, layout_tv, tiler): what make_tiled_copy_A/B/C build from a TiledMMA (src/atom/copy.jl:227-240)
+function tiled_copy_tv_query(src_bits, dst_bits, val_bits, layout_tv::Layout, tiler::Tuple, what::AbstractString)
+    buf = Vector{UInt8}(undef, CAP)
+    check(ccall((:moye_tiled_copy_tv_query, LIB), Int32,
+                (Int32, Int32, Int32, Cstring, Cstring, Cstring, Ptr{UInt8}, Csize_t),
+                Int32(src_bits), Int32(dst_bits), Int32(val_bits), string(layout_tv), string(tiler), what, buf, CAP))
+    unsafe_string(pointer(buf))
+end
+
+function tiled_copy_tv_partition(src_bits, dst_bits, val_bits, layout_tv::Layout, tiler::Tuple, thr_idx::Integer,
+                                 which::Char, x::MoYeArray{T}) where {T}
+    buf = Vector{UInt8}(undef, CAP); off = Ref{Int64}(0)
+    check(ccall((:moye_tiled_copy_tv_partition, LIB), Int32,
+                (Int32, Int32, Int32, Cstring, Cstring, Int32, Cchar, Cstring, Ptr{UInt8}, Csize_t, Ptr{Int64}),
+                Int32(src_bits), Int32(dst_bits), Int32(val_bits), string(layout_tv), string(tiler), Int32(thr_idx),
+                Cchar(which), string(MoYe.layout(x)), buf, CAP, off))
+    MoYeArray(pointer(x) + off[] * sizeof(T), parse_layout(unsafe_string(pointer(buf))))
+end
+
+"retile_S / retile_D (src/atom/copy.jl:151-166) of a fragment layout"
+function tiled_copy_tv_retile(src_bits, dst_bits, val_bits, layout_tv::Layout, tiler::Tuple, l::Layout)
+    buf = Vector{UInt8}(undef, CAP)
+    check(ccall((:moye_tiled_copy_tv_retile, LIB), Int32,
+                (Int32, Int32, Int32, Cstring, Cstring, Cstring, Ptr{UInt8}, Csize_t),
+                Int32(src_bits), Int32(dst_bits), Int32(val_bits), string(layout_tv), string(tiler), string(l), buf, CAP))
+    parse_layout(unsafe_string(pointer(buf)))
+end
+
+function tile_to_shape(l::Layout, trg_shape::Tuple, order = "")
+    buf = Vector{UInt8}(undef, CAP)
+    check(ccall((:moye_layout_tile_to_shape, LIB), Int32, (Cstring, Cstring, Cstring, Ptr{UInt8}, Csize_t),
+                string(l), string(trg_shape), string(order), buf, CAP))
+    parse_layout(unsafe_string(pointer(buf)))
+end
+
+make_layout_like(l::Layout) = @layout_call moye_layout_make_like string(l)
+
+"One wave executes the atom once through its (thr,val) tables: D(M,N) = A(M,K) * B(N,K)' on dense column-major device tiles."
+mma_atom_probe(atom::Int32, A::Ptr{Cvoid}, B::Ptr{Cvoid}, D::Ptr{Cvoid}; stream = C_NULL) =
+    check(ccall((:moye_mma_atom_probe, LIB), Int32, (Int32, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}), atom, A, B, D, stream))
+
 "A TiledCopy for the device copy: atom of `vec_bits` bits, thread and value layouts, LDS tile."
 function tiled_copy_desc(; op = COPY_UNIVERSAL, vec_bits = 128, thr = (16, 16), val = (4, 4), tiler = (64, 64))
     TiledCopyDesc(op, Int32(vec_bits), Int32.(thr), Int32.(val), Int32.(tiler), Int32(0))

@@ -18,8 +18,11 @@ from .layout import (COLON, GenColMajor, GenRowMajor, Layout, StaticInt, append,
                      flatten, index_to_coord, left_inverse, logical_divide, logical_product, make_fragment_like,
                      make_layout, make_ordered_layout, max_common_vector, prepend, raked_product, rank, recast,
                      right_inverse, shape_div, size, slice_and_offset, static, static_layout, tiled_divide,
-                     tiled_product, zipped_divide, zipped_product)
+                     tiled_product, zipped_divide, zipped_product, unflatten, group, tuple_append, tuple_prepend,
+                     zip2_by, product_each, capacity, elem_scale, filter_zeros, colex_less, elem_less, increment,
+                     coord_to_coord, iscompatible, tile_to_shape, make_layout_like)
 from .array import (CopyAtom, MoYeArray, ThrCopy, ThrMMA, TiledCopy as TiledCopyOp, TiledMMA as TiledMMAOp, copyto_,
-                    gemm_, local_partition, local_tile, make_tiled_copy, make_tiled_mma, transpose, view)
+                    gemm_, local_partition, local_tile, make_tiled_copy, make_tiled_copy_A, make_tiled_copy_B,
+                    make_tiled_copy_C, make_tiled_mma, transpose, view)
 
 __all__ = [n for n in dir() if not n.startswith("_")]

@@ -186,6 +186,20 @@ class ThrMMA:
     def partition_C(self, c):
         return self._part("C", c)
 
+    # partition_fragment_X / make_fragment_X (src/atom/mma.jl:26-47,310-337): the register-resident
+    # counterpart of a partition.  Registers have no host address, so the mirror returns the
+    # fragment's LAYOUT (what a device kernel would allocate), not an array.
+    def partition_fragment_A(self, a):
+        return L.make_fragment_like(self.partition_A(a).layout)
+
+    def partition_fragment_B(self, b):
+        return L.make_fragment_like(self.partition_B(b).layout)
+
+    def partition_fragment_C(self, c):
+        return L.make_fragment_like(self.partition_C(c).layout)
+
+    make_fragment_A, make_fragment_B, make_fragment_C = partition_fragment_A, partition_fragment_B, partition_fragment_C
+
 
 # ---- copy ------------------------------------------------------------------------------------------
 class CopyAtom:
@@ -227,6 +241,12 @@ class TiledCopy:
     def get_slice(self, thr_idx):
         return ThrCopy(self, thr_idx)
 
+    def get_layoutS_TV(self):
+        return Layout(self._q("layoutS_TV"))
+
+    def get_layoutD_TV(self):
+        return Layout(self._q("layoutD_TV"))
+
     def descriptor(self):
         d = _lib.TiledCopy()
         d.op, d.vec_bits, d.flags = self.op, self.atom.src_bits, self.flags
@@ -243,6 +263,77 @@ class TiledCopy:
 
 def make_tiled_copy(atom, thr_layout, val_layout=None, **kw):
     return TiledCopy(atom, thr_layout, val_layout, **kw)
+
+
+class TiledCopyTV:
+    """TiledCopy(atom, layout_tv, tiler) (src/atom/copy.jl:113-125), the form make_tiled_copy_A/B/C
+    produce from a TiledMMA (src/atom/copy.jl:227-240)."""
+
+    def __init__(self, atom, layout_tv, tiler):
+        self.atom, self.tiled_layout_TV, self.tiler_MN = atom, layout_tv, tuple(tiler)
+
+    def _args(self):
+        a = self.atom
+        return (a.src_bits, a.dst_bits, a.val_bits, _b(self.tiled_layout_TV.text), _b(L.tuple_text(self.tiler_MN)))
+
+    def _q(self, what):
+        return _text_out(_l().moye_tiled_copy_tv_query, *self._args(), _b(what))
+
+    def size(self):
+        return int(L.parse_tuple(self._q("size")))
+
+    def get_layoutS_TV(self):
+        return Layout(self._q("layoutS_TV"))
+
+    def get_layoutD_TV(self):
+        return Layout(self._q("layoutD_TV"))
+
+    def retile(self, x):
+        """retile_S / retile_D (src/atom/copy.jl:151-166) on a MoYeArray or a Layout."""
+        lay = x if isinstance(x, Layout) else x.layout
+        out = Layout(_text_out(_l().moye_tiled_copy_tv_retile, *self._args(), _b(lay.text)))
+        return out if isinstance(x, Layout) else x._with(out, 0)
+
+    def get_slice(self, thr_idx):
+        return ThrCopyTV(self, thr_idx)
+
+
+class ThrCopyTV:
+    def __init__(self, tiled_copy, thr_idx):
+        self.tiled_copy, self.thr_idx = tiled_copy, thr_idx
+
+    def _part(self, which, x):
+        off = C.c_int64()
+        buf = C.create_string_buffer(_CAP)
+        check(_l().moye_tiled_copy_tv_partition(*self.tiled_copy._args(), self.thr_idx, which.encode(),
+                                                _b(x.layout.text), buf, _CAP, C.byref(off)))
+        return x._with(Layout(buf.value.decode()), off.value)
+
+    def partition_S(self, s):
+        return self._part("S", s)
+
+    def partition_D(self, d):
+        return self._part("D", d)
+
+    def retile_S(self, s):
+        return self.tiled_copy.retile(s)
+
+    retile_D = retile_S
+
+
+def make_tiled_copy_A(atom, tiled_mma):
+    """src/atom/copy.jl:227-230."""
+    return TiledCopyTV(atom, tiled_mma.layout_tv("A"), (tiled_mma.tile_size(1), tiled_mma.tile_size(3)))
+
+
+def make_tiled_copy_B(atom, tiled_mma):
+    """src/atom/copy.jl:231-235."""
+    return TiledCopyTV(atom, tiled_mma.layout_tv("B"), (tiled_mma.tile_size(2), tiled_mma.tile_size(3)))
+
+
+def make_tiled_copy_C(atom, tiled_mma):
+    """src/atom/copy.jl:236-240."""
+    return TiledCopyTV(atom, tiled_mma.layout_tv("C"), (tiled_mma.tile_size(1), tiled_mma.tile_size(2)))
 
 
 class ThrCopy:

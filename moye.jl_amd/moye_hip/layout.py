@@ -137,6 +137,11 @@ def _l():
         l.moye_tiled_copy_query.argtypes = [I32, I32, I32, cs, cs, cs, cs, S]
         l.moye_tiled_copy_partition.argtypes = [I32, I32, I32, cs, cs, I32, C.c_char, cs, cs, S, I64p]
         l.moye_make_tiled_mma.argtypes = [I32, cs, cs, C.POINTER(_lib.TiledMMA)]
+        l.moye_tiled_copy_tv_query.argtypes = [I32, I32, I32, cs, cs, cs, cs, S]
+        l.moye_tiled_copy_tv_partition.argtypes = [I32, I32, I32, cs, cs, I32, C.c_char, cs, cs, S, I64p]
+        l.moye_tiled_copy_tv_retile.argtypes = [I32, I32, I32, cs, cs, cs, cs, S]
+        l.moye_layout_tile_to_shape.argtypes = [cs, cs, cs, cs, S]
+        l.moye_layout_make_like.argtypes = [cs, cs, S]
         _declared = True
     return l
 
@@ -368,3 +373,72 @@ def flat(l):
     if not isinstance(s, tuple):
         s, d = (s,), (d,)
     return [int(x) for x in s], [int(x) for x in d]
+
+
+# ---- more IntTuple helpers (src/algorithm/tuple_algorithms.jl, src/int_tuple.jl, src/stride.jl) ----
+def unflatten(flat_tuple, target):
+    return tuple_op("unflatten", flat_tuple, target)
+
+
+def group(t, b, e):
+    """group modes b..e (1-based, inclusive) — tuple_algorithms.jl:101-112."""
+    return tuple_op("group", t, b, e)
+
+
+def tuple_append(t, val, n=None):
+    return tuple_op("append", t, val, n)
+
+
+def tuple_prepend(t, val, n=None):
+    return tuple_op("prepend", t, val, n)
+
+
+def zip2_by(t, guide):
+    return tuple_op("zip2_by", t, guide)
+
+
+def product_each(t):
+    return tuple_op("product_each", t)
+
+
+def capacity(t):
+    return tuple_op("capacity", t)
+
+
+def elem_scale(x, y):
+    return tuple_op("elem_scale", x, y)
+
+
+def filter_zeros(a, x=None):
+    return tuple_op("filter_zeros", a, x)
+
+
+def colex_less(a, b):
+    return tuple_op("colex_less", a, b)
+
+
+def elem_less(a, b):
+    return tuple_op("elem_less", a, b)
+
+
+def increment(coord, shape):
+    return tuple_op("increment", coord, shape)
+
+
+def coord_to_coord(coord, src_shape, dst_shape):
+    return tuple_op("coord_to_coord", coord, src_shape, dst_shape)
+
+
+def iscompatible(a, b):
+    return tuple_op("iscompatible", a, b)
+
+
+def tile_to_shape(l, trg_shape, order=None):
+    """src/layout.jl:930-935; order None = GenColMajor."""
+    return Layout(_text_out(_l().moye_layout_tile_to_shape, _b(l.text), _b(tuple_text(trg_shape)),
+                            _b("" if order is None else tuple_text(order))))
+
+
+def make_layout_like(l):
+    """src/layout.jl:223-225."""
+    return Layout(_text_out(_l().moye_layout_make_like, _b(l.text)))

@@ -7,6 +7,8 @@ import random
 import pytest
 
 import layout_oracle as lo
+import numpy as np
+import moye_hip as mh
 import tiled_oracle as to
 from helpers import canon, load_vectors, split_top
 
@@ -395,3 +397,111 @@ def test_errors_map_to_status_codes():
     with pytest.raises(MoyeError) as e:
         ml.index_to_coord(9, (3, 4), (1, 3, 5))
     assert e.value.status == ERR_RANK
+
+
+# ---------------------------------------------------------------------------------------------
+# IntTuple helpers, tile_to_shape, make_layout_like and the TV-based TiledCopy: host vs oracle
+# ---------------------------------------------------------------------------------------------
+import numpy as np
+import moye_hip as mh
+import tiled_oracle as to
+
+
+def _o2t(x):
+    """oracle IntTuple -> text the host parses."""
+    return lo._fmt(x) if hasattr(lo, "_fmt") else str(x)
+
+
+def _same(host_value, oracle_value):
+    assert ml.tuple_text(host_value).replace(" ", "") == _o2t(oracle_value).replace(" ", ""), (host_value, oracle_value)
+
+
+def test_more_tuple_helpers_against_the_oracle():
+    S = lo.S
+    t = (S(2), (3, S(4)), ((5, 6), S(7)))
+    h = ml.parse_tuple(_o2t(t))
+    _same(ml.unflatten(ml.parse_tuple("(1,2,3,4,5,6)"), ml.parse_tuple("(0,(0,0),((0,0),0))")),
+          lo.unflatten((1, 2, 3, 4, 5, 6), (0, (0, 0), ((0, 0), 0))))
+    _same(ml.group(h, 2, 3), lo.group(t, 2, 3))
+    _same(ml.group(h, 1, 1), lo.group(t, 1, 1))
+    _same(ml.tuple_append(h, ml.StaticInt(1)), lo.append(t, S(1)))
+    _same(ml.tuple_append(h, ml.StaticInt(1), 5), lo.append(t, S(1), 5))
+    _same(ml.tuple_prepend(h, 9, 4), lo.prepend(t, 9, 4))
+    with pytest.raises(mh.MoyeError):
+        ml.tuple_append(h, 1, 2)
+    z = (((1, 2), (3, 4)), ((5, 6), (7, 8)), (9, 10))
+    _same(ml.zip2_by(ml.parse_tuple(_o2t(z)), ml.parse_tuple("((0,0),0)")), lo.zip2_by(z, ((0, 0), 0)))
+    _same(ml.product_each(h), lo.product_each(t))
+    _same(ml.elem_scale(ml.parse_tuple("(2,(3,_4))"), ml.parse_tuple("(5,((6,7),_2))")),
+          lo.elem_scale((2, (3, S(4))), (5, ((6, 7), S(2)))))
+    _same(ml.filter_zeros(ml.parse_tuple("(_0,(3,_0))"), ml.parse_tuple("(7,(8,9))")),
+          lo.filter_zeros((S(0), (3, S(0))), (7, (8, 9))))
+    _same(ml.coord_to_coord(ml.parse_tuple("(3,(2,2))"), ml.parse_tuple("(4,(2,3))"), ml.parse_tuple("(2,(6,1))")),
+          lo.coord_to_coord((3, (2, 2)), (4, (2, 3)), (2, (6, 1))))
+    # orderings and increment: all coordinates of a small hierarchical shape
+    shape = (2, (3, 2))
+    coords = [lo.index_to_coord(i, shape) for i in range(1, 13)]
+    c = coords[0]
+    for nxt in coords[1:] + coords[:1]:
+        _same(ml.increment(ml.parse_tuple(_o2t(c)), ml.parse_tuple(_o2t(shape))), lo.increment(c, shape))
+        assert lo.increment(c, shape) == nxt      # the oracle itself walks the coordinates in order
+        c = nxt
+    for a in coords[::3]:
+        for b in coords[::2]:
+            ta, tb = ml.parse_tuple(_o2t(a)), ml.parse_tuple(_o2t(b))
+            assert ml.colex_less(ta, tb) == lo.colex_less(a, b)
+            assert ml.elem_less(ta, tb) == lo.elem_less(a, b)
+    # reference known answers (test/int_tuple.jl:46-96 style)
+    assert ml.colex_less(ml.parse_tuple("(1,2,3)"), ml.parse_tuple("(1,2,4)")) is True
+    assert ml.elem_less(ml.parse_tuple("(1,2,3)"), ml.parse_tuple("(2,3,4)")) is True
+    assert ml.elem_less(ml.parse_tuple("(3,2,3)"), ml.parse_tuple("(2,3,4)")) is False
+
+
+def test_tile_to_shape_and_make_layout_like_against_the_oracle():
+    for text, trg, order in (("(_2,_2):(_1,_2)", "(_8,_6)", None), ("(_4,_2):(_2,_1)", "(_8,_8)", "(_1,_0)"),
+                             ("_4:_1", "(_8,_4,_2)", None), ("(_2,_3):(_3,_1)", "(_4,_9)", "(_0,_1)")):
+        l = lo.parse_layout(text)
+        want = lo.tile_to_shape(l, lo.parse_int_tuple(trg)) if order is None else \
+            lo.tile_to_shape(l, lo.parse_int_tuple(trg), lo.parse_int_tuple(order))
+        got = ml.tile_to_shape(ml.Layout(text), ml.parse_tuple(trg), None if order is None else ml.parse_tuple(order))
+        assert canon(got.text) == canon(str(want)), (text, trg, order)
+        # what the function is for: the result covers the target shape with copies of the block
+        assert int(lo.size(want)) == int(lo.product(lo.parse_int_tuple(trg)))
+    for text in ("(_2,(_3,_4)):(_12,(_1,_3))", "(4,_1,6):(6,_0,1)", "(_8,_8):(_8,_1)"):
+        assert canon(ml.make_layout_like(ml.Layout(text)).text) == canon(str(lo.make_layout_like(lo.parse_layout(text))))
+
+
+def test_make_tiled_copy_ABC_and_retile_against_the_oracle():
+    """make_tiled_copy_A/B/C (src/atom/copy.jl:227-240), partition_S/D and retile through the TV form."""
+    S = lo.S
+    for name, al in (("MMAOP_16x8x8_F32TF32TF32F32_TN", None), ("MMAOP_16x8x8_F16F16F16F16_TN", lo.SL((2, 2, 1))),
+                     ("MFMA_F32_16x16x32_F16", lo.SL((2, 2, 1)))):
+        op = to.REFERENCE_MMA_OPS.get(name) or to.MFMA_OPS[name]
+        omma = to.make_tiled_mma(op, al)
+        hmma = mh.TiledMMAOp(name, None if al is None else ml.Layout(str(al)))
+        vb = 32 if "TF32" in name else 16
+        oatom, hatom = to.CopyAtom(to.UniversalCopy(vb), vb), mh.CopyAtom(vb, vb)
+        for which, omake, hmake, tile in (("A", to.make_tiled_copy_A, mh.make_tiled_copy_A, (1, 3)),
+                                          ("B", to.make_tiled_copy_B, mh.make_tiled_copy_B, (2, 3)),
+                                          ("C", to.make_tiled_copy_C, mh.make_tiled_copy_C, (1, 2))):
+            otc, htc = omake(oatom, omma), hmake(hatom, hmma)
+            assert canon(htc.tiled_layout_TV.text) == canon(str(otc.tiled_layout_TV))
+            assert canon(htc.get_layoutS_TV().text) == canon(str(otc.get_layoutS_TV()))
+            assert canon(htc.get_layoutD_TV().text) == canon(str(otc.get_layoutD_TV()))
+            rows, cols = int(omma.tile_size(tile[0])), int(omma.tile_size(tile[1]))
+            buf = np.arange(rows * cols * 4, dtype=np.float32)
+            oarr = to.Array(buf, lo.make_layout((S(2 * rows), S(2 * cols))))
+            harr = mh.MoYeArray(0, mh.F32, ml.Layout("(_%d,_%d)" % (2 * rows, 2 * cols)))
+            seen = np.zeros(rows * cols * 4, dtype=np.int32)
+            for thr in range(1, int(otc.size()) + 1):
+                op_, hp_ = otc.get_slice(thr).partition_S(oarr), htc.get_slice(thr).partition_S(harr)
+                assert canon(hp_.layout.text) == canon(str(op_.layout)) and hp_.ptr == op_.offset * 4, (name, which, thr)
+                seen[op_.offsets()] += 1
+            # A is shared by the atoms along N, B by the atoms along M (src/atom/mma.jl:120-169): every element
+            # is owned that many times, C exactly once
+            mult = 1 if al is None else {"A": int(al.shape[1]), "B": int(al.shape[0]), "C": 1}[which]
+            assert (seen == mult).all(), (name, which, mult)
+            # retile of a fragment-shaped layout (atom/copy.jl:151-166)
+            frag = otc.get_slice(1).partition_D(oarr).layout
+            frag_like = lo.make_fragment_like(frag)
+            assert canon(htc.retile(ml.Layout(str(frag_like))).text) == canon(str(otc.retile(frag_like))), (name, which)

@@ -128,6 +128,15 @@ int32_t moye_copy(const moye_tiled_copy* tc, const moye_tensor* dst, const moye_
 int32_t moye_gemm(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A,
                   const moye_tensor* B, const moye_tensor* C, float alpha, void* stream);
 
+/* axpby!(a, X, b, Y) (src/algorithm/blas.jl:1-9): y[i] = iszero(b) ? a*x[i] : a*x[i] + b*y[i] over the
+ * logical elements of both layouts; X and Y have the same floating-point element type T, a and b are
+ * converted to T first, every operation is rounded in T and nothing is fused. */
+int32_t moye_axpby(double a, const moye_tensor* X, double b, const moye_tensor* Y, void* stream);
+
+/* fill!(x, value) / zeros!(x) (src/algorithm/array_algorithms.jl:158-182): value converted to x's
+ * element type */
+int32_t moye_fill(const moye_tensor* X, double value, void* stream);
+
 /* bytes of device workspace moye_gemm needs for this call (split-K partials); 0 if none.
  * The library allocates it internally on first use and keeps it. */
 int32_t moye_gemm_workspace_size(const moye_tiled_mma* mma, const moye_tensor* D,

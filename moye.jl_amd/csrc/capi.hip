@@ -157,6 +157,14 @@ int32_t moye_gemm(const moye_tiled_mma* mma, const moye_tensor* D, const moye_te
     return gemm_impl(mma, D, A, B, C, alpha, static_cast<hipStream_t>(stream));
 }
 
+int32_t moye_axpby(double a, const moye_tensor* X, double b, const moye_tensor* Y, void* stream) {
+    return axpby_dispatch(a, X, b, Y, static_cast<hipStream_t>(stream));
+}
+
+int32_t moye_fill(const moye_tensor* X, double value, void* stream) {
+    return fill_dispatch(X, value, static_cast<hipStream_t>(stream));
+}
+
 int32_t moye_gemm_workspace_size(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A,
                                  const moye_tensor* B, size_t* bytes) {
     if (!mma || !D || !A || !B || !bytes) return fail(MOYE_ERR_ARG, "moye_gemm_workspace_size: null argument");

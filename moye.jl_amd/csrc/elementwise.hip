@@ -1,0 +1,195 @@
+// axpby! and fill!/zeros! on device arrays with arbitrary layouts.
+//
+//   axpby!(a, X, b, Y)  (src/algorithm/blas.jl:1-9):  y[i] = iszero(b) ? a*x[i] : a*x[i] + b*y[i]
+//   fill!(x, val), zeros!(x)  (src/algorithm/array_algorithms.jl:158-182)
+// over the logical elements i of both layouts.  X and Y have the same element type T; a and b are
+// converted to T first and every operation is rounded in T (Julia's Float16 arithmetic computes in
+// Float32 and rounds after each operation; so does this), products and the sum never contracted
+// into an fma: the file is compiled with -ffp-contract=off.
+#include <algorithm>
+#include <cstring>
+
+#include "kernels.hpp"
+
+namespace moye {
+
+namespace {
+struct ELayout {
+    int32_t rank;
+    int64_t shape[MOYE_MAX_RANK];
+    int64_t stride[MOYE_MAX_RANK];
+};
+
+// colexicographic decomposition of a 0-based linear index (src/stride.jl:20-31)
+__device__ __forceinline__ int64_t e_offset(const ELayout& l, int64_t i) {
+    int64_t off = 0;
+#pragma unroll 1
+    for (int m = 0; m < l.rank; ++m) {
+        const int64_t s = l.shape[m], q = i / s;
+        off += (i - q * s) * l.stride[m];
+        i = q;
+    }
+    return off;
+}
+
+ELayout elayout_of(const moye_tensor& t) {
+    ELayout f;
+    f.rank = t.rank;
+    for (int i = 0; i < MOYE_MAX_RANK; ++i) {
+        f.shape[i] = i < t.rank ? t.shape[i] : 1;
+        f.stride[i] = i < t.rank ? t.stride[i] : 0;
+    }
+    return f;
+}
+
+__device__ __forceinline__ float e_bf16_round(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return f;
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return __uint_as_float(u & 0xffff0000u);
+}
+
+// element traits: load to / store from the compute type, round a compute-type value to T
+struct ElF32 {
+    typedef float compute;
+    typedef float storage;
+    static __device__ __forceinline__ float load(const float* p) { return *p; }
+    static __device__ __forceinline__ void store(float* p, float v) { *p = v; }
+    static __device__ __forceinline__ float round(float v) { return v; }
+};
+struct ElF64 {
+    typedef double compute;
+    typedef double storage;
+    static __device__ __forceinline__ double load(const double* p) { return *p; }
+    static __device__ __forceinline__ void store(double* p, double v) { *p = v; }
+    static __device__ __forceinline__ double round(double v) { return v; }
+};
+struct ElF16 {
+    typedef float compute;
+    typedef _Float16 storage;
+    static __device__ __forceinline__ float load(const _Float16* p) { return (float)*p; }
+    static __device__ __forceinline__ void store(_Float16* p, float v) { *p = (_Float16)v; }
+    static __device__ __forceinline__ float round(float v) { return (float)(_Float16)v; }
+};
+struct ElBF16 {
+    typedef float compute;
+    typedef uint16_t storage;
+    static __device__ __forceinline__ float load(const uint16_t* p) { return __uint_as_float((uint32_t)*p << 16); }
+    static __device__ __forceinline__ void store(uint16_t* p, float v) { *p = (uint16_t)(__float_as_uint(e_bf16_round(v)) >> 16); }
+    static __device__ __forceinline__ float round(float v) { return e_bf16_round(v); }
+};
+
+template <typename El>
+__global__ __launch_bounds__(256) void axpby_kernel(typename El::compute a, const typename El::storage* x, ELayout lx,
+                                                    typename El::compute b, typename El::storage* y, ELayout ly,
+                                                    int64_t n, bool b_is_zero) {
+    typedef typename El::compute T;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const T ax = El::round(a * El::load(x + e_offset(lx, i)));
+        typename El::storage* yp = y + e_offset(ly, i);
+        if (b_is_zero) {
+            El::store(yp, ax);
+        } else {
+            const T by = El::round(b * El::load(yp));
+            El::store(yp, El::round(ax + by));
+        }
+    }
+}
+
+template <int kBytes>
+__global__ __launch_bounds__(256) void fill_kernel(char* x, ELayout lx, int64_t n, uint64_t bits) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        char* p = x + e_offset(lx, i) * kBytes;
+        if constexpr (kBytes == 1) *reinterpret_cast<uint8_t*>(p) = (uint8_t)bits;
+        else if constexpr (kBytes == 2) *reinterpret_cast<uint16_t*>(p) = (uint16_t)bits;
+        else if constexpr (kBytes == 4) *reinterpret_cast<uint32_t*>(p) = (uint32_t)bits;
+        else *reinterpret_cast<uint64_t*>(p) = bits;
+    }
+}
+
+int64_t count(const moye_tensor& t) {
+    int64_t n = 1;
+    for (int i = 0; i < t.rank; ++i) n *= t.shape[i];
+    return n;
+}
+
+// host-side rounding of the scalars to T, the same way the kernels round
+float host_round_f16(float v) { return (float)(_Float16)v; }
+float host_round_bf16(float f) {
+    uint32_t u;
+    std::memcpy(&u, &f, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return f;
+    u += 0x7fffu + ((u >> 16) & 1u);
+    u &= 0xffff0000u;
+    std::memcpy(&f, &u, 4);
+    return f;
+}
+}  // namespace
+
+int32_t axpby_dispatch(double a, const moye_tensor* X, double b, const moye_tensor* Y, hipStream_t st) {
+    if (int32_t e = check_tensor(X, "X")) return e;
+    if (int32_t e = check_tensor(Y, "Y")) return e;
+    if (X->dtype != Y->dtype) return fail(MOYE_ERR_UNSUPPORTED, "axpby!: X and Y must have the same element type");
+    const int64_t n = count(*X);
+    if (count(*Y) != n) return fail(MOYE_ERR_SHAPE, "axpby!: X holds %lld elements, Y %lld", (long long)n, (long long)count(*Y));
+    if (n == 0) return MOYE_OK;
+    const dim3 grid((unsigned)std::min<int64_t>((n + 255) / 256, 256 * 16));
+    const ELayout lx = elayout_of(*X), ly = elayout_of(*Y);
+    switch (X->dtype) {
+        case MOYE_F32:
+            axpby_kernel<ElF32><<<grid, 256, 0, st>>>((float)a, static_cast<const float*>(X->ptr), lx, (float)b,
+                                                      static_cast<float*>(Y->ptr), ly, n, (float)b == 0.f);
+            break;
+        case MOYE_F64:
+            axpby_kernel<ElF64><<<grid, 256, 0, st>>>(a, static_cast<const double*>(X->ptr), lx, b,
+                                                      static_cast<double*>(Y->ptr), ly, n, b == 0.0);
+            break;
+        case MOYE_F16: {
+            const float af = host_round_f16((float)a), bf = host_round_f16((float)b);
+            axpby_kernel<ElF16><<<grid, 256, 0, st>>>(af, static_cast<const _Float16*>(X->ptr), lx, bf,
+                                                      static_cast<_Float16*>(Y->ptr), ly, n, bf == 0.f);
+            break;
+        }
+        case MOYE_BF16: {
+            const float af = host_round_bf16((float)a), bf = host_round_bf16((float)b);
+            axpby_kernel<ElBF16><<<grid, 256, 0, st>>>(af, static_cast<const uint16_t*>(X->ptr), lx, bf,
+                                                       static_cast<uint16_t*>(Y->ptr), ly, n, bf == 0.f);
+            break;
+        }
+        default:
+            return fail(MOYE_ERR_UNSUPPORTED, "axpby!: element type %s is not a floating-point type this build handles", dtype_name(X->dtype));
+    }
+    MOYE_HIP_CHECK(hipGetLastError());
+    return MOYE_OK;
+}
+
+// `value` is converted to the element type (floating-point types: round to nearest even; integer types: truncation)
+int32_t fill_dispatch(const moye_tensor* X, double value, hipStream_t st) {
+    if (int32_t e = check_tensor(X, "x")) return e;
+    const int64_t n = count(*X);
+    if (n == 0) return MOYE_OK;
+    uint64_t bits = 0;
+    switch (X->dtype) {
+        case MOYE_F32: { const float f = (float)value; uint32_t u; std::memcpy(&u, &f, 4); bits = u; break; }
+        case MOYE_F64: std::memcpy(&bits, &value, 8); break;
+        case MOYE_F16: { const _Float16 h = (_Float16)(float)value; uint16_t u; std::memcpy(&u, &h, 2); bits = u; break; }
+        case MOYE_BF16: { const float f = host_round_bf16((float)value); uint32_t u; std::memcpy(&u, &f, 4); bits = u >> 16; break; }
+        case MOYE_U8: case MOYE_U16: case MOYE_U32: case MOYE_U64: bits = (uint64_t)(int64_t)value; break;
+        default: return fail(MOYE_ERR_UNSUPPORTED, "fill!: no conversion to %s", dtype_name(X->dtype));
+    }
+    const dim3 grid((unsigned)std::min<int64_t>((n + 255) / 256, 256 * 16));
+    const ELayout lx = elayout_of(*X);
+    char* p = static_cast<char*>(X->ptr);
+    switch (dtype_bytes(X->dtype)) {
+        case 1: fill_kernel<1><<<grid, 256, 0, st>>>(p, lx, n, bits); break;
+        case 2: fill_kernel<2><<<grid, 256, 0, st>>>(p, lx, n, bits); break;
+        case 4: fill_kernel<4><<<grid, 256, 0, st>>>(p, lx, n, bits); break;
+        default: fill_kernel<8><<<grid, 256, 0, st>>>(p, lx, n, bits); break;
+    }
+    MOYE_HIP_CHECK(hipGetLastError());
+    return MOYE_OK;
+}
+
+}  // namespace moye

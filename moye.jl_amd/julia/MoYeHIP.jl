@@ -374,6 +374,24 @@ function gemm!(mma::TiledMMADesc, D::MoYeArray, A::MoYeArray, B::MoYeArray, C::U
     nothing
 end
 
+"""
+    axpby!(a, X, b, Y; stream=C_NULL)
+
+`axpby!(a, X, b, Y)` (src/algorithm/blas.jl:1-9) for device arrays of one floating-point element type.
+"""
+function axpby!(a::Real, X::MoYeArray, b::Real, Y::MoYeArray; stream::Ptr{Cvoid} = C_NULL)
+    GC.@preserve X Y check(ccall((:moye_axpby, LIB), Int32, (Cdouble, Ptr{Tensor}, Cdouble, Ptr{Tensor}, Ptr{Cvoid}),
+                                 Float64(a), Ref(Tensor(X)), Float64(b), Ref(Tensor(Y)), stream))
+    nothing
+end
+
+"`fill!(x, val)` / `zeros!(x)` (src/algorithm/array_algorithms.jl:158-182) for device arrays."
+function fill!(x::MoYeArray, val::Real; stream::Ptr{Cvoid} = C_NULL)
+    GC.@preserve x check(ccall((:moye_fill, LIB), Int32, (Ptr{Tensor}, Cdouble, Ptr{Cvoid}), Ref(Tensor(x)), Float64(val), stream))
+    x
+end
+zeros!(x::MoYeArray; stream::Ptr{Cvoid} = C_NULL) = fill!(x, 0.0; stream = stream)
+
 function gemm_workspace_size(mma::TiledMMADesc, D::MoYeArray, A::MoYeArray, B::MoYeArray)
     n = Ref{Csize_t}(0)
     check(ccall((:moye_gemm_workspace_size, LIB), Int32,

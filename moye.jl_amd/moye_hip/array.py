@@ -380,3 +380,22 @@ def gemm_(mma, D, A, B, C_=None, alpha=1.0, stream=None):
         return x if x is None or isinstance(x, _lib.Tensor) else x.tensor()
 
     device.gemm_(d, t(D), t(A), t(B), t(C_), alpha, stream)
+
+
+def axpby_(a, X, b, Y, stream=None):
+    """axpby!(a, X, b, Y) (src/algorithm/blas.jl:1-9): Y = a*X + b*Y element by element; returns Y."""
+    x = X if isinstance(X, _lib.Tensor) else X.tensor()
+    y = Y if isinstance(Y, _lib.Tensor) else Y.tensor()
+    device.axpby_(a, x, b, y, stream)
+    return Y
+
+
+def fill_(X, value, stream=None):
+    """fill!(x, value) (src/algorithm/array_algorithms.jl:158-164); returns X."""
+    device.fill_(X if isinstance(X, _lib.Tensor) else X.tensor(), value, stream)
+    return X
+
+
+def zeros_(X, stream=None):
+    """zeros!(x) (src/algorithm/array_algorithms.jl:176-182)."""
+    return fill_(X, 0.0, stream)

@@ -76,3 +76,16 @@ def mma_atom_probe(atom, a_ptr, b_ptr, d_ptr, stream=None):
     f = lib().moye_mma_atom_probe
     f.argtypes = [C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
     check(f(atom, a_ptr, b_ptr, d_ptr, stream))
+
+
+def axpby_(a, x, b, y, stream=None):
+    """axpby!(a, X, b, Y) on raw descriptors."""
+    f = lib().moye_axpby
+    f.argtypes = [C.c_double, C.c_void_p, C.c_double, C.c_void_p, C.c_void_p]
+    check(f(a, C.byref(x), b, C.byref(y), stream))
+
+
+def fill_(x, value, stream=None):
+    f = lib().moye_fill
+    f.argtypes = [C.c_void_p, C.c_double, C.c_void_p]
+    check(f(C.byref(x), value, stream))

@@ -581,6 +581,35 @@ def gemm_arrays(D, A, B, C):
     return D
 
 
+def axpby(a, X, b, Y):
+    """blas.jl:1-9 — y[i] = iszero(b) ? a*x[i] : a*x[i] + b*y[i] over the logical elements of both
+    arrays, every operation rounded in the arrays' element type (numpy's float16 arithmetic computes in
+    float32 and rounds after each operation, as Julia's does; bf16 arrays are float32 buffers holding
+    bf16 values and are rounded with round_bf16)."""
+    assert len(X) == len(Y)
+    ox, oy = X.offsets(), Y.offsets()
+    bf16 = getattr(Y, "bf16", False)
+    if bf16:
+        rnd = lambda v: round_bf16(np.asarray(v, dtype=np.float32))
+        af, bf_ = rnd(np.float32(a)), rnd(np.float32(b))
+        x, y = X.buf[ox].astype(np.float32), Y.buf[oy].astype(np.float32)
+        ax = rnd(af * x)
+        Y.buf[oy] = ax if bf_ == 0 else rnd(ax + rnd(bf_ * y))
+        return Y
+    T = Y.buf.dtype.type
+    at, bt = T(a), T(b)
+    x, y = X.buf[ox], Y.buf[oy]
+    ax = (at * x).astype(T)
+    Y.buf[oy] = ax if bt == 0 else (ax + (bt * y).astype(T)).astype(T)
+    return Y
+
+
+def fill(X, value):
+    """array_algorithms.jl:158-164 — every logical element of X becomes `value` (converted to eltype)."""
+    X.buf[X.offsets()] = X.buf.dtype.type(value)
+    return X
+
+
 def gemm_fp64(A, B):
     """The tolerance oracle: exact-input fp64 product A*B' of (M,K) and (N,K)."""
     return np.asarray(A, dtype=np.float64) @ np.asarray(B, dtype=np.float64).T

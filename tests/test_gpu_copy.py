@@ -204,3 +204,73 @@ def test_copy_errors(mh):
     assert e.value.status == mh._lib.ERR_UNSUPPORTED
     empty = torch.zeros(0, dtype=torch.int32, device="cuda")
     mh.copyto_(_tens(mh, empty, (0,), (1,)), _tens(mh, empty, (0,), (1,)))
+
+
+# ---------------------------------------------------------------------------------------------
+# axpby! and fill! / zeros! (src/algorithm/blas.jl:1-9, src/algorithm/array_algorithms.jl:158-182)
+# ---------------------------------------------------------------------------------------------
+
+AXPBY_LAYOUTS = [
+    ("(_4096)", "(_4096)"),                                      # both dense
+    ("(_64,_48):(_1,_64)", "(_64,_48):(_48,_1)"),                # column-major X into row-major Y
+    ("((_4,_8),(_2,_3)):((_1,_8),(_4,_64))", "(_32,_6):(_1,_40)"),  # hierarchical X, padded Y
+]
+
+
+@pytest.mark.parametrize("dt", ["float32", "float16", "bfloat16", "float64"])
+def test_axpby_bit_exact_against_the_oracle(mh, dt):
+    tdt = getattr(torch, dt)
+    g = torch.Generator().manual_seed(7)
+    for lx_text, ly_text in AXPBY_LAYOUTS:
+        lx, ly = lo.parse_layout(lx_text), lo.parse_layout(ly_text)
+        nx, ny = int(lo.cosize(lx)), int(lo.cosize(ly))
+        for a, b in ((1.7, 0.0), (-0.3, 2.5), (1.0 + 2.0 ** -12, 1.0)):
+            X = (torch.randn(nx, generator=g) * 3).to(tdt)
+            Y = (torch.randn(ny, generator=g) * 3).to(tdt)
+            if b == 0.0:
+                Y[::3] = float("nan")          # must be overwritten, not propagated
+            x, y = X.cuda(), Y.cuda()
+            sx, dx = _flat(lx)
+            sy, dy = _flat(ly)
+            mh.axpby_(a, _tens(mh, x, sx, dx), b, _tens(mh, y, sy, dy))
+            torch.cuda.synchronize()
+            # oracle on the same bits
+            if dt == "bfloat16":
+                ox = to.Array(X.float().numpy().copy(), lx)
+                oy = to.Array(Y.float().numpy().copy(), ly)
+                oy.bf16 = True
+                to.axpby(a, ox, b, oy)
+            else:
+                ox, oy = to.Array(X.numpy().copy(), lx), to.Array(Y.numpy().copy(), ly)
+                to.axpby(a, ox, b, oy)
+            # elements the layout does not reach keep their bits (NaN payloads included)
+            reached = torch.from_numpy(np.asarray(oy.offsets(), dtype=np.int64))
+            want = Y.clone()
+            want[reached] = torch.from_numpy(oy.buf[reached.numpy()]).to(tdt)
+            got = y.cpu()
+            itype = {2: torch.int16, 4: torch.int32, 8: torch.int64}[got.element_size()]
+            assert torch.equal(got.view(itype), want.view(itype)), (dt, lx_text, a, b)
+
+
+def test_fill_and_zeros(mh):
+    for dt, val in ((torch.float32, 3.25), (torch.float16, -1.5), (torch.bfloat16, 0.1), (torch.float64, 1e-300),
+                    (torch.int32, 77)):
+        y = torch.full((64,), 9, dtype=dt, device="cuda")
+        # a strided view: every fourth element of the first 48
+        mh.fill_(_tens(mh, y, [12], [4]), val)
+        torch.cuda.synchronize()
+        want = torch.full((64,), 9, dtype=dt)
+        want[0:48:4] = torch.tensor(val, dtype=torch.float64).to(dt) if dt != torch.int32 else 77
+        assert torch.equal(y.cpu(), want), dt
+        mh.zeros_(_tens(mh, y, [64], [1]))
+        torch.cuda.synchronize()
+        assert float(y.abs().max()) == 0.0
+
+
+def test_axpby_errors(mh):
+    x = torch.zeros(8, device="cuda")
+    y = torch.zeros(8, dtype=torch.float16, device="cuda")
+    with pytest.raises(mh.MoyeError):
+        mh.axpby_(1.0, _tens(mh, x, [8], [1]), 1.0, _tens(mh, y, [8], [1]))
+    with pytest.raises(mh.MoyeError):
+        mh.axpby_(1.0, _tens(mh, x, [8], [1]), 1.0, _tens(mh, x, [4], [1]))

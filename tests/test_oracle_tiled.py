@@ -277,3 +277,37 @@ def test_round_bf16():
         assert (to.round_bf16(t.numpy()) == t.to(torch.bfloat16).to(torch.float32).numpy()).all()
     except ImportError:
         pass
+
+
+def test_axpby_known_answers():
+    """axpby! (src/algorithm/blas.jl:1-9): hand-built cases that separate the reference's arithmetic
+    from its plausible mis-statements."""
+    f32 = np.float32
+    # b == 0 must not read Y: NaN in Y disappears (the iszero(b) branch)
+    X = to.Array(np.array([1, 2, 3], f32), lo.make_layout(S(3)))
+    Y = to.Array(np.array([np.nan, np.inf, 5], f32), lo.make_layout(S(3)))
+    to.axpby(2.0, X, 0.0, Y)
+    assert Y.buf.tolist() == [2.0, 4.0, 6.0]
+    # unfused: a*x is rounded before the add.  a = x = 1 + 2^-12: a*x = 1 + 2^-11 + 2^-24 rounds (ties to
+    # even) to 1 + 2^-11, and y = -(1 + 2^-11) cancels it exactly; an fma would leave 2^-24
+    v = f32(1 + 2.0 ** -12)
+    X = to.Array(np.array([v], f32), lo.make_layout(S(1)))
+    Y = to.Array(np.array([-(1 + 2.0 ** -11)], f32), lo.make_layout(S(1)))
+    to.axpby(float(v), X, 1.0, Y)
+    assert Y.buf[0] == 0.0
+    # fp16: every operation rounded to fp16.  a*x = 3 * 0.1(fp16) is rounded once, then b*y, then the sum
+    h = np.float16
+    X = to.Array(np.array([0.1], h), lo.make_layout(S(1)))
+    Y = to.Array(np.array([1000.0], h), lo.make_layout(S(1)))
+    to.axpby(3.0, X, 1.0, Y)
+    ax = h(h(3.0) * h(0.1))
+    assert Y.buf[0] == h(np.float32(ax) + np.float32(1000.0))
+    # through layouts: X column-major, Y row-major views of 2x3
+    X = to.Array(np.arange(6, dtype=f32), lo.make_layout((S(2), S(3))))
+    Y = to.Array(np.zeros(6, f32), lo.make_layout((S(2), S(3)), (S(3), S(1))))
+    to.axpby(1.0, X, 0.0, Y)
+    assert Y.buf.reshape(2, 3).tolist() == [[0, 2, 4], [1, 3, 5]]
+    # fill!: only the elements the layout reaches
+    Z = to.Array(np.zeros(8, f32), lo.make_layout((S(2), S(2)), (S(1), S(4))))
+    to.fill(Z, 7)
+    assert Z.buf.tolist() == [7, 7, 0, 0, 7, 7, 0, 0]

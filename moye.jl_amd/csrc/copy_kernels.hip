@@ -7,6 +7,8 @@
 //                   loads, 4x4 register transpose, XOR-swizzled LDS tile, 128-bit stores
 //   copy_flat       both sides contiguous in the same order: 128-bit streaming copy
 //   copy_generic    anything else: per-element gather/scatter with optional conversion
+#include <algorithm>
+
 #include "kernels.hpp"
 
 namespace moye {
@@ -356,7 +358,43 @@ int32_t copy_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, const m
     }
 
     // (3) generic
-    const FlatLayout ls = flat_of(*src), ld = flat_of(*dst);
+    FlatLayout ls = flat_of(*src), ld = flat_of(*dst);
+    if (same_bits) {
+        // Vectorise when the layouts allow it, which the reference computes (max_common_vector,
+        // src/layout.jl:752-761) and then leaves unused (src/algorithm/copy.jl:53-58): if logical
+        // neighbours are memory neighbours on both sides in runs of v elements, and every other stride
+        // and both pointers are multiples of v, both layouts are recast to elements of v * sizeof(T)
+        // bytes (the upcast of src/layout.jl:945-975 on flattened modes) and moved 4..16 bytes at a time.
+        const auto run = [](const FlatLayout& l) { return l.rank >= 1 && l.stride[0] == 1 ? l.shape[0] : 1; };
+        int64_t v = std::min(run(ls), run(ld));
+        // logical index i -> mode-0 coordinate i % shape[0] on each side: the runs must line up
+        if (ls.shape[0] != ld.shape[0]) v = std::__gcd(std::__gcd(ls.shape[0], ld.shape[0]), v);
+        int64_t width = 16 / sb;  // widest access in elements
+        while (width > 1) {
+            bool fits = v % width == 0 && reinterpret_cast<uintptr_t>(s) % (width * sb) == 0 &&
+                        reinterpret_cast<uintptr_t>(d) % (width * sb) == 0;
+            for (int m = 1; m < MOYE_MAX_RANK && fits; ++m)
+                fits = (ls.shape[m] == 1 || ls.stride[m] % width == 0) && (ld.shape[m] == 1 || ld.stride[m] % width == 0);
+            if (fits) break;
+            width /= 2;
+        }
+        if (width > 1 && sb * width <= 16) {
+            for (FlatLayout* l : {&ls, &ld}) {
+                l->shape[0] /= width;
+                for (int m = 1; m < MOYE_MAX_RANK; ++m) l->stride[m] /= width;
+            }
+            const int64_t nv = n / width;
+            const dim3 gv((unsigned)std::min<int64_t>((nv + 255) / 256, 256 * 64));
+            switch (sb * width) {
+                case 2: copy_generic_bits<2><<<gv, 256, 0, st>>>(s, d, ls, ld, nv); break;
+                case 4: copy_generic_bits<4><<<gv, 256, 0, st>>>(s, d, ls, ld, nv); break;
+                case 8: copy_generic_bits<8><<<gv, 256, 0, st>>>(s, d, ls, ld, nv); break;
+                default: copy_generic_bits<16><<<gv, 256, 0, st>>>(s, d, ls, ld, nv); break;
+            }
+            MOYE_HIP_CHECK(hipGetLastError());
+            return MOYE_OK;
+        }
+    }
     const dim3 g((unsigned)std::min<int64_t>((n + 255) / 256, 256 * 64));
     bool ok = true;
     if (same_bits) {

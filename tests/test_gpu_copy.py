@@ -274,3 +274,30 @@ def test_axpby_errors(mh):
         mh.axpby_(1.0, _tens(mh, x, [8], [1]), 1.0, _tens(mh, y, [8], [1]))
     with pytest.raises(mh.MoyeError):
         mh.axpby_(1.0, _tens(mh, x, [8], [1]), 1.0, _tens(mh, x, [4], [1]))
+
+
+def test_generic_copy_vectorised_paths_bit_exact(mh):
+    """Layouts whose logical neighbours are memory neighbours in runs (padded pitches, a flat source
+    into a padded destination, runs of different lengths, misaligned bases, 2-byte elements): the copy
+    may use 4..16-byte accesses, the result must not change."""
+    cases = [("(_64,_48):(_1,_64)", "(_64,_48):(_1,_80)", 0, 0),
+             ("(_3072)", "(_64,_48):(_1,_80)", 0, 0),
+             ("(_6,_8):(_1,_6)", "(_4,_12):(_1,_10)", 0, 0),
+             ("(_64,_48):(_1,_64)", "(_64,_48):(_1,_80)", 1, 0),      # source base off by one element
+             ("(_64,_48):(_1,_64)", "(_64,_48):(_1,_82)", 0, 2),      # pitch and base only 8-byte friendly
+             ("((_8,_8),_48):((_1,_16),_128)", "(_64,_48):(_1,_64)", 0, 0)]
+    for dt in (torch.int32, torch.int16):
+        for sl, dl, soff, doff in cases:
+            ls, ld = lo.parse_layout(sl), lo.parse_layout(dl)
+            ns, nd = int(lo.cosize(ls)) + soff, int(lo.cosize(ld)) + doff
+            src = _rand_bits(ns, 5).to(dt)
+            dst = torch.full((nd,), -1, dtype=dt, device="cuda")
+            sx, dx = _flat(ls)
+            sy, dy = _flat(ld)
+            mh.copyto_(_tens(mh, dst[doff:], sy, dy), _tens(mh, src[soff:], sx, dx))
+            torch.cuda.synchronize()
+            want = np.full(nd, -1, dtype=src.cpu().numpy().dtype)
+            o_src = to.Array(src.cpu().numpy()[soff:], ls)
+            o_dst = to.Array(want[doff:], ld)
+            to.copyto(o_dst, o_src)
+            assert np.array_equal(dst.cpu().numpy(), want), (dt, sl, dl, soff, doff)

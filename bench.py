@@ -226,6 +226,14 @@ def main():
                      "kernel_ms": round(kern_ms, 5)},
     }
 
+    # the matrix pipe alone on this box, same input type: what "MFMA-bound" can mean here
+    tf_r, ghz_r = mh.mfma_ceiling(mh.F16, True, 0.5)
+    tf_z, ghz_z = mh.mfma_ceiling(mh.F16, False, 0.5)
+    out["mfma_only"] = {"what": "MFMA-only loop on all CUs, fp16, no memory traffic (moye_mfma_ceiling), 0.5 s each",
+                        "random_operands": {"tflops": round(tf_r, 1), "clock_ghz": round(ghz_r, 3)},
+                        "zero_operands": {"tflops": round(tf_z, 1), "clock_ghz": round(ghz_z, 3)}}
+    out["roofline"]["frac_of_mfma_only_random"] = round(achieved / tf_r, 4)
+
     if not args.no_copy:
         n = 16384
         src = torch.randint(-2 ** 31, 2 ** 31 - 1, (n * n,), dtype=torch.int32, device="cuda")

@@ -253,6 +253,15 @@ int32_t moye_time_gemm(const moye_tiled_mma* mma, const moye_tensor* D, const mo
 int32_t moye_time_copy(const moye_tiled_copy* tc, const moye_tensor* dst, const moye_tensor* src,
                        void* stream, int32_t warmup, int32_t iters, float* ms_per_launch);
 
+/* The matrix pipe alone: every wave of every CU issues independent MFMAs of the given input type
+ * (MOYE_F16 | MOYE_BF16 | MOYE_F8E4M3 | MOYE_F32) on register operands for about `seconds`, no memory
+ * traffic.  Reports the rate and the clock the loop ran at (cycle counter over wall time); with
+ * random_operands != 0 the operands are dense pseudo-random values, else zeros.  A yardstick for the
+ * GEMM kernels' roofline fractions (the part does not hold its nominal clock under dense operands);
+ * allocates a few KiB and synchronises. */
+int32_t moye_mfma_ceiling(int32_t in_dtype, int32_t random_operands, float seconds, float* tflops,
+                          float* clock_ghz, void* stream);
+
 const char* moye_last_error(void);
 const char* moye_version(void);
 

@@ -24,6 +24,7 @@ SOURCES = {
     "gemm_mfma256.hip": [],
     "gemm_mfma256pp.hip": [],
     "gemm_mfma_skinny.hip": [],
+    "mfma_ceiling.hip": [],
     "elementwise.hip": ["-ffp-contract=off"],      # axpby!: rounded products, unfused sum
     "gemm_universal.hip": ["-ffp-contract=off"],   # UniversalFMA: mul then add, never fused
     "layout_host.cpp": ["-x", "hip"],

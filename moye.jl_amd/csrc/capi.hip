@@ -224,6 +224,11 @@ int32_t moye_time_copy(const moye_tiled_copy* tc, const moye_tensor* dst, const 
     return time_launches([&] { return copy_dispatch(tc, dst, src, st); }, st, warmup, iters, ms_per_launch);
 }
 
+int32_t moye_mfma_ceiling(int32_t in_dtype, int32_t random_operands, float seconds, float* tflops, float* clock_ghz,
+                          void* stream) {
+    return mfma_ceiling(in_dtype, random_operands, seconds, tflops, clock_ghz, static_cast<hipStream_t>(stream));
+}
+
 const char* moye_last_error(void) { return last_error().c_str(); }
 const char* moye_version(void) { return "moye_hip 0.1.0 (gfx950)"; }
 

@@ -89,3 +89,12 @@ def fill_(x, value, stream=None):
     f = lib().moye_fill
     f.argtypes = [C.c_void_p, C.c_double, C.c_void_p]
     check(f(C.byref(x), value, stream))
+
+
+def mfma_ceiling(in_dtype, random_operands=True, seconds=0.3, stream=None):
+    """(TFLOP/s, clock GHz) of an MFMA-only loop on every CU: the matrix pipe's sustained rate on this part."""
+    f = lib().moye_mfma_ceiling
+    f.argtypes = [C.c_int32, C.c_int32, C.c_float, C.POINTER(C.c_float), C.POINTER(C.c_float), C.c_void_p]
+    tf, ghz = C.c_float(), C.c_float()
+    check(f(in_dtype, 1 if random_operands else 0, seconds, C.byref(tf), C.byref(ghz), stream))
+    return tf.value, ghz.value

@@ -542,3 +542,20 @@ def test_32x32_atoms_have_no_kernel(mh):
     with pytest.raises(mh.MoyeError) as e:
         mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_32x32x16_F16, cta_tile=(128, 128, 32)), T(d), T(a), T(a))
     assert "32x32" in str(e.value)
+
+
+def test_mfma_ceiling_probe(mh):
+    """The MFMA-only yardstick: plausible numbers, and zeros never slower than dense random operands."""
+    tf_r, ghz_r = mh.mfma_ceiling(mh.F16, True, 0.2)
+    tf_z, ghz_z = mh.mfma_ceiling(mh.F16, False, 0.2)
+    print("MFMA-only fp16: random %.0f TFLOP/s at %.2f GHz, zeros %.0f TFLOP/s at %.2f GHz" % (tf_r, ghz_r, tf_z, ghz_z))
+    assert 500 < tf_r < 2600 and 500 < tf_z < 2600
+    assert 0.5 < ghz_r < 2.6 and 0.5 < ghz_z < 2.6
+    assert tf_z >= 0.95 * tf_r
+    # the rate is the clock times 1024 flop per clock per SIMD (a 16x16x32 MFMA every 16 clocks), to a few per cent
+    assert abs(tf_r / (ghz_r * 1e9 * 1024 * 1024 / 1e12) - 1) < 0.1
+    for dt, lo_, hi in ((mh.F8E4M3, 1000, 5200), (mh.F32, 50, 160), (mh.BF16, 500, 2600)):
+        tf, ghz = mh.mfma_ceiling(dt, True, 0.1)
+        assert lo_ < tf < hi and 0.5 < ghz < 2.6, (dt, tf, ghz)
+    with pytest.raises(mh.MoyeError):
+        mh.mfma_ceiling(mh.F64, True, 0.1)

@@ -116,6 +116,81 @@ static int32_t launch_transpose(const uint32_t* s, uint32_t* d, int64_t lds_, in
 }
 
 // ------------------------------------------------------------------------------------------
+// the same for 2-byte elements (fp16 / bf16 matrices)
+// ------------------------------------------------------------------------------------------
+// A 64 x 64 tile is 64 source rows (j) of 128 bytes.  Rows go to LDS as they come, 16 bytes per lane,
+// with the 16-byte chunk index XORed with j / 8; a lane then gathers the 8 values S[8c .. 8c+7][i]
+// with 2-byte LDS reads (for a wave: 8 values of i, 8 values of c -> 32 different banks) and stores them
+// as one 16-byte piece of destination row i, 8 lanes per 128-byte run.
+template <int GI>
+__global__ __launch_bounds__(256) void transpose_lds_b16(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst,
+                                                         int64_t lds_, int64_t ldd, int groups_i, int tiles_j, int sb) {
+    extern __shared__ u32x4 tile[];  // GI tiles of 64 rows x 8 chunks
+    int gi, tj;
+    tile_coords(blockIdx.x, groups_i, tiles_j, sb, &gi, &tj);
+    const int v = threadIdx.x & 7;   // 16-byte chunk inside a 128-byte run
+    const int r = threadIdx.x >> 3;  // 0..31
+
+    // ---- load: rows j = r and r + 32, elements i = 8v .. 8v+7 of each tile ----
+    const uint16_t* s = src + ((int64_t)tj * kTile + r) * lds_ + (int64_t)gi * GI * kTile + 8 * v;
+    u32x4 x[GI][2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int a = 0; a < GI; ++a)
+            x[a][h] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(s + (int64_t)(32 * h) * lds_ + a * kTile));
+#pragma unroll
+    for (int a = 0; a < GI; ++a)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int j = r + 32 * h;
+            tile[a * 512 + j * 8 + (v ^ (j >> 3))] = x[a][h];
+        }
+    __syncthreads();
+
+    // ---- store: destination rows i = r and r + 32, elements j = 8v .. 8v+7 ----
+    const uint16_t* lds16 = reinterpret_cast<const uint16_t*>(tile);
+    uint16_t* d = dst + ((int64_t)gi * GI * kTile + r) * ldd + (int64_t)tj * kTile + 8 * v;
+#pragma unroll
+    for (int a = 0; a < GI; ++a)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int i = r + 32 * h;
+            uint16_t w[8];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const int j = 8 * v + q;  // j / 8 == v
+                w[q] = lds16[a * 4096 + j * 64 + ((((i >> 3) ^ v) << 3) | (i & 7))];
+            }
+            u32x4 o;
+            o.x = w[0] | ((uint32_t)w[1] << 16);
+            o.y = w[2] | ((uint32_t)w[3] << 16);
+            o.z = w[4] | ((uint32_t)w[5] << 16);
+            o.w = w[6] | ((uint32_t)w[7] << 16);
+            __builtin_nontemporal_store(o, reinterpret_cast<u32x4*>(d + (int64_t)(a * kTile + 32 * h) * ldd));
+        }
+}
+
+template <int GI>
+static int32_t launch_transpose16(const uint16_t* s, uint16_t* d, int64_t lds_, int64_t ldd, int ti, int tj, hipStream_t st) {
+    auto kern = transpose_lds_b16<GI>;
+    constexpr int kLds = GI * kTile * kTile * 2;
+    if (kLds > 48 * 1024) {
+        static bool once = false;
+        if (!once) {
+            MOYE_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
+            once = true;
+        }
+    }
+    const int64_t groups = (int64_t)(ti / GI) * tj;
+    if (groups > 0x7fffffff) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles");
+    kern<<<(unsigned)groups, 256, kLds, st>>>(s, d, lds_, ldd, ti / GI, tj, 64);
+    MOYE_HIP_CHECK(hipGetLastError());
+    return MOYE_OK;
+}
+
+// ------------------------------------------------------------------------------------------
 // contiguous streaming copy, 16 bytes per lane per step
 // ------------------------------------------------------------------------------------------
 // each workgroup walks contiguous 16 KiB chunks (4 x 16 bytes per lane in flight): measured
@@ -326,7 +401,7 @@ int32_t copy_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, const m
         // (2) rank-2 transpose of 4-byte elements through the LDS tile
         const int tm = tc && tc->tiler_mn[0] ? tc->tiler_mn[0] : kTile;
         const int tn = tc && tc->tiler_mn[1] ? tc->tiler_mn[1] : kTile;
-        if (sb == 4 && src->rank == 2 && dst->rank == 2 && src->shape[0] == dst->shape[0] &&
+        if ((sb == 4 || sb == 2) && src->rank == 2 && dst->rank == 2 && src->shape[0] == dst->shape[0] &&
             src->shape[1] == dst->shape[1] && tm == kTile && tn == kTile) {
             const moye_tensor *a = src, *b = dst;
             bool ok = false, swap = false;
@@ -337,11 +412,20 @@ int32_t copy_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, const m
                 const int mi = swap ? 1 : 0, mj = swap ? 0 : 1;
                 const int64_t ni = a->shape[mi], nj = a->shape[mj];
                 const int64_t lds_ = a->stride[mj], ldd = b->stride[mi];
-                const bool aligned = ni % kTile == 0 && nj % kTile == 0 && lds_ % 4 == 0 && ldd % 4 == 0 &&
+                const int per16 = 16 / sb;  // elements per 16-byte access
+                const bool aligned = ni % kTile == 0 && nj % kTile == 0 && lds_ % per16 == 0 && ldd % per16 == 0 &&
                                      lds_ >= ni && ldd >= nj &&
                                      (reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d)) % 16 == 0;
                 if (aligned) {
                     const int ti = (int)(ni / kTile), tj = (int)(nj / kTile);
+                    if (sb == 2) {
+                        const uint16_t* s16 = reinterpret_cast<const uint16_t*>(s);
+                        uint16_t* d16 = reinterpret_cast<uint16_t*>(d);
+                        if (ti % 8 == 0) return launch_transpose16<8>(s16, d16, lds_, ldd, ti, tj, st);
+                        if (ti % 4 == 0) return launch_transpose16<4>(s16, d16, lds_, ldd, ti, tj, st);
+                        if (ti % 2 == 0) return launch_transpose16<2>(s16, d16, lds_, ldd, ti, tj, st);
+                        return launch_transpose16<1>(s16, d16, lds_, ldd, ti, tj, st);
+                    }
                     const uint32_t* s32 = reinterpret_cast<const uint32_t*>(s);
                     uint32_t* d32 = reinterpret_cast<uint32_t*>(d);
                     if (tc && (tc->flags & MOYE_GEMM_NO_LDS_SWIZZLE)) return launch_transpose<false, 1>(s32, d32, lds_, ldd, ti, tj, st);
@@ -353,7 +437,7 @@ int32_t copy_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, const m
         }
         if (tc && tc->op == MOYE_COPY_LDS_TILED)
             return fail(MOYE_ERR_UNSUPPORTED,
-                        "copyto!: the LDS-tiled copy needs rank-2 4-byte operands whose sizes are multiples of "
+                        "copyto!: the LDS-tiled copy needs rank-2 operands of 2- or 4-byte elements whose sizes are multiples of "
                         "64, 16-byte aligned, with the unit stride on different modes");
     }
 

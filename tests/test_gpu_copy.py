@@ -301,3 +301,28 @@ def test_generic_copy_vectorised_paths_bit_exact(mh):
             o_dst = to.Array(want[doff:], ld)
             to.copyto(o_dst, o_src)
             assert np.array_equal(dst.cpu().numpy(), want), (dt, sl, dl, soff, doff)
+
+
+@pytest.mark.parametrize("M,N", [(64, 64), (128, 192), (512, 64), (192, 128), (256, 1024), (4096, 4096)])
+def test_transpose_two_byte_elements(mh, M, N):
+    """fp16 / bf16 matrices through the 2-byte LDS tile (1, 2, 4 or 8 tiles per workgroup depending on M):
+    both orientations, padded pitches, bits compared as int16; the oracle on the small cases."""
+    src = _rand_bits(M * N, 31).to(torch.int16)
+    dst = torch.zeros(M * N, dtype=torch.int16, device="cuda")
+    tc = mh.tiled_copy_desc(op=mh.COPY_LDS_TILED, vec_bits=128, tiler=(64, 64))
+    mh.copyto_(_tens(mh, dst, (M, N), (N, 1)), _tens(mh, src, (M, N), (1, M)), tc)
+    torch.cuda.synchronize()
+    assert torch.equal(dst.view(M, N), src.view(N, M).t())
+    if M * N <= 128 * 256:
+        s = to.Array(src.cpu().numpy(), lo.make_layout((M, N), (1, M)))
+        d = to.Array(np.zeros(M * N, np.int16), lo.make_layout((M, N), (N, 1)))
+        to.copyto(d, s)
+        assert np.array_equal(d.buf, dst.cpu().numpy())
+    # the other orientation with padded pitches (multiples of 8 elements = 16 bytes)
+    lds, ldd = N + 8, M + 24
+    src2 = _rand_bits(M * lds, 32).to(torch.int16)
+    dst2 = torch.full((N * ldd,), -1, dtype=torch.int16, device="cuda")
+    mh.copyto_(_tens(mh, dst2, (M, N), (1, ldd)), _tens(mh, src2, (M, N), (lds, 1)))
+    torch.cuda.synchronize()
+    assert torch.equal(dst2.view(N, ldd)[:, :M], src2.view(M, lds)[:, :N].t())
+    assert bool((dst2.view(N, ldd)[:, M:] == -1).all())

@@ -88,6 +88,7 @@ typedef struct {
 
 #define MOYE_GEMM_NO_XCD_SWIZZLE 1   /* keep blockIdx -> tile mapping linear (for A/B studies)  */
 #define MOYE_GEMM_NO_LDS_SWIZZLE 2   /* linear LDS tiles (bank-conflict study)                  */
+#define MOYE_GEMM_NO_WORKSPACE 4      /* fail instead of transposing a non-K-major operand into the workspace */
 #define MOYE_GEMM_PINGPONG 0x100      /* 256x256 tile only: the two waves of a SIMD alternate
                                         between MFMA and memory slots, k-tiles of 64 bytes in a
                                         five-stage LDS ring (cta_tile_mnk[2] = 64 bytes of K)    */
@@ -137,8 +138,10 @@ int32_t moye_axpby(double a, const moye_tensor* X, double b, const moye_tensor* 
  * element type */
 int32_t moye_fill(const moye_tensor* X, double value, void* stream);
 
-/* bytes of device workspace moye_gemm needs for this call (split-K partials); 0 if none.
- * The library allocates it internally on first use and keeps it. */
+/* bytes of device workspace moye_gemm needs for this call: the K-major copies of MFMA operands whose
+ * unit stride is not along K (NN / NT / TT problems); 0 for TN and for UniversalFMA.  The library
+ * allocates the workspace on first use (a synchronous hipMalloc inside that one moye_gemm call), grows
+ * it when a larger call comes, and keeps it; calls that use it must not overlap on different streams. */
 int32_t moye_gemm_workspace_size(const moye_tiled_mma* mma, const moye_tensor* D,
                                  const moye_tensor* A, const moye_tensor* B, size_t* bytes);
 

@@ -62,6 +62,58 @@ static int32_t atom_input_dtype(int32_t atom) {
     }
 }
 
+// ---- workspace for operands that are not K-major -----------------------------------------------
+// The MFMA kernels read K-major operands.  An operand with its unit stride along M (or N) is first
+// transposed into a K-major copy in a workspace the library owns: allocated on first use, grown when
+// a larger operand comes, kept.  One workspace per process: calls that need it must not overlap on
+// different streams (the copy and the GEMM of one call are ordered by the stream they share).
+static std::mutex g_ws_mutex;
+static char* g_ws = nullptr;
+static size_t g_ws_bytes = 0;
+
+static int32_t ensure_workspace(size_t bytes) {
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    if (bytes <= g_ws_bytes) return MOYE_OK;
+    if (g_ws) {
+        MOYE_HIP_CHECK(hipDeviceSynchronize());
+        MOYE_HIP_CHECK(hipFree(g_ws));
+        g_ws = nullptr;
+        g_ws_bytes = 0;
+    }
+    MOYE_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&g_ws), bytes));
+    g_ws_bytes = bytes;
+    return MOYE_OK;
+}
+
+// bytes of a K-major copy of an (rows x K) operand: row pitch rounded up to 16 bytes
+static size_t kmajor_bytes(const Mat& m) {
+    const int eb = dtype_bytes(m.dtype);
+    const int64_t pitch = (m.cols * eb + 15) / 16 * 16;
+    return (size_t)(m.rows * pitch + 255) / 256 * 256;
+}
+
+static size_t gemm_workspace_bytes(const moye_tiled_mma* mma, const Mat& A, const Mat& B) {
+    if (mma->atom == MOYE_MMA_UNIVERSAL_FMA) return 0;
+    size_t n = 0;
+    if (A.cs != 1 && A.cols > 1) n += kmajor_bytes(A);
+    if (B.cs != 1 && B.cols > 1) n += kmajor_bytes(B);
+    return n;
+}
+
+// transposes `m` (unit stride along its rows index) into ws as rows x K with K contiguous and rewrites `m`
+static int32_t make_kmajor(Mat* m, char* ws, hipStream_t st) {
+    const int eb = dtype_bytes(m->dtype);
+    const int64_t pitch_e = ((m->cols * eb + 15) / 16 * 16) / eb;
+    moye_tensor src{}, dst{};
+    src.ptr = m->ptr; src.dtype = m->dtype; src.rank = 2;
+    src.shape[0] = m->rows; src.shape[1] = m->cols; src.stride[0] = m->rs; src.stride[1] = m->cs;
+    dst = src;
+    dst.ptr = ws; dst.stride[0] = pitch_e; dst.stride[1] = 1;
+    if (int32_t e = copy_dispatch(nullptr, &dst, &src, st)) return e;
+    m->ptr = ws; m->rs = pitch_e; m->cs = 1;
+    return MOYE_OK;
+}
+
 static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const moye_tensor* tA,
                          const moye_tensor* tB, const moye_tensor* tC, float alpha, hipStream_t st) {
     if (!mma) return fail(MOYE_ERR_ARG, "gemm!: null TiledMMA descriptor");
@@ -97,9 +149,24 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
     if (mma->atom == MOYE_MFMA_F32_32x32x2_F32 || mma->atom == MOYE_MFMA_F32_32x32x16_F16 ||
         mma->atom == MOYE_MFMA_F32_32x32x16_BF16 || mma->atom == MOYE_MFMA_F32_32x32x16_FP8)
         return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the 32x32 MFMA atoms are described (layouts, partitions) but the kernels issue the 16x16 forms");
-    if (K > 0 && (A.cs != 1 || B.cs != 1))
-        return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the MFMA kernels need K-major A and B (stride 1 along K, the 'TN' form)");
     if (K == 0) return fail(MOYE_ERR_SHAPE, "gemm!: K == 0");
+    // NN / NT / TT (the naming of src/arch/mma/make_mma_ops.jl:253-265): operands whose unit stride is not
+    // along K are brought to the K-major form the kernels read (one tiled transpose each)
+    if (const size_t ws_bytes = gemm_workspace_bytes(mma, A, B)) {
+        if (mma->flags & MOYE_GEMM_NO_WORKSPACE)
+            return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the MFMA kernels need K-major A and B (stride 1 along K, the 'TN' form) "
+                                              "and MOYE_GEMM_NO_WORKSPACE forbids the transposed copy");
+        if (int32_t e = ensure_workspace(ws_bytes)) return e;
+        char* ws = g_ws;
+        if (A.cs != 1 && A.cols > 1) {
+            const size_t nb = kmajor_bytes(A);
+            if (int32_t e = make_kmajor(&A, ws, st)) return e;
+            ws += nb;
+        }
+        if (B.cs != 1 && B.cols > 1) {
+            if (int32_t e = make_kmajor(&B, ws, st)) return e;
+        }
+    }
     GemmArgs g{};
     // TiledMMA.atom_layout_mnk = how many waves tile the CTA along M and N (src/atom/mma.jl:84)
     const int waves = mma->atom_layout_mnk[0] * mma->atom_layout_mnk[1];
@@ -169,6 +236,10 @@ int32_t moye_gemm_workspace_size(const moye_tiled_mma* mma, const moye_tensor* D
                                  const moye_tensor* B, size_t* bytes) {
     if (!mma || !D || !A || !B || !bytes) return fail(MOYE_ERR_ARG, "moye_gemm_workspace_size: null argument");
     *bytes = 0;
+    Mat a, b;
+    if (int32_t e = as_matrix(A, "A", &a)) return e;
+    if (int32_t e = as_matrix(B, "B", &b)) return e;
+    if (!(mma->flags & MOYE_GEMM_NO_WORKSPACE)) *bytes = gemm_workspace_bytes(mma, a, b);
     return MOYE_OK;
 }
 

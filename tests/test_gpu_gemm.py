@@ -237,8 +237,9 @@ def test_gemm_errors(mh):
     with pytest.raises(mh.MoyeError) as e:  # tile does not divide
         mh.gemm_(mma, T(d[:96]), T(a[:96]), T(b))
     assert e.value.status == E.ERR_SHAPE
-    with pytest.raises(mh.MoyeError) as e:  # M-major A is not the TN form
-        mh.gemm_(mma, T(d), T(a, (128, 64), (1, 128)), T(b))
+    with pytest.raises(mh.MoyeError) as e:  # M-major A is not the TN form, and the workspace is forbidden
+        mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(128, 128, 32), flags=E.GEMM_NO_WORKSPACE),
+                 T(d), T(a, (128, 64), (1, 128)), T(b))
     assert e.value.status == E.ERR_UNSUPPORTED
     with pytest.raises(mh.MoyeError) as e:  # wrong operand type for the atom
         a32 = a.float()
@@ -559,3 +560,57 @@ def test_mfma_ceiling_probe(mh):
         assert lo_ < tf < hi and 0.5 < ghz < 2.6, (dt, tf, ghz)
     with pytest.raises(mh.MoyeError):
         mh.mfma_ceiling(mh.F64, True, 0.1)
+
+
+# ---------------------------------------------------------------------------------------------
+# operand majors other than TN: transposed into a K-major workspace first
+# ---------------------------------------------------------------------------------------------
+
+def test_operand_majors_nn_nt_tt(mh):
+    """A with its unit stride along M and/or B with its unit stride along N (the NN / NT / TT forms of
+    src/arch/mma/make_mma_ops.jl:253-265).  Exact on integers; sizes that take the LDS-tiled transpose and
+    sizes that take the generic one; the workspace size the query announces."""
+    import ctypes as C
+    from moye_hip import _lib
+    g = torch.Generator().manual_seed(61)
+    for (M, N, K) in ((256, 384, 128), (128, 128, 96), (512, 256, 1024)):
+        A = torch.randint(-4, 5, (M, K), generator=g).to(torch.float16)
+        B = torch.randint(-4, 5, (N, K), generator=g).to(torch.float16)
+        ref = A.double() @ B.double().t()
+        a_k, b_k = A.cuda(), B.cuda()                                   # K-major
+        a_m, b_n = A.t().contiguous().cuda(), B.t().contiguous().cuda()  # M-major / N-major storage
+        for a_major, b_major in (("m", "k"), ("k", "n"), ("m", "n")):
+            ta = T(a_m, (M, K), (1, M)) if a_major == "m" else T(a_k)
+            tb = T(b_n, (N, K), (1, N)) if b_major == "n" else T(b_k)
+            d = torch.zeros(M, N, dtype=torch.float32, device="cuda")
+            mma = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 2, 1), cta_tile=(128, 128, 32))
+            nbytes = C.c_size_t(0)
+            _lib.check(_lib.lib().moye_gemm_workspace_size(C.byref(mma), C.byref(T(d)), C.byref(ta), C.byref(tb), C.byref(nbytes)))
+            want = (M * K * 2 if a_major == "m" else 0) + (N * K * 2 if b_major == "n" else 0)
+            assert want <= nbytes.value <= want + 512 + 16 * (M + N)
+            mh.gemm_(mma, T(d), ta, tb)
+            torch.cuda.synchronize()
+            assert torch.equal(d.cpu().double(), ref), (M, N, K, a_major, b_major)
+            with pytest.raises(mh.MoyeError) as e:
+                mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(128, 128, 32), flags=_lib.GEMM_NO_WORKSPACE),
+                         T(d), ta, tb)
+            assert "K-major" in str(e.value)
+
+
+def test_config1_shape_on_the_matrix_cores(mh):
+    """BASELINE config 1's operands (fp32 256^3, A and B column-major: the NN form) through the fp32 MFMA
+    atom instead of UniversalFMA: tolerance 1e-5 against fp64."""
+    M = N = K = 256
+    rng = np.random.default_rng(1001)
+    A = (rng.random((M, K), dtype=np.float32) * 2 - 1)
+    Bkn = (rng.random((K, N), dtype=np.float32) * 2 - 1)
+    a = torch.from_numpy(np.asfortranarray(A).T.copy()).cuda()       # column-major A: memory holds A' row-major
+    b = torch.from_numpy(np.asfortranarray(Bkn).T.copy()).cuda()     # column-major (K,N): memory holds (N,K) row-major
+    d = torch.zeros(N, M, device="cuda")                             # column-major C
+    mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x4_F32, atom_layout=(2, 2, 1), cta_tile=(128, 128, 16)),
+             T(d, (M, N), (1, M)), T(a, (M, K), (1, M)), T(b, (N, K), (K, 1)))
+    torch.cuda.synchronize()
+    c64 = A.astype(np.float64) @ Bkn.astype(np.float64)
+    err = to.relerr(d.t().cpu().numpy(), c64)
+    print("config1 operands on the fp32 MFMA atom: rel err %.3e" % err)
+    assert err <= 1e-5

@@ -89,6 +89,9 @@ typedef struct {
 #define MOYE_GEMM_NO_XCD_SWIZZLE 1   /* keep blockIdx -> tile mapping linear (for A/B studies)  */
 #define MOYE_GEMM_NO_LDS_SWIZZLE 2   /* linear LDS tiles (bank-conflict study)                  */
 #define MOYE_GEMM_NO_WORKSPACE 4      /* fail instead of transposing a non-K-major operand into the workspace */
+#define MOYE_GEMM_PREDICATE 0x200     /* compute residue tiles (M, N, K not multiples of the 128x128 CTA tile)
+                                        instead of failing as the reference's kernels assert; implied
+                                        when cta_tile_mnk is left to the library                        */
 #define MOYE_GEMM_PINGPONG 0x100      /* 256x256 tile only: the two waves of a SIMD alternate
                                         between MFMA and memory slots, k-tiles of 64 bytes in a
                                         five-stage LDS ring (cta_tile_mnk[2] = 64 bytes of K)    */

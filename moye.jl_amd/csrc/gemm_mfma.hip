@@ -20,7 +20,11 @@
 
 namespace moye {
 
-template <typename In, typename Out, int BM, int BN, int BKB /* bytes of K per tile row */>
+// kEdge: M, N need not be multiples of the tile and K need not be a multiple of the k-tile (only of 16
+// bytes): rows beyond M / N and k beyond K are read as zeros (the predication the reference's
+// copyto_if! is meant for, src/algorithm/copy.jl:4-16) and the epilogue stores element by element
+// inside the bounds.
+template <typename In, typename Out, int BM, int BN, int BKB /* bytes of K per tile row */, bool kEdge = false>
 __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
     constexpr int CPR = BKB / 16;                 // 16-byte chunks per tile row
     constexpr int KSTEPS = CPR / 4;               // one step = 4 chunks = one (fp8: two) MFMA k-slice
@@ -49,18 +53,31 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
     const char* a_src[A_LD];
     const char* b_src[B_LD];
     int a_dst[A_LD], b_dst[B_LD];
+    int a_lim[A_LD], b_lim[B_LD];  // kEdge: bytes of K this chunk may still read (0 for a row out of bounds)
+    const int64_t kbytes = (int64_t)p.K * In::kBytes;
 #pragma unroll
     for (int i = 0; i < A_LD; ++i) {
         const int c = tid + 256 * i, row = c / CPR, ch = c % CPR;
         a_src[i] = gA + row * kbytes_a + ch * 16;
         a_dst[i] = row * CPR + (ch ^ swz<CPR>(row));
+        a_lim[i] = (int64_t)tm * BM + row < p.M ? (int)(kbytes - ch * 16) : 0;
     }
 #pragma unroll
     for (int i = 0; i < B_LD; ++i) {
         const int c = tid + 256 * i, row = c / CPR, ch = c % CPR;
         b_src[i] = gB + row * kbytes_b + ch * 16;
         b_dst[i] = row * CPR + (ch ^ swz<CPR>(row));
+        b_lim[i] = (int64_t)tn * BN + row < p.N ? (int)(kbytes - ch * 16) : 0;
     }
+    // a chunk at byte offset koff of its row is inside the operand iff koff < lim
+    auto load_a = [&](int i, int64_t koff) -> u32x4 {
+        if (kEdge && koff >= a_lim[i]) return u32x4{0u, 0u, 0u, 0u};
+        return *reinterpret_cast<const u32x4*>(a_src[i] + koff);
+    };
+    auto load_b = [&](int i, int64_t koff) -> u32x4 {
+        if (kEdge && koff >= b_lim[i]) return u32x4{0u, 0u, 0u, 0u};
+        return *reinterpret_cast<const u32x4*>(b_src[i] + koff);
+    };
 
     f32x4 acc[MI][NI];
 #pragma unroll
@@ -68,14 +85,14 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
 #pragma unroll
         for (int j = 0; j < NI; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    const int ktiles = (int)(((int64_t)p.K * In::kBytes) / BKB);
+    const int ktiles = (int)((kbytes + BKB - 1) / BKB);
     u32x4 ra[A_LD], rb[B_LD];
 
     // prologue: tile 0 -> LDS stage 0
 #pragma unroll
-    for (int i = 0; i < A_LD; ++i) ra[i] = *reinterpret_cast<const u32x4*>(a_src[i]);
+    for (int i = 0; i < A_LD; ++i) ra[i] = load_a(i, 0);
 #pragma unroll
-    for (int i = 0; i < B_LD; ++i) rb[i] = *reinterpret_cast<const u32x4*>(b_src[i]);
+    for (int i = 0; i < B_LD; ++i) rb[i] = load_b(i, 0);
 #pragma unroll
     for (int i = 0; i < A_LD; ++i) sA0[a_dst[i]] = ra[i];
 #pragma unroll
@@ -89,9 +106,9 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
         if (more) {  // next tile: global -> registers, in flight during the MFMAs below
             const int64_t koff = (int64_t)(kt + 1) * BKB;
 #pragma unroll
-            for (int i = 0; i < A_LD; ++i) ra[i] = *reinterpret_cast<const u32x4*>(a_src[i] + koff);
+            for (int i = 0; i < A_LD; ++i) ra[i] = load_a(i, koff);
 #pragma unroll
-            for (int i = 0; i < B_LD; ++i) rb[i] = *reinterpret_cast<const u32x4*>(b_src[i] + koff);
+            for (int i = 0; i < B_LD; ++i) rb[i] = load_b(i, koff);
         }
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) {
@@ -126,6 +143,25 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
     // ---- epilogue: alpha*acc + C -> OutT -> this wave's LDS patch -> 128-bit row stores ----
     // lane holds C[m = 16 i + r16][n = 16 j + 4 kq + e], e = 0..3
     const int64_t m_base = (int64_t)tm * BM + wm0, n_base = (int64_t)tn * BN + wn0;
+    if constexpr (kEdge) {
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+            const int64_t m = m_base + 16 * i + r16;
+            if (m >= p.M) continue;
+#pragma unroll
+            for (int j = 0; j < NI; ++j) {
+                const int64_t n = n_base + 16 * j + 4 * kq;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (n + e >= p.N) continue;
+                    float x = acc[i][j][e] * p.alpha;
+                    if (p.C) x += Out::load(p.C, m * p.ldc_m + (n + e) * p.ldc_n);
+                    static_cast<OutT*>(p.D)[m * p.ldd + n + e] = Out::cvt(x);
+                }
+            }
+        }
+        return;
+    }
     constexpr int EPC = 16 / (int)sizeof(OutT);          // elements per 16-byte chunk
     constexpr int CR = WN / EPC;                         // chunks per patch row
     constexpr int PASS_MI = (sizeof(OutT) == 4 && MI > 1) ? MI / 2 : MI;  // keep the patch <= 8 KiB
@@ -171,13 +207,13 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
     }
 }
 
-template <typename In, typename Out, int BM, int BN, int BKB>
+template <typename In, typename Out, int BM, int BN, int BKB, bool kEdge = false>
 static int32_t launch(const GemmArgs& a, hipStream_t st) {
     typedef typename Out::type OutT;
     constexpr int kMain = 2 * (BM + BN) * BKB;
     constexpr int kEpi = (sizeof(OutT) == 4 && BM / 32 > 1 ? BM / 2 : BM) * BN * (int)sizeof(OutT);
     constexpr int kLds = kMain > kEpi ? kMain : kEpi;
-    auto kern = gemm_mfma_tn<In, Out, BM, BN, BKB>;
+    auto kern = gemm_mfma_tn<In, Out, BM, BN, BKB, kEdge>;
     if (kLds > 64 * 1024) {
         static bool once = false;  // raising the dynamic LDS cap is per function, idempotent
         if (!once) {
@@ -191,12 +227,12 @@ static int32_t launch(const GemmArgs& a, hipStream_t st) {
     return MOYE_OK;
 }
 
-template <typename In, int BM, int BN, int BKB>
+template <typename In, int BM, int BN, int BKB, bool kEdge = false>
 static int32_t launch_out(int32_t out_dt, const GemmArgs& a, hipStream_t st) {
     switch (out_dt) {
-        case MOYE_F32: return launch<In, OutF32, BM, BN, BKB>(a, st);
-        case MOYE_F16: return launch<In, OutF16, BM, BN, BKB>(a, st);
-        case MOYE_BF16: return launch<In, OutBF16, BM, BN, BKB>(a, st);
+        case MOYE_F32: return launch<In, OutF32, BM, BN, BKB, kEdge>(a, st);
+        case MOYE_F16: return launch<In, OutF16, BM, BN, BKB, kEdge>(a, st);
+        case MOYE_BF16: return launch<In, OutBF16, BM, BN, BKB, kEdge>(a, st);
         default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: MFMA kernels write f32, f16 or bf16, not %s", dtype_name(out_dt));
     }
 }
@@ -206,8 +242,10 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
                               GemmArgs a, hipStream_t st) {
     const int eb = dtype_bytes(in_dt);
     // a short A (at most 64 rows) is a bandwidth problem: stream B once, no CTA tiling
-    if ((bm == 0 && bn == 0 && a.M <= 64) || (bm == a.M && bm <= 64 && bn == 16))
+    if ((bm == 0 && bn == 0 && a.M <= 64 && a.M % 16 == 0 && a.N % 16 == 0 && ((int64_t)a.K * eb) % 64 == 0) ||
+        (bm == a.M && bm <= 64 && bn == 16))
         return gemm_mfma_skinny_dispatch(in_dt, out_dt, a, st);
+    const bool chosen_here = bm == 0 && bn == 0;
     if (bm == 0 && bn == 0) {
         // the library chooses: one 256x256 tile per CU when that fills the chip, else 128x128
         const bool big = a.M % 256 == 0 && a.N % 256 == 0 && a.K % (128 / eb) == 0 &&
@@ -240,9 +278,28 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         return fail(MOYE_ERR_UNSUPPORTED,
                     "gemm!: no MFMA kernel for CTA tile %dx%dx%d (%s); built: 128x128x{%d,%d} and 256x256x%d", bm, bn,
                     bk_elems, dtype_name(in_dt), 64 / eb, 128 / eb, 128 / eb);
-    if (a.M % bm || a.N % bn || a.K % bk_elems)
-        return fail(MOYE_ERR_SHAPE, "gemm!: CTA tile %dx%dx%d does not divide the problem %dx%dx%d", bm, bn,
-                    bk_elems, a.M, a.N, a.K);
+    if (a.M % bm || a.N % bn || a.K % bk_elems) {
+        // the reference's kernels assert divisibility; residue tiles are computed when the caller asks for
+        // predication or leaves the tile choice to the library
+        if (!chosen_here && !(a.xcd_swizzle & MOYE_GEMM_PREDICATE))
+            return fail(MOYE_ERR_SHAPE, "gemm!: CTA tile %dx%dx%d does not divide the problem %dx%dx%d", bm, bn,
+                        bk_elems, a.M, a.N, a.K);
+        if (((int64_t)a.K * eb) % 16)
+            return fail(MOYE_ERR_SHAPE, "gemm!: the predicated MFMA kernel needs K to be a multiple of %d elements (16 bytes), got %d",
+                        16 / eb, a.K);
+        if ((a.lda * eb) % 16 || (a.ldb * eb) % 16 ||
+            (reinterpret_cast<uintptr_t>(a.A) | reinterpret_cast<uintptr_t>(a.B)) % 16)
+            return fail(MOYE_ERR_ALIGN, "gemm!: operands of the MFMA kernels need 16-byte aligned pointers and row pitches");
+        a.tiles_m = (a.M + 127) / 128;
+        a.tiles_n = (a.N + 127) / 128;
+        switch (in_dt) {
+            case MOYE_F16: return launch_out<InF16, 128, 128, 64, true>(out_dt, a, st);
+            case MOYE_BF16: return launch_out<InBF16, 128, 128, 64, true>(out_dt, a, st);
+            case MOYE_F8E4M3: return launch_out<InFP8, 128, 128, 64, true>(out_dt, a, st);
+            case MOYE_F32: return launch_out<InF32, 128, 128, 64, true>(out_dt, a, st);
+            default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: no MFMA atom for %s inputs", dtype_name(in_dt));
+        }
+    }
     if (misaligned)
         return fail(MOYE_ERR_ALIGN, "gemm!: operands of the MFMA kernels need 16-byte aligned pointers and row pitches");
     a.tiles_m = a.M / bm;

@@ -614,3 +614,34 @@ def test_config1_shape_on_the_matrix_cores(mh):
     err = to.relerr(d.t().cpu().numpy(), c64)
     print("config1 operands on the fp32 MFMA atom: rel err %.3e" % err)
     assert err <= 1e-5
+
+
+# ---------------------------------------------------------------------------------------------
+# residue tiles: M, N, K that the CTA tile does not divide
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("M,N,K", [(100, 130, 40), (129, 127, 72), (17, 300, 200), (384, 250, 64), (1, 1, 8), (255, 257, 1032)])
+def test_residue_tiles_predicated(mh, M, N, K):
+    """cta_tile left to the library (or MOYE_GEMM_PREDICATE with an explicit 128x128 tile): rows beyond M / N
+    and k beyond K are read as zeros, stores stay inside D.  Exact on integers; the frame around D untouched."""
+    from moye_hip import _lib
+    g = torch.Generator().manual_seed(M * 7 + N)
+    A = torch.randint(-4, 5, (M, K), generator=g).to(torch.float16)
+    B = torch.randint(-4, 5, (N, K), generator=g).to(torch.float16)
+    C = torch.randint(-9, 10, (M, N), generator=g).float()
+    a, b, c = A.cuda(), B.cuda(), C.cuda()
+    ref = A.double() @ B.double().t()
+    for kw in (dict(cta_tile=(0, 0, 0)), dict(cta_tile=(128, 128, 32), flags=_lib.GEMM_PREDICATE)):
+        for out_dt in (torch.float32, torch.float16):
+            big = torch.full((M + 2, N + 3), 77.0, dtype=out_dt, device="cuda")     # D is a window of a larger buffer
+            d = big[1:M + 1, 2:N + 2]
+            mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, **kw), T(d), T(a), T(b), T(c.to(out_dt).contiguous()), 1.0)
+            torch.cuda.synchronize()
+            assert torch.equal(d.cpu().double(), (ref + C.double()).to(out_dt).double()), (M, N, K, kw, out_dt)
+            frame = big.clone()
+            frame[1:M + 1, 2:N + 2] = 77.0
+            assert bool((frame == 77.0).all()), "stores outside D"
+    with pytest.raises(mh.MoyeError) as e:      # an explicit tile without the flag keeps the reference's assertion
+        mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(128, 128, 32)),
+                 T(torch.zeros(M, N, device="cuda")), T(a), T(b))
+    assert e.value.status == _lib.ERR_SHAPE or (M % 128 == 0 and N % 128 == 0 and K % 32 == 0)

@@ -182,6 +182,7 @@ int32_t moye_layout_make_fragment_like(const char* layout, char* out, size_t cap
 int32_t moye_layout_slice(const char* layout, const char* coord, char* out, size_t cap, int64_t* offset); /* slice_and_offset, layout.jl:368-371 */
 int32_t moye_layout_make(const char* shape, int32_t row_major, char* out, size_t cap);
 int32_t moye_layout_tile_to_shape(const char* layout, const char* trg_shape, const char* order, char* out, size_t cap); /* layout.jl:930-935; order "" = GenColMajor */
+int32_t moye_layout_print(const char* layout, char* out, size_t cap);                       /* print_layout, print.jl:7-44: the index table of a rank-2 layout as text */
 int32_t moye_layout_make_like(const char* layout, char* out, size_t cap);                   /* make_layout_like, layout.jl:223-225 */        /* make_layout(shape, GenColMajor|GenRowMajor), layout.jl:154-159 */
 
 /* IntTuple helpers (src/int_tuple.jl, src/stride.jl, src/algorithm/tuple_algorithms.jl) on tuple text such as

@@ -710,6 +710,30 @@ int32_t moye_layout_tile_to_shape(const char* layout, const char* trg_shape, con
     });
 }
 
+int32_t moye_layout_print(const char* layout, char* out, size_t cap) {  // print_layout, print.jl:7-44
+    MOYE_REQUIRE(layout);
+    return guarded([&] {
+        const Layout l = parse_layout(layout);
+        if (rank(l) != 2) throw Error(MOYE_ERR_RANK, "print_layout takes a rank-2 layout");
+        const int64_t rows = size(l, 1).v, cols = size(l, 2).v;
+        const int w = (int)std::to_string(cosize(l).v).size() + 2;
+        auto lpad = [](const std::string& t, int n) { return (int)t.size() >= n ? t : std::string((size_t)n - t.size(), ' ') + t; };
+        std::string sep = "    ";
+        for (int64_t n = 0; n < cols; ++n) sep += "+" + std::string((size_t)w, '-');
+        sep += "+";
+        std::string r = to_string(l) + "\n    ";
+        for (int64_t n = 1; n <= cols; ++n) r += "  " + lpad(std::to_string(n), w - 2) + " ";
+        for (int64_t m = 1; m <= rows; ++m) {
+            r += "\n" + sep + "\n" + lpad(std::to_string(m), 2) + "  ";
+            for (int64_t n = 1; n <= cols; ++n)
+                r += "| " + lpad(std::to_string(eval(l, tup({IT(D(m)), IT(D(n))})).v), w - 2) + " ";
+            r += "|";
+        }
+        r += "\n" + sep;
+        return put(r, out, cap);
+    });
+}
+
 int32_t moye_layout_make_like(const char* layout, char* out, size_t cap) {
     MOYE_REQUIRE(layout);
     return guarded([&] { return put(to_string(make_layout_like(parse_layout(layout))), out, cap); });

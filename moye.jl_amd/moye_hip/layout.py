@@ -142,6 +142,7 @@ def _l():
         l.moye_tiled_copy_tv_retile.argtypes = [I32, I32, I32, cs, cs, cs, cs, S]
         l.moye_layout_tile_to_shape.argtypes = [cs, cs, cs, cs, S]
         l.moye_layout_make_like.argtypes = [cs, cs, S]
+        l.moye_layout_print.argtypes = [cs, cs, S]
         _declared = True
     return l
 
@@ -442,3 +443,13 @@ def tile_to_shape(l, trg_shape, order=None):
 def make_layout_like(l):
     """src/layout.jl:223-225."""
     return Layout(_text_out(_l().moye_layout_make_like, _b(l.text)))
+
+
+def print_layout(l, file=None):
+    """print_layout(layout) (src/print.jl:7-44): the index table of a rank-2 layout; returns the text."""
+    buf = C.create_string_buffer(1 << 20)
+    check(_l().moye_layout_print(_b(l.text), buf, 1 << 20))
+    text = buf.value.decode()
+    if file is not False:
+        print(text, file=file)
+    return text

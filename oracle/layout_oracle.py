@@ -1199,6 +1199,21 @@ def make_fragment_like(l):
 _TOK = re.compile(r"\s*(_?-?\d+|[(),:])")
 
 
+def print_layout(layout):
+    """print.jl:7-44 — the rank-2 index table, as a string (lines joined by newlines, no trailing newline).
+    Cells hold the 1-based index; the column width follows the number of digits of cosize."""
+    assert lrank(layout) == 2
+    idx_width = len(str(int(cosize(layout)))) + 2
+    sep = "    " + ("+" + "-" * idx_width) * int(size(layout, 2)) + "+"
+    lines = [str(layout), "    " + "".join("  " + str(n).rjust(idx_width - 2) + " " for n in range(1, int(size(layout, 2)) + 1))]
+    for m in range(1, int(size(layout, 1)) + 1):
+        lines.append(sep)
+        lines.append(str(m).rjust(2) + "  " + "".join("| " + str(int(layout((m, n)))).rjust(idx_width - 2) + " "
+                                                         for n in range(1, int(size(layout, 2)) + 1)) + "|")
+    lines.append(sep)
+    return "\n".join(lines)
+
+
 def parse_int_tuple(text):
     toks = _TOK.findall(text)
     if "".join(toks) != re.sub(r"\s+", "", text):

@@ -505,3 +505,15 @@ def test_make_tiled_copy_ABC_and_retile_against_the_oracle():
             frag = otc.get_slice(1).partition_D(oarr).layout
             frag_like = lo.make_fragment_like(frag)
             assert canon(htc.retile(ml.Layout(str(frag_like))).text) == canon(str(otc.retile(frag_like))), (name, which)
+
+
+def test_host_print_layout_matches_the_reference_docstrings():
+    import json
+    import os
+    tables = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "print_layout_tables.json")))
+    for t in tables:
+        text = ml.print_layout(ml.Layout(t["layout"]), file=False)
+        assert [line.rstrip() for line in text.split("\n")] == t["lines"], t["expression"]
+        assert text == lo.print_layout(lo.parse_layout(t["layout"]))
+    with pytest.raises(MoyeError):
+        ml.print_layout(ml.Layout("(_2,_2,_2)"), file=False)

@@ -287,3 +287,15 @@ def test_divide_of_config_shapes():
 def test_text_roundtrip():
     for text in ["(_2, (_1, _6)):(_1, (_6, _2))", "(4,):(2,)", "_12:_1", "((1, (2, 4)), 1):((_1, (1, 2)), 8)"]:
         assert repr(lo.parse_layout(text)) == text
+
+
+def test_print_layout_matches_the_reference_docstrings():
+    """The print_layout outputs the reference keeps in its docstrings (src/layout.jl), verbatim: pins the
+    text format of src/print.jl:7-44 and, once more, the index every cell holds."""
+    import json
+    import os
+    tables = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "print_layout_tables.json")))
+    assert len(tables) == 10
+    for t in tables:
+        got = [line.rstrip() for line in lo.print_layout(lo.parse_layout(t["layout"])).split("\n")]
+        assert got == t["lines"], t["expression"]

@@ -233,6 +233,15 @@ def main():
                         "random_operands": {"tflops": round(tf_r, 1), "clock_ghz": round(ghz_r, 3)},
                         "zero_operands": {"tflops": round(tf_z, 1), "clock_ghz": round(ghz_z, 3)}}
     out["roofline"]["frac_of_mfma_only_random"] = round(achieved / tf_r, 4)
+    # the same kernel on all-zero operands: same instructions, same traffic, no toggling data -> the clock the
+    # power controller allows is higher; the difference to `achieved` is what dense operands cost on this part
+    Az, Bz = torch.zeros_like(A), torch.zeros_like(B)
+    t_ramp = time.perf_counter()
+    while time.perf_counter() - t_ramp < 0.3:
+        mh.time_gemm(mma, tD, tensor_of(Az), tensor_of(Bz), None, 1.0, stream, warmup=0, iters=50)
+    zms = mh.time_gemm(mma, tD, tensor_of(Az), tensor_of(Bz), None, 1.0, stream, warmup=0, iters=max(args.steps, 10))
+    out["roofline"]["same_kernel_zero_operands_tflops"] = round(flops / (zms * 1e-3) / 1e12, 1)
+    del Az, Bz
 
     if not args.no_copy:
         n = 16384

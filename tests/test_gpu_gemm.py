@@ -645,3 +645,33 @@ def test_residue_tiles_predicated(mh, M, N, K):
         mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(128, 128, 32)),
                  T(torch.zeros(M, N, device="cuda")), T(a), T(b))
     assert e.value.status == _lib.ERR_SHAPE or (M % 128 == 0 and N % 128 == 0 and K % 32 == 0)
+
+
+# ---------------------------------------------------------------------------------------------
+# byte offsets beyond 2^31 and 2^32
+# ---------------------------------------------------------------------------------------------
+
+def test_large_offsets_gemm_and_transpose(mh):
+    """D of 49152 x 49152 fp16 (4.5 GiB) with K = 64: tile and row offsets exceed 2^32 bytes; and a 2-byte
+    transpose of 65536 x 32768 (4 GiB each side).  Sampled against closed forms."""
+    M = N = 49152
+    K = 64
+    g = torch.Generator().manual_seed(3)
+    A = torch.randint(-3, 4, (M, K), generator=g).to(torch.float16)
+    B = torch.randint(-3, 4, (N, K), generator=g).to(torch.float16)
+    a, b = A.cuda(), B.cuda()
+    d = torch.empty(M, N, dtype=torch.float16, device="cuda")
+    mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 4, 1), cta_tile=(256, 256, 64)), T(d), T(a), T(b))
+    torch.cuda.synchronize()
+    for r0 in (0, 20000, M - 256):
+        ref = A[r0:r0 + 256].double() @ B.double().t()
+        assert torch.equal(d[r0:r0 + 256].cpu().double(), ref), r0
+    del d
+    R, Cn = 65536, 32768
+    src = torch.arange(R * Cn, dtype=torch.int64, device="cuda").to(torch.int16)   # wraps: value = index mod 2^16
+    dst = torch.empty_like(src)
+    mh.copyto_(T(dst, (R, Cn), (Cn, 1)), T(src, (R, Cn), (1, R)))
+    torch.cuda.synchronize()
+    sv, dv = src.view(Cn, R), dst.view(R, Cn)
+    for (i, j) in ((0, 0), (R - 64, Cn - 64), (40000, 17000), (65000, 100)):
+        assert torch.equal(dv[i:i + 64, j:j + 64], sv[j:j + 64, i:i + 64].t()), (i, j)

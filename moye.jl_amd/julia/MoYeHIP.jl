@@ -80,6 +80,12 @@ const MFMA_F32_16x16x32_FP8 = Int32(5)
 const MFMA_F32_32x32x16_FP8 = Int32(6)
 const MFMA_F32_16x16x4_F32 = Int32(7)
 const MFMA_F32_32x32x2_F32 = Int32(8)
+# moye_tiled_mma.flags
+const GEMM_NO_XCD_SWIZZLE = Int32(1)
+const GEMM_NO_LDS_SWIZZLE = Int32(2)
+const GEMM_NO_WORKSPACE = Int32(4)      # fail instead of transposing NN/NT/TT operands into the workspace
+const GEMM_PINGPONG = Int32(0x100)      # 256x256 tile: ping-pong schedule over a five-stage LDS ring
+const GEMM_PREDICATE = Int32(0x200)     # compute residue tiles instead of asserting divisibility
 const COPY_UNIVERSAL = Int32(0)
 const COPY_LDS_TILED = Int32(1)
 
@@ -433,6 +439,20 @@ function device_info()
     check(ccall((:moye_device_info, LIB), Int32, (Ptr{UInt8}, Csize_t, Ptr{Int32}, Ptr{Int32}, Ptr{Csize_t}),
                 name, 256, cu, khz, mem))
     (name = unsafe_string(pointer(name)), compute_units = cu[], clock_khz = khz[], total_mem = Int(mem[]))
+end
+
+"(TFLOP/s, GHz) of an MFMA-only loop on every CU: what the matrix pipe sustains on this part for this input type."
+function mfma_ceiling(in_dtype::Int32; random_operands::Bool = true, seconds::Real = 0.3, stream = C_NULL)
+    tf = Ref{Cfloat}(0); ghz = Ref{Cfloat}(0)
+    check(ccall((:moye_mfma_ceiling, LIB), Int32, (Int32, Int32, Cfloat, Ptr{Cfloat}, Ptr{Cfloat}, Ptr{Cvoid}),
+                in_dtype, Int32(random_operands), Float32(seconds), tf, ghz, stream))
+    (tflops = tf[], clock_ghz = ghz[])
+end
+
+function print_layout(l::Layout)
+    buf = Vector{UInt8}(undef, 1 << 20)
+    check(ccall((:moye_layout_print, LIB), Int32, (Cstring, Ptr{UInt8}, Csize_t), string(l), buf, 1 << 20))
+    println(unsafe_string(pointer(buf)))
 end
 
 "Average milliseconds per launch of the same gemm! call, HIP events on `stream`."

@@ -366,6 +366,12 @@ LDSM = {
                           SL((32, (32, 2)), (32, (1, 1024)))),
     "LDSM_U32x4_N": _ldsm("LDSM_U32x4_N", SL((32, 128), (128, 1)),
                           SL((32, (32, 4)), (32, (1, 1024)))),
+    "LDSM_U16x2_T": _ldsm("LDSM_U16x2_T", SL(((8, 4), 128), ((128, 0), 1)),
+                          SL(((4, 8), (16, 2)), ((256, 16), (1, 128)))),
+    "LDSM_U16x4_T": _ldsm("LDSM_U16x4_T", SL(((16, 2), 128), ((128, 0), 1)),
+                          SL(((4, 8), (16, 2, 2)), ((256, 16), (1, 128, 1024)))),
+    "LDSM_U16x8_T": _ldsm("LDSM_U16x8_T", SL((32, 128), (128, 1)),
+                          SL(((4, 8), (16, 2, 4)), ((256, 16), (1, 128, 1024)))),
 }
 
 

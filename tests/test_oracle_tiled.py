@@ -189,6 +189,68 @@ def test_tiled_copy_roundtrips():
         to.make_tiled_copy(to.CopyAtom(to.LDSM[name], 16), SL((16, 2)), SL((2, 4)))
 
 
+def _ldmatrix(nmat, trans, ptrs, mem):
+    """What PTX `ldmatrix.sync.aligned.m8n8.x{nmat}[.trans].b16` does for one warp, written from the
+    instruction's definition and not from the reference's layouts: thread 8i+r supplies the
+    address of row r of matrix i (8 contiguous b16 values); thread t receives from every matrix
+    the two values at (row t//4, columns 2(t%4), 2(t%4)+1), or of the transposed matrix."""
+    out = np.zeros((32, 2 * nmat), mem.dtype)
+    for t in range(32):
+        for i in range(nmat):
+            for v in range(2):
+                r, c = (2 * (t % 4) + v, t // 4) if trans else (t // 4, 2 * (t % 4) + v)
+                out[t, 2 * i + v] = mem[ptrs[8 * i + r] + c]
+    return out
+
+
+def _ldmatrix_copy_kernel(smem_layout, tc, n, nmat, trans):
+    """test/device/tiled_copy.jl:2-22 for one warp, with the shared->register step done by the
+    instruction model above: every thread passes the address of each 8-value source slice of its
+    partition_S and stores what it receives through its partition_D."""
+    g_in = np.arange(1, n + 1, dtype=np.uint16)
+    g_out = np.zeros(n, np.uint16)
+    smem = to.Array(g_in.copy(), smem_layout, memspace="smem")
+    gout = to.Array(g_out, smem_layout)
+    src, dst = [], []
+    for tid in range(1, 33):
+        thr = tc.get_slice(tid)
+        src.append(thr.partition_S(smem).offsets())
+        dst.append(thr.partition_D(gout).offsets())
+    natoms = len(src[0]) // 8
+    assert len(dst[0]) == natoms * 2 * nmat
+    for k in range(natoms):
+        for t in range(32):  # a row handed to the instruction is 16 contiguous bytes
+            assert (np.diff(src[t][8 * k:8 * k + 8]) == 1).all()
+        regs = _ldmatrix(nmat, trans, [int(src[t][8 * k]) for t in range(32)], smem.buf)
+        for t in range(32):
+            g_out[dst[t][2 * nmat * k:2 * nmat * (k + 1)]] = regs[t]
+    return g_in, g_out
+
+
+@pytest.mark.parametrize("name,nmat", [("LDSM_U32x1_N", 1), ("LDSM_U32x2_N", 2), ("LDSM_U32x4_N", 4)])
+def test_ldmatrix_tiled_copy_roundtrips(name, nmat):
+    """test/device/tiled_copy.jl:56-90: `cu_g_out == cu_g_in` for the three ldmatrix atoms on both
+    shared layouts of that file."""
+    atom = to.CopyAtom(to.LDSM[name], 16)
+    g_in, g_out = _ldmatrix_copy_kernel(SL((32, 32), (1, 32)), to.make_tiled_copy(atom, SL((16, 2)), SL((2, 4))),
+                                        1024, nmat, False)
+    assert (g_in == g_out).all()
+    g_in, g_out = _ldmatrix_copy_kernel(SL((32, (2, 4)), (2, (1, 64))),
+                                        to.make_tiled_copy(atom, SL((32, 1)), SL((1, 8))), 256, nmat, False)
+    assert (g_in == g_out).all()
+
+
+@pytest.mark.parametrize("name,nmat", [("LDSM_U16x2_T", 1), ("LDSM_U16x4_T", 2), ("LDSM_U16x8_T", 4)])
+def test_ldmatrix_trans_tiled_copy_roundtrips(name, nmat):
+    """traits/ldmatrix.jl:22-41 has no test in the reference; the same round trip pins the tables.
+    The transposing atoms want the shared tile contiguous along the mode the registers do not
+    run along, so the tiles here are row-major and the values run down the rows."""
+    tc = to.make_tiled_copy(to.CopyAtom(to.LDSM[name], 16), SL((4, 8)), SL((8, 1)))
+    for layout, n in ((SL((32, 8), (8, 1)), 256), (SL((32, 32), (32, 1)), 1024)):
+        g_in, g_out = _ldmatrix_copy_kernel(layout, tc, n, nmat, True)
+        assert (g_in == g_out).all()
+
+
 def test_plain_copyto():
     """test/copy.jl:5-99."""
     x = to.Array(np.arange(1, 9, dtype=np.int32), lo.make_layout((4, 2)))

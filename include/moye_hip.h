@@ -95,6 +95,9 @@ typedef struct {
 #define MOYE_GEMM_PINGPONG 0x100      /* 256x256 tile only: the two waves of a SIMD alternate
                                         between MFMA and memory slots, k-tiles of 64 bytes in a
                                         five-stage LDS ring (cta_tile_mnk[2] = 64 bytes of K)    */
+#define MOYE_GEMM_WAVE4 0x400         /* 256x256 tile only: four waves with 128x128 wave tiles, one
+                                        per SIMD, the same five-stage ring; fp8 on the 16x16x128
+                                        MFMA (cta_tile_mnk[2] = 64 bytes of K, 128 for fp8)      */
 
 /* copy ops: UniversalCopy (src/arch/copy/copy.jl:26-51); the LDS-staged forms stand where the
  * reference has cp.async (copy_async.jl:8-24) and ldmatrix (ldmatrix.jl:18-48) */

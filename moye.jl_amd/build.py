@@ -23,6 +23,7 @@ SOURCES = {
     "gemm_mfma.hip": [],
     "gemm_mfma256.hip": [],
     "gemm_mfma256pp.hip": [],
+    "gemm_mfma256w4.hip": [],
     "gemm_mfma_skinny.hip": [],
     "mfma_ceiling.hip": [],
     "elementwise.hip": ["-ffp-contract=off"],      # axpby!: rounded products, unfused sum

@@ -265,12 +265,14 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
     if (bm == 256 && bn == 256) {
         if (bkb != 128 && bkb != 64)
             return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the 256x256 MFMA kernels take %d or %d elements of K per tile", 64 / eb, 128 / eb);
-        const int kmult = (a.xcd_swizzle & MOYE_GEMM_PINGPONG) ? 64 / eb : 128 / eb;
+        const int kmult = (a.xcd_swizzle & MOYE_GEMM_WAVE4) ? (in_dt == MOYE_F8E4M3 ? 128 : 64 / eb)
+                          : (a.xcd_swizzle & MOYE_GEMM_PINGPONG) ? 64 / eb : 128 / eb;
         if (a.M % 256 || a.N % 256 || a.K % kmult)
             return fail(MOYE_ERR_SHAPE, "gemm!: CTA tile 256x256x%d does not divide the problem %dx%dx%d", kmult,
                         a.M, a.N, a.K);
         if (misaligned)
             return fail(MOYE_ERR_ALIGN, "gemm!: operands of the MFMA kernels need 16-byte aligned pointers and row pitches");
+        if (a.xcd_swizzle & MOYE_GEMM_WAVE4) return gemm_mfma_tn_256_w4_dispatch(in_dt, out_dt, a, st);
         if (a.xcd_swizzle & MOYE_GEMM_PINGPONG) return gemm_mfma_tn_256_pp_dispatch(in_dt, out_dt, a, st);
         return gemm_mfma_tn_256_dispatch(in_dt, out_dt, a, waves, stages, st);
     }

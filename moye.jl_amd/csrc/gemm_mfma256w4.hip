@@ -1,0 +1,338 @@
+// gemm! on the matrix cores, one wave per SIMD: one 256 x 256 CTA tile per compute unit, four waves
+// as 2 x 2, wave tile 128 x 128 (8 x 8 MFMA tiles, 256 accumulator registers per lane, pinned in
+// the AccVGPR file), operand tiles with 64-byte rows in a ring of five 32 KiB LDS stages filled by
+// load-to-LDS instructions.
+//
+// Why this shape: a 128 x 128 wave tile needs 16 fragments for 64 MFMAs (0.25 per MFMA; a
+// 128 x 64 wave tile needs 0.375), and with one wave per SIMD the only workgroup-wide rendezvous
+// is one s_barrier per k-step of 64 MFMAs.  Nothing else may hold the matrix pipe up, so the
+// order of every instruction in the k-loop is fixed in the source:
+//  * the MFMAs are inline assembly (their order is kept, and their "+a" constraints keep all 256
+//    accumulators in AccVGPRs: with the builtins the register allocator moved accumulators
+//    between the two register files, more copies than MFMAs);
+//  * fragments are single-buffered and refilled in place: a fragment register is reloaded (for
+//    the next k-step) right after the last MFMA of this k-step that reads it, and the MFMAs are
+//    ordered so that every refill has at least 14 MFMAs (224 clocks) before its first use:
+//      first half   rows 0-3, column by column      A0-3 are free after the last column
+//      second half  row 4, row 5, then rows 6 and 7 column by column: B_j is free after its pair
+//    the next k-step starts column by column again, so B_j is needed 4j MFMAs in;
+//  * the fragment reads are inline assembly as well, with hand-placed s_waitcnt: the compiler's
+//    wait-count pass drains every LDS read at the top of the loop once sixteen are in flight
+//    across the back edge, and puts vmcnt(0) in front of LDS reads that follow load-to-LDS
+//    instructions; neither is acceptable here.  The waits: the barrier's (all reads back, eight
+//    MFMAs after the last one was issued), and partial ones in front of the first two columns;
+//  * the loads of the stage(s) five ahead are spread evenly over the MFMAs that follow the barrier.
+// A k-step is one stage (64 bytes of K) for f16/bf16/f32 and two stages for fp8, whose MFMA
+// (16x16x128, 32 bytes per lane and operand) is the only fp8 form that runs at twice the
+// 16-bit rate on gfx950.
+//
+// Ring: step s reads the fragments of step s+1 out of LDS, so when every wave has passed the
+// barrier of step s (which sits after the MFMAs that consumed the last refills of step s-1) the
+// stages of step s are free and receive the data five stages ahead.  Before the barrier a wave
+// waits until its own share of step s+1 has landed: all but the youngest 5 - 2 SPS stages' loads.
+//
+// Operand conventions as in gemm_mfma256.hip: K-major A and B, N-contiguous D, the MFMA issued
+// with B rows as its first operand so a lane holds four consecutive n of one m; the 16-byte chunk
+// index of an LDS row is XORed with (row / 2) % 4, applied on the global side of the load-to-LDS.
+#include <type_traits>
+#include <utility>
+
+#include "mfma_epilogue.hpp"
+
+#ifndef W4_EXP  // 0: the kernel; 1 and 2 drop the loads or the fragment reads for timing studies (wrong results)
+#define W4_EXP 0
+#endif
+namespace moye {
+
+typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
+
+template <class F, int... Ps>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Ps...>) {
+    (f(std::integral_constant<int, Ps>{}), ...);
+}
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>), in order
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+// The ND load-to-LDS instructions a wave issues per k-step go out evenly over the 56 MFMA positions
+// that follow the barrier (positions 8..63).  Returns the index of the load issued after MFMA P, or -1.
+constexpr int dma_index(int P, int ND) {
+    for (int k = 0; k < ND; ++k)
+        if (8 + k * 56 / ND == P) return k;
+    return -1;
+}
+
+// The same pointer, provably wave-uniform (an "s" operand of inline assembly is not legalised:
+// a uniform value the compiler happened to compute in vector registers would be passed as is).
+__device__ __forceinline__ const char* uniform_ptr(const char* p) {
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<const char*>(((uint64_t)hi << 32) | lo);
+}
+
+// 16 bytes from LDS byte address `addr` + OFF.  The compiler does not know that the result is in
+// flight: the caller waits (s_waitcnt lgkmcnt) before the first use.
+template <int OFF>
+__device__ __forceinline__ u32x4 lds_read16(uint32_t addr) {
+    u32x4 v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+    return v;
+}
+
+// fragment = what one lane feeds to one MFMA group per operand; SPS = ring stages per k-step
+struct W4F16 {
+    static constexpr int kBytes = 2, SPS = 1;
+    typedef u32x4 frag;
+    static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) {
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    }
+};
+struct W4BF16 {
+    static constexpr int kBytes = 2, SPS = 1;
+    typedef u32x4 frag;
+    static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) {
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    }
+};
+// 32 bytes per lane: the chunk of stage 0 and the chunk of stage 1 of the k-step.  Which 32 of the
+// 128 k-values a lane carries does not matter as long as A and B agree, and they do.
+struct W4FP8 {
+    static constexpr int kBytes = 1, SPS = 2;
+    struct frag { u32x4 lo, hi; };
+    static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) {
+        const u32x8 a8 = __builtin_shufflevector(a.lo, a.hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        const u32x8 b8 = __builtin_shufflevector(b.lo, b.hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(a8), "v"(b8));
+    }
+};
+// element j of the chunk goes to MFMA j (see InF32)
+struct W4F32 {
+    static constexpr int kBytes = 4, SPS = 1;
+    typedef u32x4 frag;
+    static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) {
+        asm volatile(
+            "v_mfma_f32_16x16x4_f32 %0, %1, %5, %0\n\tv_mfma_f32_16x16x4_f32 %0, %2, %6, %0\n\t"
+            "v_mfma_f32_16x16x4_f32 %0, %3, %7, %0\n\tv_mfma_f32_16x16x4_f32 %0, %4, %8, %0"
+            : "+a"(c)
+            : "v"(a.x), "v"(a.y), "v"(a.z), "v"(a.w), "v"(b.x), "v"(b.y), "v"(b.z), "v"(b.w));
+    }
+};
+
+template <typename In, typename Out>
+__global__ __launch_bounds__(256) void gemm_mfma_tn_256_w4(GemmArgs p) {
+    constexpr int BM = 256, BN = 256, CPR = 4, STAGES = 5, SPS = In::SPS;
+    constexpr int STAGE = (BM + BN) * CPR;  // in 16-byte chunks
+    constexpr int MI = 8, NI = 8, LD = 4;  // per wave and stage: 4 load-to-LDS instructions per operand
+    typedef typename In::frag frag;
+
+    extern __shared__ u32x4 smem[];
+
+    int tm, tn;
+    tile_of_block(p, &tm, &tn);
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * 128;
+    const int r16 = lane & 15, kq = lane >> 4;
+
+    const int64_t pitch_a = (int64_t)p.lda * In::kBytes, pitch_b = (int64_t)p.ldb * In::kBytes;
+    // LDS stage (32 KiB) = A tile (256 rows of 64 bytes) then B tile.  Lane l of a load-to-LDS
+    // instruction lands in physical chunk l % 4 of row l / 4 of a 16-row group; wave w brings rows
+    // 64 w .. 64 w + 63 of each operand.
+    const int lrow = wave * 64 + (lane >> 2), lch = (lane & 3) ^ swz<CPR>(lane >> 2);
+    const char* const a_tile = static_cast<const char*>(p.A) + (int64_t)tm * BM * pitch_a;  // uniform
+    const char* const b_tile = static_cast<const char*>(p.B) + (int64_t)tn * BN * pitch_b;
+    constexpr uint32_t kStageBytes = STAGE * 16, kATileBytes = BM * CPR * 16;
+
+    f32x4 acc[MI][NI];
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int nstages = (int)(((int64_t)p.K * In::kBytes) / 64);
+    const int nsteps = nstages / SPS;
+    frag fa[MI], fb[NI];
+
+    typedef __attribute__((address_space(3))) void* lptr_t;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(lptr_t)smem;  // LDS byte address of the ring
+    // Load-to-LDS instruction Q (0..3: A, 4..7: B) of this wave's share of a stage, in the scalar-base
+    // form: a uniform 64-bit pointer to the stage's first row plus a per-lane 32-bit offset that never
+    // changes, so no vector ALU work is left in the loop.  M0 carries the LDS destination of the
+    // instruction's first lane.
+    uint32_t voff[2 * LD];
+#pragma unroll
+    for (int q = 0; q < 2 * LD; ++q)
+        voff[q] = (uint32_t)((lrow + 16 * (q % LD)) * (q < LD ? pitch_a : pitch_b) + lch * 16);
+    auto dma1 = [&](int g, int ring_slot, auto qc) __attribute__((always_inline)) {
+        constexpr int Q = decltype(qc)::value;
+        const char* const base = uniform_ptr((Q < LD ? a_tile : b_tile) + (int64_t)g * 64);
+        const uint32_t dst = __builtin_amdgcn_readfirstlane(lds0 + ring_slot * kStageBytes + (Q < LD ? 0 : kATileBytes) +
+                                                            (uint32_t)(wave * 64 + 16 * (Q % LD)) * 64);
+        const uint32_t lane_off = voff[Q];  // (a captured array element cannot be an asm operand of a generic lambda)
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(base), "s"(dst)
+                     : "memory");
+    };
+#define MOYE_VMCNT(N) (((N) & 0xF) | (((N) >> 4) << 14))
+    // bare s_barrier: __syncthreads() would add a fence that drains the prefetch
+#define MOYE_BARRIER()                      \
+    {                                       \
+        asm volatile("" ::: "memory");      \
+        __builtin_amdgcn_s_barrier();       \
+        asm volatile("" ::: "memory");      \
+    }
+    // LDS byte addresses of this lane's fragment chunk in ring slot 0; 16-row block BLK adds 1024 BLK
+    const uint32_t frag_lane = (uint32_t)(r16 * 64 + ((kq ^ swz<CPR>(r16)) * 16));
+    const uint32_t fa_byte = lds0 + wm0 * 64 + frag_lane;
+    const uint32_t fb_byte = lds0 + kATileBytes + wn0 * 64 + frag_lane;
+    // the fragment of 16-row block BLK for the k-step whose stages start at byte offsets o0 (, o1)
+    auto load_frag = [&](frag& f, uint32_t base, auto blk_c, uint32_t o0, uint32_t o1) __attribute__((always_inline)) {
+        constexpr int OFF = 1024 * decltype(blk_c)::value;
+        if constexpr (SPS == 1) {
+            f = lds_read16<OFF>(base + o0);
+        } else {
+            f.lo = lds_read16<OFF>(base + o0);
+            f.hi = lds_read16<OFF>(base + o1);
+        }
+    };
+#define MOYE_BLK(N) std::integral_constant<int, (N)> {}
+
+    // prologue: all five stages requested, wait for the first k-step's
+#pragma unroll
+    for (int g = 0; g < STAGES; ++g)
+        if (g < nstages) {
+            static_for<2 * LD>([&](auto qc) __attribute__((always_inline)) { dma1(g, g, qc); });
+        }
+    if (nstages >= STAGES) __builtin_amdgcn_s_waitcnt(MOYE_VMCNT(2 * LD * (STAGES - SPS)) | 0x0F70);
+    else __builtin_amdgcn_s_waitcnt(0x0F70);
+    MOYE_BARRIER()
+    static_for<MI>([&](auto ic) __attribute__((always_inline)) {
+        load_frag(fa[decltype(ic)::value], fa_byte, ic, 0, kStageBytes);
+        if (decltype(ic)::value == 3) __builtin_amdgcn_s_waitcnt(0xC07F);  // at most 15 reads in flight
+    });
+    static_for<NI>([&](auto jc) __attribute__((always_inline)) {
+        load_frag(fb[decltype(jc)::value], fb_byte, jc, 0, kStageBytes);
+        if (decltype(jc)::value == 3) __builtin_amdgcn_s_waitcnt(0xC07F);
+    });
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+
+    // position P of the 64 MFMA groups of a k-step -> (i, j)
+#define MOYE_I(P) ((P) < 32 ? (P) % 4 : (P) < 40 ? 4 : (P) < 48 ? 5 : 6 + ((P) & 1))
+#define MOYE_J(P) ((P) < 32 ? (P) / 4 : (P) < 48 ? (P) % 8 : ((P) - 48) / 2)
+    int slot = 0;  // ring slot of the first stage of step s
+    // One k-step.  MORE: step s+1 exists (its fragments are read); AHEAD: the stages five ahead exist
+    // (they are requested, and the stages allowed to stay in flight at the barrier are the full 5 - 2 SPS).
+    // Fragment reads in program order: A0 A1 A2 A3 (after MFMA 28..31) A4 (39) A5 (47) B0 (49) B1 (51)
+    // B2 B3 B4 B5 B6 (61) A6 (62) A7 B7 (63); the next k-step needs B_j at MFMA 4 j, A0-3 at 0..3.
+    auto step = [&](auto more_c, auto ahead_c, int s) __attribute__((always_inline)) {
+        constexpr bool MORE = decltype(more_c)::value, AHEAD = decltype(ahead_c)::value;
+        int slot_n = slot + SPS;  // first stage of step s+1
+        if (slot_n >= STAGES) slot_n -= STAGES;
+        const uint32_t o0 = (uint32_t)slot_n * kStageBytes;
+        const uint32_t o1 = (uint32_t)(slot_n + 1 == STAGES ? 0 : slot_n + 1) * kStageBytes;
+        const int g_new = s * SPS + STAGES;  // first global stage requested in this step
+        static_for<64>([&](auto pc) __attribute__((always_inline)) {
+            constexpr int P = decltype(pc)::value;
+            constexpr int i = MOYE_I(P), j = MOYE_J(P);
+            // B0 is followed by 9 fragment reads, B1 by 8; a stricter count costs nothing where the older
+            // reads are hundreds of clocks old (fp8: two reads per fragment, 32-clock MFMAs)
+            if (P == 0) __builtin_amdgcn_s_waitcnt(0xC07F | ((9 * SPS < 12 ? 9 * SPS : 12) << 8));
+            if (P == 4) __builtin_amdgcn_s_waitcnt(0xC07F | ((8 * SPS < 12 ? 8 * SPS : 12) << 8));
+            In::mma(fb[j], fa[i], acc[i][j]);
+            if (P == 7) {
+                // my share of step s+1 has landed and all my fragment reads have returned (the last were
+                // issued eight MFMAs ago); after the barrier that holds for everybody
+                if (AHEAD) {
+                    __builtin_amdgcn_s_waitcnt(MOYE_VMCNT(2 * LD * (STAGES - 2 * SPS)) | 0x0070);
+                } else {
+                    // stages requested so far: min(nstages, g_new); needed: all below (s+2) SPS
+                    const int allow = min(nstages, g_new) - (s + 2) * SPS;
+                    if (allow >= 2) __builtin_amdgcn_s_waitcnt(MOYE_VMCNT(2 * LD * 2) | 0x0070);
+                    else if (allow == 1) __builtin_amdgcn_s_waitcnt(MOYE_VMCNT(2 * LD) | 0x0070);
+                    else __builtin_amdgcn_s_waitcnt(0x0070);
+                }
+                MOYE_BARRIER()
+            }
+            if constexpr (dma_index(P, 2 * LD * SPS) >= 0) {
+                constexpr int q = dma_index(P, 2 * LD * SPS);  // 0 .. 2 LD SPS - 1
+                // in the drain a k-step of two stages may still have its first stage to request
+                if (W4_EXP != 1 && (AHEAD || g_new + q / (2 * LD) < nstages)) {
+                    int sl = slot + q / (2 * LD);
+                    if (sl >= STAGES) sl -= STAGES;
+                    dma1(g_new + q / (2 * LD), sl, std::integral_constant<int, q % (2 * LD)>{});
+                }
+            }
+            if (MORE && W4_EXP != 2) {
+                if constexpr (P >= 28 && P < 32) load_frag(fa[P - 28], fa_byte, MOYE_BLK(P - 28), o0, o1);
+                if constexpr (P == 39) load_frag(fa[4], fa_byte, MOYE_BLK(4), o0, o1);
+                if constexpr (P == 47) load_frag(fa[5], fa_byte, MOYE_BLK(5), o0, o1);
+                if constexpr (P == 62) load_frag(fa[6], fa_byte, MOYE_BLK(6), o0, o1);
+                if constexpr (P == 63) load_frag(fa[7], fa_byte, MOYE_BLK(7), o0, o1);
+                if constexpr (P >= 48 && (P & 1)) load_frag(fb[(P - 48) / 2], fb_byte, MOYE_BLK((P - 48) / 2), o0, o1);
+            }
+        });
+        slot = slot_n;
+    };
+    typedef std::integral_constant<bool, true> yes;
+    typedef std::integral_constant<bool, false> no;
+    int s = 0;
+    for (; s * SPS + STAGES + SPS <= nstages; ++s) step(yes{}, yes{}, s);
+    for (; s + 1 < nsteps; ++s) step(yes{}, no{}, s);
+    step(no{}, no{}, s);
+#undef MOYE_BLK
+#undef MOYE_I
+#undef MOYE_J
+#undef MOYE_VMCNT
+#undef MOYE_BARRIER
+    // the accumulators were written by instructions the compiler did not see: let the last ones
+    // retire before anything reads them
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    __syncthreads();  // every wave is done with the operand ring before it becomes C patches
+
+    store_c_tile<Out, MI, NI>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
+}
+
+template <typename In, typename Out>
+static int32_t launch256_w4(const GemmArgs& a, hipStream_t st) {
+    constexpr int kLds = 5 * (256 + 256) * 64;  // all 160 KiB
+    auto kern = gemm_mfma_tn_256_w4<In, Out>;
+    static bool once = false;
+    if (!once) {
+        MOYE_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
+        once = true;
+    }
+    kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n)), dim3(256), kLds, st>>>(a);
+    MOYE_HIP_CHECK(hipGetLastError());
+    return MOYE_OK;
+}
+
+template <typename In>
+static int32_t launch256_w4_out(int32_t out_dt, const GemmArgs& a, hipStream_t st) {
+    switch (out_dt) {
+        case MOYE_F32: return launch256_w4<In, OutF32>(a, st);
+        case MOYE_F16: return launch256_w4<In, OutF16>(a, st);
+        case MOYE_BF16: return launch256_w4<In, OutBF16>(a, st);
+        default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: MFMA kernels write f32, f16 or bf16, not %s", dtype_name(out_dt));
+    }
+}
+
+// 256 x 256 tile, four waves; K a multiple of 64 bytes (128 for fp8); the caller has checked
+// divisibility of M and N and alignment.
+int32_t gemm_mfma_tn_256_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, hipStream_t st) {
+    a.tiles_m = a.M / 256;
+    a.tiles_n = a.N / 256;
+    // the load-to-LDS addresses are a uniform base plus a 32-bit lane offset
+    const int eb = dtype_bytes(in_dt);
+    if (256 * a.lda * eb >= (int64_t)1 << 32 || 256 * a.ldb * eb >= (int64_t)1 << 32)
+        return fail(MOYE_ERR_SHAPE, "gemm!: row pitch too large for the 256x256 MFMA kernel");
+    switch (in_dt) {
+        case MOYE_F16: return launch256_w4_out<W4F16>(out_dt, a, st);
+        case MOYE_BF16: return launch256_w4_out<W4BF16>(out_dt, a, st);
+        case MOYE_F8E4M3: return launch256_w4_out<W4FP8>(out_dt, a, st);
+        case MOYE_F32: return launch256_w4_out<W4F32>(out_dt, a, st);
+        default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: no MFMA atom for %s inputs", dtype_name(in_dt));
+    }
+}
+
+}  // namespace moye

@@ -25,6 +25,7 @@ GMEM, SMEM, RMEM = range(3)
  MFMA_F32_32x32x2_F32) = range(9)
 COPY_UNIVERSAL, COPY_LDS_TILED = 0, 1
 GEMM_NO_XCD_SWIZZLE, GEMM_NO_LDS_SWIZZLE, GEMM_NO_WORKSPACE, GEMM_PINGPONG, GEMM_PREDICATE = 1, 2, 4, 0x100, 0x200
+GEMM_WAVE4 = 0x400
 
 
 class MoyeError(RuntimeError):

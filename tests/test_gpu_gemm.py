@@ -313,6 +313,63 @@ def test_pingpong_schedule_random(mh):
     assert torch.equal(d, d2)
 
 
+def test_wave4_schedule_exact_on_integers(mh):
+    """MOYE_GEMM_WAVE4: four waves with 128x128 wave tiles, fragments refilled in place, hand-placed
+    waits.  Small integers make every sum exact, so any fragment read too early, any stage
+    overwritten too soon or any misplaced accumulator shows as a wrong integer.  K from one
+    k-step to many: the prologue, the steady state and the drain each have their own wait counts."""
+    from moye_hip import _lib
+    g = torch.Generator().manual_seed(17)
+    cases = [(torch.float16, mh.MFMA_F32_16x16x32_F16, 32), (torch.bfloat16, mh.MFMA_F32_16x16x32_BF16, 32),
+             (torch.float32, mh.MFMA_F32_16x16x4_F32, 16)]
+    if hasattr(torch, "float8_e4m3fn"):
+        cases.append((torch.float8_e4m3fn, mh.MFMA_F32_16x16x32_FP8, 128))
+    for in_dt, atom, bk in cases:
+        for (M, N, kt) in ((256, 256, 1), (256, 512, 2), (512, 256, 3), (256, 256, 4), (256, 256, 5), (256, 256, 6),
+                           (256, 256, 7), (512, 768, 37)):
+            K = kt * bk
+            A = torch.randint(-3, 4, (M, K), generator=g).float()
+            B = torch.randint(-3, 4, (N, K), generator=g).float()
+            C = torch.randint(-8, 9, (M, N), generator=g).float()
+            a, b, c = A.to(in_dt).cuda(), B.to(in_dt).cuda(), C.cuda()
+            d = torch.zeros(M, N, dtype=torch.float32, device="cuda")
+            mma = mh.tiled_mma_desc(atom, atom_layout=(2, 2, 1), cta_tile=(256, 256, bk), flags=_lib.GEMM_WAVE4)
+            print("wave4", in_dt, M, N, K, flush=True)
+            mh.gemm_(mma, T(d), T(a), T(b), T(c), 2.0)
+            torch.cuda.synchronize()
+            assert torch.equal(d.cpu().double(), 2.0 * (A.double() @ B.double().t()) + C.double()), (in_dt, M, N, K)
+
+
+def test_wave4_schedule_random(mh):
+    from moye_hip import _lib
+    M = N = K = 2048
+    g = torch.Generator().manual_seed(18)
+    A = (torch.randn(M, K, generator=g) * K ** -0.5).half()
+    B = (torch.randn(N, K, generator=g) * K ** -0.5).half()
+    a, b = A.cuda(), B.cuda()
+    d = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+    d2 = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+    mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 2, 1), cta_tile=(256, 256, 32),
+                               flags=_lib.GEMM_WAVE4), T(d), T(a), T(b))
+    mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 4, 1), cta_tile=(256, 256, 64)), T(d2), T(a), T(b))
+    torch.cuda.synchronize()
+    c64 = a.double() @ b.double().t()
+    assert relerr(d, c64) <= TOL16
+    # both schedules add the same products in the same k order within a lane
+    assert torch.equal(d, d2)
+    if hasattr(torch, "float8_e4m3fn"):
+        x = torch.randn(M, K, generator=g)
+        w = torch.randn(N, K, generator=g)
+        sa, sb = float(x.abs().max()) / 448.0, float(w.abs().max()) / 448.0
+        qa, qb = (x / sa).to(torch.float8_e4m3fn).cuda(), (w / sb).to(torch.float8_e4m3fn).cuda()
+        o = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
+        mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_FP8, atom_layout=(2, 2, 1), cta_tile=(256, 256, 128),
+                                   flags=_lib.GEMM_WAVE4), T(o), T(qa), T(qb), None, sa * sb)
+        torch.cuda.synchronize()
+        c64 = (qa.double() @ qb.double().t()) * (sa * sb)
+        assert relerr(o, c64) <= TOL16
+
+
 @pytest.mark.parametrize("tdt,atom", [("float16", "MFMA_F32_16x16x32_F16"), ("bfloat16", "MFMA_F32_16x16x32_BF16")])
 def test_256_tile_variants(mh, tdt, atom):
     """column-major D, C accumulation and alpha through the 256x256 kernel; one k-tile and many."""

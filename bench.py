@@ -138,7 +138,7 @@ def other_configs(mh, tensor_of, torch, stream):
         qa, qb = (x / sa).to(torch.float8_e4m3fn), (w / sb).to(torch.float8_e4m3fn)
         del x, w
         d = torch.zeros(n, n, dtype=torch.bfloat16, device="cuda")
-        run("fp8 e4m3 TN 8192^3, per-tensor scales, bf16 out, CTA 256x256x128", mh.MFMA_F32_16x16x32_FP8, qa, qb, d,
+        run("fp8 e4m3 TN 8192^3, per-tensor scales, bf16 out, CTA 256x256x128 (v_mfma_f32_16x16x128_f8f6f4)", mh.MFMA_F32_16x16x32_FP8, qa, qb, d,
             sa * sb, 5000.0, (256, 256, 128), (2, 4, 1), "gemm_fp8_8192_tile256")
     return res
 
@@ -242,6 +242,26 @@ def main():
     zms = mh.time_gemm(mma, tD, tensor_of(Az), tensor_of(Bz), None, 1.0, stream, warmup=0, iters=max(args.steps, 10))
     out["roofline"]["same_kernel_zero_operands_tflops"] = round(flops / (zms * 1e-3) / 1e12, 1)
     del Az, Bz
+
+    # yardstick, not the product: what the vendor library's GEMM (torch.matmul -> hipBLASLt) sustains on this box for the
+    # same operands, after the same clock ramp
+    if not args.no_other:
+        def lib():
+            torch.matmul(A, B.t(), out=D)
+        t_ramp = time.perf_counter()
+        while time.perf_counter() - t_ramp < 0.3:
+            for _ in range(50):
+                lib()
+            torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(100):
+            lib()
+        e1.record()
+        torch.cuda.synchronize()
+        out["vendor_library_tflops"] = round(flops / (e0.elapsed_time(e1) / 100 * 1e-3) / 1e12, 1)
+        mh.gemm_(mma, tD, tA, tB, None, 1.0, stream)  # leave D as the product computed it
+        torch.cuda.synchronize()
 
     if not args.no_copy:
         n = 16384

@@ -39,9 +39,6 @@
 
 #include "mfma_epilogue.hpp"
 
-#ifndef W4_EXP  // 0: the kernel; 1 and 2 drop the loads or the fragment reads for timing studies (wrong results)
-#define W4_EXP 0
-#endif
 namespace moye {
 
 typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
@@ -56,11 +53,11 @@ __device__ __forceinline__ void static_for(F&& f) {
     static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
-// The ND load-to-LDS instructions a wave issues per k-step go out evenly over the 56 MFMA positions
-// that follow the barrier (positions 8..63).  Returns the index of the load issued after MFMA P, or -1.
-constexpr int dma_index(int P, int ND) {
+// The ND load-to-LDS instructions a wave issues per k-step go out evenly over the MFMA positions that
+// follow the barrier (positions 8 .. NPOS - 1).  Returns the index of the load issued after MFMA P, or -1.
+constexpr int dma_index(int P, int ND, int NPOS) {
     for (int k = 0; k < ND; ++k)
-        if (8 + k * 56 / ND == P) return k;
+        if (8 + k * (NPOS - 8) / ND == P) return k;
     return -1;
 }
 
@@ -120,11 +117,16 @@ struct W4F32 {
     }
 };
 
-template <typename In, typename Out>
-__global__ __launch_bounds__(256) void gemm_mfma_tn_256_w4(GemmArgs p) {
+// WGN = 2: four waves (2 x 2), wave tile 128 x 128.  WGN = 4: eight waves (2 x 4), wave tile 128 x 64,
+// two waves per SIMD, so that what stalls one wave's instruction stream (an M0 write, a taken branch,
+// the barrier) leaves the matrix pipe to the other.
+template <typename In, typename Out, int WGN>
+__global__ __launch_bounds__(128 * WGN) void gemm_mfma_tn_256_w4(GemmArgs p) {
     constexpr int BM = 256, BN = 256, CPR = 4, STAGES = 5, SPS = In::SPS;
     constexpr int STAGE = (BM + BN) * CPR;  // in 16-byte chunks
-    constexpr int MI = 8, NI = 8, LD = 4;  // per wave and stage: 4 load-to-LDS instructions per operand
+    constexpr int NW = 2 * WGN, WN = BN / WGN;
+    constexpr int MI = 8, NI = WN / 16, NPOS = MI * NI;
+    constexpr int RW = BM / NW, LD = RW / 16;  // per wave and stage: RW rows, LD load-to-LDS instructions per operand
     typedef typename In::frag frag;
 
     extern __shared__ u32x4 smem[];
@@ -132,14 +134,14 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn_256_w4(GemmArgs p) {
     int tm, tn;
     tile_of_block(p, &tm, &tn);
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * 128;
+    const int wm0 = (wave / WGN) * 128, wn0 = (wave % WGN) * WN;
     const int r16 = lane & 15, kq = lane >> 4;
 
     const int64_t pitch_a = (int64_t)p.lda * In::kBytes, pitch_b = (int64_t)p.ldb * In::kBytes;
     // LDS stage (32 KiB) = A tile (256 rows of 64 bytes) then B tile.  Lane l of a load-to-LDS
     // instruction lands in physical chunk l % 4 of row l / 4 of a 16-row group; wave w brings rows
-    // 64 w .. 64 w + 63 of each operand.
-    const int lrow = wave * 64 + (lane >> 2), lch = (lane & 3) ^ swz<CPR>(lane >> 2);
+    // RW w .. RW w + RW - 1 of each operand.
+    const int lrow = wave * RW + (lane >> 2), lch = (lane & 3) ^ swz<CPR>(lane >> 2);
     const char* const a_tile = static_cast<const char*>(p.A) + (int64_t)tm * BM * pitch_a;  // uniform
     const char* const b_tile = static_cast<const char*>(p.B) + (int64_t)tn * BN * pitch_b;
     constexpr uint32_t kStageBytes = STAGE * 16, kATileBytes = BM * CPR * 16;
@@ -156,7 +158,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn_256_w4(GemmArgs p) {
 
     typedef __attribute__((address_space(3))) void* lptr_t;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(lptr_t)smem;  // LDS byte address of the ring
-    // Load-to-LDS instruction Q (0..3: A, 4..7: B) of this wave's share of a stage, in the scalar-base
+    // Load-to-LDS instruction Q (0 .. LD-1: A, LD .. 2 LD - 1: B) of this wave's share of a stage, in the scalar-base
     // form: a uniform 64-bit pointer to the stage's first row plus a per-lane 32-bit offset that never
     // changes, so no vector ALU work is left in the loop.  M0 carries the LDS destination of the
     // instruction's first lane.
@@ -168,7 +170,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn_256_w4(GemmArgs p) {
         constexpr int Q = decltype(qc)::value;
         const char* const base = uniform_ptr((Q < LD ? a_tile : b_tile) + (int64_t)g * 64);
         const uint32_t dst = __builtin_amdgcn_readfirstlane(lds0 + ring_slot * kStageBytes + (Q < LD ? 0 : kATileBytes) +
-                                                            (uint32_t)(wave * 64 + 16 * (Q % LD)) * 64);
+                                                            (uint32_t)(wave * RW + 16 * (Q % LD)) * 64);
         const uint32_t lane_off = voff[Q];  // (a captured array element cannot be an asm operand of a generic lambda)
         asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(base), "s"(dst)
                      : "memory");
@@ -212,18 +214,21 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn_256_w4(GemmArgs p) {
     });
     static_for<NI>([&](auto jc) __attribute__((always_inline)) {
         load_frag(fb[decltype(jc)::value], fb_byte, jc, 0, kStageBytes);
-        if (decltype(jc)::value == 3) __builtin_amdgcn_s_waitcnt(0xC07F);
+        if (decltype(jc)::value % 4 == 3) __builtin_amdgcn_s_waitcnt(0xC07F);
     });
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
 
-    // position P of the 64 MFMA groups of a k-step -> (i, j)
-#define MOYE_I(P) ((P) < 32 ? (P) % 4 : (P) < 40 ? 4 : (P) < 48 ? 5 : 6 + ((P) & 1))
-#define MOYE_J(P) ((P) < 32 ? (P) / 4 : (P) < 48 ? (P) % 8 : ((P) - 48) / 2)
+    // position P of the NPOS MFMA groups of a k-step -> (i, j): rows 0-3 column by column, row 4, row 5,
+    // rows 6 and 7 column by column
+#define MOYE_I(P) ((P) < 4 * NI ? (P) % 4 : (P) < 5 * NI ? 4 : (P) < 6 * NI ? 5 : 6 + (((P) - 6 * NI) & 1))
+#define MOYE_J(P) ((P) < 4 * NI ? (P) / 4 : (P) < 6 * NI ? ((P) - 4 * NI) % NI : ((P) - 6 * NI) / 2)
     int slot = 0;  // ring slot of the first stage of step s
     // One k-step.  MORE: step s+1 exists (its fragments are read); AHEAD: the stages five ahead exist
     // (they are requested, and the stages allowed to stay in flight at the barrier are the full 5 - 2 SPS).
-    // Fragment reads in program order: A0 A1 A2 A3 (after MFMA 28..31) A4 (39) A5 (47) B0 (49) B1 (51)
-    // B2 B3 B4 B5 B6 (61) A6 (62) A7 B7 (63); the next k-step needs B_j at MFMA 4 j, A0-3 at 0..3.
+    // Fragment reads in program order (128 x 128 wave tile): A0 A1 A2 A3 (after MFMA 28..31) A4 (39) A5 (47)
+    // B0 (49) B1 (51) B2 B3 B4 B5 B6 (61) A6 (62) A7 B7 (63); the next k-step needs B_j at MFMA 4 j and
+    // A0-3 at 0..3.  In general: A_i after 4 (NI - 1) + i, A4 after 5 NI - 1, A5 after 6 NI - 1, B_j after
+    // 6 NI + 2 j + 1, A6 after 8 NI - 2, A7 after 8 NI - 1.
     auto step = [&](auto more_c, auto ahead_c, int s) __attribute__((always_inline)) {
         constexpr bool MORE = decltype(more_c)::value, AHEAD = decltype(ahead_c)::value;
         int slot_n = slot + SPS;  // first stage of step s+1
@@ -231,13 +236,13 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn_256_w4(GemmArgs p) {
         const uint32_t o0 = (uint32_t)slot_n * kStageBytes;
         const uint32_t o1 = (uint32_t)(slot_n + 1 == STAGES ? 0 : slot_n + 1) * kStageBytes;
         const int g_new = s * SPS + STAGES;  // first global stage requested in this step
-        static_for<64>([&](auto pc) __attribute__((always_inline)) {
+        static_for<NPOS>([&](auto pc) __attribute__((always_inline)) {
             constexpr int P = decltype(pc)::value;
             constexpr int i = MOYE_I(P), j = MOYE_J(P);
-            // B0 is followed by 9 fragment reads, B1 by 8; a stricter count costs nothing where the older
-            // reads are hundreds of clocks old (fp8: two reads per fragment, 32-clock MFMAs)
-            if (P == 0) __builtin_amdgcn_s_waitcnt(0xC07F | ((9 * SPS < 12 ? 9 * SPS : 12) << 8));
-            if (P == 4) __builtin_amdgcn_s_waitcnt(0xC07F | ((8 * SPS < 12 ? 8 * SPS : 12) << 8));
+            // B0 is followed by NI + 1 fragment reads, B1 by NI; a stricter count costs nothing where the
+            // older reads are hundreds of clocks old (fp8: two reads per fragment, 32-clock MFMAs)
+            if (P == 0) __builtin_amdgcn_s_waitcnt(0xC07F | (((NI + 1) * SPS < 12 ? (NI + 1) * SPS : 12) << 8));
+            if (P == 4) __builtin_amdgcn_s_waitcnt(0xC07F | ((NI * SPS < 12 ? NI * SPS : 12) << 8));
             In::mma(fb[j], fa[i], acc[i][j]);
             if (P == 7) {
                 // my share of step s+1 has landed and all my fragment reads have returned (the last were
@@ -253,22 +258,23 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn_256_w4(GemmArgs p) {
                 }
                 MOYE_BARRIER()
             }
-            if constexpr (dma_index(P, 2 * LD * SPS) >= 0) {
-                constexpr int q = dma_index(P, 2 * LD * SPS);  // 0 .. 2 LD SPS - 1
+            if constexpr (dma_index(P, 2 * LD * SPS, NPOS) >= 0) {
+                constexpr int q = dma_index(P, 2 * LD * SPS, NPOS);  // 0 .. 2 LD SPS - 1
                 // in the drain a k-step of two stages may still have its first stage to request
-                if (W4_EXP != 1 && (AHEAD || g_new + q / (2 * LD) < nstages)) {
+                if (AHEAD || g_new + q / (2 * LD) < nstages) {
                     int sl = slot + q / (2 * LD);
                     if (sl >= STAGES) sl -= STAGES;
                     dma1(g_new + q / (2 * LD), sl, std::integral_constant<int, q % (2 * LD)>{});
                 }
             }
-            if (MORE && W4_EXP != 2) {
-                if constexpr (P >= 28 && P < 32) load_frag(fa[P - 28], fa_byte, MOYE_BLK(P - 28), o0, o1);
-                if constexpr (P == 39) load_frag(fa[4], fa_byte, MOYE_BLK(4), o0, o1);
-                if constexpr (P == 47) load_frag(fa[5], fa_byte, MOYE_BLK(5), o0, o1);
-                if constexpr (P == 62) load_frag(fa[6], fa_byte, MOYE_BLK(6), o0, o1);
-                if constexpr (P == 63) load_frag(fa[7], fa_byte, MOYE_BLK(7), o0, o1);
-                if constexpr (P >= 48 && (P & 1)) load_frag(fb[(P - 48) / 2], fb_byte, MOYE_BLK((P - 48) / 2), o0, o1);
+            if (MORE) {
+                constexpr int A0 = 4 * (NI - 1), B0 = 6 * NI;
+                if constexpr (P >= A0 && P < A0 + 4) load_frag(fa[P - A0], fa_byte, MOYE_BLK(P - A0), o0, o1);
+                if constexpr (P == 5 * NI - 1) load_frag(fa[4], fa_byte, MOYE_BLK(4), o0, o1);
+                if constexpr (P == 6 * NI - 1) load_frag(fa[5], fa_byte, MOYE_BLK(5), o0, o1);
+                if constexpr (P == NPOS - 2) load_frag(fa[6], fa_byte, MOYE_BLK(6), o0, o1);
+                if constexpr (P == NPOS - 1) load_frag(fa[7], fa_byte, MOYE_BLK(7), o0, o1);
+                if constexpr (P >= B0 && ((P - B0) & 1)) load_frag(fb[(P - B0) / 2], fb_byte, MOYE_BLK((P - B0) / 2), o0, o1);
             }
         });
         slot = slot_n;
@@ -292,47 +298,52 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn_256_w4(GemmArgs p) {
     store_c_tile<Out, MI, NI>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
 }
 
-template <typename In, typename Out>
+template <typename In, typename Out, int WGN>
 static int32_t launch256_w4(const GemmArgs& a, hipStream_t st) {
     constexpr int kLds = 5 * (256 + 256) * 64;  // all 160 KiB
-    auto kern = gemm_mfma_tn_256_w4<In, Out>;
+    auto kern = gemm_mfma_tn_256_w4<In, Out, WGN>;
     static bool once = false;
     if (!once) {
         MOYE_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
         once = true;
     }
-    kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n)), dim3(256), kLds, st>>>(a);
+    kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n)), dim3(128 * WGN), kLds, st>>>(a);
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;
 }
 
-template <typename In>
+template <typename In, int WGN>
 static int32_t launch256_w4_out(int32_t out_dt, const GemmArgs& a, hipStream_t st) {
     switch (out_dt) {
-        case MOYE_F32: return launch256_w4<In, OutF32>(a, st);
-        case MOYE_F16: return launch256_w4<In, OutF16>(a, st);
-        case MOYE_BF16: return launch256_w4<In, OutBF16>(a, st);
+        case MOYE_F32: return launch256_w4<In, OutF32, WGN>(a, st);
+        case MOYE_F16: return launch256_w4<In, OutF16, WGN>(a, st);
+        case MOYE_BF16: return launch256_w4<In, OutBF16, WGN>(a, st);
         default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: MFMA kernels write f32, f16 or bf16, not %s", dtype_name(out_dt));
     }
 }
 
-// 256 x 256 tile, four waves; K a multiple of 64 bytes (128 for fp8); the caller has checked
+template <int WGN>
+static int32_t launch256_w4_in(int32_t in_dt, int32_t out_dt, const GemmArgs& a, hipStream_t st) {
+    switch (in_dt) {
+        case MOYE_F16: return launch256_w4_out<W4F16, WGN>(out_dt, a, st);
+        case MOYE_BF16: return launch256_w4_out<W4BF16, WGN>(out_dt, a, st);
+        case MOYE_F8E4M3: return launch256_w4_out<W4FP8, WGN>(out_dt, a, st);
+        case MOYE_F32: return launch256_w4_out<W4F32, WGN>(out_dt, a, st);
+        default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: no MFMA atom for %s inputs", dtype_name(in_dt));
+    }
+}
+
+// 256 x 256 tile, four or eight waves; K a multiple of 64 bytes (128 for fp8); the caller has checked
 // divisibility of M and N and alignment.
-int32_t gemm_mfma_tn_256_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, hipStream_t st) {
+int32_t gemm_mfma_tn_256_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, int waves, hipStream_t st) {
     a.tiles_m = a.M / 256;
     a.tiles_n = a.N / 256;
     // the load-to-LDS addresses are a uniform base plus a 32-bit lane offset
     const int eb = dtype_bytes(in_dt);
     if (256 * a.lda * eb >= (int64_t)1 << 32 || 256 * a.ldb * eb >= (int64_t)1 << 32)
         return fail(MOYE_ERR_SHAPE, "gemm!: row pitch too large for the 256x256 MFMA kernel");
-    switch (in_dt) {
-        case MOYE_F16: return launch256_w4_out<W4F16>(out_dt, a, st);
-        case MOYE_BF16: return launch256_w4_out<W4BF16>(out_dt, a, st);
-        case MOYE_F8E4M3: return launch256_w4_out<W4FP8>(out_dt, a, st);
-        case MOYE_F32: return launch256_w4_out<W4F32>(out_dt, a, st);
-        default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: no MFMA atom for %s inputs", dtype_name(in_dt));
-    }
+    return waves == 4 ? launch256_w4_in<2>(in_dt, out_dt, a, st) : launch256_w4_in<4>(in_dt, out_dt, a, st);
 }
 
 }  // namespace moye

@@ -313,9 +313,10 @@ def test_pingpong_schedule_random(mh):
     assert torch.equal(d, d2)
 
 
-def test_wave4_schedule_exact_on_integers(mh):
-    """MOYE_GEMM_WAVE4: four waves with 128x128 wave tiles, fragments refilled in place, hand-placed
-    waits.  Small integers make every sum exact, so any fragment read too early, any stage
+@pytest.mark.parametrize("waves", [(2, 2, 1), (2, 4, 1)])
+def test_wave4_schedule_exact_on_integers(mh, waves):
+    """MOYE_GEMM_WAVE4: four waves with 128x128 wave tiles or eight with 128x64, fragments refilled in
+    place, hand-placed waits.  Small integers make every sum exact, so any fragment read too early, any stage
     overwritten too soon or any misplaced accumulator shows as a wrong integer.  K from one
     k-step to many: the prologue, the steady state and the drain each have their own wait counts."""
     from moye_hip import _lib
@@ -333,14 +334,15 @@ def test_wave4_schedule_exact_on_integers(mh):
             C = torch.randint(-8, 9, (M, N), generator=g).float()
             a, b, c = A.to(in_dt).cuda(), B.to(in_dt).cuda(), C.cuda()
             d = torch.zeros(M, N, dtype=torch.float32, device="cuda")
-            mma = mh.tiled_mma_desc(atom, atom_layout=(2, 2, 1), cta_tile=(256, 256, bk), flags=_lib.GEMM_WAVE4)
-            print("wave4", in_dt, M, N, K, flush=True)
+            mma = mh.tiled_mma_desc(atom, atom_layout=waves, cta_tile=(256, 256, bk), flags=_lib.GEMM_WAVE4)
+            print("wave4", waves, in_dt, M, N, K, flush=True)
             mh.gemm_(mma, T(d), T(a), T(b), T(c), 2.0)
             torch.cuda.synchronize()
             assert torch.equal(d.cpu().double(), 2.0 * (A.double() @ B.double().t()) + C.double()), (in_dt, M, N, K)
 
 
-def test_wave4_schedule_random(mh):
+@pytest.mark.parametrize("waves", [(2, 2, 1), (2, 4, 1)])
+def test_wave4_schedule_random(mh, waves):
     from moye_hip import _lib
     M = N = K = 2048
     g = torch.Generator().manual_seed(18)
@@ -349,7 +351,7 @@ def test_wave4_schedule_random(mh):
     a, b = A.cuda(), B.cuda()
     d = torch.zeros(M, N, dtype=torch.float16, device="cuda")
     d2 = torch.zeros(M, N, dtype=torch.float16, device="cuda")
-    mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 2, 1), cta_tile=(256, 256, 32),
+    mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=waves, cta_tile=(256, 256, 32),
                                flags=_lib.GEMM_WAVE4), T(d), T(a), T(b))
     mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 4, 1), cta_tile=(256, 256, 64)), T(d2), T(a), T(b))
     torch.cuda.synchronize()
@@ -363,7 +365,7 @@ def test_wave4_schedule_random(mh):
         sa, sb = float(x.abs().max()) / 448.0, float(w.abs().max()) / 448.0
         qa, qb = (x / sa).to(torch.float8_e4m3fn).cuda(), (w / sb).to(torch.float8_e4m3fn).cuda()
         o = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
-        mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_FP8, atom_layout=(2, 2, 1), cta_tile=(256, 256, 128),
+        mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_FP8, atom_layout=waves, cta_tile=(256, 256, 128),
                                    flags=_lib.GEMM_WAVE4), T(o), T(qa), T(qb), None, sa * sb)
         torch.cuda.synchronize()
         c64 = (qa.double() @ qb.double().t()) * (sa * sb)

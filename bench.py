@@ -26,8 +26,9 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 MEASURED_TRAFFIC = {
     "gemm_f16_4096_tile256": {"read_bytes": 197437 * 1024, "write_bytes": 33280 * 1024},
     "transpose_f32_16384": {"read_bytes": 1048622 * 1024, "write_bytes": 1049576 * 1024},
-    "gemm_bf16_8192_tile256": {"read_bytes": 1647295 * 1024, "write_bytes": 266240 * 1024},
-    "gemm_fp8_8192_tile256": {"read_bytes": 787830 * 1024, "write_bytes": 131072 * 1024},
+    "gemm_bf16_8192_tile256": {"read_bytes": 1809307 * 1024, "write_bytes": 266240 * 1024},
+    "gemm_f32_8192_tile256": {"read_bytes": 3960678 * 1024, "write_bytes": 270336 * 1024},
+    "gemm_fp8_8192_tile256": {"read_bytes": 786981 * 1024, "write_bytes": 131072 * 1024},
     "gemm_bf16_16x8192x8192": {"read_bytes": 159438 * 1024, "write_bytes": 512 * 1024},
 }
 
@@ -101,7 +102,7 @@ def other_configs(mh, tensor_of, torch, stream):
     af, bf_ = a.float(), b.float()
     df = torch.zeros(n, n, dtype=torch.float32, device="cuda")
     run("fp32 TN 8192^3 (v_mfma_f32_16x16x4_f32), CTA 256x256x32", mh.MFMA_F32_16x16x4_F32, af, bf_, df, 1.0, 157.3,
-        (256, 256, 32), (2, 4, 1), None)
+        (256, 256, 32), (2, 4, 1), "gemm_f32_8192_tile256")
     del af, bf_, df
     # short M: rotate over 3 copies of B so that the 256 MiB Infinity Cache cannot serve the stream
     a16 = a[:16].contiguous()
@@ -143,6 +144,47 @@ def other_configs(mh, tensor_of, torch, stream):
     return res
 
 
+def yardsticks(out, args, mh, torch, tensor_of, mma, A, B, D, tA, tB, tD, flops, achieved, stream):
+    """What the headline number can be held against on this box: the matrix pipe alone, the same kernel on
+    operands that do not toggle, and the vendor library's GEMM.  None of it is the product path."""
+    # the matrix pipe alone on this box, same input type: what "MFMA-bound" can mean here
+    tf_r, ghz_r = mh.mfma_ceiling(mh.F16, True, 0.5)
+    tf_z, ghz_z = mh.mfma_ceiling(mh.F16, False, 0.5)
+    out["mfma_only"] = {"what": "MFMA-only loop on all CUs, fp16, no memory traffic (moye_mfma_ceiling), 0.5 s each",
+                        "random_operands": {"tflops": round(tf_r, 1), "clock_ghz": round(ghz_r, 3)},
+                        "zero_operands": {"tflops": round(tf_z, 1), "clock_ghz": round(ghz_z, 3)}}
+    out["roofline"]["frac_of_mfma_only_random"] = round(achieved / tf_r, 4)
+    # the same kernel on all-zero operands: same instructions, same traffic, no toggling data -> the clock the
+    # power controller allows is higher; the difference to `achieved` is what dense operands cost on this part
+    Az, Bz = torch.zeros_like(A), torch.zeros_like(B)
+    t_ramp = time.perf_counter()
+    while time.perf_counter() - t_ramp < 0.3:
+        mh.time_gemm(mma, tD, tensor_of(Az), tensor_of(Bz), None, 1.0, stream, warmup=0, iters=50)
+    zms = mh.time_gemm(mma, tD, tensor_of(Az), tensor_of(Bz), None, 1.0, stream, warmup=0, iters=max(args.steps, 10))
+    out["roofline"]["same_kernel_zero_operands_tflops"] = round(flops / (zms * 1e-3) / 1e12, 1)
+    del Az, Bz
+
+    # yardstick, not the product: what the vendor library's GEMM (torch.matmul -> hipBLASLt) sustains on this box for the
+    # same operands, after the same clock ramp
+    if not args.no_other:
+        def lib():
+            torch.matmul(A, B.t(), out=D)
+        t_ramp = time.perf_counter()
+        while time.perf_counter() - t_ramp < 0.3:
+            for _ in range(50):
+                lib()
+            torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(100):
+            lib()
+        e1.record()
+        torch.cuda.synchronize()
+        out["vendor_library_tflops"] = round(flops / (e0.elapsed_time(e1) / 100 * 1e-3) / 1e12, 1)
+        mh.gemm_(mma, tD, tA, tB, None, 1.0, stream)  # leave D as the product computed it
+        torch.cuda.synchronize()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -151,6 +193,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-copy", action="store_true", help="skip the tiled-copy leg")
     ap.add_argument("--no-other", action="store_true", help="skip the bf16 / fp8 / short-M GEMM legs")
+    ap.add_argument("--no-yardsticks", action="store_true",
+                    help="skip the MFMA-only loop, the zero-operand run and the vendor-library run (for kernel traces: "
+                         "every launch of the headline kernel is then a dense-operand launch)")
     ap.add_argument("--tile", default="256,256,64", help="CTA tile bm,bn,bk of the GEMM kernel")
     ap.add_argument("--waves", default="2,4", help="waves per CTA along M,N (TiledMMA atom layout)")
     ap.add_argument("--stages", type=int, default=0, help="LDS pipeline depth (0 = kernel default)")
@@ -226,42 +271,8 @@ def main():
                      "kernel_ms": round(kern_ms, 5)},
     }
 
-    # the matrix pipe alone on this box, same input type: what "MFMA-bound" can mean here
-    tf_r, ghz_r = mh.mfma_ceiling(mh.F16, True, 0.5)
-    tf_z, ghz_z = mh.mfma_ceiling(mh.F16, False, 0.5)
-    out["mfma_only"] = {"what": "MFMA-only loop on all CUs, fp16, no memory traffic (moye_mfma_ceiling), 0.5 s each",
-                        "random_operands": {"tflops": round(tf_r, 1), "clock_ghz": round(ghz_r, 3)},
-                        "zero_operands": {"tflops": round(tf_z, 1), "clock_ghz": round(ghz_z, 3)}}
-    out["roofline"]["frac_of_mfma_only_random"] = round(achieved / tf_r, 4)
-    # the same kernel on all-zero operands: same instructions, same traffic, no toggling data -> the clock the
-    # power controller allows is higher; the difference to `achieved` is what dense operands cost on this part
-    Az, Bz = torch.zeros_like(A), torch.zeros_like(B)
-    t_ramp = time.perf_counter()
-    while time.perf_counter() - t_ramp < 0.3:
-        mh.time_gemm(mma, tD, tensor_of(Az), tensor_of(Bz), None, 1.0, stream, warmup=0, iters=50)
-    zms = mh.time_gemm(mma, tD, tensor_of(Az), tensor_of(Bz), None, 1.0, stream, warmup=0, iters=max(args.steps, 10))
-    out["roofline"]["same_kernel_zero_operands_tflops"] = round(flops / (zms * 1e-3) / 1e12, 1)
-    del Az, Bz
-
-    # yardstick, not the product: what the vendor library's GEMM (torch.matmul -> hipBLASLt) sustains on this box for the
-    # same operands, after the same clock ramp
-    if not args.no_other:
-        def lib():
-            torch.matmul(A, B.t(), out=D)
-        t_ramp = time.perf_counter()
-        while time.perf_counter() - t_ramp < 0.3:
-            for _ in range(50):
-                lib()
-            torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(100):
-            lib()
-        e1.record()
-        torch.cuda.synchronize()
-        out["vendor_library_tflops"] = round(flops / (e0.elapsed_time(e1) / 100 * 1e-3) / 1e12, 1)
-        mh.gemm_(mma, tD, tA, tB, None, 1.0, stream)  # leave D as the product computed it
-        torch.cuda.synchronize()
+    if not args.no_yardsticks:
+        yardsticks(out, args, mh, torch, tensor_of, mma, A, B, D, tA, tB, tD, flops, achieved, stream)
 
     if not args.no_copy:
         n = 16384

@@ -58,9 +58,27 @@ def cpu_baseline(cores):
     t0 = time.perf_counter()
     co.gemm(A, B, None, "f16", (32, 32, 8), cores)
     dt = time.perf_counter() - t0
-    return {"value": round(2.0 * n ** 3 / dt / 1e12, 6), "unit": "TFLOP/s", "cores": cores, "kind": "port",
-            "sample": "fp16 TN %d^3 sub-problem of the 4096^3 workload, UniversalFMA gemm! restatement "
-                      "(32x32x8 tiles, OpenMP over C tiles), %.1f s" % (n, dt)}
+    res = {"value": round(2.0 * n ** 3 / dt / 1e12, 6), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+           "sample": "fp16 TN %d^3 sub-problem of the 4096^3 workload, UniversalFMA gemm! restatement "
+                     "(32x32x8 tiles, OpenMP over C tiles), %.1f s" % (n, dt)}
+    # the same restatement on one thread (the reference's host test runs it that way per Julia thread), 512^3
+    A1, B1 = operands(512)
+    t0 = time.perf_counter()
+    co.gemm(A1, B1, None, "f16", (32, 32, 8), 1)
+    res["single_thread_tflops"] = round(2.0 * 512 ** 3 / (time.perf_counter() - t0) / 1e12, 6)
+    # what LinearAlgebra.mul! would reach on these cores: the BLAS sgemm behind torch.mm, full 4096^3 in fp32
+    try:
+        import torch
+        torch.set_num_threads(cores)
+        a32, b32 = torch.from_numpy(A[:min(n, 4096)]).contiguous(), torch.from_numpy(B[:min(n, 4096)]).contiguous()
+        torch.mm(a32, b32.t())
+        t0 = time.perf_counter()
+        torch.mm(a32, b32.t())
+        res["blas_sgemm"] = {"tflops": round(2.0 * a32.shape[0] * b32.shape[0] * a32.shape[1] / (time.perf_counter() - t0) / 1e12, 4),
+                             "threads": cores, "what": "torch.mm fp32 on the host, %d^3" % a32.shape[0]}
+    except Exception as e:  # the baseline above stands without it
+        res["blas_sgemm"] = {"error": repr(e)[:200]}
+    return res
 
 
 def other_configs(mh, tensor_of, torch, stream):

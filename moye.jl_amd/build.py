@@ -5,6 +5,7 @@
 Objects go to csrc/build/, the library next to the Python mirror as moye_hip/libmoye_hip.so.
 """
 import os
+import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -60,11 +61,65 @@ def _compile(item, force):
     return obj, err
 
 
+# Kernels whose MFMAs are inline assembly: the compiler does not know how long their results take, so any
+# instruction of its own that touches an accumulator register next to them (a copy made by the register
+# allocator, an epilogue read scheduled upwards) would read a value that is not there yet, silently.
+ASM_MFMA_SOURCES = ["gemm_mfma256w4.hip"]
+
+
+def check_accumulator_hazards(src):
+    """Compile `src` to assembly and fail if, in any basic block that holds v_mfma instructions, something
+    other than a v_mfma names an AccVGPR before the kernel's `MOYE_ACC_SETTLED` marker."""
+    path = os.path.join(CSRC, src)
+    asm = os.path.join(CSRC, "build", os.path.splitext(src)[0] + ".s")
+    if not _stale(asm, [path] + _headers()):
+        return
+    cmd = [HIPCC] + COMMON + ["-S", "--cuda-device-only", path, "-o", asm]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc -S failed for %s:\n%s" % (src, r.stdout + r.stderr))
+    fn, block, bad = None, [], []
+
+    def flush():
+        if fn and any("v_mfma" in c.split(";")[0] for _, c in block):
+            settled = False
+            for ln, c in block:
+                settled = settled or "MOYE_ACC_SETTLED" in c
+                code = c.split(";")[0]
+                if "v_mfma" in code or settled:
+                    continue
+                if re.search(r"\ba(\[\d+:\d+\]|\d+)\b", code):
+                    bad.append("%s:%d: %s   [%s]" % (os.path.basename(asm), ln, code.strip(), fn[:60]))
+        del block[:]
+
+    with open(asm) as f:
+        for ln, line in enumerate(f, 1):
+            m = re.match(r"^(_Z\w+):", line)
+            if m:
+                flush()
+                fn = m.group(1)
+                continue
+            if fn is None:
+                continue
+            if re.match(r"^\.LBB\w+:", line):
+                flush()
+            block.append((ln, line))
+            if re.search(r"\bs_(cbranch|branch|endpgm)", line):
+                flush()
+                if "s_endpgm" in line:
+                    fn = None
+    if bad:
+        os.remove(asm)
+        raise RuntimeError("accumulator registers are touched next to inline-assembly MFMAs:\n" + "\n".join(bad[:20]))
+
+
 def build(force=False, verbose=True):
     os.makedirs(os.path.join(CSRC, "build"), exist_ok=True)
     items = [(s, f) for s, f in SOURCES.items() if os.path.exists(os.path.join(CSRC, s))]
     with ThreadPoolExecutor(max_workers=min(8, len(items))) as ex:
         results = list(ex.map(lambda it: _compile(it, force), items))
+    for src in ASM_MFMA_SOURCES:
+        check_accumulator_hazards(src)
     objs = [o for o, _ in results]
     for (src, _), (_, msg) in zip(items, results):
         if msg.strip() and verbose:

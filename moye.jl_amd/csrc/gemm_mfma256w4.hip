@@ -290,9 +290,18 @@ __global__ __launch_bounds__(128 * WGN) void gemm_mfma_tn_256_w4(GemmArgs p) {
 #undef MOYE_J
 #undef MOYE_VMCNT
 #undef MOYE_BARRIER
-    // the accumulators were written by instructions the compiler did not see: let the last ones
-    // retire before anything reads them
-    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    // The accumulators were written by instructions whose latency the compiler does not know: let the last
+    // ones retire before anything reads them.  The empty statements make every later read of an accumulator
+    // depend on something that comes after the nops (volatile statements keep their order), so the epilogue's
+    // v_accvgpr_read cannot be scheduled up to the MFMA that produced the value (seen in a variant of this
+    // kernel: the read landed right behind the MFMA and returned the old value).  The build checks the
+    // generated code for the other way this could go wrong: an accumulator register named, between MFMAs,
+    // by anything that is not an MFMA (build.py, check_accumulator_hazards).
+    asm volatile("s_nop 15\n\ts_nop 15\n\t; MOYE_ACC_SETTLED" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j) asm volatile("" : "+a"(acc[i][j]));
     __syncthreads();  // every wave is done with the operand ring before it becomes C patches
 
     store_c_tile<Out, MI, NI>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);

@@ -144,6 +144,23 @@ int32_t moye_axpby(double a, const moye_tensor* X, double b, const moye_tensor* 
  * element type */
 int32_t moye_fill(const moye_tensor* X, double value, void* stream);
 
+/* Broadcast-style element-wise maps, dst .= op.(a, b) (src/broadcast.jl:5-41; map!,
+ * src/algorithm/array_algorithms.jl:192-210), over the logical elements of the layouts.  All arrays have the
+ * same floating-point element type T.  `b` may be NULL (the second operand is `scalar`, converted to T), hold
+ * as many elements as dst, or as many as a leading group of dst's modes (it then repeats over the trailing
+ * modes, as a lower-rank array does under Julia's broadcasting).  One operation, rounded in T. */
+#define MOYE_MAP_IDENTITY 0   /* dst .= a                      */
+#define MOYE_MAP_ADD 1        /* a .+ b                        */
+#define MOYE_MAP_SUB 2        /* a .- b                        */
+#define MOYE_MAP_MUL 3        /* a .* b                        */
+#define MOYE_MAP_DIV 4        /* a ./ b                        */
+#define MOYE_MAP_MAX 5        /* max.(a, b): NaN if either is  */
+#define MOYE_MAP_MIN 6        /* min.(a, b)                    */
+#define MOYE_MAP_NEG 7        /* .-a (b and scalar ignored)    */
+#define MOYE_MAP_ABS 8        /* abs.(a)                       */
+int32_t moye_map(int32_t op, const moye_tensor* dst, const moye_tensor* a, const moye_tensor* b, double scalar,
+                 void* stream);
+
 /* bytes of device workspace moye_gemm needs for this call: the K-major copies of MFMA operands whose
  * unit stride is not along K (NN / NT / TT problems); 0 for TN and for UniversalFMA.  The library
  * allocates the workspace on first use (a synchronous hipMalloc inside that one moye_gemm call), grows

@@ -232,6 +232,11 @@ int32_t moye_fill(const moye_tensor* X, double value, void* stream) {
     return fill_dispatch(X, value, static_cast<hipStream_t>(stream));
 }
 
+int32_t moye_map(int32_t op, const moye_tensor* dst, const moye_tensor* a, const moye_tensor* b, double scalar,
+                 void* stream) {
+    return map_dispatch(op, dst, a, b, scalar, static_cast<hipStream_t>(stream));
+}
+
 int32_t moye_gemm_workspace_size(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A,
                                  const moye_tensor* B, size_t* bytes) {
     if (!mma || !D || !A || !B || !bytes) return fail(MOYE_ERR_ARG, "moye_gemm_workspace_size: null argument");

@@ -1,7 +1,8 @@
-// axpby! and fill!/zeros! on device arrays with arbitrary layouts.
+// axpby!, fill!/zeros! and broadcast-style element-wise maps on device arrays with arbitrary layouts.
 //
 //   axpby!(a, X, b, Y)  (src/algorithm/blas.jl:1-9):  y[i] = iszero(b) ? a*x[i] : a*x[i] + b*y[i]
 //   fill!(x, val), zeros!(x)  (src/algorithm/array_algorithms.jl:158-182)
+//   dst .= a .+ b, a .* s, max.(a, b), ...  (src/broadcast.jl:5-41; map! src/algorithm/array_algorithms.jl:192-210)
 // over the logical elements i of both layouts.  X and Y have the same element type T; a and b are
 // converted to T first and every operation is rounded in T (Julia's Float16 arithmetic computes in
 // Float32 and rounds after each operation; so does this), products and the sum never contracted
@@ -97,6 +98,36 @@ __global__ __launch_bounds__(256) void axpby_kernel(typename El::compute a, cons
     }
 }
 
+
+// dst[i] = f(a[i], b[i % nb]) or f(a[i], s): b may be a whole array (nb == n) or span the leading modes of dst
+// and repeat over the trailing ones (Julia's broadcasting of a lower-rank array), or absent (scalar operand)
+template <typename El>
+__global__ __launch_bounds__(256) void map_kernel(int32_t op, typename El::storage* d, ELayout ld,
+                                                  const typename El::storage* a, ELayout la,
+                                                  const typename El::storage* b, ELayout lb, int64_t nb,
+                                                  typename El::compute s, int64_t n) {
+    typedef typename El::compute T;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const T x = El::load(a + e_offset(la, i));
+        const T y = b ? El::load(b + e_offset(lb, i % nb)) : s;
+        T r;
+        switch (op) {
+            case MOYE_MAP_ADD: r = x + y; break;
+            case MOYE_MAP_SUB: r = x - y; break;
+            case MOYE_MAP_MUL: r = x * y; break;
+            case MOYE_MAP_DIV: r = x / y; break;
+            // Julia's max/min for floats (base/math.jl): a NaN operand is returned; max(-0.0, 0.0) == 0.0
+            case MOYE_MAP_MAX: r = ((y > x) | (signbit(y) < signbit(x))) ? (x != x ? x : y) : (y != y ? y : x); break;
+            case MOYE_MAP_MIN: r = ((y < x) | (signbit(y) > signbit(x))) ? (x != x ? x : y) : (y != y ? y : x); break;
+            case MOYE_MAP_NEG: r = -x; break;
+            case MOYE_MAP_ABS: r = signbit(x) ? -x : x; break;
+            default: r = x; break;  // MOYE_MAP_IDENTITY
+        }
+        El::store(d + e_offset(ld, i), El::round(r));
+    }
+}
+
 template <int kBytes>
 __global__ __launch_bounds__(256) void fill_kernel(char* x, ELayout lx, int64_t n, uint64_t bits) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
@@ -160,6 +191,61 @@ int32_t axpby_dispatch(double a, const moye_tensor* X, double b, const moye_tens
         }
         default:
             return fail(MOYE_ERR_UNSUPPORTED, "axpby!: element type %s is not a floating-point type this build handles", dtype_name(X->dtype));
+    }
+    MOYE_HIP_CHECK(hipGetLastError());
+    return MOYE_OK;
+}
+
+
+// dst .= op.(A, B) / op.(A, scalar) / op.(A): every array has the same floating-point element type T, the scalar
+// is converted to T first and the result of the one operation is rounded in T
+int32_t map_dispatch(int32_t op, const moye_tensor* D, const moye_tensor* A, const moye_tensor* B, double scalar,
+                     hipStream_t st) {
+    if (op < MOYE_MAP_IDENTITY || op > MOYE_MAP_ABS) return fail(MOYE_ERR_UNSUPPORTED, "map!: unknown operation %d", op);
+    if (int32_t e = check_tensor(D, "dst")) return e;
+    if (int32_t e = check_tensor(A, "a")) return e;
+    if (B) if (int32_t e = check_tensor(B, "b")) return e;
+    if (A->dtype != D->dtype || (B && B->dtype != D->dtype))
+        return fail(MOYE_ERR_UNSUPPORTED, "map!: all arrays must have the element type of the destination (%s)", dtype_name(D->dtype));
+    const int64_t n = count(*D);
+    if (count(*A) != n) return fail(MOYE_ERR_SHAPE, "map!: dst holds %lld elements, a %lld", (long long)n, (long long)count(*A));
+    int64_t nb = 1;
+    if (B) {
+        nb = count(*B);
+        // b must be dst-sized or span a leading group of dst's modes
+        bool ok = nb == n;
+        int64_t lead = 1;
+        for (int i = 0; i < D->rank && !ok; ++i) {
+            lead *= D->shape[i];
+            ok = lead == nb;
+        }
+        if (!ok && nb != 1)
+            return fail(MOYE_ERR_SHAPE, "map!: cannot broadcast %lld elements of b over the %lld of dst", (long long)nb, (long long)n);
+    }
+    if (n == 0) return MOYE_OK;
+    const dim3 grid((unsigned)std::min<int64_t>((n + 255) / 256, 256 * 16));
+    const ELayout ld = elayout_of(*D), la = elayout_of(*A), lb = B ? elayout_of(*B) : ELayout{};
+    switch (D->dtype) {
+        case MOYE_F32:
+            map_kernel<ElF32><<<grid, 256, 0, st>>>(op, static_cast<float*>(D->ptr), ld, static_cast<const float*>(A->ptr), la,
+                                                    B ? static_cast<const float*>(B->ptr) : nullptr, lb, nb, (float)scalar, n);
+            break;
+        case MOYE_F64:
+            map_kernel<ElF64><<<grid, 256, 0, st>>>(op, static_cast<double*>(D->ptr), ld, static_cast<const double*>(A->ptr), la,
+                                                    B ? static_cast<const double*>(B->ptr) : nullptr, lb, nb, scalar, n);
+            break;
+        case MOYE_F16:
+            map_kernel<ElF16><<<grid, 256, 0, st>>>(op, static_cast<_Float16*>(D->ptr), ld, static_cast<const _Float16*>(A->ptr), la,
+                                                    B ? static_cast<const _Float16*>(B->ptr) : nullptr, lb, nb,
+                                                    host_round_f16((float)scalar), n);
+            break;
+        case MOYE_BF16:
+            map_kernel<ElBF16><<<grid, 256, 0, st>>>(op, static_cast<uint16_t*>(D->ptr), ld, static_cast<const uint16_t*>(A->ptr), la,
+                                                     B ? static_cast<const uint16_t*>(B->ptr) : nullptr, lb, nb,
+                                                     host_round_bf16((float)scalar), n);
+            break;
+        default:
+            return fail(MOYE_ERR_UNSUPPORTED, "map!: element type %s is not a floating-point type this build handles", dtype_name(D->dtype));
     }
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;

@@ -36,6 +36,7 @@ int32_t gemm_mfma_tn_256_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, 
 int32_t gemm_mfma_skinny_dispatch(int32_t in_dt, int32_t out_dt, const GemmArgs& a, hipStream_t st);
 int32_t axpby_dispatch(double a, const moye_tensor* X, double b, const moye_tensor* Y, hipStream_t st);
 int32_t fill_dispatch(const moye_tensor* X, double value, hipStream_t st);
+int32_t map_dispatch(int32_t op, const moye_tensor* D, const moye_tensor* A, const moye_tensor* B, double scalar, hipStream_t st);
 int32_t mfma_ceiling(int32_t in_dt, int32_t random_operands, float seconds, float* tflops, float* clock_ghz, hipStream_t st);
 int32_t gemm_universal_dispatch(int bm, int bn, int bk, UArgs a, hipStream_t st);
 

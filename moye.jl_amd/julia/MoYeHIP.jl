@@ -399,6 +399,33 @@ function fill!(x::MoYeArray, val::Real; stream::Ptr{Cvoid} = C_NULL)
 end
 zeros!(x::MoYeArray; stream::Ptr{Cvoid} = C_NULL) = fill!(x, 0.0; stream = stream)
 
+const MAP_OPS = Dict{Any,Int32}(identity => 0, (+) => 1, (-) => 2, (*) => 3, (/) => 4, max => 5, min => 6, abs => 8)
+
+"""
+    map!(f, dst, a, b; stream=C_NULL)     # dst .= f.(a, b), b an array or a number
+    map!(f, dst, a; stream=C_NULL)        # dst .= f.(a) for identity, -, abs
+
+The device form of the reference's broadcast (src/broadcast.jl:5-41) and `map!`
+(src/algorithm/array_algorithms.jl:192-210) for `f` in `+ - * / max min abs identity`: one operation per
+element, rounded in the arrays' element type.  A lower-rank `b` repeats over the trailing modes of `dst`.
+"""
+function map!(f, dst::MoYeArray, a::MoYeArray, b::MoYeArray; stream::Ptr{Cvoid} = C_NULL)
+    GC.@preserve dst a b check(ccall((:moye_map, LIB), Int32, (Int32, Ptr{Tensor}, Ptr{Tensor}, Ptr{Tensor}, Cdouble, Ptr{Cvoid}),
+                                     MAP_OPS[f], Ref(Tensor(dst)), Ref(Tensor(a)), Ref(Tensor(b)), 0.0, stream))
+    dst
+end
+function map!(f, dst::MoYeArray, a::MoYeArray, b::Real; stream::Ptr{Cvoid} = C_NULL)
+    GC.@preserve dst a check(ccall((:moye_map, LIB), Int32, (Int32, Ptr{Tensor}, Ptr{Tensor}, Ptr{Tensor}, Cdouble, Ptr{Cvoid}),
+                                   MAP_OPS[f], Ref(Tensor(dst)), Ref(Tensor(a)), C_NULL, Float64(b), stream))
+    dst
+end
+function map!(f, dst::MoYeArray, a::MoYeArray; stream::Ptr{Cvoid} = C_NULL)
+    op = f === (-) ? Int32(7) : MAP_OPS[f]
+    GC.@preserve dst a check(ccall((:moye_map, LIB), Int32, (Int32, Ptr{Tensor}, Ptr{Tensor}, Ptr{Tensor}, Cdouble, Ptr{Cvoid}),
+                                   op, Ref(Tensor(dst)), Ref(Tensor(a)), C_NULL, 0.0, stream))
+    dst
+end
+
 function gemm_workspace_size(mma::TiledMMADesc, D::MoYeArray, A::MoYeArray, B::MoYeArray)
     n = Ref{Csize_t}(0)
     check(ccall((:moye_gemm_workspace_size, LIB), Int32,

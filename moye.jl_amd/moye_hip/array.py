@@ -396,6 +396,25 @@ def fill_(X, value, stream=None):
     return X
 
 
+def map_(op, dst, A, B=None, scalar=0.0, stream=None):
+    """dst .= op.(A, B) or op.(A, scalar) (src/broadcast.jl:5-41; map!, src/algorithm/array_algorithms.jl:192-210);
+    op is one of "identity", "add", "sub", "mul", "div", "max", "min", "neg", "abs".  Returns dst."""
+    t = lambda x: x if isinstance(x, _lib.Tensor) else x.tensor()
+    device.map_(_lib.MAP_OPS[op] if isinstance(op, str) else op, t(dst), t(A), None if B is None else t(B), scalar, stream)
+    return dst
+
+
+def broadcast(op, A, B=None, scalar=0.0, stream=None):
+    """op.(A, B): a new array with `make_layout_like(layout(A))`, as `similar` gives the reference's broadcast
+    (src/broadcast.jl:27-31).  The memory is a torch tensor the result keeps alive."""
+    import torch
+    from .torch_interop import TORCH_DTYPES
+    lay = L.make_layout_like(A.layout)
+    buf = torch.empty(int(L.cosize(lay)), dtype=TORCH_DTYPES[A.dtype], device="cuda")
+    out = MoYeArray(buf.data_ptr(), A.dtype, lay, keep=buf)
+    return map_(op, out, A, B, scalar, stream)
+
+
 def zeros_(X, stream=None):
     """zeros!(x) (src/algorithm/array_algorithms.jl:176-182)."""
     return fill_(X, 0.0, stream)

@@ -91,6 +91,13 @@ def fill_(x, value, stream=None):
     check(f(C.byref(x), value, stream))
 
 
+def map_(op, dst, a, b=None, scalar=0.0, stream=None):
+    """dst .= op.(a, b) / op.(a, scalar) on raw descriptors (moye_map)."""
+    f = lib().moye_map
+    f.argtypes = [C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_double, C.c_void_p]
+    check(f(op, C.byref(dst), C.byref(a), C.byref(b) if b is not None else None, scalar, stream))
+
+
 def mfma_ceiling(in_dtype, random_operands=True, seconds=0.3, stream=None):
     """(TFLOP/s, clock GHz) of an MFMA-only loop on every CU: the matrix pipe's sustained rate on this part."""
     f = lib().moye_mfma_ceiling

@@ -10,6 +10,12 @@ if hasattr(torch, "float8_e4m3fn"):
     _DT[torch.float8_e4m3fn] = _lib.F8E4M3
 
 
+# moye dtype -> torch dtype (the first torch type registered for it)
+TORCH_DTYPES = {}
+for _t, _m in _DT.items():
+    TORCH_DTYPES.setdefault(_m, _t)
+
+
 def dtype_of(t):
     return _DT[t.dtype]
 

@@ -15,7 +15,7 @@ from __future__ import annotations
 
 import numpy as np
 
-from layout_oracle import (COLON, S, Layout, SL, _0, _1, append, capacity, coalesce, composition,
+from layout_oracle import (COLON, S, Layout, SL, _0, _1, append, lflatten, capacity, coalesce, composition,
                            complement, cosize, dice, dice_layout, get_congr_coord, is_static,
                            is_tuple, lappend, lgroup, logical_divide, logical_product, lprepend,
                            lrank, ltranspose, lzip, make_fragment_like, make_layout,
@@ -608,6 +608,58 @@ def axpby(a, X, b, Y):
     ax = (at * x).astype(T)
     Y.buf[oy] = ax if bt == 0 else (ax + (bt * y).astype(T)).astype(T)
     return Y
+
+
+def _julia_max(x, y):
+    """base/math.jl max(x::T, y::T): ifelse((y > x) | (signbit(y) < signbit(x)), ifelse(isnan(x), x, y), ifelse(isnan(y), y, x))."""
+    with np.errstate(invalid="ignore"):
+        cond = (y > x) | (np.signbit(y) < np.signbit(x))
+    return np.where(cond, np.where(np.isnan(x), x, y), np.where(np.isnan(y), y, x))
+
+
+def _julia_min(x, y):
+    with np.errstate(invalid="ignore"):
+        cond = (y < x) | (np.signbit(y) > np.signbit(x))
+    return np.where(cond, np.where(np.isnan(x), x, y), np.where(np.isnan(y), y, x))
+
+
+BROADCAST_OPS = {
+    "identity": lambda x, y: x, "add": lambda x, y: x + y, "sub": lambda x, y: x - y, "mul": lambda x, y: x * y,
+    "div": lambda x, y: x / y, "max": _julia_max, "min": _julia_min, "neg": lambda x, y: -x, "abs": lambda x, y: np.abs(x),
+}
+
+
+def broadcast(op, A, B=None, scalar=0.0, out=None):
+    """src/broadcast.jl:5-41 — `op.(A, B)` for arrays with static layouts.  The result is an owning array with
+    `make_layout_like(layout(A))` (broadcast.jl:27-31, `similar`) unless `out` is given (`out .= op.(A, B)`).  B
+    may be an array with as many elements as A, an array spanning a leading group of A's modes (a lower-rank
+    array: Julia repeats it over the trailing modes), or None (the second operand is `scalar`).  One operation
+    per element, rounded in the element type (Float16 computes in Float32 and rounds, as numpy does; bf16
+    arrays are float32 buffers holding bf16 values)."""
+    f = BROADCAST_OPS[op]
+    n = len(A)
+    oa = A.offsets()
+    bf16 = getattr(A, "bf16", False)
+    T = np.float32 if bf16 else A.buf.dtype.type
+    x = A.buf[oa].astype(T)
+    if B is None:
+        y = round_bf16(np.float32(scalar)) if bf16 else T(scalar)
+    else:
+        nb = len(B)
+        shp = lflatten(A.layout).shape
+        shp = [int(v) for v in shp] if isinstance(shp, tuple) else [int(shp)]
+        assert nb in (n, 1) or nb in list(np.cumprod(shp)), "cannot broadcast %d elements over %s" % (nb, shp)
+        y = B.buf[B.offsets()].astype(T)[np.arange(n) % nb]
+    with np.errstate(all="ignore"):
+        r = np.asarray(f(x, y)).astype(T)
+    if bf16:
+        r = round_bf16(r)
+    if out is None:
+        out = Array.undef(A.buf.dtype.type, make_layout_like(A.layout))
+        if bf16:
+            out.bf16 = True
+    out.buf[out.offsets()] = r
+    return out
 
 
 def fill(X, value):

@@ -267,6 +267,70 @@ def test_fill_and_zeros(mh):
         assert float(y.abs().max()) == 0.0
 
 
+MAP_LAYOUTS = [("(_4,_6):(_1,_4)", "(_4,_6):(_6,_1)", "(_4,_6):(_1,_8)"),           # dst, a, b
+               ("((_2,_3),(_2,_4)):((_1,_16),(_2,_4))", "(_6,_8):(_1,_6)", "(_6):(_2)"),   # b spans the first mode of dst
+               ("(_3,_5,_7):(_1,_3,_15)", "(_3,_5,_7):(_35,_7,_1)", "(_3,_5):(_5,_1)")]     # ... and the first two of three
+
+
+@pytest.mark.parametrize("dt", ["float32", "float64", "float16", "bfloat16"])
+def test_map_bit_exact_against_the_oracle(mh, dt):
+    """dst .= op.(a, b) for every operation, array, lower-rank and scalar second operands, through
+    hierarchical and padded layouts; NaNs and signed zeros included (Julia's max/min rules)."""
+    tdt = getattr(torch, dt)
+    g = torch.Generator().manual_seed(23)
+    for ld_text, la_text, lb_text in MAP_LAYOUTS:
+        ld, la, lb = lo.parse_layout(ld_text), lo.parse_layout(la_text), lo.parse_layout(lb_text)
+        nd, na, nb = int(lo.cosize(ld)), int(lo.cosize(la)), int(lo.cosize(lb))
+        for op in ("identity", "add", "sub", "mul", "div", "max", "min", "neg", "abs"):
+            for second in ("array", "scalar"):
+                A = (torch.randn(na, generator=g) * 3).to(tdt)
+                B = (torch.randn(nb, generator=g) * 3).to(tdt)
+                if dt in ("float32", "float64"):
+                    A[1], A[3], B[0] = float("nan"), -0.0, 0.0
+                    B[2] = float("nan")
+                Dst = torch.full((nd,), 9.0, dtype=tdt)
+                a, b, d = A.cuda(), B.cuda(), Dst.cuda()
+                sd, dd = _flat(ld)
+                sa, da = _flat(la)
+                sb, db = _flat(lb)
+                mh.map_(op, _tens(mh, d, sd, dd), _tens(mh, a, sa, da), _tens(mh, b, sb, db) if second == "array" else None, 1.75)
+                torch.cuda.synchronize()
+                conv = (lambda t: t.float().numpy().copy()) if dt == "bfloat16" else (lambda t: t.numpy().copy())
+                oa, ob, od = to.Array(conv(A), la), to.Array(conv(B), lb), to.Array(conv(Dst), ld)
+                if dt == "bfloat16":
+                    oa.bf16 = ob.bf16 = od.bf16 = True
+                to.broadcast(op, oa, ob if second == "array" else None, 1.75, out=od)
+                got, want = d.cpu(), torch.from_numpy(od.buf).to(tdt)
+                itype = {2: torch.int16, 4: torch.int32, 8: torch.int64}[got.element_size()]
+                same = got.view(itype) == want.view(itype)
+                both_nan = torch.isnan(got.float()) & torch.isnan(want.float())     # NaN payloads are not compared
+                assert bool((same | both_nan).all()), (dt, op, second, ld_text)
+
+
+def test_broadcast_returns_a_compact_array_like_the_first_operand(mh):
+    """test/broadcast.jl:3-17 on the device: `x .+ x`, `x .+ 1`, `x .+ y` with a lower-rank y."""
+    from moye_hip import MoYeArray
+    xt = torch.arange(1, 7, dtype=torch.float32, device="cuda")
+    x = MoYeArray(xt.data_ptr(), mh.F32, lo_text("(_3,_2):(_1,_3)", mh), keep=xt)
+    x2, x3 = mh.broadcast("add", x, x), mh.broadcast("add", x, None, 1.0)
+    torch.cuda.synchronize()
+    assert str(x2.layout) == str(x.layout) and x2.ptr != x.ptr
+    assert x2._keep.tolist() == [2, 4, 6, 8, 10, 12] and x3._keep.tolist() == [2, 3, 4, 5, 6, 7]
+    yt = torch.tensor([10, 0, 20, 0, 30, 0], dtype=torch.float32, device="cuda")
+    y = MoYeArray(yt.data_ptr(), mh.F32, lo_text("(_3):(_2)", mh), keep=yt)
+    z = mh.broadcast("add", x, y)
+    torch.cuda.synchronize()
+    assert str(z.layout) == str(x.layout) and z._keep.tolist() == [11, 22, 33, 14, 25, 36]
+    with pytest.raises(mh.MoyeError):
+        w = torch.zeros(4, device="cuda")
+        mh.map_("add", x, x, MoYeArray(w.data_ptr(), mh.F32, lo_text("(_4):(_1)", mh), keep=w))
+
+
+def lo_text(text, mh):
+    from moye_hip.layout import Layout
+    return Layout(text)
+
+
 def test_axpby_errors(mh):
     x = torch.zeros(8, device="cuda")
     y = torch.zeros(8, dtype=torch.float16, device="cuda")

@@ -373,3 +373,43 @@ def test_axpby_known_answers():
     Z = to.Array(np.zeros(8, f32), lo.make_layout((S(2), S(2)), (S(1), S(4))))
     to.fill(Z, 7)
     assert Z.buf.tolist() == [7, 7, 0, 0, 7, 7, 0, 0]
+
+
+def test_broadcast_layouts_and_known_answers():
+    """test/broadcast.jl:3-17: `x .+ x`, `x .+ 1` and `x .+ y` (y of lower rank) give owning arrays with x's
+    layout; values by hand."""
+    f32 = np.float32
+    x = to.Array(np.arange(1, 7, dtype=f32), lo.make_layout((S(3), S(2))))
+    x2 = to.broadcast("add", x, x)
+    x3 = to.broadcast("add", x, None, 1)
+    assert x2.layout == L("(_3,_2):(_1,_3)") and x3.layout == x2.layout
+    assert x2.buf.tolist() == [2, 4, 6, 8, 10, 12] and x3.buf.tolist() == [2, 3, 4, 5, 6, 7]
+    assert x2.buf is not x.buf                                      # an owning result (ArrayEngine), x untouched
+    y = to.Array(np.array([10, 0, 20, 0, 30, 0], f32), lo.make_layout((S(3),), (S(2),)))
+    z = to.broadcast("add", x, y)                                   # test/broadcast.jl:15-17
+    assert z.layout == x.layout
+    assert z.buf.tolist() == [11, 22, 33, 14, 25, 36]               # y repeats over the second mode
+    # through layouts: make_layout_like keeps the order of the strides (a row-major view gives a row-major result),
+    # a padded view gives a compact one; operands meet by logical index
+    xr = to.Array(np.arange(1, 7, dtype=f32), lo.make_layout((S(3), S(2)), (S(2), S(1))))
+    r = to.broadcast("mul", xr, None, 2)
+    assert r.layout == L("(_3,_2):(_2,_1)") and r.buf.tolist() == [2, 4, 6, 8, 10, 12]
+    xp = to.Array(np.arange(8, dtype=f32), lo.make_layout((S(3), S(2)), (S(1), S(4))))    # pitch 4: 0 1 2 | 4 5 6
+    rp = to.broadcast("add", xp, x)
+    assert rp.layout == L("(_3,_2):(_1,_3)") and rp.buf.tolist() == [1, 3, 5, 8, 10, 12]
+    # device/broadcast.jl:5-9 in numbers: fill!(a, 1); a .= a .* 2; sum(a) == 12
+    a = to.Array(np.zeros(6, np.float64), lo.make_layout((S(3), S(2))))
+    to.fill(a, 1.0)
+    to.broadcast("mul", a, None, 2, out=a)
+    assert a.buf.sum() == 12.0
+    # Julia's max/min on floats: the NaN operand wins, and the signs of zeros are ordered
+    u = to.Array(np.array([np.nan, 1.0, -0.0, 0.0], f32), lo.make_layout(S(4)))
+    v = to.Array(np.array([1.0, np.nan, 0.0, -0.0], f32), lo.make_layout(S(4)))
+    mx, mn = to.broadcast("max", u, v).buf, to.broadcast("min", u, v).buf
+    assert np.isnan(mx[0]) and np.isnan(mx[1]) and np.isnan(mn[0]) and np.isnan(mn[1])
+    assert not np.signbit(mx[2]) and not np.signbit(mx[3]) and np.signbit(mn[2]) and np.signbit(mn[3])
+    # fp16: one rounding per operation
+    h = np.float16
+    p = to.Array(np.array([0.1, 1000.0], h), lo.make_layout(S(2)))
+    q = to.broadcast("mul", p, None, 3.0)
+    assert q.buf[0] == h(np.float32(h(0.1)) * np.float32(3.0)) and q.buf.dtype == h

@@ -67,12 +67,12 @@ def _compile(item, force):
 ASM_MFMA_SOURCES = ["gemm_mfma256w4.hip"]
 
 
-def check_accumulator_hazards(src):
+def check_accumulator_hazards(src, force=False):
     """Compile `src` to assembly and fail if, in any basic block that holds v_mfma instructions, something
     other than a v_mfma names an AccVGPR before the kernel's `MOYE_ACC_SETTLED` marker."""
     path = os.path.join(CSRC, src)
     asm = os.path.join(CSRC, "build", os.path.splitext(src)[0] + ".s")
-    if not _stale(asm, [path] + _headers()):
+    if not force and not _stale(asm, [path] + _headers()):
         return
     cmd = [HIPCC] + COMMON + ["-S", "--cuda-device-only", path, "-o", asm]
     r = subprocess.run(cmd, capture_output=True, text=True)
@@ -119,7 +119,7 @@ def build(force=False, verbose=True):
     with ThreadPoolExecutor(max_workers=min(8, len(items))) as ex:
         results = list(ex.map(lambda it: _compile(it, force), items))
     for src in ASM_MFMA_SOURCES:
-        check_accumulator_hazards(src)
+        check_accumulator_hazards(src, force)
     objs = [o for o, _ in results]
     for (src, _), (_, msg) in zip(items, results):
         if msg.strip() and verbose:

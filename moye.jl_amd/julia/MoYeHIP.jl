@@ -204,6 +204,9 @@ function layout_index(l::Layout, coord)
     check(ccall((:moye_layout_eval, LIB), Int32, (Cstring, Cstring, Ptr{Int64}), string(l), string(coord), idx))
     idx[]
 end
+# The library computes in 64 bits; the reference's index has the integer type of the coordinate
+# (`@Layout((2,(2,2)),(2,(1,4)))(Int32(2)) isa Int32`, test/layout.jl:4-12): an Int32 coordinate gets an Int32 index back.
+layout_index(l::Layout, coord::Int32) = Int32(invoke(layout_index, Tuple{Layout,Any}, l, coord))
 
 function layout_size(l::Layout)
     n = Ref{Int64}(0)

@@ -37,18 +37,30 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_skinny(GemmArgs p) {
 #pragma unroll
         for (int t = 0; t < NTW; ++t) acc[i][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    int s = s0;
-    for (; s + U <= s1; s += U) {
+    // Every workgroup needs all of A, and workgroups that walk K in the same order ask the L2 for the same lines of A
+    // at the same moment, before any of them has them.  So a workgroup starts its walk at a step that depends on
+    // its position within its L2's share of the grid (consecutive workgroups go to consecutive L2s), in units of U
+    // steps so that a trip still covers whole 128-byte lines of B (measured at 16 x 8192 x 8192 bf16: 146 MiB
+    // fetched instead of 161, 32.9 us instead of 34.0).  The order of a column's k-sum follows the workgroup, not
+    // the time, so results stay reproducible.
+    const int len = s1 - s0;
+    const int first = len >= U && len % U == 0 ? U * (int)((blockIdx.x / 8) % (unsigned)(len / U)) : 0;
+    auto step_of = [&](int t) { const int r = t + first; return s0 + (r >= len ? r - len : r); };
+    int t0 = 0;
+    for (; t0 + U <= len; t0 += U) {
         u32x4 b[NTW][U], a[MT][U];
+        int64_t off[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) off[u] = (int64_t)step_of(t0 + u) * 64;
 #pragma unroll
         for (int t = 0; t < NTW; ++t)
 #pragma unroll
             for (int u = 0; u < U; ++u)
-                b[t][u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(bp[t] + (int64_t)(s + u) * 64));
+                b[t][u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(bp[t] + off[u]));
 #pragma unroll
         for (int i = 0; i < MT; ++i)
 #pragma unroll
-            for (int u = 0; u < U; ++u) a[i][u] = *reinterpret_cast<const u32x4*>(ap[i] + (int64_t)(s + u) * 64);
+            for (int u = 0; u < U; ++u) a[i][u] = *reinterpret_cast<const u32x4*>(ap[i] + off[u]);
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -56,13 +68,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_skinny(GemmArgs p) {
 #pragma unroll
                 for (int t = 0; t < NTW; ++t) In::mma(b[t][u], a[i][u], acc[i][t]);
     }
-    for (; s < s1; ++s) {
+    for (; t0 < len; ++t0) {
+        const int64_t off = (int64_t)step_of(t0) * 64;
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
-            const u32x4 a = *reinterpret_cast<const u32x4*>(ap[i] + (int64_t)s * 64);
+            const u32x4 a = *reinterpret_cast<const u32x4*>(ap[i] + off);
 #pragma unroll
             for (int t = 0; t < NTW; ++t)
-                In::mma(__builtin_nontemporal_load(reinterpret_cast<const u32x4*>(bp[t] + (int64_t)s * 64)), a, acc[i][t]);
+                In::mma(__builtin_nontemporal_load(reinterpret_cast<const u32x4*>(bp[t] + off)), a, acc[i][t]);
         }
     }
 

@@ -223,7 +223,12 @@ int32_t moye_local_partition(const char* layout, const char* thr_tile, const cha
 /* TiledMMA (src/atom/mma.jl): `atom` is a moye_mma_atom or the name of one of the reference's
  * NVIDIA atoms kept as data for its tests ("MMAOP_16x8x8_F16F16F16F16_TN", ...).
  * what = "thr_layout_vmnk" | "tile_shape" | "layout_a" | "layout_b" | "layout_c" |
- *        "layoutA_TV" | "layoutB_TV" | "layoutC_TV" | "size"                                  */
+ *        "layoutA_TV" | "layoutB_TV" | "layoutC_TV" | "size" |
+ *        "layoutA_MK" | "layoutB_NK" | "layoutC_MN" with "thrID_A" | "thrID_B" | "thrID_C"
+ *        (get_layoutA_MK / B_NK / C_MN, atom/mma.jl:235-262: both values of each pair) |
+ *        "print": the three tables print_typst(tiled_mma) draws (print.jl:46-93,317-323) as text,
+ *        B as (K, N), then A (M, K), then C (M, N); a cell reads T<thread index>V<value index>,
+ *        1-based as the reference prints them.  A table of a 256 x 256 tile needs about 1 MB.   */
 int32_t moye_tiled_mma_query(const char* atom, const char* atom_layout, const char* permutation,
                              const char* what, char* out, size_t cap);
 /* partition_A/B/C of get_slice(mma, thr_idx) (atom/mma.jl:171-175,292-308); operand = 'A'|'B'|'C' */
@@ -241,8 +246,11 @@ int32_t moye_tiled_copy_partition(int32_t src_bits, int32_t dst_bits, int32_t va
                                   char which, const char* layout, char* out, size_t cap, int64_t* offset);
 /* TiledCopy(atom, layout_tv, tiler) (atom/copy.jl:113-125): the form make_tiled_copy_A/B/C build from a
  * TiledMMA (atom/copy.jl:227-240: layout_tv = get_layoutA/B/C_TV(mma), tiler = its tile sizes).
- * what = "layoutS_TV" | "layoutD_TV" (atom/copy.jl:168-187) | "num_val_src" | "num_val_dst" | "size";
- * the two names are accepted by moye_tiled_copy_query too. */
+ * what = "layoutS_TV" | "layoutD_TV" (atom/copy.jl:168-187) | "layoutS_MN" | "layoutD_MN"
+ * (atom/copy.jl:175-179,188-192; their thread-id layout is size:1) | "num_val_src" | "num_val_dst" |
+ * "size" | "print": the source and destination tables print_typst(tiled_copy) draws
+ * (print.jl:200-233,337-345) as text, cells T<thread>V<value>.  The TV, MN and print names are
+ * accepted by moye_tiled_copy_query too. */
 int32_t moye_tiled_copy_tv_query(int32_t src_bits, int32_t dst_bits, int32_t val_bits, const char* layout_tv,
                                  const char* tiler, const char* what, char* out, size_t cap);
 int32_t moye_tiled_copy_tv_partition(int32_t src_bits, int32_t dst_bits, int32_t val_bits, const char* layout_tv,

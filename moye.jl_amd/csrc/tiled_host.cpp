@@ -154,7 +154,55 @@ struct TiledMMAHost {
         const Tile btile = tile_tuple({tile_colon(), tile_tuple({tile_of(make_layout(mn, tup({SI(0), SI(1)}))), tile_colon()})});
         return composition(composition(thrfrg_B(ref), tile_tuple({btile, tile_colon()})), tile_tuple({inv, tile_colon()}));
     }
+    // get_layoutC_MN / get_layoutA_MK / get_layoutB_NK (atom/mma.jl:235-262): cell of the tile -> index into the
+    // (thr, val) fragment layout, and the layout from the thread part of that index to the thread index
+    std::pair<Layout, Layout> layout_mn(char operand) const {
+        const Layout t = thr_layout_vmnk();
+        const IT c = IT::colon(), one = SI(1);
+        switch (operand) {
+            case 'C': {
+                const Layout ref = make_layout(tup({IT(tile_size(1)), IT(tile_size(2))}));
+                return {composition(right_inverse(thrfrg_C(ref)), ref), slice_layout(t, tup({c, c, c, one}))};
+            }
+            case 'A': {
+                const Layout ref = make_layout(tup({IT(tile_size(1)), IT(tile_size(3))}));
+                return {composition(right_inverse(thrfrg_A(ref)), ref), slice_layout(t, tup({c, c, one, c}))};
+            }
+            case 'B': {
+                const Layout ref = make_layout(tup({IT(tile_size(2)), IT(tile_size(3))}));
+                return {composition(right_inverse(thrfrg_B(ref)), ref), slice_layout(t, tup({c, one, c, c}))};
+            }
+            default: raise(MOYE_ERR_ARG, "operand must be 'A', 'B' or 'C'");
+        }
+    }
 };
+
+// The table print_typst draws for one operand (src/print.jl:64-71,220-228) as text: cell (m, n) holds
+// "T<thr_idx>V<val_idx>" with val_idx, thr = fldmod1(layout_mn(m, n), size(thr_id)) and thr_idx = thr_id(thr), all
+// 1-based.  `transposed` draws cell (n, m) at row m, as the reference does for B above C.
+static std::string tv_table_text(const std::string& title, const Layout& layout_mn, const Layout& thr_id, bool transposed) {
+    const int64_t nthr = size(thr_id).v;
+    const int64_t d1 = size(layout_mn, 1).v, d2 = size(layout_mn, 2).v;
+    const int64_t rows = transposed ? d2 : d1, cols = transposed ? d1 : d2;
+    const int64_t nval = (size(layout_mn).v + nthr - 1) / nthr;
+    const int w = (int)("T" + std::to_string(cosize(thr_id).v) + "V" + std::to_string(nval)).size() + 2;
+    auto lpad = [](const std::string& t, int n) { return (int)t.size() >= n ? t : std::string((size_t)n - t.size(), ' ') + t; };
+    std::string sep = "     ";
+    for (int64_t n = 0; n < cols; ++n) sep += "+" + std::string((size_t)w, '-');
+    sep += "+";
+    std::string r = title + "\n     ";
+    for (int64_t n = 1; n <= cols; ++n) r += "  " + lpad(std::to_string(n), w - 2) + " ";
+    for (int64_t m = 1; m <= rows; ++m) {
+        r += "\n" + sep + "\n" + lpad(std::to_string(m), 3) + "  ";
+        for (int64_t n = 1; n <= cols; ++n) {
+            const int64_t idx = eval(layout_mn, transposed ? tup({IT(D(n)), IT(D(m))}) : tup({IT(D(m)), IT(D(n))})).v - 1;
+            const int64_t thr = eval(thr_id, IT(D(idx % nthr + 1))).v;
+            r += "| " + lpad("T" + std::to_string(thr) + "V" + std::to_string(idx / nthr + 1), w - 2) + " ";
+        }
+        r += "|";
+    }
+    return r + "\n" + sep + "\n";
+}
 
 // CopyAtom + TiledCopy (src/atom/copy.jl:3-59,86-258) for UniversalCopy{S,D} over values of val_bits
 struct TiledCopyHost {
@@ -220,6 +268,15 @@ struct TiledCopyHost {
         const Layout ref = make_layout(tup({tiler, SI(1)}));
         const Layout t = tile2thrfrg(ref, composition(right_inverse(val_ref), trg));
         return slice_layout(t, tup({IT::colon(), IT::colon(), SI(1)}));
+    }
+    // get_layoutS_MN / get_layoutD_MN (atom/copy.jl:175-179,188-192)
+    std::pair<Layout, Layout> layout_MN(char which) const {
+        return {composition(right_inverse(layout_TV(which)), make_layout(tiler)), make_layout(IT(size(layout_tv, 1)))};
+    }
+    std::string print() const {  // print_typst(tiled_copy), src/print.jl:337-345
+        const auto s = layout_MN('S'), d = layout_MN('D');
+        return tv_table_text("S " + to_string(tiler), s.first, s.second, false) + "\n" +
+               tv_table_text("D " + to_string(tiler), d.first, d.second, false);
     }
     Layout retile(const Layout& x) const {  // atom/copy.jl:151-166
         const Int v = size(x, 1);
@@ -624,6 +681,17 @@ int32_t moye_tiled_mma_query(const char* atom, const char* atom_layout, const ch
         if (what == "layoutA_TV") return put(to_string(m.layout_tv('A')), out, cap);
         if (what == "layoutB_TV") return put(to_string(m.layout_tv('B')), out, cap);
         if (what == "layoutC_TV") return put(to_string(m.layout_tv('C')), out, cap);
+        if (what == "layoutA_MK") return put(to_string(m.layout_mn('A').first), out, cap);
+        if (what == "layoutB_NK") return put(to_string(m.layout_mn('B').first), out, cap);
+        if (what == "layoutC_MN") return put(to_string(m.layout_mn('C').first), out, cap);
+        if (what == "thrID_A") return put(to_string(m.layout_mn('A').second), out, cap);
+        if (what == "thrID_B") return put(to_string(m.layout_mn('B').second), out, cap);
+        if (what == "thrID_C") return put(to_string(m.layout_mn('C').second), out, cap);
+        if (what == "print") {  // print_typst(tiled_mma), src/print.jl:317-323: B drawn as (K, N), then A, then C
+            const auto A = m.layout_mn('A'), B = m.layout_mn('B'), C = m.layout_mn('C');
+            return put(tv_table_text("B (K, N)", B.first, B.second, true) + "\n" + tv_table_text("A (M, K)", A.first, A.second, false) +
+                           "\n" + tv_table_text("C (M, N)", C.first, C.second, false), out, cap);
+        }
         throw Error(MOYE_ERR_UNSUPPORTED, "unknown TiledMMA query \"" + what + "\"");
     });
 }
@@ -647,6 +715,9 @@ int32_t moye_tiled_copy_query(int32_t src_bits, int32_t dst_bits, int32_t val_bi
         if (what == "layout_tv") return put(to_string(tc.layout_tv), out, cap);
         if (what == "layoutS_TV") return put(to_string(tc.layout_TV('S')), out, cap);
         if (what == "layoutD_TV") return put(to_string(tc.layout_TV('D')), out, cap);
+        if (what == "layoutS_MN") return put(to_string(tc.layout_MN('S').first), out, cap);
+        if (what == "layoutD_MN") return put(to_string(tc.layout_MN('D').first), out, cap);
+        if (what == "print") return put(tc.print(), out, cap);
         if (what == "tiler") return put(to_string(tc.tiler), out, cap);
         if (what == "num_val_src") return put(to_string(IT(tc.num_val_src())), out, cap);
         if (what == "num_val_dst") return put(to_string(IT(tc.num_val_dst())), out, cap);
@@ -674,6 +745,9 @@ int32_t moye_tiled_copy_tv_query(int32_t src_bits, int32_t dst_bits, int32_t val
         const std::string what = what_;
         if (what == "layoutS_TV") return put(to_string(tc.layout_TV('S')), out, cap);
         if (what == "layoutD_TV") return put(to_string(tc.layout_TV('D')), out, cap);
+        if (what == "layoutS_MN") return put(to_string(tc.layout_MN('S').first), out, cap);
+        if (what == "layoutD_MN") return put(to_string(tc.layout_MN('D').first), out, cap);
+        if (what == "print") return put(tc.print(), out, cap);
         if (what == "num_val_src") return put(to_string(IT(tc.num_val_src())), out, cap);
         if (what == "num_val_dst") return put(to_string(IT(tc.num_val_dst())), out, cap);
         if (what == "size") return put(to_string(IT(size(tc.layout_tv, 1))), out, cap);

@@ -257,12 +257,16 @@ function make_tiled_mma(atom::Int32, atom_layout::Layout, permutation::Tuple = (
     d[]
 end
 
-function tiled_mma_query(atom::AbstractString, atom_layout::Layout, permutation, what::AbstractString)
-    buf = Vector{UInt8}(undef, CAP)
+function tiled_mma_query(atom::AbstractString, atom_layout::Layout, permutation, what::AbstractString; cap = CAP)
+    buf = Vector{UInt8}(undef, cap)
     check(ccall((:moye_tiled_mma_query, LIB), Int32, (Cstring, Cstring, Cstring, Cstring, Ptr{UInt8}, Csize_t),
-                atom, string(atom_layout), permutation === nothing ? "" : tile_text(permutation), what, buf, CAP))
+                atom, string(atom_layout), permutation === nothing ? "" : tile_text(permutation), what, buf, cap))
     unsafe_string(pointer(buf))
 end
+
+"The tables print_typst(tiled_mma) draws (src/print.jl:46-93,317-323) as text: B as (K, N), then A, then C."
+print_tv(atom::AbstractString, atom_layout::Layout, permutation = nothing) =
+    println(tiled_mma_query(atom, atom_layout, permutation, "print"; cap = 1 << 23))
 
 "partition_A/B/C(get_slice(mma, thr_idx), x) computed by the library (operand = 'A', 'B' or 'C')."
 function tiled_mma_partition(atom::AbstractString, atom_layout::Layout, permutation, thr_idx::Integer,
@@ -275,13 +279,17 @@ function tiled_mma_partition(atom::AbstractString, atom_layout::Layout, permutat
     MoYeArray(pointer(x) + off[] * sizeof(T), parse_layout(unsafe_string(pointer(buf))))
 end
 
-function tiled_copy_query(src_bits, dst_bits, val_bits, thr::Layout, val::Layout, what::AbstractString)
-    buf = Vector{UInt8}(undef, CAP)
+function tiled_copy_query(src_bits, dst_bits, val_bits, thr::Layout, val::Layout, what::AbstractString; cap = CAP)
+    buf = Vector{UInt8}(undef, cap)
     check(ccall((:moye_tiled_copy_query, LIB), Int32,
                 (Int32, Int32, Int32, Cstring, Cstring, Cstring, Ptr{UInt8}, Csize_t),
-                Int32(src_bits), Int32(dst_bits), Int32(val_bits), string(thr), string(val), what, buf, CAP))
+                Int32(src_bits), Int32(dst_bits), Int32(val_bits), string(thr), string(val), what, buf, cap))
     unsafe_string(pointer(buf))
 end
+
+"The source and destination tables print_typst(tiled_copy) draws (src/print.jl:200-233,337-345) as text."
+print_tv(src_bits::Integer, dst_bits::Integer, val_bits::Integer, thr::Layout, val::Layout) =
+    println(tiled_copy_query(src_bits, dst_bits, val_bits, thr, val, "print"; cap = 1 << 23))
 
 function tiled_copy_partition(src_bits, dst_bits, val_bits, thr::Layout, val::Layout, thr_idx::Integer,
                               which::Char, x::MoYeArray{T}) where {T}

@@ -99,6 +99,12 @@ ATOM_NAMES = ["UniversalFMA", "MFMA_F32_16x16x32_F16", "MFMA_F32_32x32x16_F16", 
               "MFMA_F32_32x32x2_F32"]
 
 
+def _emit(text, file):
+    if file is not False:
+        print(text, file=file)
+    return text
+
+
 class TiledMMA:
     """make_tiled_mma(op, atom_layout, permutations) (src/atom/mma.jl:193-233).  `op` is a
     moye_mma_atom number or an atom name (the reference's NVIDIA atoms exist by name, as data)."""
@@ -137,6 +143,15 @@ class TiledMMA:
 
     def layout_tv(self, operand):
         return Layout(self._q("layout%s_TV" % operand))
+
+    def layout_mn(self, operand):
+        """get_layoutA_MK / get_layoutB_NK / get_layoutC_MN (src/atom/mma.jl:235-262): (layout, thread-id layout)."""
+        return Layout(self._q({"A": "layoutA_MK", "B": "layoutB_NK", "C": "layoutC_MN"}[operand])), Layout(self._q("thrID_" + operand))
+
+    def print_tv(self, file=None):
+        """The three tables print_typst(tiled_mma) draws (src/print.jl:46-93,317-323), as text: B as (K, N), then A,
+        then C; a cell reads T<thread index>V<value index>.  Returns the text; file=False only returns it."""
+        return _emit(self._q("print"), file)
 
     def get_slice(self, thr_idx):
         return ThrMMA(self, thr_idx)
@@ -247,6 +262,18 @@ class TiledCopy:
     def get_layoutD_TV(self):
         return Layout(self._q("layoutD_TV"))
 
+    def get_layoutS_MN(self):
+        """src/atom/copy.jl:175-179: (layout, thread-id layout)."""
+        return Layout(self._q("layoutS_MN")), L.static_layout(self.size())
+
+    def get_layoutD_MN(self):
+        """src/atom/copy.jl:188-192."""
+        return Layout(self._q("layoutD_MN")), L.static_layout(self.size())
+
+    def print_tv(self, file=None):
+        """The source and destination tables print_typst(tiled_copy) draws (src/print.jl:200-233,337-345), as text."""
+        return _emit(self._q("print"), file)
+
     def descriptor(self):
         d = _lib.TiledCopy()
         d.op, d.vec_bits, d.flags = self.op, self.atom.src_bits, self.flags
@@ -287,6 +314,15 @@ class TiledCopyTV:
 
     def get_layoutD_TV(self):
         return Layout(self._q("layoutD_TV"))
+
+    def get_layoutS_MN(self):
+        return Layout(self._q("layoutS_MN")), L.static_layout(self.size())
+
+    def get_layoutD_MN(self):
+        return Layout(self._q("layoutD_MN")), L.static_layout(self.size())
+
+    def print_tv(self, file=None):
+        return _emit(self._q("print"), file)
 
     def retile(self, x):
         """retile_S / retile_D (src/atom/copy.jl:151-166) on a MoYeArray or a Layout."""

@@ -10,6 +10,7 @@ from . import _lib
 from ._lib import check, lib
 
 _CAP = 8192
+_BIG_CAP = 1 << 23
 
 
 class StaticInt(int):
@@ -94,7 +95,11 @@ def _tile_text(t):
 
 def _text_out(fn, *args):
     buf = C.create_string_buffer(_CAP)
-    check(fn(*args, buf, _CAP))
+    status = fn(*args, buf, _CAP)
+    if status == _lib.ERR_BUFFER:  # printed tables outgrow the usual buffer
+        buf = C.create_string_buffer(_BIG_CAP)
+        status = fn(*args, buf, _BIG_CAP)
+    check(status)
     return buf.value.decode()
 
 

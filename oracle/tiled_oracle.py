@@ -293,6 +293,37 @@ class TiledMMA:
         return composition(composition(tv, (btile, COLON)), (right_inverse(t), COLON))
 
 
+    # atom/mma.jl:235-262: cell of the tile -> index into the un-permuted (thr, val) fragment layout, together with
+    # the layout that turns the thread part of that index into a thread index (the other operand's atoms dropped)
+    def get_layoutC_MN(self):
+        ref = make_layout((self.tile_size(1), self.tile_size(2)))
+        return withshape(right_inverse(self.thrfrg_C(ref)), ref.shape), self.thr_layout_vmnk()((COLON, COLON, COLON, _1))
+
+    def get_layoutA_MK(self):
+        ref = make_layout((self.tile_size(1), self.tile_size(3)))
+        return withshape(right_inverse(self.thrfrg_A(ref)), ref.shape), self.thr_layout_vmnk()((COLON, COLON, _1, COLON))
+
+    def get_layoutB_NK(self):
+        ref = make_layout((self.tile_size(2), self.tile_size(3)))
+        return withshape(right_inverse(self.thrfrg_B(ref)), ref.shape), self.thr_layout_vmnk()((COLON, _1, COLON, COLON))
+
+
+def tv_table(layout_mn, thr_id):
+    """The cells print_typst writes (src/print.jl:64-71,220-228): for cell (m, n) of the tile,
+    `val_idx, thr = fldmod1(layout_mn(m, n), size(thr_id))` and `thr_idx = thr_id(thr)`; returns
+    table[m][n] = (thr_idx, val_idx), both 1-based as the reference prints them."""
+    nthr = int(size(thr_id))
+    rows, cols = int(size(layout_mn, 1)), int(size(layout_mn, 2))
+    out = []
+    for m in range(1, rows + 1):
+        row = []
+        for n in range(1, cols + 1):
+            idx = int(layout_mn((m, n))) - 1
+            row.append((int(thr_id(idx % nthr + 1)), idx // nthr + 1))
+        out.append(row)
+    return out
+
+
 def make_tiled_mma(op, atom_layout=None, permutations=None):
     """atom/mma.jl:193-199,229-233."""
     return TiledMMA(op, atom_layout, permutations)
@@ -437,6 +468,16 @@ class TiledCopy:
         ref = make_layout((self.tiler_MN, _1))
         return self.tile2thrfrg(ref, composition(right_inverse(a.val_layout_ref),
                                                  a.val_layout_dst))((COLON, COLON, _1))
+
+    def get_layoutS_MN(self):
+        """atom/copy.jl:175-179."""
+        return (composition(right_inverse(self.get_layoutS_TV()), make_layout(self.tiler_MN)),
+                make_layout(size(self.tiled_layout_TV, 1)))
+
+    def get_layoutD_MN(self):
+        """atom/copy.jl:188-192."""
+        return (composition(right_inverse(self.get_layoutD_TV()), make_layout(self.tiler_MN)),
+                make_layout(size(self.tiled_layout_TV, 1)))
 
     def get_slice(self, thr_idx):
         return ThrCopy(self, thr_idx)

@@ -131,3 +131,95 @@ def test_host_library_agrees_on_the_mma_figure():
         assert owners(got, rows, cols) == owners(want, rows, cols), operand
         tables.append(owners(got, rows, cols))
     assert check_figure("TF32F32.svg", [transpose(tables[1]), tables[0], tables[2]]) == 32
+
+
+# ---- the tables themselves: get_layoutX_MK/NK/MN + print_typst's cell rule, as text from the host library ----
+
+def parse_tables(text):
+    """{title: [[(thr, val), ...] per row]} from the text the host library prints."""
+    import re
+    tables, cur = {}, None
+    for line in text.splitlines():
+        cells = re.findall(r"T(\d+)V(\d+)", line)
+        if cells:
+            cur.append([(int(t), int(v)) for t, v in cells])
+        elif line and not line.startswith(" "):
+            cur = tables.setdefault(line.strip(), [])
+    return tables
+
+
+def thread_part(table):
+    return [[t for t, _ in row] for row in table]
+
+
+def check_cells_invert(table, layout_tv, rows):
+    """Every cell (m, n) names a (thread, value) that the TV layout sends back to that cell."""
+    for m, row in enumerate(table):
+        for n, (t, v) in enumerate(row):
+            assert int(layout_tv((t, v))) - 1 == m + rows * n, (m, n, t, v)
+
+
+def test_printed_mma_tables_match_the_figure_and_the_oracle():
+    import moye_hip as mh
+    mma = _tf32_mma()
+    host = mh.TiledMMAOp("MMAOP_16x8x8_F32TF32TF32F32_TN")
+    tabs = parse_tables(host.print_tv(file=False))
+    assert list(tabs) == ["B (K, N)", "A (M, K)", "C (M, N)"]
+    want = {"A (M, K)": to.tv_table(*mma.get_layoutA_MK()), "C (M, N)": to.tv_table(*mma.get_layoutC_MN()),
+            "B (K, N)": transpose(to.tv_table(*mma.get_layoutB_NK()))}
+    for k in want:
+        assert tabs[k] == [list(r) for r in want[k]], k
+    # the figure of the manual draws exactly these threads (tensor_core.md:15-19)
+    assert check_figure("TF32F32.svg", [thread_part(tabs["B (K, N)"]), thread_part(tabs["A (M, K)"]), thread_part(tabs["C (M, N)"])]) == 32
+    check_cells_invert(tabs["A (M, K)"], mma.get_layoutA_TV(), 16)
+    check_cells_invert(transpose(tabs["B (K, N)"]), mma.get_layoutB_TV(), 8)
+    check_cells_invert(tabs["C (M, N)"], mma.get_layoutC_TV(), 16)
+
+
+def test_printed_copy_tables_match_the_figures():
+    import moye_hip as mh
+    from moye_hip import layout as ml
+    tc = mh.make_tiled_copy(mh.CopyAtom(64, 64), ml.Layout("(_2,_3):(_3,_1)"), ml.Layout("(_2,_3):(_1,_2)"))
+    tabs = parse_tables(tc.print_tv(file=False))
+    s, d = tabs["S (_4, _9)"], tabs["D (_4, _9)"]
+    assert check_figure("tiled_copy.svg", [thread_part(s), thread_part(d)]) == 6
+    otc = to.make_tiled_copy(to.CopyAtom(to.UniversalCopy(64), 64), SL((2, 3), (3, 1)), SL((2, 3), (1, 2)))
+    assert s == [list(r) for r in to.tv_table(*otc.get_layoutS_MN())] and d == [list(r) for r in to.tv_table(*otc.get_layoutD_MN())]
+    check_cells_invert(s, otc.get_layoutS_TV(), 4)
+    # tiled_matmul.md:9-14 prints the thread table of this copy
+    assert thread_part(s) == [[1, 1, 1, 2, 2, 2, 3, 3, 3], [1, 1, 1, 2, 2, 2, 3, 3, 3], [4, 4, 4, 5, 5, 5, 6, 6, 6], [4, 4, 4, 5, 5, 5, 6, 6, 6]]
+    # make_tiled_copy_A over the TF32 mma: the destination table is the mma's A table (tensor_core.md:132)
+    mma = mh.TiledMMAOp("MMAOP_16x8x8_F32TF32TF32F32_TN")
+    ca = mh.make_tiled_copy_A(mh.CopyAtom(32, 32), mma)
+    tabs = parse_tables(ca.print_tv(file=False))
+    a_tab = parse_tables(mma.print_tv(file=False))["A (M, K)"]
+    assert thread_part(tabs["D (_16, _8)"]) == thread_part(a_tab)
+
+
+@pytest.mark.parametrize("atom,atom_layout,perm", [
+    ("MFMA_F32_16x16x32_F16", (2, 2, 1), None), ("MFMA_F32_16x16x32_BF16", (2, 4, 1), None),
+    ("MFMA_F32_32x32x16_F16", (2, 2, 1), None), ("MFMA_F32_16x16x4_F32", (1, 2, 1), None),
+    ("MFMA_F32_16x16x32_F16", (2, 2, 1), (64, 64, 32)), ("MMAOP_16x8x8_F32TF32TF32F32_TN", (2, 2, 1), (32, 32, 8))])
+def test_layouts_mn_of_tiled_mfma_agree_with_the_oracle(atom, atom_layout, perm):
+    """get_layoutA_MK / B_NK / C_MN (src/atom/mma.jl:235-262) of tiled gfx950 atoms: host library against the oracle,
+    and each cell's (thread, value) inverts through get_layoutX_TV."""
+    import moye_hip as mh
+    from moye_hip import layout as ml
+    op = to.MFMA_OPS.get(atom) or to.REFERENCE_MMA_OPS[atom]
+    operm = None if perm is None else tuple(S(v) for v in perm)
+    omma = to.make_tiled_mma(op, SL(atom_layout), operm)
+    host = mh.TiledMMAOp(atom, ml.static_layout(atom_layout), None if perm is None else tuple(ml.StaticInt(v) for v in perm))
+    tabs = parse_tables(host.print_tv(file=False))
+    for operand, key, fn, tv in (("A", "A (M, K)", omma.get_layoutA_MK, omma.get_layoutA_TV()),
+                                 ("B", "B (K, N)", omma.get_layoutB_NK, omma.get_layoutB_TV()),
+                                 ("C", "C (M, N)", omma.get_layoutC_MN, omma.get_layoutC_TV())):
+        want_l, want_t = fn()
+        got_l, got_t = host.layout_mn(operand)
+        assert lo.parse_layout(got_l.text) == want_l and lo.parse_layout(got_t.text) == want_t, operand
+        want = to.tv_table(want_l, want_t)
+        got = transpose(tabs[key]) if operand == "B" else tabs[key]
+        assert [list(r) for r in got] == [list(r) for r in want], operand
+        check_cells_invert(got, tv, len(got))
+        # every (thread, value) pair appears exactly once
+        flat = [c for row in got for c in row]
+        assert len(set(flat)) == len(flat)

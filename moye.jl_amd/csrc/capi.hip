@@ -146,9 +146,8 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
         return fail(MOYE_ERR_UNSUPPORTED, "gemm!: atom takes %s operands, got A %s and B %s", dtype_name(in_dt),
                     dtype_name(A.dtype), dtype_name(B.dtype));
     if (tC && C.dtype != D.dtype) return fail(MOYE_ERR_UNSUPPORTED, "gemm!: C and D must have the same element type");
-    if (mma->atom == MOYE_MFMA_F32_32x32x2_F32 || mma->atom == MOYE_MFMA_F32_32x32x16_F16 ||
-        mma->atom == MOYE_MFMA_F32_32x32x16_BF16 || mma->atom == MOYE_MFMA_F32_32x32x16_FP8)
-        return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the 32x32 MFMA atoms are described (layouts, partitions) but the kernels issue the 16x16 forms");
+    const bool atom32 = mma->atom == MOYE_MFMA_F32_32x32x2_F32 || mma->atom == MOYE_MFMA_F32_32x32x16_F16 ||
+                        mma->atom == MOYE_MFMA_F32_32x32x16_BF16 || mma->atom == MOYE_MFMA_F32_32x32x16_FP8;
     if (K == 0) return fail(MOYE_ERR_SHAPE, "gemm!: K == 0");
     // NN / NT / TT (the naming of src/arch/mma/make_mma_ops.jl:253-265): operands whose unit stride is not
     // along K are brought to the K-major form the kernels read (one tiled transpose each)
@@ -172,7 +171,7 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
     const int waves = mma->atom_layout_mnk[0] * mma->atom_layout_mnk[1];
     g.alpha = alpha;
     g.K = K;
-    g.xcd_swizzle = !(mma->flags & MOYE_GEMM_NO_XCD_SWIZZLE) | (mma->flags & 0xff00);
+    g.xcd_swizzle = !(mma->flags & MOYE_GEMM_NO_XCD_SWIZZLE) | (mma->flags & 0xff00) | (atom32 ? kGemmAtom32 : 0);
     if (D.cs == 1) {  // row-major D
         g.A = A.ptr; g.B = B.ptr; g.M = M; g.N = N; g.lda = A.rs; g.ldb = B.rs; g.ldd = D.rs;
         g.C = tC ? C.ptr : nullptr; g.ldc_m = C.rs; g.ldc_n = C.cs; g.D = D.ptr;

@@ -24,15 +24,23 @@ namespace moye {
 // bytes): rows beyond M / N and k beyond K are read as zeros (the predication the reference's
 // copyto_if! is meant for, src/algorithm/copy.jl:4-16) and the epilogue stores element by element
 // inside the bounds.
-template <typename In, typename Out, int BM, int BN, int BKB /* bytes of K per tile row */, bool kEdge = false>
+//
+// AT = 16 issues the 16x16 MFMA forms, AT = 32 the 32x32 ones (v_mfma_f32_32x32x16_{f16,bf16,fp8_fp8},
+// v_mfma_f32_32x32x2_f32).  A 32x32 MFMA reads 32 rows of each operand and half the K extent of the
+// 16x16 form: lane l holds row l % 32 and the 16-byte chunk l / 32 of a 32-byte piece of that row, and its 16
+// accumulators are four groups of four consecutive n (n = 8 g + 4 (l / 32) + 0..3) of row m = l % 32.
+template <typename In, typename Out, int BM, int BN, int BKB /* bytes of K per tile row */, bool kEdge = false, int AT = 16>
 __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
     constexpr int CPR = BKB / 16;                 // 16-byte chunks per tile row
-    constexpr int KSTEPS = CPR / 4;               // one step = 4 chunks = one (fp8: two) MFMA k-slice
+    constexpr int CS = 64 / AT;                   // chunks of a row that the lanes of one MFMA step cover
+    constexpr int KSTEPS = CPR / CS;              // one step = one (fp8: two, fp32: four) MFMA k-slice
     constexpr int A_CH = BM * CPR, B_CH = BN * CPR;
     constexpr int A_LD = A_CH / 256, B_LD = B_CH / 256;
-    constexpr int WM = BM / 2, WN = BN / 2, MI = WM / 16, NI = WN / 16;
-    static_assert(A_CH % 256 == 0 && B_CH % 256 == 0 && CPR % 4 == 0, "tile shape");
+    constexpr int WM = BM / 2, WN = BN / 2, MI = WM / AT, NI = WN / AT;
+    constexpr int G = AT * AT / 256;              // groups of four accumulators per lane and MFMA tile
+    static_assert(A_CH % 256 == 0 && B_CH % 256 == 0 && CPR % 4 == 0 && (AT == 16 || AT == 32), "tile shape");
     typedef typename Out::type OutT;
+    typedef float accv __attribute__((ext_vector_type(4 * G)));
 
     extern __shared__ u32x4 smem[];
     u32x4* const sA0 = smem;
@@ -43,7 +51,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
     tile_of_block(p, &tm, &tn);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
-    const int r16 = lane & 15, kq = lane >> 4;
+    const int r16 = lane % AT, kq = lane / AT;   // row inside an MFMA tile, chunk inside a step
 
     const int64_t kbytes_a = (int64_t)p.lda * In::kBytes, kbytes_b = (int64_t)p.ldb * In::kBytes;
     const char* gA = static_cast<const char*>(p.A) + (int64_t)tm * BM * kbytes_a;
@@ -79,11 +87,13 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
         return *reinterpret_cast<const u32x4*>(b_src[i] + koff);
     };
 
-    f32x4 acc[MI][NI];
+    accv acc[MI][NI];
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
-        for (int j = 0; j < NI; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < NI; ++j)
+#pragma unroll
+            for (int e = 0; e < 4 * G; ++e) acc[i][j][e] = 0.f;
 
     const int ktiles = (int)((kbytes + BKB - 1) / BKB);
     u32x4 ra[A_LD], rb[B_LD];
@@ -113,21 +123,24 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) {
             u32x4 fa[MI], fb[NI];
-            const int ch = ks * 4 + kq;
+            const int ch = ks * CS + kq;
 #pragma unroll
             for (int i = 0; i < MI; ++i) {
-                const int row = wm0 + 16 * i + r16;
+                const int row = wm0 + AT * i + r16;
                 fa[i] = sA[row * CPR + (ch ^ swz<CPR>(row))];
             }
 #pragma unroll
             for (int j = 0; j < NI; ++j) {
-                const int row = wn0 + 16 * j + r16;
+                const int row = wn0 + AT * j + r16;
                 fb[j] = sB[row * CPR + (ch ^ swz<CPR>(row))];
             }
 #pragma unroll
             for (int i = 0; i < MI; ++i)
 #pragma unroll
-                for (int j = 0; j < NI; ++j) In::mma(fb[j], fa[i], acc[i][j]);
+                for (int j = 0; j < NI; ++j) {
+                    if constexpr (AT == 16) In::mma(fb[j], fa[i], acc[i][j]);
+                    else In::mma32(fb[j], fa[i], acc[i][j]);
+                }
         }
         if (more) {  // registers -> the other LDS stage
             u32x4* dA = sA0 + ((kt + 1) & 1) * STAGE;
@@ -141,22 +154,25 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
     }
 
     // ---- epilogue: alpha*acc + C -> OutT -> this wave's LDS patch -> 128-bit row stores ----
-    // lane holds C[m = 16 i + r16][n = 16 j + 4 kq + e], e = 0..3
+    // lane holds C[m = AT i + r16][n = AT j + 8 g + 4 kq + e], e = 0..3 (g = 0 only for the 16x16 forms)
     const int64_t m_base = (int64_t)tm * BM + wm0, n_base = (int64_t)tn * BN + wn0;
     if constexpr (kEdge) {
 #pragma unroll
         for (int i = 0; i < MI; ++i) {
-            const int64_t m = m_base + 16 * i + r16;
+            const int64_t m = m_base + AT * i + r16;
             if (m >= p.M) continue;
 #pragma unroll
             for (int j = 0; j < NI; ++j) {
-                const int64_t n = n_base + 16 * j + 4 * kq;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    if (n + e >= p.N) continue;
-                    float x = acc[i][j][e] * p.alpha;
-                    if (p.C) x += Out::load(p.C, m * p.ldc_m + (n + e) * p.ldc_n);
-                    static_cast<OutT*>(p.D)[m * p.ldd + n + e] = Out::cvt(x);
+                for (int g = 0; g < G; ++g) {
+                    const int64_t n = n_base + AT * j + 8 * g + 4 * kq;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if (n + e >= p.N) continue;
+                        float x = acc[i][j][4 * g + e] * p.alpha;
+                        if (p.C) x += Out::load(p.C, m * p.ldc_m + (n + e) * p.ldc_n);
+                        static_cast<OutT*>(p.D)[m * p.ldd + n + e] = Out::cvt(x);
+                    }
                 }
             }
         }
@@ -165,7 +181,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
     constexpr int EPC = 16 / (int)sizeof(OutT);          // elements per 16-byte chunk
     constexpr int CR = WN / EPC;                         // chunks per patch row
     constexpr int PASS_MI = (sizeof(OutT) == 4 && MI > 1) ? MI / 2 : MI;  // keep the patch <= 8 KiB
-    constexpr int PASS_ROWS = PASS_MI * 16;
+    constexpr int PASS_ROWS = PASS_MI * AT;
     OutT* patch = reinterpret_cast<OutT*>(smem) + wave * (PASS_ROWS * WN);
     u32x4* patch16 = reinterpret_cast<u32x4*>(patch);
 
@@ -176,18 +192,22 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
             const int i = i0 + ii;
 #pragma unroll
             for (int j = 0; j < NI; ++j) {
-                float v[4] = {acc[i][j].x * p.alpha, acc[i][j].y * p.alpha, acc[i][j].z * p.alpha,
-                              acc[i][j].w * p.alpha};
-                if (p.C) {
-                    const int64_t m = m_base + 16 * i + r16, n = n_base + 16 * j + 4 * kq;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) v[e] += Out::load(p.C, m * p.ldc_m + (n + e) * p.ldc_n);
+                for (int g = 0; g < G; ++g) {
+                    float v[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * g + e] * p.alpha;
+                    if (p.C) {
+                        const int64_t m = m_base + AT * i + r16, n = n_base + AT * j + 8 * g + 4 * kq;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] += Out::load(p.C, m * p.ldc_m + (n + e) * p.ldc_n);
+                    }
+                    const int row = AT * ii + r16, col = AT * j + 8 * g + 4 * kq;
+                    const int chunk = col / EPC, within = col % EPC;
+                    OutT* dst = patch + (row * CR + (chunk ^ (row & (CR - 1)))) * EPC + within;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) dst[e] = Out::cvt(v[e]);
                 }
-                const int row = 16 * ii + r16, col = 16 * j + 4 * kq;
-                const int chunk = col / EPC, within = col % EPC;
-                OutT* dst = patch + (row * CR + (chunk ^ (row & (CR - 1)))) * EPC + within;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) dst[e] = Out::cvt(v[e]);
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -198,7 +218,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
             const int c = lane + 64 * t, row = c / CR, ch = c % CR;
             const u32x4 w = patch16[row * CR + (ch ^ (row & (CR - 1)))];
             char* d = static_cast<char*>(p.D) +
-                      ((m_base + 16 * i0 + row) * p.ldd + n_base) * (int64_t)sizeof(OutT) + ch * 16;
+                      ((m_base + AT * i0 + row) * p.ldd + n_base) * (int64_t)sizeof(OutT) + ch * 16;
             *reinterpret_cast<u32x4*>(d) = w;
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -207,13 +227,13 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
     }
 }
 
-template <typename In, typename Out, int BM, int BN, int BKB, bool kEdge = false>
+template <typename In, typename Out, int BM, int BN, int BKB, bool kEdge = false, int AT = 16>
 static int32_t launch(const GemmArgs& a, hipStream_t st) {
     typedef typename Out::type OutT;
     constexpr int kMain = 2 * (BM + BN) * BKB;
     constexpr int kEpi = (sizeof(OutT) == 4 && BM / 32 > 1 ? BM / 2 : BM) * BN * (int)sizeof(OutT);
     constexpr int kLds = kMain > kEpi ? kMain : kEpi;
-    auto kern = gemm_mfma_tn<In, Out, BM, BN, BKB, kEdge>;
+    auto kern = gemm_mfma_tn<In, Out, BM, BN, BKB, kEdge, AT>;
     if (kLds > 64 * 1024) {
         static bool once = false;  // raising the dynamic LDS cap is per function, idempotent
         if (!once) {
@@ -227,20 +247,57 @@ static int32_t launch(const GemmArgs& a, hipStream_t st) {
     return MOYE_OK;
 }
 
-template <typename In, int BM, int BN, int BKB, bool kEdge = false>
+template <typename In, int BM, int BN, int BKB, bool kEdge = false, int AT = 16>
 static int32_t launch_out(int32_t out_dt, const GemmArgs& a, hipStream_t st) {
     switch (out_dt) {
-        case MOYE_F32: return launch<In, OutF32, BM, BN, BKB, kEdge>(a, st);
-        case MOYE_F16: return launch<In, OutF16, BM, BN, BKB, kEdge>(a, st);
-        case MOYE_BF16: return launch<In, OutBF16, BM, BN, BKB, kEdge>(a, st);
+        case MOYE_F32: return launch<In, OutF32, BM, BN, BKB, kEdge, AT>(a, st);
+        case MOYE_F16: return launch<In, OutF16, BM, BN, BKB, kEdge, AT>(a, st);
+        case MOYE_BF16: return launch<In, OutBF16, BM, BN, BKB, kEdge, AT>(a, st);
         default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: MFMA kernels write f32, f16 or bf16, not %s", dtype_name(out_dt));
     }
+}
+
+template <bool kEdge>
+static int32_t launch_atom32(int32_t in_dt, int32_t out_dt, const GemmArgs& a, hipStream_t st) {
+    switch (in_dt) {
+        case MOYE_F16: return launch_out<InF16, 128, 128, 64, kEdge, 32>(out_dt, a, st);
+        case MOYE_BF16: return launch_out<InBF16, 128, 128, 64, kEdge, 32>(out_dt, a, st);
+        case MOYE_F8E4M3: return launch_out<InFP8, 128, 128, 64, kEdge, 32>(out_dt, a, st);
+        case MOYE_F32: return launch_out<InF32, 128, 128, 64, kEdge, 32>(out_dt, a, st);
+        default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: no MFMA atom for %s inputs", dtype_name(in_dt));
+    }
+}
+
+// The 32x32 atoms: CTA tile 128x128 with 64 bytes of K per row, four waves of 2 x 2 MFMA tiles each; residue
+// tiles under the same rule as for the 16x16 atoms.
+static int32_t dispatch_atom32(int32_t in_dt, int32_t out_dt, int bm, int bn, int bk_elems, GemmArgs a, hipStream_t st) {
+    const int eb = dtype_bytes(in_dt), ob = dtype_bytes(out_dt);
+    const bool chosen_here = bm == 0 && bn == 0;
+    if ((bm && bm != 128) || (bn && bn != 128) || (bk_elems && bk_elems * eb != 64))
+        return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the 32x32 MFMA atoms run with CTA tile 128x128x%d only, not %dx%dx%d", 64 / eb, bm, bn,
+                    bk_elems);
+    if ((a.lda * eb) % 16 || (a.ldb * eb) % 16 || (reinterpret_cast<uintptr_t>(a.A) | reinterpret_cast<uintptr_t>(a.B)) % 16)
+        return fail(MOYE_ERR_ALIGN, "gemm!: operands of the MFMA kernels need 16-byte aligned pointers and row pitches");
+    a.tiles_m = (a.M + 127) / 128;
+    a.tiles_n = (a.N + 127) / 128;
+    if (a.M % 128 || a.N % 128 || a.K % (64 / eb)) {
+        if (!chosen_here && !(a.xcd_swizzle & MOYE_GEMM_PREDICATE))
+            return fail(MOYE_ERR_SHAPE, "gemm!: CTA tile 128x128x%d does not divide the problem %dx%dx%d", 64 / eb, a.M, a.N, a.K);
+        if (((int64_t)a.K * eb) % 16)
+            return fail(MOYE_ERR_SHAPE, "gemm!: the predicated MFMA kernel needs K to be a multiple of %d elements (16 bytes), got %d",
+                        16 / eb, a.K);
+        return launch_atom32<true>(in_dt, out_dt, a, st);
+    }
+    if ((a.ldd * ob) % 16 || reinterpret_cast<uintptr_t>(a.D) % 16)
+        return fail(MOYE_ERR_ALIGN, "gemm!: operands of the MFMA kernels need 16-byte aligned pointers and row pitches");
+    return launch_atom32<false>(in_dt, out_dt, a, st);
 }
 
 // K-major A and B, N-contiguous D.  bk_elems = 0 picks the default K extent per tile.
 int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int bk_elems, int waves, int stages,
                               GemmArgs a, hipStream_t st) {
     const int eb = dtype_bytes(in_dt);
+    if (a.xcd_swizzle & kGemmAtom32) return dispatch_atom32(in_dt, out_dt, bm, bn, bk_elems, a, st);
     // a short A (at most 64 rows) is a bandwidth problem: stream B once, no CTA tiling
     if ((bm == 0 && bn == 0 && a.M <= 64 && a.M % 16 == 0 && a.N % 16 == 0 && ((int64_t)a.K * eb) % 64 == 0) ||
         (bm == a.M && bm <= 64 && bn == 16))

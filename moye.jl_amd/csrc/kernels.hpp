@@ -15,8 +15,9 @@ struct GemmArgs {
     int64_t lda, ldb, ldc_m, ldc_n, ldd;
     float alpha;
     int tiles_m, tiles_n;
-    int xcd_swizzle;
+    int xcd_swizzle;  // bit 0: XCD-aware tile order; bits 8-15: MOYE_GEMM_* schedule flags; kGemmAtom32
 };
+constexpr int kGemmAtom32 = 0x10000;  // in GemmArgs::xcd_swizzle: issue the 32x32 MFMA forms
 
 // UniversalFMA GEMM, any strides (gemm_universal.hip)
 struct UArgs {

@@ -8,6 +8,7 @@ namespace moye {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
@@ -17,6 +18,10 @@ struct InF16 {
     static constexpr int kBytes = 2;
     static __device__ __forceinline__ void mma(const u32x4& a, const u32x4& b, f32x4& c) {
         c = __builtin_amdgcn_mfma_f32_16x16x32_f16((f16x8)a, (f16x8)b, c, 0, 0, 0);
+    }
+    // the 32x32x16 form: 32 rows per operand, a lane's chunk is half of a 32-byte piece of its row
+    static __device__ __forceinline__ void mma32(const u32x4& a, const u32x4& b, f32x16& c) {
+        c = __builtin_amdgcn_mfma_f32_32x32x16_f16((f16x8)a, (f16x8)b, c, 0, 0, 0);
     }
     // accumulator pinned in the AccVGPR file: its reads and write-backs then stay off the
     // ArchVGPR ports that the LDS fragment loads are writing through
@@ -28,6 +33,9 @@ struct InBF16 {
     static constexpr int kBytes = 2;
     static __device__ __forceinline__ void mma(const u32x4& a, const u32x4& b, f32x4& c) {
         c = __builtin_amdgcn_mfma_f32_16x16x32_bf16((bf16x8)a, (bf16x8)b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ void mma32(const u32x4& a, const u32x4& b, f32x16& c) {
+        c = __builtin_amdgcn_mfma_f32_32x32x16_bf16((bf16x8)a, (bf16x8)b, c, 0, 0, 0);
     }
     static __device__ __forceinline__ void mma_acc(const u32x4& a, const u32x4& b, f32x4& c) {
         asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
@@ -42,6 +50,12 @@ struct InFP8 {
         const long b0 = (long)(((uint64_t)b.y << 32) | b.x), b1 = (long)(((uint64_t)b.w << 32) | b.z);
         c = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a0, b0, c, 0, 0, 0);
         c = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a1, b1, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ void mma32(const u32x4& a, const u32x4& b, f32x16& c) {
+        const long a0 = (long)(((uint64_t)a.y << 32) | a.x), a1 = (long)(((uint64_t)a.w << 32) | a.z);
+        const long b0 = (long)(((uint64_t)b.y << 32) | b.x), b1 = (long)(((uint64_t)b.w << 32) | b.z);
+        c = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(a0, b0, c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(a1, b1, c, 0, 0, 0);
     }
     static __device__ __forceinline__ void mma_acc(const u32x4& a, const u32x4& b, f32x4& c) {
         const u32x2 a0 = {a.x, a.y}, a1 = {a.z, a.w}, b0 = {b.x, b.y}, b1 = {b.z, b.w};
@@ -59,6 +73,11 @@ struct InF32 {
 #pragma unroll
         for (int j = 0; j < 4; ++j)
             c = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(a[j]), __uint_as_float(b[j]), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ void mma32(const u32x4& a, const u32x4& b, f32x16& c) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[j]), __uint_as_float(b[j]), c, 0, 0, 0);
     }
     static __device__ __forceinline__ void mma_acc(const u32x4& a, const u32x4& b, f32x4& c) { mma(a, b, c); }
 };

@@ -596,11 +596,82 @@ def test_f32_mfma_short_m(mh):
     assert torch.equal(d.cpu().double(), A.double() @ B.double().t())
 
 
-def test_32x32_atoms_have_no_kernel(mh):
+def _atoms32(mh):
+    out = [(mh.MFMA_F32_32x32x16_F16, mh.MFMA_F32_16x16x32_F16, torch.float16, 4, TOL16),
+           (mh.MFMA_F32_32x32x16_BF16, mh.MFMA_F32_16x16x32_BF16, torch.bfloat16, 4, TOL16),
+           (mh.MFMA_F32_32x32x2_F32, mh.MFMA_F32_16x16x4_F32, torch.float32, 50, TOL32)]
+    if hasattr(torch, "float8_e4m3fn"):
+        out.append((mh.MFMA_F32_32x32x16_FP8, mh.MFMA_F32_16x16x32_FP8, torch.float8_e4m3fn, 4, TOL16))
+    return out
+
+
+def test_32x32_atoms_exact_on_integers(mh):
+    """The 32x32 MFMA forms in the 128x128 kernel: small-integer inputs make every partial sum exact, so a wrong
+    k pairing between the two operands or a misplaced accumulator group is a hard mismatch.  Row-major and
+    column-major D, C accumulated with alpha, every output type."""
+    g = torch.Generator().manual_seed(32)
+    for atom, _, tdt, hi, _ in _atoms32(mh):
+        for (M, N, K) in ((128, 128, 64), (256, 384, 448)):
+            A = torch.randint(-hi, hi + 1, (M, K), generator=g).float()
+            B = torch.randint(-hi, hi + 1, (N, K), generator=g).float()
+            C = torch.randint(-9, 10, (M, N), generator=g).float()
+            a, b = A.to(tdt).cuda(), B.to(tdt).cuda()
+            ref = A.double() @ B.double().t()
+            for out_dt in (torch.float32, torch.float16, torch.bfloat16):
+                if out_dt != torch.float32 and float(ref.abs().max()) * 2 + 9 > (2048 if out_dt == torch.float16 else 256):
+                    continue        # not every integer of that size is a float of that type
+                mma = mh.tiled_mma_desc(atom, atom_layout=(2, 2, 1), cta_tile=(128, 128, 0))
+                d = torch.zeros(M, N, dtype=out_dt, device="cuda")
+                mh.gemm_(mma, T(d), T(a), T(b))
+                torch.cuda.synchronize()
+                assert torch.equal(d.cpu().double(), ref), (atom, M, N, K, out_dt)
+                c = C.to(out_dt).cuda()
+                mh.gemm_(mma, T(d), T(a), T(b), T(c), 2.0)
+                torch.cuda.synchronize()
+                assert torch.equal(d.cpu().double(), 2 * ref + C.double()), (atom, M, N, K, out_dt, "C")
+                dt_ = torch.zeros(N, M, dtype=out_dt, device="cuda")          # column-major D
+                mh.gemm_(mma, T(dt_, (M, N), (1, M)), T(a), T(b))
+                torch.cuda.synchronize()
+                assert torch.equal(dt_.t().cpu().double(), ref), (atom, M, N, K, out_dt, "col-major")
+
+
+def test_32x32_atoms_random_and_residue_tiles(mh):
+    from moye_hip import _lib
+    g = torch.Generator().manual_seed(33)
+    for atom, atom16, tdt, hi, tol in _atoms32(mh):
+        M, N, K = 256, 256, 512
+        A = (torch.randn(M, K, generator=g) * K ** -0.5).to(tdt)
+        B = (torch.randn(N, K, generator=g) * K ** -0.5).to(tdt)
+        a, b = A.cuda(), B.cuda()
+        d, d16 = torch.zeros(M, N, device="cuda"), torch.zeros(M, N, device="cuda")
+        mh.gemm_(mh.tiled_mma_desc(atom, atom_layout=(2, 2, 1), cta_tile=(128, 128, 0)), T(d), T(a), T(b))
+        mh.gemm_(mh.tiled_mma_desc(atom16, atom_layout=(2, 2, 1), cta_tile=(128, 128, 0)), T(d16), T(a), T(b))
+        torch.cuda.synchronize()
+        c64 = A.double().cuda() @ B.double().cuda().t()
+        assert relerr(d, c64) <= tol, atom
+        assert relerr(d, d16) <= 1e-5, atom            # both forms accumulate in fp32; only the order differs
+        # residue tiles: the library's tile, and the explicit tile with the predicate flag
+        for (M, N, K) in ((100, 130, 48), (129, 127, 80), (1, 1, 16)):
+            A = torch.randint(-hi, hi + 1, (M, K), generator=g).float()
+            B = torch.randint(-hi, hi + 1, (N, K), generator=g).float()
+            a, b = A.to(tdt).cuda(), B.to(tdt).cuda()
+            ref = A.double() @ B.double().t()
+            for kw in (dict(cta_tile=(0, 0, 0)), dict(cta_tile=(128, 128, 0), flags=_lib.GEMM_PREDICATE)):
+                big = torch.full((M + 2, N + 3), 77.0, device="cuda")
+                d = big[1:M + 1, 2:N + 2]
+                mh.gemm_(mh.tiled_mma_desc(atom, **kw), T(d), T(a), T(b))
+                torch.cuda.synchronize()
+                assert torch.equal(d.cpu().double(), ref), (atom, M, N, K, kw)
+                frame = big.clone()
+                frame[1:M + 1, 2:N + 2] = 77.0
+                assert bool((frame == 77.0).all()), "stores outside D"
+
+
+def test_32x32_atoms_take_the_128_tile_only(mh):
     a = torch.zeros(256, 64, dtype=torch.float16, device="cuda")
     d = torch.zeros(256, 256, dtype=torch.float16, device="cuda")
     with pytest.raises(mh.MoyeError) as e:
-        mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_32x32x16_F16, cta_tile=(128, 128, 32)), T(d), T(a), T(a))
+        mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_32x32x16_F16, atom_layout=(2, 4, 1), cta_tile=(256, 256, 64)), T(d), T(a), T(a))
     assert "32x32" in str(e.value)
 
 

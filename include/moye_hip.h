@@ -84,7 +84,11 @@ typedef struct {
     int32_t tile_mnk[3];           /* tile_size(mma, 1..3) (atom/mma.jl:178-191)               */
     int32_t cta_tile_mnk[3];       /* bM, bN, bK; 0 = let the library choose                    */
     int32_t stages;                /* LDS pipeline depth, 0 = default                           */
-    int32_t split_k;               /* 0/1 = none; >1 = deterministic two-pass split-K           */
+    int32_t split_k;               /* 0/1 = none; >1 = K cut into that many equal ranges (each a
+                                      whole number of 16-byte pieces), all computed by one launch
+                                      into fp32 partial products in the library's workspace and
+                                      summed in ascending order by a second kernel (results do not
+                                      depend on timing); MFMA atoms only                         */
     int32_t flags;                 /* MOYE_GEMM_* bits                                          */
 } moye_tiled_mma;
 
@@ -164,7 +168,8 @@ int32_t moye_map(int32_t op, const moye_tensor* dst, const moye_tensor* a, const
                  void* stream);
 
 /* bytes of device workspace moye_gemm needs for this call: the K-major copies of MFMA operands whose
- * unit stride is not along K (NN / NT / TT problems); 0 for TN and for UniversalFMA.  The library
+ * unit stride is not along K (NN / NT / TT problems) and split_k * M * N fp32 partial products of a
+ * split-K call; 0 for plain TN and for UniversalFMA.  The library
  * allocates the workspace on first use (a synchronous hipMalloc inside that one moye_gemm call), grows
  * it when a larger call comes, and keeps it; calls that use it must not overlap on different streams. */
 int32_t moye_gemm_workspace_size(const moye_tiled_mma* mma, const moye_tensor* D,

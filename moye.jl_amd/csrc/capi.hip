@@ -92,11 +92,13 @@ static size_t kmajor_bytes(const Mat& m) {
     return (size_t)(m.rows * pitch + 255) / 256 * 256;
 }
 
+// K-major copies of A and B where needed, then the fp32 partial products of a split-K call
 static size_t gemm_workspace_bytes(const moye_tiled_mma* mma, const Mat& A, const Mat& B) {
     if (mma->atom == MOYE_MMA_UNIVERSAL_FMA) return 0;
     size_t n = 0;
     if (A.cs != 1 && A.cols > 1) n += kmajor_bytes(A);
     if (B.cs != 1 && B.cols > 1) n += kmajor_bytes(B);
+    if (mma->split_k > 1) n += (size_t)mma->split_k * (size_t)A.rows * (size_t)B.rows * sizeof(float);
     return n;
 }
 
@@ -136,6 +138,8 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
     const int bm = mma->cta_tile_mnk[0], bn = mma->cta_tile_mnk[1], bk = mma->cta_tile_mnk[2];
 
     if (mma->atom == MOYE_MMA_UNIVERSAL_FMA) {
+        if (mma->split_k > 1)
+            return fail(MOYE_ERR_UNSUPPORTED, "gemm!: UniversalFMA sums k in ascending order (src/algorithm/blas.jl:63-67); split_k would change that");
         UArgs u{A.ptr, B.ptr, tC ? C.ptr : nullptr, D.ptr, M, N, K, A.rs, A.cs, B.rs, B.cs,
                 C.rs, C.cs, D.rs, D.cs, alpha, A.dtype, B.dtype, tC ? C.dtype : D.dtype, D.dtype};
         return gemm_universal_dispatch(bm, bn, bk, u, st);
@@ -151,19 +155,22 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
     if (K == 0) return fail(MOYE_ERR_SHAPE, "gemm!: K == 0");
     // NN / NT / TT (the naming of src/arch/mma/make_mma_ops.jl:253-265): operands whose unit stride is not
     // along K are brought to the K-major form the kernels read (one tiled transpose each)
+    char* ws = nullptr;
     if (const size_t ws_bytes = gemm_workspace_bytes(mma, A, B)) {
         if (mma->flags & MOYE_GEMM_NO_WORKSPACE)
-            return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the MFMA kernels need K-major A and B (stride 1 along K, the 'TN' form) "
-                                              "and MOYE_GEMM_NO_WORKSPACE forbids the transposed copy");
+            return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the MFMA kernels need K-major A and B (stride 1 along K, the 'TN' form), split_k needs room "
+                                              "for its partial products, and MOYE_GEMM_NO_WORKSPACE forbids the library's workspace");
         if (int32_t e = ensure_workspace(ws_bytes)) return e;
-        char* ws = g_ws;
+        ws = g_ws;
         if (A.cs != 1 && A.cols > 1) {
             const size_t nb = kmajor_bytes(A);
             if (int32_t e = make_kmajor(&A, ws, st)) return e;
             ws += nb;
         }
         if (B.cs != 1 && B.cols > 1) {
+            const size_t nb = kmajor_bytes(B);
             if (int32_t e = make_kmajor(&B, ws, st)) return e;
+            ws += nb;
         }
     }
     GemmArgs g{};
@@ -172,6 +179,21 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
     g.alpha = alpha;
     g.K = K;
     g.xcd_swizzle = !(mma->flags & MOYE_GEMM_NO_XCD_SWIZZLE) | (mma->flags & 0xff00) | (atom32 ? kGemmAtom32 : 0);
+    if (mma->split_k > 1) {
+        // K is cut into split_k equal ranges, all in one launch (gridDim.y); each range writes its fp32 product, compact and
+        // row-major, into the workspace; a second pass sums the ranges in ascending order, applies alpha and C and converts
+        const int split = mma->split_k, eb = dtype_bytes(in_dt);
+        if (split > 65535) return fail(MOYE_ERR_ARG, "gemm!: split_k = %d is beyond the 65535 ranges one launch holds", split);
+        if (K % split || ((int64_t)(K / split) * eb) % 16)
+            return fail(MOYE_ERR_SHAPE, "gemm!: split_k = %d needs K = %d to split into equal ranges of whole 16-byte pieces", split, K);
+        const int Ks = K / split;
+        float* P = reinterpret_cast<float*>(ws);
+        g.alpha = 1.f; g.K = Ks; g.M = M; g.N = N; g.lda = A.rs; g.ldb = B.rs; g.ldd = N; g.C = nullptr;
+        g.A = A.ptr; g.B = B.ptr; g.D = P;
+        g.split = split; g.split_ab = (int64_t)Ks * eb; g.split_d = (int64_t)M * N * (int64_t)sizeof(float);
+        if (int32_t e = gemm_mfma_tn_dispatch(in_dt, MOYE_F32, bm, bn, bk, waves, mma->stages, g, st)) return e;
+        return splitk_reduce_dispatch(P, split, M, N, alpha, tC ? C.ptr : nullptr, C.rs, C.cs, D.ptr, D.rs, D.cs, D.dtype, st);
+    }
     if (D.cs == 1) {  // row-major D
         g.A = A.ptr; g.B = B.ptr; g.M = M; g.N = N; g.lda = A.rs; g.ldb = B.rs; g.ldd = D.rs;
         g.C = tC ? C.ptr : nullptr; g.ldc_m = C.rs; g.ldc_n = C.cs; g.D = D.ptr;

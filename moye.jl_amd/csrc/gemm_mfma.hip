@@ -48,6 +48,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
     constexpr int STAGE = A_CH + B_CH;
 
     int tm, tn;
+    split_of_block(p);
     tile_of_block(p, &tm, &tn);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
@@ -242,7 +243,7 @@ static int32_t launch(const GemmArgs& a, hipStream_t st) {
             once = true;
         }
     }
-    kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n)), dim3(256), kLds, st>>>(a);
+    kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1)), dim3(256), kLds, st>>>(a);
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;
 }

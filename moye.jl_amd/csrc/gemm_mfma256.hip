@@ -37,6 +37,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
     extern __shared__ u32x4 smem[];
 
     int tm, tn;
+    split_of_block(p);
     tile_of_block(p, &tm, &tn);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm0 = (wave / WGN) * WM, wn0 = (wave % WGN) * WN;
@@ -233,6 +234,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256_ring(GemmArgs
     extern __shared__ u32x4 smem[];
 
     int tm, tn;
+    split_of_block(p);
     tile_of_block(p, &tm, &tn);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm0 = (wave / WGN) * WM, wn0 = (wave % WGN) * WN;
@@ -375,7 +377,7 @@ static int32_t launch256_ring(const GemmArgs& a, hipStream_t st) {
                                            hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
         once = true;
     }
-    kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n)), dim3(512), kLds, st>>>(a);
+    kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1)), dim3(512), kLds, st>>>(a);
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;
 }
@@ -390,7 +392,7 @@ static int32_t launch256(const GemmArgs& a, hipStream_t st) {
                                            hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
         once = true;
     }
-    kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n)), dim3(64 * WGM * WGN), kLds, st>>>(a);
+    kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1)), dim3(64 * WGM * WGN), kLds, st>>>(a);
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;
 }

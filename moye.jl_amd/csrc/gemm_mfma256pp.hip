@@ -41,6 +41,7 @@ __global__ __launch_bounds__(512) void gemm_mfma_tn_256_pp(GemmArgs p) {
     extern __shared__ u32x4 smem[];
 
     int tm, tn;
+    split_of_block(p);
     tile_of_block(p, &tm, &tn);
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int group = wave >> 2;  // wave-uniform: the waits below are scalar instructions
@@ -161,7 +162,7 @@ static int32_t launch256_pp(const GemmArgs& a, hipStream_t st) {
                                            hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
         once = true;
     }
-    kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n)), dim3(512), kLds, st>>>(a);
+    kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1)), dim3(512), kLds, st>>>(a);
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;
 }

@@ -132,6 +132,7 @@ __global__ __launch_bounds__(128 * WGN) void gemm_mfma_tn_256_w4(GemmArgs p) {
     extern __shared__ u32x4 smem[];
 
     int tm, tn;
+    split_of_block(p);
     tile_of_block(p, &tm, &tn);
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm0 = (wave / WGN) * 128, wn0 = (wave % WGN) * WN;
@@ -317,7 +318,7 @@ static int32_t launch256_w4(const GemmArgs& a, hipStream_t st) {
                                            hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
         once = true;
     }
-    kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n)), dim3(128 * WGN), kLds, st>>>(a);
+    kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1)), dim3(128 * WGN), kLds, st>>>(a);
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;
 }

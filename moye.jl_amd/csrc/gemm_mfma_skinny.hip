@@ -17,6 +17,7 @@ namespace moye {
 template <typename In, typename Out, int MT, int NTW, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_skinny(GemmArgs p) {
     typedef typename Out::type OutT;
+    split_of_block(p);
     constexpr int U = 4;  // 64-byte k-steps in flight per wave and row
     __shared__ f32x4 part[WAVES][MT * NTW][64];
     const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, r16 = lane % 16, kq = lane / 16;
@@ -106,7 +107,7 @@ static int32_t launch_skinny(const GemmArgs& a, hipStream_t st) {
     constexpr int W = 8;
     const dim3 block(W * 64);
     if (a.N % 32 == 0 && a.N / 32 >= 256) {  // two B tiles per wave once that still fills the chip
-        const dim3 grid((unsigned)(a.N / 32));
+        const dim3 grid((unsigned)(a.N / 32), (unsigned)(a.split > 1 ? a.split : 1));
         switch (a.M / 16) {
             case 1: gemm_mfma_skinny<In, Out, 1, 2, W><<<grid, block, 0, st>>>(a); break;
             case 2: gemm_mfma_skinny<In, Out, 2, 2, W><<<grid, block, 0, st>>>(a); break;
@@ -114,7 +115,7 @@ static int32_t launch_skinny(const GemmArgs& a, hipStream_t st) {
             default: gemm_mfma_skinny<In, Out, 4, 2, W><<<grid, block, 0, st>>>(a); break;
         }
     } else {
-        const dim3 grid((unsigned)(a.N / 16));
+        const dim3 grid((unsigned)(a.N / 16), (unsigned)(a.split > 1 ? a.split : 1));
         switch (a.M / 16) {
             case 1: gemm_mfma_skinny<In, Out, 1, 1, W><<<grid, block, 0, st>>>(a); break;
             case 2: gemm_mfma_skinny<In, Out, 2, 1, W><<<grid, block, 0, st>>>(a); break;

@@ -15,6 +15,10 @@ struct GemmArgs {
     int64_t lda, ldb, ldc_m, ldc_n, ldd;
     float alpha;
     int tiles_m, tiles_n;
+    // split-K: gridDim.y ranges of K in one launch; range y reads A and B split_ab bytes further along their rows
+    // and writes its product split_d bytes further (compact fp32 partial products, one after the other)
+    int split;
+    int64_t split_ab, split_d;
     int xcd_swizzle;  // bit 0: XCD-aware tile order; bits 8-15: MOYE_GEMM_* schedule flags; kGemmAtom32
 };
 constexpr int kGemmAtom32 = 0x10000;  // in GemmArgs::xcd_swizzle: issue the 32x32 MFMA forms
@@ -38,6 +42,8 @@ int32_t gemm_mfma_skinny_dispatch(int32_t in_dt, int32_t out_dt, const GemmArgs&
 int32_t axpby_dispatch(double a, const moye_tensor* X, double b, const moye_tensor* Y, hipStream_t st);
 int32_t fill_dispatch(const moye_tensor* X, double value, hipStream_t st);
 int32_t map_dispatch(int32_t op, const moye_tensor* D, const moye_tensor* A, const moye_tensor* B, double scalar, hipStream_t st);
+int32_t splitk_reduce_dispatch(const float* P, int split, int64_t M, int64_t N, float alpha, const void* C, int64_t c_rs,
+                               int64_t c_cs, void* D, int64_t d_rs, int64_t d_cs, int32_t out_dt, hipStream_t st);
 int32_t mfma_ceiling(int32_t in_dt, int32_t random_operands, float seconds, float* tflops, float* clock_ghz, hipStream_t st);
 int32_t gemm_universal_dispatch(int bm, int bn, int bk, UArgs a, hipStream_t st);
 

@@ -117,6 +117,15 @@ __device__ __forceinline__ int swz(int row) {
     else return (row / (8 / CPR)) & (CPR - 1);
 }
 
+// blockIdx.y -> the K range of a split-K launch (one range and no offsets for an ordinary launch)
+__device__ __forceinline__ void split_of_block(GemmArgs& p) {
+    if (gridDim.y > 1) {
+        p.A = static_cast<const char*>(p.A) + (int64_t)blockIdx.y * p.split_ab;
+        p.B = static_cast<const char*>(p.B) + (int64_t)blockIdx.y * p.split_ab;
+        p.D = static_cast<char*>(p.D) + (int64_t)blockIdx.y * p.split_d;
+    }
+}
+
 // blockIdx -> (tile_m, tile_n).  Hardware deals consecutive workgroup ids round-robin to the 8
 // XCDs; remapping id -> (id % 8) * (n / 8) + id / 8 hands each XCD one contiguous run of tiles,
 // and inside a run tiles are walked in bands of 8 tile-rows so that the A and B panels an

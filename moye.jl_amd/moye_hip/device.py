@@ -56,6 +56,14 @@ def gemm_(mma, D, A, B, C_=None, alpha=1.0, stream=None):
     check(lib().moye_gemm(C.byref(mma), C.byref(D), C.byref(A), C.byref(B), _ref(C_), alpha, stream))
 
 
+def gemm_workspace_size(mma, D, A, B):
+    """Bytes of library-owned device workspace this gemm! call needs (K-major copies of operands that are not K-major,
+    partial products of a split-K call); 0 for a plain TN call."""
+    n = C.c_size_t()
+    check(lib().moye_gemm_workspace_size(C.byref(mma), C.byref(D), C.byref(A), C.byref(B), C.byref(n)))
+    return n.value
+
+
 def time_gemm(mma, D, A, B, C_=None, alpha=1.0, stream=None, warmup=2, iters=10):
     """Average milliseconds per launch (HIP events on `stream`)."""
     ms = C.c_float()

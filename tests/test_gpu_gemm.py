@@ -675,6 +675,87 @@ def test_32x32_atoms_take_the_128_tile_only(mh):
     assert "32x32" in str(e.value)
 
 
+@pytest.mark.parametrize("split", [2, 4, 8])
+def test_split_k_exact_on_integers(mh, split):
+    """split_k > 1: K cut into equal ranges, fp32 partial products summed in ascending order in a second pass.
+    Exact on integers whatever the tile, with C and alpha, with a column-major D, with an operand that is not K-major
+    (its K-major copy and the partials share the workspace) and for a short A."""
+    from moye_hip import _lib
+    g = torch.Generator().manual_seed(40 + split)
+    M, N, K = 256, 384, 2048
+    A = torch.randint(-4, 5, (M, K), generator=g).to(torch.float16)
+    B = torch.randint(-4, 5, (N, K), generator=g).to(torch.float16)
+    C = torch.randint(-9, 10, (M, N), generator=g).float()
+    a, b, c = A.cuda(), B.cuda(), C.cuda()
+    ref = A.double() @ B.double().t()
+    for cta, waves in (((128, 128, 32), (2, 2, 1)), ((0, 0, 0), (1, 1, 1)), ((128, 128, 64), (2, 2, 1))):
+        mma = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=waves, cta_tile=cta, split_k=split)
+        d = torch.zeros(M, N, device="cuda")
+        mh.gemm_(mma, T(d), T(a), T(b))
+        torch.cuda.synchronize()
+        assert torch.equal(d.cpu().double(), ref), (cta, "plain")
+        mh.gemm_(mma, T(d), T(a), T(b), T(c), 2.0)
+        torch.cuda.synchronize()
+        assert torch.equal(d.cpu().double(), 2 * ref + C.double()), (cta, "alpha, C")
+        dt_ = torch.zeros(N, M, device="cuda")
+        mh.gemm_(mma, T(dt_, (M, N), (1, M)), T(a), T(b))
+        torch.cuda.synchronize()
+        assert torch.equal(dt_.t().cpu().double(), ref), (cta, "column-major D")
+        at = A.t().contiguous().cuda()                      # A stored M-major: (M,K):(1,M)
+        d.zero_()
+        mh.gemm_(mma, T(d), T(at, (M, K), (1, M)), T(b))
+        torch.cuda.synchronize()
+        assert torch.equal(d.cpu().double(), ref), (cta, "M-major A")
+    # 256x256 tile
+    M2 = N2 = 512
+    A2 = torch.randint(-4, 5, (M2, K), generator=g).to(torch.bfloat16)
+    B2 = torch.randint(-4, 5, (N2, K), generator=g).to(torch.bfloat16)
+    d2 = torch.zeros(M2, N2, dtype=torch.bfloat16, device="cuda")
+    a2, b2 = A2.cuda(), B2.cuda()
+    mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_BF16, atom_layout=(2, 4, 1), cta_tile=(256, 256, 64), split_k=split),
+             T(d2), T(a2), T(b2), None, 0.125)
+    torch.cuda.synchronize()
+    assert torch.equal(d2.cpu().double(), (0.125 * (A2.double() @ B2.double().t())).to(torch.bfloat16).double())
+    # short A
+    d3 = torch.zeros(16, N, device="cuda")
+    a16 = a[:16].contiguous()
+    mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(0, 0, 0), split_k=split), T(d3), T(a16), T(b))
+    torch.cuda.synchronize()
+    assert torch.equal(d3.cpu().double(), ref[:16])
+    # workspace size is reported; a K that does not split is refused; UniversalFMA keeps its order
+    need = mh.gemm_workspace_size(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, split_k=split), T(d), T(a), T(b))
+    assert need == split * M * N * 4
+    ak, bk_ = a[:, :K - 8].contiguous(), b[:, :K - 8].contiguous()
+    with pytest.raises(mh.MoyeError) as e:
+        mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, split_k=split), T(d), T(ak), T(bk_))
+    assert e.value.status == _lib.ERR_SHAPE
+    af, bf = a.float(), b.float()
+    with pytest.raises(mh.MoyeError) as e:
+        mh.gemm_(mh.tiled_mma_desc(mh.MMA_UNIVERSAL_FMA, cta_tile=(32, 32, 8), split_k=split), T(d), T(af), T(bf))
+    assert e.value.status == _lib.ERR_UNSUPPORTED
+
+
+def test_split_k_long_k(mh):
+    """A small C with a long K leaves most of the chip idle without a split: 256 x 256 x 65536 fp16."""
+    g = torch.Generator().manual_seed(77)
+    M = N = 256
+    K = 65536
+    A = (torch.randn(M, K, generator=g) * K ** -0.5).half()
+    B = (torch.randn(N, K, generator=g) * K ** -0.5).half()
+    a, b = A.cuda(), B.cuda()
+    c64 = a.double() @ b.double().t()
+    times = {}
+    for split in (1, 16, 64):
+        d = torch.zeros(M, N, device="cuda")
+        mma = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 2, 1), cta_tile=(128, 128, 32), split_k=split)
+        mh.gemm_(mma, T(d), T(a), T(b))
+        torch.cuda.synchronize()
+        assert relerr(d, c64) <= TOL16
+        times[split] = mh.time_gemm(mma, T(d), T(a), T(b), None, 1.0, None, warmup=2, iters=10)
+    print("256x256x65536 f16: " + ", ".join("split_k=%d %.1f us" % (k, v * 1e3) for k, v in times.items()))
+    assert times[16] < times[1]
+
+
 def test_mfma_ceiling_probe(mh):
     """The MFMA-only yardstick: plausible numbers, and zeros never slower than dense random operands."""
     tf_r, ghz_r = mh.mfma_ceiling(mh.F16, True, 0.2)
@@ -765,7 +846,8 @@ def test_residue_tiles_predicated(mh, M, N, K):
         for out_dt in (torch.float32, torch.float16):
             big = torch.full((M + 2, N + 3), 77.0, dtype=out_dt, device="cuda")     # D is a window of a larger buffer
             d = big[1:M + 1, 2:N + 2]
-            mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, **kw), T(d), T(a), T(b), T(c.to(out_dt).contiguous()), 1.0)
+            c_out = c.to(out_dt).contiguous()
+            mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, **kw), T(d), T(a), T(b), T(c_out), 1.0)
             torch.cuda.synchronize()
             assert torch.equal(d.cpu().double(), (ref + C.double()).to(out_dt).double()), (M, N, K, kw, out_dt)
             frame = big.clone()

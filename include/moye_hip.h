@@ -93,7 +93,9 @@ typedef struct {
 } moye_tiled_mma;
 
 #define MOYE_GEMM_NO_XCD_SWIZZLE 1   /* keep blockIdx -> tile mapping linear (for A/B studies)  */
-#define MOYE_GEMM_NO_LDS_SWIZZLE 2   /* linear LDS tiles (bank-conflict study)                  */
+#define MOYE_GEMM_NO_LDS_SWIZZLE 2   /* in moye_tiled_copy.flags: the LDS-tiled 32-bit transpose keeps
+                                        its tile linear (bank-conflict study); the GEMM kernels
+                                        ignore it                                               */
 #define MOYE_GEMM_NO_WORKSPACE 4      /* fail instead of transposing a non-K-major operand into the workspace */
 #define MOYE_GEMM_PREDICATE 0x200     /* compute residue tiles (M, N, K not multiples of the 128x128 CTA tile)
                                         instead of failing as the reference's kernels assert; implied
@@ -119,7 +121,7 @@ typedef struct {
     int32_t thr_shape[2];          /* thr_layout of make_tiled_copy (atom/copy.jl:249-258)      */
     int32_t val_shape[2];          /* val_layout                                                */
     int32_t tiler_mn[2];           /* tiler_MN = LDS tile, e.g. 64x64                           */
-    int32_t flags;
+    int32_t flags;                 /* 0 or MOYE_GEMM_NO_LDS_SWIZZLE                              */
 } moye_tiled_copy;
 
 /* ---- device loops ------------------------------------------------------------------------ */

@@ -24,18 +24,18 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # (the summaries are committed under profiles/), each reading scaled by what the same counter shows for the
 # 1 GiB plain copy (fetch x2.0000, write x1.0000).  Only valid for the default tile/waves/flags.
 MEASURED_TRAFFIC = {
-    "gemm_f16_4096_tile256": {"read_bytes": 197437 * 1024, "write_bytes": 33280 * 1024},
-    "transpose_f32_16384": {"read_bytes": 1048622 * 1024, "write_bytes": 1049576 * 1024},
-    "gemm_bf16_8192_tile256": {"read_bytes": 1809307 * 1024, "write_bytes": 266240 * 1024},
-    "gemm_f32_8192_tile256": {"read_bytes": 3960678 * 1024, "write_bytes": 270336 * 1024},
-    "gemm_fp8_8192_tile256": {"read_bytes": 786981 * 1024, "write_bytes": 131072 * 1024},
-    "gemm_bf16_16x8192x8192": {"read_bytes": 159438 * 1024, "write_bytes": 512 * 1024},
+    "gemm_f16_4096_tile256": {"read_bytes": 197454 * 1024, "write_bytes": 33280 * 1024},
+    "transpose_f32_16384": {"read_bytes": 1048640 * 1024, "write_bytes": 1049572 * 1024},
+    "gemm_bf16_8192_tile256": {"read_bytes": 1620806 * 1024, "write_bytes": 266240 * 1024},
+    "gemm_f32_8192_tile256": {"read_bytes": 4908081 * 1024, "write_bytes": 270336 * 1024},
+    "gemm_fp8_8192_tile256": {"read_bytes": 787072 * 1024, "write_bytes": 131072 * 1024},
+    "gemm_bf16_16x8192x8192": {"read_bytes": 149534 * 1024, "write_bytes": 512 * 1024},
 }
 
 
 def cpu_baseline(cores):
     """The reference's CPU path, restated (oracle/gemm_oracle.c): UniversalFMA gemm! over host
-    arrays, fp16 operands, 32x32x8 tiles, on a bounded sub-problem (about 12 s) of the same workload."""
+    arrays, fp16 operands, 32x32x8 tiles, on a bounded sub-problem (10-20 s) of the same workload."""
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
     import numpy as np
     import c_oracle as co
@@ -47,13 +47,13 @@ def cpu_baseline(cores):
         b = (rng.standard_normal((n, n)) / np.sqrt(4096)).astype(np.float16).astype(np.float32)
         return a, b
 
-    A, B = operands(512)
+    A, B = operands(1024)
     co.gemm(A[:64, :64], B[:64, :64], None, "f16", (32, 32, 8), cores)  # load + warm
     t0 = time.perf_counter()
     co.gemm(A, B, None, "f16", (32, 32, 8), cores)
-    rate = 2.0 * 512 ** 3 / (time.perf_counter() - t0)      # flop/s on a probe
-    # bounded sample: about 12 s of CPU work, a multiple of 256, at most the full 4096^3 problem
-    n = int(min(4096, max(512, ((rate * 12.0 / 2.0) ** (1.0 / 3.0)) // 256 * 256)))
+    rate = 2.0 * 1024 ** 3 / (time.perf_counter() - t0)     # flop/s on a probe
+    # bounded sample: about 15 s of CPU work, a multiple of 256, at most the full 4096^3 problem
+    n = int(min(4096, max(512, ((rate * 15.0 / 2.0) ** (1.0 / 3.0)) // 256 * 256)))
     A, B = operands(n)
     t0 = time.perf_counter()
     co.gemm(A, B, None, "f16", (32, 32, 8), cores)

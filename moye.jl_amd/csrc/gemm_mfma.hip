@@ -135,10 +135,13 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
                 const int row = wn0 + AT * j + r16;
                 fb[j] = sB[row * CPR + (ch ^ swz<CPR>(row))];
             }
+            // rows walked back and forth: one operand register set changes between consecutive MFMAs, which
+            // costs less power than two (the part is power-limited with dense operands)
 #pragma unroll
             for (int i = 0; i < MI; ++i)
 #pragma unroll
-                for (int j = 0; j < NI; ++j) {
+                for (int jj = 0; jj < NI; ++jj) {
+                    const int j = (i & 1) ? NI - 1 - jj : jj;
                     if constexpr (AT == 16) In::mma(fb[j], fa[i], acc[i][j]);
                     else In::mma32(fb[j], fa[i], acc[i][j]);
                 }

@@ -94,9 +94,15 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
 #define MOYE_FRAGS(BASE, KS, BUF)                                                                     \
     _Pragma("unroll") for (int i = 0; i < MI; ++i) fa[BUF][i] = (BASE)[fa_slot[KS] + 16 * CPR * i];   \
     _Pragma("unroll") for (int j = 0; j < NI; ++j) fb[BUF][j] = (BASE)[fb_slot[KS] + 16 * CPR * j];
+// Rows of the wave tile are walked back and forth, so that exactly one operand register set changes between
+// consecutive MFMAs: with dense operands the part is power-limited, and an MFMA-only loop over an 8 x 4 register
+// tile sustains 1.5-2 % more in this order than row by row (1980 against 1947 TFLOP/s).
 #define MOYE_MMA(BUF, I0, I1)                                                                         \
     _Pragma("unroll") for (int i = I0; i < I1; ++i)                                                   \
-        _Pragma("unroll") for (int j = 0; j < NI; ++j) In::mma(fb[BUF][j], fa[BUF][i], acc[i][j]);
+        _Pragma("unroll") for (int jj = 0; jj < NI; ++jj) {                                           \
+            const int j = (i & 1) ? NI - 1 - jj : jj;                                                 \
+            In::mma(fb[BUF][j], fa[BUF][i], acc[i][j]);                                               \
+        }
 
     // Issue order inside a k-step: the two waves of a SIMD leave the barrier together, so if each one
     // issued all its fragment reads first the MFMA pipe would idle for both.  Spread them instead:
@@ -285,9 +291,12 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256_ring(GemmArgs
         _Pragma("unroll") for (int i = 0; i < MI; ++i) fa[BUF][i] = base_[fa_slot + 16 * CPR * i];     \
         _Pragma("unroll") for (int j = 0; j < NI; ++j) fb[BUF][j] = base_[fb_slot + 16 * CPR * j];     \
     }
-#define MOYE_MMA(BUF, I0, I1)                                                                          \
-    _Pragma("unroll") for (int i = I0; i < I1; ++i)                                                    \
-        _Pragma("unroll") for (int j = 0; j < NI; ++j) In::mma(fb[BUF][j], fa[BUF][i], acc[i][j]);
+#define MOYE_MMA(BUF, I0, I1)                                                                         \
+    _Pragma("unroll") for (int i = I0; i < I1; ++i)                                                   \
+        _Pragma("unroll") for (int jj = 0; jj < NI; ++jj) {                                           \
+            const int j = (i & 1) ? NI - 1 - jj : jj;                                                 \
+            In::mma(fb[BUF][j], fa[BUF][i], acc[i][j]);                                               \
+        }
     // one k-step; BUF is the fragment buffer that holds tile T
 #define MOYE_STEP(T, BUF)                                                                              \
     {                                                                                                  \

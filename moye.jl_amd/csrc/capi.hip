@@ -92,13 +92,27 @@ static size_t kmajor_bytes(const Mat& m) {
     return (size_t)(m.rows * pitch + 255) / 256 * 256;
 }
 
+// split_k of the descriptor -> number of K ranges.  Negative = the library chooses: no split when the 128 x 128 tiles
+// of the problem fill half the chip or more, else the largest count up to 256 / tiles (one workgroup per CU) that cuts K into equal
+// ranges of whole 128-byte pieces of at least 512 bytes (so every kernel's k-tile divides a range).
+static int split_count(const moye_tiled_mma* mma, int64_t M, int64_t N, int64_t K, int eb) {
+    if (mma->split_k >= 0) return mma->split_k > 1 ? mma->split_k : 1;
+    if (mma->flags & MOYE_GEMM_NO_WORKSPACE) return 1;  // nowhere to put the partial products
+    const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+    if (tiles <= 0 || tiles >= 128) return 1;
+    for (int64_t s = std::min<int64_t>(256 / tiles, K); s >= 2; --s)
+        if (K % s == 0 && ((K / s) * eb) % 128 == 0 && (K / s) * eb >= 512) return (int)s;
+    return 1;
+}
+
 // K-major copies of A and B where needed, then the fp32 partial products of a split-K call
 static size_t gemm_workspace_bytes(const moye_tiled_mma* mma, const Mat& A, const Mat& B) {
     if (mma->atom == MOYE_MMA_UNIVERSAL_FMA) return 0;
     size_t n = 0;
     if (A.cs != 1 && A.cols > 1) n += kmajor_bytes(A);
     if (B.cs != 1 && B.cols > 1) n += kmajor_bytes(B);
-    if (mma->split_k > 1) n += (size_t)mma->split_k * (size_t)A.rows * (size_t)B.rows * sizeof(float);
+    const int split = split_count(mma, A.rows, B.rows, A.cols, dtype_bytes(A.dtype));
+    if (split > 1) n += (size_t)split * (size_t)A.rows * (size_t)B.rows * sizeof(float);
     return n;
 }
 
@@ -179,10 +193,10 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
     g.alpha = alpha;
     g.K = K;
     g.xcd_swizzle = !(mma->flags & MOYE_GEMM_NO_XCD_SWIZZLE) | (mma->flags & 0xff00) | (atom32 ? kGemmAtom32 : 0);
-    if (mma->split_k > 1) {
-        // K is cut into split_k equal ranges, all in one launch (gridDim.y); each range writes its fp32 product, compact and
+    if (const int split = split_count(mma, M, N, K, dtype_bytes(in_dt)); split > 1) {
+        // K is cut into `split` equal ranges, all in one launch (gridDim.y); each range writes its fp32 product, compact and
         // row-major, into the workspace; a second pass sums the ranges in ascending order, applies alpha and C and converts
-        const int split = mma->split_k, eb = dtype_bytes(in_dt);
+        const int eb = dtype_bytes(in_dt);
         if (split > 65535) return fail(MOYE_ERR_ARG, "gemm!: split_k = %d is beyond the 65535 ranges one launch holds", split);
         if (K % split || ((int64_t)(K / split) * eb) % 16)
             return fail(MOYE_ERR_SHAPE, "gemm!: split_k = %d needs K = %d to split into equal ranges of whole 16-byte pieces", split, K);

@@ -745,7 +745,7 @@ def test_split_k_long_k(mh):
     a, b = A.cuda(), B.cuda()
     c64 = a.double() @ b.double().t()
     times = {}
-    for split in (1, 16, 64):
+    for split in (1, 16, 64, -1):
         d = torch.zeros(M, N, device="cuda")
         mma = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 2, 1), cta_tile=(128, 128, 32), split_k=split)
         mh.gemm_(mma, T(d), T(a), T(b))
@@ -753,7 +753,11 @@ def test_split_k_long_k(mh):
         assert relerr(d, c64) <= TOL16
         times[split] = mh.time_gemm(mma, T(d), T(a), T(b), None, 1.0, None, warmup=2, iters=10)
     print("256x256x65536 f16: " + ", ".join("split_k=%d %.1f us" % (k, v * 1e3) for k, v in times.items()))
-    assert times[16] < times[1]
+    assert times[16] < times[1] and times[-1] < times[1]        # -1: the library chooses
+    # the library's choice: tiles that fill the chip are not split (no workspace asked for)
+    big = torch.zeros(2048, 2048, dtype=torch.float16, device="cuda")
+    assert mh.gemm_workspace_size(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, split_k=-1), T(big), T(big), T(big)) == 0
+    assert mh.gemm_workspace_size(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, split_k=-1), T(d), T(a), T(b)) > 0
 
 
 def test_mfma_ceiling_probe(mh):

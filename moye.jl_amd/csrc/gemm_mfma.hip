@@ -303,8 +303,7 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
     const int eb = dtype_bytes(in_dt);
     if (a.xcd_swizzle & kGemmAtom32) return dispatch_atom32(in_dt, out_dt, bm, bn, bk_elems, a, st);
     // a short A (at most 64 rows) is a bandwidth problem: stream B once, no CTA tiling
-    if ((bm == 0 && bn == 0 && a.M <= 64 && a.M % 16 == 0 && a.N % 16 == 0 && ((int64_t)a.K * eb) % 64 == 0) ||
-        (bm == a.M && bm <= 64 && bn == 16))
+    if ((bm == 0 && bn == 0 && a.M <= 64 && ((int64_t)a.K * eb) % 64 == 0) || (bm == a.M && bm <= 64 && bn == 16))
         return gemm_mfma_skinny_dispatch(in_dt, out_dt, a, st);
     const bool chosen_here = bm == 0 && bn == 0;
     if (bm == 0 && bn == 0) {

@@ -1,4 +1,4 @@
-// MFMA GEMM for a short A: M = 16, 32, 48 or 64 rows against a long B (N x K), K-major operands.
+// MFMA GEMM for a short A: at most 64 rows against a long B (N x K), K-major operands.
 // The work is streaming B from HBM once, so the kernel is laid out for bandwidth, not for the
 // matrix pipe: one workgroup owns 16 or 32 rows of B (that many output columns) and all of A; its waves split
 // K into contiguous ranges, each lane streams 16-byte pieces of its B row straight into the MFMA
@@ -24,14 +24,16 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_skinny(GemmArgs p) {
     const int n0 = blockIdx.x * 16 * NTW;
     const int steps = (int)(((int64_t)p.K * In::kBytes) / 64);
     const int s0 = (int)((int64_t)steps * wave / WAVES), s1 = (int)((int64_t)steps * (wave + 1) / WAVES);
+    // M and N need not be multiples of 16: a lane whose row lies beyond the operand reads the last row instead, and
+    // what it computes is not stored
     const char* bp[NTW];
 #pragma unroll
     for (int t = 0; t < NTW; ++t)
-        bp[t] = static_cast<const char*>(p.B) + (int64_t)(n0 + 16 * t + r16) * p.ldb * In::kBytes + kq * 16;
+        bp[t] = static_cast<const char*>(p.B) + (int64_t)min(n0 + 16 * t + r16, p.N - 1) * p.ldb * In::kBytes + kq * 16;
     const char* ap[MT];
 #pragma unroll
     for (int i = 0; i < MT; ++i)
-        ap[i] = static_cast<const char*>(p.A) + (int64_t)(16 * i + r16) * p.lda * In::kBytes + kq * 16;
+        ap[i] = static_cast<const char*>(p.A) + (int64_t)min(16 * i + r16, p.M - 1) * p.lda * In::kBytes + kq * 16;
     f32x4 acc[MT][NTW];
 #pragma unroll
     for (int i = 0; i < MT; ++i)
@@ -92,9 +94,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_skinny(GemmArgs p) {
 #pragma unroll
         for (int w = 1; w < WAVES; ++w) v += part[w][it][l];
         const int m = 16 * (it / NTW) + l % 16, n = n0 + 16 * (it % NTW) + 4 * (l / 16);
+        if (m >= p.M) continue;
         OutT* d = static_cast<OutT*>(p.D) + (int64_t)m * p.ldd + n;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
+            if (n + e >= p.N) continue;
             float x = v[e] * p.alpha;
             if (p.C) x += Out::load(p.C, (int64_t)m * p.ldc_m + (int64_t)(n + e) * p.ldc_n);
             d[e] = Out::cvt(x);
@@ -108,15 +112,15 @@ static int32_t launch_skinny(const GemmArgs& a, hipStream_t st) {
     const dim3 block(W * 64);
     if (a.N % 32 == 0 && a.N / 32 >= 256) {  // two B tiles per wave once that still fills the chip
         const dim3 grid((unsigned)(a.N / 32), (unsigned)(a.split > 1 ? a.split : 1));
-        switch (a.M / 16) {
+        switch ((a.M + 15) / 16) {
             case 1: gemm_mfma_skinny<In, Out, 1, 2, W><<<grid, block, 0, st>>>(a); break;
             case 2: gemm_mfma_skinny<In, Out, 2, 2, W><<<grid, block, 0, st>>>(a); break;
             case 3: gemm_mfma_skinny<In, Out, 3, 2, W><<<grid, block, 0, st>>>(a); break;
             default: gemm_mfma_skinny<In, Out, 4, 2, W><<<grid, block, 0, st>>>(a); break;
         }
     } else {
-        const dim3 grid((unsigned)(a.N / 16), (unsigned)(a.split > 1 ? a.split : 1));
-        switch (a.M / 16) {
+        const dim3 grid((unsigned)((a.N + 15) / 16), (unsigned)(a.split > 1 ? a.split : 1));
+        switch ((a.M + 15) / 16) {
             case 1: gemm_mfma_skinny<In, Out, 1, 1, W><<<grid, block, 0, st>>>(a); break;
             case 2: gemm_mfma_skinny<In, Out, 2, 1, W><<<grid, block, 0, st>>>(a); break;
             case 3: gemm_mfma_skinny<In, Out, 3, 1, W><<<grid, block, 0, st>>>(a); break;
@@ -137,11 +141,11 @@ static int32_t launch_skinny_out(int32_t out_dt, const GemmArgs& a, hipStream_t 
     }
 }
 
-// M in {16,32,48,64}, N a multiple of 16, K a multiple of 64 bytes; pointers and pitches 16-byte aligned.
+// 1 <= M <= 64, any N, K a multiple of 64 bytes; pointers and pitches 16-byte aligned.
 int32_t gemm_mfma_skinny_dispatch(int32_t in_dt, int32_t out_dt, const GemmArgs& a, hipStream_t st) {
     const int eb = dtype_bytes(in_dt);
-    if (a.M % 16 || a.M > 64 || a.N % 16 || ((int64_t)a.K * eb) % 64)
-        return fail(MOYE_ERR_SHAPE, "gemm!: the short-M MFMA kernel needs M in {16,32,48,64}, N %% 16 == 0 and K %% %d == 0, got %dx%dx%d",
+    if (a.M < 1 || a.M > 64 || a.N < 1 || ((int64_t)a.K * eb) % 64)
+        return fail(MOYE_ERR_SHAPE, "gemm!: the short-M MFMA kernel needs 1 <= M <= 64 and K %% %d == 0, got %dx%dx%d",
                     64 / eb, a.M, a.N, a.K);
     if ((a.lda * eb) % 16 || (a.ldb * eb) % 16 ||
         (reinterpret_cast<uintptr_t>(a.A) | reinterpret_cast<uintptr_t>(a.B)) % 16)

@@ -490,6 +490,31 @@ def test_short_m_exact_on_integers(mh, M):
         assert torch.equal(d.cpu().double(), 2.0 * ref + C.double()), (M, N, K, "C, alpha")
 
 
+@pytest.mark.parametrize("M", [1, 7, 20, 33, 63])
+def test_short_m_any_m_and_n(mh, M):
+    """M and N that are not multiples of 16: lanes beyond the operands read the last row and store nothing.
+    D is a window of a larger buffer whose frame must stay untouched."""
+    g = torch.Generator().manual_seed(90 + M)
+    for (N, K) in ((100, 320), (1, 64), (8200, 256), (8191, 96)):
+        A = torch.randint(-4, 5, (M, K), generator=g).to(torch.float16)
+        B = torch.randint(-4, 5, (N, K), generator=g).to(torch.float16)
+        C = torch.randint(-8, 9, (M, N), generator=g).to(torch.float32)
+        a, b, c = A.cuda(), B.cuda(), C.cuda()
+        ref = A.double() @ B.double().t()
+        big = torch.full((M + 2, N + 3), 77.0, device="cuda")
+        d = big[1:M + 1, 2:N + 2]
+        mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(0, 0, 0)), T(d), T(a), T(b), T(c), 2.0)
+        torch.cuda.synchronize()
+        assert torch.equal(d.cpu().double(), 2.0 * ref + C.double()), (M, N, K)
+        frame = big.clone()
+        frame[1:M + 1, 2:N + 2] = 77.0
+        assert bool((frame == 77.0).all()), "stores outside D"
+        dt_ = torch.zeros(N, M, device="cuda")                 # column-major D: the short side becomes N
+        mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(0, 0, 0)), T(dt_, (M, N), (1, M)), T(a), T(b))
+        torch.cuda.synchronize()
+        assert torch.equal(dt_.t().cpu().double(), ref), (M, N, K, "column-major D")
+
+
 def test_short_m_other_types(mh):
     g = torch.Generator().manual_seed(77)
     M, N, K = 16, 512, 1024

@@ -135,6 +135,12 @@ typedef struct {
  * `tc` may be NULL (plain copyto!). */
 int32_t moye_copy(const moye_tiled_copy* tc, const moye_tensor* dst, const moye_tensor* src,
                   void* stream);
+/* copyto_if!(dest, src, mask) (src/algorithm/copy.jl:4-16): as copyto!, but logical element i moves
+ * only where mask(i) is true.  The reference takes any callable; across this boundary the mask is an
+ * array of one byte per logical element (Bool: nonzero = move) with a layout of its own.  Elements
+ * of dst whose mask is false keep their value. */
+int32_t moye_copy_if(const moye_tensor* dst, const moye_tensor* src, const moye_tensor* mask,
+                     void* stream);
 
 /* gemm!(mma, D, A, B, C) (src/algorithm/blas.jl:11-17 and the dispatch tower :20-131) driven
  * over a whole problem the way the reference's user kernels drive it

@@ -272,6 +272,11 @@ int32_t moye_map(int32_t op, const moye_tensor* dst, const moye_tensor* a, const
     return map_dispatch(op, dst, a, b, scalar, static_cast<hipStream_t>(stream));
 }
 
+int32_t moye_copy_if(const moye_tensor* dst, const moye_tensor* src, const moye_tensor* mask, void* stream) {
+    if (!dst || !src || !mask) return fail(MOYE_ERR_ARG, "copyto_if!: null argument");
+    return copy_if_dispatch(nullptr, dst, src, mask, static_cast<hipStream_t>(stream));
+}
+
 int32_t moye_gemm_workspace_size(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A,
                                  const moye_tensor* B, size_t* bytes) {
     if (!mma || !D || !A || !B || !bytes) return fail(MOYE_ERR_ARG, "moye_gemm_workspace_size: null argument");

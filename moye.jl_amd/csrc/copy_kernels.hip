@@ -295,12 +295,20 @@ __device__ __forceinline__ void store_from(char* p, double v, bool src_is_f64) {
     else *reinterpret_cast<uint8_t*>(p) = f32_to_f8e4m3((float)v);
 }
 
+// copyto_if! (src/algorithm/copy.jl:4-16): element i moves only where the mask's logical element i is nonzero
+struct Mask {
+    const uint8_t* ptr;  // null = every element moves
+    FlatLayout l;
+};
+__device__ __forceinline__ bool masked_out(const Mask& m, int64_t i) { return m.ptr && !m.ptr[layout_offset(m.l, i)]; }
+
 template <int kBytes>
 __global__ __launch_bounds__(256) void copy_generic_bits(const char* __restrict__ src,
                                                          char* __restrict__ dst, FlatLayout ls,
-                                                         FlatLayout ld, int64_t n) {
+                                                         FlatLayout ld, int64_t n, Mask mask) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        if (masked_out(mask, i)) continue;
         const char* s = src + layout_offset(ls, i) * kBytes;
         char* d = dst + layout_offset(ld, i) * kBytes;
         if constexpr (kBytes == 1) *reinterpret_cast<uint8_t*>(d) = *reinterpret_cast<const uint8_t*>(s);
@@ -314,9 +322,10 @@ __global__ __launch_bounds__(256) void copy_generic_bits(const char* __restrict_
 template <int kSrc, int kDst>
 __global__ __launch_bounds__(256) void copy_generic_cvt(const char* __restrict__ src,
                                                         char* __restrict__ dst, FlatLayout ls,
-                                                        FlatLayout ld, int64_t n, int sb, int db) {
+                                                        FlatLayout ld, int64_t n, int sb, int db, Mask mask) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        if (masked_out(mask, i)) continue;
         const double v = load_as_f64<kSrc>(src + layout_offset(ls, i) * sb);
         store_from<kDst>(dst + layout_offset(ld, i) * db, v, kSrc == MOYE_F64);
     }
@@ -346,22 +355,38 @@ static bool is_contiguous(const moye_tensor& t) {
 
 template <int kSrc>
 static bool launch_cvt_dst(int32_t dd, dim3 g, hipStream_t st, const char* s, char* d, FlatLayout ls,
-                           FlatLayout ld, int64_t n, int sb, int db) {
+                           FlatLayout ld, int64_t n, int sb, int db, const Mask& mk) {
     switch (dd) {
-        case MOYE_F32: copy_generic_cvt<kSrc, MOYE_F32><<<g, 256, 0, st>>>(s, d, ls, ld, n, sb, db); return true;
-        case MOYE_F16: copy_generic_cvt<kSrc, MOYE_F16><<<g, 256, 0, st>>>(s, d, ls, ld, n, sb, db); return true;
-        case MOYE_BF16: copy_generic_cvt<kSrc, MOYE_BF16><<<g, 256, 0, st>>>(s, d, ls, ld, n, sb, db); return true;
-        case MOYE_F8E4M3: copy_generic_cvt<kSrc, MOYE_F8E4M3><<<g, 256, 0, st>>>(s, d, ls, ld, n, sb, db); return true;
-        case MOYE_F64: copy_generic_cvt<kSrc, MOYE_F64><<<g, 256, 0, st>>>(s, d, ls, ld, n, sb, db); return true;
+        case MOYE_F32: copy_generic_cvt<kSrc, MOYE_F32><<<g, 256, 0, st>>>(s, d, ls, ld, n, sb, db, mk); return true;
+        case MOYE_F16: copy_generic_cvt<kSrc, MOYE_F16><<<g, 256, 0, st>>>(s, d, ls, ld, n, sb, db, mk); return true;
+        case MOYE_BF16: copy_generic_cvt<kSrc, MOYE_BF16><<<g, 256, 0, st>>>(s, d, ls, ld, n, sb, db, mk); return true;
+        case MOYE_F8E4M3: copy_generic_cvt<kSrc, MOYE_F8E4M3><<<g, 256, 0, st>>>(s, d, ls, ld, n, sb, db, mk); return true;
+        case MOYE_F64: copy_generic_cvt<kSrc, MOYE_F64><<<g, 256, 0, st>>>(s, d, ls, ld, n, sb, db, mk); return true;
         default: return false;
     }
 }
 
 int32_t copy_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, const moye_tensor* src,
                       hipStream_t st) {
+    return copy_if_dispatch(tc, dst, src, nullptr, st);
+}
+
+// `mask` null: copyto!; else copyto_if! with a mask array of one byte per logical element (nonzero = move)
+int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, const moye_tensor* src,
+                         const moye_tensor* mask, hipStream_t st) {
     if (int32_t e = check_tensor(dst, "dst")) return e;
     if (int32_t e = check_tensor(src, "src")) return e;
     const int64_t n = tensor_size(*src);
+    Mask mk{};
+    if (mask) {
+        if (int32_t e = check_tensor(mask, "mask")) return e;
+        if (dtype_bytes(mask->dtype) != 1 || is_float_dtype(mask->dtype))
+            return fail(MOYE_ERR_UNSUPPORTED, "copyto_if!: the mask holds one byte per element (Bool), not %s", dtype_name(mask->dtype));
+        if (tensor_size(*mask) != n)
+            return fail(MOYE_ERR_SHAPE, "copyto_if!: mask holds %lld elements, src %lld", (long long)tensor_size(*mask), (long long)n);
+        mk.ptr = static_cast<const uint8_t*>(mask->ptr);
+        mk.l = flat_of(*mask);
+    }
     if (tensor_size(*dst) != n)
         return fail(MOYE_ERR_SHAPE, "copyto!: dst holds %lld elements, src %lld",
                     (long long)tensor_size(*dst), (long long)n);
@@ -383,7 +408,7 @@ int32_t copy_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, const m
     const char* s = static_cast<const char*>(src->ptr);
     char* d = static_cast<char*>(dst->ptr);
 
-    if (same_bits) {
+    if (same_bits && !mask) {
         // (1) both sides one dense run in the same order
         if (is_contiguous(*src) && is_contiguous(*dst)) {
             const int64_t bytes = n * sb;
@@ -443,7 +468,7 @@ int32_t copy_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, const m
 
     // (3) generic
     FlatLayout ls = flat_of(*src), ld = flat_of(*dst);
-    if (same_bits) {
+    if (same_bits && !mask) {
         // Vectorise when the layouts allow it, which the reference computes (max_common_vector,
         // src/layout.jl:752-761) and then leaves unused (src/algorithm/copy.jl:53-58): if logical
         // neighbours are memory neighbours on both sides in runs of v elements, and every other stride
@@ -470,10 +495,10 @@ int32_t copy_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, const m
             const int64_t nv = n / width;
             const dim3 gv((unsigned)std::min<int64_t>((nv + 255) / 256, 256 * 64));
             switch (sb * width) {
-                case 2: copy_generic_bits<2><<<gv, 256, 0, st>>>(s, d, ls, ld, nv); break;
-                case 4: copy_generic_bits<4><<<gv, 256, 0, st>>>(s, d, ls, ld, nv); break;
-                case 8: copy_generic_bits<8><<<gv, 256, 0, st>>>(s, d, ls, ld, nv); break;
-                default: copy_generic_bits<16><<<gv, 256, 0, st>>>(s, d, ls, ld, nv); break;
+                case 2: copy_generic_bits<2><<<gv, 256, 0, st>>>(s, d, ls, ld, nv, Mask{}); break;
+                case 4: copy_generic_bits<4><<<gv, 256, 0, st>>>(s, d, ls, ld, nv, Mask{}); break;
+                case 8: copy_generic_bits<8><<<gv, 256, 0, st>>>(s, d, ls, ld, nv, Mask{}); break;
+                default: copy_generic_bits<16><<<gv, 256, 0, st>>>(s, d, ls, ld, nv, Mask{}); break;
             }
             MOYE_HIP_CHECK(hipGetLastError());
             return MOYE_OK;
@@ -483,20 +508,20 @@ int32_t copy_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, const m
     bool ok = true;
     if (same_bits) {
         switch (sb) {
-            case 1: copy_generic_bits<1><<<g, 256, 0, st>>>(s, d, ls, ld, n); break;
-            case 2: copy_generic_bits<2><<<g, 256, 0, st>>>(s, d, ls, ld, n); break;
-            case 4: copy_generic_bits<4><<<g, 256, 0, st>>>(s, d, ls, ld, n); break;
-            case 8: copy_generic_bits<8><<<g, 256, 0, st>>>(s, d, ls, ld, n); break;
-            case 16: copy_generic_bits<16><<<g, 256, 0, st>>>(s, d, ls, ld, n); break;
+            case 1: copy_generic_bits<1><<<g, 256, 0, st>>>(s, d, ls, ld, n, mk); break;
+            case 2: copy_generic_bits<2><<<g, 256, 0, st>>>(s, d, ls, ld, n, mk); break;
+            case 4: copy_generic_bits<4><<<g, 256, 0, st>>>(s, d, ls, ld, n, mk); break;
+            case 8: copy_generic_bits<8><<<g, 256, 0, st>>>(s, d, ls, ld, n, mk); break;
+            case 16: copy_generic_bits<16><<<g, 256, 0, st>>>(s, d, ls, ld, n, mk); break;
             default: ok = false;
         }
     } else {
         switch (src->dtype) {
-            case MOYE_F32: ok = launch_cvt_dst<MOYE_F32>(dst->dtype, g, st, s, d, ls, ld, n, sb, db); break;
-            case MOYE_F16: ok = launch_cvt_dst<MOYE_F16>(dst->dtype, g, st, s, d, ls, ld, n, sb, db); break;
-            case MOYE_BF16: ok = launch_cvt_dst<MOYE_BF16>(dst->dtype, g, st, s, d, ls, ld, n, sb, db); break;
-            case MOYE_F8E4M3: ok = launch_cvt_dst<MOYE_F8E4M3>(dst->dtype, g, st, s, d, ls, ld, n, sb, db); break;
-            case MOYE_F64: ok = launch_cvt_dst<MOYE_F64>(dst->dtype, g, st, s, d, ls, ld, n, sb, db); break;
+            case MOYE_F32: ok = launch_cvt_dst<MOYE_F32>(dst->dtype, g, st, s, d, ls, ld, n, sb, db, mk); break;
+            case MOYE_F16: ok = launch_cvt_dst<MOYE_F16>(dst->dtype, g, st, s, d, ls, ld, n, sb, db, mk); break;
+            case MOYE_BF16: ok = launch_cvt_dst<MOYE_BF16>(dst->dtype, g, st, s, d, ls, ld, n, sb, db, mk); break;
+            case MOYE_F8E4M3: ok = launch_cvt_dst<MOYE_F8E4M3>(dst->dtype, g, st, s, d, ls, ld, n, sb, db, mk); break;
+            case MOYE_F64: ok = launch_cvt_dst<MOYE_F64>(dst->dtype, g, st, s, d, ls, ld, n, sb, db, mk); break;
             default: ok = false;
         }
     }

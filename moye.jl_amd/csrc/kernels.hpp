@@ -33,6 +33,8 @@ struct UArgs {
 };
 
 int32_t copy_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, const moye_tensor* src, hipStream_t st);
+int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, const moye_tensor* src, const moye_tensor* mask,
+                         hipStream_t st);
 int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int bk_elems, int waves, int stages,
                               GemmArgs a, hipStream_t st);
 int32_t gemm_mfma_tn_256_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, int waves, int stages, hipStream_t st);

@@ -374,6 +374,14 @@ end
 `gemm!(mma, D, A, B, C)` (src/algorithm/blas.jl:11-17) over whole device operands:
 A:(M,K), B:(N,K), C,D:(M,N); D = alpha * A * B' + C.  Returns `nothing` like the reference.
 """
+"copyto_if!(dst, src, mask) (src/algorithm/copy.jl:4-16); `mask` is a MoYeArray{Bool} (one byte per logical element)."
+function copyto_if!(dst::MoYeArray, src::MoYeArray, mask::MoYeArray{Bool}; stream::Ptr{Cvoid} = C_NULL)
+    m = Tensor(recast(UInt8, mask))
+    GC.@preserve dst src mask check(ccall((:moye_copy_if, LIB), Int32, (Ptr{Tensor}, Ptr{Tensor}, Ptr{Tensor}, Ptr{Cvoid}),
+                                          Ref(Tensor(dst)), Ref(Tensor(src)), Ref(m), stream))
+    dst
+end
+
 function gemm!(mma::TiledMMADesc, D::MoYeArray, A::MoYeArray, B::MoYeArray, C::Union{Nothing,MoYeArray} = nothing;
                alpha::Real = 1.0f0, stream::Ptr{Cvoid} = C_NULL)
     m, d, a, b = Ref(mma), Ref(Tensor(D)), Ref(Tensor(A)), Ref(Tensor(B))

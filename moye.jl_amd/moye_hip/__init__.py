@@ -21,7 +21,7 @@ from .layout import (COLON, GenColMajor, GenRowMajor, Layout, StaticInt, append,
                      tiled_product, zipped_divide, zipped_product, unflatten, group, tuple_append, tuple_prepend,
                      zip2_by, product_each, capacity, elem_scale, filter_zeros, colex_less, elem_less, increment,
                      coord_to_coord, iscompatible, tile_to_shape, make_layout_like, print_layout)
-from .array import (axpby_, fill_, zeros_, map_, broadcast, CopyAtom, MoYeArray, ThrCopy, ThrMMA, TiledCopy as TiledCopyOp, TiledMMA as TiledMMAOp, copyto_,
+from .array import (axpby_, fill_, zeros_, map_, broadcast, CopyAtom, MoYeArray, ThrCopy, ThrMMA, TiledCopy as TiledCopyOp, TiledMMA as TiledMMAOp, copyto_, copyto_if_,
                     gemm_, local_partition, local_tile, make_tiled_copy, make_tiled_copy_A, make_tiled_copy_B,
                     make_tiled_copy_C, make_tiled_mma, transpose, view)
 

@@ -78,6 +78,7 @@ def _declare(l):
     l.moye_version.restype = cs
     sig = {
         "moye_copy": [P(TiledCopy), P(Tensor), P(Tensor), vp],
+        "moye_copy_if": [P(Tensor), P(Tensor), P(Tensor), vp],
         "moye_gemm": [P(TiledMMA), P(Tensor), P(Tensor), P(Tensor), P(Tensor), C.c_float, vp],
         "moye_gemm_workspace_size": [P(TiledMMA), P(Tensor), P(Tensor), P(Tensor), P(S)],
         "moye_device_malloc": [P(vp), S], "moye_device_free": [vp],

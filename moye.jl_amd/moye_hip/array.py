@@ -404,6 +404,14 @@ def copyto_(dst, src, tiled_copy=None, stream=None):
     return dst
 
 
+def copyto_if_(dst, src, mask, stream=None):
+    """copyto_if!(dst, src, mask) (src/algorithm/copy.jl:4-16): element i moves where the mask's element i is true;
+    the mask is a MoYeArray of bytes (Bool) with its own layout.  Returns dst."""
+    t = [x if isinstance(x, _lib.Tensor) else x.tensor() for x in (dst, src, mask)]
+    device.copyto_if_(t[0], t[1], t[2], stream)
+    return dst
+
+
 def gemm_(mma, D, A, B, C_=None, alpha=1.0, stream=None):
     """gemm!(mma, D, A, B, C) (src/algorithm/blas.jl:11-17): D = alpha * A * B' + C with A:(M,K), B:(N,K),
     C,D:(M,N).  gemm_(mma, A, B, C) with three arrays accumulates in place like the reference's 3-argument form."""

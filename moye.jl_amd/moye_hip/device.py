@@ -51,6 +51,13 @@ def copyto_(dst, src, tiled_copy=None, stream=None):
     return dst
 
 
+def copyto_if_(dst, src, mask, stream=None):
+    """copyto_if!(dst, src, mask) (src/algorithm/copy.jl:4-16) on moye_tensor descriptors; the mask holds one byte per
+    logical element, nonzero = move."""
+    check(lib().moye_copy_if(C.byref(dst), C.byref(src), C.byref(mask), stream))
+    return dst
+
+
 def gemm_(mma, D, A, B, C_=None, alpha=1.0, stream=None):
     """gemm!(mma, D, A, B, C): D = alpha * A * B' + C with A:(M,K), B:(N,K), C,D:(M,N)."""
     check(lib().moye_gemm(C.byref(mma), C.byref(D), C.byref(A), C.byref(B), _ref(C_), alpha, stream))

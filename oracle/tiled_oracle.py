@@ -574,6 +574,21 @@ def copyto(dst, src, tiled_copy=None):
     return dst
 
 
+def copyto_if(dst, src, mask):
+    """algorithm/copy.jl:4-16: as copyto!, but logical element i moves only where mask(i) is true.  `mask` is an
+    Array of bytes with its own layout (the reference takes any callable of the 1-based linear index)."""
+    n = len(src)
+    if len(dst) != n or len(mask) != n:
+        raise ValueError("copyto_if!: size mismatch")
+    so, do, mo = src.offsets(), dst.offsets(), mask.offsets()
+    keep = mask.buf[mo] != 0
+    vals = src.buf[so][keep]
+    if dst.dtype != src.dtype:
+        vals = _convert(vals, dst.dtype)
+    dst.buf[do[keep]] = vals
+    return dst
+
+
 def round_bf16(x32):
     """fp32 -> bf16 (kept in fp32 storage), round to nearest even; NaN stays NaN."""
     x32 = np.asarray(x32, dtype=np.float32)

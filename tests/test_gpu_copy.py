@@ -132,6 +132,68 @@ def test_generic_copy_matches_oracle(mh, dl, sl, dtype):
     assert np.array_equal(o_dst.buf, dst_d.cpu().numpy())
 
 
+MASK_LAYOUTS = ["(4,6):(1,4)", "((2,3),(2,4)):((3,1),(6,12))", "(32,8):(8,1)", "(3,5,7):(1,3,15)", "72:1", "105:1"]
+
+
+@pytest.mark.parametrize("case", range(len(CASES)))
+@pytest.mark.parametrize("dtype", ["int8", "int32", "int64", "float16->float32", "float32->bfloat16"])
+def test_copy_if_matches_oracle(mh, case, dtype):
+    """copyto_if! (src/algorithm/copy.jl:4-16): the mask has a layout of its own; elements whose mask is false keep
+    the value dst had.  Plain and converting copies, compared bit for bit with the oracle's element loop."""
+    dl, sl = CASES[case]
+    ld, ls, lm = lo.parse_layout(dl), lo.parse_layout(sl), lo.parse_layout(MASK_LAYOUTS[case])
+    ns, nd, nm = int(lo.cosize(ls)), int(lo.cosize(ld)), int(lo.cosize(lm))
+    g = torch.Generator().manual_seed(11 + case)
+    if "->" in dtype:
+        sdt, ddt = (getattr(torch, x) for x in dtype.split("->"))
+        src = (torch.randn(ns, generator=g) * 100).to(sdt)
+        dst0 = torch.full((nd,), 5.0, dtype=ddt)
+    else:
+        sdt = ddt = getattr(torch, dtype)
+        info = torch.iinfo(sdt)
+        src = torch.randint(max(info.min, -2 ** 62), min(info.max, 2 ** 62), (ns,), dtype=sdt, generator=g)
+        dst0 = torch.full((nd,), 5, dtype=ddt)
+    mask = (torch.rand(nm, generator=g) < 0.5).to(torch.uint8) * 3          # any nonzero byte is true
+    src_d, dst_d, mask_d = src.cuda(), dst0.cuda(), mask.cuda()
+    mh.copyto_if_(_tens(mh, dst_d, *_flat(ld)), _tens(mh, src_d, *_flat(ls)), _tens(mh, mask_d, *_flat(lm)))
+    torch.cuda.synchronize()
+    as_np = lambda t: t.float().numpy().copy() if t.dtype == torch.bfloat16 else t.numpy().copy()
+    o_dst = to.Array(as_np(dst0), ld)
+    o_src = to.Array(as_np(src), ls)
+    if ddt == torch.bfloat16:       # numpy has no bfloat16: convert through torch, element by element as the oracle would
+        keep = to.Array(mask.numpy(), lm).values() != 0
+        want = dst0.clone()
+        want[torch.from_numpy(o_dst.offsets()[keep])] = src[torch.from_numpy(o_src.offsets()[keep])].to(ddt)
+        assert torch.equal(want.view(torch.int16), dst_d.cpu().view(torch.int16))
+    else:
+        to.copyto_if(o_dst, o_src, to.Array(mask.numpy(), lm))
+        assert np.array_equal(o_dst.buf.view(np.uint8), dst_d.cpu().numpy().view(np.uint8))
+    # all-true and all-false masks: copyto! and nothing
+    ones = torch.ones(nm, dtype=torch.uint8, device="cuda")
+    d1, d2 = dst0.cuda(), dst0.cuda()
+    mh.copyto_if_(_tens(mh, d1, *_flat(ld)), _tens(mh, src_d, *_flat(ls)), _tens(mh, ones, *_flat(lm)))
+    mh.copyto_(_tens(mh, d2, *_flat(ld)), _tens(mh, src_d, *_flat(ls)))
+    torch.cuda.synchronize()
+    assert torch.equal(d1.view(torch.uint8), d2.view(torch.uint8))
+    zeros = torch.zeros(nm, dtype=torch.uint8, device="cuda")
+    d3 = dst0.cuda()
+    mh.copyto_if_(_tens(mh, d3, *_flat(ld)), _tens(mh, src_d, *_flat(ls)), _tens(mh, zeros, *_flat(lm)))
+    torch.cuda.synchronize()
+    assert torch.equal(d3.cpu().view(torch.uint8), dst0.view(torch.uint8))
+
+
+def test_copy_if_errors(mh):
+    from moye_hip import _lib
+    x = torch.zeros(24, dtype=torch.float32, device="cuda")
+    m8 = torch.zeros(24, dtype=torch.uint8, device="cuda")
+    with pytest.raises(mh.MoyeError) as e:        # mask of the wrong size
+        mh.copyto_if_(_tens(mh, x, [24], [1]), _tens(mh, x, [24], [1]), _tens(mh, m8, [12], [1]))
+    assert e.value.status == _lib.ERR_SHAPE
+    with pytest.raises(mh.MoyeError) as e:        # mask that is not bytes
+        mh.copyto_if_(_tens(mh, x, [24], [1]), _tens(mh, x, [24], [1]), _tens(mh, x, [24], [1]))
+    assert e.value.status == _lib.ERR_UNSUPPORTED
+
+
 def test_contiguous_copy_and_odd_sizes(mh):
     for n in (1, 7, 4096, 1000003):
         src = _rand_bits(n, n)

@@ -413,3 +413,27 @@ def test_broadcast_layouts_and_known_answers():
     p = to.Array(np.array([0.1, 1000.0], h), lo.make_layout(S(2)))
     q = to.broadcast("mul", p, None, 3.0)
     assert q.buf[0] == h(np.float32(h(0.1)) * np.float32(3.0)) and q.buf.dtype == h
+
+
+def test_copyto_if_moves_only_where_the_mask_is_true():
+    """algorithm/copy.jl:4-12: `if mask(i) apply(copy_op, pointer(dest, i), pointer(src, i))` over the linear index;
+    checked by the element loop written out, on layouts where dst, src and mask all order their elements differently."""
+    ls, ld, lm = lo.parse_layout("(4,6):(1,4)"), lo.parse_layout("(4,6):(6,1)"), lo.parse_layout("((2,2),6):((12,1),2)")
+    rng = np.random.default_rng(5)
+    src = to.Array(rng.integers(-100, 100, 24).astype(np.int32), ls)
+    mask = to.Array((rng.random(24) < 0.5).astype(np.uint8), lm)
+    dst = to.Array(np.full(24, 7, np.int32), ld)
+    want = dst.buf.copy()
+    for i in range(1, 25):
+        if mask.buf[int(lm(i)) - 1]:
+            want[int(ld(i)) - 1] = src.buf[int(ls(i)) - 1]
+    to.copyto_if(dst, src, mask)
+    assert np.array_equal(dst.buf, want)
+    assert 0 < int((want == 7).sum()) < 24            # some moved, some kept
+    # an all-true mask is copyto!
+    d2, d3 = to.Array(np.full(24, 7, np.int32), ld), to.Array(np.full(24, 7, np.int32), ld)
+    to.copyto_if(d2, src, to.Array(np.ones(24, np.uint8), lm))
+    to.copyto(d3, src)
+    assert np.array_equal(d2.buf, d3.buf)
+    with pytest.raises(ValueError):
+        to.copyto_if(dst, src, to.Array(np.ones(12, np.uint8), lo.parse_layout("12:1")))

@@ -213,6 +213,12 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
         g.C = tC ? C.ptr : nullptr; g.ldc_m = C.rs; g.ldc_n = C.cs; g.D = D.ptr;
         return gemm_mfma_tn_dispatch(in_dt, D.dtype, bm, bn, bk, waves, mma->stages, g, st);
     }
+    if (D.rs == 1 && bm == 0 && bn == 0 && M <= 64 && ((int64_t)K * dtype_bytes(in_dt)) % 64 == 0) {
+        // column-major D with a short A: the short-M kernel writes D through both of its strides
+        g.A = A.ptr; g.B = B.ptr; g.M = M; g.N = N; g.lda = A.rs; g.ldb = B.rs; g.ldd = 1; g.ldd_n = D.cs;
+        g.C = tC ? C.ptr : nullptr; g.ldc_m = C.rs; g.ldc_n = C.cs; g.D = D.ptr;
+        return gemm_mfma_skinny_dispatch(in_dt, D.dtype, g, st);
+    }
     if (D.rs == 1) {  // column-major D: D' = B * A' is row-major
         g.A = B.ptr; g.B = A.ptr; g.M = N; g.N = M; g.lda = B.rs; g.ldb = A.rs; g.ldd = D.cs;
         g.C = tC ? C.ptr : nullptr; g.ldc_m = C.cs; g.ldc_n = C.rs; g.D = D.ptr;

@@ -310,6 +310,44 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         // the library chooses: one 256x256 tile per CU when that fills the chip, else 128x128
         const bool big = a.M % 256 == 0 && a.N % 256 == 0 && a.K % (128 / eb) == 0 &&
                          (int64_t)(a.M / 256) * (a.N / 256) >= 128;
+        // A large problem whose M or N is not a multiple of 256: the interior runs on 256x256 tiles, the fringe to the
+        // right (all interior rows, the last N % 256 columns) and the fringe below (the last M % 256 rows, all columns)
+        // on the kernels that take residue tiles.  Three launches on the same stream, disjoint parts of D.
+        const int M0 = a.M / 256 * 256, N0 = a.N / 256 * 256, ob0 = dtype_bytes(out_dt);
+        const bool aligned = !((a.lda * eb) % 16 || (a.ldb * eb) % 16 || (a.ldd * ob0) % 16 ||
+                               (reinterpret_cast<uintptr_t>(a.A) | reinterpret_cast<uintptr_t>(a.B) | reinterpret_cast<uintptr_t>(a.D)) % 16);
+        if (!big && a.split <= 1 && bk_elems == 0 && aligned && a.K % (128 / eb) == 0 && (int64_t)(M0 / 256) * (N0 / 256) >= 128) {
+            GemmArgs part = a;
+            part.M = M0; part.N = N0;
+            if (int32_t e = gemm_mfma_tn_dispatch(in_dt, out_dt, 0, 0, 0, waves, stages, part, st)) return e;
+            if (a.N > N0 && a.N - N0 <= 64 && ((int64_t)a.K * eb) % 64 == 0) {
+                // a narrow fringe is a short-M problem once transposed: D(:, N0:)' = B(N0:, :) * A'
+                part = a;
+                part.M = a.N - N0; part.N = M0;
+                part.A = static_cast<const char*>(a.B) + (int64_t)N0 * a.ldb * eb; part.lda = a.ldb;
+                part.B = a.A; part.ldb = a.lda;
+                part.D = static_cast<char*>(a.D) + (int64_t)N0 * ob0; part.ldd = 1; part.ldd_n = a.ldd;
+                if (a.C) part.C = static_cast<const char*>(a.C) + (int64_t)N0 * a.ldc_n * ob0;
+                part.ldc_m = a.ldc_n; part.ldc_n = a.ldc_m;
+                if (int32_t e = gemm_mfma_skinny_dispatch(in_dt, out_dt, part, st)) return e;
+            } else if (a.N > N0) {
+                part = a;
+                part.M = M0; part.N = a.N - N0;
+                part.B = static_cast<const char*>(a.B) + (int64_t)N0 * a.ldb * eb;
+                part.D = static_cast<char*>(a.D) + (int64_t)N0 * ob0;
+                if (a.C) part.C = static_cast<const char*>(a.C) + (int64_t)N0 * a.ldc_n * ob0;
+                if (int32_t e = gemm_mfma_tn_dispatch(in_dt, out_dt, 0, 0, 0, 0, 0, part, st)) return e;
+            }
+            if (a.M > M0) {
+                part = a;
+                part.M = a.M - M0;
+                part.A = static_cast<const char*>(a.A) + (int64_t)M0 * a.lda * eb;
+                part.D = static_cast<char*>(a.D) + (int64_t)M0 * a.ldd * ob0;
+                if (a.C) part.C = static_cast<const char*>(a.C) + (int64_t)M0 * a.ldc_m * ob0;
+                if (int32_t e = gemm_mfma_tn_dispatch(in_dt, out_dt, 0, 0, 0, 0, 0, part, st)) return e;
+            }
+            return MOYE_OK;
+        }
         bm = bn = big ? 256 : 128;
         if (bk_elems == 0) bk_elems = big || a.K % (128 / eb) == 0 ? 128 / eb : 64 / eb;
         if (big && waves <= 1) waves = 8;

@@ -95,13 +95,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_skinny(GemmArgs p) {
         for (int w = 1; w < WAVES; ++w) v += part[w][it][l];
         const int m = 16 * (it / NTW) + l % 16, n = n0 + 16 * (it % NTW) + 4 * (l / 16);
         if (m >= p.M) continue;
-        OutT* d = static_cast<OutT*>(p.D) + (int64_t)m * p.ldd + n;
+        const int64_t sn = p.ldd_n ? p.ldd_n : 1;  // D may have its unit stride along m (a column-major D, or the
+                                                   // right-hand fringe of a large problem computed as its transpose)
+        OutT* d = static_cast<OutT*>(p.D) + (int64_t)m * p.ldd + (int64_t)n * sn;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             if (n + e >= p.N) continue;
             float x = v[e] * p.alpha;
             if (p.C) x += Out::load(p.C, (int64_t)m * p.ldc_m + (int64_t)(n + e) * p.ldc_n);
-            d[e] = Out::cvt(x);
+            d[e * sn] = Out::cvt(x);
         }
     }
 }

@@ -13,6 +13,7 @@ struct GemmArgs {
     void* D;        // (M,N), N contiguous, row pitch ldd
     int M, N, K;
     int64_t lda, ldb, ldc_m, ldc_n, ldd;
+    int64_t ldd_n;  // stride of D along n; 0 = contiguous.  Only the short-M kernel takes another value.
     float alpha;
     int tiles_m, tiles_n;
     // split-K: gridDim.y ranges of K in one launch; range y reads A and B split_ab bytes further along their rows

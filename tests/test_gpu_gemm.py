@@ -700,6 +700,39 @@ def test_32x32_atoms_take_the_128_tile_only(mh):
     assert "32x32" in str(e.value)
 
 
+@pytest.mark.parametrize("M,N", [(4100, 4104), (4096 + 64, 4096), (4096, 4096 + 136), (4352 + 200, 2816 + 248)])
+def test_large_ragged_problem_runs_its_interior_on_256_tiles(mh, M, N):
+    """Tile left to the library, M or N not a multiple of 256, at least 128 tiles of 256 x 256 inside: interior, right
+    fringe and bottom fringe are three launches; exact on integers, with C and alpha, frame around D untouched."""
+    K = 512
+    g = torch.Generator().manual_seed(M + N)
+    A = torch.randint(-4, 5, (M, K), generator=g).to(torch.float16)
+    B = torch.randint(-4, 5, (N, K), generator=g).to(torch.float16)
+    C = torch.randint(-9, 10, (M, N), generator=g).float()
+    a, b, c = A.cuda(), B.cuda(), C.cuda()
+    ref = (a.double() @ b.double().t())
+    mma = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(0, 0, 0))
+    big = torch.full((M + 2, N + 8), 77.0, device="cuda")
+    d = big[1:M + 1, 4:N + 4]                       # 16-byte aligned window of a larger buffer
+    mh.gemm_(mma, T(d), T(a), T(b))
+    torch.cuda.synchronize()
+    assert torch.equal(d.double(), ref)
+    mh.gemm_(mma, T(d), T(a), T(b), T(c), 0.5)
+    torch.cuda.synchronize()
+    assert torch.equal(d.double(), 0.5 * ref + c.double())
+    frame = big.clone()
+    frame[1:M + 1, 4:N + 4] = 77.0
+    assert bool((frame == 77.0).all()), "stores outside D"
+    d16 = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+    mh.gemm_(mma, T(d16), T(a), T(b), None, 0.25)
+    torch.cuda.synchronize()
+    assert torch.equal(d16.double(), (0.25 * ref).half().double())
+    dt_ = torch.zeros(N, M, device="cuda")                                  # column-major D
+    mh.gemm_(mma, T(dt_, (M, N), (1, M)), T(a), T(b))
+    torch.cuda.synchronize()
+    assert torch.equal(dt_.t().double(), ref)
+
+
 @pytest.mark.parametrize("split", [2, 4, 8])
 def test_split_k_exact_on_integers(mh, split):
     """split_k > 1: K cut into equal ranges, fp32 partial products summed in ascending order in a second pass.

@@ -130,6 +130,22 @@ __global__ __launch_bounds__(256) void axpby_kernel(typename El::compute a, cons
 }
 
 
+template <typename T>
+__device__ __forceinline__ T map_op(int32_t op, T x, T y) {
+    switch (op) {
+        case MOYE_MAP_ADD: return x + y;
+        case MOYE_MAP_SUB: return x - y;
+        case MOYE_MAP_MUL: return x * y;
+        case MOYE_MAP_DIV: return x / y;
+        // Julia's max/min for floats (base/math.jl): a NaN operand is returned; max(-0.0, 0.0) == 0.0
+        case MOYE_MAP_MAX: return ((y > x) | (signbit(y) < signbit(x))) ? (x != x ? x : y) : (y != y ? y : x);
+        case MOYE_MAP_MIN: return ((y < x) | (signbit(y) > signbit(x))) ? (x != x ? x : y) : (y != y ? y : x);
+        case MOYE_MAP_NEG: return -x;
+        case MOYE_MAP_ABS: return signbit(x) ? -x : x;
+        default: return x;  // MOYE_MAP_IDENTITY
+    }
+}
+
 // dst[i] = f(a[i], b[i % nb]) or f(a[i], s): b may be a whole array (nb == n) or span the leading modes of dst
 // and repeat over the trailing ones (Julia's broadcasting of a lower-rank array), or absent (scalar operand)
 template <typename El>
@@ -142,20 +158,7 @@ __global__ __launch_bounds__(256) void map_kernel(int32_t op, typename El::stora
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
         const T x = El::load(a + e_offset(la, i));
         const T y = b ? El::load(b + e_offset(lb, i % nb)) : s;
-        T r;
-        switch (op) {
-            case MOYE_MAP_ADD: r = x + y; break;
-            case MOYE_MAP_SUB: r = x - y; break;
-            case MOYE_MAP_MUL: r = x * y; break;
-            case MOYE_MAP_DIV: r = x / y; break;
-            // Julia's max/min for floats (base/math.jl): a NaN operand is returned; max(-0.0, 0.0) == 0.0
-            case MOYE_MAP_MAX: r = ((y > x) | (signbit(y) < signbit(x))) ? (x != x ? x : y) : (y != y ? y : x); break;
-            case MOYE_MAP_MIN: r = ((y < x) | (signbit(y) > signbit(x))) ? (x != x ? x : y) : (y != y ? y : x); break;
-            case MOYE_MAP_NEG: r = -x; break;
-            case MOYE_MAP_ABS: r = signbit(x) ? -x : x; break;
-            default: r = x; break;  // MOYE_MAP_IDENTITY
-        }
-        El::store(d + e_offset(ld, i), El::round(r));
+        El::store(d + e_offset(ld, i), El::round(map_op(op, x, y)));
     }
 }
 
@@ -169,6 +172,130 @@ __global__ __launch_bounds__(256) void fill_kernel(char* x, ELayout lx, int64_t 
         else if constexpr (kBytes == 4) *reinterpret_cast<uint32_t*>(p) = (uint32_t)bits;
         else *reinterpret_cast<uint64_t*>(p) = bits;
     }
+}
+
+// ---- dense fast path ------------------------------------------------------------------------------------------
+// When every array of a call is one run in logical order (compact column-major after dropping size-1 modes) and
+// 16-byte aligned, logical index = memory index on all sides: 16 bytes per lane and access, four accesses of a lane
+// in flight, no index arithmetic.  The per-element arithmetic is the same code as in the general kernels.
+template <typename El>
+struct DenseVec {
+    typedef typename El::storage S;
+    static constexpr int N = 16 / (int)sizeof(S);
+    typedef S type __attribute__((ext_vector_type(N)));
+};
+constexpr int kDenseU = 4;  // 16-byte accesses of a lane in flight
+
+template <typename El>
+__global__ __launch_bounds__(256) void axpby_dense_kernel(typename El::compute a, const typename El::storage* x,
+                                                          typename El::compute b, typename El::storage* y, int64_t nvec,
+                                                          bool b_is_zero) {
+    typedef typename El::compute T;
+    typedef typename El::storage S;
+    typedef typename DenseVec<El>::type vec;
+    constexpr int N = DenseVec<El>::N;
+    const vec* xv = reinterpret_cast<const vec*>(x);
+    vec* yv = reinterpret_cast<vec*>(y);
+    auto one = [&](const vec& vx, const vec& vy) {
+        vec r;
+#pragma unroll
+        for (int k = 0; k < N; ++k) {
+            S ex = vx[k], ey = vy[k], er;
+            const T ax = El::round(a * El::load(&ex));
+            if (b_is_zero) El::store(&er, ax);
+            else El::store(&er, El::round(ax + El::round(b * El::load(&ey))));
+            r[k] = er;
+        }
+        return r;
+    };
+    const int64_t chunks = nvec / (256 * kDenseU);
+    for (int64_t c = blockIdx.x; c < chunks; c += gridDim.x) {
+        const int64_t base = c * 256 * kDenseU + threadIdx.x;
+        vec vx[kDenseU], vy[kDenseU];
+#pragma unroll
+        for (int u = 0; u < kDenseU; ++u) {
+            vx[u] = __builtin_nontemporal_load(xv + base + u * 256);
+            vy[u] = b_is_zero ? vx[u] : yv[base + u * 256];
+        }
+#pragma unroll
+        for (int u = 0; u < kDenseU; ++u) __builtin_nontemporal_store(one(vx[u], vy[u]), yv + base + u * 256);
+    }
+    for (int64_t i = chunks * 256 * kDenseU + (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256) {
+        const vec vx = xv[i];
+        yv[i] = one(vx, b_is_zero ? vx : yv[i]);
+    }
+}
+
+template <typename El>
+__global__ __launch_bounds__(256) void map_dense_kernel(int32_t op, typename El::storage* d, const typename El::storage* a,
+                                                        const typename El::storage* b, typename El::compute s, int64_t nvec) {
+    typedef typename El::compute T;
+    typedef typename El::storage S;
+    typedef typename DenseVec<El>::type vec;
+    constexpr int N = DenseVec<El>::N;
+    const vec* av = reinterpret_cast<const vec*>(a);
+    const vec* bv = reinterpret_cast<const vec*>(b);
+    vec* dv = reinterpret_cast<vec*>(d);
+    auto one = [&](const vec& va, const vec& vb) {
+        vec r;
+#pragma unroll
+        for (int k = 0; k < N; ++k) {
+            S ea = va[k], eb = vb[k], er;
+            const T x = El::load(&ea);
+            const T y = b ? El::load(&eb) : s;
+            El::store(&er, El::round(map_op(op, x, y)));
+            r[k] = er;
+        }
+        return r;
+    };
+    const int64_t chunks = nvec / (256 * kDenseU);
+    for (int64_t c = blockIdx.x; c < chunks; c += gridDim.x) {
+        const int64_t base = c * 256 * kDenseU + threadIdx.x;
+        vec va[kDenseU], vb[kDenseU];
+#pragma unroll
+        for (int u = 0; u < kDenseU; ++u) {
+            va[u] = av[base + u * 256];
+            vb[u] = b ? bv[base + u * 256] : va[u];
+        }
+#pragma unroll
+        for (int u = 0; u < kDenseU; ++u) __builtin_nontemporal_store(one(va[u], vb[u]), dv + base + u * 256);
+    }
+    for (int64_t i = chunks * 256 * kDenseU + (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256) {
+        const vec va = av[i];
+        dv[i] = one(va, b ? bv[i] : va);
+    }
+}
+
+__global__ __launch_bounds__(256) void fill_dense_kernel(u32x4* x, int64_t nvec, u32x4 pattern) {
+    const int64_t chunks = nvec / (256 * kDenseU);
+    for (int64_t c = blockIdx.x; c < chunks; c += gridDim.x) {
+        const int64_t base = c * 256 * kDenseU + threadIdx.x;
+#pragma unroll
+        for (int u = 0; u < kDenseU; ++u) __builtin_nontemporal_store(pattern, x + base + u * 256);
+    }
+    for (int64_t i = chunks * 256 * kDenseU + (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256)
+        x[i] = pattern;
+}
+
+// one run in logical order?
+bool dense(const moye_tensor& t) {
+    int64_t expect = 1;
+    for (int i = 0; i < t.rank; ++i) {
+        if (t.shape[i] == 1) continue;
+        if (t.stride[i] != expect) return false;
+        expect *= t.shape[i];
+    }
+    return true;
+}
+bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
+dim3 dense_grid(int64_t nvec) { return dim3((unsigned)std::max<int64_t>(1, std::min<int64_t>((nvec + 256 * kDenseU - 1) / (256 * kDenseU), 256 * 32))); }
+ELayout run_layout(int64_t n) {  // a rank-1 run of n elements: what is left of a dense array behind its last whole 16 bytes
+    ELayout l{};
+    l.rank = 1;
+    for (int i = 0; i < MOYE_MAX_RANK; ++i) { l.shape[i] = 1; l.stride[i] = 0; }
+    l.shape[0] = n;
+    l.stride[0] = 1;
+    return l;
 }
 
 int64_t count(const moye_tensor& t) {
@@ -190,6 +317,44 @@ float host_round_bf16(float f) {
 }
 }  // namespace
 
+template <typename El>
+static void launch_axpby(typename El::compute a, const void* x, const ELayout& lx, typename El::compute b, void* y, const ELayout& ly,
+                         int64_t n, bool is_dense, hipStream_t st) {
+    typedef typename El::storage S;
+    const S* xs = static_cast<const S*>(x);
+    S* ys = static_cast<S*>(y);
+    const bool b0 = b == (typename El::compute)0;
+    if (!is_dense) {
+        const dim3 grid((unsigned)std::min<int64_t>((n + 255) / 256, 256 * 16));
+        axpby_kernel<El><<<grid, 256, 0, st>>>(a, xs, lx, b, ys, ly, n, b0);
+        return;
+    }
+    constexpr int N = DenseVec<El>::N;
+    const int64_t nvec = n / N, tail = n - nvec * N;
+    if (nvec) axpby_dense_kernel<El><<<dense_grid(nvec), 256, 0, st>>>(a, xs, b, ys, nvec, b0);
+    if (tail) axpby_kernel<El><<<1, 64, 0, st>>>(a, xs + nvec * N, run_layout(tail), b, ys + nvec * N, run_layout(tail), tail, b0);
+}
+
+template <typename El>
+static void launch_map(int32_t op, void* d, const ELayout& ld, const void* a, const ELayout& la, const void* b, const ELayout& lb,
+                       int64_t nb, typename El::compute s, int64_t n, bool is_dense, hipStream_t st) {
+    typedef typename El::storage S;
+    S* ds = static_cast<S*>(d);
+    const S* as = static_cast<const S*>(a);
+    const S* bs = static_cast<const S*>(b);
+    if (!is_dense) {
+        const dim3 grid((unsigned)std::min<int64_t>((n + 255) / 256, 256 * 16));
+        map_kernel<El><<<grid, 256, 0, st>>>(op, ds, ld, as, la, bs, lb, nb, s, n);
+        return;
+    }
+    constexpr int N = DenseVec<El>::N;
+    const int64_t nvec = n / N, tail = n - nvec * N;
+    if (nvec) map_dense_kernel<El><<<dense_grid(nvec), 256, 0, st>>>(op, ds, as, bs, s, nvec);
+    if (tail)
+        map_kernel<El><<<1, 64, 0, st>>>(op, ds + nvec * N, run_layout(tail), as + nvec * N, run_layout(tail), bs ? bs + nvec * N : nullptr,
+                                         run_layout(tail), tail, s, tail);
+}
+
 int32_t axpby_dispatch(double a, const moye_tensor* X, double b, const moye_tensor* Y, hipStream_t st) {
     if (int32_t e = check_tensor(X, "X")) return e;
     if (int32_t e = check_tensor(Y, "Y")) return e;
@@ -197,29 +362,13 @@ int32_t axpby_dispatch(double a, const moye_tensor* X, double b, const moye_tens
     const int64_t n = count(*X);
     if (count(*Y) != n) return fail(MOYE_ERR_SHAPE, "axpby!: X holds %lld elements, Y %lld", (long long)n, (long long)count(*Y));
     if (n == 0) return MOYE_OK;
-    const dim3 grid((unsigned)std::min<int64_t>((n + 255) / 256, 256 * 16));
     const ELayout lx = elayout_of(*X), ly = elayout_of(*Y);
+    const bool fast = dense(*X) && dense(*Y) && aligned16(X->ptr) && aligned16(Y->ptr);
     switch (X->dtype) {
-        case MOYE_F32:
-            axpby_kernel<ElF32><<<grid, 256, 0, st>>>((float)a, static_cast<const float*>(X->ptr), lx, (float)b,
-                                                      static_cast<float*>(Y->ptr), ly, n, (float)b == 0.f);
-            break;
-        case MOYE_F64:
-            axpby_kernel<ElF64><<<grid, 256, 0, st>>>(a, static_cast<const double*>(X->ptr), lx, b,
-                                                      static_cast<double*>(Y->ptr), ly, n, b == 0.0);
-            break;
-        case MOYE_F16: {
-            const float af = host_round_f16((float)a), bf = host_round_f16((float)b);
-            axpby_kernel<ElF16><<<grid, 256, 0, st>>>(af, static_cast<const _Float16*>(X->ptr), lx, bf,
-                                                      static_cast<_Float16*>(Y->ptr), ly, n, bf == 0.f);
-            break;
-        }
-        case MOYE_BF16: {
-            const float af = host_round_bf16((float)a), bf = host_round_bf16((float)b);
-            axpby_kernel<ElBF16><<<grid, 256, 0, st>>>(af, static_cast<const uint16_t*>(X->ptr), lx, bf,
-                                                       static_cast<uint16_t*>(Y->ptr), ly, n, bf == 0.f);
-            break;
-        }
+        case MOYE_F32: launch_axpby<ElF32>((float)a, X->ptr, lx, (float)b, Y->ptr, ly, n, fast, st); break;
+        case MOYE_F64: launch_axpby<ElF64>(a, X->ptr, lx, b, Y->ptr, ly, n, fast, st); break;
+        case MOYE_F16: launch_axpby<ElF16>(host_round_f16((float)a), X->ptr, lx, host_round_f16((float)b), Y->ptr, ly, n, fast, st); break;
+        case MOYE_BF16: launch_axpby<ElBF16>(host_round_bf16((float)a), X->ptr, lx, host_round_bf16((float)b), Y->ptr, ly, n, fast, st); break;
         default:
             return fail(MOYE_ERR_UNSUPPORTED, "axpby!: element type %s is not a floating-point type this build handles", dtype_name(X->dtype));
     }
@@ -254,27 +403,15 @@ int32_t map_dispatch(int32_t op, const moye_tensor* D, const moye_tensor* A, con
             return fail(MOYE_ERR_SHAPE, "map!: cannot broadcast %lld elements of b over the %lld of dst", (long long)nb, (long long)n);
     }
     if (n == 0) return MOYE_OK;
-    const dim3 grid((unsigned)std::min<int64_t>((n + 255) / 256, 256 * 16));
     const ELayout ld = elayout_of(*D), la = elayout_of(*A), lb = B ? elayout_of(*B) : ELayout{};
+    const void* bp = B ? B->ptr : nullptr;
+    const bool fast = dense(*D) && dense(*A) && aligned16(D->ptr) && aligned16(A->ptr) &&
+                      (!B || (nb == n && dense(*B) && aligned16(B->ptr)));
     switch (D->dtype) {
-        case MOYE_F32:
-            map_kernel<ElF32><<<grid, 256, 0, st>>>(op, static_cast<float*>(D->ptr), ld, static_cast<const float*>(A->ptr), la,
-                                                    B ? static_cast<const float*>(B->ptr) : nullptr, lb, nb, (float)scalar, n);
-            break;
-        case MOYE_F64:
-            map_kernel<ElF64><<<grid, 256, 0, st>>>(op, static_cast<double*>(D->ptr), ld, static_cast<const double*>(A->ptr), la,
-                                                    B ? static_cast<const double*>(B->ptr) : nullptr, lb, nb, scalar, n);
-            break;
-        case MOYE_F16:
-            map_kernel<ElF16><<<grid, 256, 0, st>>>(op, static_cast<_Float16*>(D->ptr), ld, static_cast<const _Float16*>(A->ptr), la,
-                                                    B ? static_cast<const _Float16*>(B->ptr) : nullptr, lb, nb,
-                                                    host_round_f16((float)scalar), n);
-            break;
-        case MOYE_BF16:
-            map_kernel<ElBF16><<<grid, 256, 0, st>>>(op, static_cast<uint16_t*>(D->ptr), ld, static_cast<const uint16_t*>(A->ptr), la,
-                                                     B ? static_cast<const uint16_t*>(B->ptr) : nullptr, lb, nb,
-                                                     host_round_bf16((float)scalar), n);
-            break;
+        case MOYE_F32: launch_map<ElF32>(op, D->ptr, ld, A->ptr, la, bp, lb, nb, (float)scalar, n, fast, st); break;
+        case MOYE_F64: launch_map<ElF64>(op, D->ptr, ld, A->ptr, la, bp, lb, nb, scalar, n, fast, st); break;
+        case MOYE_F16: launch_map<ElF16>(op, D->ptr, ld, A->ptr, la, bp, lb, nb, host_round_f16((float)scalar), n, fast, st); break;
+        case MOYE_BF16: launch_map<ElBF16>(op, D->ptr, ld, A->ptr, la, bp, lb, nb, host_round_bf16((float)scalar), n, fast, st); break;
         default:
             return fail(MOYE_ERR_UNSUPPORTED, "map!: element type %s is not a floating-point type this build handles", dtype_name(D->dtype));
     }
@@ -296,10 +433,29 @@ int32_t fill_dispatch(const moye_tensor* X, double value, hipStream_t st) {
         case MOYE_U8: case MOYE_U16: case MOYE_U32: case MOYE_U64: bits = (uint64_t)(int64_t)value; break;
         default: return fail(MOYE_ERR_UNSUPPORTED, "fill!: no conversion to %s", dtype_name(X->dtype));
     }
+    char* p = static_cast<char*>(X->ptr);
+    const int eb = dtype_bytes(X->dtype);
+    if (dense(*X) && aligned16(p)) {  // the value repeated over 16 bytes, then what is left behind the last whole 16 bytes
+        uint64_t rep = bits;
+        for (int w = eb; w < 8; w *= 2) rep |= rep << (8 * w);
+        const u32x4 pattern = {(uint32_t)rep, (uint32_t)(rep >> 32), (uint32_t)rep, (uint32_t)(rep >> 32)};
+        const int64_t nvec = n * eb / 16, tail = n - nvec * (16 / eb);
+        if (nvec) fill_dense_kernel<<<dense_grid(nvec), 256, 0, st>>>(reinterpret_cast<u32x4*>(p), nvec, pattern);
+        if (tail) {
+            char* q = p + nvec * 16;
+            switch (eb) {
+                case 1: fill_kernel<1><<<1, 64, 0, st>>>(q, run_layout(tail), tail, bits); break;
+                case 2: fill_kernel<2><<<1, 64, 0, st>>>(q, run_layout(tail), tail, bits); break;
+                case 4: fill_kernel<4><<<1, 64, 0, st>>>(q, run_layout(tail), tail, bits); break;
+                default: fill_kernel<8><<<1, 64, 0, st>>>(q, run_layout(tail), tail, bits); break;
+            }
+        }
+        MOYE_HIP_CHECK(hipGetLastError());
+        return MOYE_OK;
+    }
     const dim3 grid((unsigned)std::min<int64_t>((n + 255) / 256, 256 * 16));
     const ELayout lx = elayout_of(*X);
-    char* p = static_cast<char*>(X->ptr);
-    switch (dtype_bytes(X->dtype)) {
+    switch (eb) {
         case 1: fill_kernel<1><<<grid, 256, 0, st>>>(p, lx, n, bits); break;
         case 2: fill_kernel<2><<<grid, 256, 0, st>>>(p, lx, n, bits); break;
         case 4: fill_kernel<4><<<grid, 256, 0, st>>>(p, lx, n, bits); break;

@@ -393,6 +393,55 @@ def lo_text(text, mh):
     return Layout(text)
 
 
+@pytest.mark.parametrize("dt", ["float32", "float64", "float16", "bfloat16"])
+def test_dense_elementwise_paths_match_the_general_kernels(mh, dt):
+    """Arrays that are one aligned run take 16-byte accesses; the same values behind a pointer that is not 16-byte
+    aligned take the general kernels.  Both must give the same bits (axpby!, map! with array and scalar operands,
+    fill!), for sizes that are not a multiple of the vector width and sizes beyond one chunk."""
+    tdt = getattr(torch, dt)
+    g = torch.Generator().manual_seed(31)
+    itype = {2: torch.int16, 4: torch.int32, 8: torch.int64}[torch.empty(0, dtype=tdt).element_size()]
+    for n in (1, 5, 4099, 1 << 20, (1 << 20) + 7):
+        X, Y = (torch.randn(n + 1, generator=g) * 3).to(tdt), (torch.randn(n + 1, generator=g) * 3).to(tdt)
+        xa, ya = X[:n].clone().cuda(), Y[:n].clone().cuda()              # aligned
+        xu_, yu_ = X.cuda(), Y.cuda()
+        xu_[1:] = xa
+        yu_[1:] = ya
+        xu, yu = xu_[1:], yu_[1:]                                         # the same values, one element off alignment
+        def t1(t):
+            return _tens(mh, t, [n], [1])
+        for b in (0.0, -1.25):
+            y1, y2 = ya.clone(), yu_.clone()
+            mh.axpby_(0.75, t1(xa), b, t1(y1))
+            mh.axpby_(0.75, t1(xu), b, t1(y2[1:]))
+            torch.cuda.synchronize()
+            assert torch.equal(y1.view(itype), y2[1:].view(itype)), (dt, n, "axpby", b)
+        for op in ("add", "mul", "max", "div", "abs"):
+            for second in ("array", "scalar"):
+                d1, d2 = torch.zeros(n, dtype=tdt, device="cuda"), torch.zeros(n + 1, dtype=tdt, device="cuda")
+                mh.map_(op, t1(d1), t1(xa), t1(ya) if second == "array" else None, 1.75)
+                mh.map_(op, t1(d2[1:]), t1(xu), t1(yu) if second == "array" else None, 1.75)
+                torch.cuda.synchronize()
+                same = d1.view(itype) == d2[1:].view(itype)
+                assert bool((same | (torch.isnan(d1.float()) & torch.isnan(d2[1:].float()))).all()), (dt, n, op, second)
+        if dt == "float32":       # and against torch where the rounding is plain IEEE
+            d1 = torch.zeros(n, dtype=tdt, device="cuda")
+            mh.map_("add", t1(d1), t1(xa), t1(ya))
+            torch.cuda.synchronize()
+            assert torch.equal(d1, xa + ya)
+        f1, f2 = torch.zeros(n, dtype=tdt, device="cuda"), torch.zeros(n + 1, dtype=tdt, device="cuda")
+        mh.fill_(t1(f1), 2.71828)
+        mh.fill_(t1(f2[1:]), 2.71828)
+        torch.cuda.synchronize()
+        assert torch.equal(f1.view(itype), f2[1:].view(itype)) and float(f2[0]) == 0.0
+        assert torch.equal(f1, torch.full((n,), 2.71828, dtype=tdt, device="cuda"))
+    for idt in (torch.uint8, torch.int16, torch.int32, torch.int64):        # fill! of integer arrays through the dense path
+        z = torch.zeros(1037, dtype=idt, device="cuda")
+        mh.fill_(_tens(mh, z, [1037], [1]), 93)
+        torch.cuda.synchronize()
+        assert bool((z == 93).all())
+
+
 def test_axpby_errors(mh):
     x = torch.zeros(8, device="cuda")
     y = torch.zeros(8, dtype=torch.float16, device="cuda")

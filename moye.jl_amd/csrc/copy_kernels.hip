@@ -331,6 +331,50 @@ __global__ __launch_bounds__(256) void copy_generic_cvt(const char* __restrict__
     }
 }
 
+// Converting copy between two dense, 16-byte aligned runs: a lane converts E = 16 / min(sizeof) elements per step, so
+// that the narrower side moves 16 bytes per access and the wider side a whole number of 16-byte accesses; two steps
+// of a lane are in flight.  Used where the destination is the narrower side (or as wide).  Element by element the same
+// conversion as copy_generic_cvt.
+template <int kSrc, int kDst, int SB, int DB>
+__global__ __launch_bounds__(256) void copy_cvt_dense(const char* __restrict__ src, char* __restrict__ dst, int64_t nsteps) {
+    constexpr int E = 16 / (SB < DB ? SB : DB), SV = E * SB / 16, DV = E * DB / 16, U = 2;
+    const u32x4* sv = reinterpret_cast<const u32x4*>(src);
+    u32x4* dv = reinterpret_cast<u32x4*>(dst);
+    auto convert = [](const u32x4 (&in)[SV], u32x4 (&out)[DV]) {
+#pragma unroll
+        for (int k = 0; k < E; ++k) {
+            char e_in[SB], e_out[DB];
+            __builtin_memcpy(e_in, reinterpret_cast<const char*>(in) + k * SB, SB);
+            store_from<kDst>(e_out, load_as_f64<kSrc>(e_in), kSrc == MOYE_F64);
+            __builtin_memcpy(reinterpret_cast<char*>(out) + k * DB, e_out, DB);
+        }
+    };
+    const int64_t stride = (int64_t)gridDim.x * 256 * U;
+    int64_t i = (int64_t)blockIdx.x * 256 * U + threadIdx.x;
+    for (; i + 256 * (U - 1) < nsteps; i += stride) {
+        u32x4 in[U][SV], out[U][DV];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int q = 0; q < SV; ++q) in[u][q] = __builtin_nontemporal_load(sv + (i + 256 * u) * SV + q);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            convert(in[u], out[u]);
+#pragma unroll
+            for (int q = 0; q < DV; ++q) __builtin_nontemporal_store(out[u][q], dv + (i + 256 * u) * DV + q);
+        }
+    }
+    for (; i < nsteps; i += 256) {  // the last, partial group of this lane's stride
+        if (i >= nsteps) break;
+        u32x4 in[SV], out[DV];
+#pragma unroll
+        for (int q = 0; q < SV; ++q) in[q] = sv[i * SV + q];
+        convert(in, out);
+#pragma unroll
+        for (int q = 0; q < DV; ++q) dv[i * DV + q] = out[q];
+    }
+}
+
 static FlatLayout flat_of(const moye_tensor& t) {
     FlatLayout f;
     f.rank = t.rank;
@@ -351,6 +395,125 @@ static bool is_contiguous(const moye_tensor& t) {
         expect *= t.shape[i];
     }
     return true;
+}
+
+// The widening direction: a lane's 16-byte store holds EW = 16 / sizeof(dst) elements, which it reads as one access of
+// EW * sizeof(src) bytes (8, 4 or 2), so that loads and stores of a wave are both contiguous; four of them in flight.
+template <int NB> struct NarrowWord;
+template <> struct NarrowWord<8> { typedef uint64_t type; };
+template <> struct NarrowWord<4> { typedef uint32_t type; };
+template <> struct NarrowWord<2> { typedef uint16_t type; };
+template <int kSrc, int kDst, int SB, int DB>
+__global__ __launch_bounds__(256) void copy_cvt_dense_widen(const char* __restrict__ src, char* __restrict__ dst, int64_t nvec) {
+    constexpr int EW = 16 / DB, NB = EW * SB, U = 4;
+    typedef typename NarrowWord<NB>::type word;
+    const word* sv = reinterpret_cast<const word*>(src);
+    u32x4* dv = reinterpret_cast<u32x4*>(dst);
+    auto convert = [](word in) {
+        u32x4 out;
+#pragma unroll
+        for (int k = 0; k < EW; ++k) {
+            char e_in[SB], e_out[DB];
+            __builtin_memcpy(e_in, reinterpret_cast<const char*>(&in) + k * SB, SB);
+            store_from<kDst>(e_out, load_as_f64<kSrc>(e_in), kSrc == MOYE_F64);
+            __builtin_memcpy(reinterpret_cast<char*>(&out) + k * DB, e_out, DB);
+        }
+        return out;
+    };
+    const int64_t chunks = nvec / (256 * U);
+    for (int64_t c = blockIdx.x; c < chunks; c += gridDim.x) {
+        const int64_t base = c * 256 * U + threadIdx.x;
+        word in[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) in[u] = __builtin_nontemporal_load(sv + base + u * 256);
+#pragma unroll
+        for (int u = 0; u < U; ++u) __builtin_nontemporal_store(convert(in[u]), dv + base + u * 256);
+    }
+    for (int64_t i = chunks * 256 * U + (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256)
+        dv[i] = convert(sv[i]);
+}
+
+// The narrowing direction when the source is at least four times as wide: a lane reads 16 bytes and stores the
+// EN = 16 / sizeof(src) converted elements as one access of 2, 4 or 8 bytes; loads and stores of a wave are contiguous.
+template <int kSrc, int kDst, int SB, int DB>
+__global__ __launch_bounds__(256) void copy_cvt_dense_narrow(const char* __restrict__ src, char* __restrict__ dst, int64_t nvec) {
+    constexpr int EN = 16 / SB, NB = EN * DB, U = 4;
+    typedef typename NarrowWord<NB>::type word;
+    const u32x4* sv = reinterpret_cast<const u32x4*>(src);
+    word* dv = reinterpret_cast<word*>(dst);
+    auto convert = [](const u32x4& in) {
+        word out;
+#pragma unroll
+        for (int k = 0; k < EN; ++k) {
+            char e_in[SB], e_out[DB];
+            __builtin_memcpy(e_in, reinterpret_cast<const char*>(&in) + k * SB, SB);
+            store_from<kDst>(e_out, load_as_f64<kSrc>(e_in), kSrc == MOYE_F64);
+            __builtin_memcpy(reinterpret_cast<char*>(&out) + k * DB, e_out, DB);
+        }
+        return out;
+    };
+    const int64_t chunks = nvec / (256 * U);
+    for (int64_t c = blockIdx.x; c < chunks; c += gridDim.x) {
+        const int64_t base = c * 256 * U + threadIdx.x;
+        u32x4 in[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) in[u] = __builtin_nontemporal_load(sv + base + u * 256);
+#pragma unroll
+        for (int u = 0; u < U; ++u) dv[base + u * 256] = convert(in[u]);
+    }
+    for (int64_t i = chunks * 256 * U + (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256)
+        dv[i] = convert(sv[i]);
+}
+
+constexpr int float_bytes(int dt) { return dt == MOYE_F64 ? 8 : dt == MOYE_F32 ? 4 : dt == MOYE_F8E4M3 ? 1 : 2; }
+
+// dense converting copy of the first n - n % E elements; returns how many elements it covered (0: not launched)
+template <int kSrc, int kDst>
+static int64_t launch_cvt_dense_pair(const char* s, char* d, int64_t n, hipStream_t st) {
+    constexpr int SB = float_bytes(kSrc), DB = float_bytes(kDst), E = 16 / (SB < DB ? SB : DB);
+    if constexpr (DB > SB) {
+        constexpr int EW = 16 / DB;
+        const int64_t nvec = n / EW;
+        if (nvec == 0) return 0;
+        const unsigned blocks = (unsigned)std::min<int64_t>((nvec + 1023) / 1024, 256 * 32);
+        copy_cvt_dense_widen<kSrc, kDst, SB, DB><<<blocks, 256, 0, st>>>(s, d, nvec);
+        return nvec * EW;
+    }
+    if constexpr (SB >= 4 * DB && (16 / SB) * DB >= 2) {
+        constexpr int EN = 16 / SB;
+        const int64_t nvec = n / EN;
+        if (nvec == 0) return 0;
+        const unsigned blocks = (unsigned)std::min<int64_t>((nvec + 1023) / 1024, 256 * 32);
+        copy_cvt_dense_narrow<kSrc, kDst, SB, DB><<<blocks, 256, 0, st>>>(s, d, nvec);
+        return nvec * EN;
+    }
+    const int64_t nsteps = n / E;
+    if (nsteps == 0) return 0;
+    const unsigned blocks = (unsigned)std::min<int64_t>((nsteps + 511) / 512, 256 * 16);
+    copy_cvt_dense<kSrc, kDst, SB, DB><<<blocks, 256, 0, st>>>(s, d, nsteps);
+    return nsteps * E;
+}
+template <int kSrc>
+static int64_t launch_cvt_dense_dst(int32_t dd, const char* s, char* d, int64_t n, hipStream_t st) {
+    switch (dd) {
+        case MOYE_F32: if constexpr (kSrc != MOYE_F32) return launch_cvt_dense_pair<kSrc, MOYE_F32>(s, d, n, st); break;
+        case MOYE_F16: if constexpr (kSrc != MOYE_F16) return launch_cvt_dense_pair<kSrc, MOYE_F16>(s, d, n, st); break;
+        case MOYE_BF16: if constexpr (kSrc != MOYE_BF16) return launch_cvt_dense_pair<kSrc, MOYE_BF16>(s, d, n, st); break;
+        case MOYE_F8E4M3: if constexpr (kSrc != MOYE_F8E4M3) return launch_cvt_dense_pair<kSrc, MOYE_F8E4M3>(s, d, n, st); break;
+        case MOYE_F64: if constexpr (kSrc != MOYE_F64) return launch_cvt_dense_pair<kSrc, MOYE_F64>(s, d, n, st); break;
+        default: break;
+    }
+    return 0;
+}
+static int64_t launch_cvt_dense(int32_t sd, int32_t dd, const char* s, char* d, int64_t n, hipStream_t st) {
+    switch (sd) {
+        case MOYE_F32: return launch_cvt_dense_dst<MOYE_F32>(dd, s, d, n, st);
+        case MOYE_F16: return launch_cvt_dense_dst<MOYE_F16>(dd, s, d, n, st);
+        case MOYE_BF16: return launch_cvt_dense_dst<MOYE_BF16>(dd, s, d, n, st);
+        case MOYE_F8E4M3: return launch_cvt_dense_dst<MOYE_F8E4M3>(dd, s, d, n, st);
+        case MOYE_F64: return launch_cvt_dense_dst<MOYE_F64>(dd, s, d, n, st);
+        default: return 0;
+    }
 }
 
 template <int kSrc>
@@ -376,7 +539,7 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
                          const moye_tensor* mask, hipStream_t st) {
     if (int32_t e = check_tensor(dst, "dst")) return e;
     if (int32_t e = check_tensor(src, "src")) return e;
-    const int64_t n = tensor_size(*src);
+    int64_t n = tensor_size(*src);
     Mask mk{};
     if (mask) {
         if (int32_t e = check_tensor(mask, "mask")) return e;
@@ -502,6 +665,24 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
             }
             MOYE_HIP_CHECK(hipGetLastError());
             return MOYE_OK;
+        }
+    }
+    if (!same_bits && !mask && is_contiguous(*src) && is_contiguous(*dst) &&
+        (reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d)) % 16 == 0) {
+        // both sides one aligned run: 16-byte accesses for all whole groups, the general kernel for what is left
+        const int64_t done = launch_cvt_dense(src->dtype, dst->dtype, s, d, n, st);
+        if (done > 0) {
+            MOYE_HIP_CHECK(hipGetLastError());
+            if (done == n) return MOYE_OK;
+            s += done * sb;
+            d += done * db;
+            n -= done;
+            for (FlatLayout* l : {&ls, &ld}) {
+                l->rank = 1;
+                for (int m = 0; m < MOYE_MAX_RANK; ++m) { l->shape[m] = 1; l->stride[m] = 0; }
+                l->shape[0] = n;
+                l->stride[0] = 1;
+            }
         }
     }
     const dim3 g((unsigned)std::min<int64_t>((n + 255) / 256, 256 * 64));

@@ -66,6 +66,39 @@ def test_transpose_other_orientation_and_pitch(mh):
     assert bool((dst.view(N, ldd)[:, M:] == -1).all())  # padding untouched
 
 
+@pytest.mark.parametrize("dt", ["float32", "float16"])
+@pytest.mark.parametrize("M,N", [(1000, 1032), (72, 4104), (8200, 136), (64, 64 + 8)])
+def test_ragged_transpose_interior_and_strips(mh, M, N, dt):
+    """Sizes that are not multiples of the 64 x 64 tile: the interior goes through the LDS tiles, the strips through the
+    general kernel; together they are the transpose, bit for bit, and nothing outside dst is written."""
+    tdt = getattr(torch, dt)
+    bits = _rand_bits(M * N, 5).view(torch.int32)
+    src = (bits.view(torch.float32) if dt == "float32" else bits.to(torch.int16).view(torch.float16)).clone()   # any bit pattern
+    big = torch.full(((N + 2) * M + 16,), 7, dtype=tdt, device="cuda")
+    dst = big[8:8 + N * M]
+    # src column-major (M, N):(1, M) ... as a row-major (M, N):(N, 1)
+    mh.copyto_(_tens(mh, dst, (M, N), (N, 1)), _tens(mh, src, (M, N), (1, M)))
+    torch.cuda.synchronize()
+    it = torch.int32 if dt == "float32" else torch.int16
+    assert torch.equal(dst.view(it).view(M, N), src.view(it).view(N, M).t())
+    assert bool((big[:8] == 7).all()) and bool((big[8 + N * M:] == 7).all())
+
+
+@pytest.mark.parametrize("dt", ["float32", "float16"])
+def test_ragged_transpose_with_padded_pitches(mh, dt):
+    """Sizes that are not even whole 16-byte pieces, inside aligned pitches: the strips go through the general kernel."""
+    tdt = getattr(torch, dt)
+    M, N, PM, PN = 1002, 205, 1008, 208
+    it = torch.int32 if dt == "float32" else torch.int16
+    src = _rand_bits(PM * N, 6).to(it).view(tdt).clone()
+    dst = torch.full((M * PN,), 7, dtype=tdt, device="cuda")
+    mh.copyto_(_tens(mh, dst, (M, N), (PN, 1)), _tens(mh, src, (M, N), (1, PM)))
+    torch.cuda.synchronize()
+    got = dst.view(it).view(M, PN)
+    assert torch.equal(got[:, :N], src.view(it).view(N, PM)[:, :M].t())
+    assert bool((dst.view(M, PN)[:, N:] == 7).all())          # the padding of dst is untouched
+
+
 def test_transpose_without_swizzle_is_identical(mh):
     M = N = 256
     src = _rand_bits(M * N, 11)

@@ -191,6 +191,81 @@ static int32_t launch_transpose16(const uint16_t* s, uint16_t* d, int64_t lds_, 
 }
 
 // ------------------------------------------------------------------------------------------
+// the same for 1-byte elements (fp8 matrices, bytes)
+// ------------------------------------------------------------------------------------------
+// A sub-tile is 256 source rows (j) of 64 bytes (i); a workgroup moves GI of them that are neighbours along i.  Rows go
+// to LDS as they come, 16 bytes per lane.  A lane then owns a block of 4 (i) x 16 (j) bytes: it reads the 16 rows'
+// dwords, transposes the bytes in registers and stores four 16-byte pieces, one to each of four consecutive
+// destination rows.  A 64-byte LDS row spans 16 of the 64 banks, so rows that are a multiple of four apart share
+// banks; the lanes of a wave read rows 16 apart, hence rows are stored with their two low index bits XORed with
+// bits 4-5: the four rows a wave reads at once then lie in four different bank groups.
+constexpr int kTileJ8 = 256;
+__device__ __forceinline__ int lds_row_b8(int j) { return (j & ~3) | ((j & 3) ^ ((j >> 4) & 3)); }
+
+template <int GI>
+__global__ __launch_bounds__(256) void transpose_lds_b8(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, int64_t lds_,
+                                                        int64_t ldd, int groups_i, int tiles_j, int sb) {
+    extern __shared__ u32x4 tile[];  // GI sub-tiles of 256 rows x 4 chunks
+    int gi, tj;
+    tile_coords(blockIdx.x, groups_i, tiles_j, sb, &gi, &tj);
+    const int v = threadIdx.x & 3;   // 16-byte chunk of a 64-byte row
+    const int r = threadIdx.x >> 2;  // 0..63
+
+    // ---- load: rows j = r + 64 h, bytes i = 16 v .. 16 v + 15 of each sub-tile ----
+    const uint8_t* s = src + ((int64_t)tj * kTileJ8 + r) * lds_ + (int64_t)gi * GI * kTile + 16 * v;
+    u32x4 x[GI][4];
+#pragma unroll
+    for (int h = 0; h < 4; ++h)
+#pragma unroll
+        for (int a = 0; a < GI; ++a)
+            x[a][h] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(s + (int64_t)(64 * h) * lds_ + a * kTile));
+#pragma unroll
+    for (int a = 0; a < GI; ++a)
+#pragma unroll
+        for (int h = 0; h < 4; ++h) tile[a * 1024 + lds_row_b8(r + 64 * h) * 4 + v] = x[a][h];
+    __syncthreads();
+
+    // ---- store: destination rows i = 4 ib .. 4 ib + 3, bytes j = 16 c .. 16 c + 15 ----
+    const uint32_t* lds32 = reinterpret_cast<const uint32_t*>(tile);
+    const int ib = threadIdx.x & 15, c = threadIdx.x >> 4;
+    uint8_t* d = dst + ((int64_t)gi * GI * kTile + 4 * ib) * ldd + (int64_t)tj * kTileJ8 + 16 * c;
+#pragma unroll
+    for (int a = 0; a < GI; ++a) {
+        uint32_t w[16];
+#pragma unroll
+        for (int q = 0; q < 16; ++q) w[q] = lds32[a * 4096 + lds_row_b8(16 * c + q) * 16 + ib];  // S[16 c + q][4 ib .. 4 ib + 3]
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            u32x4 o;
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+                o[g] = ((w[4 * g] >> (8 * e)) & 0xffu) | (((w[4 * g + 1] >> (8 * e)) & 0xffu) << 8) |
+                       (((w[4 * g + 2] >> (8 * e)) & 0xffu) << 16) | (((w[4 * g + 3] >> (8 * e)) & 0xffu) << 24);
+            __builtin_nontemporal_store(o, reinterpret_cast<u32x4*>(d + (int64_t)(a * kTile + e) * ldd));
+        }
+    }
+}
+
+template <int GI>
+static int32_t launch_transpose8(const uint8_t* s, uint8_t* d, int64_t lds_, int64_t ldd, int ti, int tj, hipStream_t st) {
+    auto kern = transpose_lds_b8<GI>;
+    constexpr int kLds = GI * kTileJ8 * kTile;
+    if (kLds > 48 * 1024) {
+        static bool once = false;
+        if (!once) {
+            MOYE_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
+            once = true;
+        }
+    }
+    const int64_t groups = (int64_t)(ti / GI) * tj;
+    if (groups > 0x7fffffff) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles");
+    kern<<<(unsigned)groups, 256, kLds, st>>>(s, d, lds_, ldd, ti / GI, tj, 64);
+    MOYE_HIP_CHECK(hipGetLastError());
+    return MOYE_OK;
+}
+
+// ------------------------------------------------------------------------------------------
 // contiguous streaming copy, 16 bytes per lane per step
 // ------------------------------------------------------------------------------------------
 // each workgroup walks contiguous 16 KiB chunks (4 x 16 bytes per lane in flight): measured
@@ -589,7 +664,7 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
         // (2) rank-2 transpose of 4-byte elements through the LDS tile
         const int tm = tc && tc->tiler_mn[0] ? tc->tiler_mn[0] : kTile;
         const int tn = tc && tc->tiler_mn[1] ? tc->tiler_mn[1] : kTile;
-        if ((sb == 4 || sb == 2) && src->rank == 2 && dst->rank == 2 && src->shape[0] == dst->shape[0] &&
+        if ((sb == 4 || sb == 2 || sb == 1) && src->rank == 2 && dst->rank == 2 && src->shape[0] == dst->shape[0] &&
             src->shape[1] == dst->shape[1] && tm == kTile && tn == kTile) {
             const moye_tensor *a = src, *b = dst;
             bool ok = false, swap = false;
@@ -601,11 +676,19 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
                 const int64_t ni = a->shape[mi], nj = a->shape[mj];
                 const int64_t lds_ = a->stride[mj], ldd = b->stride[mi];
                 const int per16 = 16 / sb;  // elements per 16-byte access
-                const bool aligned = ni % kTile == 0 && nj % kTile == 0 && lds_ % per16 == 0 && ldd % per16 == 0 &&
+                const int tile_j = sb == 1 ? kTileJ8 : kTile;  // extent of a tile along the destination's contiguous index
+                const bool aligned = ni % kTile == 0 && nj % tile_j == 0 && lds_ % per16 == 0 && ldd % per16 == 0 &&
                                      lds_ >= ni && ldd >= nj &&
                                      (reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d)) % 16 == 0;
                 if (aligned) {
-                    const int ti = (int)(ni / kTile), tj = (int)(nj / kTile);
+                    const int ti = (int)(ni / kTile), tj = (int)(nj / tile_j);
+                    if (sb == 1) {
+                        const uint8_t* s8 = reinterpret_cast<const uint8_t*>(s);
+                        uint8_t* d8 = reinterpret_cast<uint8_t*>(d);
+                        if (ti % 4 == 0) return launch_transpose8<4>(s8, d8, lds_, ldd, ti, tj, st);
+                        if (ti % 2 == 0) return launch_transpose8<2>(s8, d8, lds_, ldd, ti, tj, st);
+                        return launch_transpose8<1>(s8, d8, lds_, ldd, ti, tj, st);
+                    }
                     if (sb == 2) {
                         const uint16_t* s16 = reinterpret_cast<const uint16_t*>(s);
                         uint16_t* d16 = reinterpret_cast<uint16_t*>(d);
@@ -625,7 +708,7 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
                 // LDS tiles, the two strips that are left through the general kernel.  Three launches, disjoint parts.  (A strip
                 // touches one page per row of the other side, so it costs far more per byte than the interior: 16400 x 16392
                 // fp32 runs at 3.3 TB/s against 5.6 for 16384 x 16384; whole tiles pushed against the edge cost the same.)
-                const int64_t ni0 = ni / kTile * kTile, nj0 = nj / kTile * kTile;
+                const int64_t ni0 = ni / kTile * kTile, nj0 = nj / tile_j * tile_j;
                 if (!(tc && tc->op == MOYE_COPY_LDS_TILED) && ni0 > 0 && nj0 > 0 && lds_ % per16 == 0 && ldd % per16 == 0 &&
                     lds_ >= ni && ldd >= nj && (reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d)) % 16 == 0) {
                     // sub-array [i0, i0 + ci) x [j0, j0 + cj) of both sides

@@ -565,3 +565,34 @@ def test_transpose_two_byte_elements(mh, M, N):
     torch.cuda.synchronize()
     assert torch.equal(dst2.view(N, ldd)[:, :M], src2.view(M, lds)[:, :N].t())
     assert bool((dst2.view(N, ldd)[:, M:] == -1).all())
+
+
+@pytest.mark.parametrize("M,N", [(64, 256), (128, 512), (192, 256), (256, 1024), (4096, 4096), (8192, 2048), (200, 300), (1088, 784)])
+def test_transpose_one_byte_elements(mh, M, N):
+    """fp8 matrices / bytes through the 1-byte LDS tile (64 x 256; 1, 2 or 4 sub-tiles per workgroup depending on M), sizes
+    that are not multiples of the tile through interior + strips or the general kernel: both orientations, padded pitches,
+    compared as bytes; the oracle on the small cases."""
+    g = torch.Generator().manual_seed(M + N)
+    src = torch.randint(0, 256, (M * N,), dtype=torch.uint8, generator=g).cuda()
+    dst = torch.zeros(M * N, dtype=torch.uint8, device="cuda")
+    mh.copyto_(_tens(mh, dst, (M, N), (N, 1)), _tens(mh, src, (M, N), (1, M)))
+    torch.cuda.synchronize()
+    assert torch.equal(dst.view(M, N), src.view(N, M).t())
+    if M * N <= 128 * 512:
+        s = to.Array(src.cpu().numpy(), lo.make_layout((M, N), (1, M)))
+        d = to.Array(np.zeros(M * N, np.uint8), lo.make_layout((M, N), (N, 1)))
+        to.copyto(d, s)
+        assert np.array_equal(d.buf, dst.cpu().numpy())
+    # the other orientation with padded pitches (multiples of 16 bytes)
+    lds, ldd = N + 16, M + 48
+    src2 = torch.randint(0, 256, (M * lds,), dtype=torch.uint8, generator=g).cuda()
+    dst2 = torch.full((N * ldd,), 255, dtype=torch.uint8, device="cuda")
+    mh.copyto_(_tens(mh, dst2, (M, N), (1, ldd)), _tens(mh, src2, (M, N), (lds, 1)))
+    torch.cuda.synchronize()
+    assert torch.equal(dst2.view(N, ldd)[:, :M], src2.view(M, lds)[:, :N].t())
+    assert bool((dst2.view(N, ldd)[:, M:] == 255).all())
+    if hasattr(torch, "float8_e4m3fn") and M % 64 == 0:      # the same through the fp8 element type
+        s8, d8 = src.view(torch.float8_e4m3fn), torch.zeros(M * N, dtype=torch.uint8, device="cuda").view(torch.float8_e4m3fn)
+        mh.copyto_(_tens(mh, d8, (M, N), (N, 1)), _tens(mh, s8, (M, N), (1, M)))
+        torch.cuda.synchronize()
+        assert torch.equal(d8.view(torch.uint8), dst)

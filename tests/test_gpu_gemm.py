@@ -870,6 +870,25 @@ def test_operand_majors_nn_nt_tt(mh):
             assert "K-major" in str(e.value)
 
 
+def test_operand_majors_other_element_types(mh):
+    """The NN form (A stored M-major, B stored N-major) for fp8, bf16 and fp32 operands: their K-major copies go through
+    the 1-, 2- and 4-byte LDS-tiled transposes.  Exact on integers."""
+    cases = [(mh.MFMA_F32_16x16x32_BF16, torch.bfloat16), (mh.MFMA_F32_16x16x4_F32, torch.float32)]
+    if hasattr(torch, "float8_e4m3fn"):
+        cases.append((mh.MFMA_F32_16x16x32_FP8, torch.float8_e4m3fn))
+    g = torch.Generator().manual_seed(62)
+    for atom, tdt in cases:
+        for (M, N, K) in ((256, 512, 256), (320, 192, 448)):
+            A = torch.randint(-4, 5, (M, K), generator=g).float()
+            B = torch.randint(-4, 5, (N, K), generator=g).float()
+            ref = A.double() @ B.double().t()
+            a_m, b_n = A.t().contiguous().to(tdt).cuda(), B.t().contiguous().to(tdt).cuda()
+            d = torch.zeros(M, N, dtype=torch.float32, device="cuda")
+            mh.gemm_(mh.tiled_mma_desc(atom, cta_tile=(0, 0, 0)), T(d), T(a_m, (M, K), (1, M)), T(b_n, (N, K), (1, N)))
+            torch.cuda.synchronize()
+            assert torch.equal(d.cpu().double(), ref), (tdt, M, N, K)
+
+
 def test_config1_shape_on_the_matrix_cores(mh):
     """BASELINE config 1's operands (fp32 256^3, A and B column-major: the NN form) through the fp32 MFMA
     atom instead of UniversalFMA: tolerance 1e-5 against fp64."""

@@ -142,8 +142,10 @@ int32_t gemm_universal_dispatch(int bm, int bn, int bk, UArgs a, hipStream_t st)
     if (a.C && a.c_dt != a.d_dt)
         return fail(MOYE_ERR_UNSUPPORTED, "gemm!: C and D must have the same element type");
     if (bm == 0 && bn == 0) {
-        const bool small = (int64_t)a.M * a.N <= 512 * 512;
-        bm = bn = small ? 32 : 128;
+        // measured, fp32: 1024^3 runs at 17.4 / 8.3 / 3.7 TFLOP/s on 32 / 64 / 128 tiles, 2048^3 at 24.0 / 27.9 / 15.2,
+        // 4096^3 at 27.6 / 36.7 / 30.5 (every tile gives the same bits: k ascends strictly whatever the tile)
+        const bool small = (int64_t)a.M * a.N <= 1024 * 1024;
+        bm = bn = small ? 32 : 64;
     }
     if (bk == 0) bk = 8;
     if (bm == 32 && bn == 32 && bk == 8) return launch_u<32, 32, 8, 2, 2>(a, prod, accT, st);

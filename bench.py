@@ -24,12 +24,12 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # (the summaries are committed under profiles/), each reading scaled by what the same counter shows for the
 # 1 GiB plain copy (fetch x2.0000, write x1.0000).  Only valid for the default tile/waves/flags.
 MEASURED_TRAFFIC = {
-    "gemm_f16_4096_tile256": {"read_bytes": 197454 * 1024, "write_bytes": 33280 * 1024},
-    "transpose_f32_16384": {"read_bytes": 1048640 * 1024, "write_bytes": 1049572 * 1024},
-    "gemm_bf16_8192_tile256": {"read_bytes": 1620806 * 1024, "write_bytes": 266240 * 1024},
-    "gemm_f32_8192_tile256": {"read_bytes": 4908081 * 1024, "write_bytes": 270336 * 1024},
-    "gemm_fp8_8192_tile256": {"read_bytes": 787072 * 1024, "write_bytes": 131072 * 1024},
-    "gemm_bf16_16x8192x8192": {"read_bytes": 149534 * 1024, "write_bytes": 512 * 1024},
+    "gemm_f16_4096_tile256": {"read_bytes": 197487 * 1024, "write_bytes": 33280 * 1024},
+    "transpose_f32_16384": {"read_bytes": 1048637 * 1024, "write_bytes": 1049548 * 1024},
+    "gemm_bf16_8192_tile256": {"read_bytes": 1632408 * 1024, "write_bytes": 266240 * 1024},
+    "gemm_f32_8192_tile256": {"read_bytes": 4394669 * 1024, "write_bytes": 266240 * 1024},
+    "gemm_fp8_8192_tile256": {"read_bytes": 787037 * 1024, "write_bytes": 131072 * 1024},
+    "gemm_bf16_16x8192x8192": {"read_bytes": 149651 * 1024, "write_bytes": 512 * 1024},
 }
 
 

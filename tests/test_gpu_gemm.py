@@ -391,6 +391,43 @@ def test_library_picks_the_tile(mh):
         assert relerr(got, c64) <= TOL16
 
 
+def test_64x64_tile_exact_on_integers(mh):
+    """The 64 x 64 CTA tile (what the library picks for problems that leave CUs idle with 128 x 128): every input
+    type, both K extents per tile, C and alpha, column-major D, and the library's own choice."""
+    cases = [(mh.MFMA_F32_16x16x32_F16, torch.float16, 32), (mh.MFMA_F32_16x16x32_BF16, torch.bfloat16, 32),
+             (mh.MFMA_F32_16x16x4_F32, torch.float32, 16)]
+    if hasattr(torch, "float8_e4m3fn"):
+        cases.append((mh.MFMA_F32_16x16x32_FP8, torch.float8_e4m3fn, 64))
+    g = torch.Generator().manual_seed(64)
+    for atom, tdt, bk in cases:
+        for (M, N, K) in ((64, 64, 2 * bk), (192, 320, 256), (1024, 1024, 512)):
+            A = torch.randint(-4, 5, (M, K), generator=g).float()
+            B = torch.randint(-4, 5, (N, K), generator=g).float()
+            C = torch.randint(-9, 10, (M, N), generator=g).float()
+            a, b, c = A.to(tdt).cuda(), B.to(tdt).cuda(), C.cuda()
+            ref = A.double() @ B.double().t()
+            for cta in ((64, 64, bk), (64, 64, 2 * bk), (0, 0, 0)):
+                mma = mh.tiled_mma_desc(atom, atom_layout=(2, 2, 1), cta_tile=cta)
+                d = torch.zeros(M, N, device="cuda")
+                mh.gemm_(mma, T(d), T(a), T(b))
+                torch.cuda.synchronize()
+                assert torch.equal(d.cpu().double(), ref), (tdt, M, N, K, cta)
+                mh.gemm_(mma, T(d), T(a), T(b), T(c), 2.0)
+                torch.cuda.synchronize()
+                assert torch.equal(d.cpu().double(), 2 * ref + C.double()), (tdt, M, N, K, cta, "C")
+                dt_ = torch.zeros(N, M, device="cuda")
+                mh.gemm_(mma, T(dt_, (M, N), (1, M)), T(a), T(b))
+                torch.cuda.synchronize()
+                assert torch.equal(dt_.t().cpu().double(), ref), (tdt, M, N, K, cta, "column-major D")
+            d16 = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
+            mh.gemm_(mh.tiled_mma_desc(atom, atom_layout=(2, 2, 1), cta_tile=(64, 64, bk)), T(d16), T(a), T(b), None, 2.0 ** -6)
+            torch.cuda.synchronize()
+            assert torch.equal(d16.cpu().double(), (ref * 2.0 ** -6).to(torch.bfloat16).double()), (tdt, M, N, K, "bf16 out")
+    with pytest.raises(mh.MoyeError):          # an explicit 64 x 64 tile keeps the reference's divisibility assertion
+        x = torch.zeros(100, 64, dtype=torch.float16, device="cuda")
+        mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(64, 64, 32)), T(torch.zeros(100, 100, device="cuda")), T(x), T(x))
+
+
 def test_config4_bf16_8192(mh):
     """BASELINE config 4 (square) at full size: bf16 8192^3, fp32 accumulate and output."""
     M = N = K = 8192

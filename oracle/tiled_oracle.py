@@ -10,6 +10,13 @@ are reproduced as data because the reference's own tests and SVG fixtures are
 expressed through them (pinned by tests/test_svg_fixtures.py against the figures
 of the reference's manual); the gfx950 MFMA tables are new and are pinned on
 hardware by the one-wave atom probe test (tests/test_gpu_gemm.py).
+
+Parity unpinned in this file (the reference holds no vector for them): `copyto_if`
+(src/algorithm/copy.jl:4-16 is never called with a mask in the reference's tests;
+checked only against the element loop written out) and the printed form of
+`get_layout{A,B,C}_{MK,NK,MN}` / `get_layout{S,D}_MN` (their function values are pinned
+by the manual's figures and by inversion through the TV layouts,
+tests/test_svg_fixtures.py).
 """
 from __future__ import annotations
 

@@ -112,6 +112,17 @@ template <typename In, typename Out>
 static int32_t launch_skinny(const GemmArgs& a, hipStream_t st) {
     constexpr int W = 8;
     const dim3 block(W * 64);
+    // With K split over two or more workgroups there are enough workgroups to give each one 64 rows of B: A, which every
+    // workgroup reads whole (its K range of it), then crosses the L2-to-CU path half as often.  Pays from M = 33 on
+    // (bf16 64 x 8192 x 8192: 44.8 us with two K ranges, the second pass included, against 52.5 unsplit; M = 48: 41.3
+    // against 55.3); without the split the larger workgroup tile is slower (68.8 us).
+    if (a.split > 1 && a.M > 32 && a.N % 64 == 0 && a.N / 64 >= 128) {
+        const dim3 grid((unsigned)(a.N / 64), (unsigned)(a.split > 1 ? a.split : 1));
+        if ((a.M + 15) / 16 == 3) gemm_mfma_skinny<In, Out, 3, 4, W><<<grid, block, 0, st>>>(a);
+        else gemm_mfma_skinny<In, Out, 4, 4, W><<<grid, block, 0, st>>>(a);
+        MOYE_HIP_CHECK(hipGetLastError());
+        return MOYE_OK;
+    }
     if (a.N % 32 == 0 && a.N / 32 >= 256) {  // two B tiles per wave once that still fills the chip
         const dim3 grid((unsigned)(a.N / 32), (unsigned)(a.split > 1 ? a.split : 1));
         switch ((a.M + 15) / 16) {

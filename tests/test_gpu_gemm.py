@@ -509,7 +509,7 @@ def test_moye_array_api_on_device(mh):
 @pytest.mark.parametrize("M", [16, 32, 48, 64])
 def test_short_m_exact_on_integers(mh, M):
     g = torch.Generator().manual_seed(40 + M)
-    for (N, K) in ((256, 320), (1024, 4096), (48, 32), (8192, 288)):
+    for (N, K) in ((256, 320), (1024, 4096), (48, 32), (8192, 288), (8192, 512)):
         A = torch.randint(-4, 5, (M, K), generator=g).to(torch.float16)
         B = torch.randint(-4, 5, (N, K), generator=g).to(torch.float16)
         C = torch.randint(-8, 9, (M, N), generator=g).to(torch.float32)
@@ -525,6 +525,11 @@ def test_short_m_exact_on_integers(mh, M):
         mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(0, 0, 0)), T(d), T(a), T(b), T(c), 2.0)
         torch.cuda.synchronize()
         assert torch.equal(d.cpu().double(), 2.0 * ref + C.double()), (M, N, K, "C, alpha")
+        for split in (-1, 2):          # K ranges: from M = 33 on a workgroup then takes 64 rows of B
+            d = torch.zeros(M, N, dtype=torch.float32, device="cuda")
+            mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(0, 0, 0), split_k=split), T(d), T(a), T(b), T(c), 2.0)
+            torch.cuda.synchronize()
+            assert torch.equal(d.cpu().double(), 2.0 * ref + C.double()), (M, N, K, "split_k", split)
 
 
 @pytest.mark.parametrize("M", [1, 7, 20, 33, 63])

@@ -64,36 +64,98 @@ __global__ __launch_bounds__(256) void gemm_universal_fma(UArgs p) {
         }
 
     const bool a_kfast = p.sa_k == 1, b_kfast = p.sb_k == 1;
+    // Operand stages go global -> registers -> LDS, and the registers of stage t+1 are filled while stage t is
+    // multiplied: a small problem (few workgroups per CU) would otherwise wait out one global round trip per stage.
+    constexpr int LA = (BM * BK + 255) / 256, LB = (BN * BK + 255) / 256;
+    float ra[LA], rb[LB];
+    auto fetch = [&](int k0) {
+        const int kmax = min(BK, p.K - k0);
+#pragma unroll
+        for (int q = 0; q < LA; ++q) {
+            const int idx = tid + 256 * q;
+            const int m = a_kfast ? idx / BK : idx % BM, k = a_kfast ? idx % BK : idx / BM;
+            ra[q] = 0.0f;
+            if (idx < BM * BK && m0 + m < p.M && k < kmax) ra[q] = u_load(p.A, (int64_t)(m0 + m) * p.sa_m + (int64_t)(k0 + k) * p.sa_k, p.a_dt);
+        }
+#pragma unroll
+        for (int q = 0; q < LB; ++q) {
+            const int idx = tid + 256 * q;
+            const int n = b_kfast ? idx / BK : idx % BN, k = b_kfast ? idx % BK : idx / BN;
+            rb[q] = 0.0f;
+            if (idx < BN * BK && n0 + n < p.N && k < kmax) rb[q] = u_load(p.B, (int64_t)(n0 + n) * p.sb_n + (int64_t)(k0 + k) * p.sb_k, p.b_dt);
+        }
+    };
+    auto stash = [&]() {
+#pragma unroll
+        for (int q = 0; q < LA; ++q) {
+            const int idx = tid + 256 * q;
+            const int m = a_kfast ? idx / BK : idx % BM, k = a_kfast ? idx % BK : idx / BM;
+            if (idx < BM * BK) sA[k][m] = ra[q];
+        }
+#pragma unroll
+        for (int q = 0; q < LB; ++q) {
+            const int idx = tid + 256 * q;
+            const int n = b_kfast ? idx / BK : idx % BN, k = b_kfast ? idx % BK : idx / BN;
+            if (idx < BN * BK) sB[k][n] = rb[q];
+        }
+    };
+    auto k_step = [&](int k) {
+        float a[TM], b[TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) a[i] = sA[k][tx + TX * i];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) b[j] = sB[k][ty + TY * j];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const float prod = round_in<kProd>(__fmul_rn(a[i], b[j]));
+                acc[i][j] = round_in<kAcc>(__fadd_rn(prod, acc[i][j]));
+            }
+    };
+    if (p.K > 0) {
+        fetch(0);
+        stash();
+    }
+    __syncthreads();
     for (int k0 = 0; k0 < p.K; k0 += BK) {
         const int kmax = min(BK, p.K - k0);
-        for (int idx = tid; idx < BM * BK; idx += 256) {
-            const int m = a_kfast ? idx / BK : idx % BM, k = a_kfast ? idx % BK : idx / BM;
-            float v = 0.0f;
-            if (m0 + m < p.M && k < kmax) v = u_load(p.A, (int64_t)(m0 + m) * p.sa_m + (int64_t)(k0 + k) * p.sa_k, p.a_dt);
-            sA[k][m] = v;
-        }
-        for (int idx = tid; idx < BN * BK; idx += 256) {
-            const int n = b_kfast ? idx / BK : idx % BN, k = b_kfast ? idx % BK : idx / BN;
-            float v = 0.0f;
-            if (n0 + n < p.N && k < kmax) v = u_load(p.B, (int64_t)(n0 + n) * p.sb_n + (int64_t)(k0 + k) * p.sb_k, p.b_dt);
-            sB[k][n] = v;
-        }
-        __syncthreads();
-        for (int k = 0; k < kmax; ++k) {
-            float a[TM], b[TN];
+        const bool more = k0 + BK < p.K;
+        if (more) fetch(k0 + BK);  // in flight during the arithmetic below
+        if (kmax == BK && TM * TN <= 4) {
+            // a whole stage of a small thread tile: the fragments of eight k are read from LDS before the first product, so
+            // that one LDS latency is paid per eight k, not per k (there may be a single wave per SIMD to hide it)
 #pragma unroll
-            for (int i = 0; i < TM; ++i) a[i] = sA[k][tx + TX * i];
+            for (int kb = 0; kb < BK; kb += 8) {
+                float a[8][TM], b[8][TN];
 #pragma unroll
-            for (int j = 0; j < TN; ++j) b[j] = sB[k][ty + TY * j];
+                for (int k = 0; k < 8; ++k) {
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
+                    for (int i = 0; i < TM; ++i) a[k][i] = sA[kb + k][tx + TX * i];
 #pragma unroll
-                for (int j = 0; j < TN; ++j) {
-                    const float prod = round_in<kProd>(__fmul_rn(a[i], b[j]));
-                    acc[i][j] = round_in<kAcc>(__fadd_rn(prod, acc[i][j]));
+                    for (int j = 0; j < TN; ++j) b[k][j] = sB[kb + k][ty + TY * j];
                 }
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+#pragma unroll
+                        for (int j = 0; j < TN; ++j) {
+                            const float prod = round_in<kProd>(__fmul_rn(a[k][i], b[k][j]));
+                            acc[i][j] = round_in<kAcc>(__fadd_rn(prod, acc[i][j]));
+                        }
+            }
+        } else if (kmax == BK) {   // a whole stage: unrolled, so that the LDS reads of later k are in flight under the arithmetic
+#pragma unroll
+            for (int k = 0; k < BK; ++k) k_step(k);
+        } else {
+            for (int k = 0; k < kmax; ++k) k_step(k);
         }
-        __syncthreads();
+        __syncthreads();           // everybody is done reading this stage
+        if (more) {
+            stash();
+            __syncthreads();
+        }
     }
 
 #pragma unroll
@@ -142,12 +204,16 @@ int32_t gemm_universal_dispatch(int bm, int bn, int bk, UArgs a, hipStream_t st)
     if (a.C && a.c_dt != a.d_dt)
         return fail(MOYE_ERR_UNSUPPORTED, "gemm!: C and D must have the same element type");
     if (bm == 0 && bn == 0) {
-        // measured, fp32: 1024^3 runs at 17.4 / 8.3 / 3.7 TFLOP/s on 32 / 64 / 128 tiles, 2048^3 at 24.0 / 27.9 / 15.2,
-        // 4096^3 at 27.6 / 36.7 / 30.5 (every tile gives the same bits: k ascends strictly whatever the tile)
+        // measured, fp32: 1024^3 runs at 21.0 / 11.8 / 5.0 TFLOP/s on 32 / 64 / 128 tiles, 2048^3 at 28.0 / 36.5 / 20.3,
+        // 4096^3 at 29.9 / 39.3 / 40.1 (every tile gives the same bits: k ascends strictly whatever the tile)
         const bool small = (int64_t)a.M * a.N <= 1024 * 1024;
         bm = bn = small ? 32 : 64;
     }
     if (bk == 0) bk = 8;
+    // bK of the caller's tile is how many k the reference's kernel stages per trip; the sum over k is strictly ascending
+    // whatever that number is, so the 32 x 32 tile, which small problems use with few waves per CU, stages 32 per trip (one
+    // global round trip and one barrier pair per 32 k: fp32 256^3 17 us instead of 20, 1024^3 102 instead of 112)
+    if (bm == 32 && bn == 32 && bk == 8) return launch_u<32, 32, 32, 2, 2>(a, prod, accT, st);
     if (bm == 32 && bn == 32 && bk == 8) return launch_u<32, 32, 8, 2, 2>(a, prod, accT, st);
     if (bm == 64 && bn == 64 && bk == 8) return launch_u<64, 64, 8, 4, 4>(a, prod, accT, st);
     if (bm == 128 && bn == 128 && bk == 8) return launch_u<128, 128, 8, 8, 8>(a, prod, accT, st);

@@ -107,7 +107,8 @@ typedef struct {
                                         five-stage LDS ring (cta_tile_mnk[2] = 64 bytes of K)    */
 #define MOYE_GEMM_WAVE4 0x400         /* 256x256 tile only: four waves with 128x128 wave tiles, one
                                         per SIMD, the same five-stage ring; fp8 on the 16x16x128
-                                        MFMA (cta_tile_mnk[2] = 64 bytes of K, 128 for fp8)      */
+                                        MFMA (cta_tile_mnk[2] = 64 bytes of K, 128 for fp8; 128
+                                        bytes for f16/bf16 too: k-steps of two ring stages)      */
 
 /* copy ops: UniversalCopy (src/arch/copy/copy.jl:26-51); the LDS-staged forms stand where the
  * reference has cp.async (copy_async.jl:8-24) and ldmatrix (ldmatrix.jl:18-48) */

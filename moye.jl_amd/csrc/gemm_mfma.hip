@@ -371,14 +371,16 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         // fp8 runs at twice the 16-bit rate only on the 16x16x128 MFMA, which the hand-ordered kernel issues
         if (in_dt == MOYE_F8E4M3 && bkb == 128 && stages < 3 && !(a.xcd_swizzle & MOYE_GEMM_PINGPONG))
             a.xcd_swizzle |= MOYE_GEMM_WAVE4;
-        const int kmult = (a.xcd_swizzle & MOYE_GEMM_WAVE4) ? (in_dt == MOYE_F8E4M3 ? 128 : 64 / eb)
+        // hand-ordered kernel: k-steps of 64 bytes, or of 128 (fp8 always; the 16-bit types when the tile says so)
+        const int w4_step = in_dt == MOYE_F8E4M3 || (bkb == 128 && eb == 2) ? 128 : 64;
+        const int kmult = (a.xcd_swizzle & MOYE_GEMM_WAVE4) ? w4_step / eb
                           : (a.xcd_swizzle & MOYE_GEMM_PINGPONG) ? 64 / eb : 128 / eb;
         if (a.M % 256 || a.N % 256 || a.K % kmult)
             return fail(MOYE_ERR_SHAPE, "gemm!: CTA tile 256x256x%d does not divide the problem %dx%dx%d", kmult,
                         a.M, a.N, a.K);
         if (misaligned)
             return fail(MOYE_ERR_ALIGN, "gemm!: operands of the MFMA kernels need 16-byte aligned pointers and row pitches");
-        if (a.xcd_swizzle & MOYE_GEMM_WAVE4) return gemm_mfma_tn_256_w4_dispatch(in_dt, out_dt, a, waves, st);
+        if (a.xcd_swizzle & MOYE_GEMM_WAVE4) return gemm_mfma_tn_256_w4_dispatch(in_dt, out_dt, a, waves, w4_step, st);
         if (a.xcd_swizzle & MOYE_GEMM_PINGPONG) return gemm_mfma_tn_256_pp_dispatch(in_dt, out_dt, a, st);
         return gemm_mfma_tn_256_dispatch(in_dt, out_dt, a, waves, stages, st);
     }

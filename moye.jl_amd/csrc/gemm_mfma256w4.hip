@@ -93,6 +93,24 @@ struct W4BF16 {
         asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
     }
 };
+// The 16-bit types with k-steps of two stages (128 bytes of K): two MFMAs in a row on the same accumulator (which
+// costs nothing: 16.4 clocks per MFMA either way) and half as many barriers per K.
+struct W4F16x2 {
+    static constexpr int kBytes = 2, SPS = 2;
+    struct frag { u32x4 lo, hi; };
+    static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) {
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %3, %0\n\tv_mfma_f32_16x16x32_f16 %0, %2, %4, %0"
+                     : "+a"(c) : "v"(a.lo), "v"(a.hi), "v"(b.lo), "v"(b.hi));
+    }
+};
+struct W4BF16x2 {
+    static constexpr int kBytes = 2, SPS = 2;
+    struct frag { u32x4 lo, hi; };
+    static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) {
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %3, %0\n\tv_mfma_f32_16x16x32_bf16 %0, %2, %4, %0"
+                     : "+a"(c) : "v"(a.lo), "v"(a.hi), "v"(b.lo), "v"(b.hi));
+    }
+};
 // 32 bytes per lane: the chunk of stage 0 and the chunk of stage 1 of the k-step.  Which 32 of the
 // 128 k-values a lane carries does not matter as long as A and B agree, and they do.
 struct W4FP8 {
@@ -340,26 +358,27 @@ static int32_t launch256_w4_out(int32_t out_dt, const GemmArgs& a, hipStream_t s
 }
 
 template <int WGN>
-static int32_t launch256_w4_in(int32_t in_dt, int32_t out_dt, const GemmArgs& a, hipStream_t st) {
+static int32_t launch256_w4_in(int32_t in_dt, int32_t out_dt, const GemmArgs& a, bool two_stage_steps, hipStream_t st) {
     switch (in_dt) {
-        case MOYE_F16: return launch256_w4_out<W4F16, WGN>(out_dt, a, st);
-        case MOYE_BF16: return launch256_w4_out<W4BF16, WGN>(out_dt, a, st);
+        case MOYE_F16: return two_stage_steps ? launch256_w4_out<W4F16x2, WGN>(out_dt, a, st) : launch256_w4_out<W4F16, WGN>(out_dt, a, st);
+        case MOYE_BF16: return two_stage_steps ? launch256_w4_out<W4BF16x2, WGN>(out_dt, a, st) : launch256_w4_out<W4BF16, WGN>(out_dt, a, st);
         case MOYE_F8E4M3: return launch256_w4_out<W4FP8, WGN>(out_dt, a, st);
         case MOYE_F32: return launch256_w4_out<W4F32, WGN>(out_dt, a, st);
         default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: no MFMA atom for %s inputs", dtype_name(in_dt));
     }
 }
 
-// 256 x 256 tile, four or eight waves; K a multiple of 64 bytes (128 for fp8); the caller has checked
-// divisibility of M and N and alignment.
-int32_t gemm_mfma_tn_256_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, int waves, hipStream_t st) {
+// 256 x 256 tile, four or eight waves; K a multiple of kstep_bytes = 64 or 128 bytes (fp8: always 128; fp32: always
+// 64); the caller has checked divisibility of M and N and alignment.
+int32_t gemm_mfma_tn_256_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, int waves, int kstep_bytes, hipStream_t st) {
     a.tiles_m = a.M / 256;
     a.tiles_n = a.N / 256;
     // the load-to-LDS addresses are a uniform base plus a 32-bit lane offset
     const int eb = dtype_bytes(in_dt);
     if (256 * a.lda * eb >= (int64_t)1 << 32 || 256 * a.ldb * eb >= (int64_t)1 << 32)
         return fail(MOYE_ERR_SHAPE, "gemm!: row pitch too large for the 256x256 MFMA kernel");
-    return waves == 4 ? launch256_w4_in<2>(in_dt, out_dt, a, st) : launch256_w4_in<4>(in_dt, out_dt, a, st);
+    const bool two = kstep_bytes == 128;
+    return waves == 4 ? launch256_w4_in<2>(in_dt, out_dt, a, two, st) : launch256_w4_in<4>(in_dt, out_dt, a, two, st);
 }
 
 }  // namespace moye

@@ -322,7 +322,9 @@ def test_wave4_schedule_exact_on_integers(mh, waves):
     from moye_hip import _lib
     g = torch.Generator().manual_seed(17)
     cases = [(torch.float16, mh.MFMA_F32_16x16x32_F16, 32), (torch.bfloat16, mh.MFMA_F32_16x16x32_BF16, 32),
-             (torch.float32, mh.MFMA_F32_16x16x4_F32, 16)]
+             (torch.float32, mh.MFMA_F32_16x16x4_F32, 16),
+             # the 16-bit types with k-steps of two stages (two MFMAs in a row per accumulator)
+             (torch.float16, mh.MFMA_F32_16x16x32_F16, 64), (torch.bfloat16, mh.MFMA_F32_16x16x32_BF16, 64)]
     if hasattr(torch, "float8_e4m3fn"):
         cases.append((torch.float8_e4m3fn, mh.MFMA_F32_16x16x32_FP8, 128))
     for in_dt, atom, bk in cases:

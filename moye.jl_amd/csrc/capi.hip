@@ -195,7 +195,14 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
     const int waves = mma->atom_layout_mnk[0] * mma->atom_layout_mnk[1];
     g.alpha = alpha;
     g.K = K;
-    g.xcd_swizzle = !(mma->flags & MOYE_GEMM_NO_XCD_SWIZZLE) | (mma->flags & 0xff00) | (atom32 ? kGemmAtom32 : 0);
+    // The eight XCDs start their walk over K an eighth apart when the problem is large enough for the column blocks they
+    // ask memory for at one time to matter: more 256 x 256 tiles than CUs, or rows of 32 KiB and more (measured, 256 x 256
+    // tile, same box, alternating runs: bf16 8192^3 1408 TFLOP/s against 1372, fp16 4096 x 4096 x 16384 +4 %; fp16 4096^3
+    // 1333 against 1338, so not there)
+    static const int rotate_env = getenv("MOYE_ROTATE_K") ? atoi(getenv("MOYE_ROTATE_K")) : -1;
+    const bool rotate_k = rotate_env >= 0 ? rotate_env != 0
+                                          : ((int64_t)(M / 256) * (N / 256) > 256 || (int64_t)K * dtype_bytes(in_dt) >= 32768);
+    g.xcd_swizzle = !(mma->flags & MOYE_GEMM_NO_XCD_SWIZZLE) | (mma->flags & 0xff00) | (atom32 ? kGemmAtom32 : 0) | (rotate_k ? kGemmRotateK : 0);
     if (const int split = split_count(mma, M, N, K, dtype_bytes(in_dt)); split > 1) {
         // K is cut into `split` equal ranges, all in one launch (gridDim.y); each range writes its fp32 product, compact and
         // row-major, into the workspace; a second pass sums the ranges in ascending order, applies alpha and C and converts

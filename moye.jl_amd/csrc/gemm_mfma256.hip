@@ -118,10 +118,21 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
     }                                                                                                 \
     __builtin_amdgcn_sched_group_barrier(0x008, (MI * NI - (NV)) % (MI + NI), 0);
 
+    // Where in K this workgroup starts: the workgroups of one XCD (consecutive workgroup ids go to consecutive XCDs) walk K
+    // together, so that the panels they share are fetched into their L2 once, but the eight XCDs start an eighth of K
+    // apart, so that at any moment the chip asks memory for eight different column blocks of A and B instead of one
+    // (with K-major operands and a power-of-two pitch one column block lives in few channels).  k_of() hands out the
+    // byte offsets of successive k-tiles in that rotated order; the sum over k starts elsewhere but is the same sum.
+    int k_next = (p.xcd_swizzle & kGemmRotateK) ? (int)((int64_t)(blockIdx.x % 8) * ktiles / 8) : 0;
+    auto k_of = [&]() {
+        const int64_t off = (int64_t)k_next * 128;
+        k_next = k_next + 1 == ktiles ? 0 : k_next + 1;
+        return off;
+    };
     // prologue: tiles 0 and 1 on their way, wait for tile 0 only (LD loads per operand are younger)
-    MOYE_DMA(smem, 0)
+    { const int64_t ko = k_of(); MOYE_DMA(smem, ko) }
     if (ktiles > 1) {
-        MOYE_DMA(smem + STAGE, 128)
+        { const int64_t ko = k_of(); MOYE_DMA(smem + STAGE, ko) }
         MOYE_WAIT_BARRIER(2 * LD)
     } else {
         MOYE_WAIT_BARRIER(0)
@@ -148,7 +159,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
         __builtin_amdgcn_sched_barrier(0);                                                            \
         /* step 1: the stage tile KT lived in is free, so tile KT+2 gets a whole iteration to arrive; \
            MFMAs on buffer 1 (already in registers) while step 0 of tile KT+1 arrives in buffer 0 */  \
-        if (DMA) MOYE_DMA(cur, (int64_t)((KT) + 2) * 128)                                             \
+        if (DMA) { const int64_t ko = k_of(); MOYE_DMA(cur, ko) }                                     \
         if (NEXT) MOYE_FRAGS(nxt, 0, 0)                                                               \
         MOYE_MMA(1, 0, MI)                                                                            \
         if (NEXT) { MOYE_INTERLEAVE((DMA) ? 2 * LD : 0) }                                             \

@@ -185,9 +185,13 @@ __global__ __launch_bounds__(128 * WGN) void gemm_mfma_tn_256_w4(GemmArgs p) {
 #pragma unroll
     for (int q = 0; q < 2 * LD; ++q)
         voff[q] = (uint32_t)((lrow + 16 * (q % LD)) * (q < LD ? pitch_a : pitch_b) + lch * 16);
+    // stage g of this workgroup's walk over K is stage g + g0 (mod nstages) of the operands: the eight XCDs start an
+    // eighth of K apart when the caller asks for it (see gemm_mfma256.hip)
+    const int g0 = (p.xcd_swizzle & kGemmRotateK) ? (int)((int64_t)(blockIdx.x % 8) * nsteps / 8) * SPS : 0;
     auto dma1 = [&](int g, int ring_slot, auto qc) __attribute__((always_inline)) {
         constexpr int Q = decltype(qc)::value;
-        const char* const base = uniform_ptr((Q < LD ? a_tile : b_tile) + (int64_t)g * 64);
+        const int gr = g + g0 >= nstages ? g + g0 - nstages : g + g0;
+        const char* const base = uniform_ptr((Q < LD ? a_tile : b_tile) + (int64_t)gr * 64);
         const uint32_t dst = __builtin_amdgcn_readfirstlane(lds0 + ring_slot * kStageBytes + (Q < LD ? 0 : kATileBytes) +
                                                             (uint32_t)(wave * RW + 16 * (Q % LD)) * 64);
         const uint32_t lane_off = voff[Q];  // (a captured array element cannot be an asm operand of a generic lambda)

@@ -22,7 +22,8 @@ struct GemmArgs {
     int64_t split_ab, split_d;
     int xcd_swizzle;  // bit 0: XCD-aware tile order; bits 8-15: MOYE_GEMM_* schedule flags; kGemmAtom32
 };
-constexpr int kGemmAtom32 = 0x10000;  // in GemmArgs::xcd_swizzle: issue the 32x32 MFMA forms
+constexpr int kGemmAtom32 = 0x10000;   // in GemmArgs::xcd_swizzle: issue the 32x32 MFMA forms
+constexpr int kGemmRotateK = 0x20000;  // in GemmArgs::xcd_swizzle: each XCD starts its walk over K at its own eighth
 
 // UniversalFMA GEMM, any strides (gemm_universal.hip)
 struct UArgs {

@@ -202,7 +202,18 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
     static const int rotate_env = getenv("MOYE_ROTATE_K") ? atoi(getenv("MOYE_ROTATE_K")) : -1;
     const bool rotate_k = rotate_env >= 0 ? rotate_env != 0
                                           : ((int64_t)(M / 256) * (N / 256) > 256 || (int64_t)K * dtype_bytes(in_dt) >= 32768);
-    g.xcd_swizzle = !(mma->flags & MOYE_GEMM_NO_XCD_SWIZZLE) | (mma->flags & 0xff00) | (atom32 ? kGemmAtom32 : 0) | (rotate_k ? kGemmRotateK : 0);
+    static const int stream_env = getenv("MOYE_STREAM_D") ? atoi(getenv("MOYE_STREAM_D")) : -1;
+    // D written with non-temporal stores (measured, same box, alternating runs, ordinary -> non-temporal, TFLOP/s): fp16
+    // 4096^3 fp16 out 1339 -> 1345, fp32 out 1285 -> 1253; fp16 8192^3 fp16 out 1382 -> 1401; bf16 8192^3 fp32 out 1412 ->
+    // 1452; fp8 4096^3 bf16 out 2373 -> 2450, 8192^3 2760 -> 2745; fp16 2048^3 and 3072^3 +1.6 %.  So: 16-bit results
+    // always, except for the fp8 kernel on more tiles than CUs; 32-bit results when the launch has more 256 x 256 tiles
+    // than the chip has CUs (then the results of one round would sit in the L2s in place of the next round's operands;
+    // in a single round they are better left there for the end of the kernel to write back)
+    const bool many_tiles = (int64_t)(M / 256) * (N / 256) > 256;
+    const bool stream_d = stream_env >= 0 ? stream_env != 0
+                          : dtype_bytes(D.dtype) == 2 ? !(in_dt == MOYE_F8E4M3 && many_tiles) : many_tiles;
+    g.xcd_swizzle = !(mma->flags & MOYE_GEMM_NO_XCD_SWIZZLE) | (mma->flags & 0xff00) | (atom32 ? kGemmAtom32 : 0) | (rotate_k ? kGemmRotateK : 0) |
+                    (stream_d ? kGemmStreamD : 0);
     if (const int split = split_count(mma, M, N, K, dtype_bytes(in_dt)); split > 1) {
         // K is cut into `split` equal ranges, all in one launch (gridDim.y); each range writes its fp32 product, compact and
         // row-major, into the workspace; a second pass sums the ranges in ascending order, applies alpha and C and converts
@@ -215,6 +226,7 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
         g.alpha = 1.f; g.K = Ks; g.M = M; g.N = N; g.lda = A.rs; g.ldb = B.rs; g.ldd = N; g.C = nullptr;
         g.A = A.ptr; g.B = B.ptr; g.D = P;
         g.split = split; g.split_ab = (int64_t)Ks * eb; g.split_d = (int64_t)M * N * (int64_t)sizeof(float);
+        g.xcd_swizzle &= ~kGemmStreamD;  // the partial products are read back at once
         if (int32_t e = gemm_mfma_tn_dispatch(in_dt, MOYE_F32, bm, bn, bk, waves, mma->stages, g, st)) return e;
         return splitk_reduce_dispatch(P, split, M, N, alpha, tC ? C.ptr : nullptr, C.rs, C.cs, D.ptr, D.rs, D.cs, D.dtype, st);
     }

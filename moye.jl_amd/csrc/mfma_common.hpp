@@ -126,6 +126,16 @@ __device__ __forceinline__ void split_of_block(GemmArgs& p) {
     }
 }
 
+// One 16-byte piece of D.  With kGemmStreamD in GemmArgs::xcd_swizzle the store is non-temporal: when a launch has
+// more tiles than the chip has CUs, results written the ordinary way sit in the L2s and push out the operand panels
+// the next tiles are about to share.
+__device__ __forceinline__ void store_d_chunk(const GemmArgs& p, char* d, const u32x4& w) {
+    // (as text: the compiler merges an ordinary and a non-temporal store in the two arms of a branch into one ordinary
+    // store; the nop covers the wait states a wide store needs before its data registers are written again)
+    if (p.xcd_swizzle & kGemmStreamD) asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 1" ::"v"(d), "v"(w) : "memory");
+    else *reinterpret_cast<u32x4*>(d) = w;
+}
+
 // blockIdx -> (tile_m, tile_n).  Hardware deals consecutive workgroup ids round-robin to the 8
 // XCDs; remapping id -> (id % 8) * (n / 8) + id / 8 hands each XCD one contiguous run of tiles,
 // and inside a run tiles are walked in bands of 8 tile-rows so that the A and B panels an

@@ -51,7 +51,7 @@ __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&ac
             const u32x4 w = patch16[row * CR + (ch ^ (row & 7))];
             char* d = static_cast<char*>(p.D) +
                       ((m_base + 16 * i0 + row) * p.ldd + n_base) * (int64_t)sizeof(OutT) + ch * 16;
-            *reinterpret_cast<u32x4*>(d) = w;
+            store_d_chunk(p, d, w);
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();

@@ -148,7 +148,10 @@ int32_t moye_copy_if(const moye_tensor* dst, const moye_tensor* src, const moye_
  * (test/device/matmul.jl:3-53, docs/src/manual/tensor_core.md:265-355):
  * A:(M,K), B:(N,K), C,D:(M,N);  D = alpha * (A * B') + C.   C may be NULL (zero-init
  * accumulator, `zeros!(tCrC)`); D may alias C.  With MOYE_MMA_UNIVERSAL_FMA the arithmetic is
- * the reference's exactly (product rounded in the input type, unfused add, k ascending). */
+ * the reference's exactly (product rounded in the input type, unfused add, k ascending).
+ * Environment, read once per process, for tuning only (no result bit changes): MOYE_ROTATE_K=0|1 forces
+ * whether the XCDs start their walk over K an eighth apart, MOYE_STREAM_D=0|1 whether D is written with
+ * non-temporal stores; unset, the library decides by problem size and result type. */
 int32_t moye_gemm(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A,
                   const moye_tensor* B, const moye_tensor* C, float alpha, void* stream);
 

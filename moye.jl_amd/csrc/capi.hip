@@ -133,6 +133,11 @@ static int32_t make_kmajor(Mat* m, char* ws, hipStream_t st) {
     return MOYE_OK;
 }
 
+// C as the 256 x 256 kernels' epilogue likes it: unit stride along the kernel's n, rows that start on 16-byte boundaries
+static bool rows_in_16_byte_pieces(const void* c, int64_t ld_m, int64_t ld_n, int32_t dt) {
+    return c && ld_n == 1 && reinterpret_cast<uintptr_t>(c) % 16 == 0 && (ld_m * dtype_bytes(dt)) % 16 == 0;
+}
+
 static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const moye_tensor* tA,
                          const moye_tensor* tB, const moye_tensor* tC, float alpha, hipStream_t st) {
     if (!mma) return fail(MOYE_ERR_ARG, "gemm!: null TiledMMA descriptor");
@@ -233,6 +238,7 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
     if (D.cs == 1) {  // row-major D
         g.A = A.ptr; g.B = B.ptr; g.M = M; g.N = N; g.lda = A.rs; g.ldb = B.rs; g.ldd = D.rs;
         g.C = tC ? C.ptr : nullptr; g.ldc_m = C.rs; g.ldc_n = C.cs; g.D = D.ptr;
+        if (rows_in_16_byte_pieces(g.C, g.ldc_m, g.ldc_n, D.dtype)) g.xcd_swizzle |= kGemmRowC;
         return gemm_mfma_tn_dispatch(in_dt, D.dtype, bm, bn, bk, waves, mma->stages, g, st);
     }
     if (D.rs == 1 && bm == 0 && bn == 0 && M <= 64 && ((int64_t)K * dtype_bytes(in_dt)) % 64 == 0) {
@@ -244,6 +250,7 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
     if (D.rs == 1) {  // column-major D: D' = B * A' is row-major
         g.A = B.ptr; g.B = A.ptr; g.M = N; g.N = M; g.lda = B.rs; g.ldb = A.rs; g.ldd = D.cs;
         g.C = tC ? C.ptr : nullptr; g.ldc_m = C.cs; g.ldc_n = C.rs; g.D = D.ptr;
+        if (rows_in_16_byte_pieces(g.C, g.ldc_m, g.ldc_n, D.dtype)) g.xcd_swizzle |= kGemmRowC;
         return gemm_mfma_tn_dispatch(in_dt, D.dtype, bn, bm, bk, waves, mma->stages, g, st);
     }
     return fail(MOYE_ERR_UNSUPPORTED, "gemm!: D needs a unit stride along M or N");

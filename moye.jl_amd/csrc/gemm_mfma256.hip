@@ -20,7 +20,7 @@
 //
 // Same operand conventions as gemm_mfma.hip: K-major A and B, N-contiguous D, the MFMA issued
 // with B rows as its first operand so a lane holds four consecutive n of one m.
-#include "mfma_common.hpp"
+#include "mfma_epilogue.hpp"
 
 namespace moye {
 
@@ -32,7 +32,6 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
     constexpr int WROWS = BM / NWAVES;  // operand rows each wave brings in per tile
     constexpr int LD = WROWS / 8;       // load-to-LDS instructions per wave per operand (8 rows each)
     constexpr int WM = BM / WGM, WN = BN / WGN, MI = WM / 16, NI = WN / 16;
-    typedef typename Out::type OutT;
 
     extern __shared__ u32x4 smem[];
 
@@ -181,52 +180,9 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
 #undef MOYE_MMA
     __syncthreads();  // every wave is done with the operand stages before they become C patches
 
-    // ---- epilogue: alpha*acc + C -> OutT -> this wave's LDS patch -> 128-bit row stores ----
-    // lane holds C[m = 16 i + r16][n = 16 j + 4 kq + e], e = 0..3
-    const int64_t m_base = (int64_t)tm * BM + wm0, n_base = (int64_t)tn * BN + wn0;
-    constexpr int EPC = 16 / (int)sizeof(OutT);  // elements per 16-byte chunk
-    constexpr int CR = WN / EPC;                 // chunks per patch row
-    constexpr int PASS_MI = 2, PASS_ROWS = PASS_MI * 16;
-    static_assert(NWAVES * PASS_ROWS * WN * 4 <= 2 * STAGE * 16, "C patches fit in the operand stages");
-    OutT* patch = reinterpret_cast<OutT*>(smem) + wave * (PASS_ROWS * WN);
-    u32x4* patch16 = reinterpret_cast<u32x4*>(patch);
-
-#pragma unroll
-    for (int i0 = 0; i0 < MI; i0 += PASS_MI) {
-#pragma unroll
-        for (int ii = 0; ii < PASS_MI; ++ii) {
-            const int i = i0 + ii;
-#pragma unroll
-            for (int j = 0; j < NI; ++j) {
-                float v[4] = {acc[i][j].x * p.alpha, acc[i][j].y * p.alpha, acc[i][j].z * p.alpha,
-                              acc[i][j].w * p.alpha};
-                if (p.C) {
-                    const int64_t m = m_base + 16 * i + r16, n = n_base + 16 * j + 4 * kq;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) v[e] += Out::load(p.C, m * p.ldc_m + (n + e) * p.ldc_n);
-                }
-                const int row = 16 * ii + r16, col = 16 * j + 4 * kq;
-                const int chunk = col / EPC, within = col % EPC;
-                OutT* dst = patch + (row * CR + (chunk ^ (row & 7))) * EPC + within;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) dst[e] = Out::cvt(v[e]);
-            }
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-        for (int t = 0; t < PASS_ROWS * CR / 64; ++t) {
-            const int c = lane + 64 * t, row = c / CR, ch = c % CR;
-            const u32x4 w = patch16[row * CR + (ch ^ (row & 7))];
-            char* d = static_cast<char*>(p.D) +
-                      ((m_base + 16 * i0 + row) * p.ldd + n_base) * (int64_t)sizeof(OutT) + ch * 16;
-            store_d_chunk(p, d, w);
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    }
+    // --- epilogue (mfma_epilogue.hpp): alpha*acc + C -> OutT -> this wave's LDS patch -> 128-bit row stores
+    static_assert(NWAVES * 32 * WN * 4 <= 2 * STAGE * 16, "C patches (32 rows per wave and pass) fit in the operand stages");
+    store_c_tile<Out, MI, NI>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -246,7 +202,6 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256_ring(GemmArgs
     constexpr int LD = WROWS / 16;      // load-to-LDS instructions per wave per operand (16 rows each)
     constexpr int WM = BM / WGM, WN = BN / WGN, MI = WM / 16, NI = WN / 16;
     static_assert(LD >= 1 && STAGES >= 3, "ring shape");
-    typedef typename Out::type OutT;
 
     extern __shared__ u32x4 smem[];
 
@@ -341,50 +296,9 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256_ring(GemmArgs
 #undef MOYE_STEP
     __syncthreads();  // every wave is done with the operand ring before it becomes C patches
 
-    // ---- epilogue: alpha*acc + C -> OutT -> this wave's LDS patch -> 128-bit row stores ----
-    const int64_t m_base = (int64_t)tm * BM + wm0, n_base = (int64_t)tn * BN + wn0;
-    constexpr int EPC = 16 / (int)sizeof(OutT);
-    constexpr int CR = WN / EPC;
-    constexpr int PASS_MI = 2, PASS_ROWS = PASS_MI * 16;
-    static_assert(NWAVES * PASS_ROWS * WN * 4 <= STAGES * STAGE * 16, "C patches fit in the operand ring");
-    OutT* patch = reinterpret_cast<OutT*>(smem) + wave * (PASS_ROWS * WN);
-    u32x4* patch16 = reinterpret_cast<u32x4*>(patch);
-#pragma unroll
-    for (int i0 = 0; i0 < MI; i0 += PASS_MI) {
-#pragma unroll
-        for (int ii = 0; ii < PASS_MI; ++ii) {
-            const int i = i0 + ii;
-#pragma unroll
-            for (int j = 0; j < NI; ++j) {
-                float v[4] = {acc[i][j].x * p.alpha, acc[i][j].y * p.alpha, acc[i][j].z * p.alpha,
-                              acc[i][j].w * p.alpha};
-                if (p.C) {
-                    const int64_t m = m_base + 16 * i + r16, n = n_base + 16 * j + 4 * kq;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) v[e] += Out::load(p.C, m * p.ldc_m + (n + e) * p.ldc_n);
-                }
-                const int row = 16 * ii + r16, col = 16 * j + 4 * kq;
-                const int chunk = col / EPC, within = col % EPC;
-                OutT* dst = patch + (row * CR + (chunk ^ (row & 7))) * EPC + within;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) dst[e] = Out::cvt(v[e]);
-            }
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-        for (int t = 0; t < PASS_ROWS * CR / 64; ++t) {
-            const int c = lane + 64 * t, row = c / CR, ch = c % CR;
-            const u32x4 w = patch16[row * CR + (ch ^ (row & 7))];
-            char* d = static_cast<char*>(p.D) +
-                      ((m_base + 16 * i0 + row) * p.ldd + n_base) * (int64_t)sizeof(OutT) + ch * 16;
-            store_d_chunk(p, d, w);
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    }
+    // --- epilogue (mfma_epilogue.hpp): alpha*acc + C -> OutT -> this wave's LDS patch -> 128-bit row stores
+    static_assert(NWAVES * 32 * WN * 4 <= STAGES * STAGE * 16, "C patches (32 rows per wave and pass) fit in the operand ring");
+    store_c_tile<Out, MI, NI>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
 }
 
 template <typename In, typename Out, int STAGES>

@@ -23,6 +23,7 @@ struct GemmArgs {
     int xcd_swizzle;  // bit 0: XCD-aware tile order; bits 8-15: MOYE_GEMM_* schedule flags; kGemmAtom32
 };
 constexpr int kGemmAtom32 = 0x10000;   // in GemmArgs::xcd_swizzle: issue the 32x32 MFMA forms
+constexpr int kGemmRowC = 0x80000;    // in GemmArgs::xcd_swizzle: C has unit stride along n, 16-byte aligned rows: read in 128-bit pieces
 constexpr int kGemmStreamD = 0x40000;  // in GemmArgs::xcd_swizzle: D is written with non-temporal stores
 constexpr int kGemmRotateK = 0x20000;  // in GemmArgs::xcd_swizzle: each XCD starts its walk over K at its own eighth
 

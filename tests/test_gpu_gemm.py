@@ -1012,3 +1012,43 @@ def test_large_offsets_gemm_and_transpose(mh):
     sv, dv = src.view(Cn, R), dst.view(R, Cn)
     for (i, j) in ((0, 0), (R - 64, Cn - 64), (40000, 17000), (65000, 100)):
         assert torch.equal(dv[i:i + 64, j:j + 64], sv[j:j + 64, i:i + 64].t()), (i, j)
+
+
+@pytest.mark.parametrize("out_dt", ["float32", "float16", "bfloat16"])
+@pytest.mark.parametrize("flags", ["default", "wave4"])
+def test_256_tile_every_layout_of_c(mh, out_dt, flags):
+    """C through the 256x256 kernels' epilogue: row-major with aligned rows (read in 128-bit pieces of whole rows),
+    a row pitch and a base that are not multiples of 16 bytes, column-major, and D itself (in place).  Small integers:
+    every result is exact, so a misplaced piece of C shows as a hard mismatch."""
+    from moye_hip import _lib
+    out_dt = getattr(torch, out_dt)
+    M, N, K = 512, 768, 256
+    g = torch.Generator().manual_seed(77)
+    A = torch.randint(-3, 4, (M, K), generator=g).to(torch.float16)
+    B = torch.randint(-3, 4, (N, K), generator=g).to(torch.float16)
+    C0 = torch.randint(-8, 9, (M, N), generator=g).to(out_dt)
+    a, b = A.cuda(), B.cuda()
+    mma = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 4, 1), cta_tile=(256, 256, 64),
+                            flags=_lib.GEMM_WAVE4 if flags == "wave4" else 0)
+    want = (A.double() @ B.double().t()) * 0.5 + C0.double()
+    if out_dt != torch.float32:
+        want = want.to(out_dt).double()  # halves of odd sums round to even in the 16-bit types
+    forms = {}
+    forms["rows"] = (C0.cuda(), (N, 1), 0)
+    padded = torch.zeros(M, N + 1, dtype=out_dt)
+    padded[:, :N] = C0
+    forms["pitch N + 1"] = (padded.cuda(), (N + 1, 1), 0)
+    shifted = torch.zeros(M * N + 1, dtype=out_dt)
+    shifted[1:] = C0.reshape(-1)
+    forms["base off by one element"] = (shifted.cuda(), (N, 1), 1)
+    forms["column-major"] = (C0.t().contiguous().cuda(), (1, M), 0)
+    for name, (c, strides, off) in forms.items():
+        d = torch.zeros(M, N, dtype=out_dt, device="cuda")
+        cc = T(c.reshape(-1)[off:], (M, N), strides)
+        mh.gemm_(mma, T(d), T(a), T(b), cc, 0.5)
+        torch.cuda.synchronize()
+        assert torch.equal(d.cpu().double(), want), name
+    d = C0.cuda().clone()
+    mh.gemm_(mma, T(d), T(a), T(b), T(d), 0.5)
+    torch.cuda.synchronize()
+    assert torch.equal(d.cpu().double(), want), "in place"

@@ -188,9 +188,34 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
     constexpr int PASS_ROWS = PASS_MI * AT;
     OutT* patch = reinterpret_cast<OutT*>(smem) + wave * (PASS_ROWS * WN);
     u32x4* patch16 = reinterpret_cast<u32x4*>(patch);
+    // C with unit stride along n and 16-byte aligned rows (kGemmRowC) is read the way D is written, in 128-bit pieces
+    // of whole rows, all requested up front, and handed to the lanes through the patch (see mfma_epilogue.hpp)
+    constexpr int NCH = PASS_ROWS * CR / 64, PASSES = MI / PASS_MI;
+    const bool row_c = p.C && (p.xcd_swizzle & kGemmRowC);
+    u32x4 cw[PASSES][NCH];
+    if (row_c) {
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ++ps)
+#pragma unroll
+            for (int t = 0; t < NCH; ++t) {
+                const int c = lane + 64 * t, row = c / CR, ch = c % CR;
+                cw[ps][t] = *reinterpret_cast<const u32x4*>(static_cast<const char*>(p.C) +
+                                                            ((m_base + PASS_ROWS * ps + row) * p.ldc_m + n_base) * (int64_t)sizeof(OutT) + ch * 16);
+            }
+    }
 
 #pragma unroll
     for (int i0 = 0; i0 < MI; i0 += PASS_MI) {
+        if (row_c) {
+#pragma unroll
+            for (int t = 0; t < NCH; ++t) {
+                const int c = lane + 64 * t, row = c / CR, ch = c % CR;
+                patch16[row * CR + (ch ^ (row & (CR - 1)))] = cw[i0 / PASS_MI][t];
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
 #pragma unroll
         for (int ii = 0; ii < PASS_MI; ++ii) {
             const int i = i0 + ii;
@@ -201,14 +226,17 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
                     float v[4];
 #pragma unroll
                     for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * g + e] * p.alpha;
-                    if (p.C) {
+                    const int row = AT * ii + r16, col = AT * j + 8 * g + 4 * kq;
+                    const int chunk = col / EPC, within = col % EPC;
+                    OutT* dst = patch + (row * CR + (chunk ^ (row & (CR - 1)))) * EPC + within;
+                    if (row_c) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] += Out::load(dst, e);
+                    } else if (p.C) {
                         const int64_t m = m_base + AT * i + r16, n = n_base + AT * j + 8 * g + 4 * kq;
 #pragma unroll
                         for (int e = 0; e < 4; ++e) v[e] += Out::load(p.C, m * p.ldc_m + (n + e) * p.ldc_n);
                     }
-                    const int row = AT * ii + r16, col = AT * j + 8 * g + 4 * kq;
-                    const int chunk = col / EPC, within = col % EPC;
-                    OutT* dst = patch + (row * CR + (chunk ^ (row & (CR - 1)))) * EPC + within;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) dst[e] = Out::cvt(v[e]);
                 }

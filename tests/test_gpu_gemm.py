@@ -1015,9 +1015,9 @@ def test_large_offsets_gemm_and_transpose(mh):
 
 
 @pytest.mark.parametrize("out_dt", ["float32", "float16", "bfloat16"])
-@pytest.mark.parametrize("flags", ["default", "wave4"])
-def test_256_tile_every_layout_of_c(mh, out_dt, flags):
-    """C through the 256x256 kernels' epilogue: row-major with aligned rows (read in 128-bit pieces of whole rows),
+@pytest.mark.parametrize("flags", ["default", "wave4", "128", "64", "128 atom32"])
+def test_every_layout_of_c(mh, out_dt, flags):
+    """C through the MFMA kernels' epilogues (256x256 tile, lock-step and hand-ordered; 128x128; 64x64; 32x32 atoms): row-major with aligned rows (read in 128-bit pieces of whole rows),
     a row pitch and a base that are not multiples of 16 bytes, column-major, and D itself (in place).  Small integers:
     every result is exact, so a misplaced piece of C shows as a hard mismatch."""
     from moye_hip import _lib
@@ -1028,8 +1028,13 @@ def test_256_tile_every_layout_of_c(mh, out_dt, flags):
     B = torch.randint(-3, 4, (N, K), generator=g).to(torch.float16)
     C0 = torch.randint(-8, 9, (M, N), generator=g).to(out_dt)
     a, b = A.cuda(), B.cuda()
-    mma = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 4, 1), cta_tile=(256, 256, 64),
-                            flags=_lib.GEMM_WAVE4 if flags == "wave4" else 0)
+    if flags in ("default", "wave4"):
+        mma = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 4, 1), cta_tile=(256, 256, 64),
+                                flags=_lib.GEMM_WAVE4 if flags == "wave4" else 0)
+    elif flags == "128 atom32":
+        mma = mh.tiled_mma_desc(mh.MFMA_F32_32x32x16_F16, atom_layout=(2, 2, 1), cta_tile=(128, 128, 32))
+    else:
+        mma = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 2, 1), cta_tile=(int(flags), int(flags), 64))
     want = (A.double() @ B.double().t()) * 0.5 + C0.double()
     if out_dt != torch.float32:
         want = want.to(out_dt).double()  # halves of odd sums round to even in the 16-bit types

@@ -736,6 +736,11 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
 
     // (3) generic
     FlatLayout ls = flat_of(*src), ld = flat_of(*dst);
+    // same shape mode by mode: visit the coordinates along the destination's smallest strides first (then the source's)
+    {
+        FlatLayout* all[3] = {&ld, &ls, mask ? &mk.l : nullptr};
+        order_modes_by_stride(all, mask ? 3 : 2);
+    }
     if (same_bits && !mask) {
         // Vectorise when the layouts allow it, which the reference computes (max_common_vector,
         // src/layout.jl:752-761) and then leaves unused (src/algorithm/copy.jl:53-58): if logical

@@ -277,6 +277,86 @@ __global__ __launch_bounds__(256) void fill_dense_kernel(u32x4* x, int64_t nvec,
         x[i] = pattern;
 }
 
+// ---- rows of 16-byte pieces -----------------------------------------------------------------------------------
+// Arrays that are not one run but whose first mode (after the modes were ordered by stride) has unit stride on every
+// side, in whole aligned 16-byte pieces: the layouts are recast to 16-byte elements (first extent and every other
+// stride divided by the piece's element count) and each lane takes one piece per operand, with the arithmetic of the
+// general kernels.
+template <typename El>
+__global__ __launch_bounds__(256) void axpby_rows_kernel(typename El::compute a, const typename El::storage* x, ELayout lx,
+                                                         typename El::compute b, typename El::storage* y, ELayout ly, int64_t nvec,
+                                                         bool b_is_zero) {
+    typedef typename El::compute T;
+    typedef typename El::storage S;
+    typedef typename DenseVec<El>::type vec;
+    constexpr int N = DenseVec<El>::N;
+    const vec* xv = reinterpret_cast<const vec*>(x);
+    vec* yv = reinterpret_cast<vec*>(y);
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256) {
+        const vec vx = xv[e_offset(lx, i)];
+        vec* py = yv + e_offset(ly, i);
+        const vec vy = b_is_zero ? vx : *py;
+        vec r;
+#pragma unroll
+        for (int k = 0; k < N; ++k) {
+            S ex = vx[k], ey = vy[k], er;
+            const T ax = El::round(a * El::load(&ex));
+            if (b_is_zero) El::store(&er, ax);
+            else El::store(&er, El::round(ax + El::round(b * El::load(&ey))));
+            r[k] = er;
+        }
+        *py = r;
+    }
+}
+
+template <typename El>
+__global__ __launch_bounds__(256) void map_rows_kernel(int32_t op, typename El::storage* d, ELayout ld, const typename El::storage* a,
+                                                       ELayout la, const typename El::storage* b, ELayout lb, typename El::compute s,
+                                                       int64_t nvec) {
+    typedef typename El::compute T;
+    typedef typename El::storage S;
+    typedef typename DenseVec<El>::type vec;
+    constexpr int N = DenseVec<El>::N;
+    const vec* av = reinterpret_cast<const vec*>(a);
+    const vec* bv = reinterpret_cast<const vec*>(b);
+    vec* dv = reinterpret_cast<vec*>(d);
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256) {
+        const vec va = av[e_offset(la, i)];
+        const vec vb = b ? bv[e_offset(lb, i)] : va;
+        vec r;
+#pragma unroll
+        for (int k = 0; k < N; ++k) {
+            S ea = va[k], eb = vb[k], er;
+            const T x = El::load(&ea);
+            const T y = b ? El::load(&eb) : s;
+            El::store(&er, El::round(map_op(op, x, y)));
+            r[k] = er;
+        }
+        dv[e_offset(ld, i)] = r;
+    }
+}
+
+__global__ __launch_bounds__(256) void fill_rows_kernel(u32x4* x, ELayout lx, int64_t nvec, u32x4 pattern) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256) x[e_offset(lx, i)] = pattern;
+}
+
+// Can every one of these (same-shape, stride-ordered) layouts be recast to pieces of `per` elements?  If so, does it.
+bool recast_rows(ELayout* const* ls, const void* const* ptrs, int count, int per) {
+    if (per <= 1) return false;
+    for (int q = 0; q < count; ++q) {
+        const ELayout& l = *ls[q];
+        if (l.rank < 1 || l.stride[0] != 1 || l.shape[0] % per || reinterpret_cast<uintptr_t>(ptrs[q]) % 16) return false;
+        for (int m = 1; m < l.rank; ++m)
+            if (l.shape[m] != 1 && l.stride[m] % per) return false;
+    }
+    for (int q = 0; q < count; ++q) {
+        ELayout& l = *ls[q];
+        l.shape[0] /= per;
+        for (int m = 1; m < l.rank; ++m) l.stride[m] /= per;
+    }
+    return true;
+}
+
 // one run in logical order?
 bool dense(const moye_tensor& t) {
     int64_t expect = 1;
@@ -319,11 +399,16 @@ float host_round_bf16(float f) {
 
 template <typename El>
 static void launch_axpby(typename El::compute a, const void* x, const ELayout& lx, typename El::compute b, void* y, const ELayout& ly,
-                         int64_t n, bool is_dense, hipStream_t st) {
+                         int64_t n, bool is_dense, bool rows, hipStream_t st) {
     typedef typename El::storage S;
     const S* xs = static_cast<const S*>(x);
     S* ys = static_cast<S*>(y);
     const bool b0 = b == (typename El::compute)0;
+    if (!is_dense && rows) {  // lx, ly are in 16-byte pieces
+        const int64_t nvec = n / DenseVec<El>::N;
+        axpby_rows_kernel<El><<<dim3((unsigned)std::min<int64_t>((nvec + 255) / 256, 256 * 16)), 256, 0, st>>>(a, xs, lx, b, ys, ly, nvec, b0);
+        return;
+    }
     if (!is_dense) {
         const dim3 grid((unsigned)std::min<int64_t>((n + 255) / 256, 256 * 16));
         axpby_kernel<El><<<grid, 256, 0, st>>>(a, xs, lx, b, ys, ly, n, b0);
@@ -337,11 +422,16 @@ static void launch_axpby(typename El::compute a, const void* x, const ELayout& l
 
 template <typename El>
 static void launch_map(int32_t op, void* d, const ELayout& ld, const void* a, const ELayout& la, const void* b, const ELayout& lb,
-                       int64_t nb, typename El::compute s, int64_t n, bool is_dense, hipStream_t st) {
+                       int64_t nb, typename El::compute s, int64_t n, bool is_dense, bool rows, hipStream_t st) {
     typedef typename El::storage S;
     S* ds = static_cast<S*>(d);
     const S* as = static_cast<const S*>(a);
     const S* bs = static_cast<const S*>(b);
+    if (!is_dense && rows) {  // ld, la, lb are in 16-byte pieces
+        const int64_t nvec = n / DenseVec<El>::N;
+        map_rows_kernel<El><<<dim3((unsigned)std::min<int64_t>((nvec + 255) / 256, 256 * 16)), 256, 0, st>>>(op, ds, ld, as, la, bs, lb, s, nvec);
+        return;
+    }
     if (!is_dense) {
         const dim3 grid((unsigned)std::min<int64_t>((n + 255) / 256, 256 * 16));
         map_kernel<El><<<grid, 256, 0, st>>>(op, ds, ld, as, la, bs, lb, nb, s, n);
@@ -362,13 +452,19 @@ int32_t axpby_dispatch(double a, const moye_tensor* X, double b, const moye_tens
     const int64_t n = count(*X);
     if (count(*Y) != n) return fail(MOYE_ERR_SHAPE, "axpby!: X holds %lld elements, Y %lld", (long long)n, (long long)count(*Y));
     if (n == 0) return MOYE_OK;
-    const ELayout lx = elayout_of(*X), ly = elayout_of(*Y);
+    ELayout lx = elayout_of(*X), ly = elayout_of(*Y);
     const bool fast = dense(*X) && dense(*Y) && aligned16(X->ptr) && aligned16(Y->ptr);
+    bool rows = false;
+    if (!fast) {
+        ELayout* all[2] = {&ly, &lx};
+        const void* ptrs[2] = {Y->ptr, X->ptr};
+        rows = order_modes_by_stride(all, 2) && recast_rows(all, ptrs, 2, 16 / dtype_bytes(X->dtype));
+    }
     switch (X->dtype) {
-        case MOYE_F32: launch_axpby<ElF32>((float)a, X->ptr, lx, (float)b, Y->ptr, ly, n, fast, st); break;
-        case MOYE_F64: launch_axpby<ElF64>(a, X->ptr, lx, b, Y->ptr, ly, n, fast, st); break;
-        case MOYE_F16: launch_axpby<ElF16>(host_round_f16((float)a), X->ptr, lx, host_round_f16((float)b), Y->ptr, ly, n, fast, st); break;
-        case MOYE_BF16: launch_axpby<ElBF16>(host_round_bf16((float)a), X->ptr, lx, host_round_bf16((float)b), Y->ptr, ly, n, fast, st); break;
+        case MOYE_F32: launch_axpby<ElF32>((float)a, X->ptr, lx, (float)b, Y->ptr, ly, n, fast, rows, st); break;
+        case MOYE_F64: launch_axpby<ElF64>(a, X->ptr, lx, b, Y->ptr, ly, n, fast, rows, st); break;
+        case MOYE_F16: launch_axpby<ElF16>(host_round_f16((float)a), X->ptr, lx, host_round_f16((float)b), Y->ptr, ly, n, fast, rows, st); break;
+        case MOYE_BF16: launch_axpby<ElBF16>(host_round_bf16((float)a), X->ptr, lx, host_round_bf16((float)b), Y->ptr, ly, n, fast, rows, st); break;
         default:
             return fail(MOYE_ERR_UNSUPPORTED, "axpby!: element type %s is not a floating-point type this build handles", dtype_name(X->dtype));
     }
@@ -403,15 +499,21 @@ int32_t map_dispatch(int32_t op, const moye_tensor* D, const moye_tensor* A, con
             return fail(MOYE_ERR_SHAPE, "map!: cannot broadcast %lld elements of b over the %lld of dst", (long long)nb, (long long)n);
     }
     if (n == 0) return MOYE_OK;
-    const ELayout ld = elayout_of(*D), la = elayout_of(*A), lb = B ? elayout_of(*B) : ELayout{};
+    ELayout ld = elayout_of(*D), la = elayout_of(*A), lb = B ? elayout_of(*B) : ELayout{};
     const void* bp = B ? B->ptr : nullptr;
     const bool fast = dense(*D) && dense(*A) && aligned16(D->ptr) && aligned16(A->ptr) &&
                       (!B || (nb == n && dense(*B) && aligned16(B->ptr)));
+    bool rows = false;
+    if (!fast && (!B || nb == n)) {  // (a b that is broadcast is tied to the leading modes of dst as the caller wrote them)
+        ELayout* all[3] = {&ld, &la, &lb};
+        const void* ptrs[3] = {D->ptr, A->ptr, bp};
+        rows = order_modes_by_stride(all, B ? 3 : 2) && recast_rows(all, ptrs, B ? 3 : 2, 16 / dtype_bytes(D->dtype));
+    }
     switch (D->dtype) {
-        case MOYE_F32: launch_map<ElF32>(op, D->ptr, ld, A->ptr, la, bp, lb, nb, (float)scalar, n, fast, st); break;
-        case MOYE_F64: launch_map<ElF64>(op, D->ptr, ld, A->ptr, la, bp, lb, nb, scalar, n, fast, st); break;
-        case MOYE_F16: launch_map<ElF16>(op, D->ptr, ld, A->ptr, la, bp, lb, nb, host_round_f16((float)scalar), n, fast, st); break;
-        case MOYE_BF16: launch_map<ElBF16>(op, D->ptr, ld, A->ptr, la, bp, lb, nb, host_round_bf16((float)scalar), n, fast, st); break;
+        case MOYE_F32: launch_map<ElF32>(op, D->ptr, ld, A->ptr, la, bp, lb, nb, (float)scalar, n, fast, rows, st); break;
+        case MOYE_F64: launch_map<ElF64>(op, D->ptr, ld, A->ptr, la, bp, lb, nb, scalar, n, fast, rows, st); break;
+        case MOYE_F16: launch_map<ElF16>(op, D->ptr, ld, A->ptr, la, bp, lb, nb, host_round_f16((float)scalar), n, fast, rows, st); break;
+        case MOYE_BF16: launch_map<ElBF16>(op, D->ptr, ld, A->ptr, la, bp, lb, nb, host_round_bf16((float)scalar), n, fast, rows, st); break;
         default:
             return fail(MOYE_ERR_UNSUPPORTED, "map!: element type %s is not a floating-point type this build handles", dtype_name(D->dtype));
     }
@@ -435,6 +537,7 @@ int32_t fill_dispatch(const moye_tensor* X, double value, hipStream_t st) {
     }
     char* p = static_cast<char*>(X->ptr);
     const int eb = dtype_bytes(X->dtype);
+    if (eb < 8) bits &= (1ull << (8 * eb)) - 1;  // integer values wrap to the element's width
     if (dense(*X) && aligned16(p)) {  // the value repeated over 16 bytes, then what is left behind the last whole 16 bytes
         uint64_t rep = bits;
         for (int w = eb; w < 8; w *= 2) rep |= rep << (8 * w);
@@ -454,7 +557,20 @@ int32_t fill_dispatch(const moye_tensor* X, double value, hipStream_t st) {
         return MOYE_OK;
     }
     const dim3 grid((unsigned)std::min<int64_t>((n + 255) / 256, 256 * 16));
-    const ELayout lx = elayout_of(*X);
+    ELayout lx = elayout_of(*X);
+    {
+        ELayout* all[1] = {&lx};
+        const void* ptrs[1] = {p};
+        if (order_modes_by_stride(all, 1) && recast_rows(all, ptrs, 1, 16 / eb)) {  // the value repeated over 16 bytes
+            uint64_t rep = bits;
+            for (int w = eb; w < 8; w *= 2) rep |= rep << (8 * w);
+            const u32x4 pattern = {(uint32_t)rep, (uint32_t)(rep >> 32), (uint32_t)rep, (uint32_t)(rep >> 32)};
+            const int64_t nvec = n / (16 / eb);
+            fill_rows_kernel<<<dim3((unsigned)std::min<int64_t>((nvec + 255) / 256, 256 * 16)), 256, 0, st>>>(reinterpret_cast<u32x4*>(p), lx, nvec, pattern);
+            MOYE_HIP_CHECK(hipGetLastError());
+            return MOYE_OK;
+        }
+    }
     switch (eb) {
         case 1: fill_kernel<1><<<grid, 256, 0, st>>>(p, lx, n, bits); break;
         case 2: fill_kernel<2><<<grid, 256, 0, st>>>(p, lx, n, bits); break;

@@ -1,5 +1,6 @@
 // Shared host-side helpers of libmoye_hip: status/error text, dtype table, tensor validation.
 #pragma once
+#include <algorithm>
 
 #include <hip/hip_runtime.h>
 
@@ -64,5 +65,39 @@ struct Mat {
     int32_t dtype;
 };
 int32_t as_matrix(const moye_tensor* t, const char* what, Mat* m);
+
+// An elementwise operation over arrays of one shape, mode by mode, takes coordinate c of every operand: the order in
+// which the coordinates are visited is free.  Visit them along the smallest strides of the first layout (the
+// destination), then of the second, so that neighbouring lanes touch neighbouring memory whatever the order the caller
+// wrote the modes in (a row-major array handed over as shape (rows, cols), strides (pitch, 1) has its unit stride on
+// the last mode).  L has rank, shape[], stride[]; the same permutation is applied to every layout; returns false, and
+// changes nothing, when ranks or shapes differ.
+template <class L>
+inline bool order_modes_by_stride(L* const* layouts, int count) {
+    const L& first = *layouts[0];
+    const int r = first.rank;
+    for (int q = 1; q < count; ++q) {
+        if (layouts[q]->rank != r) return false;
+        for (int m = 0; m < r; ++m)
+            if (layouts[q]->shape[m] != first.shape[m]) return false;
+    }
+    int perm[MOYE_MAX_RANK];
+    for (int m = 0; m < r; ++m) perm[m] = m;
+    std::stable_sort(perm, perm + r, [&](int a, int b) {
+        const bool one_a = first.shape[a] == 1, one_b = first.shape[b] == 1;  // modes of one element go last
+        if (one_a != one_b) return one_b;
+        for (int q = 0; q < count; ++q)
+            if (layouts[q]->stride[a] != layouts[q]->stride[b]) return layouts[q]->stride[a] < layouts[q]->stride[b];
+        return false;
+    });
+    for (int q = 0; q < count; ++q) {
+        const L old = *layouts[q];
+        for (int m = 0; m < r; ++m) {
+            layouts[q]->shape[m] = old.shape[perm[m]];
+            layouts[q]->stride[m] = old.stride[perm[m]];
+        }
+    }
+    return true;
+}
 
 }  // namespace moye

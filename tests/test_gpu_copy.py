@@ -596,3 +596,89 @@ def test_transpose_one_byte_elements(mh, M, N):
         mh.copyto_(_tens(mh, d8, (M, N), (N, 1)), _tens(mh, s8, (M, N), (1, M)))
         torch.cuda.synchronize()
         assert torch.equal(d8.view(torch.uint8), dst)
+
+
+@pytest.mark.parametrize("dt", ["uint8", "float16", "float32", "int64"])
+def test_same_shape_copies_whatever_the_order_of_the_modes(mh, dt):
+    """Arrays of one shape whose unit stride sits on the last or the middle mode (row-major with a pitch, a batch of
+    padded matrices, permuted rank-3 strides, a source one element off alignment): the library is free to visit the
+    coordinates in the order that suits the strides; the result is the element loop's (torch.as_strided + copy_)."""
+    tdt = getattr(torch, dt)
+    g = torch.Generator().manual_seed(29)
+
+    def rand(n):
+        return torch.randint(0, 256, (n * tdt.itemsize,), dtype=torch.uint8, generator=g).view(tdt)
+
+    cases = [
+        # shape, dst strides, src strides, dst offset, src offset
+        ((96, 200), (256, 1), (208, 1), 0, 0),
+        ((96, 200), (256, 1), (208, 1), 0, 1),
+        ((96, 200), (1, 96), (208, 1), 0, 0),
+        ((5, 24, 64), (24 * 64, 64, 1), (32 * 80, 80, 1), 0, 0),
+        ((5, 24, 64), (64, 5 * 64, 1), (1, 5, 120), 0, 0),
+        ((16, 3, 40), (1, 16 * 40, 16), (3 * 48, 48, 1), 8, 16),
+        ((7, 1, 33), (33, 0, 1), (1, 0, 7), 0, 0),
+    ]
+    for shape, dstr, sstr, doff, soff in cases:
+        extent = lambda st, off: off + 1 + sum((n - 1) * s for n, s in zip(shape, st))
+        src, dst0 = rand(extent(sstr, soff)), rand(extent(dstr, doff))
+        want = dst0.clone()
+        torch.as_strided(want, shape, dstr, doff).copy_(torch.as_strided(src, shape, sstr, soff))
+        s_d, d_d = src.cuda(), dst0.cuda()
+        mh.copyto_(_tens(mh, d_d[doff:], shape, dstr), _tens(mh, s_d[soff:], shape, sstr))
+        torch.cuda.synchronize()
+        assert torch.equal(d_d.cpu().view(torch.uint8), want.view(torch.uint8)), (shape, dstr, sstr, doff, soff)
+        # with a mask of the same shape in an order of its own
+        mask = (torch.rand(shape, generator=g) < 0.5).to(torch.uint8)
+        want = dst0.clone()
+        wv, sv = torch.as_strided(want, shape, dstr, doff), torch.as_strided(src, shape, sstr, soff)
+        wv[mask.bool()] = sv[mask.bool()]
+        m_d, d_d = mask.cuda(), dst0.cuda()
+        mh.copyto_if_(_tens(mh, d_d[doff:], shape, dstr), _tens(mh, s_d[soff:], shape, sstr), _tens(mh, m_d, shape, tuple(mask.stride())))
+        torch.cuda.synchronize()
+        assert torch.equal(d_d.cpu().view(torch.uint8), want.view(torch.uint8)), ("masked", shape, dstr, sstr)
+
+
+@pytest.mark.parametrize("dt", ["float32", "float16"])
+def test_elementwise_on_arrays_with_the_unit_stride_on_a_later_mode(mh, dt):
+    """axpby!, map! and fill! over row-major arrays with a pitch and over a rank-3 array with permuted strides give
+    the bits of the same operation on dense copies, and leave the padding alone."""
+    tdt = getattr(torch, dt)
+    itype = {2: torch.int16, 4: torch.int32}[tdt.itemsize]
+    g = torch.Generator().manual_seed(41)
+    cases = [((96, 200), (256, 1), (208, 1)), ((5, 24, 64), (64, 5 * 64, 1), (1, 5, 120)), ((96, 200), (1, 96), (208, 1))]
+    for shape, ystr, xstr in cases:
+        n = int(np.prod(shape))
+        extent = lambda st: 1 + sum((k - 1) * s for k, s in zip(shape, st))
+        X, Y = (torch.randn(extent(xstr), generator=g) * 3).to(tdt), (torch.randn(extent(ystr), generator=g) * 3).to(tdt)
+        xv, yv = torch.as_strided(X, shape, xstr), torch.as_strided(Y, shape, ystr)
+        # dense copies in the order of the logical index (first mode fastest)
+        order = tuple(reversed(range(len(shape))))
+        xd, yd = xv.permute(order).contiguous().cuda(), yv.permute(order).contiguous().cuda()
+        flat = lambda t: _tens(mh, t, [n], [1])
+        yd1 = yd.clone()
+        mh.axpby_(0.75, flat(xd), -1.25, flat(yd1))
+        xs, ys = X.cuda(), Y.cuda()
+        mh.axpby_(0.75, _tens(mh, xs, shape, xstr), -1.25, _tens(mh, ys, shape, ystr))
+        torch.cuda.synchronize()
+        want = Y.clone()
+        torch.as_strided(want, shape, ystr).copy_(yd1.cpu().permute(order))
+        assert torch.equal(ys.cpu().view(itype), want.view(itype)), ("axpby", shape, ystr, xstr)
+        for second in ("array", "scalar"):
+            dd = torch.zeros(n, dtype=tdt, device="cuda")
+            mh.map_("mul", flat(dd), flat(xd), flat(yd) if second == "array" else None, 1.75)
+            D = torch.full((extent(ystr),), 7.0, dtype=tdt)
+            ds = D.cuda()
+            y2 = Y.cuda()
+            mh.map_("mul", _tens(mh, ds, shape, ystr), _tens(mh, xs, shape, xstr), _tens(mh, y2, shape, ystr) if second == "array" else None, 1.75)
+            torch.cuda.synchronize()
+            want = D.clone()
+            torch.as_strided(want, shape, ystr).copy_(dd.cpu().reshape(tuple(reversed(shape))).permute(order))
+            assert torch.equal(ds.cpu().view(itype), want.view(itype)), ("map", second, shape, ystr, xstr)
+        F = torch.full((extent(ystr),), 7.0, dtype=tdt)
+        fs = F.cuda()
+        mh.fill_(_tens(mh, fs, shape, ystr), 2.5)
+        torch.cuda.synchronize()
+        want = F.clone()
+        torch.as_strided(want, shape, ystr).fill_(2.5)
+        assert torch.equal(fs.cpu(), want), ("fill", shape, ystr)

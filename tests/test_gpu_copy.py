@@ -682,3 +682,34 @@ def test_elementwise_on_arrays_with_the_unit_stride_on_a_later_mode(mh, dt):
         want = F.clone()
         torch.as_strided(want, shape, ystr).fill_(2.5)
         assert torch.equal(fs.cpu(), want), ("fill", shape, ystr)
+
+
+@pytest.mark.parametrize("dt", ["uint8", "float16", "float32"])
+def test_batches_of_transposes(mh, dt):
+    """Rank-3 and rank-4 arrays whose two sides have their unit strides on different modes: every other mode counts
+    matrices, and each matrix goes through the tiled transpose (whole tiles, ragged edges, padded pitches).  Checked
+    against the element loop (torch.as_strided + copy_), padding included."""
+    tdt = getattr(torch, dt)
+    g = torch.Generator().manual_seed(53)
+
+    def rand(n):
+        return torch.randint(0, 256, (n * tdt.itemsize,), dtype=torch.uint8, generator=g).view(tdt)
+
+    M, N = 512, 320
+    cases = [
+        # shape, dst strides, src strides
+        ((3, M, N), (M * N, N, 1), (M * N, 1, M)),                      # batch first
+        ((M, N, 3), (N, 1, M * N), (1, M, M * N)),                      # batch last
+        ((M, 2, N), (2 * N, N, 1), (1, M * N, M)),                      # batch in the middle, interleaved rows on one side
+        ((2, M + 8, N + 16), ((M + 8) * (N + 32), N + 32, 1), ((M + 16) * (N + 16), 1, M + 16)),   # ragged sizes, padded pitches
+        ((2, M, 3, N), (3 * M * N, N, M * N, 1), (3 * M * N, 1, M * N, M)),                       # two batch modes
+    ]
+    for shape, dstr, sstr in cases:
+        extent = lambda st: 1 + sum((k - 1) * s for k, s in zip(shape, st))
+        src, dst0 = rand(extent(sstr)), rand(extent(dstr))
+        want = dst0.clone()
+        torch.as_strided(want, shape, dstr).copy_(torch.as_strided(src, shape, sstr))
+        s_d, d_d = src.cuda(), dst0.cuda()
+        mh.copyto_(_tens(mh, d_d, shape, dstr), _tens(mh, s_d, shape, sstr))
+        torch.cuda.synchronize()
+        assert torch.equal(d_d.cpu().view(torch.uint8), want.view(torch.uint8)), (shape, dstr, sstr)

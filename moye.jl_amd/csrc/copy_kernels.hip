@@ -55,8 +55,10 @@ template <bool kSwizzle, int GI>
 __global__ __launch_bounds__(256) void transpose_lds_b32(const uint32_t* __restrict__ src,
                                                          uint32_t* __restrict__ dst, int64_t lds_,
                                                          int64_t ldd, int groups_i, int tiles_j,
-                                                         int sb) {
+                                                         int sb, int64_t bs_src, int64_t bs_dst) {
     extern __shared__ u32x4 tile[];  // GI tiles of 64 x 16 chunks
+    src += (int64_t)blockIdx.y * bs_src;  // blockIdx.y counts the matrices of a batch
+    dst += (int64_t)blockIdx.y * bs_dst;
     int gi, tj;
     tile_coords(blockIdx.x, groups_i, tiles_j, sb, &gi, &tj);
 
@@ -95,7 +97,8 @@ __global__ __launch_bounds__(256) void transpose_lds_b32(const uint32_t* __restr
 }
 
 template <bool kSwizzle, int GI>
-static int32_t launch_transpose(const uint32_t* s, uint32_t* d, int64_t lds_, int64_t ldd, int ti, int tj, hipStream_t st) {
+static int32_t launch_transpose(const uint32_t* s, uint32_t* d, int64_t lds_, int64_t ldd, int ti, int tj, hipStream_t st, int64_t bs_src = 0,
+                              int64_t bs_dst = 0, int batch = 1) {
     auto kern = transpose_lds_b32<kSwizzle, GI>;
     constexpr int kLds = GI * kTile * kTile * 4;
     if (kLds > 48 * 1024) {
@@ -110,7 +113,7 @@ static int32_t launch_transpose(const uint32_t* s, uint32_t* d, int64_t lds_, in
     if (groups > 0x7fffffff) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles");
     // groups are walked with the source-contiguous index fastest in bands of 64 tile columns: the
     // workgroups in flight read whole source rows and write runs of several KiB per destination row
-    kern<<<(unsigned)groups, 256, kLds, st>>>(s, d, lds_, ldd, ti / GI, tj, 64);
+    kern<<<dim3((unsigned)groups, (unsigned)batch), 256, kLds, st>>>(s, d, lds_, ldd, ti / GI, tj, 64, bs_src, bs_dst);
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;
 }
@@ -124,8 +127,11 @@ static int32_t launch_transpose(const uint32_t* s, uint32_t* d, int64_t lds_, in
 // as one 16-byte piece of destination row i, 8 lanes per 128-byte run.
 template <int GI>
 __global__ __launch_bounds__(256) void transpose_lds_b16(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst,
-                                                         int64_t lds_, int64_t ldd, int groups_i, int tiles_j, int sb) {
+                                                         int64_t lds_, int64_t ldd, int groups_i, int tiles_j, int sb,
+                                                         int64_t bs_src, int64_t bs_dst) {
     extern __shared__ u32x4 tile[];  // GI tiles of 64 rows x 8 chunks
+    src += (int64_t)blockIdx.y * bs_src;
+    dst += (int64_t)blockIdx.y * bs_dst;
     int gi, tj;
     tile_coords(blockIdx.x, groups_i, tiles_j, sb, &gi, &tj);
     const int v = threadIdx.x & 7;   // 16-byte chunk inside a 128-byte run
@@ -172,7 +178,8 @@ __global__ __launch_bounds__(256) void transpose_lds_b16(const uint16_t* __restr
 }
 
 template <int GI>
-static int32_t launch_transpose16(const uint16_t* s, uint16_t* d, int64_t lds_, int64_t ldd, int ti, int tj, hipStream_t st) {
+static int32_t launch_transpose16(const uint16_t* s, uint16_t* d, int64_t lds_, int64_t ldd, int ti, int tj, hipStream_t st, int64_t bs_src = 0,
+                              int64_t bs_dst = 0, int batch = 1) {
     auto kern = transpose_lds_b16<GI>;
     constexpr int kLds = GI * kTile * kTile * 2;
     if (kLds > 48 * 1024) {
@@ -185,7 +192,7 @@ static int32_t launch_transpose16(const uint16_t* s, uint16_t* d, int64_t lds_, 
     }
     const int64_t groups = (int64_t)(ti / GI) * tj;
     if (groups > 0x7fffffff) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles");
-    kern<<<(unsigned)groups, 256, kLds, st>>>(s, d, lds_, ldd, ti / GI, tj, 64);
+    kern<<<dim3((unsigned)groups, (unsigned)batch), 256, kLds, st>>>(s, d, lds_, ldd, ti / GI, tj, 64, bs_src, bs_dst);
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;
 }
@@ -204,8 +211,11 @@ __device__ __forceinline__ int lds_row_b8(int j) { return (j & ~3) | ((j & 3) ^ 
 
 template <int GI>
 __global__ __launch_bounds__(256) void transpose_lds_b8(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, int64_t lds_,
-                                                        int64_t ldd, int groups_i, int tiles_j, int sb) {
+                                                        int64_t ldd, int groups_i, int tiles_j, int sb, int64_t bs_src,
+                                                        int64_t bs_dst) {
     extern __shared__ u32x4 tile[];  // GI sub-tiles of 256 rows x 4 chunks
+    src += (int64_t)blockIdx.y * bs_src;
+    dst += (int64_t)blockIdx.y * bs_dst;
     int gi, tj;
     tile_coords(blockIdx.x, groups_i, tiles_j, sb, &gi, &tj);
     const int v = threadIdx.x & 3;   // 16-byte chunk of a 64-byte row
@@ -247,7 +257,8 @@ __global__ __launch_bounds__(256) void transpose_lds_b8(const uint8_t* __restric
 }
 
 template <int GI>
-static int32_t launch_transpose8(const uint8_t* s, uint8_t* d, int64_t lds_, int64_t ldd, int ti, int tj, hipStream_t st) {
+static int32_t launch_transpose8(const uint8_t* s, uint8_t* d, int64_t lds_, int64_t ldd, int ti, int tj, hipStream_t st, int64_t bs_src = 0,
+                              int64_t bs_dst = 0, int batch = 1) {
     auto kern = transpose_lds_b8<GI>;
     constexpr int kLds = GI * kTileJ8 * kTile;
     if (kLds > 48 * 1024) {
@@ -260,7 +271,7 @@ static int32_t launch_transpose8(const uint8_t* s, uint8_t* d, int64_t lds_, int
     }
     const int64_t groups = (int64_t)(ti / GI) * tj;
     if (groups > 0x7fffffff) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles");
-    kern<<<(unsigned)groups, 256, kLds, st>>>(s, d, lds_, ldd, ti / GI, tj, 64);
+    kern<<<dim3((unsigned)groups, (unsigned)batch), 256, kLds, st>>>(s, d, lds_, ldd, ti / GI, tj, 64, bs_src, bs_dst);
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;
 }
@@ -661,6 +672,33 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
             MOYE_HIP_CHECK(hipGetLastError());
             return MOYE_OK;
         }
+        // whole tiles of an aligned matrix (or of `batch` such matrices bs / bd elements apart) through the LDS kernels
+        auto tiled_launch = [&](const char* s_, char* d_, int64_t ni, int64_t nj, int64_t lds_, int64_t ldd, int64_t bs, int64_t bd,
+                                int batch) -> int32_t {
+            const int tile_j = sb == 1 ? kTileJ8 : kTile;
+            const int ti = (int)(ni / kTile), tj = (int)(nj / tile_j);
+            if (sb == 1) {
+                const uint8_t* s8 = reinterpret_cast<const uint8_t*>(s_);
+                uint8_t* d8 = reinterpret_cast<uint8_t*>(d_);
+                if (ti % 4 == 0) return launch_transpose8<4>(s8, d8, lds_, ldd, ti, tj, st, bs, bd, batch);
+                if (ti % 2 == 0) return launch_transpose8<2>(s8, d8, lds_, ldd, ti, tj, st, bs, bd, batch);
+                return launch_transpose8<1>(s8, d8, lds_, ldd, ti, tj, st, bs, bd, batch);
+            }
+            if (sb == 2) {
+                const uint16_t* s16 = reinterpret_cast<const uint16_t*>(s_);
+                uint16_t* d16 = reinterpret_cast<uint16_t*>(d_);
+                if (ti % 8 == 0) return launch_transpose16<8>(s16, d16, lds_, ldd, ti, tj, st, bs, bd, batch);
+                if (ti % 4 == 0) return launch_transpose16<4>(s16, d16, lds_, ldd, ti, tj, st, bs, bd, batch);
+                if (ti % 2 == 0) return launch_transpose16<2>(s16, d16, lds_, ldd, ti, tj, st, bs, bd, batch);
+                return launch_transpose16<1>(s16, d16, lds_, ldd, ti, tj, st, bs, bd, batch);
+            }
+            const uint32_t* s32 = reinterpret_cast<const uint32_t*>(s_);
+            uint32_t* d32 = reinterpret_cast<uint32_t*>(d_);
+            if (tc && (tc->flags & MOYE_GEMM_NO_LDS_SWIZZLE)) return launch_transpose<false, 1>(s32, d32, lds_, ldd, ti, tj, st, bs, bd, batch);
+            if (ti % 4 == 0) return launch_transpose<true, 4>(s32, d32, lds_, ldd, ti, tj, st, bs, bd, batch);
+            if (ti % 2 == 0) return launch_transpose<true, 2>(s32, d32, lds_, ldd, ti, tj, st, bs, bd, batch);
+            return launch_transpose<true, 1>(s32, d32, lds_, ldd, ti, tj, st, bs, bd, batch);
+        };
         // (2) rank-2 transpose of 4-byte elements through the LDS tile
         const int tm = tc && tc->tiler_mn[0] ? tc->tiler_mn[0] : kTile;
         const int tn = tc && tc->tiler_mn[1] ? tc->tiler_mn[1] : kTile;
@@ -680,30 +718,7 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
                 const bool aligned = ni % kTile == 0 && nj % tile_j == 0 && lds_ % per16 == 0 && ldd % per16 == 0 &&
                                      lds_ >= ni && ldd >= nj &&
                                      (reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d)) % 16 == 0;
-                if (aligned) {
-                    const int ti = (int)(ni / kTile), tj = (int)(nj / tile_j);
-                    if (sb == 1) {
-                        const uint8_t* s8 = reinterpret_cast<const uint8_t*>(s);
-                        uint8_t* d8 = reinterpret_cast<uint8_t*>(d);
-                        if (ti % 4 == 0) return launch_transpose8<4>(s8, d8, lds_, ldd, ti, tj, st);
-                        if (ti % 2 == 0) return launch_transpose8<2>(s8, d8, lds_, ldd, ti, tj, st);
-                        return launch_transpose8<1>(s8, d8, lds_, ldd, ti, tj, st);
-                    }
-                    if (sb == 2) {
-                        const uint16_t* s16 = reinterpret_cast<const uint16_t*>(s);
-                        uint16_t* d16 = reinterpret_cast<uint16_t*>(d);
-                        if (ti % 8 == 0) return launch_transpose16<8>(s16, d16, lds_, ldd, ti, tj, st);
-                        if (ti % 4 == 0) return launch_transpose16<4>(s16, d16, lds_, ldd, ti, tj, st);
-                        if (ti % 2 == 0) return launch_transpose16<2>(s16, d16, lds_, ldd, ti, tj, st);
-                        return launch_transpose16<1>(s16, d16, lds_, ldd, ti, tj, st);
-                    }
-                    const uint32_t* s32 = reinterpret_cast<const uint32_t*>(s);
-                    uint32_t* d32 = reinterpret_cast<uint32_t*>(d);
-                    if (tc && (tc->flags & MOYE_GEMM_NO_LDS_SWIZZLE)) return launch_transpose<false, 1>(s32, d32, lds_, ldd, ti, tj, st);
-                    if (ti % 4 == 0) return launch_transpose<true, 4>(s32, d32, lds_, ldd, ti, tj, st);
-                    if (ti % 2 == 0) return launch_transpose<true, 2>(s32, d32, lds_, ldd, ti, tj, st);
-                    return launch_transpose<true, 1>(s32, d32, lds_, ldd, ti, tj, st);
-                }
+                if (aligned) return tiled_launch(s, d, ni, nj, lds_, ldd, 0, 0, 1);
                 // Sizes that are not multiples of the tile (everything else in order): the interior goes through the
                 // LDS tiles, the two strips that are left through the general kernel.  Three launches, disjoint parts.  (A strip
                 // touches one page per row of the other side, so it costs far more per byte than the interior: 16400 x 16392
@@ -729,8 +744,9 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
             }
         }
         // (2b) a batch of such transposes: arrays of one shape, rank above two, the unit strides of the two sides on
-        // different modes of 64 and more; every other mode counts matrices.  One rank-2 call per matrix while the
-        // matrices are large enough to fill the chip on their own and few enough for the launches not to matter
+        // different modes of 64 and more; every other mode counts matrices.  One launch with the matrix index in the
+        // grid when there is one such mode and the matrices are whole aligned tiles; else one rank-2 call per matrix while
+        // the matrices are large enough to fill the chip on their own and few enough for the launches not to matter
         // (64 fp32 matrices of 2048 x 2048: 1.5 TB/s through the general kernel, which reads one side in single
         // elements a pitch apart).
         if ((sb == 4 || sb == 2 || sb == 1) && src->rank == dst->rank && src->rank > 2) {
@@ -744,6 +760,18 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
             }
             if (same && mi >= 0 && mj >= 0 && mi != mj && src->shape[mi] >= kTile && src->shape[mj] >= kTile) {
                 const int64_t per = src->shape[mi] * src->shape[mj], batch = n / per;
+                // one batch mode, whole aligned tiles: one launch, the matrix index in the grid
+                int bm = -1, nbatch_modes = 0;
+                for (int m = 0; m < r; ++m)
+                    if (m != mi && m != mj && src->shape[m] > 1) { bm = m; ++nbatch_modes; }
+                {
+                    const int64_t ni = src->shape[mi], nj = src->shape[mj], lds_ = src->stride[mj], ldd = dst->stride[mi];
+                    const int per16 = 16 / sb, tile_j = sb == 1 ? kTileJ8 : kTile;
+                    if (nbatch_modes == 1 && batch <= 65535 && tm == kTile && tn == kTile && ni % kTile == 0 && nj % tile_j == 0 && lds_ % per16 == 0 && ldd % per16 == 0 &&
+                        lds_ >= ni && ldd >= nj && src->stride[bm] % per16 == 0 && dst->stride[bm] % per16 == 0 &&
+                        (reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d)) % 16 == 0)
+                        return tiled_launch(s, d, ni, nj, lds_, ldd, src->stride[bm], dst->stride[bm], (int)batch);
+                }
                 if (batch <= 4096 && per * sb >= (128 << 10)) {
                     moye_tensor ps = *src, pd = *dst;
                     ps.rank = pd.rank = 2;

@@ -24,12 +24,12 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # (the summaries are committed under profiles/), each reading scaled by what the same counter shows for the
 # 1 GiB plain copy (fetch x2.0000, write x1.0000).  Only valid for the default tile/waves/flags.
 MEASURED_TRAFFIC = {
-    "gemm_f16_4096_tile256": {"read_bytes": 198686 * 1024, "write_bytes": 34325 * 1024},
+    "gemm_f16_4096_tile256": {"read_bytes": 196894 * 1024, "write_bytes": 32781 * 1024},
     "transpose_f32_16384": {"read_bytes": 1048637 * 1024, "write_bytes": 1049561 * 1024},
-    "gemm_bf16_8192_tile256": {"read_bytes": 1574701 * 1024, "write_bytes": 262866 * 1024},
-    "gemm_f32_8192_tile256": {"read_bytes": 4783150 * 1024, "write_bytes": 262200 * 1024},
-    "gemm_fp8_8192_tile256": {"read_bytes": 787140 * 1024, "write_bytes": 131072 * 1024},
-    "gemm_bf16_16x8192x8192": {"read_bytes": 149404 * 1024, "write_bytes": 512 * 1024},
+    "gemm_bf16_8192_tile256": {"read_bytes": 1575798 * 1024, "write_bytes": 262640 * 1024},
+    "gemm_f32_8192_tile256": {"read_bytes": 6980880 * 1024, "write_bytes": 262152 * 1024},
+    "gemm_fp8_8192_tile256": {"read_bytes": 786997 * 1024, "write_bytes": 131072 * 1024},
+    "gemm_bf16_16x8192x8192": {"read_bytes": 149528 * 1024, "write_bytes": 512 * 1024},
 }
 
 

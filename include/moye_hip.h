@@ -181,13 +181,41 @@ int32_t moye_fill(const moye_tensor* X, double value, void* stream);
 int32_t moye_map(int32_t op, const moye_tensor* dst, const moye_tensor* a, const moye_tensor* b, double scalar,
                  void* stream);
 
-/* bytes of device workspace moye_gemm needs for this call: the K-major copies of MFMA operands whose
- * unit stride is not along K (NN / NT / TT problems) and split_k * M * N fp32 partial products of a
- * split-K call; 0 for plain TN and for UniversalFMA.  The library
- * allocates the workspace on first use (a synchronous hipMalloc inside that one moye_gemm call), grows
- * it when a larger call comes, and keeps it; calls that use it must not overlap on different streams. */
+/* bytes of device workspace this gemm! call needs: the K-major copies of MFMA operands whose unit stride
+ * is not along K (NN / NT / TT problems, src/arch/mma/make_mma_ops.jl:253-265) and split_k * M * N fp32
+ * partial products of a split-K call; 0 for plain TN and for UniversalFMA.
+ *   moye_gemm     keeps a workspace of its own per (device, stream): allocated by the first call on that stream
+ *                 that needs one (a synchronous hipMalloc inside that call, so not under stream capture),
+ *                 replaced by a larger one when a larger call comes, never freed inside a call.  Calls on
+ *                 different streams do not share a buffer; calls on one stream are ordered by the stream.
+ *   moye_gemm_ex  takes the workspace from the caller (256-byte aligned, at least the size reported here;
+ *                 NULL when the call needs none) and never allocates, frees or synchronises.            */
 int32_t moye_gemm_workspace_size(const moye_tiled_mma* mma, const moye_tensor* D,
                                  const moye_tensor* A, const moye_tensor* B, size_t* bytes);
+/* waits for the devices that hold workspaces of moye_gemm and frees them all (no counterpart in the
+ * reference, whose kernels own no memory) */
+int32_t moye_gemm_release_workspace(void);
+
+/* What the reference's user kernels do to the accumulator fragment between the k-loop and the store
+ * (axpby!, src/algorithm/blas.jl:1-9; a broadcast over the fragment, src/broadcast.jl:5-41), as part of the
+ * GEMM's epilogue:   D = op(alpha * (A * B') + beta * C, operand)   in fp32, then one round-to-nearest-even
+ * conversion to D's type (src/arch/copy/copy.jl:38-43).  Nothing is fused: alpha * acc, beta * c, their sum
+ * and op are four separately rounded fp32 operations; with beta == 0 C is not read (axpby!'s iszero(b)). */
+typedef struct {
+    float   alpha;
+    float   beta;
+    int32_t op;                 /* MOYE_MAP_*; MOYE_MAP_IDENTITY = none                                */
+    int32_t _pad;
+    const moye_tensor* operand; /* second argument of op: an (M,N) array of f32 or of D's type with any
+                                   strides, 0 = repeated along that mode (a bias vector is (M,N):(1,0) or
+                                   (M,N):(0,1)); NULL = `scalar`                                        */
+    double  scalar;
+} moye_gemm_epilogue;
+
+/* gemm! with the epilogue above and a caller-provided workspace */
+int32_t moye_gemm_ex(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A,
+                     const moye_tensor* B, const moye_tensor* C, const moye_gemm_epilogue* ep,
+                     void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- host-side layout algebra (no GPU needed) ------------------------------------------- */
 /* Text form of a layout: `shape:stride`, `_n` = static int, `n` = dynamic int, e.g.

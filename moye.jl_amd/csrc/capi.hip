@@ -3,7 +3,10 @@
 // Julia assertions while tracing (src/algorithm/blas.jl:55-57,79-82, src/int_tuple.jl:88,
 // src/atom/copy.jl:121-122) come back as status codes before any kernel is launched.
 #include <cstring>
+#include <map>
 #include <mutex>
+#include <utility>
+#include <vector>
 
 #include "kernels.hpp"
 
@@ -62,26 +65,35 @@ static int32_t atom_input_dtype(int32_t atom) {
     }
 }
 
-// ---- workspace for operands that are not K-major -----------------------------------------------
-// The MFMA kernels read K-major operands.  An operand with its unit stride along M (or N) is first
-// transposed into a K-major copy in a workspace the library owns: allocated on first use, grown when
-// a larger operand comes, kept.  One workspace per process: calls that need it must not overlap on
-// different streams (the copy and the GEMM of one call are ordered by the stream they share).
+// ---- workspace: K-major copies of operands that are not K-major, partial products of split-K -------
+// moye_gemm_ex takes the workspace from its caller and allocates nothing.  moye_gemm keeps the
+// library's own: one buffer per (device, stream), allocated on the first call that needs one (a
+// synchronous hipMalloc inside that call) and replaced by a larger one when a larger call comes.  A
+// replaced buffer is not freed in the call path, since work queued earlier on the stream may still
+// use it: it is parked until moye_gemm_release_workspace().  g_ws_mutex is held from the lookup to
+// the last enqueue of a call, so two host threads that share a stream cannot interleave the halves
+// (transpose, GEMM, reduction) of their calls; calls on different streams have different buffers.
+struct LibWorkspace {
+    char* ptr = nullptr;
+    size_t bytes = 0;
+};
 static std::mutex g_ws_mutex;
-static char* g_ws = nullptr;
-static size_t g_ws_bytes = 0;
+static std::map<std::pair<int, hipStream_t>, LibWorkspace> g_ws;
+static std::vector<void*> g_ws_parked;
 
-static int32_t ensure_workspace(size_t bytes) {
-    std::lock_guard<std::mutex> lock(g_ws_mutex);
-    if (bytes <= g_ws_bytes) return MOYE_OK;
-    if (g_ws) {
-        MOYE_HIP_CHECK(hipDeviceSynchronize());
-        MOYE_HIP_CHECK(hipFree(g_ws));
-        g_ws = nullptr;
-        g_ws_bytes = 0;
+// caller holds g_ws_mutex
+static int32_t library_workspace(size_t bytes, hipStream_t st, char** out) {
+    int dev = 0;
+    MOYE_HIP_CHECK(hipGetDevice(&dev));
+    LibWorkspace& w = g_ws[{dev, st}];
+    if (bytes > w.bytes) {
+        void* p = nullptr;
+        MOYE_HIP_CHECK(hipMalloc(&p, bytes));
+        if (w.ptr) g_ws_parked.push_back(w.ptr);
+        w.ptr = static_cast<char*>(p);
+        w.bytes = bytes;
     }
-    MOYE_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&g_ws), bytes));
-    g_ws_bytes = bytes;
+    *out = w.ptr;
     return MOYE_OK;
 }
 
@@ -138,8 +150,11 @@ static bool rows_in_16_byte_pieces(const void* c, int64_t ld_m, int64_t ld_n, in
     return c && ld_n == 1 && reinterpret_cast<uintptr_t>(c) % 16 == 0 && (ld_m * dtype_bytes(dt)) % 16 == 0;
 }
 
+// `caller_ws` / `caller_ws_bytes`: the workspace when the caller brings one (it must hold what
+// moye_gemm_workspace_size reports); with caller_ws == nullptr the library's own is used.
 static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const moye_tensor* tA,
-                         const moye_tensor* tB, const moye_tensor* tC, float alpha, hipStream_t st) {
+                         const moye_tensor* tB, const moye_tensor* tC, float alpha, char* caller_ws,
+                         size_t caller_ws_bytes, hipStream_t st) {
     if (!mma) return fail(MOYE_ERR_ARG, "gemm!: null TiledMMA descriptor");
     Mat A, B, C{}, D;
     if (int32_t e = as_matrix(tA, "A", &A)) return e;
@@ -178,12 +193,21 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
     // NN / NT / TT (the naming of src/arch/mma/make_mma_ops.jl:253-265): operands whose unit stride is not
     // along K are brought to the K-major form the kernels read (one tiled transpose each)
     char* ws = nullptr;
+    std::unique_lock<std::mutex> ws_lock(g_ws_mutex, std::defer_lock);
     if (const size_t ws_bytes = gemm_workspace_bytes(mma, A, B)) {
         if (mma->flags & MOYE_GEMM_NO_WORKSPACE)
             return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the MFMA kernels need K-major A and B (stride 1 along K, the 'TN' form), split_k needs room "
-                                              "for its partial products, and MOYE_GEMM_NO_WORKSPACE forbids the library's workspace");
-        if (int32_t e = ensure_workspace(ws_bytes)) return e;
-        ws = g_ws;
+                                              "for its partial products, and MOYE_GEMM_NO_WORKSPACE forbids the use of a workspace");
+        if (caller_ws) {
+            if (ws_bytes > caller_ws_bytes)
+                return fail(MOYE_ERR_ARG, "gemm!: this call needs a workspace of %zu bytes, the one passed holds %zu", ws_bytes, caller_ws_bytes);
+            if (reinterpret_cast<uintptr_t>(caller_ws) % 256)
+                return fail(MOYE_ERR_ALIGN, "gemm!: the workspace must start on a 256-byte boundary");
+            ws = caller_ws;
+        } else {
+            ws_lock.lock();  // until every kernel of this call is enqueued
+            if (int32_t e = library_workspace(ws_bytes, st, &ws)) return e;
+        }
         if (A.cs != 1 && A.cols > 1) {
             const size_t nb = kmajor_bytes(A);
             if (int32_t e = make_kmajor(&A, ws, st)) return e;
@@ -291,7 +315,40 @@ int32_t moye_copy(const moye_tiled_copy* tc, const moye_tensor* dst, const moye_
 
 int32_t moye_gemm(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A, const moye_tensor* B,
                   const moye_tensor* C, float alpha, void* stream) {
-    return gemm_impl(mma, D, A, B, C, alpha, static_cast<hipStream_t>(stream));
+    return gemm_impl(mma, D, A, B, C, alpha, nullptr, 0, static_cast<hipStream_t>(stream));
+}
+
+int32_t moye_gemm_ex(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A, const moye_tensor* B,
+                     const moye_tensor* C, const moye_gemm_epilogue* ep, void* workspace, size_t workspace_bytes,
+                     void* stream) {
+    if (!ep) return fail(MOYE_ERR_ARG, "moye_gemm_ex: null epilogue descriptor");
+    if (!workspace && workspace_bytes) return fail(MOYE_ERR_ARG, "moye_gemm_ex: null workspace of %zu bytes", workspace_bytes);
+    if (ep->beta != 0.f || ep->op != MOYE_MAP_IDENTITY)
+        return fail(MOYE_ERR_UNSUPPORTED, "moye_gemm_ex: beta and the element-wise operation are not built yet");
+    // a call that needs no workspace may pass none; one that needs it and passes none fails: this entry never allocates
+    alignas(256) static char nothing[256];
+    return gemm_impl(mma, D, A, B, C, ep->alpha, workspace ? static_cast<char*>(workspace) : nothing, workspace_bytes,
+                     static_cast<hipStream_t>(stream));
+}
+
+int32_t moye_gemm_release_workspace(void) {
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    int current = 0;
+    MOYE_HIP_CHECK(hipGetDevice(&current));
+    int last = -1;
+    for (auto& kv : g_ws) {  // ordered by device: wait once for each device that holds a buffer
+        if (kv.first.first != last) {
+            last = kv.first.first;
+            MOYE_HIP_CHECK(hipSetDevice(last));
+            MOYE_HIP_CHECK(hipDeviceSynchronize());
+        }
+        if (kv.second.ptr) g_ws_parked.push_back(kv.second.ptr);
+    }
+    MOYE_HIP_CHECK(hipSetDevice(current));
+    g_ws.clear();
+    for (void* p : g_ws_parked) (void)hipFree(p);
+    g_ws_parked.clear();
+    return MOYE_OK;
 }
 
 int32_t moye_axpby(double a, const moye_tensor* X, double b, const moye_tensor* Y, void* stream) {
@@ -366,7 +423,7 @@ int32_t moye_time_gemm(const moye_tiled_mma* mma, const moye_tensor* D, const mo
                        const moye_tensor* C, float alpha, void* stream, int32_t warmup, int32_t iters,
                        float* ms_per_launch) {
     hipStream_t st = static_cast<hipStream_t>(stream);
-    return time_launches([&] { return gemm_impl(mma, D, A, B, C, alpha, st); }, st, warmup, iters, ms_per_launch);
+    return time_launches([&] { return gemm_impl(mma, D, A, B, C, alpha, nullptr, 0, st); }, st, warmup, iters, ms_per_launch);
 }
 
 int32_t moye_time_copy(const moye_tiled_copy* tc, const moye_tensor* dst, const moye_tensor* src, void* stream,

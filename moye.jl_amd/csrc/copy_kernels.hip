@@ -102,12 +102,8 @@ static int32_t launch_transpose(const uint32_t* s, uint32_t* d, int64_t lds_, in
     auto kern = transpose_lds_b32<kSwizzle, GI>;
     constexpr int kLds = GI * kTile * kTile * 4;
     if (kLds > 48 * 1024) {
-        static bool once = false;
-        if (!once) {
-            MOYE_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
-            once = true;
-        }
+        static LdsCap cap;
+        if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
     }
     const int64_t groups = (int64_t)(ti / GI) * tj;
     if (groups > 0x7fffffff) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles");
@@ -183,12 +179,8 @@ static int32_t launch_transpose16(const uint16_t* s, uint16_t* d, int64_t lds_, 
     auto kern = transpose_lds_b16<GI>;
     constexpr int kLds = GI * kTile * kTile * 2;
     if (kLds > 48 * 1024) {
-        static bool once = false;
-        if (!once) {
-            MOYE_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
-            once = true;
-        }
+        static LdsCap cap;
+        if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
     }
     const int64_t groups = (int64_t)(ti / GI) * tj;
     if (groups > 0x7fffffff) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles");
@@ -262,12 +254,8 @@ static int32_t launch_transpose8(const uint8_t* s, uint8_t* d, int64_t lds_, int
     auto kern = transpose_lds_b8<GI>;
     constexpr int kLds = GI * kTileJ8 * kTile;
     if (kLds > 48 * 1024) {
-        static bool once = false;
-        if (!once) {
-            MOYE_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
-            once = true;
-        }
+        static LdsCap cap;
+        if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
     }
     const int64_t groups = (int64_t)(ti / GI) * tj;
     if (groups > 0x7fffffff) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles");

@@ -267,12 +267,8 @@ static int32_t launch(const GemmArgs& a, hipStream_t st) {
     constexpr int kLds = kMain > kEpi ? kMain : kEpi;
     auto kern = gemm_mfma_tn<In, Out, BM, BN, BKB, kEdge, AT>;
     if (kLds > 64 * 1024) {
-        static bool once = false;  // raising the dynamic LDS cap is per function, idempotent
-        if (!once) {
-            MOYE_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
-            once = true;
-        }
+        static LdsCap cap;
+        if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
     }
     kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1)), dim3(256), kLds, st>>>(a);
     MOYE_HIP_CHECK(hipGetLastError());

@@ -310,12 +310,8 @@ template <typename In, typename Out, int STAGES>
 static int32_t launch256_ring(const GemmArgs& a, hipStream_t st) {
     constexpr int kLds = STAGES * (256 + 256) * 64;
     auto kern = gemm_mfma_tn_256_ring<In, Out, 2, 4, STAGES>;
-    static bool once = false;
-    if (!once) {
-        MOYE_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
-        once = true;
-    }
+    static LdsCap cap;
+    if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
     kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1)), dim3(512), kLds, st>>>(a);
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;
@@ -325,12 +321,8 @@ template <typename In, typename Out, int WGM, int WGN>
 static int32_t launch256(const GemmArgs& a, hipStream_t st) {
     constexpr int kLds = 2 * (256 + 256) * 128;  // two operand stages, 128 KiB
     auto kern = gemm_mfma_tn_256<In, Out, WGM, WGN>;
-    static bool once = false;
-    if (!once) {
-        MOYE_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
-        once = true;
-    }
+    static LdsCap cap;
+    if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
     kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1)), dim3(64 * WGM * WGN), kLds, st>>>(a);
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;

@@ -340,12 +340,8 @@ template <typename In, typename Out, int WGN>
 static int32_t launch256_w4(const GemmArgs& a, hipStream_t st) {
     constexpr int kLds = 5 * (256 + 256) * 64;  // all 160 KiB
     auto kern = gemm_mfma_tn_256_w4<In, Out, WGN>;
-    static bool once = false;
-    if (!once) {
-        MOYE_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
-        once = true;
-    }
+    static LdsCap cap;
+    if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
     kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1)), dim3(128 * WGN), kLds, st>>>(a);
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;

@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
@@ -23,6 +24,21 @@ int32_t fail(moye_status st, const char* fmt, ...) __attribute__((format(printf,
         if (_e != hipSuccess)                                                             \
             return ::moye::fail(MOYE_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(_e)); \
     } while (0)
+
+// A kernel that needs more dynamic LDS than the default cap has the cap raised once per device.  The call is
+// idempotent, so two host threads that launch for the first time may both make it; the flag only saves later calls.
+struct LdsCap {
+    std::atomic<uint64_t> raised{0};  // bit d: done on device d
+};
+inline int32_t raise_lds_cap(LdsCap& cap, const void* kernel, int bytes) {
+    int dev = 0;
+    MOYE_HIP_CHECK(hipGetDevice(&dev));
+    const uint64_t bit = 1ull << (dev & 63);
+    if (cap.raised.load(std::memory_order_acquire) & bit) return MOYE_OK;
+    MOYE_HIP_CHECK(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+    cap.raised.fetch_or(bit, std::memory_order_release);
+    return MOYE_OK;
+}
 
 inline int dtype_bytes(int32_t dt) {
     switch (dt) {

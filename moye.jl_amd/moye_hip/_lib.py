@@ -56,6 +56,11 @@ class TiledCopy(C.Structure):
                 ("val_shape", C.c_int32 * 2), ("tiler_mn", C.c_int32 * 2), ("flags", C.c_int32)]
 
 
+class GemmEpilogue(C.Structure):
+    _fields_ = [("alpha", C.c_float), ("beta", C.c_float), ("op", C.c_int32), ("_pad", C.c_int32),
+                ("operand", C.POINTER(Tensor)), ("scalar", C.c_double)]
+
+
 _lib = None
 
 
@@ -80,6 +85,8 @@ def _declare(l):
         "moye_copy": [P(TiledCopy), P(Tensor), P(Tensor), vp],
         "moye_copy_if": [P(Tensor), P(Tensor), P(Tensor), vp],
         "moye_gemm": [P(TiledMMA), P(Tensor), P(Tensor), P(Tensor), P(Tensor), C.c_float, vp],
+        "moye_gemm_ex": [P(TiledMMA), P(Tensor), P(Tensor), P(Tensor), P(Tensor), P(GemmEpilogue), vp, S, vp],
+        "moye_gemm_release_workspace": [],
         "moye_gemm_workspace_size": [P(TiledMMA), P(Tensor), P(Tensor), P(Tensor), P(S)],
         "moye_device_malloc": [P(vp), S], "moye_device_free": [vp],
         "moye_memcpy_h2d": [vp, vp, S], "moye_memcpy_d2h": [vp, vp, S], "moye_memset": [vp, C.c_int, S],

@@ -63,6 +63,30 @@ def gemm_(mma, D, A, B, C_=None, alpha=1.0, stream=None):
     check(lib().moye_gemm(C.byref(mma), C.byref(D), C.byref(A), C.byref(B), _ref(C_), alpha, stream))
 
 
+def gemm_epilogue(alpha=1.0, beta=0.0, op=_lib.MAP_IDENTITY, operand=None, scalar=0.0):
+    """A moye_gemm_epilogue: D = op(alpha * A * B' + beta * C, operand or scalar), every step rounded in fp32.
+    Keeps `operand` (a moye_tensor) alive through the attribute `_operand`."""
+    e = _lib.GemmEpilogue()
+    e.alpha, e.beta, e.op, e.scalar = alpha, beta, op, scalar
+    if operand is not None:
+        e._operand = operand
+        e.operand = C.pointer(operand)
+    return e
+
+
+def gemm_ex_(mma, D, A, B, C_=None, epilogue=None, workspace=None, workspace_bytes=0, stream=None):
+    """gemm! with a fused epilogue and a caller-provided workspace (a device pointer as int, or None); never
+    allocates."""
+    ep = epilogue if epilogue is not None else gemm_epilogue()
+    check(lib().moye_gemm_ex(C.byref(mma), C.byref(D), C.byref(A), C.byref(B), _ref(C_), C.byref(ep), workspace,
+                             workspace_bytes, stream))
+
+
+def gemm_release_workspace():
+    """Frees the per-stream workspaces moye_gemm keeps (waits for the device first)."""
+    check(lib().moye_gemm_release_workspace())
+
+
 def gemm_workspace_size(mma, D, A, B):
     """Bytes of library-owned device workspace this gemm! call needs (K-major copies of operands that are not K-major,
     partial products of a split-K call); 0 for a plain TN call."""

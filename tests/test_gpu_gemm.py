@@ -1057,3 +1057,66 @@ def test_every_layout_of_c(mh, out_dt, flags):
     mh.gemm_(mma, T(d), T(a), T(b), T(d), 0.5)
     torch.cuda.synchronize()
     assert torch.equal(d.cpu().double(), want), "in place"
+
+
+# ---------------------------------------------------------------------------------------------
+# moye_gemm_ex: the workspace comes from the caller
+# ---------------------------------------------------------------------------------------------
+
+def test_gemm_ex_takes_the_callers_workspace(mh):
+    """Split-K partials and K-major copies go into the caller's buffer: same bits as moye_gemm with the library's own
+    workspace; a buffer that is too small, misaligned or missing is refused before anything is launched; two streams
+    with two workspaces do not disturb each other."""
+    from moye_hip import _lib
+    g = torch.Generator().manual_seed(90)
+    M, N, K = 256, 384, 2048
+    A = torch.randint(-4, 5, (M, K), generator=g).to(torch.float16)
+    B = torch.randint(-4, 5, (N, K), generator=g).to(torch.float16)
+    a, b = A.cuda(), B.cuda()
+    a_m = A.t().contiguous().cuda()
+    ref = A.double() @ B.double().t()
+    mma = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 2, 1), cta_tile=(128, 128, 32), split_k=4)
+    ta_m = T(a_m, (M, K), (1, M))
+    d = torch.zeros(M, N, device="cuda")
+    need = mh.gemm_workspace_size(mma, T(d), ta_m, T(b))
+    assert need >= 4 * M * N * 4 + M * K * 2
+    ws = torch.full((need + 256,), 0x5a, dtype=torch.uint8, device="cuda")
+    base = (ws.data_ptr() + 255) // 256 * 256
+    mh.gemm_ex_(mma, T(d), ta_m, T(b), None, mh.gemm_epilogue(alpha=0.5), base, need)
+    d_lib = torch.zeros(M, N, device="cuda")
+    mh.gemm_(mma, T(d_lib), ta_m, T(b), None, 0.5)
+    torch.cuda.synchronize()
+    assert torch.equal(d.cpu().double(), 0.5 * ref) and torch.equal(d, d_lib)
+    # refused: too small, misaligned, missing
+    for args in ((base, need - 256), (base + 16, need), (None, 0)):
+        with pytest.raises(mh.MoyeError) as e:
+            mh.gemm_ex_(mma, T(d), ta_m, T(b), None, None, *args)
+        assert e.value.status in (_lib.ERR_ARG, _lib.ERR_ALIGN)
+    # a plain TN call needs no workspace and may pass none
+    plain = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 2, 1), cta_tile=(128, 128, 32))
+    d.zero_()
+    mh.gemm_ex_(plain, T(d), T(a), T(b))
+    torch.cuda.synchronize()
+    assert torch.equal(d.cpu().double(), ref)
+    # two streams, each with its own workspace (and, through moye_gemm, each with the library's per-stream one)
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    ws2 = torch.zeros(need + 256, dtype=torch.uint8, device="cuda")
+    base2 = (ws2.data_ptr() + 255) // 256 * 256
+    B2 = torch.randint(-4, 5, (N, K), generator=g).to(torch.float16)
+    b2 = B2.cuda()
+    ref2 = A.double() @ B2.double().t()
+    d1, d2 = torch.zeros(M, N, device="cuda"), torch.zeros(M, N, device="cuda")
+    e1, e2 = torch.zeros(M, N, device="cuda"), torch.zeros(M, N, device="cuda")
+    torch.cuda.synchronize()
+    for _ in range(8):
+        mh.gemm_ex_(mma, T(d1), ta_m, T(b), None, None, base, need, stream=s1.cuda_stream)
+        mh.gemm_ex_(mma, T(d2), ta_m, T(b2), None, None, base2, need, stream=s2.cuda_stream)
+        mh.gemm_(mma, T(e1), ta_m, T(b), stream=s1.cuda_stream)
+        mh.gemm_(mma, T(e2), ta_m, T(b2), stream=s2.cuda_stream)
+    torch.cuda.synchronize()
+    assert torch.equal(d1.cpu().double(), ref) and torch.equal(d2.cpu().double(), ref2)
+    assert torch.equal(e1.cpu().double(), ref) and torch.equal(e2.cpu().double(), ref2)
+    mh.gemm_release_workspace()
+    mh.gemm_(mma, T(e1), ta_m, T(b))        # allocates afresh
+    torch.cuda.synchronize()
+    assert torch.equal(e1.cpu().double(), ref)

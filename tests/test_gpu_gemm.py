@@ -1120,3 +1120,60 @@ def test_gemm_ex_takes_the_callers_workspace(mh):
     mh.gemm_(mma, T(e1), ta_m, T(b))        # allocates afresh
     torch.cuda.synchronize()
     assert torch.equal(e1.cpu().double(), ref)
+
+
+# ---------------------------------------------------------------------------------------------
+# exactly what bench.py times, at the size it times
+# ---------------------------------------------------------------------------------------------
+
+def _bench_mma(mh):
+    """The descriptor of bench.py's headline leg: CTA tile 256x256x64, 2x4 waves, fp16 in and out."""
+    return mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 4, 1), tile=(256, 256, 64), cta_tile=(256, 256, 64))
+
+
+def test_bench_descriptor_f16_4096_against_fp64(mh):
+    """fp16 TN 4096^3, seed 1003, values normal(0,1)/sqrt(K), fp16 out, through the 256x256x64 kernel on all 256 CUs;
+    every row against the fp64 product of the rounded inputs: max|D - D64| / max|D64| <= 1e-2."""
+    M = N = K = 4096
+    g = torch.Generator().manual_seed(1003)
+    A = (torch.randn(M, K, generator=g) / K ** 0.5).half()
+    B = (torch.randn(N, K, generator=g) / K ** 0.5).half()
+    a, b = A.cuda(), B.cuda()
+    d = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+    mh.gemm_(_bench_mma(mh), T(d), T(a), T(b))
+    torch.cuda.synchronize()
+    c64 = a.double() @ b.double().t()
+    err = relerr(d, c64)
+    rows = np.random.default_rng(1).choice(M, 32, replace=False)
+    host = A[rows].double().numpy() @ B.double().numpy().T               # the GPU fp64 product checked on the host
+    assert np.allclose(c64[rows].cpu().numpy(), host, rtol=1e-12, atol=1e-12)
+    ref = to.gemm_universal_fma(A[rows[:8]].float().numpy(), B.float().numpy(), np.zeros((8, N), np.float32),
+                                "f16", "f16").astype(np.float16)
+    print("bench descriptor f16 4096^3 (256x256x64): rel err %.3e (reference arithmetic on 8 rows: %.3e)"
+          % (err, to.relerr(ref, host[:8])))
+    assert err <= TOL16
+    # the named tile of the baseline's config 3 gives the same product up to the order of the sum
+    d128 = torch.zeros_like(d)
+    mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 2, 1), cta_tile=(128, 128, 32)), T(d128), T(a), T(b))
+    torch.cuda.synchronize()
+    assert relerr(d128, c64) <= TOL16
+    assert float((d.double() - d128.double()).abs().max()) <= 2 ** -8 * float(c64.abs().max())
+
+
+@pytest.mark.parametrize("out_dt", ["float16", "float32"])
+def test_bench_descriptor_every_cta_exact_on_integers(mh, out_dt):
+    """4096 x 4096 x 512 on small integers through the bench descriptor: all 256 CTA positions of the XCD-aware
+    order, non-temporal stores on, bit for bit (every product and sum is exact in fp32 and in fp16)."""
+    out_dt = getattr(torch, out_dt)
+    M = N = 4096
+    K = 512
+    g = torch.Generator().manual_seed(1103)
+    A = torch.randint(-2, 3, (M, K), generator=g).half()
+    B = torch.randint(-2, 3, (N, K), generator=g).half()
+    a, b = A.cuda(), B.cuda()
+    d = torch.full((M, N), float("nan"), dtype=out_dt, device="cuda")
+    mh.gemm_(_bench_mma(mh), T(d), T(a), T(b))
+    torch.cuda.synchronize()
+    want = (a.float() @ b.float().t())           # exact: |sum| <= 4 * 512 = 2048, an integer fp16 holds
+    assert float(want.abs().max()) <= 2048
+    assert torch.equal(d.float(), want)

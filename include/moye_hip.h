@@ -217,6 +217,17 @@ int32_t moye_gemm_ex(const moye_tiled_mma* mma, const moye_tensor* D, const moye
                      const moye_tensor* B, const moye_tensor* C, const moye_gemm_epilogue* ep,
                      void* workspace, size_t workspace_bytes, void* stream);
 
+/* gemm! for callers that cannot allocate device memory (code under HIP graph capture, serving loops, harnesses
+ * that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as moye_gemm, bit for bit;
+ * the workspace (split-K partial products, K-major copies of operands that are not K-major) is a static device
+ * array of MOYE_NOALLOC_SCRATCH_BYTES inside the library, one copy per GPU, held until the process ends.  A call
+ * that needs more (moye_gemm_workspace_size) fails with MOYE_ERR_ARG before anything is launched.  Never calls
+ * hipMalloc / hipFree or synchronises.  All calls on one GPU share that GPU's array: calls that overlap on one GPU
+ * (different streams, or host threads that do not order their launches) race; calls on one stream are safe. */
+#define MOYE_NOALLOC_SCRATCH_BYTES (32u << 20)
+int32_t moye_gemm_noalloc(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A,
+                          const moye_tensor* B, const moye_tensor* C, float alpha, void* stream);
+
 /* ---- host-side layout algebra (no GPU needed) ------------------------------------------- */
 /* Text form of a layout: `shape:stride`, `_n` = static int, `n` = dynamic int, e.g.
  * "(_2, (_1, _6)):(_1, (_6, _2))"; a bare shape means the compact column-major layout

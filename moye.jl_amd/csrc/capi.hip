@@ -97,6 +97,33 @@ static int32_t library_workspace(size_t bytes, hipStream_t st, char** out) {
     return MOYE_OK;
 }
 
+// ---- moye_gemm_noalloc: the workspace is a static device array ----------------------------------
+// For callers that cannot allocate (under graph capture, in serving loops): the split-K partial
+// products and the K-major operand copies go into this array instead of an allocated buffer.  Every
+// GPU the library runs on holds its own copy at its own address until the process ends; the address
+// is asked for once per device, with that device current, and only that address (never the array's
+// name, which on the host is a stand-in) is handed to kernels.
+constexpr size_t kScratchBytes = MOYE_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static char* g_scratch_ptr[kMaxDevices];
+
+static int32_t scratch_of_current_device(char** out) {
+    int dev = 0;
+    MOYE_HIP_CHECK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(MOYE_ERR_ARG, "moye_gemm_noalloc: device index %d beyond %d", dev, kMaxDevices - 1);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        MOYE_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return fail(MOYE_ERR_HIP, "moye_gemm_noalloc: the static scratch array has no address on device %d", dev);
+        g_scratch_ptr[dev] = static_cast<char*>(p);
+    }
+    *out = g_scratch_ptr[dev];
+    return MOYE_OK;
+}
+
 // bytes of a K-major copy of an (rows x K) operand: row pitch rounded up to 16 bytes
 static size_t kmajor_bytes(const Mat& m) {
     const int eb = dtype_bytes(m.dtype);
@@ -329,6 +356,21 @@ int32_t moye_gemm_ex(const moye_tiled_mma* mma, const moye_tensor* D, const moye
     alignas(256) static char nothing[256];
     return gemm_impl(mma, D, A, B, C, ep->alpha, workspace ? static_cast<char*>(workspace) : nothing, workspace_bytes,
                      static_cast<hipStream_t>(stream));
+}
+
+int32_t moye_gemm_noalloc(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A, const moye_tensor* B,
+                          const moye_tensor* C, float alpha, void* stream) {
+    if (!mma || !D || !A || !B) return fail(MOYE_ERR_ARG, "moye_gemm_noalloc: null argument");
+    size_t need = 0;
+    if (int32_t e = moye_gemm_workspace_size(mma, D, A, B, &need)) return e;
+    if (need > kScratchBytes)
+        return fail(MOYE_ERR_ARG, "moye_gemm_noalloc: this call needs %zu bytes of workspace, the static scratch array holds %zu; "
+                                  "use moye_gemm_ex with a workspace of the caller's", need, kScratchBytes);
+    char* ws = nullptr;
+    if (int32_t e = scratch_of_current_device(&ws)) return e;
+    // every byte of the scratch a call reads it has written before (whole K-major copies, whole partial products), so
+    // nothing needs clearing between calls
+    return gemm_impl(mma, D, A, B, C, alpha, ws, kScratchBytes, static_cast<hipStream_t>(stream));
 }
 
 int32_t moye_gemm_release_workspace(void) {

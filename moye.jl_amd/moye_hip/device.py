@@ -82,6 +82,15 @@ def gemm_ex_(mma, D, A, B, C_=None, epilogue=None, workspace=None, workspace_byt
                              workspace_bytes, stream))
 
 
+NOALLOC_SCRATCH_BYTES = 32 << 20
+
+
+def gemm_noalloc_(mma, D, A, B, C_=None, alpha=1.0, stream=None):
+    """gemm! whose workspace is the library's static device array (moye_gemm_noalloc): allocates nothing; fails when
+    the call needs more than NOALLOC_SCRATCH_BYTES."""
+    check(lib().moye_gemm_noalloc(C.byref(mma), C.byref(D), C.byref(A), C.byref(B), _ref(C_), alpha, stream))
+
+
 def gemm_release_workspace():
     """Frees the per-stream workspaces moye_gemm keeps (waits for the device first)."""
     check(lib().moye_gemm_release_workspace())

@@ -114,6 +114,67 @@ static int32_t launch_transpose(const uint32_t* s, uint32_t* d, int64_t lds_, in
     return MOYE_OK;
 }
 
+// The form for large matrices: a workgroup moves GJ tiles that are neighbours along the DESTINATION's contiguous index
+// (64 destination rows of GJ * 256 bytes each) and workgroups are numbered along that index first, so consecutive
+// workgroups complete whole destination rows: 64 x ldd elements of contiguous memory per tj / GJ workgroups.  On this
+// part writes are the side that needs the locality (measured on 16384^2, one side at a time with the other left out:
+// reads of 256-byte pieces a pitch apart run at 6.9 TB/s whatever the order; writes run at 6.6-6.9 TB/s in this order
+// against 5.1 with the source-contiguous index first), and fewer workgroups in flight do better than more: one per CU
+// (6.25 TB/s) against two (6.15) or five (5.85), hence the LDS request above what the tiles need.
+template <int GJ>
+__global__ __launch_bounds__(256) void transpose_lds_b32_rows(const uint32_t* __restrict__ src, uint32_t* __restrict__ dst,
+                                                              int64_t lds_, int64_t ldd, int groups_j, int64_t bs_src,
+                                                              int64_t bs_dst) {
+    extern __shared__ u32x4 tile[];  // GJ tiles of 64 x 16 chunks
+    src += (int64_t)blockIdx.y * bs_src;
+    dst += (int64_t)blockIdx.y * bs_dst;
+    const int gj = blockIdx.x % groups_j, ti = blockIdx.x / groups_j;
+    const int lane16 = threadIdx.x & 15;  // chunk of 4 along the contiguous index of the side being accessed
+    const int grp = threadIdx.x >> 4;     // 0..15
+
+    // ---- load: source rows j = 64 b + 4 grp + q of the group, elements i = 4 lane16 .. +3 of tile column ti ----
+    const uint32_t* s = src + ((int64_t)gj * GJ * kTile + 4 * grp) * lds_ + (int64_t)ti * kTile + 4 * lane16;
+    u32x4 v[GJ][4];
+#pragma unroll
+    for (int b = 0; b < GJ; ++b)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            v[b][q] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(s + (int64_t)(b * kTile + q) * lds_));
+#pragma unroll
+    for (int b = 0; b < GJ; ++b)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int row = 4 * lane16 + e;  // i within the tile
+            tile[b * 1024 + row * 16 + lds_chunk<true>(row, grp)] = u32x4{v[b][0][e], v[b][1][e], v[b][2][e], v[b][3][e]};
+        }
+    __syncthreads();
+    // ---- store: destination rows i = grp + 16 p, elements j = 64 b + 4 lane16 .. +3 ----
+    uint32_t* d = dst + ((int64_t)ti * kTile + grp) * ldd + (int64_t)gj * GJ * kTile + 4 * lane16;
+#pragma unroll
+    for (int p = 0; p < 4; ++p)
+#pragma unroll
+        for (int b = 0; b < GJ; ++b) {
+            const int row = grp + 16 * p;
+            const u32x4 w = tile[b * 1024 + row * 16 + lds_chunk<true>(row, lane16)];
+            __builtin_nontemporal_store(w, reinterpret_cast<u32x4*>(d + (int64_t)(16 * p) * ldd + b * kTile));
+        }
+}
+
+template <int GJ>
+static int32_t launch_transpose_rows(const uint32_t* s, uint32_t* d, int64_t lds_, int64_t ldd, int ti, int tj, hipStream_t st,
+                                     int64_t bs_src = 0, int64_t bs_dst = 0, int batch = 1) {
+    auto kern = transpose_lds_b32_rows<GJ>;
+    constexpr int kLds = 96 * 1024;  // the tiles need GJ * 16 KiB; more than half of a CU's 160 KiB keeps it to one workgroup per CU
+    static_assert(GJ * kTile * kTile * 4 <= kLds, "tiles fit");
+    static LdsCap cap;
+    if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
+    const int64_t groups = (int64_t)ti * (tj / GJ);
+    if (groups > 0x7fffffff) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles");
+    kern<<<dim3((unsigned)groups, (unsigned)batch), 256, kLds, st>>>(s, d, lds_, ldd, tj / GJ, bs_src, bs_dst);
+    MOYE_HIP_CHECK(hipGetLastError());
+    return MOYE_OK;
+}
+
 // ------------------------------------------------------------------------------------------
 // the same for 2-byte elements (fp16 / bf16 matrices)
 // ------------------------------------------------------------------------------------------
@@ -683,19 +744,35 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
             const uint32_t* s32 = reinterpret_cast<const uint32_t*>(s_);
             uint32_t* d32 = reinterpret_cast<uint32_t*>(d_);
             if (tc && (tc->flags & MOYE_GEMM_NO_LDS_SWIZZLE)) return launch_transpose<false, 1>(s32, d32, lds_, ldd, ti, tj, st, bs, bd, batch);
+            // Destination rows first (transpose_lds_b32_rows) when the source's contiguous extent is at least the destination's
+            // and 2048 or more; measured, TB/s, source-first / destination-first order: 16384^2 5.68 / 6.25, 12288^2 5.20 / 5.94,
+            // 4096^2 x 16 5.81 / 6.02, 2048^2 x 64 6.30 / 6.48, 32768 x 4096 4.33 / 6.39; the other way round 4096 x 32768
+            // 5.58 / 5.08, 2048 x 65536 5.77 / 4.52, 1024^2 x 128 6.03 / 5.86.  MOYE_TRANSPOSE_ROWS=0|1 forces the choice (tuning).
+            static const int rows_env = getenv("MOYE_TRANSPOSE_ROWS") ? atoi(getenv("MOYE_TRANSPOSE_ROWS")) : -1;
+            if (tj % 4 == 0 && (rows_env >= 0 ? rows_env != 0 : (ni >= nj && ni >= 2048)))
+                return launch_transpose_rows<4>(s32, d32, lds_, ldd, ti, tj, st, bs, bd, batch);
             if (ti % 4 == 0) return launch_transpose<true, 4>(s32, d32, lds_, ldd, ti, tj, st, bs, bd, batch);
             if (ti % 2 == 0) return launch_transpose<true, 2>(s32, d32, lds_, ldd, ti, tj, st, bs, bd, batch);
             return launch_transpose<true, 1>(s32, d32, lds_, ldd, ti, tj, st, bs, bd, batch);
         };
-        // (2) rank-2 transpose of 4-byte elements through the LDS tile
-        const int tm = tc && tc->tiler_mn[0] ? tc->tiler_mn[0] : kTile;
-        const int tn = tc && tc->tiler_mn[1] ? tc->tiler_mn[1] : kTile;
+        // (2) rank-2 transpose of 1-, 2- and 4-byte elements through LDS patches
+        bool lds_pair = false;  // a rank-2 pair with the unit strides on different modes: what the LDS-tiled op is for
+        // The tiler of the descriptor (tiler_MN of make_tiled_copy, src/atom/copy.jl:249-258; 32 x 32 in the reference's own
+        // transpose kernel, test/host/copy_async.jl:51-76) must divide the array, as zipped_divide asserts; how the kernels
+        // group elements into LDS patches (64 x 64, several per workgroup) is their own business and changes no result.
+        if (tc && tc->op == MOYE_COPY_LDS_TILED && src->rank >= 2) {
+            for (int m = 0; m < 2; ++m)
+                if (tc->tiler_mn[m] < 0 || (tc->tiler_mn[m] > 0 && src->shape[m] % tc->tiler_mn[m]))
+                    return fail(MOYE_ERR_SHAPE, "copyto!: tiler extent %d does not divide mode %d of size %lld", tc->tiler_mn[m], m + 1,
+                                (long long)src->shape[m]);
+        }
         if ((sb == 4 || sb == 2 || sb == 1) && src->rank == 2 && dst->rank == 2 && src->shape[0] == dst->shape[0] &&
-            src->shape[1] == dst->shape[1] && tm == kTile && tn == kTile) {
+            src->shape[1] == dst->shape[1]) {
             const moye_tensor *a = src, *b = dst;
             bool ok = false, swap = false;
             if (a->stride[0] == 1 && b->stride[1] == 1) ok = true;
             else if (a->stride[1] == 1 && b->stride[0] == 1) ok = swap = true;
+            lds_pair = ok;
             if (ok) {
                 // normalise to: i = contiguous index of src, j = contiguous index of dst
                 const int mi = swap ? 1 : 0, mj = swap ? 0 : 1;
@@ -712,7 +789,7 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
                 // touches one page per row of the other side, so it costs far more per byte than the interior: 16400 x 16392
                 // fp32 runs at 3.3 TB/s against 5.6 for 16384 x 16384; whole tiles pushed against the edge cost the same.)
                 const int64_t ni0 = ni / kTile * kTile, nj0 = nj / tile_j * tile_j;
-                if (!(tc && tc->op == MOYE_COPY_LDS_TILED) && ni0 > 0 && nj0 > 0 && lds_ % per16 == 0 && ldd % per16 == 0 &&
+                if (ni0 > 0 && nj0 > 0 && lds_ % per16 == 0 && ldd % per16 == 0 &&
                     lds_ >= ni && ldd >= nj && (reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d)) % 16 == 0) {
                     // sub-array [i0, i0 + ci) x [j0, j0 + cj) of both sides
                     auto part = [&](int64_t i0, int64_t ci, int64_t j0, int64_t cj) -> int32_t {
@@ -723,7 +800,9 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
                             t->shape[mi] = ci;
                             t->shape[mj] = cj;
                         }
-                        return copy_if_dispatch(tc, &pd, &ps, nullptr, st);
+                        // the strips are not whole patches: they go through the general kernel whatever the descriptor says
+                        const bool interior = i0 == 0 && j0 == 0 && ci == ni0 && cj == nj0;
+                        return copy_if_dispatch(interior ? tc : nullptr, &pd, &ps, nullptr, st);
                     };
                     if (int32_t e = part(0, ni0, 0, nj0)) return e;
                     if (int32_t e = part(ni0, ni - ni0, 0, nj)) return e;
@@ -755,7 +834,7 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
                 {
                     const int64_t ni = src->shape[mi], nj = src->shape[mj], lds_ = src->stride[mj], ldd = dst->stride[mi];
                     const int per16 = 16 / sb, tile_j = sb == 1 ? kTileJ8 : kTile;
-                    if (nbatch_modes == 1 && batch <= 65535 && tm == kTile && tn == kTile && ni % kTile == 0 && nj % tile_j == 0 && lds_ % per16 == 0 && ldd % per16 == 0 &&
+                    if (nbatch_modes == 1 && batch <= 65535 && ni % kTile == 0 && nj % tile_j == 0 && lds_ % per16 == 0 && ldd % per16 == 0 &&
                         lds_ >= ni && ldd >= nj && src->stride[bm] % per16 == 0 && dst->stride[bm] % per16 == 0 &&
                         (reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d)) % 16 == 0)
                         return tiled_launch(s, d, ni, nj, lds_, ldd, src->stride[bm], dst->stride[bm], (int)batch);
@@ -785,10 +864,11 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
                 }
             }
         }
-        if (tc && tc->op == MOYE_COPY_LDS_TILED)
+        // a pair the LDS-tiled op is meant for, but smaller than a patch or not 16-byte aligned: the general kernel moves it
+        if (tc && tc->op == MOYE_COPY_LDS_TILED && !lds_pair)
             return fail(MOYE_ERR_UNSUPPORTED,
-                        "copyto!: the LDS-tiled copy needs rank-2 operands of 2- or 4-byte elements whose sizes are multiples of "
-                        "64, 16-byte aligned, with the unit stride on different modes");
+                        "copyto!: the LDS-tiled copy takes rank-2 operands (or a batch of them) of 1-, 2- or 4-byte elements "
+                        "with the unit stride on different modes");
     }
 
     // (3) generic

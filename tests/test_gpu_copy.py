@@ -325,8 +325,13 @@ def test_copy_errors(mh):
         mh.copyto_(_tens(mh, a, (8, 8), (1, 8)), _tens(mh, af, (8, 8), (1, 8)))
     assert e.value.status == mh._lib.ERR_UNSUPPORTED
     tc = mh.tiled_copy_desc(op=mh.COPY_LDS_TILED, tiler=(64, 64))
-    with pytest.raises(mh.MoyeError) as e:  # 8x8 is not a multiple of the 64x64 LDS tile
+    with pytest.raises(mh.MoyeError) as e:  # the 64x64 tiler does not divide 8x8 (zipped_divide's assertion)
         mh.copyto_(_tens(mh, a, (8, 8), (8, 1)), _tens(mh, a, (8, 8), (1, 8)), tc)
+    assert e.value.status == mh._lib.ERR_SHAPE
+    with pytest.raises(mh.MoyeError) as e:  # both sides with the unit stride on the same mode: not what the op is for
+        wide = torch.zeros(128, dtype=torch.int32, device="cuda")
+        mh.copyto_(_tens(mh, torch.zeros_like(wide), (8, 8), (1, 16)), _tens(mh, wide, (8, 8), (1, 16)),
+                   mh.tiled_copy_desc(op=mh.COPY_LDS_TILED, tiler=(8, 8)))
     assert e.value.status == mh._lib.ERR_UNSUPPORTED
     empty = torch.zeros(0, dtype=torch.int32, device="cuda")
     mh.copyto_(_tens(mh, empty, (0,), (1,)), _tens(mh, empty, (0,), (1,)))
@@ -713,3 +718,43 @@ def test_batches_of_transposes(mh, dt):
         mh.copyto_(_tens(mh, d_d, shape, dstr), _tens(mh, s_d, shape, sstr))
         torch.cuda.synchronize()
         assert torch.equal(d_d.cpu().view(torch.uint8), want.view(torch.uint8)), (shape, dstr, sstr)
+
+
+@pytest.mark.parametrize("tiler", [(32, 32), (64, 64), (16, 128), (8, 8), (0, 0)])
+def test_lds_tiled_copy_takes_any_tiler_that_divides(mh, tiler):
+    """The reference's own transpose kernel tiles 32 x 32 with 256 threads (test/host/copy_async.jl:51-76): the tiler
+    of the descriptor only has to divide the array; closed form dst[j, i] == src[i, j] bit for bit, for sizes that are
+    whole 64 x 64 patches, sizes that leave strips, and an array smaller than a patch."""
+    for (M, N) in ((2048, 4096), (4096, 2048), (96, 160), (32, 32), (2048 + 32, 2048)):
+        if tiler[0] and (M % tiler[0] or N % tiler[1]):
+            continue
+        src = _rand_bits(M * N, 31 + M)
+        dst = torch.zeros_like(src)
+        tc = mh.tiled_copy_desc(op=mh.COPY_LDS_TILED, vec_bits=128, thr_shape=(32, 8), val_shape=(1, 1), tiler=tiler)
+        mh.copyto_(_tens(mh, dst, (M, N), (N, 1)), _tens(mh, src, (M, N), (1, M)), tc)
+        torch.cuda.synchronize()
+        assert torch.equal(dst.view(M, N), src.view(N, M).t()), (M, N, tiler)
+    if tiler[0] > 8:
+        src = _rand_bits(24 * 24, 5)
+        with pytest.raises(mh.MoyeError) as e:
+            mh.copyto_(_tens(mh, torch.zeros_like(src), (24, 24), (24, 1)), _tens(mh, src, (24, 24), (1, 24)),
+                       mh.tiled_copy_desc(op=mh.COPY_LDS_TILED, tiler=tiler))
+        assert e.value.status == mh._lib.ERR_SHAPE
+
+
+def test_transpose_destination_rows_first_and_source_first_agree(mh):
+    """Large matrices take the kernel that completes destination rows first, matrices whose destination rows are the
+    longer side the one that walks the source first: both against the closed form, bit for bit, on shapes either side
+    of the rule, and on a batch."""
+    for (ni, nj) in ((4096, 2048), (2048, 4096), (2048, 2048), (8192, 1024), (1024, 8192), (2304, 2304)):
+        src = _rand_bits(ni * nj, ni + nj)
+        dst = torch.zeros_like(src)
+        mh.copyto_(_tens(mh, dst, (ni, nj), (nj, 1)), _tens(mh, src, (ni, nj), (1, ni)))
+        torch.cuda.synchronize()
+        assert torch.equal(dst.view(ni, nj), src.view(nj, ni).t()), (ni, nj)
+    ni = nj = 2048
+    src = _rand_bits(ni * nj * 3, 77)
+    dst = torch.zeros_like(src)
+    mh.copyto_(_tens(mh, dst, (ni, nj, 3), (nj, 1, ni * nj)), _tens(mh, src, (ni, nj, 3), (1, ni, ni * nj)))
+    torch.cuda.synchronize()
+    assert torch.equal(dst.view(3, ni, nj), src.view(3, nj, ni).transpose(1, 2))

@@ -21,11 +21,13 @@ COMMON = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-
 SOURCES = {
     "capi.hip": [],
     "copy_kernels.hip": [],
-    "gemm_mfma.hip": [],
-    "gemm_mfma256.hip": [],
-    "gemm_mfma256pp.hip": [],
-    "gemm_mfma256w4.hip": [],
-    "gemm_mfma_skinny.hip": [],
+    # the epilogue's alpha * acc + beta * c is two products and a sum, each rounded (the oracle composes it from axpby!):
+    # never contracted into fused operations
+    "gemm_mfma.hip": ["-ffp-contract=off"],
+    "gemm_mfma256.hip": ["-ffp-contract=off"],
+    "gemm_mfma256pp.hip": ["-ffp-contract=off"],
+    "gemm_mfma256w4.hip": ["-ffp-contract=off"],
+    "gemm_mfma_skinny.hip": ["-ffp-contract=off"],
     "mfma_ceiling.hip": [],
     "elementwise.hip": ["-ffp-contract=off"],      # axpby!: rounded products, unfused sum
     "gemm_universal.hip": ["-ffp-contract=off"],   # UniversalFMA: mul then add, never fused
@@ -74,7 +76,7 @@ def check_accumulator_hazards(src, force=False):
     asm = os.path.join(CSRC, "build", os.path.splitext(src)[0] + ".s")
     if not force and not _stale(asm, [path] + _headers()):
         return
-    cmd = [HIPCC] + COMMON + ["-S", "--cuda-device-only", path, "-o", asm]
+    cmd = [HIPCC] + COMMON + SOURCES.get(src, []) + ["-S", "--cuda-device-only", path, "-o", asm]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("hipcc -S failed for %s:\n%s" % (src, r.stdout + r.stderr))

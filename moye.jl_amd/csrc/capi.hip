@@ -177,12 +177,24 @@ static bool rows_in_16_byte_pieces(const void* c, int64_t ld_m, int64_t ld_n, in
     return c && ld_n == 1 && reinterpret_cast<uintptr_t>(c) % 16 == 0 && (ld_m * dtype_bytes(dt)) % 16 == 0;
 }
 
+// gemm!(mma, D, A, B, C) as moye_gemm has always computed it: D = alpha * A * B' + C
+static moye_gemm_epilogue plain_epilogue(float alpha) {
+    moye_gemm_epilogue e{};
+    e.alpha = alpha;
+    e.beta = 1.f;
+    e.op = MOYE_MAP_IDENTITY;
+    return e;
+}
+
 // `caller_ws` / `caller_ws_bytes`: the workspace when the caller brings one (it must hold what
 // moye_gemm_workspace_size reports); with caller_ws == nullptr the library's own is used.
 static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const moye_tensor* tA,
-                         const moye_tensor* tB, const moye_tensor* tC, float alpha, char* caller_ws,
+                         const moye_tensor* tB, const moye_tensor* tC, const moye_gemm_epilogue& ep, char* caller_ws,
                          size_t caller_ws_bytes, hipStream_t st) {
     if (!mma) return fail(MOYE_ERR_ARG, "gemm!: null TiledMMA descriptor");
+    const float alpha = ep.alpha;
+    if (ep.beta == 0.f) tC = nullptr;  // axpby!'s iszero(b): C is not read
+    if (ep.op < MOYE_MAP_IDENTITY || ep.op > MOYE_MAP_ABS) return fail(MOYE_ERR_UNSUPPORTED, "gemm!: unknown epilogue operation %d", ep.op);
     Mat A, B, C{}, D;
     if (int32_t e = as_matrix(tA, "A", &A)) return e;
     if (int32_t e = as_matrix(tB, "B", &B)) return e;
@@ -204,6 +216,9 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
     if (mma->atom == MOYE_MMA_UNIVERSAL_FMA) {
         if (mma->split_k > 1)
             return fail(MOYE_ERR_UNSUPPORTED, "gemm!: UniversalFMA sums k in ascending order (src/algorithm/blas.jl:63-67); split_k would change that");
+        if (ep.op != MOYE_MAP_IDENTITY || (tC && ep.beta != 1.f))
+            return fail(MOYE_ERR_UNSUPPORTED, "gemm!: UniversalFMA accumulates onto C as the reference does (src/algorithm/blas.jl:39-88): "
+                                              "beta other than 0 or 1 and element-wise epilogue operations belong to the MFMA atoms");
         UArgs u{A.ptr, B.ptr, tC ? C.ptr : nullptr, D.ptr, M, N, K, A.rs, A.cs, B.rs, B.cs,
                 C.rs, C.cs, D.rs, D.cs, alpha, A.dtype, B.dtype, tC ? C.dtype : D.dtype, D.dtype};
         return gemm_universal_dispatch(bm, bn, bk, u, st);
@@ -247,6 +262,20 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
         }
     }
     GemmArgs g{};
+    g.beta = ep.beta;
+    g.ep_op = ep.op;
+    g.ep_scalar = (float)ep.scalar;
+    const bool binary_op = ep.op != MOYE_MAP_IDENTITY && ep.op != MOYE_MAP_NEG && ep.op != MOYE_MAP_ABS;
+    Mat X{};
+    if (binary_op && ep.operand) {
+        if (int32_t e = as_matrix(ep.operand, "epilogue operand", &X)) return e;
+        if (X.rows != D.rows || X.cols != D.cols)
+            return fail(MOYE_ERR_SHAPE, "gemm!: the epilogue operand is (%lld,%lld), D is (%lld,%lld); repeat a vector with a stride of 0",
+                        (long long)X.rows, (long long)X.cols, (long long)D.rows, (long long)D.cols);
+        if (X.dtype != MOYE_F32 && X.dtype != D.dtype)
+            return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the epilogue operand holds f32 or D's element type, not %s", dtype_name(X.dtype));
+        g.ep_x = X.ptr; g.ep_xdt = X.dtype; g.ep_xm = X.rs; g.ep_xn = X.cs;
+    }
     // TiledMMA.atom_layout_mnk = how many waves tile the CTA along M and N (src/atom/mma.jl:84)
     const int waves = mma->atom_layout_mnk[0] * mma->atom_layout_mnk[1];
     g.alpha = alpha;
@@ -279,12 +308,15 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
             return fail(MOYE_ERR_SHAPE, "gemm!: split_k = %d needs K = %d to split into equal ranges of whole 16-byte pieces", split, K);
         const int Ks = K / split;
         float* P = reinterpret_cast<float*>(ws);
-        g.alpha = 1.f; g.K = Ks; g.M = M; g.N = N; g.lda = A.rs; g.ldb = B.rs; g.ldd = N; g.C = nullptr;
+        GemmArgs r = g;  // the epilogue belongs to the second pass
+        r.C = tC ? C.ptr : nullptr; r.ldc_m = C.rs; r.ldc_n = C.cs; r.D = D.ptr; r.ldd = D.rs; r.ldd_n = D.cs;
+        g.alpha = 1.f; g.beta = 0.f; g.ep_op = MOYE_MAP_IDENTITY; g.ep_x = nullptr;
+        g.K = Ks; g.M = M; g.N = N; g.lda = A.rs; g.ldb = B.rs; g.ldd = N; g.C = nullptr;
         g.A = A.ptr; g.B = B.ptr; g.D = P;
         g.split = split; g.split_ab = (int64_t)Ks * eb; g.split_d = (int64_t)M * N * (int64_t)sizeof(float);
         g.xcd_swizzle &= ~kGemmStreamD;  // the partial products are read back at once
         if (int32_t e = gemm_mfma_tn_dispatch(in_dt, MOYE_F32, bm, bn, bk, waves, mma->stages, g, st)) return e;
-        return splitk_reduce_dispatch(P, split, M, N, alpha, tC ? C.ptr : nullptr, C.rs, C.cs, D.ptr, D.rs, D.cs, D.dtype, st);
+        return splitk_reduce_dispatch(P, split, M, N, r, D.dtype, st);
     }
     if (D.cs == 1) {  // row-major D
         g.A = A.ptr; g.B = B.ptr; g.M = M; g.N = N; g.lda = A.rs; g.ldb = B.rs; g.ldd = D.rs;
@@ -301,6 +333,7 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
     if (D.rs == 1) {  // column-major D: D' = B * A' is row-major
         g.A = B.ptr; g.B = A.ptr; g.M = N; g.N = M; g.lda = B.rs; g.ldb = A.rs; g.ldd = D.cs;
         g.C = tC ? C.ptr : nullptr; g.ldc_m = C.cs; g.ldc_n = C.rs; g.D = D.ptr;
+        std::swap(g.ep_xm, g.ep_xn);  // the kernel's m is the caller's n
         if (rows_in_16_byte_pieces(g.C, g.ldc_m, g.ldc_n, D.dtype)) g.xcd_swizzle |= kGemmRowC;
         return gemm_mfma_tn_dispatch(in_dt, D.dtype, bn, bm, bk, waves, mma->stages, g, st);
     }
@@ -342,7 +375,7 @@ int32_t moye_copy(const moye_tiled_copy* tc, const moye_tensor* dst, const moye_
 
 int32_t moye_gemm(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A, const moye_tensor* B,
                   const moye_tensor* C, float alpha, void* stream) {
-    return gemm_impl(mma, D, A, B, C, alpha, nullptr, 0, static_cast<hipStream_t>(stream));
+    return gemm_impl(mma, D, A, B, C, plain_epilogue(alpha), nullptr, 0, static_cast<hipStream_t>(stream));
 }
 
 int32_t moye_gemm_ex(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A, const moye_tensor* B,
@@ -350,11 +383,9 @@ int32_t moye_gemm_ex(const moye_tiled_mma* mma, const moye_tensor* D, const moye
                      void* stream) {
     if (!ep) return fail(MOYE_ERR_ARG, "moye_gemm_ex: null epilogue descriptor");
     if (!workspace && workspace_bytes) return fail(MOYE_ERR_ARG, "moye_gemm_ex: null workspace of %zu bytes", workspace_bytes);
-    if (ep->beta != 0.f || ep->op != MOYE_MAP_IDENTITY)
-        return fail(MOYE_ERR_UNSUPPORTED, "moye_gemm_ex: beta and the element-wise operation are not built yet");
     // a call that needs no workspace may pass none; one that needs it and passes none fails: this entry never allocates
     alignas(256) static char nothing[256];
-    return gemm_impl(mma, D, A, B, C, ep->alpha, workspace ? static_cast<char*>(workspace) : nothing, workspace_bytes,
+    return gemm_impl(mma, D, A, B, C, *ep, workspace ? static_cast<char*>(workspace) : nothing, workspace_bytes,
                      static_cast<hipStream_t>(stream));
 }
 
@@ -370,7 +401,7 @@ int32_t moye_gemm_noalloc(const moye_tiled_mma* mma, const moye_tensor* D, const
     if (int32_t e = scratch_of_current_device(&ws)) return e;
     // every byte of the scratch a call reads it has written before (whole K-major copies, whole partial products), so
     // nothing needs clearing between calls
-    return gemm_impl(mma, D, A, B, C, alpha, ws, kScratchBytes, static_cast<hipStream_t>(stream));
+    return gemm_impl(mma, D, A, B, C, plain_epilogue(alpha), ws, kScratchBytes, static_cast<hipStream_t>(stream));
 }
 
 int32_t moye_gemm_release_workspace(void) {
@@ -465,7 +496,7 @@ int32_t moye_time_gemm(const moye_tiled_mma* mma, const moye_tensor* D, const mo
                        const moye_tensor* C, float alpha, void* stream, int32_t warmup, int32_t iters,
                        float* ms_per_launch) {
     hipStream_t st = static_cast<hipStream_t>(stream);
-    return time_launches([&] { return gemm_impl(mma, D, A, B, C, alpha, nullptr, 0, st); }, st, warmup, iters, ms_per_launch);
+    return time_launches([&] { return gemm_impl(mma, D, A, B, C, plain_epilogue(alpha), nullptr, 0, st); }, st, warmup, iters, ms_per_launch);
 }
 
 int32_t moye_time_copy(const moye_tiled_copy* tc, const moye_tensor* dst, const moye_tensor* src, void* stream,

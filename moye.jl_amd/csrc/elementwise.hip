@@ -14,31 +14,29 @@
 
 namespace moye {
 
-// Second pass of a split-K gemm!: D[m][n] = cvt(alpha * (P_0 + P_1 + ... )[m][n] + C[m][n]).  The partial
-// products P_s are fp32, compact, with n contiguous and one after the other; they are summed in ascending s,
-// so the result does not depend on timing.
+// Second pass of a split-K gemm!: D[m][n] = cvt(epilogue(P_0 + P_1 + ... )[m][n]).  The partial products P_s are
+// fp32, compact, with n contiguous and one after the other; they are summed in ascending s, so the result does not
+// depend on timing.  The epilogue (alpha, beta * C, op) is the one the GEMM kernels apply, epi_value().
 template <typename Out>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ P, int split, int64_t M, int64_t N,
-                                                            float alpha, const void* C, int64_t c_rs, int64_t c_cs,
-                                                            void* D, int64_t d_rs, int64_t d_cs) {
+                                                            GemmArgs e) {
     const int64_t total = M * N;
+    const int64_t d_cs = e.ldd_n ? e.ldd_n : 1;
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
         float sum = P[i];
         for (int s = 1; s < split; ++s) sum += P[(int64_t)s * total + i];
         const int64_t m = i / N, n = i % N;
-        float x = sum * alpha;
-        if (C) x += Out::load(C, m * c_rs + n * c_cs);
-        static_cast<typename Out::type*>(D)[m * d_rs + n * d_cs] = Out::cvt(x);
+        const float c = e.C ? Out::load(e.C, m * e.ldc_m + n * e.ldc_n) : 0.f;
+        static_cast<typename Out::type*>(e.D)[m * e.ldd + n * d_cs] = Out::cvt(epi_value(e, sum, e.C != nullptr, c, m, n));
     }
 }
 
-int32_t splitk_reduce_dispatch(const float* P, int split, int64_t M, int64_t N, float alpha, const void* C, int64_t c_rs,
-                               int64_t c_cs, void* D, int64_t d_rs, int64_t d_cs, int32_t out_dt, hipStream_t st) {
+int32_t splitk_reduce_dispatch(const float* P, int split, int64_t M, int64_t N, const GemmArgs& e, int32_t out_dt, hipStream_t st) {
     const dim3 grid((unsigned)std::min<int64_t>((M * N + 255) / 256, 256 * 32));
     switch (out_dt) {
-        case MOYE_F32: splitk_reduce_kernel<OutF32><<<grid, 256, 0, st>>>(P, split, M, N, alpha, C, c_rs, c_cs, D, d_rs, d_cs); break;
-        case MOYE_F16: splitk_reduce_kernel<OutF16><<<grid, 256, 0, st>>>(P, split, M, N, alpha, C, c_rs, c_cs, D, d_rs, d_cs); break;
-        case MOYE_BF16: splitk_reduce_kernel<OutBF16><<<grid, 256, 0, st>>>(P, split, M, N, alpha, C, c_rs, c_cs, D, d_rs, d_cs); break;
+        case MOYE_F32: splitk_reduce_kernel<OutF32><<<grid, 256, 0, st>>>(P, split, M, N, e); break;
+        case MOYE_F16: splitk_reduce_kernel<OutF16><<<grid, 256, 0, st>>>(P, split, M, N, e); break;
+        case MOYE_BF16: splitk_reduce_kernel<OutBF16><<<grid, 256, 0, st>>>(P, split, M, N, e); break;
         default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: MFMA kernels write f32, f16 or bf16, not %s", dtype_name(out_dt));
     }
     MOYE_HIP_CHECK(hipGetLastError());

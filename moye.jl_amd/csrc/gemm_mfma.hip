@@ -160,7 +160,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
     // ---- epilogue: alpha*acc + C -> OutT -> this wave's LDS patch -> 128-bit row stores ----
     // lane holds C[m = AT i + r16][n = AT j + 8 g + 4 kq + e], e = 0..3 (g = 0 only for the 16x16 forms)
     const int64_t m_base = (int64_t)tm * BM + wm0, n_base = (int64_t)tn * BN + wn0;
-    if constexpr (kEdge) {
+    // residue tiles, and any tile with an element-wise operation in the epilogue: every lane stores its own elements
+    if (kEdge || p.ep_op != MOYE_MAP_IDENTITY) {
 #pragma unroll
         for (int i = 0; i < MI; ++i) {
             const int64_t m = m_base + AT * i + r16;
@@ -173,9 +174,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         if (n + e >= p.N) continue;
-                        float x = acc[i][j][4 * g + e] * p.alpha;
-                        if (p.C) x += Out::load(p.C, m * p.ldc_m + (n + e) * p.ldc_n);
-                        static_cast<OutT*>(p.D)[m * p.ldd + n + e] = Out::cvt(x);
+                        const float c = p.C ? Out::load(p.C, m * p.ldc_m + (n + e) * p.ldc_n) : 0.f;
+                        static_cast<OutT*>(p.D)[m * p.ldd + n + e] = Out::cvt(epi_value(p, acc[i][j][4 * g + e], p.C != nullptr, c, m, n + e));
                     }
                 }
             }
@@ -223,19 +223,16 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
             for (int j = 0; j < NI; ++j) {
 #pragma unroll
                 for (int g = 0; g < G; ++g) {
-                    float v[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * g + e] * p.alpha;
                     const int row = AT * ii + r16, col = AT * j + 8 * g + 4 * kq;
                     const int chunk = col / EPC, within = col % EPC;
                     OutT* dst = patch + (row * CR + (chunk ^ (row & (CR - 1)))) * EPC + within;
-                    if (row_c) {
+                    const int64_t m = m_base + AT * i + r16, n = n_base + AT * j + 8 * g + 4 * kq;
+                    float v[4];
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) v[e] += Out::load(dst, e);
-                    } else if (p.C) {
-                        const int64_t m = m_base + AT * i + r16, n = n_base + AT * j + 8 * g + 4 * kq;
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) v[e] += Out::load(p.C, m * p.ldc_m + (n + e) * p.ldc_n);
+                    for (int e = 0; e < 4; ++e) {
+                        v[e] = __fmul_rn(acc[i][j][4 * g + e], p.alpha);
+                        if (row_c) v[e] = __fadd_rn(v[e], __fmul_rn(p.beta, Out::load(dst, e)));
+                        else if (p.C) v[e] = __fadd_rn(v[e], __fmul_rn(p.beta, Out::load(p.C, m * p.ldc_m + (n + e) * p.ldc_n)));
                     }
 #pragma unroll
                     for (int e = 0; e < 4; ++e) dst[e] = Out::cvt(v[e]);
@@ -353,6 +350,8 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
                 part.D = static_cast<char*>(a.D) + (int64_t)N0 * ob0; part.ldd = 1; part.ldd_n = a.ldd;
                 if (a.C) part.C = static_cast<const char*>(a.C) + (int64_t)N0 * a.ldc_n * ob0;
                 part.ldc_m = a.ldc_n; part.ldc_n = a.ldc_m;
+                if (a.ep_x) part.ep_x = static_cast<const char*>(a.ep_x) + (int64_t)N0 * a.ep_xn * dtype_bytes(a.ep_xdt);
+                part.ep_xm = a.ep_xn; part.ep_xn = a.ep_xm;
                 if (int32_t e = gemm_mfma_skinny_dispatch(in_dt, out_dt, part, st)) return e;
             } else if (a.N > N0) {
                 part = a;
@@ -360,6 +359,7 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
                 part.B = static_cast<const char*>(a.B) + (int64_t)N0 * a.ldb * eb;
                 part.D = static_cast<char*>(a.D) + (int64_t)N0 * ob0;
                 if (a.C) part.C = static_cast<const char*>(a.C) + (int64_t)N0 * a.ldc_n * ob0;
+                if (a.ep_x) part.ep_x = static_cast<const char*>(a.ep_x) + (int64_t)N0 * a.ep_xn * dtype_bytes(a.ep_xdt);
                 if (int32_t e = gemm_mfma_tn_dispatch(in_dt, out_dt, 0, 0, 0, 0, 0, part, st)) return e;
             }
             if (a.M > M0) {
@@ -368,6 +368,7 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
                 part.A = static_cast<const char*>(a.A) + (int64_t)M0 * a.lda * eb;
                 part.D = static_cast<char*>(a.D) + (int64_t)M0 * a.ldd * ob0;
                 if (a.C) part.C = static_cast<const char*>(a.C) + (int64_t)M0 * a.ldc_m * ob0;
+                if (a.ep_x) part.ep_x = static_cast<const char*>(a.ep_x) + (int64_t)M0 * a.ep_xm * dtype_bytes(a.ep_xdt);
                 if (int32_t e = gemm_mfma_tn_dispatch(in_dt, out_dt, 0, 0, 0, 0, 0, part, st)) return e;
             }
             return MOYE_OK;
@@ -392,8 +393,11 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
     if (bm == 256 && bn == 256) {
         if (bkb != 128 && bkb != 64)
             return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the 256x256 MFMA kernels take %d or %d elements of K per tile", 64 / eb, 128 / eb);
+        // the hand-ordered kernel has no element-wise operations in its epilogue
+        if ((a.xcd_swizzle & (MOYE_GEMM_WAVE4 | MOYE_GEMM_PINGPONG)) && a.ep_op != MOYE_MAP_IDENTITY)
+            return fail(MOYE_ERR_UNSUPPORTED, "gemm!: MOYE_GEMM_WAVE4 and MOYE_GEMM_PINGPONG take no element-wise epilogue operation; leave the schedule to the library");
         // fp8 runs at twice the 16-bit rate only on the 16x16x128 MFMA, which the hand-ordered kernel issues
-        if (in_dt == MOYE_F8E4M3 && bkb == 128 && stages < 3 && !(a.xcd_swizzle & MOYE_GEMM_PINGPONG))
+        if (in_dt == MOYE_F8E4M3 && bkb == 128 && stages < 3 && !(a.xcd_swizzle & MOYE_GEMM_PINGPONG) && a.ep_op == MOYE_MAP_IDENTITY)
             a.xcd_swizzle |= MOYE_GEMM_WAVE4;
         // hand-ordered kernel: k-steps of 64 bytes, or of 128 (fp8 always; the 16-bit types when the tile says so)
         const int w4_step = in_dt == MOYE_F8E4M3 || (bkb == 128 && eb == 2) ? 128 : 64;

@@ -24,7 +24,9 @@
 
 namespace moye {
 
-template <typename In, typename Out, int WGM, int WGN>
+// kOps: the epilogue may apply an element-wise operation (GemmArgs::ep_op).  A separate instance, so that the code and
+// the registers of that path never touch the kernel the plain gemm! runs.
+template <typename In, typename Out, int WGM, int WGN, bool kOps = false>
 __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
     constexpr int BM = 256, BN = 256, CPR = 8;  // 8 chunks of 16 bytes per tile row
     constexpr int A_CH = BM * CPR, B_CH = BN * CPR, STAGE = A_CH + B_CH;
@@ -187,7 +189,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
 
     // --- epilogue (mfma_epilogue.hpp): alpha*acc + C -> OutT -> this wave's LDS patch -> 128-bit row stores
     static_assert(NWAVES * 32 * WN * 4 <= 2 * STAGE * 16, "C patches (32 rows per wave and pass) fit in the operand stages");
-    store_c_tile<Out, MI, NI>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
+    store_c_tile<Out, MI, NI, kOps>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -303,7 +305,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256_ring(GemmArgs
 
     // --- epilogue (mfma_epilogue.hpp): alpha*acc + C -> OutT -> this wave's LDS patch -> 128-bit row stores
     static_assert(NWAVES * 32 * WN * 4 <= STAGES * STAGE * 16, "C patches (32 rows per wave and pass) fit in the operand ring");
-    store_c_tile<Out, MI, NI>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
+    store_c_tile<Out, MI, NI, false>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
 }
 
 template <typename In, typename Out, int STAGES>
@@ -320,16 +322,27 @@ static int32_t launch256_ring(const GemmArgs& a, hipStream_t st) {
 template <typename In, typename Out, int WGM, int WGN>
 static int32_t launch256(const GemmArgs& a, hipStream_t st) {
     constexpr int kLds = 2 * (256 + 256) * 128;  // two operand stages, 128 KiB
-    auto kern = gemm_mfma_tn_256<In, Out, WGM, WGN>;
+    const dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1));
+    if constexpr (WGM * WGN == 8) if (a.ep_op != MOYE_MAP_IDENTITY) {
+        auto kern = gemm_mfma_tn_256<In, Out, WGM, WGN, true>;
+        static LdsCap cap;
+        if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
+        kern<<<grid, dim3(64 * WGM * WGN), kLds, st>>>(a);
+        MOYE_HIP_CHECK(hipGetLastError());
+        return MOYE_OK;
+    }
+    auto kern = gemm_mfma_tn_256<In, Out, WGM, WGN, false>;
     static LdsCap cap;
     if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
-    kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1)), dim3(64 * WGM * WGN), kLds, st>>>(a);
+    kern<<<grid, dim3(64 * WGM * WGN), kLds, st>>>(a);
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;
 }
 
 template <typename In>
 static int32_t launch256_out(int32_t out_dt, const GemmArgs& a, int waves, int stages, hipStream_t st) {
+    if (stages >= 3 && a.ep_op != MOYE_MAP_IDENTITY)
+        return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the ring schedules (stages >= 3) take no element-wise epilogue operation; leave stages at 0");
     if (stages >= 3) {
         const bool five = stages >= 5;
         switch (out_dt) {
@@ -339,7 +352,7 @@ static int32_t launch256_out(int32_t out_dt, const GemmArgs& a, int waves, int s
             default: break;
         }
     }
-    if (waves == 4) {
+    if (waves == 4 && a.ep_op == MOYE_MAP_IDENTITY) {  // (with an element-wise operation the eight-wave form runs: 256 accumulators leave it no registers)
         switch (out_dt) {
             case MOYE_F32: return launch256<In, OutF32, 2, 2>(a, st);
             case MOYE_F16: return launch256<In, OutF16, 2, 2>(a, st);

@@ -333,7 +333,7 @@ __global__ __launch_bounds__(128 * WGN) void gemm_mfma_tn_256_w4(GemmArgs p) {
         for (int j = 0; j < NI; ++j) asm volatile("" : "+a"(acc[i][j]));
     __syncthreads();  // every wave is done with the operand ring before it becomes C patches
 
-    store_c_tile<Out, MI, NI>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
+    store_c_tile<Out, MI, NI, false>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
 }
 
 template <typename In, typename Out, int WGN>

@@ -101,9 +101,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_skinny(GemmArgs p) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             if (n + e >= p.N) continue;
-            float x = v[e] * p.alpha;
-            if (p.C) x += Out::load(p.C, (int64_t)m * p.ldc_m + (int64_t)(n + e) * p.ldc_n);
-            d[e * sn] = Out::cvt(x);
+            const float c = p.C ? Out::load(p.C, (int64_t)m * p.ldc_m + (int64_t)(n + e) * p.ldc_n) : 0.f;
+            d[e * sn] = Out::cvt(epi_value(p, v[e], p.C != nullptr, c, m, n + e));
         }
     }
 }

@@ -15,6 +15,13 @@ struct GemmArgs {
     int64_t lda, ldb, ldc_m, ldc_n, ldd;
     int64_t ldd_n;  // stride of D along n; 0 = contiguous.  Only the short-M kernel takes another value.
     float alpha;
+    // the rest of the epilogue (moye_gemm_epilogue): D = op(alpha * acc + beta * C, x), see epi_value() in mfma_common.hpp
+    float beta;        // applied to C; the host passes C = nullptr when beta == 0
+    int ep_op;         // MOYE_MAP_*; MOYE_MAP_IDENTITY = none
+    int ep_xdt;        // element type of ep_x: MOYE_F32, MOYE_F16 or MOYE_BF16
+    float ep_scalar;   // second argument of op when ep_x is null
+    const void* ep_x;  // (M,N) operand of op, element strides ep_xm / ep_xn (0 = repeated along that mode)
+    int64_t ep_xm, ep_xn;
     int tiles_m, tiles_n;
     // split-K: gridDim.y ranges of K in one launch; range y reads A and B split_ab bytes further along their rows
     // and writes its product split_d bytes further (compact fp32 partial products, one after the other)
@@ -48,8 +55,9 @@ int32_t gemm_mfma_skinny_dispatch(int32_t in_dt, int32_t out_dt, const GemmArgs&
 int32_t axpby_dispatch(double a, const moye_tensor* X, double b, const moye_tensor* Y, hipStream_t st);
 int32_t fill_dispatch(const moye_tensor* X, double value, hipStream_t st);
 int32_t map_dispatch(int32_t op, const moye_tensor* D, const moye_tensor* A, const moye_tensor* B, double scalar, hipStream_t st);
-int32_t splitk_reduce_dispatch(const float* P, int split, int64_t M, int64_t N, float alpha, const void* C, int64_t c_rs,
-                               int64_t c_cs, void* D, int64_t d_rs, int64_t d_cs, int32_t out_dt, hipStream_t st);
+// sums the `split` partial products in P in ascending order and applies the epilogue of `e` (alpha, beta, op and operand;
+// C with strides ldc_m / ldc_n; D with strides ldd / ldd_n), M x N elements
+int32_t splitk_reduce_dispatch(const float* P, int split, int64_t M, int64_t N, const GemmArgs& e, int32_t out_dt, hipStream_t st);
 int32_t mfma_ceiling(int32_t in_dt, int32_t random_operands, float seconds, float* tflops, float* clock_ghz, hipStream_t st);
 int32_t gemm_universal_dispatch(int bm, int bn, int bk, UArgs a, hipStream_t st);
 

@@ -106,6 +106,41 @@ struct OutBF16 {
     }
 };
 
+// ---- the epilogue's arithmetic on one element (include/moye_hip.h, moye_gemm_epilogue) -------------------------------
+// What the reference's user kernels do to the accumulator fragment after the k-loop: axpby! (src/algorithm/blas.jl:1-9)
+// and one broadcast operation (src/broadcast.jl:5-41), in fp32, every operation rounded on its own (the intrinsics keep
+// the compiler from contracting a product and a sum into one fused operation, which Julia does not do either).
+__device__ __forceinline__ float epi_operand(const GemmArgs& p, int64_t m, int64_t n) {
+    if (!p.ep_x) return p.ep_scalar;
+    const int64_t i = m * p.ep_xm + n * p.ep_xn;
+    switch (p.ep_xdt) {
+        case MOYE_F16: return (float)static_cast<const _Float16*>(p.ep_x)[i];
+        case MOYE_BF16: return __uint_as_float((uint32_t)static_cast<const uint16_t*>(p.ep_x)[i] << 16);
+        default: return static_cast<const float*>(p.ep_x)[i];
+    }
+}
+// max / min follow Julia: NaN if either argument is NaN, -0.0 < +0.0 (as moye_map)
+__device__ __forceinline__ float epi_op(int op, float x, float y) {
+    switch (op) {
+        case MOYE_MAP_ADD: return __fadd_rn(x, y);
+        case MOYE_MAP_SUB: return __fsub_rn(x, y);
+        case MOYE_MAP_MUL: return __fmul_rn(x, y);
+        case MOYE_MAP_DIV: return __fdiv_rn(x, y);
+        case MOYE_MAP_MAX: return ((y > x) | (signbit(y) < signbit(x))) ? (x != x ? x : y) : (y != y ? y : x);
+        case MOYE_MAP_MIN: return ((y < x) | (signbit(y) > signbit(x))) ? (x != x ? x : y) : (y != y ? y : x);
+        case MOYE_MAP_NEG: return -x;
+        case MOYE_MAP_ABS: return signbit(x) ? -x : x;
+        default: return x;
+    }
+}
+// acc: the fp32 sum over k; c: the element of C (ignored unless has_c); (m, n): the element's position in the problem
+__device__ __forceinline__ float epi_value(const GemmArgs& p, float acc, bool has_c, float c, int64_t m, int64_t n) {
+    float t = __fmul_rn(acc, p.alpha);
+    if (has_c) t = __fadd_rn(t, __fmul_rn(p.beta, c));
+    if (p.ep_op != MOYE_MAP_IDENTITY) t = epi_op(p.ep_op, t, epi_operand(p, m, n));
+    return t;
+}
+
 // XOR swizzle of the 16-byte chunk index inside an LDS tile row of CPR chunks.  The LDS has 32
 // banks of 4 bytes, so 128 bytes (8 chunks) make one sweep of the banks and a 128-bit access is
 // served 8 lanes per clock.  Rows that lie in different 128-byte sweeps get different chunk

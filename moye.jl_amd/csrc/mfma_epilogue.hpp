@@ -8,12 +8,80 @@
 
 namespace moye {
 
+// The same tile with an element-wise operation in the epilogue (GemmArgs::ep_op other than the identity).  The raw fp32
+// accumulators go through the wave's LDS patch, 32 rows at a time; the lanes then read them back along rows, apply
+// epi_value() (alpha, beta * C, the operation with its operand), convert and store 16-byte pieces.  The arithmetic
+// exists once, in a loop over the passes that is not unrolled: unrolled over all accumulators it would be several
+// thousand instructions per kernel.  `smem`: 32 x WN floats per wave.
+template <typename Out, int MI, int NI>
+__device__ __forceinline__ void store_c_tile_general(const GemmArgs& p, const f32x4 (&acc)[MI][NI], u32x4* smem, int wave,
+                                                     int lane, int64_t m_base, int64_t n_base) {
+    typedef typename Out::type OutT;
+    constexpr int WN = NI * 16, PASS_MI = 2, PASS_ROWS = 32, PASSES = MI / PASS_MI;
+    constexpr int EPC = 16 / (int)sizeof(OutT);  // elements per 16-byte piece of D
+    constexpr int CR = WN / 4;                   // 16-byte chunks of floats per patch row
+    constexpr int OUT_CH = PASS_ROWS * (WN / EPC);  // 16-byte pieces of D per pass
+    static_assert(CR >= 8 && OUT_CH % 64 == 0, "patch shape");
+    const int r16 = lane & 15, kq = lane >> 4;
+    float* patch = reinterpret_cast<float*>(smem) + wave * (PASS_ROWS * WN);
+    f32x4* patch16 = reinterpret_cast<f32x4*>(patch);
+#pragma unroll 1
+    for (int pass = 0; pass < PASSES; ++pass) {
+        // accumulators of rows 32 pass .. 32 pass + 31 -> patch (the only part that names registers, hence the static index)
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ++ps) {
+            if (pass != ps) continue;
+#pragma unroll
+            for (int ii = 0; ii < PASS_MI; ++ii)
+#pragma unroll
+                for (int j = 0; j < NI; ++j) {
+                    const int row = 16 * ii + r16, chunk = 4 * j + kq;
+                    patch16[row * CR + (chunk ^ (row & 7))] = acc[ps * PASS_MI + ii][j];
+                }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll 1
+        for (int t = 0; t < OUT_CH / 64; ++t) {
+            const int c = lane + 64 * t, row = c / (WN / EPC), och = c % (WN / EPC);
+            const int64_t m = m_base + PASS_ROWS * pass + row, n0 = n_base + och * EPC;
+            OutT out[EPC];
+#pragma unroll
+            for (int q = 0; q < EPC / 4; ++q) {
+                const int chunk = och * (EPC / 4) + q;
+                const f32x4 a = patch16[row * CR + (chunk ^ (row & 7))];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int64_t n = n0 + 4 * q + e;
+                    const float cv = p.C ? Out::load(p.C, m * p.ldc_m + n * p.ldc_n) : 0.f;
+                    out[4 * q + e] = Out::cvt(epi_value(p, a[e], p.C != nullptr, cv, m, n));
+                }
+            }
+            u32x4 w;
+            __builtin_memcpy(&w, out, 16);
+            store_d_chunk(p, static_cast<char*>(p.D) + (m * p.ldd + n0) * (int64_t)sizeof(OutT), w);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+}
+
 // acc[i][j] of a lane holds C[m = 16 i + lane % 16][n = 16 j + 4 (lane / 16) + e], e = 0..3,
 // relative to (m_base, n_base).  `smem` must be free of operand data for all waves.
-template <typename Out, int MI, int NI>
+// kWithOps = false leaves the element-wise operations out (the hand-ordered kernel: its register allocation around the
+// inline-assembly MFMAs must not change with what the epilogue needs; the host never sends it such a call).
+template <typename Out, int MI, int NI, bool kWithOps = true>
 __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&acc)[MI][NI], u32x4* smem, int wave,
                                              int lane, int64_t m_base, int64_t n_base) {
     typedef typename Out::type OutT;
+    if constexpr (kWithOps) {
+        if (p.ep_op != MOYE_MAP_IDENTITY) {
+            store_c_tile_general<Out, MI, NI>(p, acc, smem, wave, lane, m_base, n_base);
+            return;
+        }
+    }
     constexpr int WN = NI * 16;
     constexpr int EPC = 16 / (int)sizeof(OutT);  // elements per 16-byte chunk
     constexpr int CR = WN / EPC;                 // chunks per patch row
@@ -60,18 +128,23 @@ __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&ac
             const int i = i0 + ii;
 #pragma unroll
             for (int j = 0; j < NI; ++j) {
-                float v[4] = {acc[i][j].x * p.alpha, acc[i][j].y * p.alpha, acc[i][j].z * p.alpha,
-                              acc[i][j].w * p.alpha};
                 const int row = 16 * ii + r16, col = 16 * j + 4 * kq;
                 const int chunk = col / EPC, within = col % EPC;
                 OutT* dst = patch + (row * CR + (chunk ^ (row & 7))) * EPC + within;
+                const int64_t m = m_base + 16 * i + r16, n = n_base + 16 * j + 4 * kq;
+                float c[4] = {0.f, 0.f, 0.f, 0.f};
                 if (row_c) {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) v[e] += Out::load(dst, e);
+                    for (int e = 0; e < 4; ++e) c[e] = Out::load(dst, e);
                 } else if (p.C) {
-                    const int64_t m = m_base + 16 * i + r16, n = n_base + 16 * j + 4 * kq;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) v[e] += Out::load(p.C, m * p.ldc_m + (n + e) * p.ldc_n);
+                    for (int e = 0; e < 4; ++e) c[e] = Out::load(p.C, m * p.ldc_m + (n + e) * p.ldc_n);
+                }
+                float v[4] = {__fmul_rn(acc[i][j].x, p.alpha), __fmul_rn(acc[i][j].y, p.alpha), __fmul_rn(acc[i][j].z, p.alpha),
+                              __fmul_rn(acc[i][j].w, p.alpha)};
+                if (p.C) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = __fadd_rn(v[e], __fmul_rn(p.beta, c[e]));
                 }
 #pragma unroll
                 for (int e = 0; e < 4; ++e) dst[e] = Out::cvt(v[e]);

@@ -78,8 +78,24 @@ class Array:
         return int(size(self.layout))
 
     def offsets(self):
-        """0-based buffer offsets of the logical elements 1..size, in order."""
-        return np.array([self.index0(i) for i in range(1, len(self) + 1)], dtype=np.int64)
+        """0-based buffer offsets of the logical elements 1..size, in order.  Large arrays take the same
+        colexicographic decomposition (stride.jl:20-31) over the flattened modes in numpy, all elements at once;
+        tests/test_oracle_tiled.py checks the two forms against each other."""
+        n = len(self)
+        if n > 4096:
+            return self.offsets_vectorised()
+        return np.array([self.index0(i) for i in range(1, n + 1)], dtype=np.int64)
+
+    def offsets_vectorised(self):
+        flat = lflatten(self.layout)
+        shp = flat.shape if isinstance(flat.shape, tuple) else (flat.shape,)
+        strd = flat.stride if isinstance(flat.stride, tuple) else (flat.stride,)
+        idx = np.arange(len(self), dtype=np.int64)
+        off = np.full(len(self), self.offset, dtype=np.int64)
+        for s_, d_ in zip(shp, strd):
+            off += (idx % int(s_)) * int(d_)
+            idx //= int(s_)
+        return off
 
     def values(self):
         return self.buf[self.offsets()]
@@ -723,6 +739,34 @@ def broadcast(op, A, B=None, scalar=0.0, out=None):
             out.bf16 = True
     out.buf[out.offsets()] = r
     return out
+
+
+def gemm_epilogue(acc, alpha, beta, C, op, operand, scalar, out):
+    """What a user kernel of the reference does to its fp32 accumulator fragment after the k-loop, composed of the
+    reference's own pieces: axpby!(alpha, acc, beta, c) (blas.jl:1-9; iszero(beta) leaves C out), one broadcast
+    `op.(t, operand)` (broadcast.jl:5-41), and the conversion of copyto! into the result type (arch/copy/copy.jl:38-43,
+    round to nearest even).  acc: (M,N) float32; C: (M,N) in the result type or None; operand: anything numpy
+    broadcasts to (M,N) (float32, float16 or bf16-valued float32) or None for `scalar`; out: "f32" | "f16" | "bf16".
+    Every intermediate is float32 and every operation is rounded on its own."""
+    M, N = acc.shape
+    lay = make_layout((M, N))
+    X = Array(np.ascontiguousarray(acc, dtype=np.float32).reshape(-1, order="F").copy(), lay)
+    c32 = np.zeros((M, N), np.float32) if C is None else np.asarray(C).astype(np.float32)
+    Y = Array(c32.reshape(-1, order="F").copy(), lay)
+    axpby(np.float32(alpha), X, np.float32(beta if C is not None else 0.0), Y)
+    if op not in (None, "identity"):
+        if operand is None:
+            Y = broadcast(op, Y, None, scalar, out=Y)
+        else:
+            full = np.broadcast_to(np.asarray(operand).astype(np.float32), (M, N))
+            Y = broadcast(op, Y, Array(full.reshape(-1, order="F").copy(), lay), out=Y)
+    r = Y.buf.reshape(M, N, order="F")
+    if out == "f16":
+        with np.errstate(over="ignore"):
+            return r.astype(np.float16)
+    if out == "bf16":
+        return round_bf16(r)
+    return r
 
 
 def fill(X, value):

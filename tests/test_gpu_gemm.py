@@ -1177,3 +1177,153 @@ def test_bench_descriptor_every_cta_exact_on_integers(mh, out_dt):
     want = (a.float() @ b.float().t())           # exact: |sum| <= 4 * 512 = 2048, an integer fp16 holds
     assert float(want.abs().max()) <= 2048
     assert torch.equal(d.float(), want)
+
+
+# ---------------------------------------------------------------------------------------------
+# fused epilogue: D = op(alpha * A * B' + beta * C, operand)   (moye_gemm_ex)
+# ---------------------------------------------------------------------------------------------
+
+_NP_OF = {"float32": ("f32", np.float32), "float16": ("f16", np.float16), "bfloat16": ("bf16", np.float32)}
+
+
+def _epilogue_case(mh, mma, M, N, K, out_name, op, operand_kind, seed, col_major_d=False, alpha=0.375, beta=-1.25,
+                   operand_in_out_type=False):
+    """Small-integer A and B (the fp32 accumulator is exact whatever the order of the sum), random C and operand:
+    every bit of D is then fixed by the epilogue's arithmetic, which the oracle composes from axpby! and broadcast."""
+    out_dt = getattr(torch, out_name)
+    tag, _ = _NP_OF[out_name]
+    g = torch.Generator().manual_seed(seed)
+    A = torch.randint(-3, 4, (M, K), generator=g).to(torch.float16)
+    B = torch.randint(-3, 4, (N, K), generator=g).to(torch.float16)
+    C0 = torch.randn(M, N, generator=g).to(out_dt)
+    x_dt = out_dt if operand_in_out_type else torch.float32
+    if operand_kind == "row":        # one value per column n, repeated down the rows: (M,N):(0,1)
+        X0, xs = (torch.randn(N, generator=g) * 4).to(x_dt), (0, 1)
+    elif operand_kind == "col":      # one value per row m: (M,N):(1,0)
+        X0, xs = (torch.randn(M, generator=g) * 4).to(x_dt), (1, 0)
+    elif operand_kind == "full":     # a whole (M,N) array, column-major
+        X0, xs = (torch.randn(N, M, generator=g) * 4).to(x_dt), (1, M)
+    else:
+        X0, xs = None, None
+    if op == "div" and X0 is not None:
+        X0 = X0 + torch.where(X0 >= 0, 1.0, -1.0).to(x_dt)     # keep away from zero
+    acc = (A.float() @ B.float().t()).numpy()
+    assert np.abs(acc).max() < 2 ** 20
+    a, b, c = A.cuda(), B.cuda(), C0.cuda()
+    xd = X0.cuda() if X0 is not None else None
+    ep = mh.gemm_epilogue(alpha=alpha, beta=beta, op=mh._lib.MAP_OPS[op],
+                          operand=T(xd.reshape(-1), (M, N), xs) if xd is not None else None, scalar=1.5)
+    if col_major_d:
+        d = torch.zeros(N, M, dtype=out_dt, device="cuda")
+        td = T(d, (M, N), (1, M))
+    else:
+        d = torch.zeros(M, N, dtype=out_dt, device="cuda")
+        td = T(d)
+    need = mh.gemm_workspace_size(mma, td, T(a), T(b))
+    ws = torch.zeros(max(need, 1) + 256, dtype=torch.uint8, device="cuda")
+    mh.gemm_ex_(mma, td, T(a), T(b), T(c) if beta != 0 else None, ep, (ws.data_ptr() + 255) // 256 * 256, need)
+    torch.cuda.synchronize()
+    got = (d.t() if col_major_d else d).cpu()
+    cnp = C0.float().numpy().astype(np.float16) if tag == "f16" else C0.float().numpy()
+    if X0 is None:
+        xnp = None
+    else:
+        xf = X0.float().numpy()
+        xnp = xf[None, :] if operand_kind == "row" else xf[:, None] if operand_kind == "col" else xf.T
+    want = to.gemm_epilogue(acc, alpha, beta, cnp if beta != 0 else None, op, xnp, 1.5, tag)
+    gb = got.float().numpy().view(np.uint32)
+    wb = want.astype(np.float32).view(np.uint32)
+    bad = np.argwhere(gb != wb)
+    assert bad.size == 0, "%d of %d elements differ, first at %s: got %r want %r" % (
+        len(bad), M * N, bad[0], got.float().numpy()[tuple(bad[0])], want.astype(np.float32)[tuple(bad[0])])
+
+
+@pytest.mark.parametrize("out_name", ["float32", "float16", "bfloat16"])
+@pytest.mark.parametrize("op", ["identity", "add", "sub", "mul", "div", "max", "min", "neg", "abs"])
+def test_fused_epilogue_every_op_bit_exact(mh, out_name, op):
+    """256x256 tile (the default for this size): every operation with a per-column vector, alpha and beta that make
+    the products round; bit for bit against the oracle."""
+    mma = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 4, 1), cta_tile=(256, 256, 64))
+    _epilogue_case(mh, mma, 512, 768, 128, out_name, op, "row", 300 + len(op))
+
+
+@pytest.mark.parametrize("kernel", ["256", "128", "64", "128 atom32", "predicated", "short-M", "split-K", "library", "ragged"])
+@pytest.mark.parametrize("operand_kind", ["row", "col", "full", "scalar"])
+def test_fused_epilogue_every_kernel_and_operand(mh, kernel, operand_kind):
+    """bias-style add with beta * C through every kernel family that writes D, row-major and column-major D, operands
+    as row vector, column vector, whole array and scalar, in fp32 and in D's type."""
+    from moye_hip import _lib
+    F16 = mh.MFMA_F32_16x16x32_F16
+    M, N, K = 512, 512, 128
+    if kernel == "256":
+        mma = mh.tiled_mma_desc(F16, atom_layout=(2, 4, 1), cta_tile=(256, 256, 64))
+    elif kernel == "128":
+        mma = mh.tiled_mma_desc(F16, atom_layout=(2, 2, 1), cta_tile=(128, 128, 32))
+    elif kernel == "64":
+        mma = mh.tiled_mma_desc(F16, atom_layout=(2, 2, 1), cta_tile=(64, 64, 32))
+    elif kernel == "128 atom32":
+        mma = mh.tiled_mma_desc(mh.MFMA_F32_32x32x16_F16, atom_layout=(2, 2, 1), cta_tile=(128, 128, 32))
+    elif kernel == "predicated":
+        mma = mh.tiled_mma_desc(F16, cta_tile=(0, 0, 0))
+        M, N, K = 200, 136, 72
+    elif kernel == "short-M":
+        mma = mh.tiled_mma_desc(F16, cta_tile=(0, 0, 0))
+        M, N, K = 24, 640, 256
+    elif kernel == "split-K":
+        mma = mh.tiled_mma_desc(F16, atom_layout=(2, 2, 1), cta_tile=(128, 128, 32), split_k=4)
+        M, N, K = 256, 384, 512
+    elif kernel == "ragged":     # interior on 256x256 tiles, both fringes on the residue kernels
+        mma = mh.tiled_mma_desc(F16, cta_tile=(0, 0, 0))
+        M, N, K = 4096 + 40, 2048 + 72, 64
+    else:
+        mma = mh.tiled_mma_desc(F16, cta_tile=(0, 0, 0))
+        M, N, K = 2048, 4096, 64          # the library picks 256x256
+    combos = [(c, o, t) for c in (False, True) for o, t in (("float16", False), ("float32", False), ("bfloat16", True))]
+    if M * N > 1 << 20:      # the oracle takes seconds on these: one combination per layout of D
+        combos = [(False, "float16", False), (True, "bfloat16", True)]
+        if operand_kind in ("col", "scalar"):
+            combos = combos[:1] if kernel == "library" else combos[1:]
+    for col_major_d, out_name, in_out_type in combos:
+        _epilogue_case(mh, mma, M, N, K, out_name, "add", operand_kind, 17, col_major_d=col_major_d,
+                       operand_in_out_type=in_out_type)
+
+
+def test_fused_epilogue_limits(mh):
+    """beta == 0 never reads C (NaNs in it do not reach D); moye_gemm is the beta == 1 case of moye_gemm_ex, bit for
+    bit; what is not built says so."""
+    from moye_hip import _lib
+    g = torch.Generator().manual_seed(5)
+    M = N = 256
+    K = 128
+    A = (torch.randn(M, K, generator=g) / 8).half()
+    B = (torch.randn(N, K, generator=g) / 8).half()
+    a, b = A.cuda(), B.cuda()
+    nan_c = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+    mma = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(128, 128, 32))
+    d0 = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+    mh.gemm_ex_(mma, T(d0), T(a), T(b), T(nan_c), mh.gemm_epilogue(alpha=2.0, beta=0.0))
+    d1 = torch.zeros_like(d0)
+    mh.gemm_(mma, T(d1), T(a), T(b), None, 2.0)
+    torch.cuda.synchronize()
+    assert not torch.isnan(d0).any() and torch.equal(d0.view(torch.int16), d1.view(torch.int16))
+    C0 = torch.randn(M, N, generator=g).half().cuda()
+    mh.gemm_ex_(mma, T(d0), T(a), T(b), T(C0), mh.gemm_epilogue(alpha=0.3, beta=1.0))
+    mh.gemm_(mma, T(d1), T(a), T(b), T(C0), 0.3)
+    torch.cuda.synchronize()
+    assert torch.equal(d0.view(torch.int16), d1.view(torch.int16))
+    x = torch.zeros(M, N, dtype=torch.float64, device="cuda")
+    for bad, status in ((mh.gemm_epilogue(op=99), _lib.ERR_UNSUPPORTED),
+                        (mh.gemm_epilogue(op=_lib.MAP_ADD, operand=T(x)), _lib.ERR_UNSUPPORTED),
+                        (mh.gemm_epilogue(op=_lib.MAP_ADD, operand=T(d0.float()[:, :128].contiguous())), _lib.ERR_SHAPE)):
+        with pytest.raises(mh.MoyeError) as e:
+            mh.gemm_ex_(mma, T(d0), T(a), T(b), None, bad)
+        assert e.value.status == status
+    with pytest.raises(mh.MoyeError) as e:       # the hand-ordered kernel has no such epilogue
+        mh.gemm_ex_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 4, 1), cta_tile=(256, 256, 64), flags=_lib.GEMM_WAVE4),
+                    T(d0), T(a), T(b), None, mh.gemm_epilogue(op=_lib.MAP_ABS))
+    assert e.value.status == _lib.ERR_UNSUPPORTED
+    af, bf = a.float(), b.float()
+    with pytest.raises(mh.MoyeError) as e:       # UniversalFMA keeps the reference's own accumulation
+        mh.gemm_ex_(mh.tiled_mma_desc(mh.MMA_UNIVERSAL_FMA, cta_tile=(32, 32, 8)), T(d0.float()), T(af), T(bf), None,
+                    mh.gemm_epilogue(op=_lib.MAP_ABS))
+    assert e.value.status == _lib.ERR_UNSUPPORTED

@@ -437,3 +437,55 @@ def test_copyto_if_moves_only_where_the_mask_is_true():
     assert np.array_equal(d2.buf, d3.buf)
     with pytest.raises(ValueError):
         to.copyto_if(dst, src, to.Array(np.ones(12, np.uint8), lo.parse_layout("12:1")))
+
+
+def test_gemm_epilogue_oracle_known_answers():
+    """The epilogue oracle (axpby! then one broadcast, then the converting copy): hand-built cases that a fused
+    multiply-add, a dropped beta, a transposed operand or a wrong conversion would fail."""
+    import tiled_oracle as to
+    f32 = np.float32
+    # alpha * acc rounds to 1 + 2^-11 (the exact product has a further 2^-24: a tie, to even); adding -(1 + 2^-11)
+    # gives exactly 0 when the product is rounded first and 2^-24 when product and sum are fused
+    a = f32(1) + f32(2.0 ** -12)
+    acc = np.full((2, 3), a, f32)
+    C = np.full((2, 3), -(f32(1) + f32(2.0 ** -11)), f32)
+    r = to.gemm_epilogue(acc, a, 1.0, C, None, None, 0.0, "f32")
+    assert r.dtype == np.float32 and np.all(r == 0.0)
+    # beta == 0 leaves C out altogether, NaNs included (axpby!'s iszero(b))
+    r = to.gemm_epilogue(np.ones((2, 3), f32), 2.0, 0.0, np.full((2, 3), np.nan, f32), None, None, 0.0, "f32")
+    assert np.all(r == 2.0)
+    # beta scales C, then the sum: 0.5 * 3 + (-2) * 4 = -6.5; fp16 result
+    r = to.gemm_epilogue(np.full((2, 2), 3, f32), 0.5, -2.0, np.full((2, 2), 4, np.float16), None, None, 0.0, "f16")
+    assert r.dtype == np.float16 and np.all(r == np.float16(-6.5))
+    # a row vector is repeated down the rows, a column vector along them
+    acc = np.arange(6, dtype=f32).reshape(2, 3)
+    assert np.array_equal(to.gemm_epilogue(acc, 1.0, 0.0, None, "add", np.array([[10, 20, 30]], f32), 0.0, "f32"),
+                          np.array([[10, 21, 32], [13, 24, 35]], f32))
+    assert np.array_equal(to.gemm_epilogue(acc, 1.0, 0.0, None, "sub", np.array([[10], [20]], f32), 0.0, "f32"),
+                          np.array([[-10, -9, -8], [-17, -16, -15]], f32))
+    # relu through max with a scalar; Julia's max: NaN wins, +0 > -0
+    r = to.gemm_epilogue(np.array([[-1.0, np.nan, -0.0, 2.0]], f32), 1.0, 0.0, None, "max", None, 0.0, "f32")
+    assert r[0, 0] == 0 and np.isnan(r[0, 1]) and r[0, 3] == 2 and not np.signbit(r[0, 2])
+    # conversion is round-to-nearest-even after the operation: 2049 is a tie in fp16 (-> 2048), 2051 -> 2052; bf16: 257 -> 256, 259 -> 260
+    r = to.gemm_epilogue(np.array([[2048.0, 2050.0]], f32), 1.0, 0.0, None, "add", None, 1.0, "f16")
+    assert list(r[0].astype(np.float64)) == [2048.0, 2052.0]
+    r = to.gemm_epilogue(np.array([[256.0, 258.0]], f32), 1.0, 0.0, None, "add", None, 1.0, "bf16")
+    assert list(r[0].astype(np.float64)) == [256.0, 260.0]
+    # division and the unary operations
+    assert to.gemm_epilogue(np.array([[1.0]], f32), 1.0, 0.0, None, "div", None, 3.0, "f32")[0, 0] == f32(1) / f32(3)
+    assert to.gemm_epilogue(np.array([[-2.5]], f32), 1.0, 0.0, None, "abs", None, 0.0, "f32")[0, 0] == 2.5
+    assert to.gemm_epilogue(np.array([[-2.5]], f32), 1.0, 0.0, None, "neg", None, 0.0, "f32")[0, 0] == 2.5
+
+
+def test_vectorised_offsets_match_the_element_loop():
+    """Array.offsets() for large arrays decomposes all indices at once; same numbers as layout(i) element by element on
+    hierarchical, padded, zero-stride and row-major layouts."""
+    import tiled_oracle as to
+    from layout_oracle import Layout, make_layout
+    for shape, stride in [((4, 6), (1, 4)), ((4, 6), (6, 1)), (((2, 3), (2, 2)), ((1, 4), (2, 12))), ((8, 5), (0, 1)),
+                          ((3, (2, 4)), (16, (1, 2))), (12, 3), ((5, 7, 2), (1, 10, 100))]:
+        a = to.Array(np.zeros(1), Layout(shape, stride), offset=7)
+        want = np.array([a.index0(i) for i in range(1, len(a) + 1)], dtype=np.int64)
+        assert np.array_equal(a.offsets_vectorised(), want), (shape, stride)
+    big = to.Array(np.zeros(1), make_layout((96, 64)))
+    assert len(big) > 4096 and np.array_equal(big.offsets(), np.arange(96 * 64))

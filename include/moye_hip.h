@@ -235,6 +235,11 @@ int32_t moye_gemm_noalloc(const moye_tiled_mma* mma, const moye_tensor* D, const
  * Results are written to `out` (capacity `cap` bytes, NUL-terminated). */
 int32_t moye_layout_normalize(const char* layout, char* out, size_t cap);                    /* parse + print  */
 int32_t moye_layout_eval(const char* layout, const char* coord, int64_t* index);             /* layout.jl:90-102 (1-based) */
+/* the same with the result as text, which carries its integer type the way the reference's result does (Int32 stays
+ * Int32: test/layout.jl:4-12, src/utilities.jl:1-11): "_7" static, "7" an Int, "7i32" an Int32.  In all text that
+ * crosses this boundary a dynamic Int32 is written with the suffix `i32`; a result is static when every integer that
+ * went into it is, an Int32 when its dynamic inputs all are, an Int otherwise; Int32 arithmetic wraps modulo 2^32. */
+int32_t moye_layout_eval_typed(const char* layout, const char* coord, char* out, size_t cap);
 int32_t moye_layout_size(const char* layout, int64_t* size);                                 /* layout.jl:302-304 */
 int32_t moye_layout_cosize(const char* layout, int64_t* cosize);                             /* layout.jl:350-352 */
 int32_t moye_layout_rank_depth(const char* layout, int32_t* rank, int32_t* depth);           /* layout.jl:321-343 */

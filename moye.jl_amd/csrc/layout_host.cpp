@@ -24,23 +24,23 @@ int64_t trem(int64_t a, int64_t b) {
 }
 
 // Static.jl arithmetic: static op static -> static, mixed -> dynamic; a static zero absorbs `*`.
-Int add(Int a, Int b) { return Int(a.v + b.v, a.s && b.s); }
-Int sub(Int a, Int b) { return Int(a.v - b.v, a.s && b.s); }
+Int add(Int a, Int b) { return promoted(a.v + b.v, a, b); }
+Int sub(Int a, Int b) { return promoted(a.v - b.v, a, b); }
 Int mul(Int a, Int b) {
     if ((a.s && a.v == 0) || (b.s && b.v == 0)) return S(0);
-    return Int(a.v * b.v, a.s && b.s);
+    return promoted(a.v * b.v, a, b);
 }
-Int div(Int a, Int b) { return Int(tdiv(a.v, b.v), a.s && b.s); }
-Int rem(Int a, Int b) { return Int(trem(a.v, b.v), a.s && b.s); }
-Int imin(Int a, Int b) { return Int(std::min(a.v, b.v), a.s && b.s); }
-Int imax(Int a, Int b) { return Int(std::max(a.v, b.v), a.s && b.s); }
-Int iabs(Int a) { return Int(std::llabs(a.v), a.s); }
-Int isign(Int a) { return Int((a.v > 0) - (a.v < 0), a.s); }
+Int div(Int a, Int b) { return promoted(tdiv(a.v, b.v), a, b); }
+Int rem(Int a, Int b) { return promoted(trem(a.v, b.v), a, b); }
+Int imin(Int a, Int b) { return promoted(std::min(a.v, b.v), a, b); }
+Int imax(Int a, Int b) { return promoted(std::max(a.v, b.v), a, b); }
+Int iabs(Int a) { return same_type(a, std::llabs(a.v)); }
+Int isign(Int a) { return same_type(a, (a.v > 0) - (a.v < 0)); }
 Int cld(Int a, Int b) {
     if (b.v == 0) raise(MOYE_ERR_SHAPE, "division by zero in layout arithmetic");
     int64_t q = a.v / b.v;
     if ((a.v % b.v != 0) && ((a.v < 0) == (b.v < 0))) ++q;
-    return Int(q, a.s && b.s);
+    return promoted(q, a, b);
 }
 bool is_static_one(const IT& t) { return t.is_leaf() && t.leaf.s && t.leaf.v == 1; }
 bool is_static_zero(const IT& t) { return t.is_leaf() && t.leaf.s && t.leaf.v == 0; }
@@ -114,6 +114,12 @@ struct Parser {
         if (q == d0) bad("expected an integer");
         int64_t v = std::strtoll(s.substr(p, q - p).c_str(), nullptr, 10);
         p = q;
+        if (s.compare(p, 3, "i32") == 0) {  // a dynamic Int32
+            if (st) bad("a static integer has no width");
+            if (v < INT32_MIN || v > INT32_MAX) bad("value does not fit an Int32");
+            p += 3;
+            return D32(v);
+        }
         return Int(v, st);
     }
     // int tuple item; colons allowed when `colons`
@@ -226,7 +232,7 @@ Tile parse_tile(const std::string& text_in) {
 
 std::string to_string(const IT& t) {
     if (t.is_colon()) return ":";
-    if (t.is_leaf()) return (t.leaf.s ? "_" : "") + std::to_string(t.leaf.v);
+    if (t.is_leaf()) return (t.leaf.s ? "_" : "") + std::to_string(t.leaf.v) + (t.leaf.w32 ? "i32" : "");
     std::string r = "(";
     for (size_t i = 0; i < t.size(); ++i) {
         if (i) r += ", ";
@@ -305,7 +311,7 @@ Int shape_div_int(Int a, Int b) {  // int_tuple.jl:84-90
     if (b.v == 0) raise(MOYE_ERR_SHAPE, "shape_div by zero");
     const int64_t q = tdiv(a.v, b.v);
     const int64_t r = q != 0 ? q : isign(a).v * isign(b).v;
-    return Int(r, a.s && b.s);
+    return promoted(r, a, b);
 }
 }  // namespace
 
@@ -452,23 +458,23 @@ IT offset0(const IT& x) {  // stride.jl:72-80: 1-based -> 0-based, colon -> 0
         for (const IT& e : x.items) out.push_back(offset0(e));
         return IT::tuple(out);
     }
-    return IT(Int(x.leaf.v - 1, x.leaf.s));
+    return IT(same_type(x.leaf, x.leaf.v - 1));
 }
 }  // namespace
 
 Int coord_to_index(const IT& coord, const IT& shape, const IT& stride) {  // stride.jl:82-89
     const Int idx = c2i0(offset0(coord), shape, stride);
-    return Int(idx.v + 1, idx.s);
+    return same_type(idx, idx.v + 1);
 }
 
 Int coord_to_index_default(const IT& coord, const IT& shape) {  // stride.jl:56-70
     const IT c0 = offset0(coord);
-    if (c0.is_leaf()) return Int(c0.leaf.v + 1, c0.leaf.s);
+    if (c0.is_leaf()) return same_type(c0.leaf, c0.leaf.v + 1);
     const std::vector<Int> fc = flat_leaves(c0);
     const std::vector<Int> fs = flat_leaves(product_like(shape, coord));
     Int acc = fc.back();
     for (size_t i = fc.size() - 1; i-- > 0;) acc = add(fc[i], mul(fs[i], acc));
-    return Int(acc.v + 1, acc.s);
+    return same_type(acc, acc.v + 1);
 }
 
 namespace {
@@ -514,8 +520,8 @@ IT index_to_coord(Int index, const IT& shape, const IT& stride_in) {  // stride.
     }
     if (is_static_one(shape)) return IT(S(0));
     const Int st = leaf_of(stride_in);
-    const Int crd = rem(div(Int(index.v - 1, index.s), st), leaf_of(shape));
-    return IT(Int(crd.v + 1, crd.s));
+    const Int crd = rem(div(same_type(index, index.v - 1), st), leaf_of(shape));
+    return IT(same_type(crd, crd.v + 1));
 }
 
 namespace {
@@ -1008,7 +1014,7 @@ Layout upcast(const Layout& l, int64_t n) {  // layout.jl:945-965
                 const IT m = IT(S(n));
                 return Layout{shape_div(shp, shape_div(m, IT(iabs(d)))), shape_div(strd, m)};
             }
-            return Layout{shp, IT(D(tdiv(d.v, n)))};
+            return Layout{shp, IT(same_type(d, tdiv(d.v, n)))};
         }
     };
     return F{n}(l.shape, l.stride);
@@ -1235,7 +1241,7 @@ bool elem_less(const IT& a, const IT& b) {  // int_tuple.jl:197-211
 IT increment(const IT& coord, const IT& shape) {  // int_tuple.jl:218-232: next 1-based coordinate, wrapping
     if (!coord.is_tuple()) {
         const Int c = leaf_of(coord), s = leaf_of(shape);
-        return c.v < s.v ? IT(add(c, Int(1, c.s))) : IT(Int(1, c.s));
+        return c.v < s.v ? IT(same_type(c, c.v + 1)) : IT(same_type(c, 1));
     }
     if (!shape.is_tuple() || shape.size() != coord.size()) raise(MOYE_ERR_RANK, "increment: coordinate and shape differ in rank");
     const IT &c = coord[0], &s = shape[0];

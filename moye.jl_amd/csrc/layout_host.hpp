@@ -24,14 +24,23 @@ struct Error : std::runtime_error {
     Error(moye_status st, const std::string& msg) : std::runtime_error(msg), status(st) {}
 };
 
+// A dynamic integer is an Int (64 bits) or an Int32 (`w32`; src/utilities.jl:1-11: IntType = Union{Int, StaticInt,
+// Int32}).  Julia's promotion decides the type of a result: static with static stays static, a static operand takes the
+// other's type (promote_rule(StaticInt, Int32) = Int32), Int32 with Int32 is Int32, anything with an Int is an Int.
+// Int32 results wrap modulo 2^32 as Julia's do.  In text a dynamic Int32 carries the suffix `i32` ("5i32").
 struct Int {
     int64_t v = 0;
-    bool s = false;  // static
+    bool s = false;    // static
+    bool w32 = false;  // dynamic Int32 (never set on a static integer)
     Int() = default;
-    Int(int64_t v_, bool s_) : v(v_), s(s_) {}
+    Int(int64_t v_, bool s_, bool w32_ = false) : v(w32_ && !s_ ? (int64_t)(int32_t)v_ : v_), s(s_), w32(w32_ && !s_) {}
 };
 inline Int S(int64_t v) { return Int(v, true); }
 inline Int D(int64_t v) { return Int(v, false); }
+inline Int D32(int64_t v) { return Int(v, false, true); }
+// the result of an operation on a and b / on a alone, with value v
+inline Int promoted(int64_t v, Int a, Int b) { return Int(v, a.s && b.s, (a.s || a.w32) && (b.s || b.w32)); }
+inline Int same_type(Int a, int64_t v) { return Int(v, a.s, a.w32); }
 
 // An IntTuple: a leaf integer, a colon (only inside coordinates and tiles) or a tuple of IntTuples.
 struct IT {

@@ -480,6 +480,10 @@ int32_t moye_layout_eval(const char* layout, const char* coord, int64_t* index) 
         return (int32_t)MOYE_OK;
     });
 }
+int32_t moye_layout_eval_typed(const char* layout, const char* coord, char* out, size_t cap) {
+    MOYE_REQUIRE(layout && coord && out);
+    return guarded([&] { return put(to_string(IT(eval(parse_layout(layout), parse_int_tuple(coord)))), out, cap); });
+}
 int32_t moye_layout_size(const char* layout, int64_t* n) {
     MOYE_REQUIRE(layout && n);
     return guarded([&] {

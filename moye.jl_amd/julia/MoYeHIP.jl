@@ -71,6 +71,26 @@ struct TiledCopyDesc              # moye_tiled_copy
     flags::Int32
 end
 
+struct GemmEpilogue               # moye_gemm_epilogue
+    alpha::Cfloat
+    beta::Cfloat
+    op::Int32
+    _pad::Int32
+    operand::Ptr{Tensor}
+    scalar::Cdouble
+end
+
+# moye_map / epilogue operations
+const MAP_IDENTITY = Int32(0)
+const MAP_ADD = Int32(1)
+const MAP_SUB = Int32(2)
+const MAP_MUL = Int32(3)
+const MAP_DIV = Int32(4)
+const MAP_MAX = Int32(5)
+const MAP_MIN = Int32(6)
+const MAP_NEG = Int32(7)
+const MAP_ABS = Int32(8)
+
 const UNIVERSAL_FMA = Int32(0)
 const MFMA_F32_16x16x32_F16 = Int32(1)
 const MFMA_F32_32x32x16_F16 = Int32(2)
@@ -114,8 +134,17 @@ function Tensor(x::MoYeArray{T}) where {T}
 end
 
 # ---- host-side layout algebra through the library -------------------------------------------
-# Layouts cross the boundary in MoYe's own printed form; `string(layout)` is already that form.
+# Layouts cross the boundary in MoYe's own printed form (`string(layout)`), with `i32` added to run-time Int32 integers.
 # The results are parsed back with MoYe's constructors by `parse_layout` below.
+
+# Text form of an IntTuple for the library: MoYe prints an Int32 like an Int, so the width is added here ("5i32");
+# results carry it back, and an index computed from Int32 and static integers only comes back as an Int32
+# (test/layout.jl:4-12 of MoYe).
+int_text(x::Int32) = string(x, "i32")
+int_text(x::Colon) = ":"
+int_text(x::Tuple) = length(x) == 1 ? string("(", int_text(x[1]), ",)") : string("(", join((int_text(e) for e in x), ", "), ")")
+int_text(x) = string(x)
+layout_text(l::Layout) = string(int_text(shape(l)), ":", int_text(stride(l)))
 
 function parse_int_tuple(s::AbstractString)
     s = strip(s)
@@ -133,6 +162,8 @@ function parse_int_tuple(s::AbstractString)
         return Tuple(parse_int_tuple(p) for p in parts)
     elseif startswith(s, "_")
         return static(parse(Int, s[2:end]))
+    elseif endswith(s, "i32")
+        return parse(Int32, s[1:end-3])
     else
         return parse(Int, s)
     end
@@ -150,8 +181,12 @@ function parse_layout(s::AbstractString)
     MoYe.make_layout(parse_int_tuple(s))
 end
 
-tile_text(t::Tuple) = "<" * join((x isa Layout ? string(x) : x isa Colon ? ":" : string(x) for x in t), ", ") * ">"
-tile_text(x) = string(x)
+# any argument of the host algebra as text: layouts and IntTuples with their integer widths, text as it is
+txt(x::Layout) = layout_text(x)
+txt(x::AbstractString) = x
+txt(x) = int_text(x)
+tile_text(t::Tuple) = "<" * join((txt(x) for x in t), ", ") * ">"
+tile_text(x) = txt(x)
 
 macro layout_call(sym, args...)
     quote
@@ -162,72 +197,73 @@ macro layout_call(sym, args...)
     end
 end
 
-coalesce(l::Layout) = @layout_call moye_layout_coalesce string(l)
-filter(l::Layout) = @layout_call moye_layout_filter string(l)
-flatten_layout(l::Layout) = @layout_call moye_layout_flatten string(l)
-composition(a::Layout, b) = @layout_call moye_layout_composition string(a) tile_text(b)
-complement(l::Layout, cotarget = "") = @layout_call moye_layout_complement string(l) string(cotarget)
-right_inverse(l::Layout) = @layout_call moye_layout_right_inverse string(l)
-left_inverse(l::Layout) = @layout_call moye_layout_left_inverse string(l)
-logical_product(l::Layout, t) = @layout_call moye_layout_logical_product string(l) tile_text(t)
-zipped_product(l::Layout, t) = @layout_call moye_layout_zipped_product string(l) tile_text(t)
-tiled_product(l::Layout, t) = @layout_call moye_layout_tiled_product string(l) tile_text(t)
-logical_divide(l::Layout, t) = @layout_call moye_layout_logical_divide string(l) tile_text(t)
-zipped_divide(l::Layout, t) = @layout_call moye_layout_zipped_divide string(l) tile_text(t)
-tiled_divide(l::Layout, t) = @layout_call moye_layout_tiled_divide string(l) tile_text(t)
-make_fragment_like(l::Layout) = @layout_call moye_layout_make_fragment_like string(l)
-normalize(l::Layout) = @layout_call moye_layout_normalize string(l)
+coalesce(l::Layout) = @layout_call moye_layout_coalesce txt(l)
+filter(l::Layout) = @layout_call moye_layout_filter txt(l)
+flatten_layout(l::Layout) = @layout_call moye_layout_flatten txt(l)
+composition(a::Layout, b) = @layout_call moye_layout_composition txt(a) tile_text(b)
+complement(l::Layout, cotarget = "") = @layout_call moye_layout_complement txt(l) txt(cotarget)
+right_inverse(l::Layout) = @layout_call moye_layout_right_inverse txt(l)
+left_inverse(l::Layout) = @layout_call moye_layout_left_inverse txt(l)
+logical_product(l::Layout, t) = @layout_call moye_layout_logical_product txt(l) tile_text(t)
+zipped_product(l::Layout, t) = @layout_call moye_layout_zipped_product txt(l) tile_text(t)
+tiled_product(l::Layout, t) = @layout_call moye_layout_tiled_product txt(l) tile_text(t)
+logical_divide(l::Layout, t) = @layout_call moye_layout_logical_divide txt(l) tile_text(t)
+zipped_divide(l::Layout, t) = @layout_call moye_layout_zipped_divide txt(l) tile_text(t)
+tiled_divide(l::Layout, t) = @layout_call moye_layout_tiled_divide txt(l) tile_text(t)
+make_fragment_like(l::Layout) = @layout_call moye_layout_make_fragment_like txt(l)
+normalize(l::Layout) = @layout_call moye_layout_normalize txt(l)
 
 function blocked_product(block::Layout, l::Layout, coalesce_result::Bool = false)
     buf = Vector{UInt8}(undef, CAP)
     check(ccall((:moye_layout_blocked_product, LIB), Int32, (Cstring, Cstring, Int32, Ptr{UInt8}, Csize_t),
-                string(block), string(l), Int32(coalesce_result), buf, CAP))
+                txt(block), txt(l), Int32(coalesce_result), buf, CAP))
     parse_layout(unsafe_string(pointer(buf)))
 end
 
 function raked_product(block::Layout, l::Layout, coalesce_result::Bool = false)
     buf = Vector{UInt8}(undef, CAP)
     check(ccall((:moye_layout_raked_product, LIB), Int32, (Cstring, Cstring, Int32, Ptr{UInt8}, Csize_t),
-                string(block), string(l), Int32(coalesce_result), buf, CAP))
+                txt(block), txt(l), Int32(coalesce_result), buf, CAP))
     parse_layout(unsafe_string(pointer(buf)))
 end
 
 function recast(l::Layout, ::Type{New}, ::Type{Old}) where {New,Old}
     buf = Vector{UInt8}(undef, CAP)
     check(ccall((:moye_layout_recast, LIB), Int32, (Cstring, Int32, Int32, Ptr{UInt8}, Csize_t),
-                string(l), Int32(sizeof(New)), Int32(sizeof(Old)), buf, CAP))
+                txt(l), Int32(sizeof(New)), Int32(sizeof(Old)), buf, CAP))
     parse_layout(unsafe_string(pointer(buf)))
 end
 
+# `layout(coord)`.  The result has the type MoYe's own arithmetic would give it: a StaticInt when layout and coordinate
+# are static, an Int32 when their run-time integers all are (`@Layout((2,(2,2)),(2,(1,4)))(Int32(2)) isa Int32`,
+# test/layout.jl:4-12), an Int otherwise.
 function layout_index(l::Layout, coord)
-    idx = Ref{Int64}(0)
-    check(ccall((:moye_layout_eval, LIB), Int32, (Cstring, Cstring, Ptr{Int64}), string(l), string(coord), idx))
-    idx[]
+    buf = Vector{UInt8}(undef, 64)
+    check(ccall((:moye_layout_eval_typed, LIB), Int32, (Cstring, Cstring, Ptr{UInt8}, Csize_t),
+                layout_text(l), int_text(coord), buf, 64))
+    parse_int_tuple(unsafe_string(pointer(buf)))
 end
-# The library computes in 64 bits; the reference's index has the integer type of the coordinate
-# (`@Layout((2,(2,2)),(2,(1,4)))(Int32(2)) isa Int32`, test/layout.jl:4-12): an Int32 coordinate gets an Int32 index back.
-layout_index(l::Layout, coord::Int32) = Int32(invoke(layout_index, Tuple{Layout,Any}, l, coord))
 
 function layout_size(l::Layout)
     n = Ref{Int64}(0)
-    check(ccall((:moye_layout_size, LIB), Int32, (Cstring, Ptr{Int64}), string(l), n)); n[]
+    check(ccall((:moye_layout_size, LIB), Int32, (Cstring, Ptr{Int64}), txt(l), n)); n[]
 end
 
 function layout_cosize(l::Layout)
     n = Ref{Int64}(0)
-    check(ccall((:moye_layout_cosize, LIB), Int32, (Cstring, Ptr{Int64}), string(l), n)); n[]
+    check(ccall((:moye_layout_cosize, LIB), Int32, (Cstring, Ptr{Int64}), txt(l), n)); n[]
 end
 
 function max_common_vector(a::Layout, b::Layout)
     n = Ref{Int64}(0)
-    check(ccall((:moye_layout_max_common_vector, LIB), Int32, (Cstring, Cstring, Ptr{Int64}), string(a), string(b), n))
+    check(ccall((:moye_layout_max_common_vector, LIB), Int32, (Cstring, Cstring, Ptr{Int64}), txt(a), txt(b), n))
     n[]
 end
 
 function tuple_op(op::AbstractString, a, b = "", c = "")
     buf = Vector{UInt8}(undef, CAP)
     check(ccall((:moye_tuple_op, LIB), Int32, (Cstring, Cstring, Cstring, Cstring, Ptr{UInt8}, Csize_t),
-                op, string(a), string(b), string(c), buf, CAP))
+                op, txt(a), txt(b), txt(c), buf, CAP))
     unsafe_string(pointer(buf))
 end
 
@@ -235,7 +271,7 @@ end
 function local_tile(x::MoYeArray{T}, tile::Tuple, coord::Tuple, proj = "") where {T}
     buf = Vector{UInt8}(undef, CAP); off = Ref{Int64}(0)
     check(ccall((:moye_local_tile, LIB), Int32, (Cstring, Cstring, Cstring, Cstring, Ptr{UInt8}, Csize_t, Ptr{Int64}),
-                string(MoYe.layout(x)), tile_text(tile), tile_text(coord), string(proj), buf, CAP, off))
+                txt(MoYe.layout(x)), tile_text(tile), tile_text(coord), txt(proj), buf, CAP, off))
     MoYeArray(pointer(x) + off[] * sizeof(T), parse_layout(unsafe_string(pointer(buf))))
 end
 
@@ -244,7 +280,7 @@ function local_partition(x::MoYeArray{T}, thr::Layout, idx::Integer, proj = "") 
     buf = Vector{UInt8}(undef, CAP); off = Ref{Int64}(0)
     check(ccall((:moye_local_partition, LIB), Int32,
                 (Cstring, Cstring, Cstring, Cstring, Ptr{UInt8}, Csize_t, Ptr{Int64}),
-                string(MoYe.layout(x)), string(thr), string(idx), string(proj), buf, CAP, off))
+                txt(MoYe.layout(x)), txt(thr), txt(idx), txt(proj), buf, CAP, off))
     MoYeArray(pointer(x) + off[] * sizeof(T), parse_layout(unsafe_string(pointer(buf))))
 end
 
@@ -253,14 +289,14 @@ end
 function make_tiled_mma(atom::Int32, atom_layout::Layout, permutation::Tuple = ())
     d = Ref{TiledMMADesc}()
     check(ccall((:moye_make_tiled_mma, LIB), Int32, (Int32, Cstring, Cstring, Ptr{TiledMMADesc}),
-                atom, string(atom_layout), isempty(permutation) ? "" : tile_text(permutation), d))
+                atom, txt(atom_layout), isempty(permutation) ? "" : tile_text(permutation), d))
     d[]
 end
 
 function tiled_mma_query(atom::AbstractString, atom_layout::Layout, permutation, what::AbstractString; cap = CAP)
     buf = Vector{UInt8}(undef, cap)
     check(ccall((:moye_tiled_mma_query, LIB), Int32, (Cstring, Cstring, Cstring, Cstring, Ptr{UInt8}, Csize_t),
-                atom, string(atom_layout), permutation === nothing ? "" : tile_text(permutation), what, buf, cap))
+                atom, txt(atom_layout), permutation === nothing ? "" : tile_text(permutation), what, buf, cap))
     unsafe_string(pointer(buf))
 end
 
@@ -274,8 +310,8 @@ function tiled_mma_partition(atom::AbstractString, atom_layout::Layout, permutat
     buf = Vector{UInt8}(undef, CAP); off = Ref{Int64}(0)
     check(ccall((:moye_tiled_mma_partition, LIB), Int32,
                 (Cstring, Cstring, Cstring, Int32, Cchar, Cstring, Ptr{UInt8}, Csize_t, Ptr{Int64}),
-                atom, string(atom_layout), permutation === nothing ? "" : tile_text(permutation), Int32(thr_idx),
-                Cchar(operand), string(MoYe.layout(x)), buf, CAP, off))
+                atom, txt(atom_layout), permutation === nothing ? "" : tile_text(permutation), Int32(thr_idx),
+                Cchar(operand), txt(MoYe.layout(x)), buf, CAP, off))
     MoYeArray(pointer(x) + off[] * sizeof(T), parse_layout(unsafe_string(pointer(buf))))
 end
 
@@ -283,7 +319,7 @@ function tiled_copy_query(src_bits, dst_bits, val_bits, thr::Layout, val::Layout
     buf = Vector{UInt8}(undef, cap)
     check(ccall((:moye_tiled_copy_query, LIB), Int32,
                 (Int32, Int32, Int32, Cstring, Cstring, Cstring, Ptr{UInt8}, Csize_t),
-                Int32(src_bits), Int32(dst_bits), Int32(val_bits), string(thr), string(val), what, buf, cap))
+                Int32(src_bits), Int32(dst_bits), Int32(val_bits), txt(thr), txt(val), what, buf, cap))
     unsafe_string(pointer(buf))
 end
 
@@ -296,8 +332,8 @@ function tiled_copy_partition(src_bits, dst_bits, val_bits, thr::Layout, val::La
     buf = Vector{UInt8}(undef, CAP); off = Ref{Int64}(0)
     check(ccall((:moye_tiled_copy_partition, LIB), Int32,
                 (Int32, Int32, Int32, Cstring, Cstring, Int32, Cchar, Cstring, Ptr{UInt8}, Csize_t, Ptr{Int64}),
-                Int32(src_bits), Int32(dst_bits), Int32(val_bits), string(thr), string(val), Int32(thr_idx),
-                Cchar(which), string(MoYe.layout(x)), buf, CAP, off))
+                Int32(src_bits), Int32(dst_bits), Int32(val_bits), txt(thr), txt(val), Int32(thr_idx),
+                Cchar(which), txt(MoYe.layout(x)), buf, CAP, off))
     MoYeArray(pointer(x) + off[] * sizeof(T), parse_layout(unsafe_string(pointer(buf))))
 end
 
@@ -306,7 +342,7 @@ function tiled_copy_tv_query(src_bits, dst_bits, val_bits, layout_tv::Layout, ti
     buf = Vector{UInt8}(undef, CAP)
     check(ccall((:moye_tiled_copy_tv_query, LIB), Int32,
                 (Int32, Int32, Int32, Cstring, Cstring, Cstring, Ptr{UInt8}, Csize_t),
-                Int32(src_bits), Int32(dst_bits), Int32(val_bits), string(layout_tv), string(tiler), what, buf, CAP))
+                Int32(src_bits), Int32(dst_bits), Int32(val_bits), txt(layout_tv), txt(tiler), what, buf, CAP))
     unsafe_string(pointer(buf))
 end
 
@@ -315,8 +351,8 @@ function tiled_copy_tv_partition(src_bits, dst_bits, val_bits, layout_tv::Layout
     buf = Vector{UInt8}(undef, CAP); off = Ref{Int64}(0)
     check(ccall((:moye_tiled_copy_tv_partition, LIB), Int32,
                 (Int32, Int32, Int32, Cstring, Cstring, Int32, Cchar, Cstring, Ptr{UInt8}, Csize_t, Ptr{Int64}),
-                Int32(src_bits), Int32(dst_bits), Int32(val_bits), string(layout_tv), string(tiler), Int32(thr_idx),
-                Cchar(which), string(MoYe.layout(x)), buf, CAP, off))
+                Int32(src_bits), Int32(dst_bits), Int32(val_bits), txt(layout_tv), txt(tiler), Int32(thr_idx),
+                Cchar(which), txt(MoYe.layout(x)), buf, CAP, off))
     MoYeArray(pointer(x) + off[] * sizeof(T), parse_layout(unsafe_string(pointer(buf))))
 end
 
@@ -325,18 +361,18 @@ function tiled_copy_tv_retile(src_bits, dst_bits, val_bits, layout_tv::Layout, t
     buf = Vector{UInt8}(undef, CAP)
     check(ccall((:moye_tiled_copy_tv_retile, LIB), Int32,
                 (Int32, Int32, Int32, Cstring, Cstring, Cstring, Ptr{UInt8}, Csize_t),
-                Int32(src_bits), Int32(dst_bits), Int32(val_bits), string(layout_tv), string(tiler), string(l), buf, CAP))
+                Int32(src_bits), Int32(dst_bits), Int32(val_bits), txt(layout_tv), txt(tiler), txt(l), buf, CAP))
     parse_layout(unsafe_string(pointer(buf)))
 end
 
 function tile_to_shape(l::Layout, trg_shape::Tuple, order = "")
     buf = Vector{UInt8}(undef, CAP)
     check(ccall((:moye_layout_tile_to_shape, LIB), Int32, (Cstring, Cstring, Cstring, Ptr{UInt8}, Csize_t),
-                string(l), string(trg_shape), string(order), buf, CAP))
+                txt(l), txt(trg_shape), txt(order), buf, CAP))
     parse_layout(unsafe_string(pointer(buf)))
 end
 
-make_layout_like(l::Layout) = @layout_call moye_layout_make_like string(l)
+make_layout_like(l::Layout) = @layout_call moye_layout_make_like txt(l)
 
 "One wave executes the atom once through its (thr,val) tables: D(M,N) = A(M,K) * B(N,K)' on dense column-major device tiles."
 mma_atom_probe(atom::Int32, A::Ptr{Cvoid}, B::Ptr{Cvoid}, D::Ptr{Cvoid}; stream = C_NULL) =
@@ -368,12 +404,6 @@ function copyto!(dst::MoYeArray, src::MoYeArray; tiled_copy::Union{Nothing,Tiled
     dst
 end
 
-"""
-    gemm!(mma, D, A, B[, C]; alpha=1f0, stream=C_NULL)
-
-`gemm!(mma, D, A, B, C)` (src/algorithm/blas.jl:11-17) over whole device operands:
-A:(M,K), B:(N,K), C,D:(M,N); D = alpha * A * B' + C.  Returns `nothing` like the reference.
-"""
 "copyto_if!(dst, src, mask) (src/algorithm/copy.jl:4-16); `mask` is a MoYeArray{Bool} (one byte per logical element)."
 function copyto_if!(dst::MoYeArray, src::MoYeArray, mask::MoYeArray{Bool}; stream::Ptr{Cvoid} = C_NULL)
     m = Tensor(recast(UInt8, mask))
@@ -382,6 +412,12 @@ function copyto_if!(dst::MoYeArray, src::MoYeArray, mask::MoYeArray{Bool}; strea
     dst
 end
 
+"""
+    gemm!(mma, D, A, B[, C]; alpha=1f0, stream=C_NULL)
+
+`gemm!(mma, D, A, B, C)` (src/algorithm/blas.jl:11-17) over whole device operands:
+A:(M,K), B:(N,K), C,D:(M,N); D = alpha * A * B' + C.  Returns `nothing` like the reference.
+"""
 function gemm!(mma::TiledMMADesc, D::MoYeArray, A::MoYeArray, B::MoYeArray, C::Union{Nothing,MoYeArray} = nothing;
                alpha::Real = 1.0f0, stream::Ptr{Cvoid} = C_NULL)
     m, d, a, b = Ref(mma), Ref(Tensor(D)), Ref(Tensor(A)), Ref(Tensor(B))
@@ -399,6 +435,54 @@ function gemm!(mma::TiledMMADesc, D::MoYeArray, A::MoYeArray, B::MoYeArray, C::U
     end
     nothing
 end
+
+"""
+    gemm_ex!(mma, D, A, B[, C]; alpha, beta, op, operand, scalar, workspace, workspace_bytes, stream)
+
+gemm! with the epilogue a MoYe kernel applies to its accumulator fragment fused in: `axpby!` (src/algorithm/blas.jl:1-9)
+and one broadcast operation (src/broadcast.jl:5-41), D = op.(alpha * A * B' + beta * C, operand).  `operand` is an
+(M,N) MoYeArray (a stride of 0 repeats a bias vector along that mode) or `nothing` (then `scalar`).  The workspace, when
+the call needs one (`gemm_workspace_size`), comes from the caller; this entry point never allocates.
+"""
+function gemm_ex!(mma::TiledMMADesc, D::MoYeArray, A::MoYeArray, B::MoYeArray, C::Union{Nothing,MoYeArray} = nothing;
+                  alpha::Real = 1.0f0, beta::Real = C === nothing ? 0.0f0 : 1.0f0, op::Int32 = MAP_IDENTITY,
+                  operand::Union{Nothing,MoYeArray} = nothing, scalar::Real = 0.0,
+                  workspace::Ptr{Cvoid} = C_NULL, workspace_bytes::Integer = 0, stream::Ptr{Cvoid} = C_NULL)
+    m, d, a, b = Ref(mma), Ref(Tensor(D)), Ref(Tensor(A)), Ref(Tensor(B))
+    x = operand === nothing ? nothing : Ref(Tensor(operand))
+    c = C === nothing ? nothing : Ref(Tensor(C))
+    GC.@preserve D A B C operand x c begin
+        xp = x === nothing ? Ptr{Tensor}(C_NULL) : Base.unsafe_convert(Ptr{Tensor}, x)
+        cp = c === nothing ? Ptr{Tensor}(C_NULL) : Base.unsafe_convert(Ptr{Tensor}, c)
+        ep = Ref(GemmEpilogue(Float32(alpha), Float32(beta), op, Int32(0), xp, Float64(scalar)))
+        check(ccall((:moye_gemm_ex, LIB), Int32,
+                    (Ptr{TiledMMADesc}, Ptr{Tensor}, Ptr{Tensor}, Ptr{Tensor}, Ptr{Tensor}, Ptr{GemmEpilogue}, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
+                    m, d, a, b, cp, ep, workspace, workspace_bytes, stream))
+    end
+    nothing
+end
+
+"""
+    gemm_noalloc!(mma, D, A, B[, C]; alpha=1f0, stream=C_NULL)
+
+gemm! for callers that cannot allocate device memory (under graph capture): the workspace is a static 32 MiB array
+inside the library; a call that needs more throws an ArgumentError.
+"""
+function gemm_noalloc!(mma::TiledMMADesc, D::MoYeArray, A::MoYeArray, B::MoYeArray, C::Union{Nothing,MoYeArray} = nothing;
+                       alpha::Real = 1.0f0, stream::Ptr{Cvoid} = C_NULL)
+    m, d, a, b = Ref(mma), Ref(Tensor(D)), Ref(Tensor(A)), Ref(Tensor(B))
+    c = C === nothing ? nothing : Ref(Tensor(C))
+    GC.@preserve D A B C c begin
+        cp = c === nothing ? Ptr{Tensor}(C_NULL) : Base.unsafe_convert(Ptr{Tensor}, c)
+        check(ccall((:moye_gemm_noalloc, LIB), Int32,
+                    (Ptr{TiledMMADesc}, Ptr{Tensor}, Ptr{Tensor}, Ptr{Tensor}, Ptr{Tensor}, Cfloat, Ptr{Cvoid}),
+                    m, d, a, b, cp, Float32(alpha), stream))
+    end
+    nothing
+end
+
+"Frees the per-stream workspaces `gemm!` keeps for NN / NT / TT operands and split-K (waits for the device first)."
+gemm_release_workspace() = check(ccall((:moye_gemm_release_workspace, LIB), Int32, ()))
 
 """
     axpby!(a, X, b, Y; stream=C_NULL)
@@ -498,7 +582,7 @@ end
 
 function print_layout(l::Layout)
     buf = Vector{UInt8}(undef, 1 << 20)
-    check(ccall((:moye_layout_print, LIB), Int32, (Cstring, Ptr{UInt8}, Csize_t), string(l), buf, 1 << 20))
+    check(ccall((:moye_layout_print, LIB), Int32, (Cstring, Ptr{UInt8}, Csize_t), txt(l), buf, 1 << 20))
     println(unsafe_string(pointer(buf)))
 end
 

@@ -13,7 +13,7 @@ from ._lib import (BF16, COPY_LDS_TILED, COPY_UNIVERSAL, F8E4M3, F16, F32, F64, 
                    MoyeError, Tensor, TiledCopy, TiledMMA, check, lib, make_tensor)
 from . import device
 from .device import device_info, gemm_epilogue, gemm_ex_, gemm_noalloc_, gemm_release_workspace, mfma_ceiling, mma_atom_probe, tiled_copy_desc, tiled_mma_desc, time_copy, time_gemm, gemm_workspace_size, version
-from .layout import (COLON, GenColMajor, GenRowMajor, Layout, StaticInt, append, blocked_product, coalesce,
+from .layout import (COLON, GenColMajor, GenRowMajor, Int32, Layout, StaticInt, append, blocked_product, coalesce,
                      compact_col_major, compact_row_major, complement, composition, coord_to_index, cosize, depth,
                      flatten, index_to_coord, left_inverse, logical_divide, logical_product, make_fragment_like,
                      make_layout, make_ordered_layout, max_common_vector, prepend, raked_product, rank, recast,

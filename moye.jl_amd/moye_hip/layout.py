@@ -22,6 +22,16 @@ class StaticInt(int):
         return "_%d" % int(self)
 
 
+class Int32(int):
+    """A run-time 32-bit integer (Julia `Int32`), written `5i32` in text: results computed from Int32 and static
+    integers only stay Int32 (test/layout.jl:4-12 of the reference)."""
+
+    __slots__ = ()
+
+    def __repr__(self):
+        return "%di32" % int(self)
+
+
 class _Colon:
     def __repr__(self):
         return ":"
@@ -47,7 +57,7 @@ def tuple_text(t):
         return "(%s,)" % inner if len(t) == 1 else "(%s)" % inner
     if t is COLON or t is Ellipsis or t == ":":
         return ":"
-    return repr(t) if isinstance(t, StaticInt) else str(int(t))
+    return repr(t) if isinstance(t, (StaticInt, Int32)) else str(int(t))
 
 
 def parse_tuple(text):
@@ -76,6 +86,9 @@ def parse_tuple(text):
         while j < len(text) and (text[j].isdigit() or text[j] in "_-"):
             j += 1
         tok = text[pos[0]:j]
+        if text.startswith("i32", j):
+            pos[0] = j + 3
+            return Int32(int(tok))
         pos[0] = j
         return StaticInt(int(tok[1:])) if tok.startswith("_") else int(tok)
 
@@ -201,9 +214,10 @@ class Layout:
         c = coord[0] if len(coord) == 1 else tuple(coord)
         if _has_colon(c):
             return slice_and_offset(self, c)[0]
-        out = C.c_int64()
-        check(_l().moye_layout_eval(_b(self.text), _b(tuple_text(c)), C.byref(out)))
-        return out.value
+        # the typed form: a StaticInt, an Int32 or an int, as the reference's result type would be
+        f = _l().moye_layout_eval_typed
+        f.argtypes = [C.c_char_p, C.c_char_p, C.c_char_p, C.c_size_t]
+        return parse_tuple(_text_out(f, _b(self.text), _b(tuple_text(c))))
 
     def __getitem__(self, i):
         s, d = self.shape, self.stride

@@ -48,7 +48,9 @@ class S(int):
     __str__ = __repr__
 
     def _w(self, other, r):
-        return S(r) if isinstance(other, S) else int(r)
+        if isinstance(other, S):
+            return S(r)
+        return I32(r) if isinstance(other, I32) else int(r)
 
     def __add__(self, o):
         return self._w(o, int(self) + int(o))
@@ -85,6 +87,77 @@ class S(int):
 
     def __abs__(self):
         return S(abs(int(self)))
+
+
+def _wrap32(r):
+    return (int(r) + 2 ** 31) % 2 ** 32 - 2 ** 31
+
+
+class I32(int):
+    """A run-time `Int32` (src/utilities.jl:1-11: IntType = Union{Int, StaticInt, Int32}), printed `5i32`.  Julia's
+    promotion: with a static integer or another Int32 the result is an Int32 (promote_rule(StaticInt, Int32) = Int32),
+    with an Int it is an Int; Int32 arithmetic wraps modulo 2^32."""
+
+    __slots__ = ()
+
+    def __new__(cls, v):
+        return super().__new__(cls, _wrap32(v))
+
+    def __repr__(self):
+        return "%di32" % int(self)
+
+    __str__ = __repr__
+
+    def _w(self, other, r):
+        return I32(r) if isinstance(other, (I32, S)) else int(r)
+
+    def __add__(self, o):
+        return self._w(o, int(self) + int(o))
+
+    __radd__ = __add__
+
+    def __sub__(self, o):
+        return self._w(o, int(self) - int(o))
+
+    def __rsub__(self, o):
+        return self._w(o, int(o) - int(self))
+
+    def __mul__(self, o):
+        if isinstance(o, S) and int(o) == 0:
+            return S(0)
+        return self._w(o, int(self) * int(o))
+
+    __rmul__ = __mul__
+
+    def __floordiv__(self, o):
+        return self._w(o, tdiv(int(self), int(o)))
+
+    def __rfloordiv__(self, o):
+        return self._w(o, tdiv(int(o), int(self)))
+
+    def __mod__(self, o):
+        return self._w(o, trem(int(self), int(o)))
+
+    def __rmod__(self, o):
+        return self._w(o, trem(int(o), int(self)))
+
+    def __neg__(self):
+        return I32(-int(self))
+
+    def __abs__(self):
+        return I32(abs(int(self)))
+
+
+def one(x):
+    """Julia `one(x)`: 1 in the type of x."""
+    return _1 if isinstance(x, S) else I32(1) if isinstance(x, I32) else 1
+
+
+def _promote(r, *xs):
+    """r in the type Julia's promotion gives a result computed from xs."""
+    if all(isinstance(x, S) for x in xs):
+        return S(r)
+    return I32(r) if all(isinstance(x, (S, I32)) for x in xs) else int(r)
 
 
 def tdiv(a, b):
@@ -136,13 +209,11 @@ def dynamic(x):
 
 
 def smin(a, b):
-    r = min(int(a), int(b))
-    return S(r) if isinstance(a, S) and isinstance(b, S) else r
+    return _promote(min(int(a), int(b)), a, b)
 
 
 def smax(a, b):
-    r = max(int(a), int(b))
-    return S(r) if isinstance(a, S) and isinstance(b, S) else r
+    return _promote(max(int(a), int(b)), a, b)
 
 
 def sabs(a):
@@ -150,13 +221,11 @@ def sabs(a):
 
 
 def ssign(a):
-    r = (int(a) > 0) - (int(a) < 0)
-    return S(r) if isinstance(a, S) else r
+    return _promote((int(a) > 0) - (int(a) < 0), a)
 
 
 def cld(a, b):
-    r = -((-int(a)) // int(b))
-    return S(r) if isinstance(a, S) and isinstance(b, S) else r
+    return _promote(-((-int(a)) // int(b)), a, b)
 
 
 # --------------------------------------------------------------------------
@@ -368,7 +437,7 @@ def shape_div(a, b):
             raise AssertionError("Cannot divide %d by %d or vice versa" % (a, b))
     q = tdiv(int(a), int(b))
     r = q if q != 0 else int(ssign(a)) * int(ssign(b))
-    return S(r) if isinstance(a, S) and isinstance(b, S) else r
+    return _promote(r, a, b)
 
 
 def elem_scale(x, y):
@@ -521,13 +590,13 @@ def _offset(x):
         return _0
     if is_tuple(x):
         return tuple(_offset(e) for e in x)
-    return x - _1 if isinstance(x, S) else x - 1
+    return x - one(x)
 
 
 def coord_to_index(coord, shape, stride=None):
-    """stride.jl:82-89 — 1-based coordinate to 1-based index."""
+    """stride.jl:82-89 — 1-based coordinate to 1-based index; `one(idx)` keeps the integer type."""
     idx = coord_to_index0(_offset(coord), shape, stride)
-    return idx + (_1 if isinstance(idx, S) else 1)
+    return idx + one(idx)
 
 
 def index_to_coord(index, shape, stride=None):
@@ -552,8 +621,8 @@ def index_to_coord(index, shape, stride=None):
         return tuple(index_to_coord(index, s, d) for s, d in zip(shape, stride))
     if isinstance(shape, S) and shape == 1:
         return _0
-    crd = ((index - 1) // stride) % shape
-    return crd + 1
+    crd = ((index - one(index)) // stride) % shape
+    return crd + one(crd)
 
 
 def coord_to_coord(coord, src_shape, dst_shape):
@@ -1128,8 +1197,7 @@ def upcast(l, m):
             if strd == 0:
                 return Layout(shp, strd)
             return Layout(shape_div(shp, shape_div(m, sabs(strd))), shape_div(strd, m))
-        q = tdiv(int(strd), int(m))
-        return Layout(shp, q)
+        return Layout(shp, _promote(tdiv(int(strd), int(m)), strd, m))  # safe_div(stride, m()), layout.jl:943,955-958: div keeps the stride's integer type
 
     return f(l.shape, l.stride)
 
@@ -1196,7 +1264,7 @@ def make_fragment_like(l):
 # text form:  "(_2, (_1, _6)):(_1, (_6, _2))"
 # --------------------------------------------------------------------------
 
-_TOK = re.compile(r"\s*(_?-?\d+|[(),:])")
+_TOK = re.compile(r"\s*(_?-?\d+(?:i32)?|[(),:])")
 
 
 def print_layout(layout):
@@ -1233,6 +1301,8 @@ def parse_int_tuple(text):
             return tuple(out)
         if t == ":":
             return COLON
+        if t.endswith("i32"):
+            return I32(int(t[:-3]))
         return S(int(t[1:])) if t.startswith("_") else int(t)
 
     v = item()

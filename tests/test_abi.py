@@ -65,3 +65,55 @@ def test_julia_glue_binds_declared_symbols_only():
     used = set(re.findall(r":(moye_[a-z0-9_]+)", text))
     assert used, "no ccall found"
     assert used <= set(declared_functions()), sorted(used - set(declared_functions()))
+
+
+def _julia_blocks(text):
+    """A rough reading of Julia source, enough for the two mistakes that would stop `include` before anything runs:
+    returns (orphans, depth): docstrings that are not directly followed by something to document, and the balance
+    of block openers against `end`."""
+    lines = text.split("\n")
+    orphans, depth, i = [], 0, 0
+    opener = re.compile(r"^\s*(function|struct|mutable struct|module|macro|if|for|while|let|begin|quote|try|do)\b|"
+                        r"\b(begin|do|quote)\s*$|=\s*(begin|let|quote)\b|\b(function)\s*\(")
+    definition = re.compile(r"^\s*(function|struct|mutable struct|macro|const|module|abstract type|@\w+|[\w.!]+(\{.*\})?\(.*\)\s*(where\b.*)?=|[\w.!]+\s*=)")
+    while i < len(lines):
+        line = lines[i]
+        stripped = line.strip()
+        doc_end = None
+        if stripped.startswith('"""'):
+            j = i if stripped.count('"""') >= 2 and len(stripped) > 3 else i + 1
+            while j < len(lines) and '"""' not in lines[j] and j != i:
+                j += 1
+            doc_end = j
+        elif re.match(r'^"([^"\\]|\\.)*"\s*$', stripped) and not line.startswith(" "):
+            doc_end = i
+        if doc_end is not None:
+            nxt = lines[doc_end + 1] if doc_end + 1 < len(lines) else ""
+            if not definition.match(nxt):
+                orphans.append((i + 1, nxt.strip()[:60]))
+            i = doc_end + 1
+            continue
+        code = re.sub(r'"([^"\\]|\\.)*"', '""', line.split("#")[0])
+        if not re.search(r"\bend\b", code) or not re.match(r"^\s*(if|for|while|function|struct|try|let|begin|quote|macro|module)\b.*\bend\s*$", code):
+            if opener.search(code):
+                depth += 1
+            if re.match(r"^\s*end\b", code) or re.search(r"\bend\s*$", code) and not opener.search(code):
+                depth -= 1
+        i += 1
+    return orphans, depth
+
+
+def test_julia_glue_has_no_orphan_docstrings_and_balanced_blocks():
+    """Julia refuses to load a file in which a docstring is followed by another string literal or a blank line
+    ("cannot document the following expression"), and one with an unmatched `end`.  No Julia runtime exists here, so
+    the two are checked textually; the scanner is itself checked on small samples."""
+    good = 'module M\n"""\n    f(x)\n\ndoc\n"""\nfunction f(x)\n    x\nend\n"one-line doc"\ng(x) = x\nend\n'
+    assert _julia_blocks(good) == ([], 0)
+    bad = 'module M\n"""\ndoc of f\n"""\n"doc of g"\ng(x) = x\nfunction f(x)\n    x\nend\nend\n'
+    orphans, depth = _julia_blocks(bad)
+    assert len(orphans) == 1 and orphans[0][0] == 2 and depth == 0
+    assert _julia_blocks('function f(x)\n    if x\n        1\n    end\n')[1] == 1
+    path = os.path.join(ROOT, "moye.jl_amd", "julia", "MoYeHIP.jl")
+    orphans, depth = _julia_blocks(open(path).read())
+    assert not orphans, orphans
+    assert depth == 0

@@ -517,3 +517,58 @@ def test_host_print_layout_matches_the_reference_docstrings():
         assert text == lo.print_layout(lo.parse_layout(t["layout"]))
     with pytest.raises(MoyeError):
         ml.print_layout(ml.Layout("(_2,_2,_2)"), file=False)
+
+
+# ---- Int32: the coordinate's integer type survives (test/layout.jl:4-12, src/utilities.jl:1-11) -----------------------
+
+def test_int32_known_answers_through_the_abi():
+    a = ml.Layout("(_2,(_2,_2)):(_2,(_1,_4))")
+    r = a(ml.Int32(2))
+    assert type(r) is ml.Int32 and r == 3
+    assert type(a(2)) is int and type(a(ml.StaticInt(2))) is ml.StaticInt
+    b = ml.make_layout((ml.Int32(2), ml.Int32(4)))
+    assert b.text == "(2i32, 4i32):(_1, 2i32)"
+    r = b(ml.Int32(2))
+    assert type(r) is ml.Int32 and r == 2
+    assert type(b(2)) is int
+    assert repr(ml.index_to_coord(ml.Int32(7), a.shape, a.stride)) == "(2i32, (1i32, 2i32))"
+    assert repr(ml.coord_to_index((ml.Int32(2), (ml.Int32(1), ml.Int32(2))), a.shape, a.stride)) == "7i32"
+    w = ml.Layout("4i32:1073741824i32")
+    assert repr(w(ml.Int32(4))) == "-1073741823i32" and w(4) == 3 * 2 ** 30 + 1     # wraps as Julia's Int32 does
+    assert repr(ml.compact_col_major((ml.Int32(3), ml.Int32(5), ml.StaticInt(2)))) == "(_1, 3i32, 15i32)"
+    with pytest.raises(MoyeError) as e:
+        ml.Layout("_4i32:_1")                  # a static integer has no width
+    assert e.value.status == ERR_PARSE
+    with pytest.raises(MoyeError) as e:
+        ml.Layout("4294967296i32:_1")
+    assert e.value.status == ERR_PARSE
+
+
+def test_int32_random_differential():
+    """The C++ algebra against the oracle on random layouts whose dynamic integers are a mix of Int32 and Int: the
+    printed results agree, widths included."""
+    rng = random.Random(77)
+
+    def widen(text):      # every dynamic integer becomes an Int32 with probability 0.7
+        import re
+        return re.sub(r"(?<![_\d])(\d+)(?![\d])", lambda m: m.group(1) + ("i32" if rng.random() < 0.7 else ""), text)
+
+    n = 0
+    for _ in range(300):
+        ta, tb = widen(_rand_layout(rng, 0.5)), widen(_rand_layout(rng, 0.5))
+        a, b, oa, ob = ml.Layout(ta), ml.Layout(tb), lo.parse_layout(ta), lo.parse_layout(tb)
+        assert a.text == repr(oa)
+        _both(lambda: ml.coalesce(a), lambda: lo.coalesce(oa))
+        _both(lambda: ml.filter(a), lambda: lo.lfilter(oa))
+        _both(lambda: ml.composition(a, b), lambda: lo.composition(oa, ob))
+        _both(lambda: ml.logical_divide(a, b), lambda: lo.logical_divide(oa, ob))
+        _both(lambda: ml.logical_product(a, b), lambda: lo.logical_product(oa, ob))
+        _both(lambda: ml.recast(a, 2, 4), lambda: lo.recast_layout(oa, 2, 4))
+        _both(lambda: ml.recast(a, 4, 2), lambda: lo.recast_layout(oa, 4, 2))
+        for i in range(1, min(ml.size(a), 8) + 1):
+            for c, oc in ((ml.Int32(i), lo.I32(i)), (i, i), (ml.StaticInt(i), lo.S(i))):
+                assert repr(a(c)) == repr(oa(oc)), (ta, i)
+            if "0" not in [t.strip("_i32") for t in ta.split(":")[1].replace("(", "").replace(")", "").split(",")]:  # no stride of 0
+                assert repr(ml.index_to_coord(ml.Int32(i), a.shape, a.stride)) == repr(lo.index_to_coord(lo.I32(i), oa.shape, oa.stride))
+        n += 1
+    assert n == 300

@@ -299,3 +299,32 @@ def test_print_layout_matches_the_reference_docstrings():
     for t in tables:
         got = [line.rstrip() for line in lo.print_layout(lo.parse_layout(t["layout"])).split("\n")]
         assert got == t["lines"], t["expression"]
+
+
+def test_int32_known_answers():
+    """test/layout.jl:4-12 of the reference: a layout called with an Int32 gives an Int32, for a static layout
+    (promote_rule(StaticInt, Int32) = Int32, src/utilities.jl:4-6) and for a layout made of Int32 shapes; plus what
+    Julia's promotion and wrap-around fix for the other combinations."""
+    import layout_oracle as lo
+    a = lo.parse_layout("(_2,(_2,_2)):(_2,(_1,_4))")
+    r = a(lo.I32(2))
+    assert type(r) is lo.I32 and int(r) == 3 and repr(r) == "3i32"
+    b = lo.make_layout((lo.I32(2), lo.I32(4)))
+    assert repr(b) == "(2i32, 4i32):(_1, 2i32)"
+    r = b(lo.I32(2))
+    assert type(r) is lo.I32 and int(r) == 2
+    assert type(b(2)) is int and b(2) == 2                       # Int32 with an Int is an Int
+    assert type(a(2)) is int and type(a(lo.S(2))) is lo.S        # static stays static
+    assert repr(lo.parse_layout("(2i32,4):(_1,2i32)")(lo.I32(7))) == "7"   # one Int among the inputs: an Int
+    # hierarchical coordinates and the way back
+    assert repr(a((lo.I32(2), (lo.I32(1), lo.I32(2))))) == "7i32"
+    assert repr(lo.index_to_coord(lo.I32(7), a.shape, a.stride)) == "(2i32, (1i32, 2i32))"
+    assert repr(lo.index_to_coord(lo.I32(5), (lo.I32(3), lo.I32(4)))) == "(2i32, 2i32)"
+    # Int32 arithmetic wraps as Julia's does: (4 - 1) * 2^30 = 3 * 2^30 -> -2^30, plus one
+    w = lo.parse_layout("4i32:1073741824i32")
+    assert repr(w(lo.I32(4))) == "-1073741823i32" and w(4) == 3 * 2 ** 30 + 1
+    assert repr(lo.parse_int_tuple("(2i32, (_3, 4))")) == "(2i32, (_3, 4))"
+    # the algebra carries the type: products of Int32 shapes, shape_div, coalesce of dynamic modes
+    assert repr(lo.compact_col_major((lo.I32(3), lo.I32(5), lo.S(2)))) == "(_1, 3i32, 15i32)"
+    assert repr(lo.shape_div(lo.I32(12), lo.S(4))) == "3i32" and repr(lo.shape_div(lo.I32(12), 4)) == "3"
+    assert repr(lo.size(lo.parse_layout("(2i32,_3,4i32):(_1,2i32,6i32)"))) == "24i32"

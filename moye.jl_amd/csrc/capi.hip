@@ -147,15 +147,41 @@ static int split_count(const moye_tiled_mma* mma, int64_t M, int64_t N, int64_t 
     return 1;
 }
 
+// An operand with its unit stride along M (N) instead of K needs no K-major copy when the call runs on the 256 x 256
+// kernel's transposing fragment reads (gemm_mfma256.hip): f16 / bf16 through the 16x16x32 atoms, the 256 x 256 x 64 tile
+// (named, or the library's own choice for this size), eight waves, the two-stage schedule; the operand dense along its
+// rows with a pitch of whole 16-byte pieces.
+static bool majors_run_natively(const moye_tiled_mma* mma, const Mat& A, const Mat& B) {
+    if (mma->atom != MOYE_MFMA_F32_16x16x32_F16 && mma->atom != MOYE_MFMA_F32_16x16x32_BF16) return false;
+    if ((mma->flags & (MOYE_GEMM_PINGPONG | MOYE_GEMM_WAVE4)) || mma->stages >= 3) return false;
+    if (mma->atom_layout_mnk[0] * mma->atom_layout_mnk[1] == 4) return false;
+    if (mma->split_k != 0 && mma->split_k != 1) return false;  // the K ranges of a split need not be whole k-tiles
+    const int64_t M = A.rows, N = B.rows, K = A.cols;
+    const int bm = mma->cta_tile_mnk[0], bn = mma->cta_tile_mnk[1], bk = mma->cta_tile_mnk[2];
+    if (M % 256 || N % 256 || K % 64) return false;
+    const bool named = bm == 256 && bn == 256 && (bk == 0 || bk == 64);
+    const bool chosen = bm == 0 && bn == 0 && bk == 0 && (M / 256) * (N / 256) >= 128;
+    if (!named && !chosen) return false;
+    for (const Mat* x : {&A, &B}) {
+        if (x->cs == 1 || x->cols == 1) continue;  // K-major already
+        if (x->rs != 1 || (x->cs * 2) % 16 || reinterpret_cast<uintptr_t>(x->ptr) % 16 || x->cs < x->rows) return false;
+    }
+    return true;
+}
+
 // K-major copies of A and B where needed, then the fp32 partial products of a split-K call
-static size_t gemm_workspace_bytes(const moye_tiled_mma* mma, const Mat& A, const Mat& B) {
+static size_t gemm_workspace_bytes_impl(const moye_tiled_mma* mma, const Mat& A, const Mat& B, bool native) {
     if (mma->atom == MOYE_MMA_UNIVERSAL_FMA) return 0;
     size_t n = 0;
-    if (A.cs != 1 && A.cols > 1) n += kmajor_bytes(A);
-    if (B.cs != 1 && B.cols > 1) n += kmajor_bytes(B);
+    if (!native && A.cs != 1 && A.cols > 1) n += kmajor_bytes(A);
+    if (!native && B.cs != 1 && B.cols > 1) n += kmajor_bytes(B);
     const int split = split_count(mma, A.rows, B.rows, A.cols, dtype_bytes(A.dtype));
     if (split > 1) n += (size_t)split * (size_t)A.rows * (size_t)B.rows * sizeof(float);
     return n;
+}
+
+static size_t gemm_workspace_bytes(const moye_tiled_mma* mma, const Mat& A, const Mat& B) {
+    return gemm_workspace_bytes_impl(mma, A, B, majors_run_natively(mma, A, B));
 }
 
 // transposes `m` (unit stride along its rows index) into ws as rows x K with K contiguous and rewrites `m`
@@ -236,7 +262,13 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
     // along K are brought to the K-major form the kernels read (one tiled transpose each)
     char* ws = nullptr;
     std::unique_lock<std::mutex> ws_lock(g_ws_mutex, std::defer_lock);
-    if (const size_t ws_bytes = gemm_workspace_bytes(mma, A, B)) {
+    const bool native_majors = majors_run_natively(mma, A, B);
+    int major_flags = 0;  // which of the kernel's operands keep their M- (N-) major form
+    if (native_majors) {
+        if (A.cs != 1 && A.cols > 1) { major_flags |= kGemmAMajorM; A.rs = A.cs; A.cs = 1; }  // Mat::rs now holds the pitch between consecutive k
+        if (B.cs != 1 && B.cols > 1) { major_flags |= kGemmBMajorN; B.rs = B.cs; B.cs = 1; }
+    }
+    if (const size_t ws_bytes = gemm_workspace_bytes_impl(mma, A, B, native_majors)) {
         if (mma->flags & MOYE_GEMM_NO_WORKSPACE)
             return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the MFMA kernels need K-major A and B (stride 1 along K, the 'TN' form), split_k needs room "
                                               "for its partial products, and MOYE_GEMM_NO_WORKSPACE forbids the use of a workspace");
@@ -250,12 +282,12 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
             ws_lock.lock();  // until every kernel of this call is enqueued
             if (int32_t e = library_workspace(ws_bytes, st, &ws)) return e;
         }
-        if (A.cs != 1 && A.cols > 1) {
+        if (!native_majors && A.cs != 1 && A.cols > 1) {
             const size_t nb = kmajor_bytes(A);
             if (int32_t e = make_kmajor(&A, ws, st)) return e;
             ws += nb;
         }
-        if (B.cs != 1 && B.cols > 1) {
+        if (!native_majors && B.cs != 1 && B.cols > 1) {
             const size_t nb = kmajor_bytes(B);
             if (int32_t e = make_kmajor(&B, ws, st)) return e;
             ws += nb;
@@ -298,7 +330,7 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
     const bool stream_d = stream_env >= 0 ? stream_env != 0
                           : dtype_bytes(D.dtype) == 2 ? !(in_dt == MOYE_F8E4M3 && many_tiles) : many_tiles;
     g.xcd_swizzle = !(mma->flags & MOYE_GEMM_NO_XCD_SWIZZLE) | (mma->flags & 0xff00) | (atom32 ? kGemmAtom32 : 0) | (rotate_k ? kGemmRotateK : 0) |
-                    (stream_d ? kGemmStreamD : 0);
+                    (stream_d ? kGemmStreamD : 0) | major_flags;
     if (const int split = split_count(mma, M, N, K, dtype_bytes(in_dt)); split > 1) {
         // K is cut into `split` equal ranges, all in one launch (gridDim.y); each range writes its fp32 product, compact and
         // row-major, into the workspace; a second pass sums the ranges in ascending order, applies alpha and C and converts
@@ -334,6 +366,8 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
         g.A = B.ptr; g.B = A.ptr; g.M = N; g.N = M; g.lda = B.rs; g.ldb = A.rs; g.ldd = D.cs;
         g.C = tC ? C.ptr : nullptr; g.ldc_m = C.cs; g.ldc_n = C.rs; g.D = D.ptr;
         std::swap(g.ep_xm, g.ep_xn);  // the kernel's m is the caller's n
+        g.xcd_swizzle = (g.xcd_swizzle & ~(kGemmAMajorM | kGemmBMajorN)) | ((major_flags & kGemmAMajorM) ? kGemmBMajorN : 0) |
+                        ((major_flags & kGemmBMajorN) ? kGemmAMajorM : 0);
         if (rows_in_16_byte_pieces(g.C, g.ldc_m, g.ldc_n, D.dtype)) g.xcd_swizzle |= kGemmRowC;
         return gemm_mfma_tn_dispatch(in_dt, D.dtype, bn, bm, bk, waves, mma->stages, g, st);
     }

@@ -20,13 +20,26 @@
 //
 // Same operand conventions as gemm_mfma.hip: K-major A and B, N-contiguous D, the MFMA issued
 // with B rows as its first operand so a lane holds four consecutive n of one m.
+#include <type_traits>
+
 #include "mfma_epilogue.hpp"
 
 namespace moye {
 
 // kOps: the epilogue may apply an element-wise operation (GemmArgs::ep_op).  A separate instance, so that the code and
 // the registers of that path never touch the kernel the plain gemm! runs.
-template <typename In, typename Out, int WGM, int WGN, bool kOps = false>
+//
+// AMAJ / BMAJ = 1: that operand is stored with its unit stride along M (N) instead of K, the 'N' forms of
+// src/arch/mma/make_mma_ops.jl:253-265 (GemmArgs::lda / ldb is then the pitch between consecutive k).  Its LDS tile is
+// 64 k-rows of 256 operand rows (512 bytes), brought in by the same load-to-LDS instructions, and the fragments come
+// out of it with ds_read_b64_tr_b16, the transposing LDS read of gfx950, where the reference has ldmatrix.trans
+// (src/arch/copy/ldmatrix.jl:18-48): sixteen lanes that each point at four consecutive 16-bit values of a row get back
+// the four values lane j's position holds in rows 0..3 of their group (measured on the hardware: result e of lane j of a
+// group is value j % 4 of the lane 4 e + j / 4).  With lane l = 16 g + s pointing at k-row 8 g + s / 4 (+ 4 for the second
+// read), m = m0 + 4 (s % 4), two reads give lane l the eight k of row m0 + l % 16 that the K-major ds_read_b128 would.
+// The 32-byte piece index of a k-row is XORed with (row % 4) | 4 ((row / 8) % 2): the eight row pieces the 32 lanes of
+// one pass read then lie in eight different bank groups.
+template <typename In, typename Out, int WGM, int WGN, bool kOps = false, int AMAJ = 0, int BMAJ = 0>
 __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
     constexpr int BM = 256, BN = 256, CPR = 8;  // 8 chunks of 16 bytes per tile row
     constexpr int A_CH = BM * CPR, B_CH = BN * CPR, STAGE = A_CH + B_CH;
@@ -51,6 +64,27 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
     const char* gA = static_cast<const char*>(p.A) + ((int64_t)tm * BM + lrow) * pitch_a + lch * 16;
     const char* gB = static_cast<const char*>(p.B) + ((int64_t)tn * BN + lrow) * pitch_b + lch * 16;
     const int dma_slot = __builtin_amdgcn_readfirstlane(wave * WROWS * CPR);  // + 8 rows * CPR per i
+    // An M-major (N-major) operand: wave w fills k-rows KROWS w + 2 i + l / 32 of the tile, two rows (1 KiB) per
+    // instruction; lane l brings the 16-byte chunk that belongs in physical slot l % 32 of its row.
+    constexpr int KROWS = 64 / NWAVES;
+    static_assert(!(AMAJ || BMAJ) || (In::kBytes == 2 && KROWS == 2 * LD), "transposing fragment reads: 16-bit operands");
+    auto tr_swz = [](int krow) { return (krow & 3) | (((krow >> 3) & 1) << 2); };
+    [[maybe_unused]] int64_t tA[AMAJ ? LD : 1], tB[BMAJ ? LD : 1];  // byte offsets of this lane's chunk, per instruction, from the k-tile's first row
+    if constexpr (AMAJ) {
+#pragma unroll
+        for (int i = 0; i < LD; ++i) {
+            const int krow = wave * KROWS + 2 * i + (lane >> 5), p16 = lane & 31, l32 = (p16 >> 1) ^ tr_swz(krow);
+            tA[i] = krow * pitch_a + ((int64_t)tm * BM) * In::kBytes + (l32 * 2 + (p16 & 1)) * 16;
+        }
+    }
+    if constexpr (BMAJ) {
+#pragma unroll
+        for (int i = 0; i < LD; ++i) {
+            const int krow = wave * KROWS + 2 * i + (lane >> 5), p16 = lane & 31, l32 = (p16 >> 1) ^ tr_swz(krow);
+            tB[i] = krow * pitch_b + ((int64_t)tn * BN) * In::kBytes + (l32 * 2 + (p16 & 1)) * 16;
+        }
+    }
+    const int dma_slot_t = __builtin_amdgcn_readfirstlane(wave * KROWS * 32);  // + 2 rows * 32 chunks per i
 
     // fragment slots: row = w?0 + 16 i + r16, chunk = 4 ks + kq
     int fa_slot[2], fb_slot[2];
@@ -61,6 +95,12 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
         fb_slot[ks] = A_CH + (wn0 + r16) * CPR + (ch ^ swz<CPR>(r16));
     }
 
+    // transposed operands: byte offset of this lane's first read of 16-row block 0 of k-step 0 inside the operand tile;
+    // block idx adds (idx << 5) by XOR (the piece index is swizzled), k-step ks adds 32 rows, the second read 4 rows
+    const int fx = ((r16 >> 2) & 3) | ((kq & 1) << 2);
+    const int ta_lane = (8 * kq + (r16 >> 2)) * 512 + (wm0 / 128) * 256 + ((((wm0 / 16) & 7) ^ fx) << 5) + 8 * (r16 & 3);
+    const int tb_lane = (8 * kq + (r16 >> 2)) * 512 + (wn0 / 128) * 256 + ((((wn0 / 16) & 7) ^ fx) << 5) + 8 * (r16 & 3);
+
     f32x4 acc[MI][NI];
 #pragma unroll
     for (int i = 0; i < MI; ++i)
@@ -69,15 +109,36 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
 
     const int ktiles = (int)(((int64_t)p.K * In::kBytes) / 128);
     u32x4 fa[2][MI], fb[2][NI];
+    typedef short v4s __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) v4s* tr_ptr_t;
+    // the eight k of one row of a transposed operand tile: two transposing reads, 4 k-rows apart
+    auto tr_frag = [&](const u32x4* tile16, int lane_off, int idx, int ks) __attribute__((always_inline)) -> u32x4 {
+        const char* base = reinterpret_cast<const char*>(tile16) + ((lane_off ^ (idx << 5)) + ks * 32 * 512);
+        const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_ptr_t)(base));
+        const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_ptr_t)(base + 4 * 512));
+        u32x2 l2, h2;
+        __builtin_memcpy(&l2, &lo, 8);
+        __builtin_memcpy(&h2, &hi, 8);
+        return u32x4{l2.x, l2.y, h2.x, h2.y};
+    };
 
     typedef __attribute__((address_space(1))) const void* gptr_t;
     typedef __attribute__((address_space(3))) void* lptr_t;
-#define MOYE_DMA(BASE, KOFF)                                                                          \
+    // KT: index of the k-tile (128 bytes of K: 64 k of a 16-bit type)
+#define MOYE_DMA(BASE, KT)                                                                            \
     _Pragma("unroll") for (int i = 0; i < LD; ++i) {                                                  \
-        __builtin_amdgcn_global_load_lds((gptr_t)(gA + (int64_t)(8 * i) * pitch_a + (KOFF)),          \
-                                         (lptr_t)((BASE) + dma_slot + 8 * CPR * i), 16, 0, 0);        \
-        __builtin_amdgcn_global_load_lds((gptr_t)(gB + (int64_t)(8 * i) * pitch_b + (KOFF)),          \
-                                         (lptr_t)((BASE) + A_CH + dma_slot + 8 * CPR * i), 16, 0, 0); \
+        if constexpr (AMAJ)                                                                           \
+            __builtin_amdgcn_global_load_lds((gptr_t)(static_cast<const char*>(p.A) + tA[i] + (int64_t)(KT) * 64 * pitch_a), \
+                                             (lptr_t)((BASE) + dma_slot_t + 64 * i), 16, 0, 0);       \
+        else                                                                                          \
+            __builtin_amdgcn_global_load_lds((gptr_t)(gA + (int64_t)(8 * i) * pitch_a + (int64_t)(KT) * 128), \
+                                             (lptr_t)((BASE) + dma_slot + 8 * CPR * i), 16, 0, 0);    \
+        if constexpr (BMAJ)                                                                           \
+            __builtin_amdgcn_global_load_lds((gptr_t)(static_cast<const char*>(p.B) + tB[i] + (int64_t)(KT) * 64 * pitch_b), \
+                                             (lptr_t)((BASE) + A_CH + dma_slot_t + 64 * i), 16, 0, 0); \
+        else                                                                                          \
+            __builtin_amdgcn_global_load_lds((gptr_t)(gB + (int64_t)(8 * i) * pitch_b + (int64_t)(KT) * 128), \
+                                             (lptr_t)((BASE) + A_CH + dma_slot + 8 * CPR * i), 16, 0, 0); \
     }
     // Wait until at most N of this wave's load-to-LDS instructions are in flight and its own LDS reads
     // have returned, then meet the other waves.  A bare s_barrier on purpose: __syncthreads() adds a
@@ -93,8 +154,14 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
     }
 #define MOYE_WAIT_LDS() __builtin_amdgcn_s_waitcnt(0xC07F) /* lgkmcnt(0) only */
 #define MOYE_FRAGS(BASE, KS, BUF)                                                                     \
-    _Pragma("unroll") for (int i = 0; i < MI; ++i) fa[BUF][i] = (BASE)[fa_slot[KS] + 16 * CPR * i];   \
-    _Pragma("unroll") for (int j = 0; j < NI; ++j) fb[BUF][j] = (BASE)[fb_slot[KS] + 16 * CPR * j];
+    _Pragma("unroll") for (int i = 0; i < MI; ++i) {                                                  \
+        if constexpr (AMAJ) fa[BUF][i] = tr_frag((BASE), ta_lane, i, KS);                             \
+        else fa[BUF][i] = (BASE)[fa_slot[KS] + 16 * CPR * i];                                         \
+    }                                                                                                 \
+    _Pragma("unroll") for (int j = 0; j < NI; ++j) {                                                  \
+        if constexpr (BMAJ) fb[BUF][j] = tr_frag((BASE) + A_CH, tb_lane, j, KS);                      \
+        else fb[BUF][j] = (BASE)[fb_slot[KS] + 16 * CPR * j];                                         \
+    }
 // Rows of the wave tile are walked back and forth, so that exactly one operand register set changes between
 // consecutive MFMAs: with dense operands the part is power-limited, and an MFMA-only loop over an 8 x 4 register
 // tile sustains 1.5-2 % more in this order than row by row (1980 against 1947 TFLOP/s).
@@ -128,17 +195,17 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
     // together, so that the panels they share are fetched into their L2 once, but the eight XCDs start an eighth of K
     // apart, so that at any moment the chip asks memory for eight different column blocks of A and B instead of one
     // (with K-major operands and a power-of-two pitch one column block lives in few channels).  k_of() hands out the
-    // byte offsets of successive k-tiles in that rotated order; the sum over k starts elsewhere but is the same sum.
+    // indices of successive k-tiles in that rotated order; the sum over k starts elsewhere but is the same sum.
     int k_next = (p.xcd_swizzle & kGemmRotateK) ? (int)((int64_t)(blockIdx.x % 8) * ktiles / 8) : 0;
     auto k_of = [&]() {
-        const int64_t off = (int64_t)k_next * 128;
+        const int kt_now = k_next;
         k_next = k_next + 1 == ktiles ? 0 : k_next + 1;
-        return off;
+        return kt_now;
     };
     // prologue: tiles 0 and 1 on their way, wait for tile 0 only (LD loads per operand are younger)
-    { const int64_t ko = k_of(); MOYE_DMA(smem, ko) }
+    { const int ko = k_of(); MOYE_DMA(smem, ko) }
     if (ktiles > 1) {
-        { const int64_t ko = k_of(); MOYE_DMA(smem + STAGE, ko) }
+        { const int ko = k_of(); MOYE_DMA(smem + STAGE, ko) }
         MOYE_WAIT_BARRIER(2 * LD)
     } else {
         MOYE_WAIT_BARRIER(0)
@@ -165,7 +232,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
         __builtin_amdgcn_sched_barrier(0);                                                            \
         /* step 1: the stage tile KT lived in is free, so tile KT+2 gets a whole iteration to arrive; \
            MFMAs on buffer 1 (already in registers) while step 0 of tile KT+1 arrives in buffer 0 */  \
-        if (DMA) { const int64_t ko = k_of(); MOYE_DMA(cur, ko) }                                     \
+        if (DMA) { const int ko = k_of(); MOYE_DMA(cur, ko) }                                     \
         if (NEXT) MOYE_FRAGS(nxt, 0, 0)                                                               \
         MOYE_MMA(1, 0, MI)                                                                            \
         if (NEXT) { MOYE_INTERLEAVE((DMA) ? 2 * LD : 0) }                                             \
@@ -319,24 +386,33 @@ static int32_t launch256_ring(const GemmArgs& a, hipStream_t st) {
     return MOYE_OK;
 }
 
-template <typename In, typename Out, int WGM, int WGN>
-static int32_t launch256(const GemmArgs& a, hipStream_t st) {
+template <typename In, typename Out, int WGM, int WGN, bool kOps, int AMAJ, int BMAJ>
+static int32_t launch256_instance(const GemmArgs& a, hipStream_t st) {
     constexpr int kLds = 2 * (256 + 256) * 128;  // two operand stages, 128 KiB
-    const dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1));
-    if constexpr (WGM * WGN == 8) if (a.ep_op != MOYE_MAP_IDENTITY) {
-        auto kern = gemm_mfma_tn_256<In, Out, WGM, WGN, true>;
-        static LdsCap cap;
-        if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
-        kern<<<grid, dim3(64 * WGM * WGN), kLds, st>>>(a);
-        MOYE_HIP_CHECK(hipGetLastError());
-        return MOYE_OK;
-    }
-    auto kern = gemm_mfma_tn_256<In, Out, WGM, WGN, false>;
+    auto kern = gemm_mfma_tn_256<In, Out, WGM, WGN, kOps, AMAJ, BMAJ>;
     static LdsCap cap;
     if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
-    kern<<<grid, dim3(64 * WGM * WGN), kLds, st>>>(a);
+    kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1)), dim3(64 * WGM * WGN), kLds, st>>>(a);
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;
+}
+
+template <typename In, typename Out, int WGM, int WGN>
+static int32_t launch256(const GemmArgs& a, hipStream_t st) {
+    const bool am = a.xcd_swizzle & kGemmAMajorM, bm = a.xcd_swizzle & kGemmBMajorN;
+    if (am || bm) {
+        // operands that are not K-major: eight waves, 16-bit types (the host checked)
+        if constexpr (WGM * WGN == 8 && In::kBytes == 2) {
+            const bool ops = a.ep_op != MOYE_MAP_IDENTITY;
+            if (am && bm) return ops ? launch256_instance<In, Out, WGM, WGN, true, 1, 1>(a, st) : launch256_instance<In, Out, WGM, WGN, false, 1, 1>(a, st);
+            if (am) return ops ? launch256_instance<In, Out, WGM, WGN, true, 1, 0>(a, st) : launch256_instance<In, Out, WGM, WGN, false, 1, 0>(a, st);
+            return ops ? launch256_instance<In, Out, WGM, WGN, true, 0, 1>(a, st) : launch256_instance<In, Out, WGM, WGN, false, 0, 1>(a, st);
+        } else {
+            return fail(MOYE_ERR_UNSUPPORTED, "gemm!: operands that are not K-major run natively with 16-bit types on eight waves only");
+        }
+    }
+    if constexpr (WGM * WGN == 8) if (a.ep_op != MOYE_MAP_IDENTITY) return launch256_instance<In, Out, WGM, WGN, true, 0, 0>(a, st);
+    return launch256_instance<In, Out, WGM, WGN, false, 0, 0>(a, st);
 }
 
 template <typename In>

@@ -32,6 +32,8 @@ struct GemmArgs {
 constexpr int kGemmAtom32 = 0x10000;   // in GemmArgs::xcd_swizzle: issue the 32x32 MFMA forms
 constexpr int kGemmRowC = 0x80000;    // in GemmArgs::xcd_swizzle: C has unit stride along n, 16-byte aligned rows: read in 128-bit pieces
 constexpr int kGemmStreamD = 0x40000;  // in GemmArgs::xcd_swizzle: D is written with non-temporal stores
+constexpr int kGemmAMajorM = 0x100000;  // in GemmArgs::xcd_swizzle: A has its unit stride along M, lda is the pitch between consecutive k
+constexpr int kGemmBMajorN = 0x200000;  // the same for B and N (the 256 x 256 kernel's transposing fragment reads; 16-bit types)
 constexpr int kGemmRotateK = 0x20000;  // in GemmArgs::xcd_swizzle: each XCD starts its walk over K at its own eighth
 
 // UniversalFMA GEMM, any strides (gemm_universal.hip)

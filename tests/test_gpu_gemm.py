@@ -1327,3 +1327,79 @@ def test_fused_epilogue_limits(mh):
         mh.gemm_ex_(mh.tiled_mma_desc(mh.MMA_UNIVERSAL_FMA, cta_tile=(32, 32, 8)), T(d0.float()), T(af), T(bf), None,
                     mh.gemm_epilogue(op=_lib.MAP_ABS))
     assert e.value.status == _lib.ERR_UNSUPPORTED
+
+
+# ---------------------------------------------------------------------------------------------
+# operands that are not K-major, without a workspace: the 256x256 kernel's transposing fragment reads
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("tdt,atom", [("float16", "MFMA_F32_16x16x32_F16"), ("bfloat16", "MFMA_F32_16x16x32_BF16")])
+@pytest.mark.parametrize("majors", ["mk", "kn", "mn"])
+def test_operand_majors_native_exact_on_integers(mh, tdt, atom, majors):
+    """A stored M-major and / or B stored N-major (NN / NT / TT of src/arch/mma/make_mma_ops.jl:253-265) through the
+    256x256 tile with MOYE_GEMM_NO_WORKSPACE: no K-major copy is made, the fragments come out of LDS through the
+    transposing read.  Small integers, so every misplaced element shows; named tile and the library's choice, row- and
+    column-major D, C and alpha, fp32 and 16-bit results, a padded pitch, and the epilogue operation."""
+    from moye_hip import _lib
+    tdt = getattr(torch, tdt)
+    atom = getattr(mh, atom)
+    g = torch.Generator().manual_seed(71)
+    cases = [(512, 768, 256, (256, 256, 64), 0), (256, 256, 64, (256, 256, 0), 8), (2048, 4096, 128, (0, 0, 0), 0), (512, 512, 16384, (256, 256, 64), 0)]
+    for (M, N, K, cta, pad) in cases:
+        A = torch.randint(-3, 4, (M, K), generator=g).to(tdt)
+        B = torch.randint(-3, 4, (N, K), generator=g).to(tdt)
+        ref = A.double() @ B.double().t()
+        assert float(ref.abs().max()) < 2 ** 24
+        a_k, b_k = A.cuda(), B.cuda()
+        # M-major / N-major storage with a pitch of M + pad (N + pad) elements between consecutive k
+        a_m = torch.zeros(K, M + pad, dtype=tdt)
+        a_m[:, :M] = A.t()
+        b_n = torch.zeros(K, N + pad, dtype=tdt)
+        b_n[:, :N] = B.t()
+        a_m, b_n = a_m.cuda(), b_n.cuda()
+        ta = T(a_m, (M, K), (1, M + pad)) if majors[0] == "m" else T(a_k)
+        tb = T(b_n, (N, K), (1, N + pad)) if majors[1] == "n" else T(b_k)
+        mma = mh.tiled_mma_desc(atom, atom_layout=(2, 4, 1), cta_tile=cta, flags=_lib.GEMM_NO_WORKSPACE)
+        for out_dt in (torch.float32, tdt):
+            d = torch.zeros(M, N, dtype=out_dt, device="cuda")
+            assert mh.gemm_workspace_size(mma, T(d), ta, tb) == 0
+            mh.gemm_(mma, T(d), ta, tb)
+            torch.cuda.synchronize()
+            want = ref if out_dt == torch.float32 else ref.to(out_dt).double()
+            assert torch.equal(d.cpu().double(), want), (M, N, K, cta, out_dt, "row-major D")
+        C0 = torch.randint(-8, 9, (M, N), generator=g).float()
+        dt_ = torch.zeros(N, M, dtype=torch.float32, device="cuda")
+        mh.gemm_(mma, T(dt_, (M, N), (1, M)), ta, tb, T(C0.cuda()), 0.5)
+        torch.cuda.synchronize()
+        assert torch.equal(dt_.t().cpu().double(), 0.5 * ref + C0.double()), (M, N, K, cta, "column-major D, C, alpha")
+        if K <= 256:
+            bias = torch.randint(-5, 6, (N,), generator=g).float()
+            d = torch.zeros(M, N, dtype=torch.float32, device="cuda")
+            mh.gemm_ex_(mma, T(d), ta, tb, None,
+                        mh.gemm_epilogue(alpha=1.0, op=_lib.MAP_MAX, operand=T(bias.cuda(), (M, N), (0, 1))))
+            torch.cuda.synchronize()
+            assert torch.equal(d.cpu().double(), torch.maximum(ref, bias.double()[None, :])), (M, N, K, "max with a bias row")
+
+
+def test_operand_majors_native_random_and_speed(mh):
+    """fp16 NN 4096^3 (A M-major, B N-major) on random data against fp64, and its time beside the TN form's."""
+    from moye_hip import _lib
+    M = N = K = 4096
+    g = torch.Generator().manual_seed(1003)
+    A = (torch.randn(M, K, generator=g) / K ** 0.5).half()
+    B = (torch.randn(N, K, generator=g) / K ** 0.5).half()
+    a_k, b_k = A.cuda(), B.cuda()
+    a_m, b_n = A.t().contiguous().cuda(), B.t().contiguous().cuda()
+    c64 = a_k.double() @ b_k.double().t()
+    mma = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 4, 1), cta_tile=(256, 256, 64), flags=_lib.GEMM_NO_WORKSPACE)
+    times = {}
+    for name, ta, tb in (("TN", T(a_k), T(b_k)), ("NN", T(a_m, (M, K), (1, M)), T(b_n, (N, K), (1, N))),
+                         ("A M-major", T(a_m, (M, K), (1, M)), T(b_k)), ("B N-major", T(a_k), T(b_n, (N, K), (1, N)))):
+        d = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+        mh.gemm_(mma, T(d), ta, tb)
+        torch.cuda.synchronize()
+        assert relerr(d, c64) <= TOL16, name
+        mh.time_gemm(mma, T(d), ta, tb, None, 1.0, None, warmup=20, iters=100)
+        times[name] = mh.time_gemm(mma, T(d), ta, tb, None, 1.0, None, warmup=5, iters=100)
+    print("fp16 4096^3 by operand major: " + ", ".join("%s %.1f us" % (k, v * 1e3) for k, v in times.items()))
+    assert times["NN"] < 1.25 * times["TN"]

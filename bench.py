@@ -22,12 +22,15 @@ PEAK_F16_TFLOPS = 2500.0   # MI355X dense fp16/bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # Bytes that leave the L2s per launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script
 # (the summaries are committed under profiles/), each reading scaled by what the same counter shows for the
-# 1 GiB plain copy (fetch x2.0000, write x1.0000).  Only valid for the default tile/waves/flags.
+# 1 GiB plain copy (fetch x2.0000, write x1.0000).  Only valid for the default tile/waves/flags.  These are figures
+# from the profiled sessions, not from the run that prints them (TRAFFIC_SOURCE goes into every roofline object);
+# where sessions differ (the 8192^3 GEMMs: how far the XCDs drift apart varies) the median session is quoted.
+TRAFFIC_SOURCE = "profiles/*_counters.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this script in earlier sessions; not measured in this run)"
 MEASURED_TRAFFIC = {
     "gemm_f16_4096_tile256": {"read_bytes": 196894 * 1024, "write_bytes": 32781 * 1024},
     "transpose_f32_16384": {"read_bytes": 1048637 * 1024, "write_bytes": 1049561 * 1024},
     "gemm_bf16_8192_tile256": {"read_bytes": 1575798 * 1024, "write_bytes": 262640 * 1024},
-    "gemm_f32_8192_tile256": {"read_bytes": 6980880 * 1024, "write_bytes": 262152 * 1024},
+    "gemm_f32_8192_tile256": {"read_bytes": 2 * 2422808 * 1024, "write_bytes": 262152 * 1024},  # median of six sessions
     "gemm_fp8_8192_tile256": {"read_bytes": 786997 * 1024, "write_bytes": 131072 * 1024},
     "gemm_bf16_16x8192x8192": {"read_bytes": 149528 * 1024, "write_bytes": 512 * 1024},
 }
@@ -81,6 +84,54 @@ def cpu_baseline(cores):
     return res
 
 
+def headline_variants(mh, tensor_of, torch, stream, A, B, D):
+    """The headline problem (fp16 4096^3, the operands of the timed run) through other descriptors: the CTA tile the
+    baseline's config 3 names (128x128x32), operands stored M- / N-major (no K-major copy), and a fused epilogue
+    (bias row added, then max with 0 taken per element: one launch)."""
+    from moye_hip import _lib
+    res = []
+    flops = 2.0 * 4096 ** 3
+    tA, tB, tD = tensor_of(A), tensor_of(B), tensor_of(D)
+
+    def timed(name, fn, timer):
+        t_ramp = time.perf_counter()
+        while time.perf_counter() - t_ramp < 0.2:
+            for _ in range(20):
+                fn()
+            torch.cuda.synchronize()
+        ms = timer()
+        res.append({"workload": name, "kernel_ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 1),
+                    "roofline": {"bound": "mfma", "achieved": round(flops / ms / 1e9, 1), "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
+                                 "frac": round(flops / ms / 1e9 / PEAK_F16_TFLOPS, 4), "traffic": None}})
+
+    m128 = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 2, 1), tile=(128, 128, 32), cta_tile=(128, 128, 32))
+    timed("fp16 TN 4096^3 on the CTA tile config 3 names: 128x128x32, 2x2 waves",
+          lambda: mh.gemm_(m128, tD, tA, tB, None, 1.0, stream),
+          lambda: mh.time_gemm(m128, tD, tA, tB, None, 1.0, stream, warmup=3, iters=50))
+    m256 = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 4, 1), cta_tile=(256, 256, 64), flags=_lib.GEMM_NO_WORKSPACE)
+    At, Bt = A.t().contiguous(), B.t().contiguous()
+    tAm, tBn = tensor_of(At, (4096, 4096), (1, 4096)), tensor_of(Bt, (4096, 4096), (1, 4096))
+    timed("fp16 NN 4096^3 (A M-major, B N-major, no K-major copies), CTA 256x256x64",
+          lambda: mh.gemm_(m256, tD, tAm, tBn, None, 1.0, stream),
+          lambda: mh.time_gemm(m256, tD, tAm, tBn, None, 1.0, stream, warmup=3, iters=50))
+    bias = torch.randn(4096, device="cuda")
+    ep = mh.gemm_epilogue(alpha=1.0, beta=0.0, op=_lib.MAP_ADD, operand=tensor_of(bias, (4096, 4096), (0, 1)))
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def ev():
+        e0.record()
+        for _ in range(50):
+            mh.gemm_ex_(m256, tD, tA, tB, None, ep, None, 0, stream)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / 50
+    timed("fp16 TN 4096^3 with a bias row added in the epilogue (moye_gemm_ex), CTA 256x256x64",
+          lambda: mh.gemm_ex_(m256, tD, tA, tB, None, ep, None, 0, stream), ev)
+    mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 4, 1), cta_tile=(256, 256, 64)), tD, tA, tB, None, 1.0, stream)
+    torch.cuda.synchronize()
+    return res
+
+
 def other_configs(mh, tensor_of, torch, stream):
     """The remaining GEMM workloads of the baseline: bf16 8192^3 (fp32 out), fp8 e4m3 8192^3 with per-tensor
     scales (bf16 out), and the HBM-bound short-M case bf16 16 x 8192 x 8192.  Kernel time by HIP events."""
@@ -104,7 +155,8 @@ def other_configs(mh, tensor_of, torch, stream):
         if peak:
             entry["roofline"] = {"bound": "mfma", "achieved": entry["tflops"], "peak": peak, "unit": "TFLOP/s",
                                  "frac": round(entry["tflops"] / peak, 4),
-                                 "traffic": sum(MEASURED_TRAFFIC[traffic_key].values()) if traffic_key else None}
+                                 "traffic": sum(MEASURED_TRAFFIC[traffic_key].values()) if traffic_key else None,
+                                 "traffic_source": TRAFFIC_SOURCE if traffic_key else None}
         else:
             nbytes = a.numel() * a.element_size() + b.numel() * b.element_size() + d.numel() * d.element_size()
             gbs = nbytes / ms / 1e6
@@ -148,7 +200,7 @@ def other_configs(mh, tensor_of, torch, stream):
                 "rel_err_vs_fp64": float((d16.double() - c64).abs().max() / c64.abs().max()),
                 "roofline": {"bound": "hbm", "achieved": round(nbytes / ms / 1e6, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                              "frac": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4), "algorithmic_bytes": nbytes,
-                             "traffic": sum(MEASURED_TRAFFIC["gemm_bf16_16x8192x8192"].values())}})
+                             "traffic": sum(MEASURED_TRAFFIC["gemm_bf16_16x8192x8192"].values()), "traffic_source": TRAFFIC_SOURCE}})
     del bs, a, b, d
     if hasattr(torch, "float8_e4m3fn"):
         x = torch.randn(n, n, generator=g, device="cuda")
@@ -286,7 +338,7 @@ def main():
                    "rel_err_vs_fp64": err},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_F16_TFLOPS, 4), "traffic": gemm_traffic,
-                     "kernel_ms": round(kern_ms, 5)},
+                     "traffic_source": TRAFFIC_SOURCE if gemm_traffic else None, "kernel_ms": round(kern_ms, 5)},
     }
 
     if not args.no_yardsticks:
@@ -312,13 +364,14 @@ def main():
             "config": {"workload": "16384x16384 fp32 column-major -> row-major through 64x64 LDS tiles", "bit_exact_sample": ok},
             "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                          "frac": round(gbs / PEAK_HBM_GBS, 4),
-                         "traffic": sum(MEASURED_TRAFFIC["transpose_f32_16384"].values()), "kernel_ms": round(cms, 5)},
+                         "traffic": sum(MEASURED_TRAFFIC["transpose_f32_16384"].values()), "traffic_source": TRAFFIC_SOURCE,
+                         "kernel_ms": round(cms, 5)},
             "plain_copy_gbs": round(nbytes / (pms * 1e-3) / 1e9, 1),
         }
         del src, dst
 
     if not args.no_other:
-        out["other_configs"] = other_configs(mh, tensor_of, torch, stream)
+        out["other_configs"] = headline_variants(mh, tensor_of, torch, stream, A, B, D) + other_configs(mh, tensor_of, torch, stream)
 
     if not args.no_cpu:
         cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else os.cpu_count()

@@ -6,7 +6,9 @@
 // partial accumulators are summed through LDS in wave order, which makes the result independent
 // of timing.  A (at most 64 x K) is re-read by every workgroup and lives in L2; with 32 rows of B
 // per workgroup each A fragment feeds two MFMAs, which halves that L2 traffic (measured 33 us
-// against 38 us at 16 x 8192 x 8192 bf16; the bare B stream alone takes 22 us).
+// against 38 us at 16 x 8192 x 8192 bf16; the bare B stream alone takes 22 us).  More requests in flight make it
+// slower, not faster (same case, waves per workgroup x k-steps in flight per wave: 8 x 4 32.4 us, 4 x 8 34.3, 8 x 8 38.8,
+// 16 x 2 39.9, 16 x 4 41.5, 8 x 16 55.1): the kernel is not short of memory-level parallelism.
 //
 // Stands where the reference's user kernel would run gemm! (src/algorithm/blas.jl:11-131) on a
 // 16-row problem with its usual 128 x 128 tiles and waste 7/8 of each tile.
@@ -14,11 +16,10 @@
 
 namespace moye {
 
-template <typename In, typename Out, int MT, int NTW, int WAVES>
+template <typename In, typename Out, int MT, int NTW, int WAVES, int U = 4 /* 64-byte k-steps in flight per wave and row */>
 __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_skinny(GemmArgs p) {
     typedef typename Out::type OutT;
     split_of_block(p);
-    constexpr int U = 4;  // 64-byte k-steps in flight per wave and row
     __shared__ f32x4 part[WAVES][MT * NTW][64];
     const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, r16 = lane % 16, kq = lane / 16;
     const int n0 = blockIdx.x * 16 * NTW;

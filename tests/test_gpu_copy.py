@@ -752,6 +752,12 @@ def test_transpose_destination_rows_first_and_source_first_agree(mh):
         mh.copyto_(_tens(mh, dst, (ni, nj), (nj, 1)), _tens(mh, src, (ni, nj), (1, ni)))
         torch.cuda.synchronize()
         assert torch.equal(dst.view(ni, nj), src.view(nj, ni).t()), (ni, nj)
+    for (ni, nj) in ((4096, 3072), (3072, 4096), (3072, 3072), (2048, 2048)):      # the same for 2-byte elements
+        src = _rand_bits(ni * nj, ni + nj).to(torch.int16)
+        dst = torch.zeros_like(src)
+        mh.copyto_(_tens(mh, dst, (ni, nj), (nj, 1)), _tens(mh, src, (ni, nj), (1, ni)))
+        torch.cuda.synchronize()
+        assert torch.equal(dst.view(ni, nj), src.view(nj, ni).t()), (ni, nj, "int16")
     ni = nj = 2048
     src = _rand_bits(ni * nj * 3, 77)
     dst = torch.zeros_like(src)

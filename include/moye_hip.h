@@ -81,7 +81,8 @@ typedef enum {
 typedef struct {
     int32_t atom;                  /* moye_mma_atom                                           */
     int32_t atom_layout_mnk[3];    /* shape of TiledMMA.atom_layout_mnk (atom/mma.jl:84)       */
-    int32_t tile_mnk[3];           /* tile_size(mma, 1..3) (atom/mma.jl:178-191)               */
+    int32_t tile_mnk[3];           /* tile_size(mma, 1..3) (atom/mma.jl:178-191); for the record: the
+                                      kernels are chosen by cta_tile_mnk and atom_layout_mnk     */
     int32_t cta_tile_mnk[3];       /* bM, bN, bK; 0 = let the library choose                    */
     int32_t stages;                /* LDS pipeline depth, 0 = default                           */
     int32_t split_k;               /* 0/1 = none; >1 = K cut into that many equal ranges (each a
@@ -121,9 +122,12 @@ typedef enum {
 typedef struct {
     int32_t op;                    /* moye_copy_op                                             */
     int32_t vec_bits;              /* bits per access of the atom: 8..128 (UniversalCopy{UIntN}) */
-    int32_t thr_shape[2];          /* thr_layout of make_tiled_copy (atom/copy.jl:249-258)      */
+    int32_t thr_shape[2];          /* thr_layout of make_tiled_copy (atom/copy.jl:249-258); for the
+                                      record: the kernels' lane layouts are their own and no
+                                      result depends on thr_shape / val_shape                    */
     int32_t val_shape[2];          /* val_layout                                                */
-    int32_t tiler_mn[2];           /* tiler_MN = LDS tile, e.g. 64x64                           */
+    int32_t tiler_mn[2];           /* tiler_MN, e.g. 64x64 or the reference's 32x32; 0 = none.  Must
+                                      divide modes 1 and 2 of the array (zipped_divide's assertion) */
     int32_t flags;                 /* 0 or MOYE_GEMM_NO_LDS_SWIZZLE                              */
 } moye_tiled_copy;
 

@@ -214,6 +214,13 @@ static moye_gemm_epilogue plain_epilogue(float alpha) {
 
 // `caller_ws` / `caller_ws_bytes`: the workspace when the caller brings one (it must hold what
 // moye_gemm_workspace_size reports); with caller_ws == nullptr the library's own is used.
+// the epilogue operand as the 256 x 256 kernels like it: unit stride along the kernel's n, 16-byte aligned rows (or one row)
+static bool operand_rows_in_16_byte_pieces(const GemmArgs& g) {
+    if (!g.ep_x || g.ep_xn != 1) return false;
+    const int eb = dtype_bytes(g.ep_xdt);
+    return reinterpret_cast<uintptr_t>(g.ep_x) % 16 == 0 && (g.ep_xm * eb) % 16 == 0;
+}
+
 static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const moye_tensor* tA,
                          const moye_tensor* tB, const moye_tensor* tC, const moye_gemm_epilogue& ep, char* caller_ws,
                          size_t caller_ws_bytes, hipStream_t st) {
@@ -354,6 +361,7 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
         g.A = A.ptr; g.B = B.ptr; g.M = M; g.N = N; g.lda = A.rs; g.ldb = B.rs; g.ldd = D.rs;
         g.C = tC ? C.ptr : nullptr; g.ldc_m = C.rs; g.ldc_n = C.cs; g.D = D.ptr;
         if (rows_in_16_byte_pieces(g.C, g.ldc_m, g.ldc_n, D.dtype)) g.xcd_swizzle |= kGemmRowC;
+        if (operand_rows_in_16_byte_pieces(g)) g.xcd_swizzle |= kGemmEpiRowX;
         return gemm_mfma_tn_dispatch(in_dt, D.dtype, bm, bn, bk, waves, mma->stages, g, st);
     }
     if (D.rs == 1 && bm == 0 && bn == 0 && M <= 64 && ((int64_t)K * dtype_bytes(in_dt)) % 64 == 0) {
@@ -369,6 +377,7 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
         g.xcd_swizzle = (g.xcd_swizzle & ~(kGemmAMajorM | kGemmBMajorN)) | ((major_flags & kGemmAMajorM) ? kGemmBMajorN : 0) |
                         ((major_flags & kGemmBMajorN) ? kGemmAMajorM : 0);
         if (rows_in_16_byte_pieces(g.C, g.ldc_m, g.ldc_n, D.dtype)) g.xcd_swizzle |= kGemmRowC;
+        if (operand_rows_in_16_byte_pieces(g)) g.xcd_swizzle |= kGemmEpiRowX;
         return gemm_mfma_tn_dispatch(in_dt, D.dtype, bn, bm, bk, waves, mma->stages, g, st);
     }
     return fail(MOYE_ERR_UNSUPPORTED, "gemm!: D needs a unit stride along M or N");

@@ -34,6 +34,7 @@ constexpr int kGemmRowC = 0x80000;    // in GemmArgs::xcd_swizzle: C has unit st
 constexpr int kGemmStreamD = 0x40000;  // in GemmArgs::xcd_swizzle: D is written with non-temporal stores
 constexpr int kGemmAMajorM = 0x100000;  // in GemmArgs::xcd_swizzle: A has its unit stride along M, lda is the pitch between consecutive k
 constexpr int kGemmBMajorN = 0x200000;  // the same for B and N (the 256 x 256 kernel's transposing fragment reads; 16-bit types)
+constexpr int kGemmEpiRowX = 0x400000;  // in GemmArgs::xcd_swizzle: the epilogue operand has unit stride along n and 16-byte aligned rows (or one row)
 constexpr int kGemmRotateK = 0x20000;  // in GemmArgs::xcd_swizzle: each XCD starts its walk over K at its own eighth
 
 // UniversalFMA GEMM, any strides (gemm_universal.hip)

@@ -46,17 +46,73 @@ __device__ __forceinline__ void store_c_tile_general(const GemmArgs& p, const f3
         for (int t = 0; t < OUT_CH / 64; ++t) {
             const int c = lane + 64 * t, row = c / (WN / EPC), och = c % (WN / EPC);
             const int64_t m = m_base + PASS_ROWS * pass + row, n0 = n_base + och * EPC;
-            OutT out[EPC];
+            float v[EPC], x[EPC];
 #pragma unroll
             for (int q = 0; q < EPC / 4; ++q) {
                 const int chunk = och * (EPC / 4) + q;
                 const f32x4 a = patch16[row * CR + (chunk ^ (row & 7))];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int64_t n = n0 + 4 * q + e;
-                    const float cv = p.C ? Out::load(p.C, m * p.ldc_m + n * p.ldc_n) : 0.f;
-                    out[4 * q + e] = Out::cvt(epi_value(p, a[e], p.C != nullptr, cv, m, n));
+                for (int e = 0; e < 4; ++e) v[4 * q + e] = __fmul_rn(a[e], p.alpha);
+            }
+            // beta * C: a 16-byte piece of the row where C allows it (kGemmRowC), element by element otherwise
+            if (p.C) {
+                if (p.xcd_swizzle & kGemmRowC) {
+                    OutT cw[EPC];
+                    const u32x4 w = *reinterpret_cast<const u32x4*>(static_cast<const char*>(p.C) + (m * p.ldc_m + n0) * (int64_t)sizeof(OutT));
+                    __builtin_memcpy(cw, &w, 16);
+#pragma unroll
+                    for (int e = 0; e < EPC; ++e) v[e] = __fadd_rn(v[e], __fmul_rn(p.beta, Out::load(cw, e)));
+                } else {
+#pragma unroll
+                    for (int e = 0; e < EPC; ++e) v[e] = __fadd_rn(v[e], __fmul_rn(p.beta, Out::load(p.C, m * p.ldc_m + (n0 + e) * p.ldc_n)));
                 }
+            }
+            // the operand: a scalar, one value per row, a 16-byte piece (or two) of a row, or element by element
+            if (!p.ep_x) {
+#pragma unroll
+                for (int e = 0; e < EPC; ++e) x[e] = p.ep_scalar;
+            } else if (p.ep_xn == 0) {
+                const float xr = epi_operand(p, m, 0);
+#pragma unroll
+                for (int e = 0; e < EPC; ++e) x[e] = xr;
+            } else if (p.xcd_swizzle & kGemmEpiRowX) {
+                if (p.ep_xdt == MOYE_F32) {
+                    const f32x4* xp = reinterpret_cast<const f32x4*>(static_cast<const float*>(p.ep_x) + m * p.ep_xm + n0);
+#pragma unroll
+                    for (int q = 0; q < EPC / 4; ++q) {
+                        const f32x4 w = xp[q];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) x[4 * q + e] = w[e];
+                    }
+                } else {  // D's 16-bit type
+                    OutT xw[EPC];
+                    const u32x4 w = *reinterpret_cast<const u32x4*>(static_cast<const char*>(p.ep_x) + (m * p.ep_xm + n0) * (int64_t)sizeof(OutT));
+                    __builtin_memcpy(xw, &w, 16);
+#pragma unroll
+                    for (int e = 0; e < EPC; ++e) x[e] = Out::load(xw, e);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < EPC; ++e) x[e] = epi_operand(p, m, n0 + e);
+            }
+            OutT out[EPC];
+            switch (p.ep_op) {  // the operation is the same for every element: one branch per piece, not per element
+#define MOYE_EPI_CASE(OP)                                                                              \
+    case OP:                                                                                           \
+        _Pragma("unroll") for (int e = 0; e < EPC; ++e) out[e] = Out::cvt(epi_op(OP, v[e], x[e]));     \
+        break;
+                MOYE_EPI_CASE(MOYE_MAP_ADD)
+                MOYE_EPI_CASE(MOYE_MAP_SUB)
+                MOYE_EPI_CASE(MOYE_MAP_MUL)
+                MOYE_EPI_CASE(MOYE_MAP_DIV)
+                MOYE_EPI_CASE(MOYE_MAP_MAX)
+                MOYE_EPI_CASE(MOYE_MAP_MIN)
+                MOYE_EPI_CASE(MOYE_MAP_NEG)
+                MOYE_EPI_CASE(MOYE_MAP_ABS)
+#undef MOYE_EPI_CASE
+                default:
+#pragma unroll
+                    for (int e = 0; e < EPC; ++e) out[e] = Out::cvt(v[e]);
             }
             u32x4 w;
             __builtin_memcpy(&w, out, 16);

@@ -137,9 +137,13 @@ static size_t kmajor_bytes(const Mat& m) {
 static int split_count(const moye_tiled_mma* mma, int64_t M, int64_t N, int64_t K, int eb) {
     if (mma->split_k >= 0) return mma->split_k > 1 ? mma->split_k : 1;
     if (mma->flags & MOYE_GEMM_NO_WORKSPACE) return 1;  // nowhere to put the partial products
-    if (M <= 64 && mma->cta_tile_mnk[0] == 0 && mma->cta_tile_mnk[1] == 0 && (K * eb) % 64 == 0)
-        // the short-M kernel: two K ranges let a workgroup take 64 rows of B (see gemm_mfma_skinny.hip), nothing to gain below
+    if (M <= 64 && mma->cta_tile_mnk[0] == 0 && mma->cta_tile_mnk[1] == 0 && (K * eb) % 64 == 0) {
+        // the short-M kernels (gemm_mfma_skinny.hip).  The one that stages lines through LDS is fastest unsplit (bf16
+        // 64 x 8192 x 8192: 30.4 us against 41.3 with two ranges and the second pass); the one that loads into registers
+        // gains from two K ranges, which let a workgroup take 64 rows of B, from M = 33 on
+        if ((K * eb) % kSkinnyLineBytes == 0) return 1;
         return M > 32 && N % 64 == 0 && N / 64 >= 128 && (K * eb) % 256 == 0 ? 2 : 1;
+    }
     const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
     if (tiles <= 0 || tiles >= 128) return 1;
     for (int64_t s = std::min<int64_t>(256 / tiles, K); s >= 2; --s)

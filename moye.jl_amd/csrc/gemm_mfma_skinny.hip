@@ -1,14 +1,15 @@
 // MFMA GEMM for a short A: at most 64 rows against a long B (N x K), K-major operands.
-// The work is streaming B from HBM once, so the kernel is laid out for bandwidth, not for the
-// matrix pipe: one workgroup owns 16 or 32 rows of B (that many output columns) and all of A; its waves split
-// K into contiguous ranges, each lane streams 16-byte pieces of its B row straight into the MFMA
-// operand registers (no LDS staging: nothing is reused inside a workgroup), and the per-wave
-// partial accumulators are summed through LDS in wave order, which makes the result independent
-// of timing.  A (at most 64 x K) is re-read by every workgroup and lives in L2; with 32 rows of B
-// per workgroup each A fragment feeds two MFMAs, which halves that L2 traffic (measured 33 us
-// against 38 us at 16 x 8192 x 8192 bf16; the bare B stream alone takes 22 us).  More requests in flight make it
-// slower, not faster (same case, waves per workgroup x k-steps in flight per wave: 8 x 4 32.4 us, 4 x 8 34.3, 8 x 8 38.8,
-// 16 x 2 39.9, 16 x 4 41.5, 8 x 16 55.1): the kernel is not short of memory-level parallelism.
+// The work is streaming B from HBM once, so both kernels here are laid out for bandwidth, not for the matrix pipe: one
+// workgroup owns 16 or 32 rows of B (that many output columns) and all of A; its waves split K into contiguous ranges,
+// and the per-wave partial accumulators are summed through LDS in wave order, which makes the result independent of
+// timing.  A (at most 64 x K) is re-read by every workgroup and lives in L2.
+//   gemm_mfma_skinny_lds  K a multiple of 512 bytes: whole 128-byte lines of both operands go through LDS (load-to-LDS
+//                         instructions), four waves per workgroup; bf16 16 x 8192 x 8192: 21.0 us
+//   gemm_mfma_skinny      any K of whole 64-byte steps: each lane loads 16-byte pieces of its B row straight into the
+//                         MFMA operand registers, eight waves; the same problem: 32.4 us.  With 32 rows of B per
+//                         workgroup each A fragment feeds two MFMAs (33 us against 38).  More requests in flight make
+//                         it slower, not faster (waves per workgroup x k-steps in flight per wave: 8 x 4 32.4 us,
+//                         4 x 8 34.3, 8 x 8 38.8, 16 x 2 39.9, 16 x 4 41.5, 8 x 16 55.1).
 //
 // Stands where the reference's user kernel would run gemm! (src/algorithm/blas.jl:11-131) on a
 // 16-row problem with its usual 128 x 128 tiles and waste 7/8 of each tile.
@@ -108,9 +109,177 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_skinny(GemmArgs p) {
     }
 }
 
+// The same decomposition for at most 16 rows of A, with both operands staged through LDS by load-to-LDS instructions.
+// A lane that loads straight into MFMA operand registers must address row lane % 16: neighbouring lanes then ask for
+// 16 bytes each of sixteen different cache lines, and the address path of the CU handles such an instruction several
+// times slower than one whose lanes read consecutive addresses (measured on the kernel above with the lanes renumbered,
+// results wrong on purpose, same bytes: 32.4 us as it is, 30.2 with four lanes per 64 bytes, 29.0 with eight lanes per
+// 128-byte line).  Here every instruction reads eight whole 128-byte lines (eight rows of one operand, lane l the piece
+// (l % 8) ^ (l / 8) of row l / 8), the pieces land in LDS in lane order, which is the XOR-swizzled row layout that
+// ds_read_b128 reads back without bank conflicts, and no operand in flight holds a register.  Each wave streams its own
+// K range through its own ring of kStages buffers of 128 bytes of K, so the k-loop has no barrier.
+template <typename In, typename Out, int MT, int NTW, int WAVES, int kStages, int kAuxB = 2 /* nt: B is read once */>
+__global__ __launch_bounds__(WAVES * 64) void gemm_mfma_skinny_lds(GemmArgs p) {
+    typedef typename Out::type OutT;
+    typedef __attribute__((address_space(1))) const void* gptr_t;
+    typedef __attribute__((address_space(3))) void* lptr_t;
+    constexpr int ROWS = 16 * NTW + 16 * MT;  // rows of B, then the rows of A
+    constexpr int LD = ROWS / 8;              // load-to-LDS instructions per stage
+    constexpr int STAGE = ROWS * 8;           // in 16-byte pieces
+    static_assert(LD * kStages <= 63, "vmcnt counts to 63");
+    static_assert(MT * NTW * 64 <= kStages * STAGE, "the partial sums fit where the rings were");
+    extern __shared__ u32x4 smem[];
+    split_of_block(p);
+    const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, r16 = lane % 16, kq = lane / 16;
+    const int n0 = blockIdx.x * 16 * NTW;
+    u32x4* const ring = smem + __builtin_amdgcn_readfirstlane(wave * kStages * STAGE);
+
+    const int lines = (int)(((int64_t)p.K * In::kBytes) / 128);  // a multiple of WAVES (checked by the host)
+    const int len = lines / WAVES, s0 = wave * len;
+    // M and N need not be multiples of 16: a row beyond the operand is read from the last row instead, and what is
+    // computed from it is not stored
+    const int lrow = lane >> 3, lch = (lane & 7) ^ (lane >> 3);
+    const char* src[LD];
+#pragma unroll
+    for (int j = 0; j < LD; ++j) {
+        const int r = 8 * j + lrow;
+        src[j] = j < 2 * NTW ? static_cast<const char*>(p.B) + (int64_t)min(n0 + r, p.N - 1) * p.ldb * In::kBytes + lch * 16
+                             : static_cast<const char*>(p.A) + (int64_t)min(r - 16 * NTW, p.M - 1) * p.lda * In::kBytes + lch * 16;
+    }
+    // fragment of k-step ks (64 bytes of K): piece 4 ks + kq of row r16 of each 16-row block
+    int slot[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) slot[ks] = r16 * 8 + ((4 * ks + kq) ^ (r16 & 7));
+
+    f32x4 acc[MT][NTW];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int t = 0; t < NTW; ++t) acc[i][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // Workgroups that walk K in the same order ask their L2 for the same lines of A at the same moment, before any of
+    // them has them: a workgroup starts its walk at a line that depends on its position within its L2's share of the
+    // grid.  The order of a column's k-sum follows the workgroup, not the time, so results stay reproducible.
+    const int first = (int)((blockIdx.x / 8) % (unsigned)len);
+    auto line_of = [&](int t) { const int r = t + first; return s0 + (r >= len ? r - len : r); };
+#define MOYE_STAGE_LOAD(T)                                                                                      \
+    {                                                                                                           \
+        const int64_t off_ = (int64_t)line_of(T) * 128;                                                         \
+        u32x4* const dst_ = ring + ((T) % kStages) * STAGE;                                                     \
+        _Pragma("unroll") for (int j = 0; j < 2 * NTW; ++j)                                                     \
+            __builtin_amdgcn_global_load_lds((gptr_t)(src[j] + off_), (lptr_t)(dst_ + 64 * j), 16, 0, kAuxB);   \
+        _Pragma("unroll") for (int j = 2 * NTW; j < LD; ++j)                                                    \
+            __builtin_amdgcn_global_load_lds((gptr_t)(src[j] + off_), (lptr_t)(dst_ + 64 * j), 16, 0, 0);       \
+    }
+#pragma unroll
+    for (int t = 0; t < kStages - 1; ++t)
+        if (t < len) MOYE_STAGE_LOAD(t)
+    for (int t = 0; t < len; ++t) {
+        if (t + kStages - 1 < len) {
+            __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the fragment reads of trip t - 1 are out of the buffer refilled now
+            MOYE_STAGE_LOAD(t + kStages - 1)
+            __builtin_amdgcn_s_waitcnt((((kStages - 1) * LD) & 0xF) | ((((kStages - 1) * LD) >> 4) << 14) | 0x0F70);
+        } else {
+            // the tail: fewer stages are behind this one; waiting for all of them costs little over so few trips
+            __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        }
+        asm volatile("" ::: "memory");
+        const u32x4* const cur = ring + (t % kStages) * STAGE;
+        u32x4 b[2][NTW], a[2][MT];
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+            for (int j = 0; j < NTW; ++j) b[ks][j] = cur[16 * 8 * j + slot[ks]];
+#pragma unroll
+            for (int i = 0; i < MT; ++i) a[ks][i] = cur[16 * 8 * (NTW + i) + slot[ks]];
+        }
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int j = 0; j < NTW; ++j) In::mma(b[ks][j], a[ks][i], acc[i][j]);
+        asm volatile("" ::: "memory");
+    }
+#undef MOYE_STAGE_LOAD
+
+    __syncthreads();  // every wave is done with its ring before the partial sums go there
+    f32x4* const part = reinterpret_cast<f32x4*>(smem);  // [WAVES][MT * NTW][64]
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int t = 0; t < NTW; ++t) part[(wave * MT * NTW + i * NTW + t) * 64 + lane] = acc[i][t];
+    __syncthreads();
+    // lane l of tile (i, t) holds C[m = 16 i + l % 16][n = n0 + 16 t + 4 (l / 16) + 0..3]
+    for (int unit = threadIdx.x; unit < MT * NTW * 64; unit += WAVES * 64) {
+        const int it = unit / 64, l = unit % 64;
+        f32x4 v = part[unit];
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) v += part[w * MT * NTW * 64 + unit];
+        const int m = 16 * (it / NTW) + l % 16, n = n0 + 16 * (it % NTW) + 4 * (l / 16);
+        if (m >= p.M) continue;
+        const int64_t sn = p.ldd_n ? p.ldd_n : 1;  // D may have its unit stride along m
+        OutT* d = static_cast<OutT*>(p.D) + (int64_t)m * p.ldd + (int64_t)n * sn;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if (n + e >= p.N) continue;
+            const float c = p.C ? Out::load(p.C, (int64_t)m * p.ldc_m + (int64_t)(n + e) * p.ldc_n) : 0.f;
+            d[e * sn] = Out::cvt(epi_value(p, v[e], p.C != nullptr, c, m, n + e));
+        }
+    }
+}
+
+constexpr int kSkinnyLdsWaves = 4;
+static_assert(kSkinnyLineBytes == 128 * kSkinnyLdsWaves, "the host decides about K ranges by this");
+
+// K a whole number of 128-byte lines per wave
+template <typename In>
+static bool skinny_lds_takes(const GemmArgs& a) {
+    return a.K > 0 && ((int64_t)a.K * In::kBytes) % (128 * kSkinnyLdsWaves) == 0;
+}
+
+template <typename In, typename Out, int MT, int W, int NTW, int S, int AUX>
+static int32_t launch_skinny_lds_v(const GemmArgs& a, hipStream_t st) {
+    constexpr int kLds = W * S * (16 * NTW + 16 * MT) * 128;
+    static LdsCap cap;
+    auto kern = gemm_mfma_skinny_lds<In, Out, MT, NTW, W, S, AUX>;
+    if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
+    const dim3 grid((unsigned)((a.N + 16 * NTW - 1) / (16 * NTW)), (unsigned)(a.split > 1 ? a.split : 1));
+    kern<<<grid, dim3(W * 64), kLds, st>>>(a);
+    MOYE_HIP_CHECK(hipGetLastError());
+    return MOYE_OK;
+}
+template <typename In, typename Out>
+static int32_t launch_skinny_lds(const GemmArgs& a, hipStream_t st) {
+    constexpr int W = kSkinnyLdsWaves;
+    // Waves x buffers, bf16 16 x 8192 x 8192, 32 rows of B per workgroup: 8 x 3 27.2 us, 8 x 2 25.2, 4 x 2 21.2, 4 x 3 21.0,
+    // 4 x 4 21.2, 2 x 4 21.0, 2 x 3 22.6, 1 x 8 30.0; 64 rows per workgroup (half as many workgroups as CUs) 28.0-30.1;
+    // B without the non-temporal hint 23.6.  As with the transposes, less in flight is faster on this part, down to what
+    // covers the latency.  32 rows per workgroup once that gives every CU one (bf16, K = 8192: N = 16384 40.1 us against
+    // 45.3 with 16 rows; N = 4096 17.9 against 13.5).
+    const bool wide = (a.N + 31) / 32 >= 256;
+    if (wide) {
+        switch ((a.M + 15) / 16) {
+            case 1: return launch_skinny_lds_v<In, Out, 1, W, 2, 3, 2>(a, st);
+            case 2: return launch_skinny_lds_v<In, Out, 2, W, 2, 3, 2>(a, st);
+            case 3: return launch_skinny_lds_v<In, Out, 3, W, 2, 3, 2>(a, st);
+            default: return launch_skinny_lds_v<In, Out, 4, W, 2, 3, 2>(a, st);
+        }
+    }
+    switch ((a.M + 15) / 16) {
+        case 1: return launch_skinny_lds_v<In, Out, 1, W, 1, 3, 2>(a, st);
+        case 2: return launch_skinny_lds_v<In, Out, 2, W, 1, 3, 2>(a, st);
+        case 3: return launch_skinny_lds_v<In, Out, 3, W, 1, 3, 2>(a, st);
+        default: return launch_skinny_lds_v<In, Out, 4, W, 1, 3, 2>(a, st);
+    }
+}
+
 template <typename In, typename Out>
 static int32_t launch_skinny(const GemmArgs& a, hipStream_t st) {
     constexpr int W = 8;
+    // MOYE_SKINNY_LDS=0 keeps calls on the kernel above (to measure one against the other)
+    static const bool lds_off = getenv("MOYE_SKINNY_LDS") && atoi(getenv("MOYE_SKINNY_LDS")) == 0;
+    if (!lds_off && skinny_lds_takes<In>(a)) return launch_skinny_lds<In, Out>(a, st);
     const dim3 block(W * 64);
     // With K split over two or more workgroups there are enough workgroups to give each one 64 rows of B: A, which every
     // workgroup reads whole (its K range of it), then crosses the L2-to-CU path half as often.  Pays from M = 33 on

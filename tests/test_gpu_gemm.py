@@ -559,6 +559,50 @@ def test_short_m_any_m_and_n(mh, M):
         assert torch.equal(dt_.t().cpu().double(), ref), (M, N, K, "column-major D")
 
 
+@pytest.mark.parametrize("M", [1, 16, 17, 48, 64])
+def test_short_m_line_staging_kernel(mh, M):
+    """K of whole 512-byte units runs on the kernel that stages 128-byte lines through LDS: any M <= 64 and any N (16 and
+    32 rows of B per workgroup), one K line per wave and many, row- and column-major D inside a frame, C with alpha,
+    every input type; exact on small integers, so a wrong piece, row or K range is a hard mismatch."""
+    g = torch.Generator().manual_seed(300 + M)
+    for (N, K) in ((100, 256), (8191, 768), (8200, 2048), (12000, 256), (32, 4096)):
+        A = torch.randint(-4, 5, (M, K), generator=g).to(torch.float16)
+        B = torch.randint(-4, 5, (N, K), generator=g).to(torch.float16)
+        C = torch.randint(-8, 9, (M, N), generator=g).to(torch.float32)
+        a, b, c = A.cuda(), B.cuda(), C.cuda()
+        ref = A.double() @ B.double().t()
+        big = torch.full((M + 2, N + 3), 77.0, device="cuda")
+        d = big[1:M + 1, 2:N + 2]
+        mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(0, 0, 0)), T(d), T(a), T(b), T(c), 2.0)
+        torch.cuda.synchronize()
+        assert torch.equal(d.cpu().double(), 2.0 * ref + C.double()), (M, N, K)
+        frame = big.clone()
+        frame[1:M + 1, 2:N + 2] = 77.0
+        assert bool((frame == 77.0).all()), "stores outside D"
+        dt_ = torch.zeros(N, M, device="cuda")
+        mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(0, 0, 0)), T(dt_, (M, N), (1, M)), T(a), T(b))
+        torch.cuda.synchronize()
+        assert torch.equal(dt_.t().cpu().double(), ref), (M, N, K, "column-major D")
+        d2 = torch.zeros(M, N, dtype=torch.float32, device="cuda")     # two K ranges on request: each a multiple of 512 bytes or not
+        mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(0, 0, 0), split_k=2), T(d2), T(a), T(b), T(c), 2.0)
+        torch.cuda.synchronize()
+        assert torch.equal(d2.cpu().double(), 2.0 * ref + C.double()), (M, N, K, "split_k 2")
+    N, K = 8192, 1024
+    A = torch.randint(-3, 4, (M, K), generator=g).float()
+    B = torch.randint(-3, 4, (N, K), generator=g).float()
+    ref = A.double() @ B.double().t()
+    cases = [(torch.bfloat16, mh.MFMA_F32_16x16x32_BF16, torch.bfloat16), (torch.float32, mh.MFMA_F32_16x16x4_F32, torch.float32)]
+    if hasattr(torch, "float8_e4m3fn"):
+        cases.append((torch.float8_e4m3fn, mh.MFMA_F32_16x16x32_FP8, torch.float16))
+    for in_dt, atom, out_dt in cases:
+        a, b = A.to(in_dt).cuda(), B.to(in_dt).cuda()
+        d = torch.zeros(M, N, dtype=out_dt, device="cuda")
+        mh.gemm_(mh.tiled_mma_desc(atom, cta_tile=(0, 0, 0)), T(d), T(a), T(b), None, 1.0 / 64)
+        torch.cuda.synchronize()
+        want = (ref / 64).to(torch.float32).to(out_dt)
+        assert torch.equal(d.cpu(), want), (in_dt, out_dt)
+
+
 def test_short_m_other_types(mh):
     g = torch.Generator().manual_seed(77)
     M, N, K = 16, 512, 1024

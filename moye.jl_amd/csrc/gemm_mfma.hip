@@ -337,6 +337,19 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         const int M0 = a.M / 256 * 256, N0 = a.N / 256 * 256, ob0 = dtype_bytes(out_dt);
         const bool aligned = !((a.lda * eb) % 16 || (a.ldb * eb) % 16 || (a.ldd * ob0) % 16 ||
                                (reinterpret_cast<uintptr_t>(a.A) | reinterpret_cast<uintptr_t>(a.B) | reinterpret_cast<uintptr_t>(a.D)) % 16);
+        // Ragged tiles on the 256 x 256 kernel itself (its guarded instance: rows clamped, the K tail masked, stores
+        // guarded) when that fills the chip, unless the fringes are thin enough for the short-M kernel, which then costs
+        // less than a further round of tiles (fp16 4000 x 4096 x 4096: 170 us as interior + fringe on 128 x 128 tiles,
+        // vendor library 96).  Not fp8: its fast kernel is the hand-ordered one, which has no guarded form.
+        const int fr_m = a.M - M0, fr_n = a.N - N0;
+        const bool thin = fr_m <= 64 && fr_n <= 64 && a.K % (128 / eb) == 0;
+        const int64_t rtiles = (int64_t)((a.M + 255) / 256) * ((a.N + 255) / 256);
+        if (!big && !thin && a.split <= 1 && bk_elems == 0 && aligned && in_dt != MOYE_F8E4M3 && ((int64_t)a.K * eb) % 16 == 0 &&
+            rtiles >= 128 && stages < 3 && (waves <= 1 || waves == 8) &&
+            !(a.xcd_swizzle & (MOYE_GEMM_WAVE4 | MOYE_GEMM_PINGPONG | kGemmAMajorM | kGemmBMajorN | kGemmAtom32))) {
+            a.xcd_swizzle |= kGemmRagged;
+            return gemm_mfma_tn_256_dispatch(in_dt, out_dt, a, 8, stages, st);
+        }
         if (!big && a.split <= 1 && bk_elems == 0 && aligned && a.K % (128 / eb) == 0 && (int64_t)(M0 / 256) * (N0 / 256) >= 128) {
             GemmArgs part = a;
             part.M = M0; part.N = N0;

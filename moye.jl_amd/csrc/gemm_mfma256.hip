@@ -39,8 +39,15 @@ namespace moye {
 // read), m = m0 + 4 (s % 4), two reads give lane l the eight k of row m0 + l % 16 that the K-major ds_read_b128 would.
 // The 32-byte piece index of a k-row is XORed with (row % 4) | 4 ((row / 8) % 2): the eight row pieces the 32 lanes of
 // one pass read then lie in eight different bank groups.
-template <typename In, typename Out, int WGM, int WGN, bool kOps = false, int AMAJ = 0, int BMAJ = 0>
+//
+// kRagged: M and N need not be multiples of 256 and K not of the k-tile (the intent of copyto_if!,
+// src/algorithm/copy.jl:4-16, for whole tiles).  A row beyond the operand is read from the operand's last row instead and
+// what is computed from it is never stored; in the last k-tile a lane whose 16-byte piece lies beyond K reads the
+// row's first piece instead and every fragment piece beyond K is zeroed in registers before it reaches an MFMA; the
+// epilogue is the general one with its row and column guards.
+template <typename In, typename Out, int WGM, int WGN, bool kOps = false, int AMAJ = 0, int BMAJ = 0, bool kRagged = false>
 __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
+    static_assert(!kRagged || (kOps && !AMAJ && !BMAJ), "ragged tiles: K-major operands, the general epilogue");
     constexpr int BM = 256, BN = 256, CPR = 8;  // 8 chunks of 16 bytes per tile row
     constexpr int A_CH = BM * CPR, B_CH = BN * CPR, STAGE = A_CH + B_CH;
     constexpr int NWAVES = WGM * WGN;
@@ -61,8 +68,13 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
     // load-to-LDS: wave w fills rows WROWS w + 8 i + l/8 (i < LD) of each operand tile; lane l brings
     // the chunk that belongs in physical slot l % 8 of its row
     const int lrow = wave * WROWS + (lane >> 3), lch = (lane & 7) ^ (lane >> 3);
-    const char* gA = static_cast<const char*>(p.A) + ((int64_t)tm * BM + lrow) * pitch_a + lch * 16;
-    const char* gB = static_cast<const char*>(p.B) + ((int64_t)tn * BN + lrow) * pitch_b + lch * 16;
+    const int row_a0 = tm * BM + lrow, row_b0 = tn * BN + lrow;
+    const char* gA = static_cast<const char*>(p.A) + (int64_t)(kRagged ? min(row_a0, p.M - 1) : row_a0) * pitch_a + lch * 16;
+    const char* gB = static_cast<const char*>(p.B) + (int64_t)(kRagged ? min(row_b0, p.N - 1) : row_b0) * pitch_b + lch * 16;
+    // ragged tiles: how many rows below its first one this lane may go, and what to add to its address in the last k-tile
+    [[maybe_unused]] const int more_a = max(p.M - 1 - row_a0, 0), more_b = max(p.N - 1 - row_b0, 0);
+    [[maybe_unused]] const int k_rem = (int)((((int64_t)p.K * In::kBytes) % 128) / 16), k_valid = k_rem ? k_rem : 8;
+    [[maybe_unused]] const int tail_delta = lch < k_valid ? 0 : -lch * 16;
     const int dma_slot = __builtin_amdgcn_readfirstlane(wave * WROWS * CPR);  // + 8 rows * CPR per i
     // An M-major (N-major) operand: wave w fills k-rows KROWS w + 2 i + l / 32 of the tile, two rows (1 KiB) per
     // instruction; lane l brings the 16-byte chunk that belongs in physical slot l % 32 of its row.
@@ -107,7 +119,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
 #pragma unroll
         for (int j = 0; j < NI; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    const int ktiles = (int)(((int64_t)p.K * In::kBytes) / 128);
+    const int ktiles = (int)(((int64_t)p.K * In::kBytes + (kRagged ? 127 : 0)) / 128);
     u32x4 fa[2][MI], fb[2][NI];
     typedef short v4s __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) v4s* tr_ptr_t;
@@ -130,15 +142,27 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
         if constexpr (AMAJ)                                                                           \
             __builtin_amdgcn_global_load_lds((gptr_t)(static_cast<const char*>(p.A) + tA[i] + (int64_t)(KT) * 64 * pitch_a), \
                                              (lptr_t)((BASE) + dma_slot_t + 64 * i), 16, 0, 0);       \
+        else if constexpr (kRagged)                                                                   \
+            __builtin_amdgcn_global_load_lds((gptr_t)(gA + (int64_t)min(8 * i, more_a) * pitch_a + (int64_t)(KT) * 128 + ((KT) == ktiles - 1 ? tail_delta : 0)), \
+                                             (lptr_t)((BASE) + dma_slot + 8 * CPR * i), 16, 0, 0);    \
         else                                                                                          \
             __builtin_amdgcn_global_load_lds((gptr_t)(gA + (int64_t)(8 * i) * pitch_a + (int64_t)(KT) * 128), \
                                              (lptr_t)((BASE) + dma_slot + 8 * CPR * i), 16, 0, 0);    \
         if constexpr (BMAJ)                                                                           \
             __builtin_amdgcn_global_load_lds((gptr_t)(static_cast<const char*>(p.B) + tB[i] + (int64_t)(KT) * 64 * pitch_b), \
                                              (lptr_t)((BASE) + A_CH + dma_slot_t + 64 * i), 16, 0, 0); \
+        else if constexpr (kRagged)                                                                   \
+            __builtin_amdgcn_global_load_lds((gptr_t)(gB + (int64_t)min(8 * i, more_b) * pitch_b + (int64_t)(KT) * 128 + ((KT) == ktiles - 1 ? tail_delta : 0)), \
+                                             (lptr_t)((BASE) + A_CH + dma_slot + 8 * CPR * i), 16, 0, 0); \
         else                                                                                          \
             __builtin_amdgcn_global_load_lds((gptr_t)(gB + (int64_t)(8 * i) * pitch_b + (int64_t)(KT) * 128), \
                                              (lptr_t)((BASE) + A_CH + dma_slot + 8 * CPR * i), 16, 0, 0); \
+    }
+    // ragged K: the fragments of k-step KS of the last k-tile, in buffer BUF, keep only the pieces inside K
+#define MOYE_MASK_TAIL(KS, BUF)                                                                       \
+    if (kRagged && 4 * (KS) + kq >= k_valid) {                                                        \
+        _Pragma("unroll") for (int i = 0; i < MI; ++i) fa[BUF][i] = u32x4{0u, 0u, 0u, 0u};            \
+        _Pragma("unroll") for (int j = 0; j < NI; ++j) fb[BUF][j] = u32x4{0u, 0u, 0u, 0u};            \
     }
     // Wait until at most N of this wave's load-to-LDS instructions are in flight and its own LDS reads
     // have returned, then meet the other waves.  A bare s_barrier on purpose: __syncthreads() adds a
@@ -196,7 +220,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
     // apart, so that at any moment the chip asks memory for eight different column blocks of A and B instead of one
     // (with K-major operands and a power-of-two pitch one column block lives in few channels).  k_of() hands out the
     // indices of successive k-tiles in that rotated order; the sum over k starts elsewhere but is the same sum.
-    int k_next = (p.xcd_swizzle & kGemmRotateK) ? (int)((int64_t)(blockIdx.x % 8) * ktiles / 8) : 0;
+    int k_next = (!kRagged && (p.xcd_swizzle & kGemmRotateK)) ? (int)((int64_t)(blockIdx.x % 8) * ktiles / 8) : 0;  // (ragged: the last k-tile in time is the last in K)
     auto k_of = [&]() {
         const int kt_now = k_next;
         k_next = k_next + 1 == ktiles ? 0 : k_next + 1;
@@ -211,10 +235,11 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
         MOYE_WAIT_BARRIER(0)
     }
     MOYE_FRAGS(smem, 0, 0)
+    if (ktiles == 1) { MOYE_MASK_TAIL(0, 0) }
 
     // One k-tile.  DMA: tile KT+2 exists and is fetched; NEXT: tile KT+1 exists and its first fragments
     // are read.  The steady-state body has no branches, so each k-step is one scheduling region.
-#define MOYE_TILE(KT, DMA, NEXT)                                                                      \
+#define MOYE_TILE(KT, DMA, NEXT, TAIL)                                                                \
     {                                                                                                 \
         u32x4* const cur = smem + ((KT) & 1) * STAGE;                                                 \
         u32x4* const nxt = smem + (((KT) + 1) & 1) * STAGE;                                           \
@@ -224,6 +249,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
         MOYE_WAIT_LDS();                                                                              \
         __builtin_amdgcn_sched_barrier(0);                                                            \
         MOYE_FRAGS(cur, 1, 1)                                                                         \
+        if ((TAIL) == 2) { MOYE_MASK_TAIL(1, 1) }                                                     \
         MOYE_MMA(0, 0, MI)                                                                            \
         MOYE_INTERLEAVE(0)                                                                            \
         __builtin_amdgcn_sched_barrier(0);                                                            \
@@ -234,18 +260,20 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
            MFMAs on buffer 1 (already in registers) while step 0 of tile KT+1 arrives in buffer 0 */  \
         if (DMA) { const int ko = k_of(); MOYE_DMA(cur, ko) }                                     \
         if (NEXT) MOYE_FRAGS(nxt, 0, 0)                                                               \
+        if ((TAIL) == 1) { MOYE_MASK_TAIL(0, 0) }                                                     \
         MOYE_MMA(1, 0, MI)                                                                            \
         if (NEXT) { MOYE_INTERLEAVE((DMA) ? 2 * LD : 0) }                                             \
         __builtin_amdgcn_sched_barrier(0);                                                            \
     }
     int kt = 0;
-    for (; kt + 2 < ktiles; ++kt) MOYE_TILE(kt, true, true)
+    for (; kt + 2 < ktiles; ++kt) MOYE_TILE(kt, true, true, 0)
     if (kt + 1 < ktiles) {
-        MOYE_TILE(kt, false, true)
+        MOYE_TILE(kt, false, true, 1)
         ++kt;
     }
-    MOYE_TILE(kt, false, false)
+    MOYE_TILE(kt, false, false, 2)
 #undef MOYE_TILE
+#undef MOYE_MASK_TAIL
 #undef MOYE_INTERLEAVE
 #undef MOYE_DMA
 #undef MOYE_WAIT_BARRIER
@@ -256,7 +284,8 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
 
     // --- epilogue (mfma_epilogue.hpp): alpha*acc + C -> OutT -> this wave's LDS patch -> 128-bit row stores
     static_assert(NWAVES * 32 * WN * 4 <= 2 * STAGE * 16, "C patches (32 rows per wave and pass) fit in the operand stages");
-    store_c_tile<Out, MI, NI, kOps>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
+    if constexpr (kRagged) store_c_tile_general<Out, MI, NI, true>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
+    else store_c_tile<Out, MI, NI, kOps>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -386,10 +415,10 @@ static int32_t launch256_ring(const GemmArgs& a, hipStream_t st) {
     return MOYE_OK;
 }
 
-template <typename In, typename Out, int WGM, int WGN, bool kOps, int AMAJ, int BMAJ>
+template <typename In, typename Out, int WGM, int WGN, bool kOps, int AMAJ, int BMAJ, bool kRagged = false>
 static int32_t launch256_instance(const GemmArgs& a, hipStream_t st) {
     constexpr int kLds = 2 * (256 + 256) * 128;  // two operand stages, 128 KiB
-    auto kern = gemm_mfma_tn_256<In, Out, WGM, WGN, kOps, AMAJ, BMAJ>;
+    auto kern = gemm_mfma_tn_256<In, Out, WGM, WGN, kOps, AMAJ, BMAJ, kRagged>;
     static LdsCap cap;
     if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
     kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1)), dim3(64 * WGM * WGN), kLds, st>>>(a);
@@ -400,6 +429,14 @@ static int32_t launch256_instance(const GemmArgs& a, hipStream_t st) {
 template <typename In, typename Out, int WGM, int WGN>
 static int32_t launch256(const GemmArgs& a, hipStream_t st) {
     const bool am = a.xcd_swizzle & kGemmAMajorM, bm = a.xcd_swizzle & kGemmBMajorN;
+    if (a.xcd_swizzle & kGemmRagged) {
+        if constexpr (WGM * WGN == 8 && !std::is_same<In, InFP8>::value) {
+            if (am || bm) return fail(MOYE_ERR_UNSUPPORTED, "gemm!: ragged 256 x 256 tiles take K-major operands");
+            return launch256_instance<In, Out, WGM, WGN, true, 0, 0, true>(a, st);
+        } else {
+            return fail(MOYE_ERR_UNSUPPORTED, "gemm!: ragged 256 x 256 tiles run on eight waves with f16, bf16 or f32 operands");
+        }
+    }
     if (am || bm) {
         // operands that are not K-major: eight waves, 16-bit types (the host checked)
         if constexpr (WGM * WGN == 8 && In::kBytes == 2) {
@@ -446,8 +483,8 @@ static int32_t launch256_out(int32_t out_dt, const GemmArgs& a, int waves, int s
 
 // 256 x 256 x (128 bytes of K) tile; the caller has checked divisibility and alignment.
 int32_t gemm_mfma_tn_256_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, int waves, int stages, hipStream_t st) {
-    a.tiles_m = a.M / 256;
-    a.tiles_n = a.N / 256;
+    a.tiles_m = (a.M + 255) / 256;  // (whole tiles unless kGemmRagged)
+    a.tiles_n = (a.N + 255) / 256;
     switch (in_dt) {
         case MOYE_F16: return launch256_out<InF16>(out_dt, a, waves, stages, st);
         case MOYE_BF16: return launch256_out<InBF16>(out_dt, a, waves, stages, st);

@@ -35,6 +35,7 @@ constexpr int kGemmStreamD = 0x40000;  // in GemmArgs::xcd_swizzle: D is written
 constexpr int kGemmAMajorM = 0x100000;  // in GemmArgs::xcd_swizzle: A has its unit stride along M, lda is the pitch between consecutive k
 constexpr int kGemmBMajorN = 0x200000;  // the same for B and N (the 256 x 256 kernel's transposing fragment reads; 16-bit types)
 constexpr int kGemmEpiRowX = 0x400000;  // in GemmArgs::xcd_swizzle: the epilogue operand has unit stride along n and 16-byte aligned rows (or one row)
+constexpr int kGemmRagged = 0x800000;   // in GemmArgs::xcd_swizzle: the 256 x 256 kernel runs with tiles that reach beyond M, N or K (its guarded instance)
 constexpr int kGemmRotateK = 0x20000;  // in GemmArgs::xcd_swizzle: each XCD starts its walk over K at its own eighth
 
 // UniversalFMA GEMM, any strides (gemm_universal.hip)

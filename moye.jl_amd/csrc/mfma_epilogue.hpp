@@ -13,7 +13,9 @@ namespace moye {
 // epi_value() (alpha, beta * C, the operation with its operand), convert and store 16-byte pieces.  The arithmetic
 // exists once, in a loop over the passes that is not unrolled: unrolled over all accumulators it would be several
 // thousand instructions per kernel.  `smem`: 32 x WN floats per wave.
-template <typename Out, int MI, int NI>
+// kGuard: the tile may reach beyond M or N; rows beyond M are skipped, a piece that crosses N is read and stored element
+// by element up to N (rows of D start on 16-byte boundaries, so every piece inside N still goes out whole).
+template <typename Out, int MI, int NI, bool kGuard = false>
 __device__ __forceinline__ void store_c_tile_general(const GemmArgs& p, const f32x4 (&acc)[MI][NI], u32x4* smem, int wave,
                                                      int lane, int64_t m_base, int64_t n_base) {
     typedef typename Out::type OutT;
@@ -46,6 +48,8 @@ __device__ __forceinline__ void store_c_tile_general(const GemmArgs& p, const f3
         for (int t = 0; t < OUT_CH / 64; ++t) {
             const int c = lane + 64 * t, row = c / (WN / EPC), och = c % (WN / EPC);
             const int64_t m = m_base + PASS_ROWS * pass + row, n0 = n_base + och * EPC;
+            if (kGuard && (m >= p.M || n0 >= p.N)) continue;
+            const bool whole = !kGuard || n0 + EPC <= p.N;  // else only the first N - n0 elements exist
             float v[EPC], x[EPC];
 #pragma unroll
             for (int q = 0; q < EPC / 4; ++q) {
@@ -56,7 +60,7 @@ __device__ __forceinline__ void store_c_tile_general(const GemmArgs& p, const f3
             }
             // beta * C: a 16-byte piece of the row where C allows it (kGemmRowC), element by element otherwise
             if (p.C) {
-                if (p.xcd_swizzle & kGemmRowC) {
+                if ((p.xcd_swizzle & kGemmRowC) && whole) {
                     OutT cw[EPC];
                     const u32x4 w = *reinterpret_cast<const u32x4*>(static_cast<const char*>(p.C) + (m * p.ldc_m + n0) * (int64_t)sizeof(OutT));
                     __builtin_memcpy(cw, &w, 16);
@@ -64,7 +68,8 @@ __device__ __forceinline__ void store_c_tile_general(const GemmArgs& p, const f3
                     for (int e = 0; e < EPC; ++e) v[e] = __fadd_rn(v[e], __fmul_rn(p.beta, Out::load(cw, e)));
                 } else {
 #pragma unroll
-                    for (int e = 0; e < EPC; ++e) v[e] = __fadd_rn(v[e], __fmul_rn(p.beta, Out::load(p.C, m * p.ldc_m + (n0 + e) * p.ldc_n)));
+                    for (int e = 0; e < EPC; ++e)
+                        if (whole || n0 + e < p.N) v[e] = __fadd_rn(v[e], __fmul_rn(p.beta, Out::load(p.C, m * p.ldc_m + (n0 + e) * p.ldc_n)));
                 }
             }
             // the operand: a scalar, one value per row, a 16-byte piece (or two) of a row, or element by element
@@ -75,7 +80,7 @@ __device__ __forceinline__ void store_c_tile_general(const GemmArgs& p, const f3
                 const float xr = epi_operand(p, m, 0);
 #pragma unroll
                 for (int e = 0; e < EPC; ++e) x[e] = xr;
-            } else if (p.xcd_swizzle & kGemmEpiRowX) {
+            } else if ((p.xcd_swizzle & kGemmEpiRowX) && whole) {
                 if (p.ep_xdt == MOYE_F32) {
                     const f32x4* xp = reinterpret_cast<const f32x4*>(static_cast<const float*>(p.ep_x) + m * p.ep_xm + n0);
 #pragma unroll
@@ -93,7 +98,7 @@ __device__ __forceinline__ void store_c_tile_general(const GemmArgs& p, const f3
                 }
             } else {
 #pragma unroll
-                for (int e = 0; e < EPC; ++e) x[e] = epi_operand(p, m, n0 + e);
+                for (int e = 0; e < EPC; ++e) x[e] = whole || n0 + e < p.N ? epi_operand(p, m, n0 + e) : 0.f;
             }
             OutT out[EPC];
             switch (p.ep_op) {  // the operation is the same for every element: one branch per piece, not per element
@@ -114,9 +119,16 @@ __device__ __forceinline__ void store_c_tile_general(const GemmArgs& p, const f3
 #pragma unroll
                     for (int e = 0; e < EPC; ++e) out[e] = Out::cvt(v[e]);
             }
-            u32x4 w;
-            __builtin_memcpy(&w, out, 16);
-            store_d_chunk(p, static_cast<char*>(p.D) + (m * p.ldd + n0) * (int64_t)sizeof(OutT), w);
+            if (whole) {
+                u32x4 w;
+                __builtin_memcpy(&w, out, 16);
+                store_d_chunk(p, static_cast<char*>(p.D) + (m * p.ldd + n0) * (int64_t)sizeof(OutT), w);
+            } else {
+                OutT* d = static_cast<OutT*>(p.D) + m * p.ldd + n0;
+#pragma unroll
+                for (int e = 0; e < EPC; ++e)
+                    if (n0 + e < p.N) d[e] = out[e];
+            }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();

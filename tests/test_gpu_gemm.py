@@ -603,6 +603,50 @@ def test_short_m_line_staging_kernel(mh, M):
         assert torch.equal(d.cpu(), want), (in_dt, out_dt)
 
 
+@pytest.mark.parametrize("case", [(4000, 2200, 328), (3900, 2304, 120), (4096, 2048, 72), (4090, 2203, 40), (2100, 4100, 200),
+                                  (4099, 2050, 4096 + 8)])
+def test_ragged_256_tiles_exact_on_integers(mh, case):
+    """Problems the library puts on 256x256 tiles that reach beyond M, N and K: rows beyond the operands are read from
+    the last row and never stored, the K tail (1 to 7 pieces of 16 bytes, also with less than one k-tile in all) is
+    masked, pieces of D that cross N go out element by element.  D is a window of a larger buffer whose frame must stay
+    untouched; small integers make every sum exact."""
+    M, N, K = case
+    g = torch.Generator().manual_seed(M + N + K)
+    A = torch.randint(-3, 4, (M, K), generator=g).float()
+    B = torch.randint(-3, 4, (N, K), generator=g).float()
+    C = torch.randint(-8, 9, (M, N), generator=g).float()
+    if K > 4096:                      # keep |sum| small enough to be exact in fp16 too; both ends of K stay in play
+        A[:, 150:K - 150] = 0
+    ref = A.double() @ B.double().t()
+    assert float(ref.abs().max()) * 2 + 8 < 2048
+    pitch = (N + 8 + 7) // 8 * 8
+    for in_dt, atom, out_dt in ((torch.float16, mh.MFMA_F32_16x16x32_F16, torch.float16),
+                                (torch.bfloat16, mh.MFMA_F32_16x16x32_BF16, torch.float32),
+                                (torch.float32, mh.MFMA_F32_16x16x4_F32, torch.float32)):
+        a, b, c = A.to(in_dt).cuda(), B.to(in_dt).cuda(), C.to(out_dt).cuda()
+        big = torch.full((M + 2, pitch), 77.0, dtype=out_dt, device="cuda")
+        d = big[1:M + 1, 8:8 + N]
+        mh.gemm_(mh.tiled_mma_desc(atom, cta_tile=(0, 0, 0)), T(d), T(a), T(b), T(c), 2.0)
+        torch.cuda.synchronize()
+        assert torch.equal(d.cpu().double(), 2.0 * ref + C.double()), (case, in_dt, out_dt)
+        frame = big.clone()
+        frame[1:M + 1, 8:8 + N] = 77.0
+        assert bool((frame == 77.0).all()), "stores outside D"
+        d.zero_()
+        mh.gemm_(mh.tiled_mma_desc(atom, cta_tile=(0, 0, 0)), T(d), T(a), T(b))
+        torch.cuda.synchronize()
+        assert torch.equal(d.cpu().double(), ref), (case, in_dt, out_dt, "no C")
+    # NaN and Inf beyond the operands' K extent and in the rows after them must not reach D: the operands are windows too
+    Ab = torch.full((M + 1, K + 8), float("nan"), dtype=torch.float16, device="cuda")
+    Bb = torch.full((N + 1, K + 8), float("inf"), dtype=torch.float16, device="cuda")
+    Ab[:M, :K] = A.half().cuda()
+    Bb[:N, :K] = B.half().cuda()
+    d = torch.zeros(M, (N + 7) // 8 * 8, dtype=torch.float16, device="cuda")[:, :N]
+    mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(0, 0, 0)), T(d), T(Ab[:M, :K]), T(Bb[:N, :K]))
+    torch.cuda.synchronize()
+    assert torch.equal(d.cpu().double(), ref), (case, "operands inside NaN / Inf frames")
+
+
 def test_short_m_other_types(mh):
     g = torch.Generator().manual_seed(77)
     M, N, K = 16, 512, 1024
@@ -1291,7 +1335,7 @@ def test_fused_epilogue_every_op_bit_exact(mh, out_name, op):
     _epilogue_case(mh, mma, 512, 768, 128, out_name, op, "row", 300 + len(op))
 
 
-@pytest.mark.parametrize("kernel", ["256", "128", "64", "128 atom32", "predicated", "short-M", "split-K", "library", "ragged"])
+@pytest.mark.parametrize("kernel", ["256", "128", "64", "128 atom32", "predicated", "short-M", "split-K", "library", "ragged", "thin fringes"])
 @pytest.mark.parametrize("operand_kind", ["row", "col", "full", "scalar"])
 def test_fused_epilogue_every_kernel_and_operand(mh, kernel, operand_kind):
     """bias-style add with beta * C through every kernel family that writes D, row-major and column-major D, operands
@@ -1316,9 +1360,12 @@ def test_fused_epilogue_every_kernel_and_operand(mh, kernel, operand_kind):
     elif kernel == "split-K":
         mma = mh.tiled_mma_desc(F16, atom_layout=(2, 2, 1), cta_tile=(128, 128, 32), split_k=4)
         M, N, K = 256, 384, 512
-    elif kernel == "ragged":     # interior on 256x256 tiles, both fringes on the residue kernels
+    elif kernel == "ragged":     # 256x256 tiles that reach beyond M and N (the guarded instance)
         mma = mh.tiled_mma_desc(F16, cta_tile=(0, 0, 0))
         M, N, K = 4096 + 40, 2048 + 72, 64
+    elif kernel == "thin fringes":     # interior on 256x256 tiles, both fringes on the short-M kernel
+        mma = mh.tiled_mma_desc(F16, cta_tile=(0, 0, 0))
+        M, N, K = 4096 + 40, 2048 + 24, 64
     else:
         mma = mh.tiled_mma_desc(F16, cta_tile=(0, 0, 0))
         M, N, K = 2048, 4096, 64          # the library picks 256x256

@@ -21,9 +21,10 @@
 namespace moye {
 
 // kEdge: M, N need not be multiples of the tile and K need not be a multiple of the k-tile (only of 16
-// bytes): rows beyond M / N and k beyond K are read as zeros (the predication the reference's
-// copyto_if! is meant for, src/algorithm/copy.jl:4-16) and the epilogue stores element by element
-// inside the bounds.
+// bytes): a row beyond M / N is read from the operand's last row instead (what is computed from it is never
+// stored), k beyond K is read as zeros (the predication the reference's copyto_if! is meant for,
+// src/algorithm/copy.jl:4-16; only loads of the last k-tile can take that branch) and the epilogue stores
+// element by element inside the bounds.
 //
 // AT = 16 issues the 16x16 MFMA forms, AT = 32 the 32x32 ones (v_mfma_f32_32x32x16_{f16,bf16,fp8_fp8},
 // v_mfma_f32_32x32x2_f32).  A 32x32 MFMA reads 32 rows of each operand and half the K extent of the
@@ -67,16 +68,16 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
 #pragma unroll
     for (int i = 0; i < A_LD; ++i) {
         const int c = tid + 256 * i, row = c / CPR, ch = c % CPR;
-        a_src[i] = gA + row * kbytes_a + ch * 16;
+        a_src[i] = gA + (kEdge ? min(row, p.M - 1 - tm * BM) : row) * kbytes_a + ch * 16;
         a_dst[i] = row * CPR + (ch ^ swz<CPR>(row));
-        a_lim[i] = (int64_t)tm * BM + row < p.M ? (int)(kbytes - ch * 16) : 0;
+        a_lim[i] = (int)(kbytes - ch * 16);
     }
 #pragma unroll
     for (int i = 0; i < B_LD; ++i) {
         const int c = tid + 256 * i, row = c / CPR, ch = c % CPR;
-        b_src[i] = gB + row * kbytes_b + ch * 16;
+        b_src[i] = gB + (kEdge ? min(row, p.N - 1 - tn * BN) : row) * kbytes_b + ch * 16;
         b_dst[i] = row * CPR + (ch ^ swz<CPR>(row));
-        b_lim[i] = (int64_t)tn * BN + row < p.N ? (int)(kbytes - ch * 16) : 0;
+        b_lim[i] = (int)(kbytes - ch * 16);
     }
     // a chunk at byte offset koff of its row is inside the operand iff koff < lim
     auto load_a = [&](int i, int64_t koff) -> u32x4 {
@@ -460,11 +461,13 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
             return fail(MOYE_ERR_ALIGN, "gemm!: operands of the MFMA kernels need 16-byte aligned pointers and row pitches");
         a.tiles_m = (a.M + 127) / 128;
         a.tiles_n = (a.N + 127) / 128;
+        // k-tiles of 128 bytes when the library chose the tile and K is long enough to matter (half the barriers)
+        const bool wide_edge = chosen_here && (int64_t)a.K * eb >= 512;
         switch (in_dt) {
-            case MOYE_F16: return launch_out<InF16, 128, 128, 64, true>(out_dt, a, st);
-            case MOYE_BF16: return launch_out<InBF16, 128, 128, 64, true>(out_dt, a, st);
-            case MOYE_F8E4M3: return launch_out<InFP8, 128, 128, 64, true>(out_dt, a, st);
-            case MOYE_F32: return launch_out<InF32, 128, 128, 64, true>(out_dt, a, st);
+            case MOYE_F16: return wide_edge ? launch_out<InF16, 128, 128, 128, true>(out_dt, a, st) : launch_out<InF16, 128, 128, 64, true>(out_dt, a, st);
+            case MOYE_BF16: return wide_edge ? launch_out<InBF16, 128, 128, 128, true>(out_dt, a, st) : launch_out<InBF16, 128, 128, 64, true>(out_dt, a, st);
+            case MOYE_F8E4M3: return wide_edge ? launch_out<InFP8, 128, 128, 128, true>(out_dt, a, st) : launch_out<InFP8, 128, 128, 64, true>(out_dt, a, st);
+            case MOYE_F32: return wide_edge ? launch_out<InF32, 128, 128, 128, true>(out_dt, a, st) : launch_out<InF32, 128, 128, 64, true>(out_dt, a, st);
             default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: no MFMA atom for %s inputs", dtype_name(in_dt));
         }
     }

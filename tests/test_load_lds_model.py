@@ -91,3 +91,93 @@ def test_immediate_offset_variant_under_three_readings_of_the_instruction():
         k = p["q"] % 2
         plan.append(dict(p, imm=-1024 * (1 - k), voff=p["voff"] + 1024 * (1 - k), m0=p["m0"] + 1024 * (1 - k)))
     assert check(plan, pitch) == [] and check(plan, pitch, apply_imm_to_global=False)
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# gemm_mfma_tn_256 with ragged tiles (csrc/gemm_mfma256.hip, kRagged): rows clamped to the operand's last row, pieces
+# beyond K swapped for the row's first piece in the last k-tile
+# ---------------------------------------------------------------------------------------------------------------------
+
+def ragged256_plan(rows, k_bytes, pitch, tile):
+    """(byte offset from the operand's first byte, LDS byte address, row, piece) of every lane of every load-to-LDS
+    instruction that fills one operand's 256-row tile `tile`, for every k-tile; rows = M (or N)."""
+    waves, WROWS, LD = 8, 32, 4
+    ktiles = (k_bytes + 127) // 128
+    k_rem = (k_bytes % 128) // 16
+    k_valid = k_rem if k_rem else 8
+    for kt, wave, i, lane in itertools.product(range(ktiles), range(waves), range(LD), range(64)):
+        lrow, lch = wave * WROWS + (lane >> 3), (lane & 7) ^ (lane >> 3)
+        row0 = tile * 256 + lrow
+        base = min(row0, rows - 1) * pitch + lch * 16
+        more = max(rows - 1 - row0, 0)
+        tail_delta = 0 if lch < k_valid else -lch * 16
+        off = base + min(8 * i, more) * pitch + kt * 128 + (tail_delta if kt == ktiles - 1 else 0)
+        lds = (kt & 1) * (512 * 128) + (wave * WROWS * 8 + 8 * 8 * i) * 16 + 16 * lane
+        yield dict(kt=kt, off=off, lds=lds, row=min(row0 + 8 * i, rows - 1), want_row=row0 + 8 * i, piece=lch,
+                   masked=kt == ktiles - 1 and lch >= k_valid)
+
+
+def test_ragged_256_tile_addressing_stays_inside_the_operand():
+    for rows, k_elems, pad in ((4000, 4000, 0), (300, 8, 8), (257, 72, 0), (4099, 4104, 24), (256, 64, 0), (1, 40, 0)):
+        k_bytes = k_elems * 2
+        pitch = k_bytes + pad * 2
+        assert pitch % 16 == 0 and k_bytes % 16 == 0
+        for tile in range((rows + 255) // 256):
+            seen = set()
+            for p in ragged256_plan(rows, k_bytes, pitch, tile):
+                r, c = divmod(p["off"], pitch)
+                assert 0 <= p["off"] and p["off"] % 16 == 0
+                assert r < rows and c + 16 <= k_bytes, (rows, k_elems, tile, p)         # inside the operand's own bytes
+                assert r == p["row"]
+                if not p["masked"]:
+                    assert c == p["kt"] * 128 + p["piece"] * 16                          # the piece the fragment reads expect
+                assert 0 <= p["lds"] and p["lds"] + 16 <= 2 * 512 * 128 and p["lds"] % 16 == 0
+                key = (p["kt"], p["lds"])
+                assert key not in seen
+                seen.add(key)
+            assert len(seen) == ((k_bytes + 127) // 128) * 256 * 8                       # every piece of every stage, once
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# gemm_mfma_skinny_lds (csrc/gemm_mfma_skinny.hip): per-wave rings of whole 128-byte lines
+# ---------------------------------------------------------------------------------------------------------------------
+
+def skinny_lines_plan(M, N, k_bytes, MT, NTW, block, waves=4, stages=3):
+    ROWS = 16 * NTW + 16 * MT
+    LD, STAGE = ROWS // 8, ROWS * 8
+    lines = k_bytes // 128
+    length = lines // waves
+    n0 = block * 16 * NTW
+    first = (block // 8) % length
+    for wave, t, j, lane in itertools.product(range(waves), range(length), range(LD), range(64)):
+        r = 8 * j + (lane >> 3)
+        lch = (lane & 7) ^ (lane >> 3)
+        line = wave * length + (t + first) % length
+        if j < 2 * NTW:
+            operand, row = "B", min(n0 + r, N - 1)
+        else:
+            operand, row = "A", min(r - 16 * NTW, M - 1)
+        lds = (wave * stages * STAGE + (t % stages) * STAGE + 64 * j) * 16 + 16 * lane
+        yield dict(operand=operand, row=row, col=line * 128 + lch * 16, lds=lds, wave=wave, t=t, line=line)
+
+
+def test_short_m_line_staging_addressing():
+    for M, N, k_bytes, MT, NTW in ((16, 8192, 16384, 1, 2), (64, 100, 512, 4, 1), (33, 8191, 1536, 3, 2), (1, 32, 2048, 1, 1),
+                                   (48, 12000, 512, 3, 2)):
+        assert k_bytes % (128 * 4) == 0 and (M + 15) // 16 == MT
+        lds_bytes = 4 * 3 * (16 * NTW + 16 * MT) * 128
+        assert lds_bytes <= LDS_BYTES
+        blocks = (N + 16 * NTW - 1) // (16 * NTW)
+        for block in {0, 1, 9, blocks // 2, blocks - 1}:
+            seen, lines_of_wave = set(), {}
+            for p in skinny_lines_plan(M, N, k_bytes, MT, NTW, block):
+                rows = N if p["operand"] == "B" else M
+                assert 0 <= p["row"] < rows and 0 <= p["col"] and p["col"] + 16 <= k_bytes
+                assert 0 <= p["lds"] and p["lds"] + 16 <= lds_bytes
+                key = (p["wave"], p["t"], p["lds"])
+                assert key not in seen
+                seen.add(key)
+                lines_of_wave.setdefault(p["wave"], set()).add(p["line"])
+            # the waves' K ranges are disjoint and together cover K
+            allv = sorted(x for v in lines_of_wave.values() for x in v)
+            assert allv == list(range(k_bytes // 128))

@@ -647,6 +647,38 @@ def test_ragged_256_tiles_exact_on_integers(mh, case):
     assert torch.equal(d.cpu().double(), ref), (case, "operands inside NaN / Inf frames")
 
 
+def test_random_shapes_exact_on_integers(mh):
+    """Whatever kernel the library picks for a shape (short-M by registers or by lines, 64 / 128 / 256 tiles, whole,
+    predicated or ragged, interior plus thin fringes, K ranges), the result on small integers is exact.  Seeded shapes
+    from the ranges where the choice changes; row- and column-major D, with and without C."""
+    import random
+    rnd = random.Random(20240607)
+    pools = ([1, 8, 16, 17, 40, 64, 65, 96, 128, 200, 256, 300, 520], [16, 100, 128, 256, 1000, 2048, 4000, 4096, 4100, 4160, 8192, 8200],
+             [8, 32, 64, 72, 128, 256, 264, 512, 1000, 1024, 2048])
+    shapes = {(rnd.choice(pools[0]), rnd.choice(pools[1]), rnd.choice(pools[2])) for _ in range(40)}
+    shapes |= {(rnd.choice(pools[1]), rnd.choice(pools[1]), rnd.choice(pools[2][:8])) for _ in range(24)}
+    g = torch.Generator().manual_seed(5)
+    for (M, N, K) in sorted(shapes):
+        if M * N * K > 4096 * 4096 * 300:
+            K = 72
+        A = torch.randint(-2, 3, (M, K), generator=g).to(torch.float16)
+        B = torch.randint(-2, 3, (N, K), generator=g).to(torch.float16)
+        C = torch.randint(-8, 9, (M, N), generator=g).to(torch.float16)
+        a, b, c = A.cuda(), B.cuda(), C.cuda()
+        ref = (a.float() @ b.float().t()).double().cpu()            # exact: |sum| <= 4 K <= 8192 in fp32
+        if float(ref.abs().max()) * 2 + 8 >= 2048:                  # ... and representable in fp16 after alpha and C
+            continue
+        for split in (0, -1):
+            d = torch.full((M, N), 9.0, dtype=torch.float16, device="cuda")
+            mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(0, 0, 0), split_k=split), T(d), T(a), T(b), T(c), 2.0)
+            torch.cuda.synchronize()
+            assert torch.equal(d.cpu().double(), 2.0 * ref + C.double()), (M, N, K, "split_k", split)
+        dt_ = torch.full((N, M), 9.0, dtype=torch.float16, device="cuda")
+        mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(0, 0, 0)), T(dt_, (M, N), (1, M)), T(a), T(b))
+        torch.cuda.synchronize()
+        assert torch.equal(dt_.t().cpu().double(), ref), (M, N, K, "column-major D")
+
+
 def test_short_m_other_types(mh):
     g = torch.Generator().manual_seed(77)
     M, N, K = 16, 512, 1024

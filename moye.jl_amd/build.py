@@ -24,6 +24,7 @@ SOURCES = {
     # the epilogue's alpha * acc + beta * c is two products and a sum, each rounded (the oracle composes it from axpby!):
     # never contracted into fused operations
     "gemm_mfma.hip": ["-ffp-contract=off"],
+    "gemm_mfma128.hip": ["-ffp-contract=off"],
     "gemm_mfma256.hip": ["-ffp-contract=off"],
     "gemm_mfma256pp.hip": ["-ffp-contract=off"],
     "gemm_mfma256w4.hip": ["-ffp-contract=off"],

@@ -9,6 +9,7 @@
 #include <vector>
 
 #include "kernels.hpp"
+#include "gemm_plan.hpp"
 
 namespace moye {
 
@@ -131,9 +132,10 @@ static size_t kmajor_bytes(const Mat& m) {
     return (size_t)(m.rows * pitch + 255) / 256 * 256;
 }
 
-// split_k of the descriptor -> number of K ranges.  Negative = the library chooses: no split when the 128 x 128 tiles
-// of the problem fill half the chip or more, else the largest count up to 256 / tiles (one workgroup per CU) that cuts K into equal
-// ranges of whole 128-byte pieces of at least 512 bytes (so every kernel's k-tile divides a range).
+// split_k of the descriptor -> number of K ranges.  Negative = the library chooses: none for a problem that fills the chip
+// with 256 x 256 tiles; for a smaller one with the tile left to the library too, what the cost model of gemm_plan.hpp
+// finds cheapest together with the tile; with a named tile, none when the problem's 128 x 128 tiles fill half the chip,
+// else the largest count up to 256 / tiles that cuts K into equal ranges of whole 128-byte pieces of at least 512 bytes.
 static int split_count(const moye_tiled_mma* mma, int64_t M, int64_t N, int64_t K, int eb) {
     if (mma->split_k >= 0) return mma->split_k > 1 ? mma->split_k : 1;
     if (mma->flags & MOYE_GEMM_NO_WORKSPACE) return 1;  // nowhere to put the partial products
@@ -145,6 +147,10 @@ static int split_count(const moye_tiled_mma* mma, int64_t M, int64_t N, int64_t 
         return M > 32 && N % 64 == 0 && N / 64 >= 128 && (K * eb) % 256 == 0 ? 2 : 1;
     }
     const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+    if (mma->cta_tile_mnk[0] == 0 && mma->cta_tile_mnk[1] == 0 && mma->cta_tile_mnk[2] == 0 && (K * eb) % 16 == 0) {
+        if (((M + 255) / 256) * ((N + 255) / 256) >= 128) return 1;
+        return gemm_plan(M, N, K * eb, eb == 4, M % 64 == 0 && N % 64 == 0 && (K * eb) % 128 == 0, 16).split;
+    }
     if (tiles <= 0 || tiles >= 128) return 1;
     for (int64_t s = std::min<int64_t>(256 / tiles, K); s >= 2; --s)
         if (K % s == 0 && ((K / s) * eb) % 128 == 0 && (K / s) * eb >= 512) return (int)s;

@@ -16,6 +16,7 @@
 // 16x16 MFMA tiles.  The MFMA is issued with the B-matrix rows as its first operand and the
 // A-matrix rows as its second, so a lane ends up holding four CONSECUTIVE n of one m, which is
 // what a row-major D wants.
+#include "gemm_plan.hpp"
 #include "mfma_common.hpp"
 
 namespace moye {
@@ -389,10 +390,10 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         }
         bm = bn = big ? 256 : 128;
         if (bk_elems == 0) bk_elems = big || a.K % (128 / eb) == 0 ? 128 / eb : 64 / eb;
-        // a problem with fewer than 200 tiles of 128 x 128 leaves CUs idle: 64 x 64 tiles when they divide it
-        // (fp16 1024^3: 8.6 us against 14.9; 1536^3: 18.6 against 21.1; from 2048^3 on the larger tile wins)
+        // smaller problems: 64 x 64 tiles (four times the workgroups, no ragged form) where the cost model prices them
+        // below 128 x 128 tiles for the K ranges this call runs with (gemm_plan.hpp; fp16 1024^3: 8.3 us against 10.0)
         if (!big && a.M % 64 == 0 && a.N % 64 == 0 && a.K % bk_elems == 0 && !(a.xcd_swizzle & kGemmAtom32) &&
-            (int64_t)((a.M + 127) / 128) * ((a.N + 127) / 128) < 200)
+            gemm_plan(a.M, a.N, (int64_t)a.K * eb * (a.split > 1 ? a.split : 1), eb == 4, true, 16, a.split > 1 ? a.split : 1).tile == 64)
             bm = bn = 64;
         if (big && waves <= 1) waves = 8;
     }
@@ -441,6 +442,18 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
             case MOYE_F8E4M3: return wide64 ? launch_out<InFP8, 64, 64, 128>(out_dt, a, st) : launch_out<InFP8, 64, 64, 64>(out_dt, a, st);
             case MOYE_F32: return wide64 ? launch_out<InF32, 64, 64, 128>(out_dt, a, st) : launch_out<InF32, 64, 64, 64>(out_dt, a, st);
             default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: no MFMA atom for %s inputs", dtype_name(in_dt));
+        }
+    }
+    // 128 x 128 tiles with 128 bytes of K per tile run on the load-to-LDS kernel (gemm_mfma128.hip) when pointers and
+    // pitches are 16-byte aligned: whole tiles, or -- where residue tiles are asked for (MOYE_GEMM_PREDICATE, or the
+    // tile left to the library) -- tiles that reach beyond M, N and K.  The kernel below keeps 64-byte k-tiles, the
+    // 32 x 32 atoms and operands or D that are not aligned.
+    if (bm == 128 && bn == 128 && (bkb == 128 || chosen_here) && !misaligned && ((int64_t)a.K * eb) % 16 == 0) {
+        const bool whole = a.M % 128 == 0 && a.N % 128 == 0 && ((int64_t)a.K * eb) % 128 == 0;
+        if (whole) return gemm_mfma_tn_128_dispatch(in_dt, out_dt, a, st);
+        if (chosen_here || (a.xcd_swizzle & MOYE_GEMM_PREDICATE)) {
+            a.xcd_swizzle |= kGemmRagged;
+            return gemm_mfma_tn_128_dispatch(in_dt, out_dt, a, st);
         }
     }
     if (bm != 128 || bn != 128 || (bkb != 64 && bkb != 128))

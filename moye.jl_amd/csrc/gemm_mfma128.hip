@@ -1,0 +1,61 @@
+// gemm! on the matrix cores, 128 x 128 x (128 bytes of K) CTA tile with the load-to-LDS schedule of
+// gemm_mfma_lds_tile.hpp: four waves as 2 x 2 (wave tile 64 x 64, 64 accumulator registers per lane), 64 KiB of LDS, so
+// two workgroups share a CU and cover each other's barriers and load stalls.  For problems that do not fill the chip
+// with 256 x 256 tiles; against the kernel of gemm_mfma.hip, which stages its operands through registers (fp16,
+// same box): 4096^3 156 -> 123 us, 2048^3 29.5 -> 22.9 us, 256 x 8192 x 8192 98 -> 68 us, 8192 x 1024 x 4096 80 -> 63 us.
+//
+// kOps: element-wise operation in the epilogue; kRagged (with kOps): tiles that reach beyond M, N or K (rows clamped to
+// the operand's last row, the K tail masked in registers, guarded stores) -- the predication the reference's copyto_if!
+// is meant for (src/algorithm/copy.jl:4-16).
+#include "gemm_mfma_lds_tile.hpp"
+
+namespace moye {
+
+template <typename In, typename Out, bool kOps = false, bool kRagged = false>
+__global__ __launch_bounds__(256, 2) void gemm_mfma_tn_128(GemmArgs p) {
+    gemm_mfma_tn_lds_tile<In, Out, 128, 128, 2, 2, kOps, 0, 0, kRagged>(p);
+}
+
+template <typename In, typename Out, bool kOps, bool kRagged>
+static int32_t launch128_instance(const GemmArgs& a, hipStream_t st) {
+    constexpr int kLds = 2 * (128 + 128) * 128;  // two operand stages, 64 KiB
+    auto kern = gemm_mfma_tn_128<In, Out, kOps, kRagged>;
+    static LdsCap cap;
+    if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
+    kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1)), dim3(256), kLds, st>>>(a);
+    MOYE_HIP_CHECK(hipGetLastError());
+    return MOYE_OK;
+}
+
+template <typename In, typename Out>
+static int32_t launch128(const GemmArgs& a, hipStream_t st) {
+    if (a.xcd_swizzle & kGemmRagged) return launch128_instance<In, Out, true, true>(a, st);
+    if (a.ep_op != MOYE_MAP_IDENTITY) return launch128_instance<In, Out, true, false>(a, st);
+    return launch128_instance<In, Out, false, false>(a, st);
+}
+
+template <typename In>
+static int32_t launch128_out(int32_t out_dt, const GemmArgs& a, hipStream_t st) {
+    switch (out_dt) {
+        case MOYE_F32: return launch128<In, OutF32>(a, st);
+        case MOYE_F16: return launch128<In, OutF16>(a, st);
+        case MOYE_BF16: return launch128<In, OutBF16>(a, st);
+        default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: MFMA kernels write f32, f16 or bf16, not %s", dtype_name(out_dt));
+    }
+}
+
+// K-major operands, 16-byte aligned pointers and pitches (D's too); whole tiles (M, N multiples of 128, K of 128 bytes)
+// unless kGemmRagged is set in a.xcd_swizzle, in which case K only has to be a multiple of 16 bytes.  The caller checks.
+int32_t gemm_mfma_tn_128_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, hipStream_t st) {
+    a.tiles_m = (a.M + 127) / 128;
+    a.tiles_n = (a.N + 127) / 128;
+    switch (in_dt) {
+        case MOYE_F16: return launch128_out<InF16>(out_dt, a, st);
+        case MOYE_BF16: return launch128_out<InBF16>(out_dt, a, st);
+        case MOYE_F8E4M3: return launch128_out<InFP8>(out_dt, a, st);
+        case MOYE_F32: return launch128_out<InF32>(out_dt, a, st);
+        default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: no MFMA atom for %s inputs", dtype_name(in_dt));
+    }
+}
+
+}  // namespace moye

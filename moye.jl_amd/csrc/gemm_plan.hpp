@@ -1,0 +1,66 @@
+// Host-side choice of CTA tile and K ranges for a gemm! whose tile is left to the library and that does not fill the chip
+// with 256 x 256 tiles: a small cost model instead of thresholds, fitted to fp16 timings on one MI355X (256 CUs).
+//
+//   time = 3 us + k-tiles per workgroup x t(tile, workgroups resident on a CU) [x rounds] + second pass of a K split
+//
+// with k-tiles of 128 bytes of K and, per k-tile and workgroup,
+//   128 x 128 tiles (gemm_mfma128.hip, two workgroups fit a CU):   0.52 us alone on its CU, 0.94 us with a neighbour
+//   64 x 64 tiles (gemm_mfma.hip, four fit):                       0.40 / 0.47 / 0.66 / 0.84 us for 1 / 2 / 3 / 4 on a CU
+//                                                                  (alone: 0.33 while the operands fit the L2s, 0.49 beyond)
+// (256 x 8192 x 8192 on 128 workgroups of 128 x 128: 68 us; 4096^3 as two rounds of 512: 123 us; 1024^3 on 256
+// workgroups of 64 x 64: 8.3 us; 2048^3 on 1024: 31.5 us), and a second pass that moves the fp32 partial products
+// at about 6 TB/s (they are still in the caches) after 3 us of launch.  Ragged tiles cost the 128 x 128 kernel a
+// quarter more; the 64 x 64 kernel has no ragged form.  fp32 operands take six times as long per k-tile.
+#pragma once
+
+#include <cstdint>
+
+namespace moye {
+
+struct GemmPlan {
+    int tile;   // 64 or 128
+    int split;  // K ranges
+    double us;
+};
+
+inline double gemm_plan_cost(int tile, int split, int64_t M, int64_t N, int64_t k_bytes, bool f32_in) {
+    const int64_t tiles = ((M + tile - 1) / tile) * ((N + tile - 1) / tile), ctas = tiles * split;
+    const int slots = tile == 128 ? 2 : 4;
+    static const double t128[3] = {0, 0.52, 0.94}, t64[5] = {0, 0.40, 0.47, 0.66, 0.84};
+    const double ktiles = (double)((k_bytes / split + 127) / 128);
+    double per;
+    int64_t rounds = 1;
+    if (ctas <= 256 * (int64_t)slots) {
+        const int c = (int)((ctas + 255) / 256);
+        per = tile == 128 ? t128[c] : t64[c];
+    } else {
+        rounds = (ctas + 256 * slots - 1) / (256 * slots);
+        per = tile == 128 ? t128[slots] : t64[slots];
+    }
+    double us = 3.0 + (double)rounds * ktiles * per * (f32_in ? 6.0 : 1.0);
+    if (tile == 128 && (M % 128 || N % 128 || k_bytes % 128)) us *= 1.25;
+    if (split > 1) us += 3.0 + (2.0 * split * 4.0 + 4.0) * (double)M * (double)N / 6.0e6;
+    return us;
+}
+
+// `max_split` = 1 forbids K ranges (no workspace); `fixed_split` > 0 asks for the best tile for that many ranges (the
+// dispatch after the split has been made: k_bytes is then the whole K again, so both calls price the same candidates).
+inline GemmPlan gemm_plan(int64_t M, int64_t N, int64_t k_bytes, bool f32_in, bool tile64_ok, int max_split,
+                          int fixed_split = 0) {
+    GemmPlan best{128, fixed_split > 0 ? fixed_split : 1, 1e30};
+    for (int tile : {128, 64}) {
+        if (tile == 64 && !tile64_ok) continue;
+        for (int s = 1; s <= 16; s *= 2) {
+            if (fixed_split > 0 && s != fixed_split) continue;
+            if (fixed_split <= 0 && s > 1) {
+                // equal ranges of whole k-tiles, at least four of them
+                if (s > max_split || k_bytes % s || (k_bytes / s) % 128 || k_bytes / s < 512) continue;
+            }
+            const double us = gemm_plan_cost(tile, s, M, N, k_bytes, f32_in);
+            if (us < best.us) best = GemmPlan{tile, s, us};
+        }
+    }
+    return best;
+}
+
+}  // namespace moye

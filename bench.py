@@ -86,8 +86,8 @@ def cpu_baseline(cores):
 
 def headline_variants(mh, tensor_of, torch, stream, A, B, D):
     """The headline problem (fp16 4096^3, the operands of the timed run) through other descriptors: the CTA tile the
-    baseline's config 3 names (128x128x32), operands stored M- / N-major (no K-major copy), and a fused epilogue
-    (bias row added, then max with 0 taken per element: one launch)."""
+    baseline's config 3 names (128x128x32), the same tile with 64 k per k-tile on the load-to-LDS kernel, operands
+    stored M- / N-major (no K-major copy), and a fused epilogue (a bias row added: one launch)."""
     from moye_hip import _lib
     res = []
     flops = 2.0 * 4096 ** 3
@@ -108,6 +108,10 @@ def headline_variants(mh, tensor_of, torch, stream, A, B, D):
     timed("fp16 TN 4096^3 on the CTA tile config 3 names: 128x128x32, 2x2 waves",
           lambda: mh.gemm_(m128, tD, tA, tB, None, 1.0, stream),
           lambda: mh.time_gemm(m128, tD, tA, tB, None, 1.0, stream, warmup=3, iters=50))
+    m128l = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 2, 1), tile=(128, 128, 64), cta_tile=(128, 128, 64))
+    timed("fp16 TN 4096^3 on 128x128x64 tiles, 2x2 waves, load-to-LDS kernel (two workgroups per CU)",
+          lambda: mh.gemm_(m128l, tD, tA, tB, None, 1.0, stream),
+          lambda: mh.time_gemm(m128l, tD, tA, tB, None, 1.0, stream, warmup=3, iters=50))
     m256 = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 4, 1), cta_tile=(256, 256, 64), flags=_lib.GEMM_NO_WORKSPACE)
     At, Bt = A.t().contiguous(), B.t().contiguous()
     tAm, tBn = tensor_of(At, (4096, 4096), (1, 4096)), tensor_of(Bt, (4096, 4096), (1, 4096))

@@ -1278,6 +1278,12 @@ def test_bench_descriptor_f16_4096_against_fp64(mh):
     torch.cuda.synchronize()
     assert relerr(d128, c64) <= TOL16
     assert float((d.double() - d128.double()).abs().max()) <= 2 ** -8 * float(c64.abs().max())
+    # ... and so does the 128x128x64 tile on the load-to-LDS kernel (bench.py times it too)
+    d128l = torch.zeros_like(d)
+    mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 2, 1), cta_tile=(128, 128, 64)), T(d128l), T(a), T(b))
+    torch.cuda.synchronize()
+    assert relerr(d128l, c64) <= TOL16
+    assert float((d.double() - d128l.double()).abs().max()) <= 2 ** -8 * float(c64.abs().max())
 
 
 @pytest.mark.parametrize("out_dt", ["float16", "float32"])
@@ -1296,6 +1302,11 @@ def test_bench_descriptor_every_cta_exact_on_integers(mh, out_dt):
     torch.cuda.synchronize()
     want = (a.float() @ b.float().t())           # exact: |sum| <= 4 * 512 = 2048, an integer fp16 holds
     assert float(want.abs().max()) <= 2048
+    assert torch.equal(d.float(), want)
+    # the 1024 workgroups of the 128x128x64 tile on the load-to-LDS kernel, two to a CU
+    d.fill_(float("nan"))
+    mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 2, 1), cta_tile=(128, 128, 64)), T(d), T(a), T(b))
+    torch.cuda.synchronize()
     assert torch.equal(d.float(), want)
 
 

@@ -337,16 +337,17 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         // right (all interior rows, the last N % 256 columns) and the fringe below (the last M % 256 rows, all columns)
         // on the kernels that take residue tiles.  Three launches on the same stream, disjoint parts of D.
         const int M0 = a.M / 256 * 256, N0 = a.N / 256 * 256, ob0 = dtype_bytes(out_dt);
-        const bool aligned = !((a.lda * eb) % 16 || (a.ldb * eb) % 16 || (a.ldd * ob0) % 16 ||
-                               (reinterpret_cast<uintptr_t>(a.A) | reinterpret_cast<uintptr_t>(a.B) | reinterpret_cast<uintptr_t>(a.D)) % 16);
+        const bool aligned_ab = !((a.lda * eb) % 16 || (a.ldb * eb) % 16 ||
+                                  (reinterpret_cast<uintptr_t>(a.A) | reinterpret_cast<uintptr_t>(a.B)) % 16);
+        const bool aligned = aligned_ab && !((a.ldd * ob0) % 16 || reinterpret_cast<uintptr_t>(a.D) % 16);
         // Ragged tiles on the 256 x 256 kernel itself (its guarded instance: rows clamped, the K tail masked, stores
         // guarded) when that fills the chip, unless the fringes are thin enough for the short-M kernel, which then costs
         // less than a further round of tiles (fp16 4000 x 4096 x 4096: 170 us as interior + fringe on 128 x 128 tiles,
         // vendor library 96).  Not fp8: its fast kernel is the hand-ordered one, which has no guarded form.
         const int fr_m = a.M - M0, fr_n = a.N - N0;
-        const bool thin = fr_m <= 64 && fr_n <= 64 && a.K % (128 / eb) == 0;
+        const bool thin = fr_m <= 64 && fr_n <= 64 && a.K % (128 / eb) == 0 && aligned;  // (a D that is not 16-byte aligned: the guarded instance)
         const int64_t rtiles = (int64_t)((a.M + 255) / 256) * ((a.N + 255) / 256);
-        if (!big && !thin && a.split <= 1 && bk_elems == 0 && aligned && in_dt != MOYE_F8E4M3 && ((int64_t)a.K * eb) % 16 == 0 &&
+        if ((!big || !aligned) && !thin && a.split <= 1 && bk_elems == 0 && aligned_ab && in_dt != MOYE_F8E4M3 && ((int64_t)a.K * eb) % 16 == 0 &&
             rtiles >= 128 && stages < 3 && (waves <= 1 || waves == 8) &&
             !(a.xcd_swizzle & (MOYE_GEMM_WAVE4 | MOYE_GEMM_PINGPONG | kGemmAMajorM | kGemmBMajorN | kGemmAtom32))) {
             a.xcd_swizzle |= kGemmRagged;
@@ -392,7 +393,7 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         if (bk_elems == 0) bk_elems = big || a.K % (128 / eb) == 0 ? 128 / eb : 64 / eb;
         // smaller problems: 64 x 64 tiles (four times the workgroups, no ragged form) where the cost model prices them
         // below 128 x 128 tiles for the K ranges this call runs with (gemm_plan.hpp; fp16 1024^3: 8.3 us against 10.0)
-        if (!big && a.M % 64 == 0 && a.N % 64 == 0 && a.K % bk_elems == 0 && !(a.xcd_swizzle & kGemmAtom32) &&
+        if (!big && aligned && a.M % 64 == 0 && a.N % 64 == 0 && a.K % bk_elems == 0 && !(a.xcd_swizzle & kGemmAtom32) &&
             gemm_plan(a.M, a.N, (int64_t)a.K * eb * (a.split > 1 ? a.split : 1), eb == 4, true, 16, a.split > 1 ? a.split : 1).tile == 64)
             bm = bn = 64;
         if (big && waves <= 1) waves = 8;
@@ -402,9 +403,10 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
     if (bk_elems == 0) bk_elems = 64 / eb;  // 64 bytes of K per row: 32 halves / 64 fp8
     const int bkb = bk_elems * eb;
     const int ob = dtype_bytes(out_dt);
-    const bool misaligned =
-        (a.lda * eb) % 16 || (a.ldb * eb) % 16 || (a.ldd * ob) % 16 ||
-        (reinterpret_cast<uintptr_t>(a.A) | reinterpret_cast<uintptr_t>(a.B) | reinterpret_cast<uintptr_t>(a.D)) % 16;
+    const bool misaligned_ab = (a.lda * eb) % 16 || (a.ldb * eb) % 16 ||
+                               (reinterpret_cast<uintptr_t>(a.A) | reinterpret_cast<uintptr_t>(a.B)) % 16;
+    const bool misaligned_d = (a.ldd * ob) % 16 || reinterpret_cast<uintptr_t>(a.D) % 16;
+    const bool misaligned = misaligned_ab || misaligned_d;
     if (bm == 256 && bn == 256) {
         if (bkb != 128 && bkb != 64)
             return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the 256x256 MFMA kernels take %d or %d elements of K per tile", 64 / eb, 128 / eb);
@@ -446,10 +448,10 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
     }
     // 128 x 128 tiles with 128 bytes of K per tile run on the load-to-LDS kernel (gemm_mfma128.hip) when pointers and
     // pitches are 16-byte aligned: whole tiles, or -- where residue tiles are asked for (MOYE_GEMM_PREDICATE, or the
-    // tile left to the library) -- tiles that reach beyond M, N and K.  The kernel below keeps 64-byte k-tiles, the
-    // 32 x 32 atoms and operands or D that are not aligned.
-    if (bm == 128 && bn == 128 && (bkb == 128 || chosen_here) && !misaligned && ((int64_t)a.K * eb) % 16 == 0) {
-        const bool whole = a.M % 128 == 0 && a.N % 128 == 0 && ((int64_t)a.K * eb) % 128 == 0;
+    // tile left to the library) -- tiles that reach beyond M, N and K, which also take a D that is not 16-byte aligned.
+    // The kernel below keeps 64-byte k-tiles, the 32 x 32 atoms and operands that are not aligned.
+    if (bm == 128 && bn == 128 && (bkb == 128 || chosen_here) && !misaligned_ab && ((int64_t)a.K * eb) % 16 == 0) {
+        const bool whole = a.M % 128 == 0 && a.N % 128 == 0 && ((int64_t)a.K * eb) % 128 == 0 && !misaligned_d;
         if (whole) return gemm_mfma_tn_128_dispatch(in_dt, out_dt, a, st);
         if (chosen_here || (a.xcd_swizzle & MOYE_GEMM_PREDICATE)) {
             a.xcd_swizzle |= kGemmRagged;

@@ -13,8 +13,9 @@ namespace moye {
 // epi_value() (alpha, beta * C, the operation with its operand), convert and store 16-byte pieces.  The arithmetic
 // exists once, in a loop over the passes that is not unrolled: unrolled over all accumulators it would be several
 // thousand instructions per kernel.  `smem`: 32 x WN floats per wave.
-// kGuard: the tile may reach beyond M or N; rows beyond M are skipped, a piece that crosses N is read and stored element
-// by element up to N (rows of D start on 16-byte boundaries, so every piece inside N still goes out whole).
+// kGuard: the tile may reach beyond M or N, and D need not be 16-byte aligned; rows beyond M are skipped, a piece that
+// crosses N is read and stored element by element up to N, and so is a piece of D that does not start on a 16-byte
+// boundary (a pitch of D that is not a multiple of 16 bytes).
 template <typename Out, int MI, int NI, bool kGuard = false>
 __device__ __forceinline__ void store_c_tile_general(const GemmArgs& p, const f32x4 (&acc)[MI][NI], u32x4* smem, int wave,
                                                      int lane, int64_t m_base, int64_t n_base) {
@@ -50,6 +51,8 @@ __device__ __forceinline__ void store_c_tile_general(const GemmArgs& p, const f3
             const int64_t m = m_base + PASS_ROWS * pass + row, n0 = n_base + och * EPC;
             if (kGuard && (m >= p.M || n0 >= p.N)) continue;
             const bool whole = !kGuard || n0 + EPC <= p.N;  // else only the first N - n0 elements exist
+            char* const d16 = static_cast<char*>(p.D) + (m * p.ldd + n0) * (int64_t)sizeof(OutT);
+            const bool store16 = whole && (!kGuard || (reinterpret_cast<uintptr_t>(d16) & 15) == 0);
             float v[EPC], x[EPC];
 #pragma unroll
             for (int q = 0; q < EPC / 4; ++q) {
@@ -119,15 +122,15 @@ __device__ __forceinline__ void store_c_tile_general(const GemmArgs& p, const f3
 #pragma unroll
                     for (int e = 0; e < EPC; ++e) out[e] = Out::cvt(v[e]);
             }
-            if (whole) {
+            if (store16) {
                 u32x4 w;
                 __builtin_memcpy(&w, out, 16);
-                store_d_chunk(p, static_cast<char*>(p.D) + (m * p.ldd + n0) * (int64_t)sizeof(OutT), w);
+                store_d_chunk(p, d16, w);
             } else {
                 OutT* d = static_cast<OutT*>(p.D) + m * p.ldd + n0;
 #pragma unroll
                 for (int e = 0; e < EPC; ++e)
-                    if (n0 + e < p.N) d[e] = out[e];
+                    if (whole || n0 + e < p.N) d[e] = out[e];
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");

@@ -604,9 +604,9 @@ def test_short_m_line_staging_kernel(mh, M):
 
 
 @pytest.mark.parametrize("case", [(4000, 2200, 328), (3900, 2304, 120), (4096, 2048, 72), (4090, 2203, 40), (2100, 4100, 200),
-                                  (4099, 2050, 4096 + 8)])
+                                  (4099, 2050, 4096 + 8), (4096, 2048, 128), (1000, 600, 136), (384, 256, 128), (130, 2000, 72)])
 def test_ragged_256_tiles_exact_on_integers(mh, case):
-    """Problems the library puts on 256x256 tiles that reach beyond M, N and K: rows beyond the operands are read from
+    """Problems the library puts on 256x256 tiles (the larger cases) or 128x128 tiles that reach beyond M, N and K: rows beyond the operands are read from
     the last row and never stored, the K tail (1 to 7 pieces of 16 bytes, also with less than one k-tile in all) is
     masked, pieces of D that cross N go out element by element.  D is a window of a larger buffer whose frame must stay
     untouched; small integers make every sum exact."""
@@ -636,6 +636,17 @@ def test_ragged_256_tiles_exact_on_integers(mh, case):
         mh.gemm_(mh.tiled_mma_desc(atom, cta_tile=(0, 0, 0)), T(d), T(a), T(b))
         torch.cuda.synchronize()
         assert torch.equal(d.cpu().double(), ref), (case, in_dt, out_dt, "no C")
+    # a D whose rows do not start on 16-byte boundaries (pitch and first element 8 bytes off): the pieces that are not
+    # aligned go out element by element
+    a, b = A.half().cuda(), B.half().cuda()
+    big = torch.full((M + 2, N + 12 + (N % 2)), 77.0, dtype=torch.float16, device="cuda")
+    d = big[1:M + 1, 4:4 + N]
+    mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(0, 0, 0)), T(d), T(a), T(b))
+    torch.cuda.synchronize()
+    assert torch.equal(d.cpu().double(), ref), (case, "unaligned D")
+    frame = big.clone()
+    frame[1:M + 1, 4:4 + N] = 77.0
+    assert bool((frame == 77.0).all()), "stores outside an unaligned D"
     # NaN and Inf beyond the operands' K extent and in the rows after them must not reach D: the operands are windows too
     Ab = torch.full((M + 1, K + 8), float("nan"), dtype=torch.float16, device="cuda")
     Bb = torch.full((N + 1, K + 8), float("inf"), dtype=torch.float16, device="cuda")

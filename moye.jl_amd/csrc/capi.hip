@@ -132,9 +132,9 @@ static size_t kmajor_bytes(const Mat& m) {
     return (size_t)(m.rows * pitch + 255) / 256 * 256;
 }
 
-// split_k of the descriptor -> number of K ranges.  Negative = the library chooses: none for a problem that fills the chip
-// with 256 x 256 tiles; for a smaller one with the tile left to the library too, what the cost model of gemm_plan.hpp
-// finds cheapest together with the tile; with a named tile, none when the problem's 128 x 128 tiles fill half the chip,
+// split_k of the descriptor -> number of K ranges.  Negative = the library chooses: with the tile left to the library too,
+// what the cost model of gemm_plan.hpp finds cheapest together with the tile (none where 256 x 256 tiles come out
+// cheapest); with a named tile, none when the problem's 128 x 128 tiles fill half the chip,
 // else the largest count up to 256 / tiles that cuts K into equal ranges of whole 128-byte pieces of at least 512 bytes.
 static int split_count(const moye_tiled_mma* mma, int64_t M, int64_t N, int64_t K, int eb) {
     if (mma->split_k >= 0) return mma->split_k > 1 ? mma->split_k : 1;
@@ -148,8 +148,10 @@ static int split_count(const moye_tiled_mma* mma, int64_t M, int64_t N, int64_t 
     }
     const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
     if (mma->cta_tile_mnk[0] == 0 && mma->cta_tile_mnk[1] == 0 && mma->cta_tile_mnk[2] == 0 && (K * eb) % 16 == 0) {
-        if (((M + 255) / 256) * ((N + 255) / 256) >= 128) return 1;
-        return gemm_plan(M, N, K * eb, eb == 4, M % 64 == 0 && N % 64 == 0 && (K * eb) % 128 == 0, 16).split;
+        const GemmPlan pl = gemm_plan(M, N, K * eb, eb == 4, M % 64 == 0 && N % 64 == 0 && (K * eb) % 128 == 0, 16);
+        const bool ragged = M % 256 || N % 256 || (K * eb) % 128;
+        if (((M + 255) / 256) * ((N + 255) / 256) >= 64 && gemm_plan_cost_256(M, N, K * eb, eb == 4, ragged) <= pl.us) return 1;
+        return pl.split;
     }
     if (tiles <= 0 || tiles >= 128) return 1;
     for (int64_t s = std::min<int64_t>(256 / tiles, K); s >= 2; --s)

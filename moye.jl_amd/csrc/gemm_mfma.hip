@@ -330,9 +330,19 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         return gemm_mfma_skinny_dispatch(in_dt, out_dt, a, st);
     const bool chosen_here = bm == 0 && bn == 0;
     if (bm == 0 && bn == 0) {
-        // the library chooses: one 256x256 tile per CU when that fills the chip, else 128x128
-        const bool big = a.M % 256 == 0 && a.N % 256 == 0 && a.K % (128 / eb) == 0 &&
-                         (int64_t)(a.M / 256) * (a.N / 256) >= 128;
+        // the library chooses: 256 x 256 tiles, one per CU, where the cost model of gemm_plan.hpp prices them below
+        // 128 x 128 and 64 x 64 tiles (they need not fill the chip: fp16 4096 x 2304 x 4096, 144 tiles, 73 us against 93;
+        // 4096 x 2048 x 4096, 128 tiles, 72 us against 62 on 128 x 128 tiles)
+        const int64_t rtiles = (int64_t)((a.M + 255) / 256) * ((a.N + 255) / 256);
+        const int ranges = a.split > 1 ? a.split : 1;
+        const int64_t k_bytes_all = (int64_t)a.K * eb * ranges;
+        const bool whole256 = a.M % 256 == 0 && a.N % 256 == 0 && a.K % (128 / eb) == 0;
+        const GemmPlan plan = gemm_plan(a.M, a.N, k_bytes_all, eb == 4, a.M % 64 == 0 && a.N % 64 == 0 && ((int64_t)a.K * eb) % 128 == 0, 16, ranges);
+        // (operands that are not K-major were left where they lie only for the 256 x 256 kernel: no choice then)
+        const bool prefer256 = (a.xcd_swizzle & (kGemmAMajorM | kGemmBMajorN)) ? true
+                               : ranges > 1 ? rtiles >= 128
+                                            : rtiles >= 64 && gemm_plan_cost_256(a.M, a.N, k_bytes_all, eb == 4, !whole256) <= plan.us;
+        const bool big = whole256 && prefer256;
         // A large problem whose M or N is not a multiple of 256: the interior runs on 256x256 tiles, the fringe to the
         // right (all interior rows, the last N % 256 columns) and the fringe below (the last M % 256 rows, all columns)
         // on the kernels that take residue tiles.  Three launches on the same stream, disjoint parts of D.
@@ -346,14 +356,13 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         // vendor library 96).  Not fp8: its fast kernel is the hand-ordered one, which has no guarded form.
         const int fr_m = a.M - M0, fr_n = a.N - N0;
         const bool thin = fr_m <= 64 && fr_n <= 64 && a.K % (128 / eb) == 0 && aligned;  // (a D that is not 16-byte aligned: the guarded instance)
-        const int64_t rtiles = (int64_t)((a.M + 255) / 256) * ((a.N + 255) / 256);
         if ((!big || !aligned) && !thin && a.split <= 1 && bk_elems == 0 && aligned_ab && in_dt != MOYE_F8E4M3 && ((int64_t)a.K * eb) % 16 == 0 &&
-            rtiles >= 128 && stages < 3 && (waves <= 1 || waves == 8) &&
+            prefer256 && stages < 3 && (waves <= 1 || waves == 8) &&
             !(a.xcd_swizzle & (MOYE_GEMM_WAVE4 | MOYE_GEMM_PINGPONG | kGemmAMajorM | kGemmBMajorN | kGemmAtom32))) {
             a.xcd_swizzle |= kGemmRagged;
             return gemm_mfma_tn_256_dispatch(in_dt, out_dt, a, 8, stages, st);
         }
-        if (!big && a.split <= 1 && bk_elems == 0 && aligned && a.K % (128 / eb) == 0 && (int64_t)(M0 / 256) * (N0 / 256) >= 128) {
+        if (!big && a.split <= 1 && bk_elems == 0 && aligned && a.K % (128 / eb) == 0 && prefer256 && (int64_t)(M0 / 256) * (N0 / 256) >= 64) {
             GemmArgs part = a;
             part.M = M0; part.N = N0;
             if (int32_t e = gemm_mfma_tn_dispatch(in_dt, out_dt, 0, 0, 0, waves, stages, part, st)) return e;
@@ -393,8 +402,7 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         if (bk_elems == 0) bk_elems = big || a.K % (128 / eb) == 0 ? 128 / eb : 64 / eb;
         // smaller problems: 64 x 64 tiles (four times the workgroups, no ragged form) where the cost model prices them
         // below 128 x 128 tiles for the K ranges this call runs with (gemm_plan.hpp; fp16 1024^3: 8.3 us against 10.0)
-        if (!big && aligned && a.M % 64 == 0 && a.N % 64 == 0 && a.K % bk_elems == 0 && !(a.xcd_swizzle & kGemmAtom32) &&
-            gemm_plan(a.M, a.N, (int64_t)a.K * eb * (a.split > 1 ? a.split : 1), eb == 4, true, 16, a.split > 1 ? a.split : 1).tile == 64)
+        if (!big && aligned && a.M % 64 == 0 && a.N % 64 == 0 && a.K % bk_elems == 0 && !(a.xcd_swizzle & kGemmAtom32) && plan.tile == 64)
             bm = bn = 64;
         if (big && waves <= 1) waves = 8;
     }

@@ -9,8 +9,8 @@
 //                                                                  (alone: 0.33 while the operands fit the L2s, 0.49 beyond)
 // (256 x 8192 x 8192 on 128 workgroups of 128 x 128: 68 us; 4096^3 as two rounds of 512: 123 us; 1024^3 on 256
 // workgroups of 64 x 64: 8.3 us; 2048^3 on 1024: 31.5 us), and a second pass that moves the fp32 partial products
-// at about 6 TB/s (they are still in the caches) after 3 us of launch.  Ragged tiles cost the 128 x 128 kernel a
-// quarter more; the 64 x 64 kernel has no ragged form.  fp32 operands take six times as long per k-tile.
+// at about 6 TB/s (they are still in the caches) after 3 us of launch.  Ragged tiles cost the 128 x 128 kernel
+// 15 % more; the 64 x 64 kernel has no ragged form.  fp32 operands take six times as long per k-tile.
 #pragma once
 
 #include <cstdint>
@@ -38,7 +38,7 @@ inline double gemm_plan_cost(int tile, int split, int64_t M, int64_t N, int64_t 
         per = tile == 128 ? t128[slots] : t64[slots];
     }
     double us = 3.0 + (double)rounds * ktiles * per * (f32_in ? 6.0 : 1.0);
-    if (tile == 128 && (M % 128 || N % 128 || k_bytes % 128)) us *= 1.25;
+    if (tile == 128 && (M % 128 || N % 128 || k_bytes % 128)) us *= 1.15;
     if (split > 1) us += 3.0 + (2.0 * split * 4.0 + 4.0) * (double)M * (double)N / 6.0e6;
     return us;
 }
@@ -61,6 +61,19 @@ inline GemmPlan gemm_plan(int64_t M, int64_t N, int64_t k_bytes, bool f32_in, bo
         }
     }
     return best;
+}
+
+// The same problem on 256 x 256 tiles, one workgroup per CU: 9 us + per k-tile 1.44 us in a round that fills the chip,
+// 0.98 us in one that fills half of it or less (fewer requesters, and a higher clock on a part that is power-limited when
+// full), linear in between (fp16 K = 4096: 256 tiles 101 us, 224 91, 192 83, 144 73, 128 72); a quarter more for the
+// guarded instance (130 x 32768 x 4096 on 128 ragged tiles: 99 us).
+inline double gemm_plan_cost_256(int64_t M, int64_t N, int64_t k_bytes, bool f32_in, bool ragged) {
+    const int64_t tiles = ((M + 255) / 256) * ((N + 255) / 256), full = tiles / 256, rest = tiles % 256;
+    const double ktiles = (double)((k_bytes + 127) / 128);
+    const double t_rest = rest == 0 ? 0.0 : rest <= 128 ? 0.98 : 0.98 + (double)(rest - 128) / 128.0 * 0.46;
+    double us = 9.0 + 6.0 * (double)(full + (rest ? 1 : 0) - 1) + ktiles * ((double)full * 1.44 + t_rest) * (f32_in ? 6.0 : 1.0);
+    if (ragged) us *= 1.25;
+    return us;
 }
 
 }  // namespace moye

@@ -27,12 +27,12 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # where sessions differ (the 8192^3 GEMMs: how far the XCDs drift apart varies) the median session is quoted.
 TRAFFIC_SOURCE = "profiles/*_counters.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this script in earlier sessions; not measured in this run)"
 MEASURED_TRAFFIC = {
-    "gemm_f16_4096_tile256": {"read_bytes": 196907 * 1024, "write_bytes": 32782 * 1024},
-    "transpose_f32_16384": {"read_bytes": 1048618 * 1024, "write_bytes": 1050127 * 1024},
-    "gemm_bf16_8192_tile256": {"read_bytes": 1575091 * 1024, "write_bytes": 262899 * 1024},
+    "gemm_f16_4096_tile256": {"read_bytes": 196891 * 1024, "write_bytes": 32782 * 1024},
+    "transpose_f32_16384": {"read_bytes": 1048618 * 1024, "write_bytes": 1050139 * 1024},
+    "gemm_bf16_8192_tile256": {"read_bytes": 1581210 * 1024, "write_bytes": 262757 * 1024},
     "gemm_f32_8192_tile256": {"read_bytes": 2 * 2422808 * 1024, "write_bytes": 262152 * 1024},  # median of six sessions
     "gemm_fp8_8192_tile256": {"read_bytes": 787037 * 1024, "write_bytes": 131072 * 1024},
-    "gemm_bf16_16x8192x8192": {"read_bytes": 149542 * 1024, "write_bytes": 512 * 1024},
+    "gemm_bf16_16x8192x8192": {"read_bytes": 133211 * 1024, "write_bytes": 512 * 1024},
 }
 
 
@@ -199,7 +199,7 @@ def other_configs(mh, tensor_of, torch, stream):
     ms = e0.elapsed_time(e1) / iters
     nbytes = 16 * n * 2 + n * n * 2 + 16 * n * 4
     c64 = a16.float().double() @ b.float().double().t()
-    res.append({"workload": "bf16 TN 16x8192x8192, fp32 out (short-M kernel, B rotated over 3 buffers)",
+    res.append({"workload": "bf16 TN 16x8192x8192, fp32 out (short-M kernel staging 128-byte lines through LDS, B rotated over 3 buffers)",
                 "kernel_ms": round(ms, 5), "tflops": round(2.0 * 16 * n * n / ms / 1e9, 1),
                 "rel_err_vs_fp64": float((d16.double() - c64).abs().max() / c64.abs().max()),
                 "roofline": {"bound": "hbm", "achieved": round(nbytes / ms / 1e6, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",

@@ -7,19 +7,8 @@
 // 256 x 256 CTA tile halves the L2 bytes per flop of a 128 x 128 one.  4096 / 256 = 16, so a
 // 4096^2 problem is exactly 256 workgroups: one per CU, no tail.
 //
-// Schedule per k-tile (two k-steps of 32 halves / 64 fp8), operand tiles double-buffered in LDS,
-// fragments double-buffered in registers:
-//   step 0: ds_read the fragments of step 1 (buffer 1) | MFMAs of step 0 (buffer 0)
-//   s_waitcnt vmcnt(0) lgkmcnt(0), s_barrier: tile t+1 has landed, nobody reads tile t any more
-//   global_load_lds_dwordx4 of tile t+2 -> the stage tile t just vacated: the loads have a whole
-//     iteration to complete and go straight to LDS (no registers, no ds_write)
-//   step 1: ds_read the fragments of step 0 of tile t+1 (buffer 0) | MFMAs of step 1 (buffer 1)
-// so the MFMAs that follow a barrier always find their operands already in registers.
-// A load-to-LDS instruction writes lane l's 16 bytes at base + 16 l, so the XOR swizzle is
-// applied on the global side: lane l of a 64-chunk block fetches chunk (l%8)^(l/8) of row l/8.
-//
-// Same operand conventions as gemm_mfma.hip: K-major A and B, N-contiguous D, the MFMA issued
-// with B rows as its first operand so a lane holds four consecutive n of one m.
+// The k-loop and the epilogue are gemm_mfma_tn_lds_tile (gemm_mfma_lds_tile.hpp), shared with the 128 x 128 kernel of
+// gemm_mfma128.hip; the ring schedule below is a second k-loop for the same tile.
 #include "gemm_mfma_lds_tile.hpp"
 
 namespace moye {

@@ -85,7 +85,7 @@ def test_immediate_offset_variant_under_three_readings_of_the_instruction():
         assert check(plan, pitch) == []                                    # as documented: in bounds, right elements
         g = check(plan, pitch, apply_imm_to_global=False)
         assert g and {k for k, _ in g} <= {"global out of the tile", "global address is not the element's"}
-    # the 2.1 form of the variant, negative immediates (M0 = last block): the lane offsets grow instead; same verdict
+    # the first form of the variant, negative immediates (M0 = last block): the lane offsets grow instead; same verdict
     plan = []
     for p in w4_plan(8, pitch, 6):
         k = p["q"] % 2

@@ -187,7 +187,8 @@ int32_t moye_map(int32_t op, const moye_tensor* dst, const moye_tensor* a, const
 
 /* bytes of device workspace this gemm! call needs: the K-major copies of MFMA operands whose unit stride
  * is not along K (NN / NT / TT problems, src/arch/mma/make_mma_ops.jl:253-265) and split_k * M * N fp32
- * partial products of a split-K call; 0 for plain TN and for UniversalFMA.
+ * partial products of a split-K call; 0 for plain TN, for UniversalFMA, and for f16 / bf16 operands of any major
+ * that run on whole 256x256x64 or 128x128x64 tiles without K ranges (read where they lie).
  *   moye_gemm     keeps a workspace of its own per (device, stream): allocated by the first call on that stream
  *                 that needs one (a synchronous hipMalloc inside that call, so not under stream capture),
  *                 replaced by a larger one when a larger call comes, never freed inside a call.  Calls on

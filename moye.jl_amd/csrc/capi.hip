@@ -159,21 +159,26 @@ static int split_count(const moye_tiled_mma* mma, int64_t M, int64_t N, int64_t 
     return 1;
 }
 
-// An operand with its unit stride along M (N) instead of K needs no K-major copy when the call runs on the 256 x 256
-// kernel's transposing fragment reads (gemm_mfma256.hip): f16 / bf16 through the 16x16x32 atoms, the 256 x 256 x 64 tile
-// (named, or the library's own choice for this size), eight waves, the two-stage schedule; the operand dense along its
-// rows with a pitch of whole 16-byte pieces.
-static bool majors_run_natively(const moye_tiled_mma* mma, const Mat& A, const Mat& B) {
+// An operand with its unit stride along M (N) instead of K needs no K-major copy when the call runs on the transposing
+// fragment reads of the load-to-LDS kernels (gemm_mfma_lds_tile.hpp): f16 / bf16 through the 16x16x32 atoms, whole
+// 256 x 256 x 64 tiles on eight waves or whole 128 x 128 x 64 tiles (named, or the library's own choice for a problem of
+// whole 128 x 128 tiles with more than 64 rows), the two-stage schedule, no K ranges; the operand dense along its rows
+// with a pitch of whole 16-byte pieces, and D 16-byte aligned (the guarded instances, which take any D, read K-major
+// operands only).
+static bool majors_run_natively(const moye_tiled_mma* mma, const Mat& A, const Mat& B, const Mat& D) {
     if (mma->atom != MOYE_MFMA_F32_16x16x32_F16 && mma->atom != MOYE_MFMA_F32_16x16x32_BF16) return false;
     if ((mma->flags & (MOYE_GEMM_PINGPONG | MOYE_GEMM_WAVE4)) || mma->stages >= 3) return false;
-    if (mma->atom_layout_mnk[0] * mma->atom_layout_mnk[1] == 4) return false;
     if (mma->split_k != 0 && mma->split_k != 1) return false;  // the K ranges of a split need not be whole k-tiles
     const int64_t M = A.rows, N = B.rows, K = A.cols;
     const int bm = mma->cta_tile_mnk[0], bn = mma->cta_tile_mnk[1], bk = mma->cta_tile_mnk[2];
-    if (M % 256 || N % 256 || K % 64) return false;
-    const bool named = bm == 256 && bn == 256 && (bk == 0 || bk == 64);
-    const bool chosen = bm == 0 && bn == 0 && bk == 0 && (M / 256) * (N / 256) >= 128;
-    if (!named && !chosen) return false;
+    if (K % 64) return false;
+    const bool four_waves = mma->atom_layout_mnk[0] * mma->atom_layout_mnk[1] == 4;
+    const bool named256 = bm == 256 && bn == 256 && (bk == 0 || bk == 64) && !four_waves && M % 256 == 0 && N % 256 == 0;
+    const bool named128 = bm == 128 && bn == 128 && bk == 64 && M % 128 == 0 && N % 128 == 0;
+    const bool chosen = bm == 0 && bn == 0 && bk == 0 && M > 64 && M % 128 == 0 && N % 128 == 0;
+    if (!named256 && !named128 && !chosen) return false;
+    const int64_t d_pitch = D.cs == 1 ? D.rs : D.cs;
+    if ((D.cs != 1 && D.rs != 1) || (d_pitch * dtype_bytes(D.dtype)) % 16 || reinterpret_cast<uintptr_t>(D.ptr) % 16) return false;
     for (const Mat* x : {&A, &B}) {
         if (x->cs == 1 || x->cols == 1) continue;  // K-major already
         if (x->rs != 1 || (x->cs * 2) % 16 || reinterpret_cast<uintptr_t>(x->ptr) % 16 || x->cs < x->rows) return false;
@@ -192,8 +197,8 @@ static size_t gemm_workspace_bytes_impl(const moye_tiled_mma* mma, const Mat& A,
     return n;
 }
 
-static size_t gemm_workspace_bytes(const moye_tiled_mma* mma, const Mat& A, const Mat& B) {
-    return gemm_workspace_bytes_impl(mma, A, B, majors_run_natively(mma, A, B));
+static size_t gemm_workspace_bytes(const moye_tiled_mma* mma, const Mat& A, const Mat& B, const Mat& D) {
+    return gemm_workspace_bytes_impl(mma, A, B, majors_run_natively(mma, A, B, D));
 }
 
 // transposes `m` (unit stride along its rows index) into ws as rows x K with K contiguous and rewrites `m`
@@ -281,7 +286,7 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
     // along K are brought to the K-major form the kernels read (one tiled transpose each)
     char* ws = nullptr;
     std::unique_lock<std::mutex> ws_lock(g_ws_mutex, std::defer_lock);
-    const bool native_majors = majors_run_natively(mma, A, B);
+    const bool native_majors = majors_run_natively(mma, A, B, D);
     int major_flags = 0;  // which of the kernel's operands keep their M- (N-) major form
     if (native_majors) {
         if (A.cs != 1 && A.cols > 1) { major_flags |= kGemmAMajorM; A.rs = A.cs; A.cs = 1; }  // Mat::rs now holds the pitch between consecutive k
@@ -501,10 +506,11 @@ int32_t moye_gemm_workspace_size(const moye_tiled_mma* mma, const moye_tensor* D
                                  const moye_tensor* B, size_t* bytes) {
     if (!mma || !D || !A || !B || !bytes) return fail(MOYE_ERR_ARG, "moye_gemm_workspace_size: null argument");
     *bytes = 0;
-    Mat a, b;
+    Mat a, b, d;
     if (int32_t e = as_matrix(A, "A", &a)) return e;
     if (int32_t e = as_matrix(B, "B", &b)) return e;
-    if (!(mma->flags & MOYE_GEMM_NO_WORKSPACE)) *bytes = gemm_workspace_bytes(mma, a, b);
+    if (int32_t e = as_matrix(D, "D", &d)) return e;
+    if (!(mma->flags & MOYE_GEMM_NO_WORKSPACE)) *bytes = gemm_workspace_bytes(mma, a, b, d);
     return MOYE_OK;
 }
 

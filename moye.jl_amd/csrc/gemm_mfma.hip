@@ -338,9 +338,10 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         const int64_t k_bytes_all = (int64_t)a.K * eb * ranges;
         const bool whole256 = a.M % 256 == 0 && a.N % 256 == 0 && a.K % (128 / eb) == 0;
         const GemmPlan plan = gemm_plan(a.M, a.N, k_bytes_all, eb == 4, a.M % 64 == 0 && a.N % 64 == 0 && ((int64_t)a.K * eb) % 128 == 0, 16, ranges);
-        // (operands that are not K-major were left where they lie only for the 256 x 256 kernel: no choice then)
-        const bool prefer256 = (a.xcd_swizzle & (kGemmAMajorM | kGemmBMajorN)) ? true
-                               : ranges > 1 ? rtiles >= 128
+        // (operands that were left M- or N-major: the host made sure of whole 128 x 128 tiles, an aligned D and no K ranges;
+        // such a call takes whole 256 x 256 or 128 x 128 tiles, never 64 x 64 ones, ragged ones or fringes)
+        const bool majors = a.xcd_swizzle & (kGemmAMajorM | kGemmBMajorN);
+        const bool prefer256 = ranges > 1 ? rtiles >= 128
                                             : rtiles >= 64 && gemm_plan_cost_256(a.M, a.N, k_bytes_all, eb == 4, !whole256) <= plan.us;
         const bool big = whole256 && prefer256;
         // A large problem whose M or N is not a multiple of 256: the interior runs on 256x256 tiles, the fringe to the
@@ -362,7 +363,7 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
             a.xcd_swizzle |= kGemmRagged;
             return gemm_mfma_tn_256_dispatch(in_dt, out_dt, a, 8, stages, st);
         }
-        if (!big && a.split <= 1 && bk_elems == 0 && aligned && a.K % (128 / eb) == 0 && prefer256 && (int64_t)(M0 / 256) * (N0 / 256) >= 64) {
+        if (!big && !majors && a.split <= 1 && bk_elems == 0 && aligned && a.K % (128 / eb) == 0 && prefer256 && (int64_t)(M0 / 256) * (N0 / 256) >= 64) {
             GemmArgs part = a;
             part.M = M0; part.N = N0;
             if (int32_t e = gemm_mfma_tn_dispatch(in_dt, out_dt, 0, 0, 0, waves, stages, part, st)) return e;
@@ -402,7 +403,7 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         if (bk_elems == 0) bk_elems = big || a.K % (128 / eb) == 0 ? 128 / eb : 64 / eb;
         // smaller problems: 64 x 64 tiles (four times the workgroups, no ragged form) where the cost model prices them
         // below 128 x 128 tiles for the K ranges this call runs with (gemm_plan.hpp; fp16 1024^3: 8.3 us against 10.0)
-        if (!big && aligned && a.M % 64 == 0 && a.N % 64 == 0 && a.K % bk_elems == 0 && !(a.xcd_swizzle & kGemmAtom32) && plan.tile == 64)
+        if (!big && !majors && aligned && a.M % 64 == 0 && a.N % 64 == 0 && a.K % bk_elems == 0 && !(a.xcd_swizzle & kGemmAtom32) && plan.tile == 64)
             bm = bn = 64;
         if (big && waves <= 1) waves = 8;
     }

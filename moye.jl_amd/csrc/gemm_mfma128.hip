@@ -11,15 +11,15 @@
 
 namespace moye {
 
-template <typename In, typename Out, bool kOps = false, bool kRagged = false>
+template <typename In, typename Out, bool kOps = false, bool kRagged = false, int AMAJ = 0, int BMAJ = 0>
 __global__ __launch_bounds__(256, 2) void gemm_mfma_tn_128(GemmArgs p) {
-    gemm_mfma_tn_lds_tile<In, Out, 128, 128, 2, 2, kOps, 0, 0, kRagged>(p);
+    gemm_mfma_tn_lds_tile<In, Out, 128, 128, 2, 2, kOps, AMAJ, BMAJ, kRagged>(p);
 }
 
-template <typename In, typename Out, bool kOps, bool kRagged>
+template <typename In, typename Out, bool kOps, bool kRagged, int AMAJ = 0, int BMAJ = 0>
 static int32_t launch128_instance(const GemmArgs& a, hipStream_t st) {
     constexpr int kLds = 2 * (128 + 128) * 128;  // two operand stages, 64 KiB
-    auto kern = gemm_mfma_tn_128<In, Out, kOps, kRagged>;
+    auto kern = gemm_mfma_tn_128<In, Out, kOps, kRagged, AMAJ, BMAJ>;
     static LdsCap cap;
     if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
     kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1)), dim3(256), kLds, st>>>(a);
@@ -29,6 +29,19 @@ static int32_t launch128_instance(const GemmArgs& a, hipStream_t st) {
 
 template <typename In, typename Out>
 static int32_t launch128(const GemmArgs& a, hipStream_t st) {
+    const bool am = a.xcd_swizzle & kGemmAMajorM, bm = a.xcd_swizzle & kGemmBMajorN;
+    if (am || bm) {
+        // operands that are not K-major (AMAJ / BMAJ of gemm_mfma_lds_tile.hpp): 16-bit types, whole tiles (the host checked)
+        if constexpr (In::kBytes == 2) {
+            if (a.xcd_swizzle & kGemmRagged) return fail(MOYE_ERR_UNSUPPORTED, "gemm!: ragged tiles take K-major operands");
+            const bool ops = a.ep_op != MOYE_MAP_IDENTITY;
+            if (am && bm) return ops ? launch128_instance<In, Out, true, false, 1, 1>(a, st) : launch128_instance<In, Out, false, false, 1, 1>(a, st);
+            if (am) return ops ? launch128_instance<In, Out, true, false, 1, 0>(a, st) : launch128_instance<In, Out, false, false, 1, 0>(a, st);
+            return ops ? launch128_instance<In, Out, true, false, 0, 1>(a, st) : launch128_instance<In, Out, false, false, 0, 1>(a, st);
+        } else {
+            return fail(MOYE_ERR_UNSUPPORTED, "gemm!: operands that are not K-major run natively with 16-bit types only");
+        }
+    }
     if (a.xcd_swizzle & kGemmRagged) return launch128_instance<In, Out, true, true>(a, st);
     if (a.ep_op != MOYE_MAP_IDENTITY) return launch128_instance<In, Out, true, false>(a, st);
     return launch128_instance<In, Out, false, false>(a, st);

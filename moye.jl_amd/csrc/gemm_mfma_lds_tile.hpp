@@ -29,7 +29,7 @@ namespace moye {
 //
 // AMAJ / BMAJ = 1: that operand is stored with its unit stride along M (N) instead of K, the 'N' forms of
 // src/arch/mma/make_mma_ops.jl:253-265 (GemmArgs::lda / ldb is then the pitch between consecutive k).  Its LDS tile is
-// 64 k-rows of 256 operand rows (512 bytes), brought in by the same load-to-LDS instructions, and the fragments come
+// 64 k-rows of BM operand rows (512 or 256 bytes), brought in by the same load-to-LDS instructions, and the fragments come
 // out of it with ds_read_b64_tr_b16, the transposing LDS read of gfx950, where the reference has ldmatrix.trans
 // (src/arch/copy/ldmatrix.jl:18-48): sixteen lanes that each point at four consecutive 16-bit values of a row get back
 // the four values lane j's position holds in rows 0..3 of their group (measured on the hardware: result e of lane j of a
@@ -46,7 +46,7 @@ namespace moye {
 template <typename In, typename Out, int BM, int BN, int WGM, int WGN, bool kOps, int AMAJ, int BMAJ, bool kRagged>
 __device__ __forceinline__ void gemm_mfma_tn_lds_tile(GemmArgs p) {
     static_assert(!kRagged || (kOps && !AMAJ && !BMAJ), "ragged tiles: K-major operands, the general epilogue");
-    static_assert((BM == 256 && BN == 256) || (BM == 128 && BN == 128 && WGM == 2 && WGN == 2 && !AMAJ && !BMAJ), "tile shapes");
+    static_assert((BM == 256 && BN == 256) || (BM == 128 && BN == 128 && WGM == 2 && WGN == 2), "tile shapes");
     constexpr int CPR = 8;  // 8 chunks of 16 bytes per tile row
     constexpr int A_CH = BM * CPR, B_CH = BN * CPR, STAGE = A_CH + B_CH;
     constexpr int NWAVES = WGM * WGN;
@@ -85,27 +85,29 @@ __device__ __forceinline__ void gemm_mfma_tn_lds_tile(GemmArgs p) {
         }
     }
     const int dma_slot = __builtin_amdgcn_readfirstlane(wave * WROWS * CPR);  // + 8 rows * CPR per i
-    // An M-major (N-major) operand: wave w fills k-rows KROWS w + 2 i + l / 32 of the tile, two rows (1 KiB) per
-    // instruction; lane l brings the 16-byte chunk that belongs in physical slot l % 32 of its row.
+    // An M-major (N-major) operand: a k-row of the tile is TROW bytes (BM 16-bit values); wave w fills k-rows
+    // KROWS w + TRPI i + l / TLPR of the tile, TRPI rows (1 KiB) per instruction; lane l brings the 16-byte chunk that
+    // belongs in physical slot l % TLPR of its row.
     constexpr int KROWS = 64 / NWAVES;
-    static_assert(!(AMAJ || BMAJ) || (In::kBytes == 2 && KROWS == 2 * LD), "transposing fragment reads: 16-bit operands");
+    constexpr int TROW = BM * 2, TLPR = TROW / 16, TRPI = 64 / TLPR;
+    static_assert(!(AMAJ || BMAJ) || (In::kBytes == 2 && BM == BN && KROWS == TRPI * LD), "transposing fragment reads: 16-bit operands");
     auto tr_swz = [](int krow) { return (krow & 3) | (((krow >> 3) & 1) << 2); };
     [[maybe_unused]] int64_t tA[AMAJ ? LD : 1], tB[BMAJ ? LD : 1];  // byte offsets of this lane's chunk, per instruction, from the k-tile's first row
     if constexpr (AMAJ) {
 #pragma unroll
         for (int i = 0; i < LD; ++i) {
-            const int krow = wave * KROWS + 2 * i + (lane >> 5), p16 = lane & 31, l32 = (p16 >> 1) ^ tr_swz(krow);
+            const int krow = wave * KROWS + TRPI * i + lane / TLPR, p16 = lane % TLPR, l32 = (p16 >> 1) ^ tr_swz(krow);
             tA[i] = krow * pitch_a + ((int64_t)tm * BM) * In::kBytes + (l32 * 2 + (p16 & 1)) * 16;
         }
     }
     if constexpr (BMAJ) {
 #pragma unroll
         for (int i = 0; i < LD; ++i) {
-            const int krow = wave * KROWS + 2 * i + (lane >> 5), p16 = lane & 31, l32 = (p16 >> 1) ^ tr_swz(krow);
+            const int krow = wave * KROWS + TRPI * i + lane / TLPR, p16 = lane % TLPR, l32 = (p16 >> 1) ^ tr_swz(krow);
             tB[i] = krow * pitch_b + ((int64_t)tn * BN) * In::kBytes + (l32 * 2 + (p16 & 1)) * 16;
         }
     }
-    const int dma_slot_t = __builtin_amdgcn_readfirstlane(wave * KROWS * 32);  // + 2 rows * 32 chunks per i
+    const int dma_slot_t = __builtin_amdgcn_readfirstlane(wave * KROWS * TLPR);  // + 64 chunks (TRPI rows) per i
 
     // fragment slots: row = w?0 + 16 i + r16, chunk = 4 ks + kq
     int fa_slot[2], fb_slot[2];
@@ -119,8 +121,9 @@ __device__ __forceinline__ void gemm_mfma_tn_lds_tile(GemmArgs p) {
     // transposed operands: byte offset of this lane's first read of 16-row block 0 of k-step 0 inside the operand tile;
     // block idx adds (idx << 5) by XOR (the piece index is swizzled), k-step ks adds 32 rows, the second read 4 rows
     const int fx = ((r16 >> 2) & 3) | ((kq & 1) << 2);
-    const int ta_lane = (8 * kq + (r16 >> 2)) * 512 + (wm0 / 128) * 256 + ((((wm0 / 16) & 7) ^ fx) << 5) + 8 * (r16 & 3);
-    const int tb_lane = (8 * kq + (r16 >> 2)) * 512 + (wn0 / 128) * 256 + ((((wn0 / 16) & 7) ^ fx) << 5) + 8 * (r16 & 3);
+    // (the blocks of a wave tile start at a piece index whose low bits are clear, so adding the block is an XOR too)
+    const int ta_lane = (8 * kq + (r16 >> 2)) * TROW + (wm0 / 128) * 256 + ((((wm0 / 16) & 7) ^ fx) << 5) + 8 * (r16 & 3);
+    const int tb_lane = (8 * kq + (r16 >> 2)) * TROW + (wn0 / 128) * 256 + ((((wn0 / 16) & 7) ^ fx) << 5) + 8 * (r16 & 3);
 
     f32x4 acc[MI][NI];
 #pragma unroll
@@ -134,9 +137,9 @@ __device__ __forceinline__ void gemm_mfma_tn_lds_tile(GemmArgs p) {
     typedef __attribute__((address_space(3))) v4s* tr_ptr_t;
     // the eight k of one row of a transposed operand tile: two transposing reads, 4 k-rows apart
     auto tr_frag = [&](const u32x4* tile16, int lane_off, int idx, int ks) __attribute__((always_inline)) -> u32x4 {
-        const char* base = reinterpret_cast<const char*>(tile16) + ((lane_off ^ (idx << 5)) + ks * 32 * 512);
+        const char* base = reinterpret_cast<const char*>(tile16) + ((lane_off ^ (idx << 5)) + ks * 32 * TROW);
         const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_ptr_t)(base));
-        const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_ptr_t)(base + 4 * 512));
+        const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_ptr_t)(base + 4 * TROW));
         u32x2 l2, h2;
         __builtin_memcpy(&l2, &lo, 8);
         __builtin_memcpy(&h2, &hi, 8);

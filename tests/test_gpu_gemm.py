@@ -1475,21 +1475,23 @@ def test_fused_epilogue_limits(mh):
 
 
 # ---------------------------------------------------------------------------------------------
-# operands that are not K-major, without a workspace: the 256x256 kernel's transposing fragment reads
+# operands that are not K-major, without a workspace: the transposing fragment reads of the load-to-LDS kernels
 # ---------------------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("tdt,atom", [("float16", "MFMA_F32_16x16x32_F16"), ("bfloat16", "MFMA_F32_16x16x32_BF16")])
 @pytest.mark.parametrize("majors", ["mk", "kn", "mn"])
 def test_operand_majors_native_exact_on_integers(mh, tdt, atom, majors):
     """A stored M-major and / or B stored N-major (NN / NT / TT of src/arch/mma/make_mma_ops.jl:253-265) through the
-    256x256 tile with MOYE_GEMM_NO_WORKSPACE: no K-major copy is made, the fragments come out of LDS through the
+    256x256 and 128x128 tiles with MOYE_GEMM_NO_WORKSPACE: no K-major copy is made, the fragments come out of LDS through the
     transposing read.  Small integers, so every misplaced element shows; named tile and the library's choice, row- and
     column-major D, C and alpha, fp32 and 16-bit results, a padded pitch, and the epilogue operation."""
     from moye_hip import _lib
     tdt = getattr(torch, tdt)
     atom = getattr(mh, atom)
     g = torch.Generator().manual_seed(71)
-    cases = [(512, 768, 256, (256, 256, 64), 0), (256, 256, 64, (256, 256, 0), 8), (2048, 4096, 128, (0, 0, 0), 0), (512, 512, 16384, (256, 256, 64), 0)]
+    cases = [(512, 768, 256, (256, 256, 64), 0), (256, 256, 64, (256, 256, 0), 8), (2048, 4096, 128, (0, 0, 0), 0), (512, 512, 16384, (256, 256, 64), 0),
+             # the 128x128 tile of the same schedule: named, and as the library's choice for problems of whole 128x128 tiles
+             (384, 640, 256, (128, 128, 64), 8), (128, 128, 64, (128, 128, 64), 0), (1152, 896, 128, (0, 0, 0), 0), (2048, 2048, 192, (0, 0, 0), 8)]
     for (M, N, K, cta, pad) in cases:
         A = torch.randint(-3, 4, (M, K), generator=g).to(tdt)
         B = torch.randint(-3, 4, (N, K), generator=g).to(tdt)
@@ -1507,7 +1509,7 @@ def test_operand_majors_native_exact_on_integers(mh, tdt, atom, majors):
         mma = mh.tiled_mma_desc(atom, atom_layout=(2, 4, 1), cta_tile=cta, flags=_lib.GEMM_NO_WORKSPACE)
         for out_dt in (torch.float32, tdt):
             d = torch.zeros(M, N, dtype=out_dt, device="cuda")
-            assert mh.gemm_workspace_size(mma, T(d), ta, tb) == 0
+            assert mh.gemm_workspace_size(mh.tiled_mma_desc(atom, atom_layout=(2, 4, 1), cta_tile=cta), T(d), ta, tb) == 0
             mh.gemm_(mma, T(d), ta, tb)
             torch.cuda.synchronize()
             want = ref if out_dt == torch.float32 else ref.to(out_dt).double()
@@ -1548,3 +1550,19 @@ def test_operand_majors_native_random_and_speed(mh):
         times[name] = mh.time_gemm(mma, T(d), ta, tb, None, 1.0, None, warmup=5, iters=100)
     print("fp16 4096^3 by operand major: " + ", ".join("%s %.1f us" % (k, v * 1e3) for k, v in times.items()))
     assert times["NN"] < 1.25 * times["TN"]
+    # the same on a problem the library puts on 128x128 tiles
+    M = N = K = 2048
+    a_k, b_k = a_k[:M, :K].contiguous(), b_k[:N, :K].contiguous()
+    a_m, b_n = a_k.t().contiguous(), b_k.t().contiguous()
+    c64 = a_k.double() @ b_k.double().t()
+    mma = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(0, 0, 0), flags=_lib.GEMM_NO_WORKSPACE)
+    times = {}
+    for name, ta, tb in (("TN", T(a_k), T(b_k)), ("NN", T(a_m, (M, K), (1, M)), T(b_n, (N, K), (1, N)))):
+        d = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+        mh.gemm_(mma, T(d), ta, tb)
+        torch.cuda.synchronize()
+        assert relerr(d, c64) <= TOL16, name
+        mh.time_gemm(mma, T(d), ta, tb, None, 1.0, None, warmup=20, iters=100)
+        times[name] = mh.time_gemm(mma, T(d), ta, tb, None, 1.0, None, warmup=5, iters=100)
+    print("fp16 2048^3 by operand major: " + ", ".join("%s %.1f us" % (k, v * 1e3) for k, v in times.items()))
+    assert times["NN"] < 1.7 * times["TN"]      # (the 128x128 tile reads LDS near its limit already; with K-major copies: about 1.3)

@@ -252,6 +252,10 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
     if (tC) {
         if (int32_t e = as_matrix(tC, "C", &C)) return e;
     }
+    // the stride of a mode of extent 1 is never used: a one-row operand with unit stride along its columns gets the
+    // pitch a dense row-major array of its shape would have, so that it is not taken for M-major or misaligned
+    for (Mat* x : {&A, &B, &C, &D})
+        if (x->rows == 1 && x->cs == 1) x->rs = x->cols;
     // blas.jl:55-57,79-82: size(A,1)==size(C,1), size(B,1)==size(C,2), size(A,2)==size(B,2)
     if (A.rows != D.rows) return fail(MOYE_ERR_SHAPE, "gemm!: M of A (%lld) and D (%lld) differ", (long long)A.rows, (long long)D.rows);
     if (B.rows != D.cols) return fail(MOYE_ERR_SHAPE, "gemm!: N of B (%lld) and D (%lld) differ", (long long)B.rows, (long long)D.cols);
@@ -510,6 +514,8 @@ int32_t moye_gemm_workspace_size(const moye_tiled_mma* mma, const moye_tensor* D
     if (int32_t e = as_matrix(A, "A", &a)) return e;
     if (int32_t e = as_matrix(B, "B", &b)) return e;
     if (int32_t e = as_matrix(D, "D", &d)) return e;
+    for (Mat* x : {&a, &b, &d})
+        if (x->rows == 1 && x->cs == 1) x->rs = x->cols;
     if (!(mma->flags & MOYE_GEMM_NO_WORKSPACE)) *bytes = gemm_workspace_bytes(mma, a, b, d);
     return MOYE_OK;
 }

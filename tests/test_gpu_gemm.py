@@ -690,6 +690,21 @@ def test_random_shapes_exact_on_integers(mh):
         assert torch.equal(dt_.t().cpu().double(), ref), (M, N, K, "column-major D")
 
 
+def test_one_row_operands_with_any_stride_on_the_unit_mode(mh):
+    """A 1 x K operand described as (1, K):(1, 1) (what an M-major view of a one-row A looks like) and a 1 x N result
+    described the same way: the stride of the mode of extent 1 is never used and must not be taken for a pitch."""
+    g = torch.Generator().manual_seed(3)
+    for (N, K) in ((1000, 264), (8192, 512), (8, 32)):
+        A = torch.randint(-3, 4, (1, K), generator=g).half()
+        B = torch.randint(-3, 4, (N, K), generator=g).half()
+        ref = A.double() @ B.double().t()
+        a, b = A.cuda(), B.cuda()
+        d = torch.zeros(1, N, dtype=torch.float32, device="cuda")
+        mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(0, 0, 0)), T(d, (1, N), (1, 1)), T(a, (1, K), (1, 1)), T(b))
+        torch.cuda.synchronize()
+        assert torch.equal(d.cpu().double(), ref), (N, K)
+
+
 def test_short_m_other_types(mh):
     g = torch.Generator().manual_seed(77)
     M, N, K = 16, 512, 1024

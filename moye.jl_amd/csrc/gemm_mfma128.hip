@@ -42,7 +42,8 @@ static int32_t launch128(const GemmArgs& a, hipStream_t st) {
             return fail(MOYE_ERR_UNSUPPORTED, "gemm!: operands that are not K-major run natively with 16-bit types only");
         }
     }
-    if (a.xcd_swizzle & kGemmRagged) return launch128_instance<In, Out, true, true>(a, st);
+    if (a.xcd_swizzle & kGemmRagged)
+        return a.ep_op != MOYE_MAP_IDENTITY ? launch128_instance<In, Out, true, true>(a, st) : launch128_instance<In, Out, false, true>(a, st);
     if (a.ep_op != MOYE_MAP_IDENTITY) return launch128_instance<In, Out, true, false>(a, st);
     return launch128_instance<In, Out, false, false>(a, st);
 }

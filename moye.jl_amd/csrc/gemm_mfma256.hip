@@ -162,7 +162,8 @@ static int32_t launch256(const GemmArgs& a, hipStream_t st) {
     if (a.xcd_swizzle & kGemmRagged) {
         if constexpr (WGM * WGN == 8 && !std::is_same<In, InFP8>::value) {
             if (am || bm) return fail(MOYE_ERR_UNSUPPORTED, "gemm!: ragged 256 x 256 tiles take K-major operands");
-            return launch256_instance<In, Out, WGM, WGN, true, 0, 0, true>(a, st);
+            return a.ep_op != MOYE_MAP_IDENTITY ? launch256_instance<In, Out, WGM, WGN, true, 0, 0, true>(a, st)
+                                                : launch256_instance<In, Out, WGM, WGN, false, 0, 0, true>(a, st);
         } else {
             return fail(MOYE_ERR_UNSUPPORTED, "gemm!: ragged 256 x 256 tiles run on eight waves with f16, bf16 or f32 operands");
         }

@@ -42,10 +42,10 @@ namespace moye {
 // src/algorithm/copy.jl:4-16, for whole tiles).  A row beyond the operand is read from the operand's last row instead and
 // what is computed from it is never stored; in the last k-tile a lane whose 16-byte piece lies beyond K reads the
 // row's first piece instead and every fragment piece beyond K is zeroed in registers before it reaches an MFMA; the
-// epilogue is the general one with its row and column guards.
+// epilogues run with their row and column guards.
 template <typename In, typename Out, int BM, int BN, int WGM, int WGN, bool kOps, int AMAJ, int BMAJ, bool kRagged>
 __device__ __forceinline__ void gemm_mfma_tn_lds_tile(GemmArgs p) {
-    static_assert(!kRagged || (kOps && !AMAJ && !BMAJ), "ragged tiles: K-major operands, the general epilogue");
+    static_assert(!kRagged || (!AMAJ && !BMAJ), "ragged tiles: K-major operands");
     static_assert((BM == 256 && BN == 256) || (BM == 128 && BN == 128 && WGM == 2 && WGN == 2), "tile shapes");
     constexpr int CPR = 8;  // 8 chunks of 16 bytes per tile row
     constexpr int A_CH = BM * CPR, B_CH = BN * CPR, STAGE = A_CH + B_CH;
@@ -299,7 +299,7 @@ __device__ __forceinline__ void gemm_mfma_tn_lds_tile(GemmArgs p) {
     // (a kOps instance is only launched for calls with an operation or with ragged tiles: it carries the general
     // epilogue alone, which keeps the other one's registers out of its allocation)
     if constexpr (kOps) store_c_tile_general<Out, MI, NI, kRagged>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
-    else store_c_tile<Out, MI, NI, false>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
+    else store_c_tile<Out, MI, NI, false, kRagged>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
 }
 
 }  // namespace moye

@@ -143,7 +143,9 @@ __device__ __forceinline__ void store_c_tile_general(const GemmArgs& p, const f3
 // relative to (m_base, n_base).  `smem` must be free of operand data for all waves.
 // kWithOps = false leaves the element-wise operations out (the hand-ordered kernel: its register allocation around the
 // inline-assembly MFMAs must not change with what the epilogue needs; the host never sends it such a call).
-template <typename Out, int MI, int NI, bool kWithOps = true>
+// kGuard: the tile may reach beyond M or N and D need not be 16-byte aligned: nothing is read or stored beyond them, a
+// piece of D that crosses N or does not start on a 16-byte boundary goes out element by element.
+template <typename Out, int MI, int NI, bool kWithOps = true, bool kGuard = false>
 __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&acc)[MI][NI], u32x4* smem, int wave,
                                              int lane, int64_t m_base, int64_t n_base) {
     typedef typename Out::type OutT;
@@ -166,12 +168,17 @@ __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&ac
     // element by element.
     constexpr int NCH = PASS_ROWS * CR / 64, PASSES = MI / PASS_MI;
     constexpr int AHEAD = sizeof(OutT) == 2 ? PASSES : (PASSES < 2 ? PASSES : 2);
-    const bool row_c = p.C && (p.xcd_swizzle & kGemmRowC);
+    // (ragged tiles read C in whole pieces only when no piece crosses N)
+    const bool row_c = p.C && (p.xcd_swizzle & kGemmRowC) && (!kGuard || p.N % EPC == 0);
     u32x4 cw[AHEAD][NCH];
     auto fetch_c = [&](int pass, u32x4 (&into)[NCH]) __attribute__((always_inline)) {
 #pragma unroll
         for (int t = 0; t < NCH; ++t) {
             const int c = lane + 64 * t, row = c / CR, ch = c % CR;
+            if (kGuard && (m_base + PASS_ROWS * pass + row >= p.M || n_base + ch * EPC >= p.N)) {
+                into[t] = u32x4{0u, 0u, 0u, 0u};
+                continue;
+            }
             into[t] = *reinterpret_cast<const u32x4*>(static_cast<const char*>(p.C) +
                                                       ((m_base + PASS_ROWS * pass + row) * p.ldc_m + n_base) * (int64_t)sizeof(OutT) + ch * 16);
         }
@@ -209,7 +216,8 @@ __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&ac
                     for (int e = 0; e < 4; ++e) c[e] = Out::load(dst, e);
                 } else if (p.C) {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) c[e] = Out::load(p.C, m * p.ldc_m + (n + e) * p.ldc_n);
+                    for (int e = 0; e < 4; ++e)
+                        if (!kGuard || (m < p.M && n + e < p.N)) c[e] = Out::load(p.C, m * p.ldc_m + (n + e) * p.ldc_n);
                 }
                 float v[4] = {__fmul_rn(acc[i][j].x, p.alpha), __fmul_rn(acc[i][j].y, p.alpha), __fmul_rn(acc[i][j].z, p.alpha),
                               __fmul_rn(acc[i][j].w, p.alpha)};
@@ -230,6 +238,18 @@ __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&ac
             const u32x4 w = patch16[row * CR + (ch ^ (row & 7))];
             char* d = static_cast<char*>(p.D) +
                       ((m_base + 16 * i0 + row) * p.ldd + n_base) * (int64_t)sizeof(OutT) + ch * 16;
+            if constexpr (kGuard) {
+                const int64_t m = m_base + 16 * i0 + row, n0 = n_base + ch * EPC;
+                if (m >= p.M || n0 >= p.N) continue;
+                if (n0 + EPC > p.N || (reinterpret_cast<uintptr_t>(d) & 15)) {
+                    OutT o[EPC];
+                    __builtin_memcpy(o, &w, 16);
+#pragma unroll
+                    for (int e = 0; e < EPC; ++e)
+                        if (n0 + e < p.N) reinterpret_cast<OutT*>(d)[e] = o[e];
+                    continue;
+                }
+            }
             store_d_chunk(p, d, w);
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");

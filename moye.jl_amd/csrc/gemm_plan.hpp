@@ -10,7 +10,7 @@
 // (256 x 8192 x 8192 on 128 workgroups of 128 x 128: 68 us; 4096^3 as two rounds of 512: 123 us; 1024^3 on 256
 // workgroups of 64 x 64: 8.3 us; 2048^3 on 1024: 31.5 us), and a second pass that moves the fp32 partial products
 // at about 6 TB/s (they are still in the caches) after 3 us of launch.  Ragged tiles cost the 128 x 128 kernel
-// 15 % more; the 64 x 64 kernel has no ragged form.  fp32 operands take six times as long per k-tile.
+// 15 % more; the 64 x 64 kernel has no ragged form.  fp32 operands have their own per-k-tile times.
 #pragma once
 
 #include <cstdint>
@@ -26,18 +26,16 @@ struct GemmPlan {
 inline double gemm_plan_cost(int tile, int split, int64_t M, int64_t N, int64_t k_bytes, bool f32_in) {
     const int64_t tiles = ((M + tile - 1) / tile) * ((N + tile - 1) / tile), ctas = tiles * split;
     const int slots = tile == 128 ? 2 : 4;
-    static const double t128[3] = {0, 0.52, 0.94}, t64[5] = {0, 0.40, 0.47, 0.66, 0.84};
+    // per k-tile and workgroup with 1 .. slots workgroups resident on a CU.  fp32 operands run on v_mfma_f32_16x16x4_f32,
+    // an eighth of the 16-bit rate per byte of K, and are bound by it (2048^3 on 256 workgroups of 128 x 128: 128 us;
+    // 4096 x 2048 x 4096 on 512: 589 us; 1024^3 on 256 workgroups of 64 x 64: 25.7 us; 2048^3 on 1024: 156 us)
+    static const double t128_16[3] = {0, 0.52, 0.94}, t64_16[5] = {0, 0.40, 0.47, 0.66, 0.84};
+    static const double t128_32[3] = {0, 1.96, 4.58}, t64_32[5] = {0, 0.71, 1.25, 1.80, 2.40};
+    const double* t = tile == 128 ? (f32_in ? t128_32 : t128_16) : (f32_in ? t64_32 : t64_16);
     const double ktiles = (double)((k_bytes / split + 127) / 128);
-    double per;
-    int64_t rounds = 1;
-    if (ctas <= 256 * (int64_t)slots) {
-        const int c = (int)((ctas + 255) / 256);
-        per = tile == 128 ? t128[c] : t64[c];
-    } else {
-        rounds = (ctas + 256 * slots - 1) / (256 * slots);
-        per = tile == 128 ? t128[slots] : t64[slots];
-    }
-    double us = 3.0 + (double)rounds * ktiles * per * (f32_in ? 6.0 : 1.0);
+    // whole rounds of 256 x slots workgroups, then the rest with fewer neighbours
+    const int64_t full = ctas / (256 * slots), rest = ctas % (256 * slots);
+    double us = 3.0 + ktiles * ((double)full * t[slots] + (rest ? t[(rest + 255) / 256] : 0.0));
     if (tile == 128 && (M % 128 || N % 128 || k_bytes % 128)) us *= 1.15;
     if (split > 1) us += 3.0 + (2.0 * split * 4.0 + 4.0) * (double)M * (double)N / 6.0e6;
     return us;
@@ -70,8 +68,10 @@ inline GemmPlan gemm_plan(int64_t M, int64_t N, int64_t k_bytes, bool f32_in, bo
 inline double gemm_plan_cost_256(int64_t M, int64_t N, int64_t k_bytes, bool f32_in, bool ragged) {
     const int64_t tiles = ((M + 255) / 256) * ((N + 255) / 256), full = tiles / 256, rest = tiles % 256;
     const double ktiles = (double)((k_bytes + 127) / 128);
-    const double t_rest = rest == 0 ? 0.0 : rest <= 128 ? 0.98 : 0.98 + (double)(rest - 128) / 128.0 * 0.46;
-    double us = 9.0 + 6.0 * (double)(full + (rest ? 1 : 0) - 1) + ktiles * ((double)full * 1.44 + t_rest) * (f32_in ? 6.0 : 1.0);
+    // (fp32: 7.56 us per k-tile however many CUs are busy: the matrix pipe alone sets the pace, 4096 x 4096 x 1024 251 us)
+    const double t_full = f32_in ? 7.56 : 1.44;
+    const double t_rest = rest == 0 ? 0.0 : f32_in ? 7.56 : rest <= 128 ? 0.98 : 0.98 + (double)(rest - 128) / 128.0 * 0.46;
+    double us = 9.0 + 6.0 * (double)(full + (rest ? 1 : 0) - 1) + ktiles * ((double)full * t_full + t_rest);
     if (ragged) us *= 1.25;
     return us;
 }

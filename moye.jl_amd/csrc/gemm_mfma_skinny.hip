@@ -3,7 +3,7 @@
 // workgroup owns 16 or 32 rows of B (that many output columns) and all of A; its waves split K into contiguous ranges,
 // and the per-wave partial accumulators are summed through LDS in wave order, which makes the result independent of
 // timing.  A (at most 64 x K) is re-read by every workgroup and lives in L2.
-//   gemm_mfma_skinny_lds  K a multiple of 512 bytes: whole 128-byte lines of both operands go through LDS (load-to-LDS
+//   gemm_mfma_skinny_lds  K a multiple of 128 bytes: whole 128-byte lines of both operands go through LDS (load-to-LDS
 //                         instructions), four waves per workgroup; bf16 16 x 8192 x 8192: 21.0 us
 //   gemm_mfma_skinny      any K of whole 64-byte steps: each lane loads 16-byte pieces of its B row straight into the
 //                         MFMA operand registers, eight waves; the same problem: 32.4 us.  With 32 rows of B per
@@ -134,8 +134,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_skinny_lds(GemmArgs p) {
     const int n0 = blockIdx.x * 16 * NTW;
     u32x4* const ring = smem + __builtin_amdgcn_readfirstlane(wave * kStages * STAGE);
 
-    const int lines = (int)(((int64_t)p.K * In::kBytes) / 128);  // a multiple of WAVES (checked by the host)
-    const int len = lines / WAVES, s0 = wave * len;
+    // the waves' K ranges: whole 128-byte lines, as even as they come (a wave may get none of a very short K)
+    const int lines = (int)(((int64_t)p.K * In::kBytes) / 128);
+    const int s0 = (int)((int64_t)lines * wave / WAVES), len = (int)((int64_t)lines * (wave + 1) / WAVES) - s0;
     // M and N need not be multiples of 16: a row beyond the operand is read from the last row instead, and what is
     // computed from it is not stored
     const int lrow = lane >> 3, lch = (lane & 7) ^ (lane >> 3);
@@ -160,7 +161,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_skinny_lds(GemmArgs p) {
     // Workgroups that walk K in the same order ask their L2 for the same lines of A at the same moment, before any of
     // them has them: a workgroup starts its walk at a line that depends on its position within its L2's share of the
     // grid.  The order of a column's k-sum follows the workgroup, not the time, so results stay reproducible.
-    const int first = (int)((blockIdx.x / 8) % (unsigned)len);
+    const int first = len > 0 ? (int)((blockIdx.x / 8) % (unsigned)len) : 0;
     auto line_of = [&](int t) { const int r = t + first; return s0 + (r >= len ? r - len : r); };
 #define MOYE_STAGE_LOAD(T)                                                                                      \
     {                                                                                                           \
@@ -230,12 +231,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_skinny_lds(GemmArgs p) {
 }
 
 constexpr int kSkinnyLdsWaves = 4;
-static_assert(kSkinnyLineBytes == 128 * kSkinnyLdsWaves, "the host decides about K ranges by this");
+static_assert(kSkinnyLineBytes == 128, "the host decides about K ranges by this");
 
-// K a whole number of 128-byte lines per wave
+// K a whole number of 128-byte lines
 template <typename In>
 static bool skinny_lds_takes(const GemmArgs& a) {
-    return a.K > 0 && ((int64_t)a.K * In::kBytes) % (128 * kSkinnyLdsWaves) == 0;
+    return a.K > 0 && ((int64_t)a.K * In::kBytes) % kSkinnyLineBytes == 0;
 }
 
 template <typename In, typename Out, int MT, int W, int NTW, int S, int AUX>

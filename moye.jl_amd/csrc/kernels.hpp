@@ -59,7 +59,7 @@ int32_t gemm_mfma_tn_128_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, hip
 int32_t gemm_mfma_skinny_dispatch(int32_t in_dt, int32_t out_dt, const GemmArgs& a, hipStream_t st);
 // The short-M kernel stages whole 128-byte lines of K through LDS, four waves with a K range each, when K is this many
 // bytes or a multiple of it (else every lane loads its own 16-byte pieces).
-constexpr int kSkinnyLineBytes = 4 * 128;
+constexpr int kSkinnyLineBytes = 128;
 int32_t axpby_dispatch(double a, const moye_tensor* X, double b, const moye_tensor* Y, hipStream_t st);
 int32_t fill_dispatch(const moye_tensor* X, double value, hipStream_t st);
 int32_t map_dispatch(int32_t op, const moye_tensor* D, const moye_tensor* A, const moye_tensor* B, double scalar, hipStream_t st);

@@ -146,13 +146,15 @@ def skinny_lines_plan(M, N, k_bytes, MT, NTW, block, waves=4, stages=3):
     ROWS = 16 * NTW + 16 * MT
     LD, STAGE = ROWS // 8, ROWS * 8
     lines = k_bytes // 128
-    length = lines // waves
     n0 = block * 16 * NTW
-    first = (block // 8) % length
-    for wave, t, j, lane in itertools.product(range(waves), range(length), range(LD), range(64)):
+    for wave, j, lane in itertools.product(range(waves), range(LD), range(64)):
+      s0 = lines * wave // waves
+      length = lines * (wave + 1) // waves - s0          # the waves' K ranges: as even as whole lines come
+      first = (block // 8) % length if length else 0
+      for t in range(length):
         r = 8 * j + (lane >> 3)
         lch = (lane & 7) ^ (lane >> 3)
-        line = wave * length + (t + first) % length
+        line = s0 + (t + first) % length
         if j < 2 * NTW:
             operand, row = "B", min(n0 + r, N - 1)
         else:
@@ -163,8 +165,8 @@ def skinny_lines_plan(M, N, k_bytes, MT, NTW, block, waves=4, stages=3):
 
 def test_short_m_line_staging_addressing():
     for M, N, k_bytes, MT, NTW in ((16, 8192, 16384, 1, 2), (64, 100, 512, 4, 1), (33, 8191, 1536, 3, 2), (1, 32, 2048, 1, 1),
-                                   (48, 12000, 512, 3, 2)):
-        assert k_bytes % (128 * 4) == 0 and (M + 15) // 16 == MT
+                                   (48, 12000, 512, 3, 2), (16, 8192, 640, 1, 2), (7, 64, 128, 1, 1), (64, 8192, 1408, 4, 2)):
+        assert k_bytes % 128 == 0 and (M + 15) // 16 == MT
         lds_bytes = 4 * 3 * (16 * NTW + 16 * MT) * 128
         assert lds_bytes <= LDS_BYTES
         blocks = (N + 16 * NTW - 1) // (16 * NTW)

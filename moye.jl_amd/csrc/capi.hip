@@ -383,6 +383,7 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
         g.C = tC ? C.ptr : nullptr; g.ldc_m = C.rs; g.ldc_n = C.cs; g.D = D.ptr;
         if (rows_in_16_byte_pieces(g.C, g.ldc_m, g.ldc_n, D.dtype)) g.xcd_swizzle |= kGemmRowC;
         if (operand_rows_in_16_byte_pieces(g)) g.xcd_swizzle |= kGemmEpiRowX;
+        if (g.ep_op == MOYE_MAP_ADD && (!g.ep_x || g.ep_xm == 0 || g.ep_xn == 0)) g.xcd_swizzle |= kGemmEpiAddVec;  // a bias
         return gemm_mfma_tn_dispatch(in_dt, D.dtype, bm, bn, bk, waves, mma->stages, g, st);
     }
     if (D.rs == 1 && bm == 0 && bn == 0 && M <= 64 && ((int64_t)K * dtype_bytes(in_dt)) % 64 == 0) {
@@ -399,6 +400,7 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
                         ((major_flags & kGemmBMajorN) ? kGemmAMajorM : 0);
         if (rows_in_16_byte_pieces(g.C, g.ldc_m, g.ldc_n, D.dtype)) g.xcd_swizzle |= kGemmRowC;
         if (operand_rows_in_16_byte_pieces(g)) g.xcd_swizzle |= kGemmEpiRowX;
+        if (g.ep_op == MOYE_MAP_ADD && (!g.ep_x || g.ep_xm == 0 || g.ep_xn == 0)) g.xcd_swizzle |= kGemmEpiAddVec;
         return gemm_mfma_tn_dispatch(in_dt, D.dtype, bn, bm, bk, waves, mma->stages, g, st);
     }
     return fail(MOYE_ERR_UNSUPPORTED, "gemm!: D needs a unit stride along M or N");

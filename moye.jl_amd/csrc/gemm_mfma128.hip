@@ -11,15 +11,15 @@
 
 namespace moye {
 
-template <typename In, typename Out, bool kOps = false, bool kRagged = false, int AMAJ = 0, int BMAJ = 0>
+template <typename In, typename Out, bool kOps = false, bool kRagged = false, int AMAJ = 0, int BMAJ = 0, bool kBias = false>
 __global__ __launch_bounds__(256, 2) void gemm_mfma_tn_128(GemmArgs p) {
-    gemm_mfma_tn_lds_tile<In, Out, 128, 128, 2, 2, kOps, AMAJ, BMAJ, kRagged>(p);
+    gemm_mfma_tn_lds_tile<In, Out, 128, 128, 2, 2, kOps, AMAJ, BMAJ, kRagged, kBias>(p);
 }
 
-template <typename In, typename Out, bool kOps, bool kRagged, int AMAJ = 0, int BMAJ = 0>
+template <typename In, typename Out, bool kOps, bool kRagged, int AMAJ = 0, int BMAJ = 0, bool kBias = false>
 static int32_t launch128_instance(const GemmArgs& a, hipStream_t st) {
     constexpr int kLds = 2 * (128 + 128) * 128;  // two operand stages, 64 KiB
-    auto kern = gemm_mfma_tn_128<In, Out, kOps, kRagged, AMAJ, BMAJ>;
+    auto kern = gemm_mfma_tn_128<In, Out, kOps, kRagged, AMAJ, BMAJ, kBias>;
     static LdsCap cap;
     if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
     kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1)), dim3(256), kLds, st>>>(a);
@@ -44,6 +44,7 @@ static int32_t launch128(const GemmArgs& a, hipStream_t st) {
     }
     if (a.xcd_swizzle & kGemmRagged)
         return a.ep_op != MOYE_MAP_IDENTITY ? launch128_instance<In, Out, true, true>(a, st) : launch128_instance<In, Out, false, true>(a, st);
+    if (a.xcd_swizzle & kGemmEpiAddVec) return launch128_instance<In, Out, false, false, 0, 0, true>(a, st);  // a bias
     if (a.ep_op != MOYE_MAP_IDENTITY) return launch128_instance<In, Out, true, false>(a, st);
     return launch128_instance<In, Out, false, false>(a, st);
 }

@@ -13,9 +13,9 @@
 
 namespace moye {
 // The kernel body lives in gemm_mfma_lds_tile.hpp (kOps, AMAJ / BMAJ, kRagged are described there).
-template <typename In, typename Out, int WGM, int WGN, bool kOps = false, int AMAJ = 0, int BMAJ = 0, bool kRagged = false>
+template <typename In, typename Out, int WGM, int WGN, bool kOps = false, int AMAJ = 0, int BMAJ = 0, bool kRagged = false, bool kBias = false>
 __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256(GemmArgs p) {
-    gemm_mfma_tn_lds_tile<In, Out, 256, 256, WGM, WGN, kOps, AMAJ, BMAJ, kRagged>(p);
+    gemm_mfma_tn_lds_tile<In, Out, 256, 256, WGM, WGN, kOps, AMAJ, BMAJ, kRagged, kBias>(p);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -145,10 +145,10 @@ static int32_t launch256_ring(const GemmArgs& a, hipStream_t st) {
     return MOYE_OK;
 }
 
-template <typename In, typename Out, int WGM, int WGN, bool kOps, int AMAJ, int BMAJ, bool kRagged = false>
+template <typename In, typename Out, int WGM, int WGN, bool kOps, int AMAJ, int BMAJ, bool kRagged = false, bool kBias = false>
 static int32_t launch256_instance(const GemmArgs& a, hipStream_t st) {
     constexpr int kLds = 2 * (256 + 256) * 128;  // two operand stages, 128 KiB
-    auto kern = gemm_mfma_tn_256<In, Out, WGM, WGN, kOps, AMAJ, BMAJ, kRagged>;
+    auto kern = gemm_mfma_tn_256<In, Out, WGM, WGN, kOps, AMAJ, BMAJ, kRagged, kBias>;
     static LdsCap cap;
     if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
     kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1)), dim3(64 * WGM * WGN), kLds, st>>>(a);
@@ -179,7 +179,10 @@ static int32_t launch256(const GemmArgs& a, hipStream_t st) {
             return fail(MOYE_ERR_UNSUPPORTED, "gemm!: operands that are not K-major run natively with 16-bit types on eight waves only");
         }
     }
-    if constexpr (WGM * WGN == 8) if (a.ep_op != MOYE_MAP_IDENTITY) return launch256_instance<In, Out, WGM, WGN, true, 0, 0>(a, st);
+    if constexpr (WGM * WGN == 8) {
+        if (a.xcd_swizzle & kGemmEpiAddVec) return launch256_instance<In, Out, WGM, WGN, false, 0, 0, false, true>(a, st);  // a bias
+        if (a.ep_op != MOYE_MAP_IDENTITY) return launch256_instance<In, Out, WGM, WGN, true, 0, 0>(a, st);
+    }
     return launch256_instance<In, Out, WGM, WGN, false, 0, 0>(a, st);
 }
 

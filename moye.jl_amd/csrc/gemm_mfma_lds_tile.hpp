@@ -43,9 +43,13 @@ namespace moye {
 // what is computed from it is never stored; in the last k-tile a lane whose 16-byte piece lies beyond K reads the
 // row's first piece instead and every fragment piece beyond K is zeroed in registers before it reaches an MFMA; the
 // epilogues run with their row and column guards.
-template <typename In, typename Out, int BM, int BN, int WGM, int WGN, bool kOps, int AMAJ, int BMAJ, bool kRagged>
+//
+// kBias: the call adds a vector (one value per column or per row) or a scalar to the product -- a bias: an instance of
+// its own that is the plain kernel with that addition in the lanes' own epilogue, nothing of the general one.
+template <typename In, typename Out, int BM, int BN, int WGM, int WGN, bool kOps, int AMAJ, int BMAJ, bool kRagged, bool kBias = false>
 __device__ __forceinline__ void gemm_mfma_tn_lds_tile(GemmArgs p) {
     static_assert(!kRagged || (!AMAJ && !BMAJ), "ragged tiles: K-major operands");
+    static_assert(!kBias || (!kOps && !kRagged && !AMAJ && !BMAJ), "the bias instance: whole tiles, K-major operands");
     static_assert((BM == 256 && BN == 256) || (BM == 128 && BN == 128 && WGM == 2 && WGN == 2), "tile shapes");
     constexpr int CPR = 8;  // 8 chunks of 16 bytes per tile row
     constexpr int A_CH = BM * CPR, B_CH = BN * CPR, STAGE = A_CH + B_CH;
@@ -298,7 +302,8 @@ __device__ __forceinline__ void gemm_mfma_tn_lds_tile(GemmArgs p) {
     static_assert(NWAVES * 32 * WN * 4 <= 2 * STAGE * 16, "C patches (32 rows per wave and pass) fit in the operand stages");
     // (a kOps instance is only launched for calls with an operation or with ragged tiles: it carries the general
     // epilogue alone, which keeps the other one's registers out of its allocation)
-    if constexpr (kOps) store_c_tile_general<Out, MI, NI, kRagged>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
+    if constexpr (kBias) store_c_tile<Out, MI, NI, false, false, true>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
+    else if constexpr (kOps) store_c_tile_general<Out, MI, NI, kRagged>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
     else store_c_tile<Out, MI, NI, false, kRagged>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
 }
 

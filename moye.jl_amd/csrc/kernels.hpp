@@ -36,6 +36,7 @@ constexpr int kGemmAMajorM = 0x100000;  // in GemmArgs::xcd_swizzle: A has its u
 constexpr int kGemmBMajorN = 0x200000;  // the same for B and N (the 256 x 256 kernel's transposing fragment reads; 16-bit types)
 constexpr int kGemmEpiRowX = 0x400000;  // in GemmArgs::xcd_swizzle: the epilogue operand has unit stride along n and 16-byte aligned rows (or one row)
 constexpr int kGemmRagged = 0x800000;   // in GemmArgs::xcd_swizzle: the 256 x 256 kernel runs with tiles that reach beyond M, N or K (its guarded instance)
+constexpr int kGemmEpiAddVec = 0x1000000;  // in GemmArgs::xcd_swizzle: the epilogue operation adds a one-per-column or one-per-row vector or a scalar
 constexpr int kGemmRotateK = 0x20000;  // in GemmArgs::xcd_swizzle: each XCD starts its walk over K at its own eighth
 
 // UniversalFMA GEMM, any strides (gemm_universal.hip)

@@ -145,7 +145,10 @@ __device__ __forceinline__ void store_c_tile_general(const GemmArgs& p, const f3
 // inline-assembly MFMAs must not change with what the epilogue needs; the host never sends it such a call).
 // kGuard: the tile may reach beyond M or N and D need not be 16-byte aligned: nothing is read or stored beyond them, a
 // piece of D that crosses N or does not start on a 16-byte boundary goes out element by element.
-template <typename Out, int MI, int NI, bool kWithOps = true, bool kGuard = false>
+// kAddVec: the call adds a vector or a scalar (GemmArgs::ep_op == MOYE_MAP_ADD with a one-per-column, one-per-row or
+// scalar operand: a bias): the lanes add it to their own accumulators here, with the same roundings as the general
+// epilogue, instead of sending the tile through it.
+template <typename Out, int MI, int NI, bool kWithOps = true, bool kGuard = false, bool kAddVec = false>
 __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&acc)[MI][NI], u32x4* smem, int wave,
                                              int lane, int64_t m_base, int64_t n_base) {
     typedef typename Out::type OutT;
@@ -187,6 +190,15 @@ __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&ac
 #pragma unroll
         for (int a = 0; a < AHEAD; ++a) fetch_c(a, cw[a]);
     }
+    // a lane's columns are n_base + 16 j + 4 kq + 0..3: the operand values of a one-per-column vector, once for all rows
+    [[maybe_unused]] f32x4 xcol[kAddVec ? NI : 1];
+    [[maybe_unused]] const bool per_row = kAddVec && p.ep_x && p.ep_xn == 0;
+    if constexpr (kAddVec) {
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) xcol[j][e] = per_row ? 0.f : epi_operand(p, 0, n_base + 16 * j + 4 * (lane >> 4) + e);
+    }
 #pragma unroll
     for (int i0 = 0; i0 < MI; i0 += PASS_MI) {
         if (row_c) {
@@ -224,6 +236,11 @@ __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&ac
                 if (p.C) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) v[e] = __fadd_rn(v[e], __fmul_rn(p.beta, c[e]));
+                }
+                if constexpr (kAddVec) {
+                    const float xrow = per_row ? epi_operand(p, m, 0) : 0.f;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = __fadd_rn(v[e], per_row ? xrow : xcol[j][e]);
                 }
 #pragma unroll
                 for (int e = 0; e < 4; ++e) dst[e] = Out::cvt(v[e]);

@@ -522,48 +522,27 @@ __global__ __launch_bounds__(256) void copy_generic_cvt(const char* __restrict__
     }
 }
 
-// Converting copy between two dense, 16-byte aligned runs: a lane converts E = 16 / min(sizeof) elements per step, so
-// that the narrower side moves 16 bytes per access and the wider side a whole number of 16-byte accesses; two steps
-// of a lane are in flight.  Used where the destination is the narrower side (or as wide).  Element by element the same
-// conversion as copy_generic_cvt.
+// Converting copy between two dense, 16-byte aligned runs of elements of one width (fp16 <-> bf16): a lane converts the
+// elements of one 16-byte piece; one workgroup per 256 pieces, no loop.  Element by element the same conversion as
+// copy_generic_cvt.
 template <int kSrc, int kDst, int SB, int DB>
-__global__ __launch_bounds__(256) void copy_cvt_dense(const char* __restrict__ src, char* __restrict__ dst, int64_t nsteps) {
-    constexpr int E = 16 / (SB < DB ? SB : DB), SV = E * SB / 16, DV = E * DB / 16, U = 2;
+__global__ __launch_bounds__(256) void copy_cvt_dense(const char* __restrict__ src, char* __restrict__ dst, int64_t nvec) {
+    static_assert(SB == DB, "the widening and narrowing directions have kernels of their own");
+    constexpr int E = 16 / SB;
     const u32x4* sv = reinterpret_cast<const u32x4*>(src);
     u32x4* dv = reinterpret_cast<u32x4*>(dst);
-    auto convert = [](const u32x4 (&in)[SV], u32x4 (&out)[DV]) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= nvec) return;
+    const u32x4 in = __builtin_nontemporal_load(sv + i);
+    u32x4 out;
 #pragma unroll
-        for (int k = 0; k < E; ++k) {
-            char e_in[SB], e_out[DB];
-            __builtin_memcpy(e_in, reinterpret_cast<const char*>(in) + k * SB, SB);
-            store_from<kDst>(e_out, load_as_f64<kSrc>(e_in), kSrc == MOYE_F64);
-            __builtin_memcpy(reinterpret_cast<char*>(out) + k * DB, e_out, DB);
-        }
-    };
-    const int64_t stride = (int64_t)gridDim.x * 256 * U;
-    int64_t i = (int64_t)blockIdx.x * 256 * U + threadIdx.x;
-    for (; i + 256 * (U - 1) < nsteps; i += stride) {
-        u32x4 in[U][SV], out[U][DV];
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-#pragma unroll
-            for (int q = 0; q < SV; ++q) in[u][q] = __builtin_nontemporal_load(sv + (i + 256 * u) * SV + q);
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            convert(in[u], out[u]);
-#pragma unroll
-            for (int q = 0; q < DV; ++q) __builtin_nontemporal_store(out[u][q], dv + (i + 256 * u) * DV + q);
-        }
+    for (int k = 0; k < E; ++k) {
+        char e_in[SB], e_out[DB];
+        __builtin_memcpy(e_in, reinterpret_cast<const char*>(&in) + k * SB, SB);
+        store_from<kDst>(e_out, load_as_f64<kSrc>(e_in), kSrc == MOYE_F64);
+        __builtin_memcpy(reinterpret_cast<char*>(&out) + k * DB, e_out, DB);
     }
-    for (; i < nsteps; i += 256) {  // the last, partial group of this lane's stride
-        if (i >= nsteps) break;
-        u32x4 in[SV], out[DV];
-#pragma unroll
-        for (int q = 0; q < SV; ++q) in[q] = sv[i * SV + q];
-        convert(in, out);
-#pragma unroll
-        for (int q = 0; q < DV; ++q) dv[i * DV + q] = out[q];
-    }
+    __builtin_nontemporal_store(out, dv + i);
 }
 
 static FlatLayout flat_of(const moye_tensor& t) {
@@ -588,6 +567,15 @@ static bool is_contiguous(const moye_tensor& t) {
     return true;
 }
 
+// Are both one dense run in the same order: as written, or once the modes of both are ordered by stride (two row-major
+// arrays of one shape: a copy may visit the elements in any order)?
+static bool one_run_each(const moye_tensor& src, const moye_tensor& dst) {
+    if (is_contiguous(src) && is_contiguous(dst)) return true;
+    moye_tensor ts = src, td = dst;
+    moye_tensor* both[2] = {&td, &ts};
+    return order_modes_by_stride(both, 2) && is_contiguous(ts) && is_contiguous(td);
+}
+
 // The widening direction: a lane's 16-byte store holds EW = 16 / sizeof(dst) elements, which it reads as one access of
 // EW * sizeof(src) bytes (8, 4 or 2), so that loads and stores of a wave are both contiguous; four of them in flight.
 template <int NB> struct NarrowWord;
@@ -596,7 +584,7 @@ template <> struct NarrowWord<4> { typedef uint32_t type; };
 template <> struct NarrowWord<2> { typedef uint16_t type; };
 template <int kSrc, int kDst, int SB, int DB>
 __global__ __launch_bounds__(256) void copy_cvt_dense_widen(const char* __restrict__ src, char* __restrict__ dst, int64_t nvec) {
-    constexpr int EW = 16 / DB, NB = EW * SB, U = 4;
+    constexpr int EW = 16 / DB, NB = EW * SB;
     typedef typename NarrowWord<NB>::type word;
     const word* sv = reinterpret_cast<const word*>(src);
     u32x4* dv = reinterpret_cast<u32x4*>(dst);
@@ -611,24 +599,16 @@ __global__ __launch_bounds__(256) void copy_cvt_dense_widen(const char* __restri
         }
         return out;
     };
-    const int64_t chunks = nvec / (256 * U);
-    for (int64_t c = blockIdx.x; c < chunks; c += gridDim.x) {
-        const int64_t base = c * 256 * U + threadIdx.x;
-        word in[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) in[u] = __builtin_nontemporal_load(sv + base + u * 256);
-#pragma unroll
-        for (int u = 0; u < U; ++u) __builtin_nontemporal_store(convert(in[u]), dv + base + u * 256);
-    }
-    for (int64_t i = chunks * 256 * U + (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256)
-        dv[i] = convert(sv[i]);
+    // one piece per lane, one workgroup per 256 pieces, no loop (the form that is fastest for the plain copy)
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < nvec) __builtin_nontemporal_store(convert(__builtin_nontemporal_load(sv + i)), dv + i);
 }
 
-// The narrowing direction when the source is at least four times as wide: a lane reads 16 bytes and stores the
-// EN = 16 / sizeof(src) converted elements as one access of 2, 4 or 8 bytes; loads and stores of a wave are contiguous.
+// The narrowing direction: a lane reads 16 bytes and stores the EN = 16 / sizeof(src) converted elements as one access of
+// 2, 4 or 8 bytes; loads and stores of a wave are contiguous.
 template <int kSrc, int kDst, int SB, int DB>
 __global__ __launch_bounds__(256) void copy_cvt_dense_narrow(const char* __restrict__ src, char* __restrict__ dst, int64_t nvec) {
-    constexpr int EN = 16 / SB, NB = EN * DB, U = 4;
+    constexpr int EN = 16 / SB, NB = EN * DB;
     typedef typename NarrowWord<NB>::type word;
     const u32x4* sv = reinterpret_cast<const u32x4*>(src);
     word* dv = reinterpret_cast<word*>(dst);
@@ -643,17 +623,8 @@ __global__ __launch_bounds__(256) void copy_cvt_dense_narrow(const char* __restr
         }
         return out;
     };
-    const int64_t chunks = nvec / (256 * U);
-    for (int64_t c = blockIdx.x; c < chunks; c += gridDim.x) {
-        const int64_t base = c * 256 * U + threadIdx.x;
-        u32x4 in[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) in[u] = __builtin_nontemporal_load(sv + base + u * 256);
-#pragma unroll
-        for (int u = 0; u < U; ++u) dv[base + u * 256] = convert(in[u]);
-    }
-    for (int64_t i = chunks * 256 * U + (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256)
-        dv[i] = convert(sv[i]);
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < nvec) __builtin_nontemporal_store(convert(__builtin_nontemporal_load(sv + i)), dv + i);
 }
 
 constexpr int float_bytes(int dt) { return dt == MOYE_F64 ? 8 : dt == MOYE_F32 ? 4 : dt == MOYE_F8E4M3 ? 1 : 2; }
@@ -666,23 +637,27 @@ static int64_t launch_cvt_dense_pair(const char* s, char* d, int64_t n, hipStrea
         constexpr int EW = 16 / DB;
         const int64_t nvec = n / EW;
         if (nvec == 0) return 0;
-        const unsigned blocks = (unsigned)std::min<int64_t>((nvec + 1023) / 1024, 256 * 32);
+        const unsigned blocks = (unsigned)((nvec + 255) / 256);
         copy_cvt_dense_widen<kSrc, kDst, SB, DB><<<blocks, 256, 0, st>>>(s, d, nvec);
         return nvec * EW;
     }
-    if constexpr (SB >= 4 * DB && (16 / SB) * DB >= 2) {
+    if constexpr (SB > DB) {
+        static_assert((16 / SB) * DB >= 2, "a lane's store is 2, 4 or 8 bytes");
         constexpr int EN = 16 / SB;
         const int64_t nvec = n / EN;
         if (nvec == 0) return 0;
-        const unsigned blocks = (unsigned)std::min<int64_t>((nvec + 1023) / 1024, 256 * 32);
+        const unsigned blocks = (unsigned)((nvec + 255) / 256);
         copy_cvt_dense_narrow<kSrc, kDst, SB, DB><<<blocks, 256, 0, st>>>(s, d, nvec);
         return nvec * EN;
     }
-    const int64_t nsteps = n / E;
-    if (nsteps == 0) return 0;
-    const unsigned blocks = (unsigned)std::min<int64_t>((nsteps + 511) / 512, 256 * 16);
-    copy_cvt_dense<kSrc, kDst, SB, DB><<<blocks, 256, 0, st>>>(s, d, nsteps);
-    return nsteps * E;
+    if constexpr (SB == DB) {
+        const int64_t nvec = n / E;
+        if (nvec == 0) return 0;
+        const unsigned blocks = (unsigned)((nvec + 255) / 256);
+        copy_cvt_dense<kSrc, kDst, SB, DB><<<blocks, 256, 0, st>>>(s, d, nvec);
+        return nvec * E;
+    }
+    return 0;
 }
 template <int kSrc>
 static int64_t launch_cvt_dense_dst(int32_t dd, const char* s, char* d, int64_t n, hipStream_t st) {
@@ -763,15 +738,8 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
     char* d = static_cast<char*>(dst->ptr);
 
     if (same_bits && !mask) {
-        // (1) both sides one dense run in the same order: as written, or once the modes of both are ordered by stride (two
-        // row-major arrays of one shape: a copy may visit the elements in any order)
-        bool one_run = is_contiguous(*src) && is_contiguous(*dst);
-        if (!one_run) {
-            moye_tensor ts = *src, td = *dst;
-            moye_tensor* both[2] = {&td, &ts};
-            one_run = order_modes_by_stride(both, 2) && is_contiguous(ts) && is_contiguous(td);
-        }
-        if (one_run) {
+        // (1) both sides one dense run in the same order
+        if (one_run_each(*src, *dst)) {
             const int64_t bytes = n * sb;
             if (bytes % 16 == 0 && (reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d)) % 16 == 0) {
                 const int64_t n16 = bytes / 16;
@@ -972,7 +940,7 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
                 for (int m = 1; m < MOYE_MAX_RANK; ++m) l->stride[m] /= width;
             }
             const int64_t nv = n / width;
-            const dim3 gv((unsigned)std::min<int64_t>((nv + 255) / 256, 256 * 64));
+            const dim3 gv((unsigned)std::min<int64_t>((nv + 255) / 256, 0x7fffffff));  // one piece per lane
             switch (sb * width) {
                 case 2: copy_generic_bits<2><<<gv, 256, 0, st>>>(s, d, ls, ld, nv, Mask{}); break;
                 case 4: copy_generic_bits<4><<<gv, 256, 0, st>>>(s, d, ls, ld, nv, Mask{}); break;
@@ -983,7 +951,7 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
             return MOYE_OK;
         }
     }
-    if (!same_bits && !mask && is_contiguous(*src) && is_contiguous(*dst) &&
+    if (!same_bits && !mask && one_run_each(*src, *dst) &&
         (reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d)) % 16 == 0) {
         // both sides one aligned run: 16-byte accesses for all whole groups, the general kernel for what is left
         const int64_t done = launch_cvt_dense(src->dtype, dst->dtype, s, d, n, st);

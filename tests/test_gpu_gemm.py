@@ -1270,6 +1270,60 @@ def test_gemm_ex_takes_the_callers_workspace(mh):
     assert torch.equal(e1.cpu().double(), ref)
 
 
+def test_host_threads_with_their_own_streams_and_workspaces(mh):
+    """Four host threads call the library at the same time (ctypes drops the interpreter lock during a call), each on its
+    own stream with its own workspace: split-K partials, K-major copies of an M-major operand, a ragged problem, a
+    transposing copy and an axpby!.  Every thread's results are exact on small integers, every time."""
+    import threading
+    M, N, K = 256, 384, 2048
+    mma = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 2, 1), cta_tile=(128, 128, 32), split_k=4)
+    lib_choice = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16)
+    errors = []
+
+    def work(seed):
+        try:
+            g = torch.Generator().manual_seed(seed)
+            A = torch.randint(-4, 5, (M, K), generator=g).to(torch.float16)
+            B = torch.randint(-4, 5, (N, K), generator=g).to(torch.float16)
+            Ar = torch.randint(-4, 5, (300, 520), generator=g).to(torch.float16)
+            Br = torch.randint(-4, 5, (1000, 520), generator=g).to(torch.float16)
+            S = torch.randint(-1000, 1000, (512, 1024), generator=g, dtype=torch.int32)
+            ref, ref_r = A.double() @ B.double().t(), Ar.double() @ Br.double().t()
+            st = torch.cuda.Stream()
+            with torch.cuda.stream(st):
+                a_m, b, ar, br, src = A.t().contiguous().cuda(), B.cuda(), Ar.cuda(), Br.cuda(), S.cuda()
+                d, dr = torch.zeros(M, N, device="cuda"), torch.zeros(300, 1000, device="cuda")
+                dst = torch.zeros(1024, 512, dtype=torch.int32, device="cuda")
+                y = torch.ones(M, N, device="cuda")
+                ta_m = T(a_m, (M, K), (1, M))
+                need = mh.gemm_workspace_size(mma, T(d), ta_m, T(b))
+                ws = torch.zeros(need + 256, dtype=torch.uint8, device="cuda")
+                base = (ws.data_ptr() + 255) // 256 * 256
+            st.synchronize()
+            for it in range(12):
+                mh.gemm_ex_(mma, T(d), ta_m, T(b), None, None, base, need, stream=st.cuda_stream)
+                mh.gemm_ex_(lib_choice, T(dr), T(ar), T(br), stream=st.cuda_stream)
+                mh.copyto_(T(dst, (512, 1024), (1, 512)), T(src), stream=st.cuda_stream)
+                mh.axpby_(1.0, T(d), 0.0, T(y), stream=st.cuda_stream)
+                st.synchronize()
+                if not (torch.equal(d.cpu().double(), ref) and torch.equal(dr.cpu().double(), ref_r)
+                        and torch.equal(dst.cpu(), S.t()) and torch.equal(y.cpu().double(), ref)):
+                    errors.append("thread %d, pass %d: wrong result" % (seed, it))
+                    return
+                d.zero_(), dr.zero_(), dst.zero_(), y.fill_(1.0)
+                st.synchronize()
+        except Exception as e:  # noqa: BLE001 - reported below, in the test's own thread
+            errors.append("thread %d: %r" % (seed, e))
+
+    threads = [threading.Thread(target=work, args=(100 + i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
+
+
 # ---------------------------------------------------------------------------------------------
 # exactly what bench.py times, at the size it times
 # ---------------------------------------------------------------------------------------------

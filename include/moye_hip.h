@@ -90,8 +90,9 @@ typedef struct {
                                       into fp32 partial products in the library's workspace and
                                       summed in ascending order by a second kernel (results do not
                                       depend on timing); MFMA atoms only.  < 0 = the library
-                                      chooses: no split unless the problem's tiles fill less than
-                                      half the chip and K is long                                */
+                                      chooses: no split unless the problem's tiles (for M <= 64:
+                                      its workgroups of 16 columns) fill less than half the chip
+                                      and K is long                                              */
     int32_t flags;                 /* MOYE_GEMM_* bits                                          */
 } moye_tiled_mma;
 

@@ -559,6 +559,25 @@ def test_short_m_any_m_and_n(mh, M):
         assert torch.equal(dt_.t().cpu().double(), ref), (M, N, K, "column-major D")
 
 
+def test_short_m_small_n_long_k_takes_k_ranges(mh):
+    """With split_k < 0 the library cuts K into ranges for a short-M problem whose N is small and K long (its workgroups of
+    16 columns would leave most CUs idle): the workspace it asks for tells how many; none when N fills the chip or K is
+    short.  Results exact on small integers either way, the same bits as unsplit (integers: every order of the sum)."""
+    g = torch.Generator().manual_seed(41)
+    for (M, N, K, ranges) in ((16, 1024, 32768, 4), (16, 2048, 16384, 2), (32, 1024, 8192, 4), (64, 2048, 8192, 2), (16, 1000, 32768, 4),
+                              (16, 8192, 8192, 1), (16, 2048, 4096, 1), (16, 4096, 8192, 1), (16, 1024, 2048, 1)):
+        A = torch.randint(-2, 3, (M, K), generator=g).to(torch.bfloat16)
+        B = torch.randint(-2, 3, (N, K), generator=g).to(torch.bfloat16)
+        a, b = A.cuda(), B.cuda()
+        d = torch.zeros(M, N, device="cuda")
+        mma = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_BF16, split_k=-1)
+        need = mh.gemm_workspace_size(mma, T(d), T(a), T(b))
+        assert need == (ranges * M * N * 4 if ranges > 1 else 0), (M, N, K, need)
+        mh.gemm_(mma, T(d), T(a), T(b))
+        torch.cuda.synchronize()
+        assert torch.equal(d.cpu().double(), A.double() @ B.double().t()), (M, N, K)
+
+
 @pytest.mark.parametrize("M", [1, 16, 17, 48, 64])
 def test_short_m_line_staging_kernel(mh, M):
     """K of whole 128-byte lines runs on the kernel that stages them through LDS: any M <= 64 and any N (16 and

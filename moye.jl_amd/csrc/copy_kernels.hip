@@ -398,7 +398,7 @@ static int32_t launch_transpose8(const uint8_t* s, uint8_t* d, int64_t lds_, int
 // or four pieces per lane and no loop, 4.3 with eight; 6.2 without the non-temporal hints).
 __global__ __launch_bounds__(256) void copy_flat_b128(const u32x4* __restrict__ src,
                                                       u32x4* __restrict__ dst, int64_t n16) {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t i = flat_piece();
     if (i < n16) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
 }
 
@@ -531,7 +531,7 @@ __global__ __launch_bounds__(256) void copy_cvt_dense(const char* __restrict__ s
     constexpr int E = 16 / SB;
     const u32x4* sv = reinterpret_cast<const u32x4*>(src);
     u32x4* dv = reinterpret_cast<u32x4*>(dst);
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t i = flat_piece();
     if (i >= nvec) return;
     const u32x4 in = __builtin_nontemporal_load(sv + i);
     u32x4 out;
@@ -600,7 +600,7 @@ __global__ __launch_bounds__(256) void copy_cvt_dense_widen(const char* __restri
         return out;
     };
     // one piece per lane, one workgroup per 256 pieces, no loop (the form that is fastest for the plain copy)
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t i = flat_piece();
     if (i < nvec) __builtin_nontemporal_store(convert(__builtin_nontemporal_load(sv + i)), dv + i);
 }
 
@@ -623,7 +623,7 @@ __global__ __launch_bounds__(256) void copy_cvt_dense_narrow(const char* __restr
         }
         return out;
     };
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t i = flat_piece();
     if (i < nvec) __builtin_nontemporal_store(convert(__builtin_nontemporal_load(sv + i)), dv + i);
 }
 
@@ -637,8 +637,7 @@ static int64_t launch_cvt_dense_pair(const char* s, char* d, int64_t n, hipStrea
         constexpr int EW = 16 / DB;
         const int64_t nvec = n / EW;
         if (nvec == 0) return 0;
-        const unsigned blocks = (unsigned)((nvec + 255) / 256);
-        copy_cvt_dense_widen<kSrc, kDst, SB, DB><<<blocks, 256, 0, st>>>(s, d, nvec);
+        copy_cvt_dense_widen<kSrc, kDst, SB, DB><<<flat_grid(nvec), 256, 0, st>>>(s, d, nvec);
         return nvec * EW;
     }
     if constexpr (SB > DB) {
@@ -646,15 +645,13 @@ static int64_t launch_cvt_dense_pair(const char* s, char* d, int64_t n, hipStrea
         constexpr int EN = 16 / SB;
         const int64_t nvec = n / EN;
         if (nvec == 0) return 0;
-        const unsigned blocks = (unsigned)((nvec + 255) / 256);
-        copy_cvt_dense_narrow<kSrc, kDst, SB, DB><<<blocks, 256, 0, st>>>(s, d, nvec);
+        copy_cvt_dense_narrow<kSrc, kDst, SB, DB><<<flat_grid(nvec), 256, 0, st>>>(s, d, nvec);
         return nvec * EN;
     }
     if constexpr (SB == DB) {
         const int64_t nvec = n / E;
         if (nvec == 0) return 0;
-        const unsigned blocks = (unsigned)((nvec + 255) / 256);
-        copy_cvt_dense<kSrc, kDst, SB, DB><<<blocks, 256, 0, st>>>(s, d, nvec);
+        copy_cvt_dense<kSrc, kDst, SB, DB><<<flat_grid(nvec), 256, 0, st>>>(s, d, nvec);
         return nvec * E;
     }
     return 0;
@@ -743,9 +740,7 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
             const int64_t bytes = n * sb;
             if (bytes % 16 == 0 && (reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d)) % 16 == 0) {
                 const int64_t n16 = bytes / 16;
-                if ((n16 + 255) / 256 > 0x7fffffff) return fail(MOYE_ERR_SHAPE, "copyto!: more than 8 TiB in one call");
-                const unsigned blocks = (unsigned)((n16 + 255) / 256);
-                copy_flat_b128<<<blocks, 256, 0, st>>>(reinterpret_cast<const u32x4*>(s), reinterpret_cast<u32x4*>(d), n16);
+                copy_flat_b128<<<flat_grid(n16), 256, 0, st>>>(reinterpret_cast<const u32x4*>(s), reinterpret_cast<u32x4*>(d), n16);
             } else {
                 const int blocks = (int)std::min<int64_t>((bytes + 255) / 256, 256 * 32);
                 copy_flat_bytes<<<blocks, 256, 0, st>>>(reinterpret_cast<const uint8_t*>(s), reinterpret_cast<uint8_t*>(d), bytes);
@@ -940,7 +935,7 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
                 for (int m = 1; m < MOYE_MAX_RANK; ++m) l->stride[m] /= width;
             }
             const int64_t nv = n / width;
-            const dim3 gv((unsigned)std::min<int64_t>((nv + 255) / 256, 0x7fffffff));  // one piece per lane
+            const dim3 gv = strided_grid(nv);  // one piece per lane up to 16 GiB of 16-byte pieces
             switch (sb * width) {
                 case 2: copy_generic_bits<2><<<gv, 256, 0, st>>>(s, d, ls, ld, nv, Mask{}); break;
                 case 4: copy_generic_bits<4><<<gv, 256, 0, st>>>(s, d, ls, ld, nv, Mask{}); break;

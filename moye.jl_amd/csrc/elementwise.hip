@@ -208,7 +208,7 @@ __global__ __launch_bounds__(256) void axpby_dense_kernel(typename El::compute a
         }
         return r;
     };
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t i = flat_piece();
     if (i >= nvec) return;
     const vec vx = __builtin_nontemporal_load(xv + i);
     __builtin_nontemporal_store(one(vx, b_is_zero ? vx : __builtin_nontemporal_load(yv + i)), yv + i);
@@ -236,7 +236,7 @@ __global__ __launch_bounds__(256) void map_dense_kernel(int32_t op, typename El:
         }
         return r;
     };
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t i = flat_piece();
     if (i >= nvec) return;
     // (d may be a or b: every lane reads its own piece before it writes it)
     const vec va = __builtin_nontemporal_load(av + i);
@@ -244,7 +244,7 @@ __global__ __launch_bounds__(256) void map_dense_kernel(int32_t op, typename El:
 }
 
 __global__ __launch_bounds__(256) void fill_dense_kernel(u32x4* x, int64_t nvec, u32x4 pattern) {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t i = flat_piece();
     if (i < nvec) x[i] = pattern;
 }
 
@@ -350,8 +350,7 @@ bool dense_l(const ELayout& l) {
     return true;
 }
 bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
-// one workgroup per 256 pieces of 16 bytes; a launch holds 2^31 - 1 workgroups, i.e. 8 TiB per operand
-dim3 dense_grid(int64_t nvec) { return dim3((unsigned)std::max<int64_t>(1, (nvec + 255) / 256)); }
+
 ELayout run_layout(int64_t n) {  // a rank-1 run of n elements: what is left of a dense array behind its last whole 16 bytes
     ELayout l{};
     l.rank = 1;
@@ -389,7 +388,7 @@ static void launch_axpby(typename El::compute a, const void* x, const ELayout& l
     const bool b0 = b == (typename El::compute)0;
     if (!is_dense && rows) {  // lx, ly are in 16-byte pieces
         const int64_t nvec = n / DenseVec<El>::N;
-        axpby_rows_kernel<El><<<dense_grid(nvec), 256, 0, st>>>(a, xs, lx, b, ys, ly, nvec, b0);
+        axpby_rows_kernel<El><<<strided_grid(nvec), 256, 0, st>>>(a, xs, lx, b, ys, ly, nvec, b0);
         return;
     }
     if (!is_dense) {
@@ -399,7 +398,7 @@ static void launch_axpby(typename El::compute a, const void* x, const ELayout& l
     }
     constexpr int N = DenseVec<El>::N;
     const int64_t nvec = n / N, tail = n - nvec * N;
-    if (nvec) axpby_dense_kernel<El><<<dense_grid(nvec), 256, 0, st>>>(a, xs, b, ys, nvec, b0);
+    if (nvec) axpby_dense_kernel<El><<<flat_grid(nvec), 256, 0, st>>>(a, xs, b, ys, nvec, b0);
     if (tail) axpby_kernel<El><<<1, 64, 0, st>>>(a, xs + nvec * N, run_layout(tail), b, ys + nvec * N, run_layout(tail), tail, b0);
 }
 
@@ -412,7 +411,7 @@ static void launch_map(int32_t op, void* d, const ELayout& ld, const void* a, co
     const S* bs = static_cast<const S*>(b);
     if (!is_dense && rows) {  // ld, la, lb are in 16-byte pieces
         const int64_t nvec = n / DenseVec<El>::N;
-        map_rows_kernel<El><<<dense_grid(nvec), 256, 0, st>>>(op, ds, ld, as, la, bs, lb, s, nvec);
+        map_rows_kernel<El><<<strided_grid(nvec), 256, 0, st>>>(op, ds, ld, as, la, bs, lb, s, nvec);
         return;
     }
     if (!is_dense) {
@@ -422,7 +421,7 @@ static void launch_map(int32_t op, void* d, const ELayout& ld, const void* a, co
     }
     constexpr int N = DenseVec<El>::N;
     const int64_t nvec = n / N, tail = n - nvec * N;
-    if (nvec) map_dense_kernel<El><<<dense_grid(nvec), 256, 0, st>>>(op, ds, as, bs, s, nvec);
+    if (nvec) map_dense_kernel<El><<<flat_grid(nvec), 256, 0, st>>>(op, ds, as, bs, s, nvec);
     if (tail)
         map_kernel<El><<<1, 64, 0, st>>>(op, ds + nvec * N, run_layout(tail), as + nvec * N, run_layout(tail), bs ? bs + nvec * N : nullptr,
                                          run_layout(tail), tail, s, tail);
@@ -538,7 +537,7 @@ int32_t fill_dispatch(const moye_tensor* X, double value, hipStream_t st) {
         for (int w = eb; w < 8; w *= 2) rep |= rep << (8 * w);
         const u32x4 pattern = {(uint32_t)rep, (uint32_t)(rep >> 32), (uint32_t)rep, (uint32_t)(rep >> 32)};
         const int64_t nvec = n * eb / 16, tail = n - nvec * (16 / eb);
-        if (nvec) fill_dense_kernel<<<dense_grid(nvec), 256, 0, st>>>(reinterpret_cast<u32x4*>(p), nvec, pattern);
+        if (nvec) fill_dense_kernel<<<flat_grid(nvec), 256, 0, st>>>(reinterpret_cast<u32x4*>(p), nvec, pattern);
         if (tail) {
             char* q = p + nvec * 16;
             switch (eb) {
@@ -560,7 +559,7 @@ int32_t fill_dispatch(const moye_tensor* X, double value, hipStream_t st) {
             for (int w = eb; w < 8; w *= 2) rep |= rep << (8 * w);
             const u32x4 pattern = {(uint32_t)rep, (uint32_t)(rep >> 32), (uint32_t)rep, (uint32_t)(rep >> 32)};
             const int64_t nvec = n / (16 / eb);
-            fill_rows_kernel<<<dense_grid(nvec), 256, 0, st>>>(reinterpret_cast<u32x4*>(p), lx, nvec, pattern);
+            fill_rows_kernel<<<strided_grid(nvec), 256, 0, st>>>(reinterpret_cast<u32x4*>(p), lx, nvec, pattern);
             MOYE_HIP_CHECK(hipGetLastError());
             return MOYE_OK;
         }

@@ -40,6 +40,23 @@ inline int32_t raise_lds_cap(LdsCap& cap, const void* kernel, int bytes) {
     return MOYE_OK;
 }
 
+// Kernels that give every lane one piece and do not loop.  A launch holds fewer than 2^32 work-items per grid dimension,
+// so from 2^22 workgroups of 256 on (16 GiB of 16-byte pieces) the rest of the workgroups go into the grid's second
+// dimension; the lanes past the last piece of the last row of workgroups find nothing to do.
+constexpr unsigned kFlatGridX = 1u << 22;
+inline dim3 flat_grid(int64_t pieces) {
+    const int64_t blocks = pieces > 0 ? (pieces + 255) / 256 : 1;
+    if (blocks <= (int64_t)kFlatGridX) return dim3((unsigned)blocks);
+    return dim3(kFlatGridX, (unsigned)((blocks + kFlatGridX - 1) / kFlatGridX));
+}
+#if defined(__HIPCC__)
+__device__ __forceinline__ int64_t flat_piece() { return ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * 256 + threadIdx.x; }
+#endif
+// Kernels whose lanes walk the pieces with a stride of the whole grid: as many workgroups as pieces, up to 2^22.
+inline dim3 strided_grid(int64_t pieces) {
+    return dim3((unsigned)std::min<int64_t>(std::max<int64_t>(1, (pieces + 255) / 256), (int64_t)kFlatGridX));
+}
+
 inline int dtype_bytes(int32_t dt) {
     switch (dt) {
         case MOYE_F32: case MOYE_U32: return 4;

@@ -764,3 +764,40 @@ def test_transpose_destination_rows_first_and_source_first_agree(mh):
     mh.copyto_(_tens(mh, dst, (ni, nj, 3), (nj, 1, ni * nj)), _tens(mh, src, (ni, nj, 3), (1, ni, ni * nj)))
     torch.cuda.synchronize()
     assert torch.equal(dst.view(3, ni, nj), src.view(3, nj, ni).transpose(1, 2))
+
+
+def test_more_than_16_gib_in_one_call(mh):
+    """Arrays of more than 2^30 16-byte pieces: the kernels that give every lane one piece then spread their workgroups
+    over two grid dimensions (a launch holds fewer than 2^32 work-items per dimension).  fill!, a plain copy, a
+    converting copy and axpby! on 17 GiB arrays; every byte checked on the device."""
+    free, _ = torch.cuda.mem_get_info()
+    if free < 60 * 2 ** 30:
+        pytest.skip("needs 60 GiB of free device memory")
+    cols = 1 << 20
+    rows = 17 * 256 + 3                                   # 17 GiB of int32 and a little more
+    n = rows * cols
+    x = torch.empty(n, dtype=torch.int32, device="cuda")
+    mh.fill_(_tens(mh, x, [n], [1]), 0x01020304)
+    torch.cuda.synchronize()
+    assert bool((x.view(rows, cols) == 0x01020304).all())
+    pat = torch.arange(cols, dtype=torch.int32, device="cuda")
+    for r0 in range(0, rows, 512):                        # row r holds (column index) * 3 + r
+        r1 = min(rows, r0 + 512)
+        x.view(rows, cols)[r0:r1] = pat[None, :] * 3 + torch.arange(r0, r1, dtype=torch.int32, device="cuda")[:, None]
+    y = torch.zeros(n, dtype=torch.int32, device="cuda")
+    mh.copyto_(_tens(mh, y, [n], [1]), _tens(mh, x, [n], [1]))
+    torch.cuda.synchronize()
+    assert torch.equal(x, y)
+    # axpby! on the same bytes as fp32 values (small integers, exact): y = 2 x + y
+    xf, yf = x.view(torch.float32), y.view(torch.float32)
+    xf.view(rows, cols)[:] = pat[None, :].float() % 1024
+    yf.view(rows, cols)[:] = 1.0
+    mh.axpby_(2.0, _tens(mh, xf, [n], [1]), 1.0, _tens(mh, yf, [n], [1]))
+    torch.cuda.synchronize()
+    assert bool((yf.view(rows, cols) == 2 * (pat[None, :].float() % 1024) + 1).all())
+    del y, yf
+    # a narrowing conversion: fp32 -> fp16, 2^30 and more pieces on the fp32 side
+    h = torch.zeros(n, dtype=torch.float16, device="cuda")
+    mh.copyto_(_tens(mh, h, [n], [1]), _tens(mh, xf, [n], [1]))
+    torch.cuda.synchronize()
+    assert bool((h.view(rows, cols) == (pat[None, :] % 1024).half()).all())

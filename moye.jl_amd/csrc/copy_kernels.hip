@@ -106,7 +106,7 @@ static int32_t launch_transpose(const uint32_t* s, uint32_t* d, int64_t lds_, in
         if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
     }
     const int64_t groups = (int64_t)(ti / GI) * tj;
-    if (groups > 0x7fffffff) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles");
+    if (groups >= (1 << 24)) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles for one launch (2^24 workgroups of 256)");
     // groups are walked with the source-contiguous index fastest in bands of 64 tile columns: the
     // workgroups in flight read whole source rows and write runs of several KiB per destination row
     kern<<<dim3((unsigned)groups, (unsigned)batch), 256, kLds, st>>>(s, d, lds_, ldd, ti / GI, tj, 64, bs_src, bs_dst);
@@ -169,7 +169,7 @@ static int32_t launch_transpose_rows(const uint32_t* s, uint32_t* d, int64_t lds
     static LdsCap cap;
     if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
     const int64_t groups = (int64_t)ti * (tj / GJ);
-    if (groups > 0x7fffffff) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles");
+    if (groups >= (1 << 24)) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles for one launch (2^24 workgroups of 256)");
     kern<<<dim3((unsigned)groups, (unsigned)batch), 256, kLds, st>>>(s, d, lds_, ldd, tj / GJ, bs_src, bs_dst);
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;
@@ -244,7 +244,7 @@ static int32_t launch_transpose16(const uint16_t* s, uint16_t* d, int64_t lds_, 
         if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
     }
     const int64_t groups = (int64_t)(ti / GI) * tj;
-    if (groups > 0x7fffffff) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles");
+    if (groups >= (1 << 24)) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles for one launch (2^24 workgroups of 256)");
     kern<<<dim3((unsigned)groups, (unsigned)batch), 256, kLds, st>>>(s, d, lds_, ldd, ti / GI, tj, 64, bs_src, bs_dst);
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;
@@ -309,7 +309,7 @@ static int32_t launch_transpose16_rows(const uint16_t* s, uint16_t* d, int64_t l
     static LdsCap cap;
     if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
     const int64_t groups = (int64_t)ti * (tj / GJ);
-    if (groups > 0x7fffffff) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles");
+    if (groups >= (1 << 24)) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles for one launch (2^24 workgroups of 256)");
     kern<<<dim3((unsigned)groups, (unsigned)batch), 256, kLds, st>>>(s, d, lds_, ldd, tj / GJ, bs_src, bs_dst);
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;
@@ -384,7 +384,7 @@ static int32_t launch_transpose8(const uint8_t* s, uint8_t* d, int64_t lds_, int
         if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
     }
     const int64_t groups = (int64_t)(ti / GI) * tj;
-    if (groups > 0x7fffffff) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles");
+    if (groups >= (1 << 24)) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles for one launch (2^24 workgroups of 256)");
     kern<<<dim3((unsigned)groups, (unsigned)batch), 256, kLds, st>>>(s, d, lds_, ldd, ti / GI, tj, 64, bs_src, bs_dst);
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;

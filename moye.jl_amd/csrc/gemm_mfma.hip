@@ -425,6 +425,16 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         // fp8 runs at twice the 16-bit rate only on the 16x16x128 MFMA, which the hand-ordered kernel issues
         if (in_dt == MOYE_F8E4M3 && bkb == 128 && stages < 3 && !(a.xcd_swizzle & MOYE_GEMM_PINGPONG) && a.ep_op == MOYE_MAP_IDENTITY)
             a.xcd_swizzle |= MOYE_GEMM_WAVE4;
+        // ... and for the 16-bit types its form with whole 128-byte rows in two stages is the fastest k-loop of this build
+        // for a plain call (fp16 4096^3 97.6-98.6 us against 101.3-102.0 for the compiler-scheduled kernel on the same
+        // box, bf16 8192^3 726 against 754); operations in the epilogue, ragged tiles, operands that are not K-major and
+        // fp32 operands stay with that kernel, and so does a call that asks for it: stages = 2 in the descriptor, or
+        // MOYE_GEMM_HAND_ORDERED=0 in the environment (read once).
+        static const bool hand_ordered_off = getenv("MOYE_GEMM_HAND_ORDERED") && atoi(getenv("MOYE_GEMM_HAND_ORDERED")) == 0;
+        if (!hand_ordered_off && eb == 2 && bkb == 128 && stages < 2 && a.ep_op == MOYE_MAP_IDENTITY &&
+            !(a.xcd_swizzle & (MOYE_GEMM_PINGPONG | kGemmRagged | kGemmAMajorM | kGemmBMajorN | kGemmEpiAddVec | kGemmAtom32)) &&
+            256 * a.lda * eb < ((int64_t)1 << 32) && 256 * a.ldb * eb < ((int64_t)1 << 32))
+            a.xcd_swizzle |= MOYE_GEMM_WAVE4;
         // hand-ordered kernel: k-steps of 64 bytes, or of 128 (fp8 always; the 16-bit types when the tile says so)
         const int w4_step = in_dt == MOYE_F8E4M3 || (bkb == 128 && eb == 2) ? 128 : 64;
         const int kmult = (a.xcd_swizzle & MOYE_GEMM_WAVE4) ? w4_step / eb
@@ -434,7 +444,7 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
                         a.M, a.N, a.K);
         if (misaligned)
             return fail(MOYE_ERR_ALIGN, "gemm!: operands of the MFMA kernels need 16-byte aligned pointers and row pitches");
-        if (a.xcd_swizzle & MOYE_GEMM_WAVE4) return gemm_mfma_tn_256_w4_dispatch(in_dt, out_dt, a, waves, w4_step, st);
+        if (a.xcd_swizzle & MOYE_GEMM_WAVE4) return gemm_mfma_tn_256_w4_dispatch(in_dt, out_dt, a, waves, w4_step, stages >= 3, st);
         if (a.xcd_swizzle & MOYE_GEMM_PINGPONG) return gemm_mfma_tn_256_pp_dispatch(in_dt, out_dt, a, st);
         return gemm_mfma_tn_256_dispatch(in_dt, out_dt, a, waves, stages, st);
     }

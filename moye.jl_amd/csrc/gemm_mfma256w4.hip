@@ -34,6 +34,7 @@
 // Operand conventions as in gemm_mfma256.hip: K-major A and B, N-contiguous D, the MFMA issued
 // with B rows as its first operand so a lane holds four consecutive n of one m; the 16-byte chunk
 // index of an LDS row is XORed with (row / 2) % 4, applied on the global side of the load-to-LDS.
+#include <cstdlib>
 #include <type_traits>
 #include <utility>
 
@@ -55,6 +56,10 @@ __device__ __forceinline__ void static_for(F&& f) {
 
 // The ND load-to-LDS instructions a wave issues per k-step go out evenly over the MFMA positions that
 // follow the barrier (positions 8 .. NPOS - 1).  Returns the index of the load issued after MFMA P, or -1.
+// With a ring of two stages the loads of a k-step must have landed by the next barrier: every other position from 8 on.
+// (measured at fp16 4096^3, eight / four waves: every position 100.4 / 101.0 us, every other 97.7-98.7 / 97.4-98.6, every third
+// 99.3 / 98.3; the barrier after MFMA 3, 5 or 11 instead of 7: 98.2, 99.9, 98.0 / 98.5, 99.4, 97.6)
+constexpr int dma_index_early(int P, int ND) { return P >= 8 && P < 8 + 2 * ND && (P - 8) % 2 == 0 ? (P - 8) / 2 : -1; }
 constexpr int dma_index(int P, int ND, int NPOS) {
     for (int k = 0; k < ND; ++k)
         if (8 + k * (NPOS - 8) / ND == P) return k;
@@ -78,15 +83,17 @@ __device__ __forceinline__ u32x4 lds_read16(uint32_t addr) {
     return v;
 }
 
-// fragment = what one lane feeds to one MFMA group per operand; SPS = ring stages per k-step
-struct W4F16 {
+// fragment = what one lane feeds to one MFMA group per operand; SPS = ring stages per k-step; kRow = bytes of K per row
+// of a stage, kRing = stages in the ring
+struct W4Ring64 { static constexpr int kRow = 64, kRing = 5; };
+struct W4F16 : W4Ring64 {
     static constexpr int kBytes = 2, SPS = 1;
     typedef u32x4 frag;
     static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) {
         asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
     }
 };
-struct W4BF16 {
+struct W4BF16 : W4Ring64 {
     static constexpr int kBytes = 2, SPS = 1;
     typedef u32x4 frag;
     static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) {
@@ -95,7 +102,7 @@ struct W4BF16 {
 };
 // The 16-bit types with k-steps of two stages (128 bytes of K): two MFMAs in a row on the same accumulator (which
 // costs nothing: 16.4 clocks per MFMA either way) and half as many barriers per K.
-struct W4F16x2 {
+struct W4F16x2 : W4Ring64 {
     static constexpr int kBytes = 2, SPS = 2;
     struct frag { u32x4 lo, hi; };
     static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) {
@@ -103,7 +110,7 @@ struct W4F16x2 {
                      : "+a"(c) : "v"(a.lo), "v"(a.hi), "v"(b.lo), "v"(b.hi));
     }
 };
-struct W4BF16x2 {
+struct W4BF16x2 : W4Ring64 {
     static constexpr int kBytes = 2, SPS = 2;
     struct frag { u32x4 lo, hi; };
     static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) {
@@ -113,7 +120,7 @@ struct W4BF16x2 {
 };
 // 32 bytes per lane: the chunk of stage 0 and the chunk of stage 1 of the k-step.  Which 32 of the
 // 128 k-values a lane carries does not matter as long as A and B agree, and they do.
-struct W4FP8 {
+struct W4FP8 : W4Ring64 {
     static constexpr int kBytes = 1, SPS = 2;
     struct frag { u32x4 lo, hi; };
     static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) {
@@ -122,8 +129,37 @@ struct W4FP8 {
         asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(a8), "v"(b8));
     }
 };
+// The same MFMA fed from whole 128-byte rows: a stage is a k-step (64 KiB), two stages make the ring (the fragments of
+// step s+1 are read out of one while the loads of step s+2 fill the other), a lane's 32 bytes are chunks kq and kq + 4
+// of its row.  A load-to-LDS instruction then reads eight whole 128-byte lines instead of sixteen half lines.
+struct W4FP8L {
+    static constexpr int kBytes = 1, SPS = 1, kRow = 128, kRing = 2;
+    struct frag { u32x4 lo, hi; };
+    static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) {
+        const u32x8 a8 = __builtin_shufflevector(a.lo, a.hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        const u32x8 b8 = __builtin_shufflevector(b.lo, b.hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(a8), "v"(b8));
+    }
+};
+// The 16-bit types on whole-line stages: chunk kq feeds the first MFMA of an accumulator, chunk kq + 4 the second.
+struct W4F16L {
+    static constexpr int kBytes = 2, SPS = 1, kRow = 128, kRing = 2;
+    struct frag { u32x4 lo, hi; };
+    static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) {
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %3, %0\n\tv_mfma_f32_16x16x32_f16 %0, %2, %4, %0"
+                     : "+a"(c) : "v"(a.lo), "v"(a.hi), "v"(b.lo), "v"(b.hi));
+    }
+};
+struct W4BF16L {
+    static constexpr int kBytes = 2, SPS = 1, kRow = 128, kRing = 2;
+    struct frag { u32x4 lo, hi; };
+    static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) {
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %3, %0\n\tv_mfma_f32_16x16x32_bf16 %0, %2, %4, %0"
+                     : "+a"(c) : "v"(a.lo), "v"(a.hi), "v"(b.lo), "v"(b.hi));
+    }
+};
 // element j of the chunk goes to MFMA j (see InF32)
-struct W4F32 {
+struct W4F32 : W4Ring64 {
     static constexpr int kBytes = 4, SPS = 1;
     typedef u32x4 frag;
     static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) {
@@ -140,11 +176,15 @@ struct W4F32 {
 // the barrier) leaves the matrix pipe to the other.
 template <typename In, typename Out, int WGN>
 __global__ __launch_bounds__(128 * WGN) void gemm_mfma_tn_256_w4(GemmArgs p) {
-    constexpr int BM = 256, BN = 256, CPR = 4, STAGES = 5, SPS = In::SPS;
+    constexpr int BM = 256, BN = 256, kRow = In::kRow, CPR = kRow / 16, STAGES = In::kRing, SPS = In::SPS;
+    constexpr bool kLine = kRow == 128;                        // a fragment is two chunks of one row of one stage
+    constexpr int RPF = kLine ? 2 : SPS;                       // LDS reads per fragment
+    constexpr int RPI = 64 / CPR;                              // rows one load-to-LDS instruction covers
+    static_assert(!kLine || (SPS == 1 && STAGES == 2), "whole-line stages: one per k-step, two in the ring");
     constexpr int STAGE = (BM + BN) * CPR;  // in 16-byte chunks
     constexpr int NW = 2 * WGN, WN = BN / WGN;
     constexpr int MI = 8, NI = WN / 16, NPOS = MI * NI;
-    constexpr int RW = BM / NW, LD = RW / 16;  // per wave and stage: RW rows, LD load-to-LDS instructions per operand
+    constexpr int RW = BM / NW, LD = RW / RPI;  // per wave and stage: RW rows, LD load-to-LDS instructions per operand
     typedef typename In::frag frag;
 
     extern __shared__ u32x4 smem[];
@@ -160,7 +200,7 @@ __global__ __launch_bounds__(128 * WGN) void gemm_mfma_tn_256_w4(GemmArgs p) {
     // LDS stage (32 KiB) = A tile (256 rows of 64 bytes) then B tile.  Lane l of a load-to-LDS
     // instruction lands in physical chunk l % 4 of row l / 4 of a 16-row group; wave w brings rows
     // RW w .. RW w + RW - 1 of each operand.
-    const int lrow = wave * RW + (lane >> 2), lch = (lane & 3) ^ swz<CPR>(lane >> 2);
+    const int lrow = wave * RW + lane / CPR, lch = (lane % CPR) ^ swz<CPR>(lane / CPR);
     const char* const a_tile = static_cast<const char*>(p.A) + (int64_t)tm * BM * pitch_a;  // uniform
     const char* const b_tile = static_cast<const char*>(p.B) + (int64_t)tn * BN * pitch_b;
     constexpr uint32_t kStageBytes = STAGE * 16, kATileBytes = BM * CPR * 16;
@@ -171,7 +211,7 @@ __global__ __launch_bounds__(128 * WGN) void gemm_mfma_tn_256_w4(GemmArgs p) {
 #pragma unroll
         for (int j = 0; j < NI; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    const int nstages = (int)(((int64_t)p.K * In::kBytes) / 64);
+    const int nstages = (int)(((int64_t)p.K * In::kBytes) / kRow);
     const int nsteps = nstages / SPS;
     frag fa[MI], fb[NI];
 
@@ -184,16 +224,16 @@ __global__ __launch_bounds__(128 * WGN) void gemm_mfma_tn_256_w4(GemmArgs p) {
     uint32_t voff[2 * LD];
 #pragma unroll
     for (int q = 0; q < 2 * LD; ++q)
-        voff[q] = (uint32_t)((lrow + 16 * (q % LD)) * (q < LD ? pitch_a : pitch_b) + lch * 16);
+        voff[q] = (uint32_t)((lrow + RPI * (q % LD)) * (q < LD ? pitch_a : pitch_b) + lch * 16);
     // stage g of this workgroup's walk over K is stage g + g0 (mod nstages) of the operands: the eight XCDs start an
     // eighth of K apart when the caller asks for it (see gemm_mfma256.hip)
     const int g0 = (p.xcd_swizzle & kGemmRotateK) ? (int)((int64_t)(blockIdx.x % 8) * nsteps / 8) * SPS : 0;
     auto dma1 = [&](int g, int ring_slot, auto qc) __attribute__((always_inline)) {
         constexpr int Q = decltype(qc)::value;
         const int gr = g + g0 >= nstages ? g + g0 - nstages : g + g0;
-        const char* const base = uniform_ptr((Q < LD ? a_tile : b_tile) + (int64_t)gr * 64);
+        const char* const base = uniform_ptr((Q < LD ? a_tile : b_tile) + (int64_t)gr * kRow);
         const uint32_t dst = __builtin_amdgcn_readfirstlane(lds0 + ring_slot * kStageBytes + (Q < LD ? 0 : kATileBytes) +
-                                                            (uint32_t)(wave * RW + 16 * (Q % LD)) * 64);
+                                                            (uint32_t)(wave * RW + RPI * (Q % LD)) * kRow);
         const uint32_t lane_off = voff[Q];  // (a captured array element cannot be an asm operand of a generic lambda)
         asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(base), "s"(dst)
                      : "memory");
@@ -207,13 +247,18 @@ __global__ __launch_bounds__(128 * WGN) void gemm_mfma_tn_256_w4(GemmArgs p) {
         asm volatile("" ::: "memory");      \
     }
     // LDS byte addresses of this lane's fragment chunk in ring slot 0; 16-row block BLK adds 1024 BLK
-    const uint32_t frag_lane = (uint32_t)(r16 * 64 + ((kq ^ swz<CPR>(r16)) * 16));
-    const uint32_t fa_byte = lds0 + wm0 * 64 + frag_lane;
-    const uint32_t fb_byte = lds0 + kATileBytes + wn0 * 64 + frag_lane;
+    const uint32_t frag_lane = (uint32_t)(r16 * kRow + ((kq ^ swz<CPR>(r16)) * 16));
+    const uint32_t fa_byte = lds0 + wm0 * kRow + frag_lane;
+    const uint32_t fb_byte = lds0 + kATileBytes + wn0 * kRow + frag_lane;
+    // whole-line stages: the lane's second chunk, kq + 4, of the same row
+    [[maybe_unused]] const uint32_t hi_delta = (uint32_t)((((kq + 4) ^ swz<CPR>(r16)) - (kq ^ swz<CPR>(r16))) * 16);
     // the fragment of 16-row block BLK for the k-step whose stages start at byte offsets o0 (, o1)
     auto load_frag = [&](frag& f, uint32_t base, auto blk_c, uint32_t o0, uint32_t o1) __attribute__((always_inline)) {
-        constexpr int OFF = 1024 * decltype(blk_c)::value;
-        if constexpr (SPS == 1) {
+        constexpr int OFF = 16 * kRow * decltype(blk_c)::value;
+        if constexpr (kLine) {
+            f.lo = lds_read16<OFF>(base + o0);
+            f.hi = lds_read16<OFF>(base + hi_delta + o0);
+        } else if constexpr (SPS == 1) {
             f = lds_read16<OFF>(base + o0);
         } else {
             f.lo = lds_read16<OFF>(base + o0);
@@ -271,8 +316,8 @@ __global__ __launch_bounds__(128 * WGN) void gemm_mfma_tn_256_w4(GemmArgs p) {
             constexpr int i = MOYE_I(P), j = MOYE_J(P);
             // B0 is followed by NI + 1 fragment reads, B1 by NI; a stricter count costs nothing where the
             // older reads are hundreds of clocks old (fp8: two reads per fragment, 32-clock MFMAs)
-            if (P == 0) __builtin_amdgcn_s_waitcnt(0xC07F | (((NI + 1) * SPS < 12 ? (NI + 1) * SPS : 12) << 8));
-            if (P == 4) __builtin_amdgcn_s_waitcnt(0xC07F | ((NI * SPS < 12 ? NI * SPS : 12) << 8));
+            if (P == 0) __builtin_amdgcn_s_waitcnt(0xC07F | (((NI + 1) * RPF < 12 ? (NI + 1) * RPF : 12) << 8));
+            if (P == 4) __builtin_amdgcn_s_waitcnt(0xC07F | ((NI * RPF < 12 ? NI * RPF : 12) << 8));
             In::mma(fb[j], fa[i], acc[i][j]);
             if (P == 7) {
                 // my share of step s+1 has landed and all my fragment reads have returned (the last were
@@ -288,8 +333,9 @@ __global__ __launch_bounds__(128 * WGN) void gemm_mfma_tn_256_w4(GemmArgs p) {
                 }
                 MOYE_BARRIER()
             }
-            if constexpr (dma_index(P, 2 * LD * SPS, NPOS) >= 0) {
-                constexpr int q = dma_index(P, 2 * LD * SPS, NPOS);  // 0 .. 2 LD SPS - 1
+            constexpr int dma_q = kLine ? dma_index_early(P, 2 * LD) : dma_index(P, 2 * LD * SPS, NPOS);
+            if constexpr (dma_q >= 0) {
+                constexpr int q = dma_q;  // 0 .. 2 LD SPS - 1
                 // in the drain a k-step of two stages may still have its first stage to request
                 if (AHEAD || g_new + q / (2 * LD) < nstages) {
                     int sl = slot + q / (2 * LD);
@@ -338,7 +384,7 @@ __global__ __launch_bounds__(128 * WGN) void gemm_mfma_tn_256_w4(GemmArgs p) {
 
 template <typename In, typename Out, int WGN>
 static int32_t launch256_w4(const GemmArgs& a, hipStream_t st) {
-    constexpr int kLds = 5 * (256 + 256) * 64;  // all 160 KiB
+    constexpr int kLds = In::kRing * (256 + 256) * In::kRow;  // all 160 KiB, or 128 KiB for two whole-line stages
     auto kern = gemm_mfma_tn_256_w4<In, Out, WGN>;
     static LdsCap cap;
     if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
@@ -358,11 +404,15 @@ static int32_t launch256_w4_out(int32_t out_dt, const GemmArgs& a, hipStream_t s
 }
 
 template <int WGN>
-static int32_t launch256_w4_in(int32_t in_dt, int32_t out_dt, const GemmArgs& a, bool two_stage_steps, hipStream_t st) {
+static int32_t launch256_w4_in(int32_t in_dt, int32_t out_dt, const GemmArgs& a, bool two_stage_steps, bool ring, hipStream_t st) {
     switch (in_dt) {
-        case MOYE_F16: return two_stage_steps ? launch256_w4_out<W4F16x2, WGN>(out_dt, a, st) : launch256_w4_out<W4F16, WGN>(out_dt, a, st);
-        case MOYE_BF16: return two_stage_steps ? launch256_w4_out<W4BF16x2, WGN>(out_dt, a, st) : launch256_w4_out<W4BF16, WGN>(out_dt, a, st);
-        case MOYE_F8E4M3: return launch256_w4_out<W4FP8, WGN>(out_dt, a, st);
+        case MOYE_F16:
+            if (two_stage_steps && !ring) return launch256_w4_out<W4F16L, WGN>(out_dt, a, st);
+            return two_stage_steps ? launch256_w4_out<W4F16x2, WGN>(out_dt, a, st) : launch256_w4_out<W4F16, WGN>(out_dt, a, st);
+        case MOYE_BF16:
+            if (two_stage_steps && !ring) return launch256_w4_out<W4BF16L, WGN>(out_dt, a, st);
+            return two_stage_steps ? launch256_w4_out<W4BF16x2, WGN>(out_dt, a, st) : launch256_w4_out<W4BF16, WGN>(out_dt, a, st);
+        case MOYE_F8E4M3: return ring ? launch256_w4_out<W4FP8, WGN>(out_dt, a, st) : launch256_w4_out<W4FP8L, WGN>(out_dt, a, st);
         case MOYE_F32: return launch256_w4_out<W4F32, WGN>(out_dt, a, st);
         default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: no MFMA atom for %s inputs", dtype_name(in_dt));
     }
@@ -370,7 +420,7 @@ static int32_t launch256_w4_in(int32_t in_dt, int32_t out_dt, const GemmArgs& a,
 
 // 256 x 256 tile, four or eight waves; K a multiple of kstep_bytes = 64 or 128 bytes (fp8: always 128; fp32: always
 // 64); the caller has checked divisibility of M and N and alignment.
-int32_t gemm_mfma_tn_256_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, int waves, int kstep_bytes, hipStream_t st) {
+int32_t gemm_mfma_tn_256_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, int waves, int kstep_bytes, bool ring, hipStream_t st) {
     a.tiles_m = a.M / 256;
     a.tiles_n = a.N / 256;
     // the load-to-LDS addresses are a uniform base plus a 32-bit lane offset
@@ -378,7 +428,7 @@ int32_t gemm_mfma_tn_256_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, 
     if (256 * a.lda * eb >= (int64_t)1 << 32 || 256 * a.ldb * eb >= (int64_t)1 << 32)
         return fail(MOYE_ERR_SHAPE, "gemm!: row pitch too large for the 256x256 MFMA kernel");
     const bool two = kstep_bytes == 128;
-    return waves == 4 ? launch256_w4_in<2>(in_dt, out_dt, a, two, st) : launch256_w4_in<4>(in_dt, out_dt, a, two, st);
+    return waves == 4 ? launch256_w4_in<2>(in_dt, out_dt, a, two, ring, st) : launch256_w4_in<4>(in_dt, out_dt, a, two, ring, st);
 }
 
 }  // namespace moye

@@ -254,9 +254,10 @@ def test_gemm_errors(mh):
 # 256 x 256 CTA tile schedules (one workgroup per CU)
 # ---------------------------------------------------------------------------------------------
 
-@pytest.mark.parametrize("waves,stages", [((2, 4, 1), 0), ((2, 2, 1), 0), ((2, 4, 1), 4), ((2, 4, 1), 5)])
+@pytest.mark.parametrize("waves,stages", [((2, 4, 1), 0), ((2, 2, 1), 0), ((2, 4, 1), 2), ((2, 2, 1), 2), ((2, 4, 1), 4), ((2, 4, 1), 5)])
 def test_f16_tn_256_tile_exact_on_integers(mh, waves, stages):
-    """Every 256x256 schedule (8 waves, 4 waves, 4- and 5-stage ring) on small-integer inputs:
+    """Every 256x256 schedule (8 waves, 4 waves; stages 0: the library's choice, the hand-ordered kernel on whole-line
+    stages; 2: the compiler-scheduled two-stage kernel; 4- and 5-stage ring) on small-integer inputs:
     all sums are exact in fp32, so the result must equal the integer product exactly."""
     M, N, K = 512, 768, 320
     g = torch.Generator().manual_seed(12)
@@ -335,12 +336,14 @@ def test_wave4_schedule_exact_on_integers(mh, waves):
             B = torch.randint(-3, 4, (N, K), generator=g).float()
             C = torch.randint(-8, 9, (M, N), generator=g).float()
             a, b, c = A.to(in_dt).cuda(), B.to(in_dt).cuda(), C.cuda()
-            d = torch.zeros(M, N, dtype=torch.float32, device="cuda")
-            mma = mh.tiled_mma_desc(atom, atom_layout=waves, cta_tile=(256, 256, bk), flags=_lib.GEMM_WAVE4)
-            print("wave4", waves, in_dt, M, N, K, flush=True)
-            mh.gemm_(mma, T(d), T(a), T(b), T(c), 2.0)
-            torch.cuda.synchronize()
-            assert torch.equal(d.cpu().double(), 2.0 * (A.double() @ B.double().t()) + C.double()), (in_dt, M, N, K)
+            # stages 0: k-steps of 128 bytes run on two whole-line stages; 5: on the ring of five 64-byte-row stages
+            for stages in ((0, 5) if bk * a.element_size() == 128 else (0,)):
+                d = torch.zeros(M, N, dtype=torch.float32, device="cuda")
+                mma = mh.tiled_mma_desc(atom, atom_layout=waves, cta_tile=(256, 256, bk), stages=stages, flags=_lib.GEMM_WAVE4)
+                print("wave4", waves, in_dt, M, N, K, stages, flush=True)
+                mh.gemm_(mma, T(d), T(a), T(b), T(c), 2.0)
+                torch.cuda.synchronize()
+                assert torch.equal(d.cpu().double(), 2.0 * (A.double() @ B.double().t()) + C.double()), (in_dt, M, N, K, stages)
 
 
 @pytest.mark.parametrize("waves", [(2, 2, 1), (2, 4, 1)])

@@ -84,7 +84,8 @@ typedef struct {
     int32_t tile_mnk[3];           /* tile_size(mma, 1..3) (atom/mma.jl:178-191); for the record: the
                                       kernels are chosen by cta_tile_mnk and atom_layout_mnk     */
     int32_t cta_tile_mnk[3];       /* bM, bN, bK; 0 = let the library choose                    */
-    int32_t stages;                /* LDS pipeline depth, 0 = default                           */
+    int32_t stages;                /* LDS pipeline depth, 0 = the library's choice (two); 2 = two
+                                      stages on the compiler-scheduled kernel; 4, 5 = the rings   */
     int32_t split_k;               /* 0/1 = none; >1 = K cut into that many equal ranges (each a
                                       whole number of 16-byte pieces), all computed by one launch
                                       into fp32 partial products in the library's workspace and
@@ -107,10 +108,15 @@ typedef struct {
 #define MOYE_GEMM_PINGPONG 0x100      /* 256x256 tile only: the two waves of a SIMD alternate
                                         between MFMA and memory slots, k-tiles of 64 bytes in a
                                         five-stage LDS ring (cta_tile_mnk[2] = 64 bytes of K)    */
-#define MOYE_GEMM_WAVE4 0x400         /* 256x256 tile only: four waves with 128x128 wave tiles, one
-                                        per SIMD, the same five-stage ring; fp8 on the 16x16x128
-                                        MFMA (cta_tile_mnk[2] = 64 bytes of K, 128 for fp8; 128
-                                        bytes for f16/bf16 too: k-steps of two ring stages)      */
+#define MOYE_GEMM_WAVE4 0x400         /* 256x256 tile only: the hand-ordered kernel by name, four
+                                        waves (atom layout 2x2: 128x128 wave tiles, one per SIMD) or
+                                        eight.  cta_tile_mnk[2] = 128 bytes of K (fp8 always): two
+                                        LDS stages of whole 128-byte rows, or with stages >= 3 the
+                                        ring of five stages of 64-byte rows; 64 bytes of K: that
+                                        ring.  fp8 on the 16x16x128 MFMA.  Plain f16 / bf16 calls on
+                                        256x256x(128 bytes) tiles and fp8 calls run this kernel
+                                        without the flag; stages = 2 keeps a 16-bit call on the
+                                        compiler-scheduled two-stage kernel                       */
 
 /* copy ops: UniversalCopy (src/arch/copy/copy.jl:26-51); the LDS-staged forms stand where the
  * reference has cp.async (copy_async.jl:8-24) and ldmatrix (ldmatrix.jl:18-48) */

@@ -72,7 +72,8 @@ ASM_MFMA_SOURCES = ["gemm_mfma256w4.hip"]
 
 def check_accumulator_hazards(src, force=False):
     """Compile `src` to assembly and fail if, in any basic block that holds v_mfma instructions, something
-    other than a v_mfma names an AccVGPR before the kernel's `MOYE_ACC_SETTLED` marker."""
+    other than a v_mfma names an AccVGPR before the kernel's `MOYE_ACC_SETTLED` marker, or something other than a
+    v_mfma or a ds_read_b128 names a register that the ds_read_b128 of such blocks write (a fragment)."""
     path = os.path.join(CSRC, src)
     asm = os.path.join(CSRC, "build", os.path.splitext(src)[0] + ".s")
     if not force and not _stale(asm, [path] + _headers()):
@@ -81,10 +82,25 @@ def check_accumulator_hazards(src, force=False):
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("hipcc -S failed for %s:\n%s" % (src, r.stdout + r.stderr))
+    with open(asm) as f:
+        acc_bad, frag_bad = asm_mfma_hazards(f, os.path.basename(asm))
+    if acc_bad:
+        os.remove(asm)
+        raise RuntimeError("accumulator registers are touched next to inline-assembly MFMAs:\n" + "\n".join(acc_bad[:20]))
+    if frag_bad:
+        os.remove(asm)
+        raise RuntimeError("fragment registers of inline-assembly LDS reads are touched between the MFMAs:\n" + "\n".join(frag_bad[:20]))
+
+
+def asm_mfma_hazards(lines, name="asm"):
+    """The analysis of check_accumulator_hazards on the lines of an assembly listing: (accumulator findings, fragment
+    findings), each a list of 'file:line: instruction [function]'."""
     fn, block, bad = None, [], []
+    mfma_blocks = []   # (function, [(line number, text)]) of every block that holds MFMAs, for the fragment check below
 
     def flush():
         if fn and any("v_mfma" in c.split(";")[0] for _, c in block):
+            mfma_blocks.append((fn, list(block)))
             settled = False
             for ln, c in block:
                 settled = settled or "MOYE_ACC_SETTLED" in c
@@ -92,11 +108,11 @@ def check_accumulator_hazards(src, force=False):
                 if "v_mfma" in code or settled:
                     continue
                 if re.search(r"\ba(\[\d+:\d+\]|\d+)\b", code):
-                    bad.append("%s:%d: %s   [%s]" % (os.path.basename(asm), ln, code.strip(), fn[:60]))
+                    bad.append("%s:%d: %s   [%s]" % (name, ln, code.strip(), fn[:60]))
         del block[:]
 
-    with open(asm) as f:
-        for ln, line in enumerate(f, 1):
+    if True:
+        for ln, line in enumerate(lines, 1):
             m = re.match(r"^(_Z\w+):", line)
             if m:
                 flush()
@@ -111,9 +127,48 @@ def check_accumulator_hazards(src, force=False):
                 flush()
                 if "s_endpgm" in line:
                     fn = None
-    if bad:
-        os.remove(asm)
-        raise RuntimeError("accumulator registers are touched next to inline-assembly MFMAs:\n" + "\n".join(bad[:20]))
+    acc_bad, bad = bad, []
+    # The fragment registers: written by inline-assembly ds_read_b128 whose results the compiler believes are there at
+    # once; the kernel's own s_waitcnt come before the MFMAs that read them.  Anything else that names such a register
+    # between the MFMAs (a copy made by the register allocator, a spill) could read it before the data has arrived.
+    def vregs(text):
+        out = set()
+        for a, b in re.findall(r"\bv\[(\d+):(\d+)\]", text):
+            out.update(range(int(a), int(b) + 1))
+        out.update(int(a) for a in re.findall(r"\bv(\d+)\b", text))
+        return out
+
+    frags = {}
+    for f, blk in mfma_blocks:
+        for _, c in blk:
+            code = c.split(";")[0]
+            m = re.match(r"\s*ds_read_b128\s+(v\[\d+:\d+\])", code)
+            if m:
+                frags.setdefault(f, set()).update(vregs(m.group(1)))
+    # Per block: a register counts as a fragment from the block's start (the reads of an earlier block or trip may still
+    # be in flight) until something other than a ds_read_b128 writes it (the fragment is dead then and the register has
+    # a new owner); a ds_read_b128 makes it one again.
+    no_dest = re.compile(r"\s*(global_store|buffer_store|ds_write|global_load_lds|s_|v_cmp|v_readfirstlane|v_readlane)")
+    for f, blk in mfma_blocks:
+        pending = set(frags.get(f, set()))
+        settled = False
+        for ln, c in blk:
+            settled = settled or "MOYE_ACC_SETTLED" in c
+            code = c.split(";")[0]
+            if settled or not code.strip() or code.lstrip().startswith(".") or "v_mfma" in code:
+                continue
+            m = re.match(r"\s*ds_read_b128\s+(v\[\d+:\d+\])", code)
+            if m:
+                pending |= vregs(m.group(1))
+                continue
+            ops = code.strip().split(None, 1)
+            operands = ops[1].split(",") if len(ops) > 1 else []
+            dest = set() if (no_dest.match(code) or not operands) else vregs(operands[0])
+            srcs = vregs(",".join(operands[1:] if dest else operands))
+            if srcs & pending:
+                bad.append("%s:%d: %s   [%s]" % (name, ln, code.strip(), f[:60]))
+            pending -= dest
+    return acc_bad, bad
 
 
 def build(force=False, verbose=True):

@@ -1174,6 +1174,18 @@ def test_large_offsets_gemm_and_transpose(mh):
         ref = A[r0:r0 + 256].double() @ B.double().t()
         assert torch.equal(d[r0:r0 + 256].cpu().double(), ref), r0
     del d
+    # an operand whose rows lie 16 MiB apart: 256 rows span 4 GiB, beyond the 32-bit lane offsets of the hand-ordered
+    # kernel, so the call stays on the kernel with 64-bit row addresses
+    Mp, Kp, pitch = 256, 128, 1 << 23
+    abuf = torch.zeros(Mp * pitch, dtype=torch.float16, device="cuda")
+    Ap = torch.randint(-3, 4, (Mp, Kp), generator=g).to(torch.float16)
+    abuf.view(Mp, pitch)[:, :Kp] = Ap.cuda()
+    Bp = torch.randint(-3, 4, (512, Kp), generator=g).to(torch.float16)
+    dp = torch.zeros(Mp, 512, dtype=torch.float32, device="cuda")
+    mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 4, 1), cta_tile=(256, 256, 64)), T(dp), T(abuf, (Mp, Kp), (pitch, 1)), T(Bp.cuda()))
+    torch.cuda.synchronize()
+    assert torch.equal(dp.cpu().double(), Ap.double() @ Bp.double().t())
+    del abuf, dp
     R, Cn = 65536, 32768
     src = torch.arange(R * Cn, dtype=torch.int64, device="cuda").to(torch.int16)   # wraps: value = index mod 2^16
     dst = torch.empty_like(src)

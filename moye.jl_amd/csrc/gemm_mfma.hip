@@ -431,8 +431,9 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         // fp32 operands stay with that kernel, and so does a call that asks for it: stages = 2 in the descriptor, or
         // MOYE_GEMM_HAND_ORDERED=0 in the environment (read once).
         static const bool hand_ordered_off = getenv("MOYE_GEMM_HAND_ORDERED") && atoi(getenv("MOYE_GEMM_HAND_ORDERED")) == 0;
-        if (!hand_ordered_off && eb == 2 && bkb == 128 && stages < 2 && a.ep_op == MOYE_MAP_IDENTITY &&
-            !(a.xcd_swizzle & (MOYE_GEMM_PINGPONG | kGemmRagged | kGemmAMajorM | kGemmBMajorN | kGemmEpiAddVec | kGemmAtom32)) &&
+        const bool bias_no_c = (a.xcd_swizzle & kGemmEpiAddVec) && !a.C && waves != 4;  // (its bias instance: eight waves, no C)
+        if (!hand_ordered_off && eb == 2 && bkb == 128 && stages < 2 && (a.ep_op == MOYE_MAP_IDENTITY || bias_no_c) &&
+            !(a.xcd_swizzle & (MOYE_GEMM_PINGPONG | kGemmRagged | kGemmAMajorM | kGemmBMajorN | kGemmAtom32)) &&
             256 * a.lda * eb < ((int64_t)1 << 32) && 256 * a.ldb * eb < ((int64_t)1 << 32))
             a.xcd_swizzle |= MOYE_GEMM_WAVE4;
         // hand-ordered kernel: k-steps of 64 bytes, or of 128 (fp8 always; the 16-bit types when the tile says so)

@@ -174,7 +174,10 @@ struct W4F32 : W4Ring64 {
 // WGN = 2: four waves (2 x 2), wave tile 128 x 128.  WGN = 4: eight waves (2 x 4), wave tile 128 x 64,
 // two waves per SIMD, so that what stalls one wave's instruction stream (an M0 write, a taken branch,
 // the barrier) leaves the matrix pipe to the other.
-template <typename In, typename Out, int WGN>
+// kBias: the call adds a vector (one value per column or per row) or a scalar to the product and has no C: the same
+// kernel with that addition in the lanes' own epilogue (store_c_tile's kAddVec, without C's read paths, whose registers
+// this kernel cannot spare: with them the epilogue spilled 96 registers).
+template <typename In, typename Out, int WGN, bool kBias = false>
 __global__ __launch_bounds__(128 * WGN) void gemm_mfma_tn_256_w4(GemmArgs p) {
     constexpr int BM = 256, BN = 256, kRow = In::kRow, CPR = kRow / 16, STAGES = In::kRing, SPS = In::SPS;
     constexpr bool kLine = kRow == 128;                        // a fragment is two chunks of one row of one stage
@@ -379,13 +382,13 @@ __global__ __launch_bounds__(128 * WGN) void gemm_mfma_tn_256_w4(GemmArgs p) {
         for (int j = 0; j < NI; ++j) asm volatile("" : "+a"(acc[i][j]));
     __syncthreads();  // every wave is done with the operand ring before it becomes C patches
 
-    store_c_tile<Out, MI, NI, false>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
+    store_c_tile<Out, MI, NI, false, false, kBias, kBias>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
 }
 
-template <typename In, typename Out, int WGN>
+template <typename In, typename Out, int WGN, bool kBias = false>
 static int32_t launch256_w4(const GemmArgs& a, hipStream_t st) {
     constexpr int kLds = In::kRing * (256 + 256) * In::kRow;  // all 160 KiB, or 128 KiB for two whole-line stages
-    auto kern = gemm_mfma_tn_256_w4<In, Out, WGN>;
+    auto kern = gemm_mfma_tn_256_w4<In, Out, WGN, kBias>;
     static LdsCap cap;
     if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
     kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1)), dim3(128 * WGN), kLds, st>>>(a);
@@ -395,6 +398,19 @@ static int32_t launch256_w4(const GemmArgs& a, hipStream_t st) {
 
 template <typename In, int WGN>
 static int32_t launch256_w4_out(int32_t out_dt, const GemmArgs& a, hipStream_t st) {
+    if (a.xcd_swizzle & kGemmEpiAddVec) {  // a bias: the eight-wave whole-line forms of the 16-bit types carry it, for calls without C
+        if constexpr (In::kRow == 128 && In::kBytes == 2 && WGN == 4) {
+            if (a.C) return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the bias instance of the hand-ordered kernel takes no C");
+            switch (out_dt) {
+                case MOYE_F32: return launch256_w4<In, OutF32, WGN, true>(a, st);
+                case MOYE_F16: return launch256_w4<In, OutF16, WGN, true>(a, st);
+                case MOYE_BF16: return launch256_w4<In, OutBF16, WGN, true>(a, st);
+                default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: MFMA kernels write f32, f16 or bf16, not %s", dtype_name(out_dt));
+            }
+        } else {
+            return fail(MOYE_ERR_UNSUPPORTED, "gemm!: this schedule of the hand-ordered kernel takes no element-wise epilogue operation");
+        }
+    }
     switch (out_dt) {
         case MOYE_F32: return launch256_w4<In, OutF32, WGN>(a, st);
         case MOYE_F16: return launch256_w4<In, OutF16, WGN>(a, st);

@@ -148,7 +148,9 @@ __device__ __forceinline__ void store_c_tile_general(const GemmArgs& p, const f3
 // kAddVec: the call adds a vector or a scalar (GemmArgs::ep_op == MOYE_MAP_ADD with a one-per-column, one-per-row or
 // scalar operand: a bias): the lanes add it to their own accumulators here, with the same roundings as the general
 // epilogue, instead of sending the tile through it.
-template <typename Out, int MI, int NI, bool kWithOps = true, bool kGuard = false, bool kAddVec = false>
+// kNoC: the caller has no C (GemmArgs::C is null, checked on the host): nothing of C's two read paths is compiled in,
+// which frees their registers for instances that have few to spare.
+template <typename Out, int MI, int NI, bool kWithOps = true, bool kGuard = false, bool kAddVec = false, bool kNoC = false>
 __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&acc)[MI][NI], u32x4* smem, int wave,
                                              int lane, int64_t m_base, int64_t n_base) {
     typedef typename Out::type OutT;
@@ -172,8 +174,8 @@ __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&ac
     constexpr int NCH = PASS_ROWS * CR / 64, PASSES = MI / PASS_MI;
     constexpr int AHEAD = sizeof(OutT) == 2 ? PASSES : (PASSES < 2 ? PASSES : 2);
     // (ragged tiles read C in whole pieces only when no piece crosses N)
-    const bool row_c = p.C && (p.xcd_swizzle & kGemmRowC) && (!kGuard || p.N % EPC == 0);
-    u32x4 cw[AHEAD][NCH];
+    const bool row_c = !kNoC && p.C && (p.xcd_swizzle & kGemmRowC) && (!kGuard || p.N % EPC == 0);
+    [[maybe_unused]] u32x4 cw[kNoC ? 1 : AHEAD][NCH];
     auto fetch_c = [&](int pass, u32x4 (&into)[NCH]) __attribute__((always_inline)) {
 #pragma unroll
         for (int t = 0; t < NCH; ++t) {
@@ -186,9 +188,11 @@ __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&ac
                                                       ((m_base + PASS_ROWS * pass + row) * p.ldc_m + n_base) * (int64_t)sizeof(OutT) + ch * 16);
         }
     };
-    if (row_c) {
+    if constexpr (!kNoC) {
+        if (row_c) {
 #pragma unroll
-        for (int a = 0; a < AHEAD; ++a) fetch_c(a, cw[a]);
+            for (int a = 0; a < AHEAD; ++a) fetch_c(a, cw[a]);
+        }
     }
     // a lane's columns are n_base + 16 j + 4 kq + 0..3: the operand values of a one-per-column vector, once for all rows
     [[maybe_unused]] f32x4 xcol[kAddVec ? NI : 1];
@@ -201,17 +205,19 @@ __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&ac
     }
 #pragma unroll
     for (int i0 = 0; i0 < MI; i0 += PASS_MI) {
-        if (row_c) {
-            const int pass = i0 / PASS_MI;
+        if constexpr (!kNoC) {
+            if (row_c) {
+                const int pass = i0 / PASS_MI;
 #pragma unroll
-            for (int t = 0; t < NCH; ++t) {
-                const int c = lane + 64 * t, row = c / CR, ch = c % CR;
-                patch16[row * CR + (ch ^ (row & 7))] = cw[pass % AHEAD][t];
+                for (int t = 0; t < NCH; ++t) {
+                    const int c = lane + 64 * t, row = c / CR, ch = c % CR;
+                    patch16[row * CR + (ch ^ (row & 7))] = cw[pass % AHEAD][t];
+                }
+                if (pass + AHEAD < PASSES) fetch_c(pass + AHEAD, cw[pass % AHEAD]);
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
             }
-            if (pass + AHEAD < PASSES) fetch_c(pass + AHEAD, cw[pass % AHEAD]);
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         }
 #pragma unroll
         for (int ii = 0; ii < PASS_MI; ++ii) {
@@ -222,20 +228,24 @@ __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&ac
                 const int chunk = col / EPC, within = col % EPC;
                 OutT* dst = patch + (row * CR + (chunk ^ (row & 7))) * EPC + within;
                 const int64_t m = m_base + 16 * i + r16, n = n_base + 16 * j + 4 * kq;
-                float c[4] = {0.f, 0.f, 0.f, 0.f};
-                if (row_c) {
+                [[maybe_unused]] float c[4] = {0.f, 0.f, 0.f, 0.f};
+                if constexpr (!kNoC) {
+                    if (row_c) {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) c[e] = Out::load(dst, e);
-                } else if (p.C) {
+                        for (int e = 0; e < 4; ++e) c[e] = Out::load(dst, e);
+                    } else if (p.C) {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (!kGuard || (m < p.M && n + e < p.N)) c[e] = Out::load(p.C, m * p.ldc_m + (n + e) * p.ldc_n);
+                        for (int e = 0; e < 4; ++e)
+                            if (!kGuard || (m < p.M && n + e < p.N)) c[e] = Out::load(p.C, m * p.ldc_m + (n + e) * p.ldc_n);
+                    }
                 }
                 float v[4] = {__fmul_rn(acc[i][j].x, p.alpha), __fmul_rn(acc[i][j].y, p.alpha), __fmul_rn(acc[i][j].z, p.alpha),
                               __fmul_rn(acc[i][j].w, p.alpha)};
-                if (p.C) {
+                if constexpr (!kNoC) {
+                    if (p.C) {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) v[e] = __fadd_rn(v[e], __fmul_rn(p.beta, c[e]));
+                        for (int e = 0; e < 4; ++e) v[e] = __fadd_rn(v[e], __fmul_rn(p.beta, c[e]));
+                    }
                 }
                 if constexpr (kAddVec) {
                     const float xrow = per_row ? epi_operand(p, m, 0) : 0.f;

@@ -1536,6 +1536,10 @@ def test_fused_epilogue_every_kernel_and_operand(mh, kernel, operand_kind):
     for col_major_d, out_name, in_out_type in combos:
         _epilogue_case(mh, mma, M, N, K, out_name, "add", operand_kind, 17, col_major_d=col_major_d,
                        operand_in_out_type=in_out_type)
+        if kernel in ("256", "library") and operand_kind != "full":
+            # a bias and no C (beta = 0): the bias instance of the hand-ordered kernel
+            _epilogue_case(mh, mma, M, N, K, out_name, "add", operand_kind, 18, col_major_d=col_major_d, beta=0.0,
+                           operand_in_out_type=in_out_type)
 
 
 def test_fused_epilogue_limits(mh):

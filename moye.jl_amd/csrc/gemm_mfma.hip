@@ -321,6 +321,13 @@ static int32_t dispatch_atom32(int32_t in_dt, int32_t out_dt, int bm, int bn, in
 }
 
 // K-major A and B, N-contiguous D.  bk_elems = 0 picks the default K extent per tile.
+// MOYE_GEMM_HAND_ORDERED=0 in the environment (read once) keeps calls that the library would give to the hand-ordered
+// 256 x 256 kernel on the compiler-scheduled one
+static bool hand_ordered_on() {
+    static const bool off = getenv("MOYE_GEMM_HAND_ORDERED") && atoi(getenv("MOYE_GEMM_HAND_ORDERED")) == 0;
+    return !off;
+}
+
 int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int bk_elems, int waves, int stages,
                               GemmArgs a, hipStream_t st) {
     const int eb = dtype_bytes(in_dt);
@@ -361,6 +368,11 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
             prefer256 && stages < 3 && (waves <= 1 || waves == 8) &&
             !(a.xcd_swizzle & (MOYE_GEMM_WAVE4 | MOYE_GEMM_PINGPONG | kGemmAMajorM | kGemmBMajorN | kGemmAtom32))) {
             a.xcd_swizzle |= kGemmRagged;
+            // K of whole 128-byte rows, no C and no epilogue operation: the hand-ordered kernel's guarded form (rows
+            // clamped, no K tail to mask)
+            if (hand_ordered_on() && eb == 2 && ((int64_t)a.K * eb) % 128 == 0 && a.ep_op == MOYE_MAP_IDENTITY && !a.C && stages < 2 &&
+                256 * a.lda * eb < ((int64_t)1 << 32) && 256 * a.ldb * eb < ((int64_t)1 << 32))
+                return gemm_mfma_tn_256_w4_dispatch(in_dt, out_dt, a, 8, 128, false, st);
             return gemm_mfma_tn_256_dispatch(in_dt, out_dt, a, 8, stages, st);
         }
         if (!big && !majors && a.split <= 1 && bk_elems == 0 && aligned && a.K % (128 / eb) == 0 && prefer256 && (int64_t)(M0 / 256) * (N0 / 256) >= 64) {
@@ -430,9 +442,8 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         // box, bf16 8192^3 726 against 754); operations in the epilogue, ragged tiles, operands that are not K-major and
         // fp32 operands stay with that kernel, and so does a call that asks for it: stages = 2 in the descriptor, or
         // MOYE_GEMM_HAND_ORDERED=0 in the environment (read once).
-        static const bool hand_ordered_off = getenv("MOYE_GEMM_HAND_ORDERED") && atoi(getenv("MOYE_GEMM_HAND_ORDERED")) == 0;
         const bool bias_no_c = (a.xcd_swizzle & kGemmEpiAddVec) && !a.C && waves != 4;  // (its bias instance: eight waves, no C)
-        if (!hand_ordered_off && eb == 2 && bkb == 128 && stages < 2 && (a.ep_op == MOYE_MAP_IDENTITY || bias_no_c) &&
+        if (hand_ordered_on() && eb == 2 && bkb == 128 && stages < 2 && (a.ep_op == MOYE_MAP_IDENTITY || bias_no_c) &&
             !(a.xcd_swizzle & (MOYE_GEMM_PINGPONG | kGemmRagged | kGemmAMajorM | kGemmBMajorN | kGemmAtom32)) &&
             256 * a.lda * eb < ((int64_t)1 << 32) && 256 * a.ldb * eb < ((int64_t)1 << 32))
             a.xcd_swizzle |= MOYE_GEMM_WAVE4;

@@ -177,8 +177,14 @@ struct W4F32 : W4Ring64 {
 // kBias: the call adds a vector (one value per column or per row) or a scalar to the product and has no C: the same
 // kernel with that addition in the lanes' own epilogue (store_c_tile's kAddVec, without C's read paths, whose registers
 // this kernel cannot spare: with them the epilogue spilled 96 registers).
-template <typename In, typename Out, int WGN, bool kBias = false>
+// kRagged: M and N need not be multiples of 256 (K stays a whole number of 128-byte rows): a lane whose row lies beyond
+// the operand reads the operand's last row instead (its constant lane offset is computed from the clamped row), what is
+// computed from it is never stored, and the epilogue runs with its row and column guards (a D that is not 16-byte
+// aligned goes out element by element where it must).  For calls without C, like the bias instance: the guards and C's
+// read paths together spilled 64-110 registers.
+template <typename In, typename Out, int WGN, bool kBias = false, bool kRagged = false>
 __global__ __launch_bounds__(128 * WGN) void gemm_mfma_tn_256_w4(GemmArgs p) {
+    static_assert(!kRagged || (!kBias && In::kRow == 128), "ragged tiles: the plain whole-line form");
     constexpr int BM = 256, BN = 256, kRow = In::kRow, CPR = kRow / 16, STAGES = In::kRing, SPS = In::SPS;
     constexpr bool kLine = kRow == 128;                        // a fragment is two chunks of one row of one stage
     constexpr int RPF = kLine ? 2 : SPS;                       // LDS reads per fragment
@@ -225,9 +231,13 @@ __global__ __launch_bounds__(128 * WGN) void gemm_mfma_tn_256_w4(GemmArgs p) {
     // changes, so no vector ALU work is left in the loop.  M0 carries the LDS destination of the
     // instruction's first lane.
     uint32_t voff[2 * LD];
+    [[maybe_unused]] const int last_a = p.M - 1 - tm * BM, last_b = p.N - 1 - tn * BN;  // ragged: the last row of the operand, counted from the tile's first
 #pragma unroll
-    for (int q = 0; q < 2 * LD; ++q)
-        voff[q] = (uint32_t)((lrow + RPI * (q % LD)) * (q < LD ? pitch_a : pitch_b) + lch * 16);
+    for (int q = 0; q < 2 * LD; ++q) {
+        int row = lrow + RPI * (q % LD);
+        if constexpr (kRagged) row = min(row, q < LD ? last_a : last_b);
+        voff[q] = (uint32_t)(row * (q < LD ? pitch_a : pitch_b) + lch * 16);
+    }
     // stage g of this workgroup's walk over K is stage g + g0 (mod nstages) of the operands: the eight XCDs start an
     // eighth of K apart when the caller asks for it (see gemm_mfma256.hip)
     const int g0 = (p.xcd_swizzle & kGemmRotateK) ? (int)((int64_t)(blockIdx.x % 8) * nsteps / 8) * SPS : 0;
@@ -382,13 +392,13 @@ __global__ __launch_bounds__(128 * WGN) void gemm_mfma_tn_256_w4(GemmArgs p) {
         for (int j = 0; j < NI; ++j) asm volatile("" : "+a"(acc[i][j]));
     __syncthreads();  // every wave is done with the operand ring before it becomes C patches
 
-    store_c_tile<Out, MI, NI, false, false, kBias, kBias>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
+    store_c_tile<Out, MI, NI, false, kRagged, kBias, kBias || kRagged>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
 }
 
-template <typename In, typename Out, int WGN, bool kBias = false>
+template <typename In, typename Out, int WGN, bool kBias = false, bool kRagged = false>
 static int32_t launch256_w4(const GemmArgs& a, hipStream_t st) {
     constexpr int kLds = In::kRing * (256 + 256) * In::kRow;  // all 160 KiB, or 128 KiB for two whole-line stages
-    auto kern = gemm_mfma_tn_256_w4<In, Out, WGN, kBias>;
+    auto kern = gemm_mfma_tn_256_w4<In, Out, WGN, kBias, kRagged>;
     static LdsCap cap;
     if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
     kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1)), dim3(128 * WGN), kLds, st>>>(a);
@@ -398,6 +408,19 @@ static int32_t launch256_w4(const GemmArgs& a, hipStream_t st) {
 
 template <typename In, int WGN>
 static int32_t launch256_w4_out(int32_t out_dt, const GemmArgs& a, hipStream_t st) {
+    if (a.xcd_swizzle & kGemmRagged) {  // tiles that reach beyond M or N: the eight-wave whole-line forms of the 16-bit types
+        if constexpr (In::kRow == 128 && In::kBytes == 2 && WGN == 4) {
+            if (a.ep_op != MOYE_MAP_IDENTITY || a.C) return fail(MOYE_ERR_UNSUPPORTED, "gemm!: ragged tiles of the hand-ordered kernel take no C and no epilogue operation");
+            switch (out_dt) {
+                case MOYE_F32: return launch256_w4<In, OutF32, WGN, false, true>(a, st);
+                case MOYE_F16: return launch256_w4<In, OutF16, WGN, false, true>(a, st);
+                case MOYE_BF16: return launch256_w4<In, OutBF16, WGN, false, true>(a, st);
+                default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: MFMA kernels write f32, f16 or bf16, not %s", dtype_name(out_dt));
+            }
+        } else {
+            return fail(MOYE_ERR_UNSUPPORTED, "gemm!: this schedule of the hand-ordered kernel takes whole tiles only");
+        }
+    }
     if (a.xcd_swizzle & kGemmEpiAddVec) {  // a bias: the eight-wave whole-line forms of the 16-bit types carry it, for calls without C
         if constexpr (In::kRow == 128 && In::kBytes == 2 && WGN == 4) {
             if (a.C) return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the bias instance of the hand-ordered kernel takes no C");
@@ -437,8 +460,8 @@ static int32_t launch256_w4_in(int32_t in_dt, int32_t out_dt, const GemmArgs& a,
 // 256 x 256 tile, four or eight waves; K a multiple of kstep_bytes = 64 or 128 bytes (fp8: always 128; fp32: always
 // 64); the caller has checked divisibility of M and N and alignment.
 int32_t gemm_mfma_tn_256_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, int waves, int kstep_bytes, bool ring, hipStream_t st) {
-    a.tiles_m = a.M / 256;
-    a.tiles_n = a.N / 256;
+    a.tiles_m = (a.M + 255) / 256;  // (beyond whole tiles only with kGemmRagged: the caller has checked)
+    a.tiles_n = (a.N + 255) / 256;
     // the load-to-LDS addresses are a uniform base plus a 32-bit lane offset
     const int eb = dtype_bytes(in_dt);
     if (256 * a.lda * eb >= (int64_t)1 << 32 || 256 * a.ldb * eb >= (int64_t)1 << 32)

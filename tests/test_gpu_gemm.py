@@ -628,18 +628,20 @@ def test_short_m_line_staging_kernel(mh, M):
 
 
 @pytest.mark.parametrize("case", [(4000, 2200, 328), (3900, 2304, 120), (4096, 2048, 72), (4090, 2203, 40), (2100, 4100, 200),
-                                  (4099, 2050, 4096 + 8), (4096, 2048, 128), (1000, 600, 136), (384, 256, 128), (130, 2000, 72)])
+                                  (4099, 2050, 4096 + 8), (4096, 2048, 128), (1000, 600, 136), (384, 256, 128), (130, 2000, 72),
+                                  (4000, 2200, 192), (3841, 2305, 4096)])
 def test_ragged_256_tiles_exact_on_integers(mh, case):
     """Problems the library puts on 256x256 tiles (the larger cases) or 128x128 tiles that reach beyond M, N and K: rows beyond the operands are read from
     the last row and never stored, the K tail (1 to 7 pieces of 16 bytes, also with less than one k-tile in all) is
     masked, pieces of D that cross N go out element by element.  D is a window of a larger buffer whose frame must stay
-    untouched; small integers make every sum exact."""
+    untouched; small integers make every sum exact.  (K of whole 128-byte rows, 16-bit operands and no C: the guarded
+    form of the hand-ordered kernel; everything else: of the compiler-scheduled one.)"""
     M, N, K = case
     g = torch.Generator().manual_seed(M + N + K)
     A = torch.randint(-3, 4, (M, K), generator=g).float()
     B = torch.randint(-3, 4, (N, K), generator=g).float()
     C = torch.randint(-8, 9, (M, N), generator=g).float()
-    if K > 4096:                      # keep |sum| small enough to be exact in fp16 too; both ends of K stay in play
+    if K >= 4096:                     # keep |sum| small enough to be exact in fp16 too; both ends of K stay in play
         A[:, 150:K - 150] = 0
     ref = A.double() @ B.double().t()
     assert float(ref.abs().max()) * 2 + 8 < 2048

@@ -1336,18 +1336,22 @@ def test_host_threads_with_their_own_streams_and_workspaces(mh):
                 ws = torch.zeros(need + 256, dtype=torch.uint8, device="cuda")
                 base = (ws.data_ptr() + 255) // 256 * 256
             st.synchronize()
-            for it in range(12):
+            for it in range(40):
                 mh.gemm_ex_(mma, T(d), ta_m, T(b), None, None, base, need, stream=st.cuda_stream)
                 mh.gemm_ex_(lib_choice, T(dr), T(ar), T(br), stream=st.cuda_stream)
                 mh.copyto_(T(dst, (512, 1024), (1, 512)), T(src), stream=st.cuda_stream)
                 mh.axpby_(1.0, T(d), 0.0, T(y), stream=st.cuda_stream)
                 st.synchronize()
-                if not (torch.equal(d.cpu().double(), ref) and torch.equal(dr.cpu().double(), ref_r)
-                        and torch.equal(dst.cpu(), S.t()) and torch.equal(y.cpu().double(), ref)):
-                    errors.append("thread %d, pass %d: wrong result" % (seed, it))
-                    return
-                d.zero_(), dr.zero_(), dst.zero_(), y.fill_(1.0)
+                with torch.cuda.stream(st):     # (torch's own work on this thread's stream too, so that it is ordered with the calls)
+                    got = [t.cpu() for t in (d, dr, dst, y)]
+                    d.zero_(), dr.zero_(), dst.zero_(), y.fill_(1.0)
                 st.synchronize()
+                if not (torch.equal(got[0].double(), ref) and torch.equal(got[1].double(), ref_r)
+                        and torch.equal(got[2], S.t()) and torch.equal(got[3].double(), ref)):
+                    errors.append("thread %d, pass %d: wrong result (%s)" % (seed, it, [
+                        bool(torch.equal(got[0].double(), ref)), bool(torch.equal(got[1].double(), ref_r)),
+                        bool(torch.equal(got[2], S.t())), bool(torch.equal(got[3].double(), ref))]))
+                    return
         except Exception as e:  # noqa: BLE001 - reported below, in the test's own thread
             errors.append("thread %d: %r" % (seed, e))
 

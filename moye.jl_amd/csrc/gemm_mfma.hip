@@ -363,7 +363,16 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         // less than a further round of tiles (fp16 4000 x 4096 x 4096: 170 us as interior + fringe on 128 x 128 tiles,
         // vendor library 96).  Not fp8: its fast kernel is the hand-ordered one, which has no guarded form.
         const int fr_m = a.M - M0, fr_n = a.N - N0;
-        const bool thin = fr_m <= 64 && fr_n <= 64 && a.K % (128 / eb) == 0 && aligned;  // (a D that is not 16-byte aligned: the guarded instance)
+        // (a D that is not 16-byte aligned: the interior then runs on the guarded instance, which stores such rows in
+        // smaller pieces, and the short-M kernel writes D element by element anyway.)  Priced on its own: whole tiles for
+        // the interior plus a short-M launch per fringe (4.5 us and its operands at 6 TB/s), against the plan for the
+        // whole problem (fp16 4100 x 4100 x 4096: 17 x 17 ragged tiles are a second round for 33 tiles and cost more than
+        // 128 x 128 tiles, 167-173 us either way; interior and two fringes 116)
+        const bool thin_shape = (fr_m > 0 || fr_n > 0) && fr_m <= 64 && fr_n <= 64 && a.K % (128 / eb) == 0 && aligned_ab && ranges == 1;
+        const double fringe_us = (fr_n > 0 ? 4.5 + (double)(M0 + fr_n) * (double)k_bytes_all / 6.0e6 : 0.0) +
+                                 (fr_m > 0 ? 4.5 + (double)(a.N + fr_m) * (double)k_bytes_all / 6.0e6 : 0.0);
+        const bool thin = thin_shape && (int64_t)(M0 / 256) * (N0 / 256) >= 64 &&
+                          gemm_plan_cost_256(M0, N0, k_bytes_all, eb == 4, false) + fringe_us <= plan.us;
         if ((!big || !aligned) && !thin && a.split <= 1 && bk_elems == 0 && aligned_ab && in_dt != MOYE_F8E4M3 && ((int64_t)a.K * eb) % 16 == 0 &&
             prefer256 && stages < 3 && (waves <= 1 || waves == 8) &&
             !(a.xcd_swizzle & (MOYE_GEMM_WAVE4 | MOYE_GEMM_PINGPONG | kGemmAMajorM | kGemmBMajorN | kGemmAtom32))) {
@@ -375,7 +384,7 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
                 return gemm_mfma_tn_256_w4_dispatch(in_dt, out_dt, a, 8, 128, false, st);
             return gemm_mfma_tn_256_dispatch(in_dt, out_dt, a, 8, stages, st);
         }
-        if (!big && !majors && a.split <= 1 && bk_elems == 0 && aligned && a.K % (128 / eb) == 0 && prefer256 && (int64_t)(M0 / 256) * (N0 / 256) >= 64) {
+        if (!big && !majors && a.split <= 1 && bk_elems == 0 && (thin || (aligned && prefer256)) && a.K % (128 / eb) == 0 && (int64_t)(M0 / 256) * (N0 / 256) >= 64) {
             GemmArgs part = a;
             part.M = M0; part.N = N0;
             if (int32_t e = gemm_mfma_tn_dispatch(in_dt, out_dt, 0, 0, 0, waves, stages, part, st)) return e;

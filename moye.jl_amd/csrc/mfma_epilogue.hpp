@@ -126,6 +126,12 @@ __device__ __forceinline__ void store_c_tile_general(const GemmArgs& p, const f3
                 u32x4 w;
                 __builtin_memcpy(&w, out, 16);
                 store_d_chunk(p, d16, w);
+            } else if (kGuard && whole && (reinterpret_cast<uintptr_t>(d16) & 7) == 0) {
+                // a whole piece on an 8-byte boundary (a row pitch of 8 bytes modulo 16 puts every other row there)
+                u32x2 h[2];
+                __builtin_memcpy(h, out, 16);
+                reinterpret_cast<u32x2*>(d16)[0] = h[0];
+                reinterpret_cast<u32x2*>(d16)[1] = h[1];
             } else {
                 OutT* d = static_cast<OutT*>(p.D) + m * p.ldd + n0;
 #pragma unroll
@@ -268,6 +274,12 @@ __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&ac
             if constexpr (kGuard) {
                 const int64_t m = m_base + 16 * i0 + row, n0 = n_base + ch * EPC;
                 if (m >= p.M || n0 >= p.N) continue;
+                if (n0 + EPC <= p.N && (reinterpret_cast<uintptr_t>(d) & 15) == 8) {
+                    // a whole piece on an 8-byte boundary (a row pitch of 8 bytes modulo 16 puts every other row there)
+                    reinterpret_cast<u32x2*>(d)[0] = u32x2{w.x, w.y};
+                    reinterpret_cast<u32x2*>(d)[1] = u32x2{w.z, w.w};
+                    continue;
+                }
                 if (n0 + EPC > p.N || (reinterpret_cast<uintptr_t>(d) & 15)) {
                     OutT o[EPC];
                     __builtin_memcpy(o, &w, 16);

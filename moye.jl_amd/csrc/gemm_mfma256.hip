@@ -8,7 +8,11 @@
 // 4096^2 problem is exactly 256 workgroups: one per CU, no tail.
 //
 // The k-loop and the epilogue are gemm_mfma_tn_lds_tile (gemm_mfma_lds_tile.hpp), shared with the 128 x 128 kernel of
-// gemm_mfma128.hip; the ring schedule below is a second k-loop for the same tile.
+// gemm_mfma128.hip; the ring schedule below is a second k-loop for the same tile.  This k-loop is scheduled by the
+// compiler under sched_group_barrier hints.  Plain f16 / bf16 calls now run the hand-ordered kernel of
+// gemm_mfma256w4.hip instead (same tile, same LDS layout, 4 % faster); this one keeps everything that kernel has no
+// instance for: epilogue operations, a bias together with C, operands that are not K-major, a K tail, fp32 operands,
+// and calls that name it (stages = 2).
 #include "gemm_mfma_lds_tile.hpp"
 
 namespace moye {

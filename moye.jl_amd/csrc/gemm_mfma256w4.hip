@@ -1,7 +1,13 @@
-// gemm! on the matrix cores, one wave per SIMD: one 256 x 256 CTA tile per compute unit, four waves
-// as 2 x 2, wave tile 128 x 128 (8 x 8 MFMA tiles, 256 accumulator registers per lane, pinned in
-// the AccVGPR file), operand tiles with 64-byte rows in a ring of five 32 KiB LDS stages filled by
-// load-to-LDS instructions.
+// gemm! on the matrix cores, every instruction of the k-loop placed by hand: one 256 x 256 CTA tile per compute unit,
+// eight waves as 2 x 4 (wave tile 128 x 64, two waves per SIMD) or four as 2 x 2 (wave tile 128 x 128: 8 x 8 MFMA
+// tiles, 256 accumulator registers per lane, pinned in the AccVGPR file).  Two forms of the operand stages in LDS:
+//   whole lines  rows of 128 bytes of K, a stage is a k-step (64 KiB), two stages; a load-to-LDS instruction reads
+//                eight whole 128-byte lines.  What a plain f16 / bf16 call on 256 x 256 tiles and every fp8 call run
+//                (W4F16L, W4BF16L, W4FP8L; fp16 4096^3 97.4-98.7 us against 101.3-102.9 for the compiler-scheduled kernel
+//                of gemm_mfma256.hip, fp8 8192^3 3050 TFLOP/s against 2745 on the ring), with an instance that adds a
+//                bias and one for tiles that reach beyond M and N
+//   ring         rows of 64 bytes in a ring of five 32 KiB stages, a k-step one stage or two (MOYE_GEMM_WAVE4 with
+//                cta_tile_mnk[2] = 64 bytes of K, or with stages >= 3); how this kernel began, described below
 //
 // Why this shape: a 128 x 128 wave tile needs 16 fragments for 64 MFMAs (0.25 per MFMA; a
 // 128 x 64 wave tile needs 0.375), and with one wave per SIMD the only workgroup-wide rendezvous

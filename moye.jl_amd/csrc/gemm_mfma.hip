@@ -368,7 +368,11 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         // the interior plus a short-M launch per fringe (4.5 us and its operands at 6 TB/s), against the plan for the
         // whole problem (fp16 4100 x 4100 x 4096: 17 x 17 ragged tiles are a second round for 33 tiles and cost more than
         // 128 x 128 tiles, 167-173 us either way; interior and two fringes 116)
-        const bool thin_shape = (fr_m > 0 || fr_n > 0) && fr_m <= 64 && fr_n <= 64 && a.K % (128 / eb) == 0 && aligned_ab && ranges == 1;
+        // (whole interior tiles with a D that is not aligned need the guarded instance: its conditions, as below)
+        const bool guarded_takes_interior = in_dt != MOYE_F8E4M3 && stages < 3 && (waves <= 1 || waves == 8) &&
+                                            !(a.xcd_swizzle & (MOYE_GEMM_WAVE4 | MOYE_GEMM_PINGPONG | kGemmAMajorM | kGemmBMajorN | kGemmAtom32));
+        const bool thin_shape = (fr_m > 0 || fr_n > 0) && fr_m <= 64 && fr_n <= 64 && a.K % (128 / eb) == 0 && aligned_ab && ranges == 1 &&
+                                (aligned || guarded_takes_interior);
         const double fringe_us = (fr_n > 0 ? 4.5 + (double)(M0 + fr_n) * (double)k_bytes_all / 6.0e6 : 0.0) +
                                  (fr_m > 0 ? 4.5 + (double)(a.N + fr_m) * (double)k_bytes_all / 6.0e6 : 0.0);
         const bool thin = thin_shape && (int64_t)(M0 / 256) * (N0 / 256) >= 64 &&

@@ -627,6 +627,37 @@ def test_short_m_line_staging_kernel(mh, M):
         assert torch.equal(d.cpu(), want), (in_dt, out_dt)
 
 
+def test_thin_fringes_with_a_d_that_is_not_aligned(mh):
+    """At most 64 rows and columns beyond whole 256x256 tiles, D's rows 8 bytes off 16-byte boundaries: the interior
+    runs on whole tiles through the guarded instance where there is one (f16 / bf16 / f32 operands), the fringes on the
+    short-M kernel; fp8 has no guarded instance and takes the residue kernels.  Exact on small integers; the frame
+    around D stays untouched."""
+    g = torch.Generator().manual_seed(77)
+    cases = [(torch.float16, mh.MFMA_F32_16x16x32_F16, torch.float16, 4100, 4104, 2048),
+             (torch.bfloat16, mh.MFMA_F32_16x16x32_BF16, torch.float32, 4160, 4098, 2048),
+             (torch.float32, mh.MFMA_F32_16x16x4_F32, torch.float32, 4100, 4104, 64)]
+    if hasattr(torch, "float8_e4m3fn"):
+        cases.append((torch.float8_e4m3fn, mh.MFMA_F32_16x16x32_FP8, torch.bfloat16, 4100, 4104, 2048))
+    for in_dt, atom, out_dt, M, N, K in cases:
+        A = torch.randint(-1, 2, (M, K), generator=g).float()
+        B = torch.randint(-1, 2, (N, K), generator=g).float()
+        A[:, 100:K - 100] = 0                    # keeps every sum small enough for bf16 results
+        ref = A.double() @ B.double().t()
+        assert float(ref.abs().max()) < 250
+        a, b = A.to(in_dt).cuda(), B.to(in_dt).cuda()
+        off = 8 // torch.empty(0, dtype=out_dt).element_size()          # elements in 8 bytes
+        pitch = (N + 2 * off + 7) // 8 * 8 + off
+        big = torch.full((M + 2, pitch), 7.0, dtype=out_dt, device="cuda")
+        d = big[1:M + 1, off:off + N]
+        assert (d.data_ptr() % 16, (pitch * d.element_size()) % 16) in ((8, 8), (0, 8), (8, 0))
+        mh.gemm_(mh.tiled_mma_desc(atom, cta_tile=(0, 0, 0)), T(d), T(a), T(b))
+        torch.cuda.synchronize()
+        assert torch.equal(d.cpu().double(), ref), (in_dt, out_dt)
+        frame = big.clone()
+        frame[1:M + 1, off:off + N] = 7.0
+        assert bool((frame == 7.0).all()), ("stores outside D", in_dt)
+
+
 @pytest.mark.parametrize("case", [(4000, 2200, 328), (3900, 2304, 120), (4096, 2048, 72), (4090, 2203, 40), (2100, 4100, 200),
                                   (4099, 2050, 4096 + 8), (4096, 2048, 128), (1000, 600, 136), (384, 256, 128), (130, 2000, 72),
                                   (4000, 2200, 192), (3841, 2305, 4096), (4100, 2052, 4096)])

@@ -112,7 +112,7 @@ def test_transpose_without_swizzle_is_identical(mh):
 
 
 def test_transpose_full_size_involution(mh):
-    """BASELINE config 2 at full size (16384^2 fp32 bits, 1 GiB each side): closed form on sampled
+    """Benchmark configuration 2 at full size (16384^2 fp32 bits, 1 GiB each side): closed form on sampled
     tiles, an order-independent checksum, and transpose(transpose(x)) == x."""
     M = N = 16384
     src = _rand_bits(M * N, 1002)

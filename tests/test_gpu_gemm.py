@@ -41,7 +41,7 @@ def relerr(c, c64):
 # ---------------------------------------------------------------------------------------------
 
 def test_config1_fp32_256_nn_bit_exact(mh):
-    """BASELINE config 1: fp32 C = A*B, M=N=K=256, A and B column-major, 32x32x8 tiles."""
+    """Benchmark configuration 1: fp32 C = A*B, M=N=K=256, A and B column-major, 32x32x8 tiles."""
     rng = np.random.default_rng(1001)
     M = N = K = 256
     A = (rng.random((M, K), dtype=np.float32) * 2 - 1)           # A[m,k]
@@ -178,7 +178,7 @@ def test_f16_variants(mh):
 
 
 def test_config3_f16_tn_4096(mh):
-    """BASELINE config 3 at full size: fp16 TN 4096^3, fp32 accumulate, fp16 out, 128x128x32 tile."""
+    """Benchmark configuration 3 at full size: fp16 TN 4096^3, fp32 accumulate, fp16 out, 128x128x32 tile."""
     M = N = K = 4096
     got, c64, A, B = _mfma_case(mh, mh.MFMA_F32_16x16x32_F16, torch.float16, torch.float16, M, N, K, 1003,
                                 K ** -0.5, cta=(128, 128, 32))
@@ -194,7 +194,7 @@ def test_config3_f16_tn_4096(mh):
 
 
 def test_bf16_tn(mh):
-    """BASELINE config 4 (square), reduced to 1024^3 here; bf16 in, fp32 out, N(0, 0.02)."""
+    """Benchmark configuration 4 (square), reduced to 1024^3 here; bf16 in, fp32 out, N(0, 0.02)."""
     got, c64, A, B = _mfma_case(mh, mh.MFMA_F32_16x16x32_BF16, torch.bfloat16, torch.float32, 1024, 1024, 1024,
                                 1004, 0.02)
     err = relerr(got, c64)
@@ -206,7 +206,7 @@ def test_bf16_tn(mh):
 
 
 def test_fp8_tn_with_scales(mh):
-    """BASELINE config 5 reduced to 1024^3: e4m3 inputs quantised per tensor by amax/448, fp32
+    """Benchmark configuration 5 reduced to 1024^3: e4m3 inputs quantised per tensor by amax/448, fp32
     accumulate, bf16 out = acc * s_a * s_b."""
     if not hasattr(torch, "float8_e4m3fn"):
         pytest.skip("torch without float8_e4m3fn")
@@ -434,7 +434,7 @@ def test_64x64_tile_exact_on_integers(mh):
 
 
 def test_config4_bf16_8192(mh):
-    """BASELINE config 4 (square) at full size: bf16 8192^3, fp32 accumulate and output."""
+    """Benchmark configuration 4 (square) at full size: bf16 8192^3, fp32 accumulate and output."""
     M = N = K = 8192
     got, c64, A, B = _mfma_case(mh, mh.MFMA_F32_16x16x32_BF16, torch.bfloat16, torch.float32, M, N, K, 1004, 0.02,
                                 cta=(256, 256, 64))
@@ -447,7 +447,7 @@ def test_config4_bf16_8192(mh):
 
 
 def test_config5_fp8_8192(mh):
-    """BASELINE config 5 at full size: e4m3 8192^3, per-tensor scales, bf16 out."""
+    """Benchmark configuration 5 at full size: e4m3 8192^3, per-tensor scales, bf16 out."""
     if not hasattr(torch, "float8_e4m3fn"):
         pytest.skip("torch without float8_e4m3fn")
     M = N = K = 8192
@@ -783,7 +783,7 @@ def test_short_m_other_types(mh):
 
 
 def test_config4_skinny_bf16(mh):
-    """BASELINE config 4, skinny case: bf16 16 x 8192 x 8192, fp32 out; run twice, results identical."""
+    """Benchmark configuration 4, skinny case: bf16 16 x 8192 x 8192, fp32 out; run twice, results identical."""
     M, N, K = 16, 8192, 8192
     got, c64, A, B = _mfma_case(mh, mh.MFMA_F32_16x16x32_BF16, torch.bfloat16, torch.float32, M, N, K, 1004, 0.02,
                                 cta=(0, 0, 0))
@@ -1137,7 +1137,7 @@ def test_operand_majors_other_element_types(mh):
 
 
 def test_config1_shape_on_the_matrix_cores(mh):
-    """BASELINE config 1's operands (fp32 256^3, A and B column-major: the NN form) through the fp32 MFMA
+    """Benchmark configuration 1's operands (fp32 256^3, A and B column-major: the NN form) through the fp32 MFMA
     atom instead of UniversalFMA: tolerance 1e-5 against fp64."""
     M = N = K = 256
     rng = np.random.default_rng(1001)

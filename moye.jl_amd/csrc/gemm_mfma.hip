@@ -496,6 +496,13 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
     // The kernel below keeps 64-byte k-tiles, the 32 x 32 atoms and operands that are not aligned.
     if (bm == 128 && bn == 128 && (bkb == 128 || chosen_here) && !misaligned_ab && ((int64_t)a.K * eb) % 16 == 0) {
         const bool whole = a.M % 128 == 0 && a.N % 128 == 0 && ((int64_t)a.K * eb) % 128 == 0 && !misaligned_d;
+        // (plain f16 / bf16 calls with more tiles than CUs, so that some CUs hold two workgroups: the hand-ordered kernel's
+        // 128 x 128 instance, gemm_mfma256w4.hip: fp16 4096^3 on these tiles 123-124 us against 128.5-129.7, 2560^3 37.5-38.0
+        // against 39.6; with one workgroup per CU, whose load stalls then nobody covers, 2048^3 23.9 against 23.5)
+        if (whole && hand_ordered_on() && (int64_t)(a.M / 128) * (a.N / 128) > 256 && eb == 2 && a.ep_op == MOYE_MAP_IDENTITY && stages < 2 &&
+            !(a.xcd_swizzle & (kGemmAMajorM | kGemmBMajorN | kGemmEpiAddVec)) && 128 * a.lda * eb < ((int64_t)1 << 32) &&
+            128 * a.ldb * eb < ((int64_t)1 << 32))
+            return gemm_mfma_tn_128_w4_dispatch(in_dt, out_dt, a, st);
         if (whole) return gemm_mfma_tn_128_dispatch(in_dt, out_dt, a, st);
         if (chosen_here || (a.xcd_swizzle & MOYE_GEMM_PREDICATE)) {
             a.xcd_swizzle |= kGemmRagged;

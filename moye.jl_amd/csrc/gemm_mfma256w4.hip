@@ -66,6 +66,12 @@ __device__ __forceinline__ void static_for(F&& f) {
 // (measured at fp16 4096^3, eight / four waves: every position 100.4 / 101.0 us, every other 97.7-98.7 / 97.4-98.6, every third
 // 99.3 / 98.3; the barrier after MFMA 3, 5 or 11 instead of 7: 98.2, 99.9, 98.0 / 98.5, 99.4, 97.6)
 constexpr int dma_index_early(int P, int ND) { return P >= 8 && P < 8 + 2 * ND && (P - 8) % 2 == 0 ? (P - 8) / 2 : -1; }
+// The 128 x 128 tile: sixteen groups per k-step, the barrier after the fourth, eight loads over the twelve that follow.
+constexpr int dma_index_128(int P, int ND) {
+    for (int k = 0; k < ND; ++k)
+        if (4 + (3 * k) / 2 == P) return k;
+    return -1;
+}
 constexpr int dma_index(int P, int ND, int NPOS) {
     for (int k = 0; k < ND; ++k)
         if (8 + k * (NPOS - 8) / ND == P) return k;
@@ -188,17 +194,24 @@ struct W4F32 : W4Ring64 {
 // computed from it is never stored, and the epilogue runs with its row and column guards (a D that is not 16-byte
 // aligned goes out element by element where it must).  For calls without C, like the bias instance: the guards and C's
 // read paths together spilled 64-110 registers.
-template <typename In, typename Out, int WGN, bool kBias = false, bool kRagged = false>
-__global__ __launch_bounds__(128 * WGN) void gemm_mfma_tn_256_w4(GemmArgs p) {
+//
+// TILE = 128: the same kernel on a 128 x 128 CTA tile, four waves as 2 x 2 (wave tile 64 x 64, 4 x 4 MFMA tiles), two
+// whole-line stages of 32 KiB, two workgroups per CU (what gemm_mfma128.hip's kernel is to gemm_mfma256.hip's): rows 0-1
+// column by column, then rows 2-3 column by column; the barrier after the fourth MFMA group, the eight loads of a
+// wave over the twelve groups that follow.
+template <typename In, typename Out, int WGN, bool kBias = false, bool kRagged = false, int TILE = 256>
+__global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_256_w4(GemmArgs p) {
     static_assert(!kRagged || (!kBias && In::kRow == 128), "ragged tiles: the plain whole-line form");
-    constexpr int BM = 256, BN = 256, kRow = In::kRow, CPR = kRow / 16, STAGES = In::kRing, SPS = In::SPS;
+    static_assert(TILE == 256 || (TILE == 128 && WGN == 2 && In::kRow == 128 && !kBias && !kRagged), "128 x 128 tiles: the plain whole-line form, 2 x 2 waves");
+    constexpr int BM = TILE, BN = TILE, kRow = In::kRow, CPR = kRow / 16, STAGES = In::kRing, SPS = In::SPS;
     constexpr bool kLine = kRow == 128;                        // a fragment is two chunks of one row of one stage
     constexpr int RPF = kLine ? 2 : SPS;                       // LDS reads per fragment
     constexpr int RPI = 64 / CPR;                              // rows one load-to-LDS instruction covers
     static_assert(!kLine || (SPS == 1 && STAGES == 2), "whole-line stages: one per k-step, two in the ring");
     constexpr int STAGE = (BM + BN) * CPR;  // in 16-byte chunks
     constexpr int NW = 2 * WGN, WN = BN / WGN;
-    constexpr int MI = 8, NI = WN / 16, NPOS = MI * NI;
+    constexpr int MI = BM / 32, NI = WN / 16, NPOS = MI * NI, H = MI / 2;  // H: the rows of the first phase
+    constexpr int BAR = TILE == 128 ? 3 : 7;  // the MFMA group after which the waves meet
     constexpr int RW = BM / NW, LD = RW / RPI;  // per wave and stage: RW rows, LD load-to-LDS instructions per operand
     typedef typename In::frag frag;
 
@@ -208,7 +221,7 @@ __global__ __launch_bounds__(128 * WGN) void gemm_mfma_tn_256_w4(GemmArgs p) {
     split_of_block(p);
     tile_of_block(p, &tm, &tn);
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm0 = (wave / WGN) * 128, wn0 = (wave % WGN) * WN;
+    const int wm0 = (wave / WGN) * (BM / 2), wn0 = (wave % WGN) * WN;
     const int r16 = lane & 15, kq = lane >> 4;
 
     const int64_t pitch_a = (int64_t)p.lda * In::kBytes, pitch_b = (int64_t)p.ldb * In::kBytes;
@@ -310,12 +323,16 @@ __global__ __launch_bounds__(128 * WGN) void gemm_mfma_tn_256_w4(GemmArgs p) {
     // Inside each phase the walk goes back and forth, so that one operand register set changes between consecutive
     // MFMAs, not two (odd columns of rows 0-3 and of rows 6-7 run upwards, row 4 runs from the last column back): with
     // dense operands the part is power-limited and an MFMA-only loop sustains 1.5-2 % more in such an order.
+    // (H = 4 rows first, rows 4 and 5 whole, rows 6 and 7 in pairs for the 256 x 256 tile; H = 2, no whole rows, rows 2
+    // and 3 in pairs for the 128 x 128 one)
 #define MOYE_I(P)                                                                                     \
-    ((P) < 4 * NI ? ((((P) / 4) & 1) ? 3 - (P) % 4 : (P) % 4)                                          \
-     : (P) < 5 * NI ? 4                                                                               \
-     : (P) < 6 * NI ? 5                                                                               \
-                    : 6 + ((((((P) - 6 * NI) / 2) & 1) ? 1 - (((P) - 6 * NI) & 1) : (((P) - 6 * NI) & 1))))
-#define MOYE_J(P) ((P) < 4 * NI ? (P) / 4 : (P) < 5 * NI ? 5 * NI - 1 - (P) : (P) < 6 * NI ? (P) - 5 * NI : ((P) - 6 * NI) / 2)
+    ((P) < H * NI ? ((((P) / H) & 1) ? H - 1 - (P) % H : (P) % H)                                      \
+     : (P) < (MI - 2) * NI ? H + ((P) - H * NI) / NI                                                   \
+                    : MI - 2 + ((((((P) - (MI - 2) * NI) / 2) & 1) ? 1 - (((P) - (MI - 2) * NI) & 1) : (((P) - (MI - 2) * NI) & 1))))
+#define MOYE_J(P)                                                                                     \
+    ((P) < H * NI ? (P) / H                                                                            \
+     : (P) < (MI - 2) * NI ? (((((P) - H * NI) / NI) & 1) ? ((P) - H * NI) % NI : NI - 1 - ((P) - H * NI) % NI) \
+                           : ((P) - (MI - 2) * NI) / 2)
     int slot = 0;  // ring slot of the first stage of step s
     // One k-step.  MORE: step s+1 exists (its fragments are read); AHEAD: the stages five ahead exist
     // (they are requested, and the stages allowed to stay in flight at the barrier are the full 5 - 2 SPS).
@@ -336,9 +353,9 @@ __global__ __launch_bounds__(128 * WGN) void gemm_mfma_tn_256_w4(GemmArgs p) {
             // B0 is followed by NI + 1 fragment reads, B1 by NI; a stricter count costs nothing where the
             // older reads are hundreds of clocks old (fp8: two reads per fragment, 32-clock MFMAs)
             if (P == 0) __builtin_amdgcn_s_waitcnt(0xC07F | (((NI + 1) * RPF < 12 ? (NI + 1) * RPF : 12) << 8));
-            if (P == 4) __builtin_amdgcn_s_waitcnt(0xC07F | ((NI * RPF < 12 ? NI * RPF : 12) << 8));
+            if (P == H) __builtin_amdgcn_s_waitcnt(0xC07F | ((NI * RPF < 12 ? NI * RPF : 12) << 8));
             In::mma(fb[j], fa[i], acc[i][j]);
-            if (P == 7) {
+            if (P == BAR) {
                 // my share of step s+1 has landed and all my fragment reads have returned (the last were
                 // issued eight MFMAs ago); after the barrier that holds for everybody
                 if (AHEAD) {
@@ -352,7 +369,7 @@ __global__ __launch_bounds__(128 * WGN) void gemm_mfma_tn_256_w4(GemmArgs p) {
                 }
                 MOYE_BARRIER()
             }
-            constexpr int dma_q = kLine ? dma_index_early(P, 2 * LD) : dma_index(P, 2 * LD * SPS, NPOS);
+            constexpr int dma_q = TILE == 128 ? dma_index_128(P, 2 * LD) : kLine ? dma_index_early(P, 2 * LD) : dma_index(P, 2 * LD * SPS, NPOS);
             if constexpr (dma_q >= 0) {
                 constexpr int q = dma_q;  // 0 .. 2 LD SPS - 1
                 // in the drain a k-step of two stages may still have its first stage to request
@@ -363,11 +380,10 @@ __global__ __launch_bounds__(128 * WGN) void gemm_mfma_tn_256_w4(GemmArgs p) {
                 }
             }
             if (MORE) {
-                constexpr int A0 = 4 * (NI - 1), B0 = 6 * NI;
-                if constexpr (P >= A0 && P < A0 + 4) load_frag(fa[i], fa_byte, MOYE_BLK(i), o0, o1);  // rows 0-3: last use
-                if constexpr (P == 5 * NI - 1) load_frag(fa[4], fa_byte, MOYE_BLK(4), o0, o1);
-                if constexpr (P == 6 * NI - 1) load_frag(fa[5], fa_byte, MOYE_BLK(5), o0, o1);
-                if constexpr (P >= NPOS - 2) load_frag(fa[i], fa_byte, MOYE_BLK(i), o0, o1);          // rows 6, 7: last use
+                constexpr int A0 = H * (NI - 1), B0 = (MI - 2) * NI;
+                if constexpr (P >= A0 && P < A0 + H) load_frag(fa[i], fa_byte, MOYE_BLK(i), o0, o1);  // the rows of the first phase: last use
+                if constexpr (P >= H * NI && P < B0 && (P + 1) % NI == 0) load_frag(fa[i], fa_byte, MOYE_BLK(i), o0, o1);  // a whole row: its end
+                if constexpr (P >= NPOS - 2) load_frag(fa[i], fa_byte, MOYE_BLK(i), o0, o1);          // the last two rows: last use
                 if constexpr (P >= B0 && ((P - B0) & 1)) load_frag(fb[(P - B0) / 2], fb_byte, MOYE_BLK((P - B0) / 2), o0, o1);
             }
         });
@@ -401,10 +417,10 @@ __global__ __launch_bounds__(128 * WGN) void gemm_mfma_tn_256_w4(GemmArgs p) {
     store_c_tile<Out, MI, NI, false, kRagged, kBias, kBias || kRagged>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
 }
 
-template <typename In, typename Out, int WGN, bool kBias = false, bool kRagged = false>
+template <typename In, typename Out, int WGN, bool kBias = false, bool kRagged = false, int TILE = 256>
 static int32_t launch256_w4(const GemmArgs& a, hipStream_t st) {
-    constexpr int kLds = In::kRing * (256 + 256) * In::kRow;  // all 160 KiB, or 128 KiB for two whole-line stages
-    auto kern = gemm_mfma_tn_256_w4<In, Out, WGN, kBias, kRagged>;
+    constexpr int kLds = In::kRing * (TILE + TILE) * In::kRow;  // all 160 KiB, or 128 KiB for two whole-line stages (64 KiB on 128 x 128 tiles)
+    auto kern = gemm_mfma_tn_256_w4<In, Out, WGN, kBias, kRagged, TILE>;
     static LdsCap cap;
     if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
     kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1)), dim3(128 * WGN), kLds, st>>>(a);
@@ -465,6 +481,31 @@ static int32_t launch256_w4_in(int32_t in_dt, int32_t out_dt, const GemmArgs& a,
 
 // 256 x 256 tile, four or eight waves; K a multiple of kstep_bytes = 64 or 128 bytes (fp8: always 128; fp32: always
 // 64); the caller has checked divisibility of M and N and alignment.
+// The 128 x 128 tile on the same kernel: plain f16 / bf16 calls on whole tiles, K a whole number of 128-byte rows; the
+// caller has checked divisibility and alignment.
+int32_t gemm_mfma_tn_128_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, hipStream_t st) {
+    a.tiles_m = a.M / 128;
+    a.tiles_n = a.N / 128;
+    if (128 * a.lda * 2 >= (int64_t)1 << 32 || 128 * a.ldb * 2 >= (int64_t)1 << 32)
+        return fail(MOYE_ERR_SHAPE, "gemm!: row pitch too large for the hand-ordered 128x128 MFMA kernel");
+    if (in_dt == MOYE_F16) {
+        switch (out_dt) {
+            case MOYE_F32: return launch256_w4<W4F16L, OutF32, 2, false, false, 128>(a, st);
+            case MOYE_F16: return launch256_w4<W4F16L, OutF16, 2, false, false, 128>(a, st);
+            case MOYE_BF16: return launch256_w4<W4F16L, OutBF16, 2, false, false, 128>(a, st);
+            default: break;
+        }
+    } else if (in_dt == MOYE_BF16) {
+        switch (out_dt) {
+            case MOYE_F32: return launch256_w4<W4BF16L, OutF32, 2, false, false, 128>(a, st);
+            case MOYE_F16: return launch256_w4<W4BF16L, OutF16, 2, false, false, 128>(a, st);
+            case MOYE_BF16: return launch256_w4<W4BF16L, OutBF16, 2, false, false, 128>(a, st);
+            default: break;
+        }
+    }
+    return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the hand-ordered 128x128 kernel takes f16 or bf16 operands and writes f32, f16 or bf16");
+}
+
 int32_t gemm_mfma_tn_256_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, int waves, int kstep_bytes, bool ring, hipStream_t st) {
     a.tiles_m = (a.M + 255) / 256;  // (beyond whole tiles only with kGemmRagged: the caller has checked)
     a.tiles_n = (a.N + 255) / 256;

@@ -109,7 +109,7 @@ def headline_variants(mh, tensor_of, torch, stream, A, B, D):
           lambda: mh.gemm_(m128, tD, tA, tB, None, 1.0, stream),
           lambda: mh.time_gemm(m128, tD, tA, tB, None, 1.0, stream, warmup=3, iters=50))
     m128l = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 2, 1), tile=(128, 128, 64), cta_tile=(128, 128, 64))
-    timed("fp16 TN 4096^3 on 128x128x64 tiles, 2x2 waves, load-to-LDS kernel (two workgroups per CU)",
+    timed("fp16 TN 4096^3 on 128x128x64 tiles, 2x2 waves, hand-ordered whole-line kernel (two workgroups per CU)",
           lambda: mh.gemm_(m128l, tD, tA, tB, None, 1.0, stream),
           lambda: mh.time_gemm(m128l, tD, tA, tB, None, 1.0, stream, warmup=3, iters=50))
     m256 = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 4, 1), cta_tile=(256, 256, 64), flags=_lib.GEMM_NO_WORKSPACE)

@@ -506,6 +506,11 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         if (whole) return gemm_mfma_tn_128_dispatch(in_dt, out_dt, a, st);
         if (chosen_here || (a.xcd_swizzle & MOYE_GEMM_PREDICATE)) {
             a.xcd_swizzle |= kGemmRagged;
+            // (K of whole 128-byte rows, no C, no operation, more tiles than CUs: the guarded form of the hand-ordered instance)
+            if (hand_ordered_on() && (int64_t)((a.M + 127) / 128) * ((a.N + 127) / 128) > 256 && eb == 2 && ((int64_t)a.K * eb) % 128 == 0 &&
+                a.ep_op == MOYE_MAP_IDENTITY && !a.C && stages < 2 && !(a.xcd_swizzle & (kGemmAMajorM | kGemmBMajorN | kGemmEpiAddVec)) &&
+                128 * a.lda * eb < ((int64_t)1 << 32) && 128 * a.ldb * eb < ((int64_t)1 << 32))
+                return gemm_mfma_tn_128_w4_dispatch(in_dt, out_dt, a, st);
             return gemm_mfma_tn_128_dispatch(in_dt, out_dt, a, st);
         }
     }

@@ -202,7 +202,7 @@ struct W4F32 : W4Ring64 {
 template <typename In, typename Out, int WGN, bool kBias = false, bool kRagged = false, int TILE = 256>
 __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_256_w4(GemmArgs p) {
     static_assert(!kRagged || (!kBias && In::kRow == 128), "ragged tiles: the plain whole-line form");
-    static_assert(TILE == 256 || (TILE == 128 && WGN == 2 && In::kRow == 128 && !kBias && !kRagged), "128 x 128 tiles: the plain whole-line form, 2 x 2 waves");
+    static_assert(TILE == 256 || (TILE == 128 && WGN == 2 && In::kRow == 128 && !kBias), "128 x 128 tiles: the whole-line form, 2 x 2 waves, plain or ragged");
     constexpr int BM = TILE, BN = TILE, kRow = In::kRow, CPR = kRow / 16, STAGES = In::kRing, SPS = In::SPS;
     constexpr bool kLine = kRow == 128;                        // a fragment is two chunks of one row of one stage
     constexpr int RPF = kLine ? 2 : SPS;                       // LDS reads per fragment
@@ -484,8 +484,27 @@ static int32_t launch256_w4_in(int32_t in_dt, int32_t out_dt, const GemmArgs& a,
 // The 128 x 128 tile on the same kernel: plain f16 / bf16 calls on whole tiles, K a whole number of 128-byte rows; the
 // caller has checked divisibility and alignment.
 int32_t gemm_mfma_tn_128_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, hipStream_t st) {
-    a.tiles_m = a.M / 128;
-    a.tiles_n = a.N / 128;
+    a.tiles_m = (a.M + 127) / 128;  // (beyond whole tiles only with kGemmRagged: the caller has checked; then no C either)
+    a.tiles_n = (a.N + 127) / 128;
+    if (a.xcd_swizzle & kGemmRagged) {
+        if (a.C || a.ep_op != MOYE_MAP_IDENTITY) return fail(MOYE_ERR_UNSUPPORTED, "gemm!: ragged tiles of the hand-ordered kernel take no C and no epilogue operation");
+        if (in_dt == MOYE_F16) {
+            switch (out_dt) {
+                case MOYE_F32: return launch256_w4<W4F16L, OutF32, 2, false, true, 128>(a, st);
+                case MOYE_F16: return launch256_w4<W4F16L, OutF16, 2, false, true, 128>(a, st);
+                case MOYE_BF16: return launch256_w4<W4F16L, OutBF16, 2, false, true, 128>(a, st);
+                default: break;
+            }
+        } else if (in_dt == MOYE_BF16) {
+            switch (out_dt) {
+                case MOYE_F32: return launch256_w4<W4BF16L, OutF32, 2, false, true, 128>(a, st);
+                case MOYE_F16: return launch256_w4<W4BF16L, OutF16, 2, false, true, 128>(a, st);
+                case MOYE_BF16: return launch256_w4<W4BF16L, OutBF16, 2, false, true, 128>(a, st);
+                default: break;
+            }
+        }
+        return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the hand-ordered 128x128 kernel takes f16 or bf16 operands and writes f32, f16 or bf16");
+    }
     if (128 * a.lda * 2 >= (int64_t)1 << 32 || 128 * a.ldb * 2 >= (int64_t)1 << 32)
         return fail(MOYE_ERR_SHAPE, "gemm!: row pitch too large for the hand-ordered 128x128 MFMA kernel");
     if (in_dt == MOYE_F16) {

@@ -660,7 +660,8 @@ def test_thin_fringes_with_a_d_that_is_not_aligned(mh):
 
 @pytest.mark.parametrize("case", [(4000, 2200, 328), (3900, 2304, 120), (4096, 2048, 72), (4090, 2203, 40), (2100, 4100, 200),
                                   (4099, 2050, 4096 + 8), (4096, 2048, 128), (1000, 600, 136), (384, 256, 128), (130, 2000, 72),
-                                  (4000, 2200, 192), (3841, 2305, 4096), (4100, 2052, 4096)])
+                                  (4000, 2200, 192), (3841, 2305, 4096), (4100, 2052, 4096),
+                                  (3000, 2000, 192), (2100, 2900, 4096)])
 def test_ragged_256_tiles_exact_on_integers(mh, case):
     """Problems the library puts on 256x256 tiles (the larger cases) or 128x128 tiles that reach beyond M, N and K: rows beyond the operands are read from
     the last row and never stored, the K tail (1 to 7 pieces of 16 bytes, also with less than one k-tile in all) is

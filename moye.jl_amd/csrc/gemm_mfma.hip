@@ -499,7 +499,10 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         // (plain f16 / bf16 calls with more tiles than CUs, so that some CUs hold two workgroups: the hand-ordered kernel's
         // 128 x 128 instance, gemm_mfma256w4.hip: fp16 4096^3 on these tiles 123-124 us against 128.5-129.7, 2560^3 37.5-38.0
         // against 39.6; with one workgroup per CU, whose load stalls then nobody covers, 2048^3 23.9 against 23.5)
-        if (whole && hand_ordered_on() && (int64_t)(a.M / 128) * (a.N / 128) > 256 && eb == 2 && a.ep_op == MOYE_MAP_IDENTITY && stages < 2 &&
+        // (fp8 always: only this kernel issues the 16x16x128 MFMA on 128 x 128 tiles, twice the rate of the 16x16x32 one:
+        // fp8 2560^3 29.9 -> 22.1 us, 2048^3 16.9 -> 13.7, 1536^3 14.0 -> 10.8)
+        if (whole && hand_ordered_on() && (int64_t)(a.M / 128) * (a.N / 128) > (in_dt == MOYE_F8E4M3 ? 0 : 256) &&
+            (eb == 2 || in_dt == MOYE_F8E4M3) && a.ep_op == MOYE_MAP_IDENTITY && stages < 2 &&
             !(a.xcd_swizzle & (kGemmAMajorM | kGemmBMajorN | kGemmEpiAddVec)) && 128 * a.lda * eb < ((int64_t)1 << 32) &&
             128 * a.ldb * eb < ((int64_t)1 << 32))
             return gemm_mfma_tn_128_w4_dispatch(in_dt, out_dt, a, st);

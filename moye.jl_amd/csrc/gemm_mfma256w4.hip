@@ -507,6 +507,14 @@ int32_t gemm_mfma_tn_128_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, 
     }
     if (128 * a.lda * 2 >= (int64_t)1 << 32 || 128 * a.ldb * 2 >= (int64_t)1 << 32)
         return fail(MOYE_ERR_SHAPE, "gemm!: row pitch too large for the hand-ordered 128x128 MFMA kernel");
+    if (in_dt == MOYE_F8E4M3) {  // (the 16x16x128 MFMA: twice the rate of the 16x16x32 one the other 128 x 128 kernels issue)
+        switch (out_dt) {
+            case MOYE_F32: return launch256_w4<W4FP8L, OutF32, 2, false, false, 128>(a, st);
+            case MOYE_F16: return launch256_w4<W4FP8L, OutF16, 2, false, false, 128>(a, st);
+            case MOYE_BF16: return launch256_w4<W4FP8L, OutBF16, 2, false, false, 128>(a, st);
+            default: break;
+        }
+    }
     if (in_dt == MOYE_F16) {
         switch (out_dt) {
             case MOYE_F32: return launch256_w4<W4F16L, OutF32, 2, false, false, 128>(a, st);
@@ -522,7 +530,7 @@ int32_t gemm_mfma_tn_128_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, 
             default: break;
         }
     }
-    return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the hand-ordered 128x128 kernel takes f16 or bf16 operands and writes f32, f16 or bf16");
+    return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the hand-ordered 128x128 kernel takes f16, bf16 or fp8 operands and writes f32, f16 or bf16");
 }
 
 int32_t gemm_mfma_tn_256_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, int waves, int kstep_bytes, bool ring, hipStream_t st) {

@@ -346,6 +346,39 @@ def test_wave4_schedule_exact_on_integers(mh, waves):
                 assert torch.equal(d.cpu().double(), 2.0 * (A.double() @ B.double().t()) + C.double()), (in_dt, M, N, K, stages)
 
 
+def test_hand_ordered_128_tile_exact_on_integers(mh):
+    """The 128x128 instance of the hand-ordered kernel: plain f16 / bf16 calls with more tiles than CUs (17 x 17 here) and
+    every plain fp8 call on whole 128x128 tiles.  K from one k-step of 128 bytes to many (the prologue, the steady state
+    and the drain each have their own wait counts), C with alpha, every output type; exact on small integers."""
+    g = torch.Generator().manual_seed(23)
+    cases = [(torch.float16, mh.MFMA_F32_16x16x32_F16, 64, 2176, 2176), (torch.bfloat16, mh.MFMA_F32_16x16x32_BF16, 64, 2176, 2304)]
+    if hasattr(torch, "float8_e4m3fn"):
+        cases += [(torch.float8_e4m3fn, mh.MFMA_F32_16x16x32_FP8, 128, 128, 128), (torch.float8_e4m3fn, mh.MFMA_F32_16x16x32_FP8, 128, 384, 640),
+                  (torch.float8_e4m3fn, mh.MFMA_F32_16x16x32_FP8, 128, 2176, 2176)]
+    for in_dt, atom, bk, M, N in cases:
+        for kt in (1, 2, 3, 4, 5, 7, 37):
+            if M > 1000 and kt in (4, 5):
+                continue
+            K = kt * bk
+            A = torch.randint(-3, 4, (M, K), generator=g).float()
+            B = torch.randint(-3, 4, (N, K), generator=g).float()
+            C = torch.randint(-8, 9, (M, N), generator=g).float()
+            a, b, c = A.to(in_dt).cuda(), B.to(in_dt).cuda(), C.cuda()
+            ref = A.double() @ B.double().t()
+            for cta in ((0, 0, 0), (128, 128, bk)):
+                d = torch.zeros(M, N, dtype=torch.float32, device="cuda")
+                mh.gemm_(mh.tiled_mma_desc(atom, atom_layout=(2, 2, 1), cta_tile=cta), T(d), T(a), T(b), T(c), 2.0)
+                torch.cuda.synchronize()
+                assert torch.equal(d.cpu().double(), 2.0 * ref + C.double()), (in_dt, M, N, K, cta)
+            for out_dt in (torch.float16, torch.bfloat16):
+                if float(ref.abs().max()) >= (256 if out_dt == torch.bfloat16 else 2048):
+                    continue
+                d = torch.zeros(M, N, dtype=out_dt, device="cuda")
+                mh.gemm_(mh.tiled_mma_desc(atom, atom_layout=(2, 2, 1), cta_tile=(128, 128, bk)), T(d), T(a), T(b))
+                torch.cuda.synchronize()
+                assert torch.equal(d.cpu().double(), ref), (in_dt, out_dt, M, N, K)
+
+
 @pytest.mark.parametrize("waves", [(2, 2, 1), (2, 4, 1)])
 def test_wave4_schedule_random(mh, waves):
     from moye_hip import _lib

@@ -377,15 +377,17 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
                                  (fr_m > 0 ? 4.5 + (double)(a.N + fr_m) * (double)k_bytes_all / 6.0e6 : 0.0);
         const bool thin = thin_shape && (int64_t)(M0 / 256) * (N0 / 256) >= 64 &&
                           gemm_plan_cost_256(M0, N0, k_bytes_all, eb == 4, false) + fringe_us <= plan.us;
-        if ((!big || !aligned) && !thin && a.split <= 1 && bk_elems == 0 && aligned_ab && in_dt != MOYE_F8E4M3 && ((int64_t)a.K * eb) % 16 == 0 &&
+        // (fp8: only the hand-ordered kernel's guarded form, i.e. K of whole 128-byte rows, no C, no operation)
+        const bool hand_ordered_ragged = hand_ordered_on() && (eb == 2 || in_dt == MOYE_F8E4M3) && ((int64_t)a.K * eb) % 128 == 0 &&
+                                         a.ep_op == MOYE_MAP_IDENTITY && !a.C && stages < 2 &&
+                                         256 * a.lda * eb < ((int64_t)1 << 32) && 256 * a.ldb * eb < ((int64_t)1 << 32);
+        if ((!big || !aligned) && !thin && a.split <= 1 && bk_elems == 0 && aligned_ab && (in_dt != MOYE_F8E4M3 || hand_ordered_ragged) && ((int64_t)a.K * eb) % 16 == 0 &&
             prefer256 && stages < 3 && (waves <= 1 || waves == 8) &&
             !(a.xcd_swizzle & (MOYE_GEMM_WAVE4 | MOYE_GEMM_PINGPONG | kGemmAMajorM | kGemmBMajorN | kGemmAtom32))) {
             a.xcd_swizzle |= kGemmRagged;
             // K of whole 128-byte rows, no C and no epilogue operation: the hand-ordered kernel's guarded form (rows
             // clamped, no K tail to mask)
-            if (hand_ordered_on() && eb == 2 && ((int64_t)a.K * eb) % 128 == 0 && a.ep_op == MOYE_MAP_IDENTITY && !a.C && stages < 2 &&
-                256 * a.lda * eb < ((int64_t)1 << 32) && 256 * a.ldb * eb < ((int64_t)1 << 32))
-                return gemm_mfma_tn_256_w4_dispatch(in_dt, out_dt, a, 8, 128, false, st);
+            if (hand_ordered_ragged) return gemm_mfma_tn_256_w4_dispatch(in_dt, out_dt, a, 8, 128, false, st);
             return gemm_mfma_tn_256_dispatch(in_dt, out_dt, a, 8, stages, st);
         }
         if (!big && !majors && a.split <= 1 && bk_elems == 0 && (thin || (aligned && prefer256)) && a.K % (128 / eb) == 0 && (int64_t)(M0 / 256) * (N0 / 256) >= 64) {
@@ -510,7 +512,8 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         if (chosen_here || (a.xcd_swizzle & MOYE_GEMM_PREDICATE)) {
             a.xcd_swizzle |= kGemmRagged;
             // (K of whole 128-byte rows, no C, no operation, more tiles than CUs: the guarded form of the hand-ordered instance)
-            if (hand_ordered_on() && (int64_t)((a.M + 127) / 128) * ((a.N + 127) / 128) > 256 && eb == 2 && ((int64_t)a.K * eb) % 128 == 0 &&
+            if (hand_ordered_on() && (int64_t)((a.M + 127) / 128) * ((a.N + 127) / 128) > (in_dt == MOYE_F8E4M3 ? 0 : 256) &&
+                (eb == 2 || in_dt == MOYE_F8E4M3) && ((int64_t)a.K * eb) % 128 == 0 &&
                 a.ep_op == MOYE_MAP_IDENTITY && !a.C && stages < 2 && !(a.xcd_swizzle & (kGemmAMajorM | kGemmBMajorN | kGemmEpiAddVec)) &&
                 128 * a.lda * eb < ((int64_t)1 << 32) && 128 * a.ldb * eb < ((int64_t)1 << 32))
                 return gemm_mfma_tn_128_w4_dispatch(in_dt, out_dt, a, st);

@@ -711,9 +711,11 @@ def test_ragged_256_tiles_exact_on_integers(mh, case):
     ref = A.double() @ B.double().t()
     assert float(ref.abs().max()) * 2 + 8 < 2048
     pitch = (N + 8 + 7) // 8 * 8
-    for in_dt, atom, out_dt in ((torch.float16, mh.MFMA_F32_16x16x32_F16, torch.float16),
-                                (torch.bfloat16, mh.MFMA_F32_16x16x32_BF16, torch.float32),
-                                (torch.float32, mh.MFMA_F32_16x16x4_F32, torch.float32)):
+    types = [(torch.float16, mh.MFMA_F32_16x16x32_F16, torch.float16), (torch.bfloat16, mh.MFMA_F32_16x16x32_BF16, torch.float32),
+             (torch.float32, mh.MFMA_F32_16x16x4_F32, torch.float32)]
+    if hasattr(torch, "float8_e4m3fn") and K % 16 == 0:
+        types.append((torch.float8_e4m3fn, mh.MFMA_F32_16x16x32_FP8, torch.float32))
+    for in_dt, atom, out_dt in types:
         a, b, c = A.to(in_dt).cuda(), B.to(in_dt).cuda(), C.to(out_dt).cuda()
         big = torch.full((M + 2, pitch), 77.0, dtype=out_dt, device="cuda")
         d = big[1:M + 1, 8:8 + N]

@@ -462,14 +462,14 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
             !(a.xcd_swizzle & (MOYE_GEMM_PINGPONG | kGemmRagged | kGemmAMajorM | kGemmBMajorN | kGemmAtom32)) &&
             256 * a.lda * eb < ((int64_t)1 << 32) && 256 * a.ldb * eb < ((int64_t)1 << 32))
             a.xcd_swizzle |= MOYE_GEMM_WAVE4;
-        // fp32 operands: the hand-ordered kernel on its ring of 64-byte-row stages (fp32 8192^3 147.8-148.3 TFLOP/s with eight
-        // or four waves against 142.5 for the compiler-scheduled kernel)
+        // fp32 operands: the hand-ordered kernel too (fp32 8192^3 152.8 TFLOP/s on whole-line stages, 147.8 on its ring of
+        // 64-byte-row stages, 142.5 for the compiler-scheduled kernel)
         if (hand_ordered_on() && in_dt == MOYE_F32 && stages < 2 && a.ep_op == MOYE_MAP_IDENTITY && a.K % 16 == 0 &&
             !(a.xcd_swizzle & (MOYE_GEMM_PINGPONG | kGemmRagged | kGemmAMajorM | kGemmBMajorN | kGemmAtom32)) &&
             256 * a.lda * eb < ((int64_t)1 << 32) && 256 * a.ldb * eb < ((int64_t)1 << 32))
             a.xcd_swizzle |= MOYE_GEMM_WAVE4;
         // hand-ordered kernel: k-steps of 64 bytes, or of 128 (fp8 always; the 16-bit types when the tile says so)
-        const int w4_step = in_dt == MOYE_F8E4M3 || (bkb == 128 && eb == 2) ? 128 : 64;
+        const int w4_step = in_dt == MOYE_F8E4M3 || (bkb == 128 && (eb == 2 || eb == 4)) ? 128 : 64;
         const int kmult = (a.xcd_swizzle & MOYE_GEMM_WAVE4) ? w4_step / eb
                           : (a.xcd_swizzle & MOYE_GEMM_PINGPONG) ? 64 / eb : 128 / eb;
         if (a.M % 256 || a.N % 256 || a.K % kmult)
@@ -508,9 +508,10 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         // 128 x 128 instance, gemm_mfma256w4.hip: fp16 4096^3 on these tiles 123-124 us against 128.5-129.7, 2560^3 37.5-38.0
         // against 39.6; with one workgroup per CU, whose load stalls then nobody covers, 2048^3 23.9 against 23.5)
         // (fp8 always: only this kernel issues the 16x16x128 MFMA on 128 x 128 tiles, twice the rate of the 16x16x32 one:
-        // fp8 2560^3 29.9 -> 22.1 us, 2048^3 16.9 -> 13.7, 1536^3 14.0 -> 10.8)
-        if (whole && hand_ordered_on() && (int64_t)(a.M / 128) * (a.N / 128) > (in_dt == MOYE_F8E4M3 ? 0 : 256) &&
-            (eb == 2 || in_dt == MOYE_F8E4M3) && a.ep_op == MOYE_MAP_IDENTITY && stages < 2 &&
+        // fp8 2560^3 29.9 -> 22.1 us, 2048^3 16.9 -> 13.7, 1536^3 14.0 -> 10.8; fp32 always as well: 4096^3 on these tiles
+        // 1136 -> 914 us, 2048^3 128.8 -> 122.5)
+        if (whole && hand_ordered_on() && (int64_t)(a.M / 128) * (a.N / 128) > (eb == 2 ? 256 : 0) &&
+            (eb == 2 || eb == 4 || in_dt == MOYE_F8E4M3) && a.ep_op == MOYE_MAP_IDENTITY && stages < 2 &&
             !(a.xcd_swizzle & (kGemmAMajorM | kGemmBMajorN | kGemmEpiAddVec)) && 128 * a.lda * eb < ((int64_t)1 << 32) &&
             128 * a.ldb * eb < ((int64_t)1 << 32))
             return gemm_mfma_tn_128_w4_dispatch(in_dt, out_dt, a, st);

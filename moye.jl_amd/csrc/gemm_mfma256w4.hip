@@ -199,6 +199,25 @@ struct W4F32 : W4Ring64 {
 // whole-line stages of 32 KiB, two workgroups per CU (what gemm_mfma128.hip's kernel is to gemm_mfma256.hip's): rows 0-1
 // column by column, then rows 2-3 column by column; the barrier after the fourth MFMA group, the eight loads of a
 // wave over the twelve groups that follow.
+// fp32 on whole-line stages: a 128-byte row holds 32 k; chunk kq and chunk kq + 4 are four k each, element j of a chunk
+// going to MFMA j (see W4F32): eight MFMAs in a row per accumulator and k-step.
+struct W4F32L {
+    static constexpr int kBytes = 4, SPS = 1, kRow = 128, kRing = 2;
+    struct frag { u32x4 lo, hi; };
+    static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) {
+        asm volatile(
+            "v_mfma_f32_16x16x4_f32 %0, %1, %5, %0\n\tv_mfma_f32_16x16x4_f32 %0, %2, %6, %0\n\t"
+            "v_mfma_f32_16x16x4_f32 %0, %3, %7, %0\n\tv_mfma_f32_16x16x4_f32 %0, %4, %8, %0"
+            : "+a"(c)
+            : "v"(a.lo.x), "v"(a.lo.y), "v"(a.lo.z), "v"(a.lo.w), "v"(b.lo.x), "v"(b.lo.y), "v"(b.lo.z), "v"(b.lo.w));
+        asm volatile(
+            "v_mfma_f32_16x16x4_f32 %0, %1, %5, %0\n\tv_mfma_f32_16x16x4_f32 %0, %2, %6, %0\n\t"
+            "v_mfma_f32_16x16x4_f32 %0, %3, %7, %0\n\tv_mfma_f32_16x16x4_f32 %0, %4, %8, %0"
+            : "+a"(c)
+            : "v"(a.hi.x), "v"(a.hi.y), "v"(a.hi.z), "v"(a.hi.w), "v"(b.hi.x), "v"(b.hi.y), "v"(b.hi.z), "v"(b.hi.w));
+    }
+};
+
 template <typename In, typename Out, int WGN, bool kBias = false, bool kRagged = false, int TILE = 256>
 __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_256_w4(GemmArgs p) {
     static_assert(!kRagged || (!kBias && In::kRow == 128), "ragged tiles: the plain whole-line form");
@@ -474,7 +493,7 @@ static int32_t launch256_w4_in(int32_t in_dt, int32_t out_dt, const GemmArgs& a,
             if (two_stage_steps && !ring) return launch256_w4_out<W4BF16L, WGN>(out_dt, a, st);
             return two_stage_steps ? launch256_w4_out<W4BF16x2, WGN>(out_dt, a, st) : launch256_w4_out<W4BF16, WGN>(out_dt, a, st);
         case MOYE_F8E4M3: return ring ? launch256_w4_out<W4FP8, WGN>(out_dt, a, st) : launch256_w4_out<W4FP8L, WGN>(out_dt, a, st);
-        case MOYE_F32: return launch256_w4_out<W4F32, WGN>(out_dt, a, st);
+        case MOYE_F32: return two_stage_steps && !ring ? launch256_w4_out<W4F32L, WGN>(out_dt, a, st) : launch256_w4_out<W4F32, WGN>(out_dt, a, st);
         default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: no MFMA atom for %s inputs", dtype_name(in_dt));
     }
 }
@@ -513,8 +532,16 @@ int32_t gemm_mfma_tn_128_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, 
         }
         return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the hand-ordered 128x128 kernel takes f16 or bf16 operands and writes f32, f16 or bf16");
     }
-    if (128 * a.lda * 2 >= (int64_t)1 << 32 || 128 * a.ldb * 2 >= (int64_t)1 << 32)
+    if (128 * a.lda * dtype_bytes(in_dt) >= (int64_t)1 << 32 || 128 * a.ldb * dtype_bytes(in_dt) >= (int64_t)1 << 32)
         return fail(MOYE_ERR_SHAPE, "gemm!: row pitch too large for the hand-ordered 128x128 MFMA kernel");
+    if (in_dt == MOYE_F32) {
+        switch (out_dt) {
+            case MOYE_F32: return launch256_w4<W4F32L, OutF32, 2, false, false, 128>(a, st);
+            case MOYE_F16: return launch256_w4<W4F32L, OutF16, 2, false, false, 128>(a, st);
+            case MOYE_BF16: return launch256_w4<W4F32L, OutBF16, 2, false, false, 128>(a, st);
+            default: break;
+        }
+    }
     if (in_dt == MOYE_F8E4M3) {  // (the 16x16x128 MFMA: twice the rate of the 16x16x32 one the other 128 x 128 kernels issue)
         switch (out_dt) {
             case MOYE_F32: return launch256_w4<W4FP8L, OutF32, 2, false, false, 128>(a, st);

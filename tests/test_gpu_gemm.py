@@ -323,7 +323,7 @@ def test_wave4_schedule_exact_on_integers(mh, waves):
     from moye_hip import _lib
     g = torch.Generator().manual_seed(17)
     cases = [(torch.float16, mh.MFMA_F32_16x16x32_F16, 32), (torch.bfloat16, mh.MFMA_F32_16x16x32_BF16, 32),
-             (torch.float32, mh.MFMA_F32_16x16x4_F32, 16),
+             (torch.float32, mh.MFMA_F32_16x16x4_F32, 16), (torch.float32, mh.MFMA_F32_16x16x4_F32, 32),
              # the 16-bit types with k-steps of two stages (two MFMAs in a row per accumulator)
              (torch.float16, mh.MFMA_F32_16x16x32_F16, 64), (torch.bfloat16, mh.MFMA_F32_16x16x32_BF16, 64)]
     if hasattr(torch, "float8_e4m3fn"):
@@ -348,10 +348,11 @@ def test_wave4_schedule_exact_on_integers(mh, waves):
 
 def test_hand_ordered_128_tile_exact_on_integers(mh):
     """The 128x128 instance of the hand-ordered kernel: plain f16 / bf16 calls with more tiles than CUs (17 x 17 here) and
-    every plain fp8 call on whole 128x128 tiles.  K from one k-step of 128 bytes to many (the prologue, the steady state
+    every plain fp8 and fp32 call on whole 128x128 tiles.  K from one k-step of 128 bytes to many (the prologue, the steady state
     and the drain each have their own wait counts), C with alpha, every output type; exact on small integers."""
     g = torch.Generator().manual_seed(23)
-    cases = [(torch.float16, mh.MFMA_F32_16x16x32_F16, 64, 2176, 2176), (torch.bfloat16, mh.MFMA_F32_16x16x32_BF16, 64, 2176, 2304)]
+    cases = [(torch.float16, mh.MFMA_F32_16x16x32_F16, 64, 2176, 2176), (torch.bfloat16, mh.MFMA_F32_16x16x32_BF16, 64, 2176, 2304),
+             (torch.float32, mh.MFMA_F32_16x16x4_F32, 32, 128, 128), (torch.float32, mh.MFMA_F32_16x16x4_F32, 32, 384, 640)]
     if hasattr(torch, "float8_e4m3fn"):
         cases += [(torch.float8_e4m3fn, mh.MFMA_F32_16x16x32_FP8, 128, 128, 128), (torch.float8_e4m3fn, mh.MFMA_F32_16x16x32_FP8, 128, 384, 640),
                   (torch.float8_e4m3fn, mh.MFMA_F32_16x16x32_FP8, 128, 2176, 2176)]

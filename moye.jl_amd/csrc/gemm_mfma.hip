@@ -378,7 +378,7 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         const bool thin = thin_shape && (int64_t)(M0 / 256) * (N0 / 256) >= 64 &&
                           gemm_plan_cost_256(M0, N0, k_bytes_all, eb == 4, false) + fringe_us <= plan.us;
         // (fp8: only the hand-ordered kernel's guarded form, i.e. K of whole 128-byte rows, no C, no operation)
-        const bool hand_ordered_ragged = hand_ordered_on() && (eb == 2 || in_dt == MOYE_F8E4M3) && ((int64_t)a.K * eb) % 128 == 0 &&
+        const bool hand_ordered_ragged = hand_ordered_on() && (eb == 2 || eb == 4 || in_dt == MOYE_F8E4M3) && ((int64_t)a.K * eb) % 128 == 0 &&
                                          a.ep_op == MOYE_MAP_IDENTITY && !a.C && stages < 2 &&
                                          256 * a.lda * eb < ((int64_t)1 << 32) && 256 * a.ldb * eb < ((int64_t)1 << 32);
         if ((!big || !aligned) && !thin && a.split <= 1 && bk_elems == 0 && aligned_ab && (in_dt != MOYE_F8E4M3 || hand_ordered_ragged) && ((int64_t)a.K * eb) % 16 == 0 &&
@@ -519,8 +519,8 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         if (chosen_here || (a.xcd_swizzle & MOYE_GEMM_PREDICATE)) {
             a.xcd_swizzle |= kGemmRagged;
             // (K of whole 128-byte rows, no C, no operation, more tiles than CUs: the guarded form of the hand-ordered instance)
-            if (hand_ordered_on() && (int64_t)((a.M + 127) / 128) * ((a.N + 127) / 128) > (in_dt == MOYE_F8E4M3 ? 0 : 256) &&
-                (eb == 2 || in_dt == MOYE_F8E4M3) && ((int64_t)a.K * eb) % 128 == 0 &&
+            if (hand_ordered_on() && (int64_t)((a.M + 127) / 128) * ((a.N + 127) / 128) > (eb == 2 ? 256 : 0) &&
+                (eb == 2 || eb == 4 || in_dt == MOYE_F8E4M3) && ((int64_t)a.K * eb) % 128 == 0 &&
                 a.ep_op == MOYE_MAP_IDENTITY && !a.C && stages < 2 && !(a.xcd_swizzle & (kGemmAMajorM | kGemmBMajorN | kGemmEpiAddVec)) &&
                 128 * a.lda * eb < ((int64_t)1 << 32) && 128 * a.ldb * eb < ((int64_t)1 << 32))
                 return gemm_mfma_tn_128_w4_dispatch(in_dt, out_dt, a, st);

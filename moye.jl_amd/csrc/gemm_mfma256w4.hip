@@ -450,7 +450,7 @@ static int32_t launch256_w4(const GemmArgs& a, hipStream_t st) {
 template <typename In, int WGN>
 static int32_t launch256_w4_out(int32_t out_dt, const GemmArgs& a, hipStream_t st) {
     if (a.xcd_swizzle & kGemmRagged) {  // tiles that reach beyond M or N: the eight-wave whole-line forms
-        if constexpr (In::kRow == 128 && In::kBytes <= 2 && WGN == 4) {
+        if constexpr (In::kRow == 128 && WGN == 4) {
             if (a.ep_op != MOYE_MAP_IDENTITY || a.C) return fail(MOYE_ERR_UNSUPPORTED, "gemm!: ragged tiles of the hand-ordered kernel take no C and no epilogue operation");
             switch (out_dt) {
                 case MOYE_F32: return launch256_w4<In, OutF32, WGN, false, true>(a, st);
@@ -507,6 +507,14 @@ int32_t gemm_mfma_tn_128_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, 
     a.tiles_n = (a.N + 127) / 128;
     if (a.xcd_swizzle & kGemmRagged) {
         if (a.C || a.ep_op != MOYE_MAP_IDENTITY) return fail(MOYE_ERR_UNSUPPORTED, "gemm!: ragged tiles of the hand-ordered kernel take no C and no epilogue operation");
+        if (in_dt == MOYE_F32) {
+            switch (out_dt) {
+                case MOYE_F32: return launch256_w4<W4F32L, OutF32, 2, false, true, 128>(a, st);
+                case MOYE_F16: return launch256_w4<W4F32L, OutF16, 2, false, true, 128>(a, st);
+                case MOYE_BF16: return launch256_w4<W4F32L, OutBF16, 2, false, true, 128>(a, st);
+                default: break;
+            }
+        }
         if (in_dt == MOYE_F8E4M3) {
             switch (out_dt) {
                 case MOYE_F32: return launch256_w4<W4FP8L, OutF32, 2, false, true, 128>(a, st);

@@ -426,6 +426,54 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
             }
             return MOYE_OK;
         }
+        // More whole 256 x 256 tiles than CUs, and a last round that fills a small part of the chip: two launches on the
+        // same stream, the first on 256 x 256 tiles over as many tile rows (or columns) as the cost model likes, the
+        // second over the rest on the tiles the library would choose for that problem alone (fp16 6144^3, 576 tiles:
+        // 388 us in one launch, 344 as 20 + 4 tile rows, vendor library 366; 4608^3 185 -> 161-163, vendor 171;
+        // 4608 x 4608 x 8192 318 -> 270-282; 5120^3, 400 tiles, gains nothing and the model says so).  16-bit operands
+        // with everything left to the library; taken when the model sees 3 % or more.
+        if (big && eb == 2 && a.split <= 1 && ranges == 1 && !majors && bk_elems == 0 && waves <= 1 && stages == 0 &&
+            rtiles > 256 && rtiles % 256 && hand_ordered_on() && !(a.xcd_swizzle & (MOYE_GEMM_WAVE4 | MOYE_GEMM_PINGPONG | kGemmAtom32))) {
+            const int tm = a.M / 256, tn = a.N / 256;
+            const bool by_rows = tm >= tn;
+            const int nt = by_rows ? tm : tn;
+            auto alone = [&](int64_t m, int64_t n) {  // what the library would run the part as, priced
+                const double on128 = gemm_plan(m, n, k_bytes_all, false, true, 16, 1).us;
+                const double on256 = gemm_plan_cost_256(m, n, k_bytes_all, false, false);
+                return (m / 256) * (n / 256) >= 64 && on256 <= on128 ? on256 : on128;
+            };
+            const double whole_us = gemm_plan_cost_256(a.M, a.N, k_bytes_all, false, false);
+            double best_us = 0.97 * whole_us;
+            int first = 0;
+            for (int r = 1; r < nt; ++r) {
+                const int64_t m1 = by_rows ? (int64_t)r * 256 : a.M, n1 = by_rows ? a.N : (int64_t)r * 256;
+                const int64_t m2 = by_rows ? a.M - m1 : a.M, n2 = by_rows ? a.N : a.N - n1;
+                const double us = gemm_plan_cost_256(m1, n1, k_bytes_all, false, false) + 2.0 + alone(m2, n2);
+                if (us < best_us) { best_us = us; first = r; }
+            }
+            if (first > 0) {
+                GemmArgs part = a;
+                (by_rows ? part.M : part.N) = first * 256;
+                if (int32_t e = gemm_mfma_tn_dispatch(in_dt, out_dt, 256, 256, 128 / eb, 8, 0, part, st)) return e;
+                part = a;
+                if (by_rows) {
+                    const int64_t m1 = (int64_t)first * 256;
+                    part.M = a.M - (int)m1;
+                    part.A = static_cast<const char*>(a.A) + m1 * a.lda * eb;
+                    part.D = static_cast<char*>(a.D) + m1 * a.ldd * ob0;
+                    if (a.C) part.C = static_cast<const char*>(a.C) + m1 * a.ldc_m * ob0;
+                    if (a.ep_x) part.ep_x = static_cast<const char*>(a.ep_x) + m1 * a.ep_xm * dtype_bytes(a.ep_xdt);
+                } else {
+                    const int64_t n1 = (int64_t)first * 256;
+                    part.N = a.N - (int)n1;
+                    part.B = static_cast<const char*>(a.B) + n1 * a.ldb * eb;
+                    part.D = static_cast<char*>(a.D) + n1 * ob0;
+                    if (a.C) part.C = static_cast<const char*>(a.C) + n1 * a.ldc_n * ob0;
+                    if (a.ep_x) part.ep_x = static_cast<const char*>(a.ep_x) + n1 * a.ep_xn * dtype_bytes(a.ep_xdt);
+                }
+                return gemm_mfma_tn_dispatch(in_dt, out_dt, 0, 0, 0, 0, 0, part, st);
+            }
+        }
         bm = bn = big ? 256 : 128;
         if (bk_elems == 0) bk_elems = big || a.K % (128 / eb) == 0 ? 128 / eb : 64 / eb;
         // smaller problems: 64 x 64 tiles (four times the workgroups, no ragged form) where the cost model prices them

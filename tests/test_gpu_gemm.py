@@ -692,6 +692,46 @@ def test_thin_fringes_with_a_d_that_is_not_aligned(mh):
         assert bool((frame == 7.0).all()), ("stores outside D", in_dt)
 
 
+@pytest.mark.parametrize("case", [(4608, 4608, 2048), (2304, 9216, 1024), (6144, 6144, 512), (4608, 4608, 64), (5120, 5120, 1024),
+                                  (7168, 7168, 256)])
+def test_last_round_on_its_own_launch_exact_on_integers(mh, case):
+    """More whole 256x256 tiles than CUs and a last round that fills little of the chip: the library may run the first
+    tile rows (columns where N has more tiles) on 256x256 tiles and the rest as a problem of its own, on the same
+    stream.  Every element of D belongs to exactly one of the two launches: exact on small integers, with and without
+    C, D a window of a larger buffer whose frame stays untouched."""
+    M, N, K = case
+    g = torch.Generator().manual_seed(M + N + K)
+    for in_dt, atom, out_dt, with_c in ((torch.float16, mh.MFMA_F32_16x16x32_F16, torch.float16, False),
+                                        (torch.bfloat16, mh.MFMA_F32_16x16x32_BF16, torch.float32, True)):
+        A = torch.randint(-1, 2, (M, K), generator=g).float()
+        B = torch.randint(-1, 2, (N, K), generator=g).float()
+        if K > 200:
+            A[:, 100:K - 100] = 0
+        Cm = torch.randint(-3, 4, (M, N), generator=g).float()
+        ref = 0.5 * (A.double() @ B.double().t()) + (Cm.double() if with_c else 0)
+        assert float(ref.abs().max()) < 250
+        a, b = A.to(in_dt).cuda(), B.to(in_dt).cuda()
+        big = torch.full((M + 2, N + 16), 7.0, dtype=out_dt, device="cuda")
+        d = big[1:M + 1, 8:8 + N]
+        mh.gemm_(mh.tiled_mma_desc(atom, cta_tile=(0, 0, 0), split_k=-1), T(d), T(a), T(b), T(Cm.to(out_dt).cuda()) if with_c else None, 0.5)
+        torch.cuda.synchronize()
+        assert torch.equal(d.cpu().double(), ref), (in_dt, out_dt)
+        frame = big.clone()
+        frame[1:M + 1, 8:8 + N] = 7.0
+        assert bool((frame == 7.0).all()), ("stores outside D", in_dt)
+
+
+@pytest.mark.parametrize("shape,kind", [((4608, 4608, 64), "col"), ((2304, 9216, 64), "row"), ((4608, 4608, 128), "full"),
+                                        ((2304, 9216, 128), "col"), ((4608, 4608, 64), "row")])
+def test_last_round_on_its_own_launch_keeps_the_epilogue_operand_in_step(mh, shape, kind):
+    """The same two-launch shapes with a fused epilogue: the second launch reads C and the operand (a vector along
+    either mode, or a whole array) from where its part of D begins.  Bit-exact against the oracle's epilogue."""
+    M, N, K = shape
+    mma = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(0, 0, 0), split_k=-1)
+    _epilogue_case(mh, mma, M, N, K, "float16", "add", kind, seed=M + K + len(kind))
+    _epilogue_case(mh, mma, M, N, K, "float32", "max", kind, seed=N + K + len(kind), beta=0.0)
+
+
 @pytest.mark.parametrize("case", [(4000, 2200, 328), (3900, 2304, 120), (4096, 2048, 72), (4090, 2203, 40), (2100, 4100, 200),
                                   (4099, 2050, 4096 + 8), (4096, 2048, 128), (1000, 600, 136), (384, 256, 128), (130, 2000, 72),
                                   (4000, 2200, 192), (3841, 2305, 4096), (4100, 2052, 4096),

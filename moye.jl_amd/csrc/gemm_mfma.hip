@@ -430,9 +430,9 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         // same stream, the first on 256 x 256 tiles over as many tile rows (or columns) as the cost model likes, the
         // second over the rest on the tiles the library would choose for that problem alone (fp16 6144^3, 576 tiles:
         // 388 us in one launch, 344 as 20 + 4 tile rows, vendor library 366; 4608^3 185 -> 161-163, vendor 171;
-        // 4608 x 4608 x 8192 318 -> 270-282; 5120^3, 400 tiles, gains nothing and the model says so).  16-bit operands
-        // with everything left to the library; taken when the model sees 3 % or more.
-        if (big && eb == 2 && a.split <= 1 && ranges == 1 && !majors && bk_elems == 0 && waves <= 1 && stages == 0 &&
+        // 4608 x 4608 x 8192 318 -> 270-282; 5120^3, 400 tiles, gains nothing and the model says so).  16-bit and fp8
+        // operands with everything left to the library; taken when the model sees 3 % or more.
+        if (big && (eb == 2 || in_dt == MOYE_F8E4M3) && a.split <= 1 && ranges == 1 && !majors && bk_elems == 0 && waves <= 1 && stages == 0 &&
             rtiles > 256 && rtiles % 256 && hand_ordered_on() && !(a.xcd_swizzle & (MOYE_GEMM_WAVE4 | MOYE_GEMM_PINGPONG | kGemmAtom32))) {
             const int tm = a.M / 256, tn = a.N / 256;
             const bool by_rows = tm >= tn;

@@ -701,8 +701,11 @@ def test_last_round_on_its_own_launch_exact_on_integers(mh, case):
     C, D a window of a larger buffer whose frame stays untouched."""
     M, N, K = case
     g = torch.Generator().manual_seed(M + N + K)
-    for in_dt, atom, out_dt, with_c in ((torch.float16, mh.MFMA_F32_16x16x32_F16, torch.float16, False),
-                                        (torch.bfloat16, mh.MFMA_F32_16x16x32_BF16, torch.float32, True)):
+    kinds = [(torch.float16, mh.MFMA_F32_16x16x32_F16, torch.float16, False),
+             (torch.bfloat16, mh.MFMA_F32_16x16x32_BF16, torch.float32, True)]
+    if hasattr(torch, "float8_e4m3fn") and K >= 128:
+        kinds.append((torch.float8_e4m3fn, mh.MFMA_F32_16x16x32_FP8, torch.bfloat16, False))
+    for in_dt, atom, out_dt, with_c in kinds:
         A = torch.randint(-1, 2, (M, K), generator=g).float()
         B = torch.randint(-1, 2, (N, K), generator=g).float()
         if K > 200:

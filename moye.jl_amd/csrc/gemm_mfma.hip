@@ -430,25 +430,28 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         // same stream, the first on 256 x 256 tiles over as many tile rows (or columns) as the cost model likes, the
         // second over the rest on the tiles the library would choose for that problem alone (fp16 6144^3, 576 tiles:
         // 388 us in one launch, 344 as 20 + 4 tile rows, vendor library 366; 4608^3 185 -> 161-163, vendor 171;
-        // 4608 x 4608 x 8192 318 -> 270-282; 5120^3, 400 tiles, gains nothing and the model says so).  16-bit and fp8
-        // operands with everything left to the library; taken when the model sees 3 % or more.
-        if (big && (eb == 2 || in_dt == MOYE_F8E4M3) && a.split <= 1 && ranges == 1 && !majors && bk_elems == 0 && waves <= 1 && stages == 0 &&
+        // 4608 x 4608 x 8192 318 -> 270-282; 5120^3, 400 tiles, gains nothing and the model says so).  Every
+        // operand type, with everything left to the library; taken when the model sees 3 % or more (fp32: 12 %).
+        if (big && a.split <= 1 && ranges == 1 && !majors && bk_elems == 0 && waves <= 1 && stages == 0 &&
             rtiles > 256 && rtiles % 256 && hand_ordered_on() && !(a.xcd_swizzle & (MOYE_GEMM_WAVE4 | MOYE_GEMM_PINGPONG | kGemmAtom32))) {
             const int tm = a.M / 256, tn = a.N / 256;
             const bool by_rows = tm >= tn;
             const int nt = by_rows ? tm : tn;
             auto alone = [&](int64_t m, int64_t n) {  // what the library would run the part as, priced
-                const double on128 = gemm_plan(m, n, k_bytes_all, false, true, 16, 1).us;
-                const double on256 = gemm_plan_cost_256(m, n, k_bytes_all, false, false);
+                const double on128 = gemm_plan(m, n, k_bytes_all, eb == 4, true, 16, 1).us;
+                const double on256 = gemm_plan_cost_256(m, n, k_bytes_all, eb == 4, false);
                 return (m / 256) * (n / 256) >= 64 && on256 <= on128 ? on256 : on128;
             };
-            const double whole_us = gemm_plan_cost_256(a.M, a.N, k_bytes_all, false, false);
-            double best_us = 0.97 * whole_us;
+            const double whole_us = gemm_plan_cost_256(a.M, a.N, k_bytes_all, eb == 4, false);
+            // (fp32: the model prices a part-filled round like a full one, 7 % more than it takes, so it has to see 12 %;
+            // every split it then takes was priced at 20 % or more and gains: 6144^3 4065 -> 3074 us, 4352 x 4352 x 2048
+            // 912 -> 580, 7168 x 7168 x 2048 1833 -> 1494, 4608^3 2023 -> 1754)
+            double best_us = (eb == 4 ? 0.88 : 0.97) * whole_us;
             int first = 0;
             for (int r = 1; r < nt; ++r) {
                 const int64_t m1 = by_rows ? (int64_t)r * 256 : a.M, n1 = by_rows ? a.N : (int64_t)r * 256;
                 const int64_t m2 = by_rows ? a.M - m1 : a.M, n2 = by_rows ? a.N : a.N - n1;
-                const double us = gemm_plan_cost_256(m1, n1, k_bytes_all, false, false) + 2.0 + alone(m2, n2);
+                const double us = gemm_plan_cost_256(m1, n1, k_bytes_all, eb == 4, false) + 2.0 + alone(m2, n2);
                 if (us < best_us) { best_us = us; first = r; }
             }
             if (first > 0) {

@@ -705,6 +705,8 @@ def test_last_round_on_its_own_launch_exact_on_integers(mh, case):
              (torch.bfloat16, mh.MFMA_F32_16x16x32_BF16, torch.float32, True)]
     if hasattr(torch, "float8_e4m3fn") and K >= 128:
         kinds.append((torch.float8_e4m3fn, mh.MFMA_F32_16x16x32_FP8, torch.bfloat16, False))
+    if K <= 512:
+        kinds.append((torch.float32, mh.MFMA_F32_16x16x4_F32, torch.float32, False))
     for in_dt, atom, out_dt, with_c in kinds:
         A = torch.randint(-1, 2, (M, K), generator=g).float()
         B = torch.randint(-1, 2, (N, K), generator=g).float()

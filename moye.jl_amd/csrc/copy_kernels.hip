@@ -121,43 +121,49 @@ static int32_t launch_transpose(const uint32_t* s, uint32_t* d, int64_t lds_, in
 // reads of 256-byte pieces a pitch apart run at 6.9 TB/s whatever the order; writes run at 6.6-6.9 TB/s in this order
 // against 5.1 with the source-contiguous index first), and fewer workgroups in flight do better than more: one per CU
 // (6.25 TB/s) against two (6.15) or five (5.85), hence the LDS request above what the tiles need.
+// 512 lanes, eight 16-byte loads each (same box, alternating runs, 16384^2: 256 lanes with sixteen loads each 6226-6252 GB/s,
+// 512 with eight 6263-6300, 1024 with four 6236; two such workgroups per CU 6254; workgroups of 32 x 512, 128 x 256 or
+// 64 x 512 elements 5.9-6.2; ordinary stores, or half of each row stored the ordinary way, 5.89; ordinary loads 5.90).
 template <int GJ>
-__global__ __launch_bounds__(256) void transpose_lds_b32_rows(const uint32_t* __restrict__ src, uint32_t* __restrict__ dst,
+__global__ __launch_bounds__(512) void transpose_lds_b32_rows(const uint32_t* __restrict__ src, uint32_t* __restrict__ dst,
                                                               int64_t lds_, int64_t ldd, int groups_j, int64_t bs_src,
                                                               int64_t bs_dst) {
-    extern __shared__ u32x4 tile[];  // GJ tiles of 64 x 16 chunks
+    constexpr int TJ = GJ * kTile, JC = TJ / 4;  // the group's extent along j, in elements and in 16-byte chunks
+    constexpr int NG = 512 / 16, NB = JC / NG;   // lanes come as 16 chunks along i x NG row quads along j
+    static_assert(JC % NG == 0 && 512 % JC == 0, "group shape");
+    extern __shared__ u32x4 tile[];  // 64 rows (i) of JC chunks (j), the chunk index XORed with (row / 4) % 8
     src += (int64_t)blockIdx.y * bs_src;
     dst += (int64_t)blockIdx.y * bs_dst;
     const int gj = blockIdx.x % groups_j, ti = blockIdx.x / groups_j;
-    const int lane16 = threadIdx.x & 15;  // chunk of 4 along the contiguous index of the side being accessed
-    const int grp = threadIdx.x >> 4;     // 0..15
+    const int ic = threadIdx.x & 15;  // chunk of 4 along i
+    const int jr = threadIdx.x >> 4;  // 0..31: source rows 4 (jr + NG b) + q
 
-    // ---- load: source rows j = 64 b + 4 grp + q of the group, elements i = 4 lane16 .. +3 of tile column ti ----
-    const uint32_t* s = src + ((int64_t)gj * GJ * kTile + 4 * grp) * lds_ + (int64_t)ti * kTile + 4 * lane16;
-    u32x4 v[GJ][4];
+    const uint32_t* s = src + ((int64_t)gj * TJ) * lds_ + (int64_t)ti * kTile + 4 * ic;
+    u32x4 v[NB][4];
 #pragma unroll
-    for (int b = 0; b < GJ; ++b)
+    for (int b = 0; b < NB; ++b)
 #pragma unroll
         for (int q = 0; q < 4; ++q)
-            v[b][q] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(s + (int64_t)(b * kTile + q) * lds_));
+            v[b][q] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(s + (int64_t)(4 * (jr + NG * b) + q) * lds_));
+    // 4 x 4 register transpose: eight consecutive lanes write eight different rows-of-four, hence eight different bank groups
 #pragma unroll
-    for (int b = 0; b < GJ; ++b)
+    for (int b = 0; b < NB; ++b)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const int row = 4 * lane16 + e;  // i within the tile
-            tile[b * 1024 + row * 16 + lds_chunk<true>(row, grp)] = u32x4{v[b][0][e], v[b][1][e], v[b][2][e], v[b][3][e]};
+            const int row = 4 * ic + e, c = jr + NG * b;
+            tile[row * JC + (c ^ ((row >> 2) & 7))] = u32x4{v[b][0][e], v[b][1][e], v[b][2][e], v[b][3][e]};
         }
     __syncthreads();
-    // ---- store: destination rows i = grp + 16 p, elements j = 64 b + 4 lane16 .. +3 ----
-    uint32_t* d = dst + ((int64_t)ti * kTile + grp) * ldd + (int64_t)gj * GJ * kTile + 4 * lane16;
+    // ---- store: JC consecutive lanes write one destination row of the group (GJ * 256 bytes), 512 / JC rows per pass ----
+    constexpr int RPP = 512 / JC;
+    const int jc = threadIdx.x % JC, r0 = threadIdx.x / JC;
+    uint32_t* d = dst + ((int64_t)ti * kTile + r0) * ldd + (int64_t)gj * TJ + 4 * jc;
 #pragma unroll
-    for (int p = 0; p < 4; ++p)
-#pragma unroll
-        for (int b = 0; b < GJ; ++b) {
-            const int row = grp + 16 * p;
-            const u32x4 w = tile[b * 1024 + row * 16 + lds_chunk<true>(row, lane16)];
-            __builtin_nontemporal_store(w, reinterpret_cast<u32x4*>(d + (int64_t)(16 * p) * ldd + b * kTile));
-        }
+    for (int p = 0; p < kTile / RPP; ++p) {
+        const int row = r0 + RPP * p;
+        const u32x4 w = tile[row * JC + (jc ^ ((row >> 2) & 7))];
+        __builtin_nontemporal_store(w, reinterpret_cast<u32x4*>(d + (int64_t)(RPP * p) * ldd));
+    }
 }
 
 template <int GJ>
@@ -169,8 +175,8 @@ static int32_t launch_transpose_rows(const uint32_t* s, uint32_t* d, int64_t lds
     static LdsCap cap;
     if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
     const int64_t groups = (int64_t)ti * (tj / GJ);
-    if (groups >= (1 << 24)) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles for one launch (2^24 workgroups of 256)");
-    kern<<<dim3((unsigned)groups, (unsigned)batch), 256, kLds, st>>>(s, d, lds_, ldd, tj / GJ, bs_src, bs_dst);
+    if (groups >= (1 << 24)) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles for one launch (2^24 workgroups of 512)");
+    kern<<<dim3((unsigned)groups, (unsigned)batch), 512, kLds, st>>>(s, d, lds_, ldd, tj / GJ, bs_src, bs_dst);
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;
 }

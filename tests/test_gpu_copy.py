@@ -121,6 +121,10 @@ def test_transpose_full_size_involution(mh):
     mh.copyto_(_tens(mh, dst, (M, N), (N, 1)), _tens(mh, src, (M, N), (1, M)), tc)
     torch.cuda.synchronize()
     assert int(dst.sum(dtype=torch.int64)) == int(src.sum(dtype=torch.int64))
+    # every element against the closed form dst[i, j] == src[j, i] (test/host/copy_async.jl:43,95), 2048 rows at a time
+    # so that the comparison's temporaries stay small
+    for r in range(0, M, 2048):
+        assert torch.equal(dst.view(M, N)[r:r + 2048], src.view(N, M)[:, r:r + 2048].t()), "rows %d.." % r
     rng = np.random.default_rng(0)
     for _ in range(64):
         i, j = int(rng.integers(0, M - 64)), int(rng.integers(0, N - 64))

@@ -73,7 +73,8 @@ ASM_MFMA_SOURCES = ["gemm_mfma256w4.hip"]
 def check_accumulator_hazards(src, force=False):
     """Compile `src` to assembly and fail if, in any basic block that holds v_mfma instructions, something
     other than a v_mfma names an AccVGPR before the kernel's `MOYE_ACC_SETTLED` marker, or something other than a
-    v_mfma or a ds_read_b128 names a register that the ds_read_b128 of such blocks write (a fragment)."""
+    v_mfma or a fragment read (ds_read_b128, ds_read_b64_tr_b16) names a register that the fragment reads of such blocks
+    write."""
     path = os.path.join(CSRC, src)
     asm = os.path.join(CSRC, "build", os.path.splitext(src)[0] + ".s")
     if not force and not _stale(asm, [path] + _headers()):
@@ -142,7 +143,7 @@ def asm_mfma_hazards(lines, name="asm"):
     for f, blk in mfma_blocks:
         for _, c in blk:
             code = c.split(";")[0]
-            m = re.match(r"\s*ds_read_b128\s+(v\[\d+:\d+\])", code)
+            m = re.match(r"\s*ds_read_(?:b128|b64_tr_b16)\s+(v\[\d+:\d+\])", code)
             if m:
                 frags.setdefault(f, set()).update(vregs(m.group(1)))
     # Per block: a register counts as a fragment from the block's start (the reads of an earlier block or trip may still
@@ -157,7 +158,7 @@ def asm_mfma_hazards(lines, name="asm"):
             code = c.split(";")[0]
             if settled or not code.strip() or code.lstrip().startswith(".") or "v_mfma" in code:
                 continue
-            m = re.match(r"\s*ds_read_b128\s+(v\[\d+:\d+\])", code)
+            m = re.match(r"\s*ds_read_(?:b128|b64_tr_b16)\s+(v\[\d+:\d+\])", code)
             if m:
                 pending |= vregs(m.group(1))
                 continue

@@ -509,8 +509,12 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         // fp32 operands stay with that kernel, and so does a call that asks for it: stages = 2 in the descriptor, or
         // MOYE_GEMM_HAND_ORDERED=0 in the environment (read once).
         const bool bias_no_c = (a.xcd_swizzle & kGemmEpiAddVec) && !a.C && waves != 4;  // (its bias instance: eight waves, no C)
-        if (hand_ordered_on() && eb == 2 && bkb == 128 && stages < 2 && (a.ep_op == MOYE_MAP_IDENTITY || bias_no_c) &&
-            !(a.xcd_swizzle & (MOYE_GEMM_PINGPONG | kGemmRagged | kGemmAMajorM | kGemmBMajorN | kGemmAtom32)) &&
+        // (operands that keep their M- / N-major form: its transposing fragment reads, eight waves, plain calls; fp16 4096^3 NN
+        // against the compiler-scheduled kernel's: see the kernel's header)
+        const bool majors256 = a.xcd_swizzle & (kGemmAMajorM | kGemmBMajorN);
+        if (hand_ordered_on() && eb == 2 && bkb == 128 && stages < 2 && (a.ep_op == MOYE_MAP_IDENTITY || (bias_no_c && !majors256)) &&
+            (!majors256 || (waves != 4 && !(a.xcd_swizzle & kGemmEpiAddVec))) &&
+            !(a.xcd_swizzle & (MOYE_GEMM_PINGPONG | kGemmRagged | kGemmAtom32)) &&
             256 * a.lda * eb < ((int64_t)1 << 32) && 256 * a.ldb * eb < ((int64_t)1 << 32))
             a.xcd_swizzle |= MOYE_GEMM_WAVE4;
         // fp32 operands: the hand-ordered kernel too (fp32 8192^3 152.8 TFLOP/s on whole-line stages, 147.8 on its ring of

@@ -95,6 +95,18 @@ __device__ __forceinline__ u32x4 lds_read16(uint32_t addr) {
     return v;
 }
 
+// 8 bytes through the transposing LDS read of gfx950: sixteen lanes that each point at four consecutive 16-bit values
+// get back, in lane j, value j % 4 of the lanes 4 e + j / 4 (e = 0..3).  In flight like lds_read16's result.
+template <int OFF>
+__device__ __forceinline__ u32x2 lds_read_tr8(uint32_t addr) {
+    u32x2 v;
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+    return v;
+}
+// A fragment read out of an operand stage that is stored with its unit stride along M (N): four 8-byte halves, q0 q1
+// the lane's eight k of the first MFMA, q2 q3 those of the second (see the kernel's AMAJ / BMAJ).
+struct W4TrFrag { u32x2 q0, q1, q2, q3; };
+
 // fragment = what one lane feeds to one MFMA group per operand; SPS = ring stages per k-step; kRow = bytes of K per row
 // of a stage, kRing = stages in the ring
 struct W4Ring64 { static constexpr int kRow = 64, kRing = 5; };
@@ -157,18 +169,21 @@ struct W4FP8L {
 struct W4F16L {
     static constexpr int kBytes = 2, SPS = 1, kRow = 128, kRing = 2;
     struct frag { u32x4 lo, hi; };
-    static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) {
+    // the two MFMAs of an accumulator from the four 16-byte halves (what the transposing fragment reads assemble)
+    static __device__ __forceinline__ void mma4(const u32x4& alo, const u32x4& ahi, const u32x4& blo, const u32x4& bhi, f32x4& c) {
         asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %3, %0\n\tv_mfma_f32_16x16x32_f16 %0, %2, %4, %0"
-                     : "+a"(c) : "v"(a.lo), "v"(a.hi), "v"(b.lo), "v"(b.hi));
+                     : "+a"(c) : "v"(alo), "v"(ahi), "v"(blo), "v"(bhi));
     }
+    static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) { mma4(a.lo, a.hi, b.lo, b.hi, c); }
 };
 struct W4BF16L {
     static constexpr int kBytes = 2, SPS = 1, kRow = 128, kRing = 2;
     struct frag { u32x4 lo, hi; };
-    static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) {
+    static __device__ __forceinline__ void mma4(const u32x4& alo, const u32x4& ahi, const u32x4& blo, const u32x4& bhi, f32x4& c) {
         asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %3, %0\n\tv_mfma_f32_16x16x32_bf16 %0, %2, %4, %0"
-                     : "+a"(c) : "v"(a.lo), "v"(a.hi), "v"(b.lo), "v"(b.hi));
+                     : "+a"(c) : "v"(alo), "v"(ahi), "v"(blo), "v"(bhi));
     }
+    static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) { mma4(a.lo, a.hi, b.lo, b.hi, c); }
 };
 // element j of the chunk goes to MFMA j (see InF32)
 struct W4F32 : W4Ring64 {
@@ -218,8 +233,19 @@ struct W4F32L {
     }
 };
 
-template <typename In, typename Out, int WGN, bool kBias = false, bool kRagged = false, int TILE = 256>
+// AMAJ / BMAJ = 1: that operand is stored with its unit stride along M (N) instead of K, the 'N' forms of
+// src/arch/mma/make_mma_ops.jl:253-265 (GemmArgs::lda / ldb is then the pitch between consecutive k).  Its half of a stage
+// is 64 k-rows of 256 operand rows (512 bytes), filled by the same load-to-LDS instructions (two k-rows each), and the
+// fragments come out of it with ds_read_b64_tr_b16, where the reference has ldmatrix.trans
+// (src/arch/copy/ldmatrix.jl:18-48): lane 16 g + s points at k-row 8 g + s / 4 (+ 4, + 32, + 36 for the other three
+// reads) and m = m0 + 4 (s % 4), and the four reads hand it the k of row m0 + s that chunks g and g + 4 of a K-major
+// row would.  The 32-byte piece index of a k-row is XORed with (row % 4) | 4 ((row / 8) % 2), so that the eight row
+// pieces the 32 lanes of one pass read lie in eight bank groups (the layout of gemm_mfma_lds_tile.hpp).  Whole-line
+// stages of the 16-bit types on the 256 x 256 tile, eight waves, no bias, whole tiles.
+template <typename In, typename Out, int WGN, bool kBias = false, bool kRagged = false, int TILE = 256, int AMAJ = 0, int BMAJ = 0>
 __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_256_w4(GemmArgs p) {
+    static_assert(!(AMAJ || BMAJ) || (In::kRow == 128 && In::kBytes == 2 && TILE == 256 && WGN == 4 && !kBias && !kRagged),
+                  "operands that are not K-major: whole-line stages of the 16-bit types, eight waves, plain whole tiles");
     static_assert(!kRagged || (!kBias && In::kRow == 128), "ragged tiles: the plain whole-line form");
     static_assert(TILE == 256 || (TILE == 128 && WGN == 2 && In::kRow == 128 && !kBias), "128 x 128 tiles: the whole-line form, 2 x 2 waves, plain or ragged");
     constexpr int BM = TILE, BN = TILE, kRow = In::kRow, CPR = kRow / 16, STAGES = In::kRing, SPS = In::SPS;
@@ -233,8 +259,11 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
     constexpr int BAR = TILE == 128 ? 3 : 7;  // the MFMA group after which the waves meet
     constexpr int RW = BM / NW, LD = RW / RPI;  // per wave and stage: RW rows, LD load-to-LDS instructions per operand
     typedef typename In::frag frag;
+    typedef std::conditional_t<AMAJ != 0, W4TrFrag, frag> frag_a;
+    typedef std::conditional_t<BMAJ != 0, W4TrFrag, frag> frag_b;
+    constexpr int RPA = AMAJ ? 4 : RPF, RPB = BMAJ ? 4 : RPF;  // LDS reads per fragment of A and of B
 
-    extern __shared__ u32x4 smem[];
+    extern __shared__ __attribute__((aligned(256))) u32x4 smem[];
 
     int tm, tn;
     split_of_block(p);
@@ -248,8 +277,9 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
     // instruction lands in physical chunk l % 4 of row l / 4 of a 16-row group; wave w brings rows
     // RW w .. RW w + RW - 1 of each operand.
     const int lrow = wave * RW + lane / CPR, lch = (lane % CPR) ^ swz<CPR>(lane / CPR);
-    const char* const a_tile = static_cast<const char*>(p.A) + (int64_t)tm * BM * pitch_a;  // uniform
-    const char* const b_tile = static_cast<const char*>(p.B) + (int64_t)tn * BN * pitch_b;
+    // (an M-major operand: its tile starts BM elements further along the row of every k)
+    const char* const a_tile = static_cast<const char*>(p.A) + (AMAJ ? (int64_t)tm * BM * In::kBytes : (int64_t)tm * BM * pitch_a);  // uniform
+    const char* const b_tile = static_cast<const char*>(p.B) + (BMAJ ? (int64_t)tn * BN * In::kBytes : (int64_t)tn * BN * pitch_b);
     constexpr uint32_t kStageBytes = STAGE * 16, kATileBytes = BM * CPR * 16;
 
     f32x4 acc[MI][NI];
@@ -260,7 +290,8 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
 
     const int nstages = (int)(((int64_t)p.K * In::kBytes) / kRow);
     const int nsteps = nstages / SPS;
-    frag fa[MI], fb[NI];
+    frag_a fa[MI];
+    frag_b fb[NI];
 
     typedef __attribute__((address_space(3))) void* lptr_t;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(lptr_t)smem;  // LDS byte address of the ring
@@ -270,8 +301,16 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
     // instruction's first lane.
     uint32_t voff[2 * LD];
     [[maybe_unused]] const int last_a = p.M - 1 - tm * BM, last_b = p.N - 1 - tn * BN;  // ragged: the last row of the operand, counted from the tile's first
+    // an M-major (N-major) operand: instruction q % LD of wave w brings k-rows 8 w + 2 (q % LD) + lane / 32 of the stage,
+    // lane l the 16-byte piece that belongs in physical slot l % 32 of its k-row
+    auto tr_swz = [](int krow) { return (krow & 3) | (((krow >> 3) & 1) << 2); };
 #pragma unroll
     for (int q = 0; q < 2 * LD; ++q) {
+        if ((q < LD && AMAJ) || (q >= LD && BMAJ)) {
+            const int krow = wave * (64 / NW) + 2 * (q % LD) + lane / 32, p16 = lane % 32, l32 = (p16 >> 1) ^ tr_swz(krow);
+            voff[q] = (uint32_t)(krow * (q < LD ? pitch_a : pitch_b) + (l32 * 2 + (p16 & 1)) * 16);
+            continue;
+        }
         int row = lrow + RPI * (q % LD);
         if constexpr (kRagged) row = min(row, q < LD ? last_a : last_b);
         voff[q] = (uint32_t)(row * (q < LD ? pitch_a : pitch_b) + lch * 16);
@@ -282,7 +321,9 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
     auto dma1 = [&](int g, int ring_slot, auto qc) __attribute__((always_inline)) {
         constexpr int Q = decltype(qc)::value;
         const int gr = g + g0 >= nstages ? g + g0 - nstages : g + g0;
-        const char* const base = uniform_ptr((Q < LD ? a_tile : b_tile) + (int64_t)gr * kRow);
+        // (stage gr of a K-major operand starts kRow bytes further along every row, of an M-major one 64 k-rows further down)
+        const char* const base = uniform_ptr(Q < LD ? a_tile + (AMAJ ? (int64_t)gr * 64 * pitch_a : (int64_t)gr * kRow)
+                                                    : b_tile + (BMAJ ? (int64_t)gr * 64 * pitch_b : (int64_t)gr * kRow));
         const uint32_t dst = __builtin_amdgcn_readfirstlane(lds0 + ring_slot * kStageBytes + (Q < LD ? 0 : kATileBytes) +
                                                             (uint32_t)(wave * RW + RPI * (Q % LD)) * kRow);
         const uint32_t lane_off = voff[Q];  // (a captured array element cannot be an asm operand of a generic lambda)
@@ -303,10 +344,21 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
     const uint32_t fb_byte = lds0 + kATileBytes + wn0 * kRow + frag_lane;
     // whole-line stages: the lane's second chunk, kq + 4, of the same row
     [[maybe_unused]] const uint32_t hi_delta = (uint32_t)((((kq + 4) ^ swz<CPR>(r16)) - (kq ^ swz<CPR>(r16))) * 16);
+    // transposed operand halves: the byte address of this lane's first read of 16-row block 0 in ring slot 0; block BLK
+    // XORs BLK << 5 into it (the piece index is swizzled, and a wave tile starts at a piece index whose low bits are clear)
+    [[maybe_unused]] const int tr_fx = ((r16 >> 2) & 3) | ((kq & 1) << 2);
+    [[maybe_unused]] const uint32_t ta_byte = lds0 + (uint32_t)((8 * kq + (r16 >> 2)) * 512 + (wm0 / 128) * 256 + ((((wm0 / 16) & 7) ^ tr_fx) << 5) + 8 * (r16 & 3));
+    [[maybe_unused]] const uint32_t tb_byte = lds0 + kATileBytes + (uint32_t)((8 * kq + (r16 >> 2)) * 512 + (wn0 / 128) * 256 + ((((wn0 / 16) & 7) ^ tr_fx) << 5) + 8 * (r16 & 3));
     // the fragment of 16-row block BLK for the k-step whose stages start at byte offsets o0 (, o1)
-    auto load_frag = [&](frag& f, uint32_t base, auto blk_c, uint32_t o0, uint32_t o1) __attribute__((always_inline)) {
+    auto load_frag = [&](auto& f, uint32_t base, auto blk_c, uint32_t o0, uint32_t o1) __attribute__((always_inline)) {
         constexpr int OFF = 16 * kRow * decltype(blk_c)::value;
-        if constexpr (kLine) {
+        if constexpr (std::is_same_v<std::remove_reference_t<decltype(f)>, W4TrFrag>) {
+            const uint32_t at = (base ^ (uint32_t)(decltype(blk_c)::value << 5)) + o0;  // (stage offsets are multiples of 64 KiB)
+            f.q0 = lds_read_tr8<0>(at);
+            f.q1 = lds_read_tr8<4 * 512>(at);
+            f.q2 = lds_read_tr8<32 * 512>(at);
+            f.q3 = lds_read_tr8<36 * 512>(at);
+        } else if constexpr (kLine) {
             f.lo = lds_read16<OFF>(base + o0);
             f.hi = lds_read16<OFF>(base + hi_delta + o0);
         } else if constexpr (SPS == 1) {
@@ -328,12 +380,12 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
     else __builtin_amdgcn_s_waitcnt(0x0F70);
     MOYE_BARRIER()
     static_for<MI>([&](auto ic) __attribute__((always_inline)) {
-        load_frag(fa[decltype(ic)::value], fa_byte, ic, 0, kStageBytes);
-        if (decltype(ic)::value == 3) __builtin_amdgcn_s_waitcnt(0xC07F);  // at most 15 reads in flight
+        load_frag(fa[decltype(ic)::value], AMAJ ? ta_byte : fa_byte, ic, 0, kStageBytes);
+        if (decltype(ic)::value % (AMAJ ? 2 : 4) == (AMAJ ? 1 : 3)) __builtin_amdgcn_s_waitcnt(0xC07F);  // at most 15 reads in flight
     });
     static_for<NI>([&](auto jc) __attribute__((always_inline)) {
-        load_frag(fb[decltype(jc)::value], fb_byte, jc, 0, kStageBytes);
-        if (decltype(jc)::value % 4 == 3) __builtin_amdgcn_s_waitcnt(0xC07F);
+        load_frag(fb[decltype(jc)::value], BMAJ ? tb_byte : fb_byte, jc, 0, kStageBytes);
+        if (decltype(jc)::value % (BMAJ ? 2 : 4) == (BMAJ ? 1 : 3)) __builtin_amdgcn_s_waitcnt(0xC07F);
     });
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
 
@@ -371,9 +423,25 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
             constexpr int i = MOYE_I(P), j = MOYE_J(P);
             // B0 is followed by NI + 1 fragment reads, B1 by NI; a stricter count costs nothing where the
             // older reads are hundreds of clocks old (fp8: two reads per fragment, 32-clock MFMAs)
-            if (P == 0) __builtin_amdgcn_s_waitcnt(0xC07F | (((NI + 1) * RPF < 12 ? (NI + 1) * RPF : 12) << 8));
-            if (P == H) __builtin_amdgcn_s_waitcnt(0xC07F | ((NI * RPF < 12 ? NI * RPF : 12) << 8));
-            In::mma(fb[j], fa[i], acc[i][j]);
+            // (in reads: B1 .. B(NI-1) and the last two A fragments follow B0)
+            constexpr int after_b0 = (NI - 1) * RPB + 2 * RPA, after_b1 = (NI - 2) * RPB + 2 * RPA;
+            if (P == 0) __builtin_amdgcn_s_waitcnt(0xC07F | ((after_b0 < 12 ? after_b0 : 12) << 8));
+            if (P == H) __builtin_amdgcn_s_waitcnt(0xC07F | ((after_b1 < 12 ? after_b1 : 12) << 8));
+            if constexpr (AMAJ || BMAJ) {
+                // (the halves of a transposed fragment are joined where the MFMA names them: the register allocator puts
+                // the two reads' results side by side; the build checks that nothing else touches them)
+                auto lo = [](const auto& f) __attribute__((always_inline)) {
+                    if constexpr (std::is_same_v<std::remove_cv_t<std::remove_reference_t<decltype(f)>>, W4TrFrag>) return __builtin_shufflevector(f.q0, f.q1, 0, 1, 2, 3);
+                    else return f.lo;
+                };
+                auto hi = [](const auto& f) __attribute__((always_inline)) {
+                    if constexpr (std::is_same_v<std::remove_cv_t<std::remove_reference_t<decltype(f)>>, W4TrFrag>) return __builtin_shufflevector(f.q2, f.q3, 0, 1, 2, 3);
+                    else return f.hi;
+                };
+                In::mma4(lo(fb[j]), hi(fb[j]), lo(fa[i]), hi(fa[i]), acc[i][j]);
+            } else {
+                In::mma(fb[j], fa[i], acc[i][j]);
+            }
             if (P == BAR) {
                 // my share of step s+1 has landed and all my fragment reads have returned (the last were
                 // issued eight MFMAs ago); after the barrier that holds for everybody
@@ -400,10 +468,11 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
             }
             if (MORE) {
                 constexpr int A0 = H * (NI - 1), B0 = (MI - 2) * NI;
-                if constexpr (P >= A0 && P < A0 + H) load_frag(fa[i], fa_byte, MOYE_BLK(i), o0, o1);  // the rows of the first phase: last use
-                if constexpr (P >= H * NI && P < B0 && (P + 1) % NI == 0) load_frag(fa[i], fa_byte, MOYE_BLK(i), o0, o1);  // a whole row: its end
-                if constexpr (P >= NPOS - 2) load_frag(fa[i], fa_byte, MOYE_BLK(i), o0, o1);          // the last two rows: last use
-                if constexpr (P >= B0 && ((P - B0) & 1)) load_frag(fb[(P - B0) / 2], fb_byte, MOYE_BLK((P - B0) / 2), o0, o1);
+                const uint32_t fa_at = AMAJ ? ta_byte : fa_byte, fb_at = BMAJ ? tb_byte : fb_byte;
+                if constexpr (P >= A0 && P < A0 + H) load_frag(fa[i], fa_at, MOYE_BLK(i), o0, o1);  // the rows of the first phase: last use
+                if constexpr (P >= H * NI && P < B0 && (P + 1) % NI == 0) load_frag(fa[i], fa_at, MOYE_BLK(i), o0, o1);  // a whole row: its end
+                if constexpr (P >= NPOS - 2) load_frag(fa[i], fa_at, MOYE_BLK(i), o0, o1);          // the last two rows: last use
+                if constexpr (P >= B0 && ((P - B0) & 1)) load_frag(fb[(P - B0) / 2], fb_at, MOYE_BLK((P - B0) / 2), o0, o1);
             }
         });
         slot = slot_n;
@@ -436,10 +505,10 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
     store_c_tile<Out, MI, NI, false, kRagged, kBias, kBias || kRagged>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
 }
 
-template <typename In, typename Out, int WGN, bool kBias = false, bool kRagged = false, int TILE = 256>
+template <typename In, typename Out, int WGN, bool kBias = false, bool kRagged = false, int TILE = 256, int AMAJ = 0, int BMAJ = 0>
 static int32_t launch256_w4(const GemmArgs& a, hipStream_t st) {
     constexpr int kLds = In::kRing * (TILE + TILE) * In::kRow;  // all 160 KiB, or 128 KiB for two whole-line stages (64 KiB on 128 x 128 tiles)
-    auto kern = gemm_mfma_tn_256_w4<In, Out, WGN, kBias, kRagged, TILE>;
+    auto kern = gemm_mfma_tn_256_w4<In, Out, WGN, kBias, kRagged, TILE, AMAJ, BMAJ>;
     static LdsCap cap;
     if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
     kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1)), dim3(128 * WGN), kLds, st>>>(a);
@@ -447,8 +516,29 @@ static int32_t launch256_w4(const GemmArgs& a, hipStream_t st) {
     return MOYE_OK;
 }
 
+// operands that keep their M- (N-) major form: the eight-wave whole-line forms of the 16-bit types, plain calls
+template <typename In, int AMAJ, int BMAJ>
+static int32_t launch256_w4_majors(int32_t out_dt, const GemmArgs& a, hipStream_t st) {
+    switch (out_dt) {
+        case MOYE_F32: return launch256_w4<In, OutF32, 4, false, false, 256, AMAJ, BMAJ>(a, st);
+        case MOYE_F16: return launch256_w4<In, OutF16, 4, false, false, 256, AMAJ, BMAJ>(a, st);
+        case MOYE_BF16: return launch256_w4<In, OutBF16, 4, false, false, 256, AMAJ, BMAJ>(a, st);
+        default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: MFMA kernels write f32, f16 or bf16, not %s", dtype_name(out_dt));
+    }
+}
+
 template <typename In, int WGN>
 static int32_t launch256_w4_out(int32_t out_dt, const GemmArgs& a, hipStream_t st) {
+    if (a.xcd_swizzle & (kGemmAMajorM | kGemmBMajorN)) {
+        if constexpr (In::kRow == 128 && In::kBytes == 2 && WGN == 4) {
+            if ((a.xcd_swizzle & (kGemmRagged | kGemmEpiAddVec)) || a.ep_op != MOYE_MAP_IDENTITY)
+                return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the hand-ordered kernel takes operands that are not K-major in plain calls on whole tiles only");
+            const bool am = a.xcd_swizzle & kGemmAMajorM, bm = a.xcd_swizzle & kGemmBMajorN;
+            return am && bm ? launch256_w4_majors<In, 1, 1>(out_dt, a, st) : am ? launch256_w4_majors<In, 1, 0>(out_dt, a, st) : launch256_w4_majors<In, 0, 1>(out_dt, a, st);
+        } else {
+            return fail(MOYE_ERR_UNSUPPORTED, "gemm!: this schedule of the hand-ordered kernel takes K-major operands only");
+        }
+    }
     if (a.xcd_swizzle & kGemmRagged) {  // tiles that reach beyond M or N: the eight-wave whole-line forms
         if constexpr (In::kRow == 128 && WGN == 4) {
             if (a.ep_op != MOYE_MAP_IDENTITY || a.C) return fail(MOYE_ERR_UNSUPPORTED, "gemm!: ragged tiles of the hand-ordered kernel take no C and no epilogue operation");

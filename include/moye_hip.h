@@ -194,8 +194,10 @@ int32_t moye_map(int32_t op, const moye_tensor* dst, const moye_tensor* a, const
 
 /* bytes of device workspace this gemm! call needs: the K-major copies of MFMA operands whose unit stride
  * is not along K (NN / NT / TT problems, src/arch/mma/make_mma_ops.jl:253-265) and split_k * M * N fp32
- * partial products of a split-K call; 0 for plain TN, for UniversalFMA, and for f16 / bf16 operands of any major
- * that run on whole 256x256x64 or 128x128x64 tiles without K ranges (read where they lie).
+ * partial products of a split-K call; 0 for plain TN, for UniversalFMA, for f16 / bf16 operands of any major
+ * that run on whole 256x256x64 or 128x128x64 tiles without K ranges, and for fp8 / fp32 operands of any major on whole
+ * 256x256 tiles with 128 bytes of K per k-step (named so, or left to the library on problems of at least 128 such
+ * tiles) -- all read where they lie.  Assumes the plain epilogue of moye_gemm (see moye_gemm_ex_workspace_size).
  *   moye_gemm     keeps a workspace of its own per (device, stream): allocated by the first call on that stream
  *                 that needs one (a synchronous hipMalloc inside that call, so not under stream capture),
  *                 replaced by a larger one when a larger call comes, never freed inside a call.  Calls on
@@ -228,6 +230,11 @@ typedef struct {
 int32_t moye_gemm_ex(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A,
                      const moye_tensor* B, const moye_tensor* C, const moye_gemm_epilogue* ep,
                      void* workspace, size_t workspace_bytes, void* stream);
+/* moye_gemm_workspace_size for a call of moye_gemm_ex with this epilogue.  The two differ in one case: fp8 and fp32
+ * operands that are not K-major are read where they lie by plain calls only; with an element-wise operation in the
+ * epilogue they need their K-major copies.  (No counterpart in the reference: its kernels own no memory.) */
+int32_t moye_gemm_ex_workspace_size(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A,
+                                    const moye_tensor* B, const moye_gemm_epilogue* ep, size_t* bytes);
 
 /* gemm! for callers that cannot allocate device memory (code under HIP graph capture, serving loops, harnesses
  * that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as moye_gemm, bit for bit;

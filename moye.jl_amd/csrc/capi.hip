@@ -188,29 +188,46 @@ static int split_count(const moye_tiled_mma* mma, int64_t M, int64_t N, int64_t 
     return 1;
 }
 
-// An operand with its unit stride along M (N) instead of K needs no K-major copy when the call runs on the transposing
-// fragment reads of the load-to-LDS kernels (gemm_mfma_lds_tile.hpp): f16 / bf16 through the 16x16x32 atoms, whole
-// 256 x 256 x 64 tiles on eight waves or whole 128 x 128 x 64 tiles (named, or the library's own choice for a problem of
-// whole 128 x 128 tiles with more than 64 rows), the two-stage schedule, no K ranges; the operand dense along its rows
-// with a pitch of whole 16-byte pieces, and D 16-byte aligned (the guarded instances, which take any D, read K-major
-// operands only).
-static bool majors_run_natively(const moye_tiled_mma* mma, const Mat& A, const Mat& B, const Mat& D) {
-    if (mma->atom != MOYE_MFMA_F32_16x16x32_F16 && mma->atom != MOYE_MFMA_F32_16x16x32_BF16) return false;
+// An operand with its unit stride along M (N) instead of K needs no K-major copy when the call runs on kernels whose
+// fragment reads transpose: f16 / bf16 through the 16x16x32 atoms on whole 256 x 256 x 64 tiles on eight waves (the
+// hand-ordered kernel, gemm_mfma256w4.hip, for plain calls; the load-to-LDS kernel otherwise) or whole 128 x 128 x 64 tiles
+// (named, or the library's own choice for a problem of whole 128 x 128 tiles with more than 64 rows), the two-stage
+// schedule, no K ranges; fp8 and fp32 on the hand-ordered kernel's whole 256 x 256 tiles with 128 bytes of K per k-step
+// (named so, or the library's choice when the problem has at least 128 such tiles), plain calls; the operand dense
+// along its rows with a pitch of whole 16-byte pieces, and D 16-byte aligned (the guarded instances, which take any D,
+// read K-major operands only).  `force256`: the call must run on 256 x 256 tiles although it left the tile to the library.
+static bool majors_run_natively(const moye_tiled_mma* mma, const Mat& A, const Mat& B, const Mat& D, const moye_gemm_epilogue& ep,
+                                bool has_c, bool* force256 = nullptr) {
+    if (force256) *force256 = false;
+    const bool b16 = mma->atom == MOYE_MFMA_F32_16x16x32_F16 || mma->atom == MOYE_MFMA_F32_16x16x32_BF16;
+    const bool wide = mma->atom == MOYE_MFMA_F32_16x16x32_FP8 || mma->atom == MOYE_MFMA_F32_16x16x4_F32;  // hand-ordered kernel only
+    if (!b16 && !wide) return false;
     if ((mma->flags & (MOYE_GEMM_PINGPONG | MOYE_GEMM_WAVE4)) || mma->stages >= 3) return false;
     if (mma->split_k != 0 && mma->split_k != 1) return false;  // the K ranges of a split need not be whole k-tiles
     const int64_t M = A.rows, N = B.rows, K = A.cols;
+    const int eb = dtype_bytes(A.dtype);
     const int bm = mma->cta_tile_mnk[0], bn = mma->cta_tile_mnk[1], bk = mma->cta_tile_mnk[2];
-    if (K % 64) return false;
+    if ((K * eb) % 128) return false;
     const bool four_waves = mma->atom_layout_mnk[0] * mma->atom_layout_mnk[1] == 4;
-    const bool named256 = bm == 256 && bn == 256 && (bk == 0 || bk == 64) && !four_waves && M % 256 == 0 && N % 256 == 0;
-    const bool named128 = bm == 128 && bn == 128 && bk == 64 && M % 128 == 0 && N % 128 == 0;
+    const bool named256 = bm == 256 && bn == 256 && (b16 ? (bk == 0 || bk == 64) : bk * eb == 128) && !four_waves && M % 256 == 0 && N % 256 == 0;
+    const bool named128 = b16 && bm == 128 && bn == 128 && bk == 64 && M % 128 == 0 && N % 128 == 0;
     const bool chosen = bm == 0 && bn == 0 && bk == 0 && M > 64 && M % 128 == 0 && N % 128 == 0;
-    if (!named256 && !named128 && !chosen) return false;
+    if (wide) {
+        // (the hand-ordered kernel has neither an element-wise epilogue operation nor, for fp32 and fp8, another kernel behind it)
+        if (ep.op != MOYE_MAP_IDENTITY || mma->stages >= 2) return false;
+        const bool chosen256 = chosen && M % 256 == 0 && N % 256 == 0 && (M / 256) * (N / 256) >= 128;
+        if (!named256 && !chosen256) return false;
+        if (force256) *force256 = chosen256;
+    } else if (!named256 && !named128 && !chosen) {
+        return false;
+    }
+    (void)has_c;
     const int64_t d_pitch = D.cs == 1 ? D.rs : D.cs;
     if ((D.cs != 1 && D.rs != 1) || (d_pitch * dtype_bytes(D.dtype)) % 16 || reinterpret_cast<uintptr_t>(D.ptr) % 16) return false;
     for (const Mat* x : {&A, &B}) {
         if (x->cs == 1 || x->cols == 1) continue;  // K-major already
-        if (x->rs != 1 || (x->cs * 2) % 16 || reinterpret_cast<uintptr_t>(x->ptr) % 16 || x->cs < x->rows) return false;
+        if (x->rs != 1 || (x->cs * eb) % 16 || reinterpret_cast<uintptr_t>(x->ptr) % 16 || x->cs < x->rows) return false;
+        if (wide && 256 * x->cs * eb >= ((int64_t)1 << 32)) return false;  // (the kernel's 32-bit lane offsets)
     }
     return true;
 }
@@ -226,8 +243,8 @@ static size_t gemm_workspace_bytes_impl(const moye_tiled_mma* mma, const Mat& A,
     return n;
 }
 
-static size_t gemm_workspace_bytes(const moye_tiled_mma* mma, const Mat& A, const Mat& B, const Mat& D) {
-    return gemm_workspace_bytes_impl(mma, A, B, majors_run_natively(mma, A, B, D));
+static size_t gemm_workspace_bytes(const moye_tiled_mma* mma, const Mat& A, const Mat& B, const Mat& D, const moye_gemm_epilogue& ep) {
+    return gemm_workspace_bytes_impl(mma, A, B, majors_run_natively(mma, A, B, D, ep, false));
 }
 
 // transposes `m` (unit stride along its rows index) into ws as rows x K with K contiguous and rewrites `m`
@@ -294,7 +311,7 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
         return fail(MOYE_ERR_SHAPE, "gemm!: extents above 2^31-1 are not supported");
     if (A.rows == 0 || B.rows == 0) return MOYE_OK;
     const int M = (int)A.rows, N = (int)B.rows, K = (int)A.cols;
-    const int bm = mma->cta_tile_mnk[0], bn = mma->cta_tile_mnk[1], bk = mma->cta_tile_mnk[2];
+    int bm = mma->cta_tile_mnk[0], bn = mma->cta_tile_mnk[1], bk = mma->cta_tile_mnk[2];
 
     if (mma->atom == MOYE_MMA_UNIVERSAL_FMA) {
         if (mma->split_k > 1)
@@ -319,7 +336,8 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
     // along K are brought to the K-major form the kernels read (one tiled transpose each)
     char* ws = nullptr;
     std::unique_lock<std::mutex> ws_lock(g_ws_mutex, std::defer_lock);
-    const bool native_majors = majors_run_natively(mma, A, B, D);
+    bool force256 = false;
+    const bool native_majors = majors_run_natively(mma, A, B, D, ep, tC != nullptr, &force256);
     int major_flags = 0;  // which of the kernel's operands keep their M- (N-) major form
     if (native_majors) {
         if (A.cs != 1 && A.cols > 1) { major_flags |= kGemmAMajorM; A.rs = A.cs; A.cs = 1; }  // Mat::rs now holds the pitch between consecutive k
@@ -366,7 +384,12 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
         g.ep_x = X.ptr; g.ep_xdt = X.dtype; g.ep_xm = X.rs; g.ep_xn = X.cs;
     }
     // TiledMMA.atom_layout_mnk = how many waves tile the CTA along M and N (src/atom/mma.jl:84)
-    const int waves = mma->atom_layout_mnk[0] * mma->atom_layout_mnk[1];
+    int waves = mma->atom_layout_mnk[0] * mma->atom_layout_mnk[1];
+    if (force256) {  // fp8 / fp32 operands read where they lie: only the hand-ordered kernel's 256 x 256 tiles do that
+        bm = bn = 256;
+        bk = 128 / dtype_bytes(in_dt);
+        waves = 8;
+    }
     g.alpha = alpha;
     g.K = K;
     // The eight XCDs start their walk over K an eighth apart when the problem is large enough for the column blocks they
@@ -539,7 +562,13 @@ int32_t moye_copy_if(const moye_tensor* dst, const moye_tensor* src, const moye_
 
 int32_t moye_gemm_workspace_size(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A,
                                  const moye_tensor* B, size_t* bytes) {
-    if (!mma || !D || !A || !B || !bytes) return fail(MOYE_ERR_ARG, "moye_gemm_workspace_size: null argument");
+    const moye_gemm_epilogue plain = plain_epilogue(1.f);
+    return moye_gemm_ex_workspace_size(mma, D, A, B, &plain, bytes);
+}
+
+int32_t moye_gemm_ex_workspace_size(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A,
+                                    const moye_tensor* B, const moye_gemm_epilogue* ep, size_t* bytes) {
+    if (!mma || !D || !A || !B || !ep || !bytes) return fail(MOYE_ERR_ARG, "moye_gemm_workspace_size: null argument");
     *bytes = 0;
     Mat a, b, d;
     if (int32_t e = as_matrix(A, "A", &a)) return e;
@@ -547,7 +576,7 @@ int32_t moye_gemm_workspace_size(const moye_tiled_mma* mma, const moye_tensor* D
     if (int32_t e = as_matrix(D, "D", &d)) return e;
     for (Mat* x : {&a, &b, &d})
         if (x->rows == 1 && x->cs == 1) x->rs = x->cols;
-    if (!(mma->flags & MOYE_GEMM_NO_WORKSPACE)) *bytes = gemm_workspace_bytes(mma, a, b, d);
+    if (!(mma->flags & MOYE_GEMM_NO_WORKSPACE)) *bytes = gemm_workspace_bytes(mma, a, b, d, *ep);
     return MOYE_OK;
 }
 

@@ -520,7 +520,8 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         // fp32 operands: the hand-ordered kernel too (fp32 8192^3 152.8 TFLOP/s on whole-line stages, 147.8 on its ring of
         // 64-byte-row stages, 142.5 for the compiler-scheduled kernel)
         if (hand_ordered_on() && in_dt == MOYE_F32 && stages < 2 && a.ep_op == MOYE_MAP_IDENTITY && a.K % 16 == 0 &&
-            !(a.xcd_swizzle & (MOYE_GEMM_PINGPONG | kGemmRagged | kGemmAMajorM | kGemmBMajorN | kGemmAtom32)) &&
+            (!majors256 || (waves != 4 && bkb == 128)) &&
+            !(a.xcd_swizzle & (MOYE_GEMM_PINGPONG | kGemmRagged | kGemmAtom32)) &&
             256 * a.lda * eb < ((int64_t)1 << 32) && 256 * a.ldb * eb < ((int64_t)1 << 32))
             a.xcd_swizzle |= MOYE_GEMM_WAVE4;
         // hand-ordered kernel: k-steps of 64 bytes, or of 128 (fp8 always; the 16-bit types when the tile says so)

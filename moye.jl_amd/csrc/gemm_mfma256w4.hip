@@ -103,9 +103,25 @@ __device__ __forceinline__ u32x2 lds_read_tr8(uint32_t addr) {
     asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
     return v;
 }
+// The same for bytes (fp8): sixteen lanes that each point at eight consecutive bytes get back, in lane j, byte j % 8 of
+// the lanes 2 e + j / 8 (e = 0..7) (measured on the hardware with a one-off probe, like the 16-bit form).
+template <int OFF>
+__device__ __forceinline__ u32x2 lds_read_tr8_b8(uint32_t addr) {
+    u32x2 v;
+    asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+    return v;
+}
+template <int OFF>
+__device__ __forceinline__ uint32_t lds_read4(uint32_t addr) {
+    uint32_t v;
+    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+    return v;
+}
 // A fragment read out of an operand stage that is stored with its unit stride along M (N): four 8-byte halves, q0 q1
-// the lane's eight k of the first MFMA, q2 q3 those of the second (see the kernel's AMAJ / BMAJ).
+// the lane's k of the first 16 bytes of a K-major fragment, q2 q3 those of the second (see the kernel's AMAJ / BMAJ);
+// for fp32 eight single values.
 struct W4TrFrag { u32x2 q0, q1, q2, q3; };
+struct W4TrFrag32 { uint32_t e[8]; };
 
 // fragment = what one lane feeds to one MFMA group per operand; SPS = ring stages per k-step; kRow = bytes of K per row
 // of a stage, kRing = stages in the ring
@@ -159,11 +175,12 @@ struct W4FP8 : W4Ring64 {
 struct W4FP8L {
     static constexpr int kBytes = 1, SPS = 1, kRow = 128, kRing = 2;
     struct frag { u32x4 lo, hi; };
-    static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) {
-        const u32x8 a8 = __builtin_shufflevector(a.lo, a.hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        const u32x8 b8 = __builtin_shufflevector(b.lo, b.hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    static __device__ __forceinline__ void mma4(const u32x4& alo, const u32x4& ahi, const u32x4& blo, const u32x4& bhi, f32x4& c) {
+        const u32x8 a8 = __builtin_shufflevector(alo, ahi, 0, 1, 2, 3, 4, 5, 6, 7);
+        const u32x8 b8 = __builtin_shufflevector(blo, bhi, 0, 1, 2, 3, 4, 5, 6, 7);
         asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(a8), "v"(b8));
     }
+    static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) { mma4(a.lo, a.hi, b.lo, b.hi, c); }
 };
 // The 16-bit types on whole-line stages: chunk kq feeds the first MFMA of an accumulator, chunk kq + 4 the second.
 struct W4F16L {
@@ -219,17 +236,17 @@ struct W4F32 : W4Ring64 {
 struct W4F32L {
     static constexpr int kBytes = 4, SPS = 1, kRow = 128, kRing = 2;
     struct frag { u32x4 lo, hi; };
+    // four MFMAs from four values of each operand
+    static __device__ __forceinline__ void mma_quad(uint32_t a0, uint32_t a1, uint32_t a2, uint32_t a3, uint32_t b0, uint32_t b1, uint32_t b2, uint32_t b3, f32x4& c) {
+        asm volatile(
+            "v_mfma_f32_16x16x4_f32 %0, %1, %5, %0\n\tv_mfma_f32_16x16x4_f32 %0, %2, %6, %0\n\t"
+            "v_mfma_f32_16x16x4_f32 %0, %3, %7, %0\n\tv_mfma_f32_16x16x4_f32 %0, %4, %8, %0"
+            : "+a"(c)
+            : "v"(a0), "v"(a1), "v"(a2), "v"(a3), "v"(b0), "v"(b1), "v"(b2), "v"(b3));
+    }
     static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) {
-        asm volatile(
-            "v_mfma_f32_16x16x4_f32 %0, %1, %5, %0\n\tv_mfma_f32_16x16x4_f32 %0, %2, %6, %0\n\t"
-            "v_mfma_f32_16x16x4_f32 %0, %3, %7, %0\n\tv_mfma_f32_16x16x4_f32 %0, %4, %8, %0"
-            : "+a"(c)
-            : "v"(a.lo.x), "v"(a.lo.y), "v"(a.lo.z), "v"(a.lo.w), "v"(b.lo.x), "v"(b.lo.y), "v"(b.lo.z), "v"(b.lo.w));
-        asm volatile(
-            "v_mfma_f32_16x16x4_f32 %0, %1, %5, %0\n\tv_mfma_f32_16x16x4_f32 %0, %2, %6, %0\n\t"
-            "v_mfma_f32_16x16x4_f32 %0, %3, %7, %0\n\tv_mfma_f32_16x16x4_f32 %0, %4, %8, %0"
-            : "+a"(c)
-            : "v"(a.hi.x), "v"(a.hi.y), "v"(a.hi.z), "v"(a.hi.w), "v"(b.hi.x), "v"(b.hi.y), "v"(b.hi.z), "v"(b.hi.w));
+        mma_quad(a.lo.x, a.lo.y, a.lo.z, a.lo.w, b.lo.x, b.lo.y, b.lo.z, b.lo.w, c);
+        mma_quad(a.hi.x, a.hi.y, a.hi.z, a.hi.w, b.hi.x, b.hi.y, b.hi.z, b.hi.w, c);
     }
 };
 
@@ -240,12 +257,17 @@ struct W4F32L {
 // (src/arch/copy/ldmatrix.jl:18-48): lane 16 g + s points at k-row 8 g + s / 4 (+ 4, + 32, + 36 for the other three
 // reads) and m = m0 + 4 (s % 4), and the four reads hand it the k of row m0 + s that chunks g and g + 4 of a K-major
 // row would.  The 32-byte piece index of a k-row is XORed with (row % 4) | 4 ((row / 8) % 2), so that the eight row
-// pieces the 32 lanes of one pass read lie in eight bank groups (the layout of gemm_mfma_lds_tile.hpp).  Whole-line
-// stages of the 16-bit types on the 256 x 256 tile, eight waves, no bias, whole tiles.
+// pieces the 32 lanes of one pass read lie in eight bank groups (the layout of gemm_mfma_lds_tile.hpp).  fp8 the same
+// way through ds_read_b64_tr_b8 (k-rows of 256 bytes, 128 per stage; lane 16 g + s points at k-row 16 g + s / 2 (+ 8,
+// + 64, + 72) and m = m0 + 8 (s % 2); the 16-byte piece index XORed with row % 8).  fp32 needs no transposing read: an
+// MFMA takes one value per lane and operand, so a lane reads its eight values of row m0 + s with ds_read_b32 from
+// k-rows 4 g + e and 16 + 4 g + e (k-rows of 1 KiB, 32 per stage; the 64-byte piece index XORed with (row / 4) % 2, so
+// that the two k-rows the 32 lanes of a pass read lie in different halves of the banks).  Whole-line stages on the
+// 256 x 256 tile, eight waves, no bias, whole tiles.
 template <typename In, typename Out, int WGN, bool kBias = false, bool kRagged = false, int TILE = 256, int AMAJ = 0, int BMAJ = 0>
 __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_256_w4(GemmArgs p) {
-    static_assert(!(AMAJ || BMAJ) || (In::kRow == 128 && In::kBytes == 2 && TILE == 256 && WGN == 4 && !kBias && !kRagged),
-                  "operands that are not K-major: whole-line stages of the 16-bit types, eight waves, plain whole tiles");
+    static_assert(!(AMAJ || BMAJ) || (In::kRow == 128 && TILE == 256 && WGN == 4 && !kBias && !kRagged),
+                  "operands that are not K-major: whole-line stages, eight waves, plain whole tiles");
     static_assert(!kRagged || (!kBias && In::kRow == 128), "ragged tiles: the plain whole-line form");
     static_assert(TILE == 256 || (TILE == 128 && WGN == 2 && In::kRow == 128 && !kBias), "128 x 128 tiles: the whole-line form, 2 x 2 waves, plain or ragged");
     constexpr int BM = TILE, BN = TILE, kRow = In::kRow, CPR = kRow / 16, STAGES = In::kRing, SPS = In::SPS;
@@ -259,9 +281,16 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
     constexpr int BAR = TILE == 128 ? 3 : 7;  // the MFMA group after which the waves meet
     constexpr int RW = BM / NW, LD = RW / RPI;  // per wave and stage: RW rows, LD load-to-LDS instructions per operand
     typedef typename In::frag frag;
-    typedef std::conditional_t<AMAJ != 0, W4TrFrag, frag> frag_a;
-    typedef std::conditional_t<BMAJ != 0, W4TrFrag, frag> frag_b;
-    constexpr int RPA = AMAJ ? 4 : RPF, RPB = BMAJ ? 4 : RPF;  // LDS reads per fragment of A and of B
+    typedef std::conditional_t<In::kBytes == 4, W4TrFrag32, W4TrFrag> frag_t;
+    typedef std::conditional_t<AMAJ != 0, frag_t, frag> frag_a;
+    typedef std::conditional_t<BMAJ != 0, frag_t, frag> frag_b;
+    constexpr int RPT = In::kBytes == 4 ? 8 : 4;                    // LDS reads per fragment of a transposed operand
+    constexpr int RPA = AMAJ ? RPT : RPF, RPB = BMAJ ? RPT : RPF;  // LDS reads per fragment of A and of B
+    // transposed operand halves of a stage: k-rows of TROW bytes, a swizzle granule of 16 operand rows (GB bytes)
+    constexpr int TROW = 256 * In::kBytes, TKROWS = 128 / In::kBytes, TLPR = TROW / 16, TRPI = 64 / TLPR, GB = 16 * In::kBytes;
+    auto tr_swz = [](int krow) {
+        return In::kBytes == 2 ? ((krow & 3) | (((krow >> 3) & 1) << 2)) : In::kBytes == 1 ? (krow & 7) : ((krow >> 2) & 1);
+    };
 
     extern __shared__ __attribute__((aligned(256))) u32x4 smem[];
 
@@ -303,12 +332,13 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
     [[maybe_unused]] const int last_a = p.M - 1 - tm * BM, last_b = p.N - 1 - tn * BN;  // ragged: the last row of the operand, counted from the tile's first
     // an M-major (N-major) operand: instruction q % LD of wave w brings k-rows 8 w + 2 (q % LD) + lane / 32 of the stage,
     // lane l the 16-byte piece that belongs in physical slot l % 32 of its k-row
-    auto tr_swz = [](int krow) { return (krow & 3) | (((krow >> 3) & 1) << 2); };
+    static_assert(!(AMAJ || BMAJ) || TKROWS / NW == TRPI * LD, "a wave's k-rows of a transposed operand: LD instructions");
 #pragma unroll
     for (int q = 0; q < 2 * LD; ++q) {
         if ((q < LD && AMAJ) || (q >= LD && BMAJ)) {
-            const int krow = wave * (64 / NW) + 2 * (q % LD) + lane / 32, p16 = lane % 32, l32 = (p16 >> 1) ^ tr_swz(krow);
-            voff[q] = (uint32_t)(krow * (q < LD ? pitch_a : pitch_b) + (l32 * 2 + (p16 & 1)) * 16);
+            const int krow = wave * (TKROWS / NW) + TRPI * (q % LD) + lane / TLPR, p16 = lane % TLPR;
+            const int piece = (((p16 * 16 / GB) ^ tr_swz(krow)) * GB + (p16 * 16) % GB) / 16;  // the swizzle moves granules
+            voff[q] = (uint32_t)(krow * (q < LD ? pitch_a : pitch_b) + piece * 16);
             continue;
         }
         int row = lrow + RPI * (q % LD);
@@ -322,8 +352,8 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
         constexpr int Q = decltype(qc)::value;
         const int gr = g + g0 >= nstages ? g + g0 - nstages : g + g0;
         // (stage gr of a K-major operand starts kRow bytes further along every row, of an M-major one 64 k-rows further down)
-        const char* const base = uniform_ptr(Q < LD ? a_tile + (AMAJ ? (int64_t)gr * 64 * pitch_a : (int64_t)gr * kRow)
-                                                    : b_tile + (BMAJ ? (int64_t)gr * 64 * pitch_b : (int64_t)gr * kRow));
+        const char* const base = uniform_ptr(Q < LD ? a_tile + (AMAJ ? (int64_t)gr * TKROWS * pitch_a : (int64_t)gr * kRow)
+                                                    : b_tile + (BMAJ ? (int64_t)gr * TKROWS * pitch_b : (int64_t)gr * kRow));
         const uint32_t dst = __builtin_amdgcn_readfirstlane(lds0 + ring_slot * kStageBytes + (Q < LD ? 0 : kATileBytes) +
                                                             (uint32_t)(wave * RW + RPI * (Q % LD)) * kRow);
         const uint32_t lane_off = voff[Q];  // (a captured array element cannot be an asm operand of a generic lambda)
@@ -346,18 +376,39 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
     [[maybe_unused]] const uint32_t hi_delta = (uint32_t)((((kq + 4) ^ swz<CPR>(r16)) - (kq ^ swz<CPR>(r16))) * 16);
     // transposed operand halves: the byte address of this lane's first read of 16-row block 0 in ring slot 0; block BLK
     // XORs BLK << 5 into it (the piece index is swizzled, and a wave tile starts at a piece index whose low bits are clear)
-    [[maybe_unused]] const int tr_fx = ((r16 >> 2) & 3) | ((kq & 1) << 2);
-    [[maybe_unused]] const uint32_t ta_byte = lds0 + (uint32_t)((8 * kq + (r16 >> 2)) * 512 + (wm0 / 128) * 256 + ((((wm0 / 16) & 7) ^ tr_fx) << 5) + 8 * (r16 & 3));
-    [[maybe_unused]] const uint32_t tb_byte = lds0 + kATileBytes + (uint32_t)((8 * kq + (r16 >> 2)) * 512 + (wn0 / 128) * 256 + ((((wn0 / 16) & 7) ^ tr_fx) << 5) + 8 * (r16 & 3));
+    // (the lane's first k-row and its bytes inside the granule: 16-bit 8 kq + r16 / 4 and 8 (r16 % 4); bytes 16 kq + r16 / 2
+    // and 8 (r16 % 2); fp32 4 kq and 4 r16)
+    [[maybe_unused]] const int tr_row0 = In::kBytes == 2 ? 8 * kq + (r16 >> 2) : In::kBytes == 1 ? 16 * kq + (r16 >> 1) : 4 * kq;
+    [[maybe_unused]] const int tr_in = In::kBytes == 2 ? 8 * (r16 & 3) : In::kBytes == 1 ? 8 * (r16 & 1) : 4 * r16;
+    [[maybe_unused]] const int tr_fx = tr_swz(tr_row0);
+    [[maybe_unused]] const uint32_t ta_byte = lds0 + (uint32_t)(tr_row0 * TROW + ((wm0 / 16) ^ tr_fx) * GB + tr_in);
+    [[maybe_unused]] const uint32_t tb_byte = lds0 + kATileBytes + (uint32_t)(tr_row0 * TROW + ((wn0 / 16) ^ tr_fx) * GB + tr_in);
     // the fragment of 16-row block BLK for the k-step whose stages start at byte offsets o0 (, o1)
     auto load_frag = [&](auto& f, uint32_t base, auto blk_c, uint32_t o0, uint32_t o1) __attribute__((always_inline)) {
         constexpr int OFF = 16 * kRow * decltype(blk_c)::value;
         if constexpr (std::is_same_v<std::remove_reference_t<decltype(f)>, W4TrFrag>) {
-            const uint32_t at = (base ^ (uint32_t)(decltype(blk_c)::value << 5)) + o0;  // (stage offsets are multiples of 64 KiB)
-            f.q0 = lds_read_tr8<0>(at);
-            f.q1 = lds_read_tr8<4 * 512>(at);
-            f.q2 = lds_read_tr8<32 * 512>(at);
-            f.q3 = lds_read_tr8<36 * 512>(at);
+            const uint32_t at = (base ^ (uint32_t)(decltype(blk_c)::value * GB)) + o0;  // (stage offsets are multiples of 64 KiB)
+            if constexpr (In::kBytes == 2) {
+                f.q0 = lds_read_tr8<0>(at);
+                f.q1 = lds_read_tr8<4 * 512>(at);
+                f.q2 = lds_read_tr8<32 * 512>(at);
+                f.q3 = lds_read_tr8<36 * 512>(at);
+            } else {
+                f.q0 = lds_read_tr8_b8<0>(at);
+                f.q1 = lds_read_tr8_b8<8 * 256>(at);
+                f.q2 = lds_read_tr8_b8<64 * 256>(at);
+                f.q3 = lds_read_tr8_b8<72 * 256>(at);
+            }
+        } else if constexpr (std::is_same_v<std::remove_reference_t<decltype(f)>, W4TrFrag32>) {
+            const uint32_t at = (base ^ (uint32_t)(decltype(blk_c)::value * GB)) + o0;
+            f.e[0] = lds_read4<0>(at);
+            f.e[1] = lds_read4<1024>(at);
+            f.e[2] = lds_read4<2048>(at);
+            f.e[3] = lds_read4<3072>(at);
+            f.e[4] = lds_read4<16384>(at);
+            f.e[5] = lds_read4<16384 + 1024>(at);
+            f.e[6] = lds_read4<16384 + 2048>(at);
+            f.e[7] = lds_read4<16384 + 3072>(at);
         } else if constexpr (kLine) {
             f.lo = lds_read16<OFF>(base + o0);
             f.hi = lds_read16<OFF>(base + hi_delta + o0);
@@ -381,11 +432,11 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
     MOYE_BARRIER()
     static_for<MI>([&](auto ic) __attribute__((always_inline)) {
         load_frag(fa[decltype(ic)::value], AMAJ ? ta_byte : fa_byte, ic, 0, kStageBytes);
-        if (decltype(ic)::value % (AMAJ ? 2 : 4) == (AMAJ ? 1 : 3)) __builtin_amdgcn_s_waitcnt(0xC07F);  // at most 15 reads in flight
+        if ((decltype(ic)::value + 1) % (12 / RPA < 4 ? 12 / RPA : 4) == 0) __builtin_amdgcn_s_waitcnt(0xC07F);  // at most 15 reads in flight
     });
     static_for<NI>([&](auto jc) __attribute__((always_inline)) {
         load_frag(fb[decltype(jc)::value], BMAJ ? tb_byte : fb_byte, jc, 0, kStageBytes);
-        if (decltype(jc)::value % (BMAJ ? 2 : 4) == (BMAJ ? 1 : 3)) __builtin_amdgcn_s_waitcnt(0xC07F);
+        if ((decltype(jc)::value + 1) % (12 / RPB < 4 ? 12 / RPB : 4) == 0) __builtin_amdgcn_s_waitcnt(0xC07F);
     });
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
 
@@ -427,7 +478,18 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
             constexpr int after_b0 = (NI - 1) * RPB + 2 * RPA, after_b1 = (NI - 2) * RPB + 2 * RPA;
             if (P == 0) __builtin_amdgcn_s_waitcnt(0xC07F | ((after_b0 < 12 ? after_b0 : 12) << 8));
             if (P == H) __builtin_amdgcn_s_waitcnt(0xC07F | ((after_b1 < 12 ? after_b1 : 12) << 8));
-            if constexpr (AMAJ || BMAJ) {
+            if constexpr ((AMAJ || BMAJ) && In::kBytes == 4) {
+                auto el = [](const auto& f, auto tc) __attribute__((always_inline)) {
+                    constexpr int t = decltype(tc)::value;
+                    if constexpr (std::is_same_v<std::remove_cv_t<std::remove_reference_t<decltype(f)>>, W4TrFrag32>) return f.e[t];
+                    else if constexpr (t < 4) return f.lo[t];
+                    else return f.hi[t - 4];
+                };
+#define MOYE_EL(F, T) el(F, std::integral_constant<int, T>{})
+                In::mma_quad(MOYE_EL(fb[j], 0), MOYE_EL(fb[j], 1), MOYE_EL(fb[j], 2), MOYE_EL(fb[j], 3), MOYE_EL(fa[i], 0), MOYE_EL(fa[i], 1), MOYE_EL(fa[i], 2), MOYE_EL(fa[i], 3), acc[i][j]);
+                In::mma_quad(MOYE_EL(fb[j], 4), MOYE_EL(fb[j], 5), MOYE_EL(fb[j], 6), MOYE_EL(fb[j], 7), MOYE_EL(fa[i], 4), MOYE_EL(fa[i], 5), MOYE_EL(fa[i], 6), MOYE_EL(fa[i], 7), acc[i][j]);
+#undef MOYE_EL
+            } else if constexpr (AMAJ || BMAJ) {
                 // (the halves of a transposed fragment are joined where the MFMA names them: the register allocator puts
                 // the two reads' results side by side; the build checks that nothing else touches them)
                 auto lo = [](const auto& f) __attribute__((always_inline)) {
@@ -530,7 +592,7 @@ static int32_t launch256_w4_majors(int32_t out_dt, const GemmArgs& a, hipStream_
 template <typename In, int WGN>
 static int32_t launch256_w4_out(int32_t out_dt, const GemmArgs& a, hipStream_t st) {
     if (a.xcd_swizzle & (kGemmAMajorM | kGemmBMajorN)) {
-        if constexpr (In::kRow == 128 && In::kBytes == 2 && WGN == 4) {
+        if constexpr (In::kRow == 128 && WGN == 4) {
             if ((a.xcd_swizzle & (kGemmRagged | kGemmEpiAddVec)) || a.ep_op != MOYE_MAP_IDENTITY)
                 return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the hand-ordered kernel takes operands that are not K-major in plain calls on whole tiles only");
             const bool am = a.xcd_swizzle & kGemmAMajorM, bm = a.xcd_swizzle & kGemmBMajorN;

@@ -537,6 +537,17 @@ function gemm_workspace_size(mma::TiledMMADesc, D::MoYeArray, A::MoYeArray, B::M
     Int(n[])
 end
 
+# the same for a gemm_ex! call whose epilogue applies `op` (fp8 / fp32 operands that are not K-major are read where they
+# lie by plain calls only)
+function gemm_ex_workspace_size(mma::TiledMMADesc, D::MoYeArray, A::MoYeArray, B::MoYeArray; op::Int32 = MAP_IDENTITY)
+    n = Ref{Csize_t}(0)
+    ep = Ref(GemmEpilogue(1.0f0, 0.0f0, op, Int32(0), Ptr{Tensor}(C_NULL), 0.0))
+    check(ccall((:moye_gemm_ex_workspace_size, LIB), Int32,
+                (Ptr{TiledMMADesc}, Ptr{Tensor}, Ptr{Tensor}, Ptr{Tensor}, Ptr{GemmEpilogue}, Ptr{Csize_t}),
+                Ref(mma), Ref(Tensor(D)), Ref(Tensor(A)), Ref(Tensor(B)), ep, n))
+    Int(n[])
+end
+
 # ---- device memory without a Julia GPU package ------------------------------------------------
 function device_malloc(bytes::Integer)
     p = Ref{Ptr{Cvoid}}(C_NULL)

@@ -96,11 +96,15 @@ def gemm_release_workspace():
     check(lib().moye_gemm_release_workspace())
 
 
-def gemm_workspace_size(mma, D, A, B):
+def gemm_workspace_size(mma, D, A, B, epilogue=None):
     """Bytes of library-owned device workspace this gemm! call needs (K-major copies of operands that are not K-major,
-    partial products of a split-K call); 0 for a plain TN call."""
+    partial products of a split-K call); 0 for a plain TN call.  With `epilogue` (a moye_gemm_epilogue): for the
+    moye_gemm_ex call with that epilogue."""
     n = C.c_size_t()
-    check(lib().moye_gemm_workspace_size(C.byref(mma), C.byref(D), C.byref(A), C.byref(B), C.byref(n)))
+    if epilogue is None:
+        check(lib().moye_gemm_workspace_size(C.byref(mma), C.byref(D), C.byref(A), C.byref(B), C.byref(n)))
+    else:
+        check(lib().moye_gemm_ex_workspace_size(C.byref(mma), C.byref(D), C.byref(A), C.byref(B), C.byref(epilogue), C.byref(n)))
     return n.value
 
 

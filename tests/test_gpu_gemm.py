@@ -1549,26 +1549,75 @@ def test_bench_descriptor_every_cta_exact_on_integers(mh, out_dt):
 def test_operand_majors_every_cta_exact_on_integers(mh, majors):
     """4096 x 4096 x 512 on small integers with A stored M-major and / or B stored N-major (the reference's own operand
     layout: MoYeArray(Array) is column-major, src/array.jl:101-103), MOYE_GEMM_NO_WORKSPACE: all 256 CTA positions of the
-    256 x 256 tile on the transposing fragment reads, fp16 and bf16, bit for bit."""
+    256 x 256 tile on the transposing fragment reads, for fp16, bf16, fp8 and fp32 operands, named tile and the library's
+    choice, bit for bit."""
     from moye_hip import _lib
     M = N = 4096
     K = 512
     g = torch.Generator().manual_seed(1104)
-    for tdt, atom in ((torch.float16, mh.MFMA_F32_16x16x32_F16), (torch.bfloat16, mh.MFMA_F32_16x16x32_BF16)):
-        A = torch.randint(-2, 3, (M, K), generator=g).to(tdt)
-        B = torch.randint(-2, 3, (N, K), generator=g).to(tdt)
-        a_k, b_k = A.cuda(), B.cuda()
-        a_m, b_n = A.t().contiguous().cuda(), B.t().contiguous().cuda()
+    cases = [(torch.float16, mh.MFMA_F32_16x16x32_F16, 64, torch.float16), (torch.bfloat16, mh.MFMA_F32_16x16x32_BF16, 64, torch.bfloat16),
+             (torch.float32, mh.MFMA_F32_16x16x4_F32, 32, torch.float16)]
+    if hasattr(torch, "float8_e4m3fn"):
+        cases.append((torch.float8_e4m3fn, mh.MFMA_F32_16x16x32_FP8, 128, torch.bfloat16))
+    for tdt, atom, bk, out16 in cases:
+        A = torch.randint(-2, 3, (M, K), generator=g).float()
+        B = torch.randint(-2, 3, (N, K), generator=g).float()
+        a_k, b_k = A.to(tdt).cuda(), B.to(tdt).cuda()
+        a_m, b_n = A.t().contiguous().to(tdt).cuda(), B.t().contiguous().to(tdt).cuda()
         ta = T(a_m, (M, K), (1, M)) if majors[0] == "m" else T(a_k)
         tb = T(b_n, (N, K), (1, N)) if majors[1] == "n" else T(b_k)
-        want = a_k.float() @ b_k.float().t()
+        want = A.cuda() @ B.cuda().t()
         assert float(want.abs().max()) <= 2048
-        mma = mh.tiled_mma_desc(atom, atom_layout=(2, 4, 1), cta_tile=(256, 256, 64), flags=_lib.GEMM_NO_WORKSPACE)
-        for out_dt in (tdt, torch.float32):
-            d = torch.full((M, N), float("nan"), dtype=out_dt, device="cuda")
-            mh.gemm_(mma, T(d), ta, tb)
-            torch.cuda.synchronize()
-            assert torch.equal(d.float(), want), (tdt, out_dt, majors)
+        for cta in ((256, 256, bk), (0, 0, 0)):
+            mma = mh.tiled_mma_desc(atom, atom_layout=(2, 4, 1), cta_tile=cta, flags=_lib.GEMM_NO_WORKSPACE)
+            for out_dt in (out16, torch.float32):
+                d = torch.full((M, N), float("nan"), dtype=out_dt, device="cuda")
+                assert mh.gemm_workspace_size(mh.tiled_mma_desc(atom, atom_layout=(2, 4, 1), cta_tile=cta), T(d), ta, tb) == 0
+                mh.gemm_(mma, T(d), ta, tb)
+                torch.cuda.synchronize()
+                assert torch.equal(d.float(), want), (tdt, out_dt, majors, cta)
+        # with C, alpha and a column-major D (the kernel then runs the transposed problem: the majors swap with the operands)
+        C0 = torch.randint(-8, 9, (M, N), generator=g).float().cuda()
+        dt_ = torch.zeros(N, M, dtype=torch.float32, device="cuda")
+        mh.gemm_(mh.tiled_mma_desc(atom, atom_layout=(2, 4, 1), cta_tile=(256, 256, bk), flags=_lib.GEMM_NO_WORKSPACE),
+                 T(dt_, (M, N), (1, M)), ta, tb, T(C0), 0.5)
+        torch.cuda.synchronize()
+        assert torch.equal(dt_.t(), 0.5 * want + C0), (tdt, majors, "column-major D, C, alpha")
+
+
+def test_operand_majors_wide_types_random_and_workspace_rule(mh):
+    """fp8 and fp32 NN (A M-major, B N-major) at 4096^3 on random data against fp64 (tolerances 1e-2 / 1e-5), read where
+    they lie; and the one case that still copies: an element-wise epilogue operation, which moye_gemm_ex_workspace_size
+    announces and MOYE_GEMM_NO_WORKSPACE refuses."""
+    from moye_hip import _lib
+    M = N = K = 4096
+    g = torch.Generator().manual_seed(1106)
+    A = torch.randn(M, K, generator=g) / K ** 0.5
+    B = torch.randn(N, K, generator=g) / K ** 0.5
+    cases = [(torch.float32, mh.MFMA_F32_16x16x4_F32, 32, 1e-5, 1.0)]
+    if hasattr(torch, "float8_e4m3fn"):
+        cases.append((torch.float8_e4m3fn, mh.MFMA_F32_16x16x32_FP8, 128, 1e-2, 64.0))
+    for tdt, atom, bk, tol, scale in cases:
+        a_k, b_k = (A * scale).to(tdt).cuda(), (B * scale).to(tdt).cuda()
+        a_m, b_n = a_k.float().t().contiguous().to(tdt), b_k.float().t().contiguous().to(tdt)
+        c64 = a_k.double() @ b_k.double().t() if tdt == torch.float32 else a_k.float().double() @ b_k.float().double().t()
+        ta, tb = T(a_m, (M, K), (1, M)), T(b_n, (N, K), (1, N))
+        mma = mh.tiled_mma_desc(atom, atom_layout=(2, 4, 1), cta_tile=(256, 256, bk), flags=_lib.GEMM_NO_WORKSPACE)
+        d = torch.zeros(M, N, dtype=torch.float32, device="cuda")
+        mh.gemm_(mma, T(d), ta, tb)
+        torch.cuda.synchronize()
+        assert relerr(d, c64) <= tol, tdt
+        # an operation in the epilogue: the hand-ordered kernel has none, so these operands need their K-major copies
+        plain = mh.tiled_mma_desc(atom, atom_layout=(2, 4, 1), cta_tile=(256, 256, bk))
+        ep = mh.gemm_epilogue(alpha=1.0, op=_lib.MAP_ABS)
+        need = mh.gemm_workspace_size(plain, T(d), ta, tb, ep)
+        assert need >= 2 * M * K * a_k.element_size() and mh.gemm_workspace_size(plain, T(d), ta, tb) == 0
+        with pytest.raises(mh.MoyeError):
+            mh.gemm_ex_(mma, T(d), ta, tb, None, ep)
+        ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        mh.gemm_ex_(plain, T(d), ta, tb, None, ep, ws.data_ptr(), need)
+        torch.cuda.synchronize()
+        assert relerr(d, c64.abs()) <= tol, tdt
 
 
 def test_fp32_full_grid_exact_on_integers(mh):

@@ -160,9 +160,10 @@ int32_t moye_copy_if(const moye_tensor* dst, const moye_tensor* src, const moye_
  * A:(M,K), B:(N,K), C,D:(M,N);  D = alpha * (A * B') + C.   C may be NULL (zero-init
  * accumulator, `zeros!(tCrC)`); D may alias C.  With MOYE_MMA_UNIVERSAL_FMA the arithmetic is
  * the reference's exactly (product rounded in the input type, unfused add, k ascending).
- * Environment, read once per process, for tuning only (no result bit changes): MOYE_ROTATE_K=0|1 forces
- * whether the XCDs start their walk over K an eighth apart, MOYE_STREAM_D=0|1 whether D is written with
- * non-temporal stores; unset, the library decides by problem size and result type. */
+ * The library reads no environment variable: which kernel a call runs on follows from the descriptors alone
+ * (moye_gemm_explain prints it).  The MFMA kernels sum k in an order that is fixed per kernel instance and position
+ * in the grid, never by timing: a call repeated on the same device gives the same bits; the bits of an element may
+ * differ between problem shapes, descriptors or devices that put it on another kernel instance or tile. */
 int32_t moye_gemm(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A,
                   const moye_tensor* B, const moye_tensor* C, float alpha, void* stream);
 
@@ -230,6 +231,25 @@ typedef struct {
 int32_t moye_gemm_ex(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A,
                      const moye_tensor* B, const moye_tensor* C, const moye_gemm_epilogue* ep,
                      void* workspace, size_t workspace_bytes, void* stream);
+/* Which launches a gemm! call would make, as text; host arithmetic only: nothing is launched, allocated or asked of
+ * a device, the data pointers of the descriptors are compared but never dereferenced (any distinct, suitably aligned
+ * addresses will do).  No counterpart in the reference, whose kernels are written by its users; here it is how a
+ * caller -- and this library's tests -- see what the dispatcher decided.  `ep` may be NULL (the plain epilogue of
+ * moye_gemm).  `compute_units`: plan for a chip of that many CUs (32 to an XCD); 0 = the current device, or 256 CUs in 8
+ * XCDs when there is none.  One line per step:
+ *   plan: <n> step(s), workspace <bytes> bytes, <cus> CUs in <xcds> XCDs
+ *   step <i>: kernel <function<template arguments>> grid=<x>x<y> block=<lanes> lds=<bytes> tile=<m>x<n>x<k bytes>B
+ *             in=<dtype> out=<dtype> M= N= K= lda= ldb= ldd= ldd_n= A=<where> B= D= C= a16= b16= d16= split= alpha=
+ *             beta= op= flags=<names joined by |>
+ *   step <i>: kmajor_copy <where> (<rows> x <cols> <dtype>, strides ..) -> ws+<offset> (pitch <elements>)
+ *   step <i>: splitk_reduce split= M= N= partials=ws+<offset> D=<where> out=<dtype> alpha= beta= op=
+ * <where> is A+<bytes>, B+.., D+.., C+.. (inside the caller's arrays), ws+<bytes> (inside the workspace) or null;
+ * M, N, K, the pitches and the operand roles are the kernel's (a column-major D runs the transposed problem).
+ * MOYE_ERR_BUFFER when `cap` bytes do not hold the text. */
+int32_t moye_gemm_explain(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A,
+                          const moye_tensor* B, const moye_tensor* C, const moye_gemm_epilogue* ep,
+                          int32_t compute_units, char* out, size_t cap);
+
 /* moye_gemm_workspace_size for a call of moye_gemm_ex with this epilogue.  The two differ in one case: fp8 and fp32
  * operands that are not K-major are read where they lie by plain calls only; with an element-wise operation in the
  * epilogue they need their K-major copies.  (No counterpart in the reference: its kernels own no memory.) */

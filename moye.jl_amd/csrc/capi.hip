@@ -88,11 +88,18 @@ static int32_t library_workspace(size_t bytes, hipStream_t st, char** out) {
     MOYE_HIP_CHECK(hipGetDevice(&dev));
     LibWorkspace& w = g_ws[{dev, st}];
     if (bytes > w.bytes) {
+        // (at least twice the old size, so that calls that grow a little at a time park few buffers)
+        const size_t grown = std::max(bytes, 2 * w.bytes);
         void* p = nullptr;
-        MOYE_HIP_CHECK(hipMalloc(&p, bytes));
+        if (hipMalloc(&p, grown) != hipSuccess) {
+            (void)hipGetLastError();
+            MOYE_HIP_CHECK(hipMalloc(&p, bytes));
+            w.bytes = bytes;
+        } else {
+            w.bytes = grown;
+        }
         if (w.ptr) g_ws_parked.push_back(w.ptr);
         w.ptr = static_cast<char*>(p);
-        w.bytes = bytes;
     }
     *out = w.ptr;
     return MOYE_OK;
@@ -141,8 +148,8 @@ static size_t kmajor_bytes(const Mat& m) {
 // in s ranges 7.5 + the same with a workgroup's bytes divided by s, never under 10.7 (two launches).  Ranges are whole
 // lines of 2 KiB and more; at most two above M = 32 (every workgroup reads its range of all of A, which then dominates);
 // taken when the model gains a tenth, the fewest ranges within 5 % of the best.
-static int skinny_lines_split(int64_t M, int64_t N, int64_t k_bytes) {
-    if ((N + 31) / 32 >= 256) return 1;  // 32 rows of B per workgroup and every CU has one
+static int skinny_lines_split(int64_t M, int64_t N, int64_t k_bytes, int cus) {
+    if ((N + 31) / 32 >= cus) return 1;  // 32 rows of B per workgroup and every CU has one
     const double floor_us = (double)(N + M) * (double)k_bytes / 6.0e6;
     const double wg_us = (double)(16 + 16 * ((M + 15) / 16)) * (double)k_bytes / 64.0e3;
     const double t1 = 4.5 + std::max(floor_us, wg_us);
@@ -161,29 +168,85 @@ static int skinny_lines_split(int64_t M, int64_t N, int64_t k_bytes) {
     return 1;
 }
 
+// What the chip looks like to the planner (kernels.hpp).  Asked once per device; a host without a device plans for 256 / 8.
+DeviceShape device_shape_for(int cus) {
+    if (cus > 0) return DeviceShape{cus, cus >= 32 ? cus / 32 : 1};
+    return device_shape();
+}
+DeviceShape device_shape() {
+    static std::mutex m;
+    static DeviceShape cached[kMaxDevices];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return DeviceShape{256, 8};
+    }
+    std::lock_guard<std::mutex> lock(m);
+    if (cached[dev].cus == 0) {
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
+            (void)hipGetLastError();
+            return DeviceShape{256, 8};
+        }
+        cached[dev] = device_shape_for(cus);  // gfx950: 32 CUs to an XCD; a partitioned part shows fewer of both
+    }
+    return cached[dev];
+}
+
+GemmStep& GemmPlan::add_kernel(void (*kernel)(GemmArgs), const GemmArgs& a, unsigned grid_x, unsigned grid_y, unsigned block, int lds_bytes,
+                               LdsCap* cap, int tile_m, int tile_n, int tile_k_bytes, int in_dt, int out_dt, const char* fmt, ...) {
+    steps.emplace_back();
+    GemmStep& st = steps.back();
+    st.kind = GemmStep::kKernel;
+    st.kernel = kernel;
+    st.args = a;
+    st.args.xcds = shape.xcds;
+    st.grid_x = grid_x; st.grid_y = grid_y; st.block = block;
+    st.lds_bytes = lds_bytes;
+    st.cap = cap;
+    st.tile_m = tile_m; st.tile_n = tile_n; st.tile_k_bytes = tile_k_bytes;
+    st.in_dt = in_dt; st.out_dt = out_dt;
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(st.name, sizeof st.name, fmt, ap);
+    va_end(ap);
+    return st;
+}
+
+// What the library decides when tile, waves and K ranges are all left to it: one answer for the workspace sizing and the
+// dispatcher (gemm_choose, gemm_plan.hpp).  `open`: the call leaves all of that open and runs on the MFMA kernels that
+// take a choice (M above 64 or K not in whole 64-byte pieces; 16-byte pieces of K).
+struct LibraryChoice {
+    bool open = false;
+    TileChoice tile{128, 1, 0.0};
+};
+static LibraryChoice library_choice(const moye_tiled_mma* mma, int64_t M, int64_t N, int64_t K, int eb, int cus) {
+    LibraryChoice c;
+    const bool short_m = M <= 64 && (K * eb) % 64 == 0;
+    if (mma->split_k >= 0 || mma->cta_tile_mnk[0] || mma->cta_tile_mnk[1] || mma->cta_tile_mnk[2] || short_m || (K * eb) % 16) return c;
+    c.open = true;
+    c.tile = gemm_choose(M, N, K * eb, eb == 4, (mma->flags & MOYE_GEMM_NO_WORKSPACE) ? 1 : 16, cus);
+    return c;
+}
+
 // split_k of the descriptor -> number of K ranges.  Negative = the library chooses: with the tile left to the library too,
 // what the cost model of gemm_plan.hpp finds cheapest together with the tile (none where 256 x 256 tiles come out
 // cheapest); with a named tile, none when the problem's 128 x 128 tiles fill half the chip,
-// else the largest count up to 256 / tiles that cuts K into equal ranges of whole 128-byte pieces of at least 512 bytes.
-static int split_count(const moye_tiled_mma* mma, int64_t M, int64_t N, int64_t K, int eb) {
+// else the largest count up to cus / tiles that cuts K into equal ranges of whole 128-byte pieces of at least 512 bytes.
+static int split_count(const moye_tiled_mma* mma, int64_t M, int64_t N, int64_t K, int eb, int cus) {
     if (mma->split_k >= 0) return mma->split_k > 1 ? mma->split_k : 1;
     if (mma->flags & MOYE_GEMM_NO_WORKSPACE) return 1;  // nowhere to put the partial products
     if (M <= 64 && mma->cta_tile_mnk[0] == 0 && mma->cta_tile_mnk[1] == 0 && (K * eb) % 64 == 0) {
         // the short-M kernels (gemm_mfma_skinny.hip).  The one that stages lines through LDS is fastest unsplit when its
         // workgroups fill the chip (bf16 64 x 8192 x 8192: 30.4 us against 41.3 with two ranges and the second pass); the
         // one that loads into registers gains from two K ranges, which let a workgroup take 64 rows of B, from M = 33 on
-        if ((K * eb) % kSkinnyLineBytes == 0) return skinny_lines_split(M, N, K * eb);
-        return M > 32 && N % 64 == 0 && N / 64 >= 128 && (K * eb) % 256 == 0 ? 2 : 1;
+        if ((K * eb) % kSkinnyLineBytes == 0) return skinny_lines_split(M, N, K * eb, cus);
+        return M > 32 && N % 64 == 0 && N / 64 >= cus / 2 && (K * eb) % 256 == 0 ? 2 : 1;
     }
+    if (const LibraryChoice c = library_choice(mma, M, N, K, eb, cus); c.open) return c.tile.split;
     const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
-    if (mma->cta_tile_mnk[0] == 0 && mma->cta_tile_mnk[1] == 0 && mma->cta_tile_mnk[2] == 0 && (K * eb) % 16 == 0) {
-        const GemmPlan pl = gemm_plan(M, N, K * eb, eb == 4, M % 64 == 0 && N % 64 == 0 && (K * eb) % 128 == 0, 16);
-        const bool ragged = M % 256 || N % 256 || (K * eb) % 128;
-        if (((M + 255) / 256) * ((N + 255) / 256) >= 64 && gemm_plan_cost_256(M, N, K * eb, eb == 4, ragged) <= pl.us) return 1;
-        return pl.split;
-    }
-    if (tiles <= 0 || tiles >= 128) return 1;
-    for (int64_t s = std::min<int64_t>(256 / tiles, K); s >= 2; --s)
+    if (tiles <= 0 || tiles >= cus / 2) return 1;
+    for (int64_t s = std::min<int64_t>(cus / tiles, K); s >= 2; --s)
         if (K % s == 0 && ((K / s) * eb) % 128 == 0 && (K / s) * eb >= 512) return (int)s;
     return 1;
 }
@@ -233,32 +296,34 @@ static bool majors_run_natively(const moye_tiled_mma* mma, const Mat& A, const M
 }
 
 // K-major copies of A and B where needed, then the fp32 partial products of a split-K call
-static size_t gemm_workspace_bytes_impl(const moye_tiled_mma* mma, const Mat& A, const Mat& B, bool native) {
+static size_t gemm_workspace_bytes_impl(const moye_tiled_mma* mma, const Mat& A, const Mat& B, bool native, int cus) {
     if (mma->atom == MOYE_MMA_UNIVERSAL_FMA) return 0;
     size_t n = 0;
     if (!native && A.cs != 1 && A.cols > 1) n += kmajor_bytes(A);
     if (!native && B.cs != 1 && B.cols > 1) n += kmajor_bytes(B);
-    const int split = split_count(mma, A.rows, B.rows, A.cols, dtype_bytes(A.dtype));
+    const int split = split_count(mma, A.rows, B.rows, A.cols, dtype_bytes(A.dtype), cus);
     if (split > 1) n += (size_t)split * (size_t)A.rows * (size_t)B.rows * sizeof(float);
     return n;
 }
 
-static size_t gemm_workspace_bytes(const moye_tiled_mma* mma, const Mat& A, const Mat& B, const Mat& D, const moye_gemm_epilogue& ep) {
-    return gemm_workspace_bytes_impl(mma, A, B, majors_run_natively(mma, A, B, D, ep, false));
+static size_t gemm_workspace_bytes(const moye_tiled_mma* mma, const Mat& A, const Mat& B, const Mat& D, const moye_gemm_epilogue& ep, int cus) {
+    return gemm_workspace_bytes_impl(mma, A, B, majors_run_natively(mma, A, B, D, ep, false), cus);
 }
 
-// transposes `m` (unit stride along its rows index) into ws as rows x K with K contiguous and rewrites `m`
-static int32_t make_kmajor(Mat* m, char* ws, hipStream_t st) {
+// A step that transposes `m` (unit stride along its rows index) into ws as rows x K with K contiguous; rewrites `m`
+static void plan_kmajor_copy(Mat* m, char* ws, GemmPlan& plan) {
     const int eb = dtype_bytes(m->dtype);
     const int64_t pitch_e = ((m->cols * eb + 15) / 16 * 16) / eb;
-    moye_tensor src{}, dst{};
-    src.ptr = m->ptr; src.dtype = m->dtype; src.rank = 2;
+    plan.steps.emplace_back();
+    GemmStep& st = plan.steps.back();
+    st.kind = GemmStep::kKMajorCopy;
+    moye_tensor& src = st.copy_src;
+    src.ptr = m->ptr; src.dtype = m->dtype; src.rank = 2; src.memspace = MOYE_GMEM;
     src.shape[0] = m->rows; src.shape[1] = m->cols; src.stride[0] = m->rs; src.stride[1] = m->cs;
-    dst = src;
-    dst.ptr = ws; dst.stride[0] = pitch_e; dst.stride[1] = 1;
-    if (int32_t e = copy_dispatch(nullptr, &dst, &src, st)) return e;
+    st.copy_dst = src;
+    st.copy_dst.ptr = ws; st.copy_dst.stride[0] = pitch_e; st.copy_dst.stride[1] = 1;
+    snprintf(st.name, sizeof st.name, "kmajor_copy");
     m->ptr = ws; m->rs = pitch_e; m->cs = 1;
-    return MOYE_OK;
 }
 
 // C as the 256 x 256 kernels' epilogue likes it: unit stride along the kernel's n, rows that start on 16-byte boundaries
@@ -275,8 +340,7 @@ static moye_gemm_epilogue plain_epilogue(float alpha) {
     return e;
 }
 
-// `caller_ws` / `caller_ws_bytes`: the workspace when the caller brings one (it must hold what
-// moye_gemm_workspace_size reports); with caller_ws == nullptr the library's own is used.
+
 // the epilogue operand as the 256 x 256 kernels like it: unit stride along the kernel's n, 16-byte aligned rows (or one row)
 static bool operand_rows_in_16_byte_pieces(const GemmArgs& g) {
     if (!g.ep_x || g.ep_xn != 1) return false;
@@ -284,10 +348,15 @@ static bool operand_rows_in_16_byte_pieces(const GemmArgs& g) {
     return reinterpret_cast<uintptr_t>(g.ep_x) % 16 == 0 && (g.ep_xm * eb) % 16 == 0;
 }
 
-static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const moye_tensor* tA,
-                         const moye_tensor* tB, const moye_tensor* tC, const moye_gemm_epilogue& ep, char* caller_ws,
-                         size_t caller_ws_bytes, hipStream_t st) {
+// gemm!(mma, D, A, B, C) with the epilogue `ep` as a list of launches.  Pure host arithmetic on the descriptors: nothing
+// is launched, allocated or asked of a device (plan.shape says what the chip looks like).  `workspace(bytes, &ptr)` is
+// asked once, and only when the call needs a workspace, for `bytes` bytes: the caller's buffer, the library's own, the
+// static scratch array, or -- for moye_gemm_explain -- an address that is never dereferenced.
+template <typename WorkspaceSource>
+static int32_t gemm_plan_build(const moye_tiled_mma* mma, const moye_tensor* tD, const moye_tensor* tA, const moye_tensor* tB,
+                               const moye_tensor* tC, const moye_gemm_epilogue& ep, WorkspaceSource&& workspace, GemmPlan& plan) {
     if (!mma) return fail(MOYE_ERR_ARG, "gemm!: null TiledMMA descriptor");
+    const int cus = plan.shape.cus;
     const float alpha = ep.alpha;
     if (ep.beta == 0.f) tC = nullptr;  // axpby!'s iszero(b): C is not read
     if (ep.op < MOYE_MAP_IDENTITY || ep.op > MOYE_MAP_ABS) return fail(MOYE_ERR_UNSUPPORTED, "gemm!: unknown epilogue operation %d", ep.op);
@@ -319,9 +388,14 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
         if (ep.op != MOYE_MAP_IDENTITY || (tC && ep.beta != 1.f))
             return fail(MOYE_ERR_UNSUPPORTED, "gemm!: UniversalFMA accumulates onto C as the reference does (src/algorithm/blas.jl:39-88): "
                                               "beta other than 0 or 1 and element-wise epilogue operations belong to the MFMA atoms");
-        UArgs u{A.ptr, B.ptr, tC ? C.ptr : nullptr, D.ptr, M, N, K, A.rs, A.cs, B.rs, B.cs,
-                C.rs, C.cs, D.rs, D.cs, alpha, A.dtype, B.dtype, tC ? C.dtype : D.dtype, D.dtype};
-        return gemm_universal_dispatch(bm, bn, bk, u, st);
+        plan.steps.emplace_back();
+        GemmStep& st = plan.steps.back();
+        st.kind = GemmStep::kUniversal;
+        st.uargs = UArgs{A.ptr, B.ptr, tC ? C.ptr : nullptr, D.ptr, M, N, K, A.rs, A.cs, B.rs, B.cs,
+                         C.rs, C.cs, D.rs, D.cs, alpha, A.dtype, B.dtype, tC ? C.dtype : D.dtype, D.dtype};
+        st.ubm = bm; st.ubn = bn; st.ubk = bk;
+        snprintf(st.name, sizeof st.name, "gemm_universal<%d,%d,%d>", bm, bn, bk);
+        return MOYE_OK;
     }
     const int32_t in_dt = atom_input_dtype(mma->atom);
     if (in_dt < 0) return fail(MOYE_ERR_UNSUPPORTED, "gemm!: unknown MMA atom %d", mma->atom);
@@ -335,7 +409,6 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
     // NN / NT / TT (the naming of src/arch/mma/make_mma_ops.jl:253-265): operands whose unit stride is not
     // along K are brought to the K-major form the kernels read (one tiled transpose each)
     char* ws = nullptr;
-    std::unique_lock<std::mutex> ws_lock(g_ws_mutex, std::defer_lock);
     bool force256 = false;
     const bool native_majors = majors_run_natively(mma, A, B, D, ep, tC != nullptr, &force256);
     int major_flags = 0;  // which of the kernel's operands keep their M- (N-) major form
@@ -343,28 +416,21 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
         if (A.cs != 1 && A.cols > 1) { major_flags |= kGemmAMajorM; A.rs = A.cs; A.cs = 1; }  // Mat::rs now holds the pitch between consecutive k
         if (B.cs != 1 && B.cols > 1) { major_flags |= kGemmBMajorN; B.rs = B.cs; B.cs = 1; }
     }
-    if (const size_t ws_bytes = gemm_workspace_bytes_impl(mma, A, B, native_majors)) {
+    plan.workspace_bytes = gemm_workspace_bytes_impl(mma, A, B, native_majors, cus);
+    if (plan.workspace_bytes) {
         if (mma->flags & MOYE_GEMM_NO_WORKSPACE)
             return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the MFMA kernels need K-major A and B (stride 1 along K, the 'TN' form), split_k needs room "
                                               "for its partial products, and MOYE_GEMM_NO_WORKSPACE forbids the use of a workspace");
-        if (caller_ws) {
-            if (ws_bytes > caller_ws_bytes)
-                return fail(MOYE_ERR_ARG, "gemm!: this call needs a workspace of %zu bytes, the one passed holds %zu", ws_bytes, caller_ws_bytes);
-            if (reinterpret_cast<uintptr_t>(caller_ws) % 256)
-                return fail(MOYE_ERR_ALIGN, "gemm!: the workspace must start on a 256-byte boundary");
-            ws = caller_ws;
-        } else {
-            ws_lock.lock();  // until every kernel of this call is enqueued
-            if (int32_t e = library_workspace(ws_bytes, st, &ws)) return e;
-        }
+        if (int32_t e = workspace(plan.workspace_bytes, &ws)) return e;
+        plan.workspace = ws;
         if (!native_majors && A.cs != 1 && A.cols > 1) {
             const size_t nb = kmajor_bytes(A);
-            if (int32_t e = make_kmajor(&A, ws, st)) return e;
+            plan_kmajor_copy(&A, ws, plan);
             ws += nb;
         }
         if (!native_majors && B.cs != 1 && B.cols > 1) {
             const size_t nb = kmajor_bytes(B);
-            if (int32_t e = make_kmajor(&B, ws, st)) return e;
+            plan_kmajor_copy(&B, ws, plan);
             ws += nb;
         }
     }
@@ -392,26 +458,26 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
     }
     g.alpha = alpha;
     g.K = K;
-    // The eight XCDs start their walk over K an eighth apart when the problem is large enough for the column blocks they
+    g.xcds = plan.shape.xcds;
+    // The XCDs start their walk over K a share of K apart when the problem is large enough for the column blocks they
     // ask memory for at one time to matter: more 256 x 256 tiles than CUs, or rows of 32 KiB and more (measured, 256 x 256
     // tile, same box, alternating runs: bf16 8192^3 1408 TFLOP/s against 1372, fp16 4096 x 4096 x 16384 +4 %; fp16 4096^3
     // 1333 against 1338, so not there)
-    static const int rotate_env = getenv("MOYE_ROTATE_K") ? atoi(getenv("MOYE_ROTATE_K")) : -1;
-    const bool rotate_k = rotate_env >= 0 ? rotate_env != 0
-                                          : ((int64_t)(M / 256) * (N / 256) > 256 || (int64_t)K * dtype_bytes(in_dt) >= 32768);
-    static const int stream_env = getenv("MOYE_STREAM_D") ? atoi(getenv("MOYE_STREAM_D")) : -1;
+    const bool rotate_k = (int64_t)(M / 256) * (N / 256) > cus || (int64_t)K * dtype_bytes(in_dt) >= 32768;
     // D written with non-temporal stores (measured, same box, alternating runs, ordinary -> non-temporal, TFLOP/s): fp16
     // 4096^3 fp16 out 1339 -> 1345, fp32 out 1285 -> 1253; fp16 8192^3 fp16 out 1382 -> 1401; bf16 8192^3 fp32 out 1412 ->
     // 1452; fp8 4096^3 bf16 out 2373 -> 2450, 8192^3 2760 -> 2745; fp16 2048^3 and 3072^3 +1.6 %.  So: 16-bit results
     // always, except for the fp8 kernel on more tiles than CUs; 32-bit results when the launch has more 256 x 256 tiles
     // than the chip has CUs (then the results of one round would sit in the L2s in place of the next round's operands;
     // in a single round they are better left there for the end of the kernel to write back)
-    const bool many_tiles = (int64_t)(M / 256) * (N / 256) > 256;
-    const bool stream_d = stream_env >= 0 ? stream_env != 0
-                          : dtype_bytes(D.dtype) == 2 ? !(in_dt == MOYE_F8E4M3 && many_tiles) : many_tiles;
-    g.xcd_swizzle = !(mma->flags & MOYE_GEMM_NO_XCD_SWIZZLE) | (mma->flags & 0xff00) | (atom32 ? kGemmAtom32 : 0) | (rotate_k ? kGemmRotateK : 0) |
-                    (stream_d ? kGemmStreamD : 0) | major_flags;
-    if (const int split = split_count(mma, M, N, K, dtype_bytes(in_dt)); split > 1) {
+    const bool many_tiles = (int64_t)(M / 256) * (N / 256) > cus;
+    const bool stream_d = dtype_bytes(D.dtype) == 2 ? !(in_dt == MOYE_F8E4M3 && many_tiles) : many_tiles;
+    g.flags = !(mma->flags & MOYE_GEMM_NO_XCD_SWIZZLE) | (mma->flags & 0xff00) | (atom32 ? kGemmAtom32 : 0) | (rotate_k ? kGemmRotateK : 0) |
+              (stream_d ? kGemmStreamD : 0) | major_flags;
+    // tile and K ranges, where both are left to the library, are one decision (gemm_choose)
+    const LibraryChoice lib = force256 ? LibraryChoice{} : library_choice(mma, M, N, K, dtype_bytes(in_dt), cus);
+    const TileChoice* lib_tile = lib.open ? &lib.tile : nullptr;
+    if (const int split = split_count(mma, M, N, K, dtype_bytes(in_dt), cus); split > 1) {
         // K is cut into `split` equal ranges, all in one launch (gridDim.y); each range writes its fp32 product, compact and
         // row-major, into the workspace; a second pass sums the ranges in ascending order, applies alpha and C and converts
         const int eb = dtype_bytes(in_dt);
@@ -422,40 +488,163 @@ static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const
         float* P = reinterpret_cast<float*>(ws);
         GemmArgs r = g;  // the epilogue belongs to the second pass
         r.C = tC ? C.ptr : nullptr; r.ldc_m = C.rs; r.ldc_n = C.cs; r.D = D.ptr; r.ldd = D.rs; r.ldd_n = D.cs;
+        r.M = M; r.N = N;
         g.alpha = 1.f; g.beta = 0.f; g.ep_op = MOYE_MAP_IDENTITY; g.ep_x = nullptr;
         g.K = Ks; g.M = M; g.N = N; g.lda = A.rs; g.ldb = B.rs; g.ldd = N; g.C = nullptr;
         g.A = A.ptr; g.B = B.ptr; g.D = P;
         g.split = split; g.split_ab = (int64_t)Ks * eb; g.split_d = (int64_t)M * N * (int64_t)sizeof(float);
-        g.xcd_swizzle &= ~kGemmStreamD;  // the partial products are read back at once
-        if (int32_t e = gemm_mfma_tn_dispatch(in_dt, MOYE_F32, bm, bn, bk, waves, mma->stages, g, st)) return e;
-        return splitk_reduce_dispatch(P, split, M, N, r, D.dtype, st);
+        g.flags &= ~kGemmStreamD;  // the partial products are read back at once
+        if (int32_t e = gemm_mfma_tn_dispatch(in_dt, MOYE_F32, bm, bn, bk, waves, mma->stages, g, plan, lib_tile)) return e;
+        plan.steps.emplace_back();
+        GemmStep& st = plan.steps.back();
+        st.kind = GemmStep::kSplitKReduce;
+        st.partials = P; st.split = split; st.args = r; st.out_dt = D.dtype; st.in_dt = MOYE_F32;
+        snprintf(st.name, sizeof st.name, "splitk_reduce");
+        return MOYE_OK;
     }
     if (D.cs == 1) {  // row-major D
         g.A = A.ptr; g.B = B.ptr; g.M = M; g.N = N; g.lda = A.rs; g.ldb = B.rs; g.ldd = D.rs;
         g.C = tC ? C.ptr : nullptr; g.ldc_m = C.rs; g.ldc_n = C.cs; g.D = D.ptr;
-        if (rows_in_16_byte_pieces(g.C, g.ldc_m, g.ldc_n, D.dtype)) g.xcd_swizzle |= kGemmRowC;
-        if (operand_rows_in_16_byte_pieces(g)) g.xcd_swizzle |= kGemmEpiRowX;
-        if (g.ep_op == MOYE_MAP_ADD && (!g.ep_x || g.ep_xm == 0 || g.ep_xn == 0)) g.xcd_swizzle |= kGemmEpiAddVec;  // a bias
-        return gemm_mfma_tn_dispatch(in_dt, D.dtype, bm, bn, bk, waves, mma->stages, g, st);
+        if (rows_in_16_byte_pieces(g.C, g.ldc_m, g.ldc_n, D.dtype)) g.flags |= kGemmRowC;
+        if (operand_rows_in_16_byte_pieces(g)) g.flags |= kGemmEpiRowX;
+        if (g.ep_op == MOYE_MAP_ADD && (!g.ep_x || g.ep_xm == 0 || g.ep_xn == 0)) g.flags |= kGemmEpiAddVec;  // a bias
+        return gemm_mfma_tn_dispatch(in_dt, D.dtype, bm, bn, bk, waves, mma->stages, g, plan, lib_tile);
     }
     if (D.rs == 1 && bm == 0 && bn == 0 && M <= 64 && ((int64_t)K * dtype_bytes(in_dt)) % 64 == 0) {
         // column-major D with a short A: the short-M kernel writes D through both of its strides
         g.A = A.ptr; g.B = B.ptr; g.M = M; g.N = N; g.lda = A.rs; g.ldb = B.rs; g.ldd = 1; g.ldd_n = D.cs;
         g.C = tC ? C.ptr : nullptr; g.ldc_m = C.rs; g.ldc_n = C.cs; g.D = D.ptr;
-        return gemm_mfma_skinny_dispatch(in_dt, D.dtype, g, st);
+        return gemm_mfma_skinny_dispatch(in_dt, D.dtype, g, plan);
     }
     if (D.rs == 1) {  // column-major D: D' = B * A' is row-major
         g.A = B.ptr; g.B = A.ptr; g.M = N; g.N = M; g.lda = B.rs; g.ldb = A.rs; g.ldd = D.cs;
         g.C = tC ? C.ptr : nullptr; g.ldc_m = C.cs; g.ldc_n = C.rs; g.D = D.ptr;
         std::swap(g.ep_xm, g.ep_xn);  // the kernel's m is the caller's n
-        g.xcd_swizzle = (g.xcd_swizzle & ~(kGemmAMajorM | kGemmBMajorN)) | ((major_flags & kGemmAMajorM) ? kGemmBMajorN : 0) |
-                        ((major_flags & kGemmBMajorN) ? kGemmAMajorM : 0);
-        if (rows_in_16_byte_pieces(g.C, g.ldc_m, g.ldc_n, D.dtype)) g.xcd_swizzle |= kGemmRowC;
-        if (operand_rows_in_16_byte_pieces(g)) g.xcd_swizzle |= kGemmEpiRowX;
-        if (g.ep_op == MOYE_MAP_ADD && (!g.ep_x || g.ep_xm == 0 || g.ep_xn == 0)) g.xcd_swizzle |= kGemmEpiAddVec;
-        return gemm_mfma_tn_dispatch(in_dt, D.dtype, bn, bm, bk, waves, mma->stages, g, st);
+        g.flags = (g.flags & ~(kGemmAMajorM | kGemmBMajorN)) | ((major_flags & kGemmAMajorM) ? kGemmBMajorN : 0) |
+                  ((major_flags & kGemmBMajorN) ? kGemmAMajorM : 0);
+        if (rows_in_16_byte_pieces(g.C, g.ldc_m, g.ldc_n, D.dtype)) g.flags |= kGemmRowC;
+        if (operand_rows_in_16_byte_pieces(g)) g.flags |= kGemmEpiRowX;
+        if (g.ep_op == MOYE_MAP_ADD && (!g.ep_x || g.ep_xm == 0 || g.ep_xn == 0)) g.flags |= kGemmEpiAddVec;
+        // (the library's choice was priced for (M, N); the cost model is symmetric in them)
+        return gemm_mfma_tn_dispatch(in_dt, D.dtype, bn, bm, bk, waves, mma->stages, g, plan, lib_tile);
     }
     return fail(MOYE_ERR_UNSUPPORTED, "gemm!: D needs a unit stride along M or N");
+}
+
+// Enqueues the steps of a plan on `st`, in order.  The only part of gemm! that talks to the device.
+static int32_t gemm_plan_run(const GemmPlan& plan, hipStream_t st) {
+    for (const GemmStep& s : plan.steps) {
+        switch (s.kind) {
+            case GemmStep::kKernel:
+                if (s.cap)
+                    if (int32_t e = raise_lds_cap(*s.cap, reinterpret_cast<const void*>(s.kernel), s.lds_bytes)) return e;
+                hipLaunchKernelGGL(s.kernel, dim3(s.grid_x, s.grid_y), dim3(s.block), s.lds_bytes, st, s.args);
+                MOYE_HIP_CHECK(hipGetLastError());
+                break;
+            case GemmStep::kKMajorCopy:
+                if (int32_t e = copy_dispatch(nullptr, &s.copy_dst, &s.copy_src, st)) return e;
+                break;
+            case GemmStep::kSplitKReduce:
+                if (int32_t e = splitk_reduce_dispatch(s.partials, s.split, s.args.M, s.args.N, s.args, s.out_dt, st)) return e;
+                break;
+            case GemmStep::kUniversal:
+                if (int32_t e = gemm_universal_dispatch(s.ubm, s.ubn, s.ubk, s.uargs, st)) return e;
+                break;
+        }
+    }
+    return MOYE_OK;
+}
+
+// `caller_ws` / `caller_ws_bytes`: the workspace when the caller brings one (it must hold what moye_gemm_workspace_size
+// reports); with caller_brings_ws == false the library's own per-stream buffer is used.
+static int32_t gemm_impl(const moye_tiled_mma* mma, const moye_tensor* tD, const moye_tensor* tA,
+                         const moye_tensor* tB, const moye_tensor* tC, const moye_gemm_epilogue& ep, bool caller_brings_ws, char* caller_ws,
+                         size_t caller_ws_bytes, hipStream_t st) {
+    std::unique_lock<std::mutex> ws_lock(g_ws_mutex, std::defer_lock);
+    GemmPlan plan;
+    plan.shape = device_shape();
+    auto workspace = [&](size_t bytes, char** out) -> int32_t {
+        if (caller_brings_ws) {
+            if (bytes > caller_ws_bytes)
+                return fail(MOYE_ERR_ARG, "gemm!: this call needs a workspace of %zu bytes, the one passed holds %zu", bytes, caller_ws_bytes);
+            if (reinterpret_cast<uintptr_t>(caller_ws) % 256)
+                return fail(MOYE_ERR_ALIGN, "gemm!: the workspace must start on a 256-byte boundary");
+            *out = caller_ws;
+            return MOYE_OK;
+        }
+        ws_lock.lock();  // until every kernel of this call is enqueued
+        return library_workspace(bytes, st, out);
+    };
+    if (int32_t e = gemm_plan_build(mma, tD, tA, tB, tC, ep, workspace, plan)) return e;
+    return gemm_plan_run(plan, st);
+}
+
+// "A+123" / "ws+456": where a pointer of a step lies, relative to the caller's arrays or the workspace
+static void where(char* out, size_t cap, const void* p, const GemmPlan& plan, const moye_tensor* tA, const moye_tensor* tB, const moye_tensor* tD,
+                  const moye_tensor* tC) {
+    const char* q = static_cast<const char*>(p);
+    if (!p) { snprintf(out, cap, "null"); return; }
+    if (plan.workspace && q >= plan.workspace && q < plan.workspace + plan.workspace_bytes) { snprintf(out, cap, "ws+%lld", (long long)(q - plan.workspace)); return; }
+    struct { const char* name; const moye_tensor* t; } arrays[] = {{"A", tA}, {"B", tB}, {"D", tD}, {"C", tC}};
+    for (auto& a : arrays) {
+        if (!a.t || !a.t->ptr) continue;
+        const char* base = static_cast<const char*>(a.t->ptr);
+        const int64_t bytes = tensor_cosize(*a.t) * dtype_bytes(a.t->dtype);
+        if (q >= base && q < base + bytes) { snprintf(out, cap, "%s+%lld", a.name, (long long)(q - base)); return; }
+    }
+    snprintf(out, cap, "?");
+}
+
+static std::string flag_names(int f) {
+    std::string s;
+    auto add = [&](bool on, const char* n) { if (on) { if (!s.empty()) s += '|'; s += n; } };
+    add(f & 1, "xcd_order"); add(f & MOYE_GEMM_PINGPONG, "pingpong"); add(f & MOYE_GEMM_PREDICATE, "predicate"); add(f & MOYE_GEMM_WAVE4, "hand_ordered");
+    add(f & kGemmAtom32, "atom32"); add(f & kGemmRotateK, "rotate_k"); add(f & kGemmStreamD, "stream_d"); add(f & kGemmRowC, "row_c");
+    add(f & kGemmAMajorM, "a_m_major"); add(f & kGemmBMajorN, "b_n_major"); add(f & kGemmEpiRowX, "row_x"); add(f & kGemmRagged, "ragged");
+    add(f & kGemmEpiAddVec, "add_vec");
+    return s.empty() ? "0" : s;
+}
+
+static std::string explain_plan(const GemmPlan& plan, const moye_tensor* tA, const moye_tensor* tB, const moye_tensor* tD, const moye_tensor* tC) {
+    std::string out;
+    char line[1024], wa[48], wb[48], wd[48], wc[48];
+    snprintf(line, sizeof line, "plan: %zu step(s), workspace %zu bytes, %d CUs in %d XCDs\n", plan.steps.size(), plan.workspace_bytes, plan.shape.cus, plan.shape.xcds);
+    out += line;
+    for (size_t i = 0; i < plan.steps.size(); ++i) {
+        const GemmStep& s = plan.steps[i];
+        switch (s.kind) {
+            case GemmStep::kKernel: {
+                const GemmArgs& a = s.args;
+                where(wa, sizeof wa, a.A, plan, tA, tB, tD, tC); where(wb, sizeof wb, a.B, plan, tA, tB, tD, tC);
+                where(wd, sizeof wd, a.D, plan, tA, tB, tD, tC); where(wc, sizeof wc, a.C, plan, tA, tB, tD, tC);
+                snprintf(line, sizeof line,
+                         "step %zu: kernel %s grid=%ux%u block=%u lds=%d tile=%dx%dx%dB in=%s out=%s M=%d N=%d K=%d lda=%lld ldb=%lld ldd=%lld ldd_n=%lld "
+                         "A=%s B=%s D=%s C=%s a16=%d b16=%d d16=%d split=%d alpha=%g beta=%g op=%d flags=%s\n",
+                         i, s.name, s.grid_x, s.grid_y, s.block, s.lds_bytes, s.tile_m, s.tile_n, s.tile_k_bytes, dtype_name(s.in_dt), dtype_name(s.out_dt), a.M, a.N,
+                         a.K, (long long)a.lda, (long long)a.ldb, (long long)a.ldd, (long long)a.ldd_n, wa, wb, wd, wc,
+                         (int)(reinterpret_cast<uintptr_t>(a.A) % 16 == 0), (int)(reinterpret_cast<uintptr_t>(a.B) % 16 == 0),
+                         (int)(reinterpret_cast<uintptr_t>(a.D) % 16 == 0), a.split > 1 ? a.split : 1, (double)a.alpha, (double)a.beta, a.ep_op,
+                         flag_names(a.flags).c_str());
+                break;
+            }
+            case GemmStep::kKMajorCopy:
+                where(wa, sizeof wa, s.copy_src.ptr, plan, tA, tB, tD, tC); where(wd, sizeof wd, s.copy_dst.ptr, plan, tA, tB, tD, tC);
+                snprintf(line, sizeof line, "step %zu: kmajor_copy %s (%lld x %lld %s, strides %lld,%lld) -> %s (pitch %lld)\n", i, wa, (long long)s.copy_src.shape[0],
+                         (long long)s.copy_src.shape[1], dtype_name(s.copy_src.dtype), (long long)s.copy_src.stride[0], (long long)s.copy_src.stride[1], wd,
+                         (long long)s.copy_dst.stride[0]);
+                break;
+            case GemmStep::kSplitKReduce:
+                where(wa, sizeof wa, s.partials, plan, tA, tB, tD, tC); where(wd, sizeof wd, s.args.D, plan, tA, tB, tD, tC);
+                snprintf(line, sizeof line, "step %zu: splitk_reduce split=%d M=%d N=%d partials=%s D=%s out=%s alpha=%g beta=%g op=%d\n", i, s.split, s.args.M, s.args.N, wa,
+                         wd, dtype_name(s.out_dt), (double)s.args.alpha, (double)s.args.beta, s.args.ep_op);
+                break;
+            case GemmStep::kUniversal:
+                snprintf(line, sizeof line, "step %zu: kernel %s M=%d N=%d K=%d\n", i, s.name, s.uargs.M, s.uargs.N, s.uargs.K);
+                break;
+        }
+        out += line;
+    }
+    return out;
 }
 
 // Average launch time of `iters` back-to-back launches, HIP events on the launch stream.
@@ -464,8 +653,15 @@ static int32_t time_launches(F&& launch, hipStream_t st, int warmup, int iters, 
     if (!ms || iters <= 0 || warmup < 0) return fail(MOYE_ERR_ARG, "timing: bad arguments");
     for (int i = 0; i < warmup; ++i)
         if (int32_t e = launch()) return e;
-    hipEvent_t t0, t1;
+    hipEvent_t t0 = nullptr, t1 = nullptr;
     MOYE_HIP_CHECK(hipEventCreate(&t0));
+    struct Events {  // destroyed on every way out
+        hipEvent_t &a, &b;
+        ~Events() {
+            if (a) (void)hipEventDestroy(a);
+            if (b) (void)hipEventDestroy(b);
+        }
+    } events{t0, t1};
     MOYE_HIP_CHECK(hipEventCreate(&t1));
     MOYE_HIP_CHECK(hipEventRecord(t0, st));
     int32_t err = MOYE_OK;
@@ -474,8 +670,6 @@ static int32_t time_launches(F&& launch, hipStream_t st, int warmup, int iters, 
     MOYE_HIP_CHECK(hipEventSynchronize(t1));
     float total = 0.f;
     MOYE_HIP_CHECK(hipEventElapsedTime(&total, t0, t1));
-    (void)hipEventDestroy(t0);
-    (void)hipEventDestroy(t1);
     if (err) return err;
     *ms = total / (float)iters;
     return MOYE_OK;
@@ -493,7 +687,7 @@ int32_t moye_copy(const moye_tiled_copy* tc, const moye_tensor* dst, const moye_
 
 int32_t moye_gemm(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A, const moye_tensor* B,
                   const moye_tensor* C, float alpha, void* stream) {
-    return gemm_impl(mma, D, A, B, C, plain_epilogue(alpha), nullptr, 0, static_cast<hipStream_t>(stream));
+    return gemm_impl(mma, D, A, B, C, plain_epilogue(alpha), false, nullptr, 0, static_cast<hipStream_t>(stream));
 }
 
 int32_t moye_gemm_ex(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A, const moye_tensor* B,
@@ -502,9 +696,7 @@ int32_t moye_gemm_ex(const moye_tiled_mma* mma, const moye_tensor* D, const moye
     if (!ep) return fail(MOYE_ERR_ARG, "moye_gemm_ex: null epilogue descriptor");
     if (!workspace && workspace_bytes) return fail(MOYE_ERR_ARG, "moye_gemm_ex: null workspace of %zu bytes", workspace_bytes);
     // a call that needs no workspace may pass none; one that needs it and passes none fails: this entry never allocates
-    alignas(256) static char nothing[256];
-    return gemm_impl(mma, D, A, B, C, *ep, workspace ? static_cast<char*>(workspace) : nothing, workspace_bytes,
-                     static_cast<hipStream_t>(stream));
+    return gemm_impl(mma, D, A, B, C, *ep, true, static_cast<char*>(workspace), workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
 int32_t moye_gemm_noalloc(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A, const moye_tensor* B,
@@ -519,13 +711,36 @@ int32_t moye_gemm_noalloc(const moye_tiled_mma* mma, const moye_tensor* D, const
     if (int32_t e = scratch_of_current_device(&ws)) return e;
     // every byte of the scratch a call reads it has written before (whole K-major copies, whole partial products), so
     // nothing needs clearing between calls
-    return gemm_impl(mma, D, A, B, C, plain_epilogue(alpha), ws, kScratchBytes, static_cast<hipStream_t>(stream));
+    return gemm_impl(mma, D, A, B, C, plain_epilogue(alpha), true, ws, kScratchBytes, static_cast<hipStream_t>(stream));
+}
+
+int32_t moye_gemm_explain(const moye_tiled_mma* mma, const moye_tensor* D, const moye_tensor* A, const moye_tensor* B,
+                          const moye_tensor* C, const moye_gemm_epilogue* ep, int32_t compute_units, char* out, size_t cap) {
+    if (!mma || !D || !A || !B || !out || cap == 0) return fail(MOYE_ERR_ARG, "moye_gemm_explain: null argument");
+    out[0] = 0;
+    GemmPlan plan;
+    plan.shape = device_shape_for(compute_units);
+    // the workspace of a plan that is only printed: an address nothing is read from or written to
+    auto workspace = [](size_t, char** p) -> int32_t {
+        *p = reinterpret_cast<char*>(uintptr_t(1) << 40);
+        return MOYE_OK;
+    };
+    const moye_gemm_epilogue plain = plain_epilogue(1.f);
+    if (int32_t e = gemm_plan_build(mma, D, A, B, C, ep ? *ep : plain, workspace, plan)) return e;
+    const std::string text = explain_plan(plan, A, B, D, C);
+    if (text.size() + 1 > cap) return fail(MOYE_ERR_BUFFER, "moye_gemm_explain: the plan takes %zu bytes of text, the buffer holds %zu", text.size() + 1, cap);
+    memcpy(out, text.c_str(), text.size() + 1);
+    return MOYE_OK;
 }
 
 int32_t moye_gemm_release_workspace(void) {
     std::lock_guard<std::mutex> lock(g_ws_mutex);
     int current = 0;
     MOYE_HIP_CHECK(hipGetDevice(&current));
+    struct Restore {  // the caller's device is current again on every way out
+        int dev;
+        ~Restore() { (void)hipSetDevice(dev); }
+    } restore{current};
     int last = -1;
     for (auto& kv : g_ws) {  // ordered by device: wait once for each device that holds a buffer
         if (kv.first.first != last) {
@@ -535,7 +750,6 @@ int32_t moye_gemm_release_workspace(void) {
         }
         if (kv.second.ptr) g_ws_parked.push_back(kv.second.ptr);
     }
-    MOYE_HIP_CHECK(hipSetDevice(current));
     g_ws.clear();
     for (void* p : g_ws_parked) (void)hipFree(p);
     g_ws_parked.clear();
@@ -576,7 +790,7 @@ int32_t moye_gemm_ex_workspace_size(const moye_tiled_mma* mma, const moye_tensor
     if (int32_t e = as_matrix(D, "D", &d)) return e;
     for (Mat* x : {&a, &b, &d})
         if (x->rows == 1 && x->cs == 1) x->rs = x->cols;
-    if (!(mma->flags & MOYE_GEMM_NO_WORKSPACE)) *bytes = gemm_workspace_bytes(mma, a, b, d, *ep);
+    if (!(mma->flags & MOYE_GEMM_NO_WORKSPACE)) *bytes = gemm_workspace_bytes(mma, a, b, d, *ep, device_shape().cus);
     return MOYE_OK;
 }
 
@@ -623,7 +837,7 @@ int32_t moye_time_gemm(const moye_tiled_mma* mma, const moye_tensor* D, const mo
                        const moye_tensor* C, float alpha, void* stream, int32_t warmup, int32_t iters,
                        float* ms_per_launch) {
     hipStream_t st = static_cast<hipStream_t>(stream);
-    return time_launches([&] { return gemm_impl(mma, D, A, B, C, plain_epilogue(alpha), nullptr, 0, st); }, st, warmup, iters, ms_per_launch);
+    return time_launches([&] { return gemm_impl(mma, D, A, B, C, plain_epilogue(alpha), false, nullptr, 0, st); }, st, warmup, iters, ms_per_launch);
 }
 
 int32_t moye_time_copy(const moye_tiled_copy* tc, const moye_tensor* dst, const moye_tensor* src, void* stream,

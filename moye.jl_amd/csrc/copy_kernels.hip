@@ -769,10 +769,9 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
             if (sb == 2) {
                 const uint16_t* s16 = reinterpret_cast<const uint16_t*>(s_);
                 uint16_t* d16 = reinterpret_cast<uint16_t*>(d_);
-                static const int rows16_env = getenv("MOYE_TRANSPOSE_ROWS") ? atoi(getenv("MOYE_TRANSPOSE_ROWS")) : -1;
                 // measured, TB/s, source-first / destination-first: 16384^2 5.32 / 5.75, 4096^2 x 16 6.25 / 6.47, 32768 x 4096
                 // 4.07 / 6.10; 2048^2 x 64 5.83 / 5.18, 4096 x 32768 5.65 / 4.46
-                if (tj % 8 == 0 && (rows16_env >= 0 ? rows16_env != 0 : (ni >= nj && ni >= 3072)))
+                if (tj % 8 == 0 && ni >= nj && ni >= 3072)
                     return launch_transpose16_rows<8>(s16, d16, lds_, ldd, ti, tj, st, bs, bd, batch);
                 if (ti % 8 == 0) return launch_transpose16<8>(s16, d16, lds_, ldd, ti, tj, st, bs, bd, batch);
                 if (ti % 4 == 0) return launch_transpose16<4>(s16, d16, lds_, ldd, ti, tj, st, bs, bd, batch);
@@ -785,9 +784,8 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
             // Destination rows first (transpose_lds_b32_rows) when the source's contiguous extent is at least the destination's
             // and 2048 or more; measured, TB/s, source-first / destination-first order: 16384^2 5.68 / 6.25, 12288^2 5.20 / 5.94,
             // 4096^2 x 16 5.81 / 6.02, 2048^2 x 64 6.30 / 6.48, 32768 x 4096 4.33 / 6.39; the other way round 4096 x 32768
-            // 5.58 / 5.08, 2048 x 65536 5.77 / 4.52, 1024^2 x 128 6.03 / 5.86.  MOYE_TRANSPOSE_ROWS=0|1 forces the choice (tuning).
-            static const int rows_env = getenv("MOYE_TRANSPOSE_ROWS") ? atoi(getenv("MOYE_TRANSPOSE_ROWS")) : -1;
-            if (tj % 4 == 0 && (rows_env >= 0 ? rows_env != 0 : (ni >= nj && ni >= 2048)))
+            // 5.58 / 5.08, 2048 x 65536 5.77 / 4.52, 1024^2 x 128 6.03 / 5.86.
+            if (tj % 4 == 0 && ni >= nj && ni >= 2048)
                 return launch_transpose_rows<4>(s32, d32, lds_, ldd, ti, tj, st, bs, bd, batch);
             if (ti % 4 == 0) return launch_transpose<true, 4>(s32, d32, lds_, ldd, ti, tj, st, bs, bd, batch);
             if (ti % 2 == 0) return launch_transpose<true, 2>(s32, d32, lds_, ldd, ti, tj, st, bs, bd, batch);

@@ -193,7 +193,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
     // C with unit stride along n and 16-byte aligned rows (kGemmRowC) is read the way D is written, in 128-bit pieces
     // of whole rows, all requested up front, and handed to the lanes through the patch (see mfma_epilogue.hpp)
     constexpr int NCH = PASS_ROWS * CR / 64, PASSES = MI / PASS_MI;
-    const bool row_c = p.C && (p.xcd_swizzle & kGemmRowC);
+    const bool row_c = p.C && (p.flags & kGemmRowC);
     u32x4 cw[PASSES][NCH];
     if (row_c) {
 #pragma unroll
@@ -259,45 +259,42 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
 }
 
 template <typename In, typename Out, int BM, int BN, int BKB, bool kEdge = false, int AT = 16>
-static int32_t launch(const GemmArgs& a, hipStream_t st) {
+static int32_t launch(const GemmArgs& a, GemmPlan& plan) {
     typedef typename Out::type OutT;
     constexpr int kMain = 2 * (BM + BN) * BKB;
     constexpr int kEpi = (sizeof(OutT) == 4 && BM / 32 > 1 ? BM / 2 : BM) * BN * (int)sizeof(OutT);
     constexpr int kLds = kMain > kEpi ? kMain : kEpi;
-    auto kern = gemm_mfma_tn<In, Out, BM, BN, BKB, kEdge, AT>;
-    if (kLds > 64 * 1024) {
-        static LdsCap cap;
-        if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
-    }
-    kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1)), dim3(256), kLds, st>>>(a);
-    MOYE_HIP_CHECK(hipGetLastError());
+    static LdsCap cap;
+    plan.add_kernel(gemm_mfma_tn<In, Out, BM, BN, BKB, kEdge, AT>, a, (unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1), 256, kLds,
+                    kLds > 64 * 1024 ? &cap : nullptr, BM, BN, BKB, In::kDt, Out::kDt, "gemm_mfma_tn<%s,%s,%d,%d,%d,edge=%d,atom=%d>", In::kName,
+                    Out::kName, BM, BN, BKB, (int)kEdge, AT);
     return MOYE_OK;
 }
 
 template <typename In, int BM, int BN, int BKB, bool kEdge = false, int AT = 16>
-static int32_t launch_out(int32_t out_dt, const GemmArgs& a, hipStream_t st) {
+static int32_t launch_out(int32_t out_dt, const GemmArgs& a, GemmPlan& plan) {
     switch (out_dt) {
-        case MOYE_F32: return launch<In, OutF32, BM, BN, BKB, kEdge, AT>(a, st);
-        case MOYE_F16: return launch<In, OutF16, BM, BN, BKB, kEdge, AT>(a, st);
-        case MOYE_BF16: return launch<In, OutBF16, BM, BN, BKB, kEdge, AT>(a, st);
+        case MOYE_F32: return launch<In, OutF32, BM, BN, BKB, kEdge, AT>(a, plan);
+        case MOYE_F16: return launch<In, OutF16, BM, BN, BKB, kEdge, AT>(a, plan);
+        case MOYE_BF16: return launch<In, OutBF16, BM, BN, BKB, kEdge, AT>(a, plan);
         default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: MFMA kernels write f32, f16 or bf16, not %s", dtype_name(out_dt));
     }
 }
 
 template <bool kEdge>
-static int32_t launch_atom32(int32_t in_dt, int32_t out_dt, const GemmArgs& a, hipStream_t st) {
+static int32_t launch_atom32(int32_t in_dt, int32_t out_dt, const GemmArgs& a, GemmPlan& plan) {
     switch (in_dt) {
-        case MOYE_F16: return launch_out<InF16, 128, 128, 64, kEdge, 32>(out_dt, a, st);
-        case MOYE_BF16: return launch_out<InBF16, 128, 128, 64, kEdge, 32>(out_dt, a, st);
-        case MOYE_F8E4M3: return launch_out<InFP8, 128, 128, 64, kEdge, 32>(out_dt, a, st);
-        case MOYE_F32: return launch_out<InF32, 128, 128, 64, kEdge, 32>(out_dt, a, st);
+        case MOYE_F16: return launch_out<InF16, 128, 128, 64, kEdge, 32>(out_dt, a, plan);
+        case MOYE_BF16: return launch_out<InBF16, 128, 128, 64, kEdge, 32>(out_dt, a, plan);
+        case MOYE_F8E4M3: return launch_out<InFP8, 128, 128, 64, kEdge, 32>(out_dt, a, plan);
+        case MOYE_F32: return launch_out<InF32, 128, 128, 64, kEdge, 32>(out_dt, a, plan);
         default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: no MFMA atom for %s inputs", dtype_name(in_dt));
     }
 }
 
 // The 32x32 atoms: CTA tile 128x128 with 64 bytes of K per row, four waves of 2 x 2 MFMA tiles each; residue
 // tiles under the same rule as for the 16x16 atoms.
-static int32_t dispatch_atom32(int32_t in_dt, int32_t out_dt, int bm, int bn, int bk_elems, GemmArgs a, hipStream_t st) {
+static int32_t dispatch_atom32(int32_t in_dt, int32_t out_dt, int bm, int bn, int bk_elems, GemmArgs a, GemmPlan& plan) {
     const int eb = dtype_bytes(in_dt), ob = dtype_bytes(out_dt);
     const bool chosen_here = bm == 0 && bn == 0;
     if ((bm && bm != 128) || (bn && bn != 128) || (bk_elems && bk_elems * eb != 64))
@@ -308,33 +305,29 @@ static int32_t dispatch_atom32(int32_t in_dt, int32_t out_dt, int bm, int bn, in
     a.tiles_m = (a.M + 127) / 128;
     a.tiles_n = (a.N + 127) / 128;
     if (a.M % 128 || a.N % 128 || a.K % (64 / eb)) {
-        if (!chosen_here && !(a.xcd_swizzle & MOYE_GEMM_PREDICATE))
+        if (!chosen_here && !(a.flags & MOYE_GEMM_PREDICATE))
             return fail(MOYE_ERR_SHAPE, "gemm!: CTA tile 128x128x%d does not divide the problem %dx%dx%d", 64 / eb, a.M, a.N, a.K);
         if (((int64_t)a.K * eb) % 16)
             return fail(MOYE_ERR_SHAPE, "gemm!: the predicated MFMA kernel needs K to be a multiple of %d elements (16 bytes), got %d",
                         16 / eb, a.K);
-        return launch_atom32<true>(in_dt, out_dt, a, st);
+        return launch_atom32<true>(in_dt, out_dt, a, plan);
     }
     if ((a.ldd * ob) % 16 || reinterpret_cast<uintptr_t>(a.D) % 16)
         return fail(MOYE_ERR_ALIGN, "gemm!: operands of the MFMA kernels need 16-byte aligned pointers and row pitches");
-    return launch_atom32<false>(in_dt, out_dt, a, st);
+    return launch_atom32<false>(in_dt, out_dt, a, plan);
 }
 
 // K-major A and B, N-contiguous D.  bk_elems = 0 picks the default K extent per tile.
-// MOYE_GEMM_HAND_ORDERED=0 in the environment (read once) keeps calls that the library would give to the hand-ordered
-// 256 x 256 kernel on the compiler-scheduled one
-static bool hand_ordered_on() {
-    static const bool off = getenv("MOYE_GEMM_HAND_ORDERED") && atoi(getenv("MOYE_GEMM_HAND_ORDERED")) == 0;
-    return !off;
-}
-
+// `lib`: the tile (and K ranges) the host chose together with the split when everything was left to the library
+// (gemm_choose, gemm_plan.hpp); null where only the tile is open (a part of a larger problem, a split the caller named).
 int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int bk_elems, int waves, int stages,
-                              GemmArgs a, hipStream_t st) {
+                              GemmArgs a, GemmPlan& plan, const TileChoice* lib) {
     const int eb = dtype_bytes(in_dt);
-    if (a.xcd_swizzle & kGemmAtom32) return dispatch_atom32(in_dt, out_dt, bm, bn, bk_elems, a, st);
+    const int cus = plan.shape.cus;
+    if (a.flags & kGemmAtom32) return dispatch_atom32(in_dt, out_dt, bm, bn, bk_elems, a, plan);
     // a short A (at most 64 rows) is a bandwidth problem: stream B once, no CTA tiling
     if ((bm == 0 && bn == 0 && a.M <= 64 && ((int64_t)a.K * eb) % 64 == 0) || (bm == a.M && bm <= 64 && bn == 16))
-        return gemm_mfma_skinny_dispatch(in_dt, out_dt, a, st);
+        return gemm_mfma_skinny_dispatch(in_dt, out_dt, a, plan);
     const bool chosen_here = bm == 0 && bn == 0;
     if (bm == 0 && bn == 0) {
         // the library chooses: 256 x 256 tiles, one per CU, where the cost model of gemm_plan.hpp prices them below
@@ -344,12 +337,14 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         const int ranges = a.split > 1 ? a.split : 1;
         const int64_t k_bytes_all = (int64_t)a.K * eb * ranges;
         const bool whole256 = a.M % 256 == 0 && a.N % 256 == 0 && a.K % (128 / eb) == 0;
-        const GemmPlan plan = gemm_plan(a.M, a.N, k_bytes_all, eb == 4, a.M % 64 == 0 && a.N % 64 == 0 && ((int64_t)a.K * eb) % 128 == 0, 16, ranges);
+        const TileChoice choice = lib && lib->tile != 256 ? *lib
+                                  : gemm_plan(a.M, a.N, k_bytes_all, eb == 4, a.M % 64 == 0 && a.N % 64 == 0 && ((int64_t)a.K * eb) % 128 == 0, 16, cus, ranges);
         // (operands that were left M- or N-major: the host made sure of whole 128 x 128 tiles, an aligned D and no K ranges;
         // such a call takes whole 256 x 256 or 128 x 128 tiles, never 64 x 64 ones, ragged ones or fringes)
-        const bool majors = a.xcd_swizzle & (kGemmAMajorM | kGemmBMajorN);
-        const bool prefer256 = ranges > 1 ? rtiles >= 128
-                                            : rtiles >= 64 && gemm_plan_cost_256(a.M, a.N, k_bytes_all, eb == 4, !whole256) <= plan.us;
+        const bool majors = a.flags & (kGemmAMajorM | kGemmBMajorN);
+        const bool prefer256 = lib ? lib->tile == 256
+                               : ranges > 1 ? rtiles >= cus / 2
+                                            : rtiles >= cus / 4 && gemm_plan_cost_256(a.M, a.N, k_bytes_all, eb == 4, !whole256, cus) <= choice.us;
         const bool big = whole256 && prefer256;
         // A large problem whose M or N is not a multiple of 256: the interior runs on 256x256 tiles, the fringe to the
         // right (all interior rows, the last N % 256 columns) and the fringe below (the last M % 256 rows, all columns)
@@ -370,30 +365,29 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         // 128 x 128 tiles, 167-173 us either way; interior and two fringes 116)
         // (whole interior tiles with a D that is not aligned need the guarded instance: its conditions, as below)
         const bool guarded_takes_interior = in_dt != MOYE_F8E4M3 && stages < 3 && (waves <= 1 || waves == 8) &&
-                                            !(a.xcd_swizzle & (MOYE_GEMM_WAVE4 | MOYE_GEMM_PINGPONG | kGemmAMajorM | kGemmBMajorN | kGemmAtom32));
+                                            !(a.flags & (MOYE_GEMM_WAVE4 | MOYE_GEMM_PINGPONG | kGemmAMajorM | kGemmBMajorN | kGemmAtom32));
         const bool thin_shape = (fr_m > 0 || fr_n > 0) && fr_m <= 64 && fr_n <= 64 && a.K % (128 / eb) == 0 && aligned_ab && ranges == 1 &&
                                 (aligned || guarded_takes_interior);
         const double fringe_us = (fr_n > 0 ? 4.5 + (double)(M0 + fr_n) * (double)k_bytes_all / 6.0e6 : 0.0) +
                                  (fr_m > 0 ? 4.5 + (double)(a.N + fr_m) * (double)k_bytes_all / 6.0e6 : 0.0);
-        const bool thin = thin_shape && (int64_t)(M0 / 256) * (N0 / 256) >= 64 &&
-                          gemm_plan_cost_256(M0, N0, k_bytes_all, eb == 4, false) + fringe_us <= plan.us;
+        const bool thin = thin_shape && (int64_t)(M0 / 256) * (N0 / 256) >= cus / 4 &&
+                          gemm_plan_cost_256(M0, N0, k_bytes_all, eb == 4, false, cus) + fringe_us <= choice.us;
         // (fp8: only the hand-ordered kernel's guarded form, i.e. K of whole 128-byte rows, no C, no operation)
-        const bool hand_ordered_ragged = hand_ordered_on() && (eb == 2 || eb == 4 || in_dt == MOYE_F8E4M3) && ((int64_t)a.K * eb) % 128 == 0 &&
-                                         a.ep_op == MOYE_MAP_IDENTITY && !a.C && stages < 2 &&
-                                         256 * a.lda * eb < ((int64_t)1 << 32) && 256 * a.ldb * eb < ((int64_t)1 << 32);
+        const bool hand_ordered_ragged = (eb == 2 || eb == 4 || in_dt == MOYE_F8E4M3) && ((int64_t)a.K * eb) % 128 == 0 &&
+                                         a.ep_op == MOYE_MAP_IDENTITY && !a.C && stages < 2 && row_offsets_fit(a, 256, eb);
         if ((!big || !aligned) && !thin && a.split <= 1 && bk_elems == 0 && aligned_ab && (in_dt != MOYE_F8E4M3 || hand_ordered_ragged) && ((int64_t)a.K * eb) % 16 == 0 &&
             prefer256 && stages < 3 && (waves <= 1 || waves == 8) &&
-            !(a.xcd_swizzle & (MOYE_GEMM_WAVE4 | MOYE_GEMM_PINGPONG | kGemmAMajorM | kGemmBMajorN | kGemmAtom32))) {
-            a.xcd_swizzle |= kGemmRagged;
+            !(a.flags & (MOYE_GEMM_WAVE4 | MOYE_GEMM_PINGPONG | kGemmAMajorM | kGemmBMajorN | kGemmAtom32))) {
+            a.flags |= kGemmRagged;
             // K of whole 128-byte rows, no C and no epilogue operation: the hand-ordered kernel's guarded form (rows
             // clamped, no K tail to mask)
-            if (hand_ordered_ragged) return gemm_mfma_tn_256_w4_dispatch(in_dt, out_dt, a, 8, 128, false, st);
-            return gemm_mfma_tn_256_dispatch(in_dt, out_dt, a, 8, stages, st);
+            if (hand_ordered_ragged) return gemm_mfma_tn_256_w4_dispatch(in_dt, out_dt, a, 8, 128, false, plan);
+            return gemm_mfma_tn_256_dispatch(in_dt, out_dt, a, 8, stages, plan);
         }
-        if (!big && !majors && a.split <= 1 && bk_elems == 0 && (thin || (aligned && prefer256)) && a.K % (128 / eb) == 0 && (int64_t)(M0 / 256) * (N0 / 256) >= 64) {
+        if (!big && !majors && a.split <= 1 && bk_elems == 0 && (thin || (aligned && prefer256)) && a.K % (128 / eb) == 0 && (int64_t)(M0 / 256) * (N0 / 256) >= cus / 4) {
             GemmArgs part = a;
             part.M = M0; part.N = N0;
-            if (int32_t e = gemm_mfma_tn_dispatch(in_dt, out_dt, 0, 0, 0, waves, stages, part, st)) return e;
+            if (int32_t e = gemm_mfma_tn_dispatch(in_dt, out_dt, 0, 0, 0, waves, stages, part, plan)) return e;
             if (a.N > N0 && a.N - N0 <= 64 && ((int64_t)a.K * eb) % 64 == 0) {
                 // a narrow fringe is a short-M problem once transposed: D(:, N0:)' = B(N0:, :) * A'
                 part = a;
@@ -405,7 +399,7 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
                 part.ldc_m = a.ldc_n; part.ldc_n = a.ldc_m;
                 if (a.ep_x) part.ep_x = static_cast<const char*>(a.ep_x) + (int64_t)N0 * a.ep_xn * dtype_bytes(a.ep_xdt);
                 part.ep_xm = a.ep_xn; part.ep_xn = a.ep_xm;
-                if (int32_t e = gemm_mfma_skinny_dispatch(in_dt, out_dt, part, st)) return e;
+                if (int32_t e = gemm_mfma_skinny_dispatch(in_dt, out_dt, part, plan)) return e;
             } else if (a.N > N0) {
                 part = a;
                 part.M = M0; part.N = a.N - N0;
@@ -413,7 +407,7 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
                 part.D = static_cast<char*>(a.D) + (int64_t)N0 * ob0;
                 if (a.C) part.C = static_cast<const char*>(a.C) + (int64_t)N0 * a.ldc_n * ob0;
                 if (a.ep_x) part.ep_x = static_cast<const char*>(a.ep_x) + (int64_t)N0 * a.ep_xn * dtype_bytes(a.ep_xdt);
-                if (int32_t e = gemm_mfma_tn_dispatch(in_dt, out_dt, 0, 0, 0, 0, 0, part, st)) return e;
+                if (int32_t e = gemm_mfma_tn_dispatch(in_dt, out_dt, 0, 0, 0, 0, 0, part, plan)) return e;
             }
             if (a.M > M0) {
                 part = a;
@@ -422,7 +416,7 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
                 part.D = static_cast<char*>(a.D) + (int64_t)M0 * a.ldd * ob0;
                 if (a.C) part.C = static_cast<const char*>(a.C) + (int64_t)M0 * a.ldc_m * ob0;
                 if (a.ep_x) part.ep_x = static_cast<const char*>(a.ep_x) + (int64_t)M0 * a.ep_xm * dtype_bytes(a.ep_xdt);
-                if (int32_t e = gemm_mfma_tn_dispatch(in_dt, out_dt, 0, 0, 0, 0, 0, part, st)) return e;
+                if (int32_t e = gemm_mfma_tn_dispatch(in_dt, out_dt, 0, 0, 0, 0, 0, part, plan)) return e;
             }
             return MOYE_OK;
         }
@@ -433,16 +427,16 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         // 4608 x 4608 x 8192 318 -> 270-282; 5120^3, 400 tiles, gains nothing and the model says so).  Every
         // operand type, with everything left to the library; taken when the model sees 3 % or more (fp32: 12 %).
         if (big && a.split <= 1 && ranges == 1 && !majors && bk_elems == 0 && waves <= 1 && stages == 0 &&
-            rtiles > 256 && rtiles % 256 && hand_ordered_on() && !(a.xcd_swizzle & (MOYE_GEMM_WAVE4 | MOYE_GEMM_PINGPONG | kGemmAtom32))) {
+            rtiles > cus && rtiles % cus && !(a.flags & (MOYE_GEMM_WAVE4 | MOYE_GEMM_PINGPONG | kGemmAtom32))) {
             const int tm = a.M / 256, tn = a.N / 256;
             const bool by_rows = tm >= tn;
             const int nt = by_rows ? tm : tn;
             auto alone = [&](int64_t m, int64_t n) {  // what the library would run the part as, priced
-                const double on128 = gemm_plan(m, n, k_bytes_all, eb == 4, true, 16, 1).us;
-                const double on256 = gemm_plan_cost_256(m, n, k_bytes_all, eb == 4, false);
-                return (m / 256) * (n / 256) >= 64 && on256 <= on128 ? on256 : on128;
+                const double on128 = gemm_plan(m, n, k_bytes_all, eb == 4, true, 16, cus, 1).us;
+                const double on256 = gemm_plan_cost_256(m, n, k_bytes_all, eb == 4, false, cus);
+                return (m / 256) * (n / 256) >= cus / 4 && on256 <= on128 ? on256 : on128;
             };
-            const double whole_us = gemm_plan_cost_256(a.M, a.N, k_bytes_all, eb == 4, false);
+            const double whole_us = gemm_plan_cost_256(a.M, a.N, k_bytes_all, eb == 4, false, cus);
             // (fp32: the model prices a part-filled round like a full one, 7 % more than it takes, so it has to see 12 %;
             // every split it then takes was priced at 20 % or more and gains: 6144^3 4065 -> 3074 us, 4352 x 4352 x 2048
             // 912 -> 580, 7168 x 7168 x 2048 1833 -> 1494, 4608^3 2023 -> 1754)
@@ -451,13 +445,13 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
             for (int r = 1; r < nt; ++r) {
                 const int64_t m1 = by_rows ? (int64_t)r * 256 : a.M, n1 = by_rows ? a.N : (int64_t)r * 256;
                 const int64_t m2 = by_rows ? a.M - m1 : a.M, n2 = by_rows ? a.N : a.N - n1;
-                const double us = gemm_plan_cost_256(m1, n1, k_bytes_all, eb == 4, false) + 2.0 + alone(m2, n2);
+                const double us = gemm_plan_cost_256(m1, n1, k_bytes_all, eb == 4, false, cus) + 2.0 + alone(m2, n2);
                 if (us < best_us) { best_us = us; first = r; }
             }
             if (first > 0) {
                 GemmArgs part = a;
                 (by_rows ? part.M : part.N) = first * 256;
-                if (int32_t e = gemm_mfma_tn_dispatch(in_dt, out_dt, 256, 256, 128 / eb, 8, 0, part, st)) return e;
+                if (int32_t e = gemm_mfma_tn_dispatch(in_dt, out_dt, 256, 256, 128 / eb, 8, 0, part, plan)) return e;
                 part = a;
                 if (by_rows) {
                     const int64_t m1 = (int64_t)first * 256;
@@ -474,14 +468,14 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
                     if (a.C) part.C = static_cast<const char*>(a.C) + n1 * a.ldc_n * ob0;
                     if (a.ep_x) part.ep_x = static_cast<const char*>(a.ep_x) + n1 * a.ep_xn * dtype_bytes(a.ep_xdt);
                 }
-                return gemm_mfma_tn_dispatch(in_dt, out_dt, 0, 0, 0, 0, 0, part, st);
+                return gemm_mfma_tn_dispatch(in_dt, out_dt, 0, 0, 0, 0, 0, part, plan);
             }
         }
         bm = bn = big ? 256 : 128;
         if (bk_elems == 0) bk_elems = big || a.K % (128 / eb) == 0 ? 128 / eb : 64 / eb;
         // smaller problems: 64 x 64 tiles (four times the workgroups, no ragged form) where the cost model prices them
         // below 128 x 128 tiles for the K ranges this call runs with (gemm_plan.hpp; fp16 1024^3: 8.3 us against 10.0)
-        if (!big && !majors && aligned && a.M % 64 == 0 && a.N % 64 == 0 && a.K % bk_elems == 0 && !(a.xcd_swizzle & kGemmAtom32) && plan.tile == 64)
+        if (!big && !majors && aligned && a.M % 64 == 0 && a.N % 64 == 0 && a.K % bk_elems == 0 && !(a.flags & kGemmAtom32) && choice.tile == 64)
             bm = bn = 64;
         if (big && waves <= 1) waves = 8;
     }
@@ -498,44 +492,41 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         if (bkb != 128 && bkb != 64)
             return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the 256x256 MFMA kernels take %d or %d elements of K per tile", 64 / eb, 128 / eb);
         // the hand-ordered kernel has no element-wise operations in its epilogue
-        if ((a.xcd_swizzle & (MOYE_GEMM_WAVE4 | MOYE_GEMM_PINGPONG)) && a.ep_op != MOYE_MAP_IDENTITY)
+        if ((a.flags & (MOYE_GEMM_WAVE4 | MOYE_GEMM_PINGPONG)) && a.ep_op != MOYE_MAP_IDENTITY)
             return fail(MOYE_ERR_UNSUPPORTED, "gemm!: MOYE_GEMM_WAVE4 and MOYE_GEMM_PINGPONG take no element-wise epilogue operation; leave the schedule to the library");
         // fp8 runs at twice the 16-bit rate only on the 16x16x128 MFMA, which the hand-ordered kernel issues
-        if (in_dt == MOYE_F8E4M3 && bkb == 128 && stages < 3 && !(a.xcd_swizzle & MOYE_GEMM_PINGPONG) && a.ep_op == MOYE_MAP_IDENTITY)
-            a.xcd_swizzle |= MOYE_GEMM_WAVE4;
+        if (in_dt == MOYE_F8E4M3 && bkb == 128 && stages < 3 && !(a.flags & MOYE_GEMM_PINGPONG) && a.ep_op == MOYE_MAP_IDENTITY)
+            a.flags |= MOYE_GEMM_WAVE4;
         // ... and for the 16-bit types its form with whole 128-byte rows in two stages is the fastest k-loop of this build
         // for a plain call (fp16 4096^3 97.6-98.6 us against 101.3-102.0 for the compiler-scheduled kernel on the same
-        // box, bf16 8192^3 726 against 754); operations in the epilogue, ragged tiles, operands that are not K-major and
-        // fp32 operands stay with that kernel, and so does a call that asks for it: stages = 2 in the descriptor, or
-        // MOYE_GEMM_HAND_ORDERED=0 in the environment (read once).
-        const bool bias_no_c = (a.xcd_swizzle & kGemmEpiAddVec) && !a.C && waves != 4;  // (its bias instance: eight waves, no C)
+        // box, bf16 8192^3 726 against 754); operations in the epilogue and a K tail stay with that kernel, and so does a
+        // call that asks for it: stages = 2 in the descriptor.
+        const bool bias_no_c = (a.flags & kGemmEpiAddVec) && !a.C && waves != 4;  // (its bias instance: eight waves, no C)
         // (operands that keep their M- / N-major form: its transposing fragment reads, eight waves, plain calls; fp16 4096^3 NN
         // against the compiler-scheduled kernel's: see the kernel's header)
-        const bool majors256 = a.xcd_swizzle & (kGemmAMajorM | kGemmBMajorN);
-        if (hand_ordered_on() && eb == 2 && bkb == 128 && stages < 2 && (a.ep_op == MOYE_MAP_IDENTITY || (bias_no_c && !majors256)) &&
-            (!majors256 || (waves != 4 && !(a.xcd_swizzle & kGemmEpiAddVec))) &&
-            !(a.xcd_swizzle & (MOYE_GEMM_PINGPONG | kGemmRagged | kGemmAtom32)) &&
-            256 * a.lda * eb < ((int64_t)1 << 32) && 256 * a.ldb * eb < ((int64_t)1 << 32))
-            a.xcd_swizzle |= MOYE_GEMM_WAVE4;
+        const bool majors256 = a.flags & (kGemmAMajorM | kGemmBMajorN);
+        if (eb == 2 && bkb == 128 && stages < 2 && (a.ep_op == MOYE_MAP_IDENTITY || (bias_no_c && !majors256)) &&
+            (!majors256 || (waves != 4 && !(a.flags & kGemmEpiAddVec))) &&
+            !(a.flags & (MOYE_GEMM_PINGPONG | kGemmRagged | kGemmAtom32)) && row_offsets_fit(a, 256, eb))
+            a.flags |= MOYE_GEMM_WAVE4;
         // fp32 operands: the hand-ordered kernel too (fp32 8192^3 152.8 TFLOP/s on whole-line stages, 147.8 on its ring of
         // 64-byte-row stages, 142.5 for the compiler-scheduled kernel)
-        if (hand_ordered_on() && in_dt == MOYE_F32 && stages < 2 && a.ep_op == MOYE_MAP_IDENTITY && a.K % 16 == 0 &&
+        if (in_dt == MOYE_F32 && stages < 2 && a.ep_op == MOYE_MAP_IDENTITY && a.K % 16 == 0 &&
             (!majors256 || (waves != 4 && bkb == 128)) &&
-            !(a.xcd_swizzle & (MOYE_GEMM_PINGPONG | kGemmRagged | kGemmAtom32)) &&
-            256 * a.lda * eb < ((int64_t)1 << 32) && 256 * a.ldb * eb < ((int64_t)1 << 32))
-            a.xcd_swizzle |= MOYE_GEMM_WAVE4;
+            !(a.flags & (MOYE_GEMM_PINGPONG | kGemmRagged | kGemmAtom32)) && row_offsets_fit(a, 256, eb))
+            a.flags |= MOYE_GEMM_WAVE4;
         // hand-ordered kernel: k-steps of 64 bytes, or of 128 (fp8 always; the 16-bit types when the tile says so)
         const int w4_step = in_dt == MOYE_F8E4M3 || (bkb == 128 && (eb == 2 || eb == 4)) ? 128 : 64;
-        const int kmult = (a.xcd_swizzle & MOYE_GEMM_WAVE4) ? w4_step / eb
-                          : (a.xcd_swizzle & MOYE_GEMM_PINGPONG) ? 64 / eb : 128 / eb;
+        const int kmult = (a.flags & MOYE_GEMM_WAVE4) ? w4_step / eb
+                          : (a.flags & MOYE_GEMM_PINGPONG) ? 64 / eb : 128 / eb;
         if (a.M % 256 || a.N % 256 || a.K % kmult)
             return fail(MOYE_ERR_SHAPE, "gemm!: CTA tile 256x256x%d does not divide the problem %dx%dx%d", kmult,
                         a.M, a.N, a.K);
         if (misaligned)
             return fail(MOYE_ERR_ALIGN, "gemm!: operands of the MFMA kernels need 16-byte aligned pointers and row pitches");
-        if (a.xcd_swizzle & MOYE_GEMM_WAVE4) return gemm_mfma_tn_256_w4_dispatch(in_dt, out_dt, a, waves, w4_step, stages >= 3, st);
-        if (a.xcd_swizzle & MOYE_GEMM_PINGPONG) return gemm_mfma_tn_256_pp_dispatch(in_dt, out_dt, a, st);
-        return gemm_mfma_tn_256_dispatch(in_dt, out_dt, a, waves, stages, st);
+        if (a.flags & MOYE_GEMM_WAVE4) return gemm_mfma_tn_256_w4_dispatch(in_dt, out_dt, a, waves, w4_step, stages >= 3, plan);
+        if (a.flags & MOYE_GEMM_PINGPONG) return gemm_mfma_tn_256_pp_dispatch(in_dt, out_dt, a, plan);
+        return gemm_mfma_tn_256_dispatch(in_dt, out_dt, a, waves, stages, plan);
     }
     if (bm == 64 && bn == 64 && (bkb == 64 || bkb == 128)) {
         // small problems: four times as many workgroups as with 128 x 128 tiles (no predicated form)
@@ -547,10 +538,10 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         a.tiles_n = a.N / 64;
         const bool wide64 = bkb == 128;
         switch (in_dt) {
-            case MOYE_F16: return wide64 ? launch_out<InF16, 64, 64, 128>(out_dt, a, st) : launch_out<InF16, 64, 64, 64>(out_dt, a, st);
-            case MOYE_BF16: return wide64 ? launch_out<InBF16, 64, 64, 128>(out_dt, a, st) : launch_out<InBF16, 64, 64, 64>(out_dt, a, st);
-            case MOYE_F8E4M3: return wide64 ? launch_out<InFP8, 64, 64, 128>(out_dt, a, st) : launch_out<InFP8, 64, 64, 64>(out_dt, a, st);
-            case MOYE_F32: return wide64 ? launch_out<InF32, 64, 64, 128>(out_dt, a, st) : launch_out<InF32, 64, 64, 64>(out_dt, a, st);
+            case MOYE_F16: return wide64 ? launch_out<InF16, 64, 64, 128>(out_dt, a, plan) : launch_out<InF16, 64, 64, 64>(out_dt, a, plan);
+            case MOYE_BF16: return wide64 ? launch_out<InBF16, 64, 64, 128>(out_dt, a, plan) : launch_out<InBF16, 64, 64, 64>(out_dt, a, plan);
+            case MOYE_F8E4M3: return wide64 ? launch_out<InFP8, 64, 64, 128>(out_dt, a, plan) : launch_out<InFP8, 64, 64, 64>(out_dt, a, plan);
+            case MOYE_F32: return wide64 ? launch_out<InF32, 64, 64, 128>(out_dt, a, plan) : launch_out<InF32, 64, 64, 64>(out_dt, a, plan);
             default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: no MFMA atom for %s inputs", dtype_name(in_dt));
         }
     }
@@ -566,21 +557,20 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         // (fp8 always: only this kernel issues the 16x16x128 MFMA on 128 x 128 tiles, twice the rate of the 16x16x32 one:
         // fp8 2560^3 29.9 -> 22.1 us, 2048^3 16.9 -> 13.7, 1536^3 14.0 -> 10.8; fp32 always as well: 4096^3 on these tiles
         // 1136 -> 914 us, 2048^3 128.8 -> 122.5)
-        if (whole && hand_ordered_on() && (int64_t)(a.M / 128) * (a.N / 128) > (eb == 2 ? 256 : 0) &&
+        if (whole && (int64_t)(a.M / 128) * (a.N / 128) > (eb == 2 ? cus : 0) &&
             (eb == 2 || eb == 4 || in_dt == MOYE_F8E4M3) && a.ep_op == MOYE_MAP_IDENTITY && stages < 2 &&
-            !(a.xcd_swizzle & (kGemmAMajorM | kGemmBMajorN | kGemmEpiAddVec)) && 128 * a.lda * eb < ((int64_t)1 << 32) &&
-            128 * a.ldb * eb < ((int64_t)1 << 32))
-            return gemm_mfma_tn_128_w4_dispatch(in_dt, out_dt, a, st);
-        if (whole) return gemm_mfma_tn_128_dispatch(in_dt, out_dt, a, st);
-        if (chosen_here || (a.xcd_swizzle & MOYE_GEMM_PREDICATE)) {
-            a.xcd_swizzle |= kGemmRagged;
+            !(a.flags & (kGemmAMajorM | kGemmBMajorN | kGemmEpiAddVec)) && row_offsets_fit(a, 128, eb))
+            return gemm_mfma_tn_128_w4_dispatch(in_dt, out_dt, a, plan);
+        if (whole) return gemm_mfma_tn_128_dispatch(in_dt, out_dt, a, plan);
+        if (chosen_here || (a.flags & MOYE_GEMM_PREDICATE)) {
+            a.flags |= kGemmRagged;
             // (K of whole 128-byte rows, no C, no operation, more tiles than CUs: the guarded form of the hand-ordered instance)
-            if (hand_ordered_on() && (int64_t)((a.M + 127) / 128) * ((a.N + 127) / 128) > (eb == 2 ? 256 : 0) &&
+            if ((int64_t)((a.M + 127) / 128) * ((a.N + 127) / 128) > (eb == 2 ? cus : 0) &&
                 (eb == 2 || eb == 4 || in_dt == MOYE_F8E4M3) && ((int64_t)a.K * eb) % 128 == 0 &&
-                a.ep_op == MOYE_MAP_IDENTITY && !a.C && stages < 2 && !(a.xcd_swizzle & (kGemmAMajorM | kGemmBMajorN | kGemmEpiAddVec)) &&
-                128 * a.lda * eb < ((int64_t)1 << 32) && 128 * a.ldb * eb < ((int64_t)1 << 32))
-                return gemm_mfma_tn_128_w4_dispatch(in_dt, out_dt, a, st);
-            return gemm_mfma_tn_128_dispatch(in_dt, out_dt, a, st);
+                a.ep_op == MOYE_MAP_IDENTITY && !a.C && stages < 2 && !(a.flags & (kGemmAMajorM | kGemmBMajorN | kGemmEpiAddVec)) &&
+                row_offsets_fit(a, 128, eb))
+                return gemm_mfma_tn_128_w4_dispatch(in_dt, out_dt, a, plan);
+            return gemm_mfma_tn_128_dispatch(in_dt, out_dt, a, plan);
         }
     }
     if (bm != 128 || bn != 128 || (bkb != 64 && bkb != 128))
@@ -590,7 +580,7 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
     if (a.M % bm || a.N % bn || a.K % bk_elems) {
         // the reference's kernels assert divisibility; residue tiles are computed when the caller asks for
         // predication or leaves the tile choice to the library
-        if (!chosen_here && !(a.xcd_swizzle & MOYE_GEMM_PREDICATE))
+        if (!chosen_here && !(a.flags & MOYE_GEMM_PREDICATE))
             return fail(MOYE_ERR_SHAPE, "gemm!: CTA tile %dx%dx%d does not divide the problem %dx%dx%d", bm, bn,
                         bk_elems, a.M, a.N, a.K);
         if (((int64_t)a.K * eb) % 16)
@@ -604,10 +594,10 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         // k-tiles of 128 bytes when the library chose the tile and K is long enough to matter (half the barriers)
         const bool wide_edge = chosen_here && (int64_t)a.K * eb >= 512;
         switch (in_dt) {
-            case MOYE_F16: return wide_edge ? launch_out<InF16, 128, 128, 128, true>(out_dt, a, st) : launch_out<InF16, 128, 128, 64, true>(out_dt, a, st);
-            case MOYE_BF16: return wide_edge ? launch_out<InBF16, 128, 128, 128, true>(out_dt, a, st) : launch_out<InBF16, 128, 128, 64, true>(out_dt, a, st);
-            case MOYE_F8E4M3: return wide_edge ? launch_out<InFP8, 128, 128, 128, true>(out_dt, a, st) : launch_out<InFP8, 128, 128, 64, true>(out_dt, a, st);
-            case MOYE_F32: return wide_edge ? launch_out<InF32, 128, 128, 128, true>(out_dt, a, st) : launch_out<InF32, 128, 128, 64, true>(out_dt, a, st);
+            case MOYE_F16: return wide_edge ? launch_out<InF16, 128, 128, 128, true>(out_dt, a, plan) : launch_out<InF16, 128, 128, 64, true>(out_dt, a, plan);
+            case MOYE_BF16: return wide_edge ? launch_out<InBF16, 128, 128, 128, true>(out_dt, a, plan) : launch_out<InBF16, 128, 128, 64, true>(out_dt, a, plan);
+            case MOYE_F8E4M3: return wide_edge ? launch_out<InFP8, 128, 128, 128, true>(out_dt, a, plan) : launch_out<InFP8, 128, 128, 64, true>(out_dt, a, plan);
+            case MOYE_F32: return wide_edge ? launch_out<InF32, 128, 128, 128, true>(out_dt, a, plan) : launch_out<InF32, 128, 128, 64, true>(out_dt, a, plan);
             default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: no MFMA atom for %s inputs", dtype_name(in_dt));
         }
     }
@@ -618,13 +608,13 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
     const bool wide = bkb == 128;
     switch (in_dt) {
         case MOYE_F16:
-            return wide ? launch_out<InF16, 128, 128, 128>(out_dt, a, st) : launch_out<InF16, 128, 128, 64>(out_dt, a, st);
+            return wide ? launch_out<InF16, 128, 128, 128>(out_dt, a, plan) : launch_out<InF16, 128, 128, 64>(out_dt, a, plan);
         case MOYE_BF16:
-            return wide ? launch_out<InBF16, 128, 128, 128>(out_dt, a, st) : launch_out<InBF16, 128, 128, 64>(out_dt, a, st);
+            return wide ? launch_out<InBF16, 128, 128, 128>(out_dt, a, plan) : launch_out<InBF16, 128, 128, 64>(out_dt, a, plan);
         case MOYE_F8E4M3:
-            return wide ? launch_out<InFP8, 128, 128, 128>(out_dt, a, st) : launch_out<InFP8, 128, 128, 64>(out_dt, a, st);
+            return wide ? launch_out<InFP8, 128, 128, 128>(out_dt, a, plan) : launch_out<InFP8, 128, 128, 64>(out_dt, a, plan);
         case MOYE_F32:
-            return wide ? launch_out<InF32, 128, 128, 128>(out_dt, a, st) : launch_out<InF32, 128, 128, 64>(out_dt, a, st);
+            return wide ? launch_out<InF32, 128, 128, 128>(out_dt, a, plan) : launch_out<InF32, 128, 128, 64>(out_dt, a, plan);
         default:
             return fail(MOYE_ERR_UNSUPPORTED, "gemm!: no MFMA atom for %s inputs", dtype_name(in_dt));
     }

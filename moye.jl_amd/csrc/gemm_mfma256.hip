@@ -139,35 +139,33 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256_ring(GemmArgs
 }
 
 template <typename In, typename Out, int STAGES>
-static int32_t launch256_ring(const GemmArgs& a, hipStream_t st) {
+static int32_t launch256_ring(const GemmArgs& a, GemmPlan& plan) {
     constexpr int kLds = STAGES * (256 + 256) * 64;
-    auto kern = gemm_mfma_tn_256_ring<In, Out, 2, 4, STAGES>;
     static LdsCap cap;
-    if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
-    kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1)), dim3(512), kLds, st>>>(a);
-    MOYE_HIP_CHECK(hipGetLastError());
+    plan.add_kernel(gemm_mfma_tn_256_ring<In, Out, 2, 4, STAGES>, a, (unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1), 512, kLds, &cap,
+                    256, 256, 64, In::kDt, Out::kDt, "gemm_mfma_tn_256_ring<%s,%s,stages=%d>", In::kName, Out::kName, STAGES);
     return MOYE_OK;
 }
 
 template <typename In, typename Out, int WGM, int WGN, bool kOps, int AMAJ, int BMAJ, bool kRagged = false, bool kBias = false>
-static int32_t launch256_instance(const GemmArgs& a, hipStream_t st) {
+static int32_t launch256_instance(const GemmArgs& a, GemmPlan& plan) {
     constexpr int kLds = 2 * (256 + 256) * 128;  // two operand stages, 128 KiB
-    auto kern = gemm_mfma_tn_256<In, Out, WGM, WGN, kOps, AMAJ, BMAJ, kRagged, kBias>;
     static LdsCap cap;
-    if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
-    kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1)), dim3(64 * WGM * WGN), kLds, st>>>(a);
-    MOYE_HIP_CHECK(hipGetLastError());
+    plan.add_kernel(gemm_mfma_tn_256<In, Out, WGM, WGN, kOps, AMAJ, BMAJ, kRagged, kBias>, a, (unsigned)(a.tiles_m * a.tiles_n),
+                    (unsigned)(a.split > 1 ? a.split : 1), 64 * WGM * WGN, kLds, &cap, 256, 256, 128, In::kDt, Out::kDt,
+                    "gemm_mfma_tn_256<%s,%s,waves=%d,ops=%d,amaj=%d,bmaj=%d,ragged=%d,bias=%d>", In::kName, Out::kName, WGM * WGN, (int)kOps, AMAJ, BMAJ,
+                    (int)kRagged, (int)kBias);
     return MOYE_OK;
 }
 
 template <typename In, typename Out, int WGM, int WGN>
-static int32_t launch256(const GemmArgs& a, hipStream_t st) {
-    const bool am = a.xcd_swizzle & kGemmAMajorM, bm = a.xcd_swizzle & kGemmBMajorN;
-    if (a.xcd_swizzle & kGemmRagged) {
+static int32_t launch256(const GemmArgs& a, GemmPlan& plan) {
+    const bool am = a.flags & kGemmAMajorM, bm = a.flags & kGemmBMajorN;
+    if (a.flags & kGemmRagged) {
         if constexpr (WGM * WGN == 8 && !std::is_same<In, InFP8>::value) {
             if (am || bm) return fail(MOYE_ERR_UNSUPPORTED, "gemm!: ragged 256 x 256 tiles take K-major operands");
-            return a.ep_op != MOYE_MAP_IDENTITY ? launch256_instance<In, Out, WGM, WGN, true, 0, 0, true>(a, st)
-                                                : launch256_instance<In, Out, WGM, WGN, false, 0, 0, true>(a, st);
+            return a.ep_op != MOYE_MAP_IDENTITY ? launch256_instance<In, Out, WGM, WGN, true, 0, 0, true>(a, plan)
+                                                : launch256_instance<In, Out, WGM, WGN, false, 0, 0, true>(a, plan);
         } else {
             return fail(MOYE_ERR_UNSUPPORTED, "gemm!: ragged 256 x 256 tiles run on eight waves with f16, bf16 or f32 operands");
         }
@@ -176,58 +174,58 @@ static int32_t launch256(const GemmArgs& a, hipStream_t st) {
         // operands that are not K-major: eight waves, 16-bit types (the host checked)
         if constexpr (WGM * WGN == 8 && In::kBytes == 2) {
             const bool ops = a.ep_op != MOYE_MAP_IDENTITY;
-            if (am && bm) return ops ? launch256_instance<In, Out, WGM, WGN, true, 1, 1>(a, st) : launch256_instance<In, Out, WGM, WGN, false, 1, 1>(a, st);
-            if (am) return ops ? launch256_instance<In, Out, WGM, WGN, true, 1, 0>(a, st) : launch256_instance<In, Out, WGM, WGN, false, 1, 0>(a, st);
-            return ops ? launch256_instance<In, Out, WGM, WGN, true, 0, 1>(a, st) : launch256_instance<In, Out, WGM, WGN, false, 0, 1>(a, st);
+            if (am && bm) return ops ? launch256_instance<In, Out, WGM, WGN, true, 1, 1>(a, plan) : launch256_instance<In, Out, WGM, WGN, false, 1, 1>(a, plan);
+            if (am) return ops ? launch256_instance<In, Out, WGM, WGN, true, 1, 0>(a, plan) : launch256_instance<In, Out, WGM, WGN, false, 1, 0>(a, plan);
+            return ops ? launch256_instance<In, Out, WGM, WGN, true, 0, 1>(a, plan) : launch256_instance<In, Out, WGM, WGN, false, 0, 1>(a, plan);
         } else {
             return fail(MOYE_ERR_UNSUPPORTED, "gemm!: operands that are not K-major run natively with 16-bit types on eight waves only");
         }
     }
     if constexpr (WGM * WGN == 8) {
-        if (a.xcd_swizzle & kGemmEpiAddVec) return launch256_instance<In, Out, WGM, WGN, false, 0, 0, false, true>(a, st);  // a bias
-        if (a.ep_op != MOYE_MAP_IDENTITY) return launch256_instance<In, Out, WGM, WGN, true, 0, 0>(a, st);
+        if (a.flags & kGemmEpiAddVec) return launch256_instance<In, Out, WGM, WGN, false, 0, 0, false, true>(a, plan);  // a bias
+        if (a.ep_op != MOYE_MAP_IDENTITY) return launch256_instance<In, Out, WGM, WGN, true, 0, 0>(a, plan);
     }
-    return launch256_instance<In, Out, WGM, WGN, false, 0, 0>(a, st);
+    return launch256_instance<In, Out, WGM, WGN, false, 0, 0>(a, plan);
 }
 
 template <typename In>
-static int32_t launch256_out(int32_t out_dt, const GemmArgs& a, int waves, int stages, hipStream_t st) {
+static int32_t launch256_out(int32_t out_dt, const GemmArgs& a, int waves, int stages, GemmPlan& plan) {
     if (stages >= 3 && a.ep_op != MOYE_MAP_IDENTITY)
         return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the ring schedules (stages >= 3) take no element-wise epilogue operation; leave stages at 0");
     if (stages >= 3) {
         const bool five = stages >= 5;
         switch (out_dt) {
-            case MOYE_F32: return five ? launch256_ring<In, OutF32, 5>(a, st) : launch256_ring<In, OutF32, 4>(a, st);
-            case MOYE_F16: return five ? launch256_ring<In, OutF16, 5>(a, st) : launch256_ring<In, OutF16, 4>(a, st);
-            case MOYE_BF16: return five ? launch256_ring<In, OutBF16, 5>(a, st) : launch256_ring<In, OutBF16, 4>(a, st);
+            case MOYE_F32: return five ? launch256_ring<In, OutF32, 5>(a, plan) : launch256_ring<In, OutF32, 4>(a, plan);
+            case MOYE_F16: return five ? launch256_ring<In, OutF16, 5>(a, plan) : launch256_ring<In, OutF16, 4>(a, plan);
+            case MOYE_BF16: return five ? launch256_ring<In, OutBF16, 5>(a, plan) : launch256_ring<In, OutBF16, 4>(a, plan);
             default: break;
         }
     }
     if (waves == 4 && a.ep_op == MOYE_MAP_IDENTITY) {  // (with an element-wise operation the eight-wave form runs: 256 accumulators leave it no registers)
         switch (out_dt) {
-            case MOYE_F32: return launch256<In, OutF32, 2, 2>(a, st);
-            case MOYE_F16: return launch256<In, OutF16, 2, 2>(a, st);
-            case MOYE_BF16: return launch256<In, OutBF16, 2, 2>(a, st);
+            case MOYE_F32: return launch256<In, OutF32, 2, 2>(a, plan);
+            case MOYE_F16: return launch256<In, OutF16, 2, 2>(a, plan);
+            case MOYE_BF16: return launch256<In, OutBF16, 2, 2>(a, plan);
             default: break;
         }
     }
     switch (out_dt) {
-        case MOYE_F32: return launch256<In, OutF32, 2, 4>(a, st);
-        case MOYE_F16: return launch256<In, OutF16, 2, 4>(a, st);
-        case MOYE_BF16: return launch256<In, OutBF16, 2, 4>(a, st);
+        case MOYE_F32: return launch256<In, OutF32, 2, 4>(a, plan);
+        case MOYE_F16: return launch256<In, OutF16, 2, 4>(a, plan);
+        case MOYE_BF16: return launch256<In, OutBF16, 2, 4>(a, plan);
         default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: MFMA kernels write f32, f16 or bf16, not %s", dtype_name(out_dt));
     }
 }
 
 // 256 x 256 x (128 bytes of K) tile; the caller has checked divisibility and alignment.
-int32_t gemm_mfma_tn_256_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, int waves, int stages, hipStream_t st) {
+int32_t gemm_mfma_tn_256_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, int waves, int stages, GemmPlan& plan) {
     a.tiles_m = (a.M + 255) / 256;  // (whole tiles unless kGemmRagged)
     a.tiles_n = (a.N + 255) / 256;
     switch (in_dt) {
-        case MOYE_F16: return launch256_out<InF16>(out_dt, a, waves, stages, st);
-        case MOYE_BF16: return launch256_out<InBF16>(out_dt, a, waves, stages, st);
-        case MOYE_F8E4M3: return launch256_out<InFP8>(out_dt, a, waves, stages, st);
-        case MOYE_F32: return launch256_out<InF32>(out_dt, a, waves, stages, st);
+        case MOYE_F16: return launch256_out<InF16>(out_dt, a, waves, stages, plan);
+        case MOYE_BF16: return launch256_out<InBF16>(out_dt, a, waves, stages, plan);
+        case MOYE_F8E4M3: return launch256_out<InFP8>(out_dt, a, waves, stages, plan);
+        case MOYE_F32: return launch256_out<InF32>(out_dt, a, waves, stages, plan);
         default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: no MFMA atom for %s inputs", dtype_name(in_dt));
     }
 }

@@ -153,35 +153,33 @@ __global__ __launch_bounds__(512) void gemm_mfma_tn_256_pp(GemmArgs p) {
 }
 
 template <typename In, typename Out>
-static int32_t launch256_pp(const GemmArgs& a, hipStream_t st) {
+static int32_t launch256_pp(const GemmArgs& a, GemmPlan& plan) {
     constexpr int kLds = 5 * (256 + 256) * 64;  // all 160 KiB
-    auto kern = gemm_mfma_tn_256_pp<In, Out>;
     static LdsCap cap;
-    if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
-    kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1)), dim3(512), kLds, st>>>(a);
-    MOYE_HIP_CHECK(hipGetLastError());
+    plan.add_kernel(gemm_mfma_tn_256_pp<In, Out>, a, (unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1), 512, kLds, &cap, 256, 256, 64,
+                    In::kDt, Out::kDt, "gemm_mfma_tn_256_pp<%s,%s>", In::kName, Out::kName);
     return MOYE_OK;
 }
 
 template <typename In>
-static int32_t launch256_pp_out(int32_t out_dt, const GemmArgs& a, hipStream_t st) {
+static int32_t launch256_pp_out(int32_t out_dt, const GemmArgs& a, GemmPlan& plan) {
     switch (out_dt) {
-        case MOYE_F32: return launch256_pp<In, OutF32>(a, st);
-        case MOYE_F16: return launch256_pp<In, OutF16>(a, st);
-        case MOYE_BF16: return launch256_pp<In, OutBF16>(a, st);
+        case MOYE_F32: return launch256_pp<In, OutF32>(a, plan);
+        case MOYE_F16: return launch256_pp<In, OutF16>(a, plan);
+        case MOYE_BF16: return launch256_pp<In, OutBF16>(a, plan);
         default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: MFMA kernels write f32, f16 or bf16, not %s", dtype_name(out_dt));
     }
 }
 
 // 256 x 256 x (64 bytes of K) tile, ping-pong schedule; the caller has checked divisibility and alignment.
-int32_t gemm_mfma_tn_256_pp_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, hipStream_t st) {
+int32_t gemm_mfma_tn_256_pp_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, GemmPlan& plan) {
     a.tiles_m = a.M / 256;
     a.tiles_n = a.N / 256;
     switch (in_dt) {
-        case MOYE_F16: return launch256_pp_out<InF16>(out_dt, a, st);
-        case MOYE_BF16: return launch256_pp_out<InBF16>(out_dt, a, st);
-        case MOYE_F8E4M3: return launch256_pp_out<InFP8>(out_dt, a, st);
-        case MOYE_F32: return launch256_pp_out<InF32>(out_dt, a, st);
+        case MOYE_F16: return launch256_pp_out<InF16>(out_dt, a, plan);
+        case MOYE_BF16: return launch256_pp_out<InBF16>(out_dt, a, plan);
+        case MOYE_F8E4M3: return launch256_pp_out<InFP8>(out_dt, a, plan);
+        case MOYE_F32: return launch256_pp_out<InF32>(out_dt, a, plan);
         default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: no MFMA atom for %s inputs", dtype_name(in_dt));
     }
 }

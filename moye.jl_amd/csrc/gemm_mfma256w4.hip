@@ -126,15 +126,18 @@ struct W4TrFrag32 { uint32_t e[8]; };
 // fragment = what one lane feeds to one MFMA group per operand; SPS = ring stages per k-step; kRow = bytes of K per row
 // of a stage, kRing = stages in the ring
 struct W4Ring64 { static constexpr int kRow = 64, kRing = 5; };
+// (kDt / kName: the operand type of the instance, and its name in a plan)
 struct W4F16 : W4Ring64 {
-    static constexpr int kBytes = 2, SPS = 1;
+    static constexpr int kBytes = 2, SPS = 1, kDt = MOYE_F16;
+    static constexpr const char* kName = "W4F16";
     typedef u32x4 frag;
     static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) {
         asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
     }
 };
 struct W4BF16 : W4Ring64 {
-    static constexpr int kBytes = 2, SPS = 1;
+    static constexpr int kBytes = 2, SPS = 1, kDt = MOYE_BF16;
+    static constexpr const char* kName = "W4BF16";
     typedef u32x4 frag;
     static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) {
         asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
@@ -143,7 +146,8 @@ struct W4BF16 : W4Ring64 {
 // The 16-bit types with k-steps of two stages (128 bytes of K): two MFMAs in a row on the same accumulator (which
 // costs nothing: 16.4 clocks per MFMA either way) and half as many barriers per K.
 struct W4F16x2 : W4Ring64 {
-    static constexpr int kBytes = 2, SPS = 2;
+    static constexpr int kBytes = 2, SPS = 2, kDt = MOYE_F16;
+    static constexpr const char* kName = "W4F16x2";
     struct frag { u32x4 lo, hi; };
     static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) {
         asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %3, %0\n\tv_mfma_f32_16x16x32_f16 %0, %2, %4, %0"
@@ -151,7 +155,8 @@ struct W4F16x2 : W4Ring64 {
     }
 };
 struct W4BF16x2 : W4Ring64 {
-    static constexpr int kBytes = 2, SPS = 2;
+    static constexpr int kBytes = 2, SPS = 2, kDt = MOYE_BF16;
+    static constexpr const char* kName = "W4BF16x2";
     struct frag { u32x4 lo, hi; };
     static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) {
         asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %3, %0\n\tv_mfma_f32_16x16x32_bf16 %0, %2, %4, %0"
@@ -161,7 +166,8 @@ struct W4BF16x2 : W4Ring64 {
 // 32 bytes per lane: the chunk of stage 0 and the chunk of stage 1 of the k-step.  Which 32 of the
 // 128 k-values a lane carries does not matter as long as A and B agree, and they do.
 struct W4FP8 : W4Ring64 {
-    static constexpr int kBytes = 1, SPS = 2;
+    static constexpr int kBytes = 1, SPS = 2, kDt = MOYE_F8E4M3;
+    static constexpr const char* kName = "W4FP8";
     struct frag { u32x4 lo, hi; };
     static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) {
         const u32x8 a8 = __builtin_shufflevector(a.lo, a.hi, 0, 1, 2, 3, 4, 5, 6, 7);
@@ -173,7 +179,8 @@ struct W4FP8 : W4Ring64 {
 // step s+1 are read out of one while the loads of step s+2 fill the other), a lane's 32 bytes are chunks kq and kq + 4
 // of its row.  A load-to-LDS instruction then reads eight whole 128-byte lines instead of sixteen half lines.
 struct W4FP8L {
-    static constexpr int kBytes = 1, SPS = 1, kRow = 128, kRing = 2;
+    static constexpr int kBytes = 1, SPS = 1, kRow = 128, kRing = 2, kDt = MOYE_F8E4M3;
+    static constexpr const char* kName = "W4FP8L";
     struct frag { u32x4 lo, hi; };
     static __device__ __forceinline__ void mma4(const u32x4& alo, const u32x4& ahi, const u32x4& blo, const u32x4& bhi, f32x4& c) {
         const u32x8 a8 = __builtin_shufflevector(alo, ahi, 0, 1, 2, 3, 4, 5, 6, 7);
@@ -184,7 +191,8 @@ struct W4FP8L {
 };
 // The 16-bit types on whole-line stages: chunk kq feeds the first MFMA of an accumulator, chunk kq + 4 the second.
 struct W4F16L {
-    static constexpr int kBytes = 2, SPS = 1, kRow = 128, kRing = 2;
+    static constexpr int kBytes = 2, SPS = 1, kRow = 128, kRing = 2, kDt = MOYE_F16;
+    static constexpr const char* kName = "W4F16L";
     struct frag { u32x4 lo, hi; };
     // the two MFMAs of an accumulator from the four 16-byte halves (what the transposing fragment reads assemble)
     static __device__ __forceinline__ void mma4(const u32x4& alo, const u32x4& ahi, const u32x4& blo, const u32x4& bhi, f32x4& c) {
@@ -194,7 +202,8 @@ struct W4F16L {
     static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) { mma4(a.lo, a.hi, b.lo, b.hi, c); }
 };
 struct W4BF16L {
-    static constexpr int kBytes = 2, SPS = 1, kRow = 128, kRing = 2;
+    static constexpr int kBytes = 2, SPS = 1, kRow = 128, kRing = 2, kDt = MOYE_BF16;
+    static constexpr const char* kName = "W4BF16L";
     struct frag { u32x4 lo, hi; };
     static __device__ __forceinline__ void mma4(const u32x4& alo, const u32x4& ahi, const u32x4& blo, const u32x4& bhi, f32x4& c) {
         asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %3, %0\n\tv_mfma_f32_16x16x32_bf16 %0, %2, %4, %0"
@@ -204,7 +213,8 @@ struct W4BF16L {
 };
 // element j of the chunk goes to MFMA j (see InF32)
 struct W4F32 : W4Ring64 {
-    static constexpr int kBytes = 4, SPS = 1;
+    static constexpr int kBytes = 4, SPS = 1, kDt = MOYE_F32;
+    static constexpr const char* kName = "W4F32";
     typedef u32x4 frag;
     static __device__ __forceinline__ void mma(const frag& a, const frag& b, f32x4& c) {
         asm volatile(
@@ -234,7 +244,8 @@ struct W4F32 : W4Ring64 {
 // fp32 on whole-line stages: a 128-byte row holds 32 k; chunk kq and chunk kq + 4 are four k each, element j of a chunk
 // going to MFMA j (see W4F32): eight MFMAs in a row per accumulator and k-step.
 struct W4F32L {
-    static constexpr int kBytes = 4, SPS = 1, kRow = 128, kRing = 2;
+    static constexpr int kBytes = 4, SPS = 1, kRow = 128, kRing = 2, kDt = MOYE_F32;
+    static constexpr const char* kName = "W4F32L";
     struct frag { u32x4 lo, hi; };
     // four MFMAs from four values of each operand
     static __device__ __forceinline__ void mma_quad(uint32_t a0, uint32_t a1, uint32_t a2, uint32_t a3, uint32_t b0, uint32_t b1, uint32_t b2, uint32_t b3, f32x4& c) {
@@ -347,7 +358,7 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
     }
     // stage g of this workgroup's walk over K is stage g + g0 (mod nstages) of the operands: the eight XCDs start an
     // eighth of K apart when the caller asks for it (see gemm_mfma256.hip)
-    const int g0 = (p.xcd_swizzle & kGemmRotateK) ? (int)((int64_t)(blockIdx.x % 8) * nsteps / 8) * SPS : 0;
+    const int g0 = (p.flags & kGemmRotateK) ? (int)((int64_t)(blockIdx.x % p.xcds) * nsteps / p.xcds) * SPS : 0;
     auto dma1 = [&](int g, int ring_slot, auto qc) __attribute__((always_inline)) {
         constexpr int Q = decltype(qc)::value;
         const int gr = g + g0 >= nstages ? g + g0 - nstages : g + g0;
@@ -568,59 +579,59 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
 }
 
 template <typename In, typename Out, int WGN, bool kBias = false, bool kRagged = false, int TILE = 256, int AMAJ = 0, int BMAJ = 0>
-static int32_t launch256_w4(const GemmArgs& a, hipStream_t st) {
+static int32_t launch256_w4(const GemmArgs& a, GemmPlan& plan) {
     constexpr int kLds = In::kRing * (TILE + TILE) * In::kRow;  // all 160 KiB, or 128 KiB for two whole-line stages (64 KiB on 128 x 128 tiles)
-    auto kern = gemm_mfma_tn_256_w4<In, Out, WGN, kBias, kRagged, TILE, AMAJ, BMAJ>;
     static LdsCap cap;
-    if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
-    kern<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(a.split > 1 ? a.split : 1)), dim3(128 * WGN), kLds, st>>>(a);
-    MOYE_HIP_CHECK(hipGetLastError());
+    plan.add_kernel(gemm_mfma_tn_256_w4<In, Out, WGN, kBias, kRagged, TILE, AMAJ, BMAJ>, a, (unsigned)(a.tiles_m * a.tiles_n),
+                    (unsigned)(a.split > 1 ? a.split : 1), 128 * WGN, kLds, &cap, TILE, TILE, In::kRow * In::SPS, In::kDt, Out::kDt,
+                    "gemm_mfma_tn_256_w4<%s,%s,waves=%d,bias=%d,ragged=%d,tile=%d,amaj=%d,bmaj=%d>", In::kName, Out::kName, 2 * WGN, (int)kBias, (int)kRagged,
+                    TILE, AMAJ, BMAJ);
     return MOYE_OK;
 }
 
 // operands that keep their M- (N-) major form: the eight-wave whole-line forms of the 16-bit types, plain calls
 template <typename In, int AMAJ, int BMAJ>
-static int32_t launch256_w4_majors(int32_t out_dt, const GemmArgs& a, hipStream_t st) {
+static int32_t launch256_w4_majors(int32_t out_dt, const GemmArgs& a, GemmPlan& plan) {
     switch (out_dt) {
-        case MOYE_F32: return launch256_w4<In, OutF32, 4, false, false, 256, AMAJ, BMAJ>(a, st);
-        case MOYE_F16: return launch256_w4<In, OutF16, 4, false, false, 256, AMAJ, BMAJ>(a, st);
-        case MOYE_BF16: return launch256_w4<In, OutBF16, 4, false, false, 256, AMAJ, BMAJ>(a, st);
+        case MOYE_F32: return launch256_w4<In, OutF32, 4, false, false, 256, AMAJ, BMAJ>(a, plan);
+        case MOYE_F16: return launch256_w4<In, OutF16, 4, false, false, 256, AMAJ, BMAJ>(a, plan);
+        case MOYE_BF16: return launch256_w4<In, OutBF16, 4, false, false, 256, AMAJ, BMAJ>(a, plan);
         default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: MFMA kernels write f32, f16 or bf16, not %s", dtype_name(out_dt));
     }
 }
 
 template <typename In, int WGN>
-static int32_t launch256_w4_out(int32_t out_dt, const GemmArgs& a, hipStream_t st) {
-    if (a.xcd_swizzle & (kGemmAMajorM | kGemmBMajorN)) {
+static int32_t launch256_w4_out(int32_t out_dt, const GemmArgs& a, GemmPlan& plan) {
+    if (a.flags & (kGemmAMajorM | kGemmBMajorN)) {
         if constexpr (In::kRow == 128 && WGN == 4) {
-            if ((a.xcd_swizzle & (kGemmRagged | kGemmEpiAddVec)) || a.ep_op != MOYE_MAP_IDENTITY)
+            if ((a.flags & (kGemmRagged | kGemmEpiAddVec)) || a.ep_op != MOYE_MAP_IDENTITY)
                 return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the hand-ordered kernel takes operands that are not K-major in plain calls on whole tiles only");
-            const bool am = a.xcd_swizzle & kGemmAMajorM, bm = a.xcd_swizzle & kGemmBMajorN;
-            return am && bm ? launch256_w4_majors<In, 1, 1>(out_dt, a, st) : am ? launch256_w4_majors<In, 1, 0>(out_dt, a, st) : launch256_w4_majors<In, 0, 1>(out_dt, a, st);
+            const bool am = a.flags & kGemmAMajorM, bm = a.flags & kGemmBMajorN;
+            return am && bm ? launch256_w4_majors<In, 1, 1>(out_dt, a, plan) : am ? launch256_w4_majors<In, 1, 0>(out_dt, a, plan) : launch256_w4_majors<In, 0, 1>(out_dt, a, plan);
         } else {
             return fail(MOYE_ERR_UNSUPPORTED, "gemm!: this schedule of the hand-ordered kernel takes K-major operands only");
         }
     }
-    if (a.xcd_swizzle & kGemmRagged) {  // tiles that reach beyond M or N: the eight-wave whole-line forms
+    if (a.flags & kGemmRagged) {  // tiles that reach beyond M or N: the eight-wave whole-line forms
         if constexpr (In::kRow == 128 && WGN == 4) {
             if (a.ep_op != MOYE_MAP_IDENTITY || a.C) return fail(MOYE_ERR_UNSUPPORTED, "gemm!: ragged tiles of the hand-ordered kernel take no C and no epilogue operation");
             switch (out_dt) {
-                case MOYE_F32: return launch256_w4<In, OutF32, WGN, false, true>(a, st);
-                case MOYE_F16: return launch256_w4<In, OutF16, WGN, false, true>(a, st);
-                case MOYE_BF16: return launch256_w4<In, OutBF16, WGN, false, true>(a, st);
+                case MOYE_F32: return launch256_w4<In, OutF32, WGN, false, true>(a, plan);
+                case MOYE_F16: return launch256_w4<In, OutF16, WGN, false, true>(a, plan);
+                case MOYE_BF16: return launch256_w4<In, OutBF16, WGN, false, true>(a, plan);
                 default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: MFMA kernels write f32, f16 or bf16, not %s", dtype_name(out_dt));
             }
         } else {
             return fail(MOYE_ERR_UNSUPPORTED, "gemm!: this schedule of the hand-ordered kernel takes whole tiles only");
         }
     }
-    if (a.xcd_swizzle & kGemmEpiAddVec) {  // a bias: the eight-wave whole-line forms of the 16-bit types carry it, for calls without C
+    if (a.flags & kGemmEpiAddVec) {  // a bias: the eight-wave whole-line forms of the 16-bit types carry it, for calls without C
         if constexpr (In::kRow == 128 && In::kBytes == 2 && WGN == 4) {
             if (a.C) return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the bias instance of the hand-ordered kernel takes no C");
             switch (out_dt) {
-                case MOYE_F32: return launch256_w4<In, OutF32, WGN, true>(a, st);
-                case MOYE_F16: return launch256_w4<In, OutF16, WGN, true>(a, st);
-                case MOYE_BF16: return launch256_w4<In, OutBF16, WGN, true>(a, st);
+                case MOYE_F32: return launch256_w4<In, OutF32, WGN, true>(a, plan);
+                case MOYE_F16: return launch256_w4<In, OutF16, WGN, true>(a, plan);
+                case MOYE_BF16: return launch256_w4<In, OutBF16, WGN, true>(a, plan);
                 default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: MFMA kernels write f32, f16 or bf16, not %s", dtype_name(out_dt));
             }
         } else {
@@ -628,24 +639,24 @@ static int32_t launch256_w4_out(int32_t out_dt, const GemmArgs& a, hipStream_t s
         }
     }
     switch (out_dt) {
-        case MOYE_F32: return launch256_w4<In, OutF32, WGN>(a, st);
-        case MOYE_F16: return launch256_w4<In, OutF16, WGN>(a, st);
-        case MOYE_BF16: return launch256_w4<In, OutBF16, WGN>(a, st);
+        case MOYE_F32: return launch256_w4<In, OutF32, WGN>(a, plan);
+        case MOYE_F16: return launch256_w4<In, OutF16, WGN>(a, plan);
+        case MOYE_BF16: return launch256_w4<In, OutBF16, WGN>(a, plan);
         default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: MFMA kernels write f32, f16 or bf16, not %s", dtype_name(out_dt));
     }
 }
 
 template <int WGN>
-static int32_t launch256_w4_in(int32_t in_dt, int32_t out_dt, const GemmArgs& a, bool two_stage_steps, bool ring, hipStream_t st) {
+static int32_t launch256_w4_in(int32_t in_dt, int32_t out_dt, const GemmArgs& a, bool two_stage_steps, bool ring, GemmPlan& plan) {
     switch (in_dt) {
         case MOYE_F16:
-            if (two_stage_steps && !ring) return launch256_w4_out<W4F16L, WGN>(out_dt, a, st);
-            return two_stage_steps ? launch256_w4_out<W4F16x2, WGN>(out_dt, a, st) : launch256_w4_out<W4F16, WGN>(out_dt, a, st);
+            if (two_stage_steps && !ring) return launch256_w4_out<W4F16L, WGN>(out_dt, a, plan);
+            return two_stage_steps ? launch256_w4_out<W4F16x2, WGN>(out_dt, a, plan) : launch256_w4_out<W4F16, WGN>(out_dt, a, plan);
         case MOYE_BF16:
-            if (two_stage_steps && !ring) return launch256_w4_out<W4BF16L, WGN>(out_dt, a, st);
-            return two_stage_steps ? launch256_w4_out<W4BF16x2, WGN>(out_dt, a, st) : launch256_w4_out<W4BF16, WGN>(out_dt, a, st);
-        case MOYE_F8E4M3: return ring ? launch256_w4_out<W4FP8, WGN>(out_dt, a, st) : launch256_w4_out<W4FP8L, WGN>(out_dt, a, st);
-        case MOYE_F32: return two_stage_steps && !ring ? launch256_w4_out<W4F32L, WGN>(out_dt, a, st) : launch256_w4_out<W4F32, WGN>(out_dt, a, st);
+            if (two_stage_steps && !ring) return launch256_w4_out<W4BF16L, WGN>(out_dt, a, plan);
+            return two_stage_steps ? launch256_w4_out<W4BF16x2, WGN>(out_dt, a, plan) : launch256_w4_out<W4BF16, WGN>(out_dt, a, plan);
+        case MOYE_F8E4M3: return ring ? launch256_w4_out<W4FP8, WGN>(out_dt, a, plan) : launch256_w4_out<W4FP8L, WGN>(out_dt, a, plan);
+        case MOYE_F32: return two_stage_steps && !ring ? launch256_w4_out<W4F32L, WGN>(out_dt, a, plan) : launch256_w4_out<W4F32, WGN>(out_dt, a, plan);
         default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: no MFMA atom for %s inputs", dtype_name(in_dt));
     }
 }
@@ -654,89 +665,86 @@ static int32_t launch256_w4_in(int32_t in_dt, int32_t out_dt, const GemmArgs& a,
 // 64); the caller has checked divisibility of M and N and alignment.
 // The 128 x 128 tile on the same kernel: plain f16 / bf16 calls on whole tiles, K a whole number of 128-byte rows; the
 // caller has checked divisibility and alignment.
-int32_t gemm_mfma_tn_128_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, hipStream_t st) {
+int32_t gemm_mfma_tn_128_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, GemmPlan& plan) {
     a.tiles_m = (a.M + 127) / 128;  // (beyond whole tiles only with kGemmRagged: the caller has checked; then no C either)
     a.tiles_n = (a.N + 127) / 128;
-    if (a.xcd_swizzle & kGemmRagged) {
+    if (a.flags & kGemmRagged) {
         if (a.C || a.ep_op != MOYE_MAP_IDENTITY) return fail(MOYE_ERR_UNSUPPORTED, "gemm!: ragged tiles of the hand-ordered kernel take no C and no epilogue operation");
         if (in_dt == MOYE_F32) {
             switch (out_dt) {
-                case MOYE_F32: return launch256_w4<W4F32L, OutF32, 2, false, true, 128>(a, st);
-                case MOYE_F16: return launch256_w4<W4F32L, OutF16, 2, false, true, 128>(a, st);
-                case MOYE_BF16: return launch256_w4<W4F32L, OutBF16, 2, false, true, 128>(a, st);
+                case MOYE_F32: return launch256_w4<W4F32L, OutF32, 2, false, true, 128>(a, plan);
+                case MOYE_F16: return launch256_w4<W4F32L, OutF16, 2, false, true, 128>(a, plan);
+                case MOYE_BF16: return launch256_w4<W4F32L, OutBF16, 2, false, true, 128>(a, plan);
                 default: break;
             }
         }
         if (in_dt == MOYE_F8E4M3) {
             switch (out_dt) {
-                case MOYE_F32: return launch256_w4<W4FP8L, OutF32, 2, false, true, 128>(a, st);
-                case MOYE_F16: return launch256_w4<W4FP8L, OutF16, 2, false, true, 128>(a, st);
-                case MOYE_BF16: return launch256_w4<W4FP8L, OutBF16, 2, false, true, 128>(a, st);
+                case MOYE_F32: return launch256_w4<W4FP8L, OutF32, 2, false, true, 128>(a, plan);
+                case MOYE_F16: return launch256_w4<W4FP8L, OutF16, 2, false, true, 128>(a, plan);
+                case MOYE_BF16: return launch256_w4<W4FP8L, OutBF16, 2, false, true, 128>(a, plan);
                 default: break;
             }
         }
         if (in_dt == MOYE_F16) {
             switch (out_dt) {
-                case MOYE_F32: return launch256_w4<W4F16L, OutF32, 2, false, true, 128>(a, st);
-                case MOYE_F16: return launch256_w4<W4F16L, OutF16, 2, false, true, 128>(a, st);
-                case MOYE_BF16: return launch256_w4<W4F16L, OutBF16, 2, false, true, 128>(a, st);
+                case MOYE_F32: return launch256_w4<W4F16L, OutF32, 2, false, true, 128>(a, plan);
+                case MOYE_F16: return launch256_w4<W4F16L, OutF16, 2, false, true, 128>(a, plan);
+                case MOYE_BF16: return launch256_w4<W4F16L, OutBF16, 2, false, true, 128>(a, plan);
                 default: break;
             }
         } else if (in_dt == MOYE_BF16) {
             switch (out_dt) {
-                case MOYE_F32: return launch256_w4<W4BF16L, OutF32, 2, false, true, 128>(a, st);
-                case MOYE_F16: return launch256_w4<W4BF16L, OutF16, 2, false, true, 128>(a, st);
-                case MOYE_BF16: return launch256_w4<W4BF16L, OutBF16, 2, false, true, 128>(a, st);
+                case MOYE_F32: return launch256_w4<W4BF16L, OutF32, 2, false, true, 128>(a, plan);
+                case MOYE_F16: return launch256_w4<W4BF16L, OutF16, 2, false, true, 128>(a, plan);
+                case MOYE_BF16: return launch256_w4<W4BF16L, OutBF16, 2, false, true, 128>(a, plan);
                 default: break;
             }
         }
         return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the hand-ordered 128x128 kernel takes f16 or bf16 operands and writes f32, f16 or bf16");
     }
-    if (128 * a.lda * dtype_bytes(in_dt) >= (int64_t)1 << 32 || 128 * a.ldb * dtype_bytes(in_dt) >= (int64_t)1 << 32)
-        return fail(MOYE_ERR_SHAPE, "gemm!: row pitch too large for the hand-ordered 128x128 MFMA kernel");
+    if (!row_offsets_fit(a, 128, dtype_bytes(in_dt))) return fail(MOYE_ERR_SHAPE, "gemm!: row pitch too large for the hand-ordered 128x128 MFMA kernel");
     if (in_dt == MOYE_F32) {
         switch (out_dt) {
-            case MOYE_F32: return launch256_w4<W4F32L, OutF32, 2, false, false, 128>(a, st);
-            case MOYE_F16: return launch256_w4<W4F32L, OutF16, 2, false, false, 128>(a, st);
-            case MOYE_BF16: return launch256_w4<W4F32L, OutBF16, 2, false, false, 128>(a, st);
+            case MOYE_F32: return launch256_w4<W4F32L, OutF32, 2, false, false, 128>(a, plan);
+            case MOYE_F16: return launch256_w4<W4F32L, OutF16, 2, false, false, 128>(a, plan);
+            case MOYE_BF16: return launch256_w4<W4F32L, OutBF16, 2, false, false, 128>(a, plan);
             default: break;
         }
     }
     if (in_dt == MOYE_F8E4M3) {  // (the 16x16x128 MFMA: twice the rate of the 16x16x32 one the other 128 x 128 kernels issue)
         switch (out_dt) {
-            case MOYE_F32: return launch256_w4<W4FP8L, OutF32, 2, false, false, 128>(a, st);
-            case MOYE_F16: return launch256_w4<W4FP8L, OutF16, 2, false, false, 128>(a, st);
-            case MOYE_BF16: return launch256_w4<W4FP8L, OutBF16, 2, false, false, 128>(a, st);
+            case MOYE_F32: return launch256_w4<W4FP8L, OutF32, 2, false, false, 128>(a, plan);
+            case MOYE_F16: return launch256_w4<W4FP8L, OutF16, 2, false, false, 128>(a, plan);
+            case MOYE_BF16: return launch256_w4<W4FP8L, OutBF16, 2, false, false, 128>(a, plan);
             default: break;
         }
     }
     if (in_dt == MOYE_F16) {
         switch (out_dt) {
-            case MOYE_F32: return launch256_w4<W4F16L, OutF32, 2, false, false, 128>(a, st);
-            case MOYE_F16: return launch256_w4<W4F16L, OutF16, 2, false, false, 128>(a, st);
-            case MOYE_BF16: return launch256_w4<W4F16L, OutBF16, 2, false, false, 128>(a, st);
+            case MOYE_F32: return launch256_w4<W4F16L, OutF32, 2, false, false, 128>(a, plan);
+            case MOYE_F16: return launch256_w4<W4F16L, OutF16, 2, false, false, 128>(a, plan);
+            case MOYE_BF16: return launch256_w4<W4F16L, OutBF16, 2, false, false, 128>(a, plan);
             default: break;
         }
     } else if (in_dt == MOYE_BF16) {
         switch (out_dt) {
-            case MOYE_F32: return launch256_w4<W4BF16L, OutF32, 2, false, false, 128>(a, st);
-            case MOYE_F16: return launch256_w4<W4BF16L, OutF16, 2, false, false, 128>(a, st);
-            case MOYE_BF16: return launch256_w4<W4BF16L, OutBF16, 2, false, false, 128>(a, st);
+            case MOYE_F32: return launch256_w4<W4BF16L, OutF32, 2, false, false, 128>(a, plan);
+            case MOYE_F16: return launch256_w4<W4BF16L, OutF16, 2, false, false, 128>(a, plan);
+            case MOYE_BF16: return launch256_w4<W4BF16L, OutBF16, 2, false, false, 128>(a, plan);
             default: break;
         }
     }
     return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the hand-ordered 128x128 kernel takes f16, bf16 or fp8 operands and writes f32, f16 or bf16");
 }
 
-int32_t gemm_mfma_tn_256_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, int waves, int kstep_bytes, bool ring, hipStream_t st) {
+int32_t gemm_mfma_tn_256_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, int waves, int kstep_bytes, bool ring, GemmPlan& plan) {
     a.tiles_m = (a.M + 255) / 256;  // (beyond whole tiles only with kGemmRagged: the caller has checked)
     a.tiles_n = (a.N + 255) / 256;
     // the load-to-LDS addresses are a uniform base plus a 32-bit lane offset
-    const int eb = dtype_bytes(in_dt);
-    if (256 * a.lda * eb >= (int64_t)1 << 32 || 256 * a.ldb * eb >= (int64_t)1 << 32)
-        return fail(MOYE_ERR_SHAPE, "gemm!: row pitch too large for the 256x256 MFMA kernel");
+    if (!row_offsets_fit(a, 256, dtype_bytes(in_dt))) return fail(MOYE_ERR_SHAPE, "gemm!: row pitch too large for the 256x256 MFMA kernel");
     const bool two = kstep_bytes == 128;
-    return waves == 4 ? launch256_w4_in<2>(in_dt, out_dt, a, two, ring, st) : launch256_w4_in<4>(in_dt, out_dt, a, two, ring, st);
+    return waves == 4 ? launch256_w4_in<2>(in_dt, out_dt, a, two, ring, plan) : launch256_w4_in<4>(in_dt, out_dt, a, two, ring, plan);
 }
 
 }  // namespace moye

@@ -49,7 +49,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_skinny(GemmArgs p) {
     // fetched instead of 161, 32.9 us instead of 34.0).  The order of a column's k-sum follows the workgroup, not
     // the time, so results stay reproducible.
     const int len = s1 - s0;
-    const int first = len >= U && len % U == 0 ? U * (int)((blockIdx.x / 8) % (unsigned)(len / U)) : 0;
+    const int first = len >= U && len % U == 0 ? U * (int)((blockIdx.x / (unsigned)p.xcds) % (unsigned)(len / U)) : 0;
     auto step_of = [&](int t) { const int r = t + first; return s0 + (r >= len ? r - len : r); };
     int t0 = 0;
     for (; t0 + U <= len; t0 += U) {
@@ -161,7 +161,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_skinny_lds(GemmArgs p) {
     // Workgroups that walk K in the same order ask their L2 for the same lines of A at the same moment, before any of
     // them has them: a workgroup starts its walk at a line that depends on its position within its L2's share of the
     // grid.  The order of a column's k-sum follows the workgroup, not the time, so results stay reproducible.
-    const int first = len > 0 ? (int)((blockIdx.x / 8) % (unsigned)len) : 0;
+    const int first = len > 0 ? (int)((blockIdx.x / (unsigned)p.xcds) % (unsigned)len) : 0;
     auto line_of = [&](int t) { const int r = t + first; return s0 + (r >= len ? r - len : r); };
 #define MOYE_STAGE_LOAD(T)                                                                                      \
     {                                                                                                           \
@@ -240,92 +240,88 @@ static bool skinny_lds_takes(const GemmArgs& a) {
 }
 
 template <typename In, typename Out, int MT, int W, int NTW, int S, int AUX>
-static int32_t launch_skinny_lds_v(const GemmArgs& a, hipStream_t st) {
+static int32_t launch_skinny_lds_v(const GemmArgs& a, GemmPlan& plan) {
     constexpr int kLds = W * S * (16 * NTW + 16 * MT) * 128;
     static LdsCap cap;
-    auto kern = gemm_mfma_skinny_lds<In, Out, MT, NTW, W, S, AUX>;
-    if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
-    const dim3 grid((unsigned)((a.N + 16 * NTW - 1) / (16 * NTW)), (unsigned)(a.split > 1 ? a.split : 1));
-    kern<<<grid, dim3(W * 64), kLds, st>>>(a);
-    MOYE_HIP_CHECK(hipGetLastError());
+    plan.add_kernel(gemm_mfma_skinny_lds<In, Out, MT, NTW, W, S, AUX>, a, (unsigned)((a.N + 16 * NTW - 1) / (16 * NTW)), (unsigned)(a.split > 1 ? a.split : 1),
+                    W * 64, kLds, &cap, 0, 16 * NTW, 128, In::kDt, Out::kDt, "gemm_mfma_skinny_lds<%s,%s,mt=%d,ntw=%d,waves=%d,stages=%d>", In::kName, Out::kName,
+                    MT, NTW, W, S);
+    return MOYE_OK;
+}
+// the kernel whose lanes stream their own 16-byte pieces of B into registers: MT x 16 rows of A, NTW x 16 rows of B per wave
+template <typename In, typename Out, int MT, int NTW, int W>
+static int32_t launch_skinny_regs(const GemmArgs& a, unsigned grid_x, GemmPlan& plan) {
+    plan.add_kernel(gemm_mfma_skinny<In, Out, MT, NTW, W>, a, grid_x, (unsigned)(a.split > 1 ? a.split : 1), W * 64, 0, nullptr, 0, 16 * NTW, 64, In::kDt, Out::kDt,
+                    "gemm_mfma_skinny<%s,%s,mt=%d,ntw=%d,waves=%d>", In::kName, Out::kName, MT, NTW, W);
     return MOYE_OK;
 }
 template <typename In, typename Out>
-static int32_t launch_skinny_lds(const GemmArgs& a, hipStream_t st) {
+static int32_t launch_skinny_lds(const GemmArgs& a, GemmPlan& plan) {
     constexpr int W = kSkinnyLdsWaves;
     // Waves x buffers, bf16 16 x 8192 x 8192, 32 rows of B per workgroup: 8 x 3 27.2 us, 8 x 2 25.2, 4 x 2 21.2, 4 x 3 21.0,
     // 4 x 4 21.2, 2 x 4 21.0, 2 x 3 22.6, 1 x 8 30.0; 64 rows per workgroup (half as many workgroups as CUs) 28.0-30.1;
     // B without the non-temporal hint 23.6.  As with the transposes, less in flight is faster on this part, down to what
     // covers the latency.  32 rows per workgroup once that gives every CU one (bf16, K = 8192: N = 16384 40.1 us against
     // 45.3 with 16 rows; N = 4096 17.9 against 13.5).
-    const bool wide = (a.N + 31) / 32 >= 256;
+    const bool wide = (a.N + 31) / 32 >= plan.shape.cus;
     if (wide) {
         switch ((a.M + 15) / 16) {
-            case 1: return launch_skinny_lds_v<In, Out, 1, W, 2, 3, 2>(a, st);
-            case 2: return launch_skinny_lds_v<In, Out, 2, W, 2, 3, 2>(a, st);
-            case 3: return launch_skinny_lds_v<In, Out, 3, W, 2, 3, 2>(a, st);
-            default: return launch_skinny_lds_v<In, Out, 4, W, 2, 3, 2>(a, st);
+            case 1: return launch_skinny_lds_v<In, Out, 1, W, 2, 3, 2>(a, plan);
+            case 2: return launch_skinny_lds_v<In, Out, 2, W, 2, 3, 2>(a, plan);
+            case 3: return launch_skinny_lds_v<In, Out, 3, W, 2, 3, 2>(a, plan);
+            default: return launch_skinny_lds_v<In, Out, 4, W, 2, 3, 2>(a, plan);
         }
     }
     switch ((a.M + 15) / 16) {
-        case 1: return launch_skinny_lds_v<In, Out, 1, W, 1, 3, 2>(a, st);
-        case 2: return launch_skinny_lds_v<In, Out, 2, W, 1, 3, 2>(a, st);
-        case 3: return launch_skinny_lds_v<In, Out, 3, W, 1, 3, 2>(a, st);
-        default: return launch_skinny_lds_v<In, Out, 4, W, 1, 3, 2>(a, st);
+        case 1: return launch_skinny_lds_v<In, Out, 1, W, 1, 3, 2>(a, plan);
+        case 2: return launch_skinny_lds_v<In, Out, 2, W, 1, 3, 2>(a, plan);
+        case 3: return launch_skinny_lds_v<In, Out, 3, W, 1, 3, 2>(a, plan);
+        default: return launch_skinny_lds_v<In, Out, 4, W, 1, 3, 2>(a, plan);
     }
 }
 
 template <typename In, typename Out>
-static int32_t launch_skinny(const GemmArgs& a, hipStream_t st) {
+static int32_t launch_skinny(const GemmArgs& a, GemmPlan& plan) {
     constexpr int W = 8;
-    // MOYE_SKINNY_LDS=0 keeps calls on the kernel above (to measure one against the other)
-    static const bool lds_off = getenv("MOYE_SKINNY_LDS") && atoi(getenv("MOYE_SKINNY_LDS")) == 0;
-    if (!lds_off && skinny_lds_takes<In>(a)) return launch_skinny_lds<In, Out>(a, st);
-    const dim3 block(W * 64);
+    if (skinny_lds_takes<In>(a)) return launch_skinny_lds<In, Out>(a, plan);
     // With K split over two or more workgroups there are enough workgroups to give each one 64 rows of B: A, which every
     // workgroup reads whole (its K range of it), then crosses the L2-to-CU path half as often.  Pays from M = 33 on
     // (bf16 64 x 8192 x 8192: 44.8 us with two K ranges, the second pass included, against 52.5 unsplit; M = 48: 41.3
     // against 55.3); without the split the larger workgroup tile is slower (68.8 us).
-    if (a.split > 1 && a.M > 32 && a.N % 64 == 0 && a.N / 64 >= 128) {
-        const dim3 grid((unsigned)(a.N / 64), (unsigned)(a.split > 1 ? a.split : 1));
-        if ((a.M + 15) / 16 == 3) gemm_mfma_skinny<In, Out, 3, 4, W><<<grid, block, 0, st>>>(a);
-        else gemm_mfma_skinny<In, Out, 4, 4, W><<<grid, block, 0, st>>>(a);
-        MOYE_HIP_CHECK(hipGetLastError());
-        return MOYE_OK;
+    if (a.split > 1 && a.M > 32 && a.N % 64 == 0 && a.N / 64 >= plan.shape.cus / 2) {
+        if ((a.M + 15) / 16 == 3) return launch_skinny_regs<In, Out, 3, 4, W>(a, (unsigned)(a.N / 64), plan);
+        return launch_skinny_regs<In, Out, 4, 4, W>(a, (unsigned)(a.N / 64), plan);
     }
-    if (a.N % 32 == 0 && a.N / 32 >= 256) {  // two B tiles per wave once that still fills the chip
-        const dim3 grid((unsigned)(a.N / 32), (unsigned)(a.split > 1 ? a.split : 1));
+    if (a.N % 32 == 0 && a.N / 32 >= plan.shape.cus) {  // two B tiles per wave once that still fills the chip
+        const unsigned gx = (unsigned)(a.N / 32);
         switch ((a.M + 15) / 16) {
-            case 1: gemm_mfma_skinny<In, Out, 1, 2, W><<<grid, block, 0, st>>>(a); break;
-            case 2: gemm_mfma_skinny<In, Out, 2, 2, W><<<grid, block, 0, st>>>(a); break;
-            case 3: gemm_mfma_skinny<In, Out, 3, 2, W><<<grid, block, 0, st>>>(a); break;
-            default: gemm_mfma_skinny<In, Out, 4, 2, W><<<grid, block, 0, st>>>(a); break;
-        }
-    } else {
-        const dim3 grid((unsigned)((a.N + 15) / 16), (unsigned)(a.split > 1 ? a.split : 1));
-        switch ((a.M + 15) / 16) {
-            case 1: gemm_mfma_skinny<In, Out, 1, 1, W><<<grid, block, 0, st>>>(a); break;
-            case 2: gemm_mfma_skinny<In, Out, 2, 1, W><<<grid, block, 0, st>>>(a); break;
-            case 3: gemm_mfma_skinny<In, Out, 3, 1, W><<<grid, block, 0, st>>>(a); break;
-            default: gemm_mfma_skinny<In, Out, 4, 1, W><<<grid, block, 0, st>>>(a); break;
+            case 1: return launch_skinny_regs<In, Out, 1, 2, W>(a, gx, plan);
+            case 2: return launch_skinny_regs<In, Out, 2, 2, W>(a, gx, plan);
+            case 3: return launch_skinny_regs<In, Out, 3, 2, W>(a, gx, plan);
+            default: return launch_skinny_regs<In, Out, 4, 2, W>(a, gx, plan);
         }
     }
-    MOYE_HIP_CHECK(hipGetLastError());
-    return MOYE_OK;
+    const unsigned gx = (unsigned)((a.N + 15) / 16);
+    switch ((a.M + 15) / 16) {
+        case 1: return launch_skinny_regs<In, Out, 1, 1, W>(a, gx, plan);
+        case 2: return launch_skinny_regs<In, Out, 2, 1, W>(a, gx, plan);
+        case 3: return launch_skinny_regs<In, Out, 3, 1, W>(a, gx, plan);
+        default: return launch_skinny_regs<In, Out, 4, 1, W>(a, gx, plan);
+    }
 }
 
 template <typename In>
-static int32_t launch_skinny_out(int32_t out_dt, const GemmArgs& a, hipStream_t st) {
+static int32_t launch_skinny_out(int32_t out_dt, const GemmArgs& a, GemmPlan& plan) {
     switch (out_dt) {
-        case MOYE_F32: return launch_skinny<In, OutF32>(a, st);
-        case MOYE_F16: return launch_skinny<In, OutF16>(a, st);
-        case MOYE_BF16: return launch_skinny<In, OutBF16>(a, st);
+        case MOYE_F32: return launch_skinny<In, OutF32>(a, plan);
+        case MOYE_F16: return launch_skinny<In, OutF16>(a, plan);
+        case MOYE_BF16: return launch_skinny<In, OutBF16>(a, plan);
         default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: MFMA kernels write f32, f16 or bf16, not %s", dtype_name(out_dt));
     }
 }
 
 // 1 <= M <= 64, any N, K a multiple of 64 bytes; pointers and pitches 16-byte aligned.
-int32_t gemm_mfma_skinny_dispatch(int32_t in_dt, int32_t out_dt, const GemmArgs& a, hipStream_t st) {
+int32_t gemm_mfma_skinny_dispatch(int32_t in_dt, int32_t out_dt, const GemmArgs& a, GemmPlan& plan) {
     const int eb = dtype_bytes(in_dt);
     if (a.M < 1 || a.M > 64 || a.N < 1 || ((int64_t)a.K * eb) % 64)
         return fail(MOYE_ERR_SHAPE, "gemm!: the short-M MFMA kernel needs 1 <= M <= 64 and K %% %d == 0, got %dx%dx%d",
@@ -334,10 +330,10 @@ int32_t gemm_mfma_skinny_dispatch(int32_t in_dt, int32_t out_dt, const GemmArgs&
         (reinterpret_cast<uintptr_t>(a.A) | reinterpret_cast<uintptr_t>(a.B)) % 16)
         return fail(MOYE_ERR_ALIGN, "gemm!: operands of the MFMA kernels need 16-byte aligned pointers and row pitches");
     switch (in_dt) {
-        case MOYE_F16: return launch_skinny_out<InF16>(out_dt, a, st);
-        case MOYE_BF16: return launch_skinny_out<InBF16>(out_dt, a, st);
-        case MOYE_F8E4M3: return launch_skinny_out<InFP8>(out_dt, a, st);
-        case MOYE_F32: return launch_skinny_out<InF32>(out_dt, a, st);
+        case MOYE_F16: return launch_skinny_out<InF16>(out_dt, a, plan);
+        case MOYE_BF16: return launch_skinny_out<InBF16>(out_dt, a, plan);
+        case MOYE_F8E4M3: return launch_skinny_out<InFP8>(out_dt, a, plan);
+        case MOYE_F32: return launch_skinny_out<InF32>(out_dt, a, plan);
         default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: no MFMA atom for %s inputs", dtype_name(in_dt));
     }
 }

@@ -1,5 +1,6 @@
 // Host-side choice of CTA tile and K ranges for a gemm! whose tile is left to the library and that does not fill the chip
-// with 256 x 256 tiles: a small cost model instead of thresholds, fitted to fp16 timings on one MI355X (256 CUs).
+// with 256 x 256 tiles: a small cost model instead of thresholds.  Its per-k-tile times are fitted to fp16 timings on one
+// MI355X; the number of compute units that share the work is an argument (DeviceShape::cus).
 //
 //   time = 3 us + k-tiles per workgroup x t(tile, workgroups resident on a CU) [x rounds] + second pass of a K split
 //
@@ -17,13 +18,13 @@
 
 namespace moye {
 
-struct GemmPlan {
+struct TileChoice {
     int tile;   // 64 or 128
     int split;  // K ranges
     double us;
 };
 
-inline double gemm_plan_cost(int tile, int split, int64_t M, int64_t N, int64_t k_bytes, bool f32_in) {
+inline double gemm_plan_cost(int tile, int split, int64_t M, int64_t N, int64_t k_bytes, bool f32_in, int cus) {
     const int64_t tiles = ((M + tile - 1) / tile) * ((N + tile - 1) / tile), ctas = tiles * split;
     const int slots = tile == 128 ? 2 : 4;
     // per k-tile and workgroup with 1 .. slots workgroups resident on a CU.  fp32 operands run on v_mfma_f32_16x16x4_f32,
@@ -33,9 +34,9 @@ inline double gemm_plan_cost(int tile, int split, int64_t M, int64_t N, int64_t 
     static const double t128_32[3] = {0, 1.96, 4.58}, t64_32[5] = {0, 0.71, 1.25, 1.80, 2.40};
     const double* t = tile == 128 ? (f32_in ? t128_32 : t128_16) : (f32_in ? t64_32 : t64_16);
     const double ktiles = (double)((k_bytes / split + 127) / 128);
-    // whole rounds of 256 x slots workgroups, then the rest with fewer neighbours
-    const int64_t full = ctas / (256 * slots), rest = ctas % (256 * slots);
-    double us = 3.0 + ktiles * ((double)full * t[slots] + (rest ? t[(rest + 255) / 256] : 0.0));
+    // whole rounds of cus x slots workgroups, then the rest with fewer neighbours
+    const int64_t full = ctas / ((int64_t)cus * slots), rest = ctas % ((int64_t)cus * slots);
+    double us = 3.0 + ktiles * ((double)full * t[slots] + (rest ? t[(rest + cus - 1) / cus] : 0.0));
     if (tile == 128 && (M % 128 || N % 128 || k_bytes % 128)) us *= 1.15;
     if (split > 1) us += 3.0 + (2.0 * split * 4.0 + 4.0) * (double)M * (double)N / 6.0e6;
     return us;
@@ -43,9 +44,9 @@ inline double gemm_plan_cost(int tile, int split, int64_t M, int64_t N, int64_t 
 
 // `max_split` = 1 forbids K ranges (no workspace); `fixed_split` > 0 asks for the best tile for that many ranges (the
 // dispatch after the split has been made: k_bytes is then the whole K again, so both calls price the same candidates).
-inline GemmPlan gemm_plan(int64_t M, int64_t N, int64_t k_bytes, bool f32_in, bool tile64_ok, int max_split,
-                          int fixed_split = 0) {
-    GemmPlan best{128, fixed_split > 0 ? fixed_split : 1, 1e30};
+inline TileChoice gemm_plan(int64_t M, int64_t N, int64_t k_bytes, bool f32_in, bool tile64_ok, int max_split, int cus,
+                            int fixed_split = 0) {
+    TileChoice best{128, fixed_split > 0 ? fixed_split : 1, 1e30};
     for (int tile : {128, 64}) {
         if (tile == 64 && !tile64_ok) continue;
         for (int s = 1; s <= 16; s *= 2) {
@@ -54,8 +55,8 @@ inline GemmPlan gemm_plan(int64_t M, int64_t N, int64_t k_bytes, bool f32_in, bo
                 // equal ranges of whole k-tiles, at least four of them
                 if (s > max_split || k_bytes % s || (k_bytes / s) % 128 || k_bytes / s < 512) continue;
             }
-            const double us = gemm_plan_cost(tile, s, M, N, k_bytes, f32_in);
-            if (us < best.us) best = GemmPlan{tile, s, us};
+            const double us = gemm_plan_cost(tile, s, M, N, k_bytes, f32_in, cus);
+            if (us < best.us) best = TileChoice{tile, s, us};
         }
     }
     return best;
@@ -65,15 +66,30 @@ inline GemmPlan gemm_plan(int64_t M, int64_t N, int64_t k_bytes, bool f32_in, bo
 // 0.98 us in one that fills half of it or less (fewer requesters, and a higher clock on a part that is power-limited when
 // full), linear in between (fp16 K = 4096: 256 tiles 101 us, 224 91, 192 83, 144 73, 128 72); a quarter more for the
 // guarded instance (130 x 32768 x 4096 on 128 ragged tiles: 99 us).
-inline double gemm_plan_cost_256(int64_t M, int64_t N, int64_t k_bytes, bool f32_in, bool ragged) {
-    const int64_t tiles = ((M + 255) / 256) * ((N + 255) / 256), full = tiles / 256, rest = tiles % 256;
+inline double gemm_plan_cost_256(int64_t M, int64_t N, int64_t k_bytes, bool f32_in, bool ragged, int cus) {
+    const int64_t tiles = ((M + 255) / 256) * ((N + 255) / 256), full = tiles / cus, rest = tiles % cus;
+    const int half = cus / 2 > 0 ? cus / 2 : 1;
     const double ktiles = (double)((k_bytes + 127) / 128);
     // (fp32: 7.56 us per k-tile however many CUs are busy: the matrix pipe alone sets the pace, 4096 x 4096 x 1024 251 us)
     const double t_full = f32_in ? 7.56 : 1.44;
-    const double t_rest = rest == 0 ? 0.0 : f32_in ? 7.56 : rest <= 128 ? 0.98 : 0.98 + (double)(rest - 128) / 128.0 * 0.46;
+    const double t_rest = rest == 0 ? 0.0 : f32_in ? 7.56 : rest <= half ? 0.98 : 0.98 + (double)(rest - half) / (double)half * 0.46;
     double us = 9.0 + 6.0 * (double)(full + (rest ? 1 : 0) - 1) + ktiles * ((double)full * t_full + t_rest);
     if (ragged) us *= 1.25;
     return us;
+}
+
+// Everything left to the library (tile, waves, K ranges): the cheapest of 64 x 64 / 128 x 128 tiles with 1 .. max_split K
+// ranges and of unsplit 256 x 256 tiles, which are considered from a quarter of the CUs' worth of tiles on.  The one
+// place where tile and K ranges are chosen together: the workspace sizing and the dispatcher both take their answer
+// from here.
+inline TileChoice gemm_choose(int64_t M, int64_t N, int64_t k_bytes, bool f32_in, int max_split, int cus) {
+    TileChoice best = gemm_plan(M, N, k_bytes, f32_in, M % 64 == 0 && N % 64 == 0 && k_bytes % 128 == 0, max_split, cus);
+    const bool ragged = M % 256 || N % 256 || k_bytes % 128;
+    if (((M + 255) / 256) * ((N + 255) / 256) >= cus / 4) {
+        const double us = gemm_plan_cost_256(M, N, k_bytes, f32_in, ragged, cus);
+        if (us <= best.us) best = TileChoice{256, 1, us};
+    }
+    return best;
 }
 
 }  // namespace moye

@@ -1,6 +1,8 @@
 // Argument blocks and dispatch entry points shared by the kernel translation units and capi.hip.
 #pragma once
 
+#include <vector>
+
 #include "moye_common.hpp"
 
 namespace moye {
@@ -27,17 +29,19 @@ struct GemmArgs {
     // and writes its product split_d bytes further (compact fp32 partial products, one after the other)
     int split;
     int64_t split_ab, split_d;
-    int xcd_swizzle;  // bit 0: XCD-aware tile order; bits 8-15: MOYE_GEMM_* schedule flags; kGemmAtom32
+    int flags;  // bit 0: XCD-aware tile order; bits 8-15: the MOYE_GEMM_* schedule flags of the descriptor; the kGemm* bits below
+    int xcds;   // how many XCDs the hardware deals consecutive workgroup ids to (DeviceShape::xcds): the tile order and the K rotation count with it
 };
-constexpr int kGemmAtom32 = 0x10000;   // in GemmArgs::xcd_swizzle: issue the 32x32 MFMA forms
-constexpr int kGemmRowC = 0x80000;    // in GemmArgs::xcd_swizzle: C has unit stride along n, 16-byte aligned rows: read in 128-bit pieces
-constexpr int kGemmStreamD = 0x40000;  // in GemmArgs::xcd_swizzle: D is written with non-temporal stores
-constexpr int kGemmAMajorM = 0x100000;  // in GemmArgs::xcd_swizzle: A has its unit stride along M, lda is the pitch between consecutive k
-constexpr int kGemmBMajorN = 0x200000;  // the same for B and N (the 256 x 256 kernel's transposing fragment reads; 16-bit types)
-constexpr int kGemmEpiRowX = 0x400000;  // in GemmArgs::xcd_swizzle: the epilogue operand has unit stride along n and 16-byte aligned rows (or one row)
-constexpr int kGemmRagged = 0x800000;   // in GemmArgs::xcd_swizzle: the 256 x 256 kernel runs with tiles that reach beyond M, N or K (its guarded instance)
-constexpr int kGemmEpiAddVec = 0x1000000;  // in GemmArgs::xcd_swizzle: the epilogue operation adds a one-per-column or one-per-row vector or a scalar
-constexpr int kGemmRotateK = 0x20000;  // in GemmArgs::xcd_swizzle: each XCD starts its walk over K at its own eighth
+// bits of GemmArgs::flags that the host sets for the kernels (the descriptor's own flags occupy bits 0-15)
+constexpr int kGemmAtom32 = 0x10000;   // issue the 32x32 MFMA forms
+constexpr int kGemmRotateK = 0x20000;  // each XCD starts its walk over K at its own share of K
+constexpr int kGemmStreamD = 0x40000;  // D is written with non-temporal stores
+constexpr int kGemmRowC = 0x80000;     // C has unit stride along n, 16-byte aligned rows: read in 128-bit pieces
+constexpr int kGemmAMajorM = 0x100000;  // A has its unit stride along M, lda is the pitch between consecutive k
+constexpr int kGemmBMajorN = 0x200000;  // the same for B and N (the kernels' transposing fragment reads)
+constexpr int kGemmEpiRowX = 0x400000;  // the epilogue operand has unit stride along n and 16-byte aligned rows (or one row)
+constexpr int kGemmRagged = 0x800000;   // tiles reach beyond M, N or K (the guarded instances)
+constexpr int kGemmEpiAddVec = 0x1000000;  // the epilogue operation adds a one-per-column or one-per-row vector or a scalar
 
 // UniversalFMA GEMM, any strides (gemm_universal.hip)
 struct UArgs {
@@ -48,17 +52,69 @@ struct UArgs {
     int a_dt, b_dt, c_dt, d_dt;
 };
 
+// What the host needs to know of the chip to choose tiles: compute units, and the XCDs that consecutive workgroup ids are
+// dealt to (32 CUs each on gfx950; a partitioned part shows fewer of both).  Read once per device; 256 / 8 when there is
+// no device to ask (planning on a host without a GPU).
+struct DeviceShape {
+    int cus, xcds;
+};
+DeviceShape device_shape();
+// `cus` > 0 overrides what the device says, for planning (moye_gemm_explain) and its tests
+DeviceShape device_shape_for(int cus);
+
+// The load-to-LDS kernels address operand rows as a uniform base plus a 32-bit lane offset: `rows` rows of either
+// operand must span less than 4 GiB.
+inline bool row_offsets_fit(const GemmArgs& a, int rows, int elem_bytes) {
+    return (int64_t)rows * a.lda * elem_bytes < ((int64_t)1 << 32) && (int64_t)rows * a.ldb * elem_bytes < ((int64_t)1 << 32);
+}
+
+// ---- a gemm! call as a list of launches ---------------------------------------------------------------------------
+// The host code that chooses kernels (capi.hip: gemm_plan_build; gemm_mfma.hip and the kernel files' dispatch functions)
+// launches nothing: it appends steps to a GemmPlan.  gemm_plan_run (capi.hip) then enqueues them on a stream, and
+// moye_gemm_explain prints them.  Building a plan touches no device, so it runs, and is tested, on hosts without one.
+struct GemmStep {
+    enum Kind { kKernel, kKMajorCopy, kSplitKReduce, kUniversal } kind = kKernel;
+    // kKernel: one launch of an MFMA kernel instance
+    char name[160] = {0};              // kernel function and template arguments, e.g. gemm_mfma_tn_256_w4<W4F16L,OutF16,waves=8>
+    void (*kernel)(GemmArgs) = nullptr;
+    GemmArgs args{};
+    unsigned grid_x = 0, grid_y = 1, block = 0;
+    int lds_bytes = 0;
+    struct LdsCap* cap = nullptr;      // set when the kernel needs its dynamic-LDS cap raised (once per device)
+    int tile_m = 0, tile_n = 0, tile_k_bytes = 0;  // CTA tile of the instance (0: the short-M kernels, which have none)
+    int in_dt = 0, out_dt = 0;
+    // kKMajorCopy: src (rows x cols with the unit stride along rows) -> dst (cols contiguous), through moye_copy's kernels
+    moye_tensor copy_dst{}, copy_src{};
+    // kSplitKReduce: sums `split` fp32 partial products of M x N in args.D's place (P) and applies the epilogue of `args`
+    const float* partials = nullptr;
+    int split = 0;
+    // kUniversal: the UniversalFMA kernel on CTA tile (ubm, ubn, ubk)
+    UArgs uargs{};
+    int ubm = 0, ubn = 0, ubk = 0;
+};
+struct GemmPlan {
+    std::vector<GemmStep> steps;
+    DeviceShape shape{256, 8};
+    size_t workspace_bytes = 0;  // what the steps use of the workspace (K-major operand copies, then split-K partial products)
+    char* workspace = nullptr;   // where it is
+    // appends a kernel launch; `name` is printf-style
+    GemmStep& add_kernel(void (*kernel)(GemmArgs), const GemmArgs& a, unsigned grid_x, unsigned grid_y, unsigned block, int lds_bytes,
+                         struct LdsCap* cap, int tile_m, int tile_n, int tile_k_bytes, int in_dt, int out_dt, const char* fmt, ...)
+        __attribute__((format(printf, 14, 15)));
+};
 int32_t copy_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, const moye_tensor* src, hipStream_t st);
 int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, const moye_tensor* src, const moye_tensor* mask,
                          hipStream_t st);
+// The functions below choose kernel instances and append them to `plan`; none of them launches.
+struct TileChoice;  // gemm_plan.hpp
 int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int bk_elems, int waves, int stages,
-                              GemmArgs a, hipStream_t st);
-int32_t gemm_mfma_tn_256_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, int waves, int stages, hipStream_t st);
-int32_t gemm_mfma_tn_256_pp_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, hipStream_t st);
-int32_t gemm_mfma_tn_128_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, hipStream_t st);
-int32_t gemm_mfma_tn_256_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, int waves, int kstep_bytes, bool ring, hipStream_t st);
-int32_t gemm_mfma_tn_128_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, hipStream_t st);
-int32_t gemm_mfma_skinny_dispatch(int32_t in_dt, int32_t out_dt, const GemmArgs& a, hipStream_t st);
+                              GemmArgs a, GemmPlan& plan, const TileChoice* lib = nullptr);
+int32_t gemm_mfma_tn_256_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, int waves, int stages, GemmPlan& plan);
+int32_t gemm_mfma_tn_256_pp_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, GemmPlan& plan);
+int32_t gemm_mfma_tn_128_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, GemmPlan& plan);
+int32_t gemm_mfma_tn_256_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, int waves, int kstep_bytes, bool ring, GemmPlan& plan);
+int32_t gemm_mfma_tn_128_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, GemmPlan& plan);
+int32_t gemm_mfma_skinny_dispatch(int32_t in_dt, int32_t out_dt, const GemmArgs& a, GemmPlan& plan);
 // The short-M kernel stages whole 128-byte lines of K through LDS, four waves with a K range each, when K is this many
 // bytes or a multiple of it (else every lane loads its own 16-byte pieces).
 constexpr int kSkinnyLineBytes = 128;

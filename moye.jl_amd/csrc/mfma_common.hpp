@@ -15,7 +15,8 @@ typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 
 // ---- input element traits: how one pair of 16-byte chunks feeds the MFMA pipe ----------------
 struct InF16 {
-    static constexpr int kBytes = 2;
+    static constexpr int kBytes = 2, kDt = MOYE_F16;
+    static constexpr const char* kName = "InF16";
     static __device__ __forceinline__ void mma(const u32x4& a, const u32x4& b, f32x4& c) {
         c = __builtin_amdgcn_mfma_f32_16x16x32_f16((f16x8)a, (f16x8)b, c, 0, 0, 0);
     }
@@ -30,7 +31,8 @@ struct InF16 {
     }
 };
 struct InBF16 {
-    static constexpr int kBytes = 2;
+    static constexpr int kBytes = 2, kDt = MOYE_BF16;
+    static constexpr const char* kName = "InBF16";
     static __device__ __forceinline__ void mma(const u32x4& a, const u32x4& b, f32x4& c) {
         c = __builtin_amdgcn_mfma_f32_16x16x32_bf16((bf16x8)a, (bf16x8)b, c, 0, 0, 0);
     }
@@ -44,7 +46,8 @@ struct InBF16 {
 // A 16-byte chunk holds 16 fp8 values = the k-slices of two MFMAs.  Both operands split the
 // chunk the same way, so the pairing of products is unchanged.
 struct InFP8 {
-    static constexpr int kBytes = 1;
+    static constexpr int kBytes = 1, kDt = MOYE_F8E4M3;
+    static constexpr const char* kName = "InFP8";
     static __device__ __forceinline__ void mma(const u32x4& a, const u32x4& b, f32x4& c) {
         const long a0 = (long)(((uint64_t)a.y << 32) | a.x), a1 = (long)(((uint64_t)a.w << 32) | a.z);
         const long b0 = (long)(((uint64_t)b.y << 32) | b.x), b1 = (long)(((uint64_t)b.w << 32) | b.z);
@@ -68,7 +71,8 @@ struct InFP8 {
 // MFMA j multiplies the k-slices {j, 4+j, 8+j, 12+j} of a 64-byte row piece; A and B are cut the
 // same way, so every product a[m][k] * b[n][k] is formed exactly once.
 struct InF32 {
-    static constexpr int kBytes = 4;
+    static constexpr int kBytes = 4, kDt = MOYE_F32;
+    static constexpr const char* kName = "InF32";
     static __device__ __forceinline__ void mma(const u32x4& a, const u32x4& b, f32x4& c) {
 #pragma unroll
         for (int j = 0; j < 4; ++j)
@@ -85,16 +89,22 @@ struct InF32 {
 // ---- output element traits: fp32 -> OutT, round to nearest even (src/arch/copy/copy.jl:38-43) ---
 struct OutF32 {
     typedef float type;
+    static constexpr int kDt = MOYE_F32;
+    static constexpr const char* kName = "OutF32";
     static __device__ __forceinline__ float cvt(float x) { return x; }
     static __device__ __forceinline__ float load(const void* p, int64_t i) { return static_cast<const float*>(p)[i]; }
 };
 struct OutF16 {
     typedef _Float16 type;
+    static constexpr int kDt = MOYE_F16;
+    static constexpr const char* kName = "OutF16";
     static __device__ __forceinline__ _Float16 cvt(float x) { return (_Float16)x; }
     static __device__ __forceinline__ float load(const void* p, int64_t i) { return (float)static_cast<const _Float16*>(p)[i]; }
 };
 struct OutBF16 {
     typedef uint16_t type;
+    static constexpr int kDt = MOYE_BF16;
+    static constexpr const char* kName = "OutBF16";
     static __device__ __forceinline__ uint16_t cvt(float x) {
         uint32_t u = __float_as_uint(x);
         if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
@@ -161,13 +171,13 @@ __device__ __forceinline__ void split_of_block(GemmArgs& p) {
     }
 }
 
-// One 16-byte piece of D.  With kGemmStreamD in GemmArgs::xcd_swizzle the store is non-temporal: when a launch has
+// One 16-byte piece of D.  With kGemmStreamD in GemmArgs::flags the store is non-temporal: when a launch has
 // more tiles than the chip has CUs, results written the ordinary way sit in the L2s and push out the operand panels
 // the next tiles are about to share.
 __device__ __forceinline__ void store_d_chunk(const GemmArgs& p, char* d, const u32x4& w) {
     // (as text: the compiler merges an ordinary and a non-temporal store in the two arms of a branch into one ordinary
     // store; the nop covers the wait states a wide store needs before its data registers are written again)
-    if (p.xcd_swizzle & kGemmStreamD) asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 1" ::"v"(d), "v"(w) : "memory");
+    if (p.flags & kGemmStreamD) asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 1" ::"v"(d), "v"(w) : "memory");
     else *reinterpret_cast<u32x4*>(d) = w;
 }
 
@@ -178,7 +188,8 @@ __device__ __forceinline__ void store_d_chunk(const GemmArgs& p, char* d, const 
 __device__ __forceinline__ void tile_of_block(const GemmArgs& p, int* tm, int* tn) {
     int bid = blockIdx.x;
     const int n = gridDim.x;
-    if ((p.xcd_swizzle & 1) && (n % 8) == 0) bid = (bid % 8) * (n / 8) + bid / 8;
+    const int x = p.xcds;
+    if ((p.flags & 1) && x > 1 && (n % x) == 0) bid = (bid % x) * (n / x) + bid / x;
     constexpr int kGroup = 8;
     const int per_group = kGroup * p.tiles_n;
     const int g = bid / per_group;

@@ -63,7 +63,7 @@ __device__ __forceinline__ void store_c_tile_general(const GemmArgs& p, const f3
             }
             // beta * C: a 16-byte piece of the row where C allows it (kGemmRowC), element by element otherwise
             if (p.C) {
-                if ((p.xcd_swizzle & kGemmRowC) && whole) {
+                if ((p.flags & kGemmRowC) && whole) {
                     OutT cw[EPC];
                     const u32x4 w = *reinterpret_cast<const u32x4*>(static_cast<const char*>(p.C) + (m * p.ldc_m + n0) * (int64_t)sizeof(OutT));
                     __builtin_memcpy(cw, &w, 16);
@@ -83,7 +83,7 @@ __device__ __forceinline__ void store_c_tile_general(const GemmArgs& p, const f3
                 const float xr = epi_operand(p, m, 0);
 #pragma unroll
                 for (int e = 0; e < EPC; ++e) x[e] = xr;
-            } else if ((p.xcd_swizzle & kGemmEpiRowX) && whole) {
+            } else if ((p.flags & kGemmEpiRowX) && whole) {
                 if (p.ep_xdt == MOYE_F32) {
                     const f32x4* xp = reinterpret_cast<const f32x4*>(static_cast<const float*>(p.ep_x) + m * p.ep_xm + n0);
 #pragma unroll
@@ -180,7 +180,7 @@ __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&ac
     constexpr int NCH = PASS_ROWS * CR / 64, PASSES = MI / PASS_MI;
     constexpr int AHEAD = sizeof(OutT) == 2 ? PASSES : (PASSES < 2 ? PASSES : 2);
     // (ragged tiles read C in whole pieces only when no piece crosses N)
-    const bool row_c = !kNoC && p.C && (p.xcd_swizzle & kGemmRowC) && (!kGuard || p.N % EPC == 0);
+    const bool row_c = !kNoC && p.C && (p.flags & kGemmRowC) && (!kGuard || p.N % EPC == 0);
     [[maybe_unused]] u32x4 cw[kNoC ? 1 : AHEAD][NCH];
     auto fetch_c = [&](int pass, u32x4 (&into)[NCH]) __attribute__((always_inline)) {
 #pragma unroll

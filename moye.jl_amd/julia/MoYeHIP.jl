@@ -548,6 +548,26 @@ function gemm_ex_workspace_size(mma::TiledMMADesc, D::MoYeArray, A::MoYeArray, B
     Int(n[])
 end
 
+"""
+    gemm_explain(mma, D, A, B[, C]; op, compute_units) -> String
+
+The launches `gemm!` / `gemm_ex!` would make for these descriptors (kernel instance, grid, tile, sub-problem, K ranges,
+flags; one line per launch).  Host arithmetic only: nothing is launched and the arrays' memory is not touched.
+"""
+function gemm_explain(mma::TiledMMADesc, D::MoYeArray, A::MoYeArray, B::MoYeArray, C::Union{Nothing,MoYeArray} = nothing;
+                      op::Int32 = MAP_IDENTITY, compute_units::Integer = 0)
+    buf = Vector{UInt8}(undef, 1 << 16)
+    c = C === nothing ? nothing : Ref(Tensor(C))
+    GC.@preserve D A B C c buf begin
+        cp = c === nothing ? Ptr{Tensor}(C_NULL) : Base.unsafe_convert(Ptr{Tensor}, c)
+        ep = Ref(GemmEpilogue(1.0f0, C === nothing ? 0.0f0 : 1.0f0, op, Int32(0), Ptr{Tensor}(C_NULL), 0.0))
+        check(ccall((:moye_gemm_explain, LIB), Int32,
+                    (Ptr{TiledMMADesc}, Ptr{Tensor}, Ptr{Tensor}, Ptr{Tensor}, Ptr{Tensor}, Ptr{GemmEpilogue}, Int32, Ptr{UInt8}, Csize_t),
+                    Ref(mma), Ref(Tensor(D)), Ref(Tensor(A)), Ref(Tensor(B)), cp, ep, Int32(compute_units), buf, length(buf)))
+    end
+    unsafe_string(pointer(buf))
+end
+
 # ---- device memory without a Julia GPU package ------------------------------------------------
 function device_malloc(bytes::Integer)
     p = Ref{Ptr{Cvoid}}(C_NULL)

@@ -12,7 +12,7 @@ from ._lib import (BF16, COPY_LDS_TILED, COPY_UNIVERSAL, F8E4M3, F16, F32, F64, 
                    MFMA_F32_32x32x16_F16, MFMA_F32_32x32x16_FP8, MMA_UNIVERSAL_FMA, U8, U16, U32, U64, U128,
                    MoyeError, Tensor, TiledCopy, TiledMMA, check, lib, make_tensor)
 from . import device
-from .device import device_info, gemm_epilogue, gemm_ex_, gemm_noalloc_, gemm_release_workspace, mfma_ceiling, mma_atom_probe, tiled_copy_desc, tiled_mma_desc, time_copy, time_gemm, gemm_workspace_size, version
+from .device import device_info, gemm_epilogue, gemm_ex_, gemm_noalloc_, gemm_release_workspace, mfma_ceiling, mma_atom_probe, tiled_copy_desc, tiled_mma_desc, time_copy, time_gemm, gemm_workspace_size, gemm_explain, parse_plan, version
 from .layout import (COLON, GenColMajor, GenRowMajor, Int32, Layout, StaticInt, append, blocked_product, coalesce,
                      compact_col_major, compact_row_major, complement, composition, coord_to_index, cosize, depth,
                      flatten, index_to_coord, left_inverse, logical_divide, logical_product, make_fragment_like,

@@ -90,6 +90,7 @@ def _declare(l):
         "moye_gemm_noalloc": [P(TiledMMA), P(Tensor), P(Tensor), P(Tensor), P(Tensor), C.c_float, vp],
         "moye_gemm_workspace_size": [P(TiledMMA), P(Tensor), P(Tensor), P(Tensor), P(S)],
         "moye_gemm_ex_workspace_size": [P(TiledMMA), P(Tensor), P(Tensor), P(Tensor), P(GemmEpilogue), P(S)],
+        "moye_gemm_explain": [P(TiledMMA), P(Tensor), P(Tensor), P(Tensor), P(Tensor), P(GemmEpilogue), I32, cs, S],
         "moye_device_malloc": [P(vp), S], "moye_device_free": [vp],
         "moye_memcpy_h2d": [vp, vp, S], "moye_memcpy_d2h": [vp, vp, S], "moye_memset": [vp, C.c_int, S],
         "moye_device_sync": [],

@@ -108,6 +108,43 @@ def gemm_workspace_size(mma, D, A, B, epilogue=None):
     return n.value
 
 
+def gemm_explain(mma, D, A, B, C_=None, epilogue=None, compute_units=0):
+    """The launches a gemm! call would make (moye_gemm_explain): a list of dicts, one per step, with the step's `what`
+    ("kernel", "kmajor_copy", "splitk_reduce"), the kernel's `name` and the `key=value` fields of its line (integers where
+    they are integers), plus the first line's `workspace` bytes under the key "plan".  Host arithmetic only: the data
+    pointers of the descriptors are never dereferenced."""
+    buf = C.create_string_buffer(1 << 16)
+    check(lib().moye_gemm_explain(C.byref(mma), C.byref(D), C.byref(A), C.byref(B), _ref(C_),
+                                  C.byref(epilogue) if epilogue is not None else None, compute_units, buf, len(buf)))
+    return parse_plan(buf.value.decode())
+
+
+def parse_plan(text):
+    """moye_gemm_explain's text as {"workspace": bytes, "cus": n, "xcds": n, "steps": [dict, ...], "text": text}."""
+    lines = text.strip().splitlines()
+    head = lines[0].split()
+    plan = {"workspace": int(head[4]), "cus": int(head[6]), "xcds": int(head[9]), "steps": [], "text": text}
+    for line in lines[1:]:
+        body = line.split(": ", 1)[1]
+        what, rest = body.split(" ", 1)
+        step = {"what": what}
+        if what == "kernel":
+            name, _, rest = rest.partition(" ")
+            step["name"] = name
+            step["family"] = name.split("<")[0]
+        for tok in rest.split():
+            if "=" in tok:
+                k, v = tok.split("=", 1)
+                try:
+                    step[k] = int(v)
+                except ValueError:
+                    step[k] = v
+        if "flags" in step:
+            step["flags"] = set() if step["flags"] in ("0", 0) else set(str(step["flags"]).split("|"))
+        plan["steps"].append(step)
+    return plan
+
+
 def time_gemm(mma, D, A, B, C_=None, alpha=1.0, stream=None, warmup=2, iters=10):
     """Average milliseconds per launch (HIP events on `stream`)."""
     ms = C.c_float()

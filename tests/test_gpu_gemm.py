@@ -31,6 +31,12 @@ def T(t, shape=None, stride=None):
     return tensor_of(t, shape, stride)
 
 
+def kernels_of(mh, mma, d, a, b, c=None, ep=None):
+    """The kernel steps of the plan the library makes for this call (moye_gemm_explain): what a test that means a
+    specific kernel instance asserts, so that a changed threshold cannot leave the instance untested while all stays green."""
+    return [s for s in mh.gemm_explain(mma, d, a, b, c, ep)["steps"] if s["what"] == "kernel"]
+
+
 def relerr(c, c64):
     c64 = c64.double()
     return float((c.double() - c64).abs().max() / c64.abs().max())
@@ -368,6 +374,9 @@ def test_hand_ordered_128_tile_exact_on_integers(mh):
             ref = A.double() @ B.double().t()
             for cta in ((0, 0, 0), (128, 128, bk)):
                 d = torch.zeros(M, N, dtype=torch.float32, device="cuda")
+                if cta != (0, 0, 0):
+                    ks = kernels_of(mh, mh.tiled_mma_desc(atom, atom_layout=(2, 2, 1), cta_tile=cta), T(d), T(a), T(b), T(c))
+                    assert len(ks) == 1 and ks[0]["family"] == "gemm_mfma_tn_256_w4" and "tile=128" in ks[0]["name"], ks
                 mh.gemm_(mh.tiled_mma_desc(atom, atom_layout=(2, 2, 1), cta_tile=cta), T(d), T(a), T(b), T(c), 2.0)
                 torch.cuda.synchronize()
                 assert torch.equal(d.cpu().double(), 2.0 * ref + C.double()), (in_dt, M, N, K, cta)
@@ -629,6 +638,8 @@ def test_short_m_line_staging_kernel(mh, M):
         ref = A.double() @ B.double().t()
         big = torch.full((M + 2, N + 3), 77.0, device="cuda")
         d = big[1:M + 1, 2:N + 2]
+        ks = kernels_of(mh, mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(0, 0, 0)), T(d), T(a), T(b), T(c))
+        assert len(ks) == 1 and ks[0]["family"] == "gemm_mfma_skinny_lds" and "mt=%d," % ((M + 15) // 16) in ks[0]["name"], ks
         mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(0, 0, 0)), T(d), T(a), T(b), T(c), 2.0)
         torch.cuda.synchronize()
         assert torch.equal(d.cpu().double(), 2.0 * ref + C.double()), (M, N, K)
@@ -718,7 +729,15 @@ def test_last_round_on_its_own_launch_exact_on_integers(mh, case):
         a, b = A.to(in_dt).cuda(), B.to(in_dt).cuda()
         big = torch.full((M + 2, N + 16), 7.0, dtype=out_dt, device="cuda")
         d = big[1:M + 1, 8:8 + N]
-        mh.gemm_(mh.tiled_mma_desc(atom, cta_tile=(0, 0, 0), split_k=-1), T(d), T(a), T(b), T(Cm.to(out_dt).cuda()) if with_c else None, 0.5)
+        mma = mh.tiled_mma_desc(atom, cta_tile=(0, 0, 0), split_k=-1)
+        cm = T(Cm.to(out_dt).cuda()) if with_c else None
+        ks = kernels_of(mh, mma, T(d), T(a), T(b), cm)
+        if in_dt in (torch.float16, torch.bfloat16) and case == (4608, 4608, 2048):
+            # 324 tiles of 256 x 256: the first eleven tile rows on them, the rest as a problem of its own on 128 x 128 tiles
+            assert [k["tile"] for k in ks] == ["256x256x128B", "128x128x128B"] and ks[0]["M"] + ks[1]["M"] == M, ks
+        if in_dt in (torch.float16, torch.bfloat16) and case == (5120, 5120, 1024):
+            assert len(ks) == 1 and ks[0]["tile"] == "256x256x128B", ks      # 400 tiles: the model sees nothing to gain
+        mh.gemm_(mma, T(d), T(a), T(b), cm, 0.5)
         torch.cuda.synchronize()
         assert torch.equal(d.cpu().double(), ref), (in_dt, out_dt)
         frame = big.clone()
@@ -740,7 +759,7 @@ def test_last_round_on_its_own_launch_keeps_the_epilogue_operand_in_step(mh, sha
 @pytest.mark.parametrize("case", [(4000, 2200, 328), (3900, 2304, 120), (4096, 2048, 72), (4090, 2203, 40), (2100, 4100, 200),
                                   (4099, 2050, 4096 + 8), (4096, 2048, 128), (1000, 600, 136), (384, 256, 128), (130, 2000, 72),
                                   (4000, 2200, 192), (3841, 2305, 4096), (4100, 2052, 4096),
-                                  (3000, 2000, 192), (2100, 2900, 4096)])
+                                  (3000, 2000, 192), (2100, 2900, 4096), (4000, 4000, 4096), (5000, 3000, 4096)])
 def test_ragged_256_tiles_exact_on_integers(mh, case):
     """Problems the library puts on 256x256 tiles (the larger cases) or 128x128 tiles that reach beyond M, N and K: rows beyond the operands are read from
     the last row and never stored, the K tail (1 to 7 pieces of 16 bytes, also with less than one k-tile in all) is
@@ -772,6 +791,24 @@ def test_ragged_256_tiles_exact_on_integers(mh, case):
         frame[1:M + 1, 8:8 + N] = 77.0
         assert bool((frame == 77.0).all()), "stores outside D"
         d.zero_()
+        ks = kernels_of(mh, mh.tiled_mma_desc(atom, cta_tile=(0, 0, 0)), T(d), T(a), T(b))
+        kc = kernels_of(mh, mh.tiled_mma_desc(atom, cta_tile=(0, 0, 0)), T(d), T(a), T(b), T(c))
+        b16 = in_dt in (torch.float16, torch.bfloat16)
+        if case == (3841, 2305, 4096) and b16:
+            # one row and one column beyond whole tiles: the interior on whole 256 x 256 tiles, each fringe on the short-M kernel
+            assert [k["family"] for k in ks] == ["gemm_mfma_tn_256_w4", "gemm_mfma_skinny_lds", "gemm_mfma_skinny_lds"] and "ragged=0" in ks[0]["name"], ks
+        if case in ((4000, 4000, 4096), (5000, 3000, 4096)):
+            # at least 128 ragged 256 x 256 tiles, K of whole 128-byte rows: without C the guarded form of the hand-ordered
+            # kernel, with C that of the compiler-scheduled one (fp8: the hand-ordered kernel has its only guarded form)
+            assert ks[0]["family"] == "gemm_mfma_tn_256_w4" and "ragged=1" in ks[0]["name"] and "tile=256" in ks[0]["name"], ks
+            if in_dt != torch.float8_e4m3fn:
+                assert kc[0]["family"] == "gemm_mfma_tn_256" and "ragged=1" in kc[0]["name"], kc
+        if case == (2100, 2900, 4096):     # fewer than 128 tiles of 256 x 256: the hand-ordered kernel's guarded 128 x 128 instance
+            assert ks[0]["family"] == "gemm_mfma_tn_256_w4" and "ragged=1" in ks[0]["name"] and "tile=128" in ks[0]["name"], ks
+        if case == (4099, 2050, 4096 + 8) and b16:     # a K tail on 256 x 256 tiles: the compiler-scheduled kernel's guarded instance masks it
+            assert ks[0]["family"] == "gemm_mfma_tn_256" and "ragged" in ks[0]["flags"], ks
+        if case == (1000, 600, 136):     # too few tiles for 256 x 256: the 128 x 128 kernel's guarded instance
+            assert ks[0]["tile"].startswith("128x128") and "ragged" in ks[0]["flags"], ks
         mh.gemm_(mh.tiled_mma_desc(atom, cta_tile=(0, 0, 0)), T(d), T(a), T(b))
         torch.cuda.synchronize()
         assert torch.equal(d.cpu().double(), ref), (case, in_dt, out_dt, "no C")
@@ -808,6 +845,7 @@ def test_random_shapes_exact_on_integers(mh):
     shapes = {(rnd.choice(pools[0]), rnd.choice(pools[1]), rnd.choice(pools[2])) for _ in range(40)}
     shapes |= {(rnd.choice(pools[1]), rnd.choice(pools[1]), rnd.choice(pools[2][:8])) for _ in range(24)}
     g = torch.Generator().manual_seed(5)
+    seen = set()
     for (M, N, K) in sorted(shapes):
         if M * N * K > 4096 * 4096 * 300:
             K = 72
@@ -820,6 +858,8 @@ def test_random_shapes_exact_on_integers(mh):
             continue
         for split in (0, -1):
             d = torch.full((M, N), 9.0, dtype=torch.float16, device="cuda")
+            for k in kernels_of(mh, mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(0, 0, 0), split_k=split), T(d), T(a), T(b), T(c)):
+                seen.add((k["family"], k["tile"].rsplit("x", 1)[0], "ragged" in k["flags"], k["split"] > 1))
             mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(0, 0, 0), split_k=split), T(d), T(a), T(b), T(c), 2.0)
             torch.cuda.synchronize()
             assert torch.equal(d.cpu().double(), 2.0 * ref + C.double()), (M, N, K, "split_k", split)
@@ -827,6 +867,11 @@ def test_random_shapes_exact_on_integers(mh):
         mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, cta_tile=(0, 0, 0)), T(dt_, (M, N), (1, M)), T(a), T(b))
         torch.cuda.synchronize()
         assert torch.equal(dt_.t().cpu().double(), ref), (M, N, K, "column-major D")
+    # the seeded shapes do reach the kernels the docstring names
+    fams = {f for f, _, _, _ in seen}
+    # (short K keeps these shapes off 256 x 256 tiles; test_ragged_256_tiles_* and test_last_round_* cover those)
+    assert {"gemm_mfma_skinny", "gemm_mfma_skinny_lds", "gemm_mfma_tn", "gemm_mfma_tn_128"} <= fams, sorted(fams)
+    assert any(t == "64x64" for _, t, _, _ in seen) and any(r for _, _, r, _ in seen) and any(sp for _, _, _, sp in seen), sorted(seen)
 
 
 def test_one_row_operands_with_any_stride_on_the_unit_mode(mh):
@@ -1533,6 +1578,8 @@ def test_bench_descriptor_every_cta_exact_on_integers(mh, out_dt):
     B = torch.randint(-2, 3, (N, K), generator=g).half()
     a, b = A.cuda(), B.cuda()
     d = torch.full((M, N), float("nan"), dtype=out_dt, device="cuda")
+    ks = kernels_of(mh, _bench_mma(mh), T(d), T(a), T(b))
+    assert len(ks) == 1 and ks[0]["name"].startswith("gemm_mfma_tn_256_w4<W4F16L,") and ks[0]["grid"] == "256x1", ks
     mh.gemm_(_bench_mma(mh), T(d), T(a), T(b))
     torch.cuda.synchronize()
     want = (a.float() @ b.float().t())           # exact: |sum| <= 4 * 512 = 2048, an integer fp16 holds

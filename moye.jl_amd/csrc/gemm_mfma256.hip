@@ -135,7 +135,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tn_256_ring(GemmArgs
 
     // --- epilogue (mfma_epilogue.hpp): alpha*acc + C -> OutT -> this wave's LDS patch -> 128-bit row stores
     static_assert(NWAVES * 32 * WN * 4 <= STAGES * STAGE * 16, "C patches (32 rows per wave and pass) fit in the operand ring");
-    store_c_tile<Out, MI, NI, false>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
+    store_c_tile<Out, MI, NI>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
 }
 
 template <typename In, typename Out, int STAGES>

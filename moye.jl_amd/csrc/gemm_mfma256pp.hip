@@ -149,7 +149,7 @@ __global__ __launch_bounds__(512) void gemm_mfma_tn_256_pp(GemmArgs p) {
 #undef MOYE_MMA
     __syncthreads();  // every wave is done with the operand stages before they become C patches
 
-    store_c_tile<Out, MI, NI, false>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
+    store_c_tile<Out, MI, NI>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
 }
 
 template <typename In, typename Out>

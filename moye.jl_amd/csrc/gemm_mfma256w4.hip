@@ -575,7 +575,7 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
         for (int j = 0; j < NI; ++j) asm volatile("" : "+a"(acc[i][j]));
     __syncthreads();  // every wave is done with the operand ring before it becomes C patches
 
-    store_c_tile<Out, MI, NI, false, kRagged, kBias, kBias || kRagged>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
+    store_c_tile<Out, MI, NI, kRagged, kBias, kBias || kRagged>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
 }
 
 template <typename In, typename Out, int WGN, bool kBias = false, bool kRagged = false, int TILE = 256, int AMAJ = 0, int BMAJ = 0>

@@ -302,9 +302,9 @@ __device__ __forceinline__ void gemm_mfma_tn_lds_tile(GemmArgs p) {
     static_assert(NWAVES * 32 * WN * 4 <= 2 * STAGE * 16, "C patches (32 rows per wave and pass) fit in the operand stages");
     // (a kOps instance is only launched for calls with an operation or with ragged tiles: it carries the general
     // epilogue alone, which keeps the other one's registers out of its allocation)
-    if constexpr (kBias) store_c_tile<Out, MI, NI, false, false, true>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
+    if constexpr (kBias) store_c_tile<Out, MI, NI, false, true>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
     else if constexpr (kOps) store_c_tile_general<Out, MI, NI, kRagged>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
-    else store_c_tile<Out, MI, NI, false, kRagged>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
+    else store_c_tile<Out, MI, NI, kRagged>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
 }
 
 }  // namespace moye

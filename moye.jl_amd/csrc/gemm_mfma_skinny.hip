@@ -1,15 +1,11 @@
 // MFMA GEMM for a short A: at most 64 rows against a long B (N x K), K-major operands.
-// The work is streaming B from HBM once, so both kernels here are laid out for bandwidth, not for the matrix pipe: one
-// workgroup owns 16 or 32 rows of B (that many output columns) and all of A; its waves split K into contiguous ranges,
-// and the per-wave partial accumulators are summed through LDS in wave order, which makes the result independent of
-// timing.  A (at most 64 x K) is re-read by every workgroup and lives in L2.
-//   gemm_mfma_skinny_lds  K a multiple of 128 bytes: whole 128-byte lines of both operands go through LDS (load-to-LDS
-//                         instructions), four waves per workgroup; bf16 16 x 8192 x 8192: 21.0 us
-//   gemm_mfma_skinny      any K of whole 64-byte steps: each lane loads 16-byte pieces of its B row straight into the
-//                         MFMA operand registers, eight waves; the same problem: 32.4 us.  With 32 rows of B per
-//                         workgroup each A fragment feeds two MFMAs (33 us against 38).  More requests in flight make
-//                         it slower, not faster (waves per workgroup x k-steps in flight per wave: 8 x 4 32.4 us,
-//                         4 x 8 34.3, 8 x 8 38.8, 16 x 2 39.9, 16 x 4 41.5, 8 x 16 55.1).
+// The work is streaming B from HBM once, so the kernel is laid out for bandwidth, not for the matrix pipe: one workgroup
+// owns 16 or 32 rows of B (that many output columns) and all of A; its four waves split K into contiguous ranges of
+// whole 128-byte lines, both operands go through LDS by load-to-LDS instructions that read whole lines, and the per-wave
+// partial accumulators are summed through LDS in wave order, which makes the result independent of timing.  A (at most
+// 64 x K) is re-read by every workgroup and lives in L2.  bf16 16 x 8192 x 8192: 21.0 us (0.80 of the HBM peak); a
+// kernel whose lanes loaded their 16-byte pieces of B straight into MFMA operand registers took 32.4 us and is gone.
+// K need only be a whole number of 16-byte pieces: what is left after the last whole line is a masked trip of its own.
 //
 // Stands where the reference's user kernel would run gemm! (src/algorithm/blas.jl:11-131) on a
 // 16-row problem with its usual 128 x 128 tiles and waste 7/8 of each tile.
@@ -17,103 +13,11 @@
 
 namespace moye {
 
-template <typename In, typename Out, int MT, int NTW, int WAVES, int U = 4 /* 64-byte k-steps in flight per wave and row */>
-__global__ __launch_bounds__(WAVES * 64) void gemm_mfma_skinny(GemmArgs p) {
-    typedef typename Out::type OutT;
-    split_of_block(p);
-    __shared__ f32x4 part[WAVES][MT * NTW][64];
-    const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, r16 = lane % 16, kq = lane / 16;
-    const int n0 = blockIdx.x * 16 * NTW;
-    const int steps = (int)(((int64_t)p.K * In::kBytes) / 64);
-    const int s0 = (int)((int64_t)steps * wave / WAVES), s1 = (int)((int64_t)steps * (wave + 1) / WAVES);
-    // M and N need not be multiples of 16: a lane whose row lies beyond the operand reads the last row instead, and
-    // what it computes is not stored
-    const char* bp[NTW];
-#pragma unroll
-    for (int t = 0; t < NTW; ++t)
-        bp[t] = static_cast<const char*>(p.B) + (int64_t)min(n0 + 16 * t + r16, p.N - 1) * p.ldb * In::kBytes + kq * 16;
-    const char* ap[MT];
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-        ap[i] = static_cast<const char*>(p.A) + (int64_t)min(16 * i + r16, p.M - 1) * p.lda * In::kBytes + kq * 16;
-    f32x4 acc[MT][NTW];
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-        for (int t = 0; t < NTW; ++t) acc[i][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-    // Every workgroup needs all of A, and workgroups that walk K in the same order ask the L2 for the same lines of A
-    // at the same moment, before any of them has them.  So a workgroup starts its walk at a step that depends on
-    // its position within its L2's share of the grid (consecutive workgroups go to consecutive L2s), in units of U
-    // steps so that a trip still covers whole 128-byte lines of B (measured at 16 x 8192 x 8192 bf16: 146 MiB
-    // fetched instead of 161, 32.9 us instead of 34.0).  The order of a column's k-sum follows the workgroup, not
-    // the time, so results stay reproducible.
-    const int len = s1 - s0;
-    const int first = len >= U && len % U == 0 ? U * (int)((blockIdx.x / (unsigned)p.xcds) % (unsigned)(len / U)) : 0;
-    auto step_of = [&](int t) { const int r = t + first; return s0 + (r >= len ? r - len : r); };
-    int t0 = 0;
-    for (; t0 + U <= len; t0 += U) {
-        u32x4 b[NTW][U], a[MT][U];
-        int64_t off[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) off[u] = (int64_t)step_of(t0 + u) * 64;
-#pragma unroll
-        for (int t = 0; t < NTW; ++t)
-#pragma unroll
-            for (int u = 0; u < U; ++u)
-                b[t][u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(bp[t] + off[u]));
-#pragma unroll
-        for (int i = 0; i < MT; ++i)
-#pragma unroll
-            for (int u = 0; u < U; ++u) a[i][u] = *reinterpret_cast<const u32x4*>(ap[i] + off[u]);
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-#pragma unroll
-            for (int i = 0; i < MT; ++i)
-#pragma unroll
-                for (int t = 0; t < NTW; ++t) In::mma(b[t][u], a[i][u], acc[i][t]);
-    }
-    for (; t0 < len; ++t0) {
-        const int64_t off = (int64_t)step_of(t0) * 64;
-#pragma unroll
-        for (int i = 0; i < MT; ++i) {
-            const u32x4 a = *reinterpret_cast<const u32x4*>(ap[i] + off);
-#pragma unroll
-            for (int t = 0; t < NTW; ++t)
-                In::mma(__builtin_nontemporal_load(reinterpret_cast<const u32x4*>(bp[t] + off)), a, acc[i][t]);
-        }
-    }
-
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-        for (int t = 0; t < NTW; ++t) part[wave][i * NTW + t][lane] = acc[i][t];
-    __syncthreads();
-    // lane l of tile (i, t) holds C[m = 16 i + l % 16][n = n0 + 16 t + 4 (l / 16) + 0..3]
-    for (int unit = threadIdx.x; unit < MT * NTW * 64; unit += WAVES * 64) {
-        const int it = unit / 64, l = unit % 64;
-        f32x4 v = part[0][it][l];
-#pragma unroll
-        for (int w = 1; w < WAVES; ++w) v += part[w][it][l];
-        const int m = 16 * (it / NTW) + l % 16, n = n0 + 16 * (it % NTW) + 4 * (l / 16);
-        if (m >= p.M) continue;
-        const int64_t sn = p.ldd_n ? p.ldd_n : 1;  // D may have its unit stride along m (a column-major D, or the
-                                                   // right-hand fringe of a large problem computed as its transpose)
-        OutT* d = static_cast<OutT*>(p.D) + (int64_t)m * p.ldd + (int64_t)n * sn;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            if (n + e >= p.N) continue;
-            const float c = p.C ? Out::load(p.C, (int64_t)m * p.ldc_m + (int64_t)(n + e) * p.ldc_n) : 0.f;
-            d[e * sn] = Out::cvt(epi_value(p, v[e], p.C != nullptr, c, m, n + e));
-        }
-    }
-}
-
-// The same decomposition for at most 16 rows of A, with both operands staged through LDS by load-to-LDS instructions.
+// Both operands are staged through LDS by load-to-LDS instructions.
 // A lane that loads straight into MFMA operand registers must address row lane % 16: neighbouring lanes then ask for
 // 16 bytes each of sixteen different cache lines, and the address path of the CU handles such an instruction several
-// times slower than one whose lanes read consecutive addresses (measured on the kernel above with the lanes renumbered,
-// results wrong on purpose, same bytes: 32.4 us as it is, 30.2 with four lanes per 64 bytes, 29.0 with eight lanes per
+// times slower than one whose lanes read consecutive addresses (measured on such a kernel with the lanes renumbered,
+// results wrong on purpose, same bytes: 32.4 us as it was, 30.2 with four lanes per 64 bytes, 29.0 with eight lanes per
 // 128-byte line).  Here every instruction reads eight whole 128-byte lines (eight rows of one operand, lane l the piece
 // (l % 8) ^ (l / 8) of row l / 8), the pieces land in LDS in lane order, which is the XOR-swizzled row layout that
 // ds_read_b128 reads back without bank conflicts, and no operand in flight holds a register.  Each wave streams its own
@@ -134,8 +38,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_skinny_lds(GemmArgs p) {
     const int n0 = blockIdx.x * 16 * NTW;
     u32x4* const ring = smem + __builtin_amdgcn_readfirstlane(wave * kStages * STAGE);
 
-    // the waves' K ranges: whole 128-byte lines, as even as they come (a wave may get none of a very short K)
+    // the waves' K ranges: whole 128-byte lines, as even as they come (a wave may get none of a very short K); what is
+    // left of K after the last whole line (1 to 7 pieces of 16 bytes) is one more trip of the last wave
     const int lines = (int)(((int64_t)p.K * In::kBytes) / 128);
+    const int tail_pieces = (int)((((int64_t)p.K * In::kBytes) % 128) / 16);
     const int s0 = (int)((int64_t)lines * wave / WAVES), len = (int)((int64_t)lines * (wave + 1) / WAVES) - s0;
     // M and N need not be multiples of 16: a row beyond the operand is read from the last row instead, and what is
     // computed from it is not stored
@@ -202,6 +108,33 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_skinny_lds(GemmArgs p) {
                 for (int j = 0; j < NTW; ++j) In::mma(b[ks][j], a[ks][i], acc[i][j]);
         asm volatile("" ::: "memory");
     }
+    // The K tail (the intent of copyto_if!, src/algorithm/copy.jl:4-16, for the last line): a lane whose 16-byte piece lies
+    // beyond K reads its row's first piece instead (nothing is read past a row's end), and every fragment piece beyond K
+    // is zeroed in registers, of both operands (the bytes there may be NaN or Inf), before it reaches an MFMA.
+    if (tail_pieces > 0 && wave == WAVES - 1) {
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the last trip's fragment reads are out of the buffer
+        const int64_t off_ = (int64_t)lines * 128 + (lch < tail_pieces ? 0 : -lch * 16);
+#pragma unroll
+        for (int j = 0; j < 2 * NTW; ++j) __builtin_amdgcn_global_load_lds((gptr_t)(src[j] + off_), (lptr_t)(ring + 64 * j), 16, 0, kAuxB);
+#pragma unroll
+        for (int j = 2 * NTW; j < LD; ++j) __builtin_amdgcn_global_load_lds((gptr_t)(src[j] + off_), (lptr_t)(ring + 64 * j), 16, 0, 0);
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            const bool beyond = 4 * ks + kq >= tail_pieces;
+            u32x4 b[NTW], a[MT];
+#pragma unroll
+            for (int j = 0; j < NTW; ++j) b[j] = beyond ? u32x4{0u, 0u, 0u, 0u} : ring[16 * 8 * j + slot[ks]];
+#pragma unroll
+            for (int i = 0; i < MT; ++i) a[i] = beyond ? u32x4{0u, 0u, 0u, 0u} : ring[16 * 8 * (NTW + i) + slot[ks]];
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int j = 0; j < NTW; ++j) In::mma(b[j], a[i], acc[i][j]);
+        }
+        asm volatile("" ::: "memory");
+    }
 #undef MOYE_STAGE_LOAD
 
     __syncthreads();  // every wave is done with its ring before the partial sums go there
@@ -232,13 +165,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_skinny_lds(GemmArgs p) {
 
 constexpr int kSkinnyLdsWaves = 4;
 static_assert(kSkinnyLineBytes == 128, "the host decides about K ranges by this");
-
-// K a whole number of 128-byte lines
-template <typename In>
-static bool skinny_lds_takes(const GemmArgs& a) {
-    return a.K > 0 && ((int64_t)a.K * In::kBytes) % kSkinnyLineBytes == 0;
-}
-
 template <typename In, typename Out, int MT, int W, int NTW, int S, int AUX>
 static int32_t launch_skinny_lds_v(const GemmArgs& a, GemmPlan& plan) {
     constexpr int kLds = W * S * (16 * NTW + 16 * MT) * 128;
@@ -246,13 +172,6 @@ static int32_t launch_skinny_lds_v(const GemmArgs& a, GemmPlan& plan) {
     plan.add_kernel(gemm_mfma_skinny_lds<In, Out, MT, NTW, W, S, AUX>, a, (unsigned)((a.N + 16 * NTW - 1) / (16 * NTW)), (unsigned)(a.split > 1 ? a.split : 1),
                     W * 64, kLds, &cap, 0, 16 * NTW, 128, In::kDt, Out::kDt, "gemm_mfma_skinny_lds<%s,%s,mt=%d,ntw=%d,waves=%d,stages=%d>", In::kName, Out::kName,
                     MT, NTW, W, S);
-    return MOYE_OK;
-}
-// the kernel whose lanes stream their own 16-byte pieces of B into registers: MT x 16 rows of A, NTW x 16 rows of B per wave
-template <typename In, typename Out, int MT, int NTW, int W>
-static int32_t launch_skinny_regs(const GemmArgs& a, unsigned grid_x, GemmPlan& plan) {
-    plan.add_kernel(gemm_mfma_skinny<In, Out, MT, NTW, W>, a, grid_x, (unsigned)(a.split > 1 ? a.split : 1), W * 64, 0, nullptr, 0, 16 * NTW, 64, In::kDt, Out::kDt,
-                    "gemm_mfma_skinny<%s,%s,mt=%d,ntw=%d,waves=%d>", In::kName, Out::kName, MT, NTW, W);
     return MOYE_OK;
 }
 template <typename In, typename Out>
@@ -280,52 +199,22 @@ static int32_t launch_skinny_lds(const GemmArgs& a, GemmPlan& plan) {
     }
 }
 
-template <typename In, typename Out>
-static int32_t launch_skinny(const GemmArgs& a, GemmPlan& plan) {
-    constexpr int W = 8;
-    if (skinny_lds_takes<In>(a)) return launch_skinny_lds<In, Out>(a, plan);
-    // With K split over two or more workgroups there are enough workgroups to give each one 64 rows of B: A, which every
-    // workgroup reads whole (its K range of it), then crosses the L2-to-CU path half as often.  Pays from M = 33 on
-    // (bf16 64 x 8192 x 8192: 44.8 us with two K ranges, the second pass included, against 52.5 unsplit; M = 48: 41.3
-    // against 55.3); without the split the larger workgroup tile is slower (68.8 us).
-    if (a.split > 1 && a.M > 32 && a.N % 64 == 0 && a.N / 64 >= plan.shape.cus / 2) {
-        if ((a.M + 15) / 16 == 3) return launch_skinny_regs<In, Out, 3, 4, W>(a, (unsigned)(a.N / 64), plan);
-        return launch_skinny_regs<In, Out, 4, 4, W>(a, (unsigned)(a.N / 64), plan);
-    }
-    if (a.N % 32 == 0 && a.N / 32 >= plan.shape.cus) {  // two B tiles per wave once that still fills the chip
-        const unsigned gx = (unsigned)(a.N / 32);
-        switch ((a.M + 15) / 16) {
-            case 1: return launch_skinny_regs<In, Out, 1, 2, W>(a, gx, plan);
-            case 2: return launch_skinny_regs<In, Out, 2, 2, W>(a, gx, plan);
-            case 3: return launch_skinny_regs<In, Out, 3, 2, W>(a, gx, plan);
-            default: return launch_skinny_regs<In, Out, 4, 2, W>(a, gx, plan);
-        }
-    }
-    const unsigned gx = (unsigned)((a.N + 15) / 16);
-    switch ((a.M + 15) / 16) {
-        case 1: return launch_skinny_regs<In, Out, 1, 1, W>(a, gx, plan);
-        case 2: return launch_skinny_regs<In, Out, 2, 1, W>(a, gx, plan);
-        case 3: return launch_skinny_regs<In, Out, 3, 1, W>(a, gx, plan);
-        default: return launch_skinny_regs<In, Out, 4, 1, W>(a, gx, plan);
-    }
-}
-
 template <typename In>
 static int32_t launch_skinny_out(int32_t out_dt, const GemmArgs& a, GemmPlan& plan) {
     switch (out_dt) {
-        case MOYE_F32: return launch_skinny<In, OutF32>(a, plan);
-        case MOYE_F16: return launch_skinny<In, OutF16>(a, plan);
-        case MOYE_BF16: return launch_skinny<In, OutBF16>(a, plan);
+        case MOYE_F32: return launch_skinny_lds<In, OutF32>(a, plan);
+        case MOYE_F16: return launch_skinny_lds<In, OutF16>(a, plan);
+        case MOYE_BF16: return launch_skinny_lds<In, OutBF16>(a, plan);
         default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: MFMA kernels write f32, f16 or bf16, not %s", dtype_name(out_dt));
     }
 }
 
-// 1 <= M <= 64, any N, K a multiple of 64 bytes; pointers and pitches 16-byte aligned.
+// 1 <= M <= 64, any N, K a multiple of 16 bytes; pointers and pitches 16-byte aligned.
 int32_t gemm_mfma_skinny_dispatch(int32_t in_dt, int32_t out_dt, const GemmArgs& a, GemmPlan& plan) {
     const int eb = dtype_bytes(in_dt);
-    if (a.M < 1 || a.M > 64 || a.N < 1 || ((int64_t)a.K * eb) % 64)
+    if (a.M < 1 || a.M > 64 || a.N < 1 || a.K < 1 || ((int64_t)a.K * eb) % 16)
         return fail(MOYE_ERR_SHAPE, "gemm!: the short-M MFMA kernel needs 1 <= M <= 64 and K %% %d == 0, got %dx%dx%d",
-                    64 / eb, a.M, a.N, a.K);
+                    16 / eb, a.M, a.N, a.K);
     if ((a.lda * eb) % 16 || (a.ldb * eb) % 16 ||
         (reinterpret_cast<uintptr_t>(a.A) | reinterpret_cast<uintptr_t>(a.B)) % 16)
         return fail(MOYE_ERR_ALIGN, "gemm!: operands of the MFMA kernels need 16-byte aligned pointers and row pitches");

@@ -147,8 +147,8 @@ __device__ __forceinline__ void store_c_tile_general(const GemmArgs& p, const f3
 
 // acc[i][j] of a lane holds C[m = 16 i + lane % 16][n = 16 j + 4 (lane / 16) + e], e = 0..3,
 // relative to (m_base, n_base).  `smem` must be free of operand data for all waves.
-// kWithOps = false leaves the element-wise operations out (the hand-ordered kernel: its register allocation around the
-// inline-assembly MFMAs must not change with what the epilogue needs; the host never sends it such a call).
+// No element-wise operation here: a call with one runs an instance whose epilogue is store_c_tile_general alone (the host
+// decides; the hand-ordered kernel has no such instance and is never sent one).
 // kGuard: the tile may reach beyond M or N and D need not be 16-byte aligned: nothing is read or stored beyond them, a
 // piece of D that crosses N or does not start on a 16-byte boundary goes out element by element.
 // kAddVec: the call adds a vector or a scalar (GemmArgs::ep_op == MOYE_MAP_ADD with a one-per-column, one-per-row or
@@ -156,16 +156,10 @@ __device__ __forceinline__ void store_c_tile_general(const GemmArgs& p, const f3
 // epilogue, instead of sending the tile through it.
 // kNoC: the caller has no C (GemmArgs::C is null, checked on the host): nothing of C's two read paths is compiled in,
 // which frees their registers for instances that have few to spare.
-template <typename Out, int MI, int NI, bool kWithOps = true, bool kGuard = false, bool kAddVec = false, bool kNoC = false>
+template <typename Out, int MI, int NI, bool kGuard = false, bool kAddVec = false, bool kNoC = false>
 __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&acc)[MI][NI], u32x4* smem, int wave,
                                              int lane, int64_t m_base, int64_t n_base) {
     typedef typename Out::type OutT;
-    if constexpr (kWithOps) {
-        if (p.ep_op != MOYE_MAP_IDENTITY) {
-            store_c_tile_general<Out, MI, NI>(p, acc, smem, wave, lane, m_base, n_base);
-            return;
-        }
-    }
     constexpr int WN = NI * 16;
     constexpr int EPC = 16 / (int)sizeof(OutT);  // elements per 16-byte chunk
     constexpr int CR = WN / EPC;                 // chunks per patch row

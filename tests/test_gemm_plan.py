@@ -93,10 +93,10 @@ def check_kernel_step(s, eb, ob):
             assert kb % 16 == 0, s
         else:
             assert M % tm == 0 and N % tn == 0 and kb % bkb == 0 and s["d16"] == 1 and (s["ldd"] * ob) % 16 == 0, s
-    elif fam in ("gemm_mfma_skinny_lds", "gemm_mfma_skinny"):
+    elif fam == "gemm_mfma_skinny_lds":
         assert 1 <= M <= 64 and s["a16"] == 1 and s["b16"] == 1, s
         assert (s["lda"] * eb) % 16 == 0 and (s["ldb"] * eb) % 16 == 0, s
-        assert kb % (128 if fam == "gemm_mfma_skinny_lds" else 64) == 0, s
+        assert kb % 16 == 0, s                          # whole 128-byte lines plus a masked tail of 16-byte pieces
         mt = int(name.split("mt=")[1].split(",")[0])
         assert 16 * mt >= M, s
     else:
@@ -265,9 +265,9 @@ def test_known_shapes_run_on_the_instances_they_are_meant_for():
     # ... and a K-major copy where no kernel reads the operand as it lies (a short problem on 128 x 128 tiles, fp8)
     p = run_case(f8, f32, 256, 512, 256, a_major="m", b_major="n")
     assert [s["what"] for s in p["steps"]][:2] == ["kmajor_copy", "kmajor_copy"] and p["workspace"] >= 256 * 256 + 512 * 256
-    # short M: whole 128-byte lines of K through LDS; a K tail keeps the kernel that streams into registers
+    # short M: whole 128-byte lines of K through LDS, a K tail as a masked trip of the same kernel
     assert step_names(run_case(bf16, f32, 16, 8192, 8192))[0].startswith("gemm_mfma_skinny_lds<InBF16,OutF32,mt=1,ntw=2,waves=4,stages=3>")
-    assert step_names(run_case(bf16, f32, 16, 8192, 8224))[0].startswith("gemm_mfma_skinny<InBF16,OutF32,mt=1,")
+    assert step_names(run_case(bf16, f32, 16, 8192, 8224))[0].startswith("gemm_mfma_skinny_lds<InBF16,OutF32,mt=1,ntw=2,")   # a K tail too
     # small N and a long K: the library's own K ranges for the line kernel, then the reduction
     p = run_case(bf16, f32, 16, 1024, 32768, split_k=-1)
     assert p["steps"][0]["family"] == "gemm_mfma_skinny_lds" and p["steps"][0]["split"] == 4 and p["steps"][-1]["what"] == "splitk_reduce"
@@ -309,7 +309,7 @@ def test_every_branch_of_the_dispatcher_is_reached():
     if len(SEEN) < 10:
         pytest.skip("the enumerating tests did not run in this process")
     want = {"gemm_mfma_tn_256_w4", "gemm_mfma_tn_256", "gemm_mfma_tn_128", "gemm_mfma_tn", "gemm_mfma_tn_256_ring", "gemm_mfma_tn_256_pp",
-            "gemm_mfma_skinny_lds", "gemm_mfma_skinny", "kmajor_copy", "splitk_reduce",
+            "gemm_mfma_skinny_lds", "kmajor_copy", "splitk_reduce",
             "gemm_mfma_tn_256_w4:ragged=1", "gemm_mfma_tn_256_w4:bias=1", "gemm_mfma_tn_256_w4:amaj=1", "gemm_mfma_tn_256_w4:bmaj=1",
             "gemm_mfma_tn_256_w4:tile=128", "gemm_mfma_tn_256:ragged=1", "gemm_mfma_tn_256:ops=1", "gemm_mfma_tn_256:bias=1",
             "gemm_mfma_tn_256:amaj=1", "gemm_mfma_tn_128:ragged=1", "gemm_mfma_tn_128:ops=1", "gemm_mfma_tn_128:amaj=1", "gemm_mfma_tn_128:bias=1",

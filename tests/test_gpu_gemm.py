@@ -580,6 +580,37 @@ def test_short_m_exact_on_integers(mh, M):
             assert torch.equal(d.cpu().double(), 2.0 * ref + C.double()), (M, N, K, "split_k", split)
 
 
+@pytest.mark.parametrize("tdt,atom,K", [("float16", "MFMA_F32_16x16x32_F16", 8216), ("bfloat16", "MFMA_F32_16x16x32_BF16", 136),
+                                        ("float32", "MFMA_F32_16x16x4_F32", 4100), ("float8_e4m3fn", "MFMA_F32_16x16x32_FP8", 8304)])
+def test_short_m_k_tail_inside_nan_frames(mh, tdt, atom, K):
+    """A K that ends inside a 128-byte line: the short-M kernel masks the pieces beyond K in registers.  The operands
+    are windows of arrays whose other bytes are NaN (Inf), so a piece read past K and not masked shows; every type;
+    also as the K ranges of a split (whole lines, the tail in the last)."""
+    if not hasattr(torch, tdt):
+        pytest.skip("no " + tdt)
+    tdt, atom = getattr(torch, tdt), getattr(mh, atom)
+    g = torch.Generator().manual_seed(K)
+    for (M, N) in ((16, 8192), (5, 100), (64, 8200)):
+        A = torch.randint(-3, 4, (M, K), generator=g).float()
+        B = torch.randint(-3, 4, (N, K), generator=g).float()
+        if K > 4000:
+            A[:, 100:K - 100] = 0
+        pad = 16 // torch.empty(0, dtype=tdt).element_size()
+        Ab = torch.full((M + 1, K + 3 * pad), float("nan"), dtype=torch.float32).to(tdt).cuda()
+        Bb = torch.full((N + 1, K + pad), float("nan") if tdt == torch.float8_e4m3fn else float("inf"), dtype=torch.float32).to(tdt).cuda()
+        Ab[:M, :K] = A.to(tdt).cuda()
+        Bb[:N, :K] = B.to(tdt).cuda()
+        ref = A.double() @ B.double().t()
+        for split in (0, -1):
+            d = torch.zeros(M, N, dtype=torch.float32, device="cuda")
+            mma = mh.tiled_mma_desc(atom, cta_tile=(0, 0, 0), split_k=split)
+            ks = kernels_of(mh, mma, T(d), T(Ab[:M, :K]), T(Bb[:N, :K]))
+            assert ks[0]["family"] == "gemm_mfma_skinny_lds", ks
+            mh.gemm_(mma, T(d), T(Ab[:M, :K]), T(Bb[:N, :K]))
+            torch.cuda.synchronize()
+            assert torch.equal(d.cpu().double(), ref), (tdt, M, N, K, split)
+
+
 @pytest.mark.parametrize("M", [1, 7, 20, 33, 63])
 def test_short_m_any_m_and_n(mh, M):
     """M and N that are not multiples of 16: lanes beyond the operands read the last row and store nothing.
@@ -630,7 +661,9 @@ def test_short_m_line_staging_kernel(mh, M):
     32 rows of B per workgroup), K ranges of none, one and many lines per wave, even and uneven, row- and column-major D inside a frame, C with alpha,
     every input type; exact on small integers, so a wrong piece, row or K range is a hard mismatch."""
     g = torch.Generator().manual_seed(300 + M)
-    for (N, K) in ((100, 256), (8191, 768), (8200, 2048), (12000, 256), (32, 4096), (8192, 320), (100, 64), (8200, 704)):
+    # (K of whole 128-byte lines, and K with a tail of one to seven 16-byte pieces: 8, 72, 200, 4152, 56)
+    for (N, K) in ((100, 256), (8191, 768), (8200, 2048), (12000, 256), (32, 4096), (8192, 320), (100, 64), (8200, 704), (100, 8), (8191, 72),
+                   (8200, 200), (300, 4152), (8192, 56)):
         A = torch.randint(-4, 5, (M, K), generator=g).to(torch.float16)
         B = torch.randint(-4, 5, (N, K), generator=g).to(torch.float16)
         C = torch.randint(-8, 9, (M, N), generator=g).to(torch.float32)
@@ -870,7 +903,7 @@ def test_random_shapes_exact_on_integers(mh):
     # the seeded shapes do reach the kernels the docstring names
     fams = {f for f, _, _, _ in seen}
     # (short K keeps these shapes off 256 x 256 tiles; test_ragged_256_tiles_* and test_last_round_* cover those)
-    assert {"gemm_mfma_skinny", "gemm_mfma_skinny_lds", "gemm_mfma_tn", "gemm_mfma_tn_128"} <= fams, sorted(fams)
+    assert {"gemm_mfma_skinny_lds", "gemm_mfma_tn", "gemm_mfma_tn_128"} <= fams, sorted(fams)
     assert any(t == "64x64" for _, t, _, _ in seen) and any(r for _, _, r, _ in seen) and any(sp for _, _, _, sp in seen), sorted(seen)
 
 

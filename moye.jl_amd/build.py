@@ -28,6 +28,8 @@ SOURCES = {
     "gemm_mfma256.hip": ["-ffp-contract=off"],
     "gemm_mfma256pp.hip": ["-ffp-contract=off"],
     "gemm_mfma256w4.hip": ["-ffp-contract=off"],
+    "gemm_mfma256w4_majors.hip": ["-ffp-contract=off"],
+    "gemm_mfma128w4.hip": ["-ffp-contract=off"],
     "gemm_mfma_skinny.hip": ["-ffp-contract=off"],
     "mfma_ceiling.hip": [],
     "elementwise.hip": ["-ffp-contract=off"],      # axpby!: rounded products, unfused sum
@@ -67,7 +69,7 @@ def _compile(item, force):
 # Kernels whose MFMAs are inline assembly: the compiler does not know how long their results take, so any
 # instruction of its own that touches an accumulator register next to them (a copy made by the register
 # allocator, an epilogue read scheduled upwards) would read a value that is not there yet, silently.
-ASM_MFMA_SOURCES = ["gemm_mfma256w4.hip"]
+ASM_MFMA_SOURCES = ["gemm_mfma256w4.hip", "gemm_mfma256w4_majors.hip", "gemm_mfma128w4.hip"]
 
 
 def check_accumulator_hazards(src, force=False):
@@ -175,10 +177,14 @@ def asm_mfma_hazards(lines, name="asm"):
 def build(force=False, verbose=True):
     os.makedirs(os.path.join(CSRC, "build"), exist_ok=True)
     items = [(s, f) for s, f in SOURCES.items() if os.path.exists(os.path.join(CSRC, s))]
-    with ThreadPoolExecutor(max_workers=min(8, len(items))) as ex:
-        results = list(ex.map(lambda it: _compile(it, force), items))
-    for src in ASM_MFMA_SOURCES:
-        check_accumulator_hazards(src, force)
+    # (the hazard checks compile their sources to assembly: they run beside the object compiles, the longest jobs first)
+    order = sorted(items, key=lambda it: it[0] not in ASM_MFMA_SOURCES)
+    with ThreadPoolExecutor(max_workers=8) as ex:
+        checks = [ex.submit(check_accumulator_hazards, src, force) for src in ASM_MFMA_SOURCES]
+        compiled = dict(zip([it[0] for it in order], ex.map(lambda it: _compile(it, force), order)))
+        for c in checks:
+            c.result()
+    results = [compiled[it[0]] for it in items]
     objs = [o for o, _ in results]
     for (src, _), (_, msg) in zip(items, results):
         if msg.strip() and verbose:

@@ -291,7 +291,8 @@ def test_known_shapes_run_on_the_instances_they_are_meant_for():
     assert step_names(run_case(f16, f16, 4096, 4096, 4096, cta=(256, 256, 64), ep=bias))[0].startswith("gemm_mfma_tn_256_w4")
     # the tile config 3 names (128 x 128 x 32)
     p = run_case(f16, f16, 4096, 4096, 4096, cta=(128, 128, 32), waves=(2, 2, 1))
-    assert p["steps"][0]["tile"] == "128x128x64B", p["text"]
+    # (stages of 128 x 32 in a ring of four, k-steps of two stages, two workgroups to a CU)
+    assert p["steps"][0]["name"].startswith("gemm_mfma_tn_256_w4<W4F16x2R4,OutF16,waves=4,") and p["steps"][0]["lds"] == 65536, p["text"]
     # mid-size problems: 128 x 128 tiles with K ranges, or 64 x 64 tiles, by the cost model; never 256 x 256 tiles with a split
     assert run_case(f16, f16, 1024, 1024, 1024, split_k=-1)["steps"][0]["tile"].startswith("64x64")
     assert run_case(f16, f16, 256, 256, 65536, split_k=-1)["steps"][0]["split"] > 1

@@ -528,6 +528,66 @@ __global__ __launch_bounds__(256) void copy_generic_cvt(const char* __restrict__
     }
 }
 
+// The same element loops, V elements per lane: for arrays whose first mode (once the modes are ordered by stride) is a
+// run of unit stride on every side -- pitched matrices, slices of larger arrays -- with V dividing its extent and every
+// other stride, and aligned pointers.  The vectorisation the reference computes with max_common_vector
+// (src/layout.jl:752-761) and leaves unused (src/algorithm/copy.jl:53-58), here also for converting copies (the wider
+// side moves 16 bytes per lane) and for copyto_if! (the mask is read V bytes at a time; a group whose mask is all true
+// goes out in one access, a mixed one element by element, so that elements whose mask is false are never written).
+// The layouts count groups of V elements (extent of mode 0 and the other strides divided by V).  Same conversion per
+// element as copy_generic_cvt; kSrc == kDst moves bits.
+template <int N> struct BytesOf;
+template <> struct BytesOf<1> { typedef uint8_t type; };
+template <> struct BytesOf<2> { typedef uint16_t type; };
+template <> struct BytesOf<4> { typedef uint32_t type; };
+template <> struct BytesOf<8> { typedef uint64_t type; };
+template <> struct BytesOf<16> { typedef u32x4 type; };
+template <int kSrc, int kDst, int SB, int DB, int V>
+__global__ __launch_bounds__(256) void copy_groups(const char* __restrict__ src, char* __restrict__ dst, FlatLayout ls, FlatLayout ld,
+                                                   int64_t ngroups, Mask mask) {
+    typedef typename BytesOf<V * SB>::type SrcWord;
+    typedef typename BytesOf<V * DB>::type DstWord;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < ngroups; g += stride) {
+        uint8_t keep[V];
+        bool all = true, any = true;
+        if (mask.ptr) {
+            typedef typename BytesOf<V>::type MaskWord;
+            const MaskWord mw = *reinterpret_cast<const MaskWord*>(mask.ptr + layout_offset(mask.l, g) * V);
+            __builtin_memcpy(keep, &mw, V);
+            any = false;
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                all = all && keep[e];
+                any = any || keep[e];
+            }
+            if (!any) continue;
+        }
+        const SrcWord in = *reinterpret_cast<const SrcWord*>(src + layout_offset(ls, g) * (V * SB));
+        char* const d = dst + layout_offset(ld, g) * (V * DB);
+        DstWord out;
+        if constexpr (kSrc == kDst) {
+            static_assert(SB == DB, "bits");
+            __builtin_memcpy(&out, &in, V * SB);
+        } else {
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                char e_in[SB], e_out[DB];
+                __builtin_memcpy(e_in, reinterpret_cast<const char*>(&in) + e * SB, SB);
+                store_from<kDst>(e_out, load_as_f64<kSrc>(e_in), kSrc == MOYE_F64);
+                __builtin_memcpy(reinterpret_cast<char*>(&out) + e * DB, e_out, DB);
+            }
+        }
+        if (all) {
+            *reinterpret_cast<DstWord*>(d) = out;
+        } else {
+#pragma unroll
+            for (int e = 0; e < V; ++e)
+                if (keep[e]) __builtin_memcpy(d + e * DB, reinterpret_cast<const char*>(&out) + e * DB, DB);
+        }
+    }
+}
+
 // Converting copy between two dense, 16-byte aligned runs of elements of one width (fp16 <-> bf16): a lane converts the
 // elements of one 16-byte piece; one workgroup per 256 pieces, no loop.  Element by element the same conversion as
 // copy_generic_cvt.
@@ -694,6 +754,65 @@ static bool launch_cvt_dst(int32_t dd, dim3 g, hipStream_t st, const char* s, ch
         case MOYE_BF16: copy_generic_cvt<kSrc, MOYE_BF16><<<g, 256, 0, st>>>(s, d, ls, ld, n, sb, db, mk); return true;
         case MOYE_F8E4M3: copy_generic_cvt<kSrc, MOYE_F8E4M3><<<g, 256, 0, st>>>(s, d, ls, ld, n, sb, db, mk); return true;
         case MOYE_F64: copy_generic_cvt<kSrc, MOYE_F64><<<g, 256, 0, st>>>(s, d, ls, ld, n, sb, db, mk); return true;
+        default: return false;
+    }
+}
+
+template <int kSrc, int kDst, int SB, int DB>
+static void launch_groups_pair(const char* s, char* d, const FlatLayout& ls, const FlatLayout& ld, int64_t ngroups, const Mask& mk, hipStream_t st) {
+    constexpr int V = 16 / (SB > DB ? SB : DB);
+    static_assert(V >= 2, "groups of at least two elements");
+    copy_groups<kSrc, kDst, SB, DB, V><<<strided_grid(ngroups), 256, 0, st>>>(s, d, ls, ld, ngroups, mk);
+}
+template <int kSrc, int SB>
+static bool launch_groups_dst(int32_t dd, const char* s, char* d, const FlatLayout& ls, const FlatLayout& ld, int64_t ng, const Mask& mk, hipStream_t st) {
+    switch (dd) {
+        case MOYE_F32: launch_groups_pair<kSrc, MOYE_F32, SB, 4>(s, d, ls, ld, ng, mk, st); return true;
+        case MOYE_F16: launch_groups_pair<kSrc, MOYE_F16, SB, 2>(s, d, ls, ld, ng, mk, st); return true;
+        case MOYE_BF16: launch_groups_pair<kSrc, MOYE_BF16, SB, 2>(s, d, ls, ld, ng, mk, st); return true;
+        case MOYE_F8E4M3: launch_groups_pair<kSrc, MOYE_F8E4M3, SB, 1>(s, d, ls, ld, ng, mk, st); return true;
+        case MOYE_F64: launch_groups_pair<kSrc, MOYE_F64, SB, 8>(s, d, ls, ld, ng, mk, st); return true;
+        default: return false;
+    }
+}
+// Groups of V = 16 / (the wider element) elements along the first mode, when every layout of the call (the modes already
+// ordered by stride) has it as a run of unit stride that V divides, V divides every other stride that is used, and the
+// pointers are aligned to what a lane then accesses.  `same_bits`: a copy of bits (with a mask: copyto_if!).  Returns
+// false, having launched nothing, when the call does not qualify.
+static bool launch_groups(int32_t src_dt, int32_t dst_dt, const char* s, char* d, FlatLayout ls, FlatLayout ld, Mask mk, bool same_bits, int64_t n,
+                          hipStream_t st) {
+    const int sb = dtype_bytes(src_dt), db = dtype_bytes(dst_dt);
+    const int V = 16 / std::max(sb, db);
+    if (V < 2 || ls.rank < 1 || ld.rank != ls.rank) return false;
+    auto fits = [&](const FlatLayout& l, const void* p, int elem_bytes) {
+        if (l.stride[0] != 1 || l.shape[0] % V || reinterpret_cast<uintptr_t>(p) % (V * elem_bytes)) return false;
+        for (int m = 1; m < MOYE_MAX_RANK; ++m)
+            if (l.shape[m] > 1 && l.stride[m] % V) return false;
+        return true;
+    };
+    if (ls.shape[0] != ld.shape[0] || !fits(ls, s, sb) || !fits(ld, d, db)) return false;
+    if (mk.ptr && (mk.l.rank != ls.rank || mk.l.shape[0] != ls.shape[0] || !fits(mk.l, mk.ptr, 1))) return false;
+    for (FlatLayout* l : {&ls, &ld, &mk.l}) {
+        if (l == &mk.l && !mk.ptr) continue;
+        l->shape[0] /= V;
+        for (int m = 1; m < MOYE_MAX_RANK; ++m) l->stride[m] /= V;
+    }
+    const int64_t ng = n / V;
+    if (same_bits) {
+        switch (sb) {
+            case 1: copy_groups<MOYE_U8, MOYE_U8, 1, 1, 16><<<strided_grid(ng), 256, 0, st>>>(s, d, ls, ld, ng, mk); return true;
+            case 2: copy_groups<MOYE_U16, MOYE_U16, 2, 2, 8><<<strided_grid(ng), 256, 0, st>>>(s, d, ls, ld, ng, mk); return true;
+            case 4: copy_groups<MOYE_U32, MOYE_U32, 4, 4, 4><<<strided_grid(ng), 256, 0, st>>>(s, d, ls, ld, ng, mk); return true;
+            case 8: copy_groups<MOYE_U64, MOYE_U64, 8, 8, 2><<<strided_grid(ng), 256, 0, st>>>(s, d, ls, ld, ng, mk); return true;
+            default: return false;
+        }
+    }
+    switch (src_dt) {
+        case MOYE_F32: return launch_groups_dst<MOYE_F32, 4>(dst_dt, s, d, ls, ld, ng, mk, st);
+        case MOYE_F16: return launch_groups_dst<MOYE_F16, 2>(dst_dt, s, d, ls, ld, ng, mk, st);
+        case MOYE_BF16: return launch_groups_dst<MOYE_BF16, 2>(dst_dt, s, d, ls, ld, ng, mk, st);
+        case MOYE_F8E4M3: return launch_groups_dst<MOYE_F8E4M3, 1>(dst_dt, s, d, ls, ld, ng, mk, st);
+        case MOYE_F64: return launch_groups_dst<MOYE_F64, 8>(dst_dt, s, d, ls, ld, ng, mk, st);
         default: return false;
     }
 }
@@ -967,6 +1086,12 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
                 l->stride[0] = 1;
             }
         }
+    }
+    // converting copies between pitched arrays, and copyto_if!: groups of elements along the first mode where the layouts
+    // allow (a plain copy of bits has taken its vectorised path above)
+    if ((!same_bits || mask) && launch_groups(src->dtype, dst->dtype, s, d, ls, ld, mk, same_bits, n, st)) {
+        MOYE_HIP_CHECK(hipGetLastError());
+        return MOYE_OK;
     }
     const dim3 g((unsigned)std::min<int64_t>((n + 255) / 256, 256 * 64));
     bool ok = true;

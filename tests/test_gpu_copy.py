@@ -300,6 +300,53 @@ def test_dense_converting_copy_matches_the_general_kernel(mh):
                     assert bool(((a == want.view(it)) | (torch.isnan(d1.float()) & torch.isnan(want.float()))).all()), (sdt, ddt, n, "torch")
 
 
+def test_pitched_converting_copies_and_masked_copies_in_groups(mh):
+    """Pitched matrices (row-major inside wider buffers): converting copies between every pair of floating-point types, and
+    copyto_if! of bits and with conversion, take a kernel that moves groups of elements along the rows.  Checked element
+    by element: against torch's conversion of the same window (fp8 aside: against the library's own dense conversion),
+    the masked-out elements and the padding untouched.  Shapes whose rows the group does not divide, or whose windows
+    start off alignment, fall back to the element loop and must give the same bits."""
+    types = [torch.float32, torch.float16, torch.bfloat16, torch.float64]
+    if hasattr(torch, "float8_e4m3fn"):
+        types.append(torch.float8_e4m3fn)
+    g = torch.Generator().manual_seed(23)
+    it_of = {1: torch.uint8, 2: torch.int16, 4: torch.int32, 8: torch.int64}
+    for (R, Cn, ps, pd, off) in ((300, 512, 528, 640, 0), (257, 48, 64, 48, 0), (64, 200, 208, 216, 0), (33, 96, 100, 104, 0), (100, 128, 144, 160, 1)):
+        for sdt in types:
+            for ddt in types:
+                X = (torch.randn(R, ps, generator=g) * 20).to(sdt).cuda()
+                M = (torch.rand(R, Cn + 16, generator=g) < 0.4).to(torch.uint8).cuda() * 7
+                src = X[:, off:off + Cn]
+                want_full = src.to(ddt) if ddt != getattr(torch, "float8_e4m3fn", None) or sdt == ddt else None
+                if want_full is None:           # the library's own conversion of a dense copy of the window
+                    dense = src.contiguous()
+                    want_full = torch.zeros(R, Cn, dtype=ddt, device="cuda")
+                    mh.copyto_(_tens(mh, want_full, [R * Cn], [1]), _tens(mh, dense, [R * Cn], [1]))
+                it = it_of[torch.empty(0, dtype=ddt).element_size()]
+                if sdt != ddt:
+                    D = torch.full((R, pd), 3.0).to(ddt).cuda()
+                    mh.copyto_(_tens(mh, D[:, off:off + Cn], (R, Cn), (pd, 1)), _tens(mh, src, (R, Cn), (ps, 1)))
+                    torch.cuda.synchronize()
+                    got = D[:, off:off + Cn]
+                    same = (got.contiguous().view(it) == want_full.contiguous().view(it)) | (torch.isnan(got.float()) & torch.isnan(want_full.float()))
+                    assert bool(same.all()), (sdt, ddt, R, Cn, "converting copy")
+                    frame = D.clone()
+                    frame[:, off:off + Cn] = 3.0
+                    assert bool((frame.float() == 3.0).all()), (sdt, ddt, "padding of dst touched")
+                # copyto_if! with a mask that is a window of a wider byte array
+                D = torch.full((R, pd), 3.0).to(ddt).cuda()
+                mask = M[:, off:off + Cn]
+                mh.copyto_if_(_tens(mh, D[:, off:off + Cn], (R, Cn), (pd, 1)), _tens(mh, src, (R, Cn), (ps, 1)), _tens(mh, mask, (R, Cn), (Cn + 16, 1)))
+                torch.cuda.synchronize()
+                got = D[:, off:off + Cn].contiguous()
+                want = torch.where(mask != 0, want_full.float().double(), torch.full((), 3.0, dtype=torch.float64, device="cuda"))
+                gotd = got.float().double()
+                assert bool(((gotd == want) | (torch.isnan(gotd) & torch.isnan(want))).all()), (sdt, ddt, R, Cn, "copyto_if!")
+                frame = D.clone()
+                frame[:, off:off + Cn] = 3.0
+                assert bool((frame.float() == 3.0).all()), (sdt, ddt, "padding of dst touched by copyto_if!")
+
+
 def test_fp8_conversion_matches_torch(mh):
     if not hasattr(torch, "float8_e4m3fn"):
         pytest.skip("torch without float8_e4m3fn")

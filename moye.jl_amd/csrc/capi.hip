@@ -346,6 +346,13 @@ static bool operand_rows_in_16_byte_pieces(const GemmArgs& g) {
     return reinterpret_cast<uintptr_t>(g.ep_x) % 16 == 0 && (g.ep_xm * eb) % 16 == 0;
 }
 
+// an epilogue operation the lanes can apply to their own accumulators: its operand is a scalar, one value per column or one
+// per row, or it has none (a bias, a ReLU, a scale); a division stays with the general epilogue (its code is long, and the
+// lanes' form is unrolled over all accumulators)
+static bool lane_op(const GemmArgs& g) {
+    return g.ep_op != MOYE_MAP_IDENTITY && g.ep_op != MOYE_MAP_DIV && (!g.ep_x || g.ep_xm == 0 || g.ep_xn == 0);
+}
+
 // gemm!(mma, D, A, B, C) with the epilogue `ep` as a list of launches.  Pure host arithmetic on the descriptors: nothing
 // is launched, allocated or asked of a device (plan.shape says what the chip looks like).  `workspace(bytes, &ptr)` is
 // asked once, and only when the call needs a workspace, for `bytes` bytes: the caller's buffer, the library's own, the
@@ -505,7 +512,7 @@ static int32_t gemm_plan_build(const moye_tiled_mma* mma, const moye_tensor* tD,
         g.C = tC ? C.ptr : nullptr; g.ldc_m = C.rs; g.ldc_n = C.cs; g.D = D.ptr;
         if (rows_in_16_byte_pieces(g.C, g.ldc_m, g.ldc_n, D.dtype)) g.flags |= kGemmRowC;
         if (operand_rows_in_16_byte_pieces(g)) g.flags |= kGemmEpiRowX;
-        if (g.ep_op == MOYE_MAP_ADD && (!g.ep_x || g.ep_xm == 0 || g.ep_xn == 0)) g.flags |= kGemmEpiAddVec;  // a bias
+        if (lane_op(g)) g.flags |= kGemmEpiLaneOp;
         return gemm_mfma_tn_dispatch(in_dt, D.dtype, bm, bn, bk, waves, mma->stages, g, plan, lib_tile);
     }
     if (D.rs == 1 && bm == 0 && bn == 0 && M <= 64 && ((int64_t)K * dtype_bytes(in_dt)) % 16 == 0) {
@@ -522,7 +529,7 @@ static int32_t gemm_plan_build(const moye_tiled_mma* mma, const moye_tensor* tD,
                   ((major_flags & kGemmBMajorN) ? kGemmAMajorM : 0);
         if (rows_in_16_byte_pieces(g.C, g.ldc_m, g.ldc_n, D.dtype)) g.flags |= kGemmRowC;
         if (operand_rows_in_16_byte_pieces(g)) g.flags |= kGemmEpiRowX;
-        if (g.ep_op == MOYE_MAP_ADD && (!g.ep_x || g.ep_xm == 0 || g.ep_xn == 0)) g.flags |= kGemmEpiAddVec;
+        if (lane_op(g)) g.flags |= kGemmEpiLaneOp;
         // (the library's choice was priced for (M, N); the cost model is symmetric in them)
         return gemm_mfma_tn_dispatch(in_dt, D.dtype, bn, bm, bk, waves, mma->stages, g, plan, lib_tile);
     }
@@ -599,7 +606,7 @@ static std::string flag_names(int f) {
     add(f & 1, "xcd_order"); add(f & MOYE_GEMM_PINGPONG, "pingpong"); add(f & MOYE_GEMM_PREDICATE, "predicate"); add(f & MOYE_GEMM_WAVE4, "hand_ordered");
     add(f & kGemmAtom32, "atom32"); add(f & kGemmRotateK, "rotate_k"); add(f & kGemmStreamD, "stream_d"); add(f & kGemmRowC, "row_c");
     add(f & kGemmAMajorM, "a_m_major"); add(f & kGemmBMajorN, "b_n_major"); add(f & kGemmEpiRowX, "row_x"); add(f & kGemmRagged, "ragged");
-    add(f & kGemmEpiAddVec, "add_vec");
+    add(f & kGemmEpiLaneOp, "lane_op");
     return s.empty() ? "0" : s;
 }
 

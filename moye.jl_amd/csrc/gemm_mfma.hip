@@ -372,15 +372,15 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
                                  (fr_m > 0 ? 4.5 + (double)(a.N + fr_m) * (double)k_bytes_all / 6.0e6 : 0.0);
         const bool thin = thin_shape && (int64_t)(M0 / 256) * (N0 / 256) >= cus / 4 &&
                           gemm_plan_cost_256(M0, N0, k_bytes_all, eb == 4, false, cus) + fringe_us <= choice.us;
-        // (fp8: only the hand-ordered kernel's guarded form, i.e. K of whole 128-byte rows, no C, no operation)
+        // (fp8: only the hand-ordered kernel's guarded forms, i.e. K of whole 128-byte rows)
         const bool hand_ordered_ragged = (eb == 2 || eb == 4 || in_dt == MOYE_F8E4M3) && ((int64_t)a.K * eb) % 128 == 0 &&
-                                         a.ep_op == MOYE_MAP_IDENTITY && !a.C && stages < 2 && row_offsets_fit(a, 256, eb);
+                                         stages < 2 && row_offsets_fit(a, 256, eb);
         if ((!big || !aligned) && !thin && a.split <= 1 && bk_elems == 0 && aligned_ab && (in_dt != MOYE_F8E4M3 || hand_ordered_ragged) && ((int64_t)a.K * eb) % 16 == 0 &&
             prefer256 && stages < 3 && (waves <= 1 || waves == 8) &&
             !(a.flags & (MOYE_GEMM_WAVE4 | MOYE_GEMM_PINGPONG | kGemmAMajorM | kGemmBMajorN | kGemmAtom32))) {
             a.flags |= kGemmRagged;
-            // K of whole 128-byte rows, no C and no epilogue operation: the hand-ordered kernel's guarded form (rows
-            // clamped, no K tail to mask)
+            // K of whole 128-byte rows: the hand-ordered kernel's guarded forms (rows clamped, no K tail to mask; with a C
+            // or an element-wise operation the instance whose epilogue is the general one)
             if (hand_ordered_ragged) return gemm_mfma_tn_256_w4_dispatch(in_dt, out_dt, a, 8, 128, false, plan);
             return gemm_mfma_tn_256_dispatch(in_dt, out_dt, a, 8, stages, plan);
         }
@@ -491,27 +491,30 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
     if (bm == 256 && bn == 256) {
         if (bkb != 128 && bkb != 64)
             return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the 256x256 MFMA kernels take %d or %d elements of K per tile", 64 / eb, 128 / eb);
-        // the hand-ordered kernel has no element-wise operations in its epilogue
-        if ((a.flags & (MOYE_GEMM_WAVE4 | MOYE_GEMM_PINGPONG)) && a.ep_op != MOYE_MAP_IDENTITY)
-            return fail(MOYE_ERR_UNSUPPORTED, "gemm!: MOYE_GEMM_WAVE4 and MOYE_GEMM_PINGPONG take no element-wise epilogue operation; leave the schedule to the library");
+        // the ping-pong kernel has no element-wise operations in its epilogue (the hand-ordered one has them in its
+        // eight-wave whole-line form and says so itself where a caller asks for another of its schedules)
+        if ((a.flags & MOYE_GEMM_PINGPONG) && a.ep_op != MOYE_MAP_IDENTITY)
+            return fail(MOYE_ERR_UNSUPPORTED, "gemm!: MOYE_GEMM_PINGPONG takes no element-wise epilogue operation; leave the schedule to the library");
+        const bool majors256 = a.flags & (kGemmAMajorM | kGemmBMajorN);
+        // an element-wise operation: the hand-ordered kernel's eight-wave whole-line form on K-major operands
+        const bool ops_fit = a.ep_op == MOYE_MAP_IDENTITY || (waves != 4 && stages < 2 && !majors256);
         // fp8 runs at twice the 16-bit rate only on the 16x16x128 MFMA, which the hand-ordered kernel issues
-        if (in_dt == MOYE_F8E4M3 && bkb == 128 && stages < 3 && !(a.flags & MOYE_GEMM_PINGPONG) && a.ep_op == MOYE_MAP_IDENTITY)
+        if (in_dt == MOYE_F8E4M3 && bkb == 128 && stages < 3 && !(a.flags & MOYE_GEMM_PINGPONG) && ops_fit)
             a.flags |= MOYE_GEMM_WAVE4;
         // ... and for the 16-bit types its form with whole 128-byte rows in two stages is the fastest k-loop of this build
-        // for a plain call (fp16 4096^3 97.6-98.6 us against 101.3-102.0 for the compiler-scheduled kernel on the same
-        // box, bf16 8192^3 726 against 754); operations in the epilogue and a K tail stay with that kernel, and so does a
-        // call that asks for it: stages = 2 in the descriptor.
-        const bool bias_no_c = (a.flags & kGemmEpiAddVec) && !a.C && waves != 4;  // (its bias instance: eight waves, no C)
+        // (fp16 4096^3 97.6-98.6 us against 101.3-102.0 for the compiler-scheduled kernel on the same box, bf16 8192^3 726
+        // against 754); a K tail stays with that kernel, and so does a call that asks for it: stages = 2 in the descriptor.
         // (operands that keep their M- / N-major form: its transposing fragment reads, eight waves, plain calls; fp16 4096^3 NN
         // against the compiler-scheduled kernel's: see the kernel's header)
-        const bool majors256 = a.flags & (kGemmAMajorM | kGemmBMajorN);
-        if (eb == 2 && bkb == 128 && stages < 2 && (a.ep_op == MOYE_MAP_IDENTITY || (bias_no_c && !majors256)) &&
-            (!majors256 || (waves != 4 && !(a.flags & kGemmEpiAddVec))) &&
+        // (an operation the lanes apply themselves, with a C: the compiler-scheduled kernel has that form, whose epilogue
+        // costs nothing extra, where this one's general epilogue costs 11 us per round of tiles)
+        if (eb == 2 && bkb == 128 && stages < 2 && ops_fit && !((a.flags & kGemmEpiLaneOp) && a.C) &&
+            (!majors256 || (waves != 4 && !(a.flags & kGemmEpiLaneOp))) &&
             !(a.flags & (MOYE_GEMM_PINGPONG | kGemmRagged | kGemmAtom32)) && row_offsets_fit(a, 256, eb))
             a.flags |= MOYE_GEMM_WAVE4;
         // fp32 operands: the hand-ordered kernel too (fp32 8192^3 152.8 TFLOP/s on whole-line stages, 147.8 on its ring of
         // 64-byte-row stages, 142.5 for the compiler-scheduled kernel)
-        if (in_dt == MOYE_F32 && stages < 2 && a.ep_op == MOYE_MAP_IDENTITY && a.K % 16 == 0 &&
+        if (in_dt == MOYE_F32 && stages < 2 && ops_fit && (a.ep_op == MOYE_MAP_IDENTITY || bkb == 128) && a.K % 16 == 0 &&
             (!majors256 || (waves != 4 && bkb == 128)) &&
             !(a.flags & (MOYE_GEMM_PINGPONG | kGemmRagged | kGemmAtom32)) && row_offsets_fit(a, 256, eb))
             a.flags |= MOYE_GEMM_WAVE4;
@@ -559,7 +562,7 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         // 1136 -> 914 us, 2048^3 128.8 -> 122.5)
         if (whole && (int64_t)(a.M / 128) * (a.N / 128) > (eb == 2 ? cus : 0) &&
             (eb == 2 || eb == 4 || in_dt == MOYE_F8E4M3) && a.ep_op == MOYE_MAP_IDENTITY && stages < 2 &&
-            !(a.flags & (kGemmAMajorM | kGemmBMajorN | kGemmEpiAddVec)) && row_offsets_fit(a, 128, eb))
+            !(a.flags & (kGemmAMajorM | kGemmBMajorN | kGemmEpiLaneOp)) && row_offsets_fit(a, 128, eb))
             return gemm_mfma_tn_128_w4_dispatch(in_dt, out_dt, a, plan);
         if (whole) return gemm_mfma_tn_128_dispatch(in_dt, out_dt, a, plan);
         if (chosen_here || (a.flags & MOYE_GEMM_PREDICATE)) {
@@ -567,7 +570,7 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
             // (K of whole 128-byte rows, no C, no operation, more tiles than CUs: the guarded form of the hand-ordered instance)
             if ((int64_t)((a.M + 127) / 128) * ((a.N + 127) / 128) > (eb == 2 ? cus : 0) &&
                 (eb == 2 || eb == 4 || in_dt == MOYE_F8E4M3) && ((int64_t)a.K * eb) % 128 == 0 &&
-                a.ep_op == MOYE_MAP_IDENTITY && !a.C && stages < 2 && !(a.flags & (kGemmAMajorM | kGemmBMajorN | kGemmEpiAddVec)) &&
+                a.ep_op == MOYE_MAP_IDENTITY && !a.C && stages < 2 && !(a.flags & (kGemmAMajorM | kGemmBMajorN | kGemmEpiLaneOp)) &&
                 row_offsets_fit(a, 128, eb))
                 return gemm_mfma_tn_128_w4_dispatch(in_dt, out_dt, a, plan);
             return gemm_mfma_tn_128_dispatch(in_dt, out_dt, a, plan);
@@ -577,7 +580,7 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
     // configuration names): plain f16 / bf16 calls on whole tiles, K a whole number of two-stage k-steps, run the
     // hand-ordered kernel's ring of four such stages (fp16 4096^3 140-143 us against 161-171); the rest the register-staged kernel.
     if (bm == 128 && bn == 128 && bkb == 64 && eb == 2 && !misaligned && a.M % 128 == 0 && a.N % 128 == 0 && ((int64_t)a.K * eb) % 128 == 0 &&
-        a.ep_op == MOYE_MAP_IDENTITY && stages < 2 && !(a.flags & (kGemmAMajorM | kGemmBMajorN | kGemmEpiAddVec | kGemmAtom32 | kGemmRagged | MOYE_GEMM_PINGPONG)) &&
+        a.ep_op == MOYE_MAP_IDENTITY && stages < 2 && !(a.flags & (kGemmAMajorM | kGemmBMajorN | kGemmEpiLaneOp | kGemmAtom32 | kGemmRagged | MOYE_GEMM_PINGPONG)) &&
         row_offsets_fit(a, 128, eb))
         return gemm_mfma_tn_128_w4_dispatch(in_dt, out_dt, a, plan, true);
     if (bm != 128 || bn != 128 || (bkb != 64 && bkb != 128))

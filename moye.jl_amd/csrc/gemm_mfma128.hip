@@ -43,7 +43,7 @@ static int32_t launch128(const GemmArgs& a, GemmPlan& plan) {
     }
     if (a.flags & kGemmRagged)
         return a.ep_op != MOYE_MAP_IDENTITY ? launch128_instance<In, Out, true, true>(a, plan) : launch128_instance<In, Out, false, true>(a, plan);
-    if (a.flags & kGemmEpiAddVec) return launch128_instance<In, Out, false, false, 0, 0, true>(a, plan);  // a bias
+    if (a.flags & kGemmEpiLaneOp) return launch128_instance<In, Out, false, false, 0, 0, true>(a, plan);  // a bias, a ReLU, a scale: in the lanes
     if (a.ep_op != MOYE_MAP_IDENTITY) return launch128_instance<In, Out, true, false>(a, plan);
     return launch128_instance<In, Out, false, false>(a, plan);
 }

@@ -10,9 +10,10 @@
 // The k-loop and the epilogue are gemm_mfma_tn_lds_tile (gemm_mfma_lds_tile.hpp), shared with the 128 x 128 kernel of
 // gemm_mfma128.hip; the ring schedule below is a second k-loop for the same tile.  This k-loop is scheduled by the
 // compiler under sched_group_barrier hints.  Plain f16 / bf16 calls now run the hand-ordered kernel of
-// gemm_mfma256w4.hip instead (same tile, same LDS layout, 4 % faster); this one keeps everything that kernel has no
-// instance for: epilogue operations, a bias together with C, operands that are not K-major, a K tail, fp32 operands,
-// and calls that name it (stages = 2).
+// gemm_mfma256w4.hip instead (same tile, same LDS layout, 4 % faster), and so do calls with fp8 and fp32 operands, with
+// operands that are not K-major and with an element-wise operation; this one keeps what that kernel has no instance for:
+// a bias, ReLU or scale together with C, an operation on operands that are not K-major, a K tail, and calls that name it
+// (stages = 2).
 #include "gemm_mfma_lds_tile.hpp"
 
 namespace moye {
@@ -182,7 +183,7 @@ static int32_t launch256(const GemmArgs& a, GemmPlan& plan) {
         }
     }
     if constexpr (WGM * WGN == 8) {
-        if (a.flags & kGemmEpiAddVec) return launch256_instance<In, Out, WGM, WGN, false, 0, 0, false, true>(a, plan);  // a bias
+        if (a.flags & kGemmEpiLaneOp) return launch256_instance<In, Out, WGM, WGN, false, 0, 0, false, true>(a, plan);  // a bias, a ReLU, a scale: in the lanes
         if (a.ep_op != MOYE_MAP_IDENTITY) return launch256_instance<In, Out, WGM, WGN, true, 0, 0>(a, plan);
     }
     return launch256_instance<In, Out, WGM, WGN, false, 0, 0>(a, plan);

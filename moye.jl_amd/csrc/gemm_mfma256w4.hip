@@ -1,5 +1,5 @@
 // The hand-ordered kernel (gemm_mfma_w4_kernel.hpp) on the 256 x 256 tile with K-major operands: plain, bias and guarded
-// instances of every operand type and schedule.
+// instances of every operand type and schedule (those with an element-wise operation: gemm_mfma256w4_ops.hip).
 #include "gemm_mfma_w4_kernel.hpp"
 
 namespace moye {
@@ -8,16 +8,25 @@ template <typename In, int WGN>
 static int32_t launch256_w4_out(int32_t out_dt, const GemmArgs& a, GemmPlan& plan) {
     if (a.flags & (kGemmAMajorM | kGemmBMajorN)) {
         if constexpr (In::kRow == 128 && WGN == 4) {
-            if ((a.flags & (kGemmRagged | kGemmEpiAddVec)) || a.ep_op != MOYE_MAP_IDENTITY)
+            if ((a.flags & (kGemmRagged | kGemmEpiLaneOp)) || a.ep_op != MOYE_MAP_IDENTITY)
                 return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the hand-ordered kernel takes operands that are not K-major in plain calls on whole tiles only");
             return launch256_w4_majors_dispatch(In::kDt, out_dt, a, plan);
         } else {
             return fail(MOYE_ERR_UNSUPPORTED, "gemm!: this schedule of the hand-ordered kernel takes K-major operands only");
         }
     }
+    // An element-wise operation, or a C on ragged tiles: the instances whose epilogue is the general one (an operation
+    // with a scalar, one-per-column or one-per-row operand on whole tiles of the 16-bit types without C has its own form
+    // below: applied in the lanes' own accumulators)
+    const bool bias_form = (a.flags & kGemmEpiLaneOp) && !a.C && !(a.flags & kGemmRagged) && In::kBytes == 2;
+    if ((a.ep_op != MOYE_MAP_IDENTITY && !bias_form) || ((a.flags & kGemmRagged) && a.C)) {
+        if constexpr (In::kRow == 128 && WGN == 4)
+            return launch256_w4_ops_dispatch(In::kDt, out_dt, a, plan);
+        else
+            return fail(MOYE_ERR_UNSUPPORTED, "gemm!: this schedule of the hand-ordered kernel takes no element-wise epilogue operation");
+    }
     if (a.flags & kGemmRagged) {  // tiles that reach beyond M or N: the eight-wave whole-line forms
         if constexpr (In::kRow == 128 && WGN == 4) {
-            if (a.ep_op != MOYE_MAP_IDENTITY || a.C) return fail(MOYE_ERR_UNSUPPORTED, "gemm!: ragged tiles of the hand-ordered kernel take no C and no epilogue operation");
             switch (out_dt) {
                 case MOYE_F32: return launch256_w4<In, OutF32, WGN, false, true>(a, plan);
                 case MOYE_F16: return launch256_w4<In, OutF16, WGN, false, true>(a, plan);
@@ -28,9 +37,8 @@ static int32_t launch256_w4_out(int32_t out_dt, const GemmArgs& a, GemmPlan& pla
             return fail(MOYE_ERR_UNSUPPORTED, "gemm!: this schedule of the hand-ordered kernel takes whole tiles only");
         }
     }
-    if (a.flags & kGemmEpiAddVec) {  // a bias: the eight-wave whole-line forms of the 16-bit types carry it, for calls without C
+    if (bias_form) {  // a bias, a ReLU, a scale: the eight-wave whole-line forms of the 16-bit types carry it, for calls without C
         if constexpr (In::kRow == 128 && In::kBytes == 2 && WGN == 4) {
-            if (a.C) return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the bias instance of the hand-ordered kernel takes no C");
             switch (out_dt) {
                 case MOYE_F32: return launch256_w4<In, OutF32, WGN, true>(a, plan);
                 case MOYE_F16: return launch256_w4<In, OutF16, WGN, true>(a, plan);

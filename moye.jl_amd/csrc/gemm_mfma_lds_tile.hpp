@@ -44,8 +44,9 @@ namespace moye {
 // row's first piece instead and every fragment piece beyond K is zeroed in registers before it reaches an MFMA; the
 // epilogues run with their row and column guards.
 //
-// kBias: the call adds a vector (one value per column or per row) or a scalar to the product -- a bias: an instance of
-// its own that is the plain kernel with that addition in the lanes' own epilogue, nothing of the general one.
+// kBias: the call's element-wise operation has a scalar, one-per-column or one-per-row operand or none and is no division
+// (kGemmEpiLaneOp: a bias, a ReLU, a scale): an instance of its own that is the plain kernel with that operation in the
+// lanes' own epilogue, nothing of the general one.
 template <typename In, typename Out, int BM, int BN, int WGM, int WGN, bool kOps, int AMAJ, int BMAJ, bool kRagged, bool kBias = false>
 __device__ __forceinline__ void gemm_mfma_tn_lds_tile(GemmArgs p) {
     static_assert(!kRagged || (!AMAJ && !BMAJ), "ragged tiles: K-major operands");

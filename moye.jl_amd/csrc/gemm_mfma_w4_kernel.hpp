@@ -241,14 +241,17 @@ struct W4F32 : W4Ring64 {
 // WGN = 2: four waves (2 x 2), wave tile 128 x 128.  WGN = 4: eight waves (2 x 4), wave tile 128 x 64,
 // two waves per SIMD, so that what stalls one wave's instruction stream (an M0 write, a taken branch,
 // the barrier) leaves the matrix pipe to the other.
-// kBias: the call adds a vector (one value per column or per row) or a scalar to the product and has no C: the same
-// kernel with that addition in the lanes' own epilogue (store_c_tile's kAddVec, without C's read paths, whose registers
-// this kernel cannot spare: with them the epilogue spilled 96 registers).
+// kBias: the call's element-wise operation has a scalar, one-per-column or one-per-row operand (a bias, a ReLU, a scale:
+// kGemmEpiLaneOp) and the call has no C: the same kernel with that operation in the lanes' own epilogue (store_c_tile's
+// kLaneOp, without C's read paths, whose registers this kernel cannot spare: with them the epilogue spilled 96 registers).
 // kRagged: M and N need not be multiples of 256 (K stays a whole number of 128-byte rows): a lane whose row lies beyond
 // the operand reads the operand's last row instead (its constant lane offset is computed from the clamped row), what is
 // computed from it is never stored, and the epilogue runs with its row and column guards (a D that is not 16-byte
 // aligned goes out element by element where it must).  For calls without C, like the bias instance: the guards and C's
 // read paths together spilled 64-110 registers.
+// kOps: the epilogue is store_c_tile_general (any element-wise operation, any C, whole or ragged tiles): the raw
+// accumulators go through LDS 32 rows at a time and the arithmetic exists once, in a loop, which costs the 16-bit
+// outputs 9-20 spilled registers after the last MFMA and none before.  Whole-line stages, eight waves, K-major operands.
 //
 // TILE = 128: the same kernel on a 128 x 128 CTA tile, four waves as 2 x 2 (wave tile 64 x 64, 4 x 4 MFMA tiles), two
 // whole-line stages of 32 KiB, two workgroups per CU (what gemm_mfma128.hip's kernel is to gemm_mfma256.hip's): rows 0-1
@@ -288,11 +291,12 @@ struct W4F32L {
 // k-rows 4 g + e and 16 + 4 g + e (k-rows of 1 KiB, 32 per stage; the 64-byte piece index XORed with (row / 4) % 2, so
 // that the two k-rows the 32 lanes of a pass read lie in different halves of the banks).  Whole-line stages on the
 // 256 x 256 tile, eight waves, no bias, whole tiles.
-template <typename In, typename Out, int WGN, bool kBias = false, bool kRagged = false, int TILE = 256, int AMAJ = 0, int BMAJ = 0>
+template <typename In, typename Out, int WGN, bool kBias = false, bool kRagged = false, int TILE = 256, int AMAJ = 0, int BMAJ = 0, bool kOps = false>
 __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_256_w4(GemmArgs p) {
     static_assert(!(AMAJ || BMAJ) || (In::kRow == 128 && TILE == 256 && WGN == 4 && !kBias && !kRagged),
                   "operands that are not K-major: whole-line stages, eight waves, plain whole tiles");
     static_assert(!kRagged || (!kBias && In::kRow == 128), "ragged tiles: the plain whole-line form");
+    static_assert(!kOps || (In::kRow == 128 && TILE == 256 && WGN == 4 && !kBias && !AMAJ && !BMAJ), "epilogue operations: whole-line stages, eight waves, K-major operands");
     static_assert(TILE == 256 || (TILE == 128 && WGN == 2 && !kBias && (In::kRow == 128 || (In::SPS == 2 && !kRagged))),
                   "128 x 128 tiles: 2 x 2 waves; the whole-line form, plain or ragged, or the ring of 64-byte-row stages with k-steps of two stages");
     constexpr int BM = TILE, BN = TILE, kRow = In::kRow, CPR = kRow / 16, STAGES = In::kRing, SPS = In::SPS;
@@ -589,23 +593,27 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
         for (int j = 0; j < NI; ++j) asm volatile("" : "+a"(acc[i][j]));
     __syncthreads();  // every wave is done with the operand ring before it becomes C patches
 
-    store_c_tile<Out, MI, NI, kRagged, kBias, kBias || kRagged>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
+    if constexpr (kOps)
+        store_c_tile_general<Out, MI, NI, kRagged>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
+    else
+        store_c_tile<Out, MI, NI, kRagged, kBias, kBias || kRagged>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
 }
 
-template <typename In, typename Out, int WGN, bool kBias = false, bool kRagged = false, int TILE = 256, int AMAJ = 0, int BMAJ = 0>
+template <typename In, typename Out, int WGN, bool kBias = false, bool kRagged = false, int TILE = 256, int AMAJ = 0, int BMAJ = 0, bool kOps = false>
 static int32_t launch256_w4(const GemmArgs& a, GemmPlan& plan) {
     constexpr int kLds = In::kRing * (TILE + TILE) * In::kRow;  // all 160 KiB, or 128 KiB for two whole-line stages (64 KiB on 128 x 128 tiles)
     static LdsCap cap;
-    plan.add_kernel(gemm_mfma_tn_256_w4<In, Out, WGN, kBias, kRagged, TILE, AMAJ, BMAJ>, a, (unsigned)(a.tiles_m * a.tiles_n),
+    plan.add_kernel(gemm_mfma_tn_256_w4<In, Out, WGN, kBias, kRagged, TILE, AMAJ, BMAJ, kOps>, a, (unsigned)(a.tiles_m * a.tiles_n),
                     (unsigned)(a.split > 1 ? a.split : 1), 128 * WGN, kLds, &cap, TILE, TILE, In::kRow * In::SPS, In::kDt, Out::kDt,
-                    "gemm_mfma_tn_256_w4<%s,%s,waves=%d,bias=%d,ragged=%d,tile=%d,amaj=%d,bmaj=%d>", In::kName, Out::kName, 2 * WGN, (int)kBias, (int)kRagged,
-                    TILE, AMAJ, BMAJ);
+                    "gemm_mfma_tn_256_w4<%s,%s,waves=%d,bias=%d,ragged=%d,tile=%d,amaj=%d,bmaj=%d,ops=%d>", In::kName, Out::kName, 2 * WGN, (int)kBias, (int)kRagged,
+                    TILE, AMAJ, BMAJ, (int)kOps);
     return MOYE_OK;
 }
 
-// The instances live in three translation units (so that they compile side by side): gemm_mfma256w4.hip (the 256 x 256
-// tile with K-major operands), gemm_mfma256w4_majors.hip (operands that keep their M- / N-major form), gemm_mfma128w4.hip
-// (the 128 x 128 tile).
+// The instances live in four translation units (so that they compile side by side): gemm_mfma256w4.hip (the 256 x 256
+// tile with K-major operands), gemm_mfma256w4_majors.hip (operands that keep their M- / N-major form),
+// gemm_mfma256w4_ops.hip (an element-wise operation in the epilogue), gemm_mfma128w4.hip (the 128 x 128 tile).
 int32_t launch256_w4_majors_dispatch(int32_t in_dt, int32_t out_dt, const GemmArgs& a, GemmPlan& plan);
+int32_t launch256_w4_ops_dispatch(int32_t in_dt, int32_t out_dt, const GemmArgs& a, GemmPlan& plan);
 
 }  // namespace moye

@@ -41,7 +41,7 @@ constexpr int kGemmAMajorM = 0x100000;  // A has its unit stride along M, lda is
 constexpr int kGemmBMajorN = 0x200000;  // the same for B and N (the kernels' transposing fragment reads)
 constexpr int kGemmEpiRowX = 0x400000;  // the epilogue operand has unit stride along n and 16-byte aligned rows (or one row)
 constexpr int kGemmRagged = 0x800000;   // tiles reach beyond M, N or K (the guarded instances)
-constexpr int kGemmEpiAddVec = 0x1000000;  // the epilogue operation adds a one-per-column or one-per-row vector or a scalar
+constexpr int kGemmEpiLaneOp = 0x1000000;  // the epilogue operation (not a division) has a scalar, a one-per-column or a one-per-row operand, or none: a bias, a ReLU, a scale
 
 // UniversalFMA GEMM, any strides (gemm_universal.hip)
 struct UArgs {

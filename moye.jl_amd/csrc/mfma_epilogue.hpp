@@ -151,12 +151,12 @@ __device__ __forceinline__ void store_c_tile_general(const GemmArgs& p, const f3
 // decides; the hand-ordered kernel has no such instance and is never sent one).
 // kGuard: the tile may reach beyond M or N and D need not be 16-byte aligned: nothing is read or stored beyond them, a
 // piece of D that crosses N or does not start on a 16-byte boundary goes out element by element.
-// kAddVec: the call adds a vector or a scalar (GemmArgs::ep_op == MOYE_MAP_ADD with a one-per-column, one-per-row or
-// scalar operand: a bias): the lanes add it to their own accumulators here, with the same roundings as the general
-// epilogue, instead of sending the tile through it.
+// kLaneOp: the call's element-wise operation has a one-per-column, one-per-row or scalar operand or none, and is no
+// division (kGemmEpiLaneOp: a bias, a ReLU, a scale): the lanes apply it to their own accumulators here, with the same
+// roundings as the general epilogue, instead of sending the tile through it.
 // kNoC: the caller has no C (GemmArgs::C is null, checked on the host): nothing of C's two read paths is compiled in,
 // which frees their registers for instances that have few to spare.
-template <typename Out, int MI, int NI, bool kGuard = false, bool kAddVec = false, bool kNoC = false>
+template <typename Out, int MI, int NI, bool kGuard = false, bool kLaneOp = false, bool kNoC = false>
 __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&acc)[MI][NI], u32x4* smem, int wave,
                                              int lane, int64_t m_base, int64_t n_base) {
     typedef typename Out::type OutT;
@@ -195,9 +195,9 @@ __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&ac
         }
     }
     // a lane's columns are n_base + 16 j + 4 kq + 0..3: the operand values of a one-per-column vector, once for all rows
-    [[maybe_unused]] f32x4 xcol[kAddVec ? NI : 1];
-    [[maybe_unused]] const bool per_row = kAddVec && p.ep_x && p.ep_xn == 0;
-    if constexpr (kAddVec) {
+    [[maybe_unused]] f32x4 xcol[kLaneOp ? NI : 1];
+    [[maybe_unused]] const bool per_row = kLaneOp && p.ep_x && p.ep_xn == 0;
+    if constexpr (kLaneOp) {
 #pragma unroll
         for (int j = 0; j < NI; ++j)
 #pragma unroll
@@ -247,10 +247,23 @@ __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&ac
                         for (int e = 0; e < 4; ++e) v[e] = __fadd_rn(v[e], __fmul_rn(p.beta, c[e]));
                     }
                 }
-                if constexpr (kAddVec) {
+                if constexpr (kLaneOp) {
                     const float xrow = per_row ? epi_operand(p, m, 0) : 0.f;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) v[e] = __fadd_rn(v[e], per_row ? xrow : xcol[j][e]);
+                    switch (p.ep_op) {  // the same for every element: one branch per four values
+#define MOYE_LANE_CASE(OP)                                                                                          \
+    case OP:                                                                                                        \
+        _Pragma("unroll") for (int e = 0; e < 4; ++e) v[e] = epi_op(OP, v[e], per_row ? xrow : xcol[j][e]);        \
+        break;
+                        MOYE_LANE_CASE(MOYE_MAP_ADD)
+                        MOYE_LANE_CASE(MOYE_MAP_SUB)
+                        MOYE_LANE_CASE(MOYE_MAP_MUL)
+                        MOYE_LANE_CASE(MOYE_MAP_MAX)
+                        MOYE_LANE_CASE(MOYE_MAP_MIN)
+                        MOYE_LANE_CASE(MOYE_MAP_NEG)
+                        MOYE_LANE_CASE(MOYE_MAP_ABS)
+#undef MOYE_LANE_CASE
+                        default: break;
+                    }
                 }
 #pragma unroll
                 for (int e = 0; e < 4; ++e) dst[e] = Out::cvt(v[e]);

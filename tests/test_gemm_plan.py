@@ -65,11 +65,15 @@ def check_kernel_step(s, eb, ob):
         if not ragged:
             assert M % tm == 0 and N % tn == 0 and s["d16"] == 1 and (s["ldd"] * ob) % 16 == 0, s
         else:
-            assert s["C"] == "null" and s["op"] == 0 and "amaj=0" in name and "bmaj=0" in name, s
+            assert "amaj=0" in name and "bmaj=0" in name, s
+            assert "ops=1" in name or (s["C"] == "null" and s["op"] == 0), s
         if "bias=1" in name:
-            assert s["C"] == "null" and "add_vec" in flags and s["op"] == 1, s
+            assert s["C"] == "null" and "lane_op" in flags and s["op"] not in (0, _lib.MAP_DIV) and not ragged and eb == 2, s
+        elif "ops=1" in name:
+            assert "waves=8" in name and "tile=256" in name and "amaj=0" in name and "bmaj=0" in name and step_bytes == 128, s
+            assert name.split("<")[1].split(",")[0] in ("W4F16L", "W4BF16L", "W4FP8L", "W4F32L"), s
         else:
-            assert s["op"] == 0, s                       # no element-wise operation in this kernel's epilogue
+            assert s["op"] == 0, s                       # the other instances have no element-wise operation
         if "amaj=1" in name or "bmaj=1" in name:
             assert "tile=256" in name and "waves=8" in name and not ragged, s
     elif fam in ("gemm_mfma_tn_256", "gemm_mfma_tn_128"):
@@ -84,7 +88,7 @@ def check_kernel_step(s, eb, ob):
         if s["op"] != 0 and "bias=1" not in name:
             assert "ops=1" in name, s
         if "bias=1" in name:
-            assert "add_vec" in flags and s["op"] == 1, s
+            assert "lane_op" in flags and s["op"] not in (0, _lib.MAP_DIV), s
     elif fam in ("gemm_mfma_tn_256_ring", "gemm_mfma_tn_256_pp"):
         assert M % 256 == 0 and N % 256 == 0 and kb % 64 == 0 and s["d16"] == 1 and s["op"] == 0 and not ragged, s
     elif fam == "gemm_mfma_tn":
@@ -247,17 +251,17 @@ def test_known_shapes_run_on_the_instances_they_are_meant_for():
     f16, bf16, f8, f32 = mh.F16, mh.BF16, mh.F8E4M3, mh.F32
     # the headline: fp16 4096^3 on the hand-ordered whole-line kernel, one launch of 256 workgroups
     p = run_case(f16, f16, 4096, 4096, 4096, cta=(256, 256, 64))
-    assert step_names(p) == ["gemm_mfma_tn_256_w4<W4F16L,OutF16,waves=8,bias=0,ragged=0,tile=256,amaj=0,bmaj=0>"]
+    assert step_names(p) == ["gemm_mfma_tn_256_w4<W4F16L,OutF16,waves=8,bias=0,ragged=0,tile=256,amaj=0,bmaj=0,ops=0>"]
     assert p["steps"][0]["grid"] == "256x1" and {"hand_ordered", "stream_d", "xcd_order"} <= p["steps"][0]["flags"] and "rotate_k" not in p["steps"][0]["flags"]
     # the same left to the library
     assert step_names(run_case(f16, f16, 4096, 4096, 4096)) == step_names(p)
     # bf16 8192^3 fp32 out, fp8 8192^3 bf16 out, fp32 8192^3: the same kernel's other operand types; K rotation on
     p = run_case(bf16, f32, 8192, 8192, 8192, cta=(256, 256, 64))
-    assert step_names(p) == ["gemm_mfma_tn_256_w4<W4BF16L,OutF32,waves=8,bias=0,ragged=0,tile=256,amaj=0,bmaj=0>"] and "rotate_k" in p["steps"][0]["flags"]
+    assert step_names(p) == ["gemm_mfma_tn_256_w4<W4BF16L,OutF32,waves=8,bias=0,ragged=0,tile=256,amaj=0,bmaj=0,ops=0>"] and "rotate_k" in p["steps"][0]["flags"]
     p = run_case(f8, bf16, 8192, 8192, 8192, cta=(256, 256, 128))
-    assert step_names(p) == ["gemm_mfma_tn_256_w4<W4FP8L,OutBF16,waves=8,bias=0,ragged=0,tile=256,amaj=0,bmaj=0>"]
+    assert step_names(p) == ["gemm_mfma_tn_256_w4<W4FP8L,OutBF16,waves=8,bias=0,ragged=0,tile=256,amaj=0,bmaj=0,ops=0>"]
     p = run_case(f32, f32, 8192, 8192, 8192, cta=(256, 256, 32))
-    assert step_names(p) == ["gemm_mfma_tn_256_w4<W4F32L,OutF32,waves=8,bias=0,ragged=0,tile=256,amaj=0,bmaj=0>"]
+    assert step_names(p) == ["gemm_mfma_tn_256_w4<W4F32L,OutF32,waves=8,bias=0,ragged=0,tile=256,amaj=0,bmaj=0,ops=0>"]
     # the reference's own operand layout (A M-major, B N-major) needs no workspace for any operand type
     for dt, bk in ((f16, 64), (bf16, 64), (f8, 128), (f32, 32)):
         p = run_case(dt, f32, 4096, 4096, 4096, cta=(256, 256, bk), a_major="m", b_major="n", flags=_lib.GEMM_NO_WORKSPACE)
@@ -271,11 +275,28 @@ def test_known_shapes_run_on_the_instances_they_are_meant_for():
     # small N and a long K: the library's own K ranges for the line kernel, then the reduction
     p = run_case(bf16, f32, 16, 1024, 32768, split_k=-1)
     assert p["steps"][0]["family"] == "gemm_mfma_skinny_lds" and p["steps"][0]["split"] == 4 and p["steps"][-1]["what"] == "splitk_reduce"
-    # ragged problems: the guarded form of the hand-ordered kernel (no C, K of whole lines), the compiler-scheduled one otherwise
+    # ragged problems: the guarded forms of the hand-ordered kernel (K of whole lines; with a C the instance whose
+    # epilogue is the general one), the compiler-scheduled one for a K tail
     assert "ragged=1" in step_names(run_case(f16, f16, 4000, 4000, 4096))[0] and step_names(run_case(f16, f16, 4000, 4000, 4096))[0].startswith("gemm_mfma_tn_256_w4<W4F16L")
     assert step_names(run_case(f16, f16, 4096, 4096, 4000))[0].startswith("gemm_mfma_tn_256<InF16,OutF16,waves=8,ops=0,amaj=0,bmaj=0,ragged=1")
-    assert step_names(run_case(f16, f16, 4000, 4000, 4096, with_c=True))[0].startswith("gemm_mfma_tn_256<InF16,OutF16,waves=8,ops=0,amaj=0,bmaj=0,ragged=1")
-    assert step_names(run_case(f8, bf16, 4000, 4000, 4096))[0].startswith("gemm_mfma_tn_256_w4<W4FP8L,OutBF16,waves=8,bias=0,ragged=1")
+    assert step_names(run_case(f16, f16, 4000, 4000, 4096, with_c=True))[0] == "gemm_mfma_tn_256_w4<W4F16L,OutF16,waves=8,bias=0,ragged=1,tile=256,amaj=0,bmaj=0,ops=1>"
+    # an element-wise operation with a whole-matrix operand: the same k-loop with the general epilogue, every operand type
+    # (fp8 keeps its 16x16x128 MFMA)
+    def gate(m, n):
+        return mh.gemm_epilogue(alpha=0.5, op=_lib.MAP_MUL, operand=tensor(PX, f32, (m, n), (n, 1)))
+    assert step_names(run_case(f16, f16, 4096, 4096, 4096, ep=gate(4096, 4096)))[0] == "gemm_mfma_tn_256_w4<W4F16L,OutF16,waves=8,bias=0,ragged=0,tile=256,amaj=0,bmaj=0,ops=1>"
+    assert step_names(run_case(f8, bf16, 8192, 8192, 8192, ep=gate(8192, 8192)))[0] == "gemm_mfma_tn_256_w4<W4FP8L,OutBF16,waves=8,bias=0,ragged=0,tile=256,amaj=0,bmaj=0,ops=1>"
+    assert step_names(run_case(f32, f32, 4096, 4096, 4096, ep=gate(4096, 4096)))[0] == "gemm_mfma_tn_256_w4<W4F32L,OutF32,waves=8,bias=0,ragged=0,tile=256,amaj=0,bmaj=0,ops=1>"
+    assert step_names(run_case(f16, f16, 4096, 4096, 4096, ep=gate(4096, 4096), a_major="m"))[0].startswith("gemm_mfma_tn_256<InF16,OutF16,waves=8,ops=1,amaj=1")
+    # a ReLU, a scale, a bias (a scalar, one-per-column or one-per-row operand): applied in the lanes' own epilogue; the
+    # hand-ordered kernel has that form for the 16-bit types without C, the compiler-scheduled one with C; fp8 and fp32
+    # operands take the hand-ordered kernel's general epilogue
+    relu = mh.gemm_epilogue(alpha=0.5, op=_lib.MAP_MAX, scalar=0.0)
+    assert step_names(run_case(f16, f16, 4096, 4096, 4096, ep=relu))[0] == "gemm_mfma_tn_256_w4<W4F16L,OutF16,waves=8,bias=1,ragged=0,tile=256,amaj=0,bmaj=0,ops=0>"
+    relu_c = mh.gemm_epilogue(alpha=0.5, beta=1.0, op=_lib.MAP_MAX, scalar=0.0)
+    assert step_names(run_case(f16, f16, 4096, 4096, 4096, ep=relu_c, with_c=True))[0].startswith("gemm_mfma_tn_256<InF16,OutF16,waves=8,ops=0,amaj=0,bmaj=0,ragged=0,bias=1")
+    assert step_names(run_case(f8, bf16, 8192, 8192, 8192, ep=relu))[0] == "gemm_mfma_tn_256_w4<W4FP8L,OutBF16,waves=8,bias=0,ragged=0,tile=256,amaj=0,bmaj=0,ops=1>"
+    assert "ops=1" in step_names(run_case(f16, f16, 4096, 4096, 4096, ep=mh.gemm_epilogue(op=_lib.MAP_DIV, scalar=3.0)))[0]
     # thin fringes: whole tiles for the interior, the short-M kernel for each fringe (the right-hand one transposed)
     p = run_case(f16, f16, 4100, 4104, 4096)
     fams = [s["family"] for s in p["steps"]]
@@ -285,7 +306,7 @@ def test_known_shapes_run_on_the_instances_they_are_meant_for():
     p = run_case(f16, f16, 6144, 6144, 6144, waves=(1, 1, 1))
     assert [s["name"].split(",")[5] for s in p["steps"]] == ["tile=256", "tile=128"] and p["steps"][0]["M"] + p["steps"][1]["M"] == 6144
     assert len(run_case(f16, f16, 5120, 5120, 5120, waves=(1, 1, 1))["steps"]) == 1
-    # a bias row in the epilogue: the bias instance of the hand-ordered kernel; with C as well, the compiler-scheduled one
+    # a bias row in the epilogue: the bias instance of the hand-ordered kernel
     bias = mh.gemm_epilogue(alpha=1.0, op=_lib.MAP_ADD, operand=tensor(PX, f32, (4096, 4096), (0, 1)))
     assert "bias=1" in step_names(run_case(f16, f16, 4096, 4096, 4096, cta=(256, 256, 64), ep=bias))[0]
     assert step_names(run_case(f16, f16, 4096, 4096, 4096, cta=(256, 256, 64), ep=bias))[0].startswith("gemm_mfma_tn_256_w4")
@@ -311,7 +332,7 @@ def test_every_branch_of_the_dispatcher_is_reached():
         pytest.skip("the enumerating tests did not run in this process")
     want = {"gemm_mfma_tn_256_w4", "gemm_mfma_tn_256", "gemm_mfma_tn_128", "gemm_mfma_tn", "gemm_mfma_tn_256_ring", "gemm_mfma_tn_256_pp",
             "gemm_mfma_skinny_lds", "kmajor_copy", "splitk_reduce",
-            "gemm_mfma_tn_256_w4:ragged=1", "gemm_mfma_tn_256_w4:bias=1", "gemm_mfma_tn_256_w4:amaj=1", "gemm_mfma_tn_256_w4:bmaj=1",
+            "gemm_mfma_tn_256_w4:ragged=1", "gemm_mfma_tn_256_w4:bias=1", "gemm_mfma_tn_256_w4:ops=1", "gemm_mfma_tn_256_w4:amaj=1", "gemm_mfma_tn_256_w4:bmaj=1",
             "gemm_mfma_tn_256_w4:tile=128", "gemm_mfma_tn_256:ragged=1", "gemm_mfma_tn_256:ops=1", "gemm_mfma_tn_256:bias=1",
             "gemm_mfma_tn_256:amaj=1", "gemm_mfma_tn_128:ragged=1", "gemm_mfma_tn_128:ops=1", "gemm_mfma_tn_128:amaj=1", "gemm_mfma_tn_128:bias=1",
             "gemm_mfma_tn:edge=1", "gemm_mfma_tn:atom=32"}

@@ -831,11 +831,10 @@ def test_ragged_256_tiles_exact_on_integers(mh, case):
             # one row and one column beyond whole tiles: the interior on whole 256 x 256 tiles, each fringe on the short-M kernel
             assert [k["family"] for k in ks] == ["gemm_mfma_tn_256_w4", "gemm_mfma_skinny_lds", "gemm_mfma_skinny_lds"] and "ragged=0" in ks[0]["name"], ks
         if case in ((4000, 4000, 4096), (5000, 3000, 4096)):
-            # at least 128 ragged 256 x 256 tiles, K of whole 128-byte rows: without C the guarded form of the hand-ordered
-            # kernel, with C that of the compiler-scheduled one (fp8: the hand-ordered kernel has its only guarded form)
-            assert ks[0]["family"] == "gemm_mfma_tn_256_w4" and "ragged=1" in ks[0]["name"] and "tile=256" in ks[0]["name"], ks
-            if in_dt != torch.float8_e4m3fn:
-                assert kc[0]["family"] == "gemm_mfma_tn_256" and "ragged=1" in kc[0]["name"], kc
+            # at least 128 ragged 256 x 256 tiles, K of whole 128-byte rows: the guarded forms of the hand-ordered kernel,
+            # with C the one whose epilogue is the general one
+            assert ks[0]["family"] == "gemm_mfma_tn_256_w4" and "ragged=1" in ks[0]["name"] and "tile=256" in ks[0]["name"] and "ops=0" in ks[0]["name"], ks
+            assert kc[0]["family"] == "gemm_mfma_tn_256_w4" and "ragged=1" in kc[0]["name"] and "ops=1" in kc[0]["name"], kc
         if case == (2100, 2900, 4096):     # fewer than 128 tiles of 256 x 256: the hand-ordered kernel's guarded 128 x 128 instance
             assert ks[0]["family"] == "gemm_mfma_tn_256_w4" and "ragged=1" in ks[0]["name"] and "tile=128" in ks[0]["name"], ks
         if case == (4099, 2050, 4096 + 8) and b16:     # a K tail on 256 x 256 tiles: the compiler-scheduled kernel's guarded instance masks it
@@ -1725,14 +1724,14 @@ _NP_OF = {"float32": ("f32", np.float32), "float16": ("f16", np.float16), "bfloa
 
 
 def _epilogue_case(mh, mma, M, N, K, out_name, op, operand_kind, seed, col_major_d=False, alpha=0.375, beta=-1.25,
-                   operand_in_out_type=False):
+                   operand_in_out_type=False, in_dt=torch.float16, instance=None):
     """Small-integer A and B (the fp32 accumulator is exact whatever the order of the sum), random C and operand:
     every bit of D is then fixed by the epilogue's arithmetic, which the oracle composes from axpby! and broadcast."""
     out_dt = getattr(torch, out_name)
     tag, _ = _NP_OF[out_name]
     g = torch.Generator().manual_seed(seed)
-    A = torch.randint(-3, 4, (M, K), generator=g).to(torch.float16)
-    B = torch.randint(-3, 4, (N, K), generator=g).to(torch.float16)
+    A = torch.randint(-3, 4, (M, K), generator=g).float().to(in_dt)
+    B = torch.randint(-3, 4, (N, K), generator=g).float().to(in_dt)
     C0 = torch.randn(M, N, generator=g).to(out_dt)
     x_dt = out_dt if operand_in_out_type else torch.float32
     if operand_kind == "row":        # one value per column n, repeated down the rows: (M,N):(0,1)
@@ -1759,6 +1758,9 @@ def _epilogue_case(mh, mma, M, N, K, out_name, op, operand_kind, seed, col_major
         td = T(d)
     need = mh.gemm_workspace_size(mma, td, T(a), T(b))
     ws = torch.zeros(max(need, 1) + 256, dtype=torch.uint8, device="cuda")
+    if instance is not None:      # the test means one kernel instance: the plan must say so
+        ks = kernels_of(mh, mma, td, T(a), T(b), T(c) if beta != 0 else None, ep)
+        assert len(ks) == 1 and all(part in ks[0]["name"] for part in instance), (instance, ks)
     mh.gemm_ex_(mma, td, T(a), T(b), T(c) if beta != 0 else None, ep, (ws.data_ptr() + 255) // 256 * 256, need)
     torch.cuda.synchronize()
     got = (d.t() if col_major_d else d).cpu()
@@ -1833,6 +1835,37 @@ def test_fused_epilogue_every_kernel_and_operand(mh, kernel, operand_kind):
                            operand_in_out_type=in_out_type)
 
 
+@pytest.mark.parametrize("in_name,atom,out_name,K", [("float16", "MFMA_F32_16x16x32_F16", "float16", 128), ("bfloat16", "MFMA_F32_16x16x32_BF16", "float32", 192),
+                                                     ("float8_e4m3fn", "MFMA_F32_16x16x32_FP8", "bfloat16", 256), ("float32", "MFMA_F32_16x16x4_F32", "float32", 64)])
+def test_fused_epilogue_on_the_hand_ordered_kernel(mh, in_name, atom, out_name, K):
+    """The hand-ordered 256 x 256 kernel's two epilogue forms for every operand type.  An operation with a scalar, a
+    one-per-column or a one-per-row operand (a ReLU, a scale, a bias) and no C is applied in the lanes' own accumulators
+    (16-bit operands; every such operation, not only the addition); anything else -- a whole-matrix operand, a division,
+    fp8 and fp32 operands, a C on tiles that reach beyond M and N -- goes through the general epilogue behind the same
+    k-loop (fp8 so keeps its 16x16x128 MFMA).  Bit for bit against the oracle, whole and ragged tiles."""
+    in_dt = getattr(torch, in_name)
+    b16 = in_dt in (torch.float16, torch.bfloat16)
+    mma = mh.tiled_mma_desc(getattr(mh, atom), atom_layout=(2, 4, 1), cta_tile=(256, 256, 128 // in_dt.itemsize))
+    lanes = ("gemm_mfma_tn_256_w4", "bias=1", "ops=0") if b16 else ("gemm_mfma_tn_256_w4", "bias=0", "ops=1")
+    general = ("gemm_mfma_tn_256_w4", "bias=0", "ops=1", "ragged=0")
+    seed = 900 + K
+    for op, kind in (("max", "scalar"), ("mul", "row"), ("sub", "col"), ("min", "row"), ("abs", "scalar"), ("neg", "scalar")):
+        _epilogue_case(mh, mma, 512, 768, K, out_name, op, kind, seed, beta=0.0, in_dt=in_dt, instance=lanes)
+        seed += 1
+    for op, kind, beta in (("div", "row", 0.0), ("mul", "full", 0.0), ("add", "full", -1.25), ("max", "full", 0.5)):
+        _epilogue_case(mh, mma, 512, 768, K, out_name, op, kind, seed, beta=beta, in_dt=in_dt, instance=general)
+        seed += 1
+    if not b16:      # a ReLU with C: fp8 and fp32 operands stay on this kernel (the 16-bit types have the compiler-scheduled kernel's lane form)
+        _epilogue_case(mh, mma, 512, 768, K, out_name, "max", "scalar", seed, beta=0.5, in_dt=in_dt, instance=general)
+    # tiles that reach beyond M and N, the tile left to the library: with a C or an operation the guarded general epilogue
+    lib = mh.tiled_mma_desc(getattr(mh, atom), cta_tile=(0, 0, 0))
+    ragged = ("gemm_mfma_tn_256_w4", "ragged=1", "ops=1")
+    # (14 x 15 tiles; the row pitch of a 16-bit D is 8 bytes modulo 16; K long enough that the library takes these tiles)
+    M, N, Kr = 3400, 3604, {2: 1024, 1: 4096, 4: 256}[in_dt.itemsize]
+    _epilogue_case(mh, lib, M, N, Kr, out_name, "identity", "scalar", seed + 1, beta=-1.25, in_dt=in_dt, instance=ragged)
+    _epilogue_case(mh, lib, M, N, Kr, out_name, "max", "row", seed + 2, beta=0.0, in_dt=in_dt, instance=ragged, col_major_d=True)
+
+
 def test_fused_epilogue_limits(mh):
     """beta == 0 never reads C (NaNs in it do not reach D); moye_gemm is the beta == 1 case of moye_gemm_ex, bit for
     bit; what is not built says so."""
@@ -1863,8 +1896,8 @@ def test_fused_epilogue_limits(mh):
         with pytest.raises(mh.MoyeError) as e:
             mh.gemm_ex_(mma, T(d0), T(a), T(b), None, bad)
         assert e.value.status == status
-    with pytest.raises(mh.MoyeError) as e:       # the hand-ordered kernel has no such epilogue
-        mh.gemm_ex_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 4, 1), cta_tile=(256, 256, 64), flags=_lib.GEMM_WAVE4),
+    with pytest.raises(mh.MoyeError) as e:       # the hand-ordered kernel's four-wave schedule has no such epilogue
+        mh.gemm_ex_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 2, 1), cta_tile=(256, 256, 64), flags=_lib.GEMM_WAVE4),
                     T(d0), T(a), T(b), None, mh.gemm_epilogue(op=_lib.MAP_ABS))
     assert e.value.status == _lib.ERR_UNSUPPORTED
     af, bf = a.float(), b.float()

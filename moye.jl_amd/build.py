@@ -76,7 +76,7 @@ ASM_MFMA_SOURCES = ["gemm_mfma256w4.hip", "gemm_mfma256w4_majors.hip", "gemm_mfm
 def check_accumulator_hazards(src, force=False):
     """Compile `src` to assembly and fail if, in any basic block that holds v_mfma instructions, something
     other than a v_mfma names an AccVGPR before the kernel's `MOYE_ACC_SETTLED` marker, or something other than a
-    v_mfma or a fragment read (ds_read_b128, ds_read_b64_tr_b16) names a register that the fragment reads of such blocks
+    v_mfma or a fragment read (ds_read_b128, ds_read_b64_tr_b16, ds_read_b64_tr_b8, ds_read_b32) names a register that the fragment reads of such blocks
     write."""
     path = os.path.join(CSRC, src)
     asm = os.path.join(CSRC, "build", os.path.splitext(src)[0] + ".s")
@@ -94,6 +94,11 @@ def check_accumulator_hazards(src, force=False):
     if frag_bad:
         os.remove(asm)
         raise RuntimeError("fragment registers of inline-assembly LDS reads are touched between the MFMAs:\n" + "\n".join(frag_bad[:20]))
+
+
+# the LDS reads that fill MFMA operand fragments in these kernels: whole pieces, the transposing reads of M- / N-major
+# 16-bit and 8-bit operands, single values of M- / N-major fp32 operands
+FRAG_READ = re.compile(r"\s*ds_read_(?:b128|b64_tr_b16|b64_tr_b8|b32)\s+(v\[\d+:\d+\]|v\d+\b)")
 
 
 def asm_mfma_hazards(lines, name="asm"):
@@ -146,12 +151,12 @@ def asm_mfma_hazards(lines, name="asm"):
     for f, blk in mfma_blocks:
         for _, c in blk:
             code = c.split(";")[0]
-            m = re.match(r"\s*ds_read_(?:b128|b64_tr_b16)\s+(v\[\d+:\d+\])", code)
+            m = FRAG_READ.match(code)
             if m:
                 frags.setdefault(f, set()).update(vregs(m.group(1)))
     # Per block: a register counts as a fragment from the block's start (the reads of an earlier block or trip may still
-    # be in flight) until something other than a ds_read_b128 writes it (the fragment is dead then and the register has
-    # a new owner); a ds_read_b128 makes it one again.
+    # be in flight) until something other than a fragment read writes it (the fragment is dead then and the register has
+    # a new owner); a fragment read makes it one again.
     no_dest = re.compile(r"\s*(global_store|buffer_store|ds_write|global_load_lds|s_|v_cmp|v_readfirstlane|v_readlane)")
     for f, blk in mfma_blocks:
         pending = set(frags.get(f, set()))
@@ -161,7 +166,7 @@ def asm_mfma_hazards(lines, name="asm"):
             code = c.split(";")[0]
             if settled or not code.strip() or code.lstrip().startswith(".") or "v_mfma" in code:
                 continue
-            m = re.match(r"\s*ds_read_(?:b128|b64_tr_b16)\s+(v\[\d+:\d+\])", code)
+            m = FRAG_READ.match(code)
             if m:
                 pending |= vregs(m.group(1))
                 continue

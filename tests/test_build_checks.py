@@ -46,6 +46,15 @@ def test_a_copy_of_a_fragment_between_the_mfmas_is_caught():
     assert len(scan("\tglobal_store_dwordx4 v[2:3], v[10:13], off")[1]) == 1
 
 
+def test_the_fragment_reads_of_operands_that_are_not_k_major_count_too():
+    # the transposing reads (16-bit and 8-bit operands) and the single-value reads (fp32 operands) fill fragments as well
+    for read in ("ds_read_b64_tr_b16 v[40:41], v1 offset:64", "ds_read_b64_tr_b8 v[40:41], v1 offset:64", "ds_read_b32 v40, v1 offset:64"):
+        assert scan("\t" + read)[1] == []
+        acc, frag = scan("\t" + read + "\n\tv_mov_b32 v20, v40")
+        assert acc == [] and len(frag) == 1 and "v_mov_b32 v20, v40" in frag[0], read
+        assert scan("\t" + read + "\n\tv_mov_b32 v40, v2\n\tv_add_u32 v3, v40, v4")[1] == []
+
+
 def test_an_accumulator_named_by_anything_but_an_mfma_is_caught():
     acc, frag = scan("\tv_accvgpr_read_b32 v20, a2")
     assert len(acc) == 1 and "a2" in acc[0] and frag == []
@@ -54,4 +63,7 @@ def test_an_accumulator_named_by_anything_but_an_mfma_is_caught():
 
 def test_the_shipped_listing_is_checked_at_build_time():
     # build() runs the check for every source with inline-assembly MFMAs; the hand-ordered GEMM kernel is one
-    assert "gemm_mfma256w4.hip" in build.ASM_MFMA_SOURCES
+    with open(os.path.join(build.CSRC, "gemm_mfma_w4_kernel.hpp")) as f:
+        assert "v_mfma" in f.read()
+    users = [s for s in build.SOURCES if s.endswith(".hip") and "gemm_mfma_w4_kernel.hpp" in open(os.path.join(build.CSRC, s)).read()]
+    assert users and set(users) == set(build.ASM_MFMA_SOURCES)

@@ -578,7 +578,7 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
     }
     // The named tile 128 x 128 with 64 bytes of K per stage (128 x 128 x 32 for the 16-bit types: the tile the baseline's fp16
     // configuration names): plain f16 / bf16 calls on whole tiles, K a whole number of two-stage k-steps, run the
-    // hand-ordered kernel's ring of four such stages (fp16 4096^3 140-143 us against 161-171); the rest the register-staged kernel.
+    // hand-ordered kernel's ring of four such stages (fp16 4096^3 125-127 us against 161-171); the rest the register-staged kernel.
     if (bm == 128 && bn == 128 && bkb == 64 && eb == 2 && !misaligned && a.M % 128 == 0 && a.N % 128 == 0 && ((int64_t)a.K * eb) % 128 == 0 &&
         a.ep_op == MOYE_MAP_IDENTITY && stages < 2 && !(a.flags & (kGemmAMajorM | kGemmBMajorN | kGemmEpiLaneOp | kGemmAtom32 | kGemmRagged | MOYE_GEMM_PINGPONG)) &&
         row_offsets_fit(a, 128, eb))

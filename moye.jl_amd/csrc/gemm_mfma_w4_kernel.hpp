@@ -550,11 +550,17 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
             constexpr int dma_q = TILE == 128 ? dma_index_128(P, 2 * LD * SPS) : kLine ? dma_index_early(P, 2 * LD) : dma_index(P, 2 * LD * SPS, NPOS);
             if constexpr (dma_q >= 0) {
                 constexpr int q = dma_q;  // 0 .. 2 LD SPS - 1
+                // The 128 x 128 tile's k-steps of two 64-byte-row stages ask for the two halves of a 128-byte line one
+                // right after the other, so that the second finds the line in the L1 the first brought it into (a stage
+                // after the other, eight waves of two workgroups put 32 KiB between them: the L1's size); all loads of a
+                // k-step are waited for together there (the ring holds two k-steps), so their order is free.
+                constexpr bool kPairHalves = TILE == 128 && SPS == 2 && STAGES == 2 * SPS;
+                constexpr int q_stage = kPairHalves ? q % 2 : q / (2 * LD), q_instr = kPairHalves ? q / 2 : q % (2 * LD);
                 // in the drain a k-step of two stages may still have its first stage to request
-                if (AHEAD || g_new + q / (2 * LD) < nstages) {
-                    int sl = slot + q / (2 * LD);
+                if (AHEAD || g_new + q_stage < nstages) {
+                    int sl = slot + q_stage;
                     if (sl >= STAGES) sl -= STAGES;
-                    dma1(g_new + q / (2 * LD), sl, std::integral_constant<int, q % (2 * LD)>{});
+                    dma1(g_new + q_stage, sl, std::integral_constant<int, q_instr>{});
                 }
             }
             if (MORE) {

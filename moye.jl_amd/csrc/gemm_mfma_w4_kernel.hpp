@@ -166,8 +166,9 @@ struct W4BF16x2 : W4Ring64 {
     }
 };
 // ... in a ring of four stages, i.e. two k-steps: what the 128 x 128 tile named with 64 bytes of K per stage runs on (64 KiB,
-// two workgroups to a CU; fp16 4096^3, same box: 140-143 us, against 155-159 in a ring of five and 151-153 of six, one workgroup
-// to a CU, and 161-171 for the register-staged kernel)
+// two workgroups to a CU; fp16 4096^3: 125-127 us with the two halves of every 128-byte line requested back to back, 140-143
+// a stage after the other, on the same box as 155-159 in a ring of five and 151-153 of six, one workgroup to a CU, and
+// 161-171 for the register-staged kernel)
 struct W4F16x2R4 : W4F16x2 {
     static constexpr int kRing = 4;
     static constexpr const char* kName = "W4F16x2R4";

@@ -20,20 +20,32 @@ sys.path.insert(0, os.path.join(ROOT, "moye.jl_amd"))
 
 PEAK_F16_TFLOPS = 2500.0   # MI355X dense fp16/bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
-# Bytes that leave the L2s per launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script
-# (the summaries are committed under profiles/), each reading scaled by what the same counter shows for the
-# 1 GiB plain copy (fetch x2.0000, write x1.0000).  Only valid for the default tile/waves/flags.  These are figures
-# from the profiled sessions, not from the run that prints them (TRAFFIC_SOURCE goes into every roofline object);
-# where sessions differ (the 8192^3 GEMMs: how far the XCDs drift apart varies) the median session is quoted.
-TRAFFIC_SOURCE = "profiles/*_counters.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this script in earlier sessions; not measured in this run)"
+# Bytes that leave the L2s per launch: rows of the table "Traffic leaving the L2s per dispatch" in
+# profiles/gemm_f16_4096_and_transpose_f32_16384_counters.txt, copied as they stand there (kernel name, mean FETCH_SIZE
+# and mean WRITE_SIZE in KiB per dispatch, from one rocprofv3 --pmc run of this script each; tests/test_bench_traffic.py
+# holds the two against each other).  FETCH_SIZE is scaled by what the same counter shows for the 1 GiB plain copy of
+# that run (it reads half of what the copy moved: x2), WRITE_SIZE is left as read (x0.999).  Only valid for the default
+# tile/waves/flags.  These are figures of the profiled session, not of the run that prints them (TRAFFIC_SOURCE goes
+# into every roofline object); how far the XCDs drift apart varies between sessions and moves the 8192^3 figures by a
+# few percent.
+TRAFFIC_SOURCE = "profiles/gemm_f16_4096_and_transpose_f32_16384_counters.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this script in an earlier session; not measured in this run)"
+FETCH_SCALE = 2.0
+TRAFFIC_CALIBRATION = ("copy_flat_b128", 524294.5, 1049473.9)     # the 1 GiB plain copy of the same runs: 1048576 KiB each way
 MEASURED_TRAFFIC = {
-    "gemm_f16_4096_tile256": {"read_bytes": 196952 * 1024, "write_bytes": 32795 * 1024},
-    "transpose_f32_16384": {"read_bytes": 1048617 * 1024, "write_bytes": 1050175 * 1024},
-    "gemm_bf16_8192_tile256": {"read_bytes": 1581210 * 1024, "write_bytes": 262757 * 1024},
-    "gemm_f32_8192_tile256": {"read_bytes": 2 * 1611569 * 1024, "write_bytes": 262235 * 1024},
-    "gemm_fp8_8192_tile256": {"read_bytes": 787962 * 1024, "write_bytes": 131072 * 1024},
-    "gemm_bf16_16x8192x8192": {"read_bytes": 133216 * 1024, "write_bytes": 512 * 1024},
+    # key: (kernel as the profile names it, FETCH_SIZE KiB, WRITE_SIZE KiB)
+    "gemm_f16_4096_tile256": ("gemm_mfma_tn_256_w4<W4F16L, OutF16, 4, false, false, 256, 0, 0, false>", 98486.0, 32792.8),
+    "transpose_f32_16384": ("transpose_lds_b32_rows<4>", 524308.0, 1050126.2),
+    "gemm_bf16_8192_tile256": ("gemm_mfma_tn_256_w4<W4BF16L, OutF32, 4, false, false, 256, 0, 0, false>", 878095.6, 262462.0),
+    "gemm_f32_8192_tile256": ("gemm_mfma_tn_256_w4<W4F32L, OutF32, 4, false, false, 256, 0, 0, false>", 1667201.7, 262325.5),
+    "gemm_fp8_8192_tile256": ("gemm_mfma_tn_256_w4<W4FP8L, OutBF16, 4, false, false, 256, 0, 0, false>", 393736.9, 131072.0),
+    "gemm_bf16_16x8192x8192": ("gemm_mfma_skinny_lds<InBF16, OutF32, 1, 2, 4, 3, 2>", 66616.5, 512.0),
 }
+
+
+def traffic_bytes(key):
+    """HBM-side bytes per launch of the workload `key`: scaled fetch plus write, from the profiled session."""
+    _, fetch_kib, write_kib = MEASURED_TRAFFIC[key]
+    return int(round(fetch_kib * FETCH_SCALE * 1024)) + int(round(write_kib * 1024))
 
 
 def cpu_baseline(cores):
@@ -93,31 +105,34 @@ def headline_variants(mh, tensor_of, torch, stream, A, B, D):
     flops = 2.0 * 4096 ** 3
     tA, tB, tD = tensor_of(A), tensor_of(B), tensor_of(D)
 
-    def timed(name, fn, timer):
+    def timed(name, fn, timer, kernels):
         t_ramp = time.perf_counter()
         while time.perf_counter() - t_ramp < 0.2:
             for _ in range(20):
                 fn()
             torch.cuda.synchronize()
         ms = timer()
-        res.append({"workload": name, "kernel_ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 1),
+        res.append({"workload": name, "kernels": kernels, "kernel_ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 1),
                     "roofline": {"bound": "mfma", "achieved": round(flops / ms / 1e9, 1), "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
                                  "frac": round(flops / ms / 1e9 / PEAK_F16_TFLOPS, 4), "traffic": None}})
 
+    def names(mma, a, b, ep=None):
+        return [s_.get("name", s_["what"]) for s_ in mh.gemm_explain(mma, tD, a, b, None, ep)["steps"]]
+
     m128 = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 2, 1), tile=(128, 128, 32), cta_tile=(128, 128, 32))
-    timed("fp16 TN 4096^3 on the CTA tile config 3 names: 128x128x32, 2x2 waves",
+    timed("fp16 TN 4096^3 on the CTA tile config 3 names: 128x128x32, 2x2 waves (hand-ordered kernel, ring of four 128x32 stages, two workgroups per CU)",
           lambda: mh.gemm_(m128, tD, tA, tB, None, 1.0, stream),
-          lambda: mh.time_gemm(m128, tD, tA, tB, None, 1.0, stream, warmup=3, iters=50))
+          lambda: mh.time_gemm(m128, tD, tA, tB, None, 1.0, stream, warmup=3, iters=50), names(m128, tA, tB))
     m128l = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 2, 1), tile=(128, 128, 64), cta_tile=(128, 128, 64))
     timed("fp16 TN 4096^3 on 128x128x64 tiles, 2x2 waves, hand-ordered whole-line kernel (two workgroups per CU)",
           lambda: mh.gemm_(m128l, tD, tA, tB, None, 1.0, stream),
-          lambda: mh.time_gemm(m128l, tD, tA, tB, None, 1.0, stream, warmup=3, iters=50))
+          lambda: mh.time_gemm(m128l, tD, tA, tB, None, 1.0, stream, warmup=3, iters=50), names(m128l, tA, tB))
     m256 = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 4, 1), cta_tile=(256, 256, 64), flags=_lib.GEMM_NO_WORKSPACE)
     At, Bt = A.t().contiguous(), B.t().contiguous()
     tAm, tBn = tensor_of(At, (4096, 4096), (1, 4096)), tensor_of(Bt, (4096, 4096), (1, 4096))
-    timed("fp16 NN 4096^3 (A M-major, B N-major, no K-major copies), CTA 256x256x64",
+    timed("fp16 NN 4096^3 (A M-major, B N-major, read where they lie: transposing LDS fragment reads of the hand-ordered kernel), CTA 256x256x64",
           lambda: mh.gemm_(m256, tD, tAm, tBn, None, 1.0, stream),
-          lambda: mh.time_gemm(m256, tD, tAm, tBn, None, 1.0, stream, warmup=3, iters=50))
+          lambda: mh.time_gemm(m256, tD, tAm, tBn, None, 1.0, stream, warmup=3, iters=50), names(m256, tAm, tBn))
     bias = torch.randn(4096, device="cuda")
     ep = mh.gemm_epilogue(alpha=1.0, beta=0.0, op=_lib.MAP_ADD, operand=tensor_of(bias, (4096, 4096), (0, 1)))
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -130,7 +145,7 @@ def headline_variants(mh, tensor_of, torch, stream, A, B, D):
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / 50
     timed("fp16 TN 4096^3 with a bias row added in the epilogue (moye_gemm_ex), CTA 256x256x64",
-          lambda: mh.gemm_ex_(m256, tD, tA, tB, None, ep, None, 0, stream), ev)
+          lambda: mh.gemm_ex_(m256, tD, tA, tB, None, ep, None, 0, stream), ev, names(m256, tA, tB, ep))
     mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 4, 1), cta_tile=(256, 256, 64)), tD, tA, tB, None, 1.0, stream)
     torch.cuda.synchronize()
     return res
@@ -155,11 +170,12 @@ def other_configs(mh, tensor_of, torch, stream):
             alpha * (a[rows].float().double() @ b.float().double().t())
         err = float((d[rows].double() - c64).abs().max() / c64.abs().max())
         flops = 2.0 * M * N * K
-        entry = {"workload": name, "kernel_ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 1), "rel_err_vs_fp64": err}
+        entry = {"workload": name, "kernels": [s_.get("name", s_["what"]) for s_ in mh.gemm_explain(mma, tensor_of(d), tensor_of(a), tensor_of(b))["steps"]],
+                 "kernel_ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 1), "rel_err_vs_fp64": err}
         if peak:
             entry["roofline"] = {"bound": "mfma", "achieved": entry["tflops"], "peak": peak, "unit": "TFLOP/s",
                                  "frac": round(entry["tflops"] / peak, 4),
-                                 "traffic": sum(MEASURED_TRAFFIC[traffic_key].values()) if traffic_key else None,
+                                 "traffic": traffic_bytes(traffic_key) if traffic_key else None,
                                  "traffic_source": TRAFFIC_SOURCE if traffic_key else None}
         else:
             nbytes = a.numel() * a.element_size() + b.numel() * b.element_size() + d.numel() * d.element_size()
@@ -200,11 +216,11 @@ def other_configs(mh, tensor_of, torch, stream):
     nbytes = 16 * n * 2 + n * n * 2 + 16 * n * 4
     c64 = a16.float().double() @ b.float().double().t()
     res.append({"workload": "bf16 TN 16x8192x8192, fp32 out (short-M kernel staging 128-byte lines through LDS, B rotated over 3 buffers)",
-                "kernel_ms": round(ms, 5), "tflops": round(2.0 * 16 * n * n / ms / 1e9, 1),
+                "kernels": [s_.get("name", s_["what"]) for s_ in mh.gemm_explain(mma, tD, tA, tBs[0])["steps"]], "kernel_ms": round(ms, 5), "tflops": round(2.0 * 16 * n * n / ms / 1e9, 1),
                 "rel_err_vs_fp64": float((d16.double() - c64).abs().max() / c64.abs().max()),
                 "roofline": {"bound": "hbm", "achieved": round(nbytes / ms / 1e6, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                              "frac": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4), "algorithmic_bytes": nbytes,
-                             "traffic": sum(MEASURED_TRAFFIC["gemm_bf16_16x8192x8192"].values()), "traffic_source": TRAFFIC_SOURCE}})
+                             "traffic": traffic_bytes("gemm_bf16_16x8192x8192"), "traffic_source": TRAFFIC_SOURCE}})
     del bs, a, b, d
     if hasattr(torch, "float8_e4m3fn"):
         x = torch.randn(n, n, generator=g, device="cuda")
@@ -330,8 +346,7 @@ def main():
         sys.exit("bench.py: result check failed, rel err %.3e" % err)
 
     default_cfg = (bm, bn, bk, wm, wn, args.stages, args.flags) == (256, 256, 64, 2, 4, 0, 0)
-    t = MEASURED_TRAFFIC["gemm_f16_4096_tile256"]
-    gemm_traffic = t["read_bytes"] + t["write_bytes"] if default_cfg else None
+    gemm_traffic = traffic_bytes("gemm_f16_4096_tile256") if default_cfg else None
     out = {
         "metric": "GEMM TFLOP/s (fp16 4096^3) + % MFMA peak; tiled-copy GB/s + % HBM peak",
         "value": round(value, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -339,7 +354,7 @@ def main():
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": "fp16 TN GEMM M=N=K=4096, A row-major (MxK), B col-major (KxN), fp32 accumulate, "
                                "fp16 out; CTA tile %dx%dx%d, %dx%d waves of v_mfma_f32_16x16x32_f16" % (bm, bn, bk, wm, wn),
-                   "rel_err_vs_fp64": err},
+                   "kernels": [s_.get("name", s_["what"]) for s_ in mh.gemm_explain(mma, tD, tA, tB)["steps"]], "rel_err_vs_fp64": err},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_F16_TFLOPS, 4), "traffic": gemm_traffic,
                      "traffic_source": TRAFFIC_SOURCE if gemm_traffic else None, "kernel_ms": round(kern_ms, 5)},
@@ -368,7 +383,7 @@ def main():
             "config": {"workload": "16384x16384 fp32 column-major -> row-major through 64x64 LDS tiles", "bit_exact_sample": ok},
             "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                          "frac": round(gbs / PEAK_HBM_GBS, 4),
-                         "traffic": sum(MEASURED_TRAFFIC["transpose_f32_16384"].values()), "traffic_source": TRAFFIC_SOURCE,
+                         "traffic": traffic_bytes("transpose_f32_16384"), "traffic_source": TRAFFIC_SOURCE,
                          "kernel_ms": round(cms, 5)},
             "plain_copy_gbs": round(nbytes / (pms * 1e-3) / 1e9, 1),
         }

@@ -506,9 +506,7 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         // against 754); a K tail stays with that kernel, and so does a call that asks for it: stages = 2 in the descriptor.
         // (operands that keep their M- / N-major form: its transposing fragment reads, eight waves, plain calls; fp16 4096^3 NN
         // against the compiler-scheduled kernel's: see the kernel's header)
-        // (an operation the lanes apply themselves, with a C: the compiler-scheduled kernel has that form, whose epilogue
-        // costs nothing extra, where this one's general epilogue costs 11 us per round of tiles)
-        if (eb == 2 && bkb == 128 && stages < 2 && ops_fit && !((a.flags & kGemmEpiLaneOp) && a.C) &&
+        if (eb == 2 && bkb == 128 && stages < 2 && ops_fit &&
             (!majors256 || (waves != 4 && !(a.flags & kGemmEpiLaneOp))) &&
             !(a.flags & (MOYE_GEMM_PINGPONG | kGemmRagged | kGemmAtom32)) && row_offsets_fit(a, 256, eb))
             a.flags |= MOYE_GEMM_WAVE4;

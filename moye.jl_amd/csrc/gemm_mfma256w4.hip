@@ -1,4 +1,4 @@
-// The hand-ordered kernel (gemm_mfma_w4_kernel.hpp) on the 256 x 256 tile with K-major operands: plain, bias and guarded
+// The hand-ordered kernel (gemm_mfma_w4_kernel.hpp) on the 256 x 256 tile with K-major operands: plain and guarded
 // instances of every operand type and schedule (those with an element-wise operation: gemm_mfma256w4_ops.hip).
 #include "gemm_mfma_w4_kernel.hpp"
 
@@ -15,11 +15,9 @@ static int32_t launch256_w4_out(int32_t out_dt, const GemmArgs& a, GemmPlan& pla
             return fail(MOYE_ERR_UNSUPPORTED, "gemm!: this schedule of the hand-ordered kernel takes K-major operands only");
         }
     }
-    // An element-wise operation, or a C on ragged tiles: the instances whose epilogue is the general one (an operation
-    // with a scalar, one-per-column or one-per-row operand on whole tiles of the 16-bit types without C has its own form
-    // below: applied in the lanes' own accumulators)
-    const bool bias_form = (a.flags & kGemmEpiLaneOp) && !a.C && !(a.flags & kGemmRagged) && In::kBytes == 2;
-    if ((a.ep_op != MOYE_MAP_IDENTITY && !bias_form) || ((a.flags & kGemmRagged) && a.C)) {
+    // An element-wise operation, or a C on ragged tiles: gemm_mfma256w4_ops.hip (the operation in the lanes' own epilogue
+    // where its operand is a scalar, one per column or one per row and the tiles are whole; the general epilogue otherwise)
+    if (a.ep_op != MOYE_MAP_IDENTITY || ((a.flags & kGemmRagged) && a.C)) {
         if constexpr (In::kRow == 128 && WGN == 4)
             return launch256_w4_ops_dispatch(In::kDt, out_dt, a, plan);
         else
@@ -35,18 +33,6 @@ static int32_t launch256_w4_out(int32_t out_dt, const GemmArgs& a, GemmPlan& pla
             }
         } else {
             return fail(MOYE_ERR_UNSUPPORTED, "gemm!: this schedule of the hand-ordered kernel takes whole tiles only");
-        }
-    }
-    if (bias_form) {  // a bias, a ReLU, a scale: the eight-wave whole-line forms of the 16-bit types carry it, for calls without C
-        if constexpr (In::kRow == 128 && In::kBytes == 2 && WGN == 4) {
-            switch (out_dt) {
-                case MOYE_F32: return launch256_w4<In, OutF32, WGN, true>(a, plan);
-                case MOYE_F16: return launch256_w4<In, OutF16, WGN, true>(a, plan);
-                case MOYE_BF16: return launch256_w4<In, OutBF16, WGN, true>(a, plan);
-                default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: MFMA kernels write f32, f16 or bf16, not %s", dtype_name(out_dt));
-            }
-        } else {
-            return fail(MOYE_ERR_UNSUPPORTED, "gemm!: this schedule of the hand-ordered kernel takes no element-wise epilogue operation");
         }
     }
     switch (out_dt) {

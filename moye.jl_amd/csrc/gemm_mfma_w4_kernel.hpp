@@ -243,13 +243,13 @@ struct W4F32 : W4Ring64 {
 // two waves per SIMD, so that what stalls one wave's instruction stream (an M0 write, a taken branch,
 // the barrier) leaves the matrix pipe to the other.
 // kBias: the call's element-wise operation has a scalar, one-per-column or one-per-row operand (a bias, a ReLU, a scale:
-// kGemmEpiLaneOp) and the call has no C: the same kernel with that operation in the lanes' own epilogue (store_c_tile's
-// kLaneOp, without C's read paths, whose registers this kernel cannot spare: with them the epilogue spilled 96 registers).
+// kGemmEpiLaneOp): the same kernel with that operation in the lanes' own epilogue (store_c_tile's kLaneOp, which asks
+// for C one pass ahead only: with the plain form's four passes ahead the epilogue spilled 96 registers, so it spills 2-3).
 // kRagged: M and N need not be multiples of 256 (K stays a whole number of 128-byte rows): a lane whose row lies beyond
 // the operand reads the operand's last row instead (its constant lane offset is computed from the clamped row), what is
 // computed from it is never stored, and the epilogue runs with its row and column guards (a D that is not 16-byte
-// aligned goes out element by element where it must).  For calls without C, like the bias instance: the guards and C's
-// read paths together spilled 64-110 registers.
+// aligned goes out element by element where it must).  For calls without C (its epilogue is compiled without C's read
+// paths: with them and the guards it spilled 64-110 registers); a ragged call with C runs the kOps instance.
 // kOps: the epilogue is store_c_tile_general (any element-wise operation, any C, whole or ragged tiles): the raw
 // accumulators go through LDS 32 rows at a time and the arithmetic exists once, in a loop, which costs the 16-bit
 // outputs 9-20 spilled registers after the last MFMA and none before.  Whole-line stages, eight waves, K-major operands.
@@ -603,7 +603,7 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
     if constexpr (kOps)
         store_c_tile_general<Out, MI, NI, kRagged>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
     else
-        store_c_tile<Out, MI, NI, kRagged, kBias, kBias || kRagged>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
+        store_c_tile<Out, MI, NI, kRagged, kBias, kRagged>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
 }
 
 template <typename In, typename Out, int WGN, bool kBias = false, bool kRagged = false, int TILE = 256, int AMAJ = 0, int BMAJ = 0, bool kOps = false>

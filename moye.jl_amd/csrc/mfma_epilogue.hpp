@@ -172,7 +172,8 @@ __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&ac
     // pieces of the next AHEAD - 1 passes are already requested while a pass is worked on.  Any other C is read
     // element by element.
     constexpr int NCH = PASS_ROWS * CR / 64, PASSES = MI / PASS_MI;
-    constexpr int AHEAD = sizeof(OutT) == 2 ? PASSES : (PASSES < 2 ? PASSES : 2);
+    // (an instance that also applies an operation in the lanes has fewer registers to spare: one pass ahead)
+    constexpr int AHEAD = kLaneOp ? 1 : sizeof(OutT) == 2 ? PASSES : (PASSES < 2 ? PASSES : 2);
     // (ragged tiles read C in whole pieces only when no piece crosses N)
     const bool row_c = !kNoC && p.C && (p.flags & kGemmRowC) && (!kGuard || p.N % EPC == 0);
     [[maybe_unused]] u32x4 cw[kNoC ? 1 : AHEAD][NCH];

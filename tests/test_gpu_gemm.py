@@ -1839,24 +1839,25 @@ def test_fused_epilogue_every_kernel_and_operand(mh, kernel, operand_kind):
                                                      ("float8_e4m3fn", "MFMA_F32_16x16x32_FP8", "bfloat16", 256), ("float32", "MFMA_F32_16x16x4_F32", "float32", 64)])
 def test_fused_epilogue_on_the_hand_ordered_kernel(mh, in_name, atom, out_name, K):
     """The hand-ordered 256 x 256 kernel's two epilogue forms for every operand type.  An operation with a scalar, a
-    one-per-column or a one-per-row operand (a ReLU, a scale, a bias) and no C is applied in the lanes' own accumulators
-    (16-bit operands; every such operation, not only the addition); anything else -- a whole-matrix operand, a division,
-    fp8 and fp32 operands, a C on tiles that reach beyond M and N -- goes through the general epilogue behind the same
-    k-loop (fp8 so keeps its 16x16x128 MFMA).  Bit for bit against the oracle, whole and ragged tiles."""
+    one-per-column or a one-per-row operand (a ReLU, a scale, a bias), with or without C, is applied in the lanes' own
+    accumulators (every such operation, not only the addition); anything else -- a whole-matrix operand, a division, a C
+    or an operation on tiles that reach beyond M and N -- goes through the general epilogue behind the same k-loop (fp8
+    so keeps its 16x16x128 MFMA).  Bit for bit against the oracle, whole and ragged tiles."""
     in_dt = getattr(torch, in_name)
-    b16 = in_dt in (torch.float16, torch.bfloat16)
     mma = mh.tiled_mma_desc(getattr(mh, atom), atom_layout=(2, 4, 1), cta_tile=(256, 256, 128 // in_dt.itemsize))
-    lanes = ("gemm_mfma_tn_256_w4", "bias=1", "ops=0") if b16 else ("gemm_mfma_tn_256_w4", "bias=0", "ops=1")
+    lanes = ("gemm_mfma_tn_256_w4", "bias=1", "ops=0")
     general = ("gemm_mfma_tn_256_w4", "bias=0", "ops=1", "ragged=0")
     seed = 900 + K
-    for op, kind in (("max", "scalar"), ("mul", "row"), ("sub", "col"), ("min", "row"), ("abs", "scalar"), ("neg", "scalar")):
-        _epilogue_case(mh, mma, 512, 768, K, out_name, op, kind, seed, beta=0.0, in_dt=in_dt, instance=lanes)
+    for op, kind, beta in (("max", "scalar", 0.0), ("mul", "row", 0.0), ("sub", "col", -1.25), ("min", "row", 0.5), ("abs", "scalar", 0.0), ("neg", "scalar", 0.75),
+                           ("add", "col", 0.0), ("add", "row", -1.25)):
+        _epilogue_case(mh, mma, 512, 768, K, out_name, op, kind, seed, beta=beta, in_dt=in_dt, instance=lanes)
         seed += 1
+    # (a column-major D: the kernel runs the transposed problem, C and the operand are then read through their other stride)
+    _epilogue_case(mh, mma, 512, 768, K, out_name, "sub", "row", seed, beta=0.5, in_dt=in_dt, instance=lanes, col_major_d=True)
+    seed += 1
     for op, kind, beta in (("div", "row", 0.0), ("mul", "full", 0.0), ("add", "full", -1.25), ("max", "full", 0.5)):
         _epilogue_case(mh, mma, 512, 768, K, out_name, op, kind, seed, beta=beta, in_dt=in_dt, instance=general)
         seed += 1
-    if not b16:      # a ReLU with C: fp8 and fp32 operands stay on this kernel (the 16-bit types have the compiler-scheduled kernel's lane form)
-        _epilogue_case(mh, mma, 512, 768, K, out_name, "max", "scalar", seed, beta=0.5, in_dt=in_dt, instance=general)
     # tiles that reach beyond M and N, the tile left to the library: with a C or an operation the guarded general epilogue
     lib = mh.tiled_mma_desc(getattr(mh, atom), cta_tile=(0, 0, 0))
     ragged = ("gemm_mfma_tn_256_w4", "ragged=1", "ops=1")

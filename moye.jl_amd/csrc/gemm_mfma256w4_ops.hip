@@ -9,6 +9,14 @@ namespace moye {
 template <typename In>
 static int32_t launch256_w4_ops(int32_t out_dt, const GemmArgs& a, GemmPlan& plan) {
     if ((a.flags & kGemmEpiLaneOp) && !(a.flags & kGemmRagged)) {
+        if (!a.C) {  // (the form without C's read paths)
+            switch (out_dt) {
+                case MOYE_F32: return launch256_w4<In, OutF32, 4, true, false, 256, 0, 0, false, true>(a, plan);
+                case MOYE_F16: return launch256_w4<In, OutF16, 4, true, false, 256, 0, 0, false, true>(a, plan);
+                case MOYE_BF16: return launch256_w4<In, OutBF16, 4, true, false, 256, 0, 0, false, true>(a, plan);
+                default: return fail(MOYE_ERR_UNSUPPORTED, "gemm!: MFMA kernels write f32, f16 or bf16, not %s", dtype_name(out_dt));
+            }
+        }
         switch (out_dt) {
             case MOYE_F32: return launch256_w4<In, OutF32, 4, true>(a, plan);
             case MOYE_F16: return launch256_w4<In, OutF16, 4, true>(a, plan);

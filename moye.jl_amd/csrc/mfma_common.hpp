@@ -136,8 +136,14 @@ __device__ __forceinline__ float epi_op(int op, float x, float y) {
         case MOYE_MAP_SUB: return __fsub_rn(x, y);
         case MOYE_MAP_MUL: return __fmul_rn(x, y);
         case MOYE_MAP_DIV: return __fdiv_rn(x, y);
-        case MOYE_MAP_MAX: return ((y > x) | (signbit(y) < signbit(x))) ? (x != x ? x : y) : (y != y ? y : x);
-        case MOYE_MAP_MIN: return ((y < x) | (signbit(y) > signbit(x))) ? (x != x ? x : y) : (y != y ? y : x);
+        // v_max_f32 / v_min_f32 order the zeros as Julia does (-0.0 < +0.0) and differ from it only when an operand is a NaN:
+        // no lane of the wave has one (a wave-uniform test), and the instruction's result is the answer
+        case MOYE_MAP_MAX:
+            if (__builtin_amdgcn_ballot_w64((x != x) | (y != y)) == 0) return __builtin_fmaxf(x, y);
+            return ((y > x) | (signbit(y) < signbit(x))) ? (x != x ? x : y) : (y != y ? y : x);
+        case MOYE_MAP_MIN:
+            if (__builtin_amdgcn_ballot_w64((x != x) | (y != y)) == 0) return __builtin_fminf(x, y);
+            return ((y < x) | (signbit(y) > signbit(x))) ? (x != x ? x : y) : (y != y ? y : x);
         case MOYE_MAP_NEG: return -x;
         case MOYE_MAP_ABS: return signbit(x) ? -x : x;
         default: return x;

@@ -250,21 +250,29 @@ __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&ac
                 }
                 if constexpr (kLaneOp) {
                     const float xrow = per_row ? epi_operand(p, m, 0) : 0.f;
-                    switch (p.ep_op) {  // the same for every element: one branch per four values
-#define MOYE_LANE_CASE(OP)                                                                                          \
-    case OP:                                                                                                        \
-        _Pragma("unroll") for (int e = 0; e < 4; ++e) v[e] = epi_op(OP, v[e], per_row ? xrow : xcol[j][e]);        \
+                    // the same for every element: one uniform branch per four values; the addition (a bias) and the
+                    // maximum (a ReLU) are asked first, so that they pay one or two compares and not a chain of them
+#define MOYE_LANE_APPLY(OP) _Pragma("unroll") for (int e = 0; e < 4; ++e) v[e] = epi_op(OP, v[e], per_row ? xrow : xcol[j][e]);
+#define MOYE_LANE_CASE(OP) \
+    case OP:               \
+        MOYE_LANE_APPLY(OP) \
         break;
-                        MOYE_LANE_CASE(MOYE_MAP_ADD)
-                        MOYE_LANE_CASE(MOYE_MAP_SUB)
-                        MOYE_LANE_CASE(MOYE_MAP_MUL)
-                        MOYE_LANE_CASE(MOYE_MAP_MAX)
-                        MOYE_LANE_CASE(MOYE_MAP_MIN)
-                        MOYE_LANE_CASE(MOYE_MAP_NEG)
-                        MOYE_LANE_CASE(MOYE_MAP_ABS)
-#undef MOYE_LANE_CASE
-                        default: break;
+                    if (p.ep_op == MOYE_MAP_ADD) {
+                        MOYE_LANE_APPLY(MOYE_MAP_ADD)
+                    } else if (p.ep_op == MOYE_MAP_MAX) {
+                        MOYE_LANE_APPLY(MOYE_MAP_MAX)
+                    } else {
+                        switch (p.ep_op) {
+                            MOYE_LANE_CASE(MOYE_MAP_SUB)
+                            MOYE_LANE_CASE(MOYE_MAP_MUL)
+                            MOYE_LANE_CASE(MOYE_MAP_MIN)
+                            MOYE_LANE_CASE(MOYE_MAP_NEG)
+                            MOYE_LANE_CASE(MOYE_MAP_ABS)
+                            default: break;
+                        }
                     }
+#undef MOYE_LANE_CASE
+#undef MOYE_LANE_APPLY
                 }
 #pragma unroll
                 for (int e = 0; e < 4; ++e) dst[e] = Out::cvt(v[e]);

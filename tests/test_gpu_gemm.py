@@ -1867,6 +1867,48 @@ def test_fused_epilogue_on_the_hand_ordered_kernel(mh, in_name, atom, out_name, 
     _epilogue_case(mh, lib, M, N, Kr, out_name, "max", "row", seed + 2, beta=0.0, in_dt=in_dt, instance=ragged, col_major_d=True)
 
 
+@pytest.mark.parametrize("op", ["max", "min"])
+def test_fused_epilogue_max_min_follow_julia_on_nans_and_signed_zeros(mh, op):
+    """max / min in the epilogue: NaN if either argument is one, -0.0 below +0.0 (base/math.jl, as `moye_map`), through
+    the three places the operation is applied: the lanes' own epilogue, the general epilogue, and the second pass of a
+    split-K call.  The product is made +0, -0, NaN and ordinary values by rows (zero rows of A, a negative alpha, a NaN in
+    A), the operand carries the same set by columns; bit for bit against the oracle."""
+    from moye_hip import _lib
+    M, N, K = 256, 512, 128
+    g = torch.Generator().manual_seed(77)
+    A = torch.randint(-2, 3, (M, K), generator=g).to(torch.float16)
+    A[0::4] = 0                      # rows whose product is a zero; its sign is alpha's
+    A[1::16, 5] = float("nan")       # rows whose product is NaN
+    B = torch.randint(-2, 3, (N, K), generator=g).to(torch.float16)
+    B[:, 5] = 1
+    xs = torch.tensor([0.0, -0.0, float("nan"), 1.5, -1.5, float("inf"), -float("inf"), 3.0]).repeat(N // 8)
+    acc = A.float() @ B.float().t()
+    a, b, xd = A.cuda(), B.cuda(), xs.cuda()
+    full = xs[None, :].repeat(M, 1).contiguous()
+    fd = full.cuda()
+    seen = set()
+    for alpha in (1.0, -1.0):
+        for name, mma, operand, xnp in (
+                ("lanes", mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 4, 1), cta_tile=(256, 256, 64)), T(xd, (M, N), (0, 1)), xs.numpy()[None, :]),
+                ("general", mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 4, 1), cta_tile=(256, 256, 64)), T(fd), full.numpy()),
+                ("lanes 128", mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 2, 1), cta_tile=(128, 128, 64)), T(xd, (M, N), (0, 1)), xs.numpy()[None, :]),
+                ("split-K", mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 2, 1), cta_tile=(128, 128, 32), split_k=2), T(xd, (M, N), (0, 1)), xs.numpy()[None, :])):
+            ep = mh.gemm_epilogue(alpha=alpha, beta=0.0, op=_lib.MAP_OPS[op], operand=operand)
+            d = torch.zeros(M, N, dtype=torch.float32, device="cuda")
+            seen.update(k["name"] for k in kernels_of(mh, mma, T(d), T(a), T(b), None, ep))
+            need = mh.gemm_workspace_size(mma, T(d), T(a), T(b), ep)
+            ws = torch.zeros(need + 256, dtype=torch.uint8, device="cuda")
+            mh.gemm_ex_(mma, T(d), T(a), T(b), None, ep, (ws.data_ptr() + 255) // 256 * 256, need)
+            torch.cuda.synchronize()
+            want = to.gemm_epilogue(acc.numpy(), alpha, 0.0, None, op, xnp, 0.0, "f32")
+            gb, wb = d.cpu().numpy().view(np.uint32), want.astype(np.float32).view(np.uint32)
+            nan_both = np.isnan(d.cpu().numpy()) & np.isnan(want)
+            bad = np.argwhere((gb != wb) & ~nan_both)
+            assert bad.size == 0, (name, alpha, bad[:4], d.cpu().numpy()[tuple(bad[0])], want[tuple(bad[0])])
+            assert np.isnan(want).any() and (wb == 0x80000000).any() and (wb == 0).any()     # the cases are in the data
+    assert any("gemm_mfma_tn_256_w4" in k and "bias=1" in k for k in seen) and any("gemm_mfma_tn_256_w4" in k and "ops=1" in k for k in seen), seen
+
+
 def test_fused_epilogue_limits(mh):
     """beta == 0 never reads C (NaNs in it do not reach D); moye_gemm is the beta == 1 case of moye_gemm_ex, bit for
     bit; what is not built says so."""

@@ -372,15 +372,15 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
                                  (fr_m > 0 ? 4.5 + (double)(a.N + fr_m) * (double)k_bytes_all / 6.0e6 : 0.0);
         const bool thin = thin_shape && (int64_t)(M0 / 256) * (N0 / 256) >= cus / 4 &&
                           gemm_plan_cost_256(M0, N0, k_bytes_all, eb == 4, false, cus) + fringe_us <= choice.us;
-        // (fp8: only the hand-ordered kernel's guarded forms, i.e. K of whole 128-byte rows)
-        const bool hand_ordered_ragged = (eb == 2 || eb == 4 || in_dt == MOYE_F8E4M3) && ((int64_t)a.K * eb) % 128 == 0 &&
+        // (the hand-ordered kernel's guarded forms: K of whole 16-byte pieces)
+        const bool hand_ordered_ragged = (eb == 2 || eb == 4 || in_dt == MOYE_F8E4M3) && ((int64_t)a.K * eb) % 16 == 0 &&
                                          stages < 2 && row_offsets_fit(a, 256, eb);
         if ((!big || !aligned) && !thin && a.split <= 1 && bk_elems == 0 && aligned_ab && (in_dt != MOYE_F8E4M3 || hand_ordered_ragged) && ((int64_t)a.K * eb) % 16 == 0 &&
             prefer256 && stages < 3 && (waves <= 1 || waves == 8) &&
             !(a.flags & (MOYE_GEMM_WAVE4 | MOYE_GEMM_PINGPONG | kGemmAMajorM | kGemmBMajorN | kGemmAtom32))) {
             a.flags |= kGemmRagged;
-            // K of whole 128-byte rows: the hand-ordered kernel's guarded forms (rows clamped, no K tail to mask; with a C
-            // or an element-wise operation the instance whose epilogue is the general one)
+            // the hand-ordered kernel's guarded forms (rows clamped, a K tail masked in registers; with a C or an
+            // element-wise operation the instance whose epilogue is the general one)
             if (hand_ordered_ragged) return gemm_mfma_tn_256_w4_dispatch(in_dt, out_dt, a, 8, 128, false, plan);
             return gemm_mfma_tn_256_dispatch(in_dt, out_dt, a, 8, stages, plan);
         }
@@ -565,9 +565,9 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         if (whole) return gemm_mfma_tn_128_dispatch(in_dt, out_dt, a, plan);
         if (chosen_here || (a.flags & MOYE_GEMM_PREDICATE)) {
             a.flags |= kGemmRagged;
-            // (K of whole 128-byte rows, no C, no operation, more tiles than CUs: the guarded form of the hand-ordered instance)
+            // (no C, no operation, more tiles than CUs: the guarded form of the hand-ordered instance, which masks a K tail in registers)
             if ((int64_t)((a.M + 127) / 128) * ((a.N + 127) / 128) > (eb == 2 ? cus : 0) &&
-                (eb == 2 || eb == 4 || in_dt == MOYE_F8E4M3) && ((int64_t)a.K * eb) % 128 == 0 &&
+                (eb == 2 || eb == 4 || in_dt == MOYE_F8E4M3) && ((int64_t)a.K * eb) % 16 == 0 &&
                 a.ep_op == MOYE_MAP_IDENTITY && !a.C && stages < 2 && !(a.flags & (kGemmAMajorM | kGemmBMajorN | kGemmEpiLaneOp)) &&
                 row_offsets_fit(a, 128, eb))
                 return gemm_mfma_tn_128_w4_dispatch(in_dt, out_dt, a, plan);

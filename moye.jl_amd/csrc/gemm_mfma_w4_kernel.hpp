@@ -247,7 +247,7 @@ struct W4F32 : W4Ring64 {
 // for C one pass ahead only: with the plain form's four passes ahead the epilogue spilled 96 registers, so it spills 2-3).
 // kNoC: the call has no C (checked on the host): C's read paths are not compiled in (fp16 4096^3 with a bias row: +1.8 %
 // over the plain call, +4.2 % with the paths compiled in and not taken).
-// kRagged: M and N need not be multiples of 256 (K stays a whole number of 128-byte rows): a lane whose row lies beyond
+// kRagged: M and N need not be multiples of 256 and K only of 16 bytes (its tail: see tail_pieces): a lane whose row lies beyond
 // the operand reads the operand's last row instead (its constant lane offset is computed from the clamped row), what is
 // computed from it is never stored, and the epilogue runs with its row and column guards (a D that is not 16-byte
 // aligned goes out element by element where it must).  For calls without C (its epilogue is compiled without C's read
@@ -298,7 +298,7 @@ template <typename In, typename Out, int WGN, bool kBias = false, bool kRagged =
 __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_256_w4(GemmArgs p) {
     static_assert(!(AMAJ || BMAJ) || (In::kRow == 128 && TILE == 256 && WGN == 4 && !kBias && !kRagged),
                   "operands that are not K-major: whole-line stages, eight waves, plain whole tiles");
-    static_assert(!kRagged || (!kBias && In::kRow == 128), "ragged tiles: the plain whole-line form");
+    static_assert(!kRagged || (!kBias && In::kRow == 128 && !AMAJ && !BMAJ), "ragged tiles: the plain whole-line form, K-major operands");
     static_assert(!kOps || (In::kRow == 128 && TILE == 256 && WGN == 4 && !kBias && !AMAJ && !BMAJ), "epilogue operations: whole-line stages, eight waves, K-major operands");
     static_assert(TILE == 256 || (TILE == 128 && WGN == 2 && !kBias && (In::kRow == 128 || (In::SPS == 2 && !kRagged))),
                   "128 x 128 tiles: 2 x 2 waves; the whole-line form, plain or ragged, or the ring of 64-byte-row stages with k-steps of two stages");
@@ -349,7 +349,12 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
 #pragma unroll
         for (int j = 0; j < NI; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    const int nstages = (int)(((int64_t)p.K * In::kBytes) / kRow);
+    // Ragged instances also take a K that ends inside a 128-byte row (a whole number of 16-byte pieces): the last stage
+    // then holds tail_pieces valid pieces per row.  The lanes whose piece lies beyond K read the row's first piece of that
+    // stage instead (inside the operand), and every fragment half that lies beyond K is zeroed in registers before the
+    // last k-step's MFMAs (what was loaded there may be NaN or Inf, and must not reach an accumulator).
+    [[maybe_unused]] const int tail_pieces = kRagged ? (int)((((int64_t)p.K * In::kBytes) % kRow) / 16) : 0;  // 0: whole rows
+    const int nstages = (int)(((int64_t)p.K * In::kBytes + (kRagged ? kRow - 1 : 0)) / kRow);
     const int nsteps = nstages / SPS;
     frag_a fa[MI];
     frag_b fb[NI];
@@ -378,8 +383,11 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
         voff[q] = (uint32_t)(row * (q < LD ? pitch_a : pitch_b) + lch * 16);
     }
     // stage g of this workgroup's walk over K is stage g + g0 (mod nstages) of the operands: the eight XCDs start an
-    // eighth of K apart when the caller asks for it (see gemm_mfma256.hip)
-    const int g0 = (p.flags & kGemmRotateK) ? (int)((int64_t)(blockIdx.x % p.xcds) * nsteps / p.xcds) * SPS : 0;
+    // eighth of K apart when the caller asks for it (see gemm_mfma256.hip); not with a K tail, whose stage has to be
+    // the last in time as well
+    const int g0 = ((p.flags & kGemmRotateK) && !tail_pieces) ? (int)((int64_t)(blockIdx.x % p.xcds) * nsteps / p.xcds) * SPS : 0;
+    // what a lane whose piece lies beyond K in the last stage subtracts from its offset to land on the row's first piece
+    [[maybe_unused]] const uint32_t tail_cut = (kRagged && tail_pieces && lch >= tail_pieces) ? (uint32_t)lch * 16 : 0;
     auto dma1 = [&](int g, int ring_slot, auto qc) __attribute__((always_inline)) {
         constexpr int Q = decltype(qc)::value;
         const int gr = g + g0 >= nstages ? g + g0 - nstages : g + g0;
@@ -388,7 +396,8 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
                                                     : b_tile + (BMAJ ? (int64_t)gr * TKROWS * pitch_b : (int64_t)gr * kRow));
         const uint32_t dst = __builtin_amdgcn_readfirstlane(lds0 + ring_slot * kStageBytes + (Q < LD ? 0 : kATileBytes) +
                                                             (uint32_t)(wave * RW + RPI * (Q % LD)) * kRow);
-        const uint32_t lane_off = voff[Q];  // (a captured array element cannot be an asm operand of a generic lambda)
+        uint32_t lane_off = voff[Q];  // (a captured array element cannot be an asm operand of a generic lambda)
+        if constexpr (kRagged) lane_off -= gr == nstages - 1 ? tail_cut : 0u;  // (a uniform choice; tail_cut is zero without a tail)
         asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(base), "s"(dst)
                      : "memory");
     };
@@ -496,6 +505,27 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
     // 5 NI - 1, A5 after 6 NI - 1, B_j after 6 NI + 2 j + 1, rows 6 and 7 after 8 NI - 2 and 8 NI - 1.
     auto step = [&](auto more_c, auto ahead_c, int s) __attribute__((always_inline)) {
         constexpr bool MORE = decltype(more_c)::value, AHEAD = decltype(ahead_c)::value;
+        if constexpr (kRagged && !MORE) {
+            // the last k-step of a K that ends inside a row: the fragment halves beyond K become zeros (a lane's halves
+            // are pieces kq and kq + 4 of its row).  In a block of its own, after every fragment read has returned.
+            if (tail_pieces) {
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                const bool cut_lo = kq >= tail_pieces, cut_hi = kq + 4 >= tail_pieces;
+                auto cut = [&](auto& f) __attribute__((always_inline)) {
+                    // (only the two-piece fragments of the whole-line forms exist in ragged instances; the test keeps
+                    // the other instantiations of this lambda well-formed)
+                    if constexpr (std::is_class_v<std::remove_reference_t<decltype(f)>>) {
+                        const u32x4 zero = {0u, 0u, 0u, 0u};
+                        f.lo = cut_lo ? zero : f.lo;
+                        f.hi = cut_hi ? zero : f.hi;
+                    }
+                };
+#pragma unroll
+                for (int i = 0; i < MI; ++i) cut(fa[i]);
+#pragma unroll
+                for (int j = 0; j < NI; ++j) cut(fb[j]);
+            }
+        }
         int slot_n = slot + SPS;  // first stage of step s+1
         if (slot_n >= STAGES) slot_n -= STAGES;
         const uint32_t o0 = (uint32_t)slot_n * kStageBytes;

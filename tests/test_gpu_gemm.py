@@ -792,13 +792,14 @@ def test_last_round_on_its_own_launch_keeps_the_epilogue_operand_in_step(mh, sha
 @pytest.mark.parametrize("case", [(4000, 2200, 328), (3900, 2304, 120), (4096, 2048, 72), (4090, 2203, 40), (2100, 4100, 200),
                                   (4099, 2050, 4096 + 8), (4096, 2048, 128), (1000, 600, 136), (384, 256, 128), (130, 2000, 72),
                                   (4000, 2200, 192), (3841, 2305, 4096), (4100, 2052, 4096),
-                                  (3000, 2000, 192), (2100, 2900, 4096), (4000, 4000, 4096), (5000, 3000, 4096)])
+                                  (3000, 2000, 192), (2100, 2900, 4096), (4000, 4000, 4096), (5000, 3000, 4096), (4000, 4000, 4096 + 48),
+                                  (2100, 2900, 4096 + 16)])
 def test_ragged_256_tiles_exact_on_integers(mh, case):
     """Problems the library puts on 256x256 tiles (the larger cases) or 128x128 tiles that reach beyond M, N and K: rows beyond the operands are read from
     the last row and never stored, the K tail (1 to 7 pieces of 16 bytes, also with less than one k-tile in all) is
     masked, pieces of D that cross N go out element by element.  D is a window of a larger buffer whose frame must stay
-    untouched; small integers make every sum exact.  (K of whole 128-byte rows, 16-bit operands and no C: the guarded
-    form of the hand-ordered kernel; everything else: of the compiler-scheduled one.)"""
+    untouched; small integers make every sum exact.  (The guarded forms of the hand-ordered kernel, K tails included:
+    with C the one whose epilogue is the general one.)"""
     M, N, K = case
     g = torch.Generator().manual_seed(M + N + K)
     A = torch.randint(-3, 4, (M, K), generator=g).float()
@@ -835,10 +836,11 @@ def test_ragged_256_tiles_exact_on_integers(mh, case):
             # with C the one whose epilogue is the general one
             assert ks[0]["family"] == "gemm_mfma_tn_256_w4" and "ragged=1" in ks[0]["name"] and "tile=256" in ks[0]["name"] and "ops=0" in ks[0]["name"], ks
             assert kc[0]["family"] == "gemm_mfma_tn_256_w4" and "ragged=1" in kc[0]["name"] and "ops=1" in kc[0]["name"], kc
-        if case == (2100, 2900, 4096):     # fewer than 128 tiles of 256 x 256: the hand-ordered kernel's guarded 128 x 128 instance
+        if case in ((2100, 2900, 4096), (2100, 2900, 4096 + 16)):     # fewer than 128 tiles of 256 x 256: the hand-ordered kernel's guarded 128 x 128 instance
             assert ks[0]["family"] == "gemm_mfma_tn_256_w4" and "ragged=1" in ks[0]["name"] and "tile=128" in ks[0]["name"], ks
-        if case == (4099, 2050, 4096 + 8) and b16:     # a K tail on 256 x 256 tiles: the compiler-scheduled kernel's guarded instance masks it
-            assert ks[0]["family"] == "gemm_mfma_tn_256" and "ragged" in ks[0]["flags"], ks
+        if (case == (4099, 2050, 4096 + 8) and b16) or case == (4000, 4000, 4096 + 48):     # a K tail on 256 x 256 tiles: the same guarded forms mask it in registers
+            assert ks[0]["family"] == "gemm_mfma_tn_256_w4" and "ragged=1" in ks[0]["name"] and "tile=256" in ks[0]["name"], ks
+            assert kc[0]["family"] == "gemm_mfma_tn_256_w4" and "ragged=1" in kc[0]["name"] and "ops=1" in kc[0]["name"], kc
         if case == (1000, 600, 136):     # too few tiles for 256 x 256: the 128 x 128 kernel's guarded instance
             assert ks[0]["tile"].startswith("128x128") and "ragged" in ks[0]["flags"], ks
         mh.gemm_(mh.tiled_mma_desc(atom, cta_tile=(0, 0, 0)), T(d), T(a), T(b))

@@ -95,7 +95,9 @@ def test_immediate_offset_variant_under_three_readings_of_the_instruction():
 
 # ---------------------------------------------------------------------------------------------------------------------
 # gemm_mfma_tn_256 with ragged tiles (csrc/gemm_mfma256.hip, kRagged): rows clamped to the operand's last row, pieces
-# beyond K swapped for the row's first piece in the last k-tile
+# beyond K swapped for the row's first piece in the last k-tile.  The guarded instances of the hand-ordered kernel
+# (csrc/gemm_mfma_w4_kernel.hpp) address their stages the same way: wave w brings rows 32 w + 8 i + lane / 8 (clamped),
+# lane l logical piece (l % 8) ^ (l / 8 % 8), a lane beyond K in the last stage minus its piece offset (tail_cut).
 # ---------------------------------------------------------------------------------------------------------------------
 
 def ragged256_plan(rows, k_bytes, pitch, tile):

@@ -253,12 +253,12 @@ static int split_count(const moye_tiled_mma* mma, int64_t M, int64_t N, int64_t 
 // fragment reads transpose: f16 / bf16 through the 16x16x32 atoms on whole 256 x 256 x 64 tiles on eight waves (the
 // hand-ordered kernel, gemm_mfma256w4.hip, for plain calls; the load-to-LDS kernel otherwise) or whole 128 x 128 x 64 tiles
 // (named, or the library's own choice for a problem of whole 128 x 128 tiles with more than 64 rows), the two-stage
-// schedule, no K ranges; fp8 and fp32 on the hand-ordered kernel's whole 256 x 256 tiles with 128 bytes of K per k-step
-// (named so, or the library's choice when the problem has at least 128 such tiles), plain calls; the operand dense
+// schedule, no K ranges; fp8 and fp32 on the hand-ordered kernel's whole 256 x 256 or 128 x 128 tiles with 128 bytes of K
+// per k-step (named so, or left to the library: 256 x 256 tiles when the problem has at least 128 of them), plain calls; the operand dense
 // along its rows with a pitch of whole 16-byte pieces, and D 16-byte aligned (the guarded instances, which take any D,
 // read K-major operands only).  `force256`: the call must run on 256 x 256 tiles although it left the tile to the library.
 static bool majors_run_natively(const moye_tiled_mma* mma, const Mat& A, const Mat& B, const Mat& D, const moye_gemm_epilogue& ep,
-                                bool has_c, bool* force256 = nullptr) {
+                                bool has_c, int cus, bool* force256 = nullptr) {
     if (force256) *force256 = false;
     const bool b16 = mma->atom == MOYE_MFMA_F32_16x16x32_F16 || mma->atom == MOYE_MFMA_F32_16x16x32_BF16;
     const bool wide = mma->atom == MOYE_MFMA_F32_16x16x32_FP8 || mma->atom == MOYE_MFMA_F32_16x16x4_F32;  // hand-ordered kernel only
@@ -271,13 +271,17 @@ static bool majors_run_natively(const moye_tiled_mma* mma, const Mat& A, const M
     if ((K * eb) % 128) return false;
     const bool four_waves = mma->atom_layout_mnk[0] * mma->atom_layout_mnk[1] == 4;
     const bool named256 = bm == 256 && bn == 256 && (b16 ? (bk == 0 || bk == 64) : bk * eb == 128) && !four_waves && M % 256 == 0 && N % 256 == 0;
-    const bool named128 = b16 && bm == 128 && bn == 128 && bk == 64 && M % 128 == 0 && N % 128 == 0;
+    const bool named128 = bm == 128 && bn == 128 && bk * eb == 128 && M % 128 == 0 && N % 128 == 0;
     const bool chosen = bm == 0 && bn == 0 && bk == 0 && M > 64 && M % 128 == 0 && N % 128 == 0;
     if (wide) {
-        // (the hand-ordered kernel has neither an element-wise epilogue operation nor, for fp32 and fp8, another kernel behind it)
+        // (the hand-ordered kernel reads such operands in plain calls only, and fp32 and fp8 have no other kernel that does)
         if (ep.op != MOYE_MAP_IDENTITY || mma->stages >= 2) return false;
+        // (left to the library: 256 x 256 tiles when the problem has at least 128 of them, 128 x 128 tiles otherwise)
         const bool chosen256 = chosen && M % 256 == 0 && N % 256 == 0 && (M / 256) * (N / 256) >= 128;
-        if (!named256 && !chosen256) return false;
+        if (!named256 && !named128 && !chosen) return false;
+        // (fp32, left to the library, fewer 128 x 128 tiles than CUs: K-major copies and 64 x 64 tiles cost less than a
+        // part-filled chip on the slow fp32 MFMA: 1024^3 38.5 us against 68.9)
+        if (chosen && !chosen256 && eb == 4 && (M / 128) * (N / 128) < cus) return false;
         if (force256) *force256 = chosen256;
     } else if (!named256 && !named128 && !chosen) {
         return false;
@@ -305,7 +309,7 @@ static size_t gemm_workspace_bytes_impl(const moye_tiled_mma* mma, const Mat& A,
 }
 
 static size_t gemm_workspace_bytes(const moye_tiled_mma* mma, const Mat& A, const Mat& B, const Mat& D, const moye_gemm_epilogue& ep, int cus) {
-    return gemm_workspace_bytes_impl(mma, A, B, majors_run_natively(mma, A, B, D, ep, false), cus);
+    return gemm_workspace_bytes_impl(mma, A, B, majors_run_natively(mma, A, B, D, ep, false, cus), cus);
 }
 
 // A step that transposes `m` (unit stride along its rows index) into ws as rows x K with K contiguous; rewrites `m`
@@ -415,7 +419,7 @@ static int32_t gemm_plan_build(const moye_tiled_mma* mma, const moye_tensor* tD,
     // along K are brought to the K-major form the kernels read (one tiled transpose each)
     char* ws = nullptr;
     bool force256 = false;
-    const bool native_majors = majors_run_natively(mma, A, B, D, ep, tC != nullptr, &force256);
+    const bool native_majors = majors_run_natively(mma, A, B, D, ep, tC != nullptr, plan.shape.cus, &force256);
     int major_flags = 0;  // which of the kernel's operands keep their M- (N-) major form
     if (native_majors) {
         if (A.cs != 1 && A.cols > 1) { major_flags |= kGemmAMajorM; A.rs = A.cs; A.cs = 1; }  // Mat::rs now holds the pitch between consecutive k

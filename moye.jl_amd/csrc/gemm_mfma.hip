@@ -558,9 +558,11 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
         // (fp8 always: only this kernel issues the 16x16x128 MFMA on 128 x 128 tiles, twice the rate of the 16x16x32 one:
         // fp8 2560^3 29.9 -> 22.1 us, 2048^3 16.9 -> 13.7, 1536^3 14.0 -> 10.8; fp32 always as well: 4096^3 on these tiles
         // 1136 -> 914 us, 2048^3 128.8 -> 122.5)
-        if (whole && (int64_t)(a.M / 128) * (a.N / 128) > (eb == 2 ? cus : 0) &&
+        // (operands that keep their M- / N-major form: its transposing fragment reads, every operand type)
+        const bool majors128 = a.flags & (kGemmAMajorM | kGemmBMajorN);
+        if (whole && (majors128 || (int64_t)(a.M / 128) * (a.N / 128) > (eb == 2 ? cus : 0)) &&
             (eb == 2 || eb == 4 || in_dt == MOYE_F8E4M3) && a.ep_op == MOYE_MAP_IDENTITY && stages < 2 &&
-            !(a.flags & (kGemmAMajorM | kGemmBMajorN | kGemmEpiLaneOp)) && row_offsets_fit(a, 128, eb))
+            !(a.flags & kGemmEpiLaneOp) && row_offsets_fit(a, 128, eb))
             return gemm_mfma_tn_128_w4_dispatch(in_dt, out_dt, a, plan);
         if (whole) return gemm_mfma_tn_128_dispatch(in_dt, out_dt, a, plan);
         if (chosen_here || (a.flags & MOYE_GEMM_PREDICATE)) {

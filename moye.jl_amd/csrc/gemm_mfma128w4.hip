@@ -66,6 +66,7 @@ int32_t gemm_mfma_tn_128_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, 
         return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the hand-ordered 128x128 kernel takes f16 or bf16 operands and writes f32, f16 or bf16");
     }
     if (!row_offsets_fit(a, 128, dtype_bytes(in_dt))) return fail(MOYE_ERR_SHAPE, "gemm!: row pitch too large for the hand-ordered 128x128 MFMA kernel");
+    if (a.flags & (kGemmAMajorM | kGemmBMajorN)) return launch128_w4_majors_dispatch(in_dt, out_dt, a, plan);  // (plain calls on whole tiles)
     if (in_dt == MOYE_F32) {
         switch (out_dt) {
             case MOYE_F32: return launch256_w4<W4F32L, OutF32, 2, false, false, 128>(a, plan);

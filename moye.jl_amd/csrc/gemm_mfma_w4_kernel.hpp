@@ -289,14 +289,15 @@ struct W4F32L {
 // row would.  The 32-byte piece index of a k-row is XORed with (row % 4) | 4 ((row / 8) % 2), so that the eight row
 // pieces the 32 lanes of one pass read lie in eight bank groups (the layout of gemm_mfma_lds_tile.hpp).  fp8 the same
 // way through ds_read_b64_tr_b8 (k-rows of 256 bytes, 128 per stage; lane 16 g + s points at k-row 16 g + s / 2 (+ 8,
-// + 64, + 72) and m = m0 + 8 (s % 2); the 16-byte piece index XORed with row % 8).  fp32 needs no transposing read: an
+// + 64, + 72) and m = m0 + 8 (s % 2); the 16-byte piece index XORed with row % 8 and, in bit 3, with (row / 16) % 2: see
+// tr_swz).  fp32 needs no transposing read: an
 // MFMA takes one value per lane and operand, so a lane reads its eight values of row m0 + s with ds_read_b32 from
 // k-rows 4 g + e and 16 + 4 g + e (k-rows of 1 KiB, 32 per stage; the 64-byte piece index XORed with (row / 4) % 2, so
-// that the two k-rows the 32 lanes of a pass read lie in different halves of the banks).  Whole-line stages on the
-// 256 x 256 tile, eight waves, no bias, whole tiles.
+// that the two k-rows the 32 lanes of a pass read lie in different halves of the banks).  Whole-line stages, plain calls
+// on whole tiles: the 256 x 256 tile with eight waves, the 128 x 128 tile with four (k-rows of 128 operand rows).
 template <typename In, typename Out, int WGN, bool kBias = false, bool kRagged = false, int TILE = 256, int AMAJ = 0, int BMAJ = 0, bool kOps = false, bool kNoC = false>
 __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_256_w4(GemmArgs p) {
-    static_assert(!(AMAJ || BMAJ) || (In::kRow == 128 && TILE == 256 && WGN == 4 && !kBias && !kRagged),
+    static_assert(!(AMAJ || BMAJ) || (In::kRow == 128 && ((TILE == 256 && WGN == 4) || (TILE == 128 && WGN == 2)) && !kBias && !kRagged),
                   "operands that are not K-major: whole-line stages, eight waves, plain whole tiles");
     static_assert(!kRagged || (!kBias && In::kRow == 128 && !AMAJ && !BMAJ), "ragged tiles: the plain whole-line form, K-major operands");
     static_assert(!kOps || (In::kRow == 128 && TILE == 256 && WGN == 4 && !kBias && !AMAJ && !BMAJ), "epilogue operations: whole-line stages, eight waves, K-major operands");
@@ -319,10 +320,17 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
     constexpr int RPT = In::kBytes == 4 ? 8 : 4;                    // LDS reads per fragment of a transposed operand
     constexpr int RPA = AMAJ ? RPT : RPF, RPB = BMAJ ? RPT : RPF;  // LDS reads per fragment of A and of B
     // transposed operand halves of a stage: k-rows of TROW bytes, a swizzle granule of 16 operand rows (GB bytes)
-    constexpr int TROW = 256 * In::kBytes, TKROWS = 128 / In::kBytes, TLPR = TROW / 16, TRPI = 64 / TLPR, GB = 16 * In::kBytes;
+    constexpr int TROW = TILE * In::kBytes, TKROWS = 128 / In::kBytes, TLPR = TROW / 16, TRPI = 64 / TLPR, GB = 16 * In::kBytes;
+    // (bytes: the 32 lanes of a pass read k-rows 0-7 and 16-23.  On the 256 x 256 tile a k-row has sixteen 16-byte granules
+    // and bit 4 of the row picks the half of them; on the 128 x 128 tile it has eight, a k-row is half a sweep of the
+    // banks, and the k-rows whose bit 4 is set are stored with their neighbour's place instead (tr_place), so that rows
+    // j and 16 + j lie in different halves.  Without either, every such read took two more cycles.)
     auto tr_swz = [](int krow) {
-        return In::kBytes == 2 ? ((krow & 3) | (((krow >> 3) & 1) << 2)) : In::kBytes == 1 ? (krow & 7) : ((krow >> 2) & 1);
+        return In::kBytes == 2   ? ((krow & 3) | (((krow >> 3) & 1) << 2))
+               : In::kBytes == 1 ? ((krow & 7) | (TROW >= 256 ? ((krow >> 4) & 1) << 3 : 0))
+                                 : ((krow >> 2) & 1);
     };
+    auto tr_place = [](int krow) { return In::kBytes == 1 && TROW < 256 ? krow ^ ((krow >> 4) & 1) : krow; };  // its own inverse
 
     extern __shared__ __attribute__((aligned(256))) u32x4 smem[];
 
@@ -373,7 +381,8 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
 #pragma unroll
     for (int q = 0; q < 2 * LD; ++q) {
         if ((q < LD && AMAJ) || (q >= LD && BMAJ)) {
-            const int krow = wave * (TKROWS / NW) + TRPI * (q % LD) + lane / TLPR, p16 = lane % TLPR;
+            // (the k-row whose place in the stage this lane fills)
+            const int krow = tr_place(wave * (TKROWS / NW) + TRPI * (q % LD) + lane / TLPR), p16 = lane % TLPR;
             const int piece = (((p16 * 16 / GB) ^ tr_swz(krow)) * GB + (p16 * 16) % GB) / 16;  // the swizzle moves granules
             voff[q] = (uint32_t)(krow * (q < LD ? pitch_a : pitch_b) + piece * 16);
             continue;
@@ -422,8 +431,10 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
     [[maybe_unused]] const int tr_row0 = In::kBytes == 2 ? 8 * kq + (r16 >> 2) : In::kBytes == 1 ? 16 * kq + (r16 >> 1) : 4 * kq;
     [[maybe_unused]] const int tr_in = In::kBytes == 2 ? 8 * (r16 & 3) : In::kBytes == 1 ? 8 * (r16 & 1) : 4 * r16;
     [[maybe_unused]] const int tr_fx = tr_swz(tr_row0);
-    [[maybe_unused]] const uint32_t ta_byte = lds0 + (uint32_t)(tr_row0 * TROW + ((wm0 / 16) ^ tr_fx) * GB + tr_in);
-    [[maybe_unused]] const uint32_t tb_byte = lds0 + kATileBytes + (uint32_t)(tr_row0 * TROW + ((wn0 / 16) ^ tr_fx) * GB + tr_in);
+    // (the other reads of a fragment add 8, 64 and 72 k-rows (bytes) to the first: neither bit 0, which tr_place may flip,
+    // nor the bits the swizzle looks at change)
+    [[maybe_unused]] const uint32_t ta_byte = lds0 + (uint32_t)(tr_place(tr_row0) * TROW + ((wm0 / 16) ^ tr_fx) * GB + tr_in);
+    [[maybe_unused]] const uint32_t tb_byte = lds0 + kATileBytes + (uint32_t)(tr_place(tr_row0) * TROW + ((wn0 / 16) ^ tr_fx) * GB + tr_in);
     // the fragment of 16-row block BLK for the k-step whose stages start at byte offsets o0 (, o1)
     auto load_frag = [&](auto& f, uint32_t base, auto blk_c, uint32_t o0, uint32_t o1) __attribute__((always_inline)) {
         constexpr int OFF = 16 * kRow * decltype(blk_c)::value;
@@ -431,25 +442,25 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
             const uint32_t at = (base ^ (uint32_t)(decltype(blk_c)::value * GB)) + o0;  // (stage offsets are multiples of 64 KiB)
             if constexpr (In::kBytes == 2) {
                 f.q0 = lds_read_tr8<0>(at);
-                f.q1 = lds_read_tr8<4 * 512>(at);
-                f.q2 = lds_read_tr8<32 * 512>(at);
-                f.q3 = lds_read_tr8<36 * 512>(at);
+                f.q1 = lds_read_tr8<4 * TROW>(at);
+                f.q2 = lds_read_tr8<32 * TROW>(at);
+                f.q3 = lds_read_tr8<36 * TROW>(at);
             } else {
                 f.q0 = lds_read_tr8_b8<0>(at);
-                f.q1 = lds_read_tr8_b8<8 * 256>(at);
-                f.q2 = lds_read_tr8_b8<64 * 256>(at);
-                f.q3 = lds_read_tr8_b8<72 * 256>(at);
+                f.q1 = lds_read_tr8_b8<8 * TROW>(at);
+                f.q2 = lds_read_tr8_b8<64 * TROW>(at);
+                f.q3 = lds_read_tr8_b8<72 * TROW>(at);
             }
         } else if constexpr (std::is_same_v<std::remove_reference_t<decltype(f)>, W4TrFrag32>) {
             const uint32_t at = (base ^ (uint32_t)(decltype(blk_c)::value * GB)) + o0;
             f.e[0] = lds_read4<0>(at);
-            f.e[1] = lds_read4<1024>(at);
-            f.e[2] = lds_read4<2048>(at);
-            f.e[3] = lds_read4<3072>(at);
-            f.e[4] = lds_read4<16384>(at);
-            f.e[5] = lds_read4<16384 + 1024>(at);
-            f.e[6] = lds_read4<16384 + 2048>(at);
-            f.e[7] = lds_read4<16384 + 3072>(at);
+            f.e[1] = lds_read4<TROW>(at);
+            f.e[2] = lds_read4<2 * TROW>(at);
+            f.e[3] = lds_read4<3 * TROW>(at);
+            f.e[4] = lds_read4<16 * TROW>(at);
+            f.e[5] = lds_read4<17 * TROW>(at);
+            f.e[6] = lds_read4<18 * TROW>(at);
+            f.e[7] = lds_read4<19 * TROW>(at);
         } else if constexpr (kLine) {
             f.lo = lds_read16<OFF>(base + o0);
             f.hi = lds_read16<OFF>(base + hi_delta + o0);
@@ -649,10 +660,12 @@ static int32_t launch256_w4(const GemmArgs& a, GemmPlan& plan) {
     return MOYE_OK;
 }
 
-// The instances live in four translation units (so that they compile side by side): gemm_mfma256w4.hip (the 256 x 256
+// The instances live in five translation units (so that they compile side by side): gemm_mfma256w4.hip (the 256 x 256
 // tile with K-major operands), gemm_mfma256w4_majors.hip (operands that keep their M- / N-major form),
-// gemm_mfma256w4_ops.hip (an element-wise operation in the epilogue), gemm_mfma128w4.hip (the 128 x 128 tile).
+// gemm_mfma256w4_ops.hip (an element-wise operation in the epilogue), gemm_mfma128w4.hip (the 128 x 128 tile),
+// gemm_mfma128w4_majors.hip (the 128 x 128 tile with M- / N-major operands).
 int32_t launch256_w4_majors_dispatch(int32_t in_dt, int32_t out_dt, const GemmArgs& a, GemmPlan& plan);
 int32_t launch256_w4_ops_dispatch(int32_t in_dt, int32_t out_dt, const GemmArgs& a, GemmPlan& plan);
+int32_t launch128_w4_majors_dispatch(int32_t in_dt, int32_t out_dt, const GemmArgs& a, GemmPlan& plan);
 
 }  // namespace moye

@@ -75,7 +75,8 @@ def check_kernel_step(s, eb, ob):
         else:
             assert s["op"] == 0, s                       # the other instances have no element-wise operation
         if "amaj=1" in name or "bmaj=1" in name:
-            assert "tile=256" in name and "waves=8" in name and not ragged, s
+            assert (("tile=256" in name and "waves=8" in name) or ("tile=128" in name and "waves=4" in name)) and not ragged, s
+            assert "bias=0" in name and "ops=0" in name and s["op"] == 0 and step_bytes == 128, s
     elif fam in ("gemm_mfma_tn_256", "gemm_mfma_tn_128"):
         assert ("ragged=1" in name) == ragged
         assert ("amaj=1" in name) == ("a_m_major" in flags) and ("bmaj=1" in name) == ("b_n_major" in flags)
@@ -266,9 +267,14 @@ def test_known_shapes_run_on_the_instances_they_are_meant_for():
     for dt, bk in ((f16, 64), (bf16, 64), (f8, 128), (f32, 32)):
         p = run_case(dt, f32, 4096, 4096, 4096, cta=(256, 256, bk), a_major="m", b_major="n", flags=_lib.GEMM_NO_WORKSPACE)
         assert p["workspace"] == 0 and len(p["steps"]) == 1 and "amaj=1,bmaj=1" in p["steps"][0]["name"] and p["steps"][0]["family"] == "gemm_mfma_tn_256_w4"
-    # ... and a K-major copy where no kernel reads the operand as it lies (a short problem on 128 x 128 tiles, fp8)
+    # ... also on 128 x 128 tiles (a small problem left to the library; a named tile)
     p = run_case(f8, f32, 256, 512, 256, a_major="m", b_major="n")
-    assert [s["what"] for s in p["steps"]][:2] == ["kmajor_copy", "kmajor_copy"] and p["workspace"] >= 256 * 256 + 512 * 256
+    assert p["workspace"] == 0 and step_names(p) == ["gemm_mfma_tn_256_w4<W4FP8L,OutF32,waves=4,bias=0,ragged=0,tile=128,amaj=1,bmaj=1,ops=0>"]
+    p = run_case(f16, f16, 2048, 2048, 2048, cta=(128, 128, 64), waves=(2, 2, 1), a_major="m")
+    assert p["workspace"] == 0 and step_names(p) == ["gemm_mfma_tn_256_w4<W4F16L,OutF16,waves=4,bias=0,ragged=0,tile=128,amaj=1,bmaj=0,ops=0>"]
+    # ... and a K-major copy where no kernel reads the operand as it lies (tiles that reach beyond M, fp8)
+    p = run_case(f8, f32, 200, 512, 256, a_major="m", b_major="n")
+    assert [s["what"] for s in p["steps"]][:2] == ["kmajor_copy", "kmajor_copy"] and p["workspace"] >= 200 * 256 + 512 * 256
     # short M: whole 128-byte lines of K through LDS, a K tail as a masked trip of the same kernel
     assert step_names(run_case(bf16, f32, 16, 8192, 8192))[0].startswith("gemm_mfma_skinny_lds<InBF16,OutF32,mt=1,ntw=2,waves=4,stages=3>")
     assert step_names(run_case(bf16, f32, 16, 8192, 8224))[0].startswith("gemm_mfma_skinny_lds<InBF16,OutF32,mt=1,ntw=2,")   # a K tail too

@@ -1666,6 +1666,45 @@ def test_operand_majors_every_cta_exact_on_integers(mh, majors):
         assert torch.equal(dt_.t(), 0.5 * want + C0), (tdt, majors, "column-major D, C, alpha")
 
 
+@pytest.mark.parametrize("majors", ["mk", "kn", "mn"])
+def test_operand_majors_on_128_tiles_every_type_exact_on_integers(mh, majors):
+    """Mid-size problems with A stored M-major and / or B stored N-major on the 128 x 128 tile of the hand-ordered kernel
+    (two workgroups per CU): fp16, bf16, fp8 and fp32 operands read where they lie, the tile named and left to the
+    library, MOYE_GEMM_NO_WORKSPACE; 2048 x 2304 x 384 (288 tiles: every CU holds two workgroups for part of the run) on
+    small integers, bit for bit; with C, alpha and a column-major D as well."""
+    from moye_hip import _lib
+    M, N, K = 2048, 2304, 384
+    g = torch.Generator().manual_seed(1108)
+    cases = [(torch.float16, mh.MFMA_F32_16x16x32_F16, 64, torch.float16), (torch.bfloat16, mh.MFMA_F32_16x16x32_BF16, 64, torch.float32),
+             (torch.float32, mh.MFMA_F32_16x16x4_F32, 32, torch.float32)]
+    if hasattr(torch, "float8_e4m3fn"):
+        cases.append((torch.float8_e4m3fn, mh.MFMA_F32_16x16x32_FP8, 128, torch.bfloat16))
+    for tdt, atom, bk, out_dt in cases:
+        A = torch.randint(-2, 3, (M, K), generator=g).float()
+        B = torch.randint(-2, 3, (N, K), generator=g).float()
+        a_k, b_k = A.to(tdt).cuda(), B.to(tdt).cuda()
+        a_m, b_n = A.t().contiguous().to(tdt).cuda(), B.t().contiguous().to(tdt).cuda()
+        ta = T(a_m, (M, K), (1, M)) if majors[0] == "m" else T(a_k)
+        tb = T(b_n, (N, K), (1, N)) if majors[1] == "n" else T(b_k)
+        want = A.cuda() @ B.cuda().t()
+        assert float(want.abs().max()) <= 256          # exact in bf16 too
+        for cta, waves in (((128, 128, bk), (2, 2, 1)), ((0, 0, 0), (1, 1, 1))):
+            mma = mh.tiled_mma_desc(atom, atom_layout=waves, cta_tile=cta, flags=_lib.GEMM_NO_WORKSPACE)
+            d = torch.full((M, N), float("nan"), dtype=out_dt, device="cuda")
+            ks = kernels_of(mh, mma, T(d), ta, tb)
+            want_name = ("amaj=%d" % (majors[0] == "m"), "bmaj=%d" % (majors[1] == "n"), "tile=128", "waves=4")
+            assert len(ks) == 1 and ks[0]["family"] == "gemm_mfma_tn_256_w4" and all(w in ks[0]["name"] for w in want_name), (tdt, cta, ks)
+            mh.gemm_(mma, T(d), ta, tb)
+            torch.cuda.synchronize()
+            assert torch.equal(d.float(), want), (tdt, majors, cta)
+        C0 = torch.randint(-8, 9, (M, N), generator=g).float().cuda()
+        dt_ = torch.zeros(N, M, dtype=torch.float32, device="cuda")
+        mh.gemm_(mh.tiled_mma_desc(atom, atom_layout=(2, 2, 1), cta_tile=(128, 128, bk), flags=_lib.GEMM_NO_WORKSPACE),
+                 T(dt_, (M, N), (1, M)), ta, tb, T(C0), 0.5)
+        torch.cuda.synchronize()
+        assert torch.equal(dt_.t(), 0.5 * want + C0), (tdt, majors, "column-major D, C, alpha")
+
+
 def test_operand_majors_wide_types_random_and_workspace_rule(mh):
     """fp8 and fp32 NN (A M-major, B N-major) at 4096^3 on random data against fp64 (tolerances 1e-2 / 1e-5), read where
     they lie; and the one case that still copies: an element-wise epilogue operation, which moye_gemm_ex_workspace_size

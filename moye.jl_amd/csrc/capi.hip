@@ -282,7 +282,9 @@ static bool majors_run_natively(const moye_tiled_mma* mma, const Mat& A, const M
         // (fp32, left to the library, fewer 128 x 128 tiles than CUs: K-major copies and 64 x 64 tiles cost less than a
         // part-filled chip on the slow fp32 MFMA: 1024^3 38.5 us against 68.9)
         if (chosen && !chosen256 && eb == 4 && (M / 128) * (N / 128) < cus) return false;
-        if (force256) *force256 = chosen256;
+        // (only a call that has such an operand is held to these tiles)
+        const bool any = (A.cs != 1 && A.cols > 1) || (B.cs != 1 && B.cols > 1);
+        if (force256) *force256 = chosen256 && any;
     } else if (!named256 && !named128 && !chosen) {
         return false;
     }

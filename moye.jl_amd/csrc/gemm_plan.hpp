@@ -15,6 +15,7 @@
 #pragma once
 
 #include <cstdint>
+#include <initializer_list>
 
 namespace moye {
 
@@ -28,10 +29,11 @@ inline double gemm_plan_cost(int tile, int split, int64_t M, int64_t N, int64_t 
     const int64_t tiles = ((M + tile - 1) / tile) * ((N + tile - 1) / tile), ctas = tiles * split;
     const int slots = tile == 128 ? 2 : 4;
     // per k-tile and workgroup with 1 .. slots workgroups resident on a CU.  fp32 operands run on v_mfma_f32_16x16x4_f32,
-    // an eighth of the 16-bit rate per byte of K, and are bound by it (2048^3 on 256 workgroups of 128 x 128: 128 us;
-    // 4096 x 2048 x 4096 on 512: 589 us; 1024^3 on 256 workgroups of 64 x 64: 25.7 us; 2048^3 on 1024: 156 us)
+    // an eighth of the 16-bit rate per byte of K, and are bound by it (2048^3 on 256 workgroups of 128 x 128: 124.5 us;
+    // 4096 x 2048 x 4096 on 512: 465 us; 2560^3 on 400: 291 us; 3072^3 on 576: 522 us; 1024^3 on 256 workgroups of
+    // 64 x 64: 25.7 us; 2048^3 on 1024: 156 us; 3072^3 on 2304: 509 us)
     static const double t128_16[3] = {0, 0.52, 0.94}, t64_16[5] = {0, 0.40, 0.47, 0.66, 0.84};
-    static const double t128_32[3] = {0, 1.96, 4.58}, t64_32[5] = {0, 0.71, 1.25, 1.80, 2.40};
+    static const double t128_32[3] = {0, 1.92, 3.62}, t64_32[5] = {0, 0.71, 1.25, 1.80, 2.40};
     const double* t = tile == 128 ? (f32_in ? t128_32 : t128_16) : (f32_in ? t64_32 : t64_16);
     const double ktiles = (double)((k_bytes / split + 127) / 128);
     // whole rounds of cus x slots workgroups, then the rest with fewer neighbours
@@ -70,9 +72,10 @@ inline double gemm_plan_cost_256(int64_t M, int64_t N, int64_t k_bytes, bool f32
     const int64_t tiles = ((M + 255) / 256) * ((N + 255) / 256), full = tiles / cus, rest = tiles % cus;
     const int half = cus / 2 > 0 ? cus / 2 : 1;
     const double ktiles = (double)((k_bytes + 127) / 128);
-    // (fp32: 7.56 us per k-tile however many CUs are busy: the matrix pipe alone sets the pace, 4096 x 4096 x 1024 251 us)
-    const double t_full = f32_in ? 7.56 : 1.44;
-    const double t_rest = rest == 0 ? 0.0 : f32_in ? 7.56 : rest <= half ? 0.98 : 0.98 + (double)(rest - half) / (double)half * 0.46;
+    // (fp32: 7.05 us per k-tile however many CUs are busy: the matrix pipe alone sets the pace; 4096^3 909 us,
+    // 3072^3 on 144 tiles 687 us, 4096 x 2048 x 4096 on 128 tiles 913 us)
+    const double t_full = f32_in ? 7.05 : 1.44;
+    const double t_rest = rest == 0 ? 0.0 : f32_in ? 7.05 : rest <= half ? 0.98 : 0.98 + (double)(rest - half) / (double)half * 0.46;
     double us = 9.0 + 6.0 * (double)(full + (rest ? 1 : 0) - 1) + ktiles * ((double)full * t_full + t_rest);
     if (ragged) us *= 1.25;
     return us;

@@ -834,13 +834,17 @@ def test_ragged_256_tiles_exact_on_integers(mh, case):
         if case in ((4000, 4000, 4096), (5000, 3000, 4096)):
             # at least 128 ragged 256 x 256 tiles, K of whole 128-byte rows: the guarded forms of the hand-ordered kernel,
             # with C the one whose epilogue is the general one
-            assert ks[0]["family"] == "gemm_mfma_tn_256_w4" and "ragged=1" in ks[0]["name"] and "tile=256" in ks[0]["name"] and "ops=0" in ks[0]["name"], ks
-            assert kc[0]["family"] == "gemm_mfma_tn_256_w4" and "ragged=1" in kc[0]["name"] and "ops=1" in kc[0]["name"], kc
+            # (fp32, whose pace the matrix pipe sets whatever the fill, is cheaper on 128 x 128 tiles here: the same kernel's guarded 128 x 128 form)
+            assert ks[0]["family"] == "gemm_mfma_tn_256_w4" and "ragged=1" in ks[0]["name"] and "ops=0" in ks[0]["name"], ks
+            assert "tile=256" in ks[0]["name"] or in_dt == torch.float32, ks
+            if in_dt != torch.float32:
+                assert kc[0]["family"] == "gemm_mfma_tn_256_w4" and "ragged=1" in kc[0]["name"] and "ops=1" in kc[0]["name"], kc
         if case in ((2100, 2900, 4096), (2100, 2900, 4096 + 16)):     # fewer than 128 tiles of 256 x 256: the hand-ordered kernel's guarded 128 x 128 instance
             assert ks[0]["family"] == "gemm_mfma_tn_256_w4" and "ragged=1" in ks[0]["name"] and "tile=128" in ks[0]["name"], ks
         if (case == (4099, 2050, 4096 + 8) and b16) or case == (4000, 4000, 4096 + 48):     # a K tail on 256 x 256 tiles: the same guarded forms mask it in registers
-            assert ks[0]["family"] == "gemm_mfma_tn_256_w4" and "ragged=1" in ks[0]["name"] and "tile=256" in ks[0]["name"], ks
-            assert kc[0]["family"] == "gemm_mfma_tn_256_w4" and "ragged=1" in kc[0]["name"] and "ops=1" in kc[0]["name"], kc
+            assert ks[0]["family"] == "gemm_mfma_tn_256_w4" and "ragged=1" in ks[0]["name"] and ("tile=256" in ks[0]["name"] or in_dt == torch.float32), ks
+            if in_dt != torch.float32:
+                assert kc[0]["family"] == "gemm_mfma_tn_256_w4" and "ragged=1" in kc[0]["name"] and "ops=1" in kc[0]["name"], kc
         if case == (1000, 600, 136):     # too few tiles for 256 x 256: the 128 x 128 kernel's guarded instance
             assert ks[0]["tile"].startswith("128x128") and "ragged" in ks[0]["flags"], ks
         mh.gemm_(mh.tiled_mma_desc(atom, cta_tile=(0, 0, 0)), T(d), T(a), T(b))
@@ -1901,7 +1905,9 @@ def test_fused_epilogue_on_the_hand_ordered_kernel(mh, in_name, atom, out_name, 
         seed += 1
     # tiles that reach beyond M and N, the tile left to the library: with a C or an operation the guarded general epilogue
     lib = mh.tiled_mma_desc(getattr(mh, atom), cta_tile=(0, 0, 0))
-    ragged = ("gemm_mfma_tn_256_w4", "ragged=1", "ops=1")
+    # (fp32 problems of this size are cheaper on 128 x 128 tiles, whose guarded form with a C or an operation is the
+    # compiler-scheduled kernel's: whatever runs must give the same bits)
+    ragged = ("gemm_mfma_tn_256_w4", "ragged=1", "ops=1") if in_dt != torch.float32 else ("ragged=1",)
     # (14 x 15 tiles; the row pitch of a 16-bit D is 8 bytes modulo 16; K long enough that the library takes these tiles)
     M, N, Kr = 3400, 3604, {2: 1024, 1: 4096, 4: 256}[in_dt.itemsize]
     _epilogue_case(mh, lib, M, N, Kr, out_name, "identity", "scalar", seed + 1, beta=-1.25, in_dt=in_dt, instance=ragged)

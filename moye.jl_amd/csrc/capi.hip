@@ -256,10 +256,9 @@ static int split_count(const moye_tiled_mma* mma, int64_t M, int64_t N, int64_t 
 // schedule, no K ranges; fp8 and fp32 on the hand-ordered kernel's whole 256 x 256 or 128 x 128 tiles with 128 bytes of K
 // per k-step (named so, or left to the library: 256 x 256 tiles when the problem has at least 128 of them), plain calls; the operand dense
 // along its rows with a pitch of whole 16-byte pieces, and D 16-byte aligned (the guarded instances, which take any D,
-// read K-major operands only).  `force256`: the call must run on 256 x 256 tiles although it left the tile to the library.
+// read K-major operands only).
 static bool majors_run_natively(const moye_tiled_mma* mma, const Mat& A, const Mat& B, const Mat& D, const moye_gemm_epilogue& ep,
-                                bool has_c, int cus, bool* force256 = nullptr) {
-    if (force256) *force256 = false;
+                                bool has_c, int cus) {
     const bool b16 = mma->atom == MOYE_MFMA_F32_16x16x32_F16 || mma->atom == MOYE_MFMA_F32_16x16x32_BF16;
     const bool wide = mma->atom == MOYE_MFMA_F32_16x16x32_FP8 || mma->atom == MOYE_MFMA_F32_16x16x4_F32;  // hand-ordered kernel only
     if (!b16 && !wide) return false;
@@ -276,15 +275,11 @@ static bool majors_run_natively(const moye_tiled_mma* mma, const Mat& A, const M
     if (wide) {
         // (the hand-ordered kernel reads such operands in plain calls only, and fp32 and fp8 have no other kernel that does)
         if (ep.op != MOYE_MAP_IDENTITY || mma->stages >= 2) return false;
-        // (left to the library: 256 x 256 tiles when the problem has at least 128 of them, 128 x 128 tiles otherwise)
-        const bool chosen256 = chosen && M % 256 == 0 && N % 256 == 0 && (M / 256) * (N / 256) >= 128;
+        // (left to the library: whole 256 x 256 or 128 x 128 tiles, whichever the cost model prefers)
         if (!named256 && !named128 && !chosen) return false;
         // (fp32, left to the library, fewer 128 x 128 tiles than CUs: K-major copies and 64 x 64 tiles cost less than a
         // part-filled chip on the slow fp32 MFMA: 1024^3 38.5 us against 68.9)
-        if (chosen && !chosen256 && eb == 4 && (M / 128) * (N / 128) < cus) return false;
-        // (only a call that has such an operand is held to these tiles)
-        const bool any = (A.cs != 1 && A.cols > 1) || (B.cs != 1 && B.cols > 1);
-        if (force256) *force256 = chosen256 && any;
+        if (chosen && eb == 4 && (M / 128) * (N / 128) < cus) return false;
     } else if (!named256 && !named128 && !chosen) {
         return false;
     }
@@ -420,8 +415,7 @@ static int32_t gemm_plan_build(const moye_tiled_mma* mma, const moye_tensor* tD,
     // NN / NT / TT (the naming of src/arch/mma/make_mma_ops.jl:253-265): operands whose unit stride is not
     // along K are brought to the K-major form the kernels read (one tiled transpose each)
     char* ws = nullptr;
-    bool force256 = false;
-    const bool native_majors = majors_run_natively(mma, A, B, D, ep, tC != nullptr, plan.shape.cus, &force256);
+    const bool native_majors = majors_run_natively(mma, A, B, D, ep, tC != nullptr, plan.shape.cus);
     int major_flags = 0;  // which of the kernel's operands keep their M- (N-) major form
     if (native_majors) {
         if (A.cs != 1 && A.cols > 1) { major_flags |= kGemmAMajorM; A.rs = A.cs; A.cs = 1; }  // Mat::rs now holds the pitch between consecutive k
@@ -462,11 +456,6 @@ static int32_t gemm_plan_build(const moye_tiled_mma* mma, const moye_tensor* tD,
     }
     // TiledMMA.atom_layout_mnk = how many waves tile the CTA along M and N (src/atom/mma.jl:84)
     int waves = mma->atom_layout_mnk[0] * mma->atom_layout_mnk[1];
-    if (force256) {  // fp8 / fp32 operands read where they lie: only the hand-ordered kernel's 256 x 256 tiles do that
-        bm = bn = 256;
-        bk = 128 / dtype_bytes(in_dt);
-        waves = 8;
-    }
     g.alpha = alpha;
     g.K = K;
     g.xcds = plan.shape.xcds;
@@ -486,7 +475,7 @@ static int32_t gemm_plan_build(const moye_tiled_mma* mma, const moye_tensor* tD,
     g.flags = !(mma->flags & MOYE_GEMM_NO_XCD_SWIZZLE) | (mma->flags & 0xff00) | (atom32 ? kGemmAtom32 : 0) | (rotate_k ? kGemmRotateK : 0) |
               (stream_d ? kGemmStreamD : 0) | major_flags;
     // tile and K ranges, where both are left to the library, are one decision (gemm_choose)
-    const LibraryChoice lib = force256 ? LibraryChoice{} : library_choice(mma, M, N, K, dtype_bytes(in_dt), cus);
+    const LibraryChoice lib = library_choice(mma, M, N, K, dtype_bytes(in_dt), cus);
     const TileChoice* lib_tile = lib.open ? &lib.tile : nullptr;
     if (const int split = split_count(mma, M, N, K, dtype_bytes(in_dt), cus); split > 1) {
         // K is cut into `split` equal ranges, all in one launch (gridDim.y); each range writes its fp32 product, compact and

@@ -63,7 +63,9 @@ typedef struct {
 /* MMA atoms: UniversalFMA (src/arch/mma/mma.jl:53-64) plus the gfx950 MFMA instructions that
  * take the place of the reference's MMAOP_* table (src/arch/mma/make_mma_ops.jl:426-438).
  * The 16x16 forms run with every CTA tile moye_gemm offers (64x64, 128x128, 256x256 and the
- * short-M form), the 32x32 forms with the 128x128 tile (plain and predicated). */
+ * short-M form), the 32x32 forms with the 256x256 tile (whole tiles, 2 x 4 waves) and the 128x128 tile (plain and
+ * predicated); with the tile left to the library they take 256x256 tiles where those divide the problem and fill half
+ * the chip. */
 typedef enum {
     MOYE_MMA_UNIVERSAL_FMA = 0,
     MOYE_MFMA_F32_16x16x32_F16 = 1,

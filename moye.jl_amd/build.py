@@ -26,6 +26,7 @@ SOURCES = {
     "gemm_mfma.hip": ["-ffp-contract=off"],
     "gemm_mfma128.hip": ["-ffp-contract=off"],
     "gemm_mfma256.hip": ["-ffp-contract=off"],
+    "gemm_mfma256_atom32.hip": ["-ffp-contract=off"],
     "gemm_mfma256pp.hip": ["-ffp-contract=off"],
     "gemm_mfma256w4.hip": ["-ffp-contract=off"],
     "gemm_mfma256w4_majors.hip": ["-ffp-contract=off"],

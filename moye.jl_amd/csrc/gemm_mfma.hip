@@ -292,16 +292,31 @@ static int32_t launch_atom32(int32_t in_dt, int32_t out_dt, const GemmArgs& a, G
     }
 }
 
-// The 32x32 atoms: CTA tile 128x128 with 64 bytes of K per row, four waves of 2 x 2 MFMA tiles each; residue
-// tiles under the same rule as for the 16x16 atoms.
-static int32_t dispatch_atom32(int32_t in_dt, int32_t out_dt, int bm, int bn, int bk_elems, GemmArgs a, GemmPlan& plan) {
+// The 32x32 atoms: CTA tile 256x256 with 128 bytes of K per row on eight waves of 4 x 2 MFMA tiles each (whole tiles;
+// gemm_mfma256_atom32.hip), or 128x128 with 64 bytes of K per row, four waves of 2 x 2 MFMA tiles each, residue tiles
+// under the same rule as for the 16x16 atoms.  Left to the library: 256x256 tiles when they divide the problem and
+// fill at least half of the chip.
+static int32_t dispatch_atom32(int32_t in_dt, int32_t out_dt, int bm, int bn, int bk_elems, int waves, int stages, GemmArgs a, GemmPlan& plan) {
     const int eb = dtype_bytes(in_dt), ob = dtype_bytes(out_dt);
     const bool chosen_here = bm == 0 && bn == 0;
-    if ((bm && bm != 128) || (bn && bn != 128) || (bk_elems && bk_elems * eb != 64))
-        return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the 32x32 MFMA atoms run with CTA tile 128x128x%d only, not %dx%dx%d", 64 / eb, bm, bn,
+    const bool named256 = bm == 256 && bn == 256 && (bk_elems == 0 || bk_elems * eb == 128);
+    if (!named256 && ((bm && bm != 128) || (bn && bn != 128) || (bk_elems && bk_elems * eb != 64)))
+        return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the 32x32 MFMA atoms run with CTA tile 256x256x%d or 128x128x%d, not %dx%dx%d", 128 / eb, 64 / eb, bm, bn,
                     bk_elems);
     if ((a.lda * eb) % 16 || (a.ldb * eb) % 16 || (reinterpret_cast<uintptr_t>(a.A) | reinterpret_cast<uintptr_t>(a.B)) % 16)
         return fail(MOYE_ERR_ALIGN, "gemm!: operands of the MFMA kernels need 16-byte aligned pointers and row pitches");
+    const bool whole256 = a.M % 256 == 0 && a.N % 256 == 0 && a.K % (128 / eb) == 0;
+    const bool aligned_d = !((a.ldd * ob) % 16 || reinterpret_cast<uintptr_t>(a.D) % 16);
+    if (named256) {
+        if (!whole256) return fail(MOYE_ERR_SHAPE, "gemm!: the 32x32 MFMA atoms take whole 256x256x%d tiles, the problem is %dx%dx%d", 128 / eb, a.M, a.N, a.K);
+        if (!aligned_d) return fail(MOYE_ERR_ALIGN, "gemm!: operands of the MFMA kernels need 16-byte aligned pointers and row pitches");
+        if ((waves > 1 && waves != 8) || stages >= 3 || (a.flags & (MOYE_GEMM_WAVE4 | MOYE_GEMM_PINGPONG)))
+            return fail(MOYE_ERR_UNSUPPORTED, "gemm!: the 32x32 MFMA atoms on 256x256 tiles run on 2 x 4 waves with two LDS stages");
+        return gemm_mfma_tn_256_atom32_dispatch(in_dt, out_dt, a, plan);
+    }
+    if (chosen_here && whole256 && aligned_d && (int64_t)(a.M / 256) * (a.N / 256) >= plan.shape.cus / 2 && stages < 3 &&
+        !(a.flags & (MOYE_GEMM_WAVE4 | MOYE_GEMM_PINGPONG)))
+        return gemm_mfma_tn_256_atom32_dispatch(in_dt, out_dt, a, plan);
     a.tiles_m = (a.M + 127) / 128;
     a.tiles_n = (a.N + 127) / 128;
     if (a.M % 128 || a.N % 128 || a.K % (64 / eb)) {
@@ -324,7 +339,7 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
                               GemmArgs a, GemmPlan& plan, const TileChoice* lib) {
     const int eb = dtype_bytes(in_dt);
     const int cus = plan.shape.cus;
-    if (a.flags & kGemmAtom32) return dispatch_atom32(in_dt, out_dt, bm, bn, bk_elems, a, plan);
+    if (a.flags & kGemmAtom32) return dispatch_atom32(in_dt, out_dt, bm, bn, bk_elems, waves, stages, a, plan);
     // a short A (at most 64 rows) is a bandwidth problem: stream B once, no CTA tiling
     if ((bm == 0 && bn == 0 && a.M <= 64 && ((int64_t)a.K * eb) % 16 == 0) || (bm == a.M && bm <= 64 && bn == 16))
         return gemm_mfma_skinny_dispatch(in_dt, out_dt, a, plan);

@@ -47,8 +47,15 @@ namespace moye {
 // kBias: the call's element-wise operation has a scalar, one-per-column or one-per-row operand or none and is no division
 // (kGemmEpiLaneOp: a bias, a ReLU, a scale): an instance of its own that is the plain kernel with that operation in the
 // lanes' own epilogue, nothing of the general one.
-template <typename In, typename Out, int BM, int BN, int WGM, int WGN, bool kOps, int AMAJ, int BMAJ, bool kRagged, bool kBias = false>
+//
+// AT = 32: the 32 x 32 MFMA forms (v_mfma_f32_32x32x16_{f16,bf16,fp8_fp8}, v_mfma_f32_32x32x2_f32), which the reference's
+// make_tiled_mma takes like any other atom (src/atom/mma.jl:80-107).  A 32 x 32 MFMA reads 32 rows of each operand and
+// half the K extent of the 16 x 16 form: lane l holds row l % 32 and the 16-byte chunk l / 32 of a 32-byte piece of that
+// row, so a fragment of a k-step is two chunks (two MFMAs in a row per accumulator tile) and the LDS tile, the loads and
+// the number of fragment reads are those of the 16 x 16 forms.  Whole tiles, K-major operands.
+template <typename In, typename Out, int BM, int BN, int WGM, int WGN, bool kOps, int AMAJ, int BMAJ, bool kRagged, bool kBias = false, int AT = 16>
 __device__ __forceinline__ void gemm_mfma_tn_lds_tile(GemmArgs p) {
+    static_assert(AT == 16 || (AT == 32 && !AMAJ && !BMAJ && !kRagged), "32 x 32 MFMA tiles: whole tiles, K-major operands");
     static_assert(!kRagged || (!AMAJ && !BMAJ), "ragged tiles: K-major operands");
     static_assert(!kBias || (!kOps && !kRagged && !AMAJ && !BMAJ), "the bias instance: whole tiles, K-major operands");
     static_assert((BM == 256 && BN == 256) || (BM == 128 && BN == 128 && WGM == 2 && WGN == 2), "tile shapes");
@@ -57,7 +64,9 @@ __device__ __forceinline__ void gemm_mfma_tn_lds_tile(GemmArgs p) {
     constexpr int NWAVES = WGM * WGN;
     constexpr int WROWS = BM / NWAVES;  // operand rows each wave brings in per tile
     constexpr int LD = WROWS / 8;       // load-to-LDS instructions per wave per operand (8 rows each)
-    constexpr int WM = BM / WGM, WN = BN / WGN, MI = WM / 16, NI = WN / 16;
+    constexpr int WM = BM / WGM, WN = BN / WGN, MI = WM / AT, NI = WN / AT;
+    constexpr int FT = AT / 16;  // 16-byte chunks (MFMAs in a row) per fragment and k-step
+    typedef float accv __attribute__((ext_vector_type(AT * AT / 64)));
 
     extern __shared__ u32x4 smem[];
 
@@ -66,7 +75,7 @@ __device__ __forceinline__ void gemm_mfma_tn_lds_tile(GemmArgs p) {
     tile_of_block(p, &tm, &tn);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm0 = (wave / WGN) * WM, wn0 = (wave % WGN) * WN;
-    const int r16 = lane & 15, kq = lane >> 4;
+    const int r16 = lane % AT, kq = lane / AT;  // row inside an MFMA tile, chunk inside the piece of a row one MFMA reads
 
     const int64_t pitch_a = (int64_t)p.lda * In::kBytes, pitch_b = (int64_t)p.ldb * In::kBytes;
     // load-to-LDS: wave w fills rows WROWS w + 8 i + l/8 (i < LD) of each operand tile; lane l brings
@@ -90,6 +99,12 @@ __device__ __forceinline__ void gemm_mfma_tn_lds_tile(GemmArgs p) {
         }
     }
     const int dma_slot = __builtin_amdgcn_readfirstlane(wave * WROWS * CPR);  // + 8 rows * CPR per i
+    // The 32 x 32 forms read rows r and r + 16 of a fragment in the same pass of a 128-bit LDS read (lanes l and l + 16), so
+    // the chunk permutation of a row also looks at bit 4 of the row: rows 16-31 of every 32 trade neighbouring chunks.
+    // On the load side that is the other 16-byte piece of a 32-byte pair for the instructions that bring such rows.
+    static_assert(AT == 16 || WROWS % 32 == 0, "bit 4 of a tile row is bit 1 of the instruction index");
+    [[maybe_unused]] const int pair_delta = (lch & 1) ? -16 : 16;
+#define MOYE_PAIR(I) (AT == 32 && (((I) >> 1) & 1) ? pair_delta : 0)
     // An M-major (N-major) operand: a k-row of the tile is TROW bytes (BM 16-bit values); wave w fills k-rows
     // KROWS w + TRPI i + l / TLPR of the tile, TRPI rows (1 KiB) per instruction; lane l brings the 16-byte chunk that
     // belongs in physical slot l % TLPR of its row.
@@ -114,14 +129,16 @@ __device__ __forceinline__ void gemm_mfma_tn_lds_tile(GemmArgs p) {
     }
     const int dma_slot_t = __builtin_amdgcn_readfirstlane(wave * KROWS * TLPR);  // + 64 chunks (TRPI rows) per i
 
-    // fragment slots: row = w?0 + 16 i + r16, chunk = 4 ks + kq
-    int fa_slot[2], fb_slot[2];
+    // fragment slots: row = w?0 + AT i + r16, chunk = 4 ks + (4 / FT) t + kq
+    int fa_slot[2][FT], fb_slot[2][FT];
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-        const int ch = 4 * ks + kq;
-        fa_slot[ks] = (wm0 + r16) * CPR + (ch ^ swz<CPR>(r16));
-        fb_slot[ks] = A_CH + (wn0 + r16) * CPR + (ch ^ swz<CPR>(r16));
-    }
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+        for (int t = 0; t < FT; ++t) {
+            const int ch = 4 * ks + (4 / FT) * t + kq, perm = swz<CPR>(r16) ^ (AT == 32 ? (r16 >> 4) & 1 : 0);
+            fa_slot[ks][t] = (wm0 + r16) * CPR + (ch ^ perm);
+            fb_slot[ks][t] = A_CH + (wn0 + r16) * CPR + (ch ^ perm);
+        }
 
     // transposed operands: byte offset of this lane's first read of 16-row block 0 of k-step 0 inside the operand tile;
     // block idx adds (idx << 5) by XOR (the piece index is swizzled), k-step ks adds 32 rows, the second read 4 rows
@@ -130,14 +147,16 @@ __device__ __forceinline__ void gemm_mfma_tn_lds_tile(GemmArgs p) {
     const int ta_lane = (8 * kq + (r16 >> 2)) * TROW + (wm0 / 128) * 256 + ((((wm0 / 16) & 7) ^ fx) << 5) + 8 * (r16 & 3);
     const int tb_lane = (8 * kq + (r16 >> 2)) * TROW + (wn0 / 128) * 256 + ((((wn0 / 16) & 7) ^ fx) << 5) + 8 * (r16 & 3);
 
-    f32x4 acc[MI][NI];
+    accv acc[MI][NI];
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
-        for (int j = 0; j < NI; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < NI; ++j)
+#pragma unroll
+            for (int e = 0; e < AT * AT / 64; ++e) acc[i][j][e] = 0.f;
 
     const int ktiles = (int)(((int64_t)p.K * In::kBytes + (kRagged ? 127 : 0)) / 128);
-    u32x4 fa[2][MI], fb[2][NI];
+    u32x4 fa[2][MI * FT], fb[2][NI * FT];  // (fragment i, chunk t at [FT i + t])
     typedef short v4s __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) v4s* tr_ptr_t;
     // the eight k of one row of a transposed operand tile: two transposing reads, 4 k-rows apart
@@ -163,7 +182,7 @@ __device__ __forceinline__ void gemm_mfma_tn_lds_tile(GemmArgs p) {
             __builtin_amdgcn_global_load_lds((gptr_t)(gA + (kKeepRowOffsets ? ro_a[kKeepRowOffsets ? i : 0] : (int64_t)min(8 * i, more_a) * pitch_a) + (int64_t)(KT) * 128 + ((KT) == ktiles - 1 ? tail_delta : 0)), \
                                              (lptr_t)((BASE) + dma_slot + 8 * CPR * i), 16, 0, 0);    \
         else                                                                                          \
-            __builtin_amdgcn_global_load_lds((gptr_t)(gA + (int64_t)(8 * i) * pitch_a + (int64_t)(KT) * 128), \
+            __builtin_amdgcn_global_load_lds((gptr_t)(gA + (int64_t)(8 * i) * pitch_a + (int64_t)(KT) * 128 + MOYE_PAIR(i)), \
                                              (lptr_t)((BASE) + dma_slot + 8 * CPR * i), 16, 0, 0);    \
         if constexpr (BMAJ)                                                                           \
             __builtin_amdgcn_global_load_lds((gptr_t)(static_cast<const char*>(p.B) + tB[i] + (int64_t)(KT) * 64 * pitch_b), \
@@ -172,14 +191,14 @@ __device__ __forceinline__ void gemm_mfma_tn_lds_tile(GemmArgs p) {
             __builtin_amdgcn_global_load_lds((gptr_t)(gB + (kKeepRowOffsets ? ro_b[kKeepRowOffsets ? i : 0] : (int64_t)min(8 * i, more_b) * pitch_b) + (int64_t)(KT) * 128 + ((KT) == ktiles - 1 ? tail_delta : 0)), \
                                              (lptr_t)((BASE) + A_CH + dma_slot + 8 * CPR * i), 16, 0, 0); \
         else                                                                                          \
-            __builtin_amdgcn_global_load_lds((gptr_t)(gB + (int64_t)(8 * i) * pitch_b + (int64_t)(KT) * 128), \
+            __builtin_amdgcn_global_load_lds((gptr_t)(gB + (int64_t)(8 * i) * pitch_b + (int64_t)(KT) * 128 + MOYE_PAIR(i)), \
                                              (lptr_t)((BASE) + A_CH + dma_slot + 8 * CPR * i), 16, 0, 0); \
     }
     // ragged K: the fragments of k-step KS of the last k-tile, in buffer BUF, keep only the pieces inside K
 #define MOYE_MASK_TAIL(KS, BUF)                                                                       \
     if (kRagged && 4 * (KS) + kq >= k_valid) {                                                        \
-        _Pragma("unroll") for (int i = 0; i < MI; ++i) fa[BUF][i] = u32x4{0u, 0u, 0u, 0u};            \
-        _Pragma("unroll") for (int j = 0; j < NI; ++j) fb[BUF][j] = u32x4{0u, 0u, 0u, 0u};            \
+        _Pragma("unroll") for (int i = 0; i < MI * FT; ++i) fa[BUF][i] = u32x4{0u, 0u, 0u, 0u};       \
+        _Pragma("unroll") for (int j = 0; j < NI * FT; ++j) fb[BUF][j] = u32x4{0u, 0u, 0u, 0u};       \
     }
     // Wait until at most N of this wave's load-to-LDS instructions are in flight and its own LDS reads
     // have returned, then meet the other waves.  A bare s_barrier on purpose: __syncthreads() adds a
@@ -195,13 +214,13 @@ __device__ __forceinline__ void gemm_mfma_tn_lds_tile(GemmArgs p) {
     }
 #define MOYE_WAIT_LDS() __builtin_amdgcn_s_waitcnt(0xC07F) /* lgkmcnt(0) only */
 #define MOYE_FRAGS(BASE, KS, BUF)                                                                     \
-    _Pragma("unroll") for (int i = 0; i < MI; ++i) {                                                  \
+    _Pragma("unroll") for (int i = 0; i < MI * FT; ++i) {                                             \
         if constexpr (AMAJ) fa[BUF][i] = tr_frag((BASE), ta_lane, i, KS);                             \
-        else fa[BUF][i] = (BASE)[fa_slot[KS] + 16 * CPR * i];                                         \
+        else fa[BUF][i] = (BASE)[fa_slot[KS][i % FT] + AT * CPR * (i / FT)];                          \
     }                                                                                                 \
-    _Pragma("unroll") for (int j = 0; j < NI; ++j) {                                                  \
+    _Pragma("unroll") for (int j = 0; j < NI * FT; ++j) {                                             \
         if constexpr (BMAJ) fb[BUF][j] = tr_frag((BASE) + A_CH, tb_lane, j, KS);                      \
-        else fb[BUF][j] = (BASE)[fb_slot[KS] + 16 * CPR * j];                                         \
+        else fb[BUF][j] = (BASE)[fb_slot[KS][j % FT] + AT * CPR * (j / FT)];                          \
     }
 // Rows of the wave tile are walked back and forth, so that exactly one operand register set changes between
 // consecutive MFMAs: with dense operands the part is power-limited, and an MFMA-only loop over an 8 x 4 register
@@ -210,7 +229,12 @@ __device__ __forceinline__ void gemm_mfma_tn_lds_tile(GemmArgs p) {
     _Pragma("unroll") for (int i = I0; i < I1; ++i)                                                   \
         _Pragma("unroll") for (int jj = 0; jj < NI; ++jj) {                                           \
             const int j = (i & 1) ? NI - 1 - jj : jj;                                                 \
-            In::mma(fb[BUF][j], fa[BUF][i], acc[i][j]);                                               \
+            if constexpr (AT == 16) {                                                                 \
+                In::mma(fb[BUF][j], fa[BUF][i], acc[i][j]);                                           \
+            } else {                                                                                  \
+                In::mma32(fb[BUF][2 * j], fa[BUF][2 * i], acc[i][j]);                                 \
+                In::mma32(fb[BUF][2 * j + 1], fa[BUF][2 * i + 1], acc[i][j]);                         \
+            }                                                                                         \
         }
 
     // Issue order inside a k-step: the two waves of a SIMD leave the barrier together, so if each one
@@ -220,17 +244,29 @@ __device__ __forceinline__ void gemm_mfma_tn_lds_tile(GemmArgs p) {
     // against 1305, 1340, 1310; with zero operands 1871 against 1773, 1846, 1761.  All eight waves of a workgroup leave the
     // barrier together, and 64 loads in as many MFMA slots are more than the vector memory pipe takes without holding
     // up the waves that issue them.)
-    constexpr int kLoadGap = 2;
+    // (the 32 x 32 forms: half as many MFMAs of twice the length per k-step, the same loads and fragment reads)
+    constexpr int kLoadGap = AT == 16 ? 2 : 1;
+    constexpr int NMMA = MI * NI * FT, NREAD = (MI + NI) * FT;  // per k-step (16-bit operands; more MFMAs per call otherwise)
 #define MOYE_INTERLEAVE(NV)                                                                           \
-    _Pragma("unroll") for (int q = 0; q < (NV); ++q) {                                                \
-        __builtin_amdgcn_sched_group_barrier(0x010, 1, 0); /* VMEM   */                               \
-        __builtin_amdgcn_sched_group_barrier(0x008, kLoadGap, 0); /* MFMA   */                        \
-    }                                                                                                 \
-    _Pragma("unroll") for (int q = 0; q < MI + NI; ++q) {                                             \
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); /* DS read */                              \
-        __builtin_amdgcn_sched_group_barrier(0x008, (MI * NI - kLoadGap * (NV)) / (MI + NI), 0);      \
-    }                                                                                                 \
-    __builtin_amdgcn_sched_group_barrier(0x008, (MI * NI - kLoadGap * (NV)) % (MI + NI), 0);
+    {                                                                                                 \
+        _Pragma("unroll") for (int q = 0; q < (NV); ++q) {                                            \
+            __builtin_amdgcn_sched_group_barrier(0x010, 1, 0); /* VMEM   */                           \
+            __builtin_amdgcn_sched_group_barrier(0x008, kLoadGap, 0); /* MFMA   */                    \
+        }                                                                                             \
+        constexpr int kLeft = NMMA - kLoadGap * (NV); /* MFMAs after the loads */                     \
+        if constexpr (kLeft >= NREAD || kLeft <= 0) {                                                 \
+            _Pragma("unroll") for (int q = 0; q < NREAD; ++q) {                                       \
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); /* DS read */                      \
+                __builtin_amdgcn_sched_group_barrier(0x008, kLeft / NREAD, 0);                        \
+            }                                                                                         \
+            __builtin_amdgcn_sched_group_barrier(0x008, kLeft % NREAD, 0);                            \
+        } else { /* fewer MFMAs than reads: several reads per MFMA */                                 \
+            _Pragma("unroll") for (int q = 0; q < kLeft; ++q) {                                       \
+                __builtin_amdgcn_sched_group_barrier(0x100, (NREAD + kLeft - 1) / kLeft, 0);          \
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                    \
+            }                                                                                         \
+        }                                                                                             \
+    }
 
     // Where in K this workgroup starts: the workgroups of one XCD (consecutive workgroup ids go to consecutive XCDs) walk K
     // together, so that the panels they share are fetched into their L2 once, but the eight XCDs start an eighth of K
@@ -293,6 +329,7 @@ __device__ __forceinline__ void gemm_mfma_tn_lds_tile(GemmArgs p) {
 #undef MOYE_MASK_TAIL
 #undef MOYE_INTERLEAVE
 #undef MOYE_DMA
+#undef MOYE_PAIR
 #undef MOYE_WAIT_BARRIER
 #undef MOYE_WAIT_LDS
 #undef MOYE_FRAGS
@@ -303,9 +340,9 @@ __device__ __forceinline__ void gemm_mfma_tn_lds_tile(GemmArgs p) {
     static_assert(NWAVES * 32 * WN * 4 <= 2 * STAGE * 16, "C patches (32 rows per wave and pass) fit in the operand stages");
     // (a kOps instance is only launched for calls with an operation or with ragged tiles: it carries the general
     // epilogue alone, which keeps the other one's registers out of its allocation)
-    if constexpr (kBias) store_c_tile<Out, MI, NI, false, true>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
-    else if constexpr (kOps) store_c_tile_general<Out, MI, NI, kRagged>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
-    else store_c_tile<Out, MI, NI, kRagged>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
+    if constexpr (kBias) store_c_tile<Out, MI, NI, false, true, false, AT>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
+    else if constexpr (kOps) store_c_tile_general<Out, MI, NI, kRagged, AT>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
+    else store_c_tile<Out, MI, NI, kRagged, false, false, AT>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
 }
 
 }  // namespace moye

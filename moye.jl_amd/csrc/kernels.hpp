@@ -111,6 +111,7 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
                               GemmArgs a, GemmPlan& plan, const TileChoice* lib = nullptr);
 int32_t gemm_mfma_tn_256_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, int waves, int stages, GemmPlan& plan);
 int32_t gemm_mfma_tn_256_pp_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, GemmPlan& plan);
+int32_t gemm_mfma_tn_256_atom32_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, GemmPlan& plan);
 int32_t gemm_mfma_tn_128_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, GemmPlan& plan, bool stage64 = false);
 int32_t gemm_mfma_tn_256_w4_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, int waves, int kstep_bytes, bool ring, GemmPlan& plan);
 int32_t gemm_mfma_tn_128_dispatch(int32_t in_dt, int32_t out_dt, GemmArgs a, GemmPlan& plan);

@@ -16,16 +16,17 @@ namespace moye {
 // kGuard: the tile may reach beyond M or N, and D need not be 16-byte aligned; rows beyond M are skipped, a piece that
 // crosses N is read and stored element by element up to N, and so is a piece of D that does not start on a 16-byte
 // boundary (a pitch of D that is not a multiple of 16 bytes).
-template <typename Out, int MI, int NI, bool kGuard = false>
-__device__ __forceinline__ void store_c_tile_general(const GemmArgs& p, const f32x4 (&acc)[MI][NI], u32x4* smem, int wave,
-                                                     int lane, int64_t m_base, int64_t n_base) {
+// AT: the MFMA tile (16 or 32; see store_c_tile).
+template <typename Out, int MI, int NI, bool kGuard = false, int AT = 16>
+__device__ __forceinline__ void store_c_tile_general(const GemmArgs& p, const float __attribute__((ext_vector_type(AT * AT / 64))) (&acc)[MI][NI],
+                                                     u32x4* smem, int wave, int lane, int64_t m_base, int64_t n_base) {
     typedef typename Out::type OutT;
-    constexpr int WN = NI * 16, PASS_MI = 2, PASS_ROWS = 32, PASSES = MI / PASS_MI;
+    constexpr int WN = NI * AT, PASS_MI = 32 / AT, PASS_ROWS = 32, PASSES = MI / PASS_MI, G = AT * AT / 256;
     constexpr int EPC = 16 / (int)sizeof(OutT);  // elements per 16-byte piece of D
     constexpr int CR = WN / 4;                   // 16-byte chunks of floats per patch row
     constexpr int OUT_CH = PASS_ROWS * (WN / EPC);  // 16-byte pieces of D per pass
     static_assert(CR >= 8 && OUT_CH % 64 == 0, "patch shape");
-    const int r16 = lane & 15, kq = lane >> 4;
+    const int r16 = lane % AT, kq = lane / AT;
     float* patch = reinterpret_cast<float*>(smem) + wave * (PASS_ROWS * WN);
     f32x4* patch16 = reinterpret_cast<f32x4*>(patch);
 #pragma unroll 1
@@ -37,10 +38,13 @@ __device__ __forceinline__ void store_c_tile_general(const GemmArgs& p, const f3
 #pragma unroll
             for (int ii = 0; ii < PASS_MI; ++ii)
 #pragma unroll
-                for (int j = 0; j < NI; ++j) {
-                    const int row = 16 * ii + r16, chunk = 4 * j + kq;
-                    patch16[row * CR + (chunk ^ (row & 7))] = acc[ps * PASS_MI + ii][j];
-                }
+                for (int j = 0; j < NI; ++j)
+#pragma unroll
+                    for (int g = 0; g < G; ++g) {
+                        const int row = AT * ii + r16, chunk = (AT / 4) * j + 2 * g + kq;
+                        const auto& a = acc[ps * PASS_MI + ii][j];
+                        patch16[row * CR + (chunk ^ (row & 7))] = f32x4{a[4 * g], a[4 * g + 1], a[4 * g + 2], a[4 * g + 3]};
+                    }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -146,7 +150,8 @@ __device__ __forceinline__ void store_c_tile_general(const GemmArgs& p, const f3
 }
 
 // acc[i][j] of a lane holds C[m = 16 i + lane % 16][n = 16 j + 4 (lane / 16) + e], e = 0..3,
-// relative to (m_base, n_base).  `smem` must be free of operand data for all waves.
+// relative to (m_base, n_base); with the 32 x 32 MFMA tiles (AT = 32) its sixteen values are
+// C[m = 32 i + lane % 32][n = 32 j + 8 g + 4 (lane / 32) + e], g = 0..3.  `smem` must be free of operand data for all waves.
 // No element-wise operation here: a call with one runs an instance whose epilogue is store_c_tile_general alone (the host
 // decides; the hand-ordered kernel has no such instance and is never sent one).
 // kGuard: the tile may reach beyond M or N and D need not be 16-byte aligned: nothing is read or stored beyond them, a
@@ -156,15 +161,15 @@ __device__ __forceinline__ void store_c_tile_general(const GemmArgs& p, const f3
 // roundings as the general epilogue, instead of sending the tile through it.
 // kNoC: the caller has no C (GemmArgs::C is null, checked on the host): nothing of C's two read paths is compiled in,
 // which frees their registers for instances that have few to spare.
-template <typename Out, int MI, int NI, bool kGuard = false, bool kLaneOp = false, bool kNoC = false>
-__device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&acc)[MI][NI], u32x4* smem, int wave,
-                                             int lane, int64_t m_base, int64_t n_base) {
+template <typename Out, int MI, int NI, bool kGuard = false, bool kLaneOp = false, bool kNoC = false, int AT = 16>
+__device__ __forceinline__ void store_c_tile(const GemmArgs& p, const float __attribute__((ext_vector_type(AT * AT / 64))) (&acc)[MI][NI], u32x4* smem,
+                                             int wave, int lane, int64_t m_base, int64_t n_base) {
     typedef typename Out::type OutT;
-    constexpr int WN = NI * 16;
+    constexpr int WN = NI * AT, G = AT * AT / 256;  // G: groups of four consecutive n per lane and MFMA tile
     constexpr int EPC = 16 / (int)sizeof(OutT);  // elements per 16-byte chunk
     constexpr int CR = WN / EPC;                 // chunks per patch row
-    constexpr int PASS_MI = 2, PASS_ROWS = PASS_MI * 16;
-    const int r16 = lane & 15, kq = lane >> 4;
+    constexpr int PASS_MI = 32 / AT, PASS_ROWS = PASS_MI * AT;
+    const int r16 = lane % AT, kq = lane / AT;
     OutT* patch = reinterpret_cast<OutT*>(smem) + wave * (PASS_ROWS * WN);
     u32x4* patch16 = reinterpret_cast<u32x4*>(patch);
     // C with unit stride along n and 16-byte aligned rows (kGemmRowC, decided on the host) comes in the way D goes
@@ -195,14 +200,14 @@ __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&ac
             for (int a = 0; a < AHEAD; ++a) fetch_c(a, cw[a]);
         }
     }
-    // a lane's columns are n_base + 16 j + 4 kq + 0..3: the operand values of a one-per-column vector, once for all rows
-    [[maybe_unused]] f32x4 xcol[kLaneOp ? NI : 1];
+    // a lane's columns are n_base + AT j + 8 g + 4 kq + 0..3: the operand values of a one-per-column vector, once for all rows
+    [[maybe_unused]] f32x4 xcol[kLaneOp ? NI * G : 1];
     [[maybe_unused]] const bool per_row = kLaneOp && p.ep_x && p.ep_xn == 0;
     if constexpr (kLaneOp) {
 #pragma unroll
-        for (int j = 0; j < NI; ++j)
+        for (int j = 0; j < NI * G; ++j)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) xcol[j][e] = per_row ? 0.f : epi_operand(p, 0, n_base + 16 * j + 4 * (lane >> 4) + e);
+            for (int e = 0; e < 4; ++e) xcol[j][e] = per_row ? 0.f : epi_operand(p, 0, n_base + AT * (j / G) + 8 * (j % G) + 4 * kq + e);
     }
 #pragma unroll
     for (int i0 = 0; i0 < MI; i0 += PASS_MI) {
@@ -224,11 +229,12 @@ __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&ac
         for (int ii = 0; ii < PASS_MI; ++ii) {
             const int i = i0 + ii;
 #pragma unroll
-            for (int j = 0; j < NI; ++j) {
-                const int row = 16 * ii + r16, col = 16 * j + 4 * kq;
+            for (int jg = 0; jg < NI * G; ++jg) {
+                const int j = jg / G, g = jg % G;
+                const int row = AT * ii + r16, col = AT * j + 8 * g + 4 * kq;
                 const int chunk = col / EPC, within = col % EPC;
                 OutT* dst = patch + (row * CR + (chunk ^ (row & 7))) * EPC + within;
-                const int64_t m = m_base + 16 * i + r16, n = n_base + 16 * j + 4 * kq;
+                const int64_t m = m_base + AT * i + r16, n = n_base + col;
                 [[maybe_unused]] float c[4] = {0.f, 0.f, 0.f, 0.f};
                 if constexpr (!kNoC) {
                     if (row_c) {
@@ -240,8 +246,8 @@ __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&ac
                             if (!kGuard || (m < p.M && n + e < p.N)) c[e] = Out::load(p.C, m * p.ldc_m + (n + e) * p.ldc_n);
                     }
                 }
-                float v[4] = {__fmul_rn(acc[i][j].x, p.alpha), __fmul_rn(acc[i][j].y, p.alpha), __fmul_rn(acc[i][j].z, p.alpha),
-                              __fmul_rn(acc[i][j].w, p.alpha)};
+                float v[4] = {__fmul_rn(acc[i][j][4 * g], p.alpha), __fmul_rn(acc[i][j][4 * g + 1], p.alpha), __fmul_rn(acc[i][j][4 * g + 2], p.alpha),
+                              __fmul_rn(acc[i][j][4 * g + 3], p.alpha)};
                 if constexpr (!kNoC) {
                     if (p.C) {
 #pragma unroll
@@ -252,7 +258,7 @@ __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&ac
                     const float xrow = per_row ? epi_operand(p, m, 0) : 0.f;
                     // the same for every element: one uniform branch per four values; the addition (a bias) and the
                     // maximum (a ReLU) are asked first, so that they pay one or two compares and not a chain of them
-#define MOYE_LANE_APPLY(OP) _Pragma("unroll") for (int e = 0; e < 4; ++e) v[e] = epi_op(OP, v[e], per_row ? xrow : xcol[j][e]);
+#define MOYE_LANE_APPLY(OP) _Pragma("unroll") for (int e = 0; e < 4; ++e) v[e] = epi_op(OP, v[e], per_row ? xrow : xcol[jg][e]);
 #define MOYE_LANE_CASE(OP) \
     case OP:               \
         MOYE_LANE_APPLY(OP) \
@@ -286,9 +292,9 @@ __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const f32x4 (&ac
             const int c = lane + 64 * t, row = c / CR, ch = c % CR;
             const u32x4 w = patch16[row * CR + (ch ^ (row & 7))];
             char* d = static_cast<char*>(p.D) +
-                      ((m_base + 16 * i0 + row) * p.ldd + n_base) * (int64_t)sizeof(OutT) + ch * 16;
+                      ((m_base + AT * i0 + row) * p.ldd + n_base) * (int64_t)sizeof(OutT) + ch * 16;
             if constexpr (kGuard) {
-                const int64_t m = m_base + 16 * i0 + row, n0 = n_base + ch * EPC;
+                const int64_t m = m_base + AT * i0 + row, n0 = n_base + ch * EPC;
                 if (m >= p.M || n0 >= p.N) continue;
                 if (n0 + EPC <= p.N && (reinterpret_cast<uintptr_t>(d) & 15) == 8) {
                     // a whole piece on an 8-byte boundary (a row pitch of 8 bytes modulo 16 puts every other row there)

@@ -90,6 +90,12 @@ def check_kernel_step(s, eb, ob):
             assert "ops=1" in name, s
         if "bias=1" in name:
             assert "lane_op" in flags and s["op"] not in (0, _lib.MAP_DIV), s
+    elif fam == "gemm_mfma_tn_256_atom32":
+        assert gx == (M // 256) * (N // 256) and s["a16"] == 1 and s["b16"] == 1 and "atom32" in flags, s
+        assert (s["lda"] * eb) % 16 == 0 and (s["ldb"] * eb) % 16 == 0, s
+        assert M % 256 == 0 and N % 256 == 0 and kb % 128 == 0 and s["d16"] == 1 and (s["ldd"] * ob) % 16 == 0 and not ragged, s
+        assert "a_m_major" not in flags and "b_n_major" not in flags, s
+        assert ("ops=1" in name) == (s["op"] != 0), s
     elif fam in ("gemm_mfma_tn_256_ring", "gemm_mfma_tn_256_pp"):
         assert M % 256 == 0 and N % 256 == 0 and kb % 64 == 0 and s["d16"] == 1 and s["op"] == 0 and not ragged, s
     elif fam == "gemm_mfma_tn":
@@ -329,9 +335,15 @@ def test_known_shapes_run_on_the_instances_they_are_meant_for():
     # mid-size problems: 128 x 128 tiles with K ranges, or 64 x 64 tiles, by the cost model; never 256 x 256 tiles with a split
     assert run_case(f16, f16, 1024, 1024, 1024, split_k=-1)["steps"][0]["tile"].startswith("64x64")
     assert run_case(f16, f16, 256, 256, 65536, split_k=-1)["steps"][0]["split"] > 1
-    # the 32 x 32 atoms: the register-staged 128 x 128 kernel; refused on the 256 x 256 tile
+    # the 32 x 32 atoms: the register-staged 128 x 128 kernel, or whole 256 x 256 tiles (named, or chosen when they fill
+    # half the chip)
     assert "atom=32" in step_names(run_case(f16, f32, 512, 512, 512, atom=mh.MFMA_F32_32x32x16_F16, cta=(128, 128, 32), waves=(2, 2, 1)))[0]
-    assert isinstance(run_case(f16, f32, 512, 512, 512, atom=mh.MFMA_F32_32x32x16_F16, cta=(256, 256, 64)), mh.MoyeError)
+    assert step_names(run_case(f16, f32, 512, 512, 512, atom=mh.MFMA_F32_32x32x16_F16, cta=(256, 256, 64)))[0] == "gemm_mfma_tn_256_atom32<InF16,OutF32,ops=0>"
+    assert step_names(run_case(f16, f16, 4096, 4096, 4096, atom=mh.MFMA_F32_32x32x16_F16))[0] == "gemm_mfma_tn_256_atom32<InF16,OutF16,ops=0>"
+    assert step_names(run_case(f16, f16, 4096, 4096, 4096, atom=mh.MFMA_F32_32x32x16_F16, ep=mh.gemm_epilogue(op=_lib.MAP_MAX, scalar=0.0)))[0] == "gemm_mfma_tn_256_atom32<InF16,OutF16,ops=1>"
+    assert "atom=32" in step_names(run_case(f16, f16, 1024, 1024, 1024, atom=mh.MFMA_F32_32x32x16_F16))[0]
+    assert isinstance(run_case(f16, f32, 500, 512, 512, atom=mh.MFMA_F32_32x32x16_F16, cta=(256, 256, 64)), mh.MoyeError)
+    assert isinstance(run_case(f16, f32, 512, 512, 512, atom=mh.MFMA_F32_32x32x16_F16, cta=(256, 256, 32)), mh.MoyeError)
     # a partitioned part (64 CUs in 2 XCDs): the same kernel, planned for fewer CUs
     p = run_case(f16, f16, 4096, 4096, 4096, cus=64)
     assert p["cus"] == 64 and p["xcds"] == 2 and p["steps"][0]["family"] == "gemm_mfma_tn_256_w4"

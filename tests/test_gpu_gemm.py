@@ -1104,12 +1104,73 @@ def test_32x32_atoms_random_and_residue_tiles(mh):
                 assert bool((frame == 77.0).all()), "stores outside D"
 
 
-def test_32x32_atoms_take_the_128_tile_only(mh):
+def test_32x32_atoms_on_256_tiles_exact_on_integers(mh):
+    """The 32x32 MFMA forms on the 256x256 CTA tile (eight waves of 4 x 2 MFMA tiles): every operand type, every output
+    type, named and left to the library, with C and alpha, with an operation in the epilogue (general form), column-major
+    D (the operands swapped); small integers, so a misplaced accumulator group or k pairing is a hard mismatch."""
+    from moye_hip import _lib
+    g = torch.Generator().manual_seed(3232)
+    for atom, _, tdt, hi, _ in _atoms32(mh):
+        eb = tdt.itemsize
+        for (M, N, K, cta) in ((256, 256, 128 // eb, (256, 256, 128 // eb)), (512, 768, 5 * 128 // eb, (256, 256, 0)), (2816, 3072, 256 // eb, (0, 0, 0))):
+            A = torch.randint(-hi, hi + 1, (M, K), generator=g).float()
+            B = torch.randint(-hi, hi + 1, (N, K), generator=g).float()
+            C = torch.randint(-9, 10, (M, N), generator=g).float()
+            X = torch.randint(-3, 4, (N,), generator=g).float()
+            a, b = A.to(tdt).cuda(), B.to(tdt).cuda()
+            ref = A.double() @ B.double().t()
+            for out_dt in (torch.float32, torch.float16, torch.bfloat16):
+                if out_dt != torch.float32 and float(ref.abs().max()) * 2 + 12 > (2048 if out_dt == torch.float16 else 256):
+                    continue        # not every integer of that size is a float of that type
+                mma = mh.tiled_mma_desc(atom, atom_layout=(2, 4, 1), cta_tile=cta)
+                d = torch.zeros(M, N, dtype=out_dt, device="cuda")
+                c = C.to(out_dt).cuda()
+                names = [s["name"] for s in mh.gemm_explain(mma, T(d), T(a), T(b))["steps"]]
+                assert names == ["gemm_mfma_tn_256_atom32<%s,%s,ops=0>" % ({2: "InF16" if tdt == torch.float16 else "InBF16", 1: "InFP8", 4: "InF32"}[eb],
+                                                                             {torch.float32: "OutF32", torch.float16: "OutF16", torch.bfloat16: "OutBF16"}[out_dt])], names
+                mh.gemm_(mma, T(d), T(a), T(b))
+                torch.cuda.synchronize()
+                assert torch.equal(d.cpu().double(), ref), (atom, M, N, K, out_dt)
+                mh.gemm_(mma, T(d), T(a), T(b), T(c), 2.0)
+                torch.cuda.synchronize()
+                assert torch.equal(d.cpu().double(), 2 * ref + C.double()), (atom, M, N, K, out_dt, "C")
+                x = X.cuda()
+                ep = mh.gemm_epilogue(alpha=1.0, beta=1.0, op=_lib.MAP_MAX, operand=T(x, (M, N), (0, 1)))
+                mh.gemm_ex_(mma, T(d), T(a), T(b), T(c), ep)
+                torch.cuda.synchronize()
+                assert torch.equal(d.cpu().double(), torch.maximum(ref + C.double(), X.double().expand(M, N))), (atom, M, N, K, out_dt, "max")
+                dt_ = torch.zeros(N, M, dtype=out_dt, device="cuda")          # column-major D
+                mh.gemm_(mma, T(dt_, (M, N), (1, M)), T(a), T(b))
+                torch.cuda.synchronize()
+                assert torch.equal(dt_.t().cpu().double(), ref), (atom, M, N, K, out_dt, "col-major")
+
+
+def test_32x32_atoms_on_256_tiles_random_against_fp64_and_limits(mh):
+    g = torch.Generator().manual_seed(3233)
+    for atom, atom16, tdt, hi, tol in _atoms32(mh):
+        M, N, K = 512, 512, 1024
+        A = (torch.randn(M, K, generator=g) * K ** -0.5).to(tdt)
+        B = (torch.randn(N, K, generator=g) * K ** -0.5).to(tdt)
+        a, b = A.cuda(), B.cuda()
+        d, d16 = torch.zeros(M, N, device="cuda"), torch.zeros(M, N, device="cuda")
+        mh.gemm_(mh.tiled_mma_desc(atom, atom_layout=(2, 4, 1), cta_tile=(256, 256, 0)), T(d), T(a), T(b))
+        mh.gemm_(mh.tiled_mma_desc(atom16, atom_layout=(2, 4, 1), cta_tile=(256, 256, 0)), T(d16), T(a), T(b))
+        torch.cuda.synchronize()
+        c64 = A.double().cuda() @ B.double().cuda().t()
+        assert relerr(d, c64) <= tol, atom
+        assert relerr(d, d16) <= 1e-5, atom            # both forms accumulate in fp32; only the order differs
+    # whole tiles only, 128 bytes of K per tile row, 2 x 4 waves
     a = torch.zeros(256, 64, dtype=torch.float16, device="cuda")
     d = torch.zeros(256, 256, dtype=torch.float16, device="cuda")
+    for kw, word in ((dict(atom_layout=(2, 4, 1), cta_tile=(256, 256, 32)), "32x32"), (dict(atom_layout=(2, 2, 1), cta_tile=(256, 256, 64)), "2 x 4 waves")):
+        with pytest.raises(mh.MoyeError) as e:
+            mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_32x32x16_F16, **kw), T(d), T(a), T(a))
+        assert word in str(e.value), str(e.value)
+    a = torch.zeros(300, 64, dtype=torch.float16, device="cuda")
+    d = torch.zeros(300, 300, dtype=torch.float16, device="cuda")
     with pytest.raises(mh.MoyeError) as e:
         mh.gemm_(mh.tiled_mma_desc(mh.MFMA_F32_32x32x16_F16, atom_layout=(2, 4, 1), cta_tile=(256, 256, 64)), T(d), T(a), T(a))
-    assert "32x32" in str(e.value)
+    assert "whole 256x256" in str(e.value)
 
 
 @pytest.mark.parametrize("M,N", [(4100, 4104), (4096 + 64, 4096), (4096, 4096 + 136), (4352 + 200, 2816 + 248)])

@@ -56,6 +56,10 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
     const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
     const int r16 = lane % AT, kq = lane / AT;   // row inside an MFMA tile, chunk inside a step
 
+    // the chunk permutation of a tile row.  A 128-bit LDS read serves lanes l and l + 16 in one pass: with the 32x32 forms
+    // those are rows r and r + 16 of a fragment, so bit 4 of the row takes part as well (rows 16-31 of every 32 trade
+    // neighbouring chunks)
+    auto perm = [](int row) { return swz<CPR>(row) ^ (AT == 32 ? (row >> 4) & 1 : 0); };
     const int64_t kbytes_a = (int64_t)p.lda * In::kBytes, kbytes_b = (int64_t)p.ldb * In::kBytes;
     const char* gA = static_cast<const char*>(p.A) + (int64_t)tm * BM * kbytes_a;
     const char* gB = static_cast<const char*>(p.B) + (int64_t)tn * BN * kbytes_b;
@@ -70,14 +74,14 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
     for (int i = 0; i < A_LD; ++i) {
         const int c = tid + 256 * i, row = c / CPR, ch = c % CPR;
         a_src[i] = gA + (kEdge ? min(row, p.M - 1 - tm * BM) : row) * kbytes_a + ch * 16;
-        a_dst[i] = row * CPR + (ch ^ swz<CPR>(row));
+        a_dst[i] = row * CPR + (ch ^ perm(row));
         a_lim[i] = (int)(kbytes - ch * 16);
     }
 #pragma unroll
     for (int i = 0; i < B_LD; ++i) {
         const int c = tid + 256 * i, row = c / CPR, ch = c % CPR;
         b_src[i] = gB + (kEdge ? min(row, p.N - 1 - tn * BN) : row) * kbytes_b + ch * 16;
-        b_dst[i] = row * CPR + (ch ^ swz<CPR>(row));
+        b_dst[i] = row * CPR + (ch ^ perm(row));
         b_lim[i] = (int)(kbytes - ch * 16);
     }
     // a chunk at byte offset koff of its row is inside the operand iff koff < lim
@@ -130,12 +134,12 @@ __global__ __launch_bounds__(256) void gemm_mfma_tn(GemmArgs p) {
 #pragma unroll
             for (int i = 0; i < MI; ++i) {
                 const int row = wm0 + AT * i + r16;
-                fa[i] = sA[row * CPR + (ch ^ swz<CPR>(row))];
+                fa[i] = sA[row * CPR + (ch ^ perm(row))];
             }
 #pragma unroll
             for (int j = 0; j < NI; ++j) {
                 const int row = wn0 + AT * j + r16;
-                fb[j] = sB[row * CPR + (ch ^ swz<CPR>(row))];
+                fb[j] = sB[row * CPR + (ch ^ perm(row))];
             }
             // rows walked back and forth: one operand register set changes between consecutive MFMAs, which
             // costs less power than two (the part is power-limited with dense operands)

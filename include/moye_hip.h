@@ -119,6 +119,10 @@ typedef struct {
                                         256x256x(128 bytes) tiles and fp8 calls run this kernel
                                         without the flag; stages = 2 keeps a 16-bit call on the
                                         compiler-scheduled two-stage kernel                       */
+#define MOYE_GEMM_NO_PERSIST 0x800    /* one workgroup per CTA tile also where the library would run
+                                        one workgroup per CU that walks over the tiles (a problem
+                                        with more 256x256 tiles than CUs and a 16-bit D; for A/B
+                                        studies)                                                  */
 
 /* copy ops: UniversalCopy (src/arch/copy/copy.jl:26-51); the LDS-staged forms stand where the
  * reference has cp.async (copy_async.jl:8-24) and ldmatrix (ldmatrix.jl:18-48) */

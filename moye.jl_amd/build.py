@@ -31,6 +31,7 @@ SOURCES = {
     "gemm_mfma256w4.hip": ["-ffp-contract=off"],
     "gemm_mfma256w4_majors.hip": ["-ffp-contract=off"],
     "gemm_mfma256w4_ops.hip": ["-ffp-contract=off"],
+    "gemm_mfma256w4_persist.hip": ["-ffp-contract=off"],
     "gemm_mfma128w4.hip": ["-ffp-contract=off"],
     "gemm_mfma128w4_majors.hip": ["-ffp-contract=off"],
     "gemm_mfma_skinny.hip": ["-ffp-contract=off"],
@@ -72,7 +73,7 @@ def _compile(item, force):
 # Kernels whose MFMAs are inline assembly: the compiler does not know how long their results take, so any
 # instruction of its own that touches an accumulator register next to them (a copy made by the register
 # allocator, an epilogue read scheduled upwards) would read a value that is not there yet, silently.
-ASM_MFMA_SOURCES = ["gemm_mfma256w4.hip", "gemm_mfma256w4_majors.hip", "gemm_mfma256w4_ops.hip", "gemm_mfma128w4.hip", "gemm_mfma128w4_majors.hip"]
+ASM_MFMA_SOURCES = ["gemm_mfma256w4.hip", "gemm_mfma256w4_majors.hip", "gemm_mfma256w4_ops.hip", "gemm_mfma256w4_persist.hip", "gemm_mfma128w4.hip", "gemm_mfma128w4_majors.hip"]
 
 
 def check_accumulator_hazards(src, force=False):

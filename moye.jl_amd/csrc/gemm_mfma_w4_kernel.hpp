@@ -295,12 +295,14 @@ struct W4F32L {
 // k-rows 4 g + e and 16 + 4 g + e (k-rows of 1 KiB, 32 per stage; the 64-byte piece index XORed with (row / 4) % 2, so
 // that the two k-rows the 32 lanes of a pass read lie in different halves of the banks).  Whole-line stages, plain calls
 // on whole tiles: the 256 x 256 tile with eight waves, the 128 x 128 tile with four (k-rows of 128 operand rows).
-template <typename In, typename Out, int WGN, bool kBias = false, bool kRagged = false, int TILE = 256, int AMAJ = 0, int BMAJ = 0, bool kOps = false, bool kNoC = false>
+template <typename In, typename Out, int WGN, bool kBias = false, bool kRagged = false, int TILE = 256, int AMAJ = 0, int BMAJ = 0, bool kOps = false, bool kNoC = false, bool kPersist = false>
 __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_256_w4(GemmArgs p) {
     static_assert(!(AMAJ || BMAJ) || (In::kRow == 128 && ((TILE == 256 && WGN == 4) || (TILE == 128 && WGN == 2)) && !kBias && !kRagged),
                   "operands that are not K-major: whole-line stages, eight waves, plain whole tiles");
     static_assert(!kRagged || (!kBias && In::kRow == 128 && !AMAJ && !BMAJ), "ragged tiles: the plain whole-line form, K-major operands");
     static_assert(!kOps || (In::kRow == 128 && TILE == 256 && WGN == 4 && !kBias && !AMAJ && !BMAJ), "epilogue operations: whole-line stages, eight waves, K-major operands");
+    static_assert(!kPersist || (In::kRow == 128 && TILE == 256 && WGN == 4 && !kRagged && !kOps && !AMAJ && !BMAJ && sizeof(typename Out::type) == 2),
+                  "the persistent form: whole-line stages, eight waves, whole tiles, K-major operands, a 16-bit D (its C patches lie beside the stages)");
     static_assert(TILE == 256 || (TILE == 128 && WGN == 2 && !kBias && (In::kRow == 128 || (In::SPS == 2 && !kRagged))),
                   "128 x 128 tiles: 2 x 2 waves; the whole-line form, plain or ragged, or the ring of 64-byte-row stages with k-steps of two stages");
     constexpr int BM = TILE, BN = TILE, kRow = In::kRow, CPR = kRow / 16, STAGES = In::kRing, SPS = In::SPS;
@@ -334,10 +336,35 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
 
     extern __shared__ __attribute__((aligned(256))) u32x4 smem[];
 
+    // kPersist: a workgroup per CU that takes tile blockIdx.x, blockIdx.x + gridDim.x, ... of the launch (problems with
+    // more tiles than CUs).  The first two stages of the next tile are requested before the epilogue of the tile just
+    // computed, whose C patches lie beside the operand stages, so the stores of one tile and the first loads of the next
+    // are in flight together and a tile's k-loop starts on data that is already there.
     int tm, tn;
     split_of_block(p);
-    tile_of_block(p, &tm, &tn);
-    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    [[maybe_unused]] int tile = blockIdx.x;
+    [[maybe_unused]] const int ntiles = p.tiles_m * p.tiles_n;
+    // (the persistent form: the tile's place comes out of integer divisions, which run on the vector unit; their inputs go
+    // through an empty statement so that no reciprocal is kept in a vector register across the k-loop, and the results
+    // are made scalars again)
+    auto locate = [&](int bid) __attribute__((always_inline)) {
+        int tiles_m = p.tiles_m, tiles_n = p.tiles_n, xcds = p.xcds, n = ntiles;
+        asm volatile("" : "+s"(tiles_m), "+s"(tiles_n), "+s"(xcds), "+s"(n), "+s"(bid));
+        tile_of_index(tiles_m, tiles_n, xcds, p.flags, bid, n, &tm, &tn);
+        tm = __builtin_amdgcn_readfirstlane(tm);
+        tn = __builtin_amdgcn_readfirstlane(tn);
+    };
+    if constexpr (kPersist) locate(tile);
+    else tile_of_block(p, &tm, &tn);
+    [[maybe_unused]] bool first_tile = true;
+    // (a persistent workgroup comes back here for every tile.  Everything a lane computes from its number is computed
+    // again: the lane number goes through an empty statement, so that none of it is kept in registers across the epilogue
+    // of the tile before, which needs them itself; a spilled value would come back through a scratch load, and a wait for
+    // that load is a wait for every store and load issued before it)
+    for (;;) {
+    int lane_now = threadIdx.x & 63;
+    if constexpr (kPersist) asm volatile("" : "+v"(lane_now));
+    const int tid = threadIdx.x, lane = lane_now, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm0 = (wave / WGN) * (BM / 2), wn0 = (wave % WGN) * WN;
     const int r16 = lane & 15, kq = lane >> 4;
 
@@ -347,15 +374,11 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
     // RW w .. RW w + RW - 1 of each operand.
     const int lrow = wave * RW + lane / CPR, lch = (lane % CPR) ^ swz<CPR>(lane / CPR);
     // (an M-major operand: its tile starts BM elements further along the row of every k)
-    const char* const a_tile = static_cast<const char*>(p.A) + (AMAJ ? (int64_t)tm * BM * In::kBytes : (int64_t)tm * BM * pitch_a);  // uniform
-    const char* const b_tile = static_cast<const char*>(p.B) + (BMAJ ? (int64_t)tn * BN * In::kBytes : (int64_t)tn * BN * pitch_b);
+    const char* a_tile = static_cast<const char*>(p.A) + (AMAJ ? (int64_t)tm * BM * In::kBytes : (int64_t)tm * BM * pitch_a);  // uniform
+    const char* b_tile = static_cast<const char*>(p.B) + (BMAJ ? (int64_t)tn * BN * In::kBytes : (int64_t)tn * BN * pitch_b);
     constexpr uint32_t kStageBytes = STAGE * 16, kATileBytes = BM * CPR * 16;
 
     f32x4 acc[MI][NI];
-#pragma unroll
-    for (int i = 0; i < MI; ++i)
-#pragma unroll
-        for (int j = 0; j < NI; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     // Ragged instances also take a K that ends inside a 128-byte row (a whole number of 16-byte pieces): the last stage
     // then holds tail_pieces valid pieces per row.  The lanes whose piece lies beyond K read the row's first piece of that
@@ -473,13 +496,29 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
     };
 #define MOYE_BLK(N) std::integral_constant<int, (N)> {}
 
-    // prologue: all five stages requested, wait for the first k-step's
+    // prologue: all stages of the ring requested, wait for the first k-step's
+    auto request_ring = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int g = 0; g < STAGES; ++g)
-        if (g < nstages) {
-            static_for<2 * LD>([&](auto qc) __attribute__((always_inline)) { dma1(g, g, qc); });
-        }
-    if (nstages >= STAGES) __builtin_amdgcn_s_waitcnt(MOYE_VMCNT(2 * LD * (STAGES - SPS)) | 0x0F70);
+        for (int g = 0; g < STAGES; ++g)
+            if (g < nstages) {
+                static_for<2 * LD>([&](auto qc) __attribute__((always_inline)) { dma1(g, g, qc); });
+            }
+    };
+    if (first_tile) request_ring();  // (a later tile of a persistent workgroup: requested before the epilogue of the tile before)
+    // (the persistent form: a zero made here, so that the compiler does not keep one in vector registers across the tiles,
+    // where it would be spilled and come back through a scratch load)
+    float zero = 0.f;
+    if constexpr (kPersist) asm volatile("v_mov_b32 %0, 0" : "=v"(zero));
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j) acc[i][j] = f32x4{zero, zero, zero, zero};
+    // A later tile of a persistent workgroup: after this tile's two stages the wave issued the previous tile's epilogue,
+    // at least sixteen 16-byte stores (128 x 64 values of 16 bits), and vector memory operations complete in the order
+    // they were issued: with at most the second stage's loads and eight more operations in flight the first stage is there.
+    constexpr int kEpilogueOps = 8;
+    if (kPersist && !first_tile && nstages >= STAGES) __builtin_amdgcn_s_waitcnt(MOYE_VMCNT(2 * LD * (STAGES - SPS) + kEpilogueOps) | 0x0F70);
+    else if (nstages >= STAGES) __builtin_amdgcn_s_waitcnt(MOYE_VMCNT(2 * LD * (STAGES - SPS)) | 0x0F70);
     else __builtin_amdgcn_s_waitcnt(0x0F70);
     MOYE_BARRIER()
     static_for<MI>([&](auto ic) __attribute__((always_inline)) {
@@ -507,7 +546,7 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
     ((P) < H * NI ? (P) / H                                                                            \
      : (P) < (MI - 2) * NI ? (((((P) - H * NI) / NI) & 1) ? ((P) - H * NI) % NI : NI - 1 - ((P) - H * NI) % NI) \
                            : ((P) - (MI - 2) * NI) / 2)
-    int slot = 0;  // ring slot of the first stage of step s
+    int slot;  // ring slot of the first stage of step s
     // One k-step.  MORE: step s+1 exists (its fragments are read); AHEAD: the stages five ahead exist
     // (they are requested, and the stages allowed to stay in flight at the barrier are the full 5 - 2 SPS).
     // Fragment reads in program order (128 x 128 wave tile): A3 A2 A1 A0 (after MFMA 28..31, each after its last
@@ -621,14 +660,10 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
     typedef std::integral_constant<bool, true> yes;
     typedef std::integral_constant<bool, false> no;
     int s = 0;
+    slot = 0;
     for (; s * SPS + STAGES + SPS <= nstages; ++s) step(yes{}, yes{}, s);
     for (; s + 1 < nsteps; ++s) step(yes{}, no{}, s);
     step(no{}, no{}, s);
-#undef MOYE_BLK
-#undef MOYE_I
-#undef MOYE_J
-#undef MOYE_VMCNT
-#undef MOYE_BARRIER
     // The accumulators were written by instructions whose latency the compiler does not know: let the last
     // ones retire before anything reads them.  The empty statements make every later read of an accumulator
     // depend on something that comes after the nops (volatile statements keep their order), so the epilogue's
@@ -641,22 +676,58 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
     for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < NI; ++j) asm volatile("" : "+a"(acc[i][j]));
-    __syncthreads();  // every wave is done with the operand ring before it becomes C patches
+    __syncthreads();  // every wave is done with the operand ring before it becomes C patches (or the next tile's stages)
 
-    if constexpr (kOps)
-        store_c_tile_general<Out, MI, NI, kRagged>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
-    else
-        store_c_tile<Out, MI, NI, kRagged, kBias, kRagged || kNoC>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
+    if constexpr (kPersist) {
+        const int64_t m_done = (int64_t)tm * BM + wm0, n_done = (int64_t)tn * BN + wn0;
+        const int next = tile + (int)gridDim.x;
+        if (next < ntiles) {
+            locate(next);
+            a_tile = static_cast<const char*>(p.A) + (int64_t)tm * BM * pitch_a;
+            b_tile = static_cast<const char*>(p.B) + (int64_t)tn * BN * pitch_b;
+            request_ring();
+        }
+        // the C patches: 32 rows of 64 16-bit values per wave, 32 KiB beside the two stages.  (The lane number goes through
+        // an empty statement so that nothing of the epilogue's per-lane address arithmetic is moved out of the loop over
+        // the tiles: it would stay in registers through the k-loop, which has none to spare, and be spilled; a reload in
+        // the epilogue waits for every store before it.)
+        int lane_here = threadIdx.x & 63;
+        asm volatile("" : "+v"(lane_here));
+        store_c_tile<Out, MI, NI, false, kBias, kNoC>(p, acc, smem + STAGES * STAGE, wave, lane_here, m_done, n_done);
+        if (next >= ntiles) break;
+        tile = next;
+        first_tile = false;
+    } else {
+        if constexpr (kOps)
+            store_c_tile_general<Out, MI, NI, kRagged>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
+        else
+            store_c_tile<Out, MI, NI, kRagged, kBias, kRagged || kNoC>(p, acc, smem, wave, lane, (int64_t)tm * BM + wm0, (int64_t)tn * BN + wn0);
+        break;
+    }
+    }  // for (;;)
+#undef MOYE_BLK
+#undef MOYE_I
+#undef MOYE_J
+#undef MOYE_VMCNT
+#undef MOYE_BARRIER
 }
 
-template <typename In, typename Out, int WGN, bool kBias = false, bool kRagged = false, int TILE = 256, int AMAJ = 0, int BMAJ = 0, bool kOps = false, bool kNoC = false>
+template <typename In, typename Out, int WGN, bool kBias = false, bool kRagged = false, int TILE = 256, int AMAJ = 0, int BMAJ = 0, bool kOps = false, bool kNoC = false,
+          bool kPersist = false>
 static int32_t launch256_w4(const GemmArgs& a, GemmPlan& plan) {
-    constexpr int kLds = In::kRing * (TILE + TILE) * In::kRow;  // all 160 KiB, or 128 KiB for two whole-line stages (64 KiB on 128 x 128 tiles)
+    // all 160 KiB, or 128 KiB for two whole-line stages (64 KiB on 128 x 128 tiles); the persistent form: 32 KiB of C patches more
+    constexpr int kLds = In::kRing * (TILE + TILE) * In::kRow + (kPersist ? 8 * 32 * 64 * 2 : 0);
     static LdsCap cap;
-    plan.add_kernel(gemm_mfma_tn_256_w4<In, Out, WGN, kBias, kRagged, TILE, AMAJ, BMAJ, kOps, kNoC>, a, (unsigned)(a.tiles_m * a.tiles_n),
+    unsigned grid = (unsigned)(a.tiles_m * a.tiles_n);
+    if constexpr (kPersist) {
+        // one workgroup per CU, a whole number of them per XCD
+        const unsigned per_round = (unsigned)(plan.shape.cus / plan.shape.xcds * plan.shape.xcds);
+        if (per_round && grid > per_round) grid = per_round;
+    }
+    plan.add_kernel(gemm_mfma_tn_256_w4<In, Out, WGN, kBias, kRagged, TILE, AMAJ, BMAJ, kOps, kNoC, kPersist>, a, grid,
                     (unsigned)(a.split > 1 ? a.split : 1), 128 * WGN, kLds, &cap, TILE, TILE, In::kRow * In::SPS, In::kDt, Out::kDt,
-                    "gemm_mfma_tn_256_w4<%s,%s,waves=%d,bias=%d,ragged=%d,tile=%d,amaj=%d,bmaj=%d,ops=%d>", In::kName, Out::kName, 2 * WGN, (int)kBias, (int)kRagged,
-                    TILE, AMAJ, BMAJ, (int)kOps);
+                    "gemm_mfma_tn_256_w4<%s,%s,waves=%d,bias=%d,ragged=%d,tile=%d,amaj=%d,bmaj=%d,ops=%d%s>", In::kName, Out::kName, 2 * WGN, (int)kBias, (int)kRagged,
+                    TILE, AMAJ, BMAJ, (int)kOps, kPersist ? ",persist=1" : "");
     return MOYE_OK;
 }
 
@@ -667,5 +738,6 @@ static int32_t launch256_w4(const GemmArgs& a, GemmPlan& plan) {
 int32_t launch256_w4_majors_dispatch(int32_t in_dt, int32_t out_dt, const GemmArgs& a, GemmPlan& plan);
 int32_t launch256_w4_ops_dispatch(int32_t in_dt, int32_t out_dt, const GemmArgs& a, GemmPlan& plan);
 int32_t launch128_w4_majors_dispatch(int32_t in_dt, int32_t out_dt, const GemmArgs& a, GemmPlan& plan);
+int32_t launch256_w4_persist_dispatch(int32_t in_dt, int32_t out_dt, const GemmArgs& a, GemmPlan& plan);
 
 }  // namespace moye

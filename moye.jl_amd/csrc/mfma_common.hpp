@@ -191,19 +191,23 @@ __device__ __forceinline__ void store_d_chunk(const GemmArgs& p, char* d, const 
 // XCDs; remapping id -> (id % 8) * (n / 8) + id / 8 hands each XCD one contiguous run of tiles,
 // and inside a run tiles are walked in bands of 8 tile-rows so that the A and B panels an
 // XCD's L2 holds are reused by the workgroups that follow.
-__device__ __forceinline__ void tile_of_block(const GemmArgs& p, int* tm, int* tn) {
-    int bid = blockIdx.x;
-    const int n = gridDim.x;
-    const int x = p.xcds;
-    if ((p.flags & 1) && x > 1 && (n % x) == 0) bid = (bid % x) * (n / x) + bid / x;
+// (`bid` of `n` tiles: a persistent kernel walks bid = blockIdx.x, blockIdx.x + gridDim.x, ... with gridDim.x a multiple of
+// the number of XCDs, so every tile of a workgroup comes from its own XCD's run)
+__device__ __forceinline__ void tile_of_index(int tiles_m, int tiles_n, int xcds, int flags, int bid, int n, int* tm, int* tn) {
+    const int x = xcds;
+    if ((flags & 1) && x > 1 && (n % x) == 0) bid = (bid % x) * (n / x) + bid / x;
     constexpr int kGroup = 8;
-    const int per_group = kGroup * p.tiles_n;
+    const int per_group = kGroup * tiles_n;
     const int g = bid / per_group;
     const int first_m = g * kGroup;
-    const int gsize = min(p.tiles_m - first_m, kGroup);
+    const int gsize = min(tiles_m - first_m, kGroup);
     const int r = bid - g * per_group;
     *tm = first_m + r % gsize;
     *tn = r / gsize;
 }
+__device__ __forceinline__ void tile_of_index(const GemmArgs& p, int bid, int n, int* tm, int* tn) {
+    tile_of_index(p.tiles_m, p.tiles_n, p.xcds, p.flags, bid, n, tm, tn);
+}
+__device__ __forceinline__ void tile_of_block(const GemmArgs& p, int* tm, int* tn) { tile_of_index(p, blockIdx.x, gridDim.x, tm, tn); }
 
 }  // namespace moye

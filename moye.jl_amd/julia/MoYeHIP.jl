@@ -107,6 +107,7 @@ const GEMM_NO_WORKSPACE = Int32(4)      # fail instead of transposing NN/NT/TT o
 const GEMM_PINGPONG = Int32(0x100)      # 256x256 tile: ping-pong schedule over a five-stage LDS ring
 const GEMM_WAVE4 = Int32(0x400)         # 256x256 tile: four waves with 128x128 wave tiles, fp8 on the 16x16x128 MFMA
 const GEMM_PREDICATE = Int32(0x200)     # compute residue tiles instead of asserting divisibility
+const GEMM_NO_PERSIST = Int32(0x800)    # one workgroup per CTA tile, never one per CU that walks over the tiles
 const COPY_UNIVERSAL = Int32(0)
 const COPY_LDS_TILED = Int32(1)
 

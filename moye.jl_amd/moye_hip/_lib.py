@@ -26,6 +26,7 @@ GMEM, SMEM, RMEM = range(3)
 COPY_UNIVERSAL, COPY_LDS_TILED = 0, 1
 GEMM_NO_XCD_SWIZZLE, GEMM_NO_LDS_SWIZZLE, GEMM_NO_WORKSPACE, GEMM_PINGPONG, GEMM_PREDICATE = 1, 2, 4, 0x100, 0x200
 GEMM_WAVE4 = 0x400
+GEMM_NO_PERSIST = 0x800
 # moye_map operations (include/moye_hip.h)
 MAP_IDENTITY, MAP_ADD, MAP_SUB, MAP_MUL, MAP_DIV, MAP_MAX, MAP_MIN, MAP_NEG, MAP_ABS = range(9)
 MAP_OPS = {"identity": 0, "add": 1, "sub": 2, "mul": 3, "div": 4, "max": 5, "min": 6, "neg": 7, "abs": 8}

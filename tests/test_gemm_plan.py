@@ -37,7 +37,7 @@ def operands(M, N, K, in_dt, out_dt, a_major="k", b_major="k", d_major="n", pad=
     return A, B, D
 
 
-def check_kernel_step(s, eb, ob):
+def check_kernel_step(s, eb, ob, cus=256, xcds=8):
     """What every kernel instance requires of the sub-problem it was given (the launchers' own documented conditions)."""
     fam, name, flags = s["family"], s["name"], s["flags"]
     M, N, K = s["M"], s["N"], s["K"]
@@ -51,7 +51,13 @@ def check_kernel_step(s, eb, ob):
     assert gy == s["split"]
     ragged = "ragged" in flags
     if fam in ("gemm_mfma_tn_256_w4", "gemm_mfma_tn_256", "gemm_mfma_tn_128", "gemm_mfma_tn_256_ring", "gemm_mfma_tn_256_pp", "gemm_mfma_tn"):
-        assert gx == -(-M // tm) * -(-N // tn), s
+        if "persist=1" in name:
+            # one workgroup per CU (a whole number per XCD) that walks over more tiles than there are CUs
+            assert fam == "gemm_mfma_tn_256_w4" and gx == cus // xcds * xcds and gx < (M // tm) * (N // tn) and gy == 1, s
+            assert "tile=256" in name and "waves=8" in name and "bias=0" in name and "ragged=0" in name and "amaj=0" in name and "bmaj=0" in name and "ops=0" in name, s
+            assert ob == 2 and s["lds"] == 163840 and name.split("<")[1].split(",")[0] in ("W4F16L", "W4BF16L", "W4FP8L"), s
+        else:
+            assert gx == -(-M // tm) * -(-N // tn), s
         assert s["a16"] == 1 and s["b16"] == 1, s
         a_m, b_n = "a_m_major" in flags, "b_n_major" in flags
         assert (s["lda"] * eb) % 16 == 0 and (s["ldb"] * eb) % 16 == 0, s
@@ -178,7 +184,7 @@ def run_case(in_dt, out_dt, M, N, K, **kw):
             for key in ("ragged=1", "bias=1", "amaj=1", "bmaj=1", "ops=1", "edge=1", "atom=32", "tile=128"):
                 if key in s["name"]:
                     SEEN.add(s["family"] + ":" + key)
-            check_kernel_step(s, eb, 4 if reduces else ob)
+            check_kernel_step(s, eb, 4 if reduces else ob, plan["cus"], plan["xcds"])
             if str(s["D"]).startswith("ws+"):
                 ws_used = max(ws_used, int(s["D"][3:]) + s["split"] * s["M"] * s["N"] * 4)
         elif s["what"] == "kmajor_copy":
@@ -266,7 +272,14 @@ def test_known_shapes_run_on_the_instances_they_are_meant_for():
     p = run_case(bf16, f32, 8192, 8192, 8192, cta=(256, 256, 64))
     assert step_names(p) == ["gemm_mfma_tn_256_w4<W4BF16L,OutF32,waves=8,bias=0,ragged=0,tile=256,amaj=0,bmaj=0,ops=0>"] and "rotate_k" in p["steps"][0]["flags"]
     p = run_case(f8, bf16, 8192, 8192, 8192, cta=(256, 256, 128))
-    assert step_names(p) == ["gemm_mfma_tn_256_w4<W4FP8L,OutBF16,waves=8,bias=0,ragged=0,tile=256,amaj=0,bmaj=0,ops=0>"]
+    # (more tiles than CUs and a 16-bit D: one workgroup per CU that walks over the tiles; not when the caller asks for a
+    # workgroup per tile, and not with an fp32 D)
+    assert step_names(p) == ["gemm_mfma_tn_256_w4<W4FP8L,OutBF16,waves=8,bias=0,ragged=0,tile=256,amaj=0,bmaj=0,ops=0,persist=1>"] and p["steps"][0]["grid"] == "256x1"
+    p = run_case(f8, bf16, 8192, 8192, 8192, cta=(256, 256, 128), flags=_lib.GEMM_NO_PERSIST)
+    assert step_names(p) == ["gemm_mfma_tn_256_w4<W4FP8L,OutBF16,waves=8,bias=0,ragged=0,tile=256,amaj=0,bmaj=0,ops=0>"] and p["steps"][0]["grid"] == "1024x1"
+    assert "persist" not in step_names(run_case(f16, f16, 4096, 4096, 4096))[0]
+    assert step_names(run_case(f16, f16, 4096, 8192, 4096))[0].endswith("ops=0,persist=1>")
+    assert step_names(run_case(f16, f16, 4096, 4096, 4096, cus=64))[0].endswith("ops=0,persist=1>")
     p = run_case(f32, f32, 8192, 8192, 8192, cta=(256, 256, 32))
     assert step_names(p) == ["gemm_mfma_tn_256_w4<W4F32L,OutF32,waves=8,bias=0,ragged=0,tile=256,amaj=0,bmaj=0,ops=0>"]
     # the reference's own operand layout (A M-major, B N-major) needs no workspace for any operand type

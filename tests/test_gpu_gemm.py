@@ -1173,6 +1173,57 @@ def test_32x32_atoms_on_256_tiles_random_against_fp64_and_limits(mh):
     assert "whole 256x256" in str(e.value)
 
 
+def test_persistent_workgroups_on_more_tiles_than_cus_exact_on_integers(mh):
+    """More 256x256 tiles than CUs and a 16-bit D: one workgroup per CU walks over the tiles, and a tile's first loads are
+    requested before the epilogue of the tile before.  Every operand type, both outputs, tile counts that are and are not
+    multiples of the CUs (and of the XCDs), K of one to nine k-steps, with and without C; exact on small integers inside
+    NaN frames, and bit-identical to a workgroup per tile."""
+    from moye_hip import _lib
+    g = torch.Generator(device="cuda").manual_seed(77)
+    atoms = {torch.float16: mh.MFMA_F32_16x16x32_F16, torch.bfloat16: mh.MFMA_F32_16x16x32_BF16, torch.float8_e4m3fn: mh.MFMA_F32_16x16x32_FP8}
+    for tdt, out_dt in ((torch.float16, torch.float16), (torch.bfloat16, torch.bfloat16), (torch.float8_e4m3fn, torch.bfloat16), (torch.float16, torch.bfloat16),
+                        (torch.float8_e4m3fn, torch.float16)):
+        eb = tdt.itemsize
+        for (M, N, K) in ((4352, 4096, 128 // eb), (8192, 8192, 256 // eb), (4352, 4352, 1152 // eb), (16384, 4352, 384 // eb)):
+            A = torch.randint(-2, 3, (M, K), generator=g, device="cuda").float() * (torch.rand(M, K, generator=g, device="cuda") < 0.25)
+            B = torch.randint(-2, 3, (N, K), generator=g, device="cuda").float() * (torch.rand(N, K, generator=g, device="cuda") < 0.25)
+            C = torch.randint(-3, 4, (M, N), generator=g, device="cuda").float()
+            a, b, c = A.to(tdt), B.to(tdt), C.to(out_dt)
+            ref = A @ B.t()
+            assert float(ref.abs().max()) * 2 + 3 <= 256
+            got = {}
+            for flags in (0, _lib.GEMM_NO_PERSIST):
+                mma = mh.tiled_mma_desc(atoms[tdt], atom_layout=(2, 4, 1), cta_tile=(256, 256, 128 // eb), flags=flags)
+                big = torch.full((M + 2, N + 16), float("nan"), dtype=out_dt, device="cuda")
+                d = big[1:M + 1, 8:8 + N]
+                name = mh.gemm_explain(mma, T(d), T(a), T(b))["steps"][0]["name"]
+                assert ("persist=1" in name) == (flags == 0), name
+                mh.gemm_(mma, T(d), T(a), T(b))
+                torch.cuda.synchronize()
+                assert torch.equal(d.float(), ref), (tdt, out_dt, M, N, K, flags)
+                mh.gemm_(mma, T(d), T(a), T(b), T(c), 2.0)
+                torch.cuda.synchronize()
+                assert torch.equal(d.float(), 2 * ref + C), (tdt, out_dt, M, N, K, flags, "C")
+                frame = big.clone()
+                frame[1:M + 1, 8:8 + N] = float("nan")
+                assert bool(torch.isnan(frame).all()), "stores outside D"
+                got[flags] = d.clone()
+            assert torch.equal(got[0].view(torch.int16), got[_lib.GEMM_NO_PERSIST].view(torch.int16))
+    # random operands: the two forms add in the same order, so they agree bit for bit
+    for tdt, out_dt in ((torch.float16, torch.float16), (torch.float8_e4m3fn, torch.bfloat16)):
+        M, N, K = 4608, 4352, 2048
+        a = (torch.randn(M, K, generator=g, device="cuda") / 8).to(tdt)
+        b = (torch.randn(N, K, generator=g, device="cuda") / 8).to(tdt)
+        outs = []
+        for flags in (0, _lib.GEMM_NO_PERSIST):
+            d = torch.zeros(M, N, dtype=out_dt, device="cuda")
+            mh.gemm_(mh.tiled_mma_desc(atoms[tdt], cta_tile=(0, 0, 0), flags=flags), T(d), T(a), T(b))
+            torch.cuda.synchronize()
+            outs.append(d)
+        assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+        assert relerr(outs[0][:256], a[:256].double() @ b.double().t()) <= TOL16
+
+
 @pytest.mark.parametrize("M,N", [(4100, 4104), (4096 + 64, 4096), (4096, 4096 + 136), (4352 + 200, 2816 + 248)])
 def test_large_ragged_problem_runs_its_interior_on_256_tiles(mh, M, N):
     """Tile left to the library, M or N not a multiple of 256, at least 128 tiles of 256 x 256 inside: interior, right

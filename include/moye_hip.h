@@ -121,8 +121,7 @@ typedef struct {
                                         compiler-scheduled two-stage kernel                       */
 #define MOYE_GEMM_NO_PERSIST 0x800    /* one workgroup per CTA tile also where the library would run
                                         one workgroup per CU that walks over the tiles (a problem
-                                        with more 256x256 tiles than CUs and a 16-bit D; for A/B
-                                        studies)                                                  */
+                                        with more 256x256 tiles than CUs; for A/B studies)        */
 
 /* copy ops: UniversalCopy (src/arch/copy/copy.jl:26-51); the LDS-staged forms stand where the
  * reference has cp.async (copy_async.jl:8-24) and ldmatrix (ldmatrix.jl:18-48) */

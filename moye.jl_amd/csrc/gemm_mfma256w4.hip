@@ -35,9 +35,9 @@ static int32_t launch256_w4_out(int32_t out_dt, const GemmArgs& a, GemmPlan& pla
             return fail(MOYE_ERR_UNSUPPORTED, "gemm!: this schedule of the hand-ordered kernel takes whole tiles only");
         }
     }
-    // more tiles than CUs, a 16-bit D: one workgroup per CU that walks over the tiles (gemm_mfma256w4_persist.hip)
+    // more tiles than CUs: one workgroup per CU that walks over the tiles (gemm_mfma256w4_persist.hip)
     if constexpr (In::kRow == 128 && WGN == 4 && In::kBytes <= 2) {
-        if ((out_dt == MOYE_F16 || out_dt == MOYE_BF16) && a.split <= 1 && (int64_t)a.tiles_m * a.tiles_n > plan.shape.cus && !(a.flags & MOYE_GEMM_NO_PERSIST))
+        if (a.split <= 1 && (int64_t)a.tiles_m * a.tiles_n > plan.shape.cus && !(a.flags & MOYE_GEMM_NO_PERSIST))
             return launch256_w4_persist_dispatch(In::kDt, out_dt, a, plan);
     }
     switch (out_dt) {

@@ -301,8 +301,8 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
                   "operands that are not K-major: whole-line stages, eight waves, plain whole tiles");
     static_assert(!kRagged || (!kBias && In::kRow == 128 && !AMAJ && !BMAJ), "ragged tiles: the plain whole-line form, K-major operands");
     static_assert(!kOps || (In::kRow == 128 && TILE == 256 && WGN == 4 && !kBias && !AMAJ && !BMAJ), "epilogue operations: whole-line stages, eight waves, K-major operands");
-    static_assert(!kPersist || (In::kRow == 128 && TILE == 256 && WGN == 4 && !kRagged && !kOps && !AMAJ && !BMAJ && sizeof(typename Out::type) == 2),
-                  "the persistent form: whole-line stages, eight waves, whole tiles, K-major operands, a 16-bit D (its C patches lie beside the stages)");
+    static_assert(!kPersist || (In::kRow == 128 && TILE == 256 && WGN == 4 && !kRagged && !kOps && !AMAJ && !BMAJ),
+                  "the persistent form: whole-line stages, eight waves, whole tiles, K-major operands (its C patches lie beside the stages)");
     static_assert(TILE == 256 || (TILE == 128 && WGN == 2 && !kBias && (In::kRow == 128 || (In::SPS == 2 && !kRagged))),
                   "128 x 128 tiles: 2 x 2 waves; the whole-line form, plain or ragged, or the ring of 64-byte-row stages with k-steps of two stages");
     constexpr int BM = TILE, BN = TILE, kRow = In::kRow, CPR = kRow / 16, STAGES = In::kRing, SPS = In::SPS;
@@ -687,13 +687,13 @@ __global__ __launch_bounds__(128 * WGN, TILE == 128 ? 2 : 1) void gemm_mfma_tn_2
             b_tile = static_cast<const char*>(p.B) + (int64_t)tn * BN * pitch_b;
             request_ring();
         }
-        // the C patches: 32 rows of 64 16-bit values per wave, 32 KiB beside the two stages.  (The lane number goes through
+        // the C patches: 32 rows of 64 16-bit values per wave (16 rows of 32-bit ones), 32 KiB beside the two stages.  (The lane number goes through
         // an empty statement so that nothing of the epilogue's per-lane address arithmetic is moved out of the loop over
         // the tiles: it would stay in registers through the k-loop, which has none to spare, and be spilled; a reload in
         // the epilogue waits for every store before it.)
         int lane_here = threadIdx.x & 63;
         asm volatile("" : "+v"(lane_here));
-        store_c_tile<Out, MI, NI, false, kBias, kNoC>(p, acc, smem + STAGES * STAGE, wave, lane_here, m_done, n_done);
+        store_c_tile<Out, MI, NI, false, kBias, kNoC, 16, sizeof(typename Out::type) == 2 ? 32 : 16>(p, acc, smem + STAGES * STAGE, wave, lane_here, m_done, n_done);
         if (next >= ntiles) break;
         tile = next;
         first_tile = false;

@@ -161,14 +161,16 @@ __device__ __forceinline__ void store_c_tile_general(const GemmArgs& p, const fl
 // roundings as the general epilogue, instead of sending the tile through it.
 // kNoC: the caller has no C (GemmArgs::C is null, checked on the host): nothing of C's two read paths is compiled in,
 // which frees their registers for instances that have few to spare.
-template <typename Out, int MI, int NI, bool kGuard = false, bool kLaneOp = false, bool kNoC = false, int AT = 16>
+// PR: rows of the wave tile per pass through the patch (32, or 16 where only half the room is there).
+template <typename Out, int MI, int NI, bool kGuard = false, bool kLaneOp = false, bool kNoC = false, int AT = 16, int PR = 32>
 __device__ __forceinline__ void store_c_tile(const GemmArgs& p, const float __attribute__((ext_vector_type(AT * AT / 64))) (&acc)[MI][NI], u32x4* smem,
                                              int wave, int lane, int64_t m_base, int64_t n_base) {
     typedef typename Out::type OutT;
     constexpr int WN = NI * AT, G = AT * AT / 256;  // G: groups of four consecutive n per lane and MFMA tile
     constexpr int EPC = 16 / (int)sizeof(OutT);  // elements per 16-byte chunk
     constexpr int CR = WN / EPC;                 // chunks per patch row
-    constexpr int PASS_MI = 32 / AT, PASS_ROWS = PASS_MI * AT;
+    static_assert(PR % AT == 0 && MI % (PR / AT) == 0, "whole MFMA tiles per pass");
+    constexpr int PASS_MI = PR / AT, PASS_ROWS = PASS_MI * AT;
     const int r16 = lane % AT, kq = lane / AT;
     OutT* patch = reinterpret_cast<OutT*>(smem) + wave * (PASS_ROWS * WN);
     u32x4* patch16 = reinterpret_cast<u32x4*>(patch);

@@ -1174,15 +1174,15 @@ def test_32x32_atoms_on_256_tiles_random_against_fp64_and_limits(mh):
 
 
 def test_persistent_workgroups_on_more_tiles_than_cus_exact_on_integers(mh):
-    """More 256x256 tiles than CUs and a 16-bit D: one workgroup per CU walks over the tiles, and a tile's first loads are
-    requested before the epilogue of the tile before.  Every operand type, both outputs, tile counts that are and are not
+    """More 256x256 tiles than CUs: one workgroup per CU walks over the tiles, and a tile's first loads are
+    requested before the epilogue of the tile before.  Every operand type, every output type, tile counts that are and are not
     multiples of the CUs (and of the XCDs), K of one to nine k-steps, with and without C; exact on small integers inside
     NaN frames, and bit-identical to a workgroup per tile."""
     from moye_hip import _lib
     g = torch.Generator(device="cuda").manual_seed(77)
     atoms = {torch.float16: mh.MFMA_F32_16x16x32_F16, torch.bfloat16: mh.MFMA_F32_16x16x32_BF16, torch.float8_e4m3fn: mh.MFMA_F32_16x16x32_FP8}
     for tdt, out_dt in ((torch.float16, torch.float16), (torch.bfloat16, torch.bfloat16), (torch.float8_e4m3fn, torch.bfloat16), (torch.float16, torch.bfloat16),
-                        (torch.float8_e4m3fn, torch.float16)):
+                        (torch.float8_e4m3fn, torch.float16), (torch.bfloat16, torch.float32), (torch.float16, torch.float32)):
         eb = tdt.itemsize
         for (M, N, K) in ((4352, 4096, 128 // eb), (8192, 8192, 256 // eb), (4352, 4352, 1152 // eb), (16384, 4352, 384 // eb)):
             A = torch.randint(-2, 3, (M, K), generator=g, device="cuda").float() * (torch.rand(M, K, generator=g, device="cuda") < 0.25)
@@ -1208,7 +1208,8 @@ def test_persistent_workgroups_on_more_tiles_than_cus_exact_on_integers(mh):
                 frame[1:M + 1, 8:8 + N] = float("nan")
                 assert bool(torch.isnan(frame).all()), "stores outside D"
                 got[flags] = d.clone()
-            assert torch.equal(got[0].view(torch.int16), got[_lib.GEMM_NO_PERSIST].view(torch.int16))
+            bits = torch.int16 if out_dt.itemsize == 2 else torch.int32
+            assert torch.equal(got[0].contiguous().view(bits), got[_lib.GEMM_NO_PERSIST].contiguous().view(bits))
     # random operands: the two forms add in the same order, so they agree bit for bit
     for tdt, out_dt in ((torch.float16, torch.float16), (torch.float8_e4m3fn, torch.bfloat16)):
         M, N, K = 4608, 4352, 2048

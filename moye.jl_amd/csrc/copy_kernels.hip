@@ -380,6 +380,77 @@ __global__ __launch_bounds__(256) void transpose_lds_b8(const uint8_t* __restric
     }
 }
 
+// The same for matrices whose source rows come in whole runs of 256 bytes: a workgroup moves a tile of 256 x 256 bytes,
+// four of the sub-tiles above side by side along i, and both sides move whole 256-byte runs per instruction: a load
+// instruction reads four source rows of 256 bytes (sixteen lanes each), a store instruction writes four destination rows
+// of 256 bytes.  (The kernel above reads and writes 64-byte pieces of sixteen rows per instruction: half lines, which the
+// address path takes several times slower, and four waves complete a destination row's run between them.)  A lane of the
+// store phase owns 4 (i) x 16 (j) bytes of each sub-tile as above; the sixteen lanes of a run read LDS rows 16 apart and
+// the four runs of a wave four neighbouring dwords, so besides the row swizzle above the dword position of a row is
+// XORed with 4 ((j / 64) % 4): the 64 dwords a wave reads at once then lie in 64 banks.  The 4 x 4 byte blocks are
+// transposed with v_perm_b32, eight per block.
+// Workgroups are numbered along the destination's contiguous index first (see transpose_lds_b32_rows), one per CU.
+__device__ __forceinline__ void transpose_bytes_4x4(uint32_t r0, uint32_t r1, uint32_t r2, uint32_t r3, uint32_t (&o)[4]) {
+    const uint32_t t0 = __builtin_amdgcn_perm(r1, r0, 0x05010400u), t1 = __builtin_amdgcn_perm(r1, r0, 0x07030602u);
+    const uint32_t t2 = __builtin_amdgcn_perm(r3, r2, 0x05010400u), t3 = __builtin_amdgcn_perm(r3, r2, 0x07030602u);
+    o[0] = __builtin_amdgcn_perm(t2, t0, 0x05040100u);
+    o[1] = __builtin_amdgcn_perm(t2, t0, 0x07060302u);
+    o[2] = __builtin_amdgcn_perm(t3, t1, 0x05040100u);
+    o[3] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
+}
+
+__global__ __launch_bounds__(256) void transpose_lds_b8_wide(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, int64_t lds_,
+                                                             int64_t ldd, int tiles_j, int64_t bs_src, int64_t bs_dst) {
+    extern __shared__ u32x4 tile[];  // four sub-tiles of 256 rows x 4 chunks
+    src += (int64_t)blockIdx.y * bs_src;
+    dst += (int64_t)blockIdx.y * bs_dst;
+    const int tj = blockIdx.x % tiles_j, gi = blockIdx.x / tiles_j;
+    // ---- load: rows j = r + 16 h, bytes i = 64 a + 16 v .. + 15: a row's sixteen lanes read 256 contiguous bytes ----
+    const int v = threadIdx.x & 3, a = (threadIdx.x >> 2) & 3, r = threadIdx.x >> 4;
+    const uint8_t* s = src + ((int64_t)tj * kTileJ8 + r) * lds_ + (int64_t)gi * 4 * kTile + 64 * a + 16 * v;
+    u32x4 x[16];
+#pragma unroll
+    for (int h = 0; h < 16; ++h) x[h] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(s + (int64_t)(16 * h) * lds_));
+#pragma unroll
+    for (int h = 0; h < 16; ++h) {
+        const int j = r + 16 * h;
+        tile[a * 1024 + lds_row_b8(j) * 4 + (v ^ ((j >> 6) & 3))] = x[h];
+    }
+    __syncthreads();
+
+    // ---- store: destination rows i = 64 a + 4 ib .. + 3, bytes j = 16 c .. 16 c + 15: sixteen lanes write 256 contiguous bytes ----
+    const uint32_t* lds32 = reinterpret_cast<const uint32_t*>(tile);
+    const int c = threadIdx.x & 15, ib = threadIdx.x >> 4;
+    uint8_t* d = dst + ((int64_t)gi * 4 * kTile + 4 * ib) * ldd + (int64_t)tj * kTileJ8 + 16 * c;
+    const int pos = ib ^ ((c >> 2) << 2);  // (16 c + q) / 64 == c / 4
+#pragma unroll
+    for (int a2 = 0; a2 < 4; ++a2) {
+        uint32_t w[16];
+#pragma unroll
+        for (int q = 0; q < 16; ++q) w[q] = lds32[a2 * 4096 + lds_row_b8(16 * c + q) * 16 + pos];  // S[16 c + q][64 a2 + 4 ib .. + 3]
+        uint32_t o[4][4];  // [g][e]
+#pragma unroll
+        for (int g = 0; g < 4; ++g) transpose_bytes_4x4(w[4 * g], w[4 * g + 1], w[4 * g + 2], w[4 * g + 3], o[g]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            __builtin_nontemporal_store(u32x4{o[0][e], o[1][e], o[2][e], o[3][e]}, reinterpret_cast<u32x4*>(d + (int64_t)(a2 * kTile + e) * ldd));
+    }
+}
+
+static int32_t launch_transpose8_wide(const uint8_t* s, uint8_t* d, int64_t lds_, int64_t ldd, int ti, int tj, hipStream_t st, int64_t bs_src = 0,
+                                      int64_t bs_dst = 0, int batch = 1) {
+    auto kern = transpose_lds_b8_wide;
+    constexpr int kLds = 96 * 1024;  // the tile needs 64 KiB; the request keeps it to one workgroup per CU (+2-3 % on large matrices)
+    static_assert(4 * kTileJ8 * kTile <= kLds, "the tile fits");
+    static LdsCap cap;
+    if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
+    const int64_t groups = (int64_t)(ti / 4) * tj;
+    if (groups >= (1 << 24)) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles for one launch (2^24 workgroups of 256)");
+    kern<<<dim3((unsigned)groups, (unsigned)batch), 256, kLds, st>>>(s, d, lds_, ldd, tj, bs_src, bs_dst);
+    MOYE_HIP_CHECK(hipGetLastError());
+    return MOYE_OK;
+}
+
 template <int GI>
 static int32_t launch_transpose8(const uint8_t* s, uint8_t* d, int64_t lds_, int64_t ldd, int ti, int tj, hipStream_t st, int64_t bs_src = 0,
                               int64_t bs_dst = 0, int batch = 1) {
@@ -881,7 +952,10 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
             if (sb == 1) {
                 const uint8_t* s8 = reinterpret_cast<const uint8_t*>(s_);
                 uint8_t* d8 = reinterpret_cast<uint8_t*>(d_);
-                if (ti % 4 == 0) return launch_transpose8<4>(s8, d8, lds_, ldd, ti, tj, st, bs, bd, batch);
+                // whole 256-byte runs on both sides, destination rows first (measured, TB/s, the 64-byte-piece kernel in
+                // super-block order / this one: 16384^2 2.91 / 4.82, 32768^2 3.20 / 5.89, 8192^2 3.29 / 4.94, 32768 x 4096
+                // 3.32 / 5.70, 4096 x 32768 3.46 / 4.99, 65536 x 16384 3.09 / 6.12; this one in super-block order 4.35-5.05)
+                if (ti % 4 == 0) return launch_transpose8_wide(s8, d8, lds_, ldd, ti, tj, st, bs, bd, batch);
                 if (ti % 2 == 0) return launch_transpose8<2>(s8, d8, lds_, ldd, ti, tj, st, bs, bd, batch);
                 return launch_transpose8<1>(s8, d8, lds_, ldd, ti, tj, st, bs, bd, batch);
             }

@@ -623,9 +623,11 @@ def test_transpose_two_byte_elements(mh, M, N):
     assert bool((dst2.view(N, ldd)[:, M:] == -1).all())
 
 
-@pytest.mark.parametrize("M,N", [(64, 256), (128, 512), (192, 256), (256, 1024), (4096, 4096), (8192, 2048), (200, 300), (1088, 784)])
+@pytest.mark.parametrize("M,N", [(64, 256), (128, 512), (192, 256), (256, 1024), (512, 256), (768, 1280), (4096, 4096), (8192, 2048), (200, 300), (1088, 784),
+                                 (16384, 12288)])
 def test_transpose_one_byte_elements(mh, M, N):
-    """fp8 matrices / bytes through the 1-byte LDS tile (64 x 256; 1, 2 or 4 sub-tiles per workgroup depending on M), sizes
+    """fp8 matrices / bytes through the 1-byte LDS tiles (256 x 256 bytes in whole 256-byte runs where M is a multiple of 256,
+    else 64 x 256 with 1 or 2 sub-tiles per workgroup), sizes
     that are not multiples of the tile through interior + strips or the general kernel: both orientations, padded pitches,
     compared as bytes; the oracle on the small cases."""
     g = torch.Generator().manual_seed(M + N)

@@ -182,6 +182,64 @@ static int32_t launch_transpose_rows(const uint32_t* s, uint32_t* d, int64_t lds
 }
 
 // ------------------------------------------------------------------------------------------
+// the same for 8-byte elements (Float64 / Int64 matrices), destination rows first
+// ------------------------------------------------------------------------------------------
+// A workgroup moves 64 (i) x 128 (j) elements, 64 KiB like the 4-byte form: a source row's piece is 512 bytes (32 lanes of
+// two elements), a destination row's 1 KiB (64 lanes of two elements).  A lane loads two elements along i from each of two
+// neighbouring source rows, turns the 2 x 2 block in registers and writes two elements along j into each of two LDS rows;
+// the chunk index of an LDS row is XORed with (row / 2) % 8.
+constexpr int kTileJ64 = 128;
+__global__ __launch_bounds__(512) void transpose_lds_b64_rows(const uint64_t* __restrict__ src, uint64_t* __restrict__ dst, int64_t lds_,
+                                                              int64_t ldd, int groups_j, int64_t bs_src, int64_t bs_dst) {
+    constexpr int JC = kTileJ64 / 2;            // 16-byte chunks (two elements) per LDS row
+    constexpr int NG = 512 / 32, NB = JC / NG;  // lanes come as 32 chunks along i x NG row pairs along j
+    extern __shared__ u32x4 tile[];             // 64 rows (i) of JC chunks (j)
+    src += (int64_t)blockIdx.y * bs_src;
+    dst += (int64_t)blockIdx.y * bs_dst;
+    const int gj = blockIdx.x % groups_j, ti = blockIdx.x / groups_j;
+    const int ic = threadIdx.x & 31;  // chunk of 2 along i
+    const int jr = threadIdx.x >> 5;  // 0..15: source rows 2 (jr + NG b) + q
+    const uint64_t* s = src + ((int64_t)gj * kTileJ64) * lds_ + (int64_t)ti * kTile + 2 * ic;
+    u32x4 v[NB][2];
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int q = 0; q < 2; ++q)
+            v[b][q] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(s + (int64_t)(2 * (jr + NG * b) + q) * lds_));
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const int row = 2 * ic + e, c = jr + NG * b;
+            tile[row * JC + (c ^ ((row >> 1) & 7))] = u32x4{v[b][0][2 * e], v[b][0][2 * e + 1], v[b][1][2 * e], v[b][1][2 * e + 1]};
+        }
+    __syncthreads();
+    // ---- store: JC consecutive lanes write one destination row of the group (1 KiB), 512 / JC rows per pass ----
+    constexpr int RPP = 512 / JC;
+    const int jc = threadIdx.x % JC, r0 = threadIdx.x / JC;
+    uint64_t* d = dst + ((int64_t)ti * kTile + r0) * ldd + (int64_t)gj * kTileJ64 + 2 * jc;
+#pragma unroll
+    for (int p = 0; p < kTile / RPP; ++p) {
+        const int row = r0 + RPP * p;
+        const u32x4 w = tile[row * JC + (jc ^ ((row >> 1) & 7))];
+        __builtin_nontemporal_store(w, reinterpret_cast<u32x4*>(d + (int64_t)(RPP * p) * ldd));
+    }
+}
+
+static int32_t launch_transpose64_rows(const uint64_t* s, uint64_t* d, int64_t lds_, int64_t ldd, int ti, int tj, hipStream_t st,
+                                       int64_t bs_src = 0, int64_t bs_dst = 0, int batch = 1) {
+    auto kern = transpose_lds_b64_rows;
+    constexpr int kLds = 96 * 1024;  // the tile needs 64 KiB; the request keeps it to one workgroup per CU
+    static LdsCap cap;
+    if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
+    const int64_t groups = (int64_t)ti * tj;
+    if (groups >= (1 << 24)) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles for one launch (2^24 workgroups of 512)");
+    kern<<<dim3((unsigned)groups, (unsigned)batch), 512, kLds, st>>>(s, d, lds_, ldd, tj, bs_src, bs_dst);
+    MOYE_HIP_CHECK(hipGetLastError());
+    return MOYE_OK;
+}
+
+// ------------------------------------------------------------------------------------------
 // the same for 2-byte elements (fp16 / bf16 matrices)
 // ------------------------------------------------------------------------------------------
 // A 64 x 64 tile is 64 source rows (j) of 128 bytes.  Rows go to LDS as they come, 16 bytes per lane,
@@ -947,8 +1005,10 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
         // whole tiles of an aligned matrix (or of `batch` such matrices bs / bd elements apart) through the LDS kernels
         auto tiled_launch = [&](const char* s_, char* d_, int64_t ni, int64_t nj, int64_t lds_, int64_t ldd, int64_t bs, int64_t bd,
                                 int batch) -> int32_t {
-            const int tile_j = sb == 1 ? kTileJ8 : kTile;
+            const int tile_j = sb == 1 ? kTileJ8 : sb == 8 ? kTileJ64 : kTile;
             const int ti = (int)(ni / kTile), tj = (int)(nj / tile_j);
+            if (sb == 8)
+                return launch_transpose64_rows(reinterpret_cast<const uint64_t*>(s_), reinterpret_cast<uint64_t*>(d_), lds_, ldd, ti, tj, st, bs, bd, batch);
             if (sb == 1) {
                 const uint8_t* s8 = reinterpret_cast<const uint8_t*>(s_);
                 uint8_t* d8 = reinterpret_cast<uint8_t*>(d_);
@@ -995,7 +1055,7 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
                     return fail(MOYE_ERR_SHAPE, "copyto!: tiler extent %d does not divide mode %d of size %lld", tc->tiler_mn[m], m + 1,
                                 (long long)src->shape[m]);
         }
-        if ((sb == 4 || sb == 2 || sb == 1) && src->rank == 2 && dst->rank == 2 && src->shape[0] == dst->shape[0] &&
+        if ((sb == 8 || sb == 4 || sb == 2 || sb == 1) && src->rank == 2 && dst->rank == 2 && src->shape[0] == dst->shape[0] &&
             src->shape[1] == dst->shape[1]) {
             const moye_tensor *a = src, *b = dst;
             bool ok = false, swap = false;
@@ -1008,7 +1068,7 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
                 const int64_t ni = a->shape[mi], nj = a->shape[mj];
                 const int64_t lds_ = a->stride[mj], ldd = b->stride[mi];
                 const int per16 = 16 / sb;  // elements per 16-byte access
-                const int tile_j = sb == 1 ? kTileJ8 : kTile;  // extent of a tile along the destination's contiguous index
+                const int tile_j = sb == 1 ? kTileJ8 : sb == 8 ? kTileJ64 : kTile;  // extent of a tile along the destination's contiguous index
                 const bool aligned = ni % kTile == 0 && nj % tile_j == 0 && lds_ % per16 == 0 && ldd % per16 == 0 &&
                                      lds_ >= ni && ldd >= nj &&
                                      (reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d)) % 16 == 0;
@@ -1045,7 +1105,7 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
         // the matrices are large enough to fill the chip on their own and few enough for the launches not to matter
         // (64 fp32 matrices of 2048 x 2048: 1.5 TB/s through the general kernel, which reads one side in single
         // elements a pitch apart).
-        if ((sb == 4 || sb == 2 || sb == 1) && src->rank == dst->rank && src->rank > 2) {
+        if ((sb == 8 || sb == 4 || sb == 2 || sb == 1) && src->rank == dst->rank && src->rank > 2) {
             const int r = src->rank;
             bool same = true;
             int mi = -1, mj = -1;
@@ -1062,7 +1122,7 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
                     if (m != mi && m != mj && src->shape[m] > 1) { bm = m; ++nbatch_modes; }
                 {
                     const int64_t ni = src->shape[mi], nj = src->shape[mj], lds_ = src->stride[mj], ldd = dst->stride[mi];
-                    const int per16 = 16 / sb, tile_j = sb == 1 ? kTileJ8 : kTile;
+                    const int per16 = 16 / sb, tile_j = sb == 1 ? kTileJ8 : sb == 8 ? kTileJ64 : kTile;
                     if (nbatch_modes == 1 && batch <= 65535 && ni % kTile == 0 && nj % tile_j == 0 && lds_ % per16 == 0 && ldd % per16 == 0 &&
                         lds_ >= ni && ldd >= nj && src->stride[bm] % per16 == 0 && dst->stride[bm] % per16 == 0 &&
                         (reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d)) % 16 == 0)

@@ -656,6 +656,40 @@ def test_transpose_one_byte_elements(mh, M, N):
         assert torch.equal(d8.view(torch.uint8), dst)
 
 
+@pytest.mark.parametrize("M,N", [(64, 128), (128, 256), (192, 384), (4096, 2048), (200, 300), (1088, 896), (8192, 4096)])
+def test_transpose_eight_byte_elements(mh, M, N):
+    """Float64 / Int64 matrices through the 8-byte LDS tile (64 x 128 elements, destination rows first), sizes that are not
+    multiples of the tile through interior + strips or the general kernel: both orientations, padded pitches, a batch of
+    matrices in one launch; compared as bits; the oracle on the small cases."""
+    g = torch.Generator().manual_seed(M * 3 + N)
+    src = torch.randint(-2 ** 62, 2 ** 62, (M * N,), dtype=torch.int64, generator=g).cuda()
+    dst = torch.zeros(M * N, dtype=torch.int64, device="cuda")
+    mh.copyto_(_tens(mh, dst, (M, N), (N, 1)), _tens(mh, src, (M, N), (1, M)))
+    torch.cuda.synchronize()
+    assert torch.equal(dst.view(M, N), src.view(N, M).t())
+    if M * N <= 128 * 256:
+        s = to.Array(src.cpu().numpy(), lo.make_layout((M, N), (1, M)))
+        d = to.Array(np.zeros(M * N, np.int64), lo.make_layout((M, N), (N, 1)))
+        to.copyto(d, s)
+        assert np.array_equal(d.buf, dst.cpu().numpy())
+    # the other orientation with padded pitches (multiples of 16 bytes), as Float64
+    lds, ldd = N + 2, M + 6
+    src2 = torch.randn(M * lds, dtype=torch.float64, generator=g).cuda()
+    dst2 = torch.full((N * ldd,), -1.0, dtype=torch.float64, device="cuda")
+    mh.copyto_(_tens(mh, dst2, (M, N), (1, ldd)), _tens(mh, src2, (M, N), (lds, 1)))
+    torch.cuda.synchronize()
+    assert torch.equal(dst2.view(N, ldd)[:, :M], src2.view(M, lds)[:, :N].t())
+    assert bool((dst2.view(N, ldd)[:, M:] == -1.0).all())
+    # a batch of three such matrices: one launch when they are whole tiles
+    if M <= 4096:
+        B = 3
+        src3 = torch.randint(-2 ** 62, 2 ** 62, (B, N, M), dtype=torch.int64, generator=g).cuda()      # [b][n][m]: m contiguous
+        dst3 = torch.zeros(B, M, N, dtype=torch.int64, device="cuda")                                  # [b][m][n]: n contiguous
+        mh.copyto_(_tens(mh, dst3, (M, N, B), (N, 1, M * N)), _tens(mh, src3, (M, N, B), (1, M, M * N)))
+        torch.cuda.synchronize()
+        assert torch.equal(dst3, src3.transpose(1, 2))
+
+
 @pytest.mark.parametrize("dt", ["uint8", "float16", "float32", "int64"])
 def test_same_shape_copies_whatever_the_order_of_the_modes(mh, dt):
     """Arrays of one shape whose unit stride sits on the last or the middle mode (row-major with a pitch, a batch of

@@ -55,10 +55,10 @@ template <bool kSwizzle, int GI>
 __global__ __launch_bounds__(256) void transpose_lds_b32(const uint32_t* __restrict__ src,
                                                          uint32_t* __restrict__ dst, int64_t lds_,
                                                          int64_t ldd, int groups_i, int tiles_j,
-                                                         int sb, int64_t bs_src, int64_t bs_dst) {
+                                                         int sb, int64_t bs_src, int64_t bs_dst, int64_t bz_src, int64_t bz_dst) {
     extern __shared__ u32x4 tile[];  // GI tiles of 64 x 16 chunks
-    src += (int64_t)blockIdx.y * bs_src;  // blockIdx.y counts the matrices of a batch
-    dst += (int64_t)blockIdx.y * bs_dst;
+    src += (int64_t)blockIdx.y * bs_src + (int64_t)blockIdx.z * bz_src;  // blockIdx.y counts the matrices of a batch
+    dst += (int64_t)blockIdx.y * bs_dst + (int64_t)blockIdx.z * bz_dst;
     int gi, tj;
     tile_coords(blockIdx.x, groups_i, tiles_j, sb, &gi, &tj);
 
@@ -98,7 +98,7 @@ __global__ __launch_bounds__(256) void transpose_lds_b32(const uint32_t* __restr
 
 template <bool kSwizzle, int GI>
 static int32_t launch_transpose(const uint32_t* s, uint32_t* d, int64_t lds_, int64_t ldd, int ti, int tj, hipStream_t st, int64_t bs_src = 0,
-                              int64_t bs_dst = 0, int batch = 1) {
+                              int64_t bs_dst = 0, int batch = 1, int64_t bz_src = 0, int64_t bz_dst = 0, int batch2 = 1) {
     auto kern = transpose_lds_b32<kSwizzle, GI>;
     constexpr int kLds = GI * kTile * kTile * 4;
     if (kLds > 48 * 1024) {
@@ -109,7 +109,7 @@ static int32_t launch_transpose(const uint32_t* s, uint32_t* d, int64_t lds_, in
     if (groups >= (1 << 24)) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles for one launch (2^24 workgroups of 256)");
     // groups are walked with the source-contiguous index fastest in bands of 64 tile columns: the
     // workgroups in flight read whole source rows and write runs of several KiB per destination row
-    kern<<<dim3((unsigned)groups, (unsigned)batch), 256, kLds, st>>>(s, d, lds_, ldd, ti / GI, tj, 64, bs_src, bs_dst);
+    kern<<<dim3((unsigned)groups, (unsigned)batch, (unsigned)batch2), 256, kLds, st>>>(s, d, lds_, ldd, ti / GI, tj, 64, bs_src, bs_dst, bz_src, bz_dst);
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;
 }
@@ -127,13 +127,13 @@ static int32_t launch_transpose(const uint32_t* s, uint32_t* d, int64_t lds_, in
 template <int GJ>
 __global__ __launch_bounds__(512) void transpose_lds_b32_rows(const uint32_t* __restrict__ src, uint32_t* __restrict__ dst,
                                                               int64_t lds_, int64_t ldd, int groups_j, int64_t bs_src,
-                                                              int64_t bs_dst) {
+                                                              int64_t bs_dst, int64_t bz_src, int64_t bz_dst) {
     constexpr int TJ = GJ * kTile, JC = TJ / 4;  // the group's extent along j, in elements and in 16-byte chunks
     constexpr int NG = 512 / 16, NB = JC / NG;   // lanes come as 16 chunks along i x NG row quads along j
     static_assert(JC % NG == 0 && 512 % JC == 0, "group shape");
     extern __shared__ u32x4 tile[];  // 64 rows (i) of JC chunks (j), the chunk index XORed with (row / 4) % 8
-    src += (int64_t)blockIdx.y * bs_src;
-    dst += (int64_t)blockIdx.y * bs_dst;
+    src += (int64_t)blockIdx.y * bs_src + (int64_t)blockIdx.z * bz_src;
+    dst += (int64_t)blockIdx.y * bs_dst + (int64_t)blockIdx.z * bz_dst;
     const int gj = blockIdx.x % groups_j, ti = blockIdx.x / groups_j;
     const int ic = threadIdx.x & 15;  // chunk of 4 along i
     const int jr = threadIdx.x >> 4;  // 0..31: source rows 4 (jr + NG b) + q
@@ -168,7 +168,7 @@ __global__ __launch_bounds__(512) void transpose_lds_b32_rows(const uint32_t* __
 
 template <int GJ>
 static int32_t launch_transpose_rows(const uint32_t* s, uint32_t* d, int64_t lds_, int64_t ldd, int ti, int tj, hipStream_t st,
-                                     int64_t bs_src = 0, int64_t bs_dst = 0, int batch = 1) {
+                                     int64_t bs_src = 0, int64_t bs_dst = 0, int batch = 1, int64_t bz_src = 0, int64_t bz_dst = 0, int batch2 = 1) {
     auto kern = transpose_lds_b32_rows<GJ>;
     constexpr int kLds = 96 * 1024;  // the tiles need GJ * 16 KiB; more than half of a CU's 160 KiB keeps it to one workgroup per CU
     static_assert(GJ * kTile * kTile * 4 <= kLds, "tiles fit");
@@ -176,7 +176,7 @@ static int32_t launch_transpose_rows(const uint32_t* s, uint32_t* d, int64_t lds
     if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
     const int64_t groups = (int64_t)ti * (tj / GJ);
     if (groups >= (1 << 24)) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles for one launch (2^24 workgroups of 512)");
-    kern<<<dim3((unsigned)groups, (unsigned)batch), 512, kLds, st>>>(s, d, lds_, ldd, tj / GJ, bs_src, bs_dst);
+    kern<<<dim3((unsigned)groups, (unsigned)batch, (unsigned)batch2), 512, kLds, st>>>(s, d, lds_, ldd, tj / GJ, bs_src, bs_dst, bz_src, bz_dst);
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;
 }
@@ -190,12 +190,12 @@ static int32_t launch_transpose_rows(const uint32_t* s, uint32_t* d, int64_t lds
 // the chunk index of an LDS row is XORed with (row / 2) % 8.
 constexpr int kTileJ64 = 128;
 __global__ __launch_bounds__(512) void transpose_lds_b64_rows(const uint64_t* __restrict__ src, uint64_t* __restrict__ dst, int64_t lds_,
-                                                              int64_t ldd, int groups_j, int64_t bs_src, int64_t bs_dst) {
+                                                              int64_t ldd, int groups_j, int64_t bs_src, int64_t bs_dst, int64_t bz_src, int64_t bz_dst) {
     constexpr int JC = kTileJ64 / 2;            // 16-byte chunks (two elements) per LDS row
     constexpr int NG = 512 / 32, NB = JC / NG;  // lanes come as 32 chunks along i x NG row pairs along j
     extern __shared__ u32x4 tile[];             // 64 rows (i) of JC chunks (j)
-    src += (int64_t)blockIdx.y * bs_src;
-    dst += (int64_t)blockIdx.y * bs_dst;
+    src += (int64_t)blockIdx.y * bs_src + (int64_t)blockIdx.z * bz_src;
+    dst += (int64_t)blockIdx.y * bs_dst + (int64_t)blockIdx.z * bz_dst;
     const int gj = blockIdx.x % groups_j, ti = blockIdx.x / groups_j;
     const int ic = threadIdx.x & 31;  // chunk of 2 along i
     const int jr = threadIdx.x >> 5;  // 0..15: source rows 2 (jr + NG b) + q
@@ -227,14 +227,14 @@ __global__ __launch_bounds__(512) void transpose_lds_b64_rows(const uint64_t* __
 }
 
 static int32_t launch_transpose64_rows(const uint64_t* s, uint64_t* d, int64_t lds_, int64_t ldd, int ti, int tj, hipStream_t st,
-                                       int64_t bs_src = 0, int64_t bs_dst = 0, int batch = 1) {
+                                       int64_t bs_src = 0, int64_t bs_dst = 0, int batch = 1, int64_t bz_src = 0, int64_t bz_dst = 0, int batch2 = 1) {
     auto kern = transpose_lds_b64_rows;
     constexpr int kLds = 96 * 1024;  // the tile needs 64 KiB; the request keeps it to one workgroup per CU
     static LdsCap cap;
     if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
     const int64_t groups = (int64_t)ti * tj;
     if (groups >= (1 << 24)) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles for one launch (2^24 workgroups of 512)");
-    kern<<<dim3((unsigned)groups, (unsigned)batch), 512, kLds, st>>>(s, d, lds_, ldd, tj, bs_src, bs_dst);
+    kern<<<dim3((unsigned)groups, (unsigned)batch, (unsigned)batch2), 512, kLds, st>>>(s, d, lds_, ldd, tj, bs_src, bs_dst, bz_src, bz_dst);
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;
 }
@@ -249,10 +249,10 @@ static int32_t launch_transpose64_rows(const uint64_t* s, uint64_t* d, int64_t l
 template <int GI>
 __global__ __launch_bounds__(256) void transpose_lds_b16(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst,
                                                          int64_t lds_, int64_t ldd, int groups_i, int tiles_j, int sb,
-                                                         int64_t bs_src, int64_t bs_dst) {
+                                                         int64_t bs_src, int64_t bs_dst, int64_t bz_src, int64_t bz_dst) {
     extern __shared__ u32x4 tile[];  // GI tiles of 64 rows x 8 chunks
-    src += (int64_t)blockIdx.y * bs_src;
-    dst += (int64_t)blockIdx.y * bs_dst;
+    src += (int64_t)blockIdx.y * bs_src + (int64_t)blockIdx.z * bz_src;
+    dst += (int64_t)blockIdx.y * bs_dst + (int64_t)blockIdx.z * bz_dst;
     int gi, tj;
     tile_coords(blockIdx.x, groups_i, tiles_j, sb, &gi, &tj);
     const int v = threadIdx.x & 7;   // 16-byte chunk inside a 128-byte run
@@ -300,7 +300,7 @@ __global__ __launch_bounds__(256) void transpose_lds_b16(const uint16_t* __restr
 
 template <int GI>
 static int32_t launch_transpose16(const uint16_t* s, uint16_t* d, int64_t lds_, int64_t ldd, int ti, int tj, hipStream_t st, int64_t bs_src = 0,
-                              int64_t bs_dst = 0, int batch = 1) {
+                              int64_t bs_dst = 0, int batch = 1, int64_t bz_src = 0, int64_t bz_dst = 0, int batch2 = 1) {
     auto kern = transpose_lds_b16<GI>;
     constexpr int kLds = GI * kTile * kTile * 2;
     if (kLds > 48 * 1024) {
@@ -309,7 +309,7 @@ static int32_t launch_transpose16(const uint16_t* s, uint16_t* d, int64_t lds_, 
     }
     const int64_t groups = (int64_t)(ti / GI) * tj;
     if (groups >= (1 << 24)) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles for one launch (2^24 workgroups of 256)");
-    kern<<<dim3((unsigned)groups, (unsigned)batch), 256, kLds, st>>>(s, d, lds_, ldd, ti / GI, tj, 64, bs_src, bs_dst);
+    kern<<<dim3((unsigned)groups, (unsigned)batch, (unsigned)batch2), 256, kLds, st>>>(s, d, lds_, ldd, ti / GI, tj, 64, bs_src, bs_dst, bz_src, bz_dst);
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;
 }
@@ -320,10 +320,10 @@ static int32_t launch_transpose16(const uint16_t* s, uint16_t* d, int64_t lds_, 
 template <int GJ>
 __global__ __launch_bounds__(256) void transpose_lds_b16_rows(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst,
                                                               int64_t lds_, int64_t ldd, int groups_j, int64_t bs_src,
-                                                              int64_t bs_dst) {
+                                                              int64_t bs_dst, int64_t bz_src, int64_t bz_dst) {
     extern __shared__ u32x4 tile[];  // GJ tiles of 64 rows x 8 chunks
-    src += (int64_t)blockIdx.y * bs_src;
-    dst += (int64_t)blockIdx.y * bs_dst;
+    src += (int64_t)blockIdx.y * bs_src + (int64_t)blockIdx.z * bz_src;
+    dst += (int64_t)blockIdx.y * bs_dst + (int64_t)blockIdx.z * bz_dst;
     const int gj = blockIdx.x % groups_j, ti = blockIdx.x / groups_j;
     const int v = threadIdx.x & 7;   // 16-byte chunk inside a 128-byte run
     const int r = threadIdx.x >> 3;  // 0..31
@@ -366,7 +366,7 @@ __global__ __launch_bounds__(256) void transpose_lds_b16_rows(const uint16_t* __
 
 template <int GJ>
 static int32_t launch_transpose16_rows(const uint16_t* s, uint16_t* d, int64_t lds_, int64_t ldd, int ti, int tj, hipStream_t st,
-                                       int64_t bs_src = 0, int64_t bs_dst = 0, int batch = 1) {
+                                       int64_t bs_src = 0, int64_t bs_dst = 0, int batch = 1, int64_t bz_src = 0, int64_t bz_dst = 0, int batch2 = 1) {
     auto kern = transpose_lds_b16_rows<GJ>;
     constexpr int kLds = 96 * 1024;  // the tiles need GJ * 8 KiB; the request keeps it to one workgroup per CU
     static_assert(GJ * kTile * kTile * 2 <= kLds, "tiles fit");
@@ -374,7 +374,7 @@ static int32_t launch_transpose16_rows(const uint16_t* s, uint16_t* d, int64_t l
     if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
     const int64_t groups = (int64_t)ti * (tj / GJ);
     if (groups >= (1 << 24)) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles for one launch (2^24 workgroups of 256)");
-    kern<<<dim3((unsigned)groups, (unsigned)batch), 256, kLds, st>>>(s, d, lds_, ldd, tj / GJ, bs_src, bs_dst);
+    kern<<<dim3((unsigned)groups, (unsigned)batch, (unsigned)batch2), 256, kLds, st>>>(s, d, lds_, ldd, tj / GJ, bs_src, bs_dst, bz_src, bz_dst);
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;
 }
@@ -394,10 +394,10 @@ __device__ __forceinline__ int lds_row_b8(int j) { return (j & ~3) | ((j & 3) ^ 
 template <int GI>
 __global__ __launch_bounds__(256) void transpose_lds_b8(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, int64_t lds_,
                                                         int64_t ldd, int groups_i, int tiles_j, int sb, int64_t bs_src,
-                                                        int64_t bs_dst) {
+                                                        int64_t bs_dst, int64_t bz_src, int64_t bz_dst) {
     extern __shared__ u32x4 tile[];  // GI sub-tiles of 256 rows x 4 chunks
-    src += (int64_t)blockIdx.y * bs_src;
-    dst += (int64_t)blockIdx.y * bs_dst;
+    src += (int64_t)blockIdx.y * bs_src + (int64_t)blockIdx.z * bz_src;
+    dst += (int64_t)blockIdx.y * bs_dst + (int64_t)blockIdx.z * bz_dst;
     int gi, tj;
     tile_coords(blockIdx.x, groups_i, tiles_j, sb, &gi, &tj);
     const int v = threadIdx.x & 3;   // 16-byte chunk of a 64-byte row
@@ -458,10 +458,10 @@ __device__ __forceinline__ void transpose_bytes_4x4(uint32_t r0, uint32_t r1, ui
 }
 
 __global__ __launch_bounds__(256) void transpose_lds_b8_wide(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, int64_t lds_,
-                                                             int64_t ldd, int tiles_j, int64_t bs_src, int64_t bs_dst) {
+                                                             int64_t ldd, int tiles_j, int64_t bs_src, int64_t bs_dst, int64_t bz_src, int64_t bz_dst) {
     extern __shared__ u32x4 tile[];  // four sub-tiles of 256 rows x 4 chunks
-    src += (int64_t)blockIdx.y * bs_src;
-    dst += (int64_t)blockIdx.y * bs_dst;
+    src += (int64_t)blockIdx.y * bs_src + (int64_t)blockIdx.z * bz_src;
+    dst += (int64_t)blockIdx.y * bs_dst + (int64_t)blockIdx.z * bz_dst;
     const int tj = blockIdx.x % tiles_j, gi = blockIdx.x / tiles_j;
     // ---- load: rows j = r + 16 h, bytes i = 64 a + 16 v .. + 15: a row's sixteen lanes read 256 contiguous bytes ----
     const int v = threadIdx.x & 3, a = (threadIdx.x >> 2) & 3, r = threadIdx.x >> 4;
@@ -496,7 +496,7 @@ __global__ __launch_bounds__(256) void transpose_lds_b8_wide(const uint8_t* __re
 }
 
 static int32_t launch_transpose8_wide(const uint8_t* s, uint8_t* d, int64_t lds_, int64_t ldd, int ti, int tj, hipStream_t st, int64_t bs_src = 0,
-                                      int64_t bs_dst = 0, int batch = 1) {
+                                      int64_t bs_dst = 0, int batch = 1, int64_t bz_src = 0, int64_t bz_dst = 0, int batch2 = 1) {
     auto kern = transpose_lds_b8_wide;
     constexpr int kLds = 96 * 1024;  // the tile needs 64 KiB; the request keeps it to one workgroup per CU (+2-3 % on large matrices)
     static_assert(4 * kTileJ8 * kTile <= kLds, "the tile fits");
@@ -504,14 +504,14 @@ static int32_t launch_transpose8_wide(const uint8_t* s, uint8_t* d, int64_t lds_
     if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
     const int64_t groups = (int64_t)(ti / 4) * tj;
     if (groups >= (1 << 24)) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles for one launch (2^24 workgroups of 256)");
-    kern<<<dim3((unsigned)groups, (unsigned)batch), 256, kLds, st>>>(s, d, lds_, ldd, tj, bs_src, bs_dst);
+    kern<<<dim3((unsigned)groups, (unsigned)batch, (unsigned)batch2), 256, kLds, st>>>(s, d, lds_, ldd, tj, bs_src, bs_dst, bz_src, bz_dst);
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;
 }
 
 template <int GI>
 static int32_t launch_transpose8(const uint8_t* s, uint8_t* d, int64_t lds_, int64_t ldd, int ti, int tj, hipStream_t st, int64_t bs_src = 0,
-                              int64_t bs_dst = 0, int batch = 1) {
+                              int64_t bs_dst = 0, int batch = 1, int64_t bz_src = 0, int64_t bz_dst = 0, int batch2 = 1) {
     auto kern = transpose_lds_b8<GI>;
     constexpr int kLds = GI * kTileJ8 * kTile;
     if (kLds > 48 * 1024) {
@@ -520,7 +520,7 @@ static int32_t launch_transpose8(const uint8_t* s, uint8_t* d, int64_t lds_, int
     }
     const int64_t groups = (int64_t)(ti / GI) * tj;
     if (groups >= (1 << 24)) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles for one launch (2^24 workgroups of 256)");
-    kern<<<dim3((unsigned)groups, (unsigned)batch), 256, kLds, st>>>(s, d, lds_, ldd, ti / GI, tj, 64, bs_src, bs_dst);
+    kern<<<dim3((unsigned)groups, (unsigned)batch, (unsigned)batch2), 256, kLds, st>>>(s, d, lds_, ldd, ti / GI, tj, 64, bs_src, bs_dst, bz_src, bz_dst);
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;
 }
@@ -1002,22 +1002,57 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
             MOYE_HIP_CHECK(hipGetLastError());
             return MOYE_OK;
         }
+        // Arrays of one shape of rank three and more: modes of extent 1 go, and modes that are neighbours in memory on both
+        // sides become one (NCHW -> NHWC: H and W), so that what follows sees a matrix or a batch of matrices where there is
+        // one (the tiler of the descriptor speaks of the caller's modes: it is checked here, then dropped)
+        if (src->rank == dst->rank && src->rank > 2) {
+            bool same = true;
+            for (int m = 0; m < src->rank; ++m) same = same && src->shape[m] == dst->shape[m];
+            moye_tensor cs = *src, cd = *dst;
+            int r = 0;
+            for (int m = 0; same && m < src->rank; ++m) {
+                if (src->shape[m] == 1) continue;
+                if (r > 0 && src->stride[m] == cs.stride[r - 1] * cs.shape[r - 1] && dst->stride[m] == cd.stride[r - 1] * cd.shape[r - 1]) {
+                    cs.shape[r - 1] *= src->shape[m];
+                    cd.shape[r - 1] = cs.shape[r - 1];
+                } else {
+                    cs.shape[r] = cd.shape[r] = src->shape[m];
+                    cs.stride[r] = src->stride[m];
+                    cd.stride[r] = dst->stride[m];
+                    ++r;
+                }
+            }
+            if (same && r >= 1 && r < src->rank) {
+                moye_tiled_copy plain{};
+                if (tc) {
+                    if (tc->op == MOYE_COPY_LDS_TILED)
+                        for (int m = 0; m < 2; ++m)
+                            if (tc->tiler_mn[m] < 0 || (tc->tiler_mn[m] > 0 && src->shape[m] % tc->tiler_mn[m]))
+                                return fail(MOYE_ERR_SHAPE, "copyto!: tiler extent %d does not divide mode %d of size %lld", tc->tiler_mn[m], m + 1,
+                                            (long long)src->shape[m]);
+                    plain = *tc;
+                    plain.tiler_mn[0] = plain.tiler_mn[1] = 0;
+                }
+                cs.rank = cd.rank = r;
+                return copy_if_dispatch(tc ? &plain : nullptr, &cd, &cs, nullptr, st);
+            }
+        }
         // whole tiles of an aligned matrix (or of `batch` such matrices bs / bd elements apart) through the LDS kernels
         auto tiled_launch = [&](const char* s_, char* d_, int64_t ni, int64_t nj, int64_t lds_, int64_t ldd, int64_t bs, int64_t bd,
-                                int batch) -> int32_t {
+                                int batch, int64_t bs2 = 0, int64_t bd2 = 0, int batch2 = 1) -> int32_t {
             const int tile_j = sb == 1 ? kTileJ8 : sb == 8 ? kTileJ64 : kTile;
             const int ti = (int)(ni / kTile), tj = (int)(nj / tile_j);
             if (sb == 8)
-                return launch_transpose64_rows(reinterpret_cast<const uint64_t*>(s_), reinterpret_cast<uint64_t*>(d_), lds_, ldd, ti, tj, st, bs, bd, batch);
+                return launch_transpose64_rows(reinterpret_cast<const uint64_t*>(s_), reinterpret_cast<uint64_t*>(d_), lds_, ldd, ti, tj, st, bs, bd, batch, bs2, bd2, batch2);
             if (sb == 1) {
                 const uint8_t* s8 = reinterpret_cast<const uint8_t*>(s_);
                 uint8_t* d8 = reinterpret_cast<uint8_t*>(d_);
                 // whole 256-byte runs on both sides, destination rows first (measured, TB/s, the 64-byte-piece kernel in
                 // super-block order / this one: 16384^2 2.91 / 4.82, 32768^2 3.20 / 5.89, 8192^2 3.29 / 4.94, 32768 x 4096
                 // 3.32 / 5.70, 4096 x 32768 3.46 / 4.99, 65536 x 16384 3.09 / 6.12; this one in super-block order 4.35-5.05)
-                if (ti % 4 == 0) return launch_transpose8_wide(s8, d8, lds_, ldd, ti, tj, st, bs, bd, batch);
-                if (ti % 2 == 0) return launch_transpose8<2>(s8, d8, lds_, ldd, ti, tj, st, bs, bd, batch);
-                return launch_transpose8<1>(s8, d8, lds_, ldd, ti, tj, st, bs, bd, batch);
+                if (ti % 4 == 0) return launch_transpose8_wide(s8, d8, lds_, ldd, ti, tj, st, bs, bd, batch, bs2, bd2, batch2);
+                if (ti % 2 == 0) return launch_transpose8<2>(s8, d8, lds_, ldd, ti, tj, st, bs, bd, batch, bs2, bd2, batch2);
+                return launch_transpose8<1>(s8, d8, lds_, ldd, ti, tj, st, bs, bd, batch, bs2, bd2, batch2);
             }
             if (sb == 2) {
                 const uint16_t* s16 = reinterpret_cast<const uint16_t*>(s_);
@@ -1025,24 +1060,24 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
                 // measured, TB/s, source-first / destination-first: 16384^2 5.32 / 5.75, 4096^2 x 16 6.25 / 6.47, 32768 x 4096
                 // 4.07 / 6.10; 2048^2 x 64 5.83 / 5.18, 4096 x 32768 5.65 / 4.46
                 if (tj % 8 == 0 && ni >= nj && ni >= 3072)
-                    return launch_transpose16_rows<8>(s16, d16, lds_, ldd, ti, tj, st, bs, bd, batch);
-                if (ti % 8 == 0) return launch_transpose16<8>(s16, d16, lds_, ldd, ti, tj, st, bs, bd, batch);
-                if (ti % 4 == 0) return launch_transpose16<4>(s16, d16, lds_, ldd, ti, tj, st, bs, bd, batch);
-                if (ti % 2 == 0) return launch_transpose16<2>(s16, d16, lds_, ldd, ti, tj, st, bs, bd, batch);
-                return launch_transpose16<1>(s16, d16, lds_, ldd, ti, tj, st, bs, bd, batch);
+                    return launch_transpose16_rows<8>(s16, d16, lds_, ldd, ti, tj, st, bs, bd, batch, bs2, bd2, batch2);
+                if (ti % 8 == 0) return launch_transpose16<8>(s16, d16, lds_, ldd, ti, tj, st, bs, bd, batch, bs2, bd2, batch2);
+                if (ti % 4 == 0) return launch_transpose16<4>(s16, d16, lds_, ldd, ti, tj, st, bs, bd, batch, bs2, bd2, batch2);
+                if (ti % 2 == 0) return launch_transpose16<2>(s16, d16, lds_, ldd, ti, tj, st, bs, bd, batch, bs2, bd2, batch2);
+                return launch_transpose16<1>(s16, d16, lds_, ldd, ti, tj, st, bs, bd, batch, bs2, bd2, batch2);
             }
             const uint32_t* s32 = reinterpret_cast<const uint32_t*>(s_);
             uint32_t* d32 = reinterpret_cast<uint32_t*>(d_);
-            if (tc && (tc->flags & MOYE_GEMM_NO_LDS_SWIZZLE)) return launch_transpose<false, 1>(s32, d32, lds_, ldd, ti, tj, st, bs, bd, batch);
+            if (tc && (tc->flags & MOYE_GEMM_NO_LDS_SWIZZLE)) return launch_transpose<false, 1>(s32, d32, lds_, ldd, ti, tj, st, bs, bd, batch, bs2, bd2, batch2);
             // Destination rows first (transpose_lds_b32_rows) when the source's contiguous extent is at least the destination's
             // and 2048 or more; measured, TB/s, source-first / destination-first order: 16384^2 5.68 / 6.25, 12288^2 5.20 / 5.94,
             // 4096^2 x 16 5.81 / 6.02, 2048^2 x 64 6.30 / 6.48, 32768 x 4096 4.33 / 6.39; the other way round 4096 x 32768
             // 5.58 / 5.08, 2048 x 65536 5.77 / 4.52, 1024^2 x 128 6.03 / 5.86.
             if (tj % 4 == 0 && ni >= nj && ni >= 2048)
-                return launch_transpose_rows<4>(s32, d32, lds_, ldd, ti, tj, st, bs, bd, batch);
-            if (ti % 4 == 0) return launch_transpose<true, 4>(s32, d32, lds_, ldd, ti, tj, st, bs, bd, batch);
-            if (ti % 2 == 0) return launch_transpose<true, 2>(s32, d32, lds_, ldd, ti, tj, st, bs, bd, batch);
-            return launch_transpose<true, 1>(s32, d32, lds_, ldd, ti, tj, st, bs, bd, batch);
+                return launch_transpose_rows<4>(s32, d32, lds_, ldd, ti, tj, st, bs, bd, batch, bs2, bd2, batch2);
+            if (ti % 4 == 0) return launch_transpose<true, 4>(s32, d32, lds_, ldd, ti, tj, st, bs, bd, batch, bs2, bd2, batch2);
+            if (ti % 2 == 0) return launch_transpose<true, 2>(s32, d32, lds_, ldd, ti, tj, st, bs, bd, batch, bs2, bd2, batch2);
+            return launch_transpose<true, 1>(s32, d32, lds_, ldd, ti, tj, st, bs, bd, batch, bs2, bd2, batch2);
         };
         // (2) rank-2 transpose of 1-, 2- and 4-byte elements through LDS patches
         bool lds_pair = false;  // a rank-2 pair with the unit strides on different modes: what the LDS-tiled op is for
@@ -1101,7 +1136,7 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
         }
         // (2b) a batch of such transposes: arrays of one shape, rank above two, the unit strides of the two sides on
         // different modes of 64 and more; every other mode counts matrices.  One launch with the matrix index in the
-        // grid when there is one such mode and the matrices are whole aligned tiles; else one rank-2 call per matrix while
+        // grid when there are one or two such modes and the matrices are whole aligned tiles; else one rank-2 call per matrix while
         // the matrices are large enough to fill the chip on their own and few enough for the launches not to matter
         // (64 fp32 matrices of 2048 x 2048: 1.5 TB/s through the general kernel, which reads one side in single
         // elements a pitch apart).
@@ -1116,17 +1151,26 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
             }
             if (same && mi >= 0 && mj >= 0 && mi != mj && src->shape[mi] >= kTile && src->shape[mj] >= kTile) {
                 const int64_t per = src->shape[mi] * src->shape[mj], batch = n / per;
-                // one batch mode, whole aligned tiles: one launch, the matrix index in the grid
-                int bm = -1, nbatch_modes = 0;
+                // one or two batch modes, whole aligned tiles: one launch, the matrix indices in the grid
+                // (fp16 [16, 2048, 32, 128] -> [16, 32, 128, 2048], 512 matrices in two modes: 1645 us as 512 launches)
+                int bm[2] = {-1, -1}, nbatch_modes = 0;
                 for (int m = 0; m < r; ++m)
-                    if (m != mi && m != mj && src->shape[m] > 1) { bm = m; ++nbatch_modes; }
-                {
+                    if (m != mi && m != mj && src->shape[m] > 1) {
+                        if (nbatch_modes < 2) bm[nbatch_modes] = m;
+                        ++nbatch_modes;
+                    }
+                if (nbatch_modes == 1 || nbatch_modes == 2) {
                     const int64_t ni = src->shape[mi], nj = src->shape[mj], lds_ = src->stride[mj], ldd = dst->stride[mi];
                     const int per16 = 16 / sb, tile_j = sb == 1 ? kTileJ8 : sb == 8 ? kTileJ64 : kTile;
-                    if (nbatch_modes == 1 && batch <= 65535 && ni % kTile == 0 && nj % tile_j == 0 && lds_ % per16 == 0 && ldd % per16 == 0 &&
-                        lds_ >= ni && ldd >= nj && src->stride[bm] % per16 == 0 && dst->stride[bm] % per16 == 0 &&
-                        (reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d)) % 16 == 0)
-                        return tiled_launch(s, d, ni, nj, lds_, ldd, src->stride[bm], dst->stride[bm], (int)batch);
+                    bool fits = ni % kTile == 0 && nj % tile_j == 0 && lds_ % per16 == 0 && ldd % per16 == 0 && lds_ >= ni && ldd >= nj &&
+                                (reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d)) % 16 == 0;
+                    for (int b = 0; b < nbatch_modes; ++b)
+                        fits = fits && src->shape[bm[b]] <= 65535 && src->stride[bm[b]] % per16 == 0 && dst->stride[bm[b]] % per16 == 0;
+                    if (fits) {
+                        const bool two = nbatch_modes == 2;
+                        return tiled_launch(s, d, ni, nj, lds_, ldd, src->stride[bm[0]], dst->stride[bm[0]], (int)src->shape[bm[0]],
+                                            two ? src->stride[bm[1]] : 0, two ? dst->stride[bm[1]] : 0, two ? (int)src->shape[bm[1]] : 1);
+                    }
                 }
                 if (batch <= 4096 && per * sb >= (128 << 10)) {
                     moye_tensor ps = *src, pd = *dst;

@@ -690,6 +690,43 @@ def test_transpose_eight_byte_elements(mh, M, N):
         assert torch.equal(dst3, src3.transpose(1, 2))
 
 
+@pytest.mark.parametrize("dt", ["uint8", "float16", "float32", "float64"])
+def test_permutations_that_are_batches_of_transposes(mh, dt):
+    """Rank-4 permutations whose modes merge into a batch of matrices (NCHW <-> NHWC: H and W are neighbours in memory on
+    both sides) or that count matrices in two modes ([B, S, H, D] -> [B, H, D, S]); one launch each where the matrices are
+    whole tiles, the rank-2 route per matrix otherwise.  Against torch's permute, as bits."""
+    tdt = getattr(torch, dt)
+    g = torch.Generator().manual_seed(41)
+
+    def rand(*shape):
+        n = int(np.prod(shape))
+        return torch.randint(0, 256, (n * tdt.itemsize,), dtype=torch.uint8, generator=g).view(tdt).view(*shape).cuda()
+
+    def check(x, perm):
+        view = x.permute(*perm)
+        want = view.contiguous()
+        dst = torch.zeros_like(want)
+        shape = tuple(reversed(want.shape))
+        mh.copyto_(_tens(mh, dst, shape, tuple(reversed(dst.stride()))), _tens(mh, x, shape, tuple(reversed(view.stride()))))
+        torch.cuda.synchronize()
+        bits = {1: torch.uint8, 2: torch.int16, 4: torch.int32, 8: torch.int64}[tdt.itemsize]
+        assert torch.equal(dst.view(bits), want.view(bits)), (dt, tuple(x.shape), perm)
+
+    x = rand(3, 256, 16, 16)          # NCHW, H W = 256: whole tiles for every element size
+    check(x, (0, 2, 3, 1))
+    check(x.permute(0, 2, 3, 1).contiguous(), (0, 3, 1, 2))
+    x = rand(2, 128, 14, 14)          # H W = 196: ragged matrices
+    check(x, (0, 2, 3, 1))
+    check(x.permute(0, 2, 3, 1).contiguous(), (0, 3, 1, 2))
+    x = rand(2, 256, 3, 128)          # [B, S, H, D] -> [B, H, D, S]: matrices D x S, counted by H and B
+    check(x, (0, 2, 3, 1))
+    check(x, (0, 2, 1, 3))            # [B, H, S, D]: rows move, nothing is transposed
+    x = rand(2, 1, 256, 1, 128)       # modes of extent 1 in between
+    check(x, (0, 1, 3, 4, 2))
+    x = rand(2, 3, 2, 64, 256)        # three modes that count matrices: not one launch
+    check(x, (0, 1, 2, 4, 3))
+
+
 @pytest.mark.parametrize("dt", ["uint8", "float16", "float32", "int64"])
 def test_same_shape_copies_whatever_the_order_of_the_modes(mh, dt):
     """Arrays of one shape whose unit stride sits on the last or the middle mode (row-major with a pitch, a batch of

@@ -943,6 +943,94 @@ static int64_t launch_cvt_dense(int32_t sd, int32_t dd, const char* s, char* d, 
     }
 }
 
+// ------------------------------------------------------------------------------------------
+// a transpose that converts on the way (copyto! between arrays of different element types whose unit strides lie on
+// different modes: src/algorithm/copy.jl:38-43 with the layouts of a transpose)
+// ------------------------------------------------------------------------------------------
+// A tile is TI elements along the source's contiguous index i (at least 128 bytes of a source row) by TJ along the
+// destination's (at least 256 bytes of a destination row).  A lane loads 16-byte pieces of source rows, converts their
+// elements and writes them one by one into an LDS tile of destination elements, [i][j]; a lane then reads 16 bytes of an
+// LDS row and stores them as 16 bytes of a destination row.  Workgroups are numbered along j first, as in the other
+// destination-order kernels.  An LDS row is 16 bytes longer than its data, which spreads the rows over the banks.
+template <int kSrc, int kDst, int SB, int DB>
+__global__ __launch_bounds__(256) void transpose_cvt_lds(const char* __restrict__ src, char* __restrict__ dst, int64_t lds_, int64_t ldd, int tiles_j) {
+    constexpr int TI = SB == 1 ? 128 : 64, TJ = DB == 1 ? 256 : 128;
+    constexpr int ES = 16 / SB, ED = 16 / DB;  // elements per 16-byte piece
+    constexpr int PI = TI / ES, RJ = 256 / PI, NL = TJ / RJ;  // pieces per source row of the tile, source rows per pass, passes
+    constexpr int PITCH = TJ * DB + 16;
+    extern __shared__ char cvt_tile[];  // TI rows of PITCH bytes
+    const int tj = blockIdx.x % tiles_j, ti = blockIdx.x / tiles_j;
+    const int pi = threadIdx.x % PI, jr = threadIdx.x / PI;
+    const char* s = src + (((int64_t)tj * TJ + jr) * lds_ + (int64_t)ti * TI + ES * pi) * SB;
+    constexpr int CH = NL < 8 ? NL : 8;  // loads in flight per lane
+#pragma unroll 1
+    for (int h0 = 0; h0 < NL; h0 += CH) {
+        u32x4 x[CH];
+#pragma unroll
+        for (int h = 0; h < CH; ++h) x[h] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(s + (int64_t)(RJ * (h0 + h)) * lds_ * SB));
+#pragma unroll
+        for (int h = 0; h < CH; ++h) {
+            const int j = jr + RJ * (h0 + h);
+#pragma unroll
+            for (int e = 0; e < ES; ++e) {
+                char e_in[SB];
+                __builtin_memcpy(e_in, reinterpret_cast<const char*>(&x[h]) + e * SB, SB);
+                store_from<kDst>(cvt_tile + (ES * pi + e) * PITCH + j * DB, load_as_f64<kSrc>(e_in), kSrc == MOYE_F64);
+            }
+        }
+    }
+    __syncthreads();
+    constexpr int PJ = TJ / ED, RP = 256 / PJ;  // pieces per destination row of the tile, destination rows per pass
+    const int pj = threadIdx.x % PJ, r0 = threadIdx.x / PJ;
+    char* d = dst + (((int64_t)ti * TI + r0) * ldd + (int64_t)tj * TJ + ED * pj) * DB;
+#pragma unroll
+    for (int p = 0; p < TI / RP; ++p) {
+        const u32x4 w = *reinterpret_cast<const u32x4*>(cvt_tile + (r0 + RP * p) * PITCH + pj * 16);
+        __builtin_nontemporal_store(w, reinterpret_cast<u32x4*>(d + (int64_t)(RP * p) * ldd * DB));
+    }
+}
+
+// tile extents of transpose_cvt_lds for elements of sb and db bytes
+static int cvt_tile_i(int sb) { return sb == 1 ? 128 : 64; }
+static int cvt_tile_j(int db) { return db == 1 ? 256 : 128; }
+
+template <int kSrc, int kDst, int SB, int DB>
+static int32_t launch_transpose_cvt_pair(const char* s, char* d, int64_t lds_, int64_t ldd, int64_t ni, int64_t nj, hipStream_t st) {
+    auto kern = transpose_cvt_lds<kSrc, kDst, SB, DB>;
+    constexpr int TI = SB == 1 ? 128 : 64, TJ = DB == 1 ? 256 : 128, kLds = TI * (TJ * DB + 16);
+    if (kLds > 48 * 1024) {
+        static LdsCap cap;
+        if (int32_t e = raise_lds_cap(cap, reinterpret_cast<const void*>(kern), kLds)) return e;
+    }
+    const int64_t groups = (ni / TI) * (nj / TJ);
+    if (groups >= (1 << 24)) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles for one launch (2^24 workgroups of 256)");
+    kern<<<dim3((unsigned)groups), 256, kLds, st>>>(s, d, lds_, ldd, (int)(nj / TJ));
+    MOYE_HIP_CHECK(hipGetLastError());
+    return MOYE_OK;
+}
+template <int kSrc, int SB>
+static int32_t launch_transpose_cvt_dst(int32_t dd, const char* s, char* d, int64_t lds_, int64_t ldd, int64_t ni, int64_t nj, hipStream_t st) {
+    switch (dd) {
+        case MOYE_F32: if constexpr (kSrc != MOYE_F32) return launch_transpose_cvt_pair<kSrc, MOYE_F32, SB, 4>(s, d, lds_, ldd, ni, nj, st); break;
+        case MOYE_F16: if constexpr (kSrc != MOYE_F16) return launch_transpose_cvt_pair<kSrc, MOYE_F16, SB, 2>(s, d, lds_, ldd, ni, nj, st); break;
+        case MOYE_BF16: if constexpr (kSrc != MOYE_BF16) return launch_transpose_cvt_pair<kSrc, MOYE_BF16, SB, 2>(s, d, lds_, ldd, ni, nj, st); break;
+        case MOYE_F8E4M3: if constexpr (kSrc != MOYE_F8E4M3) return launch_transpose_cvt_pair<kSrc, MOYE_F8E4M3, SB, 1>(s, d, lds_, ldd, ni, nj, st); break;
+        case MOYE_F64: if constexpr (kSrc != MOYE_F64) return launch_transpose_cvt_pair<kSrc, MOYE_F64, SB, 8>(s, d, lds_, ldd, ni, nj, st); break;
+        default: break;
+    }
+    return fail(MOYE_ERR_UNSUPPORTED, "copyto!: no conversion between these element types");
+}
+static int32_t launch_transpose_cvt(int32_t sd, int32_t dd, const char* s, char* d, int64_t lds_, int64_t ldd, int64_t ni, int64_t nj, hipStream_t st) {
+    switch (sd) {
+        case MOYE_F32: return launch_transpose_cvt_dst<MOYE_F32, 4>(dd, s, d, lds_, ldd, ni, nj, st);
+        case MOYE_F16: return launch_transpose_cvt_dst<MOYE_F16, 2>(dd, s, d, lds_, ldd, ni, nj, st);
+        case MOYE_BF16: return launch_transpose_cvt_dst<MOYE_BF16, 2>(dd, s, d, lds_, ldd, ni, nj, st);
+        case MOYE_F8E4M3: return launch_transpose_cvt_dst<MOYE_F8E4M3, 1>(dd, s, d, lds_, ldd, ni, nj, st);
+        case MOYE_F64: return launch_transpose_cvt_dst<MOYE_F64, 8>(dd, s, d, lds_, ldd, ni, nj, st);
+        default: return fail(MOYE_ERR_UNSUPPORTED, "copyto!: no conversion between these element types");
+    }
+}
+
 template <int kSrc>
 static bool launch_cvt_dst(int32_t dd, dim3 g, hipStream_t st, const char* s, char* d, FlatLayout ls,
                            FlatLayout ld, int64_t n, int sb, int db, const Mask& mk) {
@@ -1280,6 +1368,40 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
             return fail(MOYE_ERR_UNSUPPORTED,
                         "copyto!: the LDS-tiled copy takes rank-2 operands (or a batch of them) of 1-, 2- or 4-byte elements "
                         "with the unit stride on different modes");
+    }
+
+    // (2c) a transpose that converts: a rank-2 pair of one shape, floating-point types that differ, the unit strides on
+    // different modes.  Whole aligned tiles through transpose_cvt_lds; other sizes as an interior of whole tiles plus two
+    // strips for the general kernel (8192^2 f32 -> f16: 294 us through the general kernel, which reads one side in single
+    // elements a pitch apart).
+    if (!same_bits && !mask && src->rank == 2 && dst->rank == 2 && src->shape[0] == dst->shape[0] && src->shape[1] == dst->shape[1] &&
+        is_float_dtype(src->dtype) && is_float_dtype(dst->dtype) && !(tc && tc->op == MOYE_COPY_LDS_TILED && (tc->tiler_mn[0] || tc->tiler_mn[1]))) {
+        int mi = -1;
+        if (src->stride[0] == 1 && dst->stride[1] == 1) mi = 0;
+        else if (src->stride[1] == 1 && dst->stride[0] == 1) mi = 1;
+        if (mi >= 0) {
+            const int mj = 1 - mi;
+            const int64_t ni = src->shape[mi], nj = src->shape[mj], lds_ = src->stride[mj], ldd = dst->stride[mi];
+            const int ti = cvt_tile_i(sb), tj = cvt_tile_j(db);
+            const bool lines = (lds_ * sb) % 16 == 0 && (ldd * db) % 16 == 0 && lds_ >= ni && ldd >= nj &&
+                               (reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d)) % 16 == 0;
+            if (lines && ni % ti == 0 && nj % tj == 0) return launch_transpose_cvt(src->dtype, dst->dtype, s, d, lds_, ldd, ni, nj, st);
+            const int64_t ni0 = ni / ti * ti, nj0 = nj / tj * tj;
+            if (lines && ni0 > 0 && nj0 > 0) {
+                auto part = [&](int64_t i0, int64_t ci, int64_t j0, int64_t cj) -> int32_t {
+                    if (ci == 0 || cj == 0) return MOYE_OK;
+                    moye_tensor ps = *src, pd = *dst;
+                    ps.ptr = static_cast<char*>(ps.ptr) + (i0 * ps.stride[mi] + j0 * ps.stride[mj]) * sb;
+                    pd.ptr = static_cast<char*>(pd.ptr) + (i0 * pd.stride[mi] + j0 * pd.stride[mj]) * db;
+                    ps.shape[mi] = pd.shape[mi] = ci;
+                    ps.shape[mj] = pd.shape[mj] = cj;
+                    return copy_if_dispatch(nullptr, &pd, &ps, nullptr, st);
+                };
+                if (int32_t e = part(0, ni0, 0, nj0)) return e;
+                if (int32_t e = part(ni0, ni - ni0, 0, nj)) return e;
+                return part(0, ni0, nj0, nj - nj0);
+            }
+        }
     }
 
     // (3) generic

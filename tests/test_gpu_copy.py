@@ -690,6 +690,45 @@ def test_transpose_eight_byte_elements(mh, M, N):
         assert torch.equal(dst3, src3.transpose(1, 2))
 
 
+@pytest.mark.parametrize("pair", ["float32->float16", "float16->float32", "float32->bfloat16", "bfloat16->float16", "float16->float8_e4m3fn",
+                                  "float8_e4m3fn->float32", "float64->float16", "float32->float64", "float64->float8_e4m3fn", "float8_e4m3fn->bfloat16"])
+def test_transpose_that_converts(mh, pair):
+    """copyto! between matrices of different floating-point types whose unit strides lie on different modes: whole tiles
+    through the LDS kernel that converts on the way, other sizes as interior + strips, both orientations, padded pitches.
+    Bit for bit what the library's dense conversion makes of the transposed source (that conversion is pinned against the
+    oracle elsewhere), values that round differently in every target among them; the frame of the destination untouched."""
+    sname, dname = pair.split("->")
+    sdt, ddt = getattr(torch, sname), getattr(torch, dname)
+    g = torch.Generator().manual_seed(len(pair) * 7)
+    bits = {1: torch.uint8, 2: torch.int16, 4: torch.int32, 8: torch.int64}
+
+    def dense(x):       # the library's conversion of a contiguous array
+        out = torch.zeros(x.shape, dtype=ddt, device="cuda")
+        mh.copyto_(_tens(mh, out, (x.numel(),), (1,)), _tens(mh, x.contiguous(), (x.numel(),), (1,)))
+        torch.cuda.synchronize()
+        return out
+
+    for (M, N) in ((128, 256), (256, 512), (1024, 768), (200, 300), (1088, 784), (4096, 2048)):
+        vals = (torch.randn(M, N, generator=g, dtype=torch.float64) * 3).to(torch.float32)
+        vals[0, :8] = torch.tensor([0.0, -0.0, 1e-8, 65520.0, -70000.0, 448.0, 464.0, float("inf")])
+        src = vals.to(sdt).cuda()                                   # (M, N) row-major: N contiguous
+        lds, ldd = N + 16, M + 32
+        sbuf = torch.zeros(M, lds, dtype=sdt, device="cuda")
+        sbuf[:, :N] = src
+        dbuf = torch.full((N, ldd), 3.0, device="cuda").to(ddt)     # destination (M, N) with M contiguous: stored as (N, ldd)
+        mh.copyto_(_tens(mh, dbuf, (M, N), (1, ldd)), _tens(mh, sbuf, (M, N), (lds, 1)))
+        torch.cuda.synchronize()
+        want = dense(src.t())
+        assert torch.equal(dbuf[:, :M].contiguous().view(bits[ddt.itemsize]), want.view(bits[ddt.itemsize])), (pair, M, N)
+        assert bool((dbuf[:, M:].float() == 3.0).all()), "stores outside the destination"
+        # the other orientation: source with M contiguous, destination row-major
+        s2 = src.t().contiguous()                                   # stored (N, M): element (m, n) at n * M + m
+        d2 = torch.zeros(M, N, dtype=ddt, device="cuda")
+        mh.copyto_(_tens(mh, d2, (M, N), (N, 1)), _tens(mh, s2, (M, N), (1, M)))
+        torch.cuda.synchronize()
+        assert torch.equal(d2.view(bits[ddt.itemsize]), dense(src).view(bits[ddt.itemsize])), (pair, M, N, "other orientation")
+
+
 @pytest.mark.parametrize("dt", ["uint8", "float16", "float32", "float64"])
 def test_permutations_that_are_batches_of_transposes(mh, dt):
     """Rank-4 permutations whose modes merge into a batch of matrices (NCHW <-> NHWC: H and W are neighbours in memory on

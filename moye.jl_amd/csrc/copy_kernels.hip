@@ -953,12 +953,15 @@ static int64_t launch_cvt_dense(int32_t sd, int32_t dd, const char* s, char* d, 
 // LDS row and stores them as 16 bytes of a destination row.  Workgroups are numbered along j first, as in the other
 // destination-order kernels.  An LDS row is 16 bytes longer than its data, which spreads the rows over the banks.
 template <int kSrc, int kDst, int SB, int DB>
-__global__ __launch_bounds__(256) void transpose_cvt_lds(const char* __restrict__ src, char* __restrict__ dst, int64_t lds_, int64_t ldd, int tiles_j) {
+__global__ __launch_bounds__(256) void transpose_cvt_lds(const char* __restrict__ src, char* __restrict__ dst, int64_t lds_, int64_t ldd, int tiles_j,
+                                                         int64_t bs_src, int64_t bs_dst, int64_t bz_src, int64_t bz_dst) {
     constexpr int TI = SB == 1 ? 128 : 64, TJ = DB == 1 ? 256 : 128;
     constexpr int ES = 16 / SB, ED = 16 / DB;  // elements per 16-byte piece
     constexpr int PI = TI / ES, RJ = 256 / PI, NL = TJ / RJ;  // pieces per source row of the tile, source rows per pass, passes
     constexpr int PITCH = TJ * DB + 16;
     extern __shared__ char cvt_tile[];  // TI rows of PITCH bytes
+    src += ((int64_t)blockIdx.y * bs_src + (int64_t)blockIdx.z * bz_src) * SB;  // (a batch of matrices: their indices in the grid)
+    dst += ((int64_t)blockIdx.y * bs_dst + (int64_t)blockIdx.z * bz_dst) * DB;
     const int tj = blockIdx.x % tiles_j, ti = blockIdx.x / tiles_j;
     const int pi = threadIdx.x % PI, jr = threadIdx.x / PI;
     const char* s = src + (((int64_t)tj * TJ + jr) * lds_ + (int64_t)ti * TI + ES * pi) * SB;
@@ -995,7 +998,7 @@ static int cvt_tile_i(int sb) { return sb == 1 ? 128 : 64; }
 static int cvt_tile_j(int db) { return db == 1 ? 256 : 128; }
 
 template <int kSrc, int kDst, int SB, int DB>
-static int32_t launch_transpose_cvt_pair(const char* s, char* d, int64_t lds_, int64_t ldd, int64_t ni, int64_t nj, hipStream_t st) {
+static int32_t launch_transpose_cvt_pair(const char* s, char* d, int64_t lds_, int64_t ldd, int64_t ni, int64_t nj, hipStream_t st, const int64_t (&bt)[6]) {
     auto kern = transpose_cvt_lds<kSrc, kDst, SB, DB>;
     constexpr int TI = SB == 1 ? 128 : 64, TJ = DB == 1 ? 256 : 128, kLds = TI * (TJ * DB + 16);
     if (kLds > 48 * 1024) {
@@ -1004,29 +1007,32 @@ static int32_t launch_transpose_cvt_pair(const char* s, char* d, int64_t lds_, i
     }
     const int64_t groups = (ni / TI) * (nj / TJ);
     if (groups >= (1 << 24)) return fail(MOYE_ERR_SHAPE, "copyto!: too many tiles for one launch (2^24 workgroups of 256)");
-    kern<<<dim3((unsigned)groups), 256, kLds, st>>>(s, d, lds_, ldd, (int)(nj / TJ));
+    kern<<<dim3((unsigned)groups, (unsigned)bt[4], (unsigned)bt[5]), 256, kLds, st>>>(s, d, lds_, ldd, (int)(nj / TJ), bt[0], bt[1], bt[2], bt[3]);
     MOYE_HIP_CHECK(hipGetLastError());
     return MOYE_OK;
 }
 template <int kSrc, int SB>
-static int32_t launch_transpose_cvt_dst(int32_t dd, const char* s, char* d, int64_t lds_, int64_t ldd, int64_t ni, int64_t nj, hipStream_t st) {
+static int32_t launch_transpose_cvt_dst(int32_t dd, const char* s, char* d, int64_t lds_, int64_t ldd, int64_t ni, int64_t nj, hipStream_t st, const int64_t (&bt)[6]) {
     switch (dd) {
-        case MOYE_F32: if constexpr (kSrc != MOYE_F32) return launch_transpose_cvt_pair<kSrc, MOYE_F32, SB, 4>(s, d, lds_, ldd, ni, nj, st); break;
-        case MOYE_F16: if constexpr (kSrc != MOYE_F16) return launch_transpose_cvt_pair<kSrc, MOYE_F16, SB, 2>(s, d, lds_, ldd, ni, nj, st); break;
-        case MOYE_BF16: if constexpr (kSrc != MOYE_BF16) return launch_transpose_cvt_pair<kSrc, MOYE_BF16, SB, 2>(s, d, lds_, ldd, ni, nj, st); break;
-        case MOYE_F8E4M3: if constexpr (kSrc != MOYE_F8E4M3) return launch_transpose_cvt_pair<kSrc, MOYE_F8E4M3, SB, 1>(s, d, lds_, ldd, ni, nj, st); break;
-        case MOYE_F64: if constexpr (kSrc != MOYE_F64) return launch_transpose_cvt_pair<kSrc, MOYE_F64, SB, 8>(s, d, lds_, ldd, ni, nj, st); break;
+        case MOYE_F32: if constexpr (kSrc != MOYE_F32) return launch_transpose_cvt_pair<kSrc, MOYE_F32, SB, 4>(s, d, lds_, ldd, ni, nj, st, bt); break;
+        case MOYE_F16: if constexpr (kSrc != MOYE_F16) return launch_transpose_cvt_pair<kSrc, MOYE_F16, SB, 2>(s, d, lds_, ldd, ni, nj, st, bt); break;
+        case MOYE_BF16: if constexpr (kSrc != MOYE_BF16) return launch_transpose_cvt_pair<kSrc, MOYE_BF16, SB, 2>(s, d, lds_, ldd, ni, nj, st, bt); break;
+        case MOYE_F8E4M3: if constexpr (kSrc != MOYE_F8E4M3) return launch_transpose_cvt_pair<kSrc, MOYE_F8E4M3, SB, 1>(s, d, lds_, ldd, ni, nj, st, bt); break;
+        case MOYE_F64: if constexpr (kSrc != MOYE_F64) return launch_transpose_cvt_pair<kSrc, MOYE_F64, SB, 8>(s, d, lds_, ldd, ni, nj, st, bt); break;
         default: break;
     }
     return fail(MOYE_ERR_UNSUPPORTED, "copyto!: no conversion between these element types");
 }
-static int32_t launch_transpose_cvt(int32_t sd, int32_t dd, const char* s, char* d, int64_t lds_, int64_t ldd, int64_t ni, int64_t nj, hipStream_t st) {
+// bt: the strides (in elements) of one or two modes that count matrices, source and destination, and their extents
+// {bs_src, bs_dst, bz_src, bz_dst, batch, batch2}; {0, 0, 0, 0, 1, 1} for one matrix
+static int32_t launch_transpose_cvt(int32_t sd, int32_t dd, const char* s, char* d, int64_t lds_, int64_t ldd, int64_t ni, int64_t nj, hipStream_t st,
+                                    const int64_t (&bt)[6]) {
     switch (sd) {
-        case MOYE_F32: return launch_transpose_cvt_dst<MOYE_F32, 4>(dd, s, d, lds_, ldd, ni, nj, st);
-        case MOYE_F16: return launch_transpose_cvt_dst<MOYE_F16, 2>(dd, s, d, lds_, ldd, ni, nj, st);
-        case MOYE_BF16: return launch_transpose_cvt_dst<MOYE_BF16, 2>(dd, s, d, lds_, ldd, ni, nj, st);
-        case MOYE_F8E4M3: return launch_transpose_cvt_dst<MOYE_F8E4M3, 1>(dd, s, d, lds_, ldd, ni, nj, st);
-        case MOYE_F64: return launch_transpose_cvt_dst<MOYE_F64, 8>(dd, s, d, lds_, ldd, ni, nj, st);
+        case MOYE_F32: return launch_transpose_cvt_dst<MOYE_F32, 4>(dd, s, d, lds_, ldd, ni, nj, st, bt);
+        case MOYE_F16: return launch_transpose_cvt_dst<MOYE_F16, 2>(dd, s, d, lds_, ldd, ni, nj, st, bt);
+        case MOYE_BF16: return launch_transpose_cvt_dst<MOYE_BF16, 2>(dd, s, d, lds_, ldd, ni, nj, st, bt);
+        case MOYE_F8E4M3: return launch_transpose_cvt_dst<MOYE_F8E4M3, 1>(dd, s, d, lds_, ldd, ni, nj, st, bt);
+        case MOYE_F64: return launch_transpose_cvt_dst<MOYE_F64, 8>(dd, s, d, lds_, ldd, ni, nj, st, bt);
         default: return fail(MOYE_ERR_UNSUPPORTED, "copyto!: no conversion between these element types");
     }
 }
@@ -1154,6 +1160,41 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
     const char* s = static_cast<const char*>(src->ptr);
     char* d = static_cast<char*>(dst->ptr);
 
+    // Arrays of one shape of rank three and more: modes of extent 1 go, and modes that are neighbours in memory on both
+    // sides become one (NCHW -> NHWC: H and W), so that what follows sees a matrix or a batch of matrices where there is
+    // one (the tiler of the descriptor speaks of the caller's modes: it is checked here, then dropped)
+    if (!mask && src->rank == dst->rank && src->rank > 2) {
+        bool same = true;
+        for (int m = 0; m < src->rank; ++m) same = same && src->shape[m] == dst->shape[m];
+        moye_tensor cs = *src, cd = *dst;
+        int r = 0;
+        for (int m = 0; same && m < src->rank; ++m) {
+            if (src->shape[m] == 1) continue;
+            if (r > 0 && src->stride[m] == cs.stride[r - 1] * cs.shape[r - 1] && dst->stride[m] == cd.stride[r - 1] * cd.shape[r - 1]) {
+                cs.shape[r - 1] *= src->shape[m];
+                cd.shape[r - 1] = cs.shape[r - 1];
+            } else {
+                cs.shape[r] = cd.shape[r] = src->shape[m];
+                cs.stride[r] = src->stride[m];
+                cd.stride[r] = dst->stride[m];
+                ++r;
+            }
+        }
+        if (same && r >= 1 && r < src->rank) {
+            moye_tiled_copy plain{};
+            if (tc) {
+                if (tc->op == MOYE_COPY_LDS_TILED)
+                    for (int m = 0; m < 2; ++m)
+                        if (tc->tiler_mn[m] < 0 || (tc->tiler_mn[m] > 0 && src->shape[m] % tc->tiler_mn[m]))
+                            return fail(MOYE_ERR_SHAPE, "copyto!: tiler extent %d does not divide mode %d of size %lld", tc->tiler_mn[m], m + 1,
+                                        (long long)src->shape[m]);
+                plain = *tc;
+                plain.tiler_mn[0] = plain.tiler_mn[1] = 0;
+            }
+            cs.rank = cd.rank = r;
+            return copy_if_dispatch(tc ? &plain : nullptr, &cd, &cs, nullptr, st);
+        }
+    }
     if (same_bits && !mask) {
         // (1) both sides one dense run in the same order
         if (one_run_each(*src, *dst)) {
@@ -1167,41 +1208,6 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
             }
             MOYE_HIP_CHECK(hipGetLastError());
             return MOYE_OK;
-        }
-        // Arrays of one shape of rank three and more: modes of extent 1 go, and modes that are neighbours in memory on both
-        // sides become one (NCHW -> NHWC: H and W), so that what follows sees a matrix or a batch of matrices where there is
-        // one (the tiler of the descriptor speaks of the caller's modes: it is checked here, then dropped)
-        if (src->rank == dst->rank && src->rank > 2) {
-            bool same = true;
-            for (int m = 0; m < src->rank; ++m) same = same && src->shape[m] == dst->shape[m];
-            moye_tensor cs = *src, cd = *dst;
-            int r = 0;
-            for (int m = 0; same && m < src->rank; ++m) {
-                if (src->shape[m] == 1) continue;
-                if (r > 0 && src->stride[m] == cs.stride[r - 1] * cs.shape[r - 1] && dst->stride[m] == cd.stride[r - 1] * cd.shape[r - 1]) {
-                    cs.shape[r - 1] *= src->shape[m];
-                    cd.shape[r - 1] = cs.shape[r - 1];
-                } else {
-                    cs.shape[r] = cd.shape[r] = src->shape[m];
-                    cs.stride[r] = src->stride[m];
-                    cd.stride[r] = dst->stride[m];
-                    ++r;
-                }
-            }
-            if (same && r >= 1 && r < src->rank) {
-                moye_tiled_copy plain{};
-                if (tc) {
-                    if (tc->op == MOYE_COPY_LDS_TILED)
-                        for (int m = 0; m < 2; ++m)
-                            if (tc->tiler_mn[m] < 0 || (tc->tiler_mn[m] > 0 && src->shape[m] % tc->tiler_mn[m]))
-                                return fail(MOYE_ERR_SHAPE, "copyto!: tiler extent %d does not divide mode %d of size %lld", tc->tiler_mn[m], m + 1,
-                                            (long long)src->shape[m]);
-                    plain = *tc;
-                    plain.tiler_mn[0] = plain.tiler_mn[1] = 0;
-                }
-                cs.rank = cd.rank = r;
-                return copy_if_dispatch(tc ? &plain : nullptr, &cd, &cs, nullptr, st);
-            }
         }
         // whole tiles of an aligned matrix (or of `batch` such matrices bs / bd elements apart) through the LDS kernels
         auto tiled_launch = [&](const char* s_, char* d_, int64_t ni, int64_t nj, int64_t lds_, int64_t ldd, int64_t bs, int64_t bd,
@@ -1385,7 +1391,7 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
             const int ti = cvt_tile_i(sb), tj = cvt_tile_j(db);
             const bool lines = (lds_ * sb) % 16 == 0 && (ldd * db) % 16 == 0 && lds_ >= ni && ldd >= nj &&
                                (reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d)) % 16 == 0;
-            if (lines && ni % ti == 0 && nj % tj == 0) return launch_transpose_cvt(src->dtype, dst->dtype, s, d, lds_, ldd, ni, nj, st);
+            if (lines && ni % ti == 0 && nj % tj == 0) return launch_transpose_cvt(src->dtype, dst->dtype, s, d, lds_, ldd, ni, nj, st, {0, 0, 0, 0, 1, 1});
             const int64_t ni0 = ni / ti * ti, nj0 = nj / tj * tj;
             if (lines && ni0 > 0 && nj0 > 0) {
                 auto part = [&](int64_t i0, int64_t ci, int64_t j0, int64_t cj) -> int32_t {
@@ -1400,6 +1406,39 @@ int32_t copy_if_dispatch(const moye_tiled_copy* tc, const moye_tensor* dst, cons
                 if (int32_t e = part(0, ni0, 0, nj0)) return e;
                 if (int32_t e = part(ni0, ni - ni0, 0, nj)) return e;
                 return part(0, ni0, nj0, nj - nj0);
+            }
+        }
+    }
+
+    // (2d) a batch of such converting transposes, counted by one or two modes (NCHW f32 -> NHWC f16 after H and W have
+    // become one mode): whole aligned tiles, one launch
+    if (!same_bits && !mask && src->rank == dst->rank && src->rank > 2 && is_float_dtype(src->dtype) && is_float_dtype(dst->dtype) &&
+        !(tc && tc->op == MOYE_COPY_LDS_TILED && (tc->tiler_mn[0] || tc->tiler_mn[1]))) {
+        const int r = src->rank;
+        bool same = true;
+        int mi = -1, mj = -1;
+        for (int m = 0; m < r; ++m) {
+            same = same && src->shape[m] == dst->shape[m];
+            if (src->shape[m] > 1 && src->stride[m] == 1 && mi < 0) mi = m;
+            if (dst->shape[m] > 1 && dst->stride[m] == 1 && mj < 0) mj = m;
+        }
+        if (same && mi >= 0 && mj >= 0 && mi != mj) {
+            int bm[2] = {-1, -1}, nb = 0;
+            for (int m = 0; m < r; ++m)
+                if (m != mi && m != mj && src->shape[m] > 1) {
+                    if (nb < 2) bm[nb] = m;
+                    ++nb;
+                }
+            const int64_t ni = src->shape[mi], nj = src->shape[mj], lds_ = src->stride[mj], ldd = dst->stride[mi];
+            bool fits = (nb == 1 || nb == 2) && ni % cvt_tile_i(sb) == 0 && nj % cvt_tile_j(db) == 0 && (lds_ * sb) % 16 == 0 && (ldd * db) % 16 == 0 &&
+                        lds_ >= ni && ldd >= nj && (reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d)) % 16 == 0;
+            for (int b = 0; fits && b < nb; ++b)
+                fits = src->shape[bm[b]] <= 65535 && (src->stride[bm[b]] * sb) % 16 == 0 && (dst->stride[bm[b]] * db) % 16 == 0;
+            if (fits) {
+                const bool two = nb == 2;
+                return launch_transpose_cvt(src->dtype, dst->dtype, s, d, lds_, ldd, ni, nj, st,
+                                            {src->stride[bm[0]], dst->stride[bm[0]], two ? src->stride[bm[1]] : 0, two ? dst->stride[bm[1]] : 0,
+                                             src->shape[bm[0]], two ? src->shape[bm[1]] : 1});
             }
         }
     }

@@ -729,6 +729,39 @@ def test_transpose_that_converts(mh, pair):
         assert torch.equal(d2.view(bits[ddt.itemsize]), dense(src).view(bits[ddt.itemsize])), (pair, M, N, "other orientation")
 
 
+@pytest.mark.parametrize("pair", ["float32->float16", "float16->float32", "bfloat16->float8_e4m3fn", "float64->float32"])
+def test_permutations_that_convert(mh, pair):
+    """Rank-4 permutations between arrays of different floating-point types: modes merged, then a batch of converting
+    transposes in one launch where the matrices are whole tiles (NCHW -> NHWC), counted by two modes ([B, S, H, D] ->
+    [B, H, D, S]), the general kernel otherwise.  Bit for bit the library's dense conversion of torch's permuted source."""
+    sname, dname = pair.split("->")
+    sdt, ddt = getattr(torch, sname), getattr(torch, dname)
+    g = torch.Generator().manual_seed(len(pair))
+    bits = {1: torch.uint8, 2: torch.int16, 4: torch.int32, 8: torch.int64}[ddt.itemsize]
+
+    def dense(x):
+        out = torch.zeros(x.shape, dtype=ddt, device="cuda")
+        mh.copyto_(_tens(mh, out, (x.numel(),), (1,)), _tens(mh, x.contiguous(), (x.numel(),), (1,)))
+        torch.cuda.synchronize()
+        return out
+
+    def check(shape, perm):
+        x = (torch.randn(*shape, generator=g) * 4).to(sdt).cuda()
+        view = x.permute(*perm)
+        want = dense(view.contiguous())
+        dst = torch.zeros(want.shape, dtype=ddt, device="cuda")
+        lshape = tuple(reversed(want.shape))
+        mh.copyto_(_tens(mh, dst, lshape, tuple(reversed(dst.stride()))), _tens(mh, x, lshape, tuple(reversed(view.stride()))))
+        torch.cuda.synchronize()
+        assert torch.equal(dst.view(bits), want.view(bits)), (pair, shape, perm)
+
+    check((3, 256, 16, 16), (0, 2, 3, 1))      # NCHW -> NHWC, H W = 256
+    check((3, 16, 16, 256), (0, 3, 1, 2))      # NHWC -> NCHW
+    check((2, 128, 14, 14), (0, 2, 3, 1))      # H W = 196: not whole tiles
+    check((2, 256, 3, 128), (0, 2, 3, 1))      # [B, S, H, D] -> [B, H, D, S]
+    check((2, 256, 3, 128), (0, 2, 1, 3))      # rows move
+
+
 @pytest.mark.parametrize("dt", ["uint8", "float16", "float32", "float64"])
 def test_permutations_that_are_batches_of_transposes(mh, dt):
     """Rank-4 permutations whose modes merge into a batch of matrices (NCHW <-> NHWC: H and W are neighbours in memory on

@@ -62,6 +62,31 @@ __device__ __forceinline__ int64_t e_offset(const ELayout& l, int64_t i) {
     return off;
 }
 
+// The same for up to three layouts of one shape, mode by mode, and an index below 2^31: the index is taken apart once,
+// with 32-bit divisions, and the coordinates are weighed with each layout's strides (the 64-bit divisions of e_offset,
+// once per layout and mode, set the pace of these kernels otherwise).
+__device__ __forceinline__ void e_offsets(const ELayout& a, const ELayout& b, const ELayout& c, uint32_t i, int64_t* oa, int64_t* ob, int64_t* oc) {
+    int64_t xa = 0, xb = 0, xc = 0;
+#pragma unroll 1
+    for (int m = 0; m < a.rank; ++m) {
+        const uint32_t extent = (uint32_t)a.shape[m], q = i / extent, r = i - q * extent;
+        xa += (int64_t)r * a.stride[m];
+        xb += (int64_t)r * b.stride[m];
+        xc += (int64_t)r * c.stride[m];
+        i = q;
+    }
+    *oa = xa;
+    *ob = xb;
+    *oc = xc;
+}
+// layouts of one shape mode by mode, few enough elements for 32-bit indices (host side)
+bool same_modes_32(const ELayout& a, const ELayout& b, int64_t n) {
+    if (a.rank != b.rank || n >= ((int64_t)1 << 31)) return false;
+    for (int m = 0; m < a.rank; ++m)
+        if (a.shape[m] != b.shape[m] || a.shape[m] <= 0) return false;
+    return true;
+}
+
 ELayout elayout_of(const moye_tensor& t) {
     ELayout f;
     f.rank = t.rank;
@@ -112,12 +137,15 @@ struct ElBF16 {
 template <typename El>
 __global__ __launch_bounds__(256) void axpby_kernel(typename El::compute a, const typename El::storage* x, ELayout lx,
                                                     typename El::compute b, typename El::storage* y, ELayout ly,
-                                                    int64_t n, bool b_is_zero) {
+                                                    int64_t n, bool b_is_zero, bool same = false) {
     typedef typename El::compute T;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
-        const T ax = El::round(a * El::load(x + e_offset(lx, i)));
-        typename El::storage* yp = y + e_offset(ly, i);
+        int64_t ox, oy, unused;
+        if (same) e_offsets(lx, ly, ly, (uint32_t)i, &ox, &oy, &unused);
+        else ox = e_offset(lx, i), oy = e_offset(ly, i);
+        const T ax = El::round(a * El::load(x + ox));
+        typename El::storage* yp = y + oy;
         if (b_is_zero) {
             El::store(yp, ax);
         } else {
@@ -150,13 +178,21 @@ template <typename El>
 __global__ __launch_bounds__(256) void map_kernel(int32_t op, typename El::storage* d, ELayout ld,
                                                   const typename El::storage* a, ELayout la,
                                                   const typename El::storage* b, ELayout lb, int64_t nb,
-                                                  typename El::compute s, int64_t n) {
+                                                  typename El::compute s, int64_t n, bool same = false) {
     typedef typename El::compute T;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
-        const T x = El::load(a + e_offset(la, i));
-        const T y = b ? El::load(b + e_offset(lb, i % nb)) : s;
-        El::store(d + e_offset(ld, i), El::round(map_op(op, x, y)));
+        int64_t oa, ob = 0, od;
+        if (same) {
+            e_offsets(la, lb, ld, (uint32_t)i, &oa, &ob, &od);  // (lb unused without b: its strides weigh nothing that is read)
+        } else {
+            oa = e_offset(la, i);
+            if (b) ob = e_offset(lb, i % nb);
+            od = e_offset(ld, i);
+        }
+        const T x = El::load(a + oa);
+        const T y = b ? El::load(b + ob) : s;
+        El::store(d + od, El::round(map_op(op, x, y)));
     }
 }
 
@@ -256,7 +292,7 @@ __global__ __launch_bounds__(256) void fill_dense_kernel(u32x4* x, int64_t nvec,
 template <typename El>
 __global__ __launch_bounds__(256) void axpby_rows_kernel(typename El::compute a, const typename El::storage* x, ELayout lx,
                                                          typename El::compute b, typename El::storage* y, ELayout ly, int64_t nvec,
-                                                         bool b_is_zero) {
+                                                         bool b_is_zero, bool same) {
     typedef typename El::compute T;
     typedef typename El::storage S;
     typedef typename DenseVec<El>::type vec;
@@ -264,8 +300,11 @@ __global__ __launch_bounds__(256) void axpby_rows_kernel(typename El::compute a,
     const vec* xv = reinterpret_cast<const vec*>(x);
     vec* yv = reinterpret_cast<vec*>(y);
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256) {
-        const vec vx = xv[e_offset(lx, i)];
-        vec* py = yv + e_offset(ly, i);
+        int64_t ox, oy, unused;
+        if (same) e_offsets(lx, ly, ly, (uint32_t)i, &ox, &oy, &unused);
+        else ox = e_offset(lx, i), oy = e_offset(ly, i);
+        const vec vx = xv[ox];
+        vec* py = yv + oy;
         const vec vy = b_is_zero ? vx : *py;
         vec r;
 #pragma unroll
@@ -283,7 +322,7 @@ __global__ __launch_bounds__(256) void axpby_rows_kernel(typename El::compute a,
 template <typename El>
 __global__ __launch_bounds__(256) void map_rows_kernel(int32_t op, typename El::storage* d, ELayout ld, const typename El::storage* a,
                                                        ELayout la, const typename El::storage* b, ELayout lb, typename El::compute s,
-                                                       int64_t nvec) {
+                                                       int64_t nvec, bool same) {
     typedef typename El::compute T;
     typedef typename El::storage S;
     typedef typename DenseVec<El>::type vec;
@@ -292,8 +331,16 @@ __global__ __launch_bounds__(256) void map_rows_kernel(int32_t op, typename El::
     const vec* bv = reinterpret_cast<const vec*>(b);
     vec* dv = reinterpret_cast<vec*>(d);
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256) {
-        const vec va = av[e_offset(la, i)];
-        const vec vb = b ? bv[e_offset(lb, i)] : va;
+        int64_t oa, ob = 0, od;
+        if (same) {
+            e_offsets(la, lb, ld, (uint32_t)i, &oa, &ob, &od);  // (lb unused without b: its strides weigh nothing that is read)
+        } else {
+            oa = e_offset(la, i);
+            if (b) ob = e_offset(lb, i);
+            od = e_offset(ld, i);
+        }
+        const vec va = av[oa];
+        const vec vb = b ? bv[ob] : va;
         vec r;
 #pragma unroll
         for (int k = 0; k < N; ++k) {
@@ -303,7 +350,7 @@ __global__ __launch_bounds__(256) void map_rows_kernel(int32_t op, typename El::
             El::store(&er, El::round(map_op(op, x, y)));
             r[k] = er;
         }
-        dv[e_offset(ld, i)] = r;
+        dv[od] = r;
     }
 }
 
@@ -388,12 +435,12 @@ static void launch_axpby(typename El::compute a, const void* x, const ELayout& l
     const bool b0 = b == (typename El::compute)0;
     if (!is_dense && rows) {  // lx, ly are in 16-byte pieces
         const int64_t nvec = n / DenseVec<El>::N;
-        axpby_rows_kernel<El><<<strided_grid(nvec), 256, 0, st>>>(a, xs, lx, b, ys, ly, nvec, b0);
+        axpby_rows_kernel<El><<<strided_grid(nvec), 256, 0, st>>>(a, xs, lx, b, ys, ly, nvec, b0, same_modes_32(lx, ly, nvec));
         return;
     }
     if (!is_dense) {
         const dim3 grid((unsigned)std::min<int64_t>((n + 255) / 256, 256 * 16));
-        axpby_kernel<El><<<grid, 256, 0, st>>>(a, xs, lx, b, ys, ly, n, b0);
+        axpby_kernel<El><<<grid, 256, 0, st>>>(a, xs, lx, b, ys, ly, n, b0, same_modes_32(lx, ly, n));
         return;
     }
     constexpr int N = DenseVec<El>::N;
@@ -411,12 +458,14 @@ static void launch_map(int32_t op, void* d, const ELayout& ld, const void* a, co
     const S* bs = static_cast<const S*>(b);
     if (!is_dense && rows) {  // ld, la, lb are in 16-byte pieces
         const int64_t nvec = n / DenseVec<El>::N;
-        map_rows_kernel<El><<<strided_grid(nvec), 256, 0, st>>>(op, ds, ld, as, la, bs, lb, s, nvec);
+        map_rows_kernel<El><<<strided_grid(nvec), 256, 0, st>>>(op, ds, ld, as, la, bs, lb, s, nvec,
+                                                                same_modes_32(ld, la, nvec) && (!bs || same_modes_32(ld, lb, nvec)));
         return;
     }
     if (!is_dense) {
         const dim3 grid((unsigned)std::min<int64_t>((n + 255) / 256, 256 * 16));
-        map_kernel<El><<<grid, 256, 0, st>>>(op, ds, ld, as, la, bs, lb, nb, s, n);
+        map_kernel<El><<<grid, 256, 0, st>>>(op, ds, ld, as, la, bs, lb, nb, s, n,
+                                             same_modes_32(ld, la, n) && (!bs || (nb == n && same_modes_32(ld, lb, n))));
         return;
     }
     constexpr int N = DenseVec<El>::N;

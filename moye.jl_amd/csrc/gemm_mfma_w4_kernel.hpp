@@ -731,10 +731,11 @@ static int32_t launch256_w4(const GemmArgs& a, GemmPlan& plan) {
     return MOYE_OK;
 }
 
-// The instances live in five translation units (so that they compile side by side): gemm_mfma256w4.hip (the 256 x 256
+// The instances live in six translation units (so that they compile side by side): gemm_mfma256w4.hip (the 256 x 256
 // tile with K-major operands), gemm_mfma256w4_majors.hip (operands that keep their M- / N-major form),
-// gemm_mfma256w4_ops.hip (an element-wise operation in the epilogue), gemm_mfma128w4.hip (the 128 x 128 tile),
-// gemm_mfma128w4_majors.hip (the 128 x 128 tile with M- / N-major operands).
+// gemm_mfma256w4_ops.hip (an element-wise operation in the epilogue), gemm_mfma256w4_persist.hip (one workgroup per CU
+// that walks over the tiles), gemm_mfma128w4.hip (the 128 x 128 tile), gemm_mfma128w4_majors.hip (the 128 x 128 tile with
+// M- / N-major operands).
 int32_t launch256_w4_majors_dispatch(int32_t in_dt, int32_t out_dt, const GemmArgs& a, GemmPlan& plan);
 int32_t launch256_w4_ops_dispatch(int32_t in_dt, int32_t out_dt, const GemmArgs& a, GemmPlan& plan);
 int32_t launch128_w4_majors_dispatch(int32_t in_dt, int32_t out_dt, const GemmArgs& a, GemmPlan& plan);

@@ -567,12 +567,8 @@ __device__ __forceinline__ int64_t layout_offset(const FlatLayout& l, int64_t i)
 
 __device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
 
-__device__ __forceinline__ uint16_t f32_to_bf16(float f) {  // round to nearest even
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);  // quiet NaN
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
-}
+// round to nearest even, a NaN made quiet: v_cvt_pk_bf16_f32 (the same bits as the integer form for all 2^32 inputs)
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
 
 __device__ __forceinline__ float f8e4m3_to_f32(uint8_t b) {  // OCP e4m3fn
     const uint32_t sign = (uint32_t)(b & 0x80) << 24;

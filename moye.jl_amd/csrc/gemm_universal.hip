@@ -12,11 +12,10 @@
 
 namespace moye {
 
+// (a NaN stays as it is; everything else through v_cvt_pk_bf16_f32, round to nearest even)
 __device__ __forceinline__ float u_bf16_round(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return f;
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return __uint_as_float(u & 0xffff0000u);
+    if (f != f) return f;
+    return __uint_as_float((uint32_t)__builtin_bit_cast(uint16_t, (__bf16)f) << 16);
 }
 
 __device__ __forceinline__ float u_load(const void* p, int64_t i, int dt) {

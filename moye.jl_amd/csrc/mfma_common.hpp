@@ -105,12 +105,10 @@ struct OutBF16 {
     typedef uint16_t type;
     static constexpr int kDt = MOYE_BF16;
     static constexpr const char* kName = "OutBF16";
-    static __device__ __forceinline__ uint16_t cvt(float x) {
-        uint32_t u = __float_as_uint(x);
-        if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
-        u += 0x7fffu + ((u >> 16) & 1u);
-        return (uint16_t)(u >> 16);
-    }
+    // v_cvt_pk_bf16_f32: round to nearest even, a NaN keeps its sign and upper payload bits and becomes quiet.  Checked on
+    // the hardware over all 2^32 inputs against the integer form (add 0x7fff + the lowest kept bit, shift; NaN: shift, set
+    // bit 6), which costs six instructions an element where this costs half of one.
+    static __device__ __forceinline__ uint16_t cvt(float x) { return __builtin_bit_cast(uint16_t, (__bf16)x); }
     static __device__ __forceinline__ float load(const void* p, int64_t i) {
         return __uint_as_float((uint32_t)static_cast<const uint16_t*>(p)[i] << 16);
     }

@@ -30,15 +30,15 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # few percent.
 TRAFFIC_SOURCE = "profiles/gemm_f16_4096_and_transpose_f32_16384_counters.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this script in an earlier session; not measured in this run)"
 FETCH_SCALE = 2.0
-TRAFFIC_CALIBRATION = ("copy_flat_b128", 524294.5, 1049478.0)     # the 1 GiB plain copy of the same runs: 1048576 KiB each way
+TRAFFIC_CALIBRATION = ("copy_flat_b128", 524297.5, 1049490.6)     # the 1 GiB plain copy of the same runs: 1048576 KiB each way
 MEASURED_TRAFFIC = {
     # key: (kernel as the profile names it, FETCH_SIZE KiB, WRITE_SIZE KiB)
-    "gemm_f16_4096_tile256": ("gemm_mfma_tn_256_w4<W4F16L, OutF16, 4, false, false, 256, 0, 0, false, false, false>", 98481.5, 32778.7),
-    "transpose_f32_16384": ("transpose_lds_b32_rows<4>", 524308.0, 1050128.1),
-    "gemm_bf16_8192_tile256": ("gemm_mfma_tn_256_w4<W4BF16L, OutF32, 4, false, false, 256, 0, 0, false, false, true>", 829282.8, 263184.2),
-    "gemm_f32_8192_tile256": ("gemm_mfma_tn_256_w4<W4F32L, OutF32, 4, false, false, 256, 0, 0, false, false, false>", 1638174.0, 262266.9),
-    "gemm_fp8_8192_tile256": ("gemm_mfma_tn_256_w4<W4FP8L, OutBF16, 4, false, false, 256, 0, 0, false, false, true>", 395207.0, 132096.0),
-    "gemm_bf16_16x8192x8192": ("gemm_mfma_skinny_lds<InBF16, OutF32, 1, 2, 4, 3, 2>", 66617.5, 512.0),
+    "gemm_f16_4096_tile256": ("gemm_mfma_tn_256_w4<W4F16L, OutF16, 4, false, false, 256, 0, 0, false, false, false>", 98481.0, 32789.1),
+    "transpose_f32_16384": ("transpose_lds_b32_rows<4>", 524309.0, 1050103.0),
+    "gemm_bf16_8192_tile256": ("gemm_mfma_tn_256_w4<W4BF16L, OutF32, 4, false, false, 256, 0, 0, false, false, true>", 827548.5, 263348.6),
+    "gemm_f32_8192_tile256": ("gemm_mfma_tn_256_w4<W4F32L, OutF32, 4, false, false, 256, 0, 0, false, false, false>", 1653069.0, 262269.2),
+    "gemm_fp8_8192_tile256": ("gemm_mfma_tn_256_w4<W4FP8L, OutBF16, 4, false, false, 256, 0, 0, false, false, true>", 395120.7, 132096.0),
+    "gemm_bf16_16x8192x8192": ("gemm_mfma_skinny_lds<InBF16, OutF32, 1, 2, 4, 3, 2>", 66612.0, 512.0),
 }
 
 

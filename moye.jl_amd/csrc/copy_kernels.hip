@@ -570,29 +570,16 @@ __device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __uint_as_floa
 // round to nearest even, a NaN made quiet: v_cvt_pk_bf16_f32 (the same bits as the integer form for all 2^32 inputs)
 __device__ __forceinline__ uint16_t f32_to_bf16(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
 
-__device__ __forceinline__ float f8e4m3_to_f32(uint8_t b) {  // OCP e4m3fn
-    const uint32_t sign = (uint32_t)(b & 0x80) << 24;
-    const int e = (b >> 3) & 0xf;
-    const int m = b & 7;
-    if (e == 0xf && m == 7) return __uint_as_float(sign | 0x7fc00000u);
-    if (e == 0) return __uint_as_float(sign) + (sign ? -1.f : 1.f) * (float)m * 0.001953125f;  // m * 2^-9
-    return __uint_as_float(sign | ((uint32_t)(e + 120) << 23) | ((uint32_t)m << 20));
+// OCP e4m3fn <-> fp32 through v_cvt_f32_fp8 / v_cvt_pk_fp8_f32.  Narrowing rounds to nearest even and turns NaN, infinities
+// and everything beyond the last tie (|x| > 464) into NaN, as the integer form these replaced did: a one-off kernel compared
+// the two over all 2^32 inputs (and all 256 the other way) on the hardware.  They differ in one thing only, the sign of a NaN:
+// the instructions make every NaN negative, here a NaN keeps the sign it came with.
+__device__ __forceinline__ float f8e4m3_to_f32(uint8_t b) {
+    return b == 0x7f ? __uint_as_float(0x7fc00000u) : __builtin_amdgcn_cvt_f32_fp8((int)b, 0);
 }
-
-__device__ __forceinline__ uint8_t f32_to_f8e4m3(float f) {  // RNE; |x| > 464 and NaN -> NaN
-    const uint32_t u = __float_as_uint(f);
-    const uint8_t sign = (uint8_t)((u >> 24) & 0x80);
-    const float a = fabsf(f);
-    if (!(a <= 464.f)) return sign | 0x7f;           // NaN, inf, overflow past the last tie
-    if (a < 0.015625f) {                              // below 2^-6: subnormal grid of 2^-9
-        const float r = rintf(a * 512.f);             // rintf = round half to even
-        return sign | (uint8_t)r;                     // r == 8 lands on the first normal, 0x08
-    }
-    uint32_t au = u & 0x7fffffffu;
-    au += 0x7ffffu + ((au >> 20) & 1u);               // RNE to 3 mantissa bits
-    const int e = (int)(au >> 23) - 120;
-    const uint32_t m = (au >> 20) & 7u;
-    return sign | (uint8_t)((e << 3) | m);
+__device__ __forceinline__ uint8_t f32_to_f8e4m3(float f) {
+    const uint8_t h = (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(f, f, 0, false) & 0xff);
+    return f != f ? (uint8_t)(((__float_as_uint(f) >> 24) & 0x80) | 0x7f) : h;
 }
 
 template <int kDt>

@@ -183,6 +183,11 @@ static int32_t launch_skinny_lds(const GemmArgs& a, GemmPlan& plan) {
     // covers the latency.  32 rows per workgroup once that gives every CU one (bf16, K = 8192: N = 16384 40.1 us against
     // 45.3 with 16 rows; N = 4096 17.9 against 13.5).
     const bool wide = (a.N + 31) / 32 >= plan.shape.cus;
+    // More than 32 rows of A and enough columns for 64 rows of B per workgroup on every CU: every workgroup reads all of A
+    // out of the L2s, which with 32 rows of B is twice B's own bytes (bf16 64 x 28672 x 8192: 118.8 us with 32 rows, 95.3 with 64).
+    // Two buffers instead of three, for the LDS.
+    if ((a.M + 15) / 16 >= 3 && (a.N + 63) / 64 >= plan.shape.cus)
+        return (a.M + 15) / 16 == 3 ? launch_skinny_lds_v<In, Out, 3, W, 4, 2, 2>(a, plan) : launch_skinny_lds_v<In, Out, 4, W, 4, 2, 2>(a, plan);
     if (wide) {
         switch ((a.M + 15) / 16) {
             case 1: return launch_skinny_lds_v<In, Out, 1, W, 2, 3, 2>(a, plan);

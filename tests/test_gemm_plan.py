@@ -296,6 +296,10 @@ def test_known_shapes_run_on_the_instances_they_are_meant_for():
     # short M: whole 128-byte lines of K through LDS, a K tail as a masked trip of the same kernel
     assert step_names(run_case(bf16, f32, 16, 8192, 8192))[0].startswith("gemm_mfma_skinny_lds<InBF16,OutF32,mt=1,ntw=2,waves=4,stages=3>")
     assert step_names(run_case(bf16, f32, 16, 8192, 8224))[0].startswith("gemm_mfma_skinny_lds<InBF16,OutF32,mt=1,ntw=2,")   # a K tail too
+    # more than 32 rows of A: 64 rows of B per workgroup once that still gives every CU one, 32 below that
+    assert step_names(run_case(bf16, bf16, 64, 28672, 8192))[0].startswith("gemm_mfma_skinny_lds<InBF16,OutBF16,mt=4,ntw=4,waves=4,stages=2>")
+    assert step_names(run_case(bf16, bf16, 48, 16384, 4096))[0].startswith("gemm_mfma_skinny_lds<InBF16,OutBF16,mt=3,ntw=4,waves=4,stages=2>")
+    assert ",ntw=2," in step_names(run_case(bf16, bf16, 64, 8192, 8192))[0]
     # small N and a long K: the library's own K ranges for the line kernel, then the reduction
     p = run_case(bf16, f32, 16, 1024, 32768, split_k=-1)
     assert p["steps"][0]["family"] == "gemm_mfma_skinny_lds" and p["steps"][0]["split"] == 4 and p["steps"][-1]["what"] == "splitk_reduce"

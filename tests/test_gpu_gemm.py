@@ -655,6 +655,31 @@ def test_short_m_small_n_long_k_takes_k_ranges(mh):
         assert torch.equal(d.cpu().double(), A.double() @ B.double().t()), (M, N, K)
 
 
+@pytest.mark.parametrize("M", [33, 48, 64])
+def test_short_m_sixty_four_rows_of_b_per_workgroup(mh, M):
+    """More than 32 rows of A and an N that gives every CU a workgroup of 64 rows of B: the form with ntw=4 and two
+    stages; N ragged against 64, K with and without a tail, every input type, D inside a frame; exact on small integers."""
+    g = torch.Generator().manual_seed(700 + M)
+    for (tdt, atom) in ((torch.float16, mh.MFMA_F32_16x16x32_F16), (torch.bfloat16, mh.MFMA_F32_16x16x32_BF16),
+                        (torch.float8_e4m3fn, mh.MFMA_F32_16x16x32_FP8)):
+        eb = tdt.itemsize
+        for (N, K) in ((16384, 256 // eb), (16400 + M, 1280 // eb), (16385, 464 // eb)):
+            A = torch.randint(-2, 3, (M, K), generator=g).float()
+            B = torch.randint(-2, 3, (N, K), generator=g).float()
+            a, b = A.cuda().to(tdt), B.cuda().to(tdt)
+            big = torch.full((M + 2, N + 3), 77.0, device="cuda")
+            d = big[1:M + 1, 2:N + 2]
+            mma = mh.tiled_mma_desc(atom, cta_tile=(0, 0, 0))
+            ks = kernels_of(mh, mma, T(d), T(a), T(b))
+            assert len(ks) == 1 and "mt=%d,ntw=4,waves=4,stages=2" % ((M + 15) // 16) in ks[0]["name"], ks
+            mh.gemm_(mma, T(d), T(a), T(b))
+            torch.cuda.synchronize()
+            assert torch.equal(d.cpu().double(), A.double() @ B.double().t()), (tdt, M, N, K)
+            frame = big.clone()
+            frame[1:M + 1, 2:N + 2] = 77.0
+            assert bool((frame == 77.0).all()), "stores outside D"
+
+
 @pytest.mark.parametrize("M", [1, 16, 17, 48, 64])
 def test_short_m_line_staging_kernel(mh, M):
     """K of whole 128-byte lines runs on the kernel that stages them through LDS: any M <= 64 and any N (16 and

@@ -51,6 +51,9 @@ inline TileChoice gemm_plan(int64_t M, int64_t N, int64_t k_bytes, bool f32_in, 
     TileChoice best{128, fixed_split > 0 ? fixed_split : 1, 1e30};
     for (int tile : {128, 64}) {
         if (tile == 64 && !tile64_ok) continue;
+        // (one row of tiles: the 64 x 64 kernel has nothing to share B with, and the model does not know
+        // -- bf16 64 x 65536 x 2048: 51.9 us against 43.3 on 128 x 128 tiles; 64 x 32768 x 2048: 26.7 against 27.4)
+        if (tile == 64 && M <= 64) continue;
         for (int s = 1; s <= 16; s *= 2) {
             if (fixed_split > 0 && s != fixed_split) continue;
             if (fixed_split <= 0 && s > 1) {
@@ -93,6 +96,21 @@ inline TileChoice gemm_choose(int64_t M, int64_t N, int64_t k_bytes, bool f32_in
         if (us <= best.us) best = TileChoice{256, 1, us};
     }
     return best;
+}
+
+// A short A (at most 64 rows, K in 16-byte pieces) goes to the kernel that streams B once and reads all of A per workgroup
+// (gemm_mfma_skinny.hip) -- except more than 16 rows with a short K and many columns: each of that kernel's waves then
+// has too few lines of K to cover the latency and A comes out of the L2s as often as B out of memory, and 128 x 128
+// tiles, part empty as they are, take less.  bf16, us on that kernel / on tiles: 64 x 65536 x 2048 62.9 / 43.3;
+// 32 x 65536 x 2048 62.8 / 40.1; 64 x 65536 x 256 30.6 / 15.1; 64 x 32768 x 2048 31.3 / 27.4; 64 x 24576 x 256 14.5 / 8.9;
+// 64 x 65536 x 3072 94.2 / 76.7; 64 x 131072 x 4096 228.6 / 177.2.  But 64 x 16384 x 2048 16.0 / 24.3;
+// 64 x 32768 x 4096 54.5 / 60.6; 64 x 65536 x 4096 111.9 / 124.4; 16 x 32768 x 2048 22.4 / 26.2.
+inline bool gemm_short_m(int64_t M, int64_t N, int64_t k_bytes, int cus) {
+    if (M > 64 || k_bytes % 16) return false;
+    if (M <= 16) return true;
+    const int64_t tiles = N / 128;
+    return !((tiles >= 3 * (int64_t)cus / 4 && k_bytes <= 4096) || (tiles >= 2 * (int64_t)cus && k_bytes <= 6144) ||
+             (tiles >= 4 * (int64_t)cus && k_bytes <= 8192));
 }
 
 }  // namespace moye

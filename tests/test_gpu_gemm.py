@@ -680,6 +680,34 @@ def test_short_m_sixty_four_rows_of_b_per_workgroup(mh, M):
             assert bool((frame == 77.0).all()), "stores outside D"
 
 
+@pytest.mark.parametrize("M", [17, 40, 64])
+def test_short_a_with_a_short_k_and_many_columns_runs_on_tiles(mh, M):
+    """More than 16 rows of A, K of at most 4096 bytes and columns for 128-wide tiles on three quarters of the CUs: the
+    library takes tiles, not the short-M kernel; row- and column-major D inside a frame, exact on small integers."""
+    g = torch.Generator().manual_seed(800 + M)
+    for (tdt, atom) in ((torch.float16, mh.MFMA_F32_16x16x32_F16), (torch.float8_e4m3fn, mh.MFMA_F32_16x16x32_FP8)):
+        for (N, K) in ((24576, 256), (24576 + 40, 1024 // tdt.itemsize), (65536, 128)):
+            A = torch.randint(-2, 3, (M, K), generator=g).float()
+            B = torch.randint(-2, 3, (N, K), generator=g).float()
+            a, b = A.cuda().to(tdt), B.cuda().to(tdt)
+            ref = A.double() @ B.double().t()
+            mma = mh.tiled_mma_desc(atom, cta_tile=(0, 0, 0))
+            big = torch.full((M + 2, N + 8), 77.0, device="cuda")
+            d = big[1:M + 1, 4:N + 4]
+            ks = kernels_of(mh, mma, T(d), T(a), T(b))
+            assert ks[0]["family"] != "gemm_mfma_skinny_lds", ks
+            mh.gemm_(mma, T(d), T(a), T(b))
+            torch.cuda.synchronize()
+            assert torch.equal(d.cpu().double(), ref), (tdt, M, N, K)
+            frame = big.clone()
+            frame[1:M + 1, 4:N + 4] = 77.0
+            assert bool((frame == 77.0).all()), "stores outside D"
+            dt_ = torch.zeros(N, M, device="cuda")                 # column-major D
+            mh.gemm_(mma, T(dt_, (M, N), (1, M)), T(a), T(b))
+            torch.cuda.synchronize()
+            assert torch.equal(dt_.t().cpu().double(), ref), (tdt, M, N, K, "column-major D")
+
+
 @pytest.mark.parametrize("M", [1, 16, 17, 48, 64])
 def test_short_m_line_staging_kernel(mh, M):
     """K of whole 128-byte lines runs on the kernel that stages them through LDS: any M <= 64 and any N (16 and

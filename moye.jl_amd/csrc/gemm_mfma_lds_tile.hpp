@@ -273,7 +273,8 @@ __device__ __forceinline__ void gemm_mfma_tn_lds_tile(GemmArgs p) {
     // apart, so that at any moment the chip asks memory for eight different column blocks of A and B instead of one
     // (with K-major operands and a power-of-two pitch one column block lives in few channels).  k_of() hands out the
     // indices of successive k-tiles in that rotated order; the sum over k starts elsewhere but is the same sum.
-    int k_next = (!kRagged && (p.flags & kGemmRotateK)) ? (int)((int64_t)(blockIdx.x % p.xcds) * ktiles / p.xcds) : 0;  // (ragged: the last k-tile in time is the last in K)
+    // (a K tail: the k-tile that holds it is masked as the last in time, so it has to be the last in K as well)
+    int k_next = ((p.flags & kGemmRotateK) && !(kRagged && k_rem)) ? (int)((int64_t)(blockIdx.x % p.xcds) * ktiles / p.xcds) : 0;
     auto k_of = [&]() {
         const int kt_now = k_next;
         k_next = k_next + 1 == ktiles ? 0 : k_next + 1;

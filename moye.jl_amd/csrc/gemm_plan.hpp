@@ -99,18 +99,21 @@ inline TileChoice gemm_choose(int64_t M, int64_t N, int64_t k_bytes, bool f32_in
 }
 
 // A short A (at most 64 rows, K in 16-byte pieces) goes to the kernel that streams B once and reads all of A per workgroup
-// (gemm_mfma_skinny.hip) -- except more than 16 rows with a short K and many columns: each of that kernel's waves then
-// has too few lines of K to cover the latency and A comes out of the L2s as often as B out of memory, and 128 x 128
-// tiles, part empty as they are, take less.  bf16, us on that kernel / on tiles: 64 x 65536 x 2048 62.9 / 43.3;
-// 32 x 65536 x 2048 62.8 / 40.1; 64 x 65536 x 256 30.6 / 15.1; 64 x 32768 x 2048 31.3 / 27.4; 64 x 24576 x 256 14.5 / 8.9;
-// 64 x 65536 x 3072 94.2 / 76.7; 64 x 131072 x 4096 228.6 / 177.2.  But 64 x 16384 x 2048 16.0 / 24.3;
-// 64 x 32768 x 4096 54.5 / 60.6; 64 x 65536 x 4096 111.9 / 124.4; 16 x 32768 x 2048 22.4 / 26.2.
+// (gemm_mfma_skinny.hip) -- except more than 16 rows with many columns: that kernel then brings A out of the L2s as
+// often as B out of memory and has one stage in flight per wave, which holds it near 5 TB/s of B, and 128 x 128 tiles,
+// part empty as they are, take less once there are more of them than CUs (the hand-ordered instance with two workgroups
+// on a CU) or, with a very short K, from three quarters of the CUs on.  bf16, us with a different B on every call (so
+// that the memory-side cache does not serve it), that kernel / tiles: 64 x 65536 x 2048 63.8 / 47.1; 32 x 65536 x 2048
+// 59.8 / 46.3; 64 x 36864 x 2048 44.9 / 40.0; 64 x 65536 x 4096 107.9 / 92.8; 64 x 65536 x 8192 201.3 / 181.5;
+// 24 x 65536 x 1024 37.4 / 25.7; 64 x 262144 x 2048 265.0 / 209.7; 64 x 32768 x 1024 22.7 / 21.5; 64 x 24576 x 512
+// 16.3 / 12.6.  But 64 x 32768 x 2048 32.7 / 36.7; 64 x 28672 x 8192 95.7 / 134.8; 48 x 49152 x 8192 132.8 / 149.3;
+// 16 x 65536 x 2048 42.4 / 46 and 64 x 16384 x 2048 17.6 / 34.3.
 inline bool gemm_short_m(int64_t M, int64_t N, int64_t k_bytes, int cus) {
     if (M > 64 || k_bytes % 16) return false;
     if (M <= 16) return true;
-    const int64_t tiles = N / 128;
-    return !((tiles >= 3 * (int64_t)cus / 4 && k_bytes <= 4096) || (tiles >= 2 * (int64_t)cus && k_bytes <= 6144) ||
-             (tiles >= 4 * (int64_t)cus && k_bytes <= 8192));
+    const int64_t tiles = (N + 127) / 128;
+    if (tiles > cus) return !(k_bytes <= 8192 || (M > 48 && tiles >= 2 * (int64_t)cus));
+    return !(4 * tiles >= 3 * (int64_t)cus && k_bytes <= 2048);
 }
 
 }  // namespace moye

@@ -300,10 +300,11 @@ def test_known_shapes_run_on_the_instances_they_are_meant_for():
     assert step_names(run_case(bf16, bf16, 64, 28672, 8192))[0].startswith("gemm_mfma_skinny_lds<InBF16,OutBF16,mt=4,ntw=4,waves=4,stages=2>")
     assert step_names(run_case(bf16, bf16, 48, 16384, 4096))[0].startswith("gemm_mfma_skinny_lds<InBF16,OutBF16,mt=3,ntw=4,waves=4,stages=2>")
     assert ",ntw=2," in step_names(run_case(bf16, bf16, 64, 8192, 8192))[0]
-    # more than 16 rows, a short K and columns for 128-wide tiles on three quarters of the CUs: tiles, not the short-M kernel
+    # more than 16 rows and more 128-wide tiles than CUs (a very short K: three quarters of the CUs): tiles, not the short-M kernel
     for (M, N, K, fam) in ((64, 65536, 2048, "gemm_mfma_tn_256_w4"), (17, 24576, 512, "gemm_mfma_tn_128"), (64, 65536, 3072, "gemm_mfma_tn_256_w4"),
-                           (64, 131072, 4096, "gemm_mfma_tn_256_w4"), (64, 65536, 4096, "gemm_mfma_skinny_lds"), (64, 24448, 512, "gemm_mfma_skinny_lds"),
-                           (16, 65536, 512, "gemm_mfma_skinny_lds"), (64, 32768, 2056, "gemm_mfma_skinny_lds")):
+                           (64, 131072, 4096, "gemm_mfma_tn_256_w4"), (64, 65536, 4096, "gemm_mfma_tn_256_w4"), (64, 24448, 512, "gemm_mfma_skinny_lds"),
+                           (64, 65536, 8192, "gemm_mfma_tn_256_w4"), (48, 49152, 8192, "gemm_mfma_skinny_lds"), (64, 32768, 2048, "gemm_mfma_skinny_lds"),
+                           (64, 32768, 1024, "gemm_mfma_tn_128"), (16, 65536, 512, "gemm_mfma_skinny_lds"), (64, 32768, 2056, "gemm_mfma_skinny_lds")):
         assert run_case(bf16, bf16, M, N, K)["steps"][0]["family"] == fam, (M, N, K)
     # small N and a long K: the library's own K ranges for the line kernel, then the reduction
     p = run_case(bf16, f32, 16, 1024, 32768, split_k=-1)

@@ -357,6 +357,134 @@ __global__ __launch_bounds__(256) void fill_rows_kernel(u32x4* x, ELayout lx, in
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256) x[e_offset(lx, i)] = pattern;
 }
 
+// ---- an operand whose unit stride lies on another mode than the destination's -----------------------------------------
+// (d = a + b' with b' a transposed view, axpby! between a column-major and a row-major array.)  The general kernels
+// read such an operand in single elements a pitch apart.  Here a workgroup takes a TILE x TILE block of the two modes
+// concerned -- mode 0, the destination's unit stride, and mode j, that operand's --, brings the operand's block into LDS
+// along mode j (rows padded by one element: both directions free of bank conflicts for 4-byte elements) and computes
+// along mode 0, reading the destination and every operand that is laid out like it directly.  The modes beside these
+// two are taken apart once per workgroup.  The arithmetic is the general kernels'.
+struct EwTiled {
+    ELayout ld, l0, l1;      // destination, first and second operand (same modes, ordered by the destination's strides)
+    int32_t j;               // the mode whose stride is 1 in the operands that go through LDS
+    int32_t tiles_p, tiles_q;
+    bool lds0, lds1, has1;
+};
+
+template <typename El, int TILE, bool kMap>
+__global__ __launch_bounds__(256) void ew_tiled_kernel(int32_t op, typename El::compute ca, typename El::compute cb, bool b_is_zero,
+                                                       typename El::storage* d, const typename El::storage* u0,
+                                                       const typename El::storage* u1, EwTiled g) {
+    typedef typename El::compute T;
+    typedef typename El::storage S;
+    extern __shared__ __align__(16) char tile_bytes[];  // one padded block per operand that goes through LDS
+    S* const tile0 = reinterpret_cast<S*>(tile_bytes);
+    S* const tile1 = tile0 + (g.lds0 ? TILE * (TILE + 1) : 0);
+    const uint32_t bid = blockIdx.x;
+    const uint32_t tp = bid % (uint32_t)g.tiles_p, rest0 = bid / (uint32_t)g.tiles_p;
+    const uint32_t tq = rest0 % (uint32_t)g.tiles_q;
+    uint32_t rest = rest0 / (uint32_t)g.tiles_q;
+    int64_t bd = 0, b0 = 0, b1 = 0;  // where this workgroup's block starts in each array, the two tiled modes aside
+#pragma unroll 1
+    for (int m = 1; m < g.ld.rank; ++m) {
+        if (m == g.j) continue;
+        const uint32_t extent = (uint32_t)g.ld.shape[m], q = rest / extent, r = rest - q * extent;
+        bd += (int64_t)r * g.ld.stride[m];
+        b0 += (int64_t)r * g.l0.stride[m];
+        b1 += (int64_t)r * g.l1.stride[m];
+        rest = q;
+    }
+    const int64_t p0 = (int64_t)tp * TILE, q0 = (int64_t)tq * TILE;
+    const int np = (int)min((int64_t)TILE, g.ld.shape[0] - p0), nq = (int)min((int64_t)TILE, g.ld.shape[g.j] - q0);
+    const int lo = threadIdx.x % TILE, hi0 = threadIdx.x / TILE;
+    constexpr int STEP = 256 / TILE, IT = TILE / STEP;
+    // (every loop below has IT trips with the bounds as predicates, so that a lane's IT loads are in flight together)
+    // the operands that run along mode j: lanes along j, the block's rows of mode 0 one after the other
+    if (g.lds0 || g.lds1) {
+        S r0[IT], r1[IT];
+#pragma unroll
+        for (int k = 0; k < IT; ++k) {
+            const int lp = hi0 + k * STEP;
+            r0[k] = r1[k] = S(0);
+            if (lo < nq && lp < np) {
+                if (g.lds0) r0[k] = u0[b0 + (p0 + lp) * g.l0.stride[0] + (q0 + lo)];
+                if (g.lds1) r1[k] = u1[b1 + (p0 + lp) * g.l1.stride[0] + (q0 + lo)];
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < IT; ++k) {
+            const int lp = hi0 + k * STEP;
+            if (g.lds0) tile0[lp * (TILE + 1) + lo] = r0[k];
+            if (g.lds1) tile1[lp * (TILE + 1) + lo] = r1[k];
+        }
+        __syncthreads();
+    }
+    S e0[IT], e1[IT], old[IT];
+#pragma unroll
+    for (int k = 0; k < IT; ++k) {
+        const int lq = hi0 + k * STEP;
+        const bool in = lo < np && lq < nq;
+        e0[k] = e1[k] = old[k] = S(0);
+        if (g.lds0) e0[k] = tile0[lo * (TILE + 1) + lq];
+        else if (in) e0[k] = u0[b0 + (p0 + lo) * g.l0.stride[0] + (q0 + lq) * g.l0.stride[g.j]];
+        if (kMap && g.has1) {
+            if (g.lds1) e1[k] = tile1[lo * (TILE + 1) + lq];
+            else if (in) e1[k] = u1[b1 + (p0 + lo) * g.l1.stride[0] + (q0 + lq) * g.l1.stride[g.j]];
+        }
+        if (!kMap && !b_is_zero && in) old[k] = d[bd + (p0 + lo) + (q0 + lq) * g.ld.stride[g.j]];
+    }
+#pragma unroll
+    for (int k = 0; k < IT; ++k) {
+        const int lq = hi0 + k * STEP;
+        if (lo >= np || lq >= nq) continue;
+        S* const dp = d + bd + (p0 + lo) + (q0 + lq) * g.ld.stride[g.j];
+        const T x = El::load(&e0[k]);
+        if constexpr (kMap) {
+            const T y = g.has1 ? El::load(&e1[k]) : cb;  // (cb: the scalar operand)
+            El::store(dp, El::round(map_op(op, x, y)));
+        } else {
+            const T ax = El::round(ca * x);
+            if (b_is_zero) El::store(dp, ax);
+            else El::store(dp, El::round(ax + El::round(cb * El::load(&old[k]))));
+        }
+    }
+}
+
+// Does the tiled kernel apply?  Layouts of one shape, ordered by the destination's strides (order_modes_by_stride), the
+// destination's unit stride on mode 0, and an operand whose unit stride lies on another mode j with at least 16
+// elements along both; every other operand runs along mode 0 or along j as well, or is read as it comes.
+bool plan_tiled(const ELayout& ld, const ELayout* const* ops, int nops, int tile, EwTiled* g) {
+    if (ld.rank < 2 || ld.stride[0] != 1 || ld.shape[0] < 16) return false;
+    int j = -1;
+    for (int q = 0; q < nops && j < 0; ++q) {
+        if (ops[q]->stride[0] == 1) continue;
+        for (int m = 1; m < ld.rank; ++m)
+            if (ops[q]->stride[m] == 1 && ld.shape[m] >= 16) { j = m; break; }
+    }
+    if (j < 0) return false;
+    g->ld = ld;
+    g->l0 = *ops[0];
+    g->l1 = nops > 1 ? *ops[1] : *ops[0];
+    g->has1 = nops > 1;
+    g->j = j;
+    g->lds0 = ops[0]->stride[0] != 1 && ops[0]->stride[j] == 1;
+    g->lds1 = nops > 1 && ops[1]->stride[0] != 1 && ops[1]->stride[j] == 1;
+    const int64_t tp = (ld.shape[0] + tile - 1) / tile, tq = (ld.shape[j] + tile - 1) / tile;
+    int64_t rest = 1;
+    for (int m = 1; m < ld.rank; ++m)
+        if (m != j) rest *= ld.shape[m];
+    if (tp * tq * rest >= ((int64_t)1 << 31) || rest >= ((int64_t)1 << 31)) return false;
+    g->tiles_p = (int32_t)tp;
+    g->tiles_q = (int32_t)tq;
+    return true;
+}
+template <typename El>
+constexpr int tiled_edge() { return sizeof(typename El::storage) == 8 ? 32 : 64; }
+template <typename El>
+size_t tiled_lds(const EwTiled& g) {
+    return (size_t)((g.lds0 ? 1 : 0) + (g.lds1 ? 1 : 0)) * tiled_edge<El>() * (tiled_edge<El>() + 1) * sizeof(typename El::storage);
+}
+
 // Can every one of these (same-shape, stride-ordered) layouts be recast to pieces of `per` elements?  If so, does it.
 bool recast_rows(ELayout* const* ls, const void* const* ptrs, int count, int per) {
     if (per <= 1) return false;
@@ -427,7 +555,7 @@ float host_round_bf16(float f) {
 
 template <typename El>
 static void launch_axpby(typename El::compute a, const void* x, const ELayout& lx, typename El::compute b, void* y, const ELayout& ly,
-                         int64_t n, bool is_dense, bool rows, hipStream_t st) {
+                         int64_t n, bool is_dense, bool rows, bool ordered, hipStream_t st) {
     typedef typename El::storage S;
     const S* xs = static_cast<const S*>(x);
     S* ys = static_cast<S*>(y);
@@ -438,6 +566,13 @@ static void launch_axpby(typename El::compute a, const void* x, const ELayout& l
         return;
     }
     if (!is_dense) {
+        EwTiled g;
+        const ELayout* ops[1] = {&lx};
+        if (ordered && plan_tiled(ly, ops, 1, tiled_edge<El>(), &g)) {
+            const int64_t blocks = (int64_t)g.tiles_p * g.tiles_q * (n / (ly.shape[0] * ly.shape[g.j]));
+            ew_tiled_kernel<El, tiled_edge<El>(), false><<<(unsigned)blocks, 256, tiled_lds<El>(g), st>>>(0, a, b, b0, ys, xs, xs, g);
+            return;
+        }
         const dim3 grid((unsigned)std::min<int64_t>((n + 255) / 256, 256 * 16));
         axpby_kernel<El><<<grid, 256, 0, st>>>(a, xs, lx, b, ys, ly, n, b0, same_modes_32(lx, ly, n));
         return;
@@ -450,7 +585,7 @@ static void launch_axpby(typename El::compute a, const void* x, const ELayout& l
 
 template <typename El>
 static void launch_map(int32_t op, void* d, const ELayout& ld, const void* a, const ELayout& la, const void* b, const ELayout& lb,
-                       int64_t nb, typename El::compute s, int64_t n, bool is_dense, bool rows, hipStream_t st) {
+                       int64_t nb, typename El::compute s, int64_t n, bool is_dense, bool rows, bool ordered, hipStream_t st) {
     typedef typename El::storage S;
     S* ds = static_cast<S*>(d);
     const S* as = static_cast<const S*>(a);
@@ -462,6 +597,13 @@ static void launch_map(int32_t op, void* d, const ELayout& ld, const void* a, co
         return;
     }
     if (!is_dense) {
+        EwTiled g;
+        const ELayout* ops[2] = {&la, &lb};
+        if (ordered && plan_tiled(ld, ops, bs ? 2 : 1, tiled_edge<El>(), &g)) {
+            const int64_t blocks = (int64_t)g.tiles_p * g.tiles_q * (n / (ld.shape[0] * ld.shape[g.j]));
+            ew_tiled_kernel<El, tiled_edge<El>(), true><<<(unsigned)blocks, 256, tiled_lds<El>(g), st>>>(op, s, s, false, ds, as, bs ? bs : as, g);
+            return;
+        }
         const dim3 grid((unsigned)std::min<int64_t>((n + 255) / 256, 256 * 16));
         map_kernel<El><<<grid, 256, 0, st>>>(op, ds, ld, as, la, bs, lb, nb, s, n,
                                              same_modes_32(ld, la, n) && (!bs || (nb == n && same_modes_32(ld, lb, n))));
@@ -484,20 +626,21 @@ int32_t axpby_dispatch(double a, const moye_tensor* X, double b, const moye_tens
     if (n == 0) return MOYE_OK;
     ELayout lx = elayout_of(*X), ly = elayout_of(*Y);
     bool fast = dense(*X) && dense(*Y) && aligned16(X->ptr) && aligned16(Y->ptr);
-    bool rows = false;
+    bool rows = false, ordered = false;  // ordered: the layouts have one shape mode by mode and are sorted by Y's strides
     if (!fast) {
         ELayout* all[2] = {&ly, &lx};
         const void* ptrs[2] = {Y->ptr, X->ptr};
         if (order_modes_by_stride(all, 2)) {
+            ordered = true;
             if (dense_l(lx) && dense_l(ly) && aligned16(X->ptr) && aligned16(Y->ptr)) fast = true;  // one run each, in the same order
             else rows = recast_rows(all, ptrs, 2, 16 / dtype_bytes(X->dtype));
         }
     }
     switch (X->dtype) {
-        case MOYE_F32: launch_axpby<ElF32>((float)a, X->ptr, lx, (float)b, Y->ptr, ly, n, fast, rows, st); break;
-        case MOYE_F64: launch_axpby<ElF64>(a, X->ptr, lx, b, Y->ptr, ly, n, fast, rows, st); break;
-        case MOYE_F16: launch_axpby<ElF16>(host_round_f16((float)a), X->ptr, lx, host_round_f16((float)b), Y->ptr, ly, n, fast, rows, st); break;
-        case MOYE_BF16: launch_axpby<ElBF16>(host_round_bf16((float)a), X->ptr, lx, host_round_bf16((float)b), Y->ptr, ly, n, fast, rows, st); break;
+        case MOYE_F32: launch_axpby<ElF32>((float)a, X->ptr, lx, (float)b, Y->ptr, ly, n, fast, rows, ordered, st); break;
+        case MOYE_F64: launch_axpby<ElF64>(a, X->ptr, lx, b, Y->ptr, ly, n, fast, rows, ordered, st); break;
+        case MOYE_F16: launch_axpby<ElF16>(host_round_f16((float)a), X->ptr, lx, host_round_f16((float)b), Y->ptr, ly, n, fast, rows, ordered, st); break;
+        case MOYE_BF16: launch_axpby<ElBF16>(host_round_bf16((float)a), X->ptr, lx, host_round_bf16((float)b), Y->ptr, ly, n, fast, rows, ordered, st); break;
         default:
             return fail(MOYE_ERR_UNSUPPORTED, "axpby!: element type %s is not a floating-point type this build handles", dtype_name(X->dtype));
     }
@@ -536,20 +679,21 @@ int32_t map_dispatch(int32_t op, const moye_tensor* D, const moye_tensor* A, con
     const void* bp = B ? B->ptr : nullptr;
     bool fast = dense(*D) && dense(*A) && aligned16(D->ptr) && aligned16(A->ptr) &&
                 (!B || (nb == n && dense(*B) && aligned16(B->ptr)));
-    bool rows = false;
+    bool rows = false, ordered = false;
     if (!fast && (!B || nb == n)) {  // (a b that is broadcast is tied to the leading modes of dst as the caller wrote them)
         ELayout* all[3] = {&ld, &la, &lb};
         const void* ptrs[3] = {D->ptr, A->ptr, bp};
         if (order_modes_by_stride(all, B ? 3 : 2)) {
+            ordered = true;
             if (dense_l(ld) && dense_l(la) && (!B || dense_l(lb)) && aligned16(D->ptr) && aligned16(A->ptr) && (!B || aligned16(B->ptr))) fast = true;
             else rows = recast_rows(all, ptrs, B ? 3 : 2, 16 / dtype_bytes(D->dtype));
         }
     }
     switch (D->dtype) {
-        case MOYE_F32: launch_map<ElF32>(op, D->ptr, ld, A->ptr, la, bp, lb, nb, (float)scalar, n, fast, rows, st); break;
-        case MOYE_F64: launch_map<ElF64>(op, D->ptr, ld, A->ptr, la, bp, lb, nb, scalar, n, fast, rows, st); break;
-        case MOYE_F16: launch_map<ElF16>(op, D->ptr, ld, A->ptr, la, bp, lb, nb, host_round_f16((float)scalar), n, fast, rows, st); break;
-        case MOYE_BF16: launch_map<ElBF16>(op, D->ptr, ld, A->ptr, la, bp, lb, nb, host_round_bf16((float)scalar), n, fast, rows, st); break;
+        case MOYE_F32: launch_map<ElF32>(op, D->ptr, ld, A->ptr, la, bp, lb, nb, (float)scalar, n, fast, rows, ordered, st); break;
+        case MOYE_F64: launch_map<ElF64>(op, D->ptr, ld, A->ptr, la, bp, lb, nb, scalar, n, fast, rows, ordered, st); break;
+        case MOYE_F16: launch_map<ElF16>(op, D->ptr, ld, A->ptr, la, bp, lb, nb, host_round_f16((float)scalar), n, fast, rows, ordered, st); break;
+        case MOYE_BF16: launch_map<ElBF16>(op, D->ptr, ld, A->ptr, la, bp, lb, nb, host_round_bf16((float)scalar), n, fast, rows, ordered, st); break;
         default:
             return fail(MOYE_ERR_UNSUPPORTED, "map!: element type %s is not a floating-point type this build handles", dtype_name(D->dtype));
     }

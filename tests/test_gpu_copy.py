@@ -562,6 +562,61 @@ def test_dense_elementwise_paths_match_the_general_kernels(mh, dt):
         assert bool((z == 93).all())
 
 
+@pytest.mark.parametrize("dt", ["float32", "float64", "float16", "bfloat16"])
+def test_elementwise_with_a_transposed_operand_matches_the_dense_kernels(mh, dt):
+    """An operand whose unit stride lies on another mode than the destination's goes through LDS tiles: the same bits as the
+    dense kernels give on a contiguous copy of that operand.  Ragged extents, a batch mode, a pitched destination inside a
+    frame, one or both operands transposed, a scalar second operand, axpby! with and without the old Y."""
+    tdt = getattr(torch, dt)
+    g = torch.Generator(device="cuda").manual_seed(57)
+    itype = {2: torch.int16, 4: torch.int32, 8: torch.int64}[tdt.itemsize]
+
+    def rnd(*shape):
+        return (torch.randn(*shape, generator=g, device="cuda") * 3).to(tdt)
+
+    def flat(x):
+        return _tens(mh, x, [x.numel()], [1])
+
+    for (R, C, Bn) in ((64, 64, 1), (200, 77, 1), (130, 1000, 3), (16, 16, 5), (1025, 129, 2)):
+        # destination d[b][r][c] with c contiguous and a pitch of C + 3 inside a frame; xt[b][c][r] with r contiguous
+        frame = torch.full((Bn, R, C + 3), 55.0, device="cuda").to(tdt)
+        x_same, xt, yt = rnd(Bn, R, C), rnd(Bn, C, R), rnd(Bn, C, R)
+        shape, d_str = (C, R, Bn), (1, C + 3, R * (C + 3))
+        same_str, t_str = (1, C, R * C), (R, 1, R * C)
+        xt_c, yt_c = xt.transpose(1, 2).contiguous(), yt.transpose(1, 2).contiguous()   # what the transposed views hold, dense
+        for op in ("add", "max", "div"):
+            for (a_t, b_kind) in ((True, "same"), (False, "t"), (True, "t"), (True, "scalar")):
+                a_dense = xt_c if a_t else x_same
+                b_dense = {"same": x_same, "t": yt_c, "scalar": None}[b_kind]
+                want = torch.zeros(Bn, R, C, device="cuda").to(tdt)
+                mh.map_(op, flat(want), flat(a_dense), flat(b_dense) if b_dense is not None else None, 1.75)
+                d = frame.clone()
+                ta = _tens(mh, xt, shape, t_str) if a_t else _tens(mh, x_same, shape, same_str)
+                tb = {"same": lambda: _tens(mh, x_same, shape, same_str), "t": lambda: _tens(mh, yt, shape, t_str), "scalar": lambda: None}[b_kind]()
+                mh.map_(op, _tens(mh, d, shape, d_str), ta, tb, 1.75)
+                torch.cuda.synchronize()
+                got = d[:, :, :C].contiguous()
+                same = got.view(itype) == want.view(itype)
+                assert bool((same | (torch.isnan(got.float()) & torch.isnan(want.float()))).all()), (dt, R, C, Bn, op, a_t, b_kind)
+                assert bool((d[:, :, C:].float() == 55.0).all()), "stores into the padding"
+        for b in (0.0, -1.25):
+            y0 = rnd(Bn, R, C)
+            want = y0.clone()
+            mh.axpby_(0.75, flat(xt_c), b, flat(want))
+            d = frame.clone()
+            d[:, :, :C] = y0
+            mh.axpby_(0.75, _tens(mh, xt, shape, t_str), b, _tens(mh, d, shape, d_str))
+            torch.cuda.synchronize()
+            assert torch.equal(d[:, :, :C].contiguous().view(itype), want.view(itype)), (dt, R, C, Bn, "axpby", b)
+            assert bool((d[:, :, C:].float() == 55.0).all()), "stores into the padding"
+    if dt == "float32":   # and against torch where the rounding is plain IEEE
+        x, y = rnd(300, 500), rnd(500, 300)
+        d = torch.zeros(300, 500, device="cuda")
+        mh.map_("add", _tens(mh, d, (500, 300), (1, 500)), _tens(mh, x, (500, 300), (1, 500)), _tens(mh, y, (500, 300), (300, 1)))
+        torch.cuda.synchronize()
+        assert torch.equal(d, x + y.t())
+
+
 def test_axpby_errors(mh):
     x = torch.zeros(8, device="cuda")
     y = torch.zeros(8, dtype=torch.float16, device="cuda")

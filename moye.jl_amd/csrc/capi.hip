@@ -463,10 +463,12 @@ static int32_t gemm_plan_build(const moye_tiled_mma* mma, const moye_tensor* tD,
     // ask memory for at one time to matter: more 256 x 256 tiles than CUs, or rows of 32 KiB and more (measured, 256 x 256
     // tile, same box, alternating runs: bf16 8192^3 1408 TFLOP/s against 1372, fp16 4096 x 4096 x 16384 +4 %; fp16 4096^3
     // 1333 against 1338, so not there)
-    // A short A or B on tiles is a bandwidth problem whose workgroups all walk K in step: with a power-of-two pitch they
-    // then ask few memory channels for everything at one time (bf16 64 x 65536 x 2048 on 128 x 128 tiles, a B that is not
-    // in the memory-side cache: 68.2 us, 46.8 with the XCDs an eighth of K apart; 64 x 65536 x 4096 124.2 -> 92.2).
-    const bool rotate_k = (int64_t)(M / 256) * (N / 256) > cus || (int64_t)K * dtype_bytes(in_dt) >= 32768 || M <= 64 || N <= 64;
+    // A problem with a short side leans on memory, and its workgroups all walk K in step: with a power-of-two pitch they
+    // then ask few memory channels for everything at one time.  bf16, a B that is not in the memory-side cache, us without ->
+    // with the XCDs an eighth of K apart: 64 x 65536 x 2048 on 128 x 128 tiles 68.2 -> 46.8; 64 x 65536 x 4096 124.2 -> 92.2;
+    // 128 x 65536 x 4096 126.3 -> 98.1; 256 x 65536 x 2048 75.3 -> 68.3; 512 x 16384 x 4096 80.9 -> 77.3; 1024 x 16384 x 2048
+    // 58.3 -> 57.1; 2048 x 8192 x 2048 57.5 -> 56.9; 4096 x 4096 x 2048 52.4 -> 52.2.  So: a side of at most 1024.
+    const bool rotate_k = (int64_t)(M / 256) * (N / 256) > cus || (int64_t)K * dtype_bytes(in_dt) >= 32768 || std::min(M, N) <= 1024;
     // D written with non-temporal stores (measured, same box, alternating runs, ordinary -> non-temporal, TFLOP/s): fp16
     // 4096^3 fp16 out 1339 -> 1345, fp32 out 1285 -> 1253; fp16 8192^3 fp16 out 1382 -> 1401; bf16 8192^3 fp32 out 1412 ->
     // 1452; fp8 4096^3 bf16 out 2373 -> 2450, 8192^3 2760 -> 2745; fp16 2048^3 and 3072^3 +1.6 %.  So: 16-bit results

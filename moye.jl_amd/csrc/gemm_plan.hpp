@@ -1,17 +1,19 @@
 // Host-side choice of CTA tile and K ranges for a gemm! whose tile is left to the library and that does not fill the chip
-// with 256 x 256 tiles: a small cost model instead of thresholds.  Its per-k-tile times are fitted to fp16 timings on one
-// MI355X; the number of compute units that share the work is an argument (DeviceShape::cus).
+// with 256 x 256 tiles: a small cost model instead of thresholds.  Its per-k-tile times are fitted to bf16 timings on one
+// MI355X with a different B on every call (operands that stay in the 256 MiB memory-side cache between calls run the
+// kernels with one workgroup per CU up to 1.4 times faster, which real callers with several weight matrices do not see);
+// the number of compute units that share the work is an argument (DeviceShape::cus).
 //
 //   time = 3 us + k-tiles per workgroup x t(tile, workgroups resident on a CU) [x rounds] + second pass of a K split
 //
 // with k-tiles of 128 bytes of K and, per k-tile and workgroup,
-//   128 x 128 tiles (gemm_mfma128.hip, two workgroups fit a CU):   0.52 us alone on its CU, 0.94 us with a neighbour
-//   64 x 64 tiles (gemm_mfma.hip, four fit):                       0.40 / 0.47 / 0.66 / 0.84 us for 1 / 2 / 3 / 4 on a CU
-//                                                                  (alone: 0.33 while the operands fit the L2s, 0.49 beyond)
-// (256 x 8192 x 8192 on 128 workgroups of 128 x 128: 68 us; 4096^3 as two rounds of 512: 123 us; 1024^3 on 256
-// workgroups of 64 x 64: 8.3 us; 2048^3 on 1024: 31.5 us), and a second pass that moves the fp32 partial products
-// at about 6 TB/s (they are still in the caches) after 3 us of launch.  Ragged tiles cost the 128 x 128 kernel
-// 15 % more; the 64 x 64 kernel has no ragged form.  fp32 operands have their own per-k-tile times.
+//   128 x 128 tiles (gemm_mfma128.hip, two workgroups fit a CU):   0.85 us alone on its CU, 1.08 us with a neighbour
+//   64 x 64 tiles (gemm_mfma.hip, four fit):                       0.48 / 0.73 / 0.86 / 1.00 us for 1 / 2 / 3 / 4 on a CU
+// (512 x 8192 x 8192 on 256 workgroups of 128 x 128: 111.8 us, in two K ranges on 512: 89.4; 1024 x 4096 x 14336 on 256:
+// 198.5; 2048 x 4096 x 4096 on 512: 72.3; 2048^3 on 1024 workgroups of 64 x 64: 33.0; 512 x 4096 x 4096 on 512: 49.8), and a
+// second pass that moves the fp32 partial products at about 6 TB/s (they are still in the caches) after 3 us of launch.
+// Ragged tiles cost the 128 x 128 kernel 15 % more; the 64 x 64 kernel has no ragged form.  fp32 operands have their own
+// per-k-tile times.
 #pragma once
 
 #include <cstdint>
@@ -32,7 +34,7 @@ inline double gemm_plan_cost(int tile, int split, int64_t M, int64_t N, int64_t 
     // an eighth of the 16-bit rate per byte of K, and are bound by it (2048^3 on 256 workgroups of 128 x 128: 124.5 us;
     // 4096 x 2048 x 4096 on 512: 465 us; 2560^3 on 400: 291 us; 3072^3 on 576: 522 us; 1024^3 on 256 workgroups of
     // 64 x 64: 25.7 us; 2048^3 on 1024: 156 us; 3072^3 on 2304: 509 us)
-    static const double t128_16[3] = {0, 0.52, 0.94}, t64_16[5] = {0, 0.40, 0.47, 0.66, 0.84};
+    static const double t128_16[3] = {0, 0.85, 1.08}, t64_16[5] = {0, 0.48, 0.73, 0.86, 1.00};
     static const double t128_32[3] = {0, 1.92, 3.62}, t64_32[5] = {0, 0.71, 1.25, 1.80, 2.40};
     const double* t = tile == 128 ? (f32_in ? t128_32 : t128_16) : (f32_in ? t64_32 : t64_16);
     const double ktiles = (double)((k_bytes / split + 127) / 128);
@@ -68,19 +70,21 @@ inline TileChoice gemm_plan(int64_t M, int64_t N, int64_t k_bytes, bool f32_in, 
 }
 
 // The same problem on 256 x 256 tiles, one workgroup per CU: 9 us + per k-tile 1.44 us in a round that fills the chip,
-// 0.98 us in one that fills half of it or less (fewer requesters, and a higher clock on a part that is power-limited when
-// full), linear in between (fp16 K = 4096: 256 tiles 101 us, 224 91, 192 83, 144 73, 128 72); a quarter more for the
-// guarded instance (130 x 32768 x 4096 on 128 ragged tiles: 99 us).
-inline double gemm_plan_cost_256(int64_t M, int64_t N, int64_t k_bytes, bool f32_in, bool ragged, int cus) {
-    const int64_t tiles = ((M + 255) / 256) * ((N + 255) / 256), full = tiles / cus, rest = tiles % cus;
+// 1.30 us in one that fills half of it or less, linear in between (bf16, B not cached: 512 x 8192 x 8192 on 64 tiles 176 us,
+// in two K ranges 109.1, in four 79.4; with B cached 0.98 us per k-tile up to half the chip: fp16 K = 4096, 144 tiles 73 us,
+// 128 72); a quarter more for the guarded instance (130 x 32768 x 4096 on 128 ragged tiles: 99 us).  `split` K ranges:
+// that many times the workgroups with a share of K each, and the second pass.
+inline double gemm_plan_cost_256(int64_t M, int64_t N, int64_t k_bytes, bool f32_in, bool ragged, int cus, int split = 1) {
+    const int64_t tiles = ((M + 255) / 256) * ((N + 255) / 256) * split, full = tiles / cus, rest = tiles % cus;
     const int half = cus / 2 > 0 ? cus / 2 : 1;
-    const double ktiles = (double)((k_bytes + 127) / 128);
+    const double ktiles = (double)((k_bytes / split + 127) / 128);
     // (fp32: 7.05 us per k-tile however many CUs are busy: the matrix pipe alone sets the pace; 4096^3 909 us,
     // 3072^3 on 144 tiles 687 us, 4096 x 2048 x 4096 on 128 tiles 913 us)
     const double t_full = f32_in ? 7.05 : 1.44;
-    const double t_rest = rest == 0 ? 0.0 : f32_in ? 7.05 : rest <= half ? 0.98 : 0.98 + (double)(rest - half) / (double)half * 0.46;
+    const double t_rest = rest == 0 ? 0.0 : f32_in ? 7.05 : rest <= half ? 1.30 : 1.30 + (double)(rest - half) / (double)half * 0.14;
     double us = 9.0 + 6.0 * (double)(full + (rest ? 1 : 0) - 1) + ktiles * ((double)full * t_full + t_rest);
     if (ragged) us *= 1.25;
+    if (split > 1) us += 3.0 + (2.0 * split * 4.0 + 4.0) * (double)M * (double)N / 6.0e6;  // the second pass, as in gemm_plan_cost
     return us;
 }
 
@@ -94,6 +98,17 @@ inline TileChoice gemm_choose(int64_t M, int64_t N, int64_t k_bytes, bool f32_in
     if (((M + 255) / 256) * ((N + 255) / 256) >= cus / 4) {
         const double us = gemm_plan_cost_256(M, N, k_bytes, f32_in, ragged, cus);
         if (us <= best.us) best = TileChoice{256, 1, us};
+    }
+    // few whole 256 x 256 tiles and a long K: K ranges that bring the workgroups up to one per CU at most (bf16, a B that is
+    // not cached: 512 x 8192 x 8192 on 128 x 128 tiles 111.8 us, in two ranges 89.4, on 256 x 256 tiles in four ranges
+    // 79.4; 1024 x 4096 x 14336 198.5 / 145.2 / 113.5)
+    if (!ragged && !f32_in) {
+        const int64_t tiles = (M / 256) * (N / 256);
+        for (int s = 2; s <= max_split && tiles * s <= cus; s *= 2) {
+            if (k_bytes % s || (k_bytes / s) % 128 || k_bytes / s < 512) continue;
+            const double us = gemm_plan_cost_256(M, N, k_bytes, f32_in, false, cus, s);
+            if (us < best.us) best = TileChoice{256, s, us};
+        }
     }
     return best;
 }

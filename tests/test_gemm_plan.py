@@ -194,7 +194,8 @@ def run_case(in_dt, out_dt, M, N, K, **kw):
         assert len(reduces) == 1 and reduces[0]["split"] == kernels[-1]["split"] > 1 and plan["steps"][-1] is reduces[0], plan["text"]
         assert reduces[0]["M"] * reduces[0]["N"] == M * N
         if kw.get("split_k", 0) < 0 and cta == (0, 0, 0):
-            assert all(not s["tile"].startswith("256x") for s in kernels), plan["text"]   # tile and K ranges are one decision
+            # tile and K ranges are one decision: 256 x 256 tiles in K ranges only to bring the workgroups up to one per CU
+            assert all(not s["tile"].startswith("256x") or (M // 256) * (N // 256) * s["split"] <= plan["cus"] for s in kernels), plan["text"]
     elif kw.get("d_major", "n") == "n" and M > 1 and kernels and not kernels[0]["family"].startswith("gemm_universal"):
         covers_exactly_once(d_rectangles(plan, M, N, ob, N + kw.get("pad", (0, 0, 0))[2]), M, N)
     return plan

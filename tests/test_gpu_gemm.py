@@ -1371,6 +1371,42 @@ def test_split_k_exact_on_integers(mh, split):
     assert e.value.status == _lib.ERR_UNSUPPORTED
 
 
+@pytest.mark.parametrize("out_dt", [torch.float32, torch.float16, torch.bfloat16])
+def test_split_k_second_pass_in_pieces_of_four_gives_the_scalar_pass_its_bits(mh, out_dt):
+    """The second pass of a K split sums four neighbouring columns per lane when D's rows start on whole pieces of four
+    results; a D one element off that, or with an N that is no multiple of four, takes the element-wise pass.  Random
+    data, with C, alpha and an operation with a bias row: the same bits from both."""
+    from moye_hip import _lib
+    g = torch.Generator(device="cuda").manual_seed(61)
+    M, N, K = 384, 512, 4096
+    a = (torch.randn(M, K, generator=g, device="cuda") * K ** -0.5).half()
+    b = (torch.randn(N, K, generator=g, device="cuda") * K ** -0.5).half()
+    c = torch.randn(M, N, generator=g, device="cuda").to(out_dt)
+    bias = torch.randn(N, generator=g, device="cuda")
+    for split in (2, 4):
+        for cta, waves in (((128, 128, 64), (2, 2, 1)), ((256, 256, 64), (2, 4, 1))):
+            if cta[0] == 256 and M % 256: continue
+            mma = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=waves, cta_tile=cta, split_k=split)
+            for ep in (None, mh.gemm_epilogue(alpha=0.75, beta=-0.5, op=_lib.MAP_OPS["add"], operand=T(bias, (M, N), (0, 1)))):
+                d1 = torch.zeros(M, N, dtype=out_dt, device="cuda")
+                buf = torch.zeros(M, N + 8, dtype=out_dt, device="cuda")
+                d2 = buf[:, 1:N + 1]                                    # rows start one element off
+                need = mh.gemm_workspace_size(mma, T(d1), T(a), T(b), ep)
+                ws = torch.empty(need + 256, dtype=torch.uint8, device="cuda")
+                wp = (ws.data_ptr() + 255) // 256 * 256
+                mh.gemm_ex_(mma, T(d1), T(a), T(b), T(c) if ep else None, ep, wp, need)
+                mh.gemm_ex_(mma, T(d2), T(a), T(b), T(c) if ep else None, ep, wp, need)
+                torch.cuda.synchronize()
+                assert torch.equal(d1, d2), (out_dt, split, cta, ep is not None)
+                assert float(buf[:, 0].abs().max()) == 0.0 and float(buf[:, N + 1:].abs().max()) == 0.0, "stores outside D"
+    M = 256
+    mma = mh.tiled_mma_desc(mh.MFMA_F32_16x16x32_F16, atom_layout=(2, 2, 1), cta_tile=(128, 128, 64), split_k=2)
+    d = torch.zeros(M, N, dtype=out_dt, device="cuda")
+    mh.gemm_(mma, T(d), T(a[:M]), T(b))
+    torch.cuda.synchronize()
+    assert relerr(d, a[:M].double() @ b.double().t()) <= TOL16
+
+
 def test_split_k_long_k(mh):
     """A small C with a long K leaves most of the chip idle without a split: 256 x 256 x 65536 fp16."""
     g = torch.Generator().manual_seed(77)

@@ -222,7 +222,7 @@ struct LibraryChoice {
 };
 static LibraryChoice library_choice(const moye_tiled_mma* mma, int64_t M, int64_t N, int64_t K, int eb, int cus) {
     LibraryChoice c;
-    const bool short_m = gemm_short_m(M, N, K * eb, cus);
+    const bool short_m = gemm_short_m(M, N, K * eb, eb == 4, cus);
     if (mma->split_k >= 0 || mma->cta_tile_mnk[0] || mma->cta_tile_mnk[1] || mma->cta_tile_mnk[2] || short_m || (K * eb) % 16) return c;
     c.open = true;
     c.tile = gemm_choose(M, N, K * eb, eb == 4, (mma->flags & MOYE_GEMM_NO_WORKSPACE) ? 1 : 16, cus);
@@ -236,7 +236,7 @@ static LibraryChoice library_choice(const moye_tiled_mma* mma, int64_t M, int64_
 static int split_count(const moye_tiled_mma* mma, int64_t M, int64_t N, int64_t K, int eb, int cus) {
     if (mma->split_k >= 0) return mma->split_k > 1 ? mma->split_k : 1;
     if (mma->flags & MOYE_GEMM_NO_WORKSPACE) return 1;  // nowhere to put the partial products
-    if (mma->cta_tile_mnk[0] == 0 && mma->cta_tile_mnk[1] == 0 && gemm_short_m(M, N, K * eb, cus)) {
+    if (mma->cta_tile_mnk[0] == 0 && mma->cta_tile_mnk[1] == 0 && gemm_short_m(M, N, K * eb, eb == 4, cus)) {
         // the short-M kernel (gemm_mfma_skinny.hip): fastest unsplit when its workgroups fill the chip (bf16 64 x 8192 x 8192:
         // 30.4 us against 41.3 with two ranges and the second pass); K ranges are whole lines
         return skinny_lines_split(M, N, K * eb, cus);
@@ -515,7 +515,7 @@ static int32_t gemm_plan_build(const moye_tiled_mma* mma, const moye_tensor* tD,
         if (lane_op(g)) g.flags |= kGemmEpiLaneOp;
         return gemm_mfma_tn_dispatch(in_dt, D.dtype, bm, bn, bk, waves, mma->stages, g, plan, lib_tile);
     }
-    if (D.rs == 1 && bm == 0 && bn == 0 && gemm_short_m(M, N, (int64_t)K * dtype_bytes(in_dt), plan.shape.cus)) {
+    if (D.rs == 1 && bm == 0 && bn == 0 && gemm_short_m(M, N, (int64_t)K * dtype_bytes(in_dt), dtype_bytes(in_dt) == 4, plan.shape.cus)) {
         // column-major D with a short A: the short-M kernel writes D through both of its strides
         g.A = A.ptr; g.B = B.ptr; g.M = M; g.N = N; g.lda = A.rs; g.ldb = B.rs; g.ldd = 1; g.ldd_n = D.cs;
         g.C = tC ? C.ptr : nullptr; g.ldc_m = C.rs; g.ldc_n = C.cs; g.D = D.ptr;

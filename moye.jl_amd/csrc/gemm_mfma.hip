@@ -345,7 +345,7 @@ int32_t gemm_mfma_tn_dispatch(int32_t in_dt, int32_t out_dt, int bm, int bn, int
     const int cus = plan.shape.cus;
     if (a.flags & kGemmAtom32) return dispatch_atom32(in_dt, out_dt, bm, bn, bk_elems, waves, stages, a, plan);
     // a short A (at most 64 rows) is a bandwidth problem: stream B once, no CTA tiling
-    if ((bm == 0 && bn == 0 && gemm_short_m(a.M, a.N, (int64_t)a.K * eb * (a.split > 1 ? a.split : 1), cus)) || (bm == a.M && bm <= 64 && bn == 16))
+    if ((bm == 0 && bn == 0 && gemm_short_m(a.M, a.N, (int64_t)a.K * eb * (a.split > 1 ? a.split : 1), eb == 4, cus)) || (bm == a.M && bm <= 64 && bn == 16))
         return gemm_mfma_skinny_dispatch(in_dt, out_dt, a, plan);
     const bool chosen_here = bm == 0 && bn == 0;
     if (bm == 0 && bn == 0) {

@@ -123,9 +123,11 @@ inline TileChoice gemm_choose(int64_t M, int64_t N, int64_t k_bytes, bool f32_in
 // 24 x 65536 x 1024 37.4 / 25.7; 64 x 262144 x 2048 265.0 / 209.7; 64 x 32768 x 1024 22.7 / 21.5; 64 x 24576 x 512
 // 16.3 / 12.6.  But 64 x 32768 x 2048 32.7 / 36.7; 64 x 28672 x 8192 95.7 / 134.8; 48 x 49152 x 8192 132.8 / 149.3;
 // 16 x 65536 x 2048 42.4 / 46 and 64 x 16384 x 2048 17.6 / 34.3.
-inline bool gemm_short_m(int64_t M, int64_t N, int64_t k_bytes, int cus) {
+// (fp32 operands stay on that kernel: their MFMA is slow enough for the empty part of a tile to cost more than it saves,
+// 32 x 65536 x 1024 73.2 us against 138.5 on tiles, 64 x 65536 x 2048 165.2 against 252.3.)
+inline bool gemm_short_m(int64_t M, int64_t N, int64_t k_bytes, bool f32_in, int cus) {
     if (M > 64 || k_bytes % 16) return false;
-    if (M <= 16) return true;
+    if (M <= 16 || f32_in) return true;
     const int64_t tiles = (N + 127) / 128;
     if (tiles > cus) return !(k_bytes <= 8192 || (M > 48 && tiles >= 2 * (int64_t)cus));
     return !(4 * tiles >= 3 * (int64_t)cus && k_bytes <= 2048);

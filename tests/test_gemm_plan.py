@@ -307,6 +307,7 @@ def test_known_shapes_run_on_the_instances_they_are_meant_for():
                            (64, 65536, 8192, "gemm_mfma_tn_256_w4"), (48, 49152, 8192, "gemm_mfma_skinny_lds"), (64, 32768, 2048, "gemm_mfma_skinny_lds"),
                            (64, 32768, 1024, "gemm_mfma_tn_128"), (16, 65536, 512, "gemm_mfma_skinny_lds"), (64, 32768, 2056, "gemm_mfma_skinny_lds")):
         assert run_case(bf16, bf16, M, N, K)["steps"][0]["family"] == fam, (M, N, K)
+    assert run_case(mh.F32, mh.F32, 64, 65536, 512)["steps"][0]["family"] == "gemm_mfma_skinny_lds"   # fp32 operands stay on the short-M kernel
     # small N and a long K: the library's own K ranges for the line kernel, then the reduction
     p = run_case(bf16, f32, 16, 1024, 32768, split_k=-1)
     assert p["steps"][0]["family"] == "gemm_mfma_skinny_lds" and p["steps"][0]["split"] == 4 and p["steps"][-1]["what"] == "splitk_reduce"

@@ -413,12 +413,15 @@ struct EwTiled {
     bool lds0, lds1, has1;
 };
 
-template <typename El, int TILE, bool kMap>
+// V = 2: a lane takes two neighbouring elements wherever it runs along a unit stride (4- and 8-byte accesses for 2- and
+// 4-byte elements); extents, pitches and pointers then have to be even (pairs_ok below).
+template <typename El, int TILE, int V, bool kMap>
 __global__ __launch_bounds__(256) void ew_tiled_kernel(int32_t op, typename El::compute ca, typename El::compute cb, bool b_is_zero,
                                                        typename El::storage* d, const typename El::storage* u0,
                                                        const typename El::storage* u1, EwTiled g) {
     typedef typename El::compute T;
     typedef typename El::storage S;
+    typedef S SV __attribute__((ext_vector_type(V == 1 ? 1 : 2)));
     extern __shared__ __align__(16) char tile_bytes[];  // one padded block per operand that goes through LDS
     S* const tile0 = reinterpret_cast<S*>(tile_bytes);
     S* const tile1 = tile0 + (g.lds0 ? TILE * (TILE + 1) : 0);
@@ -438,58 +441,95 @@ __global__ __launch_bounds__(256) void ew_tiled_kernel(int32_t op, typename El::
     }
     const int64_t p0 = (int64_t)tp * TILE, q0 = (int64_t)tq * TILE;
     const int np = (int)min((int64_t)TILE, g.ld.shape[0] - p0), nq = (int)min((int64_t)TILE, g.ld.shape[g.j] - q0);
-    const int lo = threadIdx.x % TILE, hi0 = threadIdx.x / TILE;
-    constexpr int STEP = 256 / TILE, IT = TILE / STEP;
+    constexpr int LR = TILE / V;  // lanes along a row of the block
+    const int lo = V * (threadIdx.x % LR), hi0 = threadIdx.x / LR;
+    constexpr int STEP = 256 / LR, IT = TILE / STEP;
     // (every loop below has IT trips with the bounds as predicates, so that a lane's IT loads are in flight together)
     // the operands that run along mode j: lanes along j, the block's rows of mode 0 one after the other
     if (g.lds0 || g.lds1) {
-        S r0[IT], r1[IT];
+        SV r0[IT], r1[IT];
 #pragma unroll
         for (int k = 0; k < IT; ++k) {
             const int lp = hi0 + k * STEP;
-            r0[k] = r1[k] = S(0);
+            r0[k] = r1[k] = SV(S(0));
             if (lo < nq && lp < np) {
-                if (g.lds0) r0[k] = u0[b0 + (p0 + lp) * g.l0.stride[0] + (q0 + lo)];
-                if (g.lds1) r1[k] = u1[b1 + (p0 + lp) * g.l1.stride[0] + (q0 + lo)];
+                if (g.lds0) r0[k] = *reinterpret_cast<const SV*>(u0 + b0 + (p0 + lp) * g.l0.stride[0] + (q0 + lo));
+                if (g.lds1) r1[k] = *reinterpret_cast<const SV*>(u1 + b1 + (p0 + lp) * g.l1.stride[0] + (q0 + lo));
             }
         }
 #pragma unroll
         for (int k = 0; k < IT; ++k) {
             const int lp = hi0 + k * STEP;
-            if (g.lds0) tile0[lp * (TILE + 1) + lo] = r0[k];
-            if (g.lds1) tile1[lp * (TILE + 1) + lo] = r1[k];
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                if (g.lds0) tile0[lp * (TILE + 1) + lo + e] = r0[k][e];
+                if (g.lds1) tile1[lp * (TILE + 1) + lo + e] = r1[k][e];
+            }
         }
         __syncthreads();
     }
-    S e0[IT], e1[IT], old[IT];
+    SV e0[IT], e1[IT], old[IT];
 #pragma unroll
     for (int k = 0; k < IT; ++k) {
         const int lq = hi0 + k * STEP;
         const bool in = lo < np && lq < nq;
-        e0[k] = e1[k] = old[k] = S(0);
-        if (g.lds0) e0[k] = tile0[lo * (TILE + 1) + lq];
-        else if (in) e0[k] = u0[b0 + (p0 + lo) * g.l0.stride[0] + (q0 + lq) * g.l0.stride[g.j]];
-        if (kMap && g.has1) {
-            if (g.lds1) e1[k] = tile1[lo * (TILE + 1) + lq];
-            else if (in) e1[k] = u1[b1 + (p0 + lo) * g.l1.stride[0] + (q0 + lq) * g.l1.stride[g.j]];
+        e0[k] = e1[k] = old[k] = SV(S(0));
+        if (g.lds0) {
+#pragma unroll
+            for (int e = 0; e < V; ++e) e0[k][e] = tile0[(lo + e) * (TILE + 1) + lq];
+        } else if (in) {
+            // (V = 2: the host has made sure of a unit stride along mode 0 for every operand read here)
+            e0[k] = *reinterpret_cast<const SV*>(u0 + b0 + (p0 + lo) * g.l0.stride[0] + (q0 + lq) * g.l0.stride[g.j]);
         }
-        if (!kMap && !b_is_zero && in) old[k] = d[bd + (p0 + lo) + (q0 + lq) * g.ld.stride[g.j]];
+        if (kMap && g.has1) {
+            if (g.lds1) {
+#pragma unroll
+                for (int e = 0; e < V; ++e) e1[k][e] = tile1[(lo + e) * (TILE + 1) + lq];
+            } else if (in) {
+                e1[k] = *reinterpret_cast<const SV*>(u1 + b1 + (p0 + lo) * g.l1.stride[0] + (q0 + lq) * g.l1.stride[g.j]);
+            }
+        }
+        if (!kMap && !b_is_zero && in) old[k] = *reinterpret_cast<const SV*>(d + bd + (p0 + lo) + (q0 + lq) * g.ld.stride[g.j]);
     }
 #pragma unroll
     for (int k = 0; k < IT; ++k) {
         const int lq = hi0 + k * STEP;
         if (lo >= np || lq >= nq) continue;
-        S* const dp = d + bd + (p0 + lo) + (q0 + lq) * g.ld.stride[g.j];
-        const T x = El::load(&e0[k]);
-        if constexpr (kMap) {
-            const T y = g.has1 ? El::load(&e1[k]) : cb;  // (cb: the scalar operand)
-            El::store(dp, El::round(map_op(op, x, y)));
-        } else {
-            const T ax = El::round(ca * x);
-            if (b_is_zero) El::store(dp, ax);
-            else El::store(dp, El::round(ax + El::round(cb * El::load(&old[k]))));
+        SV out;
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+            const S xe = e0[k][e], ye = e1[k][e], oe = old[k][e];
+            S re;
+            const T x = El::load(&xe);
+            if constexpr (kMap) {
+                const T y = g.has1 ? El::load(&ye) : cb;  // (cb: the scalar operand)
+                El::store(&re, El::round(map_op(op, x, y)));
+            } else {
+                const T ax = El::round(ca * x);
+                if (b_is_zero) El::store(&re, ax);
+                else El::store(&re, El::round(ax + El::round(cb * El::load(&oe))));
+            }
+            out[e] = re;
         }
+        *reinterpret_cast<SV*>(d + bd + (p0 + lo) + (q0 + lq) * g.ld.stride[g.j]) = out;
     }
+}
+
+// May the lanes take pairs?  Even extents along the two tiled modes, every array with a unit stride along the mode its
+// lanes run on, even strides elsewhere and a pointer on a whole pair.
+bool pairs_ok(const EwTiled& g, const void* d, const void* u0, const void* u1, size_t elem) {
+    if (elem > 4 || g.ld.shape[0] % 2 || g.ld.shape[g.j] % 2) return false;
+    auto even_but = [&](const ELayout& l, int unit) {
+        if (l.stride[unit] != 1) return false;
+        for (int m = 0; m < l.rank; ++m)
+            if (m != unit && l.shape[m] != 1 && l.stride[m] % 2) return false;
+        return true;
+    };
+    auto on_pair = [&](const void* p) { return reinterpret_cast<uintptr_t>(p) % (2 * elem) == 0; };
+    if (!even_but(g.ld, 0) || !on_pair(d)) return false;
+    if (!even_but(g.l0, g.lds0 ? g.j : 0) || !on_pair(u0)) return false;
+    if (g.has1 && (!even_but(g.l1, g.lds1 ? g.j : 0) || !on_pair(u1))) return false;
+    return true;
 }
 
 // Does the tiled kernel apply?  Layouts of one shape, ordered by the destination's strides (order_modes_by_stride), the
@@ -523,8 +563,30 @@ bool plan_tiled(const ELayout& ld, const ELayout* const* ops, int nops, int tile
 template <typename El>
 constexpr int tiled_edge() { return sizeof(typename El::storage) == 8 ? 32 : 64; }
 template <typename El>
-size_t tiled_lds(const EwTiled& g) {
-    return (size_t)((g.lds0 ? 1 : 0) + (g.lds1 ? 1 : 0)) * tiled_edge<El>() * (tiled_edge<El>() + 1) * sizeof(typename El::storage);
+constexpr int tiled_edge_pairs() { return sizeof(typename El::storage) == 2 ? 128 : 64; }
+template <typename El>
+size_t tiled_lds(const EwTiled& g, int edge) {
+    return (size_t)((g.lds0 ? 1 : 0) + (g.lds1 ? 1 : 0)) * edge * (edge + 1) * sizeof(typename El::storage);
+}
+// (the block edge of the pair form differs for 2-byte elements: the plan is made again for it)
+template <typename El, bool kMap>
+bool launch_tiled(int32_t op, typename El::compute ca, typename El::compute cb, bool b_is_zero, typename El::storage* d, const ELayout& ld,
+                  const typename El::storage* u0, const typename El::storage* u1, const ELayout* const* ops, int nops, int64_t n, hipStream_t st) {
+    EwTiled g;
+    if (!plan_tiled(ld, ops, nops, tiled_edge<El>(), &g)) return false;
+    const int64_t rest = n / (ld.shape[0] * ld.shape[g.j]);
+    if constexpr (sizeof(typename El::storage) <= 4) {
+        EwTiled g2;
+        constexpr int E2 = tiled_edge_pairs<El>();
+        // (two 2-byte operands through LDS would take 66 KB: above what a launch gets without asking)
+        if (pairs_ok(g, d, u0, u1, sizeof(typename El::storage)) && plan_tiled(ld, ops, nops, E2, &g2) && tiled_lds<El>(g2, E2) <= 65536) {
+            ew_tiled_kernel<El, E2, 2, kMap><<<(unsigned)((int64_t)g2.tiles_p * g2.tiles_q * rest), 256, tiled_lds<El>(g2, E2), st>>>(op, ca, cb, b_is_zero, d, u0, u1, g2);
+            return true;
+        }
+    }
+    constexpr int E1 = tiled_edge<El>();
+    ew_tiled_kernel<El, E1, 1, kMap><<<(unsigned)((int64_t)g.tiles_p * g.tiles_q * rest), 256, tiled_lds<El>(g, E1), st>>>(op, ca, cb, b_is_zero, d, u0, u1, g);
+    return true;
 }
 
 // Can every one of these (same-shape, stride-ordered) layouts be recast to pieces of `per` elements?  If so, does it.
@@ -608,13 +670,8 @@ static void launch_axpby(typename El::compute a, const void* x, const ELayout& l
         return;
     }
     if (!is_dense) {
-        EwTiled g;
         const ELayout* ops[1] = {&lx};
-        if (ordered && plan_tiled(ly, ops, 1, tiled_edge<El>(), &g)) {
-            const int64_t blocks = (int64_t)g.tiles_p * g.tiles_q * (n / (ly.shape[0] * ly.shape[g.j]));
-            ew_tiled_kernel<El, tiled_edge<El>(), false><<<(unsigned)blocks, 256, tiled_lds<El>(g), st>>>(0, a, b, b0, ys, xs, xs, g);
-            return;
-        }
+        if (ordered && launch_tiled<El, false>(0, a, b, b0, ys, ly, xs, xs, ops, 1, n, st)) return;
         const dim3 grid((unsigned)std::min<int64_t>((n + 255) / 256, 256 * 16));
         axpby_kernel<El><<<grid, 256, 0, st>>>(a, xs, lx, b, ys, ly, n, b0, same_modes_32(lx, ly, n));
         return;
@@ -639,13 +696,8 @@ static void launch_map(int32_t op, void* d, const ELayout& ld, const void* a, co
         return;
     }
     if (!is_dense) {
-        EwTiled g;
         const ELayout* ops[2] = {&la, &lb};
-        if (ordered && plan_tiled(ld, ops, bs ? 2 : 1, tiled_edge<El>(), &g)) {
-            const int64_t blocks = (int64_t)g.tiles_p * g.tiles_q * (n / (ld.shape[0] * ld.shape[g.j]));
-            ew_tiled_kernel<El, tiled_edge<El>(), true><<<(unsigned)blocks, 256, tiled_lds<El>(g), st>>>(op, s, s, false, ds, as, bs ? bs : as, g);
-            return;
-        }
+        if (ordered && launch_tiled<El, true>(op, s, s, false, ds, ld, as, bs ? bs : as, ops, bs ? 2 : 1, n, st)) return;
         const dim3 grid((unsigned)std::min<int64_t>((n + 255) / 256, 256 * 16));
         map_kernel<El><<<grid, 256, 0, st>>>(op, ds, ld, as, la, bs, lb, nb, s, n,
                                              same_modes_32(ld, la, n) && (!bs || (nb == n && same_modes_32(ld, lb, n))));

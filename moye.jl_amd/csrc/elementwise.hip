@@ -413,15 +413,15 @@ struct EwTiled {
     bool lds0, lds1, has1;
 };
 
-// V = 2: a lane takes two neighbouring elements wherever it runs along a unit stride (4- and 8-byte accesses for 2- and
-// 4-byte elements); extents, pitches and pointers then have to be even (pairs_ok below).
+// V > 1: a lane takes that many neighbouring elements wherever it runs along a unit stride (eight 2-byte or two 4-byte
+// elements); extents, pitches and pointers then have to be multiples of V (groups_ok below).
 template <typename El, int TILE, int V, bool kMap>
 __global__ __launch_bounds__(256) void ew_tiled_kernel(int32_t op, typename El::compute ca, typename El::compute cb, bool b_is_zero,
                                                        typename El::storage* d, const typename El::storage* u0,
                                                        const typename El::storage* u1, EwTiled g) {
     typedef typename El::compute T;
     typedef typename El::storage S;
-    typedef S SV __attribute__((ext_vector_type(V == 1 ? 1 : 2)));
+    typedef S SV __attribute__((ext_vector_type(V)));
     extern __shared__ __align__(16) char tile_bytes[];  // one padded block per operand that goes through LDS
     S* const tile0 = reinterpret_cast<S*>(tile_bytes);
     S* const tile1 = tile0 + (g.lds0 ? TILE * (TILE + 1) : 0);
@@ -515,20 +515,20 @@ __global__ __launch_bounds__(256) void ew_tiled_kernel(int32_t op, typename El::
     }
 }
 
-// May the lanes take pairs?  Even extents along the two tiled modes, every array with a unit stride along the mode its
-// lanes run on, even strides elsewhere and a pointer on a whole pair.
-bool pairs_ok(const EwTiled& g, const void* d, const void* u0, const void* u1, size_t elem) {
-    if (elem > 4 || g.ld.shape[0] % 2 || g.ld.shape[g.j] % 2) return false;
-    auto even_but = [&](const ELayout& l, int unit) {
+// May the lanes take groups of v?  Extents along the two tiled modes that are multiples of v, every array with a unit
+// stride along the mode its lanes run on, strides elsewhere that are multiples of v and a pointer on a whole group.
+bool groups_ok(const EwTiled& g, const void* d, const void* u0, const void* u1, size_t elem, int v) {
+    if (g.ld.shape[0] % v || g.ld.shape[g.j] % v) return false;
+    auto whole_but = [&](const ELayout& l, int unit) {
         if (l.stride[unit] != 1) return false;
         for (int m = 0; m < l.rank; ++m)
-            if (m != unit && l.shape[m] != 1 && l.stride[m] % 2) return false;
+            if (m != unit && l.shape[m] != 1 && l.stride[m] % v) return false;
         return true;
     };
-    auto on_pair = [&](const void* p) { return reinterpret_cast<uintptr_t>(p) % (2 * elem) == 0; };
-    if (!even_but(g.ld, 0) || !on_pair(d)) return false;
-    if (!even_but(g.l0, g.lds0 ? g.j : 0) || !on_pair(u0)) return false;
-    if (g.has1 && (!even_but(g.l1, g.lds1 ? g.j : 0) || !on_pair(u1))) return false;
+    auto on_group = [&](const void* p) { return reinterpret_cast<uintptr_t>(p) % (v * elem) == 0; };
+    if (!whole_but(g.ld, 0) || !on_group(d)) return false;
+    if (!whole_but(g.l0, g.lds0 ? g.j : 0) || !on_group(u0)) return false;
+    if (g.has1 && (!whole_but(g.l1, g.lds1 ? g.j : 0) || !on_group(u1))) return false;
     return true;
 }
 
@@ -568,7 +568,7 @@ template <typename El>
 size_t tiled_lds(const EwTiled& g, int edge) {
     return (size_t)((g.lds0 ? 1 : 0) + (g.lds1 ? 1 : 0)) * edge * (edge + 1) * sizeof(typename El::storage);
 }
-// (the block edge of the pair form differs for 2-byte elements: the plan is made again for it)
+// (the block edge of the form with groups differs for 2-byte elements: the plan is made again for it)
 template <typename El, bool kMap>
 bool launch_tiled(int32_t op, typename El::compute ca, typename El::compute cb, bool b_is_zero, typename El::storage* d, const ELayout& ld,
                   const typename El::storage* u0, const typename El::storage* u1, const ELayout* const* ops, int nops, int64_t n, hipStream_t st) {
@@ -577,10 +577,12 @@ bool launch_tiled(int32_t op, typename El::compute ca, typename El::compute cb, 
     const int64_t rest = n / (ld.shape[0] * ld.shape[g.j]);
     if constexpr (sizeof(typename El::storage) <= 4) {
         EwTiled g2;
-        constexpr int E2 = tiled_edge_pairs<El>();
+        // (8192^2, axpby! with X transposed / map! add with b transposed, TB/s: f32 two per lane 3.95 / 4.01, four 3.64 / 3.97;
+        // f16 two per lane 3.04 / 2.50, four 5.14 / 3.23, eight 5.90 / 3.61)
+        constexpr int E2 = tiled_edge_pairs<El>(), V2 = sizeof(typename El::storage) == 2 ? 8 : 2;
         // (two 2-byte operands through LDS would take 66 KB: above what a launch gets without asking)
-        if (pairs_ok(g, d, u0, u1, sizeof(typename El::storage)) && plan_tiled(ld, ops, nops, E2, &g2) && tiled_lds<El>(g2, E2) <= 65536) {
-            ew_tiled_kernel<El, E2, 2, kMap><<<(unsigned)((int64_t)g2.tiles_p * g2.tiles_q * rest), 256, tiled_lds<El>(g2, E2), st>>>(op, ca, cb, b_is_zero, d, u0, u1, g2);
+        if (groups_ok(g, d, u0, u1, sizeof(typename El::storage), V2) && plan_tiled(ld, ops, nops, E2, &g2) && tiled_lds<El>(g2, E2) <= 65536) {
+            ew_tiled_kernel<El, E2, V2, kMap><<<(unsigned)((int64_t)g2.tiles_p * g2.tiles_q * rest), 256, tiled_lds<El>(g2, E2), st>>>(op, ca, cb, b_is_zero, d, u0, u1, g2);
             return true;
         }
     }

@@ -577,10 +577,10 @@ def test_elementwise_with_a_transposed_operand_matches_the_dense_kernels(mh, dt)
     def flat(x):
         return _tens(mh, x, [x.numel()], [1])
 
-    # (even extents and pitches take the form with two elements per lane, odd ones the one with single elements)
-    for (R, C, Bn) in ((64, 64, 1), (200, 77, 1), (130, 1000, 3), (16, 16, 5), (1025, 129, 2), (258, 130, 2), (128, 384, 1), (1000, 61, 1)):
-        # destination d[b][r][c] with c contiguous and a pitch of C + 3 or C + 4 inside a frame; xt[b][c][r] with r contiguous
-        pad = 3 if C % 2 else 4           # (an even pitch lets the lanes take pairs)
+    # (extents and pitches that are multiples of two (4-byte elements) or eight (2-byte) take the form with groups per lane)
+    for (R, C, Bn) in ((64, 64, 1), (200, 77, 1), (130, 1000, 3), (16, 16, 5), (1025, 129, 2), (258, 130, 2), (128, 384, 1), (1000, 61, 1), (136, 264, 2)):
+        # destination d[b][r][c] with c contiguous and a pitch of C + 3 or C + 8 inside a frame; xt[b][c][r] with r contiguous
+        pad = 3 if C % 2 else 8           # (extents and pitches that are multiples of two or eight let the lanes take groups)
         frame = torch.full((Bn, R, C + pad), 55.0, device="cuda").to(tdt)
         x_same, xt, yt = rnd(Bn, R, C), rnd(Bn, C, R), rnd(Bn, C, R)
         shape, d_str = (C, R, Bn), (1, C + pad, R * (C + pad))

@@ -619,6 +619,29 @@ def test_elementwise_with_a_transposed_operand_matches_the_dense_kernels(mh, dt)
         assert torch.equal(d, x + y.t())
 
 
+@pytest.mark.parametrize("dt", ["float32", "float16", "float64"])
+def test_map_with_operands_that_repeat_along_a_mode(mh, dt):
+    """Operands with a zero stride (one value per row or per column of dst), alone and next to a transposed operand, which
+    sends the call through the LDS blocks: one rounded operation, so torch's result bit for bit."""
+    tdt = getattr(torch, dt)
+    g = torch.Generator(device="cuda").manual_seed(3)
+    for (R, C) in ((64, 64), (200, 136), (130, 77), (1024, 512)):
+        a = torch.randn(R, C, generator=g, device="cuda").to(tdt)
+        at = torch.randn(C, R, generator=g, device="cuda").to(tdt)
+        col = torch.randn(R, generator=g, device="cuda").to(tdt)
+        row = torch.randn(C, generator=g, device="cuda").to(tdt)
+        for name, ta, tb, want in (
+                ("a + one per row", _tens(mh, a, (R, C), (C, 1)), _tens(mh, col, (R, C), (1, 0)), a + col[:, None]),
+                ("a + one per column", _tens(mh, a, (R, C), (C, 1)), _tens(mh, row, (R, C), (0, 1)), a + row[None, :]),
+                ("a' + one per row", _tens(mh, at, (R, C), (1, R)), _tens(mh, col, (R, C), (1, 0)), at.t() + col[:, None]),
+                ("a' + one per column", _tens(mh, at, (R, C), (1, R)), _tens(mh, row, (R, C), (0, 1)), at.t() + row[None, :]),
+                ("one per row + a'", _tens(mh, col, (R, C), (1, 0)), _tens(mh, at, (R, C), (1, R)), col[:, None] + at.t())):
+            d = torch.zeros(R, C, device="cuda", dtype=tdt)
+            mh.map_("add", _tens(mh, d, (R, C), (C, 1)), ta, tb)
+            torch.cuda.synchronize()
+            assert torch.equal(d, want.to(tdt)), (dt, R, C, name)
+
+
 def test_axpby_errors(mh):
     x = torch.zeros(8, device="cuda")
     y = torch.zeros(8, dtype=torch.float16, device="cuda")

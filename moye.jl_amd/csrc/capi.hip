@@ -139,27 +139,24 @@ static size_t kmajor_bytes(const Mat& m) {
     return (size_t)(m.rows * pitch + 255) / 256 * 256;
 }
 
-// K ranges for the short-M kernel that stages lines through LDS, when N is small and K long: its workgroups take 16
-// rows of B each (32 once that still gives every CU one), so N = 1024 puts 64 workgroups on 256 CUs, and a workgroup
-// streams its rows at about 64 GB/s whatever the others do.  A model of the two forms, in microseconds, fitted to bf16
-// timings (M = 16: 1024 x 32768 37.8 unsplit, 18.3 in four ranges; 2048 x 16384 22.2, 17.1 in two; 1024 x 8192 12.1,
-// 10.7 in four; 2048 x 8192 12.6, 11.7 in two: left alone; M = 32, 1024 x 8192 15.6, 10.7 in four; M = 64, 2048 x 8192
-// 22.7, 17.9 in two, 20.4 in four): unsplit 4.5 + the longer of all bytes at 6 TB/s and a workgroup's bytes at 64 GB/s;
-// in s ranges 7.5 + the same with a workgroup's bytes divided by s, never under 10.7 (two launches).  Ranges are whole
-// lines of 2 KiB and more; at most two above M = 32 (every workgroup reads its range of all of A, which then dominates);
-// taken when the model gains a tenth, the fewest ranges within 5 % of the best.
+// K ranges for the short-M kernel that stages lines through LDS, when N is small and K long: N = 1024 puts 64 workgroups
+// of 16 rows of B on 256 CUs, and a workgroup streams its rows at about 64 GB/s whatever the others do.  The model of
+// gemm_short_m_us (gemm_plan.hpp), fitted to bf16 timings (M = 16: 1024 x 32768 37.8 unsplit, 18.3 in four ranges;
+// 2048 x 16384 22.2, 17.1 in two; 1024 x 8192 12.1, 10.7 in four; 2048 x 8192 12.6, 11.7 in two: left alone; M = 32,
+// 1024 x 8192 15.6, 10.7 in four; M = 64, 2048 x 8192 22.7, 17.9 in two, 20.4 in four).  Ranges are whole lines of 2 KiB
+// and more; at most two above M = 32 (every workgroup reads its range of all of A, which then dominates); taken when
+// the model gains a tenth, the fewest ranges within 5 % of the best.
 static int skinny_lines_split(int64_t M, int64_t N, int64_t k_bytes, int cus) {
     if ((N + 31) / 32 >= cus) return 1;  // 32 rows of B per workgroup and every CU has one
-    const double floor_us = (double)(N + M) * (double)k_bytes / 6.0e6;
-    const double wg_us = (double)(16 + 16 * ((M + 15) / 16)) * (double)k_bytes / 64.0e3;
-    const double t1 = 4.5 + std::max(floor_us, wg_us);
+    double t1;
+    gemm_short_m_ntw(M, N, k_bytes, cus, 1, &t1);
     double t[9];
     double best = t1;
     const int max_split = M > 32 ? 2 : 8;
     for (int sp = 2; sp <= max_split; ++sp) {
         t[sp] = 1e30;
         if (k_bytes % ((int64_t)sp * kSkinnyLineBytes) || k_bytes / sp < 2048) continue;
-        t[sp] = std::max(10.7, 7.5 + std::max(floor_us, wg_us / sp));
+        gemm_short_m_ntw(M, N, k_bytes, cus, sp, &t[sp]);
         best = std::min(best, t[sp]);
     }
     if (best > 0.9 * t1) return 1;

@@ -10,6 +10,7 @@
 // Stands where the reference's user kernel would run gemm! (src/algorithm/blas.jl:11-131) on a
 // 16-row problem with its usual 128 x 128 tiles and waste 7/8 of each tile.
 #include "mfma_common.hpp"
+#include "gemm_plan.hpp"
 
 namespace moye {
 
@@ -182,13 +183,14 @@ static int32_t launch_skinny_lds(const GemmArgs& a, GemmPlan& plan) {
     // B without the non-temporal hint 23.6.  As with the transposes, less in flight is faster on this part, down to what
     // covers the latency.  32 rows per workgroup once that gives every CU one (bf16, K = 8192: N = 16384 40.1 us against
     // 45.3 with 16 rows; N = 4096 17.9 against 13.5).
-    const bool wide = (a.N + 31) / 32 >= plan.shape.cus;
-    // More than 32 rows of A and enough columns for 64 rows of B per workgroup on every CU: every workgroup reads all of A
-    // out of the L2s, which with 32 rows of B is twice B's own bytes (bf16 64 x 28672 x 8192: 118.8 us with 32 rows, 95.3 with 64).
-    // Two buffers instead of three, for the LDS.
-    if ((a.M + 15) / 16 >= 3 && (a.N + 63) / 64 >= plan.shape.cus)
+    // (which of them: gemm_short_m_ntw, gemm_plan.hpp -- the rounds the workgroups of a launch need on the CUs decide)
+    const int ranges = a.split > 1 ? a.split : 1;
+    const int ntw = gemm_short_m_ntw(a.M, a.N, (int64_t)a.K * In::kBytes * ranges, plan.shape.cus, ranges);
+    // (64 rows: two buffers instead of three, for the LDS; from 33 rows of A on, where every workgroup's reads of all of A
+    // out of the L2s weigh most: bf16 64 x 28672 x 8192 118.8 us with 32 rows, 95.3 with 64)
+    if (ntw == 4)
         return (a.M + 15) / 16 == 3 ? launch_skinny_lds_v<In, Out, 3, W, 4, 2, 2>(a, plan) : launch_skinny_lds_v<In, Out, 4, W, 4, 2, 2>(a, plan);
-    if (wide) {
+    if (ntw == 2) {
         switch ((a.M + 15) / 16) {
             case 1: return launch_skinny_lds_v<In, Out, 1, W, 2, 3, 2>(a, plan);
             case 2: return launch_skinny_lds_v<In, Out, 2, W, 2, 3, 2>(a, plan);

@@ -133,4 +133,34 @@ inline bool gemm_short_m(int64_t M, int64_t N, int64_t k_bytes, bool f32_in, int
     return !(4 * tiles >= 3 * (int64_t)cus && k_bytes <= 2048);
 }
 
+// The short-M kernel's workgroups take 16, 32 or (from 33 rows of A on) 64 rows of B and all of A, one workgroup on a CU
+// at a time (its rings fill the LDS), and a workgroup streams its rows at about 64 GB/s whatever the others do (52 with
+// 64 rows of B: two buffers instead of three).  A launch therefore takes as many rounds as its workgroups -- times the K
+// ranges of a split -- need on the CUs: bf16 64 x 12288 x 8192 57.7 us on 384 workgroups of 32 rows, 46.3 on 192 of 64;
+// 64 x 14336 x 4096 33.6 / 27.2; 48 x 10240 x 8192 51.1 / 40.1; but 64 x 8192 x 8192 31.1 on 256 of 32 rows, 43.8 on 128
+// of 64; 64 x 4096 x 14336 42.0 unsplit on 256 workgroups of 16 rows, 47.0 in two K ranges on 512.  In microseconds:
+// 4.5 (two launches of a split: 7.5, and never under 10.7) + the longer of all bytes at 6 TB/s and rounds x a workgroup's
+// bytes at its rate.
+inline double gemm_short_m_us(int64_t M, int64_t N, int64_t k_bytes, int cus, int ntw, int split) {
+    const int mt = (int)((M + 15) / 16);
+    const int64_t wgs = (N + 16 * ntw - 1) / (16 * ntw) * split, rounds = (wgs + cus - 1) / cus;
+    const double wg_us = (double)(16 * ntw + 16 * mt) * ((double)k_bytes / split) / (ntw == 4 ? 52.0e3 : 64.0e3);
+    const double floor_us = (double)(N + M) * (double)k_bytes / 6.0e6;
+    const double t = floor_us > (double)rounds * wg_us ? floor_us : (double)rounds * wg_us;
+    if (split > 1) return 7.5 + t > 10.7 ? 7.5 + t : 10.7;
+    return 4.5 + t;
+}
+// 16-row blocks of B per workgroup for a launch in `split` K ranges: the cheapest, more rows on a tie (fewer rounds)
+inline int gemm_short_m_ntw(int64_t M, int64_t N, int64_t k_bytes, int cus, int split, double* us = nullptr) {
+    int best = 1;
+    double best_us = 1e30;
+    for (int ntw : {1, 2, 4}) {
+        if (ntw == 4 && M <= 32) continue;
+        const double t = gemm_short_m_us(M, N, k_bytes, cus, ntw, split);
+        if (t <= best_us) { best_us = t; best = ntw; }
+    }
+    if (us) *us = best_us;
+    return best;
+}
+
 }  // namespace moye

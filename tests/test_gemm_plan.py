@@ -297,10 +297,15 @@ def test_known_shapes_run_on_the_instances_they_are_meant_for():
     # short M: whole 128-byte lines of K through LDS, a K tail as a masked trip of the same kernel
     assert step_names(run_case(bf16, f32, 16, 8192, 8192))[0].startswith("gemm_mfma_skinny_lds<InBF16,OutF32,mt=1,ntw=2,waves=4,stages=3>")
     assert step_names(run_case(bf16, f32, 16, 8192, 8224))[0].startswith("gemm_mfma_skinny_lds<InBF16,OutF32,mt=1,ntw=2,")   # a K tail too
-    # more than 32 rows of A: 64 rows of B per workgroup once that still gives every CU one, 32 below that
+    # more than 32 rows of A: 64 rows of B per workgroup where 32 rows would need more rounds on the CUs
     assert step_names(run_case(bf16, bf16, 64, 28672, 8192))[0].startswith("gemm_mfma_skinny_lds<InBF16,OutBF16,mt=4,ntw=4,waves=4,stages=2>")
     assert step_names(run_case(bf16, bf16, 48, 16384, 4096))[0].startswith("gemm_mfma_skinny_lds<InBF16,OutBF16,mt=3,ntw=4,waves=4,stages=2>")
     assert ",ntw=2," in step_names(run_case(bf16, bf16, 64, 8192, 8192))[0]
+    assert ",ntw=4," in step_names(run_case(bf16, bf16, 64, 12288, 8192))[0] and ",ntw=2," in step_names(run_case(bf16, bf16, 16, 6144, 8192))[0]
+    assert ",ntw=1," in step_names(run_case(bf16, bf16, 16, 4096, 8192))[0]
+    # K ranges count against the CUs as well: 256 workgroups of 16 rows stay whole, 128 of 32 rows take two ranges
+    p = run_case(bf16, f32, 64, 4096, 14336, split_k=-1)
+    assert p["steps"][0]["split"] == 2 and ",ntw=2," in p["steps"][0]["name"], p["text"]
     # more than 16 rows and more 128-wide tiles than CUs (a very short K: three quarters of the CUs): tiles, not the short-M kernel
     for (M, N, K, fam) in ((64, 65536, 2048, "gemm_mfma_tn_256_w4"), (17, 24576, 512, "gemm_mfma_tn_128"), (64, 65536, 3072, "gemm_mfma_tn_256_w4"),
                            (64, 131072, 4096, "gemm_mfma_tn_256_w4"), (64, 65536, 4096, "gemm_mfma_tn_256_w4"), (64, 24448, 512, "gemm_mfma_skinny_lds"),

@@ -657,13 +657,14 @@ def test_short_m_small_n_long_k_takes_k_ranges(mh):
 
 @pytest.mark.parametrize("M", [33, 48, 64])
 def test_short_m_sixty_four_rows_of_b_per_workgroup(mh, M):
-    """More than 32 rows of A and an N that gives every CU a workgroup of 64 rows of B: the form with ntw=4 and two
-    stages; N ragged against 64, K with and without a tail, every input type, D inside a frame; exact on small integers."""
+    """More than 32 rows of A and an N whose workgroups of 32 rows of B would need a second round on the CUs while those of
+    64 rows need one: the form with ntw=4 and two stages; N ragged against 64, K with and without a tail, every input
+    type, D inside a frame; exact on small integers."""
     g = torch.Generator().manual_seed(700 + M)
     for (tdt, atom) in ((torch.float16, mh.MFMA_F32_16x16x32_F16), (torch.bfloat16, mh.MFMA_F32_16x16x32_BF16),
                         (torch.float8_e4m3fn, mh.MFMA_F32_16x16x32_FP8)):
         eb = tdt.itemsize
-        for (N, K) in ((16384, 256 // eb), (16400 + M, 1280 // eb), (16385, 464 // eb)):
+        for (N, K) in ((16384, 256 // eb), (16256 + M, 1280 // eb), (12289, 464 // eb)):   # 256, 255 and 193 workgroups of 64 rows
             A = torch.randint(-2, 3, (M, K), generator=g).float()
             B = torch.randint(-2, 3, (N, K), generator=g).float()
             a, b = A.cuda().to(tdt), B.cuda().to(tdt)
